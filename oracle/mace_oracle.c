@@ -1,0 +1,459 @@
+/*
+ * CPU oracle for MACE's matrix-multiplication path.  TEST INFRASTRUCTURE ONLY: see
+ * mace_oracle.h.  Build: make -C oracle  (gcc -O2 -ffp-contract=off -fopenmp).
+ *
+ * The loops are written in the order the reference writes them so that float results
+ * carry the same rounding sequence; `nthreads` only splits the outermost independent
+ * index (rows), which never changes a result.
+ */
+#include "mace_oracle.h"
+
+#include <limits.h>
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#define ORC_PARALLEL_FOR(nt) _Pragma("omp parallel for schedule(static) num_threads(nt)")
+#else
+#define ORC_PARALLEL_FOR(nt)
+#endif
+
+static int orc_threads(int nthreads) { return nthreads < 1 ? 1 : nthreads; }
+
+/* mace/ops/common/matrix.h:48-80: (r,c) -> r*rows_stride + c*cols_stride with
+ * stride = cols for RowMajor, rows for ColMajor. */
+static inline int64_t orc_idx(int major, int64_t rows, int64_t cols, int64_t r, int64_t c) {
+  return major == ORC_COL_MAJOR ? r + c * rows : r * cols + c;
+}
+
+/* ------------------------------------------------------------------------------------
+ * Scalar helpers
+ * ---------------------------------------------------------------------------------- */
+
+/* mace/core/quantize.h:68-78  Saturate<uint8_t>: truncate to int, clamp to [0,255].
+ * The reference's float->int cast is undefined for |v| >= 2^31; the oracle clamps in the
+ * float domain first, which agrees with the reference wherever the reference is defined. */
+uint8_t orc_saturate_u8(float v) {
+  if (!(v > 0.0f)) return 0;          /* also NaN -> 0 */
+  if (v >= 255.0f) return 255;
+  int r = (int)v;
+  return (uint8_t)r;
+}
+
+/* mace/core/quantize.h:80-83 */
+uint8_t orc_quantize_u8(float value, float scale, int32_t zero_point) {
+  return orc_saturate_u8(roundf(value / scale + (float)zero_point));
+}
+
+/* mace/core/quantize.h:104-114 */
+void orc_quantize_multiplier(double multiplier, int32_t *out_mult, int *out_exp) {
+  int e = 0;
+  const double q = frexp(multiplier, &e);
+  int64_t qint = (int64_t)roundl((long double)(q * (double)(1ll << 31)));
+  if (qint == (1ll << 31)) {
+    qint /= 2;
+    ++e;
+  }
+  *out_mult = (int32_t)qint;
+  *out_exp = e;
+}
+
+/* mace/core/quantize.h:116-126.  Returns 0 on success, 1 where the reference CHECK-fails
+ * (multiplier outside (0,1) or negative right shift). */
+int orc_get_output_multiplier_and_shift(float lhs_scale, float rhs_scale, float out_scale,
+                                        int32_t *mult, int *right_shift) {
+  float real_multiplier = lhs_scale * rhs_scale / out_scale;
+  if (!(real_multiplier > 0.f && real_multiplier < 1.f)) return 1;
+  int e;
+  orc_quantize_multiplier((double)real_multiplier, mult, &e);
+  *right_shift = -e;
+  return *right_shift >= 0 ? 0 : 1;
+}
+
+/* gemmlowp fixedpoint/fixedpoint.h SaturatingRoundingDoublingHighMul (int32). */
+int32_t orc_srdhm(int32_t a, int32_t b) {
+  if (a == INT32_MIN && b == INT32_MIN) return INT32_MAX;
+  int64_t ab = (int64_t)a * (int64_t)b;
+  int64_t nudge = ab >= 0 ? (1ll << 30) : (1 - (1ll << 30));
+  return (int32_t)((ab + nudge) / (1ll << 31));  /* C division truncates toward zero */
+}
+
+/* gemmlowp fixedpoint/fixedpoint.h RoundingDivideByPOT (int32). */
+int32_t orc_rdivpot(int32_t x, int exponent) {
+  const int32_t mask = (int32_t)((1ll << exponent) - 1);
+  const int32_t remainder = x & mask;
+  const int32_t threshold = (mask >> 1) + (x < 0 ? 1 : 0);
+  /* >> on a negative int32 is an arithmetic shift with gcc/clang (what gemmlowp relies on) */
+  return (x >> exponent) + (remainder > threshold ? 1 : 0);
+}
+
+/* gemmlowp public/output_stages.h: OutputStageQuantizeDownInt32ToUint8ScaleByFixedPoint
+ * followed by OutputStageSaturatingCastToUint8, as assembled at
+ * mace/ops/common/gemmlowp_util.h:37-74.  [clamp_min, clamp_max] narrows the saturating
+ * cast (0,255 = the reference); it realises the quantised ReLUx of
+ * mace/ops/arm/q8/activation.cc:59-94 when fused. */
+uint8_t orc_requant_fixed_u8(int32_t acc, int32_t mult, int right_shift,
+                             int32_t offset_after_shift, int clamp_min, int clamp_max) {
+  int32_t y = orc_srdhm(acc, mult);
+  int64_t z = (int64_t)orc_rdivpot(y, right_shift) + (int64_t)offset_after_shift;
+  if (z < clamp_min) z = clamp_min;
+  if (z > clamp_max) z = clamp_max;
+  return (uint8_t)z;
+}
+
+/* mace/ops/arm/q8/quantization_util.cc:20-46 */
+int orc_get_bias_data(const int32_t *bias, float bias_scale, float input_scale,
+                      float filter_scale, int64_t channels, int32_t *out) {
+  if (bias == NULL) {
+    memset(out, 0, (size_t)channels * sizeof(int32_t));
+    return 0;
+  }
+  float prod = input_scale * filter_scale;
+  int adjust = fabs((double)(float)(prod - bias_scale)) > 1e-6;
+  if (!adjust) {
+    memcpy(out, bias, (size_t)channels * sizeof(int32_t));
+    return 0;
+  }
+  float adjust_scale = bias_scale / prod;
+  for (int64_t i = 0; i < channels; ++i) {
+    out[i] = (int32_t)roundf((float)bias[i] * adjust_scale);
+  }
+  return 1;
+}
+
+/* ------------------------------------------------------------------------------------
+ * fp32 Gemm / Gemv
+ * ---------------------------------------------------------------------------------- */
+
+/* mace/ops/ref/gemm.cc:58-106: float sum = 0; for d ascending: sum += l * r. */
+void orc_gemm_f32(const float *lhs, const float *rhs, int64_t batch, int64_t rows,
+                  int64_t cols, int64_t depth, int lhs_major, int rhs_major,
+                  int out_major, int lhs_batched, int rhs_batched, float *out,
+                  int nthreads) {
+  const int nt = orc_threads(nthreads);
+  for (int64_t b = 0; b < batch; ++b) {
+    const float *l = lhs + (lhs_batched ? 1 : 0) * b * rows * depth;
+    const float *r = rhs + (rhs_batched ? 1 : 0) * b * depth * cols;
+    float *o = out + b * rows * cols;
+    ORC_PARALLEL_FOR(nt)
+    for (int64_t i = 0; i < rows; ++i) {
+      for (int64_t c = 0; c < cols; ++c) {
+        float sum = 0;
+        for (int64_t d = 0; d < depth; ++d) {
+          sum += l[orc_idx(lhs_major, rows, depth, i, d)] *
+                 r[orc_idx(rhs_major, depth, cols, d, c)];
+        }
+        o[orc_idx(out_major, rows, cols, i, c)] = sum;
+      }
+    }
+  }
+}
+
+void orc_gemm_f32_acc64(const float *lhs, const float *rhs, int64_t batch, int64_t rows,
+                        int64_t cols, int64_t depth, int lhs_major, int rhs_major,
+                        int out_major, int lhs_batched, int rhs_batched, float *out,
+                        int nthreads) {
+  const int nt = orc_threads(nthreads);
+  for (int64_t b = 0; b < batch; ++b) {
+    const float *l = lhs + (lhs_batched ? 1 : 0) * b * rows * depth;
+    const float *r = rhs + (rhs_batched ? 1 : 0) * b * depth * cols;
+    float *o = out + b * rows * cols;
+    ORC_PARALLEL_FOR(nt)
+    for (int64_t i = 0; i < rows; ++i) {
+      for (int64_t c = 0; c < cols; ++c) {
+        double sum = 0;
+        for (int64_t d = 0; d < depth; ++d) {
+          sum += (double)l[orc_idx(lhs_major, rows, depth, i, d)] *
+                 (double)r[orc_idx(rhs_major, depth, cols, d, c)];
+        }
+        o[orc_idx(out_major, rows, cols, i, c)] = (float)sum;
+      }
+    }
+  }
+}
+
+/* mace/ops/ref/gemv.cc:46-81: float sum = bias ? bias[h] : 0; for w ascending. */
+void orc_gemv_f32(const float *lhs, const float *rhs, const float *bias, int64_t batch,
+                  int64_t height, int64_t width, int lhs_batched, int rhs_batched,
+                  float *out, int nthreads) {
+  const int nt = orc_threads(nthreads);
+  for (int64_t b = 0; b < batch; ++b) {
+    const float *l = lhs + (lhs_batched ? 1 : 0) * b * height * width;
+    const float *r = rhs + (rhs_batched ? 1 : 0) * b * width;
+    ORC_PARALLEL_FOR(nt)
+    for (int64_t h = 0; h < height; ++h) {
+      float sum = bias ? bias[h] : 0.f;
+      for (int64_t w = 0; w < width; ++w) {
+        sum += l[h * width + w] * r[w];
+      }
+      out[b * height + h] = sum;
+    }
+  }
+}
+
+/* mace/ops/ref/bias_add.cc:74-100 (NCHW, rank-1 bias) */
+void orc_bias_add_nchw_f32(float *data, const float *bias, int64_t batch,
+                           int64_t channels, int64_t hw) {
+  for (int64_t b = 0; b < batch; ++b)
+    for (int64_t c = 0; c < channels; ++c) {
+      float *p = data + (b * channels + c) * hw;
+      const float bv = bias[c];
+      for (int64_t i = 0; i < hw; ++i) p[i] = p[i] + bv;
+    }
+}
+
+/* mace/ops/ref/activation.cc:61-75: RELU = max(0,x); RELUX = max(0, min(limit, x)) */
+void orc_activation_f32(float *data, int64_t n, int act, float limit) {
+  if (act == ORC_ACT_RELU) {
+    for (int64_t i = 0; i < n; ++i) data[i] = data[i] > 0.f ? data[i] : 0.f;
+  } else if (act == ORC_ACT_RELUX) {
+    for (int64_t i = 0; i < n; ++i) {
+      float m = data[i] < limit ? data[i] : limit;   /* std::min(limit_, x) */
+      data[i] = m > 0.f ? m : 0.f;                   /* std::max(0.f, m)    */
+    }
+  }
+}
+
+/* ------------------------------------------------------------------------------------
+ * q8 Gemv
+ * ---------------------------------------------------------------------------------- */
+
+/* mace/ops/ref/q8/gemv.cc:124-162 */
+void orc_q8_gemv_i32(const uint8_t *lhs, const uint8_t *rhs, const int32_t *bias,
+                     int64_t batch, int64_t height, int64_t width, int lhs_batched,
+                     int rhs_batched, int32_t lhs_zp, int32_t rhs_zp, int32_t *out,
+                     int nthreads) {
+  const int nt = orc_threads(nthreads);
+  for (int64_t b = 0; b < batch; ++b) {
+    const uint8_t *l = lhs + (lhs_batched ? 1 : 0) * b * height * width;
+    const uint8_t *r = rhs + (rhs_batched ? 1 : 0) * b * width;
+    ORC_PARALLEL_FOR(nt)
+    for (int64_t h = 0; h < height; ++h) {
+      int32_t sum = bias ? bias[h] : 0;
+      for (int64_t w = 0; w < width; ++w) {
+        sum += ((int32_t)l[h * width + w] - lhs_zp) * ((int32_t)r[w] - rhs_zp);
+      }
+      out[b * height + h] = sum;
+    }
+  }
+}
+
+/* mace/ops/ref/q8/gemv.cc:80-122 (mode REF) and the requantisation line of
+ * mace/ops/arm/q8/gemv.cc:159-161 (mode NEON).  The multiplier is formed in binary32,
+ * left to right: (lhs_scale * rhs_scale) / out_scale. */
+void orc_q8_gemv_u8(const uint8_t *lhs, const uint8_t *rhs, const int32_t *bias,
+                    int64_t batch, int64_t height, int64_t width, int lhs_batched,
+                    int rhs_batched, int32_t lhs_zp, int32_t rhs_zp, float lhs_scale,
+                    float rhs_scale, float out_scale, int32_t out_zp, int mode,
+                    uint8_t *out, int nthreads) {
+  const int nt = orc_threads(nthreads);
+  const float m = lhs_scale * rhs_scale / out_scale;
+  for (int64_t b = 0; b < batch; ++b) {
+    const uint8_t *l = lhs + (lhs_batched ? 1 : 0) * b * height * width;
+    const uint8_t *r = rhs + (rhs_batched ? 1 : 0) * b * width;
+    ORC_PARALLEL_FOR(nt)
+    for (int64_t h = 0; h < height; ++h) {
+      int32_t sum = bias ? bias[h] : 0;
+      for (int64_t w = 0; w < width; ++w) {
+        sum += ((int32_t)l[h * width + w] - lhs_zp) * ((int32_t)r[w] - rhs_zp);
+      }
+      float scaled = (float)sum * m;
+      if (mode == ORC_REQUANT_NEON) scaled = scaled + (float)out_zp;
+      out[b * height + h] = orc_saturate_u8(roundf(scaled));
+    }
+  }
+}
+
+/* mace/ops/arm/q8/gemv.cc:72-157: dot, sum_lhs, sum_rhs in uint32 and the expansion
+ * ret = dot - sum_lhs*rhs_zp - sum_rhs*lhs_zp + lhs_zp*rhs_zp*W (+ bias). */
+void orc_q8_gemv_i32_expanded(const uint8_t *lhs, const uint8_t *rhs, const int32_t *bias,
+                              int64_t batch, int64_t height, int64_t width,
+                              int lhs_batched, int rhs_batched, int32_t lhs_zp,
+                              int32_t rhs_zp, int32_t *out) {
+  for (int64_t b = 0; b < batch; ++b) {
+    const uint8_t *l = lhs + (lhs_batched ? 1 : 0) * b * height * width;
+    const uint8_t *r = rhs + (rhs_batched ? 1 : 0) * b * width;
+    uint32_t sum_rhs = 0;
+    for (int64_t i = 0; i < width; ++i) sum_rhs += (uint32_t)r[i];
+    for (int64_t h = 0; h < height; ++h) {
+      uint32_t dot = 0, sum_lhs = 0;
+      for (int64_t w = 0; w < width; ++w) {
+        dot += (uint32_t)l[h * width + w] * (uint32_t)r[w];
+        sum_lhs += (uint32_t)l[h * width + w];
+      }
+      const uint32_t zero_point_dot =
+          (uint32_t)lhs_zp * (uint32_t)rhs_zp * (uint32_t)width;
+      uint32_t ret = dot - sum_lhs * (uint32_t)rhs_zp - sum_rhs * (uint32_t)lhs_zp +
+                     zero_point_dot;
+      if (bias) ret += (uint32_t)bias[h];
+      out[b * height + h] = (int32_t)ret;
+    }
+  }
+}
+
+/* ------------------------------------------------------------------------------------
+ * q8 GEMM: what gemmlowp::GemmWithOutputPipeline computes at mace/ops/matmul.cc:298-300,
+ * 383-385 and mace/ops/conv_2d.cc:312-315:
+ *   acc[i,j] = sum_k (lhs[i,k] + lhs_offset) * (rhs[k,j] + rhs_offset)   (exact int32)
+ * ---------------------------------------------------------------------------------- */
+
+void orc_q8_gemm_i32_naive(const uint8_t *lhs, const uint8_t *rhs, int64_t batch,
+                           int64_t rows, int64_t cols, int64_t depth, int lhs_order,
+                           int rhs_order, int out_order, int lhs_batched,
+                           int rhs_batched, int32_t lhs_offset, int32_t rhs_offset,
+                           int32_t *out) {
+  for (int64_t b = 0; b < batch; ++b) {
+    const uint8_t *l = lhs + (lhs_batched ? 1 : 0) * b * rows * depth;
+    const uint8_t *r = rhs + (rhs_batched ? 1 : 0) * b * depth * cols;
+    int32_t *o = out + b * rows * cols;
+    for (int64_t i = 0; i < rows; ++i)
+      for (int64_t j = 0; j < cols; ++j) {
+        int32_t acc = 0;
+        for (int64_t k = 0; k < depth; ++k) {
+          acc += ((int32_t)l[orc_idx(lhs_order, rows, depth, i, k)] + lhs_offset) *
+                 ((int32_t)r[orc_idx(rhs_order, depth, cols, k, j)] + rhs_offset);
+        }
+        o[orc_idx(out_order, rows, cols, i, j)] = acc;
+      }
+  }
+}
+
+/* Blocked form: copies both operands into K-contiguous int16 panels (values already offset),
+ * then int32 dot products that the compiler vectorises.  Exact, so equal to the naive loop
+ * whenever no int32 overflow occurs (|acc| <= 255*255*depth < 2^31 for depth <= 33025). */
+void orc_q8_gemm_i32(const uint8_t *lhs, const uint8_t *rhs, int64_t batch, int64_t rows,
+                     int64_t cols, int64_t depth, int lhs_order, int rhs_order,
+                     int out_order, int lhs_batched, int rhs_batched, int32_t lhs_offset,
+                     int32_t rhs_offset, int32_t *out, int nthreads) {
+  const int nt = orc_threads(nthreads);
+  if (rows <= 0 || cols <= 0 || batch <= 0) return;
+  const int64_t dpad = depth > 0 ? depth : 1;
+  int16_t *lp = (int16_t *)malloc((size_t)rows * dpad * sizeof(int16_t));
+  int16_t *rp = (int16_t *)malloc((size_t)cols * dpad * sizeof(int16_t));
+  for (int64_t b = 0; b < batch; ++b) {
+    const uint8_t *l = lhs + (lhs_batched ? 1 : 0) * b * rows * depth;
+    const uint8_t *r = rhs + (rhs_batched ? 1 : 0) * b * depth * cols;
+    int32_t *o = out + b * rows * cols;
+    if (b == 0 || lhs_batched) {
+      ORC_PARALLEL_FOR(nt)
+      for (int64_t i = 0; i < rows; ++i)
+        for (int64_t k = 0; k < depth; ++k)
+          lp[i * depth + k] =
+              (int16_t)((int32_t)l[orc_idx(lhs_order, rows, depth, i, k)] + lhs_offset);
+    }
+    if (b == 0 || rhs_batched) {
+      ORC_PARALLEL_FOR(nt)
+      for (int64_t j = 0; j < cols; ++j)
+        for (int64_t k = 0; k < depth; ++k)
+          rp[j * depth + k] =
+              (int16_t)((int32_t)r[orc_idx(rhs_order, depth, cols, k, j)] + rhs_offset);
+    }
+    const int64_t JB = 64;
+    ORC_PARALLEL_FOR(nt)
+    for (int64_t i0 = 0; i0 < rows; i0 += 8) {
+      const int64_t i1 = i0 + 8 < rows ? i0 + 8 : rows;
+      for (int64_t j0 = 0; j0 < cols; j0 += JB) {
+        const int64_t j1 = j0 + JB < cols ? j0 + JB : cols;
+        for (int64_t i = i0; i < i1; ++i) {
+          const int16_t *a = lp + i * depth;
+          for (int64_t j = j0; j < j1; ++j) {
+            const int16_t *bb = rp + j * depth;
+            int32_t acc = 0;
+            for (int64_t k = 0; k < depth; ++k) acc += (int32_t)a[k] * (int32_t)bb[k];
+            o[orc_idx(out_order, rows, cols, i, j)] = acc;
+          }
+        }
+      }
+    }
+  }
+  free(lp);
+  free(rp);
+}
+
+/* mace/ops/common/gemmlowp_util.h:37-74: bias (one per result ROW) -> fixed-point
+ * quantize-down -> saturating cast. */
+void orc_output_pipeline_u8(const int32_t *acc, int64_t batch, int64_t rows, int64_t cols,
+                            int order, const int32_t *bias, int32_t mult, int right_shift,
+                            int32_t offset_after_shift, int clamp_min, int clamp_max,
+                            uint8_t *out) {
+  for (int64_t b = 0; b < batch; ++b)
+    for (int64_t i = 0; i < rows; ++i)
+      for (int64_t j = 0; j < cols; ++j) {
+        const int64_t at = b * rows * cols + orc_idx(order, rows, cols, i, j);
+        /* gemmlowp adds the bias in int32 (wrapping); unsigned add keeps C defined */
+        int32_t x = (int32_t)((uint32_t)acc[at] + (uint32_t)(bias ? bias[i] : 0));
+        out[at] = orc_requant_fixed_u8(x, mult, right_shift, offset_after_shift,
+                                       clamp_min, clamp_max);
+      }
+}
+
+void orc_q8_gemm_u8(const uint8_t *lhs, const uint8_t *rhs, int64_t batch, int64_t rows,
+                    int64_t cols, int64_t depth, int lhs_order, int rhs_order,
+                    int out_order, int lhs_batched, int rhs_batched, int32_t lhs_offset,
+                    int32_t rhs_offset, const int32_t *bias, int32_t mult,
+                    int right_shift, int32_t offset_after_shift, int clamp_min,
+                    int clamp_max, uint8_t *out, int nthreads) {
+  if (rows <= 0 || cols <= 0 || batch <= 0) return;
+  int32_t *acc = (int32_t *)malloc((size_t)batch * rows * cols * sizeof(int32_t));
+  orc_q8_gemm_i32(lhs, rhs, batch, rows, cols, depth, lhs_order, rhs_order, out_order,
+                  lhs_batched, rhs_batched, lhs_offset, rhs_offset, acc, nthreads);
+  orc_output_pipeline_u8(acc, batch, rows, cols, out_order, bias, mult, right_shift,
+                         offset_after_shift, clamp_min, clamp_max, out);
+  free(acc);
+}
+
+/* ------------------------------------------------------------------------------------
+ * Conv2D 1x1
+ * ---------------------------------------------------------------------------------- */
+
+/* mace/ops/conv_2d.cc:201-318 with filter 1x1, stride 1 (im2col_required == false):
+ * lhs = filter RowMajor [cout x cin], rhs = input ColMajor [cin x n*h*w],
+ * result ColMajor [cout x n*h*w]; lhs_offset = -filter_zp, rhs_offset = -input_zp;
+ * pipeline multiplier from (filter_scale, input_scale, out_scale) (:308-310); bias via
+ * GetBiasData (:271-275).  Returns 1 where the reference CHECK-fails. */
+int orc_conv1x1_q8_nhwc(const uint8_t *input, const uint8_t *filter, const int32_t *bias,
+                        int64_t n, int64_t h, int64_t w, int64_t cin, int64_t cout,
+                        float input_scale, int32_t input_zp, float filter_scale,
+                        int32_t filter_zp, float bias_scale, float out_scale,
+                        int32_t out_zp, int clamp_min, int clamp_max, uint8_t *out,
+                        int nthreads) {
+  int32_t mult;
+  int shift;
+  if (orc_get_output_multiplier_and_shift(filter_scale, input_scale, out_scale, &mult,
+                                          &shift))
+    return 1;
+  int32_t *b2 = (int32_t *)malloc((size_t)(cout > 0 ? cout : 1) * sizeof(int32_t));
+  orc_get_bias_data(bias, bias_scale, input_scale, filter_scale, cout, b2);
+  orc_q8_gemm_u8(filter, input, 1, cout, n * h * w, cin, ORC_ROW_MAJOR, ORC_COL_MAJOR,
+                 ORC_COL_MAJOR, 0, 0, -filter_zp, -input_zp, b2, mult, shift, out_zp,
+                 clamp_min, clamp_max, out, nthreads);
+  free(b2);
+  return 0;
+}
+
+void orc_conv1x1_q8_nhwc_direct_i32(const uint8_t *input, const uint8_t *filter,
+                                    int64_t n, int64_t h, int64_t w, int64_t cin,
+                                    int64_t cout, int32_t input_zp, int32_t filter_zp,
+                                    int32_t *out) {
+  for (int64_t p = 0; p < n * h * w; ++p)
+    for (int64_t co = 0; co < cout; ++co) {
+      int32_t acc = 0;
+      for (int64_t ci = 0; ci < cin; ++ci)
+        acc += ((int32_t)filter[co * cin + ci] - filter_zp) *
+               ((int32_t)input[p * cin + ci] - input_zp);
+      out[p * cout + co] = acc;
+    }
+}
+
+/* mace/ops/arm/base/conv_2d_1x1.cc:66-68 (Gemm with lhs = filter not batched, rhs = input
+ * batched, all RowMajor), then mace/ops/conv_2d.cc:171-173 (BiasAdd, Activation). */
+void orc_conv1x1_f32_nchw(const float *input, const float *filter, const float *bias,
+                          int64_t n, int64_t cin, int64_t hw, int64_t cout, int act,
+                          float limit, float *out, int nthreads) {
+  orc_gemm_f32(filter, input, n, cout, hw, cin, ORC_ROW_MAJOR, ORC_ROW_MAJOR,
+               ORC_ROW_MAJOR, 0, 1, out, nthreads);
+  if (bias) orc_bias_add_nchw_f32(out, bias, n, cout, hw);
+  orc_activation_f32(out, n * cout * hw, act, limit);
+}
