@@ -1,0 +1,224 @@
+/*
+ * mace_hip.h -- C ABI of libmace_hip.so: MACE's matrix-multiplication path on one MI355X.
+ *
+ * Every compute entry point replaces one CPU interface of the reference (cited per
+ * function, paths relative to the reference tree).  Plain pointers and sizes only; the
+ * library never frees caller memory, never aborts and never throws: contract violations
+ * that the reference handles with MACE_CHECK (fatal) come back as MACE_HIP_INVALID_ARGS.
+ *
+ * Status codes are MaceStatus::Code values (include/mace/public/mace.h:244-250).
+ *
+ * Pointers: the plain entry points take DEVICE pointers and are ordered on the context's
+ * stream (call mace_hip_sync before reading results on the host).  The *_host variants take
+ * HOST pointers, stage through a grow-only device arena owned by the context (the
+ * counterpart of the scratch the reference rents with RENT_SCRATCH,
+ * mace/ops/arm/base/gemm.cc:545-552) and return after the result is back in host memory.
+ *
+ * Threading: one context = one stream + one arena.  Calls on one context must be
+ * serialised by the caller, as MACE serialises ops on the engine thread
+ * (mace/core/net/serial_net.cc:103-124); different contexts are independent.
+ */
+#ifndef MACE_HIP_H_
+#define MACE_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct mace_hip_ctx mace_hip_ctx;
+
+/* include/mace/public/mace.h:244-250 */
+enum {
+  MACE_HIP_SUCCESS = 0,
+  MACE_HIP_INVALID_ARGS = 1,
+  MACE_HIP_OUT_OF_RESOURCES = 2,
+  MACE_HIP_UNSUPPORTED = 3,
+  MACE_HIP_RUNTIME_ERROR = 4
+};
+
+/* mace/ops/common/matrix.h:22-25 (MatrixMajor) == gemmlowp::MapOrder */
+enum { MACE_HIP_ROW_MAJOR = 0, MACE_HIP_COL_MAJOR = 1 };
+
+/* uint8 Gemv requantisation: mace/ops/ref/q8/gemv.cc:117-118 (REF, ignores the output
+ * zero point) and mace/ops/arm/q8/gemv.cc:159-161 (NEON, adds it). */
+enum { MACE_HIP_REQUANT_REF = 0, MACE_HIP_REQUANT_NEON = 1 };
+
+/* mace/ops/common/activation_type.h (subset applied by the fp32 1x1 convolution) */
+enum { MACE_HIP_ACT_NOOP = 0, MACE_HIP_ACT_RELU = 1, MACE_HIP_ACT_RELUX = 2 };
+
+/* ---- context ------------------------------------------------------------------------ */
+
+/* Replaces the per-engine CpuRuntime that owns the thread pool and gemmlowp context
+ * (mace/runtimes/cpu/cpu_runtime.cc:28-38,103-108). */
+int mace_hip_ctx_create(int device, mace_hip_ctx **out);
+int mace_hip_ctx_destroy(mace_hip_ctx *ctx);
+/* Borrow a caller-owned hipStream_t (NULL = back to the context's own stream). */
+int mace_hip_ctx_set_stream(mace_hip_ctx *ctx, void *hip_stream);
+int mace_hip_sync(mace_hip_ctx *ctx);
+/* Message of the last failing call on this context ("" if none); valid until the next call. */
+const char *mace_hip_last_error(const mace_hip_ctx *ctx);
+/* Names the device ("gfx950...") and reports CU count and LDS bytes per workgroup. */
+int mace_hip_device_info(mace_hip_ctx *ctx, char *arch, size_t arch_len, int *cu_count,
+                         int *lds_bytes);
+/* HIP-event stopwatch on the context's stream (kernel time, not host time). */
+int mace_hip_timer_start(mace_hip_ctx *ctx);
+int mace_hip_timer_stop(mace_hip_ctx *ctx, float *elapsed_ms);
+/* Test hook, the counterpart of MACE_RUNTIME_FAILURE_RATIO
+ * (mace/core/runtime_failure_mock.cc:24-48): the next n arena allocations fail. */
+int mace_hip_ctx_fail_next_allocs(mace_hip_ctx *ctx, int n);
+
+/* Device memory helpers for hosts that do not otherwise link a HIP runtime. */
+int mace_hip_malloc(mace_hip_ctx *ctx, size_t bytes, void **dev_ptr);
+int mace_hip_free(mace_hip_ctx *ctx, void *dev_ptr);
+int mace_hip_memcpy_h2d(mace_hip_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);
+int mace_hip_memcpy_d2h(mace_hip_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);
+
+/* ---- quantisation scalars (host) ------------------------------------------------------ */
+
+/* mace/core/quantize.h:104-114 QuantizeMultiplier */
+void mace_hip_quantize_multiplier(double multiplier, int32_t *quantized_multiplier,
+                                  int *exponent);
+/* mace/core/quantize.h:116-126 GetOutputMultiplierAndShift; INVALID_ARGS where the
+ * reference CHECK-fails (real multiplier outside (0,1), negative right shift). */
+int mace_hip_get_output_multiplier_and_shift(float lhs_scale, float rhs_scale,
+                                             float output_scale,
+                                             int32_t *quantized_multiplier,
+                                             int *right_shift);
+/* mace/core/quantize.h:80-83 Quantize<uint8_t>(value, scale, zero_point) */
+uint8_t mace_hip_quantize_u8(float value, float scale, int32_t zero_point);
+/* The device epilogue's arithmetic evaluated on the host, for CPU-side tests:
+ * gemmlowp quantize-down-by-fixed-point + saturating cast (see mace_hip_gemm_q8_u8). */
+uint8_t mace_hip_requant_fixed_u8(int32_t acc, int32_t multiplier, int right_shift,
+                                  int32_t offset_after_shift, int clamp_min, int clamp_max);
+/* The Gemv float requantisation evaluated on the host (see mace_hip_gemv_q8_u8). */
+uint8_t mace_hip_requant_float_u8(int32_t acc, float multiplier, int32_t out_zp, int mode);
+
+/* ---- fp32 ------------------------------------------------------------------------------ */
+
+/* delegator::Gemm::Compute, major form (mace/ops/delegator/gemm.h:42-54; semantics
+ * mace/ops/ref/gemm.cc:58-106): out[b] (rows x cols, out_major) =
+ * lhs[b or 0] (rows x depth, lhs_major) * rhs[b or 0] (depth x cols, rhs_major). */
+int mace_hip_gemm_f32(mace_hip_ctx *ctx, const float *lhs, const float *rhs, int64_t batch,
+                      int64_t rows, int64_t cols, int64_t depth, int lhs_major,
+                      int rhs_major, int out_major, int lhs_batched, int rhs_batched,
+                      float *out);
+/* delegator::Gemm::Compute, transpose form (mace/ops/delegator/gemm.h:56-69;
+ * mace/ops/ref/gemm.cc:108-146): INVALID_ARGS on inconsistent depth. */
+int mace_hip_gemm_f32_transpose(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
+                                int64_t batch, int64_t lhs_rows, int64_t lhs_cols,
+                                int64_t rhs_rows, int64_t rhs_cols, int transpose_lhs,
+                                int transpose_rhs, int transpose_out, int lhs_batched,
+                                int rhs_batched, float *out);
+/* delegator::Gemv::Compute for float (mace/ops/delegator/gemv.h:35-44;
+ * mace/ops/ref/gemv.cc:46-81): out[b,h] = bias[h] + sum_w lhs[b?,h,w] * rhs[b?,w]. */
+int mace_hip_gemv_f32(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
+                      const float *bias /* or NULL */, int64_t batch, int64_t height,
+                      int64_t width, int lhs_batched, int rhs_batched, float *out);
+/* arm::Conv2dK1x1<float>::Compute (mace/ops/arm/base/conv_2d_1x1.cc:27-72) followed by the
+ * BiasAdd and Activation delegators as Conv2dOp runs them (mace/ops/conv_2d.cc:171-173):
+ * input [n][cin][hw], filter [cout][cin], out [n][cout][hw]. */
+int mace_hip_conv1x1_f32_nchw(mace_hip_ctx *ctx, const float *input, const float *filter,
+                              const float *bias /* or NULL */, int64_t n, int64_t cin,
+                              int64_t hw, int64_t cout, int activation, float max_limit,
+                              float *out);
+
+/* ---- uint8 Gemv (FullyConnected) ------------------------------------------------------- */
+
+/* ref::q8::Gemv<uint8_t> (mace/ops/ref/q8/gemv.cc:80-122) / arm::q8::Gemv<uint8_t>
+ * (mace/ops/arm/q8/gemv.cc:36-171), selected by requant_mode.  INVALID_ARGS when
+ * out_scale <= 0 (both CHECK it) or, in NEON mode, when the multiplier is outside (0,1)
+ * (arm/q8/gemv.cc:55-63). */
+int mace_hip_gemv_q8_u8(mace_hip_ctx *ctx, const uint8_t *lhs, const uint8_t *rhs,
+                        const int32_t *bias /* or NULL */, int64_t batch, int64_t height,
+                        int64_t width, int lhs_batched, int rhs_batched, int32_t lhs_zp,
+                        int32_t rhs_zp, float lhs_scale, float rhs_scale, float out_scale,
+                        int32_t out_zp, int requant_mode, uint8_t *out);
+/* ref::q8::Gemv<int32_t> (mace/ops/ref/q8/gemv.cc:124-162) */
+int mace_hip_gemv_q8_i32(mace_hip_ctx *ctx, const uint8_t *lhs, const uint8_t *rhs,
+                         const int32_t *bias /* or NULL */, int64_t batch, int64_t height,
+                         int64_t width, int lhs_batched, int rhs_batched, int32_t lhs_zp,
+                         int32_t rhs_zp, int32_t *out);
+
+/* ---- uint8 GEMM (the gemmlowp call) ---------------------------------------------------- */
+
+/* gemmlowp::GemmWithOutputPipeline<uint8_t, int32_t, ...> with an empty pipeline, looped
+ * over the batch as at mace/ops/matmul.cc:366-386:
+ *   out[b][i,j] = sum_k (lhs[i,k] + lhs_offset) * (rhs[k,j] + rhs_offset). */
+int mace_hip_gemm_q8_i32(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order,
+                         const uint8_t *rhs, int rhs_order, int32_t *out, int out_order,
+                         int64_t batch, int64_t rows, int64_t depth, int64_t cols,
+                         int lhs_batched, int rhs_batched, int32_t lhs_offset,
+                         int32_t rhs_offset);
+/* gemmlowp::GemmWithOutputPipeline<uint8_t, uint8_t, ...> with the pipeline of
+ * mace/ops/common/gemmlowp_util.h:37-74 (call sites mace/ops/matmul.cc:280-300,
+ * mace/ops/conv_2d.cc:308-315): x = acc + bias[row]; y = SRDHM(x, multiplier);
+ * z = RoundingDivideByPOT(y, right_shift) + offset_after_shift; out = clamp(z).
+ * clamp_min/clamp_max (0/255 = the reference's saturating cast) fuse the quantised
+ * ReLU/ReLUx of mace/ops/arm/q8/activation.cc:59-94. */
+int mace_hip_gemm_q8_u8(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order,
+                        const uint8_t *rhs, int rhs_order, uint8_t *out, int out_order,
+                        int64_t batch, int64_t rows, int64_t depth, int64_t cols,
+                        int lhs_batched, int rhs_batched, int32_t lhs_offset,
+                        int32_t rhs_offset, const int32_t *bias /* [rows] or NULL */,
+                        int32_t multiplier, int right_shift, int32_t offset_after_shift,
+                        int clamp_min, int clamp_max);
+/* Conv2dOp<RT_CPU, uint8_t>::Run for a 1x1 filter, stride 1, dilation 1
+ * (mace/ops/conv_2d.cc:201-318 with im2col_required == false): input NHWC, filter OHWI
+ * [cout][cin], bias int32 [cout] or NULL with its own scale (rescaled as GetBiasData does,
+ * mace/ops/arm/q8/quantization_util.cc:20-46), output NHWC. */
+int mace_hip_conv1x1_q8_nhwc(mace_hip_ctx *ctx, const uint8_t *input, const uint8_t *filter,
+                             const int32_t *bias /* or NULL */, int64_t n, int64_t h,
+                             int64_t w, int64_t cin, int64_t cout, float input_scale,
+                             int32_t input_zp, float filter_scale, int32_t filter_zp,
+                             float bias_scale, float out_scale, int32_t out_zp,
+                             int clamp_min, int clamp_max, uint8_t *out);
+
+/* ---- host-pointer variants (same contracts; synchronous) -------------------------------- */
+int mace_hip_gemm_f32_host(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
+                           int64_t batch, int64_t rows, int64_t cols, int64_t depth,
+                           int lhs_major, int rhs_major, int out_major, int lhs_batched,
+                           int rhs_batched, float *out);
+int mace_hip_gemv_f32_host(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
+                           const float *bias, int64_t batch, int64_t height, int64_t width,
+                           int lhs_batched, int rhs_batched, float *out);
+int mace_hip_conv1x1_f32_nchw_host(mace_hip_ctx *ctx, const float *input,
+                                   const float *filter, const float *bias, int64_t n,
+                                   int64_t cin, int64_t hw, int64_t cout, int activation,
+                                   float max_limit, float *out);
+int mace_hip_gemv_q8_u8_host(mace_hip_ctx *ctx, const uint8_t *lhs, const uint8_t *rhs,
+                             const int32_t *bias, int64_t batch, int64_t height,
+                             int64_t width, int lhs_batched, int rhs_batched, int32_t lhs_zp,
+                             int32_t rhs_zp, float lhs_scale, float rhs_scale,
+                             float out_scale, int32_t out_zp, int requant_mode,
+                             uint8_t *out);
+int mace_hip_gemv_q8_i32_host(mace_hip_ctx *ctx, const uint8_t *lhs, const uint8_t *rhs,
+                              const int32_t *bias, int64_t batch, int64_t height,
+                              int64_t width, int lhs_batched, int rhs_batched,
+                              int32_t lhs_zp, int32_t rhs_zp, int32_t *out);
+int mace_hip_gemm_q8_i32_host(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order,
+                              const uint8_t *rhs, int rhs_order, int32_t *out,
+                              int out_order, int64_t batch, int64_t rows, int64_t depth,
+                              int64_t cols, int lhs_batched, int rhs_batched,
+                              int32_t lhs_offset, int32_t rhs_offset);
+int mace_hip_gemm_q8_u8_host(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order,
+                             const uint8_t *rhs, int rhs_order, uint8_t *out, int out_order,
+                             int64_t batch, int64_t rows, int64_t depth, int64_t cols,
+                             int lhs_batched, int rhs_batched, int32_t lhs_offset,
+                             int32_t rhs_offset, const int32_t *bias, int32_t multiplier,
+                             int right_shift, int32_t offset_after_shift, int clamp_min,
+                             int clamp_max);
+int mace_hip_conv1x1_q8_nhwc_host(mace_hip_ctx *ctx, const uint8_t *input,
+                                  const uint8_t *filter, const int32_t *bias, int64_t n,
+                                  int64_t h, int64_t w, int64_t cin, int64_t cout,
+                                  float input_scale, int32_t input_zp, float filter_scale,
+                                  int32_t filter_zp, float bias_scale, float out_scale,
+                                  int32_t out_zp, int clamp_min, int clamp_max,
+                                  uint8_t *out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif  /* MACE_HIP_H_ */

@@ -1,0 +1,148 @@
+// Internal definitions shared by the translation units of libmace_hip.so.
+#ifndef MACE_AMD_CSRC_COMMON_H_
+#define MACE_AMD_CSRC_COMMON_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "mace_hip.h"
+
+struct mace_hip_ctx {
+  int device = 0;
+  hipStream_t own_stream = nullptr;
+  hipStream_t stream = nullptr;     // own_stream or a borrowed one
+  hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+  // grow-only device arena; offsets handed out per call by ArenaScope
+  char *arena = nullptr;
+  size_t arena_bytes = 0;
+  size_t arena_used = 0;
+  int fail_allocs = 0;              // test hook
+  int cu_count = 0;
+  int lds_bytes = 0;
+  char arch[64] = {0};
+  char err[512] = {0};
+};
+
+int mh_fail(mace_hip_ctx *ctx, int code, const char *fmt, ...);
+
+#define MH_HIP(ctx, expr)                                                            \
+  do {                                                                               \
+    hipError_t e__ = (expr);                                                         \
+    if (e__ != hipSuccess)                                                           \
+      return mh_fail((ctx),                                                          \
+                     e__ == hipErrorOutOfMemory ? MACE_HIP_OUT_OF_RESOURCES          \
+                                                : MACE_HIP_RUNTIME_ERROR,            \
+                     "%s failed: %s", #expr, hipGetErrorString(e__));                \
+  } while (0)
+
+#define MH_CHECK(ctx, cond, ...)                                                     \
+  do {                                                                               \
+    if (!(cond)) return mh_fail((ctx), MACE_HIP_INVALID_ARGS, __VA_ARGS__);          \
+  } while (0)
+
+#define MH_RETURN_IF_ERROR(expr)                                                     \
+  do {                                                                               \
+    int s__ = (expr);                                                                \
+    if (s__ != MACE_HIP_SUCCESS) return s__;                                         \
+  } while (0)
+
+// Arena: every call that needs scratch opens a scope, takes aligned slices and lets the
+// scope rewind the arena on exit.  Growth reallocates (after a stream sync), so slices
+// must be taken before any kernel of the call is launched: mh_arena_reserve() first.
+int mh_arena_reserve(mace_hip_ctx *ctx, size_t bytes);
+void *mh_arena_take(mace_hip_ctx *ctx, size_t bytes);   // 256-byte aligned, after reserve
+inline size_t mh_align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+struct ArenaScope {
+  mace_hip_ctx *ctx;
+  size_t mark;
+  explicit ArenaScope(mace_hip_ctx *c) : ctx(c), mark(c->arena_used) {}
+  ~ArenaScope() { ctx->arena_used = mark; }
+};
+
+// ---- arithmetic shared by device epilogues and the host-side test exports ------------
+
+// gemmlowp SaturatingRoundingDoublingHighMul: floor(a*b / 2^31 + 1/2), except
+// INT32_MIN * INT32_MIN which saturates.  (ab + nudge) / 2^31 with truncating division and
+// nudge = ab >= 0 ? 2^30 : 1 - 2^30 equals the arithmetic shift below for every other input.
+__host__ __device__ inline int32_t mh_srdhm(int32_t a, int32_t b) {
+  if (a == INT32_MIN && b == INT32_MIN) return INT32_MAX;
+  const int64_t ab = (int64_t)a * (int64_t)b;
+  return (int32_t)((ab + ((int64_t)1 << 30)) >> 31);
+}
+
+// gemmlowp RoundingDivideByPOT: x / 2^e rounded to nearest, ties away from zero.
+__host__ __device__ inline int32_t mh_rdivpot(int32_t x, int e) {
+  const int32_t mask = (int32_t)(((uint32_t)1 << e) - 1u);
+  const int32_t rem = x & mask;
+  const int32_t thr = (mask >> 1) + (x < 0 ? 1 : 0);
+  return (x >> e) + (rem > thr ? 1 : 0);
+}
+
+__host__ __device__ inline int32_t mh_requant_fixed(int32_t acc, int32_t mult, int shift,
+                                                    int32_t zp, int lo, int hi) {
+  const int64_t z = (int64_t)mh_rdivpot(mh_srdhm(acc, mult), shift) + (int64_t)zp;
+  return (int32_t)(z < lo ? lo : (z > hi ? hi : z));
+}
+
+// roundf (ties away from zero) without relying on a library implementation: the
+// fractional part v - trunc(v) is exact in binary32.
+__host__ __device__ inline float mh_roundf(float v) {
+  const float t = truncf(v);
+  const float d = v - t;
+  if (d >= 0.5f) return t + 1.0f;
+  if (d <= -0.5f) return t - 1.0f;
+  return t;
+}
+
+// mace/core/quantize.h:68-78 Saturate<uint8_t>; clamps in the float domain first so that
+// out-of-int-range values (undefined in the reference) saturate instead.
+__host__ __device__ inline uint8_t mh_saturate_u8(float v) {
+  if (!(v > 0.0f)) return 0;
+  if (v >= 255.0f) return 255;
+  return (uint8_t)(int)v;
+}
+
+// Float requantisation of the q8 Gemv: Saturate(roundf(acc * m [+ zp])), no contraction.
+__host__ __device__ inline uint8_t mh_requant_float(int32_t acc, float m, int32_t zp,
+                                                    int neon_mode) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  float v = __fmul_rn((float)acc, m);
+  if (neon_mode) v = __fadd_rn(v, (float)zp);
+#else
+  volatile float prod = (float)acc * m;   // volatile: keep the product rounded to binary32
+  float v = prod;
+  if (neon_mode) {
+    volatile float s = v + (float)zp;
+    v = s;
+  }
+#endif
+  return mh_saturate_u8(mh_roundf(v));
+}
+
+// ---- internal launch entry points (defined next to their kernels) ----------------------
+
+struct Q8GemmEpilogue {
+  const int32_t *bias;      // per result row, or nullptr
+  int32_t mult;
+  int shift;
+  int32_t zp;
+  int lo, hi;
+};
+
+int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8_t *rhs,
+               int rhs_order, void *out, int out_order, bool out_u8, int64_t batch,
+               int64_t rows, int64_t depth, int64_t cols, int lhs_batched, int rhs_batched,
+               int32_t lhs_offset, int32_t rhs_offset, const Q8GemmEpilogue &ep);
+
+struct F32Epilogue {
+  const float *bias_row;    // added per result row (NCHW channel), or nullptr
+  int act;
+  float limit;
+};
+int mh_f32_gemm(mace_hip_ctx *ctx, const float *lhs, const float *rhs, int64_t batch,
+                int64_t rows, int64_t cols, int64_t depth, int lhs_major, int rhs_major,
+                int out_major, int lhs_batched, int rhs_batched, float *out,
+                const F32Epilogue &ep);
+
+#endif  // MACE_AMD_CSRC_COMMON_H_

@@ -1,0 +1,474 @@
+// Context, arena, timers, scalar host helpers and the host-pointer staging wrappers.
+#include <math.h>
+#include <stdarg.h>
+#include <string.h>
+
+#include <new>
+
+#include "common.h"
+
+int mh_fail(mace_hip_ctx *ctx, int code, const char *fmt, ...) {
+  if (ctx) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(ctx->err, sizeof(ctx->err), fmt, ap);
+    va_end(ap);
+  }
+  return code;
+}
+
+int mh_arena_reserve(mace_hip_ctx *ctx, size_t bytes) {
+  // headroom for the per-slice alignment
+  const size_t need = ctx->arena_used + bytes + 16 * 256;
+  if (need <= ctx->arena_bytes) return MACE_HIP_SUCCESS;
+  if (ctx->fail_allocs > 0) {
+    --ctx->fail_allocs;
+    return mh_fail(ctx, MACE_HIP_OUT_OF_RESOURCES, "arena allocation of %zu bytes failed (mock)",
+                   need);
+  }
+  if (ctx->arena_used != 0)
+    return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena grown while slices are live");
+  MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  if (ctx->arena) {
+    MH_HIP(ctx, hipFree(ctx->arena));
+    ctx->arena = nullptr;
+    ctx->arena_bytes = 0;
+  }
+  const size_t want = mh_align_up(need + need / 4, 1 << 20);
+  void *p = nullptr;
+  hipError_t e = hipMalloc(&p, want);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return mh_fail(ctx, MACE_HIP_OUT_OF_RESOURCES, "hipMalloc(%zu) failed: %s", want,
+                   hipGetErrorString(e));
+  }
+  ctx->arena = (char *)p;
+  ctx->arena_bytes = want;
+  return MACE_HIP_SUCCESS;
+}
+
+void *mh_arena_take(mace_hip_ctx *ctx, size_t bytes) {
+  const size_t at = mh_align_up(ctx->arena_used, 256);
+  if (at + bytes > ctx->arena_bytes) return nullptr;   // reserve() was too small: a bug
+  ctx->arena_used = at + bytes;
+  return ctx->arena + at;
+}
+
+extern "C" {
+
+int mace_hip_ctx_create(int device, mace_hip_ctx **out) {
+  if (!out) return MACE_HIP_INVALID_ARGS;
+  *out = nullptr;
+  int count = 0;
+  if (hipGetDeviceCount(&count) != hipSuccess || device < 0 || device >= count) {
+    (void)hipGetLastError();
+    return MACE_HIP_RUNTIME_ERROR;
+  }
+  mace_hip_ctx *ctx = new (std::nothrow) mace_hip_ctx();
+  if (!ctx) return MACE_HIP_OUT_OF_RESOURCES;
+  ctx->device = device;
+  hipDeviceProp_t prop;
+  if (hipSetDevice(device) != hipSuccess || hipGetDeviceProperties(&prop, device) != hipSuccess ||
+      hipStreamCreate(&ctx->own_stream) != hipSuccess ||
+      hipEventCreate(&ctx->ev_start) != hipSuccess ||
+      hipEventCreate(&ctx->ev_stop) != hipSuccess) {
+    (void)hipGetLastError();
+    delete ctx;
+    return MACE_HIP_RUNTIME_ERROR;
+  }
+  ctx->stream = ctx->own_stream;
+  ctx->cu_count = prop.multiProcessorCount;
+  ctx->lds_bytes = (int)prop.sharedMemPerBlock;
+  snprintf(ctx->arch, sizeof(ctx->arch), "%s", prop.gcnArchName);
+  if (strncmp(ctx->arch, "gfx950", 6) != 0) {
+    // the code objects in this library exist for gfx950 only
+    (void)hipStreamDestroy(ctx->own_stream);
+    (void)hipEventDestroy(ctx->ev_start);
+    (void)hipEventDestroy(ctx->ev_stop);
+    delete ctx;
+    return MACE_HIP_UNSUPPORTED;
+  }
+  *out = ctx;
+  return MACE_HIP_SUCCESS;
+}
+
+int mace_hip_ctx_destroy(mace_hip_ctx *ctx) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  (void)hipSetDevice(ctx->device);
+  (void)hipStreamSynchronize(ctx->stream);
+  if (ctx->arena) (void)hipFree(ctx->arena);
+  (void)hipEventDestroy(ctx->ev_start);
+  (void)hipEventDestroy(ctx->ev_stop);
+  (void)hipStreamDestroy(ctx->own_stream);
+  delete ctx;
+  return MACE_HIP_SUCCESS;
+}
+
+int mace_hip_ctx_set_stream(mace_hip_ctx *ctx, void *hip_stream) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  ctx->stream = hip_stream ? (hipStream_t)hip_stream : ctx->own_stream;
+  return MACE_HIP_SUCCESS;
+}
+
+int mace_hip_sync(mace_hip_ctx *ctx) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  return MACE_HIP_SUCCESS;
+}
+
+const char *mace_hip_last_error(const mace_hip_ctx *ctx) { return ctx ? ctx->err : ""; }
+
+int mace_hip_device_info(mace_hip_ctx *ctx, char *arch, size_t arch_len, int *cu_count,
+                         int *lds_bytes) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  if (arch && arch_len) snprintf(arch, arch_len, "%s", ctx->arch);
+  if (cu_count) *cu_count = ctx->cu_count;
+  if (lds_bytes) *lds_bytes = ctx->lds_bytes;
+  return MACE_HIP_SUCCESS;
+}
+
+int mace_hip_timer_start(mace_hip_ctx *ctx) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_HIP(ctx, hipEventRecord(ctx->ev_start, ctx->stream));
+  return MACE_HIP_SUCCESS;
+}
+
+int mace_hip_timer_stop(mace_hip_ctx *ctx, float *elapsed_ms) {
+  if (!ctx || !elapsed_ms) return MACE_HIP_INVALID_ARGS;
+  MH_HIP(ctx, hipEventRecord(ctx->ev_stop, ctx->stream));
+  MH_HIP(ctx, hipEventSynchronize(ctx->ev_stop));
+  MH_HIP(ctx, hipEventElapsedTime(elapsed_ms, ctx->ev_start, ctx->ev_stop));
+  return MACE_HIP_SUCCESS;
+}
+
+int mace_hip_ctx_fail_next_allocs(mace_hip_ctx *ctx, int n) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  ctx->fail_allocs = n;
+  return MACE_HIP_SUCCESS;
+}
+
+int mace_hip_malloc(mace_hip_ctx *ctx, size_t bytes, void **dev_ptr) {
+  if (!ctx || !dev_ptr) return MACE_HIP_INVALID_ARGS;
+  *dev_ptr = nullptr;
+  if (bytes == 0) return MACE_HIP_SUCCESS;
+  hipError_t e = hipMalloc(dev_ptr, bytes);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return mh_fail(ctx, MACE_HIP_OUT_OF_RESOURCES, "hipMalloc(%zu) failed: %s", bytes,
+                   hipGetErrorString(e));
+  }
+  return MACE_HIP_SUCCESS;
+}
+
+int mace_hip_free(mace_hip_ctx *ctx, void *dev_ptr) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  if (!dev_ptr) return MACE_HIP_SUCCESS;
+  MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  MH_HIP(ctx, hipFree(dev_ptr));
+  return MACE_HIP_SUCCESS;
+}
+
+int mace_hip_memcpy_h2d(mace_hip_ctx *ctx, void *dst, const void *src, size_t bytes) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  if (bytes == 0) return MACE_HIP_SUCCESS;
+  MH_HIP(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+  MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  return MACE_HIP_SUCCESS;
+}
+
+int mace_hip_memcpy_d2h(mace_hip_ctx *ctx, void *dst, const void *src, size_t bytes) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  if (bytes == 0) return MACE_HIP_SUCCESS;
+  MH_HIP(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+  MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  return MACE_HIP_SUCCESS;
+}
+
+// ---- quantisation scalars -----------------------------------------------------------------
+
+void mace_hip_quantize_multiplier(double multiplier, int32_t *quantized_multiplier,
+                                  int *exponent) {
+  int e = 0;
+  const double q = frexp(multiplier, &e);
+  int64_t qint = (int64_t)roundl((long double)(q * (double)(1ll << 31)));
+  if (qint == (1ll << 31)) {
+    qint /= 2;
+    ++e;
+  }
+  *quantized_multiplier = (int32_t)qint;
+  *exponent = e;
+}
+
+int mace_hip_get_output_multiplier_and_shift(float lhs_scale, float rhs_scale,
+                                             float output_scale,
+                                             int32_t *quantized_multiplier,
+                                             int *right_shift) {
+  volatile float prod = lhs_scale * rhs_scale;      // binary32, left to right
+  volatile float real = prod / output_scale;
+  const float r = real;
+  if (!(r > 0.f && r < 1.f)) return MACE_HIP_INVALID_ARGS;
+  int e = 0;
+  mace_hip_quantize_multiplier((double)r, quantized_multiplier, &e);
+  *right_shift = -e;
+  return *right_shift >= 0 ? MACE_HIP_SUCCESS : MACE_HIP_INVALID_ARGS;
+}
+
+uint8_t mace_hip_quantize_u8(float value, float scale, int32_t zero_point) {
+  volatile float q = value / scale;
+  volatile float s = q + (float)zero_point;
+  return mh_saturate_u8(mh_roundf(s));
+}
+
+uint8_t mace_hip_requant_fixed_u8(int32_t acc, int32_t multiplier, int right_shift,
+                                  int32_t offset_after_shift, int clamp_min, int clamp_max) {
+  return (uint8_t)mh_requant_fixed(acc, multiplier, right_shift, offset_after_shift,
+                                   clamp_min, clamp_max);
+}
+
+uint8_t mace_hip_requant_float_u8(int32_t acc, float multiplier, int32_t out_zp, int mode) {
+  return mh_requant_float(acc, multiplier, out_zp, mode == MACE_HIP_REQUANT_NEON);
+}
+
+// ---- host-pointer staging --------------------------------------------------------------------
+
+namespace {
+
+struct Stage {
+  mace_hip_ctx *ctx;
+  ArenaScope scope;
+  explicit Stage(mace_hip_ctx *c) : ctx(c), scope(c) {}
+  // returns nullptr for a null/empty host pointer
+  int in(const void *host, size_t bytes, void **dev) {
+    *dev = nullptr;
+    if (!host || bytes == 0) return MACE_HIP_SUCCESS;
+    *dev = mh_arena_take(ctx, bytes);
+    if (!*dev) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
+    MH_HIP(ctx, hipMemcpyAsync(*dev, host, bytes, hipMemcpyHostToDevice, ctx->stream));
+    return MACE_HIP_SUCCESS;
+  }
+  int out(size_t bytes, void **dev) {
+    *dev = mh_arena_take(ctx, bytes ? bytes : 1);
+    if (!*dev) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
+    return MACE_HIP_SUCCESS;
+  }
+  int back(void *host, const void *dev, size_t bytes) {
+    if (bytes) MH_HIP(ctx, hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return MACE_HIP_SUCCESS;
+  }
+};
+
+inline bool nonneg(int64_t a, int64_t b, int64_t c, int64_t d) {
+  return a >= 0 && b >= 0 && c >= 0 && d >= 0;
+}
+
+// scratch the device-pointer call itself takes from the arena (generous upper bounds:
+// packed copies of both operands plus the correction vectors)
+inline size_t q8_gemm_scratch(int64_t batch, int64_t rows, int64_t depth, int64_t cols) {
+  const size_t kp = mh_align_up((size_t)depth, 64) + 64;
+  return (size_t)batch * ((size_t)rows + (size_t)cols) * (kp + 8) + (1 << 16);
+}
+
+}  // namespace
+
+int mace_hip_gemm_f32_host(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
+                           int64_t batch, int64_t rows, int64_t cols, int64_t depth,
+                           int lhs_major, int rhs_major, int out_major, int lhs_batched,
+                           int rhs_batched, float *out) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_CHECK(ctx, nonneg(batch, rows, cols, depth), "negative dimension");
+  const size_t lb = sizeof(float) * (lhs_batched ? batch : 1) * rows * depth;
+  const size_t rb = sizeof(float) * (rhs_batched ? batch : 1) * depth * cols;
+  const size_t ob = sizeof(float) * batch * rows * cols;
+  MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, lb + rb + ob));
+  Stage st(ctx);
+  void *dl, *dr, *dout;
+  MH_RETURN_IF_ERROR(st.in(lhs, lb, &dl));
+  MH_RETURN_IF_ERROR(st.in(rhs, rb, &dr));
+  MH_RETURN_IF_ERROR(st.out(ob, &dout));
+  MH_RETURN_IF_ERROR(mace_hip_gemm_f32(ctx, (const float *)dl, (const float *)dr, batch, rows,
+                                       cols, depth, lhs_major, rhs_major, out_major,
+                                       lhs_batched, rhs_batched, (float *)dout));
+  return st.back(out, dout, ob);
+}
+
+int mace_hip_gemv_f32_host(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
+                           const float *bias, int64_t batch, int64_t height, int64_t width,
+                           int lhs_batched, int rhs_batched, float *out) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_CHECK(ctx, nonneg(batch, height, width, 0), "negative dimension");
+  const size_t lb = sizeof(float) * (lhs_batched ? batch : 1) * height * width;
+  const size_t rb = sizeof(float) * (rhs_batched ? batch : 1) * width;
+  const size_t bb = bias ? sizeof(float) * height : 0;
+  const size_t ob = sizeof(float) * batch * height;
+  MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, lb + rb + bb + ob));
+  Stage st(ctx);
+  void *dl, *dr, *db, *dout;
+  MH_RETURN_IF_ERROR(st.in(lhs, lb, &dl));
+  MH_RETURN_IF_ERROR(st.in(rhs, rb, &dr));
+  MH_RETURN_IF_ERROR(st.in(bias, bb, &db));
+  MH_RETURN_IF_ERROR(st.out(ob, &dout));
+  MH_RETURN_IF_ERROR(mace_hip_gemv_f32(ctx, (const float *)dl, (const float *)dr,
+                                       (const float *)db, batch, height, width, lhs_batched,
+                                       rhs_batched, (float *)dout));
+  return st.back(out, dout, ob);
+}
+
+int mace_hip_conv1x1_f32_nchw_host(mace_hip_ctx *ctx, const float *input,
+                                   const float *filter, const float *bias, int64_t n,
+                                   int64_t cin, int64_t hw, int64_t cout, int activation,
+                                   float max_limit, float *out) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_CHECK(ctx, nonneg(n, cin, hw, cout), "negative dimension");
+  const size_t ib = sizeof(float) * n * cin * hw;
+  const size_t fb = sizeof(float) * cout * cin;
+  const size_t bb = bias ? sizeof(float) * cout : 0;
+  const size_t ob = sizeof(float) * n * cout * hw;
+  MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, ib + fb + bb + ob));
+  Stage st(ctx);
+  void *di, *df, *db, *dout;
+  MH_RETURN_IF_ERROR(st.in(input, ib, &di));
+  MH_RETURN_IF_ERROR(st.in(filter, fb, &df));
+  MH_RETURN_IF_ERROR(st.in(bias, bb, &db));
+  MH_RETURN_IF_ERROR(st.out(ob, &dout));
+  MH_RETURN_IF_ERROR(mace_hip_conv1x1_f32_nchw(ctx, (const float *)di, (const float *)df,
+                                               (const float *)db, n, cin, hw, cout,
+                                               activation, max_limit, (float *)dout));
+  return st.back(out, dout, ob);
+}
+
+int mace_hip_gemv_q8_u8_host(mace_hip_ctx *ctx, const uint8_t *lhs, const uint8_t *rhs,
+                             const int32_t *bias, int64_t batch, int64_t height,
+                             int64_t width, int lhs_batched, int rhs_batched, int32_t lhs_zp,
+                             int32_t rhs_zp, float lhs_scale, float rhs_scale,
+                             float out_scale, int32_t out_zp, int requant_mode,
+                             uint8_t *out) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_CHECK(ctx, nonneg(batch, height, width, 0), "negative dimension");
+  const size_t lb = (size_t)(lhs_batched ? batch : 1) * height * width;
+  const size_t rb = (size_t)(rhs_batched ? batch : 1) * width;
+  const size_t bb = bias ? sizeof(int32_t) * height : 0;
+  const size_t ob = (size_t)batch * height;
+  MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, lb + rb + bb + ob));
+  Stage st(ctx);
+  void *dl, *dr, *db, *dout;
+  MH_RETURN_IF_ERROR(st.in(lhs, lb, &dl));
+  MH_RETURN_IF_ERROR(st.in(rhs, rb, &dr));
+  MH_RETURN_IF_ERROR(st.in(bias, bb, &db));
+  MH_RETURN_IF_ERROR(st.out(ob, &dout));
+  MH_RETURN_IF_ERROR(mace_hip_gemv_q8_u8(ctx, (const uint8_t *)dl, (const uint8_t *)dr,
+                                         (const int32_t *)db, batch, height, width,
+                                         lhs_batched, rhs_batched, lhs_zp, rhs_zp, lhs_scale,
+                                         rhs_scale, out_scale, out_zp, requant_mode,
+                                         (uint8_t *)dout));
+  return st.back(out, dout, ob);
+}
+
+int mace_hip_gemv_q8_i32_host(mace_hip_ctx *ctx, const uint8_t *lhs, const uint8_t *rhs,
+                              const int32_t *bias, int64_t batch, int64_t height,
+                              int64_t width, int lhs_batched, int rhs_batched,
+                              int32_t lhs_zp, int32_t rhs_zp, int32_t *out) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_CHECK(ctx, nonneg(batch, height, width, 0), "negative dimension");
+  const size_t lb = (size_t)(lhs_batched ? batch : 1) * height * width;
+  const size_t rb = (size_t)(rhs_batched ? batch : 1) * width;
+  const size_t bb = bias ? sizeof(int32_t) * height : 0;
+  const size_t ob = sizeof(int32_t) * batch * height;
+  MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, lb + rb + bb + ob));
+  Stage st(ctx);
+  void *dl, *dr, *db, *dout;
+  MH_RETURN_IF_ERROR(st.in(lhs, lb, &dl));
+  MH_RETURN_IF_ERROR(st.in(rhs, rb, &dr));
+  MH_RETURN_IF_ERROR(st.in(bias, bb, &db));
+  MH_RETURN_IF_ERROR(st.out(ob, &dout));
+  MH_RETURN_IF_ERROR(mace_hip_gemv_q8_i32(ctx, (const uint8_t *)dl, (const uint8_t *)dr,
+                                          (const int32_t *)db, batch, height, width,
+                                          lhs_batched, rhs_batched, lhs_zp, rhs_zp,
+                                          (int32_t *)dout));
+  return st.back(out, dout, ob);
+}
+
+int mace_hip_gemm_q8_i32_host(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order,
+                              const uint8_t *rhs, int rhs_order, int32_t *out,
+                              int out_order, int64_t batch, int64_t rows, int64_t depth,
+                              int64_t cols, int lhs_batched, int rhs_batched,
+                              int32_t lhs_offset, int32_t rhs_offset) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_CHECK(ctx, nonneg(batch, rows, depth, cols), "negative dimension");
+  const size_t lb = (size_t)(lhs_batched ? batch : 1) * rows * depth;
+  const size_t rb = (size_t)(rhs_batched ? batch : 1) * depth * cols;
+  const size_t ob = sizeof(int32_t) * batch * rows * cols;
+  MH_RETURN_IF_ERROR(
+      mh_arena_reserve(ctx, lb + rb + ob + q8_gemm_scratch(batch, rows, depth, cols)));
+  Stage st(ctx);
+  void *dl, *dr, *dout;
+  MH_RETURN_IF_ERROR(st.in(lhs, lb, &dl));
+  MH_RETURN_IF_ERROR(st.in(rhs, rb, &dr));
+  MH_RETURN_IF_ERROR(st.out(ob, &dout));
+  MH_RETURN_IF_ERROR(mace_hip_gemm_q8_i32(ctx, (const uint8_t *)dl, lhs_order,
+                                          (const uint8_t *)dr, rhs_order, (int32_t *)dout,
+                                          out_order, batch, rows, depth, cols, lhs_batched,
+                                          rhs_batched, lhs_offset, rhs_offset));
+  return st.back(out, dout, ob);
+}
+
+int mace_hip_gemm_q8_u8_host(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order,
+                             const uint8_t *rhs, int rhs_order, uint8_t *out, int out_order,
+                             int64_t batch, int64_t rows, int64_t depth, int64_t cols,
+                             int lhs_batched, int rhs_batched, int32_t lhs_offset,
+                             int32_t rhs_offset, const int32_t *bias, int32_t multiplier,
+                             int right_shift, int32_t offset_after_shift, int clamp_min,
+                             int clamp_max) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_CHECK(ctx, nonneg(batch, rows, depth, cols), "negative dimension");
+  const size_t lb = (size_t)(lhs_batched ? batch : 1) * rows * depth;
+  const size_t rb = (size_t)(rhs_batched ? batch : 1) * depth * cols;
+  const size_t bb = bias ? sizeof(int32_t) * rows : 0;
+  const size_t ob = (size_t)batch * rows * cols;
+  MH_RETURN_IF_ERROR(
+      mh_arena_reserve(ctx, lb + rb + bb + ob + q8_gemm_scratch(batch, rows, depth, cols)));
+  Stage st(ctx);
+  void *dl, *dr, *db, *dout;
+  MH_RETURN_IF_ERROR(st.in(lhs, lb, &dl));
+  MH_RETURN_IF_ERROR(st.in(rhs, rb, &dr));
+  MH_RETURN_IF_ERROR(st.in(bias, bb, &db));
+  MH_RETURN_IF_ERROR(st.out(ob, &dout));
+  MH_RETURN_IF_ERROR(mace_hip_gemm_q8_u8(ctx, (const uint8_t *)dl, lhs_order,
+                                         (const uint8_t *)dr, rhs_order, (uint8_t *)dout,
+                                         out_order, batch, rows, depth, cols, lhs_batched,
+                                         rhs_batched, lhs_offset, rhs_offset,
+                                         (const int32_t *)db, multiplier, right_shift,
+                                         offset_after_shift, clamp_min, clamp_max));
+  return st.back(out, dout, ob);
+}
+
+int mace_hip_conv1x1_q8_nhwc_host(mace_hip_ctx *ctx, const uint8_t *input,
+                                  const uint8_t *filter, const int32_t *bias, int64_t n,
+                                  int64_t h, int64_t w, int64_t cin, int64_t cout,
+                                  float input_scale, int32_t input_zp, float filter_scale,
+                                  int32_t filter_zp, float bias_scale, float out_scale,
+                                  int32_t out_zp, int clamp_min, int clamp_max,
+                                  uint8_t *out) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_CHECK(ctx, nonneg(n, h, w, 0) && nonneg(cin, cout, 0, 0), "negative dimension");
+  const int64_t pix = n * h * w;
+  const size_t ib = (size_t)pix * cin, fb = (size_t)cout * cin;
+  const size_t bb = bias ? sizeof(int32_t) * cout : 0;
+  const size_t ob = (size_t)pix * cout;
+  MH_RETURN_IF_ERROR(mh_arena_reserve(
+      ctx, ib + fb + bb + ob + q8_gemm_scratch(1, cout, cin, pix) + sizeof(int32_t) * cout));
+  Stage st(ctx);
+  void *di, *df, *db, *dout;
+  MH_RETURN_IF_ERROR(st.in(input, ib, &di));
+  MH_RETURN_IF_ERROR(st.in(filter, fb, &df));
+  MH_RETURN_IF_ERROR(st.in(bias, bb, &db));
+  MH_RETURN_IF_ERROR(st.out(ob, &dout));
+  MH_RETURN_IF_ERROR(mace_hip_conv1x1_q8_nhwc(
+      ctx, (const uint8_t *)di, (const uint8_t *)df, (const int32_t *)db, n, h, w, cin, cout,
+      input_scale, input_zp, filter_scale, filter_zp, bias_scale, out_scale, out_zp,
+      clamp_min, clamp_max, (uint8_t *)dout));
+  return st.back(out, dout, ob);
+}
+
+}  // extern "C"

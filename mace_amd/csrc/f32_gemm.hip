@@ -1,0 +1,291 @@
+// fp32 Gemm / Gemv on CDNA4.
+//
+// Gemm replaces delegator::Gemm for float (contract mace/ops/delegator/gemm.h:42-69,
+// semantics mace/ops/ref/gemm.cc:58-146; the NEON implementation it stands in for is
+// mace/ops/arm/base/gemm.cc:520-683): out[b] = lhs[b or 0] * rhs[b or 0] with each of the
+// three matrices RowMajor or ColMajor.  The NEON kernel packs both operands into cache
+// panels; here the panels are LDS tiles ([k][m] and [k][n], so a wavefront's fragment read
+// is one conflict-free row segment) feeding v_mfma_f32_32x32x2_f32.  Products and sums are
+// binary32; the summation order differs from the reference's serial k loop, which the
+// reference's own tolerance (1e-4 relative + 1e-2 absolute) covers.
+//
+// Gemv replaces delegator::Gemv for float (mace/ops/delegator/gemv.h:35-44,
+// mace/ops/ref/gemv.cc:46-81): one wavefront per output row, lane-strided loads.
+#include "common.h"
+
+namespace {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int TM = 128, TN = 128, TK = 16;
+constexpr int LDT = TM + 4;   // padded LDS row (floats)
+
+struct F32GemmParams {
+  const float *lhs, *rhs;
+  float *out;
+  int64_t lrs, lcs;   // lhs element strides for (row, depth)
+  int64_t rrs, rcs;   // rhs element strides for (depth, col)
+  int64_t ors, ocs;   // out element strides for (row, col)
+  int64_t lbs, rbs, obs;
+  int M, N, K;
+  const float *bias_row;
+  int act;
+  float limit;
+  int tiles_m;
+};
+
+__device__ inline float apply_act(float v, int act, float limit) {
+  // mace/ops/ref/activation.cc:61-75
+  if (act == MACE_HIP_ACT_RELU) return fmaxf(0.f, v);
+  if (act == MACE_HIP_ACT_RELUX) return fmaxf(0.f, fminf(limit, v));
+  return v;
+}
+
+// LK / RK: the operand is contiguous along depth (true) or along its outer index (false);
+// it only selects which thread reads which element so that global loads coalesce.
+template <bool LK, bool RK>
+__global__ __launch_bounds__(256) void f32_gemm_kernel(F32GemmParams p) {
+  __shared__ float sA[2][TK][LDT];
+  __shared__ float sB[2][TK][LDT];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave & 1, wn = wave >> 1;
+  const int m0 = (blockIdx.x % p.tiles_m) * TM, n0 = (blockIdx.x / p.tiles_m) * TN;
+  const int b = blockIdx.z;
+  const float *A = p.lhs + (int64_t)b * p.lbs;
+  const float *B = p.rhs + (int64_t)b * p.rbs;
+
+  constexpr int PER = TM * TK / 256;   // elements per thread per operand tile
+  float ra[PER], rb[PER];
+  int am[PER], ak[PER], bn[PER], bk[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int e = tid + i * 256;
+    if (LK) { ak[i] = e % TK; am[i] = e / TK; } else { am[i] = e % TM; ak[i] = e / TM; }
+    if (RK) { bk[i] = e % TK; bn[i] = e / TK; } else { bn[i] = e % TN; bk[i] = e / TN; }
+  }
+  auto load_global = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int m = m0 + am[i], k = k0 + ak[i];
+      ra[i] = (m < p.M && k < p.K) ? A[(int64_t)m * p.lrs + (int64_t)k * p.lcs] : 0.f;
+      const int n = n0 + bn[i], k2 = k0 + bk[i];
+      rb[i] = (n < p.N && k2 < p.K) ? B[(int64_t)k2 * p.rrs + (int64_t)n * p.rcs] : 0.f;
+    }
+  };
+  auto store_lds = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      sA[buf][ak[i]][am[i]] = ra[i];
+      sB[buf][bk[i]][bn[i]] = rb[i];
+    }
+  };
+
+  v16f acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int nk = (p.K + TK - 1) / TK;
+  load_global(0);
+  store_lds(0);
+  __syncthreads();
+  for (int kt = 0; kt < nk; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < nk) load_global((kt + 1) * TK);
+#pragma unroll
+    for (int ks = 0; ks < TK / 2; ++ks) {
+      // v_mfma_f32_32x32x2: lane l supplies A[row l % 32][k = l / 32], B[k = l / 32][col l % 32]
+      const int kk = ks * 2 + (lane >> 5);
+      float a[2], bb[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) a[i] = sA[buf][kk][wm * 64 + i * 32 + (lane & 31)];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) bb[j] = sB[buf][kk][wn * 64 + j * 32 + (lane & 31)];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], bb[j], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < nk) store_lds(buf ^ 1);
+    __syncthreads();
+  }
+
+  float *O = p.out + (int64_t)b * p.obs;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int n = n0 + wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (m < p.M && n < p.N) {
+          float v = acc[i][j][r];
+          if (p.bias_row) v = v + p.bias_row[m];
+          v = apply_act(v, p.act, p.limit);
+          O[(int64_t)m * p.ors + (int64_t)n * p.ocs] = v;
+        }
+      }
+    }
+}
+
+// depth == 0: the reference's loop leaves sum = 0
+__global__ void f32_fill_kernel(F32GemmParams p, int64_t total) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t bm = i / p.N;
+    const int m = (int)(bm % p.M);
+    float v = 0.f;
+    if (p.bias_row) v = v + p.bias_row[m];
+    const int64_t bb = bm / p.M;
+    const int n = (int)(i - bm * p.N);
+    p.out[bb * p.obs + (int64_t)m * p.ors + (int64_t)n * p.ocs] = apply_act(v, p.act, p.limit);
+  }
+}
+
+struct F32GemvParams {
+  const float *lhs, *rhs, *bias;
+  float *out;
+  int64_t lbs, rbs;
+  int H, W;
+};
+
+__global__ __launch_bounds__(256) void f32_gemv_kernel(F32GemvParams p) {
+  const int lane = threadIdx.x & 63;
+  const int h = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (h >= p.H) return;
+  const int b = blockIdx.y;
+  const float *l = p.lhs + (int64_t)b * p.lbs + (int64_t)h * p.W;
+  const float *r = p.rhs + (int64_t)b * p.rbs;
+  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  int w = lane;
+  for (; w + 192 < p.W; w += 256) {
+    s0 += l[w] * r[w];
+    s1 += l[w + 64] * r[w + 64];
+    s2 += l[w + 128] * r[w + 128];
+    s3 += l[w + 192] * r[w + 192];
+  }
+  for (; w < p.W; w += 64) s0 += l[w] * r[w];
+  float s = (s0 + s1) + (s2 + s3);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+  if (lane == 0) p.out[(int64_t)b * p.H + h] = (p.bias ? p.bias[h] : 0.f) + s;
+}
+
+}  // namespace
+
+int mh_f32_gemm(mace_hip_ctx *ctx, const float *lhs, const float *rhs, int64_t batch,
+                int64_t rows, int64_t cols, int64_t depth, int lhs_major, int rhs_major,
+                int out_major, int lhs_batched, int rhs_batched, float *out,
+                const F32Epilogue &ep) {
+  MH_CHECK(ctx, batch >= 0 && rows >= 0 && cols >= 0 && depth >= 0, "negative dimension");
+  MH_CHECK(ctx, (lhs_major | 1) == 1 && (rhs_major | 1) == 1 && (out_major | 1) == 1,
+           "matrix major must be RowMajor (0) or ColMajor (1)");
+  MH_CHECK(ctx, rows < (1ll << 31) && cols < (1ll << 31) && depth < (1ll << 31) && batch < 65536,
+           "dimension too large");
+  if (batch == 0 || rows == 0 || cols == 0) return MACE_HIP_SUCCESS;
+  MH_CHECK(ctx, out && (depth == 0 || (lhs && rhs)), "null operand");
+  F32GemmParams p{};
+  p.lhs = lhs; p.rhs = rhs; p.out = out;
+  // mace/ops/common/matrix.h:48-80: stride = cols (RowMajor) or rows (ColMajor)
+  p.lrs = lhs_major == MACE_HIP_ROW_MAJOR ? depth : 1;
+  p.lcs = lhs_major == MACE_HIP_ROW_MAJOR ? 1 : rows;
+  p.rrs = rhs_major == MACE_HIP_ROW_MAJOR ? cols : 1;
+  p.rcs = rhs_major == MACE_HIP_ROW_MAJOR ? 1 : depth;
+  p.ors = out_major == MACE_HIP_ROW_MAJOR ? cols : 1;
+  p.ocs = out_major == MACE_HIP_ROW_MAJOR ? 1 : rows;
+  p.lbs = lhs_batched ? rows * depth : 0;
+  p.rbs = rhs_batched ? depth * cols : 0;
+  p.obs = rows * cols;
+  p.M = (int)rows; p.N = (int)cols; p.K = (int)depth;
+  p.bias_row = ep.bias_row; p.act = ep.act; p.limit = ep.limit;
+  if (depth == 0) {
+    const int64_t total = batch * rows * cols;
+    hipLaunchKernelGGL(f32_fill_kernel, dim3((unsigned)((total + 255) / 256 > 65535 ? 65535 : (total + 255) / 256)),
+                       dim3(256), 0, ctx->stream, p, total);
+    MH_HIP(ctx, hipGetLastError());
+    return MACE_HIP_SUCCESS;
+  }
+  p.tiles_m = (p.M + TM - 1) / TM;
+  const int64_t tiles = (int64_t)p.tiles_m * ((p.N + TN - 1) / TN);
+  MH_CHECK(ctx, tiles < (1ll << 31), "too many tiles");
+  dim3 grid((unsigned)tiles, 1, (unsigned)batch), block(256);
+  const bool lk = lhs_major == MACE_HIP_ROW_MAJOR;   // depth contiguous
+  const bool rk = rhs_major == MACE_HIP_COL_MAJOR;
+  if (lk && rk) hipLaunchKernelGGL((f32_gemm_kernel<true, true>), grid, block, 0, ctx->stream, p);
+  else if (lk) hipLaunchKernelGGL((f32_gemm_kernel<true, false>), grid, block, 0, ctx->stream, p);
+  else if (rk) hipLaunchKernelGGL((f32_gemm_kernel<false, true>), grid, block, 0, ctx->stream, p);
+  else hipLaunchKernelGGL((f32_gemm_kernel<false, false>), grid, block, 0, ctx->stream, p);
+  MH_HIP(ctx, hipGetLastError());
+  return MACE_HIP_SUCCESS;
+}
+
+extern "C" {
+
+int mace_hip_gemm_f32(mace_hip_ctx *ctx, const float *lhs, const float *rhs, int64_t batch,
+                      int64_t rows, int64_t cols, int64_t depth, int lhs_major,
+                      int rhs_major, int out_major, int lhs_batched, int rhs_batched,
+                      float *out) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  F32Epilogue ep{nullptr, MACE_HIP_ACT_NOOP, 0.f};
+  return mh_f32_gemm(ctx, lhs, rhs, batch, rows, cols, depth, lhs_major, rhs_major, out_major,
+                     lhs_batched, rhs_batched, out, ep);
+}
+
+int mace_hip_gemm_f32_transpose(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
+                                int64_t batch, int64_t lhs_rows, int64_t lhs_cols,
+                                int64_t rhs_rows, int64_t rhs_cols, int transpose_lhs,
+                                int transpose_rhs, int transpose_out, int lhs_batched,
+                                int rhs_batched, float *out) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  // mace/ops/ref/gemm.cc:122-131
+  const int64_t rows = transpose_lhs ? lhs_cols : lhs_rows;
+  const int64_t depth = transpose_lhs ? lhs_rows : lhs_cols;
+  const int64_t cols = transpose_rhs ? rhs_rows : rhs_cols;
+  const int64_t depth2 = transpose_rhs ? rhs_cols : rhs_rows;
+  MH_CHECK(ctx, depth == depth2,
+           "Matrices that multiply have inconsistent depth dim: %lld vs. %lld",
+           (long long)depth, (long long)depth2);
+  return mace_hip_gemm_f32(ctx, lhs, rhs, batch, rows, cols, depth,
+                           transpose_lhs ? MACE_HIP_COL_MAJOR : MACE_HIP_ROW_MAJOR,
+                           transpose_rhs ? MACE_HIP_COL_MAJOR : MACE_HIP_ROW_MAJOR,
+                           transpose_out ? MACE_HIP_COL_MAJOR : MACE_HIP_ROW_MAJOR,
+                           lhs_batched, rhs_batched, out);
+}
+
+int mace_hip_gemv_f32(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
+                      const float *bias, int64_t batch, int64_t height, int64_t width,
+                      int lhs_batched, int rhs_batched, float *out) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_CHECK(ctx, batch >= 0 && height >= 0 && width >= 0, "negative dimension");
+  MH_CHECK(ctx, height < (1ll << 31) && width < (1ll << 31) && batch <= 65535,
+           "dimension too large");
+  if (batch == 0 || height == 0) return MACE_HIP_SUCCESS;
+  MH_CHECK(ctx, out && (width == 0 || (lhs && rhs)), "null operand");
+  F32GemvParams p{lhs, rhs, bias, out, lhs_batched ? height * width : 0,
+                  rhs_batched ? width : 0, (int)height, (int)width};
+  dim3 grid((unsigned)((height + 3) / 4), (unsigned)batch);
+  hipLaunchKernelGGL(f32_gemv_kernel, grid, dim3(256), 0, ctx->stream, p);
+  MH_HIP(ctx, hipGetLastError());
+  return MACE_HIP_SUCCESS;
+}
+
+int mace_hip_conv1x1_f32_nchw(mace_hip_ctx *ctx, const float *input, const float *filter,
+                              const float *bias, int64_t n, int64_t cin, int64_t hw,
+                              int64_t cout, int activation, float max_limit, float *out) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_CHECK(ctx, activation >= MACE_HIP_ACT_NOOP && activation <= MACE_HIP_ACT_RELUX,
+           "unsupported activation %d", activation);
+  // mace/ops/arm/base/conv_2d_1x1.cc:66-68: Gemm(filter, input, batch, cout, cin, cin, hw,
+  // no transposes, lhs_batched = false, rhs_batched = true); bias and activation follow
+  // (mace/ops/conv_2d.cc:171-173) and are fused into the store here.
+  F32Epilogue ep{bias, activation, max_limit};
+  return mh_f32_gemm(ctx, filter, input, n, cout, hw, cin, MACE_HIP_ROW_MAJOR,
+                     MACE_HIP_ROW_MAJOR, MACE_HIP_ROW_MAJOR, 0, 1, out, ep);
+}
+
+}  // extern "C"

@@ -1,0 +1,490 @@
+// uint8 GEMM on the CDNA4 int8 matrix cores.
+//
+// Replaces gemmlowp::GemmWithOutputPipeline as MACE calls it (mace/ops/matmul.cc:280-300,
+// 366-386; mace/ops/conv_2d.cc:301-315):
+//   acc[i,j] = sum_k (lhs[i,k] + lhs_offset) * (rhs[k,j] + rhs_offset)          (int32)
+//   out      = acc                                       (int32 result, empty pipeline)
+//   out      = clamp(RDivPOT(SRDHM(acc + bias[i], mult), shift) + zp)   (uint8 result)
+//
+// The matrix cores multiply SIGNED bytes, so both operands are shifted by 128 (a byte XOR
+// with 0x80) and the zero points move with them:
+//   sum_k (l - zl)(r - zr),  l' = l - 128, r' = r - 128, zl' = zl - 128, zr' = zr - 128
+//   = sum_k l' r'  -  zr' * sum_k l'[i,k]  -  zl' * sum_k r'[k,j]  +  K zl' zr'
+// The two sums are one int32 per result row / column ("correction vectors", which also
+// absorb the bias); the kernel adds them to the MFMA accumulators in its epilogue.
+//
+// Canonical operand form: a "panel" P[n][k], k contiguous, 16-byte aligned rows.  The kernel
+// computes OUT[y][x] = sum_k X[x][k] * Y[y][k] with x contiguous in the output.  A RowMajor
+// result takes X = rhs columns, Y = lhs rows; a ColMajor result takes X = lhs rows, Y = rhs
+// columns, so each lane's four consecutive accumulator rows are contiguous in memory.
+// Operands that are already k-contiguous (lhs RowMajor, rhs ColMajor) with depth % 16 == 0
+// are read in place; anything else is first repacked (transposed and/or padded with 0x80,
+// which is zero after the shift) into the context's arena.
+#include <algorithm>
+
+#include "common.h"
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr int BK = 64;            // bytes of k per LDS tile
+constexpr int LDS_ROW = BK + 16;  // padded row: any 8 consecutive rows cover all banks once
+
+struct GemmParams {
+  const uint8_t *X;   // [XN][ldx] panel
+  const uint8_t *Y;   // [YN][ldy] panel
+  int64_t ldx, ldy;
+  int64_t xbs, ybs;   // batch strides in bytes (0 = shared across the batch)
+  int XN, YN, K;      // K = bytes of k to read per row (multiple of 16)
+  const int32_t *corrX;  // [batch or 1][XN]
+  const int32_t *corrY;  // [batch or 1][YN]
+  int64_t cxbs, cybs;    // batch strides of the correction vectors (elements)
+  void *out;
+  int64_t ldo;        // elements between consecutive y
+  int64_t obs;        // elements per batch
+  int32_t mult, zp;
+  int shift, lo, hi;
+  int tiles_x, tiles_y;
+};
+
+// XCD-aware tile order: consecutive workgroup ids are dealt round-robin to the 8 XCDs, so
+// workgroup w runs on XCD w % 8.  Give every XCD a contiguous span of the tile sequence and
+// walk that sequence in column groups of GROUP_Y tiles so that the tiles resident on one
+// XCD at a time share X and Y panels in its L2.
+__device__ inline void tile_of_block(int bid, int nblocks, int tiles_x, int tiles_y, int *tx,
+                                     int *ty) {
+  constexpr int XCDS = 8;
+  int t = bid;
+  if (nblocks % XCDS == 0) t = (bid % XCDS) * (nblocks / XCDS) + bid / XCDS;
+  constexpr int GROUP_Y = 8;
+  const int per_group = GROUP_Y * tiles_x;
+  const int g = t / per_group;
+  const int first_y = g * GROUP_Y;
+  const int gsize = min(GROUP_Y, tiles_y - first_y);
+  const int r = t - g * per_group;
+  *ty = first_y + r % gsize;
+  *tx = r / gsize;
+}
+
+template <int WX, int WY, int FX, int FY, typename OutT>
+__global__ __launch_bounds__(WX *WY * 64) void q8_gemm_kernel(GemmParams p) {
+  constexpr int NT = WX * WY * 64;
+  constexpr int TX = WX * FX * 32;
+  constexpr int TY = WY * FY * 32;
+  constexpr int CHUNKS_X = TX * (BK / 16) / NT;   // 16-byte chunks per thread per tile
+  constexpr int CHUNKS_Y = TY * (BK / 16) / NT;
+  static_assert(CHUNKS_X >= 1 && CHUNKS_Y >= 1, "tile too small for the block");
+  static_assert(TX * (BK / 16) % NT == 0 && TY * (BK / 16) % NT == 0, "uneven tile load");
+
+  extern __shared__ __align__(16) uint8_t lds[];
+  constexpr int BUF_BYTES = (TX + TY) * LDS_ROW;   // X tile then Y tile, two buffers
+  constexpr int Y_OFF = TX * LDS_ROW;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wx = wave % WX, wy = wave / WX;
+
+  int tile_x, tile_y;
+  tile_of_block(blockIdx.x, gridDim.x, p.tiles_x, p.tiles_y, &tile_x, &tile_y);
+  const int x0 = tile_x * TX, y0 = tile_y * TY;
+  const int b = blockIdx.z;
+
+  const uint8_t *Xb = p.X + (int64_t)b * p.xbs;
+  const uint8_t *Yb = p.Y + (int64_t)b * p.ybs;
+
+  // per-thread global row pointers (rows beyond the edge re-read the last row; their
+  // results are never stored)
+  const uint8_t *gx[CHUNKS_X];
+  const uint8_t *gy[CHUNKS_Y];
+  int lx[CHUNKS_X], ly[CHUNKS_Y], kx[CHUNKS_X], ky[CHUNKS_Y];
+#pragma unroll
+  for (int i = 0; i < CHUNKS_X; ++i) {
+    const int c = tid + i * NT;
+    const int row = c / (BK / 16), kc = c % (BK / 16);
+    gx[i] = Xb + (int64_t)min(x0 + row, p.XN - 1) * p.ldx + kc * 16;
+    lx[i] = row * LDS_ROW + kc * 16;
+    kx[i] = kc * 16;
+  }
+#pragma unroll
+  for (int i = 0; i < CHUNKS_Y; ++i) {
+    const int c = tid + i * NT;
+    const int row = c / (BK / 16), kc = c % (BK / 16);
+    gy[i] = Yb + (int64_t)min(y0 + row, p.YN - 1) * p.ldy + kc * 16;
+    ly[i] = row * LDS_ROW + kc * 16;
+    ky[i] = kc * 16;
+  }
+
+  v4i rx[CHUNKS_X], ry[CHUNKS_Y];
+  const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+  const v4i zero4 = {0, 0, 0, 0};
+
+  auto load_global = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < CHUNKS_X; ++i)
+      rx[i] = (k0 + kx[i] < p.K) ? (*(const v4i *)(gx[i] + k0) ^ flip) : zero4;
+#pragma unroll
+    for (int i = 0; i < CHUNKS_Y; ++i)
+      ry[i] = (k0 + ky[i] < p.K) ? (*(const v4i *)(gy[i] + k0) ^ flip) : zero4;
+  };
+  auto store_lds = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < CHUNKS_X; ++i) *(v4i *)(lds + buf * BUF_BYTES + lx[i]) = rx[i];
+#pragma unroll
+    for (int i = 0; i < CHUNKS_Y; ++i) *(v4i *)(lds + buf * BUF_BYTES + Y_OFF + ly[i]) = ry[i];
+  };
+
+  v16i acc[FX][FY];
+#pragma unroll
+  for (int i = 0; i < FX; ++i)
+#pragma unroll
+    for (int j = 0; j < FY; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+  // fragment addresses: lane l supplies row (l % 32), k bytes [16*(l/32), +16) of each
+  // 32-byte k step, for both operands (the pairing of k positions is what matters)
+  const int frag_off = (lane & 31) * LDS_ROW + (lane >> 5) * 16;
+  const int fx_base = wx * FX * 32 * LDS_ROW + frag_off;
+  const int fy_base = wy * FY * 32 * LDS_ROW + frag_off;
+
+  const int nk = (p.K + BK - 1) / BK;
+  load_global(0);
+  store_lds(0);
+  __syncthreads();
+  for (int kt = 0; kt < nk; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < nk) load_global((kt + 1) * BK);
+#pragma unroll
+    for (int ks = 0; ks < BK / 32; ++ks) {
+      v4i a[FX], bf[FY];
+#pragma unroll
+      for (int i = 0; i < FX; ++i)
+        a[i] = *(const v4i *)(lds + buf * BUF_BYTES + fx_base + i * 32 * LDS_ROW + ks * 32);
+#pragma unroll
+      for (int j = 0; j < FY; ++j)
+        bf[j] = *(const v4i *)(lds + buf * BUF_BYTES + Y_OFF + fy_base + j * 32 * LDS_ROW + ks * 32);
+#pragma unroll
+      for (int i = 0; i < FX; ++i)
+#pragma unroll
+        for (int j = 0; j < FY; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], bf[j], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < nk) store_lds(buf ^ 1);
+    __syncthreads();
+  }
+
+  // epilogue: accumulator register r of a 32x32 tile holds
+  //   x (MFMA row)    = 8 * (r / 4) + 4 * (lane / 32) + r % 4
+  //   y (MFMA column) = lane % 32
+  const int32_t *cX = p.corrX + (int64_t)b * p.cxbs;
+  const int32_t *cY = p.corrY + (int64_t)b * p.cybs;
+  OutT *outb = (OutT *)p.out + (int64_t)b * p.obs;
+  const bool vec_ok = (p.ldo % 4 == 0) && (((uintptr_t)outb) % (4 * sizeof(OutT)) == 0);
+#pragma unroll
+  for (int j = 0; j < FY; ++j) {
+    const int y = y0 + (wy * FY + j) * 32 + (lane & 31);
+    if (y >= p.YN) continue;
+    const uint32_t cy = (uint32_t)cY[y];
+    OutT *orow = outb + (int64_t)y * p.ldo;
+#pragma unroll
+    for (int i = 0; i < FX; ++i) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int x = x0 + (wx * FX + i) * 32 + 8 * q + 4 * (lane >> 5);
+        if (x >= p.XN) continue;
+        int32_t v[4];
+        const bool full = x + 3 < p.XN;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const uint32_t cx = (uint32_t)cX[min(x + e, p.XN - 1)];
+          v[e] = (int32_t)((uint32_t)acc[i][j][q * 4 + e] + cx + cy);
+        }
+        if constexpr (sizeof(OutT) == 4) {
+          if (full && vec_ok) {
+            *(v4i *)(orow + x) = v4i{v[0], v[1], v[2], v[3]};
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (x + e < p.XN) orow[x + e] = (OutT)v[e];
+          }
+        } else {
+          uint32_t packed = 0;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const uint32_t u = (uint32_t)mh_requant_fixed(v[e], p.mult, p.shift, p.zp, p.lo, p.hi);
+            packed |= u << (8 * e);
+          }
+          if (full && vec_ok) {
+            *(uint32_t *)(orow + x) = packed;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (x + e < p.XN) orow[x + e] = (OutT)((packed >> (8 * e)) & 0xff);
+          }
+        }
+      }
+    }
+  }
+}
+
+// ---- repacking ---------------------------------------------------------------------------
+
+// src is k-contiguous already ([n][k], row stride = k) but k is not a multiple of 16 or the
+// base is misaligned: copy into [n][kp] rows padded with 0x80.
+__global__ void q8_pack_rows_kernel(const uint8_t *src, int64_t src_bs, uint8_t *dst,
+                                    int64_t dst_bs, int n, int k, int kp) {
+  const int64_t total = (int64_t)n * kp;
+  const uint8_t *s = src + (int64_t)blockIdx.z * src_bs;
+  uint8_t *d = dst + (int64_t)blockIdx.z * dst_bs;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / kp;
+    const int c = (int)(i - r * kp);
+    d[i] = c < k ? s[r * k + c] : (uint8_t)0x80;
+  }
+}
+
+// src is [k][n] with n contiguous (row stride = n): write dst [n][kp], padding k..kp with
+// 0x80.  64x64-byte tiles through LDS; 16-byte global accesses when n % 16 == 0 and the
+// base is aligned, byte accesses otherwise.
+__global__ __launch_bounds__(256) void q8_pack_transpose_kernel(const uint8_t *src,
+                                                                int64_t src_bs, uint8_t *dst,
+                                                                int64_t dst_bs, int n, int k,
+                                                                int kp, int vec_ok) {
+  __shared__ uint8_t tile[64][64 + 4];
+  const uint8_t *s = src + (int64_t)blockIdx.z * src_bs;
+  uint8_t *d = dst + (int64_t)blockIdx.z * dst_bs;
+  const int n0 = blockIdx.x * 64, k0 = blockIdx.y * 64;
+  const int tid = threadIdx.x;
+  {
+    const int kk = tid >> 2, nc = (tid & 3) * 16;   // row kk of the tile, 16 bytes of n
+    const int gk = k0 + kk, gn = n0 + nc;
+    uint8_t v[16];
+    if (gk < k && vec_ok && gn + 15 < n) {
+      *(uint4 *)v = *(const uint4 *)(s + (int64_t)gk * n + gn);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+        v[e] = (gk < k && gn + e < n) ? s[(int64_t)gk * n + gn + e] : (uint8_t)0x80;
+    }
+#pragma unroll
+    for (int e = 0; e < 16; ++e) tile[kk][nc + e] = v[e];
+  }
+  __syncthreads();
+  {
+    const int nn = tid >> 2, kc = (tid & 3) * 16;   // output row nn, 16 bytes of k
+    const int gn = n0 + nn, gk = k0 + kc;
+    if (gn < n && gk < kp) {
+      uint8_t v[16];
+#pragma unroll
+      for (int e = 0; e < 16; ++e) v[e] = tile[kc + e][nn];
+      // kp is a multiple of 64, so the 16-byte store stays inside the padded row
+      *(uint4 *)(d + (int64_t)gn * kp + gk) = *(uint4 *)v;
+    }
+  }
+}
+
+// ---- correction vectors --------------------------------------------------------------------
+
+// corr[b][n] = coef * sum_k (P[b][n][k] - 128) + add + (bias ? bias[n] : 0), modulo 2^32.
+// One wavefront per panel row.
+__global__ __launch_bounds__(256) void q8_panel_sums_kernel(const uint8_t *P, int64_t ld,
+                                                            int64_t pbs, int n, int k,
+                                                            int32_t coef, int32_t add,
+                                                            const int32_t *bias,
+                                                            int32_t *corr) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= n) return;
+  const uint8_t *r = P + (int64_t)blockIdx.z * pbs + (int64_t)row * ld;
+  uint32_t s = 0;
+  for (int c = lane * 16; c < k; c += 64 * 16) {
+    const uint4 v = *(const uint4 *)(r + c);
+    s = __builtin_amdgcn_udot4(v.x, 0x01010101u, s, false);
+    s = __builtin_amdgcn_udot4(v.y, 0x01010101u, s, false);
+    s = __builtin_amdgcn_udot4(v.z, 0x01010101u, s, false);
+    s = __builtin_amdgcn_udot4(v.w, 0x01010101u, s, false);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+  if (lane == 0) {
+    const uint32_t shifted = s - 128u * (uint32_t)k;   // sum of (byte - 128)
+    uint32_t v = (uint32_t)coef * shifted + (uint32_t)add;
+    if (bias) v += (uint32_t)bias[row];
+    corr[(int64_t)blockIdx.z * n + row] = (int32_t)v;
+  }
+}
+
+template <int WX, int WY, int FX, int FY>
+int launch_gemm(mace_hip_ctx *ctx, GemmParams &p, bool out_u8, int batch) {
+  constexpr int TX = WX * FX * 32, TY = WY * FY * 32;
+  p.tiles_x = (p.XN + TX - 1) / TX;
+  p.tiles_y = (p.YN + TY - 1) / TY;
+  const size_t lds = 2 * (size_t)(TX + TY) * LDS_ROW;
+  dim3 grid(p.tiles_x * p.tiles_y, 1, batch), block(WX * WY * 64);
+  if (out_u8) {
+    auto k = q8_gemm_kernel<WX, WY, FX, FY, uint8_t>;
+    if (lds > 64 * 1024)
+      MH_HIP(ctx, hipFuncSetAttribute((const void *)k,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p);
+  } else {
+    auto k = q8_gemm_kernel<WX, WY, FX, FY, int32_t>;
+    if (lds > 64 * 1024)
+      MH_HIP(ctx, hipFuncSetAttribute((const void *)k,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p);
+  }
+  MH_HIP(ctx, hipGetLastError());
+  return MACE_HIP_SUCCESS;
+}
+
+}  // namespace
+
+int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8_t *rhs,
+               int rhs_order, void *out, int out_order, bool out_u8, int64_t batch,
+               int64_t rows, int64_t depth, int64_t cols, int lhs_batched, int rhs_batched,
+               int32_t lhs_offset, int32_t rhs_offset, const Q8GemmEpilogue &ep) {
+  MH_CHECK(ctx, batch >= 0 && rows >= 0 && depth >= 0 && cols >= 0, "negative dimension");
+  MH_CHECK(ctx, (lhs_order | 1) == 1 && (rhs_order | 1) == 1 && (out_order | 1) == 1,
+           "matrix order must be RowMajor (0) or ColMajor (1)");
+  MH_CHECK(ctx, rows < (1ll << 31) && cols < (1ll << 31) && depth < (1ll << 31) - 64 &&
+                    batch < 65536,
+           "dimension too large");
+  if (out_u8) {
+    MH_CHECK(ctx, ep.shift >= 0 && ep.shift <= 31, "right shift %d outside [0,31]", ep.shift);
+    MH_CHECK(ctx, ep.lo >= 0 && ep.hi <= 255 && ep.lo <= ep.hi, "clamp range [%d,%d] invalid",
+             ep.lo, ep.hi);
+  }
+  if (batch == 0 || rows == 0 || cols == 0) return MACE_HIP_SUCCESS;
+  MH_CHECK(ctx, lhs && rhs && out, "null operand");
+
+  const int lhs_nb = lhs_batched ? (int)batch : 1, rhs_nb = rhs_batched ? (int)batch : 1;
+  const int64_t kp = (int64_t)mh_align_up((size_t)(depth > 0 ? depth : 1), 64);
+
+  // which operands can be read in place
+  const bool lhs_direct = lhs_order == MACE_HIP_ROW_MAJOR && depth % 16 == 0 && depth > 0 &&
+                          ((uintptr_t)lhs % 16 == 0);
+  const bool rhs_direct = rhs_order == MACE_HIP_COL_MAJOR && depth % 16 == 0 && depth > 0 &&
+                          ((uintptr_t)rhs % 16 == 0);
+
+  size_t need = sizeof(int32_t) * ((size_t)lhs_nb * rows + (size_t)rhs_nb * cols) + 4096;
+  if (!lhs_direct) need += (size_t)lhs_nb * rows * kp + 256;
+  if (!rhs_direct) need += (size_t)rhs_nb * cols * kp + 256;
+  MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, need));
+  ArenaScope scope(ctx);
+
+  struct Panel {
+    const uint8_t *ptr;
+    int64_t ld, bs;
+    int k;   // readable bytes of k per row
+  } L, R;
+
+  auto prepare = [&](const uint8_t *src, int order_is_kcontig, bool direct, int nb, int64_t n,
+                     Panel *P) -> int {
+    if (direct) {
+      *P = Panel{src, depth, nb > 1 ? n * depth : 0, (int)depth};
+      return MACE_HIP_SUCCESS;
+    }
+    uint8_t *dst = (uint8_t *)mh_arena_take(ctx, (size_t)nb * n * kp);
+    if (!dst) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
+    if (depth == 0) {
+      MH_HIP(ctx, hipMemsetAsync(dst, 0x80, (size_t)nb * n * kp, ctx->stream));
+    } else if (order_is_kcontig) {
+      const int64_t total = n * kp;
+      dim3 grid((unsigned)std::min<int64_t>((total + 255) / 256, 65535), 1, nb);
+      hipLaunchKernelGGL(q8_pack_rows_kernel, grid, dim3(256), 0, ctx->stream, src,
+                         n * depth, dst, n * kp, (int)n, (int)depth, (int)kp);
+    } else {
+      MH_CHECK(ctx, (kp / 64) <= 65535, "depth too large to repack");
+      dim3 grid((unsigned)((n + 63) / 64), (unsigned)(kp / 64), nb);
+      const int vec_ok = (n % 16 == 0) && ((uintptr_t)src % 16 == 0);
+      hipLaunchKernelGGL(q8_pack_transpose_kernel, grid, dim3(256), 0, ctx->stream, src,
+                         n * depth, dst, n * kp, (int)n, (int)depth, (int)kp, vec_ok);
+    }
+    MH_HIP(ctx, hipGetLastError());
+    *P = Panel{dst, kp, nb > 1 ? n * kp : 0, (int)kp};
+    return MACE_HIP_SUCCESS;
+  };
+  MH_RETURN_IF_ERROR(prepare(lhs, lhs_order == MACE_HIP_ROW_MAJOR, lhs_direct, lhs_nb, rows, &L));
+  MH_RETURN_IF_ERROR(prepare(rhs, rhs_order == MACE_HIP_COL_MAJOR, rhs_direct, rhs_nb, cols, &R));
+
+  // correction vectors.  zl' = -lhs_offset - 128, zr' = -rhs_offset - 128.
+  //   corrL[i] = -zr' * sum_k l'[i,k] + bias[i];   corrR[j] = -zl' * sum_k r'[k,j] + K zl' zr'
+  int32_t *corrL = (int32_t *)mh_arena_take(ctx, sizeof(int32_t) * lhs_nb * rows);
+  int32_t *corrR = (int32_t *)mh_arena_take(ctx, sizeof(int32_t) * rhs_nb * cols);
+  if (!corrL || !corrR) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
+  const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
+  {
+    dim3 gl((unsigned)((rows + 3) / 4), 1, lhs_nb), gr((unsigned)((cols + 3) / 4), 1, rhs_nb);
+    hipLaunchKernelGGL(q8_panel_sums_kernel, gl, dim3(256), 0, ctx->stream, L.ptr, L.ld,
+                       L.bs, (int)rows, L.k, (int32_t)(0u - zr), 0,
+                       out_u8 ? ep.bias : nullptr, corrL);
+    hipLaunchKernelGGL(q8_panel_sums_kernel, gr, dim3(256), 0, ctx->stream, R.ptr, R.ld,
+                       R.bs, (int)cols, R.k, (int32_t)(0u - zl),
+                       (int32_t)((uint32_t)depth * zl * zr), (const int32_t *)nullptr, corrR);
+    MH_HIP(ctx, hipGetLastError());
+  }
+
+  GemmParams p;
+  const bool x_is_lhs = out_order == MACE_HIP_COL_MAJOR;
+  const Panel &PX = x_is_lhs ? L : R;
+  const Panel &PY = x_is_lhs ? R : L;
+  p.X = PX.ptr; p.ldx = PX.ld; p.xbs = PX.bs;
+  p.Y = PY.ptr; p.ldy = PY.ld; p.ybs = PY.bs;
+  p.XN = (int)(x_is_lhs ? rows : cols);
+  p.YN = (int)(x_is_lhs ? cols : rows);
+  p.K = L.k < R.k ? L.k : R.k;    // padded tails are zero after the shift, so the shorter wins
+  p.corrX = x_is_lhs ? corrL : corrR;
+  p.corrY = x_is_lhs ? corrR : corrL;
+  p.cxbs = (x_is_lhs ? lhs_nb : rhs_nb) > 1 ? p.XN : 0;
+  p.cybs = (x_is_lhs ? rhs_nb : lhs_nb) > 1 ? p.YN : 0;
+  p.out = out;
+  p.ldo = p.XN;
+  p.obs = rows * cols;
+  p.mult = ep.mult; p.shift = ep.shift; p.zp = ep.zp; p.lo = ep.lo; p.hi = ep.hi;
+
+  // tile shape: the largest that still yields enough workgroups to fill the CUs
+  const int64_t cu = ctx->cu_count > 0 ? ctx->cu_count : 256;
+  auto tiles = [&](int tx, int ty) {
+    return (int64_t)((p.XN + tx - 1) / tx) * ((p.YN + ty - 1) / ty) * batch;
+  };
+  if (p.XN > 128 && p.YN > 128 && tiles(256, 256) >= cu)
+    return launch_gemm<2, 2, 4, 4>(ctx, p, out_u8, (int)batch);
+  if (p.XN <= 64 && p.YN > 128 && tiles(64, 256) >= cu)
+    return launch_gemm<1, 4, 2, 2>(ctx, p, out_u8, (int)batch);
+  if (p.XN > 64 && p.YN > 64 && tiles(128, 128) >= cu)
+    return launch_gemm<2, 2, 2, 2>(ctx, p, out_u8, (int)batch);
+  return launch_gemm<2, 2, 1, 1>(ctx, p, out_u8, (int)batch);
+}
+
+extern "C" {
+
+int mace_hip_gemm_q8_i32(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order,
+                         const uint8_t *rhs, int rhs_order, int32_t *out, int out_order,
+                         int64_t batch, int64_t rows, int64_t depth, int64_t cols,
+                         int lhs_batched, int rhs_batched, int32_t lhs_offset,
+                         int32_t rhs_offset) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  Q8GemmEpilogue ep{nullptr, 0, 0, 0, 0, 255};
+  return mh_q8_gemm(ctx, lhs, lhs_order, rhs, rhs_order, out, out_order, false, batch, rows,
+                    depth, cols, lhs_batched, rhs_batched, lhs_offset, rhs_offset, ep);
+}
+
+int mace_hip_gemm_q8_u8(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order,
+                        const uint8_t *rhs, int rhs_order, uint8_t *out, int out_order,
+                        int64_t batch, int64_t rows, int64_t depth, int64_t cols,
+                        int lhs_batched, int rhs_batched, int32_t lhs_offset,
+                        int32_t rhs_offset, const int32_t *bias, int32_t multiplier,
+                        int right_shift, int32_t offset_after_shift, int clamp_min,
+                        int clamp_max) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  Q8GemmEpilogue ep{bias, multiplier, right_shift, offset_after_shift, clamp_min, clamp_max};
+  return mh_q8_gemm(ctx, lhs, lhs_order, rhs, rhs_order, out, out_order, true, batch, rows,
+                    depth, cols, lhs_batched, rhs_batched, lhs_offset, rhs_offset, ep);
+}
+
+}  // extern "C"

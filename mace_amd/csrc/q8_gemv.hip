@@ -1,0 +1,225 @@
+// uint8 Gemv (FullyConnected): a streaming kernel bound by HBM bandwidth.
+//
+// Replaces ref::q8::Gemv<uint8_t|int32_t> (mace/ops/ref/q8/gemv.cc:80-162) and
+// arm::q8::Gemv (mace/ops/arm/q8/gemv.cc:36-171):
+//   sum[b,h] = bias[h] + sum_w (lhs[b?,h,w] - lhs_zp) * (rhs[b?,w] - rhs_zp)      (int32)
+// evaluated, like the NEON kernel, from unsigned dot products and byte sums:
+//   sum = dot(l, r) - rhs_zp * sum(l) - lhs_zp * sum(r) + W * lhs_zp * rhs_zp + bias
+// in modulo-2^32 arithmetic (identical to the definition whenever it does not overflow).
+//
+// One wavefront owns one weight row: 64 lanes x 16-byte loads cover 1 KiB per step, all
+// loads of a row are issued before the first dot product so a CU keeps tens of KiB in
+// flight.  Up to NB batch rows of the right-hand vector are consumed per pass over the
+// weights, so the weight matrix is streamed once for batch <= 8.
+#include "common.h"
+
+namespace {
+
+struct GemvParams {
+  const uint8_t *lhs;
+  const uint8_t *rhs;
+  const int32_t *bias;
+  void *out;
+  int64_t lhs_bs, rhs_bs;   // bytes between batches (0 = shared)
+  int H, W;
+  int batch;
+  int32_t lhs_zp, rhs_zp;
+  float mult;               // (lhs_scale * rhs_scale) / out_scale in binary32
+  int32_t out_zp;
+  int neon_mode;
+};
+
+__device__ inline uint32_t wave_sum(uint32_t v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+__device__ inline uint32_t dot16(const uint4 &a, const uint4 &b, uint32_t acc) {
+  acc = __builtin_amdgcn_udot4(a.x, b.x, acc, false);
+  acc = __builtin_amdgcn_udot4(a.y, b.y, acc, false);
+  acc = __builtin_amdgcn_udot4(a.z, b.z, acc, false);
+  acc = __builtin_amdgcn_udot4(a.w, b.w, acc, false);
+  return acc;
+}
+
+// VEC: rows are 16-byte aligned and W % 16 == 0.  NB: batch rows per pass.
+// grid.x covers rows (4 per block), grid.y covers batch passes.
+template <int NB, bool VEC, typename OutT>
+__global__ __launch_bounds__(256) void q8_gemv_kernel(GemvParams p) {
+  const int lane = threadIdx.x & 63;
+  const int h = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (h >= p.H) return;
+  const int b0 = blockIdx.y * NB;
+  const int nb = min(NB, p.batch - b0);
+  const uint8_t *l = p.lhs + (int64_t)b0 * p.lhs_bs + (int64_t)h * p.W;
+  const uint8_t *r = p.rhs + (int64_t)b0 * p.rhs_bs;
+
+  uint32_t dot[NB], sum_r[NB], sum_l = 0;
+#pragma unroll
+  for (int b = 0; b < NB; ++b) dot[b] = sum_r[b] = 0;
+
+  if constexpr (VEC) {
+    const uint4 ones = {0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u};
+    const int nchunk = p.W >> 4;
+    // four chunks per lane per step: 4 KiB of the row in flight per wavefront
+    int c = lane;
+    for (; c + 192 < nchunk; c += 256) {
+      uint4 w0 = *(const uint4 *)(l + (int64_t)c * 16);
+      uint4 w1 = *(const uint4 *)(l + (int64_t)(c + 64) * 16);
+      uint4 w2 = *(const uint4 *)(l + (int64_t)(c + 128) * 16);
+      uint4 w3 = *(const uint4 *)(l + (int64_t)(c + 192) * 16);
+      sum_l = dot16(w0, ones, sum_l);
+      sum_l = dot16(w1, ones, sum_l);
+      sum_l = dot16(w2, ones, sum_l);
+      sum_l = dot16(w3, ones, sum_l);
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        if (b < nb) {
+          const uint8_t *rb = r + (int64_t)b * p.rhs_bs;
+          const uint4 x0 = *(const uint4 *)(rb + (int64_t)c * 16);
+          const uint4 x1 = *(const uint4 *)(rb + (int64_t)(c + 64) * 16);
+          const uint4 x2 = *(const uint4 *)(rb + (int64_t)(c + 128) * 16);
+          const uint4 x3 = *(const uint4 *)(rb + (int64_t)(c + 192) * 16);
+          dot[b] = dot16(w0, x0, dot[b]);
+          dot[b] = dot16(w1, x1, dot[b]);
+          dot[b] = dot16(w2, x2, dot[b]);
+          dot[b] = dot16(w3, x3, dot[b]);
+          sum_r[b] = dot16(x0, ones, sum_r[b]);
+          sum_r[b] = dot16(x1, ones, sum_r[b]);
+          sum_r[b] = dot16(x2, ones, sum_r[b]);
+          sum_r[b] = dot16(x3, ones, sum_r[b]);
+        }
+      }
+    }
+    for (; c < nchunk; c += 64) {
+      const uint4 w0 = *(const uint4 *)(l + (int64_t)c * 16);
+      sum_l = dot16(w0, ones, sum_l);
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        if (b < nb) {
+          const uint4 x0 = *(const uint4 *)(r + (int64_t)b * p.rhs_bs + (int64_t)c * 16);
+          dot[b] = dot16(w0, x0, dot[b]);
+          sum_r[b] = dot16(x0, ones, sum_r[b]);
+        }
+      }
+    }
+  } else {
+    for (int w = lane; w < p.W; w += 64) {
+      const uint32_t lv = l[w];
+      sum_l += lv;
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        if (b < nb) {
+          const uint32_t rv = r[(int64_t)b * p.rhs_bs + w];
+          dot[b] += lv * rv;
+          sum_r[b] += rv;
+        }
+      }
+    }
+  }
+
+  sum_l = wave_sum(sum_l);
+  const uint32_t zl = (uint32_t)p.lhs_zp, zr = (uint32_t)p.rhs_zp;
+  const uint32_t fixed = (uint32_t)p.W * zl * zr + (p.bias ? (uint32_t)p.bias[h] : 0u);
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    if (b < nb) {
+      const uint32_t d = wave_sum(dot[b]);
+      const uint32_t sr = wave_sum(sum_r[b]);
+      if (lane == 0) {
+        // when lhs is batched every batch has its own row, hence its own sum_l: NB is 1 then
+        const int32_t ret = (int32_t)(d - sum_l * zr - sr * zl + fixed);
+        OutT *o = (OutT *)p.out + (int64_t)(b0 + b) * p.H + h;
+        if constexpr (sizeof(OutT) == 4) {
+          *o = (OutT)ret;
+        } else {
+          *o = (OutT)mh_requant_float(ret, p.mult, p.out_zp, p.neon_mode);
+        }
+      }
+    }
+  }
+}
+
+template <typename OutT>
+int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
+  const bool vec = (p.W % 16 == 0) && ((uintptr_t)p.lhs % 16 == 0) &&
+                   ((uintptr_t)p.rhs % 16 == 0);
+  // a batched lhs gives every batch its own weights: one batch row per pass
+  int nb = lhs_batched ? 1 : (p.batch >= 8 ? 8 : (p.batch >= 4 ? 4 : (p.batch >= 2 ? 2 : 1)));
+  dim3 block(256);
+  dim3 grid((unsigned)((p.H + 3) / 4), (unsigned)((p.batch + nb - 1) / nb));
+#define MH_GEMV_LAUNCH(NB_)                                                              \
+  do {                                                                                   \
+    if (vec)                                                                             \
+      hipLaunchKernelGGL((q8_gemv_kernel<NB_, true, OutT>), grid, block, 0, ctx->stream, p); \
+    else                                                                                 \
+      hipLaunchKernelGGL((q8_gemv_kernel<NB_, false, OutT>), grid, block, 0, ctx->stream, p); \
+  } while (0)
+  switch (nb) {
+    case 8: MH_GEMV_LAUNCH(8); break;
+    case 4: MH_GEMV_LAUNCH(4); break;
+    case 2: MH_GEMV_LAUNCH(2); break;
+    default: MH_GEMV_LAUNCH(1); break;
+  }
+#undef MH_GEMV_LAUNCH
+  MH_HIP(ctx, hipGetLastError());
+  return MACE_HIP_SUCCESS;
+}
+
+int gemv_common(mace_hip_ctx *ctx, GemvParams &p, int64_t batch, int64_t height,
+                int64_t width, int lhs_batched, int rhs_batched, bool out_u8) {
+  MH_CHECK(ctx, batch >= 0 && height >= 0 && width >= 0, "negative dimension");
+  MH_CHECK(ctx, height < (1ll << 31) && width < (1ll << 31) && batch < (1ll << 31),
+           "dimension too large");
+  if (batch == 0 || height == 0) return MACE_HIP_SUCCESS;
+  MH_CHECK(ctx, p.out && (width == 0 || (p.lhs && p.rhs)), "null operand");
+  MH_CHECK(ctx, (height + 3) / 4 <= 0x7fffffff && batch <= 65535 * 8, "grid too large");
+  p.H = (int)height;
+  p.W = (int)width;
+  p.batch = (int)batch;
+  p.lhs_bs = lhs_batched ? height * width : 0;
+  p.rhs_bs = rhs_batched ? width : 0;
+  return out_u8 ? launch_gemv<uint8_t>(ctx, p, lhs_batched)
+                : launch_gemv<int32_t>(ctx, p, lhs_batched);
+}
+
+}  // namespace
+
+extern "C" {
+
+int mace_hip_gemv_q8_u8(mace_hip_ctx *ctx, const uint8_t *lhs, const uint8_t *rhs,
+                        const int32_t *bias, int64_t batch, int64_t height, int64_t width,
+                        int lhs_batched, int rhs_batched, int32_t lhs_zp, int32_t rhs_zp,
+                        float lhs_scale, float rhs_scale, float out_scale, int32_t out_zp,
+                        int requant_mode, uint8_t *out) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_CHECK(ctx, requant_mode == MACE_HIP_REQUANT_REF || requant_mode == MACE_HIP_REQUANT_NEON,
+           "unknown requant mode %d", requant_mode);
+  MH_CHECK(ctx, out_scale > 0.f, "output scale must not be zero");
+  volatile float prod = lhs_scale * rhs_scale;
+  volatile float m = prod / out_scale;
+  if (requant_mode == MACE_HIP_REQUANT_NEON) {
+    const float mm = m;
+    MH_CHECK(ctx, mm > 0.f && mm < 1.f, "output multiplier %g outside (0,1)", (double)mm);
+  }
+  GemvParams p{};
+  p.lhs = lhs; p.rhs = rhs; p.bias = bias; p.out = out;
+  p.lhs_zp = lhs_zp; p.rhs_zp = rhs_zp;
+  p.mult = m; p.out_zp = out_zp;
+  p.neon_mode = requant_mode == MACE_HIP_REQUANT_NEON;
+  return gemv_common(ctx, p, batch, height, width, lhs_batched, rhs_batched, true);
+}
+
+int mace_hip_gemv_q8_i32(mace_hip_ctx *ctx, const uint8_t *lhs, const uint8_t *rhs,
+                         const int32_t *bias, int64_t batch, int64_t height, int64_t width,
+                         int lhs_batched, int rhs_batched, int32_t lhs_zp, int32_t rhs_zp,
+                         int32_t *out) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  GemvParams p{};
+  p.lhs = lhs; p.rhs = rhs; p.bias = bias; p.out = out;
+  p.lhs_zp = lhs_zp; p.rhs_zp = rhs_zp;
+  return gemv_common(ctx, p, batch, height, width, lhs_batched, rhs_batched, false);
+}
+
+}  // extern "C"

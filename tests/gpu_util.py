@@ -1,0 +1,47 @@
+"""Helpers shared by the GPU parity tests: host-pointer and device-pointer call paths."""
+import ctypes as C
+
+import numpy as np
+
+from mace_amd import lib as mh
+
+
+def ptr(a):
+    """void* of a numpy array (or None)."""
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def c_(a, dtype):
+    return None if a is None else np.ascontiguousarray(a, dtype=dtype)
+
+
+class Dev:
+    """Device copies of numpy arrays through torch, for the device-pointer entry points."""
+
+    def __init__(self):
+        import torch
+        self.torch = torch
+        self.keep = []
+
+    def put(self, a):
+        if a is None:
+            return None
+        t = self.torch.from_numpy(np.ascontiguousarray(a)).cuda()
+        self.keep.append(t)
+        return C.c_void_p(t.data_ptr())
+
+    def empty(self, n, dtype):
+        tdt = {np.uint8: self.torch.uint8, np.int32: self.torch.int32,
+               np.float32: self.torch.float32}[dtype]
+        t = self.torch.empty(max(int(n), 1), dtype=tdt, device="cuda")
+        self.keep.append(t)
+        return t, C.c_void_p(t.data_ptr())
+
+    def sync(self):
+        self.torch.cuda.synchronize()
+
+
+def as_major(mat, major):
+    if major == mh.ROW_MAJOR:
+        return np.ascontiguousarray(mat).reshape(-1)
+    return np.ascontiguousarray(np.swapaxes(mat, -1, -2)).reshape(-1)

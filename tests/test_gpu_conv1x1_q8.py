@@ -1,0 +1,102 @@
+"""Quantized Conv2D 1x1 (NHWC) on the GPU vs the CPU oracle and the reference's one bit-exact
+known answer (conv_2d_test.cc:1240-1275 -> 230)."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from mace_amd import lib as mh
+from oracle import mace_oracle as orc
+from gpu_util import Dev, c_, ptr
+
+pytestmark = pytest.mark.gpu
+GOLDEN = json.load(open(os.path.join(os.path.dirname(__file__), "golden",
+                                     "reference_vectors.json")))
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = mh.Context(0)
+    yield c
+    c.close()
+
+
+def conv_host(ctx, x, f, bias, n, h, w, cin, cout, s_in, z_in, s_f, z_f, s_b, s_o, z_o,
+              lo=0, hi=255):
+    out = np.empty(n * h * w * cout, np.uint8)
+    ctx.call("mace_hip_conv1x1_q8_nhwc_host", ptr(c_(x, np.uint8)), ptr(c_(f, np.uint8)),
+             ptr(c_(bias, np.int32)), n, h, w, cin, cout, s_in, z_in, s_f, z_f, s_b, s_o, z_o,
+             lo, hi, ptr(out))
+    return out.reshape(n, h, w, cout)
+
+
+def test_conv_q8_known_answer(ctx):
+    k = GOLDEN["conv_q8_kat"]
+    out = conv_host(ctx, np.array(k["input"], np.uint8), np.array(k["filter"], np.uint8),
+                    np.array(k["bias"], np.int32), 1, 1, 1, 18, 1, k["input_scale"],
+                    k["input_zp"], k["filter_scale"], k["filter_zp"], k["bias_scale"],
+                    k["out_scale"], k["out_zp"])
+    assert out.reshape(-1).tolist() == [k["expected"]]
+
+
+# MobileNetV1 pointwise shapes of BASELINE config 4 at batch 1-2 (batch 64 runs in the
+# benchmark), the reference's random 1x1 case (conv_2d_test.cc:1383: batch 1, 128 <- 64, 32x32)
+# and ragged shapes
+CASES = [(2, 112, 112, 32, 64), (2, 56, 56, 128, 128), (2, 28, 28, 256, 256),
+         (2, 14, 14, 512, 512), (2, 7, 7, 1024, 1024), (1, 32, 32, 64, 128),
+         (1, 33, 31, 63, 129), (3, 5, 7, 16, 8), (1, 1, 1, 1, 1)]
+
+
+@pytest.mark.parametrize("n,h,w,cin,cout", CASES)
+def test_conv1x1_q8_parity(ctx, n, h, w, cin, cout):
+    rng = np.random.default_rng(4 + h * 3 + cin)
+    x = rng.integers(0, 256, (n, h, w, cin), dtype=np.uint8)
+    f = rng.integers(1, 256, (cout, cin), dtype=np.uint8)     # non-zero weights
+    bias = rng.integers(-2 ** 15, 2 ** 15, cout).astype(np.int32)
+    z_in, z_f = int(rng.integers(118, 138)), int(rng.integers(118, 138))
+    s_in, s_f = np.float32(0.02), np.float32(0.01)
+    sigma = 74.0 * 74.0 * np.sqrt(cin) * float(s_in * s_f)
+    # ReLU6 as the converter folds it: output range [0, 6] -> zp 0, scale 6/255
+    s_relu6 = np.float32(max(6.0, 3 * sigma) / 255.0)
+    spread = 0
+    for (s_o, z_o, lo, hi, s_b, bb) in (
+            (s_relu6, 0, 0, 255, np.float32(s_in * s_f), bias),
+            (np.float32(sigma / 40.0), 120, 0, 255, np.float32(s_in * s_f), bias),
+            (np.float32(sigma / 40.0), 120, 120, 200, np.float32(s_in * s_f), None),
+            (np.float32(sigma / 40.0), 10, 0, 255, np.float32(4.0 * s_in * s_f + 3e-5), bias)):
+        want = orc.conv1x1_q8_nhwc(x, f, bb, n, h, w, cin, cout, s_in, z_in, s_f, z_f, s_b, s_o,
+                                   z_o, lo, hi)
+        got = conv_host(ctx, x, f, bb, n, h, w, cin, cout, s_in, z_in, s_f, z_f, s_b, s_o, z_o,
+                        lo, hi)
+        np.testing.assert_array_equal(got, want)
+        spread = max(spread, len(np.unique(want)))
+    # far-off zero points: everything saturates, still bit-exact
+    want = orc.conv1x1_q8_nhwc(x, f, bias, n, h, w, cin, cout, s_in, 3, s_f, 250, 1.0, 0.5, 7)
+    got = conv_host(ctx, x, f, bias, n, h, w, cin, cout, s_in, 3, s_f, 250, 1.0, 0.5, 7)
+    np.testing.assert_array_equal(got, want)
+    if n * h * w * cout > 1000:
+        assert spread > 20          # the comparison above is not vacuous
+
+
+def test_conv1x1_q8_generic_relux_clamp(ctx):
+    """Unfused quantised ReLUx (arm/q8/activation.cc:59-94) == clamp to [zp, Q(limit)]."""
+    rng = np.random.default_rng(8)
+    n, h, w, cin, cout = 1, 9, 9, 64, 32
+    x = rng.integers(0, 256, (n, h, w, cin), dtype=np.uint8)
+    f = rng.integers(0, 256, (cout, cin), dtype=np.uint8)
+    s_in, s_f, s_o, z_o = np.float32(0.02), np.float32(0.01), np.float32(0.06), 40
+    lo, hi = orc.quantized_relux_bounds(6.0, s_o, z_o)
+    assert (lo, hi) == (40, 140) == (z_o, mh.load().mace_hip_quantize_u8(6.0, s_o, z_o))
+    plain = conv_host(ctx, x, f, None, n, h, w, cin, cout, s_in, 128, s_f, 128, 1.0, s_o, z_o)
+    fused = conv_host(ctx, x, f, None, n, h, w, cin, cout, s_in, 128, s_f, 128, 1.0, s_o, z_o, lo, hi)
+    np.testing.assert_array_equal(fused, np.clip(plain, lo, hi))
+    assert (plain < lo).any() and (plain > hi).any()
+
+
+def test_conv1x1_q8_errors(ctx):
+    z = np.zeros(64, np.uint8)
+    # filter_scale * input_scale / out_scale must lie in (0,1) (quantize.h:120)
+    st = ctx.status("mace_hip_conv1x1_q8_nhwc_host", ptr(z), ptr(z), None, 1, 2, 2, 4, 4, 1.0, 0,
+                    1.0, 0, 1.0, 0.5, 0, 0, 255, ptr(z))
+    assert st == mh.INVALID_ARGS and "multiplier" in ctx.last_error()

@@ -1,0 +1,166 @@
+"""fp32 Gemm / Gemv / Conv2D-1x1 on the GPU vs the CPU oracle.  Tolerance is the reference's
+own for this comparison (matmul_test.cc:142-143): |got - want| <= 1e-2 + 1e-4 * |want|,
+checked against both the binary32 serial oracle and the binary64-accumulated one; the
+BASELINE bound (1e-4 relative error) is asserted on the normwise relative error."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from mace_amd import lib as mh
+from oracle import mace_oracle as orc
+from gpu_util import Dev, as_major, c_, ptr
+
+pytestmark = pytest.mark.gpu
+R, Cm = mh.ROW_MAJOR, mh.COL_MAJOR
+GOLDEN = json.load(open(os.path.join(os.path.dirname(__file__), "golden",
+                                     "reference_vectors.json")))
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = mh.Context(0)
+    yield c
+    c.close()
+
+
+def near(got, want):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    assert np.all(np.abs(got - want) <= 1e-2 + 1e-4 * np.abs(want))
+
+
+def gemm_host(ctx, l, r, batch, rows, cols, depth, lm, rm, om, lb, rb):
+    out = np.empty(batch * rows * cols, np.float32)
+    ctx.call("mace_hip_gemm_f32_host", ptr(c_(l, np.float32)), ptr(c_(r, np.float32)), batch,
+             rows, cols, depth, lm, rm, om, int(lb), int(rb), ptr(out))
+    return out
+
+
+GEMM_CASES = [(1, 47, 69, 37, lm, rm, om, True, True)
+              for lm in (R, Cm) for rm in (R, Cm) for om in (R, Cm)]
+GEMM_CASES += [(3, 47, 69, 37, lm, rm, om, True, True)
+               for lm in (R, Cm) for rm in (R, Cm) for om in (R, Cm)]
+GEMM_CASES += [(3, 47, 69, 37, R, R, R, True, False), (3, 47, 69, 37, R, R, R, False, True),
+               (16, 31, 61, 67, R, Cm, R, True, True), (2, 300, 257, 129, R, R, R, True, True),
+               (1, 1, 5, 1, R, R, R, True, True), (2, 128, 128, 16, Cm, Cm, Cm, True, True)]
+
+
+@pytest.mark.parametrize("batch,rows,cols,depth,lm,rm,om,lb,rb", GEMM_CASES)
+def test_gemm_f32_parity(ctx, batch, rows, cols, depth, lm, rm, om, lb, rb):
+    rng = np.random.default_rng(rows * 1000 + cols + lm * 4 + rm * 2 + om)
+    L = rng.standard_normal(((batch if lb else 1), rows, depth)).astype(np.float32)
+    Rr = rng.standard_normal(((batch if rb else 1), depth, cols)).astype(np.float32)
+    l, r = as_major(L, lm), as_major(Rr, rm)
+    got = gemm_host(ctx, l, r, batch, rows, cols, depth, lm, rm, om, lb, rb)
+    near(got, orc.gemm_f32(l, r, batch, rows, cols, depth, lm, rm, om, lb, rb))
+    near(got, orc.gemm_f32(l, r, batch, rows, cols, depth, lm, rm, om, lb, rb, acc64=True))
+
+
+@pytest.mark.parametrize("case", GOLDEN["matmul_f32"], ids=lambda c: c["source"][-20:])
+def test_gemm_f32_reference_goldens(ctx, case):
+    """matmul_test.cc:55-72 through the transpose-form entry point, as MatMulOp calls it."""
+    a = np.array(case["a"], np.float32)
+    b = np.array(case["b"], np.float32)
+    batch, lr, lc = case["a_shape"]
+    _, rr, rc = case["b_shape"]
+    d = Dev()
+    t, p = d.empty(batch * lr * rc, np.float32)
+    da, db = d.put(a), d.put(b)
+    d.sync()
+    ctx.call("mace_hip_gemm_f32_transpose", da, db, batch, lr, lc, rr, rc, 0, 0, 0, 1, 1, p)
+    ctx.sync()
+    np.testing.assert_allclose(t.cpu().numpy(), np.array(case["c"], np.float32), rtol=1e-5,
+                               atol=1e-8)
+    # inconsistent depth is the reference's CHECK failure (ref/gemm.cc:127-131)
+    assert ctx.status("mace_hip_gemm_f32_transpose", da, db, batch, lr, lc, rr + 1, rc, 0, 0, 0,
+                      1, 1, p) == mh.INVALID_ARGS
+
+
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_gemm_f32_config2(ctx, ta, tb):
+    """BASELINE config 2 at batch 4, 512^3 (the 1024^3 size runs in the benchmark; the
+    scalar oracle needs ~1 s per 512^3 batch): N(0,1), all four transpose combinations,
+    plus one non-batched lhs."""
+    rng = np.random.default_rng(2)
+    b, n = 4, 512
+    A = rng.standard_normal((b, n, n)).astype(np.float32)
+    B = rng.standard_normal((b, n, n)).astype(np.float32)
+    d = Dev()
+    t, p = d.empty(b * n * n, np.float32)
+    dA, dB = d.put(A), d.put(B)
+    d.sync()
+    ctx.call("mace_hip_gemm_f32_transpose", dA, dB, b, n, n, n, n, ta, tb, 0, 1, 1, p)
+    ctx.sync()
+    got = t.cpu().numpy().copy()
+    lm, rm = (Cm if ta else R), (Cm if tb else R)
+    want = orc.gemm_f32(A, B, b, n, n, n, lm, rm, R)
+    want64 = orc.gemm_f32(A, B, b, n, n, n, lm, rm, R, acc64=True)
+    near(got, want)
+    near(got, want64)
+    rel = np.linalg.norm(got.astype(np.float64) - want64) / np.linalg.norm(want64)
+    assert rel <= 1e-4, rel
+    if ta == 0 and tb == 0:
+        ctx.call("mace_hip_gemm_f32_transpose", dA, dB, b, n, n, n, n, 0, 0, 0, 0, 1, p)
+        ctx.sync()
+        near(t.cpu().numpy(), orc.gemm_f32(A[0], B, b, n, n, n, R, R, R, False, True, acc64=True))
+
+
+GEMV_CASES = [(1, 16, 4, True, True), (1, 16, 256, True, True), (2, 16, 256, True, True),
+              (3, 63, 257, True, True), (2, 16, 256, False, True), (3, 63, 257, False, True),
+              (2, 16, 256, True, False), (3, 63, 257, True, False), (1, 253, 30001, False, True),
+              (2, 300, 253, True, True)]
+
+
+@pytest.mark.parametrize("batch,h,w,lb,rb", GEMV_CASES)
+def test_gemv_f32_parity(ctx, batch, h, w, lb, rb):
+    rng = np.random.default_rng(h * 7 + w)
+    L = rng.standard_normal(((batch if lb else 1), h, w)).astype(np.float32)
+    x = rng.standard_normal(((batch if rb else 1), w)).astype(np.float32)
+    bias = rng.standard_normal(h).astype(np.float32)
+    for bb in (bias, None):
+        out = np.empty(batch * h, np.float32)
+        ctx.call("mace_hip_gemv_f32_host", ptr(L), ptr(x), ptr(bb), batch, h, w, int(lb),
+                 int(rb), ptr(out))
+        near(out, orc.gemv_f32(L, x, bb, batch, h, w, lb, rb))
+
+
+def test_fully_connected_f32_goldens(ctx):
+    """fully_connected_test.cc:74-93 as Gemv(weight, input, bias, batch, O, I*H*W, false, true)."""
+    for case in GOLDEN["fully_connected_f32"]:
+        x = np.array(case["input"], np.float32)
+        w = np.array(case["weight"], np.float32)
+        bias = np.array(case["bias"], np.float32)
+        batch, o = case["input_shape"][0], case["weight_shape"][0]
+        i = int(np.prod(case["weight_shape"][1:]))
+        out = np.empty(batch * o, np.float32)
+        ctx.call("mace_hip_gemv_f32_host", ptr(w), ptr(x), ptr(bias), batch, o, i, 0, 1, ptr(out))
+        np.testing.assert_allclose(out, np.array(case["output"], np.float32), rtol=1e-5, atol=1e-8)
+
+
+def test_conv1x1_f32_golden_and_random(ctx):
+    g = GOLDEN["conv1x1_f32"]
+    n, h, w, cin, cout = g["n"], g["h"], g["w"], g["cin"], g["cout"]
+    x = np.full((n, cin, h * w), g["input_fill"], np.float32)
+    out = np.empty(n * cout * h * w, np.float32)
+    ctx.call("mace_hip_conv1x1_f32_nchw_host", ptr(x), ptr(np.array(g["filter"], np.float32)),
+             ptr(np.array(g["bias"], np.float32)), n, cin, h * w, cout, mh.ACT_NOOP, 0.0, ptr(out))
+    nhwc = np.transpose(out.reshape(n, cout, h, w), (0, 2, 3, 1)).reshape(-1)
+    np.testing.assert_allclose(nhwc, np.tile(np.array(g["expected_per_pixel"], np.float32),
+                                             n * h * w), rtol=1e-5, atol=1e-8)
+    rng = np.random.default_rng(6)
+    for (n, cin, hw, cout) in ((2, 32, 14 * 14, 64), (3, 130, 49, 70), (1, 5, 30, 2)):
+        x = rng.standard_normal((n, cin, hw)).astype(np.float32)
+        f = rng.standard_normal((cout, cin)).astype(np.float32)
+        b = rng.standard_normal(cout).astype(np.float32)
+        for act, limit, bb in ((mh.ACT_NOOP, 0.0, b), (mh.ACT_RELU, 0.0, b),
+                               (mh.ACT_RELUX, 6.0, b), (mh.ACT_RELUX, 1.5, None)):
+            out = np.empty(n * cout * hw, np.float32)
+            ctx.call("mace_hip_conv1x1_f32_nchw_host", ptr(x), ptr(f), ptr(bb), n, cin, hw, cout,
+                     act, limit, ptr(out))
+            want = orc.conv1x1_f32_nchw(x, f, bb, n, cin, hw, cout, act, limit).reshape(-1)
+            near(out, want)
+            if act != mh.ACT_NOOP:
+                assert out.min() >= 0.0 and (act != mh.ACT_RELUX or out.max() <= limit)
+    assert ctx.status("mace_hip_conv1x1_f32_nchw_host", ptr(x), ptr(f), None, n, cin, hw, cout,
+                      9, 0.0, ptr(out)) == mh.INVALID_ARGS

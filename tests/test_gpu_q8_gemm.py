@@ -1,0 +1,184 @@
+"""uint8 GEMM on the int8 matrix cores vs the CPU oracle: int32 accumulators and requantized
+uint8 outputs bit-exact, every combination of operand / result order, batching on one or
+both sides, aligned and ragged shapes (shape lists from the reference's matmul_test.cc:400-455
+and arm/fp32/gemm_test.cc:98-121)."""
+import numpy as np
+import pytest
+
+from mace_amd import lib as mh
+from oracle import mace_oracle as orc
+from gpu_util import Dev, as_major, c_, ptr
+
+pytestmark = pytest.mark.gpu
+R, Cm = mh.ROW_MAJOR, mh.COL_MAJOR
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = mh.Context(0)
+    yield c
+    c.close()
+
+
+def gemm_i32_host(ctx, l, lo, r, ro, oo, batch, rows, depth, cols, lb, rb, loff, roff):
+    out = np.empty(batch * rows * cols, np.int32)
+    ctx.call("mace_hip_gemm_q8_i32_host", ptr(l), lo, ptr(r), ro, ptr(out), oo, batch, rows,
+             depth, cols, int(lb), int(rb), loff, roff)
+    return out
+
+
+def gemm_u8_host(ctx, l, lo, r, ro, oo, batch, rows, depth, cols, lb, rb, loff, roff, bias,
+                 mult, shift, zp, lo_c=0, hi_c=255):
+    out = np.empty(batch * rows * cols, np.uint8)
+    bias = c_(bias, np.int32)
+    ctx.call("mace_hip_gemm_q8_u8_host", ptr(l), lo, ptr(r), ro, ptr(out), oo, batch, rows,
+             depth, cols, int(lb), int(rb), loff, roff, ptr(bias), mult, shift, zp, lo_c, hi_c)
+    return out
+
+
+def scales_for(depth):
+    """(mult, shift) such that acc / sigma spreads over the uint8 range."""
+    sigma = 74.0 * 74.0 * np.sqrt(max(depth, 1))
+    real = min(0.9, 40.0 / sigma)
+    m, e = orc.quantize_multiplier(real)
+    return m, -e
+
+
+SHAPES = [  # batch, rows, depth, cols, lhs_batched, rhs_batched
+    (1, 64, 128, 32, True, True), (1, 64, 32, 128, True, True), (6, 64, 32, 128, True, True),
+    (1, 47, 37, 69, True, True), (3, 47, 37, 69, True, True), (16, 31, 61, 67, True, True),
+    (6, 31, 61, 67, False, True), (6, 31, 61, 67, True, False),
+    (1, 1, 3000, 256, True, True), (1, 3000, 256, 1, True, True), (3, 128, 256, 1, True, True),
+    (1, 128, 256, 128, True, True),          # BASELINE config 1
+    (1, 300, 512, 260, True, True), (2, 257, 80, 513, True, True), (1, 5, 16, 7, True, True),
+    (1, 1, 1, 1, True, True), (2, 130, 1000, 70, False, False),
+]
+
+
+@pytest.mark.parametrize("batch,rows,depth,cols,lb,rb", SHAPES)
+@pytest.mark.parametrize("lo,ro,oo", [(R, R, R), (R, Cm, R), (Cm, R, R), (Cm, Cm, R),
+                                      (R, Cm, Cm), (Cm, R, Cm), (R, R, Cm), (Cm, Cm, Cm)])
+def test_q8_gemm_parity(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo):
+    rng = np.random.default_rng(rows * 31 + depth * 7 + cols + lo * 4 + ro * 2 + oo)
+    L = rng.integers(0, 256, ((batch if lb else 1), rows, depth), dtype=np.uint8)
+    Rr = rng.integers(0, 256, ((batch if rb else 1), depth, cols), dtype=np.uint8)
+    l, r = as_major(L, lo), as_major(Rr, ro)
+    lzp, rzp = int(rng.integers(0, 256)), int(rng.integers(0, 256))
+    want = orc.q8_gemm_i32(l, r, batch, rows, cols, depth, -lzp, -rzp, lo, ro, oo, lb, rb)
+    got = gemm_i32_host(ctx, l, lo, r, ro, oo, batch, rows, depth, cols, lb, rb, -lzp, -rzp)
+    np.testing.assert_array_equal(got, want)
+    mult, shift = scales_for(depth)
+    bias = rng.integers(-2 ** 15, 2 ** 15, rows).astype(np.int32)
+    for bb, zp, clamp in ((None, 128, (0, 255)), (bias, 3, (0, 255)), (bias, 100, (100, 180))):
+        want8 = orc.q8_gemm_u8(l, r, batch, rows, cols, depth, -128, -128, bb, mult, shift, zp,
+                               clamp[0], clamp[1], lo, ro, oo, lb, rb)
+        got8 = gemm_u8_host(ctx, l, lo, r, ro, oo, batch, rows, depth, cols, lb, rb, -128, -128,
+                            bb, mult, shift, zp, clamp[0], clamp[1])
+        np.testing.assert_array_equal(got8, want8)
+    if rows * cols >= 64:
+        assert len(np.unique(want8)) > 8       # the uint8 check is not vacuous
+
+
+def test_q8_gemm_config1_matmul(ctx):
+    """BASELINE config 1: A [128x256], B [256x128], zero points 128/128/128, scales
+    0.02/0.015/0.05 -> (1649267328, shift 7)."""
+    rng = np.random.default_rng(1)
+    A = rng.integers(0, 256, (128, 256), dtype=np.uint8)
+    B = rng.integers(0, 256, (256, 128), dtype=np.uint8)
+    mult, shift = mh.get_output_multiplier_and_shift(0.02, 0.015, 0.05)
+    assert (mult, shift) == (1649267328, 7) == orc.get_output_multiplier_and_shift(0.02, 0.015, 0.05)
+    want32 = orc.matmul_q8(A, B, 128, 128, out_int32=True)
+    want8 = orc.matmul_q8(A, B, 128, 128, a_scale=0.02, b_scale=0.015, out_scale=0.05, out_zp=128)
+    got32 = gemm_i32_host(ctx, A, R, B, R, R, 1, 128, 256, 128, True, True, -128, -128)
+    got8 = gemm_u8_host(ctx, A, R, B, R, R, 1, 128, 256, 128, True, True, -128, -128, None,
+                        mult, shift, 128)
+    np.testing.assert_array_equal(got32.reshape(128, 128), want32)
+    np.testing.assert_array_equal(got8.reshape(128, 128), want8)
+    assert 0 < (want8 == 0).mean() + (want8 == 255).mean() < 0.9
+
+
+@pytest.mark.parametrize("n,lo,ro,oo", [(1024, R, R, R), (1024, R, Cm, Cm), (2048, R, R, R)])
+def test_q8_gemm_large_device_pointers(ctx, n, lo, ro, oo):
+    """Square GEMMs through the device-pointer entry points (the 256x256 tile path), random
+    zero points, both outputs checked in full against the oracle."""
+    rng = np.random.default_rng(5 + n)
+    A = rng.integers(0, 256, (n, n), dtype=np.uint8)
+    B = rng.integers(0, 256, (n, n), dtype=np.uint8)
+    za, zb, zc = int(rng.integers(120, 137)), int(rng.integers(120, 137)), int(rng.integers(100, 157))
+    l, r = as_major(A, lo), as_major(B, ro)
+    d = Dev()
+    dl, dr = d.put(l), d.put(r)
+    t32, p32 = d.empty(n * n, np.int32)
+    t8, p8 = d.empty(n * n, np.uint8)
+    d.sync()
+    ctx.call("mace_hip_gemm_q8_i32", dl, lo, dr, ro, p32, oo, 1, n, n, n, 1, 1, -za, -zb)
+    mult, shift = scales_for(n)
+    ctx.call("mace_hip_gemm_q8_u8", dl, lo, dr, ro, p8, oo, 1, n, n, n, 1, 1, -za, -zb, None,
+             mult, shift, zc, 0, 255)
+    ctx.sync()
+    want32 = orc.q8_gemm_i32(l, r, 1, n, n, n, -za, -zb, lo, ro, oo)
+    np.testing.assert_array_equal(t32.cpu().numpy(), want32)
+    want8 = orc.output_pipeline_u8(want32, 1, n, n, oo, None, mult, shift, zc)
+    np.testing.assert_array_equal(t8.cpu().numpy(), want8)
+    sat = (want8 == 0).mean() + (want8 == 255).mean()
+    assert sat < 0.5, sat
+
+
+def test_q8_gemm_batched_512(ctx):
+    """BASELINE config 5's batched case at a size the oracle finishes quickly: 8 x 512^3."""
+    rng = np.random.default_rng(9)
+    b, n = 8, 512
+    A = rng.integers(0, 256, (b, n, n), dtype=np.uint8)
+    B = rng.integers(0, 256, (b, n, n), dtype=np.uint8)
+    want = orc.q8_gemm_i32(A, B, b, n, n, n, -17, -240)
+    got = gemm_i32_host(ctx, A, R, B, R, R, b, n, n, n, True, True, -17, -240)
+    np.testing.assert_array_equal(got, want)
+
+
+def test_q8_gemm_freivalds_4096(ctx):
+    """4096^3: the oracle would take minutes, so check C x == A (B x) in int64 for random
+    vectors x (size-independent property), plus 32 full rows exactly."""
+    import torch
+    n = 4096
+    g = torch.Generator(device="cuda").manual_seed(7)
+    A = torch.randint(0, 256, (n, n), dtype=torch.uint8, device="cuda", generator=g)
+    B = torch.randint(0, 256, (n, n), dtype=torch.uint8, device="cuda", generator=g)
+    Cout = torch.empty((n, n), dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()
+    za, zb = 101, 200
+    ctx.call("mace_hip_gemm_q8_i32", A.data_ptr(), R, B.data_ptr(), R, Cout.data_ptr(), R, 1, n,
+             n, n, 1, 1, -za, -zb)
+    ctx.sync()
+    Ad = (A.to(torch.float64) - za)
+    Bd = (B.to(torch.float64) - zb)
+    for seed in (1, 2):
+        x = torch.randint(-8, 9, (n, 1), generator=torch.Generator().manual_seed(seed)).to(
+            device="cuda", dtype=torch.float64)
+        lhs = Cout.to(torch.float64) @ x            # exact: |values| < 2^53
+        rhs = Ad @ (Bd @ x)
+        assert torch.equal(lhs, rhs)
+    rows = np.random.default_rng(7).choice(n, 32, replace=False)
+    a_rows = A[rows].cpu().numpy()
+    want = orc.q8_gemm_i32(a_rows, B.cpu().numpy(), 1, 32, n, n, -za, -zb)
+    np.testing.assert_array_equal(Cout[rows].cpu().numpy().reshape(-1), want)
+
+
+def test_q8_gemm_errors(ctx):
+    z = np.zeros(64, np.uint8)
+    o = np.zeros(64, np.uint8)
+    base = (ptr(z), R, ptr(z), R, ptr(o), R, 1, 8, 8, 8, 1, 1, 0, 0, None)
+    assert ctx.status("mace_hip_gemm_q8_u8_host", *base, 2 ** 30, -1, 0, 0, 255) == mh.INVALID_ARGS
+    assert ctx.status("mace_hip_gemm_q8_u8_host", *base, 2 ** 30, 32, 0, 0, 255) == mh.INVALID_ARGS
+    assert ctx.status("mace_hip_gemm_q8_u8_host", *base, 2 ** 30, 1, 0, 10, 5) == mh.INVALID_ARGS
+    assert ctx.status("mace_hip_gemm_q8_u8_host", ptr(z), 2, ptr(z), R, ptr(o), R, 1, 8, 8, 8, 1,
+                      1, 0, 0, None, 2 ** 30, 1, 0, 0, 255) == mh.INVALID_ARGS
+    assert ctx.status("mace_hip_gemm_q8_u8_host", *base, 2 ** 30, 1, 0, 0, 255) == mh.SUCCESS
+    # allocation failure comes back as OUT_OF_RESOURCES and leaves the context usable
+    big = np.zeros(4096 * 2048, np.uint8)
+    out = np.zeros(4096 * 4096, np.int32)
+    ctx.call("mace_hip_ctx_fail_next_allocs", 1)
+    st = ctx.status("mace_hip_gemm_q8_i32_host", ptr(big), R, ptr(big), R, ptr(out), R, 1, 4096,
+                    2048, 4096, 1, 1, 0, 0)
+    ctx.call("mace_hip_ctx_fail_next_allocs", 0)
+    assert st in (mh.OUT_OF_RESOURCES, mh.SUCCESS)   # SUCCESS only if the arena was already big
+    assert ctx.status("mace_hip_gemm_q8_u8_host", *base, 2 ** 30, 1, 0, 0, 255) == mh.SUCCESS

@@ -1,0 +1,109 @@
+"""uint8 Gemv on the GPU vs the CPU oracle: bit-exact int32 accumulators and uint8 outputs in
+both requantisation flavours (ref/q8/gemv.cc:80-162, arm/q8/gemv.cc:36-171)."""
+import numpy as np
+import pytest
+
+from mace_amd import lib as mh
+from oracle import mace_oracle as orc
+from gpu_util import Dev, c_, ptr
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = mh.Context(0)
+    yield c
+    c.close()
+
+
+def run_host(ctx, L, x, bias, batch, h, w, lb, rb, lzp, rzp, u8, scales=None, ozp=0, mode=0):
+    L, x, bias = c_(L, np.uint8), c_(x, np.uint8), c_(bias, np.int32)
+    if u8:
+        out = np.empty(batch * h, np.uint8)
+        ctx.call("mace_hip_gemv_q8_u8_host", ptr(L), ptr(x), ptr(bias), batch, h, w, int(lb),
+                 int(rb), lzp, rzp, scales[0], scales[1], scales[2], ozp, mode, ptr(out))
+    else:
+        out = np.empty(batch * h, np.int32)
+        ctx.call("mace_hip_gemv_q8_i32_host", ptr(L), ptr(x), ptr(bias), batch, h, w, int(lb),
+                 int(rb), lzp, rzp, ptr(out))
+    return out
+
+
+# arm/q8/gemv_test.cc:179-201 plus wider / odd / multi-pass shapes
+CASES = [(1, 16, 4, True, True), (1, 16, 256, True, True), (2, 16, 256, True, True),
+         (3, 63, 257, True, True), (2, 16, 256, False, True), (3, 63, 257, False, True),
+         (2, 16, 256, True, False), (3, 63, 257, True, False),
+         (1, 129, 4096, False, True), (8, 70, 4096 + 16, False, True),
+         (11, 37, 1040, False, True), (5, 33, 8192, False, True), (4, 5, 30001, False, True),
+         (2, 3, 1, False, True), (3, 7, 48, False, False)]
+
+
+@pytest.mark.parametrize("batch,h,w,lb,rb", CASES)
+def test_q8_gemv_parity(ctx, batch, h, w, lb, rb):
+    rng = np.random.default_rng(1000 + batch * 7 + h * 3 + w)
+    L = rng.integers(0, 256, ((batch if lb else 1), h, w), dtype=np.uint8)
+    x = rng.integers(0, 256, ((batch if rb else 1), w), dtype=np.uint8)
+    bias = rng.integers(-2 ** 15, 2 ** 15, h).astype(np.int32)
+    for lzp, rzp in ((0, 0), (23, 45), (127, 128), (255, 255)):
+        for bb in (bias, None):
+            want = orc.q8_gemv_i32(L, x, bb, batch, h, w, lzp, rzp, lb, rb)
+            got = run_host(ctx, L, x, bb, batch, h, w, lb, rb, lzp, rzp, False)
+            np.testing.assert_array_equal(got, want)
+    # uint8: scale so that the outputs spread over the range instead of saturating
+    sigma = 74.0 * 74.0 * np.sqrt(w)
+    scales = (np.float32(0.01), np.float32(0.02), np.float32(0.0002 * sigma / 40.0))
+    for ozp in (0, 57, 128):
+        for mode in (mh.REQUANT_REF, mh.REQUANT_NEON):
+            want = orc.q8_gemv_u8(L, x, bias, batch, h, w, 127, 128, *scales, ozp, mode, lb, rb)
+            got = run_host(ctx, L, x, bias, batch, h, w, lb, rb, 127, 128, True, scales, ozp, mode)
+            np.testing.assert_array_equal(got, want)
+    assert len(np.unique(got)) > min(10, h // 2)
+
+
+def test_q8_gemv_config_4096(ctx):
+    """BASELINE config: weight [4096 x 4096], batch 1 and 8, weight_zp 127, input_zp 128,
+    int32 bias in [-2^15, 2^15]; device-pointer path."""
+    rng = np.random.default_rng(3)
+    H = W = 4096
+    Wt = rng.integers(0, 256, (H, W), dtype=np.uint8)
+    bias = rng.integers(-2 ** 15, 2 ** 15, H).astype(np.int32)
+    d = Dev()
+    dW, dB = d.put(Wt), d.put(bias)
+    for batch in (1, 8):
+        x = rng.integers(0, 256, (batch, W), dtype=np.uint8)
+        dx = d.put(x)
+        t32, p32 = d.empty(batch * H, np.int32)
+        d.sync()
+        ctx.call("mace_hip_gemv_q8_i32", dW, dx, dB, batch, H, W, 0, 1, 127, 128, p32)
+        ctx.sync()
+        want = orc.q8_gemv_i32(Wt, x, bias, batch, H, W, 127, 128)
+        np.testing.assert_array_equal(t32.cpu().numpy()[:batch * H], want)
+        for ozp in (0, 128):
+            for mode in (mh.REQUANT_REF, mh.REQUANT_NEON):
+                t8, p8 = d.empty(batch * H, np.uint8)
+                d.sync()
+                ctx.call("mace_hip_gemv_q8_u8", dW, dx, dB, batch, H, W, 0, 1, 127, 128,
+                         0.01, 0.02, 1.75, ozp, mode, p8)
+                ctx.sync()
+                want8 = orc.q8_gemv_u8(Wt, x, bias, batch, H, W, 127, 128, 0.01, 0.02, 1.75,
+                                       ozp, mode)
+                np.testing.assert_array_equal(t8.cpu().numpy()[:batch * H], want8)
+        assert len(np.unique(want8)) > 50
+
+
+def test_q8_gemv_errors(ctx):
+    z = np.zeros(16, np.uint8)
+    o = np.zeros(4, np.uint8)
+    a = (ptr(z), ptr(z), None, 1, 4, 4, 0, 1, 0, 0)
+    # out.scale must be > 0 (ref/q8/gemv.cc:100)
+    assert ctx.status("mace_hip_gemv_q8_u8_host", *a, 0.5, 0.5, 0.0, 0, 0, ptr(o)) == mh.INVALID_ARGS
+    assert "scale" in ctx.last_error()
+    # NEON flavour CHECKs 0 < multiplier < 1 (arm/q8/gemv.cc:55-63 via quantize.h:120)
+    assert ctx.status("mace_hip_gemv_q8_u8_host", *a, 2.0, 2.0, 1.0, 0, 1, ptr(o)) == mh.INVALID_ARGS
+    # REF flavour does not
+    assert ctx.status("mace_hip_gemv_q8_u8_host", *a, 2.0, 2.0, 1.0, 0, 0, ptr(o)) == mh.SUCCESS
+    assert ctx.status("mace_hip_gemv_q8_u8_host", *a, 0.5, 0.5, 1.0, 0, 7, ptr(o)) == mh.INVALID_ARGS
+    # empty problems succeed and write nothing
+    assert ctx.status("mace_hip_gemv_q8_i32_host", ptr(z), ptr(z), None, 0, 4, 4, 0, 1, 0, 0,
+                      ptr(np.zeros(1, np.int32))) == mh.SUCCESS
