@@ -1,0 +1,230 @@
+#!/usr/bin/env python3
+"""Benchmark of the matrix-multiplication hot path on ONE MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one pass of the quantized MatMul hot path over one synthetic batch: the uint8 GEMM
+M = N = K = 8192 (MatMul defaults: A RowMajor, B RowMajor, result RowMajor), int32
+accumulation, fixed-point requantization to uint8 -- everything mace_hip_gemm_q8_u8 launches
+(operand repack, correction vectors, the MFMA kernel with its fused epilogue), inputs already
+resident in HBM.  `value` is 2*M*N*K / step time in TOPS.
+
+`roofline` describes the dominant kernel (the int8 MFMA GEMM kernel alone), timed with HIP
+events recorded on the library's stream around that kernel.  `gemv` reports the second half of
+the metric: the uint8 Gemv 4096x4096 in GB/s of algorithmic bytes, with the weights both
+re-read from a rotating set larger than the last-level cache (the HBM figure) and left
+resident.  `cpu_baseline` times the CPU oracle (a port of the reference's CPU path) on a
+bounded sample of the same GEMM on the host cores and, while at it, checks the GPU rows
+against it bit for bit.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+METRIC = "uint8 GEMM int8-TOPS + q8 Gemv HBM GB/s, % of MI355X roofline, 1 GPU"
+PEAK_INT8_TOPS = 5000.0      # MI355X dense int8 MFMA, published
+PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, published
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--size", type=int, default=8192, help="M = N = K of the uint8 GEMM")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-gemv", action="store_true")
+    ap.add_argument("--cpu-rows", type=int, default=8192,
+                    help="rows of A the CPU baseline multiplies by the whole of B")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        log("bench.py measures one GPU: the path needs no exchange between GPUs, and this "
+            "build launches nothing on a second one.  Run with --gpus 1.")
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from mace_amd import lib as mh
+
+    if not torch.cuda.is_available():
+        log("bench.py needs a GPU (no CPU fallback exists)")
+        sys.exit(1)
+    torch.cuda.set_device(0)
+    ctx = mh.Context(0)
+    arch, cus, lds = ctx.device_info()
+    log("device %s, %d CUs, %d B LDS/workgroup" % (arch, cus, lds))
+
+    n = args.size
+    g = torch.Generator(device="cuda").manual_seed(5)
+    A = torch.randint(0, 256, (n, n), dtype=torch.uint8, device="cuda", generator=g)
+    B = torch.randint(0, 256, (n, n), dtype=torch.uint8, device="cuda", generator=g)
+    out8 = torch.empty((n, n), dtype=torch.uint8, device="cuda")
+    za, zb, zc = 131, 122, 128
+    # real multiplier ~ 40 / sigma(acc): outputs spread over the uint8 range, few saturate
+    sigma = 74.0 * 74.0 * (n ** 0.5)
+    mult, e = mh.quantize_multiplier(min(0.9, 40.0 / sigma))
+    shift = -e
+    torch.cuda.synchronize()
+
+    def step():
+        ctx.call("mace_hip_gemm_q8_u8", A.data_ptr(), mh.ROW_MAJOR, B.data_ptr(), mh.ROW_MAJOR,
+                 out8.data_ptr(), mh.ROW_MAJOR, 1, n, n, n, 1, 1, -za, -zb, None, mult, shift, zc,
+                 0, 255)
+
+    for _ in range(args.warmup):
+        step()
+    ctx.sync()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ctx.timer_start()
+    for _ in range(args.steps):
+        step()
+    ev_ms = ctx.timer_stop()
+    ctx.sync()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms_per_step = wall_ms / args.steps
+    ops = 2.0 * n * n * n
+    value = ops / (ms_per_step * 1e-3) / 1e12
+    log("whole path: %.3f ms/step wall (%.3f ms by events) -> %.1f TOPS"
+        % (ms_per_step, ev_ms / args.steps, value))
+
+    # dominant kernel alone, HIP events on the launch stream around that kernel
+    ctx.profile(True)
+    kms = []
+    for _ in range(args.steps):
+        step()
+        kms.append(ctx.last_kernel_ms())
+    ctx.profile(False)
+    k_avg = sum(kms) / len(kms)
+    achieved = ops / (k_avg * 1e-3) / 1e12
+    log("dominant kernel: avg %.3f ms (min %.3f) -> %.1f TOPS = %.1f%% of %.0f"
+        % (k_avg, min(kms), achieved, 100 * achieved / PEAK_INT8_TOPS, PEAK_INT8_TOPS))
+    sat = float(((out8 == 0) | (out8 == 255)).float().mean().item())
+
+    result = {
+        "metric": METRIC, "value": round(value, 2), "unit": "TOPS", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8",
+        "data": "synthetic",
+        "config": {"workload": "q8_matmul_%dx%dx%d_u8out" % (n, n, n), "M": n, "N": n, "K": n,
+                   "lhs_order": "RowMajor", "rhs_order": "RowMajor", "out_order": "RowMajor",
+                   "zero_points": [za, zb, zc], "multiplier": mult, "right_shift": shift,
+                   "saturated_fraction": round(sat, 4), "device": arch, "cus": cus},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_INT8_TOPS,
+                     "unit": "TOP/s", "frac": round(achieved / PEAK_INT8_TOPS, 4),
+                     "traffic": None, "kernel": "q8_gemm_kernel<2,2,4,4,uint8_t>",
+                     "kernel_ms_avg": round(k_avg, 4), "kernel_ms_min": round(min(kms), 4),
+                     "ops_per_launch": ops},
+    }
+
+    if not args.no_gemv:
+        result["gemv"] = bench_gemv(ctx, mh, torch, args)
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(np, torch, A, B, out8, n, za, zb, zc, mult, shift,
+                                              args.cpu_rows)
+    ctx.close()
+    print(json.dumps(result), flush=True)
+
+
+def bench_gemv(ctx, mh, torch, args):
+    """uint8 Gemv 4096x4096 (FullyConnected), batch 1 and 8.  Algorithmic bytes per launch:
+    H*W weights + B*W input + 4*H bias + B*H output."""
+    H = W = 4096
+    nbuf = 40                                    # 40 x 16 MiB = 640 MiB > 256 MiB last-level cache
+    g = torch.Generator(device="cuda").manual_seed(3)
+    weights = torch.randint(0, 256, (nbuf, H, W), dtype=torch.uint8, device="cuda", generator=g)
+    bias = torch.randint(-2 ** 15, 2 ** 15, (H,), dtype=torch.int32, device="cuda", generator=g)
+    out = {}
+    for batch in (1, 8):
+        x = torch.randint(0, 256, (batch, W), dtype=torch.uint8, device="cuda", generator=g)
+        y = torch.empty((batch, H), dtype=torch.uint8, device="cuda")
+        torch.cuda.synchronize()
+        nbytes = H * W + batch * W + 4 * H + batch * H
+
+        def call(i):
+            ctx.call("mace_hip_gemv_q8_u8", weights[i].data_ptr(), x.data_ptr(), bias.data_ptr(),
+                     batch, H, W, 0, 1, 127, 128, 0.01, 0.02, 1.75, 128, mh.REQUANT_NEON,
+                     y.data_ptr())
+
+        res = {"bytes_per_launch": nbytes}
+        for name, rotate in (("hbm", True), ("cache_resident", False)):
+            for i in range(nbuf):
+                call(i if rotate else 0)
+            ctx.profile(True)
+            ks = []
+            for i in range(3 * nbuf):
+                call(i % nbuf if rotate else 0)
+                ks.append(ctx.last_kernel_ms())
+            ctx.profile(False)
+            # back-to-back launches, no host sync in between: what a serving loop sees
+            reps = 10 * nbuf
+            ctx.sync()
+            ctx.timer_start()
+            for i in range(reps):
+                call(i % nbuf if rotate else 0)
+            loop_ms = ctx.timer_stop() / reps
+            k_avg = sum(ks) / len(ks)
+            gbs = nbytes / (k_avg * 1e-3) / 1e9
+            res[name] = {"kernel_us_avg": round(k_avg * 1e3, 3),
+                         "kernel_us_min": round(min(ks) * 1e3, 3),
+                         "GBps": round(gbs, 1), "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBS, 4),
+                         "back_to_back_us": round(loop_ms * 1e3, 3),
+                         "back_to_back_GBps": round(nbytes / (loop_ms * 1e-3) / 1e9, 1)}
+            log("gemv batch %d %s: kernel %.2f us -> %.0f GB/s (%.1f%% of HBM peak); "
+                "back-to-back %.2f us" % (batch, name, k_avg * 1e3, gbs,
+                                          100 * gbs / PEAK_HBM_GBS, loop_ms * 1e3))
+        out["batch%d" % batch] = res
+    hb = out["batch1"]["hbm"]
+    out["roofline"] = {"bound": "hbm", "achieved": hb["GBps"], "peak": PEAK_HBM_GBS,
+                       "unit": "GB/s", "frac": hb["frac_of_hbm_peak"], "traffic": None,
+                       "kernel": "q8_gemv_kernel<1,true,uint8_t>"}
+    return out
+
+
+def cpu_baseline(np, torch, A, B, out8, n, za, zb, zc, mult, shift, rows):
+    """The oracle (a port of the reference's CPU path: exact integer GEMM standing in for
+    gemmlowp + the fixed-point output pipeline) on `rows` rows of A times the whole of B, on
+    the host cores.  The same rows of the GPU result are compared with it."""
+    from oracle import mace_oracle as orc
+    try:
+        cores = len(os.sched_getaffinity(0))
+    except AttributeError:
+        cores = os.cpu_count() or 1
+    cores = max(1, min(cores, 16))
+    rows = min(rows, n)
+    a = A[:rows].cpu().numpy()
+    b = B.cpu().numpy()
+    t0 = time.perf_counter()
+    want = orc.q8_gemm_u8(a, b, 1, rows, n, n, -za, -zb, None, mult, shift, zc, 0, 255,
+                          nthreads=cores)
+    dt = time.perf_counter() - t0
+    got = out8[:rows].cpu().numpy().reshape(-1)
+    exact = bool(np.array_equal(got, want))
+    tops = 2.0 * rows * n * n / dt / 1e12
+    log("cpu baseline: %d x %d x %d on %d threads in %.2f s -> %.4f TOPS; GPU rows bit-exact: %s"
+        % (rows, n, n, cores, dt, tops, exact))
+    if not exact:
+        log("ERROR: GPU result differs from the CPU oracle")
+        sys.exit(3)
+    return {"value": round(tops, 5), "unit": "TOPS", "cores": cores, "kind": "port",
+            "sample": "rows 0..%d of A times all of B (%d x %d x %d), oracle/mace_oracle.c "
+                      "q8_gemm_u8, gcc -O2 -fopenmp, %.2f s" % (rows - 1, rows, n, n, dt),
+            "gpu_rows_bit_exact": exact}
+
+
+if __name__ == "__main__":
+    main()

@@ -66,6 +66,12 @@ int mace_hip_device_info(mace_hip_ctx *ctx, char *arch, size_t arch_len, int *cu
 /* HIP-event stopwatch on the context's stream (kernel time, not host time). */
 int mace_hip_timer_start(mace_hip_ctx *ctx);
 int mace_hip_timer_stop(mace_hip_ctx *ctx, float *elapsed_ms);
+/* Dominant-kernel stopwatch (the counterpart of the per-op timing SerialNet::Run records into
+ * RunMetadata, mace/core/net/serial_net.cc:122-168): while enabled, every GEMM / Gemv call
+ * brackets its main kernel (not the repack or correction-vector passes) with HIP events on
+ * the context's stream; last_kernel_ms waits for that kernel and returns its duration. */
+int mace_hip_profile_enable(mace_hip_ctx *ctx, int on);
+int mace_hip_profile_last_kernel_ms(mace_hip_ctx *ctx, float *elapsed_ms);
 /* Test hook, the counterpart of MACE_RUNTIME_FAILURE_RATIO
  * (mace/core/runtime_failure_mock.cc:24-48): the next n arena allocations fail. */
 int mace_hip_ctx_fail_next_allocs(mace_hip_ctx *ctx, int n);

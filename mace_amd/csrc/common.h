@@ -13,6 +13,9 @@ struct mace_hip_ctx {
   hipStream_t own_stream = nullptr;
   hipStream_t stream = nullptr;     // own_stream or a borrowed one
   hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+  hipEvent_t ev_k0 = nullptr, ev_k1 = nullptr;   // dominant-kernel stopwatch
+  int prof_on = 0;
+  int prof_valid = 0;
   // grow-only device arena; offsets handed out per call by ArenaScope
   char *arena = nullptr;
   size_t arena_bytes = 0;
@@ -45,6 +48,19 @@ int mh_fail(mace_hip_ctx *ctx, int code, const char *fmt, ...);
   do {                                                                               \
     int s__ = (expr);                                                                \
     if (s__ != MACE_HIP_SUCCESS) return s__;                                         \
+  } while (0)
+
+// Brackets a kernel launch with the dominant-kernel stopwatch when profiling is enabled.
+#define MH_PROF_BEGIN(ctx)                                                           \
+  do {                                                                               \
+    if ((ctx)->prof_on) MH_HIP((ctx), hipEventRecord((ctx)->ev_k0, (ctx)->stream));  \
+  } while (0)
+#define MH_PROF_END(ctx)                                                             \
+  do {                                                                               \
+    if ((ctx)->prof_on) {                                                            \
+      MH_HIP((ctx), hipEventRecord((ctx)->ev_k1, (ctx)->stream));                    \
+      (ctx)->prof_valid = 1;                                                         \
+    }                                                                                \
   } while (0)
 
 // Arena: every call that needs scratch opens a scope, takes aligned slices and lets the

@@ -71,7 +71,8 @@ int mace_hip_ctx_create(int device, mace_hip_ctx **out) {
   if (hipSetDevice(device) != hipSuccess || hipGetDeviceProperties(&prop, device) != hipSuccess ||
       hipStreamCreate(&ctx->own_stream) != hipSuccess ||
       hipEventCreate(&ctx->ev_start) != hipSuccess ||
-      hipEventCreate(&ctx->ev_stop) != hipSuccess) {
+      hipEventCreate(&ctx->ev_stop) != hipSuccess ||
+      hipEventCreate(&ctx->ev_k0) != hipSuccess || hipEventCreate(&ctx->ev_k1) != hipSuccess) {
     (void)hipGetLastError();
     delete ctx;
     return MACE_HIP_RUNTIME_ERROR;
@@ -99,6 +100,8 @@ int mace_hip_ctx_destroy(mace_hip_ctx *ctx) {
   if (ctx->arena) (void)hipFree(ctx->arena);
   (void)hipEventDestroy(ctx->ev_start);
   (void)hipEventDestroy(ctx->ev_stop);
+  (void)hipEventDestroy(ctx->ev_k0);
+  (void)hipEventDestroy(ctx->ev_k1);
   (void)hipStreamDestroy(ctx->own_stream);
   delete ctx;
   return MACE_HIP_SUCCESS;
@@ -139,6 +142,21 @@ int mace_hip_timer_stop(mace_hip_ctx *ctx, float *elapsed_ms) {
   MH_HIP(ctx, hipEventRecord(ctx->ev_stop, ctx->stream));
   MH_HIP(ctx, hipEventSynchronize(ctx->ev_stop));
   MH_HIP(ctx, hipEventElapsedTime(elapsed_ms, ctx->ev_start, ctx->ev_stop));
+  return MACE_HIP_SUCCESS;
+}
+
+int mace_hip_profile_enable(mace_hip_ctx *ctx, int on) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  ctx->prof_on = on ? 1 : 0;
+  ctx->prof_valid = 0;
+  return MACE_HIP_SUCCESS;
+}
+
+int mace_hip_profile_last_kernel_ms(mace_hip_ctx *ctx, float *elapsed_ms) {
+  if (!ctx || !elapsed_ms) return MACE_HIP_INVALID_ARGS;
+  MH_CHECK(ctx, ctx->prof_valid, "no kernel has been timed since profiling was enabled");
+  MH_HIP(ctx, hipEventSynchronize(ctx->ev_k1));
+  MH_HIP(ctx, hipEventElapsedTime(elapsed_ms, ctx->ev_k0, ctx->ev_k1));
   return MACE_HIP_SUCCESS;
 }
 

@@ -216,10 +216,12 @@ int mh_f32_gemm(mace_hip_ctx *ctx, const float *lhs, const float *rhs, int64_t b
   dim3 grid((unsigned)tiles, 1, (unsigned)batch), block(256);
   const bool lk = lhs_major == MACE_HIP_ROW_MAJOR;   // depth contiguous
   const bool rk = rhs_major == MACE_HIP_COL_MAJOR;
+  MH_PROF_BEGIN(ctx);
   if (lk && rk) hipLaunchKernelGGL((f32_gemm_kernel<true, true>), grid, block, 0, ctx->stream, p);
   else if (lk) hipLaunchKernelGGL((f32_gemm_kernel<true, false>), grid, block, 0, ctx->stream, p);
   else if (rk) hipLaunchKernelGGL((f32_gemm_kernel<false, true>), grid, block, 0, ctx->stream, p);
   else hipLaunchKernelGGL((f32_gemm_kernel<false, false>), grid, block, 0, ctx->stream, p);
+  MH_PROF_END(ctx);
   MH_HIP(ctx, hipGetLastError());
   return MACE_HIP_SUCCESS;
 }
@@ -269,7 +271,9 @@ int mace_hip_gemv_f32(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
   F32GemvParams p{lhs, rhs, bias, out, lhs_batched ? height * width : 0,
                   rhs_batched ? width : 0, (int)height, (int)width};
   dim3 grid((unsigned)((height + 3) / 4), (unsigned)batch);
+  MH_PROF_BEGIN(ctx);
   hipLaunchKernelGGL(f32_gemv_kernel, grid, dim3(256), 0, ctx->stream, p);
+  MH_PROF_END(ctx);
   MH_HIP(ctx, hipGetLastError());
   return MACE_HIP_SUCCESS;
 }

@@ -119,21 +119,39 @@ __global__ __launch_bounds__(WX *WY * 64) void q8_gemm_kernel(GemmParams p) {
 
   v4i rx[CHUNKS_X], ry[CHUNKS_Y];
   const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
-  const v4i zero4 = {0, 0, 0, 0};
 
-  auto load_global = [&](int k0) {
+  // Loads only issue here; the 0x80 flip is applied on the way to LDS so that nothing
+  // consumes the data (and waits for it) before the MFMA work of the current tile is issued.
+  auto load_full = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < CHUNKS_X; ++i)
-      rx[i] = (k0 + kx[i] < p.K) ? (*(const v4i *)(gx[i] + k0) ^ flip) : zero4;
+    for (int i = 0; i < CHUNKS_X; ++i) rx[i] = *(const v4i *)(gx[i] + k0);
 #pragma unroll
-    for (int i = 0; i < CHUNKS_Y; ++i)
-      ry[i] = (k0 + ky[i] < p.K) ? (*(const v4i *)(gy[i] + k0) ^ flip) : zero4;
+    for (int i = 0; i < CHUNKS_Y; ++i) ry[i] = *(const v4i *)(gy[i] + k0);
+  };
+  // Last, partial tile (K % BK != 0): chunks at or beyond K read offset 0 of their row (always
+  // valid) and are replaced by 0x80 bytes, which the flip turns into zeros.  Branch-free.
+  auto load_tail = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < CHUNKS_X; ++i) {
+      const bool ok = k0 + kx[i] < p.K;
+      const v4i v = *(const v4i *)(gx[i] + (ok ? k0 : -kx[i]));
+      const int m = ok ? -1 : 0;
+      rx[i] = (v & v4i{m, m, m, m}) | (flip & v4i{~m, ~m, ~m, ~m});
+    }
+#pragma unroll
+    for (int i = 0; i < CHUNKS_Y; ++i) {
+      const bool ok = k0 + ky[i] < p.K;
+      const v4i v = *(const v4i *)(gy[i] + (ok ? k0 : -ky[i]));
+      const int m = ok ? -1 : 0;
+      ry[i] = (v & v4i{m, m, m, m}) | (flip & v4i{~m, ~m, ~m, ~m});
+    }
   };
   auto store_lds = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < CHUNKS_X; ++i) *(v4i *)(lds + buf * BUF_BYTES + lx[i]) = rx[i];
+    for (int i = 0; i < CHUNKS_X; ++i) *(v4i *)(lds + buf * BUF_BYTES + lx[i]) = rx[i] ^ flip;
 #pragma unroll
-    for (int i = 0; i < CHUNKS_Y; ++i) *(v4i *)(lds + buf * BUF_BYTES + Y_OFF + ly[i]) = ry[i];
+    for (int i = 0; i < CHUNKS_Y; ++i)
+      *(v4i *)(lds + buf * BUF_BYTES + Y_OFF + ly[i]) = ry[i] ^ flip;
   };
 
   v16i acc[FX][FY];
@@ -150,30 +168,43 @@ __global__ __launch_bounds__(WX *WY * 64) void q8_gemm_kernel(GemmParams p) {
   const int fx_base = wx * FX * 32 * LDS_ROW + frag_off;
   const int fy_base = wy * FY * 32 * LDS_ROW + frag_off;
 
-  const int nk = (p.K + BK - 1) / BK;
-  load_global(0);
-  store_lds(0);
-  __syncthreads();
-  for (int kt = 0; kt < nk; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < nk) load_global((kt + 1) * BK);
+  auto mfma_step = [&](int buf, int ks) {
+    v4i a[FX], bf[FY];
 #pragma unroll
-    for (int ks = 0; ks < BK / 32; ++ks) {
-      v4i a[FX], bf[FY];
+    for (int i = 0; i < FX; ++i)
+      a[i] = *(const v4i *)(lds + buf * BUF_BYTES + fx_base + i * 32 * LDS_ROW + ks * 32);
 #pragma unroll
-      for (int i = 0; i < FX; ++i)
-        a[i] = *(const v4i *)(lds + buf * BUF_BYTES + fx_base + i * 32 * LDS_ROW + ks * 32);
+    for (int j = 0; j < FY; ++j)
+      bf[j] = *(const v4i *)(lds + buf * BUF_BYTES + Y_OFF + fy_base + j * 32 * LDS_ROW + ks * 32);
+#pragma unroll
+    for (int i = 0; i < FX; ++i)
 #pragma unroll
       for (int j = 0; j < FY; ++j)
-        bf[j] = *(const v4i *)(lds + buf * BUF_BYTES + Y_OFF + fy_base + j * 32 * LDS_ROW + ks * 32);
-#pragma unroll
-      for (int i = 0; i < FX; ++i)
-#pragma unroll
-        for (int j = 0; j < FY; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], bf[j], acc[i][j], 0, 0, 0);
-    }
-    if (kt + 1 < nk) store_lds(buf ^ 1);
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], bf[j], acc[i][j], 0, 0, 0);
+  };
+
+  // full tiles: global loads of tile kt+1 are in flight while tile kt is multiplied
+  const int nfull = p.K / BK;
+  if (nfull > 0) {
+    load_full(0);
+    store_lds(0);
     __syncthreads();
+    for (int kt = 0; kt < nfull; ++kt) {
+      const int buf = kt & 1;
+      if (kt + 1 < nfull) load_full((kt + 1) * BK);
+#pragma unroll
+      for (int ks = 0; ks < BK / 32; ++ks) mfma_step(buf, ks);
+      if (kt + 1 < nfull) store_lds(buf ^ 1);
+      __syncthreads();
+    }
+  }
+  // partial last tile
+  const int ktail = p.K - nfull * BK;
+  if (ktail > 0) {
+    load_tail(nfull * BK);
+    store_lds(0);
+    __syncthreads();
+    for (int ks = 0; ks < (ktail + 31) / 32; ++ks) mfma_step(0, ks);
   }
 
   // epilogue: accumulator register r of a 32x32 tile holds
@@ -330,14 +361,17 @@ int launch_gemm(mace_hip_ctx *ctx, GemmParams &p, bool out_u8, int batch) {
     if (lds > 64 * 1024)
       MH_HIP(ctx, hipFuncSetAttribute((const void *)k,
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    MH_PROF_BEGIN(ctx);
     hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p);
   } else {
     auto k = q8_gemm_kernel<WX, WY, FX, FY, int32_t>;
     if (lds > 64 * 1024)
       MH_HIP(ctx, hipFuncSetAttribute((const void *)k,
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    MH_PROF_BEGIN(ctx);
     hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p);
   }
+  MH_PROF_END(ctx);
   MH_HIP(ctx, hipGetLastError());
   return MACE_HIP_SUCCESS;
 }

@@ -156,6 +156,7 @@ int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
     else                                                                                 \
       hipLaunchKernelGGL((q8_gemv_kernel<NB_, false, OutT>), grid, block, 0, ctx->stream, p); \
   } while (0)
+  MH_PROF_BEGIN(ctx);
   switch (nb) {
     case 8: MH_GEMV_LAUNCH(8); break;
     case 4: MH_GEMV_LAUNCH(4); break;
@@ -163,6 +164,7 @@ int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
     default: MH_GEMV_LAUNCH(1); break;
   }
 #undef MH_GEMV_LAUNCH
+  MH_PROF_END(ctx);
   MH_HIP(ctx, hipGetLastError());
   return MACE_HIP_SUCCESS;
 }

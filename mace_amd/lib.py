@@ -42,6 +42,8 @@ SIGNATURES = {
                                     C.POINTER(_int)]),
     "mace_hip_timer_start": (_int, [_p]),
     "mace_hip_timer_stop": (_int, [_p, C.POINTER(_f32)]),
+    "mace_hip_profile_enable": (_int, [_p, _int]),
+    "mace_hip_profile_last_kernel_ms": (_int, [_p, C.POINTER(_f32)]),
     "mace_hip_ctx_fail_next_allocs": (_int, [_p, _int]),
     "mace_hip_malloc": (_int, [_p, C.c_size_t, C.POINTER(_p)]),
     "mace_hip_free": (_int, [_p, _p]),
@@ -91,6 +93,13 @@ def load():
             raise FileNotFoundError(
                 "%s is missing: build it with `make -C mace_amd/csrc` "
                 "(no CPU fallback exists)" % LIB_PATH)
+        try:
+            # PyTorch ships its own HIP runtime under the same soname; when both live in one
+            # process the first one loaded is the one both use, and only PyTorch's request
+            # resolves to a copy that is already there.  So let it go first when present.
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         lib = C.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(lib, name)          # AttributeError if the symbol is not exported
@@ -157,6 +166,15 @@ class Context:
     def timer_stop(self):
         ms = _f32()
         self.check(self.lib.mace_hip_timer_stop(self.handle, C.byref(ms)))
+        return ms.value
+
+
+    def profile(self, on):
+        self.check(self.lib.mace_hip_profile_enable(self.handle, int(on)))
+
+    def last_kernel_ms(self):
+        ms = _f32()
+        self.check(self.lib.mace_hip_profile_last_kernel_ms(self.handle, C.byref(ms)))
         return ms.value
 
 
