@@ -79,12 +79,24 @@ struct ArenaScope {
 // ---- arithmetic shared by device epilogues and the host-side test exports ------------
 
 // gemmlowp SaturatingRoundingDoublingHighMul: floor(a*b / 2^31 + 1/2), except
-// INT32_MIN * INT32_MIN which saturates.  (ab + nudge) / 2^31 with truncating division and
-// nudge = ab >= 0 ? 2^30 : 1 - 2^30 equals the arithmetic shift below for every other input.
+// INT32_MIN * INT32_MIN which saturates.  gemmlowp writes (ab + nudge) / 2^31 with truncating
+// division and nudge = ab >= 0 ? 2^30 : 1 - 2^30, which equals (ab + 2^30) >> 31 (arithmetic)
+// for every other input.  Evaluated in 32-bit pieces: ab = hi * 2^32 + lo, so
+// (ab + 2^30) >> 31 = 2 * (hi + carry) + ((lo + 2^30) mod 2^32 >> 31).
+__host__ __device__ inline int32_t mh_mulhi_i32(int32_t a, int32_t b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __mulhi(a, b);
+#else
+  return (int32_t)(((int64_t)a * (int64_t)b) >> 32);
+#endif
+}
 __host__ __device__ inline int32_t mh_srdhm(int32_t a, int32_t b) {
-  if (a == INT32_MIN && b == INT32_MIN) return INT32_MAX;
-  const int64_t ab = (int64_t)a * (int64_t)b;
-  return (int32_t)((ab + ((int64_t)1 << 30)) >> 31);
+  const uint32_t lo = (uint32_t)a * (uint32_t)b;
+  const uint32_t hi = (uint32_t)mh_mulhi_i32(a, b);
+  const uint32_t t = lo + 0x40000000u;
+  const uint32_t carry = t < lo ? 1u : 0u;
+  const int32_t r = (int32_t)(((hi + carry) << 1) | (t >> 31));
+  return (a == INT32_MIN && b == INT32_MIN) ? INT32_MAX : r;
 }
 
 // gemmlowp RoundingDivideByPOT: x / 2^e rounded to nearest, ties away from zero.
@@ -95,10 +107,39 @@ __host__ __device__ inline int32_t mh_rdivpot(int32_t x, int e) {
   return (x >> e) + (rem > thr ? 1 : 0);
 }
 
-__host__ __device__ inline int32_t mh_requant_fixed(int32_t acc, int32_t mult, int shift,
-                                                    int32_t zp, int lo, int hi) {
-  const int64_t z = (int64_t)mh_rdivpot(mh_srdhm(acc, mult), shift) + (int64_t)zp;
-  return (int32_t)(z < lo ? lo : (z > hi ? hi : z));
+// The uint8 output pipeline with everything that does not depend on the accumulator folded
+// on the host: clamp(RDivPOT(SRDHM(x, mult), shift) + zp, lo, hi)
+//            = clamp(RDivPOT(SRDHM(x, mult), shift), lo - zp, hi - zp) + zp.
+struct RequantFixed {
+  int32_t mult;
+  int32_t shift;
+  int32_t mask;      // 2^shift - 1
+  int32_t half;      // mask >> 1
+  int32_t blo, bhi;  // lo - zp, hi - zp (must fit int32; checked by mh_make_requant)
+  int32_t zp;
+};
+// false when lo - zp or hi - zp leaves the int32 range (then the reference's own int32
+// addition of the offset overflows for some accumulators)
+inline bool mh_make_requant(int32_t mult, int shift, int32_t zp, int lo, int hi,
+                            RequantFixed *r) {
+  const int64_t blo = (int64_t)lo - zp, bhi = (int64_t)hi - zp;
+  if (blo < INT32_MIN || bhi > INT32_MAX || shift < 0 || shift > 31) return false;
+  r->mult = mult;
+  r->shift = shift;
+  r->mask = (int32_t)(((uint32_t)1 << shift) - 1u);
+  r->half = r->mask >> 1;
+  r->blo = (int32_t)blo;
+  r->bhi = (int32_t)bhi;
+  r->zp = zp;
+  return true;
+}
+__host__ __device__ inline int32_t mh_requant_fixed(int32_t acc, const RequantFixed &q) {
+  const int32_t y = mh_srdhm(acc, q.mult);
+  const int32_t rem = y & q.mask;
+  const int32_t thr = q.half - (y >> 31);            // half + (y < 0)
+  int32_t z = (y >> q.shift) + (rem > thr ? 1 : 0);
+  z = z < q.blo ? q.blo : (z > q.bhi ? q.bhi : z);
+  return z + q.zp;
 }
 
 // roundf (ties away from zero) without relying on a library implementation: the

@@ -240,8 +240,10 @@ uint8_t mace_hip_quantize_u8(float value, float scale, int32_t zero_point) {
 
 uint8_t mace_hip_requant_fixed_u8(int32_t acc, int32_t multiplier, int right_shift,
                                   int32_t offset_after_shift, int clamp_min, int clamp_max) {
-  return (uint8_t)mh_requant_fixed(acc, multiplier, right_shift, offset_after_shift,
-                                   clamp_min, clamp_max);
+  RequantFixed q;
+  if (!mh_make_requant(multiplier, right_shift, offset_after_shift, clamp_min, clamp_max, &q))
+    return 0;
+  return (uint8_t)mh_requant_fixed(acc, q);
 }
 
 uint8_t mace_hip_requant_float_u8(int32_t acc, float multiplier, int32_t out_zp, int mode) {

@@ -21,6 +21,7 @@
 // are read in place; anything else is first repacked (transposed and/or padded with 0x80,
 // which is zero after the shift) into the context's arena.
 #include <algorithm>
+#include <type_traits>
 
 #include "common.h"
 
@@ -44,9 +45,9 @@ struct GemmParams {
   void *out;
   int64_t ldo;        // elements between consecutive y
   int64_t obs;        // elements per batch
-  int32_t mult, zp;
-  int shift, lo, hi;
+  RequantFixed rq;    // uint8 output pipeline
   int tiles_x, tiles_y;
+  long long *dbg;     // lab instrumentation only (nullptr in the library)
 };
 
 // XCD-aware tile order: consecutive workgroup ids are dealt round-robin to the 8 XCDs, so
@@ -66,6 +67,73 @@ __device__ inline void tile_of_block(int bid, int nblocks, int tiles_x, int tile
   const int r = t - g * per_group;
   *ty = first_y + r % gsize;
   *tx = r / gsize;
+}
+
+// Epilogue shared by the GEMM kernels: adds the correction vectors to the accumulators and
+// stores int32 results or requantized bytes.  Accumulator register r of a 32x32 tile holds
+//   x (MFMA row)    = 8 * (r / 4) + 4 * (lane / 32) + r % 4
+//   y (MFMA column) = lane % 32
+// so every lane owns runs of four consecutive x, stored as one 16-byte (int32) or 4-byte
+// (uint8) access.  The correction vectors of the tile are staged through LDS first (the
+// operand buffers are dead by then), so the stores do not wait on scattered global loads.
+template <int WX, int WY, int FX, int FY, typename OutT>
+__device__ inline void gemm_epilogue(v16i (&acc)[FX][FY], const GemmParams &p, uint8_t *lds,
+                                     int b, int x0, int y0, int wx, int wy, int tid) {
+  constexpr int NT = WX * WY * 64;
+  constexpr int TX = WX * FX * 32, TY = WY * FY * 32;
+  const int lane = tid & 63;
+  const int32_t *cX = p.corrX + (int64_t)b * p.cxbs;
+  const int32_t *cY = p.corrY + (int64_t)b * p.cybs;
+  int32_t *sc = (int32_t *)lds;   // [TX] corrections along x, then [TY] along y
+  __syncthreads();                // every wavefront is done reading operand tiles
+  for (int i = tid; i < TX; i += NT) sc[i] = cX[min(x0 + i, p.XN - 1)];
+  for (int i = tid; i < TY; i += NT) sc[TX + i] = cY[min(y0 + i, p.YN - 1)];
+  __syncthreads();
+
+  OutT *outb = (OutT *)p.out + (int64_t)b * p.obs;
+  const bool vec_ok = (p.ldo % 4 == 0) && (((uintptr_t)outb) % (4 * sizeof(OutT)) == 0);
+  const bool interior = vec_ok && x0 + TX <= p.XN && y0 + TY <= p.YN;
+  const RequantFixed rq = p.rq;
+#pragma unroll
+  for (int j = 0; j < FY; ++j) {
+    const int yl = (wy * FY + j) * 32 + (lane & 31);
+    const int y = y0 + yl;
+    const uint32_t cy = (uint32_t)sc[TX + yl];
+    OutT *orow = outb + (int64_t)y * p.ldo + x0;
+#pragma unroll
+    for (int i = 0; i < FX; ++i) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int xl = (wx * FX + i) * 32 + 8 * q + 4 * (lane >> 5);
+        const v4i cx = *(const v4i *)(sc + xl);
+        int32_t v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          v[e] = (int32_t)((uint32_t)acc[i][j][q * 4 + e] + (uint32_t)cx[e] + cy);
+        if constexpr (sizeof(OutT) == 4) {
+          if (interior) {
+            *(v4i *)(orow + xl) = v4i{v[0], v[1], v[2], v[3]};
+          } else if (y < p.YN) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (x0 + xl + e < p.XN) orow[xl + e] = (OutT)v[e];
+          }
+        } else {
+          uint32_t packed = 0;
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            packed |= (uint32_t)mh_requant_fixed(v[e], rq) << (8 * e);
+          if (interior) {
+            *(uint32_t *)(orow + xl) = packed;
+          } else if (y < p.YN) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (x0 + xl + e < p.XN) orow[xl + e] = (OutT)((packed >> (8 * e)) & 0xff);
+          }
+        }
+      }
+    }
+  }
 }
 
 template <int WX, int WY, int FX, int FY, typename OutT>
@@ -207,58 +275,219 @@ __global__ __launch_bounds__(WX *WY * 64) void q8_gemm_kernel(GemmParams p) {
     for (int ks = 0; ks < (ktail + 31) / 32; ++ks) mfma_step(0, ks);
   }
 
-  // epilogue: accumulator register r of a 32x32 tile holds
-  //   x (MFMA row)    = 8 * (r / 4) + 4 * (lane / 32) + r % 4
-  //   y (MFMA column) = lane % 32
-  const int32_t *cX = p.corrX + (int64_t)b * p.cxbs;
-  const int32_t *cY = p.corrY + (int64_t)b * p.cybs;
-  OutT *outb = (OutT *)p.out + (int64_t)b * p.obs;
-  const bool vec_ok = (p.ldo % 4 == 0) && (((uintptr_t)outb) % (4 * sizeof(OutT)) == 0);
+  gemm_epilogue<WX, WY, FX, FY, OutT>(acc, p, lds, b, x0, y0, wx, wy, tid);
+}
+
+// ---- the streaming GEMM kernel: global -> LDS without passing through registers ----------
+//
+// A ring of STAGES LDS buffers, each one 64-byte k slab of the X and Y tiles, is filled by
+// global_load_lds_dwordx4 (one instruction moves 64 lanes x 16 bytes = 16 rows x 64 bytes
+// straight into LDS, STAGES-1 slabs ahead of the one being multiplied), so the wavefronts
+// only read fragments and issue MFMAs.  A slab row is 64 bytes = four 16-byte chunks; chunk c
+// of row r is stored at slot c ^ ((r >> 2) & 3), which makes the 16 rows a group of lanes
+// reads in one fragment load fall into 16 distinct bank groups without padding (the DMA
+// writes lane-contiguous bytes, so padding is not available anyway; the swizzle is applied by
+// choosing which global chunk each lane fetches).  The 0x80 flip is applied to the fragments.
+//
+// Requirements (checked by the host): K % 64 == 0 and K >= 64 * (STAGES - 1).
+constexpr int SLAB = 64;   // bytes of k per ring stage
+
+__device__ inline void dma_16B(const uint8_t *g, uint8_t *lds_wave_base) {
+  __builtin_amdgcn_global_load_lds(
+      (const void __attribute__((address_space(1))) *)g,
+      (void __attribute__((address_space(3))) *)lds_wave_base, 16, 0, 0);
+}
+
+// s_waitcnt vmcnt(N) alone (expcnt / lgkmcnt fields left at "no wait")
+template <int N>
+__device__ inline void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit field");
+  __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
+}
+
+template <int WX, int WY, int FX, int FY, int STAGES, typename OutT, int OCC = 1, int ABLATE = 0>
+__global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParams p) {
+  constexpr int NW = WX * WY;
+  constexpr int TX = WX * FX * 32;
+  constexpr int TY = WY * FY * 32;
+  constexpr int LX = TX / 16 / NW;   // DMA instructions per wavefront per slab, X tile
+  constexpr int LY = TY / 16 / NW;
+  static_assert(TX % (16 * NW) == 0 && TY % (16 * NW) == 0, "uneven slab load");
+  constexpr int STAGE_BYTES = (TX + TY) * SLAB;
+  constexpr int Y_OFF = TX * SLAB;
+  static_assert(STAGES >= 3 && STAGES <= 5, "ring depth");
+  static_assert((STAGES - 2) * (LX + LY) < 64, "too many loads in flight for vmcnt");
+
+  extern __shared__ __align__(16) uint8_t lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wx = wave % WX, wy = wave / WX;
+
+  int tile_x, tile_y;
+  tile_of_block(blockIdx.x, gridDim.x, p.tiles_x, p.tiles_y, &tile_x, &tile_y);
+  const int x0 = tile_x * TX, y0 = tile_y * TY;
+  const int b = blockIdx.z;
+  const uint8_t *Xb = p.X + (int64_t)b * p.xbs;
+  const uint8_t *Yb = p.Y + (int64_t)b * p.ybs;
+
+  // DMA source pointers: instruction j of this wavefront fills rows [(j*NW + wave)*16, +16) of
+  // the slab; lane l lands in row l/4, slot l%4 and therefore fetches chunk slot ^ swizzle(row)
+  const uint8_t *gx[LX];
+  const uint8_t *gy[LY];
 #pragma unroll
-  for (int j = 0; j < FY; ++j) {
-    const int y = y0 + (wy * FY + j) * 32 + (lane & 31);
-    if (y >= p.YN) continue;
-    const uint32_t cy = (uint32_t)cY[y];
-    OutT *orow = outb + (int64_t)y * p.ldo;
+  for (int j = 0; j < LX; ++j) {
+    const int row = (j * NW + wave) * 16 + (lane >> 2);
+    const int kc = (lane & 3) ^ ((row >> 2) & 3);
+    gx[j] = Xb + (int64_t)min(x0 + row, p.XN - 1) * p.ldx + kc * 16;
+  }
 #pragma unroll
-    for (int i = 0; i < FX; ++i) {
+  for (int j = 0; j < LY; ++j) {
+    const int row = (j * NW + wave) * 16 + (lane >> 2);
+    const int kc = (lane & 3) ^ ((row >> 2) & 3);
+    gy[j] = Yb + (int64_t)min(y0 + row, p.YN - 1) * p.ldy + kc * 16;
+  }
+  auto issue_slab = [&](int stage, int k0) {
+    uint8_t *sx = lds + stage * STAGE_BYTES + wave * 1024;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int x = x0 + (wx * FX + i) * 32 + 8 * q + 4 * (lane >> 5);
-        if (x >= p.XN) continue;
-        int32_t v[4];
-        const bool full = x + 3 < p.XN;
+    for (int j = 0; j < LX; ++j) dma_16B(gx[j] + k0, sx + j * NW * 1024);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const uint32_t cx = (uint32_t)cX[min(x + e, p.XN - 1)];
-          v[e] = (int32_t)((uint32_t)acc[i][j][q * 4 + e] + cx + cy);
-        }
-        if constexpr (sizeof(OutT) == 4) {
-          if (full && vec_ok) {
-            *(v4i *)(orow + x) = v4i{v[0], v[1], v[2], v[3]};
-          } else {
+    for (int j = 0; j < LY; ++j) dma_16B(gy[j] + k0, sx + Y_OFF + j * NW * 1024);
+  };
+
+  v16i acc[FX][FY];
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (x + e < p.XN) orow[x + e] = (OutT)v[e];
-          }
-        } else {
-          uint32_t packed = 0;
+  for (int i = 0; i < FX; ++i)
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const uint32_t u = (uint32_t)mh_requant_fixed(v[e], p.mult, p.shift, p.zp, p.lo, p.hi);
-            packed |= u << (8 * e);
-          }
-          if (full && vec_ok) {
-            *(uint32_t *)(orow + x) = packed;
-          } else {
+    for (int j = 0; j < FY; ++j)
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (x + e < p.XN) orow[x + e] = (OutT)((packed >> (8 * e)) & 0xff);
-          }
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+  // fragment addresses: lane l reads row (l % 32) of a 32-row block, chunk 2*ks + l/32.
+  // Block bases are multiples of 32 rows, so the swizzle depends on l only.
+  const int frow = lane & 31;
+  const int fsw = (frow >> 2) & 3;
+  int foff[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) foff[ks] = frow * SLAB + (((2 * ks + (lane >> 5)) ^ fsw) << 4);
+  const int fx_base = wx * FX * 32 * SLAB;
+  const int fy_base = Y_OFF + wy * FY * 32 * SLAB;
+  const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+
+  auto read_frags = [&](int stage, int ks, v4i (&a)[FX], v4i (&bf)[FY]) {
+    const uint8_t *s = lds + stage * STAGE_BYTES + foff[ks];
+#pragma unroll
+    for (int i = 0; i < FX; ++i) a[i] = *(const v4i *)(s + fx_base + i * 32 * SLAB);
+#pragma unroll
+    for (int j = 0; j < FY; ++j) bf[j] = *(const v4i *)(s + fy_base + j * 32 * SLAB);
+  };
+  auto flip_frags = [&](v4i (&a)[FX], v4i (&bf)[FY]) {
+#pragma unroll
+    for (int i = 0; i < FX; ++i) a[i] ^= flip;
+#pragma unroll
+    for (int j = 0; j < FY; ++j) bf[j] ^= flip;
+  };
+  // One k step of 32 for the whole wavefront tile, written as FX*FY "slots": slot m issues
+  // MFMA m on the current (already flipped) fragments and, in the 8 passes the matrix core
+  // needs for it, one piece of the work for what comes next: the LDS read of fragment m of
+  // the following step (slots 0 .. FX+FY-1), the flip of a fragment read DELAY slots earlier,
+  // and (DMA = true) one global->LDS transfer of the slab STAGES-1 ahead.  The order inside a
+  // slot is pinned with sched_barrier so that the compiler neither clusters the LDS reads in
+  // front of a wait nor the flips behind the last MFMA.
+  constexpr int NM = FX * FY, NF = FX + FY;
+  constexpr int DELAY = NM - NF > 0 ? NM - NF : 0;
+  auto frag_ptr = [&](int stage, int ks, int f) -> const v4i * {
+    const uint8_t *s = lds + stage * STAGE_BYTES + foff[ks];
+    return (const v4i *)(f < FX ? s + fx_base + f * 32 * SLAB : s + fy_base + (f - FX) * 32 * SLAB);
+  };
+  auto k_step = [&](auto dma_tag, v4i (&ca)[FX], v4i (&cb)[FY], v4i (&na)[FX], v4i (&nb)[FY],
+                    int nstage, int nks, int dstage, int dk0) {
+    constexpr bool dma = decltype(dma_tag)::value;
+    uint8_t *dsx = lds + dstage * STAGE_BYTES + wave * 1024;
+#pragma unroll
+    for (int m = 0; m < NM; ++m) {
+      acc[m / FY][m % FY] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ca[m / FY], cb[m % FY],
+                                                                  acc[m / FY][m % FY], 0, 0, 0);
+      constexpr int READS_PER_SLOT = (NF + NM - 1) / NM;
+#pragma unroll
+      for (int f = m * READS_PER_SLOT; f < (m + 1) * READS_PER_SLOT; ++f) {
+        if (f < FX) na[f] = *frag_ptr(nstage, nks, f);
+        else if (f < NF) nb[f - FX] = *frag_ptr(nstage, nks, f);
+      }
+      if (DELAY > 0 && m >= DELAY && m - DELAY < NF) {
+        const int f = m - DELAY;
+        if (f < FX) na[f] ^= flip;
+        else nb[f - FX] ^= flip;
+      }
+      if constexpr (dma) {
+        // LX + LY transfers spread over the slots from slot 0 on
+        constexpr int PER_SLOT = (LX + LY + NM - 1) / NM;
+#pragma unroll
+        for (int d = m * PER_SLOT; d < (m + 1) * PER_SLOT; ++d) {
+          if (d < LX) dma_16B(gx[d] + dk0, dsx + d * NW * 1024);
+          else if (d < LX + LY) dma_16B(gy[d - LX] + dk0, dsx + Y_OFF + (d - LX) * NW * 1024);
         }
       }
+      __builtin_amdgcn_sched_barrier(0);
     }
+    // small wavefront tiles have too few slots to hide the flips: do what is left here
+#pragma unroll
+    for (int f = 0; f < NF; ++f)
+      if (DELAY == 0 || f + DELAY >= NM) {
+        if (f < FX) na[f] ^= flip;
+        else nb[f - FX] ^= flip;
+      }
+  };
+
+  long long dbg_c0 = 0, dbg_w0 = 0;
+  if (ABLATE & 4) { dbg_c0 = clock64(); dbg_w0 = wall_clock64(); }
+  const int nslab = p.K / SLAB;
+  // prologue: slabs 0 .. STAGES-2 in flight
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; ++s) issue_slab(s, s * SLAB);
+  wait_vmcnt<(STAGES - 2) * (LX + LY)>();   // slab 0 of this wavefront has landed
+  __builtin_amdgcn_s_barrier();             // ... and everybody else's part of it
+  asm volatile("" ::: "memory");
+
+  v4i a0[FX], b0[FY], a1[FX], b1[FY];
+  read_frags(0, 0, a0, b0);
+  flip_frags(a0, b0);
+  int stage = 0;
+  for (int kt = 0; kt < nslab; ++kt) {
+    // first half of slab kt; fetches its second half
+    k_step(std::false_type{}, a0, b0, a1, b1, stage, 1, 0, 0);
+    // Slab kt+1 must be complete, and every wavefront must be done with slab kt-1 (whose
+    // stage the next DMA overwrites), before going on: one barrier covers both.
+    // Slabs 0 .. kt+STAGES-2 have been issued so far; those after slab kt+1 may stay in flight.
+    // Slabs up to kt+STAGES-2 have been issued (past the end: repeats of the last slab, see
+    // below), so exactly STAGES-3 slabs newer than kt+1 may stay in flight.
+    wait_vmcnt<(STAGES - 3) * (LX + LY)>();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    int next = stage + 1;
+    if (next == STAGES) next = 0;
+    int dst = stage + STAGES - 1;
+    if (dst >= STAGES) dst -= STAGES;
+    // Second half of slab kt; fetches the first half of slab kt+1 and feeds the ring with slab
+    // kt+STAGES-1.  Near the end there is no such slab: the last one is fetched again into a
+    // stage nobody reads any more, which keeps the loop free of branches and the in-flight
+    // count constant; likewise the fragments fetched after the last slab are never used.
+    const int ks = min(kt + STAGES - 1, nslab - 1);
+    k_step(std::true_type{}, a1, b1, a0, b0, next, 0, dst, ks * SLAB);
+    stage = next;
   }
+
+  if (ABLATE & 4) {
+    const long long c1 = clock64(), w1 = wall_clock64();
+    gemm_epilogue<WX, WY, FX, FY, OutT>(acc, p, lds, b, x0, y0, wx, wy, tid);
+    if (tid == 0 && blockIdx.x == 8) {
+      p.dbg[0] = c1 - dbg_c0; p.dbg[1] = w1 - dbg_w0;
+      p.dbg[2] = clock64() - c1; p.dbg[3] = wall_clock64() - w1;
+    }
+    return;
+  }
+  gemm_epilogue<WX, WY, FX, FY, OutT>(acc, p, lds, b, x0, y0, wx, wy, tid);
 }
 
 // ---- repacking ---------------------------------------------------------------------------
@@ -376,6 +605,34 @@ int launch_gemm(mace_hip_ctx *ctx, GemmParams &p, bool out_u8, int batch) {
   return MACE_HIP_SUCCESS;
 }
 
+// the streaming kernel; the caller has checked K % 64 == 0 and K >= 64 * (STAGES - 1)
+template <int WX, int WY, int FX, int FY, int STAGES, int OCC>
+int launch_gemm_dma(mace_hip_ctx *ctx, GemmParams &p, bool out_u8, int batch) {
+  constexpr int TX = WX * FX * 32, TY = WY * FY * 32;
+  p.tiles_x = (p.XN + TX - 1) / TX;
+  p.tiles_y = (p.YN + TY - 1) / TY;
+  const size_t lds = (size_t)STAGES * (TX + TY) * SLAB;
+  dim3 grid(p.tiles_x * p.tiles_y, 1, batch), block(WX * WY * 64);
+  if (out_u8) {
+    auto k = q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, uint8_t, OCC>;
+    if (lds > 64 * 1024)
+      MH_HIP(ctx, hipFuncSetAttribute((const void *)k,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    MH_PROF_BEGIN(ctx);
+    hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p);
+  } else {
+    auto k = q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, int32_t, OCC>;
+    if (lds > 64 * 1024)
+      MH_HIP(ctx, hipFuncSetAttribute((const void *)k,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    MH_PROF_BEGIN(ctx);
+    hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p);
+  }
+  MH_PROF_END(ctx);
+  MH_HIP(ctx, hipGetLastError());
+  return MACE_HIP_SUCCESS;
+}
+
 }  // namespace
 
 int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8_t *rhs,
@@ -388,10 +645,13 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   MH_CHECK(ctx, rows < (1ll << 31) && cols < (1ll << 31) && depth < (1ll << 31) - 64 &&
                     batch < 65536,
            "dimension too large");
+  RequantFixed rq{};
   if (out_u8) {
     MH_CHECK(ctx, ep.shift >= 0 && ep.shift <= 31, "right shift %d outside [0,31]", ep.shift);
     MH_CHECK(ctx, ep.lo >= 0 && ep.hi <= 255 && ep.lo <= ep.hi, "clamp range [%d,%d] invalid",
              ep.lo, ep.hi);
+    MH_CHECK(ctx, mh_make_requant(ep.mult, ep.shift, ep.zp, ep.lo, ep.hi, &rq),
+             "offset_after_shift %d outside the supported range", ep.zp);
   }
   if (batch == 0 || rows == 0 || cols == 0) return MACE_HIP_SUCCESS;
   MH_CHECK(ctx, lhs && rhs && out, "null operand");
@@ -479,19 +739,27 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   p.out = out;
   p.ldo = p.XN;
   p.obs = rows * cols;
-  p.mult = ep.mult; p.shift = ep.shift; p.zp = ep.zp; p.lo = ep.lo; p.hi = ep.hi;
+  p.rq = rq;
 
   // tile shape: the largest that still yields enough workgroups to fill the CUs
   const int64_t cu = ctx->cu_count > 0 ? ctx->cu_count : 256;
   auto tiles = [&](int tx, int ty) {
     return (int64_t)((p.XN + tx - 1) / tx) * ((p.YN + ty - 1) / ty) * batch;
   };
-  if (p.XN > 128 && p.YN > 128 && tiles(256, 256) >= cu)
-    return launch_gemm<2, 2, 4, 4>(ctx, p, out_u8, (int)batch);
-  if (p.XN <= 64 && p.YN > 128 && tiles(64, 256) >= cu)
-    return launch_gemm<1, 4, 2, 2>(ctx, p, out_u8, (int)batch);
-  if (p.XN > 64 && p.YN > 64 && tiles(128, 128) >= cu)
-    return launch_gemm<2, 2, 2, 2>(ctx, p, out_u8, (int)batch);
+  p.dbg = nullptr;
+  const bool big = p.XN > 128 && p.YN > 128 && tiles(256, 256) >= cu;
+  const bool skinny = !big && p.XN <= 64 && p.YN > 128 && tiles(64, 256) >= cu;
+  const bool medium = !big && !skinny && p.XN > 64 && p.YN > 64 && tiles(128, 128) >= cu;
+  // the streaming kernel needs whole 64-byte slabs and enough of them to fill its ring
+  if (p.K % SLAB == 0 && p.K >= SLAB * 3) {
+    if (big) return launch_gemm_dma<2, 2, 4, 4, 4, 1>(ctx, p, out_u8, (int)batch);
+    if (skinny) return launch_gemm_dma<1, 4, 2, 2, 4, 2>(ctx, p, out_u8, (int)batch);
+    if (medium) return launch_gemm_dma<2, 2, 2, 2, 4, 2>(ctx, p, out_u8, (int)batch);
+    return launch_gemm_dma<2, 2, 1, 1, 4, 4>(ctx, p, out_u8, (int)batch);
+  }
+  if (big) return launch_gemm<2, 2, 4, 4>(ctx, p, out_u8, (int)batch);
+  if (skinny) return launch_gemm<1, 4, 2, 2>(ctx, p, out_u8, (int)batch);
+  if (medium) return launch_gemm<2, 2, 2, 2>(ctx, p, out_u8, (int)batch);
   return launch_gemm<2, 2, 1, 1>(ctx, p, out_u8, (int)batch);
 }
 
