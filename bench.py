@@ -45,6 +45,7 @@ def main():
     ap.add_argument("--size", type=int, default=8192, help="M = N = K of the uint8 GEMM")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemv", action="store_true")
+    ap.add_argument("--only-gemv", action="store_true", help="development: skip the GEMM part")
     ap.add_argument("--cpu-rows", type=int, default=8192,
                     help="rows of A the CPU baseline multiplies by the whole of B")
     args = ap.parse_args()
@@ -66,6 +67,9 @@ def main():
     arch, cus, lds = ctx.device_info()
     log("device %s, %d CUs, %d B LDS/workgroup" % (arch, cus, lds))
 
+    if args.only_gemv:
+        print(json.dumps(bench_gemv(ctx, mh, torch, args)))
+        return
     n = args.size
     g = torch.Generator(device="cuda").manual_seed(5)
     A = torch.randint(0, 256, (n, n), dtype=torch.uint8, device="cuda", generator=g)

@@ -11,6 +11,8 @@
 // loads of a row are issued before the first dot product so a CU keeps tens of KiB in
 // flight.  Up to NB batch rows of the right-hand vector are consumed per pass over the
 // weights, so the weight matrix is streamed once for batch <= 8.
+#include <type_traits>
+
 #include "common.h"
 
 namespace {
@@ -29,10 +31,24 @@ struct GemvParams {
   int neon_mode;
 };
 
+// Sum over the 64 lanes of a wavefront with DPP adds (VALU rate; the shuffle-based form goes
+// through the LDS crossbar and costs an LDS round trip per step).  Every lane gets the total.
 __device__ inline uint32_t wave_sum(uint32_t v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-  return v;
+  int x = (int)v;
+  x += __builtin_amdgcn_update_dpp(0, x, 0xB1, 0xF, 0xF, true);    // quad_perm [1,0,3,2]
+  x += __builtin_amdgcn_update_dpp(0, x, 0x4E, 0xF, 0xF, true);    // quad_perm [2,3,0,1]
+  x += __builtin_amdgcn_update_dpp(0, x, 0x141, 0xF, 0xF, true);   // row_half_mirror
+  x += __builtin_amdgcn_update_dpp(0, x, 0x140, 0xF, 0xF, true);   // row_mirror: row sums
+  x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xA, 0xF, false);  // row_bcast:15 -> rows 1,3
+  x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xC, 0xF, false);  // row_bcast:31 -> rows 2,3
+  return (uint32_t)__builtin_amdgcn_readlane(x, 63);               // lane 63 holds the total
+}
+
+// 16-byte load marked non-temporal: the weight matrix is read once per call
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+__device__ inline uint4 load_stream16(const uint8_t *p) {
+  const u32x4 v = __builtin_nontemporal_load((const u32x4 *)p);
+  return uint4{v.x, v.y, v.z, v.w};
 }
 
 __device__ inline uint32_t dot16(const uint4 &a, const uint4 &b, uint32_t acc) {
@@ -141,6 +157,113 @@ __global__ __launch_bounds__(256) void q8_gemv_kernel(GemvParams p) {
   }
 }
 
+// Fast path for a shared weight matrix (lhs not batched) with 16-byte aligned rows: one
+// wavefront owns R consecutive weight rows and one workgroup NWAVES*R rows; with 16 wavefronts
+// a 4096 x 4096 matrix is one workgroup per CU, every wavefront requesting its whole row
+// before anything is consumed.  The right-hand vectors of the pass (NB batch rows) are staged
+// in LDS once per workgroup instead of being re-read by every wavefront.  W is walked in
+// blocks of 4 KiB per row: lane l holds chunks l, l+64, l+128, l+192 of the block.
+template <int R, int NB, int NWAVES, typename OutT>
+__global__ __launch_bounds__(NWAVES * 64) void q8_gemv_rows_kernel(GemvParams p) {
+  extern __shared__ __align__(16) uint8_t sx[];   // [NB][W]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int h0 = (blockIdx.x * NWAVES + wave) * R;
+  const int b0 = blockIdx.y * NB;
+  const int nb = min(NB, p.batch - b0);
+  const int nchunk = p.W >> 4;
+  const uint4 ones = {0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u};
+  const uint4 zero = {0u, 0u, 0u, 0u};
+
+  // rows past the end re-read the last row; their results are not stored
+  const uint8_t *lrow[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) lrow[r] = p.lhs + (int64_t)min(h0 + r, p.H - 1) * p.W;
+
+  uint32_t dot[R][NB], sum_l[R], sum_r[NB];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    sum_l[r] = 0;
+#pragma unroll
+    for (int b = 0; b < NB; ++b) dot[r][b] = 0;
+  }
+
+  __shared__ uint32_t part[NB][NWAVES];   // per-wavefront partial sums of the right-hand rows
+  auto block_of_w = [&](auto masked_tag, int c0) {
+    constexpr bool masked = decltype(masked_tag)::value;
+    // weights of this block: R x 4 loads of 16 bytes in flight per lane
+    uint4 w[R][4];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int c = c0 + lane + 64 * u;
+        w[r][u] = load_stream16(lrow[r] + (int64_t)(masked ? min(c, nchunk - 1) : c) * 16);
+      }
+    if (c0 == 0) {
+      // Stage the right-hand vectors while the weights are on their way, and sum their
+      // bytes once per workgroup (every output needs sum(r) of its batch row).
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        uint32_t s = 0;
+        if (b < nb) {
+          const uint8_t *src = p.rhs + (int64_t)(b0 + b) * p.rhs_bs;
+          for (int c = tid; c < nchunk; c += NWAVES * 64) {
+            const uint4 x = *(const uint4 *)(src + (int64_t)c * 16);
+            *(uint4 *)(sx + ((size_t)b * nchunk + c) * 16) = x;
+            s = dot16(x, ones, s);
+          }
+        }
+        s = wave_sum(s);
+        if (lane == 0) part[b][wave] = s;
+      }
+      __syncthreads();
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int c = c0 + lane + 64 * u;
+      const bool ok = !masked || c < nchunk;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        if (masked && !ok) w[r][u] = zero;
+        sum_l[r] = dot16(w[r][u], ones, sum_l[r]);
+      }
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        if (b < nb) {
+          const uint4 x =
+              *(const uint4 *)(sx + ((size_t)b * nchunk + (masked ? min(c, nchunk - 1) : c)) * 16);
+#pragma unroll
+          for (int r = 0; r < R; ++r) dot[r][b] = dot16(w[r][u], x, dot[r][b]);   // w is 0 if !ok
+        }
+      }
+    }
+  };
+  const int nfull = nchunk & ~255;
+  for (int c0 = 0; c0 < nfull; c0 += 256) block_of_w(std::false_type{}, c0);
+  if (nfull < nchunk) block_of_w(std::true_type{}, nfull);
+
+  const uint32_t zl = (uint32_t)p.lhs_zp, zr = (uint32_t)p.rhs_zp;
+#pragma unroll
+  for (int b = 0; b < NB; ++b) sum_r[b] = wave_sum(lane < NWAVES ? part[b][lane] : 0u);
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const uint32_t sl = wave_sum(sum_l[r]);
+    const int h = h0 + r;
+    const uint32_t fixed =
+        (uint32_t)p.W * zl * zr + ((p.bias && h < p.H) ? (uint32_t)p.bias[h] : 0u);
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const uint32_t d = wave_sum(dot[r][b]);
+      if (lane == 0 && b < nb && h < p.H) {
+        const int32_t ret = (int32_t)(d - sl * zr - sum_r[b] * zl + fixed);
+        OutT *o = (OutT *)p.out + (int64_t)(b0 + b) * p.H + h;
+        if constexpr (sizeof(OutT) == 4) *o = (OutT)ret;
+        else *o = (OutT)mh_requant_float(ret, p.mult, p.out_zp, p.neon_mode);
+      }
+    }
+  }
+}
+
 template <typename OutT>
 int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
   const bool vec = (p.W % 16 == 0) && ((uintptr_t)p.lhs % 16 == 0) &&
@@ -148,6 +271,24 @@ int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
   // a batched lhs gives every batch its own weights: one batch row per pass
   int nb = lhs_batched ? 1 : (p.batch >= 8 ? 8 : (p.batch >= 4 ? 4 : (p.batch >= 2 ? 2 : 1)));
   dim3 block(256);
+  // shared weights, aligned rows, right-hand vectors of one pass fit in LDS: row-block kernel
+  if (vec && !lhs_batched && p.W >= 16 && (size_t)nb * p.W <= 64 * 1024) {
+    constexpr int R = 1, NWAVES = 16;
+    dim3 grid((unsigned)((p.H + NWAVES * R - 1) / (NWAVES * R)),
+              (unsigned)((p.batch + nb - 1) / nb));
+    dim3 wg(NWAVES * 64);
+    const size_t lds = (size_t)nb * p.W;
+    MH_PROF_BEGIN(ctx);
+    switch (nb) {
+      case 8: hipLaunchKernelGGL((q8_gemv_rows_kernel<R, 8, NWAVES, OutT>), grid, wg, lds, ctx->stream, p); break;
+      case 4: hipLaunchKernelGGL((q8_gemv_rows_kernel<R, 4, NWAVES, OutT>), grid, wg, lds, ctx->stream, p); break;
+      case 2: hipLaunchKernelGGL((q8_gemv_rows_kernel<R, 2, NWAVES, OutT>), grid, wg, lds, ctx->stream, p); break;
+      default: hipLaunchKernelGGL((q8_gemv_rows_kernel<R, 1, NWAVES, OutT>), grid, wg, lds, ctx->stream, p); break;
+    }
+    MH_PROF_END(ctx);
+    MH_HIP(ctx, hipGetLastError());
+    return MACE_HIP_SUCCESS;
+  }
   dim3 grid((unsigned)((p.H + 3) / 4), (unsigned)((p.batch + nb - 1) / nb));
 #define MH_GEMV_LAUNCH(NB_)                                                              \
   do {                                                                                   \
