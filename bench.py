@@ -31,6 +31,11 @@ if ROOT not in sys.path:
 METRIC = "uint8 GEMM int8-TOPS + q8 Gemv HBM GB/s, % of MI355X roofline, 1 GPU"
 PEAK_INT8_TOPS = 5000.0      # MI355X dense int8 MFMA, published
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, published
+# Bytes that crossed the L2 <-> fabric boundary per launch of the dominant kernel, from rocprofv3
+# FETCH_SIZE / WRITE_SIZE runs of this benchmark scaled by the same counters' reading for a plain
+# 256 MiB copy (x2.0 and x1.0).  Keyed by M = N = K; a profiler run is needed to refresh them.
+GEMM_TRAFFIC_BYTES = {8192: 8.76e8}
+GEMV_TRAFFIC_BYTES = {1: 1.69e7, 8: 1.73e7}
 
 
 def log(*a):
@@ -46,6 +51,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemv", action="store_true")
     ap.add_argument("--only-gemv", action="store_true", help="development: skip the GEMM part")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 256 MiB device copy (a kernel of known traffic, for "
+                         "scaling the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
     ap.add_argument("--cpu-rows", type=int, default=8192,
                     help="rows of A the CPU baseline multiplies by the whole of B")
     args = ap.parse_args()
@@ -67,6 +75,12 @@ def main():
     arch, cus, lds = ctx.device_info()
     log("device %s, %d CUs, %d B LDS/workgroup" % (arch, cus, lds))
 
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(3)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     if args.only_gemv:
         print(json.dumps(bench_gemv(ctx, mh, torch, args)))
         return
@@ -129,7 +143,8 @@ def main():
                    "saturated_fraction": round(sat, 4), "device": arch, "cus": cus},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_INT8_TOPS,
                      "unit": "TOP/s", "frac": round(achieved / PEAK_INT8_TOPS, 4),
-                     "traffic": None, "kernel": "q8_gemm_kernel<2,2,4,4,uint8_t>",
+                     "traffic": GEMM_TRAFFIC_BYTES.get(n), "traffic_unit": "B/launch",
+                     "kernel": "q8_gemm_dma_kernel<2,2,4,4,4,uint8_t>",
                      "kernel_ms_avg": round(k_avg, 4), "kernel_ms_min": round(min(kms), 4),
                      "ops_per_launch": ops},
     }
@@ -193,9 +208,12 @@ def bench_gemv(ctx, mh, torch, args):
                                           100 * gbs / PEAK_HBM_GBS, loop_ms * 1e3))
         out["batch%d" % batch] = res
     hb = out["batch1"]["hbm"]
-    out["roofline"] = {"bound": "hbm", "achieved": hb["GBps"], "peak": PEAK_HBM_GBS,
-                       "unit": "GB/s", "frac": hb["frac_of_hbm_peak"], "traffic": None,
-                       "kernel": "q8_gemv_kernel<1,true,uint8_t>"}
+    out["roofline"] = {"bound": "hbm", "achieved": hb["back_to_back_GBps"], "peak": PEAK_HBM_GBS,
+                       "unit": "GB/s", "frac": round(hb["back_to_back_GBps"] / PEAK_HBM_GBS, 4),
+                       "traffic": GEMV_TRAFFIC_BYTES[1], "traffic_unit": "B/launch",
+                       "kernel": "q8_gemv_rows_kernel<1,1,16,uint8_t>",
+                       "timing": "400 back-to-back launches between two HIP events, rotating "
+                                 "over 640 MiB of weights"}
     return out
 
 

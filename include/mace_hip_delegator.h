@@ -1,0 +1,573 @@
+// mace_hip_delegator.h -- C++ host side above the C ABI (mace_hip.h).
+//
+// Header-only mirror of the reference interfaces this path plugs into, with the same names,
+// argument meaning and error behaviour, so that a MACE maintainer can see the drop-in without
+// building MACE:
+//   * delegator::Gemm / delegator::Gemv / delegator::Conv2d virtual signatures
+//     (mace/ops/delegator/gemm.h:35-70, gemv.h:27-46, conv_2d.h:60-82),
+//   * DelegatorInfo keys, OpDelegatorRegistry::Register / GetCreator with the reference's
+//     fallback rule (mace/core/registry/op_delegator_registry.cc:39-103),
+//   * the shape derivation and dispatch of MatMulOp, FullyConnectedOp and the quantized 1x1
+//     Conv2dOp (mace/ops/matmul.cc:55-83,110-215,397-483; fully_connected.cc:82-121,141-179;
+//     conv_2d.cc:201-318; arm/base/conv_2d_1x1.cc:27-72).
+// Everything lives in namespace mace_hip so the header can sit next to the real MACE headers.
+// In a MACE tree the hip:: classes derive from mace::ops::delegator::* instead and are
+// registered under the keys the ops ask for.
+//
+// Contract violations the reference handles with MACE_CHECK (process abort) are reported as
+// MaceStatus::MACE_INVALID_ARGS here.
+#ifndef MACE_HIP_DELEGATOR_H_
+#define MACE_HIP_DELEGATOR_H_
+
+#include <cstdint>
+#include <functional>
+#include <memory>
+#include <numeric>
+#include <sstream>
+#include <type_traits>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "mace_hip.h"
+
+namespace mace_hip {
+
+typedef int64_t index_t;
+
+// include/mace/public/mace.h:244-250
+enum class MaceStatus {
+  MACE_SUCCESS = 0,
+  MACE_INVALID_ARGS = 1,
+  MACE_OUT_OF_RESOURCES = 2,
+  MACE_UNSUPPORTED = 3,
+  MACE_RUNTIME_ERROR = 4
+};
+inline MaceStatus ToStatus(int code) { return static_cast<MaceStatus>(code); }
+
+enum DataType { DT_INVALID = 0, DT_FLOAT = 1, DT_UINT8 = 2, DT_INT32 = 4 };  // mace.proto
+enum RuntimeType { RT_CPU = 0, RT_OPENCL = 2 };            // include/mace/public/mace.h
+enum ImplType { REF = 0, NEON };                            // mace/core/ops/op_delegator.h:25-28
+const ImplType kCpuImplType = ImplType::REF;                // :30-34 on a non-NEON host
+enum MatrixMajor { RowMajor = MACE_HIP_ROW_MAJOR, ColMajor = MACE_HIP_COL_MAJOR };
+enum ActivationType { NOOP = MACE_HIP_ACT_NOOP, RELU = MACE_HIP_ACT_RELU,
+                      RELUX = MACE_HIP_ACT_RELUX };
+
+template <typename T> struct DataTypeToEnum;
+template <> struct DataTypeToEnum<float> { static const DataType value = DT_FLOAT; };
+template <> struct DataTypeToEnum<uint8_t> { static const DataType value = DT_UINT8; };
+template <> struct DataTypeToEnum<int32_t> { static const DataType value = DT_INT32; };
+
+// The part of mace::Tensor the delegators use (mace/core/tensor.h:147-256): typed data
+// pointer, shape, scale / zero point, weight flag.  Memory is owned by the caller; it is host
+// memory unless on_device is set.
+class Tensor {
+ public:
+  Tensor() = default;
+  Tensor(void *data, DataType dtype, std::vector<index_t> shape, float scale = 0.f,
+         int32_t zero_point = 0, bool is_weight = false, bool on_device = false)
+      : data_(data), dtype_(dtype), shape_(std::move(shape)), scale_(scale),
+        zero_point_(zero_point), is_weight_(is_weight), on_device_(on_device) {}
+  template <typename T> const T *data() const { return static_cast<const T *>(data_); }
+  template <typename T> T *mutable_data() { return static_cast<T *>(data_); }
+  const std::vector<index_t> &shape() const { return shape_; }
+  index_t dim_size() const { return static_cast<index_t>(shape_.size()); }
+  index_t dim(index_t i) const { return shape_[i]; }
+  index_t size() const {
+    return std::accumulate(shape_.begin(), shape_.end(), index_t(1), std::multiplies<index_t>());
+  }
+  DataType dtype() const { return dtype_; }
+  float scale() const { return scale_; }
+  int32_t zero_point() const { return zero_point_; }
+  void SetScale(float s) { scale_ = s; }
+  void SetZeroPoint(int32_t z) { zero_point_ = z; }
+  bool is_weight() const { return is_weight_; }
+  bool on_device() const { return on_device_; }
+  // The caller allocates; Resize only records the shape and checks it fits (capacity in
+  // elements, 0 = unchecked).
+  MaceStatus Resize(const std::vector<index_t> &shape, index_t capacity = 0) {
+    shape_ = shape;
+    if (capacity > 0 && size() > capacity) return MaceStatus::MACE_OUT_OF_RESOURCES;
+    return MaceStatus::MACE_SUCCESS;
+  }
+
+ private:
+  void *data_ = nullptr;
+  DataType dtype_ = DT_INVALID;
+  std::vector<index_t> shape_;
+  float scale_ = 0.f;
+  int32_t zero_point_ = 0;
+  bool is_weight_ = false;
+  bool on_device_ = false;
+};
+
+// mace/core/ops/op_context.h:24-41: what an op hands to its delegators.  Here it carries the
+// library context (stream + scratch arena) instead of a CPU runtime with a thread pool.
+class OpContext {
+ public:
+  explicit OpContext(mace_hip_ctx *ctx) : ctx_(ctx) {}
+  mace_hip_ctx *hip() const { return ctx_; }
+
+ private:
+  mace_hip_ctx *ctx_;
+};
+
+struct DelegatorParam {            // mace/core/ops/op_delegator.h:36-40
+  DelegatorParam() = default;
+  virtual ~DelegatorParam() = default;
+};
+class OpDelegator {                // mace/core/ops/op_delegator.h:42-55
+ public:
+  explicit OpDelegator(const DelegatorParam &) {}
+  virtual ~OpDelegator() = default;
+  template <class DerivedType, class ParamType>
+  static std::unique_ptr<OpDelegator> DefaultCreator(const DelegatorParam &param) {
+    return std::unique_ptr<OpDelegator>(
+        new DerivedType(static_cast<const ParamType &>(param)));
+  }
+};
+
+// ---- registry (mace/core/registry/op_delegator_registry.{h,cc}) --------------------------------
+typedef std::function<std::unique_ptr<OpDelegator>(const DelegatorParam &)> DelegatorCreator;
+static const char *const kDefaultTag = "general";
+
+struct DelegatorInfo {
+  DelegatorInfo(const char *name, DataType dt, RuntimeType rt, ImplType impl,
+                const char *in_tag = kDefaultTag)
+      : delegator_name(name), data_type(dt), runtime(rt), impl_type(impl), tag(in_tag) {}
+  std::string ToString() const {      // op_delegator_registry.cc:39-44
+    std::stringstream ss;
+    ss << delegator_name << "_" << data_type << "_" << runtime << "_" << impl_type << "_" << tag;
+    return ss.str();
+  }
+  bool operator==(const DelegatorInfo &o) const {
+    return runtime == o.runtime && impl_type == o.impl_type && data_type == o.data_type &&
+           delegator_name == o.delegator_name && tag == o.tag;
+  }
+  std::string delegator_name;
+  DataType data_type;
+  RuntimeType runtime;
+  ImplType impl_type;
+  std::string tag;
+};
+
+class OpDelegatorRegistry {
+ public:
+  // op_delegator_registry.cc:52-58: a duplicate key is a CHECK failure in the reference
+  MaceStatus Register(const DelegatorInfo &key, DelegatorCreator creator) {
+    if (registry_.count(key.ToString()) > 0) return MaceStatus::MACE_INVALID_ARGS;
+    registry_[key.ToString()] = std::move(creator);
+    return MaceStatus::MACE_SUCCESS;
+  }
+  // op_delegator_registry.cc:64-103: exact key, then NEON -> general tag -> REF (+tag) ->
+  // REF general.  The reference LOG(FATAL)s when nothing matches; an empty creator here.
+  DelegatorCreator GetCreator(const DelegatorInfo &key) const {
+    auto find = [&](const DelegatorInfo &k) { return registry_.find(k.ToString()); };
+    auto it = find(key);
+    if (it != registry_.end()) return it->second;
+    DelegatorInfo info = key;
+    if (key.impl_type == ImplType::NEON) {
+      if (info.tag != kDefaultTag) {
+        info.tag = kDefaultTag;
+        if ((it = find(info)) != registry_.end()) return it->second;
+        info.tag = key.tag;
+      }
+      info.impl_type = ImplType::REF;
+      if ((it = find(info)) != registry_.end()) return it->second;
+    }
+    if (info.tag != kDefaultTag) {
+      info.tag = kDefaultTag;
+      if ((it = find(info)) != registry_.end()) return it->second;
+    }
+    return DelegatorCreator();
+  }
+
+ private:
+  std::unordered_map<std::string, DelegatorCreator> registry_;
+};
+
+#define MACE_HIP_DELEGATOR_KEY(name, rt, DT, impl) \
+  ::mace_hip::DelegatorInfo(#name, ::mace_hip::DataTypeToEnum<DT>::value, rt, impl)
+#define MACE_HIP_DELEGATOR_KEY_EX(name, rt, DT, impl, tag) \
+  ::mace_hip::DelegatorInfo(#name, ::mace_hip::DataTypeToEnum<DT>::value, rt, impl, #tag)
+#define MACE_HIP_REGISTER_DELEGATOR(registry, class_name, param_name, key) \
+  (registry)->Register(key, ::mace_hip::OpDelegator::DefaultCreator<class_name, param_name>)
+
+// ---- abstract delegators ---------------------------------------------------------------------------
+namespace delegator {
+
+struct GemmParam : public DelegatorParam {     // mace/ops/delegator/gemm.h:28-33
+  explicit GemmParam(const bool should_cache_pack = false)
+      : should_cache_pack_(should_cache_pack) {}
+  const bool should_cache_pack_;
+};
+
+class Gemm : public OpDelegator {              // mace/ops/delegator/gemm.h:35-70
+ public:
+  explicit Gemm(const GemmParam &param) : OpDelegator(param) {}
+  virtual MaceStatus Compute(const OpContext *context, const Tensor *lhs, const Tensor *rhs,
+                             const index_t batch, const index_t rows, const index_t cols,
+                             const index_t depth, const MatrixMajor lhs_major,
+                             const MatrixMajor rhs_major, const MatrixMajor output_major,
+                             const bool lhs_batched, const bool rhs_batched,
+                             Tensor *output) = 0;
+  // Original matrix before transpose has row-major
+  virtual MaceStatus Compute(const OpContext *context, const Tensor *lhs, const Tensor *rhs,
+                             const index_t batch, const index_t lhs_rows,
+                             const index_t lhs_cols, const index_t rhs_rows,
+                             const index_t rhs_cols, const bool transpose_lhs,
+                             const bool transpose_rhs, const bool transpose_out,
+                             const bool lhs_batched, const bool rhs_batched,
+                             Tensor *output) = 0;
+};
+
+class Gemv : public OpDelegator {              // mace/ops/delegator/gemv.h:27-46
+ public:
+  explicit Gemv(const DelegatorParam &param) : OpDelegator(param) {}
+  // Always row-major after transpose
+  virtual MaceStatus Compute(const OpContext *context, const Tensor *lhs, const Tensor *rhs,
+                             const Tensor *bias, const index_t batch,
+                             const index_t lhs_height, const index_t lhs_width,
+                             const bool lhs_batched, const bool rhs_batched,
+                             Tensor *output) = 0;
+};
+
+struct Conv2dParam : public DelegatorParam {   // mace/ops/delegator/conv_2d.h:37-58 (subset)
+  Conv2dParam() = default;
+};
+class Conv2d : public OpDelegator {            // mace/ops/delegator/conv_2d.h:60-82
+ public:
+  explicit Conv2d(const Conv2dParam &param) : OpDelegator(param) {}
+  virtual MaceStatus Compute(const OpContext *context, const Tensor *input,
+                             const Tensor *filter, Tensor *output) = 0;
+};
+
+}  // namespace delegator
+
+// ---- the GPU delegators --------------------------------------------------------------------------------
+namespace hip {
+
+template <typename T> class Gemm;
+template <>
+class Gemm<float> : public delegator::Gemm {   // replaces ref::Gemm<float> / arm::Gemm<float>
+ public:
+  explicit Gemm(const delegator::GemmParam &param) : delegator::Gemm(param) {}
+  MaceStatus Compute(const OpContext *context, const Tensor *lhs, const Tensor *rhs,
+                     const index_t batch, const index_t rows, const index_t cols,
+                     const index_t depth, const MatrixMajor lhs_major,
+                     const MatrixMajor rhs_major, const MatrixMajor output_major,
+                     const bool lhs_batched, const bool rhs_batched,
+                     Tensor *output) override {
+    auto fn = output->on_device() ? mace_hip_gemm_f32 : mace_hip_gemm_f32_host;
+    return ToStatus(fn(context->hip(), lhs->data<float>(), rhs->data<float>(), batch, rows,
+                       cols, depth, lhs_major, rhs_major, output_major, lhs_batched,
+                       rhs_batched, output->mutable_data<float>()));
+  }
+  MaceStatus Compute(const OpContext *context, const Tensor *lhs, const Tensor *rhs,
+                     const index_t batch, const index_t lhs_rows, const index_t lhs_cols,
+                     const index_t rhs_rows, const index_t rhs_cols, const bool transpose_lhs,
+                     const bool transpose_rhs, const bool transpose_out,
+                     const bool lhs_batched, const bool rhs_batched,
+                     Tensor *output) override {
+    // mace/ops/ref/gemm.cc:122-145
+    const index_t rows = transpose_lhs ? lhs_cols : lhs_rows;
+    const index_t depth = transpose_lhs ? lhs_rows : lhs_cols;
+    const index_t cols = transpose_rhs ? rhs_rows : rhs_cols;
+    const index_t depth2 = transpose_rhs ? rhs_cols : rhs_rows;
+    if (depth != depth2) return MaceStatus::MACE_INVALID_ARGS;
+    return Compute(context, lhs, rhs, batch, rows, cols, depth,
+                   transpose_lhs ? ColMajor : RowMajor, transpose_rhs ? ColMajor : RowMajor,
+                   transpose_out ? ColMajor : RowMajor, lhs_batched, rhs_batched, output);
+  }
+};
+
+template <typename T> class Gemv;
+template <>
+class Gemv<float> : public delegator::Gemv {   // replaces ref::Gemv<float> / arm::Gemv<float>
+ public:
+  explicit Gemv(const DelegatorParam &param) : delegator::Gemv(param) {}
+  MaceStatus Compute(const OpContext *context, const Tensor *lhs, const Tensor *rhs,
+                     const Tensor *bias, const index_t batch, const index_t lhs_height,
+                     const index_t lhs_width, const bool lhs_batched, const bool rhs_batched,
+                     Tensor *output) override {
+    auto fn = output->on_device() ? mace_hip_gemv_f32 : mace_hip_gemv_f32_host;
+    return ToStatus(fn(context->hip(), lhs->data<float>(), rhs->data<float>(),
+                       bias ? bias->data<float>() : nullptr, batch, lhs_height, lhs_width,
+                       lhs_batched, rhs_batched, output->mutable_data<float>()));
+  }
+};
+// Replaces ref::q8::Gemv<uint8_t> (requant_mode REF) / arm::q8::Gemv<uint8_t> (NEON).
+template <>
+class Gemv<uint8_t> : public delegator::Gemv {
+ public:
+  explicit Gemv(const DelegatorParam &param, int requant_mode = MACE_HIP_REQUANT_NEON)
+      : delegator::Gemv(param), requant_mode_(requant_mode) {}
+  MaceStatus Compute(const OpContext *context, const Tensor *lhs, const Tensor *rhs,
+                     const Tensor *bias, const index_t batch, const index_t lhs_height,
+                     const index_t lhs_width, const bool lhs_batched, const bool rhs_batched,
+                     Tensor *output) override {
+    auto fn = output->on_device() ? mace_hip_gemv_q8_u8 : mace_hip_gemv_q8_u8_host;
+    return ToStatus(fn(context->hip(), lhs->data<uint8_t>(), rhs->data<uint8_t>(),
+                       bias ? bias->data<int32_t>() : nullptr, batch, lhs_height, lhs_width,
+                       lhs_batched, rhs_batched, lhs->zero_point(), rhs->zero_point(),
+                       lhs->scale(), rhs->scale(), output->scale(), output->zero_point(),
+                       requant_mode_, output->mutable_data<uint8_t>()));
+  }
+
+ private:
+  int requant_mode_;
+};
+template <>
+class Gemv<int32_t> : public delegator::Gemv {   // replaces ref::q8::Gemv<int32_t>
+ public:
+  explicit Gemv(const DelegatorParam &param) : delegator::Gemv(param) {}
+  MaceStatus Compute(const OpContext *context, const Tensor *lhs, const Tensor *rhs,
+                     const Tensor *bias, const index_t batch, const index_t lhs_height,
+                     const index_t lhs_width, const bool lhs_batched, const bool rhs_batched,
+                     Tensor *output) override {
+    auto fn = output->on_device() ? mace_hip_gemv_q8_i32 : mace_hip_gemv_q8_i32_host;
+    return ToStatus(fn(context->hip(), lhs->data<uint8_t>(), rhs->data<uint8_t>(),
+                       bias ? bias->data<int32_t>() : nullptr, batch, lhs_height, lhs_width,
+                       lhs_batched, rhs_batched, lhs->zero_point(), rhs->zero_point(),
+                       output->mutable_data<int32_t>()));
+  }
+};
+
+// Replaces arm::Conv2dK1x1<float> (mace/ops/arm/base/conv_2d_1x1.cc:27-72): NCHW input
+// {n, cin, h, w}, OIHW filter {cout, cin, 1, 1}, output {n, cout, h, w}; the op adds bias and
+// activation afterwards (see Conv2dK1x1Op below), so the delegator itself computes the Gemm.
+template <typename T> class Conv2dK1x1;
+template <>
+class Conv2dK1x1<float> : public delegator::Conv2d {
+ public:
+  explicit Conv2dK1x1(const delegator::Conv2dParam &param) : delegator::Conv2d(param) {}
+  MaceStatus Compute(const OpContext *context, const Tensor *input, const Tensor *filter,
+                     Tensor *output) override {
+    if (input->dim_size() != 4 || filter->dim_size() != 4 || filter->dim(2) != 1 ||
+        filter->dim(3) != 1 || filter->dim(1) != input->dim(1))
+      return MaceStatus::MACE_INVALID_ARGS;
+    const index_t n = input->dim(0), cin = input->dim(1), hw = input->dim(2) * input->dim(3);
+    const index_t cout = filter->dim(0);
+    MaceStatus st = output->Resize({n, cout, input->dim(2), input->dim(3)});
+    if (st != MaceStatus::MACE_SUCCESS) return st;
+    auto fn = output->on_device() ? mace_hip_conv1x1_f32_nchw : mace_hip_conv1x1_f32_nchw_host;
+    return ToStatus(fn(context->hip(), input->data<float>(), filter->data<float>(), nullptr, n,
+                       cin, hw, cout, MACE_HIP_ACT_NOOP, 0.f, output->mutable_data<float>()));
+  }
+};
+
+// mace/ops/registry/op_delegators_registry.cc:87-143 registers ref:: and arm:: delegators; this
+// registers the GPU ones under the keys the ops ask for (kCpuImplType), in their place.
+inline MaceStatus RegisterAllHipDelegators(OpDelegatorRegistry *registry) {
+  MaceStatus st = MACE_HIP_REGISTER_DELEGATOR(
+      registry, Gemm<float>, delegator::GemmParam,
+      MACE_HIP_DELEGATOR_KEY(Gemm, RT_CPU, float, kCpuImplType));
+  if (st != MaceStatus::MACE_SUCCESS) return st;
+  st = MACE_HIP_REGISTER_DELEGATOR(registry, Gemv<float>, DelegatorParam,
+                                   MACE_HIP_DELEGATOR_KEY(Gemv, RT_CPU, float, kCpuImplType));
+  if (st != MaceStatus::MACE_SUCCESS) return st;
+  st = MACE_HIP_REGISTER_DELEGATOR(registry, Gemv<uint8_t>, DelegatorParam,
+                                   MACE_HIP_DELEGATOR_KEY(Gemv, RT_CPU, uint8_t, kCpuImplType));
+  if (st != MaceStatus::MACE_SUCCESS) return st;
+  st = MACE_HIP_REGISTER_DELEGATOR(registry, Gemv<int32_t>, DelegatorParam,
+                                   MACE_HIP_DELEGATOR_KEY(Gemv, RT_CPU, int32_t, kCpuImplType));
+  if (st != MaceStatus::MACE_SUCCESS) return st;
+  return MACE_HIP_REGISTER_DELEGATOR(
+      registry, Conv2dK1x1<float>, delegator::Conv2dParam,
+      MACE_HIP_DELEGATOR_KEY_EX(Conv2d, RT_CPU, float, kCpuImplType, K1x1));
+}
+
+}  // namespace hip
+
+// ---- ops: shape derivation and dispatch ------------------------------------------------------------------
+namespace ops {
+
+struct MatMulShape {
+  index_t rows, cols, depth, batch;
+  index_t lhs_rows, lhs_cols, rhs_rows, rhs_cols;
+  bool lhs_batched, rhs_batched;
+  std::vector<index_t> output_shape;
+};
+
+// MatMulOpBase::Validate (mace/ops/matmul.cc:55-83) + the head of Run (:117-154)
+inline MaceStatus MatMulInferShape(const Tensor *A, const Tensor *B, bool transpose_a,
+                                   bool transpose_b, MatMulShape *s) {
+  const index_t lhs_rank = A->dim_size(), rhs_rank = B->dim_size();
+  if (lhs_rank < 2 || rhs_rank < 2) return MaceStatus::MACE_INVALID_ARGS;
+  if (lhs_rank == rhs_rank) {
+    for (index_t i = 0; i < lhs_rank - 2; ++i)
+      if (A->dim(i) != B->dim(i)) return MaceStatus::MACE_INVALID_ARGS;
+  } else if (lhs_rank != 2 && rhs_rank != 2) {
+    return MaceStatus::MACE_INVALID_ARGS;
+  }
+  s->lhs_rows = A->dim(lhs_rank - 2); s->lhs_cols = A->dim(lhs_rank - 1);
+  s->rhs_rows = B->dim(rhs_rank - 2); s->rhs_cols = B->dim(rhs_rank - 1);
+  const index_t lhs_depth = transpose_a ? s->lhs_rows : s->lhs_cols;
+  const index_t rhs_depth = transpose_b ? s->rhs_cols : s->rhs_rows;
+  if (lhs_depth != rhs_depth) return MaceStatus::MACE_INVALID_ARGS;
+  s->rows = transpose_a ? s->lhs_cols : s->lhs_rows;
+  s->cols = transpose_b ? s->rhs_rows : s->rhs_cols;
+  s->depth = lhs_depth;
+  auto lead = [](const Tensor *t) {
+    return std::accumulate(t->shape().begin(), t->shape().end() - 2, index_t(1),
+                           std::multiplies<index_t>());
+  };
+  if (lhs_rank >= rhs_rank) { s->output_shape = A->shape(); s->batch = lead(A); }
+  else { s->output_shape = B->shape(); s->batch = lead(B); }
+  s->output_shape[s->output_shape.size() - 2] = s->rows;
+  s->output_shape[s->output_shape.size() - 1] = s->cols;
+  s->lhs_batched = !(lhs_rank < rhs_rank);
+  s->rhs_batched = !(rhs_rank < lhs_rank);
+  return MaceStatus::MACE_SUCCESS;
+}
+
+// MatMulOp<RT_CPU, float>::Run (mace/ops/matmul.cc:110-215).  The optional bias of the Gemm
+// branch (:195-211) is a host loop in the reference and stays one here (host tensors only).
+class MatMulOpFloat {
+ public:
+  MatMulOpFloat(OpDelegatorRegistry *registry, bool transpose_a, bool transpose_b)
+      : transpose_a_(transpose_a), transpose_b_(transpose_b) {
+    auto gc = registry->GetCreator(MACE_HIP_DELEGATOR_KEY(Gemm, RT_CPU, float, kCpuImplType));
+    auto vc = registry->GetCreator(MACE_HIP_DELEGATOR_KEY(Gemv, RT_CPU, float, kCpuImplType));
+    if (gc) gemm_.reset(static_cast<delegator::Gemm *>(gc(delegator::GemmParam()).release()));
+    if (vc) gemv_.reset(static_cast<delegator::Gemv *>(vc(DelegatorParam()).release()));
+  }
+  MaceStatus Run(OpContext *context, const Tensor *lhs, const Tensor *rhs, const Tensor *bias,
+                 Tensor *C) {
+    if (!gemm_ || !gemv_) return MaceStatus::MACE_RUNTIME_ERROR;
+    MatMulShape s;
+    MaceStatus st = MatMulInferShape(lhs, rhs, transpose_a_, transpose_b_, &s);
+    if (st != MaceStatus::MACE_SUCCESS) return st;
+    if ((st = C->Resize(s.output_shape)) != MaceStatus::MACE_SUCCESS) return st;
+    if (s.rows == 1 && transpose_b_)
+      return gemv_->Compute(context, rhs, lhs, bias, s.batch, s.cols, s.depth, s.rhs_batched,
+                            s.lhs_batched, C);
+    if (s.cols == 1 && !transpose_a_)
+      return gemv_->Compute(context, lhs, rhs, bias, s.batch, s.rows, s.depth, s.lhs_batched,
+                            s.rhs_batched, C);
+    st = gemm_->Compute(context, lhs, rhs, s.batch, s.lhs_rows, s.lhs_cols, s.rhs_rows,
+                        s.rhs_cols, transpose_a_, transpose_b_, false, s.lhs_batched,
+                        s.rhs_batched, C);
+    if (st == MaceStatus::MACE_SUCCESS && bias != nullptr) {
+      if (bias->dim_size() != 1 || bias->dim(0) != s.cols || C->on_device())
+        return MaceStatus::MACE_INVALID_ARGS;
+      const float *b = bias->data<float>();
+      float *c = C->mutable_data<float>();
+      for (index_t i = 0; i < s.batch * s.rows; ++i)
+        for (index_t w = 0; w < s.cols; ++w) c[i * s.cols + w] += b[w];
+    }
+    return st;
+  }
+
+ private:
+  bool transpose_a_, transpose_b_;
+  std::unique_ptr<delegator::Gemm> gemm_;
+  std::unique_ptr<delegator::Gemv> gemv_;
+};
+
+// MatMulOp<RT_CPU, uint8_t>::Run (mace/ops/matmul.cc:397-483) with MatMulFixpointImpl
+// (:227-394): transposes become Col orders, the result is RowMajor, no bias; the uint8 result
+// uses the pipeline MakeNoBias(A.scale, B.scale, C.scale, C.zero_point), the int32 result
+// sets C.scale = A.scale * B.scale and C.zero_point = 0.  The gemmlowp call is not behind a
+// delegator in the reference, so the op calls the C ABI directly.
+class MatMulOpQuant {
+ public:
+  MatMulOpQuant(bool transpose_a, bool transpose_b, DataType output_type)
+      : transpose_a_(transpose_a), transpose_b_(transpose_b), output_type_(output_type) {}
+  MaceStatus Run(OpContext *context, const Tensor *A, const Tensor *B, Tensor *C) {
+    MatMulShape s;
+    MaceStatus st = MatMulInferShape(A, B, transpose_a_, transpose_b_, &s);
+    if (st != MaceStatus::MACE_SUCCESS) return st;
+    if ((st = C->Resize(s.output_shape)) != MaceStatus::MACE_SUCCESS) return st;
+    const int a_order = transpose_a_ ? MACE_HIP_COL_MAJOR : MACE_HIP_ROW_MAJOR;
+    const int b_order = transpose_b_ ? MACE_HIP_COL_MAJOR : MACE_HIP_ROW_MAJOR;
+    if (output_type_ == DT_INT32) {
+      C->SetScale(A->scale() * B->scale());
+      C->SetZeroPoint(0);
+      auto fn = C->on_device() ? mace_hip_gemm_q8_i32 : mace_hip_gemm_q8_i32_host;
+      return ToStatus(fn(context->hip(), A->data<uint8_t>(), a_order, B->data<uint8_t>(),
+                         b_order, C->mutable_data<int32_t>(), MACE_HIP_ROW_MAJOR, s.batch,
+                         s.rows, s.depth, s.cols, s.lhs_batched, s.rhs_batched,
+                         -A->zero_point(), -B->zero_point()));
+    }
+    int32_t multiplier = 0;
+    int shift = 0;
+    if (mace_hip_get_output_multiplier_and_shift(A->scale(), B->scale(), C->scale(),
+                                                 &multiplier, &shift) != MACE_HIP_SUCCESS)
+      return MaceStatus::MACE_INVALID_ARGS;
+    auto fn = C->on_device() ? mace_hip_gemm_q8_u8 : mace_hip_gemm_q8_u8_host;
+    return ToStatus(fn(context->hip(), A->data<uint8_t>(), a_order, B->data<uint8_t>(), b_order,
+                       C->mutable_data<uint8_t>(), MACE_HIP_ROW_MAJOR, s.batch, s.rows,
+                       s.depth, s.cols, s.lhs_batched, s.rhs_batched, -A->zero_point(),
+                       -B->zero_point(), nullptr, multiplier, shift, C->zero_point(), 0, 255));
+  }
+
+ private:
+  bool transpose_a_, transpose_b_;
+  DataType output_type_;
+};
+
+// FullyConnectedOp<RT_CPU, uint8_t>::Run (mace/ops/fully_connected.cc:141-179) and the float op
+// (:82-121) up to the Gemv call: weight OIHW, output {N,1,1,O} (uint8) / {N,O,1,1} (float).
+template <typename T>
+class FullyConnectedOp {
+ public:
+  explicit FullyConnectedOp(OpDelegatorRegistry *registry) {
+    auto vc = registry->GetCreator(MACE_HIP_DELEGATOR_KEY(Gemv, RT_CPU, T, kCpuImplType));
+    if (vc) gemv_.reset(static_cast<delegator::Gemv *>(vc(DelegatorParam()).release()));
+  }
+  MaceStatus Run(OpContext *context, const Tensor *input, const Tensor *weight,
+                 const Tensor *bias, Tensor *output) {
+    if (!gemv_) return MaceStatus::MACE_RUNTIME_ERROR;
+    if (input->dim_size() != 4 || weight->dim_size() != 4 || input->dim(1) != weight->dim(1) ||
+        input->dim(2) != weight->dim(2) || input->dim(3) != weight->dim(3))
+      return MaceStatus::MACE_INVALID_ARGS;
+    if (bias && weight->dim(0) != bias->dim(0)) return MaceStatus::MACE_INVALID_ARGS;
+    std::vector<index_t> out_shape =
+        std::is_same<T, uint8_t>::value
+            ? std::vector<index_t>{input->dim(0), 1, 1, weight->dim(0)}
+            : std::vector<index_t>{input->dim(0), weight->dim(0), 1, 1};
+    MaceStatus st = output->Resize(out_shape);
+    if (st != MaceStatus::MACE_SUCCESS) return st;
+    const index_t input_size = weight->dim(1) * weight->dim(2) * weight->dim(3);
+    return gemv_->Compute(context, weight, input, bias, input->dim(0), weight->dim(0),
+                          input_size, false, true, output);
+  }
+
+ private:
+  std::unique_ptr<delegator::Gemv> gemv_;
+};
+
+// Conv2dOp<RT_CPU, uint8_t>::Run for a 1x1 / stride 1 / dilation 1 filter
+// (mace/ops/conv_2d.cc:201-318): NHWC input, OHWI filter, NHWC output.  UNSUPPORTED for any
+// other filter (the reference's im2col path is outside this library).
+class Conv2dK1x1OpQuant {
+ public:
+  Conv2dK1x1OpQuant(int clamp_min = 0, int clamp_max = 255)
+      : clamp_min_(clamp_min), clamp_max_(clamp_max) {}
+  MaceStatus Run(OpContext *context, const Tensor *input, const Tensor *filter,
+                 const Tensor *bias, Tensor *output) {
+    if (input->dim_size() != 4 || filter->dim_size() != 4) return MaceStatus::MACE_INVALID_ARGS;
+    if (filter->dim(1) != 1 || filter->dim(2) != 1) return MaceStatus::MACE_UNSUPPORTED;
+    if (filter->dim(3) != input->dim(3)) return MaceStatus::MACE_INVALID_ARGS;
+    if (bias && bias->dim(0) != filter->dim(0)) return MaceStatus::MACE_INVALID_ARGS;
+    MaceStatus st =
+        output->Resize({input->dim(0), input->dim(1), input->dim(2), filter->dim(0)});
+    if (st != MaceStatus::MACE_SUCCESS) return st;
+    auto fn = output->on_device() ? mace_hip_conv1x1_q8_nhwc : mace_hip_conv1x1_q8_nhwc_host;
+    return ToStatus(fn(context->hip(), input->data<uint8_t>(), filter->data<uint8_t>(),
+                       bias ? bias->data<int32_t>() : nullptr, input->dim(0), input->dim(1),
+                       input->dim(2), input->dim(3), filter->dim(0), input->scale(),
+                       input->zero_point(), filter->scale(), filter->zero_point(),
+                       bias ? bias->scale() : 0.f, output->scale(), output->zero_point(),
+                       clamp_min_, clamp_max_, output->mutable_data<uint8_t>()));
+  }
+
+ private:
+  int clamp_min_, clamp_max_;
+};
+
+}  // namespace ops
+}  // namespace mace_hip
+
+#endif  // MACE_HIP_DELEGATOR_H_

@@ -1,0 +1,186 @@
+// C++ tests of the delegator adapter (include/mace_hip_delegator.h).
+//   test_delegator.bin registry   -- registry keys and fallback rule; needs no GPU
+//   test_delegator.bin compute    -- ops through the registry on the GPU, checked against the
+//                                    reference's golden vectors and the CPU oracle
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <vector>
+
+#include "mace_hip_delegator.h"
+#include "../../oracle/mace_oracle.h"
+
+using namespace mace_hip;
+
+static int g_fail = 0;
+#define EXPECT(cond)                                                              \
+  do {                                                                            \
+    if (!(cond)) { printf("FAIL %s:%d: %s\n", __FILE__, __LINE__, #cond); ++g_fail; } \
+  } while (0)
+
+struct DummyGemv : public delegator::Gemv {
+  explicit DummyGemv(const DelegatorParam &p) : delegator::Gemv(p) {}
+  MaceStatus Compute(const OpContext *, const Tensor *, const Tensor *, const Tensor *,
+                     const index_t, const index_t, const index_t, const bool, const bool,
+                     Tensor *) override { return MaceStatus::MACE_UNSUPPORTED; }
+};
+
+static int test_registry() {
+  OpDelegatorRegistry reg;
+  // key string: name_dtype_runtime_impl_tag (op_delegator_registry.cc:39-44)
+  EXPECT(MACE_HIP_DELEGATOR_KEY(Gemm, RT_CPU, float, REF).ToString() == "Gemm_1_0_0_general");
+  EXPECT(MACE_HIP_DELEGATOR_KEY_EX(Conv2d, RT_CPU, float, NEON, K1x1).ToString() ==
+         "Conv2d_1_0_1_K1x1");
+  EXPECT(hip::RegisterAllHipDelegators(&reg) == MaceStatus::MACE_SUCCESS);
+  // duplicate keys are rejected (a CHECK failure in the reference, :52-58)
+  EXPECT(hip::RegisterAllHipDelegators(&reg) == MaceStatus::MACE_INVALID_ARGS);
+  EXPECT((bool)reg.GetCreator(MACE_HIP_DELEGATOR_KEY(Gemm, RT_CPU, float, kCpuImplType)));
+  EXPECT((bool)reg.GetCreator(MACE_HIP_DELEGATOR_KEY(Gemv, RT_CPU, uint8_t, kCpuImplType)));
+  // fallback: NEON + tag -> NEON general -> REF + tag -> REF general (:64-103)
+  EXPECT((bool)reg.GetCreator(MACE_HIP_DELEGATOR_KEY(Gemv, RT_CPU, float, NEON)));
+  EXPECT((bool)reg.GetCreator(MACE_HIP_DELEGATOR_KEY_EX(Gemv, RT_CPU, float, NEON, K3x3)));
+  EXPECT((bool)reg.GetCreator(MACE_HIP_DELEGATOR_KEY_EX(Conv2d, RT_CPU, float, NEON, K1x1)));
+  // a tagged-only registration does not serve the general key
+  EXPECT(!reg.GetCreator(MACE_HIP_DELEGATOR_KEY(Conv2d, RT_CPU, float, REF)));
+  EXPECT(!reg.GetCreator(MACE_HIP_DELEGATOR_KEY(Gemm, RT_OPENCL, float, REF)));
+  // an exact NEON registration wins over the REF fallback
+  EXPECT(MACE_HIP_REGISTER_DELEGATOR(&reg, DummyGemv, DelegatorParam,
+                                     MACE_HIP_DELEGATOR_KEY(Gemv, RT_CPU, float, NEON)) ==
+         MaceStatus::MACE_SUCCESS);
+  auto c = reg.GetCreator(MACE_HIP_DELEGATOR_KEY_EX(Gemv, RT_CPU, float, NEON, K3x3));
+  std::unique_ptr<OpDelegator> d = c(DelegatorParam());
+  EXPECT(dynamic_cast<DummyGemv *>(d.get()) != nullptr);
+  // MatMul shape derivation (matmul.cc:55-83, 117-154)
+  ops::MatMulShape s;
+  Tensor a(nullptr, DT_FLOAT, {2, 3, 31, 61}), b(nullptr, DT_FLOAT, {61, 67});
+  EXPECT(ops::MatMulInferShape(&a, &b, false, false, &s) == MaceStatus::MACE_SUCCESS);
+  EXPECT(s.batch == 6 && s.rows == 31 && s.cols == 67 && s.depth == 61 && s.lhs_batched &&
+         !s.rhs_batched && s.output_shape == (std::vector<index_t>{2, 3, 31, 67}));
+  Tensor a3(nullptr, DT_FLOAT, {2, 3, 4}), b3(nullptr, DT_FLOAT, {3, 4, 5});
+  EXPECT(ops::MatMulInferShape(&a3, &b3, false, false, &s) == MaceStatus::MACE_INVALID_ARGS);
+  Tensor a1(nullptr, DT_FLOAT, {3}), b2(nullptr, DT_FLOAT, {3, 2});
+  EXPECT(ops::MatMulInferShape(&a1, &b2, false, false, &s) == MaceStatus::MACE_INVALID_ARGS);
+  Tensor a2(nullptr, DT_FLOAT, {3, 4}), b4(nullptr, DT_FLOAT, {5, 6});
+  EXPECT(ops::MatMulInferShape(&a2, &b4, false, false, &s) == MaceStatus::MACE_INVALID_ARGS);
+  EXPECT(ops::MatMulInferShape(&a2, &b4, true, false, &s) == MaceStatus::MACE_INVALID_ARGS);
+  Tensor b5(nullptr, DT_FLOAT, {6, 4});
+  EXPECT(ops::MatMulInferShape(&a2, &b5, false, true, &s) == MaceStatus::MACE_SUCCESS);
+  EXPECT(s.rows == 3 && s.cols == 6 && s.depth == 4 && s.batch == 1);
+  return g_fail;
+}
+
+static bool near(const std::vector<float> &got, const std::vector<float> &want) {
+  if (got.size() != want.size()) return false;
+  for (size_t i = 0; i < got.size(); ++i)
+    if (std::fabs(got[i] - want[i]) > 1e-5 * std::fabs(want[i]) + 1e-8 + 1e-5) return false;
+  return true;
+}
+
+static int test_compute() {
+  mace_hip_ctx *hctx = nullptr;
+  if (mace_hip_ctx_create(0, &hctx) != MACE_HIP_SUCCESS) { printf("FAIL: no context\n"); return 1; }
+  OpContext context(hctx);
+  OpDelegatorRegistry reg;
+  EXPECT(hip::RegisterAllHipDelegators(&reg) == MaceStatus::MACE_SUCCESS);
+
+  {  // matmul_test.cc:56-58 SimpleCPU
+    std::vector<float> a = {1, 2, 3, 4, 5, 6}, b = {1, 2, 3, 4, 5, 6}, c(4);
+    Tensor A(a.data(), DT_FLOAT, {1, 2, 3}), B(b.data(), DT_FLOAT, {1, 3, 2}), C(c.data(), DT_FLOAT, {});
+    ops::MatMulOpFloat op(&reg, false, false);
+    EXPECT(op.Run(&context, &A, &B, nullptr, &C) == MaceStatus::MACE_SUCCESS);
+    EXPECT(C.shape() == (std::vector<index_t>{1, 2, 2}));
+    EXPECT(near(c, {22, 28, 49, 64}));
+    // rows == 1 && transpose_b -> Gemv branch with bias as initial value (matmul.cc:158-168)
+    std::vector<float> x = {1, 2, 3}, w = {1, 0, 1, 2, 2, 2}, bias = {10, 20}, y(2);
+    Tensor X(x.data(), DT_FLOAT, {1, 3}), W(w.data(), DT_FLOAT, {2, 3}), Bi(bias.data(), DT_FLOAT, {2}),
+        Y(y.data(), DT_FLOAT, {});
+    ops::MatMulOpFloat opv(&reg, false, true);
+    EXPECT(opv.Run(&context, &X, &W, &Bi, &Y) == MaceStatus::MACE_SUCCESS);
+    EXPECT(near(y, {14, 32}));
+    // Gemm branch with per-column bias (matmul.cc:195-211)
+    std::vector<float> bias2 = {0.5f, -1.f}, c2(4);
+    Tensor Bi2(bias2.data(), DT_FLOAT, {2}), C2(c2.data(), DT_FLOAT, {});
+    EXPECT(op.Run(&context, &A, &B, &Bi2, &C2) == MaceStatus::MACE_SUCCESS);
+    EXPECT(near(c2, {22.5f, 27, 49.5f, 63}));
+  }
+  {  // fully_connected_test.cc:78-81 SimpleCPU (second case) and :89-93 WithBatch
+    std::vector<float> x = {1, 2, 3, 4, 5, 6, 7, 8, 9, 10};
+    std::vector<float> w = {1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 10, 20, 30, 40, 50, 60, 70, 80, 90, 100};
+    std::vector<float> bias = {2, 3}, y(2);
+    Tensor X(x.data(), DT_FLOAT, {1, 1, 2, 5}), W(w.data(), DT_FLOAT, {2, 1, 2, 5}, 0, 0, true),
+        Bi(bias.data(), DT_FLOAT, {2}), Y(y.data(), DT_FLOAT, {});
+    ops::FullyConnectedOp<float> fc(&reg);
+    EXPECT(fc.Run(&context, &X, &W, &Bi, &Y) == MaceStatus::MACE_SUCCESS);
+    EXPECT(Y.shape() == (std::vector<index_t>{1, 2, 1, 1}));
+    EXPECT(near(y, {387, 3853}));
+    Tensor Wbad(w.data(), DT_FLOAT, {2, 1, 5, 2});
+    EXPECT(fc.Run(&context, &X, &Wbad, &Bi, &Y) == MaceStatus::MACE_INVALID_ARGS);
+  }
+  {  // conv_2d_test.cc:1240-1275: the quantized known answer 230, as a 1x1 conv over 18 channels
+    std::vector<uint8_t> f = {102, 150, 123, 135, 1, 216, 137, 47, 53, 75, 145, 130, 171, 62, 255, 122, 72, 211};
+    std::vector<uint8_t> in = {1, 75, 117, 161, 127, 119, 94, 151, 203, 151, 84, 61, 55, 142, 113, 139, 3, 255};
+    std::vector<int32_t> bias = {2};
+    std::vector<uint8_t> out(1);
+    Tensor F(f.data(), DT_UINT8, {1, 1, 1, 18}, 0.0226f, 127, true), I(in.data(), DT_UINT8, {1, 1, 1, 18}, 0.0204f, 93),
+        Bi(bias.data(), DT_INT32, {1}, 0.00046104f, 0, true), O(out.data(), DT_UINT8, {}, 0.000711f, 1);
+    ops::Conv2dK1x1OpQuant conv;
+    EXPECT(conv.Run(&context, &I, &F, &Bi, &O) == MaceStatus::MACE_SUCCESS);
+    EXPECT(out[0] == 230);
+    Tensor F3(f.data(), DT_UINT8, {1, 3, 3, 2}, 0.0226f, 127, true);
+    EXPECT(conv.Run(&context, &I, &F3, &Bi, &O) == MaceStatus::MACE_UNSUPPORTED);
+  }
+  {  // quantized MatMul and FullyConnected vs the oracle, seeded
+    std::mt19937 rng(7);
+    const index_t batch = 3, rows = 31, depth = 61, cols = 67;
+    std::vector<uint8_t> a(batch * depth * rows), b(cols * depth);
+    for (auto &v : a) v = rng() & 255;
+    for (auto &v : b) v = rng() & 255;
+    // transpose_a = transpose_b = true, rhs not batched (matmul_test.cc:425)
+    Tensor A(a.data(), DT_UINT8, {batch, depth, rows}, 0.02f, 77), B(b.data(), DT_UINT8, {cols, depth}, 0.015f, 201);
+    std::vector<int32_t> c32(batch * rows * cols), want32(c32.size());
+    Tensor C32(c32.data(), DT_INT32, {});
+    ops::MatMulOpQuant op32(true, true, DT_INT32);
+    EXPECT(op32.Run(&context, &A, &B, &C32) == MaceStatus::MACE_SUCCESS);
+    EXPECT(C32.zero_point() == 0 && C32.scale() == 0.02f * 0.015f);
+    orc_q8_gemm_i32(a.data(), b.data(), batch, rows, cols, depth, ORC_COL_MAJOR, ORC_COL_MAJOR,
+                    ORC_ROW_MAJOR, 1, 0, -77, -201, want32.data(), 4);
+    EXPECT(c32 == want32);
+    std::vector<uint8_t> c8(c32.size()), want8(c32.size());
+    Tensor C8(c8.data(), DT_UINT8, {}, 40.f, 128);
+    ops::MatMulOpQuant op8(true, true, DT_UINT8);
+    EXPECT(op8.Run(&context, &A, &B, &C8) == MaceStatus::MACE_SUCCESS);
+    int32_t mult; int shift;
+    EXPECT(orc_get_output_multiplier_and_shift(0.02f, 0.015f, 40.f, &mult, &shift) == 0);
+    orc_q8_gemm_u8(a.data(), b.data(), batch, rows, cols, depth, ORC_COL_MAJOR, ORC_COL_MAJOR,
+                   ORC_ROW_MAJOR, 1, 0, -77, -201, nullptr, mult, shift, 128, 0, 255, want8.data(), 4);
+    EXPECT(c8 == want8);
+    Tensor Cbad(c8.data(), DT_UINT8, {}, 1e-6f, 128);   // multiplier >= 1: the reference CHECKs
+    EXPECT(op8.Run(&context, &A, &B, &Cbad) == MaceStatus::MACE_INVALID_ARGS);
+
+    const index_t n = 2, o = 40, isz = 7 * 7 * 32;
+    std::vector<uint8_t> x(n * isz), w(o * isz), y(n * o), wanty(n * o);
+    std::vector<int32_t> bias(o);
+    for (auto &v : x) v = rng() & 255;
+    for (auto &v : w) v = rng() & 255;
+    for (auto &v : bias) v = (int32_t)(rng() % 65536) - 32768;
+    Tensor X(x.data(), DT_UINT8, {n, 7, 7, 32}, 0.02f, 128), W(w.data(), DT_UINT8, {o, 7, 7, 32}, 0.01f, 127, true),
+        Bi(bias.data(), DT_INT32, {o}, 0.0002f, 0, true), Y(y.data(), DT_UINT8, {}, 0.9f, 30);
+    ops::FullyConnectedOp<uint8_t> fc(&reg);
+    EXPECT(fc.Run(&context, &X, &W, &Bi, &Y) == MaceStatus::MACE_SUCCESS);
+    EXPECT(Y.shape() == (std::vector<index_t>{n, 1, 1, o}));
+    orc_q8_gemv_u8(w.data(), x.data(), bias.data(), n, o, isz, 0, 1, 127, 128, 0.01f, 0.02f, 0.9f, 30,
+                   ORC_REQUANT_NEON, wanty.data(), 4);
+    EXPECT(y == wanty);
+  }
+  mace_hip_ctx_destroy(hctx);
+  return g_fail;
+}
+
+int main(int argc, char **argv) {
+  const char *mode = argc > 1 ? argv[1] : "registry";
+  int fails = strcmp(mode, "compute") == 0 ? test_compute() : test_registry();
+  printf("%s: %s (%d failures)\n", mode, fails ? "FAILED" : "ok", fails);
+  return fails ? 1 : 0;
+}
