@@ -50,6 +50,8 @@ def main():
     ap.add_argument("--size", type=int, default=8192, help="M = N = K of the uint8 GEMM")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemv", action="store_true")
+    ap.add_argument("--no-other", action="store_true",
+                    help="skip the secondary configurations (conv1x1, smaller GEMMs, fp32)")
     ap.add_argument("--only-gemv", action="store_true", help="development: skip the GEMM part")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a kernel of known traffic, for "
@@ -151,6 +153,8 @@ def main():
 
     if not args.no_gemv:
         result["gemv"] = bench_gemv(ctx, mh, torch, args)
+    if not args.no_other:
+        result["other_configs"] = bench_other(ctx, mh, torch)
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(np, torch, A, B, out8, n, za, zb, zc, mult, shift,
@@ -214,6 +218,102 @@ def bench_gemv(ctx, mh, torch, args):
                        "kernel": "q8_gemv_rows_kernel<1,1,16,uint8_t>",
                        "timing": "400 back-to-back launches between two HIP events, rotating "
                                  "over 640 MiB of weights"}
+    return out
+
+
+def time_kernel(ctx, call, reps=10, warm=3):
+    """(average whole-call ms between two HIP events over `reps` launches, average ms of the
+    call's dominant kernel)."""
+    for _ in range(warm):
+        call()
+    ctx.sync()
+    ctx.timer_start()
+    for _ in range(reps):
+        call()
+    whole = ctx.timer_stop() / reps
+    ctx.profile(True)
+    ks = []
+    for _ in range(reps):
+        call()
+        ks.append(ctx.last_kernel_ms())
+    ctx.profile(False)
+    return whole, sum(ks) / len(ks)
+
+
+def bench_other(ctx, mh, torch):
+    """The remaining BASELINE configurations, timed the same way (device-resident inputs, HIP
+    events on the launch stream): not the headline, reported for coverage.  Each entry gives the
+    dominant kernel's rate against the roofline that bounds it."""
+    out = []
+    g = torch.Generator(device="cuda").manual_seed(11)
+
+    def u8(*shape):
+        return torch.randint(0, 256, shape, dtype=torch.uint8, device="cuda", generator=g)
+
+    # config 1: uint8 MatMul 128x256 . 256x128 (launch-latency bound)
+    A, B, C = u8(128, 256), u8(256, 128), torch.empty((128, 128), dtype=torch.uint8, device="cuda")
+    mult, shift = mh.get_output_multiplier_and_shift(0.02, 0.015, 0.05)
+    torch.cuda.synchronize()
+    whole, k = time_kernel(ctx, lambda: ctx.call(
+        "mace_hip_gemm_q8_u8", A.data_ptr(), 0, B.data_ptr(), 0, C.data_ptr(), 0, 1, 128, 256, 128,
+        1, 1, -128, -128, None, mult, shift, 128, 0, 255), reps=50)
+    out.append({"workload": "q8_matmul_128x256x128", "call_us": round(whole * 1e3, 2),
+                "kernel_us": round(k * 1e3, 2), "GOPS": round(2 * 128 * 256 * 128 / (k * 1e-3) / 1e9, 1)})
+
+    # config 5: smaller and batched uint8 GEMMs, uint8 output
+    for (b, n) in ((1, 2048), (1, 4096), (32, 512)):
+        A, B = u8(b, n, n), u8(b, n, n)
+        C = torch.empty((b, n, n), dtype=torch.uint8, device="cuda")
+        e = mh.quantize_multiplier(min(0.9, 40.0 / (74.0 * 74.0 * n ** 0.5)))
+        torch.cuda.synchronize()
+        whole, k = time_kernel(ctx, lambda: ctx.call(
+            "mace_hip_gemm_q8_u8", A.data_ptr(), 0, B.data_ptr(), 0, C.data_ptr(), 0, b, n, n, n, 1,
+            1, -131, -122, None, e[0], -e[1], 128, 0, 255))
+        ops = 2.0 * b * n ** 3
+        out.append({"workload": "q8_matmul_%dx%d^3" % (b, n), "call_ms": round(whole, 4),
+                    "kernel_ms": round(k, 4), "TOPS": round(ops / (k * 1e-3) / 1e12, 1),
+                    "frac_of_int8_peak": round(ops / (k * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4)})
+
+    # config 4: quantized conv 1x1, NHWC, batch 64, MobileNetV1 pointwise shapes, ReLU6 range
+    for (hw, cin, cout) in ((112, 32, 64), (56, 128, 128), (28, 256, 256), (14, 512, 512),
+                            (7, 1024, 1024)):
+        n = 64
+        x, f = u8(n, hw, hw, cin), u8(cout, cin)
+        bias = torch.randint(-2 ** 15, 2 ** 15, (cout,), dtype=torch.int32, device="cuda", generator=g)
+        y = torch.empty((n, hw, hw, cout), dtype=torch.uint8, device="cuda")
+        s_in, s_f = 0.02, 0.01
+        s_out = max(6.0, 3 * 74.0 * 74.0 * cin ** 0.5 * s_in * s_f) / 255.0
+        torch.cuda.synchronize()
+        whole, k = time_kernel(ctx, lambda: ctx.call(
+            "mace_hip_conv1x1_q8_nhwc", x.data_ptr(), f.data_ptr(), bias.data_ptr(), n, hw, hw, cin,
+            cout, s_in, 128, s_f, 127, s_in * s_f, s_out, 0, 0, 255, y.data_ptr()))
+        pix = n * hw * hw
+        ops = 2.0 * pix * cin * cout
+        nbytes = pix * cin + cout * cin + 4 * cout + pix * cout
+        ai = ops / nbytes
+        roof_tops = min(PEAK_INT8_TOPS, ai * PEAK_HBM_GBS / 1e3)
+        tops = ops / (k * 1e-3) / 1e12
+        out.append({"workload": "q8_conv1x1_n64_%dx%dx%d_to_%d" % (hw, hw, cin, cout),
+                    "call_ms": round(whole, 4), "kernel_ms": round(k, 4), "TOPS": round(tops, 1),
+                    "GBps": round(nbytes / (k * 1e-3) / 1e9, 1), "ops_per_byte": round(ai, 1),
+                    "roofline_TOPS": round(roof_tops, 1), "frac_of_roofline": round(tops / roof_tops, 4)})
+
+    # config 2: fp32 Gemm, batch 4, 1024^3, the four transpose combinations
+    A = torch.randn((4, 1024, 1024), dtype=torch.float32, device="cuda", generator=g)
+    B = torch.randn((4, 1024, 1024), dtype=torch.float32, device="cuda", generator=g)
+    C = torch.empty((4, 1024, 1024), dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()
+    for ta in (0, 1):
+        for tb in (0, 1):
+            whole, k = time_kernel(ctx, lambda: ctx.call(
+                "mace_hip_gemm_f32_transpose", A.data_ptr(), B.data_ptr(), 4, 1024, 1024, 1024, 1024,
+                ta, tb, 0, 1, 1, C.data_ptr()))
+            flops = 2.0 * 4 * 1024 ** 3
+            tf = flops / (k * 1e-3) / 1e12
+            out.append({"workload": "f32_gemm_4x1024^3_ta%d_tb%d" % (ta, tb), "kernel_ms": round(k, 4),
+                        "TFLOPS": round(tf, 1), "frac_of_fp32_mfma_peak": round(tf / 157.3, 4)})
+    for o in out:
+        log("other:", json.dumps(o))
     return out
 
 

@@ -550,18 +550,25 @@ __global__ __launch_bounds__(256) void q8_pack_transpose_kernel(const uint8_t *s
 // ---- correction vectors --------------------------------------------------------------------
 
 // corr[b][n] = coef * sum_k (P[b][n][k] - 128) + add + (bias ? bias[n] : 0), modulo 2^32.
-// One wavefront per panel row.
+// LPR lanes share a panel row (LPR a power of two, 1..64): short rows (the NHWC input of a
+// conv with few channels) pack several rows into one wavefront so that every 16-byte load is
+// useful, long rows get the whole wavefront.  Rows are consecutive in memory whenever
+// ld == k, which then makes a wavefront's loads one contiguous run.
+template <int LPR>
 __global__ __launch_bounds__(256) void q8_panel_sums_kernel(const uint8_t *P, int64_t ld,
                                                             int64_t pbs, int n, int k,
                                                             int32_t coef, int32_t add,
                                                             const int32_t *bias,
                                                             int32_t *corr) {
+  constexpr int RPW = 64 / LPR;   // rows per wavefront
   const int lane = threadIdx.x & 63;
-  const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  if (row >= n) return;
-  const uint8_t *r = P + (int64_t)blockIdx.z * pbs + (int64_t)row * ld;
+  const int sub = lane % LPR;
+  const int64_t row = ((int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * RPW +
+                      lane / LPR;
+  const bool live = row < n;
+  const uint8_t *r = P + (int64_t)blockIdx.z * pbs + (live ? row : 0) * ld;
   uint32_t s = 0;
-  for (int c = lane * 16; c < k; c += 64 * 16) {
+  for (int c = sub * 16; c < k; c += LPR * 16) {
     const uint4 v = *(const uint4 *)(r + c);
     s = __builtin_amdgcn_udot4(v.x, 0x01010101u, s, false);
     s = __builtin_amdgcn_udot4(v.y, 0x01010101u, s, false);
@@ -569,13 +576,40 @@ __global__ __launch_bounds__(256) void q8_panel_sums_kernel(const uint8_t *P, in
     s = __builtin_amdgcn_udot4(v.w, 0x01010101u, s, false);
   }
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
-  if (lane == 0) {
+  for (int off = LPR / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+  if (sub == 0 && live) {
     const uint32_t shifted = s - 128u * (uint32_t)k;   // sum of (byte - 128)
     uint32_t v = (uint32_t)coef * shifted + (uint32_t)add;
     if (bias) v += (uint32_t)bias[row];
     corr[(int64_t)blockIdx.z * n + row] = (int32_t)v;
   }
+}
+
+int launch_panel_sums(mace_hip_ctx *ctx, const uint8_t *P, int64_t ld, int64_t pbs, int64_t n,
+                      int k, int nb, int32_t coef, int32_t add, const int32_t *bias,
+                      int32_t *corr) {
+  const int chunks = k / 16;
+  int lpr = 1;
+  while (lpr < 64 && lpr < chunks) lpr *= 2;
+  const int rows_per_block = 4 * (64 / lpr);
+  const int64_t blocks = (n + rows_per_block - 1) / rows_per_block;
+  MH_CHECK(ctx, blocks < (1ll << 31), "panel too tall");
+  dim3 grid((unsigned)blocks, 1, nb), block(256);
+#define MH_SUMS(L_)                                                                       \
+  hipLaunchKernelGGL((q8_panel_sums_kernel<L_>), grid, block, 0, ctx->stream, P, ld, pbs, \
+                     (int)n, k, coef, add, bias, corr)
+  switch (lpr) {
+    case 1: MH_SUMS(1); break;
+    case 2: MH_SUMS(2); break;
+    case 4: MH_SUMS(4); break;
+    case 8: MH_SUMS(8); break;
+    case 16: MH_SUMS(16); break;
+    case 32: MH_SUMS(32); break;
+    default: MH_SUMS(64); break;
+  }
+#undef MH_SUMS
+  MH_HIP(ctx, hipGetLastError());
+  return MACE_HIP_SUCCESS;
 }
 
 template <int WX, int WY, int FX, int FY>
@@ -713,13 +747,12 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   if (!corrL || !corrR) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
   const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
   {
-    dim3 gl((unsigned)((rows + 3) / 4), 1, lhs_nb), gr((unsigned)((cols + 3) / 4), 1, rhs_nb);
-    hipLaunchKernelGGL(q8_panel_sums_kernel, gl, dim3(256), 0, ctx->stream, L.ptr, L.ld,
-                       L.bs, (int)rows, L.k, (int32_t)(0u - zr), 0,
-                       out_u8 ? ep.bias : nullptr, corrL);
-    hipLaunchKernelGGL(q8_panel_sums_kernel, gr, dim3(256), 0, ctx->stream, R.ptr, R.ld,
-                       R.bs, (int)cols, R.k, (int32_t)(0u - zl),
-                       (int32_t)((uint32_t)depth * zl * zr), (const int32_t *)nullptr, corrR);
+    MH_RETURN_IF_ERROR(launch_panel_sums(ctx, L.ptr, L.ld, L.bs, rows, L.k, lhs_nb,
+                                         (int32_t)(0u - zr), 0, out_u8 ? ep.bias : nullptr,
+                                         corrL));
+    MH_RETURN_IF_ERROR(launch_panel_sums(ctx, R.ptr, R.ld, R.bs, cols, R.k, rhs_nb,
+                                         (int32_t)(0u - zl),
+                                         (int32_t)((uint32_t)depth * zl * zr), nullptr, corrR));
     MH_HIP(ctx, hipGetLastError());
   }
 
@@ -747,9 +780,22 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     return (int64_t)((p.XN + tx - 1) / tx) * ((p.YN + ty - 1) / ty) * batch;
   };
   p.dbg = nullptr;
-  const bool big = p.XN > 128 && p.YN > 128 && tiles(256, 256) >= cu;
-  const bool skinny = !big && p.XN <= 64 && p.YN > 128 && tiles(64, 256) >= cu;
-  const bool medium = !big && !skinny && p.XN > 64 && p.YN > 64 && tiles(128, 128) >= cu;
+  // Tile shape: bigger tiles do more MFMA work per byte moved and per barrier, smaller ones
+  // keep more CUs busy.  Score = relative efficiency of the shape x the fraction of CU slots
+  // its last round of workgroups fills.
+  auto score = [&](int tx, int ty, double weight) {
+    const int64_t t = tiles(tx, ty);
+    const int64_t rounds = (t + cu - 1) / cu;
+    return weight * (double)t / (double)(rounds * cu);
+  };
+  const double s_big = (p.XN > 128 && p.YN > 128) ? score(256, 256, 1.0) : 0.0;
+  const double s_skinny = (p.XN <= 64 && p.YN > 128) ? score(64, 256, 0.6) : 0.0;
+  const double s_medium = (p.XN > 64 && p.YN > 64) ? score(128, 128, 0.6) : 0.0;
+  const double s_small = score(64, 64, 0.3);
+  const double best = std::max(std::max(s_big, s_skinny), std::max(s_medium, s_small));
+  const bool big = s_big == best;
+  const bool skinny = !big && s_skinny == best;
+  const bool medium = !big && !skinny && s_medium == best;
   // the streaming kernel needs whole 64-byte slabs and enough of them to fill its ring
   if (p.K % SLAB == 0 && p.K >= SLAB * 3) {
     if (big) return launch_gemm_dma<2, 2, 4, 4, 4, 1>(ctx, p, out_u8, (int)batch);
