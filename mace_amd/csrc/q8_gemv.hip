@@ -187,7 +187,7 @@ __global__ __launch_bounds__(NWAVES * 64) void q8_gemv_rows_kernel(GemvParams p)
     for (int b = 0; b < NB; ++b) dot[r][b] = 0;
   }
 
-  __shared__ uint32_t part[NB][NWAVES];   // per-wavefront partial sums of the right-hand rows
+  __shared__ uint32_t sum_x[NB];   // byte sums of the right-hand rows of this pass
   auto block_of_w = [&](auto masked_tag, int c0) {
     constexpr bool masked = decltype(masked_tag)::value;
     // weights of this block: R x 4 loads of 16 bytes in flight per lane
@@ -200,21 +200,32 @@ __global__ __launch_bounds__(NWAVES * 64) void q8_gemv_rows_kernel(GemvParams p)
         w[r][u] = load_stream16(lrow[r] + (int64_t)(masked ? min(c, nchunk - 1) : c) * 16);
       }
     if (c0 == 0) {
-      // Stage the right-hand vectors while the weights are on their way, and sum their
-      // bytes once per workgroup (every output needs sum(r) of its batch row).
+      // Stage the right-hand vectors while the weights are on their way, and sum their bytes
+      // once per workgroup (every output needs sum(r) of its batch row).  The pass holds at
+      // most 64 KiB = 4096 chunks, i.e. at most 4 per thread: all loads are issued before the
+      // first one is consumed.
+      constexpr int NT = NWAVES * 64;
+      const int total = NB * nchunk;   // rows past the batch re-stage the last one
+      uint4 xs[4];
+      int xb[4];
 #pragma unroll
-      for (int b = 0; b < NB; ++b) {
-        uint32_t s = 0;
-        if (b < nb) {
-          const uint8_t *src = p.rhs + (int64_t)(b0 + b) * p.rhs_bs;
-          for (int c = tid; c < nchunk; c += NWAVES * 64) {
-            const uint4 x = *(const uint4 *)(src + (int64_t)c * 16);
-            *(uint4 *)(sx + ((size_t)b * nchunk + c) * 16) = x;
-            s = dot16(x, ones, s);
-          }
+      for (int j = 0; j < 4; ++j) {
+        const int i = tid + j * NT;
+        xb[j] = i < total ? i / nchunk : -1;
+        const int c = i - max(xb[j], 0) * nchunk;
+        xs[j] = zero;
+        if (xb[j] >= 0)
+          xs[j] = *(const uint4 *)(p.rhs + (int64_t)min(b0 + xb[j], p.batch - 1) * p.rhs_bs +
+                                   (int64_t)c * 16);
+      }
+      if (tid < NB) sum_x[tid] = 0;
+      __syncthreads();
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (xb[j] >= 0) {
+          *(uint4 *)(sx + (size_t)(tid + j * NT) * 16) = xs[j];   // [b][c] is the flat index
+          atomicAdd(&sum_x[xb[j]], dot16(xs[j], ones, 0u));
         }
-        s = wave_sum(s);
-        if (lane == 0) part[b][wave] = s;
       }
       __syncthreads();
     }
@@ -229,12 +240,10 @@ __global__ __launch_bounds__(NWAVES * 64) void q8_gemv_rows_kernel(GemvParams p)
       }
 #pragma unroll
       for (int b = 0; b < NB; ++b) {
-        if (b < nb) {
-          const uint4 x =
-              *(const uint4 *)(sx + ((size_t)b * nchunk + (masked ? min(c, nchunk - 1) : c)) * 16);
+        const uint4 x =
+            *(const uint4 *)(sx + ((size_t)b * nchunk + (masked ? min(c, nchunk - 1) : c)) * 16);
 #pragma unroll
-          for (int r = 0; r < R; ++r) dot[r][b] = dot16(w[r][u], x, dot[r][b]);   // w is 0 if !ok
-        }
+        for (int r = 0; r < R; ++r) dot[r][b] = dot16(w[r][u], x, dot[r][b]);   // w is 0 if !ok
       }
     }
   };
@@ -244,7 +253,7 @@ __global__ __launch_bounds__(NWAVES * 64) void q8_gemv_rows_kernel(GemvParams p)
 
   const uint32_t zl = (uint32_t)p.lhs_zp, zr = (uint32_t)p.rhs_zp;
 #pragma unroll
-  for (int b = 0; b < NB; ++b) sum_r[b] = wave_sum(lane < NWAVES ? part[b][lane] : 0u);
+  for (int b = 0; b < NB; ++b) sum_r[b] = sum_x[b];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const uint32_t sl = wave_sum(sum_l[r]);
