@@ -188,6 +188,45 @@ __global__ __launch_bounds__(NWAVES * 64) void q8_gemv_rows_kernel(GemvParams p)
   }
 
   __shared__ uint32_t sum_x[NB];   // byte sums of the right-hand rows of this pass
+  // The right-hand vectors of the pass are staged in LDS once per workgroup, together with
+  // their byte sums (every output needs sum(r) of its batch row).  The pass holds at most
+  // 64 KiB = 4096 chunks, i.e. at most 4 per thread.  Their loads are issued first, the weight
+  // loads of the first block right behind them; loads return in order, so the staging only
+  // waits for its own data and the dot products start while later weight chunks are still in
+  // flight.  Raw barriers: __syncthreads() would also wait for every outstanding load.
+  constexpr int NT = NWAVES * 64;
+  uint4 xs[4];
+  int xb[4];
+  {
+    const int total = NB * nchunk;   // rows past the batch re-stage the last one
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = tid + j * NT;
+      xb[j] = i < total ? i / nchunk : -1;
+      const int c = i - max(xb[j], 0) * nchunk;
+      xs[j] = zero;
+      if (xb[j] >= 0)
+        xs[j] = *(const uint4 *)(p.rhs + (int64_t)min(b0 + xb[j], p.batch - 1) * p.rhs_bs +
+                                 (int64_t)c * 16);
+    }
+  }
+  auto lds_barrier = [&]() {
+    __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): this wavefront's LDS traffic is done
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+  auto stage_rhs = [&]() {
+    if (tid < NB) sum_x[tid] = 0;
+    lds_barrier();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (xb[j] >= 0) {
+        *(uint4 *)(sx + (size_t)(tid + j * NT) * 16) = xs[j];   // [b][c] is the flat index
+        atomicAdd(&sum_x[xb[j]], dot16(xs[j], ones, 0u));
+      }
+    }
+    lds_barrier();
+  };
   auto block_of_w = [&](auto masked_tag, int c0) {
     constexpr bool masked = decltype(masked_tag)::value;
     // weights of this block: R x 4 loads of 16 bytes in flight per lane
@@ -199,36 +238,7 @@ __global__ __launch_bounds__(NWAVES * 64) void q8_gemv_rows_kernel(GemvParams p)
         const int c = c0 + lane + 64 * u;
         w[r][u] = load_stream16(lrow[r] + (int64_t)(masked ? min(c, nchunk - 1) : c) * 16);
       }
-    if (c0 == 0) {
-      // Stage the right-hand vectors while the weights are on their way, and sum their bytes
-      // once per workgroup (every output needs sum(r) of its batch row).  The pass holds at
-      // most 64 KiB = 4096 chunks, i.e. at most 4 per thread: all loads are issued before the
-      // first one is consumed.
-      constexpr int NT = NWAVES * 64;
-      const int total = NB * nchunk;   // rows past the batch re-stage the last one
-      uint4 xs[4];
-      int xb[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int i = tid + j * NT;
-        xb[j] = i < total ? i / nchunk : -1;
-        const int c = i - max(xb[j], 0) * nchunk;
-        xs[j] = zero;
-        if (xb[j] >= 0)
-          xs[j] = *(const uint4 *)(p.rhs + (int64_t)min(b0 + xb[j], p.batch - 1) * p.rhs_bs +
-                                   (int64_t)c * 16);
-      }
-      if (tid < NB) sum_x[tid] = 0;
-      __syncthreads();
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        if (xb[j] >= 0) {
-          *(uint4 *)(sx + (size_t)(tid + j * NT) * 16) = xs[j];   // [b][c] is the flat index
-          atomicAdd(&sum_x[xb[j]], dot16(xs[j], ones, 0u));
-        }
-      }
-      __syncthreads();
-    }
+    if (c0 == 0) stage_rhs();
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int c = c0 + lane + 64 * u;
