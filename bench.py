@@ -48,6 +48,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--size", type=int, default=8192, help="M = N = K of the uint8 GEMM")
+    ap.add_argument("--rhs-order", choices=["row", "col"], default="row",
+                    help="row = MatMul default; col = transpose_b (B is read in place, no repack)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemv", action="store_true")
     ap.add_argument("--no-other", action="store_true",
@@ -98,8 +100,10 @@ def main():
     shift = -e
     torch.cuda.synchronize()
 
+    rhs_order = mh.ROW_MAJOR if args.rhs_order == "row" else mh.COL_MAJOR
+
     def step():
-        ctx.call("mace_hip_gemm_q8_u8", A.data_ptr(), mh.ROW_MAJOR, B.data_ptr(), mh.ROW_MAJOR,
+        ctx.call("mace_hip_gemm_q8_u8", A.data_ptr(), mh.ROW_MAJOR, B.data_ptr(), rhs_order,
                  out8.data_ptr(), mh.ROW_MAJOR, 1, n, n, n, 1, 1, -za, -zb, None, mult, shift, zc,
                  0, 255)
 
@@ -140,7 +144,9 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8",
         "data": "synthetic",
         "config": {"workload": "q8_matmul_%dx%dx%d_u8out" % (n, n, n), "M": n, "N": n, "K": n,
-                   "lhs_order": "RowMajor", "rhs_order": "RowMajor", "out_order": "RowMajor",
+                   "lhs_order": "RowMajor",
+                   "rhs_order": "RowMajor" if args.rhs_order == "row" else "ColMajor",
+                   "out_order": "RowMajor",
                    "zero_points": [za, zb, zc], "multiplier": mult, "right_shift": shift,
                    "saturated_fraction": round(sat, 4), "device": arch, "cus": cus},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_INT8_TOPS,
@@ -158,7 +164,7 @@ def main():
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(np, torch, A, B, out8, n, za, zb, zc, mult, shift,
-                                              args.cpu_rows)
+                                              args.cpu_rows, rhs_order)
     ctx.close()
     print(json.dumps(result), flush=True)
 
@@ -317,7 +323,7 @@ def bench_other(ctx, mh, torch):
     return out
 
 
-def cpu_baseline(np, torch, A, B, out8, n, za, zb, zc, mult, shift, rows):
+def cpu_baseline(np, torch, A, B, out8, n, za, zb, zc, mult, shift, rows, rhs_order=0):
     """The oracle (a port of the reference's CPU path: exact integer GEMM standing in for
     gemmlowp + the fixed-point output pipeline) on `rows` rows of A times the whole of B, on
     the host cores.  The same rows of the GPU result are compared with it."""
@@ -332,7 +338,7 @@ def cpu_baseline(np, torch, A, B, out8, n, za, zb, zc, mult, shift, rows):
     b = B.cpu().numpy()
     t0 = time.perf_counter()
     want = orc.q8_gemm_u8(a, b, 1, rows, n, n, -za, -zb, None, mult, shift, zc, 0, 255,
-                          nthreads=cores)
+                          rhs_order=rhs_order, nthreads=cores)
     dt = time.perf_counter() - t0
     got = out8[:rows].cpu().numpy().reshape(-1)
     exact = bool(np.array_equal(got, want))

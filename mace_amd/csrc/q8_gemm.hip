@@ -46,6 +46,11 @@ struct GemmParams {
   int64_t ldo;        // elements between consecutive y
   int64_t obs;        // elements per batch
   RequantFixed rq;    // uint8 output pipeline
+  // When the kernel sums the Y panel itself (SUMY): corrY[y] = ycoef * sum_k Y'[y][k] + yadd
+  // (+ ybias[y]) is formed in the epilogue and corrY is not read.
+  int32_t ycoef, yadd;
+  const int32_t *ybias;
+  bool sum_y;
   int tiles_x, tiles_y;
   long long *dbg;     // lab instrumentation only (nullptr in the library)
 };
@@ -69,6 +74,15 @@ __device__ inline void tile_of_block(int bid, int nblocks, int tiles_x, int tile
   *tx = r / gsize;
 }
 
+// sum of the 16 signed bytes of a (flipped) fragment, added to acc
+__device__ inline int sum16_i8(const v4i &f, int acc) {
+  acc = __builtin_amdgcn_sdot4(f.x, 0x01010101, acc, false);
+  acc = __builtin_amdgcn_sdot4(f.y, 0x01010101, acc, false);
+  acc = __builtin_amdgcn_sdot4(f.z, 0x01010101, acc, false);
+  acc = __builtin_amdgcn_sdot4(f.w, 0x01010101, acc, false);
+  return acc;
+}
+
 // Epilogue shared by the GEMM kernels: adds the correction vectors to the accumulators and
 // stores int32 results or requantized bytes.  Accumulator register r of a 32x32 tile holds
 //   x (MFMA row)    = 8 * (r / 4) + 4 * (lane / 32) + r % 4
@@ -76,9 +90,10 @@ __device__ inline void tile_of_block(int bid, int nblocks, int tiles_x, int tile
 // so every lane owns runs of four consecutive x, stored as one 16-byte (int32) or 4-byte
 // (uint8) access.  The correction vectors of the tile are staged through LDS first (the
 // operand buffers are dead by then), so the stores do not wait on scattered global loads.
-template <int WX, int WY, int FX, int FY, typename OutT>
-__device__ inline void gemm_epilogue(v16i (&acc)[FX][FY], const GemmParams &p, uint8_t *lds,
-                                     int b, int x0, int y0, int wx, int wy, int tid) {
+template <int WX, int WY, int FX, int FY, typename OutT, bool SUMY>
+__device__ inline void gemm_epilogue(v16i (&acc)[FX][FY], const int (&ysum)[FY],
+                                     const GemmParams &p, uint8_t *lds, int b, int x0, int y0,
+                                     int wx, int wy, int tid) {
   constexpr int NT = WX * WY * 64;
   constexpr int TX = WX * FX * 32, TY = WY * FY * 32;
   const int lane = tid & 63;
@@ -87,7 +102,8 @@ __device__ inline void gemm_epilogue(v16i (&acc)[FX][FY], const GemmParams &p, u
   int32_t *sc = (int32_t *)lds;   // [TX] corrections along x, then [TY] along y
   __syncthreads();                // every wavefront is done reading operand tiles
   for (int i = tid; i < TX; i += NT) sc[i] = cX[min(x0 + i, p.XN - 1)];
-  for (int i = tid; i < TY; i += NT) sc[TX + i] = cY[min(y0 + i, p.YN - 1)];
+  if (!SUMY)
+    for (int i = tid; i < TY; i += NT) sc[TX + i] = cY[min(y0 + i, p.YN - 1)];
   __syncthreads();
 
   OutT *outb = (OutT *)p.out + (int64_t)b * p.obs;
@@ -98,7 +114,15 @@ __device__ inline void gemm_epilogue(v16i (&acc)[FX][FY], const GemmParams &p, u
   for (int j = 0; j < FY; ++j) {
     const int yl = (wy * FY + j) * 32 + (lane & 31);
     const int y = y0 + yl;
-    const uint32_t cy = (uint32_t)sc[TX + yl];
+    uint32_t cy;
+    if constexpr (SUMY) {
+      // lanes l and l ^ 32 hold the two 16-byte halves of every 32-byte k step of row y
+      const int total = ysum[j] + __shfl_xor(ysum[j], 32, 64);
+      cy = (uint32_t)p.ycoef * (uint32_t)total + (uint32_t)p.yadd;
+      if (p.ybias) cy += (uint32_t)p.ybias[min(y, p.YN - 1)];
+    } else {
+      cy = (uint32_t)sc[TX + yl];
+    }
     OutT *orow = outb + (int64_t)y * p.ldo + x0;
 #pragma unroll
     for (int i = 0; i < FX; ++i) {
@@ -136,7 +160,7 @@ __device__ inline void gemm_epilogue(v16i (&acc)[FX][FY], const GemmParams &p, u
   }
 }
 
-template <int WX, int WY, int FX, int FY, typename OutT>
+template <int WX, int WY, int FX, int FY, typename OutT, bool SUMY = false>
 __global__ __launch_bounds__(WX *WY * 64) void q8_gemm_kernel(GemmParams p) {
   constexpr int NT = WX * WY * 64;
   constexpr int TX = WX * FX * 32;
@@ -230,6 +254,10 @@ __global__ __launch_bounds__(WX *WY * 64) void q8_gemm_kernel(GemmParams p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
+  int ysum[FY];
+#pragma unroll
+  for (int j = 0; j < FY; ++j) ysum[j] = 0;
+
   // fragment addresses: lane l supplies row (l % 32), k bytes [16*(l/32), +16) of each
   // 32-byte k step, for both operands (the pairing of k positions is what matters)
   const int frag_off = (lane & 31) * LDS_ROW + (lane >> 5) * 16;
@@ -249,6 +277,10 @@ __global__ __launch_bounds__(WX *WY * 64) void q8_gemm_kernel(GemmParams p) {
 #pragma unroll
       for (int j = 0; j < FY; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], bf[j], acc[i][j], 0, 0, 0);
+    if constexpr (SUMY) {
+#pragma unroll
+      for (int j = 0; j < FY; ++j) ysum[j] = sum16_i8(bf[j], ysum[j]);
+    }
   };
 
   // full tiles: global loads of tile kt+1 are in flight while tile kt is multiplied
@@ -275,7 +307,7 @@ __global__ __launch_bounds__(WX *WY * 64) void q8_gemm_kernel(GemmParams p) {
     for (int ks = 0; ks < (ktail + 31) / 32; ++ks) mfma_step(0, ks);
   }
 
-  gemm_epilogue<WX, WY, FX, FY, OutT>(acc, p, lds, b, x0, y0, wx, wy, tid);
+  gemm_epilogue<WX, WY, FX, FY, OutT, SUMY>(acc, ysum, p, lds, b, x0, y0, wx, wy, tid);
 }
 
 // ---- the streaming GEMM kernel: global -> LDS without passing through registers ----------
@@ -305,7 +337,8 @@ __device__ inline void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
 }
 
-template <int WX, int WY, int FX, int FY, int STAGES, typename OutT, int OCC = 1, int ABLATE = 0>
+template <int WX, int WY, int FX, int FY, int STAGES, typename OutT, int OCC = 1, int ABLATE = 0,
+          bool SUMY = false>
 __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParams p) {
   constexpr int NW = WX * WY;
   constexpr int TX = WX * FX * 32;
@@ -363,6 +396,9 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
     for (int j = 0; j < FY; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+  int ysum[FY];
+#pragma unroll
+  for (int j = 0; j < FY; ++j) ysum[j] = 0;
 
   // fragment addresses: lane l reads row (l % 32) of a 32-row block, chunk 2*ks + l/32.
   // Block bases are multiples of 32 rows, so the swizzle depends on l only.
@@ -409,6 +445,12 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
     for (int m = 0; m < NM; ++m) {
       acc[m / FY][m % FY] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ca[m / FY], cb[m % FY],
                                                                   acc[m / FY][m % FY], 0, 0, 0);
+      if constexpr (SUMY) {
+        constexpr int SUMS_PER_SLOT = (FY + NM - 1) / NM;
+#pragma unroll
+        for (int j = m * SUMS_PER_SLOT; j < (m + 1) * SUMS_PER_SLOT; ++j)
+          if (j < FY) ysum[j] = sum16_i8(cb[j], ysum[j]);
+      }
       constexpr int READS_PER_SLOT = (NF + NM - 1) / NM;
 #pragma unroll
       for (int f = m * READS_PER_SLOT; f < (m + 1) * READS_PER_SLOT; ++f) {
@@ -417,8 +459,8 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
       }
       if (DELAY > 0 && m >= DELAY && m - DELAY < NF) {
         const int f = m - DELAY;
-        if (f < FX) na[f] ^= flip;
-        else nb[f - FX] ^= flip;
+        if (f < FX) { if (!(ABLATE & 16)) na[f] ^= flip; }
+        else { if (!(ABLATE & 8)) nb[f - FX] ^= flip; }
       }
       if constexpr (dma) {
         // LX + LY transfers spread over the slots from slot 0 on
@@ -480,14 +522,14 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
 
   if (ABLATE & 4) {
     const long long c1 = clock64(), w1 = wall_clock64();
-    gemm_epilogue<WX, WY, FX, FY, OutT>(acc, p, lds, b, x0, y0, wx, wy, tid);
+    gemm_epilogue<WX, WY, FX, FY, OutT, SUMY>(acc, ysum, p, lds, b, x0, y0, wx, wy, tid);
     if (tid == 0 && blockIdx.x == 8) {
       p.dbg[0] = c1 - dbg_c0; p.dbg[1] = w1 - dbg_w0;
       p.dbg[2] = clock64() - c1; p.dbg[3] = wall_clock64() - w1;
     }
     return;
   }
-  gemm_epilogue<WX, WY, FX, FY, OutT>(acc, p, lds, b, x0, y0, wx, wy, tid);
+  gemm_epilogue<WX, WY, FX, FY, OutT, SUMY>(acc, ysum, p, lds, b, x0, y0, wx, wy, tid);
 }
 
 // ---- repacking ---------------------------------------------------------------------------
@@ -619,20 +661,22 @@ int launch_gemm(mace_hip_ctx *ctx, GemmParams &p, bool out_u8, int batch) {
   p.tiles_y = (p.YN + TY - 1) / TY;
   const size_t lds = 2 * (size_t)(TX + TY) * LDS_ROW;
   dim3 grid(p.tiles_x * p.tiles_y, 1, batch), block(WX * WY * 64);
-  if (out_u8) {
-    auto k = q8_gemm_kernel<WX, WY, FX, FY, uint8_t>;
+  auto launch = [&](auto k) -> int {
     if (lds > 64 * 1024)
       MH_HIP(ctx, hipFuncSetAttribute((const void *)k,
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     MH_PROF_BEGIN(ctx);
     hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p);
+    return MACE_HIP_SUCCESS;
+  };
+  if (out_u8 && p.sum_y) {
+    MH_RETURN_IF_ERROR(launch(q8_gemm_kernel<WX, WY, FX, FY, uint8_t, true>));
+  } else if (out_u8) {
+    MH_RETURN_IF_ERROR(launch(q8_gemm_kernel<WX, WY, FX, FY, uint8_t, false>));
+  } else if (p.sum_y) {
+    MH_RETURN_IF_ERROR(launch(q8_gemm_kernel<WX, WY, FX, FY, int32_t, true>));
   } else {
-    auto k = q8_gemm_kernel<WX, WY, FX, FY, int32_t>;
-    if (lds > 64 * 1024)
-      MH_HIP(ctx, hipFuncSetAttribute((const void *)k,
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    MH_PROF_BEGIN(ctx);
-    hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p);
+    MH_RETURN_IF_ERROR(launch(q8_gemm_kernel<WX, WY, FX, FY, int32_t, false>));
   }
   MH_PROF_END(ctx);
   MH_HIP(ctx, hipGetLastError());
@@ -647,20 +691,22 @@ int launch_gemm_dma(mace_hip_ctx *ctx, GemmParams &p, bool out_u8, int batch) {
   p.tiles_y = (p.YN + TY - 1) / TY;
   const size_t lds = (size_t)STAGES * (TX + TY) * SLAB;
   dim3 grid(p.tiles_x * p.tiles_y, 1, batch), block(WX * WY * 64);
-  if (out_u8) {
-    auto k = q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, uint8_t, OCC>;
+  auto launch = [&](auto k) -> int {
     if (lds > 64 * 1024)
       MH_HIP(ctx, hipFuncSetAttribute((const void *)k,
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     MH_PROF_BEGIN(ctx);
     hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p);
+    return MACE_HIP_SUCCESS;
+  };
+  if (out_u8 && p.sum_y) {
+    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, uint8_t, OCC, 0, true>));
+  } else if (out_u8) {
+    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, uint8_t, OCC, 0, false>));
+  } else if (p.sum_y) {
+    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, int32_t, OCC, 0, true>));
   } else {
-    auto k = q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, int32_t, OCC>;
-    if (lds > 64 * 1024)
-      MH_HIP(ctx, hipFuncSetAttribute((const void *)k,
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    MH_PROF_BEGIN(ctx);
-    hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p);
+    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, int32_t, OCC, 0, false>));
   }
   MH_PROF_END(ctx);
   MH_HIP(ctx, hipGetLastError());
@@ -746,18 +792,25 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   int32_t *corrR = (int32_t *)mh_arena_take(ctx, sizeof(int32_t) * rhs_nb * cols);
   if (!corrL || !corrR) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
   const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
+  const bool x_is_lhs = out_order == MACE_HIP_COL_MAJOR;
+  // The Y operand's row sums can be taken inside the GEMM kernel from the fragments it already
+  // holds, which saves one pass over that operand; worth it when the GEMM is short in K and the
+  // extra pass is a visible share of the memory traffic.
+  const bool sum_y = depth > 0 && depth <= 1024;
+  const int32_t l_coef = (int32_t)(0u - zr), l_add = 0;
+  const int32_t r_coef = (int32_t)(0u - zl), r_add = (int32_t)((uint32_t)depth * zl * zr);
+  const int32_t *l_bias = out_u8 ? ep.bias : nullptr;
   {
-    MH_RETURN_IF_ERROR(launch_panel_sums(ctx, L.ptr, L.ld, L.bs, rows, L.k, lhs_nb,
-                                         (int32_t)(0u - zr), 0, out_u8 ? ep.bias : nullptr,
-                                         corrL));
-    MH_RETURN_IF_ERROR(launch_panel_sums(ctx, R.ptr, R.ld, R.bs, cols, R.k, rhs_nb,
-                                         (int32_t)(0u - zl),
-                                         (int32_t)((uint32_t)depth * zl * zr), nullptr, corrR));
+    if (!(sum_y && !x_is_lhs))
+      MH_RETURN_IF_ERROR(launch_panel_sums(ctx, L.ptr, L.ld, L.bs, rows, L.k, lhs_nb, l_coef,
+                                           l_add, l_bias, corrL));
+    if (!(sum_y && x_is_lhs))
+      MH_RETURN_IF_ERROR(launch_panel_sums(ctx, R.ptr, R.ld, R.bs, cols, R.k, rhs_nb, r_coef,
+                                           r_add, nullptr, corrR));
     MH_HIP(ctx, hipGetLastError());
   }
 
   GemmParams p;
-  const bool x_is_lhs = out_order == MACE_HIP_COL_MAJOR;
   const Panel &PX = x_is_lhs ? L : R;
   const Panel &PY = x_is_lhs ? R : L;
   p.X = PX.ptr; p.ldx = PX.ld; p.xbs = PX.bs;
@@ -773,6 +826,10 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   p.ldo = p.XN;
   p.obs = rows * cols;
   p.rq = rq;
+  p.sum_y = sum_y;
+  p.ycoef = x_is_lhs ? r_coef : l_coef;
+  p.yadd = x_is_lhs ? r_add : l_add;
+  p.ybias = x_is_lhs ? nullptr : l_bias;
 
   // tile shape: the largest that still yields enough workgroups to fill the CUs
   const int64_t cu = ctx->cu_count > 0 ? ctx->cu_count : 256;
