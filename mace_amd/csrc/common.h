@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <string.h>
 
 #include "mace_hip.h"
 
@@ -25,6 +26,11 @@ struct mace_hip_ctx {
   int lds_bytes = 0;
   char arch[64] = {0};
   char err[512] = {0};
+  // last few requantization comparison tables built on this context (mult, shift, blo, n)
+  int32_t rq_cache_key[4][4] = {};
+  int32_t rq_cache_tab[4][258] = {};
+  int rq_cache_valid[4] = {0, 0, 0, 0};
+  int rq_cache_next = 0;
 };
 
 int mh_fail(mace_hip_ctx *ctx, int code, const char *fmt, ...);
@@ -117,7 +123,35 @@ struct RequantFixed {
   int32_t half;      // mask >> 1
   int32_t blo, bhi;  // lo - zp, hi - zp (must fit int32; checked by mh_make_requant)
   int32_t zp;
+  // Threshold form (see mh_requant_threshold): usable when table != 0
+  int32_t table;     // 1 = the kernels may requantize by threshold lookup
+  int32_t n;         // bhi - blo: number of thresholds
+  int32_t lo;        // lo = blo + zp: the output value below the first threshold
+  float inv, off;    // float estimate of the step index: floor(acc * inv + off)
 };
+
+// The pipeline z(x) = clamp(RDivPOT(SRDHM(x, mult), shift), blo, bhi) is a non-decreasing step
+// function of x when mult > 0, so z(x) = blo + #{ j in 1..n : x >= T[j] } with
+//   T[j] = min { x : RDivPOT(SRDHM(x, mult), shift) >= blo + j }.
+// RDivPOT(y, s) >= v  <=>  y >= Y(v), Y(v) = v 2^s - 2^(s-1) (+1 if v <= 0: ties go away from
+// zero), Y(v) = v for s = 0; SRDHM(x, m) = floor((x m + 2^30) / 2^31) >= Y
+//   <=>  x >= ceil((Y 2^31 - 2^30) / m).
+// Returns T[j] clamped to [INT32_MIN, INT32_MAX + 1] as int64.
+__host__ __device__ inline int64_t mh_requant_threshold(int32_t mult, int shift, int32_t blo,
+                                                        int j) {
+  const int64_t v = (int64_t)blo + j;
+  int64_t y = v;
+  if (shift > 0) y = v * ((int64_t)1 << shift) - ((int64_t)1 << (shift - 1)) + (v <= 0 ? 1 : 0);
+  if (y > (int64_t)INT32_MAX) return (int64_t)INT32_MAX + 1;   // never reached
+  if (y < (int64_t)INT32_MIN) return (int64_t)INT32_MIN;       // always reached
+  const int64_t num = y * ((int64_t)1 << 31) - ((int64_t)1 << 30);
+  int64_t q = num / mult;
+  if (num % mult > 0) ++q;   // ceil for a positive divisor
+  if (q > (int64_t)INT32_MAX) return (int64_t)INT32_MAX + 1;
+  if (q < (int64_t)INT32_MIN) return (int64_t)INT32_MIN;
+  return q;
+}
+
 // false when lo - zp or hi - zp leaves the int32 range (then the reference's own int32
 // addition of the offset overflows for some accumulators)
 inline bool mh_make_requant(int32_t mult, int shift, int32_t zp, int lo, int hi,
@@ -131,7 +165,55 @@ inline bool mh_make_requant(int32_t mult, int shift, int32_t zp, int lo, int hi,
   r->blo = (int32_t)blo;
   r->bhi = (int32_t)bhi;
   r->zp = zp;
+  // Threshold form: needs a monotone pipeline (mult > 0), a window close enough to zero for
+  // the float estimate of the step index to be within its error budget (|v| <= 2^15 gives an
+  // absolute error below 0.02 where it matters), and every threshold above INT32_MIN so that
+  // "x >= T" can be tested as "x > T - 1" in int32.
+  r->n = (int32_t)(bhi - blo);
+  r->lo = lo;
+  r->table = 0;
+  r->inv = 0.f;
+  r->off = 0.f;
+  if (mult > 0 && blo >= -32768 && bhi <= 32768 && r->n + 2 <= 258 &&
+      (r->n == 0 || mh_requant_threshold(mult, shift, r->blo, 1) > (int64_t)INT32_MIN)) {
+    r->table = 1;
+    r->inv = (float)((double)mult / 2147483648.0 / (double)((int64_t)1 << shift));
+    r->off = (float)(0.2 - (double)blo);
+  }
   return true;
+}
+// Entry j of the comparison table kept in LDS by the kernels: x >= T[j] <=> x > table[j];
+// entry n + 1 is a sentinel no x exceeds.
+constexpr int MH_REQUANT_TABLE_MAX = 258;   // n + 2 entries, n <= 256
+__host__ __device__ inline int32_t mh_requant_table_entry(const RequantFixed &q, int j) {
+  if (j > q.n) return INT32_MAX;
+  const int64_t t = mh_requant_threshold(q.mult, q.shift, q.blo, j) - 1;
+  return t > (int64_t)INT32_MAX ? INT32_MAX : (int32_t)t;
+}
+// The table of q (n + 2 entries) into tab; the context remembers the last few it built, since
+// a layer calls with the same parameters every time.
+inline void mh_requant_table_cached(mace_hip_ctx *ctx, const RequantFixed &q, int32_t *tab) {
+  const int32_t key[4] = {q.mult, q.shift, q.blo, q.n};
+  for (int e = 0; e < 4; ++e)
+    if (ctx->rq_cache_valid[e] && memcmp(ctx->rq_cache_key[e], key, sizeof(key)) == 0) {
+      memcpy(tab, ctx->rq_cache_tab[e], sizeof(int32_t) * (q.n + 2));
+      return;
+    }
+  const int e = ctx->rq_cache_next;
+  ctx->rq_cache_next = (e + 1) % 4;
+  for (int j = 0; j <= q.n + 1; ++j) ctx->rq_cache_tab[e][j] = mh_requant_table_entry(q, j);
+  memcpy(ctx->rq_cache_key[e], key, sizeof(key));
+  ctx->rq_cache_valid[e] = 1;
+  memcpy(tab, ctx->rq_cache_tab[e], sizeof(int32_t) * (q.n + 2));
+}
+// Step index of accumulator x: k with z = blo + k, out = lo + k.  c = floor(x * inv + off),
+// clamped to [0, n], is k or k - 1 (SRDHM and RDivPOT each move the value by at most half a
+// step of their own, 0.75 output steps together; 0.2 centres that band), one look-up decides.
+__device__ inline int mh_requant_step(int32_t x, const RequantFixed &q, const int32_t *table) {
+  float u = __fmaf_rn((float)x, q.inv, q.off);
+  u = __builtin_amdgcn_fmed3f(u, 0.0f, (float)q.n + 0.5f);
+  const int c = (int)u;   // u >= 0: truncation is floor
+  return c + (x > table[c + 1] ? 1 : 0);
 }
 __host__ __device__ inline int32_t mh_requant_fixed(int32_t acc, const RequantFixed &q) {
   const int32_t y = mh_srdhm(acc, q.mult);

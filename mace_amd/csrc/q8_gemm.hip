@@ -29,9 +29,17 @@ namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
 
 constexpr int BK = 64;            // bytes of k per LDS tile
 constexpr int LDS_ROW = BK + 16;  // padded row: any 8 consecutive rows cover all banks once
+
+// Comparison table of the threshold requantization (RequantFixed::table), second kernel
+// argument.  The kernels never name it: they read it from the argument segment, right after
+// GemmParams, with a lane-dependent index.
+struct RequantTable {
+  int32_t t[MH_REQUANT_TABLE_MAX];
+};
 
 struct GemmParams {
   const uint8_t *X;   // [XN][ldx] panel
@@ -91,7 +99,7 @@ __device__ inline int sum16_i8(const v4i &f, int acc) {
 // (uint8) access.  The correction vectors of the tile are staged through LDS first (the
 // operand buffers are dead by then), so the stores do not wait on scattered global loads.
 template <int WX, int WY, int FX, int FY, typename OutT, bool SUMY>
-__device__ inline void gemm_epilogue(v16i (&acc)[FX][FY], const int (&ysum)[FY],
+__device__ __forceinline__ void gemm_epilogue(v16i (&acc)[FX][FY], const int (&ysum)[FY],
                                      const GemmParams &p, uint8_t *lds, int b, int x0, int y0,
                                      int wx, int wy, int tid) {
   constexpr int NT = WX * WY * 64;
@@ -104,64 +112,129 @@ __device__ inline void gemm_epilogue(v16i (&acc)[FX][FY], const int (&ysum)[FY],
   for (int i = tid; i < TX; i += NT) sc[i] = cX[min(x0 + i, p.XN - 1)];
   if (!SUMY)
     for (int i = tid; i < TY; i += NT) sc[TX + i] = cY[min(y0 + i, p.YN - 1)];
+  const RequantFixed rq = p.rq;
+  int32_t *tab = sc + TX + TY;    // [n + 2] comparison table of the threshold requantization
+  if constexpr (sizeof(OutT) == 1) {
+    if (rq.table) {
+      // The table is the kernel's second argument, placed right behind GemmParams in the
+      // argument segment (indexing a by-value copy with a lane-dependent index would spill it)
+      static_assert(sizeof(GemmParams) % alignof(RequantTable) == 0, "argument layout");
+      const int32_t *arg_tab = (const int32_t *)((const char *)__builtin_amdgcn_kernarg_segment_ptr() +
+                                                 sizeof(GemmParams));
+      for (int j = tid; j <= rq.n + 1; j += NT) tab[j] = arg_tab[j];
+    }
+  }
   __syncthreads();
 
   OutT *outb = (OutT *)p.out + (int64_t)b * p.obs;
   const bool vec_ok = (p.ldo % 4 == 0) && (((uintptr_t)outb) % (4 * sizeof(OutT)) == 0);
   const bool interior = vec_ok && x0 + TX <= p.XN && y0 + TY <= p.YN;
-  const RequantFixed rq = p.rq;
+  const bool interior16 = interior && (p.ldo % 16 == 0) && (((uintptr_t)outb) % 16 == 0);
+
+  // One fully unrolled copy of the store loop per combination that occurs: TABLE = threshold
+  // requantization, WIDE = whole tile inside the matrix and 16-byte aligned rows.
+  auto store_tile = [&](auto table_tag, auto wide_tag) __attribute__((always_inline)) {
+    constexpr bool TABLE = decltype(table_tag)::value;
+    constexpr bool WIDE = decltype(wide_tag)::value;
 #pragma unroll
-  for (int j = 0; j < FY; ++j) {
-    const int yl = (wy * FY + j) * 32 + (lane & 31);
-    const int y = y0 + yl;
-    uint32_t cy;
-    if constexpr (SUMY) {
-      // lanes l and l ^ 32 hold the two 16-byte halves of every 32-byte k step of row y
-      const int total = ysum[j] + __shfl_xor(ysum[j], 32, 64);
-      cy = (uint32_t)p.ycoef * (uint32_t)total + (uint32_t)p.yadd;
-      if (p.ybias) cy += (uint32_t)p.ybias[min(y, p.YN - 1)];
-    } else {
-      cy = (uint32_t)sc[TX + yl];
-    }
-    OutT *orow = outb + (int64_t)y * p.ldo + x0;
+    for (int j = 0; j < FY; ++j) {
+      const int yl = (wy * FY + j) * 32 + (lane & 31);
+      const int y = y0 + yl;
+      uint32_t cy;
+      if constexpr (SUMY) {
+        // lanes l and l ^ 32 hold the two 16-byte halves of every 32-byte k step of row y
+        const int total = ysum[j] + __shfl_xor(ysum[j], 32, 64);
+        cy = (uint32_t)p.ycoef * (uint32_t)total + (uint32_t)p.yadd;
+        if (p.ybias) cy += (uint32_t)p.ybias[min(y, p.YN - 1)];
+      } else {
+        cy = (uint32_t)sc[TX + yl];
+      }
+      OutT *orow = outb + (int64_t)y * p.ldo + x0;
 #pragma unroll
-    for (int i = 0; i < FX; ++i) {
+      for (int i = 0; i < FX; ++i) {
+        const int xb = (wx * FX + i) * 32 + 4 * (lane >> 5);   // x of register group q: xb + 8 q
+        int32_t v[16];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int xl = (wx * FX + i) * 32 + 8 * q + 4 * (lane >> 5);
-        const v4i cx = *(const v4i *)(sc + xl);
-        int32_t v[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-          v[e] = (int32_t)((uint32_t)acc[i][j][q * 4 + e] + (uint32_t)cx[e] + cy);
-        if constexpr (sizeof(OutT) == 4) {
-          if (interior) {
-            *(v4i *)(orow + xl) = v4i{v[0], v[1], v[2], v[3]};
-          } else if (y < p.YN) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (x0 + xl + e < p.XN) orow[xl + e] = (OutT)v[e];
-          }
-        } else {
-          uint32_t packed = 0;
+        for (int q = 0; q < 4; ++q) {
+          const v4i cx = *(const v4i *)(sc + xb + 8 * q);
 #pragma unroll
           for (int e = 0; e < 4; ++e)
-            packed |= (uint32_t)mh_requant_fixed(v[e], rq) << (8 * e);
-          if (interior) {
-            *(uint32_t *)(orow + xl) = packed;
-          } else if (y < p.YN) {
+            v[q * 4 + e] = (int32_t)((uint32_t)acc[i][j][q * 4 + e] + (uint32_t)cx[e] + cy);
+        }
+        if constexpr (sizeof(OutT) == 4) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (x0 + xl + e < p.XN) orow[xl + e] = (OutT)((packed >> (8 * e)) & 0xff);
+          for (int q = 0; q < 4; ++q) {
+            const int xl = xb + 8 * q;
+            if (interior) {
+              *(v4i *)(orow + xl) = v4i{v[q * 4], v[q * 4 + 1], v[q * 4 + 2], v[q * 4 + 3]};
+            } else if (y < p.YN) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                if (x0 + xl + e < p.XN) orow[xl + e] = (OutT)v[q * 4 + e];
+            }
+          }
+        } else {
+          uint32_t packed[4] = {0, 0, 0, 0};
+          if constexpr (TABLE) {
+            // estimates first, then all look-ups, then the compares: sixteen LDS reads in
+            // flight instead of one round trip per element
+            int c[16], t[16];
+            const float top = (float)rq.n + 0.5f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              c[r] = (int)__builtin_amdgcn_fmed3f(__fmaf_rn((float)v[r], rq.inv, rq.off), 0.0f, top);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) t[r] = tab[c[r] + 1];
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              packed[r / 4] |= (uint32_t)(c[r] + (v[r] > t[r] ? 1 : 0)) << (8 * (r % 4));
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              packed[q] += (uint32_t)rq.lo * 0x01010101u;   // lo + k <= 255: no carries
+          } else {
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              packed[r / 4] |= (uint32_t)mh_requant_fixed(v[r], rq) << (8 * (r % 4));
+          }
+          if constexpr (WIDE) {
+            // Lane (y, h = lane / 32) holds bytes x = 8 q + 4 h + 0..3 of this 32-wide block
+            // in packed[q].  Swapping the upper half of one register with the lower half of
+            // another gives lane (y, 0) bytes 0..15 and lane (y, 1) bytes 16..31.
+            const v2u s02 = __builtin_amdgcn_permlane32_swap(packed[0], packed[2], false, false);
+            const v2u s13 = __builtin_amdgcn_permlane32_swap(packed[1], packed[3], false, false);
+            const v4i w = {(int)s02.x, (int)s02.y, (int)s13.x, (int)s13.y};
+            *(v4i *)(orow + (wx * FX + i) * 32 + 16 * (lane >> 5)) = w;
+          } else {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const int xl = xb + 8 * q;
+              if (interior) {
+                *(uint32_t *)(orow + xl) = packed[q];
+              } else if (y < p.YN) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                  if (x0 + xl + e < p.XN) orow[xl + e] = (OutT)((packed[q] >> (8 * e)) & 0xff);
+              }
+            }
           }
         }
+        // keep the 32x32 blocks apart: hoisting the next block's look-ups over this one's
+        // stores only costs registers
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
+  };
+  if constexpr (sizeof(OutT) == 4) {
+    store_tile(std::false_type{}, std::false_type{});
+  } else {
+    if (rq.table && interior16) store_tile(std::true_type{}, std::true_type{});
+    else if (rq.table) store_tile(std::true_type{}, std::false_type{});
+    else store_tile(std::false_type{}, std::false_type{});
   }
 }
 
 template <int WX, int WY, int FX, int FY, typename OutT, bool SUMY = false>
-__global__ __launch_bounds__(WX *WY * 64) void q8_gemm_kernel(GemmParams p) {
+__global__ __launch_bounds__(WX *WY * 64) void q8_gemm_kernel(GemmParams p, RequantTable) {
   constexpr int NT = WX * WY * 64;
   constexpr int TX = WX * FX * 32;
   constexpr int TY = WY * FY * 32;
@@ -339,7 +412,7 @@ __device__ inline void wait_vmcnt() {
 
 template <int WX, int WY, int FX, int FY, int STAGES, typename OutT, int OCC = 1, int ABLATE = 0,
           bool SUMY = false>
-__global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParams p) {
+__global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParams p, RequantTable) {
   constexpr int NW = WX * WY;
   constexpr int TX = WX * FX * 32;
   constexpr int TY = WY * FY * 32;
@@ -655,7 +728,8 @@ int launch_panel_sums(mace_hip_ctx *ctx, const uint8_t *P, int64_t ld, int64_t p
 }
 
 template <int WX, int WY, int FX, int FY>
-int launch_gemm(mace_hip_ctx *ctx, GemmParams &p, bool out_u8, int batch) {
+int launch_gemm(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, bool out_u8,
+                int batch) {
   constexpr int TX = WX * FX * 32, TY = WY * FY * 32;
   p.tiles_x = (p.XN + TX - 1) / TX;
   p.tiles_y = (p.YN + TY - 1) / TY;
@@ -666,7 +740,7 @@ int launch_gemm(mace_hip_ctx *ctx, GemmParams &p, bool out_u8, int batch) {
       MH_HIP(ctx, hipFuncSetAttribute((const void *)k,
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     MH_PROF_BEGIN(ctx);
-    hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p);
+    hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, tab);
     return MACE_HIP_SUCCESS;
   };
   if (out_u8 && p.sum_y) {
@@ -685,7 +759,8 @@ int launch_gemm(mace_hip_ctx *ctx, GemmParams &p, bool out_u8, int batch) {
 
 // the streaming kernel; the caller has checked K % 64 == 0 and K >= 64 * (STAGES - 1)
 template <int WX, int WY, int FX, int FY, int STAGES, int OCC>
-int launch_gemm_dma(mace_hip_ctx *ctx, GemmParams &p, bool out_u8, int batch) {
+int launch_gemm_dma(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, bool out_u8,
+                    int batch) {
   constexpr int TX = WX * FX * 32, TY = WY * FY * 32;
   p.tiles_x = (p.XN + TX - 1) / TX;
   p.tiles_y = (p.YN + TY - 1) / TY;
@@ -696,7 +771,7 @@ int launch_gemm_dma(mace_hip_ctx *ctx, GemmParams &p, bool out_u8, int batch) {
       MH_HIP(ctx, hipFuncSetAttribute((const void *)k,
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     MH_PROF_BEGIN(ctx);
-    hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p);
+    hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, tab);
     return MACE_HIP_SUCCESS;
   };
   if (out_u8 && p.sum_y) {
@@ -826,6 +901,8 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   p.ldo = p.XN;
   p.obs = rows * cols;
   p.rq = rq;
+  RequantTable tab;
+  if (out_u8 && rq.table) mh_requant_table_cached(ctx, rq, tab.t);
   p.sum_y = sum_y;
   p.ycoef = x_is_lhs ? r_coef : l_coef;
   p.yadd = x_is_lhs ? r_add : l_add;
@@ -855,15 +932,15 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   const bool medium = !big && !skinny && s_medium == best;
   // the streaming kernel needs whole 64-byte slabs and enough of them to fill its ring
   if (p.K % SLAB == 0 && p.K >= SLAB * 3) {
-    if (big) return launch_gemm_dma<2, 2, 4, 4, 4, 1>(ctx, p, out_u8, (int)batch);
-    if (skinny) return launch_gemm_dma<1, 4, 2, 2, 4, 2>(ctx, p, out_u8, (int)batch);
-    if (medium) return launch_gemm_dma<2, 2, 2, 2, 4, 2>(ctx, p, out_u8, (int)batch);
-    return launch_gemm_dma<2, 2, 1, 1, 4, 4>(ctx, p, out_u8, (int)batch);
+    if (big) return launch_gemm_dma<2, 2, 4, 4, 4, 1>(ctx, p, tab, out_u8, (int)batch);
+    if (skinny) return launch_gemm_dma<1, 4, 2, 2, 4, 2>(ctx, p, tab, out_u8, (int)batch);
+    if (medium) return launch_gemm_dma<2, 2, 2, 2, 4, 2>(ctx, p, tab, out_u8, (int)batch);
+    return launch_gemm_dma<2, 2, 1, 1, 4, 4>(ctx, p, tab, out_u8, (int)batch);
   }
-  if (big) return launch_gemm<2, 2, 4, 4>(ctx, p, out_u8, (int)batch);
-  if (skinny) return launch_gemm<1, 4, 2, 2>(ctx, p, out_u8, (int)batch);
-  if (medium) return launch_gemm<2, 2, 2, 2>(ctx, p, out_u8, (int)batch);
-  return launch_gemm<2, 2, 1, 1>(ctx, p, out_u8, (int)batch);
+  if (big) return launch_gemm<2, 2, 4, 4>(ctx, p, tab, out_u8, (int)batch);
+  if (skinny) return launch_gemm<1, 4, 2, 2>(ctx, p, tab, out_u8, (int)batch);
+  if (medium) return launch_gemm<2, 2, 2, 2>(ctx, p, tab, out_u8, (int)batch);
+  return launch_gemm<2, 2, 1, 1>(ctx, p, tab, out_u8, (int)batch);
 }
 
 extern "C" {
