@@ -99,6 +99,16 @@ uint8_t mace_hip_quantize_u8(float value, float scale, int32_t zero_point);
  * gemmlowp quantize-down-by-fixed-point + saturating cast (see mace_hip_gemm_q8_u8). */
 uint8_t mace_hip_requant_fixed_u8(int32_t acc, int32_t multiplier, int right_shift,
                                   int32_t offset_after_shift, int clamp_min, int clamp_max);
+/* The same pipeline in the form the GEMM kernels use for their uint8 stores, evaluated on the
+ * host for CPU-side tests: the pipeline is a non-decreasing step function of the accumulator,
+ * so the kernels locate the step with one float multiply-add and one comparison against a
+ * table of exact thresholds.  Returns 1 when that form applies to the parameters, 0 when the
+ * kernels fall back to the arithmetic of mace_hip_requant_fixed_u8 (non-positive multiplier,
+ * clamp window further than 2^15 from the offset), -1 on invalid arguments; *out is the
+ * requantized value in the first two cases. */
+int mace_hip_requant_table_u8(int32_t acc, int32_t multiplier, int right_shift,
+                              int32_t offset_after_shift, int clamp_min, int clamp_max,
+                              uint8_t *out);
 /* The Gemv float requantisation evaluated on the host (see mace_hip_gemv_q8_u8). */
 uint8_t mace_hip_requant_float_u8(int32_t acc, float multiplier, int32_t out_zp, int mode);
 

@@ -3,6 +3,7 @@
 #define MACE_AMD_CSRC_COMMON_H_
 
 #include <hip/hip_runtime.h>
+#include <math.h>
 #include <stdint.h>
 #include <stdio.h>
 #include <string.h>
@@ -209,9 +210,16 @@ inline void mh_requant_table_cached(mace_hip_ctx *ctx, const RequantFixed &q, in
 // Step index of accumulator x: k with z = blo + k, out = lo + k.  c = floor(x * inv + off),
 // clamped to [0, n], is k or k - 1 (SRDHM and RDivPOT each move the value by at most half a
 // step of their own, 0.75 output steps together; 0.2 centres that band), one look-up decides.
-__device__ inline int mh_requant_step(int32_t x, const RequantFixed &q, const int32_t *table) {
+__host__ __device__ inline int mh_requant_step(int32_t x, const RequantFixed &q,
+                                               const int32_t *table) {
+#if defined(__HIP_DEVICE_COMPILE__)
   float u = __fmaf_rn((float)x, q.inv, q.off);
   u = __builtin_amdgcn_fmed3f(u, 0.0f, (float)q.n + 0.5f);
+#else
+  float u = fmaf((float)x, q.inv, q.off);
+  const float top = (float)q.n + 0.5f;
+  u = u < 0.0f ? 0.0f : (u > top ? top : u);
+#endif
   const int c = (int)u;   // u >= 0: truncation is floor
   return c + (x > table[c + 1] ? 1 : 0);
 }

@@ -246,6 +246,23 @@ uint8_t mace_hip_requant_fixed_u8(int32_t acc, int32_t multiplier, int right_shi
   return (uint8_t)mh_requant_fixed(acc, q);
 }
 
+int mace_hip_requant_table_u8(int32_t acc, int32_t multiplier, int right_shift,
+                              int32_t offset_after_shift, int clamp_min, int clamp_max,
+                              uint8_t *out) {
+  RequantFixed q;
+  if (!out || clamp_min < 0 || clamp_max > 255 || clamp_min > clamp_max ||
+      !mh_make_requant(multiplier, right_shift, offset_after_shift, clamp_min, clamp_max, &q))
+    return -1;
+  if (!q.table) {
+    *out = (uint8_t)mh_requant_fixed(acc, q);
+    return 0;
+  }
+  int32_t tab[MH_REQUANT_TABLE_MAX];
+  for (int j = 0; j <= q.n + 1; ++j) tab[j] = mh_requant_table_entry(q, j);
+  *out = (uint8_t)(q.lo + mh_requant_step(acc, q, tab));
+  return 1;
+}
+
 uint8_t mace_hip_requant_float_u8(int32_t acc, float multiplier, int32_t out_zp, int mode) {
   return mh_requant_float(acc, multiplier, out_zp, mode == MACE_HIP_REQUANT_NEON);
 }

@@ -54,6 +54,7 @@ SIGNATURES = {
                                                         C.POINTER(_int)]),
     "mace_hip_quantize_u8": (C.c_uint8, [_f32, _f32, _i32]),
     "mace_hip_requant_fixed_u8": (C.c_uint8, [_i32, _i32, _int, _i32, _int, _int]),
+    "mace_hip_requant_table_u8": (_int, [_i32, _i32, _int, _i32, _int, _int, C.POINTER(C.c_uint8)]),
     "mace_hip_requant_float_u8": (C.c_uint8, [_i32, _f32, _i32, _int]),
     "mace_hip_gemm_f32": (_int, _GEMM_F32),
     "mace_hip_gemm_f32_transpose": (_int, [_p, _p, _p, _i64, _i64, _i64, _i64, _i64, _int,

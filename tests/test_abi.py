@@ -64,6 +64,59 @@ def test_fixed_point_requant_matches_oracle():
                 orc.requant_fixed_u8(acc, 2 ** 30, shift, 100, 0, 255)
 
 
+def test_threshold_requant_matches_oracle_at_every_step():
+    """The kernels' uint8 stores locate the output step with a float estimate and one exact
+    threshold comparison.  Pin that form where it can go wrong: one below, at and one above
+    every point where the oracle's output changes (found by bisection on the oracle, which is
+    monotone for a positive multiplier), plus the int32 extremes and random accumulators."""
+    import ctypes as C
+    lib = mh.load()
+    rng = np.random.default_rng(7)
+    out = C.c_uint8()
+
+    def table(acc, mult, shift, zp, lo, hi):
+        rc = lib.mace_hip_requant_table_u8(acc, mult, shift, zp, lo, hi, C.byref(out))
+        assert rc >= 0
+        return rc, out.value
+
+    cases = [(1649267328, 7, 128, 0, 255), (2 ** 30, 0, 0, 0, 255), (2 ** 31 - 1, 0, 3, 0, 255),
+             (2 ** 30, 31, 0, 0, 255), (2 ** 31 - 1, 31, 255, 0, 255), (1419781096, 13, 128, 0, 255),
+             (2 ** 30 + 1, 1, 57, 17, 201), (1 << 30, 2, -300, 0, 255), (1518500250, 3, 700, 0, 255),
+             (1, 0, 10, 0, 255), (3, 1, 250, 0, 255), (2 ** 30, 5, 32000, 0, 255),
+             (2 ** 30, 5, -32000, 0, 255), (2 ** 31 - 1, 30, 77, 77, 77)]
+    for _ in range(12):
+        lo = int(rng.integers(0, 200))
+        cases.append((int(rng.integers(2 ** 30, 2 ** 31)), int(rng.integers(0, 32)),
+                      int(rng.integers(-400, 700)), lo, int(rng.integers(lo, 256))))
+    used_table = 0
+    for (mult, shift, zp, lo, hi) in cases:
+        def ref(acc):
+            return orc.requant_fixed_u8(acc, mult, shift, zp, lo, hi)
+        probes = {-2 ** 31, -2 ** 31 + 1, 2 ** 31 - 1, 2 ** 31 - 2, 0, -1, 1}
+        probes.update(int(a) for a in rng.integers(-2 ** 31, 2 ** 31, 200))
+        vmin, vmax = ref(-2 ** 31), ref(2 ** 31 - 1)
+        for v in range(vmin + 1, vmax + 1):          # smallest acc with output >= v
+            a, b = -2 ** 31, 2 ** 31 - 1             # ref(a) < v <= ref(b)
+            while b - a > 1:
+                m = (a + b) // 2
+                if ref(m) >= v:
+                    b = m
+                else:
+                    a = m
+            probes.update((b - 2, b - 1, b, b + 1))
+        for acc in probes:
+            if -2 ** 31 <= acc < 2 ** 31:
+                rc, got = table(acc, mult, shift, zp, lo, hi)
+                used_table += rc
+                assert got == ref(acc), (acc, mult, shift, zp, lo, hi, rc)
+    assert used_table > 0
+    # parameters outside the threshold form fall back to the plain arithmetic
+    for (mult, shift, zp) in ((-2 ** 31, 3, 10), (-5, 0, 0), (2 ** 30, 4, 40000), (2 ** 30, 4, -40000)):
+        for acc in (-2 ** 31, -12345, 0, 999, 2 ** 31 - 1):
+            rc, got = table(acc, mult, shift, zp, 0, 255)
+            assert rc == 0 and got == orc.requant_fixed_u8(acc, mult, shift, zp, 0, 255)
+
+
 def test_float_requant_matches_oracle():
     lib = mh.load()
     rng = np.random.default_rng(2)

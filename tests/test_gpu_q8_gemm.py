@@ -97,6 +97,54 @@ def test_q8_gemm_config1_matmul(ctx):
     assert 0 < (want8 == 0).mean() + (want8 == 255).mean() < 0.9
 
 
+@pytest.mark.parametrize("mult,shift,zp,clamp", [
+    (1649267328, 7, 128, (0, 255)), (2 ** 30, 0, 0, (0, 255)), (2 ** 31 - 1, 12, 3, (0, 255)),
+    (1419781096, 13, 200, (17, 201)), (1518500250, 20, -300, (0, 255)),
+    (2 ** 30, 9, 40000, (0, 255)),       # window too far from the offset: arithmetic fallback
+    (-2 ** 31, 5, 100, (0, 255)),        # non-monotone multiplier: arithmetic fallback
+])
+@pytest.mark.parametrize("rows,cols,oo", [(256, 256, R), (256, 256, Cm), (250, 251, R)])
+def test_q8_gemm_requant_at_every_step(ctx, mult, shift, zp, clamp, rows, cols, oo):
+    """Accumulators placed on and around every point where the requantized output changes:
+    row i adds bias[i] = the smallest accumulator that reaches output step i + 1 (bisection on
+    the oracle), and column j contributes j - 128, so each row sweeps 256 consecutive
+    accumulators across its threshold."""
+    depth = 16
+    lo_c, hi_c = clamp
+
+    def ref(acc):
+        return orc.requant_fixed_u8(acc, mult, shift, zp, lo_c, hi_c)
+
+    bias = np.zeros(rows, np.int32)
+    vmin, vmax = ref(-2 ** 31 + 200), ref(2 ** 31 - 200)
+    monotone = mult > 0
+    for i in range(rows):
+        v = min(vmin, vmax) + 1 + i
+        if monotone and v <= max(vmin, vmax):
+            a, b = -2 ** 31 + 200, 2 ** 31 - 200
+            while b - a > 1:
+                m = (a + b) // 2
+                a, b = (a, m) if ref(m) >= v else (m, b)
+            bias[i] = b
+        else:
+            bias[i] = np.int32((i * 16777259) % (2 ** 32) - 2 ** 31) // 2
+    L = np.full((1, rows, depth), 77, np.uint8)        # lhs + lhs_offset = 0 ...
+    L[0, :, 0] = 78                                    # ... except a single 1 per row
+    Rr = np.full((1, depth, cols), 128, np.uint8)
+    Rr[0, 0, :] = (np.arange(cols) % 256).astype(np.uint8)   # rhs + rhs_offset = j - 128
+    want32 = orc.q8_gemm_i32(L, Rr, 1, rows, cols, depth, -77, -128, R, R, oo)
+    exp = (np.arange(cols) % 256 - 128)[None, :].repeat(rows, 0)
+    np.testing.assert_array_equal(want32.reshape((rows, cols) if oo == R else (cols, rows)),
+                                  exp if oo == R else exp.T)
+    want8 = orc.q8_gemm_u8(L, Rr, 1, rows, cols, depth, -77, -128, bias, mult, shift, zp, lo_c,
+                           hi_c, R, R, oo)
+    got8 = gemm_u8_host(ctx, L, R, Rr, R, oo, 1, rows, depth, cols, True, True, -77, -128, bias,
+                        mult, shift, zp, lo_c, hi_c)
+    np.testing.assert_array_equal(got8, want8)
+    if monotone and abs(zp) < 30000:
+        assert len(np.unique(want8)) > 100
+
+
 @pytest.mark.parametrize("n,lo,ro,oo", [(1024, R, R, R), (1024, R, Cm, Cm), (2048, R, R, R)])
 def test_q8_gemm_large_device_pointers(ctx, n, lo, ro, oo):
     """Square GEMMs through the device-pointer entry points (the 256x256 tile path), random
