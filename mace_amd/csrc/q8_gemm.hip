@@ -59,6 +59,9 @@ struct GemmParams {
   int32_t ycoef, yadd;
   const int32_t *ybias;
   bool sum_y;
+  // Same for the X panel (streaming kernel only, which sums both panels itself)
+  int32_t xcoef, xadd;
+  const int32_t *xbias;
   int tiles_x, tiles_y;
   long long *dbg;     // lab instrumentation only (nullptr in the library)
 };
@@ -605,6 +608,142 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
   gemm_epilogue<WX, WY, FX, FY, OutT, SUMY>(acc, ysum, p, lds, b, x0, y0, wx, wy, tid);
 }
 
+// ---- the streaming kernel for a small X panel ------------------------------------------------
+//
+// When the X panel is small in both directions (a 1x1 convolution's filter; the host sends
+// XN <= 128 rows of K <= 64 bytes here, where it measured a gain) the product is bound by streaming Y in and the result out, and the
+// tiled kernels above spend their time in per-tile latency chains (fill LDS, barrier, multiply,
+// barrier, stage corrections, store).  Here nothing is tiled: every wavefront keeps its share
+// of X as MFMA A-fragments in registers for the whole kernel and walks over blocks of 32 Y
+// rows.  A Y block needs no LDS either -- lane l loads the 16 bytes of row l % 32 that the
+// MFMA expects from it straight from global memory, 1 KiB contiguous per wavefront and k
+// step -- so a block is: loads (issued D blocks ahead), flip, row sums, FX * KS MFMAs, the
+// requantizing epilogue, 16-byte stores.  Both correction vectors are computed here (X once
+// per workgroup, into LDS; Y per block from the fragments), so the call is this one launch.
+//
+// XN = 32 * FX * XW exactly, K = 32 * KS exactly, uint8 output by threshold look-up only,
+// result rows (ldo = XN bytes) and base 16-byte aligned: the host checks all of that.
+template <int FX, int KS, int XW, int D>
+__global__ __launch_bounds__(256) void q8_gemm_stream_kernel(GemmParams p, RequantTable) {
+  constexpr int YW = 4 / XW;   // wavefronts of the workgroup along Y
+  __shared__ int32_t s_cx[32 * FX * XW];
+  __shared__ int32_t s_tab[MH_REQUANT_TABLE_MAX];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wx = wave % XW, wy = wave / XW;
+  const int h = lane >> 5, r32 = lane & 31;
+  const int b = blockIdx.z;
+  const uint8_t *Xb = p.X + (int64_t)b * p.xbs;
+  const uint8_t *Yb = p.Y + (int64_t)b * p.ybs;
+  uint8_t *outb = (uint8_t *)p.out + (int64_t)b * p.obs;
+  const RequantFixed rq = p.rq;
+  const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+
+  // this wavefront's X fragments, shifted to int8, and their row sums
+  v4i xf[FX][KS];
+#pragma unroll
+  for (int i = 0; i < FX; ++i) {
+    const int x = (wx * FX + i) * 32 + r32;
+    const uint8_t *src = Xb + (int64_t)x * p.ldx + 16 * h;
+    int xs = 0;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      xf[i][ks] = *(const v4i *)(src + 32 * ks) ^ flip;
+      xs = sum16_i8(xf[i][ks], xs);
+    }
+    xs += __shfl_xor(xs, 32, 64);
+    if (wy == 0 && h == 0) {
+      uint32_t c = (uint32_t)p.xcoef * (uint32_t)xs + (uint32_t)p.xadd;
+      if (p.xbias) c += (uint32_t)p.xbias[x];
+      s_cx[x] = (int32_t)c;
+    }
+  }
+  {
+    const int32_t *arg_tab = (const int32_t *)((const char *)__builtin_amdgcn_kernarg_segment_ptr() +
+                                               sizeof(GemmParams));
+    for (int j = tid; j <= rq.n + 1; j += 256) s_tab[j] = arg_tab[j];
+  }
+  __syncthreads();
+
+  const int nblk = (p.YN + 31) / 32;
+  const int stride = gridDim.x * YW;
+  int blk = blockIdx.x * YW + wy;
+  // rows past the end are clamped to the last one: always readable, never stored
+  auto load_y = [&](int bk, v4i (&yf)[KS]) {
+    const int row = min(bk * 32 + r32, p.YN - 1);
+    const uint8_t *src = Yb + (int64_t)row * p.ldy + 16 * h;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) yf[ks] = __builtin_nontemporal_load((const v4i *)(src + 32 * ks));
+  };
+  v4i yf[D][KS];
+#pragma unroll
+  for (int d = 0; d < D; ++d) load_y(blk + d * stride, yf[d]);
+  const float top = (float)rq.n + 0.5f;
+  const uint32_t lo4 = (uint32_t)rq.lo * 0x01010101u;
+
+  while (blk < nblk) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const int cur = blk + d * stride;
+      if (cur < nblk) {   // uniform over the wavefront
+        v4i f[KS];
+        int ys = 0;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          f[ks] = yf[d][ks] ^ flip;
+          ys = sum16_i8(f[ks], ys);
+        }
+        load_y(cur + D * stride, yf[d]);   // refill this slot for D blocks ahead
+        ys += __shfl_xor(ys, 32, 64);
+        const int y = cur * 32 + r32;
+        uint32_t cy = (uint32_t)p.ycoef * (uint32_t)ys + (uint32_t)p.yadd;
+        if (p.ybias) cy += (uint32_t)p.ybias[min(y, p.YN - 1)];
+        uint8_t *orow = outb + (int64_t)y * p.ldo + 16 * h;
+#pragma unroll
+        for (int i = 0; i < FX; ++i) {
+          v16i acc;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[r] = 0;
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks)
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(xf[i][ks], f[ks], acc, 0, 0, 0);
+          // register r: x = 8 (r / 4) + 4 h + r % 4 of this 32-row X block, y = lane % 32
+          const int xb = (wx * FX + i) * 32 + 4 * h;
+          int32_t v[16];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const v4i cx = *(const v4i *)(s_cx + xb + 8 * q);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              v[q * 4 + e] = (int32_t)((uint32_t)acc[q * 4 + e] + (uint32_t)cx[e] + cy);
+          }
+          int c[16], t[16];
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            c[r] = (int)__builtin_amdgcn_fmed3f(__fmaf_rn((float)v[r], rq.inv, rq.off), 0.0f, top);
+#pragma unroll
+          for (int r = 0; r < 16; ++r) t[r] = s_tab[c[r] + 1];
+          uint32_t packed[4] = {0, 0, 0, 0};
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            packed[r / 4] |= (uint32_t)(c[r] + (v[r] > t[r] ? 1 : 0)) << (8 * (r % 4));
+#pragma unroll
+          for (int q = 0; q < 4; ++q) packed[q] += lo4;
+          const v2u s02 = __builtin_amdgcn_permlane32_swap(packed[0], packed[2], false, false);
+          const v2u s13 = __builtin_amdgcn_permlane32_swap(packed[1], packed[3], false, false);
+          const v4i w = {(int)s02.x, (int)s02.y, (int)s13.x, (int)s13.y};
+          // plain stores: measured faster here than non-temporal ones
+          if (y < p.YN) *(v4i *)(orow + (wx * FX + i) * 32) = w;
+        }
+      }
+    }
+    blk += D * stride;
+  }
+}
+
+
 // ---- repacking ---------------------------------------------------------------------------
 
 // src is k-contiguous already ([n][k], row stride = k) but k is not a multiple of 16 or the
@@ -788,6 +927,28 @@ int launch_gemm_dma(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, b
   return MACE_HIP_SUCCESS;
 }
 
+// the streaming kernel; the caller has checked its preconditions (see the kernel)
+template <int FX, int XW>
+int launch_gemm_stream(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, int batch) {
+  constexpr int YW = 4 / XW;
+  const int nblk = (p.YN + 31) / 32;
+  const int ks = p.K / 32;
+  // resident workgroups per CU by register footprint (X fragments dominate)
+  const int per_cu = FX * ks <= 4 ? 4 : (FX * ks <= 16 ? 2 : 1);
+  const int cu = ctx->cu_count > 0 ? ctx->cu_count : 256;
+  const int wgs = std::max(1, std::min((nblk + YW - 1) / YW, cu * per_cu));
+  dim3 grid(wgs, 1, batch), block(256);
+  MH_PROF_BEGIN(ctx);
+  switch (ks) {
+    case 1: hipLaunchKernelGGL((q8_gemm_stream_kernel<FX, 1, XW, 4>), grid, block, 0, ctx->stream, p, tab); break;
+    case 2: hipLaunchKernelGGL((q8_gemm_stream_kernel<FX, 2, XW, 4>), grid, block, 0, ctx->stream, p, tab); break;
+    default: return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "streaming kernel: unsupported depth");
+  }
+  MH_PROF_END(ctx);
+  MH_HIP(ctx, hipGetLastError());
+  return MACE_HIP_SUCCESS;
+}
+
 }  // namespace
 
 int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8_t *rhs,
@@ -875,7 +1036,14 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   const int32_t l_coef = (int32_t)(0u - zr), l_add = 0;
   const int32_t r_coef = (int32_t)(0u - zl), r_add = (int32_t)((uint32_t)depth * zl * zr);
   const int32_t *l_bias = out_u8 ? ep.bias : nullptr;
-  {
+  // A small X panel (at most 128 rows of at most 64 bytes: an early 1x1 convolution's filter) against a
+  // long Y panel goes to the streaming kernel, which also sums both panels itself.
+  const int64_t xn = x_is_lhs ? rows : cols, yn = x_is_lhs ? cols : rows;
+  // (Measured: it wins for K <= 64; from K = 128 on the tiled kernels are as fast.)
+  const bool stream = out_u8 && rq.table && lhs_direct && rhs_direct &&
+                      (depth == 32 || depth == 64) && (xn == 32 || xn == 64 || xn == 128) &&
+                      yn >= 1024 && ((uintptr_t)out % 16 == 0);
+  if (!stream) {
     if (!(sum_y && !x_is_lhs))
       MH_RETURN_IF_ERROR(launch_panel_sums(ctx, L.ptr, L.ld, L.bs, rows, L.k, lhs_nb, l_coef,
                                            l_add, l_bias, corrL));
@@ -907,6 +1075,18 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   p.ycoef = x_is_lhs ? r_coef : l_coef;
   p.yadd = x_is_lhs ? r_add : l_add;
   p.ybias = x_is_lhs ? nullptr : l_bias;
+  p.xcoef = x_is_lhs ? l_coef : r_coef;
+  p.xadd = x_is_lhs ? l_add : r_add;
+  p.xbias = x_is_lhs ? l_bias : nullptr;
+  p.tiles_x = p.tiles_y = 0;
+  p.dbg = nullptr;
+  if (stream) {
+    switch (p.XN) {
+      case 32: return launch_gemm_stream<1, 1>(ctx, p, tab, (int)batch);
+      case 64: return launch_gemm_stream<2, 1>(ctx, p, tab, (int)batch);
+      default: return launch_gemm_stream<4, 1>(ctx, p, tab, (int)batch);
+    }
+  }
 
   // tile shape: the largest that still yields enough workgroups to fill the CUs
   const int64_t cu = ctx->cu_count > 0 ? ctx->cu_count : 256;

@@ -145,6 +145,37 @@ def test_q8_gemm_requant_at_every_step(ctx, mult, shift, zp, clamp, rows, cols, 
         assert len(np.unique(want8)) > 100
 
 
+@pytest.mark.parametrize("xn,depth,yn,batch", [
+    (64, 32, 4096, 1), (32, 32, 1031, 1), (128, 128, 2048, 1), (256, 256, 1500, 1),
+    (64, 64, 1024, 3), (128, 32, 5000, 1), (256, 64, 1111, 2), (32, 256, 1025, 1),
+    (128, 64, 3000, 2), (64, 32, 2049, 1), (64, 128, 1056, 1), (32, 64, 40000, 1),
+])
+@pytest.mark.parametrize("x_is_lhs", [True, False])
+def test_q8_gemm_small_panel_streaming(ctx, xn, depth, yn, batch, x_is_lhs):
+    """A small operand (at most 256 x 256) against a long one, both k-contiguous, uint8 result
+    with the small dimension contiguous: the shapes of a 1x1 convolution (filter as the
+    left-hand side, column-major result) and of a MatMul with a narrow right-hand side.  Long
+    dimensions include non-multiples of 32; the bias runs along either side."""
+    rng = np.random.default_rng(xn * 7 + depth * 3 + yn + batch)
+    if x_is_lhs:    # lhs [xn x depth] RowMajor, rhs [depth x yn] ColMajor, result ColMajor
+        rows, cols, oo = xn, yn, Cm
+    else:           # lhs [yn x depth] RowMajor, rhs [depth x xn] ColMajor, result RowMajor
+        rows, cols, oo = yn, xn, R
+    L = rng.integers(0, 256, (batch, rows, depth), dtype=np.uint8)
+    Rr = rng.integers(0, 256, (batch, depth, cols), dtype=np.uint8)
+    l, r = as_major(L, R), as_major(Rr, Cm)
+    lzp, rzp = int(rng.integers(120, 136)), int(rng.integers(120, 136))   # keeps the mean small
+    mult, shift = scales_for(depth)
+    bias = rng.integers(-2 ** 15, 2 ** 15, rows).astype(np.int32)
+    for bb, zp, clamp in ((bias, 90, (90, 200)), (None, 0, (0, 255)), (bias, 128, (0, 255))):
+        want8 = orc.q8_gemm_u8(l, r, batch, rows, cols, depth, -lzp, -rzp, bb, mult, shift, zp,
+                               clamp[0], clamp[1], R, Cm, oo, True, True)
+        got8 = gemm_u8_host(ctx, l, R, r, Cm, oo, batch, rows, depth, cols, True, True, -lzp,
+                            -rzp, bb, mult, shift, zp, clamp[0], clamp[1])
+        np.testing.assert_array_equal(got8, want8)
+    assert len(np.unique(want8)) > 8       # zero point 128: both signs of the sums survive
+
+
 @pytest.mark.parametrize("n,lo,ro,oo", [(1024, R, R, R), (1024, R, Cm, Cm), (2048, R, R, R)])
 def test_q8_gemm_large_device_pointers(ctx, n, lo, ro, oo):
     """Square GEMMs through the device-pointer entry points (the 256x256 tile path), random
