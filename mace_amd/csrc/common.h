@@ -267,6 +267,22 @@ __host__ __device__ inline uint8_t mh_requant_float(int32_t acc, float m, int32_
   return mh_saturate_u8(mh_roundf(v));
 }
 
+#if defined(__HIPCC__)
+// global_load_lds_dwordx4: every lane fetches 16 bytes from its own global address; the wave's
+// 64 x 16 bytes land contiguously in LDS from lds_wave_base (which must be wave-uniform) on.
+__device__ inline void mh_dma_16B(const uint8_t *g, uint8_t *lds_wave_base) {
+  __builtin_amdgcn_global_load_lds(
+      (const void __attribute__((address_space(1))) *)g,
+      (void __attribute__((address_space(3))) *)lds_wave_base, 16, 0, 0);
+}
+// the same transfer marked non-temporal (cache-policy bit 1): for data read once per call
+__device__ inline void mh_dma_16B_stream(const uint8_t *g, uint8_t *lds_wave_base) {
+  __builtin_amdgcn_global_load_lds(
+      (const void __attribute__((address_space(1))) *)g,
+      (void __attribute__((address_space(3))) *)lds_wave_base, 16, 0, 2);
+}
+#endif
+
 // ---- internal launch entry points (defined next to their kernels) ----------------------
 
 struct Q8GemmEpilogue {

@@ -11,6 +11,7 @@
 // loads of a row are issued before the first dot product so a CU keeps tens of KiB in
 // flight.  Up to NB batch rows of the right-hand vector are consumed per pass over the
 // weights, so the weight matrix is streamed once for batch <= 8.
+#include <algorithm>
 #include <type_traits>
 
 #include "common.h"
@@ -283,6 +284,190 @@ __global__ __launch_bounds__(NWAVES * 64) void q8_gemv_rows_kernel(GemvParams p)
   }
 }
 
+// Shared weights against several right-hand vectors (batch >= 2): the per-lane dot products of
+// the kernel above cost NB LDS reads and NB dot instructions per weight chunk and become the
+// bound.  Here the batch rides on the matrix cores instead: one workgroup owns 16 weight rows,
+// its four wavefronts split the width, and each k step of 64 is one
+// v_mfma_i32_16x16x64_i8 with the weights as the 16 x 64 A operand (lane l: row l % 16, bytes
+// [16 (l / 16), +16) of the step, loaded straight from global memory) and, as the 64 x 16 B
+// operand, column b < NB = right-hand vector b (same bytes of the step, loaded from global /
+// L2), column 15 = all ones (its result column is the row sum of the weights), other columns
+// zero.  Bytes are shifted to int8 (XOR 0x80) on the way in:
+//   sum (w - zl)(x - zr) = sum w'x' - zr' sum w' - zl' sum x' + W zl' zr',  z' = z - 128.
+// A k step past the end of the row contributes zeros on the weight side.  The wavefronts'
+// partial 16 x 16 results meet in LDS (integer atomics: the order does not matter).
+typedef int gv4i __attribute__((ext_vector_type(4)));
+
+template <typename OutT>
+__global__ __launch_bounds__(256) void q8_gemv_mfma_kernel(GemvParams p) {
+  constexpr int NBMAX = 15, ONES_COL = 15, STEPS = 16;   // k steps in flight per wavefront
+  __shared__ int32_t s_acc[16][17];
+  __shared__ int32_t s_sx[16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, q = lane >> 4;
+  const int h0 = blockIdx.x * 16;
+  const int b0 = blockIdx.y * NBMAX;
+  const int nb = min(NBMAX, p.batch - b0);
+  const int nchunk = p.W >> 4;
+  const int nstep = (nchunk + 3) >> 2;
+  const int per_wave = (nstep + 3) >> 2;
+  const int ks0 = wave * per_wave, ks1 = min(nstep, ks0 + per_wave);
+
+  for (int i = tid; i < 16 * 17; i += 256) (&s_acc[0][0])[i] = 0;
+  if (tid < 16) s_sx[tid] = 0;
+
+  const uint8_t *arow = p.lhs + (int64_t)min(h0 + r, p.H - 1) * p.W;
+  const uint8_t *xrow = p.rhs + (int64_t)min(b0 + r, p.batch - 1) * p.rhs_bs;
+  const bool is_x = r < nb;
+  const gv4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+  const gv4i zero = {0, 0, 0, 0};
+  const gv4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+  const gv4i other = r == ONES_COL ? ones : zero;
+
+  gv4i acc = zero;
+  int sx = 0;
+  for (int ks = ks0; ks < ks1; ks += STEPS) {
+    gv4i a[STEPS], x[STEPS];
+#pragma unroll
+    for (int u = 0; u < STEPS; ++u) {
+      const int c = min(4 * (ks + u) + q, nchunk - 1);
+      a[u] = __builtin_nontemporal_load((const gv4i *)(arow + (int64_t)c * 16));
+    }
+#pragma unroll
+    for (int u = 0; u < STEPS; ++u) {
+      const int c = min(4 * (ks + u) + q, nchunk - 1);
+      x[u] = flip;
+      if (is_x) x[u] = *(const gv4i *)(xrow + (int64_t)c * 16);
+    }
+#pragma unroll
+    for (int u = 0; u < STEPS; ++u) {
+      const bool valid = (ks + u < ks1) && (4 * (ks + u) + q < nchunk);
+      const gv4i av = valid ? (a[u] ^ flip) : zero;
+      gv4i xv = is_x ? (x[u] ^ flip) : other;
+      if (!valid) xv = zero;
+      if (is_x) {
+        sx = __builtin_amdgcn_sdot4(xv.x, 0x01010101, sx, false);
+        sx = __builtin_amdgcn_sdot4(xv.y, 0x01010101, sx, false);
+        sx = __builtin_amdgcn_sdot4(xv.z, 0x01010101, sx, false);
+        sx = __builtin_amdgcn_sdot4(xv.w, 0x01010101, sx, false);
+      }
+      acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, xv, acc, 0, 0, 0);
+    }
+  }
+  __syncthreads();   // the zeroed LDS is visible
+  // result register i of lane l: row 4 (l / 16) + i, column l % 16
+#pragma unroll
+  for (int i = 0; i < 4; ++i) atomicAdd(&s_acc[4 * q + i][r], acc[i]);
+  if (is_x) atomicAdd(&s_sx[r], sx);
+  __syncthreads();
+
+  if (tid < 16 * nb) {
+    const int row = tid & 15, b = tid >> 4;
+    const int h = h0 + row;
+    if (h < p.H) {
+      const uint32_t zl = (uint32_t)p.lhs_zp - 128u, zr = (uint32_t)p.rhs_zp - 128u;
+      const uint32_t ret = (uint32_t)s_acc[row][b] - zr * (uint32_t)s_acc[row][ONES_COL] -
+                           zl * (uint32_t)s_sx[b] + (uint32_t)p.W * zl * zr +
+                           (p.bias ? (uint32_t)p.bias[h] : 0u);
+      OutT *o = (OutT *)p.out + (int64_t)(b0 + b) * p.H + h;
+      if constexpr (sizeof(OutT) == 4) *o = (OutT)(int32_t)ret;
+      else *o = (OutT)mh_requant_float((int32_t)ret, p.mult, p.out_zp, p.neon_mode);
+    }
+  }
+}
+
+// The same product with the operands staged through LDS.  In the kernel above neighbouring
+// lanes hold neighbouring ROWS (the MFMA operand layout), so every lane's 16 bytes are a
+// memory request of their own.  Here the weights and vectors are moved global -> LDS with
+// global_load_lds_dwordx4 (lane-contiguous: one instruction moves 1 KiB of one row), all
+// transfers of the workgroup issued up front, and the MFMA fragments are read from LDS
+// (row pitch = a multiple of 1 KiB plus 16 bytes: the 16 rows of a fragment read fall into
+// 16 distinct bank groups).  Needs (16 + NB) rows of LDS: the host falls back to the direct
+// kernel when that does not fit.
+template <typename OutT>
+__global__ __launch_bounds__(256) void q8_gemv_mfma_lds_kernel(GemvParams p, int pitch) {
+  constexpr int NBMAX = 15, ONES_COL = 15;
+  extern __shared__ __align__(16) uint8_t lds_rows[];   // [16 + nb][pitch]
+  __shared__ int32_t s_acc[16][17];
+  __shared__ int32_t s_sx[16];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, q = lane >> 4;
+  const int h0 = blockIdx.x * 16;
+  const int b0 = blockIdx.y * NBMAX;
+  const int nb = min(NBMAX, p.batch - b0);
+  const int nchunk = p.W >> 4;
+  const int nj = (nchunk + 63) >> 6;            // 1 KiB transfers per row
+  const int nstep = (nchunk + 3) >> 2;
+  const int per_wave = (nstep + 3) >> 2;
+  const int ks0 = wave * per_wave, ks1 = min(nstep, ks0 + per_wave);
+
+  // rows 4 wave .. 4 wave + 3 of the weights, vectors wave, wave + 4, ...; chunks past the end
+  // of a row re-read its last chunk (never used: masked below)
+  for (int rr = 0; rr < 4; ++rr) {
+    const int row = 4 * wave + rr;
+    const uint8_t *src = p.lhs + (int64_t)min(h0 + row, p.H - 1) * p.W;
+    uint8_t *dst = lds_rows + row * pitch;
+    for (int j = 0; j < nj; ++j)
+      mh_dma_16B_stream(src + (int64_t)min(64 * j + lane, nchunk - 1) * 16, dst + j * 1024);
+  }
+  for (int b = wave; b < nb; b += 4) {
+    const uint8_t *src = p.rhs + (int64_t)(b0 + b) * p.rhs_bs;
+    uint8_t *dst = lds_rows + (16 + b) * pitch;
+    for (int j = 0; j < nj; ++j)
+      mh_dma_16B(src + (int64_t)min(64 * j + lane, nchunk - 1) * 16, dst + j * 1024);
+  }
+  for (int i = tid; i < 16 * 17; i += 256) (&s_acc[0][0])[i] = 0;
+  if (tid < 16) s_sx[tid] = 0;
+  __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0), lgkmcnt(0): own transfers and LDS stores done
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+
+  const bool is_x = r < nb;
+  const gv4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+  const gv4i zero = {0, 0, 0, 0};
+  const gv4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+  const gv4i other = r == ONES_COL ? ones : zero;
+  const uint8_t *arow = lds_rows + r * pitch + q * 16;
+  const uint8_t *xrow = lds_rows + (16 + (is_x ? r : 0)) * pitch + q * 16;
+
+  gv4i acc = zero;
+  int sx = 0;
+#pragma unroll 4
+  for (int ks = ks0; ks < ks1; ++ks) {
+    const bool valid = 4 * ks + q < nchunk;
+    const gv4i av = valid ? (*(const gv4i *)(arow + ks * 64) ^ flip) : zero;
+    gv4i xv = other;
+    if (is_x) xv = *(const gv4i *)(xrow + ks * 64) ^ flip;
+    if (!valid) xv = zero;
+    if (is_x) {
+      sx = __builtin_amdgcn_sdot4(xv.x, 0x01010101, sx, false);
+      sx = __builtin_amdgcn_sdot4(xv.y, 0x01010101, sx, false);
+      sx = __builtin_amdgcn_sdot4(xv.z, 0x01010101, sx, false);
+      sx = __builtin_amdgcn_sdot4(xv.w, 0x01010101, sx, false);
+    }
+    acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, xv, acc, 0, 0, 0);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) atomicAdd(&s_acc[4 * q + i][r], acc[i]);
+  if (is_x) atomicAdd(&s_sx[r], sx);
+  __syncthreads();
+
+  if (tid < 16 * nb) {
+    const int row = tid & 15, b = tid >> 4;
+    const int h = h0 + row;
+    if (h < p.H) {
+      const uint32_t zl = (uint32_t)p.lhs_zp - 128u, zr = (uint32_t)p.rhs_zp - 128u;
+      const uint32_t ret = (uint32_t)s_acc[row][b] - zr * (uint32_t)s_acc[row][ONES_COL] -
+                           zl * (uint32_t)s_sx[b] + (uint32_t)p.W * zl * zr +
+                           (p.bias ? (uint32_t)p.bias[h] : 0u);
+      OutT *o = (OutT *)p.out + (int64_t)(b0 + b) * p.H + h;
+      if constexpr (sizeof(OutT) == 4) *o = (OutT)(int32_t)ret;
+      else *o = (OutT)mh_requant_float((int32_t)ret, p.mult, p.out_zp, p.neon_mode);
+    }
+  }
+}
+
 template <typename OutT>
 int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
   const bool vec = (p.W % 16 == 0) && ((uintptr_t)p.lhs % 16 == 0) &&
@@ -290,6 +475,29 @@ int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
   // a batched lhs gives every batch its own weights: one batch row per pass
   int nb = lhs_batched ? 1 : (p.batch >= 8 ? 8 : (p.batch >= 4 ? 4 : (p.batch >= 2 ? 2 : 1)));
   dim3 block(256);
+  // shared weights against two or more vectors: the batch goes through the matrix cores
+  if (vec && !lhs_batched && p.W >= 64 && p.batch >= 2 && p.rhs_bs % 16 == 0) {
+    dim3 grid((unsigned)((p.H + 15) / 16), (unsigned)((p.batch + 14) / 15));
+    MH_CHECK(ctx, grid.y <= 65535, "batch too large");
+    const int nb_pass = (int)std::min<int64_t>(p.batch, 15);
+    const int pitch = ((p.W / 16 + 63) / 64) * 1024 + 16;
+    const size_t lds = (size_t)(16 + nb_pass) * pitch;
+    const size_t lds_max = (ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536) - 2048;
+    if (lds <= lds_max) {
+      auto k = q8_gemv_mfma_lds_kernel<OutT>;
+      if (lds > 48 * 1024)
+        MH_HIP(ctx, hipFuncSetAttribute((const void *)k,
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      MH_PROF_BEGIN(ctx);
+      hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, pitch);
+    } else {
+      MH_PROF_BEGIN(ctx);
+      hipLaunchKernelGGL(q8_gemv_mfma_kernel<OutT>, grid, block, 0, ctx->stream, p);
+    }
+    MH_PROF_END(ctx);
+    MH_HIP(ctx, hipGetLastError());
+    return MACE_HIP_SUCCESS;
+  }
   // shared weights, aligned rows, right-hand vectors of one pass fit in LDS: row-block kernel
   if (vec && !lhs_batched && p.W >= 16 && (size_t)nb * p.W <= 64 * 1024) {
     constexpr int R = 1, NWAVES = 16;

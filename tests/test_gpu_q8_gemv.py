@@ -36,7 +36,10 @@ CASES = [(1, 16, 4, True, True), (1, 16, 256, True, True), (2, 16, 256, True, Tr
          (2, 16, 256, True, False), (3, 63, 257, True, False),
          (1, 129, 4096, False, True), (8, 70, 4096 + 16, False, True),
          (11, 37, 1040, False, True), (5, 33, 8192, False, True), (4, 5, 30001, False, True),
-         (2, 3, 1, False, True), (3, 7, 48, False, False)]
+         (2, 3, 1, False, True), (3, 7, 48, False, False),
+         # shared weights, batch >= 2: more than 15 vectors (two passes), width tails, shared rhs
+         (16, 50, 272, False, True), (31, 17, 64, False, True), (3, 40, 128, False, False),
+         (15, 16, 80, False, True), (2, 100, 2000, False, True)]
 
 
 @pytest.mark.parametrize("batch,h,w,lb,rb", CASES)
