@@ -318,6 +318,20 @@ def bench_other(ctx, mh, torch):
             tf = flops / (k * 1e-3) / 1e12
             out.append({"workload": "f32_gemm_4x1024^3_ta%d_tb%d" % (ta, tb), "kernel_ms": round(k, 4),
                         "TFLOPS": round(tf, 1), "frac_of_fp32_mfma_peak": round(tf / 157.3, 4)})
+    # the steps either side of a quantized op: Quantize / Dequantize, 64 Mi elements each
+    n = 64 << 20
+    xf = torch.randn((n,), dtype=torch.float32, device="cuda", generator=g)
+    q = torch.empty((n,), dtype=torch.uint8, device="cuda")
+    torch.cuda.synchronize()
+    for (name, nbytes, call) in (
+            ("quantize_u8_64Mi", 5 * n, lambda: ctx.call(
+                "mace_hip_quantize_tensor_u8", xf.data_ptr(), n, 0.03, 128, q.data_ptr())),
+            ("dequantize_u8_64Mi", 5 * n, lambda: ctx.call(
+                "mace_hip_dequantize_tensor_u8", q.data_ptr(), n, 0.03, 128, xf.data_ptr()))):
+        whole, k = time_kernel(ctx, call)
+        gbs = nbytes / (k * 1e-3) / 1e9
+        out.append({"workload": name, "kernel_ms": round(k, 4), "GBps": round(gbs, 1),
+                    "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBS, 4)})
     for o in out:
         log("other:", json.dumps(o))
     return out

@@ -112,6 +112,46 @@ int mace_hip_requant_table_u8(int32_t acc, int32_t multiplier, int right_shift,
 /* The Gemv float requantisation evaluated on the host (see mace_hip_gemv_q8_u8). */
 uint8_t mace_hip_requant_float_u8(int32_t acc, float multiplier, int32_t out_zp, int mode);
 
+/* ---- Quantize / Dequantize -------------------------------------------------------------- */
+
+/* mace/core/quantize.h:28-66 AdjustRange<uint8_t>(in_min, in_max, non_zero, &scale,
+ * &zero_point): the range is widened to contain 0 (and, with non_zero, so that the minimum
+ * quantizes to a value >= 1). */
+void mace_hip_adjust_range_u8(float in_min, float in_max, int non_zero, float *scale,
+                              int32_t *zero_point);
+/* mace/core/quantize.h:91-102 FindMinMax over a device tensor (NaNs are skipped, as std::max /
+ * std::min skip them).  Synchronizes the context's stream: the results are returned by value.
+ * INVALID_ARGS for an empty tensor (the reference CHECK-fails on it, quantize.h:172). */
+int mace_hip_find_min_max_f32(mace_hip_ctx *ctx, const float *input, int64_t size,
+                              float *min_val, float *max_val);
+/* QuantizeUtil<float, uint8_t>::QuantizeWithScaleAndZeropoint (mace/core/quantize.h:138-150),
+ * the branch QuantizeOp takes when the output tensor carries a scale
+ * (mace/ops/arm/q8/quantize.cc:46-52): out[i] = Saturate(roundf(zero_point + (1/scale) x[i])). */
+int mace_hip_quantize_tensor_u8(mace_hip_ctx *ctx, const float *input, int64_t size,
+                                float scale, int32_t zero_point, uint8_t *out);
+/* QuantizeUtil<float, uint8_t>::Quantize (mace/core/quantize.h:152-166), QuantizeOp's other
+ * branch (quantize.cc:53-64): range from the data, AdjustRange, quantize; the scale and zero
+ * point found are returned for the output tensor.  Synchronizes the stream once. */
+int mace_hip_quantize_tensor_dynamic_u8(mace_hip_ctx *ctx, const float *input, int64_t size,
+                                        int non_zero, uint8_t *out, float *scale,
+                                        int32_t *zero_point);
+/* QuantizeUtil<float, Q>::Dequantize (mace/core/quantize.h:188-198), DequantizeOp
+ * (mace/ops/arm/q8/quantize.cc:74-103): out[i] = scale * (q[i] - zero_point). */
+int mace_hip_dequantize_tensor_u8(mace_hip_ctx *ctx, const uint8_t *input, int64_t size,
+                                  float scale, int32_t zero_point, float *out);
+int mace_hip_dequantize_tensor_i32(mace_hip_ctx *ctx, const int32_t *input, int64_t size,
+                                   float scale, int32_t zero_point, float *out);
+/* The same with host pointers (staged through the context arena, synchronous). */
+int mace_hip_quantize_tensor_u8_host(mace_hip_ctx *ctx, const float *input, int64_t size,
+                                     float scale, int32_t zero_point, uint8_t *out);
+int mace_hip_quantize_tensor_dynamic_u8_host(mace_hip_ctx *ctx, const float *input,
+                                             int64_t size, int non_zero, uint8_t *out,
+                                             float *scale, int32_t *zero_point);
+int mace_hip_dequantize_tensor_u8_host(mace_hip_ctx *ctx, const uint8_t *input, int64_t size,
+                                       float scale, int32_t zero_point, float *out);
+int mace_hip_dequantize_tensor_i32_host(mace_hip_ctx *ctx, const int32_t *input, int64_t size,
+                                        float scale, int32_t zero_point, float *out);
+
 /* ---- fp32 ------------------------------------------------------------------------------ */
 
 /* delegator::Gemm::Compute, major form (mace/ops/delegator/gemm.h:42-54; semantics

@@ -567,6 +567,62 @@ class Conv2dK1x1OpQuant {
   int clamp_min_, clamp_max_;
 };
 
+// QuantizeOp<RT_CPU, uint8_t> (mace/ops/arm/q8/quantize.cc:31-72): float -> uint8.  An output
+// tensor that already carries a scale is quantized with it; otherwise (or with
+// find_range_every_time) the range is taken from the data and the scale / zero point found are
+// stored on the output tensor.
+class QuantizeOp {
+ public:
+  explicit QuantizeOp(bool non_zero = false, bool find_range_every_time = false)
+      : non_zero_(non_zero), find_range_every_time_(find_range_every_time) {}
+  MaceStatus Run(OpContext *context, const Tensor *input, Tensor *output) {
+    MaceStatus st = output->Resize(input->shape());   // ResizeLike
+    if (st != MaceStatus::MACE_SUCCESS) return st;
+    if (!find_range_every_time_ && output->scale() > 0.f) {
+      auto fn = output->on_device() ? mace_hip_quantize_tensor_u8 : mace_hip_quantize_tensor_u8_host;
+      return ToStatus(fn(context->hip(), input->data<float>(), input->size(), output->scale(),
+                         output->zero_point(), output->mutable_data<uint8_t>()));
+    }
+    float scale = 0.f;
+    int32_t zero_point = 0;
+    auto fn = output->on_device() ? mace_hip_quantize_tensor_dynamic_u8
+                                  : mace_hip_quantize_tensor_dynamic_u8_host;
+    st = ToStatus(fn(context->hip(), input->data<float>(), input->size(), non_zero_ ? 1 : 0,
+                     output->mutable_data<uint8_t>(), &scale, &zero_point));
+    if (st != MaceStatus::MACE_SUCCESS) return st;
+    output->SetScale(scale);
+    output->SetZeroPoint(zero_point);
+    return st;
+  }
+
+ private:
+  bool non_zero_, find_range_every_time_;
+};
+
+// DequantizeOp<RT_CPU, T> (mace/ops/arm/q8/quantize.cc:74-103), T = uint8_t or int32_t.
+template <typename T>
+class DequantizeOp {
+ public:
+  MaceStatus Run(OpContext *context, const Tensor *input, Tensor *output) {
+    MaceStatus st = output->Resize(input->shape());
+    if (st != MaceStatus::MACE_SUCCESS) return st;
+    return ToStatus(Call(context->hip(), input->data<T>(), input->size(), input->scale(),
+                         input->zero_point(), output->mutable_data<float>(), output->on_device()));
+  }
+
+ private:
+  static int Call(mace_hip_ctx *c, const uint8_t *in, index_t n, float s, int32_t z, float *out,
+                  bool dev) {
+    return dev ? mace_hip_dequantize_tensor_u8(c, in, n, s, z, out)
+               : mace_hip_dequantize_tensor_u8_host(c, in, n, s, z, out);
+  }
+  static int Call(mace_hip_ctx *c, const int32_t *in, index_t n, float s, int32_t z, float *out,
+                  bool dev) {
+    return dev ? mace_hip_dequantize_tensor_i32(c, in, n, s, z, out)
+               : mace_hip_dequantize_tensor_i32_host(c, in, n, s, z, out);
+  }
+};
+
 }  // namespace ops
 }  // namespace mace_hip
 

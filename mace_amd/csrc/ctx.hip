@@ -271,31 +271,6 @@ uint8_t mace_hip_requant_float_u8(int32_t acc, float multiplier, int32_t out_zp,
 
 namespace {
 
-struct Stage {
-  mace_hip_ctx *ctx;
-  ArenaScope scope;
-  explicit Stage(mace_hip_ctx *c) : ctx(c), scope(c) {}
-  // returns nullptr for a null/empty host pointer
-  int in(const void *host, size_t bytes, void **dev) {
-    *dev = nullptr;
-    if (!host || bytes == 0) return MACE_HIP_SUCCESS;
-    *dev = mh_arena_take(ctx, bytes);
-    if (!*dev) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
-    MH_HIP(ctx, hipMemcpyAsync(*dev, host, bytes, hipMemcpyHostToDevice, ctx->stream));
-    return MACE_HIP_SUCCESS;
-  }
-  int out(size_t bytes, void **dev) {
-    *dev = mh_arena_take(ctx, bytes ? bytes : 1);
-    if (!*dev) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
-    return MACE_HIP_SUCCESS;
-  }
-  int back(void *host, const void *dev, size_t bytes) {
-    if (bytes) MH_HIP(ctx, hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
-    MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
-    return MACE_HIP_SUCCESS;
-  }
-};
-
 inline bool nonneg(int64_t a, int64_t b, int64_t c, int64_t d) {
   return a >= 0 && b >= 0 && c >= 0 && d >= 0;
 }

@@ -433,7 +433,6 @@ __global__ __launch_bounds__(256) void q8_gemv_mfma_lds_kernel(GemvParams p, int
 
   gv4i acc = zero;
   int sx = 0;
-#pragma unroll 4
   for (int ks = ks0; ks < ks1; ++ks) {
     const bool valid = 4 * ks + q < nchunk;
     const gv4i av = valid ? (*(const gv4i *)(arow + ks * 64) ^ flip) : zero;

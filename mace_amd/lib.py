@@ -54,6 +54,16 @@ SIGNATURES = {
                                                         C.POINTER(_int)]),
     "mace_hip_quantize_u8": (C.c_uint8, [_f32, _f32, _i32]),
     "mace_hip_requant_fixed_u8": (C.c_uint8, [_i32, _i32, _int, _i32, _int, _int]),
+    "mace_hip_adjust_range_u8": (None, [_f32, _f32, _int, C.POINTER(C.c_float), C.POINTER(C.c_int32)]),
+    "mace_hip_find_min_max_f32": (_int, [_p, _p, _i64, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
+    "mace_hip_quantize_tensor_u8": (_int, [_p, _p, _i64, _f32, _i32, _p]),
+    "mace_hip_quantize_tensor_dynamic_u8": (_int, [_p, _p, _i64, _int, _p, C.POINTER(C.c_float), C.POINTER(C.c_int32)]),
+    "mace_hip_dequantize_tensor_u8": (_int, [_p, _p, _i64, _f32, _i32, _p]),
+    "mace_hip_dequantize_tensor_i32": (_int, [_p, _p, _i64, _f32, _i32, _p]),
+    "mace_hip_quantize_tensor_u8_host": (_int, [_p, _p, _i64, _f32, _i32, _p]),
+    "mace_hip_quantize_tensor_dynamic_u8_host": (_int, [_p, _p, _i64, _int, _p, C.POINTER(C.c_float), C.POINTER(C.c_int32)]),
+    "mace_hip_dequantize_tensor_u8_host": (_int, [_p, _p, _i64, _f32, _i32, _p]),
+    "mace_hip_dequantize_tensor_i32_host": (_int, [_p, _p, _i64, _f32, _i32, _p]),
     "mace_hip_requant_table_u8": (_int, [_i32, _i32, _int, _i32, _int, _int, C.POINTER(C.c_uint8)]),
     "mace_hip_requant_float_u8": (C.c_uint8, [_i32, _f32, _i32, _int]),
     "mace_hip_gemm_f32": (_int, _GEMM_F32),

@@ -9,6 +9,7 @@
 #include "mace_oracle.h"
 
 #include <limits.h>
+#include <float.h>
 #include <math.h>
 #include <stdlib.h>
 #include <string.h>
@@ -121,6 +122,78 @@ int orc_get_bias_data(const int32_t *bias, float bias_scale, float input_scale,
     out[i] = (int32_t)roundf((float)bias[i] * adjust_scale);
   }
   return 1;
+}
+
+/* ------------------------------------------------------------------------------------
+ * Quantize / Dequantize (the ops either side of every quantized op)
+ * ---------------------------------------------------------------------------------- */
+
+/* mace/core/quantize.h:28-66 AdjustRange<uint8_t>: widen [min,max] to contain 0, optionally
+ * nudge so the minimum quantizes to a value >= 1, and place the zero point. */
+void orc_adjust_range_u8(float in_min, float in_max, int non_zero, float *scale,
+                         int32_t *zero_point) {
+  const int qmin = 0, qmax = 255;
+  float out_max = 0.f > in_max ? 0.f : in_max;          /* std::max(0.f, in_max) */
+  float out_min = in_min < 0.f ? in_min : 0.f;          /* std::min(0.f, in_min) */
+  if (non_zero) {
+    const float cand = in_min - (out_max - in_min) / (float)(qmax - qmin - 1);
+    out_min = cand < out_min ? cand : out_min;           /* std::min(out_min, cand) */
+  }
+  *scale = (out_max - out_min) / (float)(qmax - qmin);
+  const float eps = 1e-6f;
+  if (out_min < -eps && out_max > eps) {
+    const float qz = -out_min / *scale;
+    const int32_t near = (int32_t)roundf(qz);
+    *zero_point = near;
+    if (fabsf(qz - (float)near) > eps && non_zero) *zero_point = (int32_t)ceilf(qz);
+  } else if (out_min > -eps) {
+    *zero_point = qmin;
+  } else {
+    *zero_point = qmax;
+  }
+}
+
+/* mace/core/quantize.h:91-102 FindMinMax: std::max / std::min keep the running value when the
+ * comparison is false, so NaNs are skipped. */
+void orc_find_min_max(const float *input, int64_t size, float *min_val, float *max_val) {
+  float max_v = -FLT_MAX, min_v = FLT_MAX;
+  for (int64_t i = 0; i < size; ++i) {
+    max_v = max_v < input[i] ? input[i] : max_v;
+    min_v = input[i] < min_v ? input[i] : min_v;
+  }
+  *min_val = min_v;
+  *max_val = max_v;
+}
+
+/* mace/core/quantize.h:138-150 QuantizeWithScaleAndZeropoint (the generic template: what an x86
+ * build runs): Saturate(roundf(zero_point + (1 / scale) * x)), every operation in binary32. */
+void orc_quantize_with_scale_u8(const float *input, int64_t size, float scale,
+                                int32_t zero_point, uint8_t *out) {
+  const float recip = 1 / scale;
+  for (int64_t i = 0; i < size; ++i) {
+    volatile float prod = recip * input[i];
+    out[i] = orc_saturate_u8(roundf((float)zero_point + prod));
+  }
+}
+
+/* mace/core/quantize.h:152-166 Quantize with the range found from the data */
+void orc_quantize_dynamic_u8(const float *input, int64_t size, int non_zero, uint8_t *out,
+                             float *scale, int32_t *zero_point) {
+  float mn, mx;
+  orc_find_min_max(input, size, &mn, &mx);
+  orc_adjust_range_u8(mn, mx, non_zero, scale, zero_point);
+  orc_quantize_with_scale_u8(input, size, *scale, *zero_point, out);
+}
+
+/* mace/core/quantize.h:188-198 Dequantize: scale * (q - zero_point), the difference in int32 */
+void orc_dequantize_u8(const uint8_t *input, int64_t size, float scale, int32_t zero_point,
+                       float *out) {
+  for (int64_t i = 0; i < size; ++i) out[i] = scale * (float)((int32_t)input[i] - zero_point);
+}
+void orc_dequantize_i32(const int32_t *input, int64_t size, float scale, int32_t zero_point,
+                        float *out) {
+  for (int64_t i = 0; i < size; ++i)
+    out[i] = scale * (float)(int32_t)((uint32_t)input[i] - (uint32_t)zero_point);
 }
 
 /* ------------------------------------------------------------------------------------

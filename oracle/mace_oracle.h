@@ -54,6 +54,19 @@ uint8_t orc_requant_fixed_u8(int32_t acc, int32_t mult, int right_shift,
 int orc_get_bias_data(const int32_t *bias, float bias_scale, float input_scale,
                       float filter_scale, int64_t channels, int32_t *out);
 
+/* ---- Quantize / Dequantize ---------------------------------------------------------- */
+void orc_adjust_range_u8(float in_min, float in_max, int non_zero, float *scale,
+                         int32_t *zero_point);
+void orc_find_min_max(const float *input, int64_t size, float *min_val, float *max_val);
+void orc_quantize_with_scale_u8(const float *input, int64_t size, float scale,
+                                int32_t zero_point, uint8_t *out);
+void orc_quantize_dynamic_u8(const float *input, int64_t size, int non_zero, uint8_t *out,
+                             float *scale, int32_t *zero_point);
+void orc_dequantize_u8(const uint8_t *input, int64_t size, float scale, int32_t zero_point,
+                       float *out);
+void orc_dequantize_i32(const int32_t *input, int64_t size, float scale, int32_t zero_point,
+                        float *out);
+
 /* ---- fp32 ------------------------------------------------------------------------ */
 void orc_gemm_f32(const float *lhs, const float *rhs, int64_t batch, int64_t rows,
                   int64_t cols, int64_t depth, int lhs_major, int rhs_major,

@@ -55,6 +55,18 @@ def lib():
         L.orc_rdivpot.argtypes = [_i32, _int]
         L.orc_requant_fixed_u8.restype = C.c_uint8
         L.orc_requant_fixed_u8.argtypes = [_i32, _i32, _int, _i32, _int, _int]
+        L.orc_adjust_range_u8.restype = None
+        L.orc_adjust_range_u8.argtypes = [_f32, _f32, _int, _p, _p]
+        L.orc_find_min_max.restype = None
+        L.orc_find_min_max.argtypes = [_p, _i64, _p, _p]
+        L.orc_quantize_with_scale_u8.restype = None
+        L.orc_quantize_with_scale_u8.argtypes = [_p, _i64, _f32, _i32, _p]
+        L.orc_quantize_dynamic_u8.restype = None
+        L.orc_quantize_dynamic_u8.argtypes = [_p, _i64, _int, _p, _p, _p]
+        L.orc_dequantize_u8.restype = None
+        L.orc_dequantize_u8.argtypes = [_p, _i64, _f32, _i32, _p]
+        L.orc_dequantize_i32.restype = None
+        L.orc_dequantize_i32.argtypes = [_p, _i64, _f32, _i32, _p]
         L.orc_get_bias_data.restype = _int
         L.orc_get_bias_data.argtypes = [_p, _f32, _f32, _f32, _i64, _p]
         gemm_f32 = [_p, _p, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _int, _p, _int]
@@ -154,6 +166,52 @@ def rdivpot(x, e):
 def requant_fixed_u8(acc, mult, shift, zp, clamp_min=0, clamp_max=255):
     return int(lib().orc_requant_fixed_u8(int(acc), int(mult), int(shift), int(zp),
                                           int(clamp_min), int(clamp_max)))
+
+
+def adjust_range_u8(in_min, in_max, non_zero=False):
+    """(scale, zero_point) of mace/core/quantize.h:28-66 AdjustRange<uint8_t>."""
+    scale, zp = C.c_float(), C.c_int32()
+    lib().orc_adjust_range_u8(np.float32(in_min), np.float32(in_max), int(bool(non_zero)),
+                              C.byref(scale), C.byref(zp))
+    return np.float32(scale.value), int(zp.value)
+
+
+def find_min_max(x):
+    x = _c(x, np.float32)
+    mn, mx = C.c_float(), C.c_float()
+    lib().orc_find_min_max(_ptr(x), x.size, C.byref(mn), C.byref(mx))
+    return np.float32(mn.value), np.float32(mx.value)
+
+
+def quantize_with_scale_u8(x, scale, zero_point):
+    x = _c(x, np.float32)
+    out = np.empty(x.size, dtype=np.uint8)
+    lib().orc_quantize_with_scale_u8(_ptr(x), x.size, np.float32(scale), int(zero_point), _ptr(out))
+    return out
+
+
+def quantize_dynamic_u8(x, non_zero=False):
+    """(quantized, scale, zero_point): the Quantize op when the output carries no scale."""
+    x = _c(x, np.float32)
+    out = np.empty(x.size, dtype=np.uint8)
+    scale, zp = C.c_float(), C.c_int32()
+    lib().orc_quantize_dynamic_u8(_ptr(x), x.size, int(bool(non_zero)), _ptr(out),
+                                  C.byref(scale), C.byref(zp))
+    return out, np.float32(scale.value), int(zp.value)
+
+
+def dequantize_u8(q, scale, zero_point):
+    q = _c(q, np.uint8)
+    out = np.empty(q.size, dtype=np.float32)
+    lib().orc_dequantize_u8(_ptr(q), q.size, np.float32(scale), int(zero_point), _ptr(out))
+    return out
+
+
+def dequantize_i32(q, scale, zero_point):
+    q = _c(q, np.int32)
+    out = np.empty(q.size, dtype=np.float32)
+    lib().orc_dequantize_i32(_ptr(q), q.size, np.float32(scale), int(zero_point), _ptr(out))
+    return out
 
 
 def get_bias_data(bias, bias_scale, input_scale, filter_scale, channels):

@@ -174,6 +174,35 @@ static int test_compute() {
                    ORC_REQUANT_NEON, wanty.data(), 4);
     EXPECT(y == wanty);
   }
+  {
+    // Quantize -> Dequantize as in the reference's test (quantize_test.cc:24-76): round trip
+    // within 0.1, every quantized value > 0 when non_zero is set; bit-exact against the oracle
+    const std::vector<std::vector<float>> inputs = {
+        {-2, -1, 0, 1, 2, 3, 4}, {0, 1, 2, 3, 4}, {2, 3, 4, 5, 6}, {2, 4, 6, 8}, {-2, -4, -6, -8}};
+    for (const auto &in : inputs)
+      for (int non_zero = 0; non_zero < 2; ++non_zero) {
+        const index_t n = (index_t)in.size();
+        std::vector<float> x = in, back(n), wantback(n);
+        std::vector<uint8_t> q(n), wantq(n);
+        Tensor X(x.data(), DT_FLOAT, {n}), Q(q.data(), DT_UINT8, {}), Y(back.data(), DT_FLOAT, {});
+        ops::QuantizeOp quantize(non_zero != 0);
+        EXPECT(quantize.Run(&context, &X, &Q) == MaceStatus::MACE_SUCCESS);
+        float ws; int32_t wz;
+        orc_quantize_dynamic_u8(x.data(), n, non_zero, wantq.data(), &ws, &wz);
+        EXPECT(q == wantq && Q.scale() == ws && Q.zero_point() == wz);
+        if (non_zero) for (auto v : q) EXPECT(v > 0);
+        ops::DequantizeOp<uint8_t> dequantize;
+        EXPECT(dequantize.Run(&context, &Q, &Y) == MaceStatus::MACE_SUCCESS);
+        orc_dequantize_u8(q.data(), n, ws, wz, wantback.data());
+        EXPECT(back == wantback && Y.shape() == X.shape());
+        for (index_t i = 0; i < n; ++i) EXPECT(std::fabs(back[i] - x[i]) <= 0.1f);
+        // an output that already carries a scale is quantized with it
+        Tensor Q2(q.data(), DT_UINT8, {}, 0.05f, 100);
+        EXPECT(quantize.Run(&context, &X, &Q2) == MaceStatus::MACE_SUCCESS);
+        orc_quantize_with_scale_u8(x.data(), n, 0.05f, 100, wantq.data());
+        EXPECT(q == wantq && Q2.scale() == 0.05f && Q2.zero_point() == 100);
+      }
+  }
   mace_hip_ctx_destroy(hctx);
   return g_fail;
 }

@@ -146,3 +146,18 @@ def test_context_needs_a_gpu_or_fails_cleanly():
         assert e.status in (mh.RUNTIME_ERROR, mh.UNSUPPORTED)
     else:
         raise AssertionError("context creation must fail without a GPU")
+
+
+def test_adjust_range_matches_oracle():
+    import ctypes as C
+    lib = mh.load()
+    rng = np.random.default_rng(11)
+    s, z = C.c_float(), C.c_int32()
+    cases = [(-2, 4), (0, 4), (2, 6), (-8, -2), (0, 0), (-1e-7, 1e-7), (-3, 0), (1e-8, 5)]
+    cases += [tuple(np.sort(rng.normal(0, 10, 2))) for _ in range(2000)]
+    cases += [tuple(np.sort(np.abs(rng.normal(0, 10, 2)))) for _ in range(300)]
+    for (a, b) in cases:
+        for nz in (0, 1):
+            lib.mace_hip_adjust_range_u8(np.float32(a), np.float32(b), nz, C.byref(s), C.byref(z))
+            want = orc.adjust_range_u8(a, b, bool(nz))
+            assert (np.float32(s.value), z.value) == want, (a, b, nz)
