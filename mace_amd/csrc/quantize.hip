@@ -10,7 +10,7 @@
 // those of the reference's generic (non-NEON) code bit for bit.
 //
 // All three are bound by HBM bandwidth: 5 bytes per element (quantize, dequantize) or 4
-// (range).  Each lane moves 16 elements per step with 16-byte accesses.
+// (range).  Every access of a wavefront is one contiguous piece of memory (see the kernels).
 #include <float.h>
 
 #include <algorithm>
@@ -28,47 +28,57 @@ __device__ inline uint32_t quantize_one(float x, float recip, float zp) {
   return (uint32_t)mh_saturate_u8(mh_roundf(v));
 }
 
-// VEC: both pointers 16-byte aligned; the last, partial group of 16 is done element by element
+// A wavefront covers 1024 consecutive elements per step as four runs of 256: in run j lane l owns
+// elements 256 j + 4 l .. + 3, so every access of the wavefront is one contiguous piece of memory
+// (1 KiB of floats, 256 bytes of uint8).  VEC: both pointers 16-byte aligned; the last, partial
+// block of 1024 is done element by element.
 template <bool VEC>
 __global__ __launch_bounds__(256) void quantize_u8_kernel(const float *in, int64_t size,
                                                          float recip, float zp, uint8_t *out) {
-  const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;   // group of 16 elements
-  const int64_t base = g * 16;
-  if (base >= size) return;
-  if (VEC && base + 16 <= size) {
-    u4 packed;
+  const int lane = threadIdx.x & 63;
+  const int64_t wbase = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 1024;
+  if (wbase >= size) return;
+  if (VEC && wbase + 1024 <= size) {
+    f4 x[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      x[j] = __builtin_nontemporal_load((const f4 *)(in + wbase + 256 * j) + lane);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const f4 x = __builtin_nontemporal_load((const f4 *)(in + base) + j);
-      packed[j] = quantize_one(x.x, recip, zp) | (quantize_one(x.y, recip, zp) << 8) |
-                  (quantize_one(x.z, recip, zp) << 16) | (quantize_one(x.w, recip, zp) << 24);
+      const uint32_t packed =
+          quantize_one(x[j].x, recip, zp) | (quantize_one(x[j].y, recip, zp) << 8) |
+          (quantize_one(x[j].z, recip, zp) << 16) | (quantize_one(x[j].w, recip, zp) << 24);
+      *((uint32_t *)(out + wbase + 256 * j) + lane) = packed;
     }
-    *(u4 *)(out + base) = packed;
   } else {
-    const int64_t end = base + 16 < size ? base + 16 : size;
-    for (int64_t i = base; i < end; ++i) out[i] = (uint8_t)quantize_one(in[i], recip, zp);
+    const int64_t end = wbase + 1024 < size ? wbase + 1024 : size;
+    for (int64_t i = wbase + lane; i < end; i += 64) out[i] = (uint8_t)quantize_one(in[i], recip, zp);
   }
 }
 
 template <bool VEC>
 __global__ __launch_bounds__(256) void dequantize_u8_kernel(const uint8_t *in, int64_t size,
                                                            float scale, int32_t zp, float *out) {
-  const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int64_t base = g * 16;
-  if (base >= size) return;
-  if (VEC && base + 16 <= size) {
-    const u4 q = __builtin_nontemporal_load((const u4 *)(in + base));
+  const int lane = threadIdx.x & 63;
+  const int64_t wbase = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 1024;
+  if (wbase >= size) return;
+  if (VEC && wbase + 1024 <= size) {
+    uint32_t q[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      q[j] = __builtin_nontemporal_load((const uint32_t *)(in + wbase + 256 * j) + lane);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       f4 v;
 #pragma unroll
       for (int e = 0; e < 4; ++e)
         v[e] = __fmul_rn(scale, (float)((int32_t)((q[j] >> (8 * e)) & 0xff) - zp));
-      *((f4 *)(out + base) + j) = v;
+      *((f4 *)(out + wbase + 256 * j) + lane) = v;
     }
   } else {
-    const int64_t end = base + 16 < size ? base + 16 : size;
-    for (int64_t i = base; i < end; ++i) out[i] = __fmul_rn(scale, (float)((int32_t)in[i] - zp));
+    const int64_t end = wbase + 1024 < size ? wbase + 1024 : size;
+    for (int64_t i = wbase + lane; i < end; i += 64)
+      out[i] = __fmul_rn(scale, (float)((int32_t)in[i] - zp));
   }
 }
 
@@ -199,7 +209,7 @@ int mace_hip_quantize_tensor_u8(mace_hip_ctx *ctx, const float *input, int64_t s
   MH_RETURN_IF_ERROR(check_size(ctx, size, input, out));
   if (size == 0) return MACE_HIP_SUCCESS;
   volatile float recip = 1 / scale;
-  const unsigned blocks = (unsigned)((size + 16 * 256 - 1) / (16 * 256));
+  const unsigned blocks = (unsigned)((size + 4095) / 4096);
   MH_PROF_BEGIN(ctx);
   if (aligned16(input, out))
     hipLaunchKernelGGL(quantize_u8_kernel<true>, dim3(blocks), dim3(256), 0, ctx->stream, input,
@@ -259,7 +269,7 @@ int mace_hip_dequantize_tensor_u8(mace_hip_ctx *ctx, const uint8_t *input, int64
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   MH_RETURN_IF_ERROR(check_size(ctx, size, input, out));
   if (size == 0) return MACE_HIP_SUCCESS;
-  const unsigned blocks = (unsigned)((size + 16 * 256 - 1) / (16 * 256));
+  const unsigned blocks = (unsigned)((size + 4095) / 4096);
   MH_PROF_BEGIN(ctx);
   if (aligned16(input, out))
     hipLaunchKernelGGL(dequantize_u8_kernel<true>, dim3(blocks), dim3(256), 0, ctx->stream,
