@@ -801,6 +801,68 @@ __global__ __launch_bounds__(256) void q8_pack_transpose_kernel(const uint8_t *s
   }
 }
 
+// The same repack for n % 16 == 0 and a 16-byte aligned source: 128 x 128-byte tiles, whole
+// 128-byte lines on both sides.  A thread loads 16 bytes of one k row (four times) and parks
+// them in LDS as dwords of 4 n each, laid out [n / 4][k]; then it picks up 16 consecutive k of
+// one n group (4 n x 16 k), transposes the four 4 x 4 byte blocks in registers (8 v_perm each)
+// and stores 16 bytes of k for each of its 4 n.  Row pitch 130 dwords: the 8 x 8 (n group, k)
+// pattern of a wavefront's LDS stores falls into 64 distinct banks.
+__device__ inline void transpose4x4_bytes(const uint32_t (&d)[4], uint32_t (&o)[4]) {
+  const uint32_t t0 = __builtin_amdgcn_perm(d[1], d[0], 0x05010400);   // d0.b0 d1.b0 d0.b1 d1.b1
+  const uint32_t t1 = __builtin_amdgcn_perm(d[1], d[0], 0x07030602);   // d0.b2 d1.b2 d0.b3 d1.b3
+  const uint32_t t2 = __builtin_amdgcn_perm(d[3], d[2], 0x05010400);
+  const uint32_t t3 = __builtin_amdgcn_perm(d[3], d[2], 0x07030602);
+  o[0] = __builtin_amdgcn_perm(t2, t0, 0x05040100);
+  o[1] = __builtin_amdgcn_perm(t2, t0, 0x07060302);
+  o[2] = __builtin_amdgcn_perm(t3, t1, 0x05040100);
+  o[3] = __builtin_amdgcn_perm(t3, t1, 0x07060302);
+}
+
+__global__ __launch_bounds__(256) void q8_pack_transpose128_kernel(const uint8_t *src,
+                                                                   int64_t src_bs, uint8_t *dst,
+                                                                   int64_t dst_bs, int n, int k,
+                                                                   int kp) {
+  constexpr int PITCH = 130;
+  __shared__ uint32_t tile[32 * PITCH];   // [n / 4][k]
+  const uint8_t *s = src + (int64_t)blockIdx.z * src_bs;
+  uint8_t *d = dst + (int64_t)blockIdx.z * dst_bs;
+  const int n0 = blockIdx.x * 128, k0 = blockIdx.y * 128;
+  const int tid = threadIdx.x;
+  {
+    const int nc = (tid & 7) * 16;   // 16 bytes of n, rows kk = tid / 8 + 32 j
+    const int gn = n0 + nc;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int kk = (tid >> 3) + 32 * j;
+      const int gk = k0 + kk;
+      uint4 v = {0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u};
+      if (gk < k && gn < n) v = *(const uint4 *)(s + (int64_t)gk * n + gn);   // n % 16 == 0
+      uint32_t *t = tile + (nc >> 2) * PITCH + kk;
+      t[0] = v.x; t[PITCH] = v.y; t[2 * PITCH] = v.z; t[3 * PITCH] = v.w;
+    }
+  }
+  __syncthreads();
+  {
+    const int kc = tid & 7, g = tid >> 3;   // 16 k starting at 16 kc, n = 4 g .. 4 g + 3
+    const uint32_t *t = tile + g * PITCH + 16 * kc;
+    uint32_t o[4][4];                       // [k block][n]
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const uint32_t din[4] = {t[4 * b], t[4 * b + 1], t[4 * b + 2], t[4 * b + 3]};
+      transpose4x4_bytes(din, o[b]);
+    }
+    const int gk = k0 + 16 * kc;
+    if (gk < kp) {   // kp is a multiple of 64: a 16-byte piece is inside the row or outside
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int gn = n0 + 4 * g + j;
+        if (gn < n)
+          *(uint4 *)(d + (int64_t)gn * kp + gk) = uint4{o[0][j], o[1][j], o[2][j], o[3][j]};
+      }
+    }
+  }
+}
+
 // ---- correction vectors --------------------------------------------------------------------
 
 // corr[b][n] = coef * sum_k (P[b][n][k] - 128) + add + (bias ? bias[n] : 0), modulo 2^32.
@@ -1010,10 +1072,16 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
                          n * depth, dst, n * kp, (int)n, (int)depth, (int)kp);
     } else {
       MH_CHECK(ctx, (kp / 64) <= 65535, "depth too large to repack");
-      dim3 grid((unsigned)((n + 63) / 64), (unsigned)(kp / 64), nb);
       const int vec_ok = (n % 16 == 0) && ((uintptr_t)src % 16 == 0);
-      hipLaunchKernelGGL(q8_pack_transpose_kernel, grid, dim3(256), 0, ctx->stream, src,
-                         n * depth, dst, n * kp, (int)n, (int)depth, (int)kp, vec_ok);
+      if (vec_ok) {
+        dim3 grid((unsigned)((n + 127) / 128), (unsigned)((kp + 127) / 128), nb);
+        hipLaunchKernelGGL(q8_pack_transpose128_kernel, grid, dim3(256), 0, ctx->stream, src,
+                           n * depth, dst, n * kp, (int)n, (int)depth, (int)kp);
+      } else {
+        dim3 grid((unsigned)((n + 63) / 64), (unsigned)(kp / 64), nb);
+        hipLaunchKernelGGL(q8_pack_transpose_kernel, grid, dim3(256), 0, ctx->stream, src,
+                           n * depth, dst, n * kp, (int)n, (int)depth, (int)kp, 0);
+      }
     }
     MH_HIP(ctx, hipGetLastError());
     *P = Panel{dst, kp, nb > 1 ? n * kp : 0, (int)kp};
