@@ -231,6 +231,32 @@ int mace_hip_conv1x1_q8_nhwc(mace_hip_ctx *ctx, const uint8_t *input, const uint
                              int32_t input_zp, float filter_scale, int32_t filter_zp,
                              float bias_scale, float out_scale, int32_t out_zp,
                              int clamp_min, int clamp_max, uint8_t *out);
+/* Conv2dOp<RT_CPU, uint8_t>::Run for any filter size and stride, dilation 1
+ * (mace/ops/conv_2d.cc:201-318): input NHWC [n][in_h][in_w][cin], filter OHWI
+ * [cout][k_h][k_w][cin], output NHWC [n][out_h][out_w][cout] with the output size given by the
+ * FLOOR rule out = floor((in + pad - k) / stride) + 1 (conv_pool_2d_util.cc:194-200; it agrees
+ * with mace_hip_calc_padding_and_output_size for VALID / SAME / FULL).  pad_h / pad_w are the
+ * TOTAL paddings per dimension as MACE passes them: pad >> 1 rows / columns go on the top / left
+ * (conv_2d.cc:345-348), the rest on the bottom / right; padded positions hold the input zero
+ * point (Im2col, conv_2d.cc:321-412).  A 1x1 filter at stride 1 without padding multiplies the
+ * input in place; everything else is gathered into an im2col matrix in the context arena first.
+ * INVALID_ARGS where the reference CHECK-fails (multiplier outside (0,1)) and for a filter larger
+ * than the padded input. */
+int mace_hip_conv2d_q8_nhwc(mace_hip_ctx *ctx, const uint8_t *input, const uint8_t *filter,
+                            const int32_t *bias /* or NULL */, int64_t n, int64_t in_h,
+                            int64_t in_w, int64_t cin, int64_t cout, int64_t k_h, int64_t k_w,
+                            int stride_h, int stride_w, int pad_h, int pad_w, float input_scale,
+                            int32_t input_zp, float filter_scale, int32_t filter_zp,
+                            float bias_scale, float out_scale, int32_t out_zp, int clamp_min,
+                            int clamp_max, uint8_t *out);
+/* CalcPaddingAndOutputSize, spatial part (mace/ops/common/conv_pool_2d_util.cc:30-120):
+ * padding 0 = VALID, 1 = SAME, 2 = FULL (mace::Padding); pad_h / pad_w are totals.
+ * INVALID_ARGS where the reference CHECK-fails (strides / dilations <= 0, dilation with stride,
+ * unknown padding type). */
+int mace_hip_calc_padding_and_output_size(int64_t in_h, int64_t in_w, int64_t k_h, int64_t k_w,
+                                          int dilation_h, int dilation_w, int stride_h,
+                                          int stride_w, int padding, int64_t *out_h,
+                                          int64_t *out_w, int *pad_h, int *pad_w);
 
 /* ---- host-pointer variants (same contracts; synchronous) -------------------------------- */
 int mace_hip_gemm_f32_host(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
@@ -273,6 +299,13 @@ int mace_hip_conv1x1_q8_nhwc_host(mace_hip_ctx *ctx, const uint8_t *input,
                                   int32_t filter_zp, float bias_scale, float out_scale,
                                   int32_t out_zp, int clamp_min, int clamp_max,
                                   uint8_t *out);
+int mace_hip_conv2d_q8_nhwc_host(mace_hip_ctx *ctx, const uint8_t *input, const uint8_t *filter,
+                                 const int32_t *bias, int64_t n, int64_t in_h, int64_t in_w,
+                                 int64_t cin, int64_t cout, int64_t k_h, int64_t k_w,
+                                 int stride_h, int stride_w, int pad_h, int pad_w,
+                                 float input_scale, int32_t input_zp, float filter_scale,
+                                 int32_t filter_zp, float bias_scale, float out_scale,
+                                 int32_t out_zp, int clamp_min, int clamp_max, uint8_t *out);
 
 #ifdef __cplusplus
 }

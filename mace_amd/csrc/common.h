@@ -321,7 +321,9 @@ struct Q8GemmEpilogue {
 int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8_t *rhs,
                int rhs_order, void *out, int out_order, bool out_u8, int64_t batch,
                int64_t rows, int64_t depth, int64_t cols, int lhs_batched, int rhs_batched,
-               int32_t lhs_offset, int32_t rhs_offset, const Q8GemmEpilogue &ep);
+               int32_t lhs_offset, int32_t rhs_offset, const Q8GemmEpilogue &ep,
+               int64_t rhs_ld = 0);   // rhs_ld != 0: ColMajor rhs whose columns are rhs_ld bytes
+                                      // apart (multiple of 16), bytes depth..rhs_ld-1 being 0x80
 
 struct F32Epilogue {
   const float *bias_row;    // added per result row (NCHW channel), or nullptr

@@ -483,4 +483,41 @@ int mace_hip_conv1x1_q8_nhwc_host(mace_hip_ctx *ctx, const uint8_t *input,
   return st.back(out, dout, ob);
 }
 
+int mace_hip_conv2d_q8_nhwc_host(mace_hip_ctx *ctx, const uint8_t *input, const uint8_t *filter,
+                                 const int32_t *bias, int64_t n, int64_t in_h, int64_t in_w,
+                                 int64_t cin, int64_t cout, int64_t k_h, int64_t k_w,
+                                 int stride_h, int stride_w, int pad_h, int pad_w,
+                                 float input_scale, int32_t input_zp, float filter_scale,
+                                 int32_t filter_zp, float bias_scale, float out_scale,
+                                 int32_t out_zp, int clamp_min, int clamp_max, uint8_t *out) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_CHECK(ctx, nonneg(n, in_h, in_w, 0) && nonneg(cin, cout, 0, 0), "negative dimension");
+  MH_CHECK(ctx, k_h >= 1 && k_w >= 1 && stride_h >= 1 && stride_w >= 1 && pad_h >= 0 &&
+                    pad_w >= 0, "filter / stride < 1 or negative padding");
+  const int64_t num_h = in_h + pad_h - k_h, num_w = in_w + pad_w - k_w;
+  MH_CHECK(ctx, num_h >= -stride_h && num_w >= -stride_w, "filter larger than the padded input");
+  const int64_t out_h = (num_h >= 0 ? num_h / stride_h : -1) + 1;
+  const int64_t out_w = (num_w >= 0 ? num_w / stride_w : -1) + 1;
+  const int64_t columns = n * out_h * out_w, depth = k_h * k_w * cin;
+  const size_t ib = (size_t)n * in_h * in_w * cin, fb = (size_t)cout * depth;
+  const size_t bb = bias ? sizeof(int32_t) * cout : 0;
+  const size_t ob = (size_t)columns * cout;
+  // staged tensors + the im2col matrix + what the GEMM takes for itself
+  MH_RETURN_IF_ERROR(mh_arena_reserve(
+      ctx, ib + fb + bb + ob + (size_t)columns * (mh_align_up((size_t)depth + 1, 64) + 8) +
+               q8_gemm_scratch(1, cout, depth, 0) + sizeof(int32_t) * (4 * cout + columns) +
+               (1 << 17)));
+  Stage st(ctx);
+  void *di, *df, *db, *dout;
+  MH_RETURN_IF_ERROR(st.in(input, ib, &di));
+  MH_RETURN_IF_ERROR(st.in(filter, fb, &df));
+  MH_RETURN_IF_ERROR(st.in(bias, bb, &db));
+  MH_RETURN_IF_ERROR(st.out(ob, &dout));
+  MH_RETURN_IF_ERROR(mace_hip_conv2d_q8_nhwc(
+      ctx, (const uint8_t *)di, (const uint8_t *)df, (const int32_t *)db, n, in_h, in_w, cin,
+      cout, k_h, k_w, stride_h, stride_w, pad_h, pad_w, input_scale, input_zp, filter_scale,
+      filter_zp, bias_scale, out_scale, out_zp, clamp_min, clamp_max, (uint8_t *)dout));
+  return st.back(out, dout, ob);
+}
+
 }  // extern "C"

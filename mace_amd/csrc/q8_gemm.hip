@@ -1016,7 +1016,8 @@ int launch_gemm_stream(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab
 int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8_t *rhs,
                int rhs_order, void *out, int out_order, bool out_u8, int64_t batch,
                int64_t rows, int64_t depth, int64_t cols, int lhs_batched, int rhs_batched,
-               int32_t lhs_offset, int32_t rhs_offset, const Q8GemmEpilogue &ep) {
+               int32_t lhs_offset, int32_t rhs_offset, const Q8GemmEpilogue &ep,
+               int64_t rhs_ld) {
   MH_CHECK(ctx, batch >= 0 && rows >= 0 && depth >= 0 && cols >= 0, "negative dimension");
   MH_CHECK(ctx, (lhs_order | 1) == 1 && (rhs_order | 1) == 1 && (out_order | 1) == 1,
            "matrix order must be RowMajor (0) or ColMajor (1)");
@@ -1040,8 +1041,11 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   // which operands can be read in place
   const bool lhs_direct = lhs_order == MACE_HIP_ROW_MAJOR && depth % 16 == 0 && depth > 0 &&
                           ((uintptr_t)lhs % 16 == 0);
-  const bool rhs_direct = rhs_order == MACE_HIP_COL_MAJOR && depth % 16 == 0 && depth > 0 &&
-                          ((uintptr_t)rhs % 16 == 0);
+  MH_CHECK(ctx, rhs_ld == 0 || (rhs_order == MACE_HIP_COL_MAJOR && rhs_ld >= depth &&
+                               rhs_ld % 16 == 0 && depth > 0 && ((uintptr_t)rhs % 16 == 0)),
+           "padded right-hand panel must be ColMajor, 16-byte aligned, pitch a multiple of 16");
+  const bool rhs_direct = rhs_ld != 0 || (rhs_order == MACE_HIP_COL_MAJOR && depth % 16 == 0 &&
+                                          depth > 0 && ((uintptr_t)rhs % 16 == 0));
 
   size_t need = sizeof(int32_t) * ((size_t)lhs_nb * rows + (size_t)rhs_nb * cols) + 4096;
   if (!lhs_direct) need += (size_t)lhs_nb * rows * kp + 256;
@@ -1056,9 +1060,10 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   } L, R;
 
   auto prepare = [&](const uint8_t *src, int order_is_kcontig, bool direct, int nb, int64_t n,
-                     Panel *P) -> int {
+                     int64_t ld, Panel *P) -> int {
     if (direct) {
-      *P = Panel{src, depth, nb > 1 ? n * depth : 0, (int)depth};
+      // a caller-padded panel (ld > depth) is readable, and zero after the shift, up to ld
+      *P = Panel{src, ld, nb > 1 ? n * ld : 0, (int)ld};
       return MACE_HIP_SUCCESS;
     }
     uint8_t *dst = (uint8_t *)mh_arena_take(ctx, (size_t)nb * n * kp);
@@ -1087,8 +1092,9 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     *P = Panel{dst, kp, nb > 1 ? n * kp : 0, (int)kp};
     return MACE_HIP_SUCCESS;
   };
-  MH_RETURN_IF_ERROR(prepare(lhs, lhs_order == MACE_HIP_ROW_MAJOR, lhs_direct, lhs_nb, rows, &L));
-  MH_RETURN_IF_ERROR(prepare(rhs, rhs_order == MACE_HIP_COL_MAJOR, rhs_direct, rhs_nb, cols, &R));
+  MH_RETURN_IF_ERROR(prepare(lhs, lhs_order == MACE_HIP_ROW_MAJOR, lhs_direct, lhs_nb, rows, depth, &L));
+  MH_RETURN_IF_ERROR(prepare(rhs, rhs_order == MACE_HIP_COL_MAJOR, rhs_direct, rhs_nb, cols,
+                             rhs_ld != 0 ? rhs_ld : depth, &R));
 
   // correction vectors.  zl' = -lhs_offset - 128, zr' = -rhs_offset - 128.
   //   corrL[i] = -zr' * sum_k l'[i,k] + bias[i];   corrR[j] = -zl' * sum_k r'[k,j] + K zl' zr'

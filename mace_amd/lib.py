@@ -29,6 +29,8 @@ _GEMV_Q8_I32 = [_p, _p, _p, _p, _i64, _i64, _i64, _int, _int, _i32, _i32, _p]
 _GEMM_Q8_I32 = [_p, _p, _int, _p, _int, _p, _int, _i64, _i64, _i64, _i64, _int, _int, _i32,
                 _i32]
 _GEMM_Q8_U8 = _GEMM_Q8_I32 + [_p, _i32, _int, _i32, _int, _int]
+_CONV2D_Q8 = [_p, _p, _p, _p] + [_i64] * 7 + [_int] * 4 + [_f32, _i32, _f32, _i32, _f32, _f32, _i32,
+                                                         _int, _int, _p]
 _CONV_Q8 = [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _f32, _i32, _f32, _i32, _f32, _f32,
             _i32, _int, _int, _p]
 
@@ -84,6 +86,12 @@ SIGNATURES = {
     "mace_hip_gemm_q8_i32_host": (_int, _GEMM_Q8_I32),
     "mace_hip_gemm_q8_u8_host": (_int, _GEMM_Q8_U8),
     "mace_hip_conv1x1_q8_nhwc_host": (_int, _CONV_Q8),
+    "mace_hip_conv2d_q8_nhwc": (_int, _CONV2D_Q8),
+    "mace_hip_conv2d_q8_nhwc_host": (_int, _CONV2D_Q8),
+    "mace_hip_calc_padding_and_output_size": (_int, [_i64, _i64, _i64, _i64, _int, _int, _int, _int,
+                                                     _int, C.POINTER(C.c_int64),
+                                                     C.POINTER(C.c_int64), C.POINTER(_int),
+                                                     C.POINTER(_int)]),
 }
 
 

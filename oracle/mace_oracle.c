@@ -530,3 +530,134 @@ void orc_conv1x1_f32_nchw(const float *input, const float *filter, const float *
   if (bias) orc_bias_add_nchw_f32(out, bias, n, cout, hw);
   orc_activation_f32(out, n * cout * hw, act, limit);
 }
+
+/* ------------------------------------------------------------------------------------
+ * General quantized Conv2D (im2col + the same GEMM)
+ * ---------------------------------------------------------------------------------- */
+
+/* mace/ops/common/conv_pool_2d_util.cc:30-120 CalcPaddingAndOutputSize, spatial part
+ * (padding: 0 VALID, 1 SAME, 2 FULL as in mace::Padding; paddings are totals per dimension).
+ * Returns 1 where the reference CHECK-fails. */
+int orc_calc_padding_and_output_size(int64_t in_h, int64_t in_w, int64_t k_h, int64_t k_w,
+                                     int dil_h, int dil_w, int stride_h, int stride_w,
+                                     int padding, int64_t *out_h, int64_t *out_w, int *pad_h,
+                                     int *pad_w) {
+  if (dil_h <= 0 || dil_w <= 0 || stride_h <= 0 || stride_w <= 0) return 1;
+  if (!((dil_h == 1 || stride_h == 1) && (dil_w == 1 || stride_w == 1))) return 1;
+  const int64_t ext_h = (k_h - 1) * dil_h + 1, ext_w = (k_w - 1) * dil_w + 1;
+  int64_t oh, ow;
+  switch (padding) {
+    case 0: oh = (in_h - ext_h) / stride_h + 1; ow = (in_w - ext_w) / stride_w + 1; break;
+    case 1: oh = (in_h - 1) / stride_h + 1; ow = (in_w - 1) / stride_w + 1; break;
+    case 2: oh = (in_h + ext_h - 2) / stride_h + 1; ow = (in_w + ext_w - 2) / stride_w + 1; break;
+    default: return 1;
+  }
+  const int64_t ph = (oh - 1) * stride_h + ext_h - in_h, pw = (ow - 1) * stride_w + ext_w - in_w;
+  *pad_h = (int)(ph > 0 ? ph : 0);
+  *pad_w = (int)(pw > 0 ? pw : 0);
+  *out_h = oh;
+  *out_w = ow;
+  return 0;
+}
+
+/* conv_pool_2d_util.cc:146-222 CalcOutputSize with RoundType::FLOOR and dilation 1 (what the
+ * quantized Conv2D uses for explicit paddings, conv_2d.cc:225-234) */
+void orc_calc_output_size_floor(int64_t in_h, int64_t in_w, int64_t k_h, int64_t k_w,
+                                int stride_h, int stride_w, int pad_h, int pad_w,
+                                int64_t *out_h, int64_t *out_w) {
+  *out_h = (int64_t)floor(1.0 * (double)(in_h + pad_h - k_h) / stride_h) + 1;
+  *out_w = (int64_t)floor(1.0 * (double)(in_w + pad_w - k_w) / stride_w) + 1;
+}
+
+/* mace/ops/conv_2d.cc:321-412 Im2col: column (b, h, w) of the [depth x columns] matrix holds
+ * the filter_h x filter_w x cin patch whose top-left input position is
+ * (h*stride_h - pad_h/2, w*stride_w - pad_w/2), in (kh, kw, c) order; positions outside the
+ * input hold the input zero point.  Written here per element; the reference fills the same
+ * bytes with fill_n / copy_n runs. */
+void orc_im2col_u8(const uint8_t *in, int64_t n, int64_t in_h, int64_t in_w, int64_t cin,
+                   int64_t k_h, int64_t k_w, int stride_h, int stride_w, uint8_t zero_point,
+                   int pad_h, int pad_w, int64_t out_h, int64_t out_w, uint8_t *out) {
+  const int64_t depth = k_h * k_w * cin;
+  for (int64_t b = 0; b < n; ++b)
+    for (int64_t h = 0; h < out_h; ++h)
+      for (int64_t w = 0; w < out_w; ++w) {
+        uint8_t *col = out + ((b * out_h + h) * out_w + w) * depth;
+        const int64_t ih0 = h * stride_h - (pad_h >> 1), iw0 = w * stride_w - (pad_w >> 1);
+        for (int64_t kh = 0; kh < k_h; ++kh)
+          for (int64_t kw = 0; kw < k_w; ++kw) {
+            const int64_t ih = ih0 + kh, iw = iw0 + kw;
+            uint8_t *dst = col + (kh * k_w + kw) * cin;
+            if (ih >= 0 && ih < in_h && iw >= 0 && iw < in_w)
+              memcpy(dst, in + ((b * in_h + ih) * in_w + iw) * cin, (size_t)cin);
+            else
+              memset(dst, zero_point, (size_t)cin);
+          }
+      }
+}
+
+/* mace/ops/conv_2d.cc:201-318, any filter / stride (dilation 1): output size by the FLOOR rule
+ * from the total paddings, im2col unless the filter is 1x1 / stride 1, then the GEMM with
+ * lhs = filter RowMajor [cout x depth], rhs = im2col ColMajor, result ColMajor.
+ * Returns 1 where the reference CHECK-fails (multiplier range), 2 for an empty output. */
+int orc_conv2d_q8_nhwc(const uint8_t *input, const uint8_t *filter, const int32_t *bias,
+                       int64_t n, int64_t in_h, int64_t in_w, int64_t cin, int64_t cout,
+                       int64_t k_h, int64_t k_w, int stride_h, int stride_w, int pad_h,
+                       int pad_w, float input_scale, int32_t input_zp, float filter_scale,
+                       int32_t filter_zp, float bias_scale, float out_scale, int32_t out_zp,
+                       int clamp_min, int clamp_max, uint8_t *out, int nthreads) {
+  int32_t mult;
+  int shift;
+  if (orc_get_output_multiplier_and_shift(filter_scale, input_scale, out_scale, &mult, &shift))
+    return 1;
+  int64_t out_h, out_w;
+  orc_calc_output_size_floor(in_h, in_w, k_h, k_w, stride_h, stride_w, pad_h, pad_w, &out_h,
+                             &out_w);
+  if (out_h <= 0 || out_w <= 0 || n <= 0) return 2;
+  const int64_t depth = k_h * k_w * cin, columns = n * out_h * out_w;
+  /* conv_2d.cc:278-279 skips im2col for a 1x1 filter at stride 1 whatever the padding; with
+   * padding the output has more positions than the input and the reference's GEMM then reads
+   * past the input tensor (undefined).  The oracle gathers in that case, which is what the
+   * definition of the convolution gives. */
+  const int need = k_h != 1 || k_w != 1 || stride_h != 1 || stride_w != 1 || pad_h != 0 ||
+                   pad_w != 0;
+  uint8_t *cols = NULL;
+  if (need) {
+    cols = (uint8_t *)malloc((size_t)(depth * columns > 0 ? depth * columns : 1));
+    orc_im2col_u8(input, n, in_h, in_w, cin, k_h, k_w, stride_h, stride_w, (uint8_t)input_zp,
+                  pad_h, pad_w, out_h, out_w, cols);
+  }
+  int32_t *b2 = (int32_t *)malloc((size_t)(cout > 0 ? cout : 1) * sizeof(int32_t));
+  orc_get_bias_data(bias, bias_scale, input_scale, filter_scale, cout, b2);
+  orc_q8_gemm_u8(filter, need ? cols : input, 1, cout, columns, depth, ORC_ROW_MAJOR,
+                 ORC_COL_MAJOR, ORC_COL_MAJOR, 0, 0, -filter_zp, -input_zp, b2, mult, shift,
+                 out_zp, clamp_min, clamp_max, out, nthreads);
+  free(b2);
+  free(cols);
+  return 0;
+}
+
+/* The convolution written as the textbook sum, padding included (a padded position holds the
+ * zero point, i.e. contributes (zp - zp) = 0): pins im2col's layout and padding claims. */
+void orc_conv2d_q8_nhwc_direct_i32(const uint8_t *input, const uint8_t *filter, int64_t n,
+                                   int64_t in_h, int64_t in_w, int64_t cin, int64_t cout,
+                                   int64_t k_h, int64_t k_w, int stride_h, int stride_w,
+                                   int pad_h, int pad_w, int64_t out_h, int64_t out_w,
+                                   int32_t input_zp, int32_t filter_zp, int32_t *out) {
+  for (int64_t b = 0; b < n; ++b)
+    for (int64_t h = 0; h < out_h; ++h)
+      for (int64_t w = 0; w < out_w; ++w)
+        for (int64_t co = 0; co < cout; ++co) {
+          int32_t acc = 0;
+          for (int64_t kh = 0; kh < k_h; ++kh)
+            for (int64_t kw = 0; kw < k_w; ++kw) {
+              const int64_t ih = h * stride_h - (pad_h >> 1) + kh;
+              const int64_t iw = w * stride_w - (pad_w >> 1) + kw;
+              if (ih < 0 || ih >= in_h || iw < 0 || iw >= in_w) continue;
+              const uint8_t *x = input + ((b * in_h + ih) * in_w + iw) * cin;
+              const uint8_t *f = filter + ((co * k_h + kh) * k_w + kw) * cin;
+              for (int64_t c = 0; c < cin; ++c)
+                acc += ((int32_t)f[c] - filter_zp) * ((int32_t)x[c] - input_zp);
+            }
+          out[((b * out_h + h) * out_w + w) * cout + co] = acc;
+        }
+}

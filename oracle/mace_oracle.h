@@ -140,6 +140,29 @@ void orc_conv1x1_q8_nhwc_direct_i32(const uint8_t *input, const uint8_t *filter,
                                     int64_t cout, int32_t input_zp, int32_t filter_zp,
                                     int32_t *out);
 
+/* ---- general quantized Conv2D (im2col) --------------------------------------------- */
+int orc_calc_padding_and_output_size(int64_t in_h, int64_t in_w, int64_t k_h, int64_t k_w,
+                                     int dil_h, int dil_w, int stride_h, int stride_w,
+                                     int padding, int64_t *out_h, int64_t *out_w, int *pad_h,
+                                     int *pad_w);
+void orc_calc_output_size_floor(int64_t in_h, int64_t in_w, int64_t k_h, int64_t k_w,
+                                int stride_h, int stride_w, int pad_h, int pad_w,
+                                int64_t *out_h, int64_t *out_w);
+void orc_im2col_u8(const uint8_t *in, int64_t n, int64_t in_h, int64_t in_w, int64_t cin,
+                   int64_t k_h, int64_t k_w, int stride_h, int stride_w, uint8_t zero_point,
+                   int pad_h, int pad_w, int64_t out_h, int64_t out_w, uint8_t *out);
+int orc_conv2d_q8_nhwc(const uint8_t *input, const uint8_t *filter, const int32_t *bias,
+                       int64_t n, int64_t in_h, int64_t in_w, int64_t cin, int64_t cout,
+                       int64_t k_h, int64_t k_w, int stride_h, int stride_w, int pad_h,
+                       int pad_w, float input_scale, int32_t input_zp, float filter_scale,
+                       int32_t filter_zp, float bias_scale, float out_scale, int32_t out_zp,
+                       int clamp_min, int clamp_max, uint8_t *out, int nthreads);
+void orc_conv2d_q8_nhwc_direct_i32(const uint8_t *input, const uint8_t *filter, int64_t n,
+                                   int64_t in_h, int64_t in_w, int64_t cin, int64_t cout,
+                                   int64_t k_h, int64_t k_w, int stride_h, int stride_w,
+                                   int pad_h, int pad_w, int64_t out_h, int64_t out_w,
+                                   int32_t input_zp, int32_t filter_zp, int32_t *out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -67,6 +67,18 @@ def lib():
         L.orc_dequantize_u8.argtypes = [_p, _i64, _f32, _i32, _p]
         L.orc_dequantize_i32.restype = None
         L.orc_dequantize_i32.argtypes = [_p, _i64, _f32, _i32, _p]
+        L.orc_calc_padding_and_output_size.restype = _int
+        L.orc_calc_padding_and_output_size.argtypes = [_i64] * 4 + [_int] * 5 + [_p] * 4
+        L.orc_calc_output_size_floor.restype = None
+        L.orc_calc_output_size_floor.argtypes = [_i64] * 4 + [_int] * 4 + [_p, _p]
+        L.orc_im2col_u8.restype = None
+        L.orc_im2col_u8.argtypes = [_p] + [_i64] * 6 + [_int, _int, C.c_uint8, _int, _int, _i64, _i64, _p]
+        L.orc_conv2d_q8_nhwc.restype = _int
+        L.orc_conv2d_q8_nhwc.argtypes = ([_p, _p, _p] + [_i64] * 7 + [_int] * 4 +
+                                         [_f32, _i32, _f32, _i32, _f32, _f32, _i32, _int, _int, _p, _int])
+        L.orc_conv2d_q8_nhwc_direct_i32.restype = None
+        L.orc_conv2d_q8_nhwc_direct_i32.argtypes = ([_p, _p] + [_i64] * 7 + [_int] * 4 +
+                                                    [_i64, _i64, _i32, _i32, _p])
         L.orc_get_bias_data.restype = _int
         L.orc_get_bias_data.argtypes = [_p, _f32, _f32, _f32, _i64, _p]
         gemm_f32 = [_p, _p, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _int, _p, _int]
@@ -345,6 +357,64 @@ def conv1x1_q8_nhwc_direct_i32(inp, filt, n, h, w, cin, cout, input_zp, filter_z
     lib().orc_conv1x1_q8_nhwc_direct_i32(_ptr(inp), _ptr(filt), n, h, w, cin, cout,
                                          input_zp, filter_zp, _ptr(out))
     return out.reshape(n, h, w, cout)
+
+
+PAD_VALID, PAD_SAME, PAD_FULL = 0, 1, 2
+
+
+def calc_padding_and_output_size(in_h, in_w, k_h, k_w, strides, padding, dilations=(1, 1)):
+    """(out_h, out_w, pad_h, pad_w) of conv_pool_2d_util.cc:30-120; paddings are totals."""
+    oh, ow, ph, pw = C.c_int64(), C.c_int64(), C.c_int(), C.c_int()
+    rc = lib().orc_calc_padding_and_output_size(in_h, in_w, k_h, k_w, dilations[0], dilations[1],
+                                                strides[0], strides[1], padding, C.byref(oh),
+                                                C.byref(ow), C.byref(ph), C.byref(pw))
+    if rc:
+        raise ValueError("invalid strides / dilations / padding type")
+    return oh.value, ow.value, ph.value, pw.value
+
+
+def calc_output_size_floor(in_h, in_w, k_h, k_w, strides, pads):
+    oh, ow = C.c_int64(), C.c_int64()
+    lib().orc_calc_output_size_floor(in_h, in_w, k_h, k_w, strides[0], strides[1], pads[0],
+                                     pads[1], C.byref(oh), C.byref(ow))
+    return oh.value, ow.value
+
+
+def im2col_u8(inp, n, in_h, in_w, cin, k_h, k_w, strides, zero_point, pads, out_h, out_w):
+    inp = _c(inp, np.uint8)
+    assert inp.size == n * in_h * in_w * cin
+    out = np.empty(n * out_h * out_w * k_h * k_w * cin, dtype=np.uint8)
+    lib().orc_im2col_u8(_ptr(inp), n, in_h, in_w, cin, k_h, k_w, strides[0], strides[1],
+                        zero_point, pads[0], pads[1], out_h, out_w, _ptr(out))
+    return out.reshape(n * out_h * out_w, k_h * k_w * cin)
+
+
+def conv2d_q8_nhwc(inp, filt, bias, n, in_h, in_w, cin, cout, k_h, k_w, strides, pads,
+                   input_scale, input_zp, filter_scale, filter_zp, bias_scale, out_scale, out_zp,
+                   clamp_min=0, clamp_max=255, nthreads=8):
+    """Quantized Conv2D, NHWC input, OHWI filter, total paddings `pads` (top/left = pad >> 1)."""
+    inp, filt, bias = _c(inp, np.uint8), _c(filt, np.uint8), _c(bias, np.int32)
+    assert inp.size == n * in_h * in_w * cin and filt.size == cout * k_h * k_w * cin
+    oh, ow = calc_output_size_floor(in_h, in_w, k_h, k_w, strides, pads)
+    out = np.empty(max(n * oh * ow * cout, 0), dtype=np.uint8)
+    rc = lib().orc_conv2d_q8_nhwc(_ptr(inp), _ptr(filt), _ptr(bias), n, in_h, in_w, cin, cout,
+                                  k_h, k_w, strides[0], strides[1], pads[0], pads[1],
+                                  np.float32(input_scale), input_zp, np.float32(filter_scale),
+                                  filter_zp, np.float32(bias_scale), np.float32(out_scale),
+                                  out_zp, clamp_min, clamp_max, _ptr(out), nthreads)
+    if rc == 1:
+        raise ValueError("output multiplier outside (0,1)")
+    return out.reshape(n, oh, ow, cout)
+
+
+def conv2d_q8_nhwc_direct_i32(inp, filt, n, in_h, in_w, cin, cout, k_h, k_w, strides, pads,
+                              out_h, out_w, input_zp, filter_zp):
+    inp, filt = _c(inp, np.uint8), _c(filt, np.uint8)
+    out = np.empty(n * out_h * out_w * cout, dtype=np.int32)
+    lib().orc_conv2d_q8_nhwc_direct_i32(_ptr(inp), _ptr(filt), n, in_h, in_w, cin, cout, k_h,
+                                        k_w, strides[0], strides[1], pads[0], pads[1], out_h,
+                                        out_w, input_zp, filter_zp, _ptr(out))
+    return out.reshape(n, out_h, out_w, cout)
 
 
 def conv1x1_f32_nchw(inp, filt, bias, n, cin, hw, cout, act=ACT_NOOP, limit=0.0,

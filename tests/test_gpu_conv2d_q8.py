@@ -1,0 +1,127 @@
+"""General quantized Conv2D (NHWC, any filter / stride, zero-point padding) on the GPU vs the
+CPU oracle, bit for bit: the reference's one bit-exact value run as a real 3x3 convolution
+(conv_2d_test.cc:1240-1275), the reference's shape list (conv_2d_test.cc:1382-1397: 1x1, 3x3,
+1x5, 5x1, 5x5, 7x7; VALID / SAME / FULL; strides 1-3; batch 9; ragged 129 <- 63 on 33x31), channel
+counts that are not multiples of 16 (the byte-wise gather) and explicit paddings."""
+import ctypes as C
+import json
+import os
+
+import numpy as np
+import pytest
+
+from mace_amd import lib as mh
+from oracle import mace_oracle as orc
+from gpu_util import c_, ptr
+
+pytestmark = pytest.mark.gpu
+GOLDEN = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_vectors.json")))
+V, S, Fu = orc.PAD_VALID, orc.PAD_SAME, orc.PAD_FULL
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = mh.Context(0)
+    yield c
+    c.close()
+
+
+def conv_host(ctx, x, f, bias, n, in_h, in_w, cin, cout, k_h, k_w, st, pads, s_in, z_in, s_f, z_f,
+              s_b, s_o, z_o, lo=0, hi=255):
+    oh, ow = orc.calc_output_size_floor(in_h, in_w, k_h, k_w, st, pads)
+    out = np.empty(n * oh * ow * cout, np.uint8)
+    ctx.call("mace_hip_conv2d_q8_nhwc_host", ptr(c_(x, np.uint8)), ptr(c_(f, np.uint8)),
+             ptr(c_(bias, np.int32)), n, in_h, in_w, cin, cout, k_h, k_w, st[0], st[1], pads[0],
+             pads[1], s_in, z_in, s_f, z_f, s_b, s_o, z_o, lo, hi, ptr(out))
+    return out.reshape(n, oh, ow, cout)
+
+
+def test_reference_3x3_known_answer(ctx):
+    k = GOLDEN["conv_q8_kat"]
+    out = conv_host(ctx, np.array(k["input"], np.uint8), np.array(k["filter"], np.uint8),
+                    np.array(k["bias"], np.int32), 1, 3, 3, 2, 1, 3, 3, (1, 1), (0, 0),
+                    k["input_scale"], k["input_zp"], k["filter_scale"], k["filter_zp"],
+                    k["bias_scale"], k["out_scale"], k["out_zp"])
+    assert out.reshape(-1).tolist() == [k["expected"]]
+
+
+def test_padding_rule_matches_oracle(ctx):
+    lib = mh.load()
+    oh, ow, ph, pw = C.c_int64(), C.c_int64(), C.c_int(), C.c_int()
+    for in_h, in_w in ((32, 32), (33, 31), (7, 9), (224, 224)):
+        for k_h, k_w in ((1, 1), (3, 3), (1, 5), (7, 7)):
+            for st in ((1, 1), (2, 2), (3, 3), (1, 2)):
+                for pad in (V, S, Fu):
+                    rc = lib.mace_hip_calc_padding_and_output_size(
+                        in_h, in_w, k_h, k_w, 1, 1, st[0], st[1], pad, C.byref(oh), C.byref(ow),
+                        C.byref(ph), C.byref(pw))
+                    assert rc == mh.SUCCESS
+                    assert (oh.value, ow.value, ph.value, pw.value) == \
+                        orc.calc_padding_and_output_size(in_h, in_w, k_h, k_w, st, pad)
+    assert lib.mace_hip_calc_padding_and_output_size(8, 8, 3, 3, 2, 2, 2, 2, S, C.byref(oh),
+                                                     C.byref(ow), C.byref(ph), C.byref(pw)) == mh.INVALID_ARGS
+
+
+CASES = [  # batch, cout, cin, in_h, in_w, k_h, k_w, padding, strides: the reference's list
+    (1, 128, 64, 32, 32, 1, 1, V, (1, 1)), (1, 128, 64, 32, 32, 3, 3, V, (1, 1)),
+    (1, 128, 64, 32, 32, 3, 3, S, (1, 1)), (1, 128, 64, 32, 32, 3, 3, Fu, (1, 1)),
+    (1, 128, 64, 32, 32, 3, 3, S, (2, 2)), (1, 129, 63, 33, 31, 3, 3, S, (1, 1)),
+    (9, 128, 64, 32, 32, 3, 3, S, (1, 1)), (1, 128, 64, 32, 32, 1, 5, S, (1, 1)),
+    (1, 128, 64, 32, 32, 5, 5, S, (1, 1)), (1, 128, 64, 32, 32, 5, 1, S, (1, 1)),
+    (1, 128, 64, 32, 32, 7, 7, S, (1, 1)), (1, 128, 64, 32, 32, 7, 7, S, (2, 2)),
+    (1, 128, 64, 32, 32, 7, 7, S, (3, 3)),
+    # beyond it: first layer of a MobileNet (3 input channels), 1x1 at stride 2, tiny and odd
+    (2, 32, 3, 64, 64, 3, 3, S, (2, 2)), (2, 64, 32, 17, 17, 1, 1, V, (2, 2)),
+    (2, 5, 3, 6, 11, 2, 4, Fu, (1, 2)), (1, 1, 1, 1, 1, 1, 1, S, (1, 1)),
+    (3, 40, 16, 9, 9, 3, 3, S, (1, 1)), (1, 64, 32, 56, 56, 3, 3, S, (1, 1)),
+]
+
+
+@pytest.mark.parametrize("n,cout,cin,in_h,in_w,k_h,k_w,pad,st", CASES)
+def test_conv2d_q8_parity(ctx, n, cout, cin, in_h, in_w, k_h, k_w, pad, st):
+    rng = np.random.default_rng(cout * 31 + cin + k_h * 7 + k_w + pad + st[0])
+    x = rng.integers(0, 256, (n, in_h, in_w, cin), dtype=np.uint8)
+    f = rng.integers(1, 256, (cout, k_h, k_w, cin), dtype=np.uint8)
+    bias = rng.integers(-2 ** 15, 2 ** 15, cout).astype(np.int32)
+    z_in, z_f = int(rng.integers(100, 156)), int(rng.integers(118, 138))
+    s_in, s_f = np.float32(0.02), np.float32(0.01)
+    depth = k_h * k_w * cin
+    s_out = np.float32(max(6.0, 3 * 74.0 * 74.0 * np.sqrt(depth) * float(s_in * s_f)) / 255.0)
+    oh, ow, ph, pw = orc.calc_padding_and_output_size(in_h, in_w, k_h, k_w, st, pad)
+    for (bb, s_b, z_o, lo, hi) in ((bias, np.float32(s_in * s_f), 0, 0, 255),
+                                   (bias, np.float32(2.5 * float(s_in * s_f)), 100, 100, 230),
+                                   (None, np.float32(0), 128, 0, 255)):
+        want = orc.conv2d_q8_nhwc(x, f, bb, n, in_h, in_w, cin, cout, k_h, k_w, st, (ph, pw), s_in,
+                                  z_in, s_f, z_f, s_b, s_out, z_o, lo, hi)
+        got = conv_host(ctx, x, f, bb, n, in_h, in_w, cin, cout, k_h, k_w, st, (ph, pw), s_in,
+                        z_in, s_f, z_f, s_b, s_out, z_o, lo, hi)
+        assert got.shape == (n, oh, ow, cout)
+        np.testing.assert_array_equal(got, want)
+    if want.size >= 64:
+        assert len(np.unique(want)) > 8
+
+
+def test_conv2d_q8_explicit_paddings_and_errors(ctx):
+    """Asymmetric totals (odd paddings put the extra row / column at the bottom / right) and a
+    padded 1x1 (which takes the gather path here)."""
+    rng = np.random.default_rng(5)
+    n, in_h, in_w, cin, cout = 2, 10, 12, 16, 24
+    x = rng.integers(0, 256, (n, in_h, in_w, cin), dtype=np.uint8)
+    for (k_h, k_w, st, pads) in ((3, 3, (1, 1), (1, 3)), (3, 3, (2, 1), (5, 0)), (1, 1, (1, 1), (2, 2)),
+                                 (4, 2, (1, 1), (3, 1))):
+        f = rng.integers(1, 256, (cout, k_h, k_w, cin), dtype=np.uint8)
+        want = orc.conv2d_q8_nhwc(x, f, None, n, in_h, in_w, cin, cout, k_h, k_w, st, pads, 0.02, 90,
+                                  0.01, 127, 0.0, 0.9, 128)
+        got = conv_host(ctx, x, f, None, n, in_h, in_w, cin, cout, k_h, k_w, st, pads,
+                        np.float32(0.02), 90, np.float32(0.01), 127, np.float32(0.0), np.float32(0.9), 128)
+        np.testing.assert_array_equal(got, want)
+    f = rng.integers(1, 256, (cout, 3, 3, cin), dtype=np.uint8)
+    out = np.zeros(16, np.uint8)
+    args = (ptr(x), ptr(f), None, n, in_h, in_w, cin, cout, 3, 3)
+    tail = (np.float32(0.02), 90, np.float32(0.01), 127, np.float32(0.0), np.float32(0.9), 128, 0, 255, ptr(out))
+    assert ctx.status("mace_hip_conv2d_q8_nhwc_host", *args, 0, 1, 0, 0, *tail) == mh.INVALID_ARGS   # stride 0
+    assert ctx.status("mace_hip_conv2d_q8_nhwc_host", *args, 1, 1, -1, 0, *tail) == mh.INVALID_ARGS  # negative pad
+    tail_bad = (np.float32(0.02), 90, np.float32(0.01), 127, np.float32(0.0), np.float32(1e-6), 128, 0, 255, ptr(out))
+    assert ctx.status("mace_hip_conv2d_q8_nhwc_host", *args, 1, 1, 0, 0, *tail_bad) == mh.INVALID_ARGS  # multiplier >= 1
+    big = (ptr(x), ptr(f), None, n, 2, 2, cin, cout, 5, 5)
+    assert ctx.status("mace_hip_conv2d_q8_nhwc_host", *big, 1, 1, 0, 0, *tail) == mh.INVALID_ARGS    # filter > input
