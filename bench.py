@@ -304,6 +304,30 @@ def bench_other(ctx, mh, torch):
                     "GBps": round(nbytes / (k * 1e-3) / 1e9, 1), "ops_per_byte": round(ai, 1),
                     "roofline_TOPS": round(roof_tops, 1), "frac_of_roofline": round(tops / roof_tops, 4)})
 
+    # beyond the 1x1 shapes: a 3x3 convolution through the im2col path (SAME padding, stride 1)
+    for (hw, cin, cout, k) in ((56, 64, 64, 3), (28, 128, 128, 3)):
+        n = 64
+        x, f = u8(n, hw, hw, cin), u8(cout, k, k, cin)
+        bias = torch.randint(-2 ** 15, 2 ** 15, (cout,), dtype=torch.int32, device="cuda", generator=g)
+        y = torch.empty((n, hw, hw, cout), dtype=torch.uint8, device="cuda")
+        s_in, s_f = 0.02, 0.01
+        s_out = max(6.0, 3 * 74.0 * 74.0 * (k * k * cin) ** 0.5 * s_in * s_f) / 255.0
+        torch.cuda.synchronize()
+        whole, kms = time_kernel(ctx, lambda: ctx.call(
+            "mace_hip_conv2d_q8_nhwc", x.data_ptr(), f.data_ptr(), bias.data_ptr(), n, hw, hw, cin,
+            cout, k, k, 1, 1, k - 1, k - 1, s_in, 128, s_f, 127, s_in * s_f, s_out, 0, 0, 255,
+            y.data_ptr()))
+        pix = n * hw * hw
+        ops = 2.0 * pix * k * k * cin * cout
+        nbytes = pix * cin + cout * k * k * cin + 4 * cout + pix * cout
+        roof_tops = min(PEAK_INT8_TOPS, ops / nbytes * PEAK_HBM_GBS / 1e3)
+        tops = ops / (whole * 1e-3) / 1e12
+        out.append({"workload": "q8_conv%dx%d_n64_%dx%dx%d_to_%d" % (k, k, hw, hw, cin, cout),
+                    "call_ms": round(whole, 4), "gemm_kernel_ms": round(kms, 4),
+                    "TOPS_whole_call": round(tops, 1), "roofline_TOPS": round(roof_tops, 1),
+                    "frac_of_roofline": round(tops / roof_tops, 4),
+                    "note": "im2col matrix materialised (%d MB)" % (pix * k * k * cin // 10 ** 6)})
+
     # config 2: fp32 Gemm, batch 4, 1024^3, the four transpose combinations
     A = torch.randn((4, 1024, 1024), dtype=torch.float32, device="cuda", generator=g)
     B = torch.randn((4, 1024, 1024), dtype=torch.float32, device="cuda", generator=g)

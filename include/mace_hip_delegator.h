@@ -21,6 +21,7 @@
 
 #include <cstdint>
 #include <functional>
+#include <cmath>
 #include <memory>
 #include <numeric>
 #include <sstream>
@@ -538,33 +539,78 @@ class FullyConnectedOp {
   std::unique_ptr<delegator::Gemv> gemv_;
 };
 
-// Conv2dOp<RT_CPU, uint8_t>::Run for a 1x1 / stride 1 / dilation 1 filter
-// (mace/ops/conv_2d.cc:201-318): NHWC input, OHWI filter, NHWC output.  UNSUPPORTED for any
-// other filter (the reference's im2col path is outside this library).
-class Conv2dK1x1OpQuant {
+enum Padding { VALID = 0, SAME = 1, FULL = 2 };   // mace/ops/common/conv_pool_2d_util.h
+
+// Conv2dOp<RT_CPU, uint8_t>::Run (mace/ops/conv_2d.cc:201-318): NHWC input, OHWI filter, NHWC
+// output, dilation 1.  The output shape comes from the padding type (CalcPaddingAndOutputSize)
+// or, when explicit paddings are given, from the FLOOR rule (CalcOutputSize), exactly as the
+// op does (:213-235).  A fused quantized ReLUx is the clamp range.
+class Conv2dOpQuant {
  public:
-  Conv2dK1x1OpQuant(int clamp_min = 0, int clamp_max = 255)
-      : clamp_min_(clamp_min), clamp_max_(clamp_max) {}
+  Conv2dOpQuant(std::vector<int> strides = {1, 1}, Padding padding_type = SAME,
+                std::vector<int> paddings = {}, std::vector<int> dilations = {1, 1},
+                int clamp_min = 0, int clamp_max = 255)
+      : strides_(std::move(strides)), padding_type_(padding_type), paddings_(std::move(paddings)),
+        dilations_(std::move(dilations)), clamp_min_(clamp_min), clamp_max_(clamp_max) {}
   MaceStatus Run(OpContext *context, const Tensor *input, const Tensor *filter,
                  const Tensor *bias, Tensor *output) {
     if (input->dim_size() != 4 || filter->dim_size() != 4) return MaceStatus::MACE_INVALID_ARGS;
-    if (filter->dim(1) != 1 || filter->dim(2) != 1) return MaceStatus::MACE_UNSUPPORTED;
+    if (strides_.size() != 2 || dilations_.size() != 2) return MaceStatus::MACE_INVALID_ARGS;
+    // "Quantization convolution does not support dilation > 1 yet." (:207-208)
+    if (dilations_[0] != 1 || dilations_[1] != 1) return MaceStatus::MACE_INVALID_ARGS;
     if (filter->dim(3) != input->dim(3)) return MaceStatus::MACE_INVALID_ARGS;
     if (bias && bias->dim(0) != filter->dim(0)) return MaceStatus::MACE_INVALID_ARGS;
-    MaceStatus st =
-        output->Resize({input->dim(0), input->dim(1), input->dim(2), filter->dim(0)});
+    int64_t out_h = 0, out_w = 0;
+    int pads[2] = {0, 0};
+    if (paddings_.empty()) {
+      MaceStatus st = ToStatus(mace_hip_calc_padding_and_output_size(
+          input->dim(1), input->dim(2), filter->dim(1), filter->dim(2), dilations_[0],
+          dilations_[1], strides_[0], strides_[1], padding_type_, &out_h, &out_w, &pads[0],
+          &pads[1]));
+      if (st != MaceStatus::MACE_SUCCESS) return st;
+    } else {
+      if (paddings_.size() != 2 || strides_[0] <= 0 || strides_[1] <= 0)
+        return MaceStatus::MACE_INVALID_ARGS;
+      pads[0] = paddings_[0];
+      pads[1] = paddings_[1];
+      out_h = static_cast<int64_t>(
+          std::floor(1.0 * (input->dim(1) + pads[0] - filter->dim(1)) / strides_[0]) + 1);
+      out_w = static_cast<int64_t>(
+          std::floor(1.0 * (input->dim(2) + pads[1] - filter->dim(2)) / strides_[1]) + 1);
+    }
+    MaceStatus st = output->Resize({input->dim(0), out_h, out_w, filter->dim(0)});
     if (st != MaceStatus::MACE_SUCCESS) return st;
-    auto fn = output->on_device() ? mace_hip_conv1x1_q8_nhwc : mace_hip_conv1x1_q8_nhwc_host;
+    auto fn = output->on_device() ? mace_hip_conv2d_q8_nhwc : mace_hip_conv2d_q8_nhwc_host;
     return ToStatus(fn(context->hip(), input->data<uint8_t>(), filter->data<uint8_t>(),
                        bias ? bias->data<int32_t>() : nullptr, input->dim(0), input->dim(1),
-                       input->dim(2), input->dim(3), filter->dim(0), input->scale(),
+                       input->dim(2), input->dim(3), filter->dim(0), filter->dim(1),
+                       filter->dim(2), strides_[0], strides_[1], pads[0], pads[1], input->scale(),
                        input->zero_point(), filter->scale(), filter->zero_point(),
                        bias ? bias->scale() : 0.f, output->scale(), output->zero_point(),
                        clamp_min_, clamp_max_, output->mutable_data<uint8_t>()));
   }
 
  private:
+  std::vector<int> strides_;
+  Padding padding_type_;
+  std::vector<int> paddings_, dilations_;
   int clamp_min_, clamp_max_;
+};
+
+// The 1x1 / stride 1 / no padding case under its earlier name.
+class Conv2dK1x1OpQuant {
+ public:
+  Conv2dK1x1OpQuant(int clamp_min = 0, int clamp_max = 255)
+      : op_({1, 1}, VALID, {}, {1, 1}, clamp_min, clamp_max) {}
+  MaceStatus Run(OpContext *context, const Tensor *input, const Tensor *filter,
+                 const Tensor *bias, Tensor *output) {
+    if (filter->dim_size() == 4 && (filter->dim(1) != 1 || filter->dim(2) != 1))
+      return MaceStatus::MACE_UNSUPPORTED;
+    return op_.Run(context, input, filter, bias, output);
+  }
+
+ private:
+  Conv2dOpQuant op_;
 };
 
 // QuantizeOp<RT_CPU, uint8_t> (mace/ops/arm/q8/quantize.cc:31-72): float -> uint8.  An output

@@ -1104,10 +1104,10 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
   const bool x_is_lhs = out_order == MACE_HIP_COL_MAJOR;
   // The Y operand's row sums can be taken inside the GEMM kernel from the fragments it already
-  // holds, which saves one pass over that operand; worth it when the GEMM is short in K and the
-  // extra pass is a visible share of the memory traffic.  (At K = 8192 the extra dot
-  // instructions in the main loop cost 37 us per launch and the saved pass 11 us.)
-  const bool sum_y = depth > 0 && depth <= 1024;
+  // holds, which saves one pass over that operand.  The pass costs YN * K bytes of HBM traffic,
+  // the in-kernel sums about 7 % of the GEMM's own time (measured at 8192^3: +37 us against an
+  // 11 us pass), i.e. the ratio grows with XN only: in-kernel wins below XN of about 2500.
+  const bool sum_y = depth > 0 && (depth <= 1024 || (x_is_lhs ? rows : cols) <= 2048);
   const int32_t l_coef = (int32_t)(0u - zr), l_add = 0;
   const int32_t r_coef = (int32_t)(0u - zl), r_add = (int32_t)((uint32_t)depth * zl * zr);
   const int32_t *l_bias = out_u8 ? ep.bias : nullptr;

@@ -130,6 +130,34 @@ static int test_compute() {
     EXPECT(out[0] == 230);
     Tensor F3(f.data(), DT_UINT8, {1, 3, 3, 2}, 0.0226f, 127, true);
     EXPECT(conv.Run(&context, &I, &F3, &Bi, &O) == MaceStatus::MACE_UNSUPPORTED);
+    // the same test as the reference runs it: a 3x3 VALID convolution over a 3x3x2 input
+    Tensor I3(in.data(), DT_UINT8, {1, 3, 3, 2}, 0.0204f, 93);
+    ops::Conv2dOpQuant conv3({1, 1}, ops::VALID);
+    out[0] = 0;
+    EXPECT(conv3.Run(&context, &I3, &F3, &Bi, &O) == MaceStatus::MACE_SUCCESS);
+    EXPECT(out[0] == 230 && O.shape() == (std::vector<index_t>{1, 1, 1, 1}));
+    ops::Conv2dOpQuant dilated({1, 1}, ops::SAME, {}, {2, 2});
+    EXPECT(dilated.Run(&context, &I3, &F3, &Bi, &O) == MaceStatus::MACE_INVALID_ARGS);
+  }
+  {  // 3x3 SAME stride 2 against the oracle (conv_2d_test.cc:1387 shape, smaller)
+    std::mt19937 rng(11);
+    const index_t n = 2, h = 9, w = 11, cin = 16, cout = 24;
+    std::vector<uint8_t> x(n * h * w * cin), f(cout * 9 * cin);
+    std::vector<int32_t> bias(cout);
+    for (auto &v : x) v = rng() & 255;
+    for (auto &v : f) v = rng() & 255;
+    for (auto &v : bias) v = (int32_t)(rng() % 65536) - 32768;
+    int64_t oh, ow; int ph, pw;
+    EXPECT(orc_calc_padding_and_output_size(h, w, 3, 3, 1, 1, 2, 2, 1, &oh, &ow, &ph, &pw) == 0);
+    std::vector<uint8_t> y(n * oh * ow * cout), want(y.size());
+    Tensor X(x.data(), DT_UINT8, {n, h, w, cin}, 0.02f, 120), F(f.data(), DT_UINT8, {cout, 3, 3, cin}, 0.01f, 130, true),
+        Bi(bias.data(), DT_INT32, {cout}, 0.0002f, 0, true), Y(y.data(), DT_UINT8, {}, 0.5f, 100);
+    ops::Conv2dOpQuant conv({2, 2}, ops::SAME, {}, {1, 1}, 100, 200);   // fused ReLUx as a clamp
+    EXPECT(conv.Run(&context, &X, &F, &Bi, &Y) == MaceStatus::MACE_SUCCESS);
+    EXPECT(Y.shape() == (std::vector<index_t>{n, oh, ow, cout}));
+    EXPECT(orc_conv2d_q8_nhwc(x.data(), f.data(), bias.data(), n, h, w, cin, cout, 3, 3, 2, 2, ph, pw, 0.02f,
+                              120, 0.01f, 130, 0.0002f, 0.5f, 100, 100, 200, want.data(), 4) == 0);
+    EXPECT(y == want);
   }
   {  // quantized MatMul and FullyConnected vs the oracle, seeded
     std::mt19937 rng(7);
