@@ -63,7 +63,6 @@ struct GemmParams {
   int32_t xcoef, xadd;
   const int32_t *xbias;
   int tiles_x, tiles_y;
-  long long *dbg;     // lab instrumentation only (nullptr in the library)
 };
 
 // XCD-aware tile order: consecutive workgroup ids are dealt round-robin to the 8 XCDs, so
@@ -413,7 +412,7 @@ __device__ inline void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
 }
 
-template <int WX, int WY, int FX, int FY, int STAGES, typename OutT, int OCC = 1, int ABLATE = 0,
+template <int WX, int WY, int FX, int FY, int STAGES, typename OutT, int OCC = 1,
           bool SUMY = false>
 __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParams p, RequantTable) {
   constexpr int NW = WX * WY;
@@ -535,8 +534,8 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
       }
       if (DELAY > 0 && m >= DELAY && m - DELAY < NF) {
         const int f = m - DELAY;
-        if (f < FX) { if (!(ABLATE & 16)) na[f] ^= flip; }
-        else { if (!(ABLATE & 8)) nb[f - FX] ^= flip; }
+        if (f < FX) na[f] ^= flip;
+        else nb[f - FX] ^= flip;
       }
       if constexpr (dma) {
         // LX + LY transfers spread over the slots from slot 0 on
@@ -558,8 +557,6 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
       }
   };
 
-  long long dbg_c0 = 0, dbg_w0 = 0;
-  if (ABLATE & 4) { dbg_c0 = clock64(); dbg_w0 = wall_clock64(); }
   const int nslab = p.K / SLAB;
   // prologue: slabs 0 .. STAGES-2 in flight
 #pragma unroll
@@ -596,15 +593,6 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
     stage = next;
   }
 
-  if (ABLATE & 4) {
-    const long long c1 = clock64(), w1 = wall_clock64();
-    gemm_epilogue<WX, WY, FX, FY, OutT, SUMY>(acc, ysum, p, lds, b, x0, y0, wx, wy, tid);
-    if (tid == 0 && blockIdx.x == 8) {
-      p.dbg[0] = c1 - dbg_c0; p.dbg[1] = w1 - dbg_w0;
-      p.dbg[2] = clock64() - c1; p.dbg[3] = wall_clock64() - w1;
-    }
-    return;
-  }
   gemm_epilogue<WX, WY, FX, FY, OutT, SUMY>(acc, ysum, p, lds, b, x0, y0, wx, wy, tid);
 }
 
@@ -976,13 +964,13 @@ int launch_gemm_dma(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, b
     return MACE_HIP_SUCCESS;
   };
   if (out_u8 && p.sum_y) {
-    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, uint8_t, OCC, 0, true>));
+    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, uint8_t, OCC, true>));
   } else if (out_u8) {
-    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, uint8_t, OCC, 0, false>));
+    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, uint8_t, OCC, false>));
   } else if (p.sum_y) {
-    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, int32_t, OCC, 0, true>));
+    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, int32_t, OCC, true>));
   } else {
-    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, int32_t, OCC, 0, false>));
+    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, int32_t, OCC, false>));
   }
   MH_PROF_END(ctx);
   MH_HIP(ctx, hipGetLastError());
@@ -1154,7 +1142,6 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   p.xadd = x_is_lhs ? l_add : r_add;
   p.xbias = x_is_lhs ? l_bias : nullptr;
   p.tiles_x = p.tiles_y = 0;
-  p.dbg = nullptr;
   if (stream) {
     switch (p.XN) {
       case 32: return launch_gemm_stream<1, 1>(ctx, p, tab, (int)batch);
@@ -1168,7 +1155,6 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   auto tiles = [&](int tx, int ty) {
     return (int64_t)((p.XN + tx - 1) / tx) * ((p.YN + ty - 1) / ty) * batch;
   };
-  p.dbg = nullptr;
   // Tile shape: bigger tiles do more MFMA work per byte moved and per barrier, smaller ones
   // keep more CUs busy.  Score = relative efficiency of the shape x the fraction of CU slots
   // its last round of workgroups fills.
