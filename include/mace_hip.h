@@ -84,6 +84,19 @@ int mace_hip_memcpy_d2h(mace_hip_ctx *ctx, void *dst_host, const void *src_dev, 
 
 /* ---- quantisation scalars (host) ------------------------------------------------------ */
 
+/* Constant operands ("weights").  MACE's delegators may keep a packed copy of a weight across
+ * calls (GemmParam::should_cache_pack_ with Tensor::is_weight(), mace/ops/delegator/gemm.h:28-33,
+ * mace/ops/arm/base/gemm.cc:560-576).  The counterpart here: once a device buffer is registered,
+ * every uint8 GEMM / Conv2D call on this context whose lhs or rhs pointer equals device_ptr (and
+ * fits in `bytes`) reuses the k-contiguous panel and the row sums derived from it on first use
+ * instead of rebuilding them per call.  The caller must not change the buffer while it is
+ * registered; register it again (or unregister it) after a change.  Unregistering frees what
+ * was derived (after synchronizing the stream); so does destroying the context. */
+int mace_hip_weight_register(mace_hip_ctx *ctx, const void *device_ptr, size_t bytes);
+int mace_hip_weight_unregister(mace_hip_ctx *ctx, const void *device_ptr);
+/* Number of times a registered weight's panel was built / reused so far (for tests). */
+int mace_hip_weight_cache_stats(mace_hip_ctx *ctx, int64_t *builds, int64_t *hits);
+
 /* mace/core/quantize.h:104-114 QuantizeMultiplier */
 void mace_hip_quantize_multiplier(double multiplier, int32_t *quantized_multiplier,
                                   int *exponent);

@@ -8,7 +8,35 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <vector>
+
 #include "mace_hip.h"
+
+// A constant operand (registered with mace_hip_weight_register) keeps what the uint8 GEMM derives
+// from it across calls: the k-contiguous, padded panel (when the caller's layout is not that
+// already) and the sums of its shifted rows.
+struct mh_weight_panel {
+  int kcontig;          // caller's layout was k-contiguous
+  int64_t n, depth;
+  int nb;
+  uint8_t *panel;       // device memory owned by the cache, or nullptr: read the weight in place
+  int64_t ld;
+  int k;
+  int32_t *sums;        // [nb][n], device memory owned by the cache
+};
+struct mh_weight {
+  const void *ptr;
+  size_t bytes;
+  std::vector<mh_weight_panel> panels;
+};
+
+inline void mh_weight_drop_panels(mh_weight *w) {
+  for (mh_weight_panel &c : w->panels) {
+    if (c.panel) (void)hipFree(c.panel);
+    if (c.sums) (void)hipFree(c.sums);
+  }
+  w->panels.clear();
+}
 
 struct mace_hip_ctx {
   int device = 0;
@@ -32,6 +60,8 @@ struct mace_hip_ctx {
   int32_t rq_cache_tab[4][258] = {};
   int rq_cache_valid[4] = {0, 0, 0, 0};
   int rq_cache_next = 0;
+  std::vector<mh_weight> weights;
+  long weight_hits = 0, weight_builds = 0;   // statistics for tests
 };
 
 int mh_fail(mace_hip_ctx *ctx, int code, const char *fmt, ...);

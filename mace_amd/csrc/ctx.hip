@@ -98,12 +98,46 @@ int mace_hip_ctx_destroy(mace_hip_ctx *ctx) {
   (void)hipSetDevice(ctx->device);
   (void)hipStreamSynchronize(ctx->stream);
   if (ctx->arena) (void)hipFree(ctx->arena);
+  for (mh_weight &w : ctx->weights) mh_weight_drop_panels(&w);
   (void)hipEventDestroy(ctx->ev_start);
   (void)hipEventDestroy(ctx->ev_stop);
   (void)hipEventDestroy(ctx->ev_k0);
   (void)hipEventDestroy(ctx->ev_k1);
   (void)hipStreamDestroy(ctx->own_stream);
   delete ctx;
+  return MACE_HIP_SUCCESS;
+}
+
+int mace_hip_weight_register(mace_hip_ctx *ctx, const void *device_ptr, size_t bytes) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_CHECK(ctx, device_ptr && bytes > 0, "null or empty weight");
+  for (mh_weight &w : ctx->weights)
+    if (w.ptr == device_ptr) {   // registered again: whatever was derived from it is stale
+      MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
+      mh_weight_drop_panels(&w);
+      w.bytes = bytes;
+      return MACE_HIP_SUCCESS;
+    }
+  ctx->weights.push_back(mh_weight{device_ptr, bytes, {}});
+  return MACE_HIP_SUCCESS;
+}
+
+int mace_hip_weight_unregister(mace_hip_ctx *ctx, const void *device_ptr) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  for (size_t i = 0; i < ctx->weights.size(); ++i)
+    if (ctx->weights[i].ptr == device_ptr) {
+      MH_HIP(ctx, hipStreamSynchronize(ctx->stream));   // kernels may still read the panels
+      mh_weight_drop_panels(&ctx->weights[i]);
+      ctx->weights.erase(ctx->weights.begin() + (long)i);
+      return MACE_HIP_SUCCESS;
+    }
+  return mh_fail(ctx, MACE_HIP_INVALID_ARGS, "weight %p is not registered", device_ptr);
+}
+
+int mace_hip_weight_cache_stats(mace_hip_ctx *ctx, int64_t *builds, int64_t *hits) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  if (builds) *builds = ctx->weight_builds;
+  if (hits) *hits = ctx->weight_hits;
   return MACE_HIP_SUCCESS;
 }
 

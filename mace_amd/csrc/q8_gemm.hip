@@ -47,19 +47,18 @@ struct GemmParams {
   int64_t ldx, ldy;
   int64_t xbs, ybs;   // batch strides in bytes (0 = shared across the batch)
   int XN, YN, K;      // K = bytes of k to read per row (multiple of 16)
-  const int32_t *corrX;  // [batch or 1][XN]
-  const int32_t *corrY;  // [batch or 1][YN]
+  const int32_t *corrX;  // [batch or 1][XN] sums of the shifted bytes of every X row
+  const int32_t *corrY;  // [batch or 1][YN] (not read when the kernel sums Y itself)
   int64_t cxbs, cybs;    // batch strides of the correction vectors (elements)
   void *out;
   int64_t ldo;        // elements between consecutive y
   int64_t obs;        // elements per batch
   RequantFixed rq;    // uint8 output pipeline
-  // When the kernel sums the Y panel itself (SUMY): corrY[y] = ycoef * sum_k Y'[y][k] + yadd
-  // (+ ybias[y]) is formed in the epilogue and corrY is not read.
+  // correction term of result (x, y): xcoef * sumX[x] + xadd (+ xbias[x]) + ycoef * sumY[y] +
+  // yadd (+ ybias[y]), formed in the epilogue
   int32_t ycoef, yadd;
   const int32_t *ybias;
   bool sum_y;
-  // Same for the X panel (streaming kernel only, which sums both panels itself)
   int32_t xcoef, xadd;
   const int32_t *xbias;
   int tiles_x, tiles_y;
@@ -111,9 +110,20 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[FX][FY], const int (&y
   const int32_t *cY = p.corrY + (int64_t)b * p.cybs;
   int32_t *sc = (int32_t *)lds;   // [TX] corrections along x, then [TY] along y
   __syncthreads();                // every wavefront is done reading operand tiles
-  for (int i = tid; i < TX; i += NT) sc[i] = cX[min(x0 + i, p.XN - 1)];
+  // panel sums -> correction terms: coef * sum + add (+ bias on the side the result rows are on)
+  for (int i = tid; i < TX; i += NT) {
+    const int x = min(x0 + i, p.XN - 1);
+    uint32_t c = (uint32_t)p.xcoef * (uint32_t)cX[x] + (uint32_t)p.xadd;
+    if (p.xbias) c += (uint32_t)p.xbias[x];
+    sc[i] = (int32_t)c;
+  }
   if (!SUMY)
-    for (int i = tid; i < TY; i += NT) sc[TX + i] = cY[min(y0 + i, p.YN - 1)];
+    for (int i = tid; i < TY; i += NT) {
+      const int y = min(y0 + i, p.YN - 1);
+      uint32_t c = (uint32_t)p.ycoef * (uint32_t)cY[y] + (uint32_t)p.yadd;
+      if (p.ybias) c += (uint32_t)p.ybias[y];
+      sc[TX + i] = (int32_t)c;
+    }
   const RequantFixed rq = p.rq;
   int32_t *tab = sc + TX + TY;    // [n + 2] comparison table of the threshold requantization
   if constexpr (sizeof(OutT) == 1) {
@@ -861,9 +871,7 @@ __global__ __launch_bounds__(256) void q8_pack_transpose128_kernel(const uint8_t
 template <int LPR>
 __global__ __launch_bounds__(256) void q8_panel_sums_kernel(const uint8_t *P, int64_t ld,
                                                             int64_t pbs, int n, int k,
-                                                            int32_t coef, int32_t add,
-                                                            const int32_t *bias,
-                                                            int32_t *corr) {
+                                                            int32_t *sums) {
   constexpr int RPW = 64 / LPR;   // rows per wavefront
   const int lane = threadIdx.x & 63;
   const int sub = lane % LPR;
@@ -882,16 +890,13 @@ __global__ __launch_bounds__(256) void q8_panel_sums_kernel(const uint8_t *P, in
 #pragma unroll
   for (int off = LPR / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
   if (sub == 0 && live) {
-    const uint32_t shifted = s - 128u * (uint32_t)k;   // sum of (byte - 128)
-    uint32_t v = (uint32_t)coef * shifted + (uint32_t)add;
-    if (bias) v += (uint32_t)bias[row];
-    corr[(int64_t)blockIdx.z * n + row] = (int32_t)v;
+    // sum of (byte - 128); the epilogue turns it into the correction term
+    sums[(int64_t)blockIdx.z * n + row] = (int32_t)(s - 128u * (uint32_t)k);
   }
 }
 
 int launch_panel_sums(mace_hip_ctx *ctx, const uint8_t *P, int64_t ld, int64_t pbs, int64_t n,
-                      int k, int nb, int32_t coef, int32_t add, const int32_t *bias,
-                      int32_t *corr) {
+                      int k, int nb, int32_t *sums) {
   const int chunks = k / 16;
   int lpr = 1;
   while (lpr < 64 && lpr < chunks) lpr *= 2;
@@ -901,7 +906,7 @@ int launch_panel_sums(mace_hip_ctx *ctx, const uint8_t *P, int64_t ld, int64_t p
   dim3 grid((unsigned)blocks, 1, nb), block(256);
 #define MH_SUMS(L_)                                                                       \
   hipLaunchKernelGGL((q8_panel_sums_kernel<L_>), grid, block, 0, ctx->stream, P, ld, pbs, \
-                     (int)n, k, coef, add, bias, corr)
+                     (int)n, k, sums)
   switch (lpr) {
     case 1: MH_SUMS(1); break;
     case 2: MH_SUMS(2); break;
@@ -1035,30 +1040,31 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   const bool rhs_direct = rhs_ld != 0 || (rhs_order == MACE_HIP_COL_MAJOR && depth % 16 == 0 &&
                                           depth > 0 && ((uintptr_t)rhs % 16 == 0));
 
+  // operands registered as constant weights keep their panel and sums in the context
+  auto find_weight = [&](const uint8_t *src, size_t bytes) -> mh_weight * {
+    if (depth == 0) return nullptr;
+    for (mh_weight &w : ctx->weights)
+      if (w.ptr == (const void *)src && bytes <= w.bytes) return &w;
+    return nullptr;
+  };
+  mh_weight *lhs_w = find_weight(lhs, (size_t)lhs_nb * rows * depth);
+  mh_weight *rhs_w = rhs_ld != 0 ? nullptr : find_weight(rhs, (size_t)rhs_nb * cols * depth);
+
   size_t need = sizeof(int32_t) * ((size_t)lhs_nb * rows + (size_t)rhs_nb * cols) + 4096;
-  if (!lhs_direct) need += (size_t)lhs_nb * rows * kp + 256;
-  if (!rhs_direct) need += (size_t)rhs_nb * cols * kp + 256;
+  if (!lhs_direct && !lhs_w) need += (size_t)lhs_nb * rows * kp + 256;
+  if (!rhs_direct && !rhs_w) need += (size_t)rhs_nb * cols * kp + 256;
   MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, need));
   ArenaScope scope(ctx);
 
   struct Panel {
     const uint8_t *ptr;
     int64_t ld, bs;
-    int k;   // readable bytes of k per row
+    int k;                  // readable bytes of k per row
+    const int32_t *sums;    // cached row sums of a registered weight, or nullptr
   } L, R;
 
-  auto prepare = [&](const uint8_t *src, int order_is_kcontig, bool direct, int nb, int64_t n,
-                     int64_t ld, Panel *P) -> int {
-    if (direct) {
-      // a caller-padded panel (ld > depth) is readable, and zero after the shift, up to ld
-      *P = Panel{src, ld, nb > 1 ? n * ld : 0, (int)ld};
-      return MACE_HIP_SUCCESS;
-    }
-    uint8_t *dst = (uint8_t *)mh_arena_take(ctx, (size_t)nb * n * kp);
-    if (!dst) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
-    if (depth == 0) {
-      MH_HIP(ctx, hipMemsetAsync(dst, 0x80, (size_t)nb * n * kp, ctx->stream));
-    } else if (order_is_kcontig) {
+  auto pack = [&](const uint8_t *src, int order_is_kcontig, int nb, int64_t n, uint8_t *dst) -> int {
+    if (order_is_kcontig) {
       const int64_t total = n * kp;
       dim3 grid((unsigned)std::min<int64_t>((total + 255) / 256, 65535), 1, nb);
       hipLaunchKernelGGL(q8_pack_rows_kernel, grid, dim3(256), 0, ctx->stream, src,
@@ -1077,12 +1083,64 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
       }
     }
     MH_HIP(ctx, hipGetLastError());
-    *P = Panel{dst, kp, nb > 1 ? n * kp : 0, (int)kp};
     return MACE_HIP_SUCCESS;
   };
-  MH_RETURN_IF_ERROR(prepare(lhs, lhs_order == MACE_HIP_ROW_MAJOR, lhs_direct, lhs_nb, rows, depth, &L));
+
+  // a registered weight: reuse (or build once, in memory of its own) its panel and row sums
+  auto prepare_weight = [&](mh_weight *w, const uint8_t *src, int order_is_kcontig, bool direct,
+                            int nb, int64_t n, Panel *P) -> int {
+    for (const mh_weight_panel &c : w->panels)
+      if (c.kcontig == order_is_kcontig && c.n == n && c.depth == depth && c.nb == nb) {
+        *P = Panel{c.panel ? c.panel : src, c.ld, nb > 1 ? n * c.ld : 0, c.k, c.sums};
+        ++ctx->weight_hits;
+        return MACE_HIP_SUCCESS;
+      }
+    mh_weight_panel c{order_is_kcontig, n, depth, nb, nullptr, direct ? depth : kp,
+                      (int)(direct ? depth : kp), nullptr};
+    if (!direct) {
+      MH_HIP(ctx, hipMalloc((void **)&c.panel, (size_t)nb * n * kp));
+      const int rc = pack(src, order_is_kcontig, nb, n, c.panel);
+      if (rc != MACE_HIP_SUCCESS) { (void)hipFree(c.panel); return rc; }
+    }
+    hipError_t e = hipMalloc((void **)&c.sums, sizeof(int32_t) * (size_t)nb * n);
+    if (e != hipSuccess) {
+      if (c.panel) (void)hipFree(c.panel);
+      MH_HIP(ctx, e);
+    }
+    const int rc = launch_panel_sums(ctx, c.panel ? c.panel : src, c.ld, nb > 1 ? n * c.ld : 0, n,
+                                     c.k, nb, c.sums);
+    if (rc != MACE_HIP_SUCCESS) {
+      if (c.panel) (void)hipFree(c.panel);
+      (void)hipFree(c.sums);
+      return rc;
+    }
+    w->panels.push_back(c);
+    ++ctx->weight_builds;
+    *P = Panel{c.panel ? c.panel : src, c.ld, nb > 1 ? n * c.ld : 0, c.k, c.sums};
+    return MACE_HIP_SUCCESS;
+  };
+
+  auto prepare = [&](const uint8_t *src, int order_is_kcontig, bool direct, int nb, int64_t n,
+                     int64_t ld, mh_weight *w, Panel *P) -> int {
+    if (w) return prepare_weight(w, src, order_is_kcontig, direct, nb, n, P);
+    if (direct) {
+      // a caller-padded panel (ld > depth) is readable, and zero after the shift, up to ld
+      *P = Panel{src, ld, nb > 1 ? n * ld : 0, (int)ld, nullptr};
+      return MACE_HIP_SUCCESS;
+    }
+    uint8_t *dst = (uint8_t *)mh_arena_take(ctx, (size_t)nb * n * kp);
+    if (!dst) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
+    if (depth == 0) {
+      MH_HIP(ctx, hipMemsetAsync(dst, 0x80, (size_t)nb * n * kp, ctx->stream));
+    } else {
+      MH_RETURN_IF_ERROR(pack(src, order_is_kcontig, nb, n, dst));
+    }
+    *P = Panel{dst, kp, nb > 1 ? n * kp : 0, (int)kp, nullptr};
+    return MACE_HIP_SUCCESS;
+  };
+  MH_RETURN_IF_ERROR(prepare(lhs, lhs_order == MACE_HIP_ROW_MAJOR, lhs_direct, lhs_nb, rows, depth, lhs_w, &L));
   MH_RETURN_IF_ERROR(prepare(rhs, rhs_order == MACE_HIP_COL_MAJOR, rhs_direct, rhs_nb, cols,
-                             rhs_ld != 0 ? rhs_ld : depth, &R));
+                             rhs_ld != 0 ? rhs_ld : depth, rhs_w, &R));
 
   // correction vectors.  zl' = -lhs_offset - 128, zr' = -rhs_offset - 128.
   //   corrL[i] = -zr' * sum_k l'[i,k] + bias[i];   corrR[j] = -zl' * sum_k r'[k,j] + K zl' zr'
@@ -1095,7 +1153,8 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   // holds, which saves one pass over that operand.  The pass costs YN * K bytes of HBM traffic,
   // the in-kernel sums about 7 % of the GEMM's own time (measured at 8192^3: +37 us against an
   // 11 us pass), i.e. the ratio grows with XN only: in-kernel wins below XN of about 2500.
-  const bool sum_y = depth > 0 && (depth <= 1024 || (x_is_lhs ? rows : cols) <= 2048);
+  const bool sum_y = depth > 0 && (depth <= 1024 || (x_is_lhs ? rows : cols) <= 2048) &&
+                     !(x_is_lhs ? R.sums : L.sums);   // cached sums cost nothing
   const int32_t l_coef = (int32_t)(0u - zr), l_add = 0;
   const int32_t r_coef = (int32_t)(0u - zl), r_add = (int32_t)((uint32_t)depth * zl * zr);
   const int32_t *l_bias = out_u8 ? ep.bias : nullptr;
@@ -1106,13 +1165,12 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   const bool stream = out_u8 && rq.table && lhs_direct && rhs_direct &&
                       (depth == 32 || depth == 64) && (xn == 32 || xn == 64 || xn == 128) &&
                       yn >= 1024 && ((uintptr_t)out % 16 == 0);
+  const int32_t *sumL = L.sums ? L.sums : corrL, *sumR = R.sums ? R.sums : corrR;
   if (!stream) {
-    if (!(sum_y && !x_is_lhs))
-      MH_RETURN_IF_ERROR(launch_panel_sums(ctx, L.ptr, L.ld, L.bs, rows, L.k, lhs_nb, l_coef,
-                                           l_add, l_bias, corrL));
-    if (!(sum_y && x_is_lhs))
-      MH_RETURN_IF_ERROR(launch_panel_sums(ctx, R.ptr, R.ld, R.bs, cols, R.k, rhs_nb, r_coef,
-                                           r_add, nullptr, corrR));
+    if (!L.sums && !(sum_y && !x_is_lhs))
+      MH_RETURN_IF_ERROR(launch_panel_sums(ctx, L.ptr, L.ld, L.bs, rows, L.k, lhs_nb, corrL));
+    if (!R.sums && !(sum_y && x_is_lhs))
+      MH_RETURN_IF_ERROR(launch_panel_sums(ctx, R.ptr, R.ld, R.bs, cols, R.k, rhs_nb, corrR));
     MH_HIP(ctx, hipGetLastError());
   }
 
@@ -1124,8 +1182,8 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   p.XN = (int)(x_is_lhs ? rows : cols);
   p.YN = (int)(x_is_lhs ? cols : rows);
   p.K = L.k < R.k ? L.k : R.k;    // padded tails are zero after the shift, so the shorter wins
-  p.corrX = x_is_lhs ? corrL : corrR;
-  p.corrY = x_is_lhs ? corrR : corrL;
+  p.corrX = x_is_lhs ? sumL : sumR;
+  p.corrY = x_is_lhs ? sumR : sumL;
   p.cxbs = (x_is_lhs ? lhs_nb : rhs_nb) > 1 ? p.XN : 0;
   p.cybs = (x_is_lhs ? rhs_nb : lhs_nb) > 1 ? p.YN : 0;
   p.out = out;
