@@ -100,3 +100,43 @@ def test_conv1x1_q8_errors(ctx):
     st = ctx.status("mace_hip_conv1x1_q8_nhwc_host", ptr(z), ptr(z), None, 1, 2, 2, 4, 4, 1.0, 0,
                     1.0, 0, 1.0, 0.5, 0, 0, 255, ptr(z))
     assert st == mh.INVALID_ARGS and "multiplier" in ctx.last_error()
+
+
+@pytest.mark.parametrize("hw,cin,cout", [(112, 32, 64), (56, 128, 128), (28, 256, 256),
+                                         (14, 512, 512), (7, 1024, 1024)])
+def test_conv1x1_q8_batch64_sampled(ctx, hw, cin, cout):
+    """BASELINE config 4 at its full batch of 64, device pointers: every output channel of 3000
+    randomly chosen pixels (plus the first and last 64) against the oracle run on just those
+    pixels -- a pixel's outputs depend on that pixel alone -- and a checksum identity over the
+    whole tensor: the sum over pixels of the int32 outputs equals filter . (sum of the shifted
+    pixels), evaluated in int64."""
+    import torch
+    n = 64
+    rng = np.random.default_rng(hw + cin)
+    x = rng.integers(0, 256, (n * hw * hw, cin), dtype=np.uint8)
+    f = rng.integers(1, 256, (cout, cin), dtype=np.uint8)
+    bias = rng.integers(-2 ** 15, 2 ** 15, cout).astype(np.int32)
+    z_in, z_f = 128, 127
+    s_in, s_f = np.float32(0.02), np.float32(0.01)
+    s_o = np.float32(max(6.0, 3 * 74.0 * 74.0 * np.sqrt(cin) * float(s_in * s_f)) / 255.0)
+    dx, df, db = torch.from_numpy(x).cuda(), torch.from_numpy(f).cuda(), torch.from_numpy(bias).cuda()
+    dy = torch.empty((n * hw * hw, cout), dtype=torch.uint8, device="cuda")
+    torch.cuda.synchronize()
+    ctx.call("mace_hip_conv1x1_q8_nhwc", dx.data_ptr(), df.data_ptr(), db.data_ptr(), n, hw, hw, cin,
+             cout, s_in, z_in, s_f, z_f, np.float32(s_in * s_f), s_o, 0, 0, 255, dy.data_ptr())
+    ctx.sync()
+    pix = np.unique(np.concatenate([np.arange(64), np.arange(n * hw * hw - 64, n * hw * hw),
+                                    rng.integers(0, n * hw * hw, 3000)]))
+    want = orc.conv1x1_q8_nhwc(x[pix], f, bias, 1, 1, len(pix), cin, cout, s_in, z_in, s_f, z_f,
+                               s_in * s_f, s_o, 0).reshape(len(pix), cout)
+    got = dy.cpu().numpy()
+    np.testing.assert_array_equal(got[pix], want)
+    assert len(np.unique(want)) > 20
+    # whole-tensor identity on the int32 accumulators (the same kernels, int32 epilogue)
+    d32 = torch.empty((n * hw * hw, cout), dtype=torch.int32, device="cuda")
+    ctx.call("mace_hip_gemm_q8_i32", df.data_ptr(), mh.ROW_MAJOR, dx.data_ptr(), mh.COL_MAJOR,
+             d32.data_ptr(), mh.COL_MAJOR, 1, cout, cin, n * hw * hw, 1, 1, -z_f, -z_in)
+    ctx.sync()
+    total = d32.to(torch.int64).sum(dim=0).cpu().numpy()
+    xs = (x.astype(np.int64) - z_in).sum(axis=0)
+    np.testing.assert_array_equal(total, (f.astype(np.int64) - z_f) @ xs)
