@@ -204,14 +204,19 @@ def test_q8_gemm_large_device_pointers(ctx, n, lo, ro, oo):
 
 
 def test_q8_gemm_batched_512(ctx):
-    """BASELINE config 5's batched case at a size the oracle finishes quickly: 8 x 512^3."""
+    """BASELINE config 5's batched case in full: 32 x 512^3, int32 accumulators and uint8 output."""
     rng = np.random.default_rng(9)
-    b, n = 8, 512
+    b, n = 32, 512
     A = rng.integers(0, 256, (b, n, n), dtype=np.uint8)
     B = rng.integers(0, 256, (b, n, n), dtype=np.uint8)
     want = orc.q8_gemm_i32(A, B, b, n, n, n, -17, -240)
     got = gemm_i32_host(ctx, A, R, B, R, R, b, n, n, n, True, True, -17, -240)
     np.testing.assert_array_equal(got, want)
+    mult, shift = scales_for(n)
+    want8 = orc.q8_gemm_u8(A, B, b, n, n, n, -131, -122, None, mult, shift, 128)
+    got8 = gemm_u8_host(ctx, A, R, B, R, R, b, n, n, n, True, True, -131, -122, None, mult, shift, 128)
+    np.testing.assert_array_equal(got8, want8)
+    assert len(np.unique(want8)) > 100
 
 
 def test_q8_gemm_freivalds_4096(ctx):
