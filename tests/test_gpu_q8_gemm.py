@@ -219,32 +219,46 @@ def test_q8_gemm_batched_512(ctx):
     assert len(np.unique(want8)) > 100
 
 
-def test_q8_gemm_freivalds_4096(ctx):
-    """4096^3: the oracle would take minutes, so check C x == A (B x) in int64 for random
-    vectors x (size-independent property), plus 32 full rows exactly."""
+@pytest.mark.parametrize("n", [4096, 8192])
+def test_q8_gemm_freivalds_large(ctx, n):
+    """4096^3 and 8192^3 (BASELINE config 5): the oracle would take minutes, so (i) check
+    C x == A (B x) exactly for random vectors x (a size-independent property; float64 holds these
+    integers exactly), (ii) compare 32 full rows with the oracle, (iii) check the WHOLE uint8
+    output by applying the oracle's output pipeline to the int32 output verified in (i)/(ii)."""
     import torch
-    n = 4096
     g = torch.Generator(device="cuda").manual_seed(7)
     A = torch.randint(0, 256, (n, n), dtype=torch.uint8, device="cuda", generator=g)
     B = torch.randint(0, 256, (n, n), dtype=torch.uint8, device="cuda", generator=g)
     Cout = torch.empty((n, n), dtype=torch.int32, device="cuda")
+    C8 = torch.empty((n, n), dtype=torch.uint8, device="cuda")
     torch.cuda.synchronize()
-    za, zb = 101, 200
+    za, zb = 131, 122
+    mult, shift = scales_for(n)
     ctx.call("mace_hip_gemm_q8_i32", A.data_ptr(), R, B.data_ptr(), R, Cout.data_ptr(), R, 1, n,
              n, n, 1, 1, -za, -zb)
+    ctx.call("mace_hip_gemm_q8_u8", A.data_ptr(), R, B.data_ptr(), R, C8.data_ptr(), R, 1, n, n, n,
+             1, 1, -za, -zb, None, mult, shift, 128, 0, 255)
     ctx.sync()
-    Ad = (A.to(torch.float64) - za)
     Bd = (B.to(torch.float64) - zb)
     for seed in (1, 2):
         x = torch.randint(-8, 9, (n, 1), generator=torch.Generator().manual_seed(seed)).to(
             device="cuda", dtype=torch.float64)
-        lhs = Cout.to(torch.float64) @ x            # exact: |values| < 2^53
-        rhs = Ad @ (Bd @ x)
+        y = Bd @ x                                  # exact: |values| < 2^53 throughout
+        rhs = torch.empty((n, 1), dtype=torch.float64, device="cuda")
+        lhs = torch.empty((n, 1), dtype=torch.float64, device="cuda")
+        for r0 in range(0, n, 2048):                # in slabs: keeps the float64 copies small
+            rhs[r0:r0 + 2048] = (A[r0:r0 + 2048].to(torch.float64) - za) @ y
+            lhs[r0:r0 + 2048] = Cout[r0:r0 + 2048].to(torch.float64) @ x
         assert torch.equal(lhs, rhs)
+    del Bd
     rows = np.random.default_rng(7).choice(n, 32, replace=False)
     a_rows = A[rows].cpu().numpy()
     want = orc.q8_gemm_i32(a_rows, B.cpu().numpy(), 1, 32, n, n, -za, -zb)
     np.testing.assert_array_equal(Cout[rows].cpu().numpy().reshape(-1), want)
+    want8 = orc.output_pipeline_u8(Cout.cpu().numpy(), 1, n, n, R, None, mult, shift, 128)
+    got8 = C8.cpu().numpy().reshape(-1)
+    np.testing.assert_array_equal(got8, want8)
+    assert 0 < ((got8 == 0) | (got8 == 255)).mean() < 0.1 and len(np.unique(got8)) > 200
 
 
 def test_q8_gemm_errors(ctx):
