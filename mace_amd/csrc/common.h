@@ -348,12 +348,23 @@ struct Q8GemmEpilogue {
   int lo, hi;
 };
 
+// The right operand of a convolution's GEMM described instead of materialised: column
+// (image, oh, ow) is the k_h x k_w x cin patch at (oh*stride_h - pad_top, ow*stride_w - pad_left)
+// of an NHWC input, k in (kh, kw, channel) order, positions outside the input = zero_point.
+// mh_q8_gemm takes it with rhs = the input tensor, cols = images*out_h*out_w, depth = k_h*k_w*cin,
+// lhs RowMajor, result ColMajor, batch 1; cin % 64 == 0 and depth >= 192.
+struct Q8ConvGather {
+  int in_h, in_w, cin, k_h, k_w, stride_h, stride_w, pad_top, pad_left, out_h, out_w;
+  int zero_point;
+};
+
 int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8_t *rhs,
                int rhs_order, void *out, int out_order, bool out_u8, int64_t batch,
                int64_t rows, int64_t depth, int64_t cols, int lhs_batched, int rhs_batched,
                int32_t lhs_offset, int32_t rhs_offset, const Q8GemmEpilogue &ep,
-               int64_t rhs_ld = 0);   // rhs_ld != 0: ColMajor rhs whose columns are rhs_ld bytes
+               int64_t rhs_ld = 0,    // rhs_ld != 0: ColMajor rhs whose columns are rhs_ld bytes
                                       // apart (multiple of 16), bytes depth..rhs_ld-1 being 0x80
+               const Q8ConvGather *cv = nullptr);
 
 struct F32Epilogue {
   const float *bias_row;    // added per result row (NCHW channel), or nullptr

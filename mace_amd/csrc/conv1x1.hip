@@ -82,7 +82,7 @@ int conv_gemm(mace_hip_ctx *ctx, const uint8_t *filter, const uint8_t *rhs, int6
               const int32_t *bias, int64_t cout, int64_t depth, int64_t columns,
               float input_scale, int32_t input_zp, float filter_scale, int32_t filter_zp,
               float bias_scale, int32_t mult, int shift, int32_t out_zp, int clamp_min,
-              int clamp_max, uint8_t *out) {
+              int clamp_max, uint8_t *out, const Q8ConvGather *cv = nullptr) {
   // GetBiasData (mace/ops/arm/q8/quantization_util.cc:20-46)
   volatile float prod = input_scale * filter_scale;
   volatile float diff = prod - bias_scale;
@@ -100,7 +100,7 @@ int conv_gemm(mace_hip_ctx *ctx, const uint8_t *filter, const uint8_t *rhs, int6
   Q8GemmEpilogue ep{bias_used, mult, shift, out_zp, clamp_min, clamp_max};
   return mh_q8_gemm(ctx, filter, MACE_HIP_ROW_MAJOR, rhs, MACE_HIP_COL_MAJOR, out,
                     MACE_HIP_COL_MAJOR, true, 1, cout, depth, columns, 0, 0, -filter_zp,
-                    -input_zp, ep, rhs_ld);
+                    -input_zp, ep, rhs_ld, cv);
 }
 
 // scratch the GEMM takes from the arena for a [cout x depth] . [depth x columns] product
@@ -147,13 +147,25 @@ extern "C" int mace_hip_conv2d_q8_nhwc(mace_hip_ctx *ctx, const uint8_t *input,
   // still skips it and reads past the input; here a padded 1x1 takes the im2col path.)
   const bool in_place = k_h == 1 && k_w == 1 && stride_h == 1 && stride_w == 1 && pad_h == 0 &&
                         pad_w == 0;
+  // With cin a multiple of 64 (and at least three 64-byte slabs of depth) the GEMM's loader
+  // gathers the patches itself and no im2col matrix is written.
+  const bool gather = !in_place && cin % 64 == 0 && depth >= 192 && ((uintptr_t)input % 16 == 0) &&
+                      ((uintptr_t)filter % 16 == 0) && in_h * in_w * cin < (1ll << 31);
   const int64_t kp = (int64_t)mh_align_up((size_t)(depth > 0 ? depth : 1), 64);
-  size_t need = sizeof(int32_t) * cout + 4096 + conv_gemm_scratch(cout, depth, columns, !in_place || depth % 16 == 0);
-  if (!in_place) need += (size_t)columns * kp + 4096;
+  size_t need = sizeof(int32_t) * cout + 4096 +
+                conv_gemm_scratch(cout, depth, columns, !in_place || depth % 16 == 0);
+  if (!in_place && !gather) need += (size_t)columns * kp + 4096;
   MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, need));
   ArenaScope scope(ctx);
   const uint8_t *rhs = input;
   int64_t rhs_ld = 0;
+  if (gather) {
+    const Q8ConvGather cv{(int)in_h, (int)in_w, (int)cin, (int)k_h, (int)k_w, stride_h, stride_w,
+                          pad_h >> 1, pad_w >> 1, (int)out_h, (int)out_w, input_zp};
+    return conv_gemm(ctx, filter, input, 0, bias, cout, depth, columns, input_scale, input_zp,
+                     filter_scale, filter_zp, bias_scale, mult, shift, out_zp, clamp_min,
+                     clamp_max, out, &cv);
+  }
   if (!in_place) {
     uint8_t *cols = (uint8_t *)mh_arena_take(ctx, (size_t)columns * kp);
     if (!cols) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");

@@ -62,6 +62,11 @@ struct GemmParams {
   int32_t xcoef, xadd;
   const int32_t *xbias;
   int tiles_x, tiles_y;
+  // CONV kernels: Y rows are output pixels of a convolution gathered on the fly; Y is the NHWC
+  // input, row y = (image, oh, ow), k = (kh, kw, channel) with cin % 64 == 0
+  int cv_in_h, cv_in_w, cv_cin, cv_kw, cv_sh, cv_sw, cv_pt, cv_pl, cv_oh, cv_ow;
+  const uint8_t *cv_zero;   // >= 64 bytes holding the input zero point (padding positions)
+  bool conv;
 };
 
 // XCD-aware tile order: consecutive workgroup ids are dealt round-robin to the 8 XCDs, so
@@ -423,7 +428,7 @@ __device__ inline void wait_vmcnt() {
 }
 
 template <int WX, int WY, int FX, int FY, int STAGES, typename OutT, int OCC = 1,
-          bool SUMY = false>
+          bool SUMY = false, bool CONV = false>
 __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParams p, RequantTable) {
   constexpr int NW = WX * WY;
   constexpr int TX = WX * FX * 32;
@@ -460,18 +465,44 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
     const int kc = (lane & 3) ^ ((row >> 2) & 3);
     gx[j] = Xb + (int64_t)min(x0 + row, p.XN - 1) * p.ldx + kc * 16;
   }
+  // CONV: what the gather needs per row: top-left input position of the pixel's patch and the
+  // lane's chunk offset; gy[j] is the image base.  A 64-byte slab lies inside one filter tap
+  // (cin % 64 == 0), so the tap is the same for the whole wavefront.
+  int cv_ih0[CONV ? LY : 1], cv_iw0[CONV ? LY : 1], cv_kc[CONV ? LY : 1];
 #pragma unroll
   for (int j = 0; j < LY; ++j) {
     const int row = (j * NW + wave) * 16 + (lane >> 2);
     const int kc = (lane & 3) ^ ((row >> 2) & 3);
-    gy[j] = Yb + (int64_t)min(y0 + row, p.YN - 1) * p.ldy + kc * 16;
+    const int y = min(y0 + row, p.YN - 1);
+    if constexpr (CONV) {
+      const int ow = y % p.cv_ow, t = y / p.cv_ow;
+      const int oh = t % p.cv_oh, img = t / p.cv_oh;
+      cv_ih0[j] = oh * p.cv_sh - p.cv_pt;
+      cv_iw0[j] = ow * p.cv_sw - p.cv_pl;
+      cv_kc[j] = kc * 16;
+      gy[j] = Yb + (int64_t)img * p.cv_in_h * p.cv_in_w * p.cv_cin;
+    } else {
+      gy[j] = Yb + (int64_t)y * p.ldy + kc * 16;
+    }
   }
+  auto y_src = [&](int j, int k0) -> const uint8_t * {
+    if constexpr (CONV) {
+      const int tap = k0 / p.cv_cin, c0 = k0 - tap * p.cv_cin;   // wave-uniform
+      const int kh = tap / p.cv_kw, kw = tap - kh * p.cv_kw;
+      const int ih = cv_ih0[j] + kh, iw = cv_iw0[j] + kw;
+      const bool inside = (unsigned)ih < (unsigned)p.cv_in_h && (unsigned)iw < (unsigned)p.cv_in_w;
+      const uint8_t *src = gy[j] + ((int64_t)ih * p.cv_in_w + iw) * p.cv_cin + c0 + cv_kc[j];
+      return inside ? src : p.cv_zero + cv_kc[j];
+    } else {
+      return gy[j] + k0;
+    }
+  };
   auto issue_slab = [&](int stage, int k0) {
     uint8_t *sx = lds + stage * STAGE_BYTES + wave * 1024;
 #pragma unroll
     for (int j = 0; j < LX; ++j) dma_16B(gx[j] + k0, sx + j * NW * 1024);
 #pragma unroll
-    for (int j = 0; j < LY; ++j) dma_16B(gy[j] + k0, sx + Y_OFF + j * NW * 1024);
+    for (int j = 0; j < LY; ++j) dma_16B(y_src(j, k0), sx + Y_OFF + j * NW * 1024);
   };
 
   v16i acc[FX][FY];
@@ -553,7 +584,7 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
 #pragma unroll
         for (int d = m * PER_SLOT; d < (m + 1) * PER_SLOT; ++d) {
           if (d < LX) dma_16B(gx[d] + dk0, dsx + d * NW * 1024);
-          else if (d < LX + LY) dma_16B(gy[d - LX] + dk0, dsx + Y_OFF + (d - LX) * NW * 1024);
+          else if (d < LX + LY) dma_16B(y_src(d - LX, dk0), dsx + Y_OFF + (d - LX) * NW * 1024);
         }
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -968,7 +999,12 @@ int launch_gemm_dma(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, b
     hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, tab);
     return MACE_HIP_SUCCESS;
   };
-  if (out_u8 && p.sum_y) {
+  if (p.conv) {   // gathered convolution rows: always with in-kernel Y sums
+    if (out_u8)
+      MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, uint8_t, OCC, true, true>));
+    else
+      MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, int32_t, OCC, true, true>));
+  } else if (out_u8 && p.sum_y) {
     MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, uint8_t, OCC, true>));
   } else if (out_u8) {
     MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, uint8_t, OCC, false>));
@@ -1010,7 +1046,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
                int rhs_order, void *out, int out_order, bool out_u8, int64_t batch,
                int64_t rows, int64_t depth, int64_t cols, int lhs_batched, int rhs_batched,
                int32_t lhs_offset, int32_t rhs_offset, const Q8GemmEpilogue &ep,
-               int64_t rhs_ld) {
+               int64_t rhs_ld, const Q8ConvGather *cv) {
   MH_CHECK(ctx, batch >= 0 && rows >= 0 && depth >= 0 && cols >= 0, "negative dimension");
   MH_CHECK(ctx, (lhs_order | 1) == 1 && (rhs_order | 1) == 1 && (out_order | 1) == 1,
            "matrix order must be RowMajor (0) or ColMajor (1)");
@@ -1037,8 +1073,16 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   MH_CHECK(ctx, rhs_ld == 0 || (rhs_order == MACE_HIP_COL_MAJOR && rhs_ld >= depth &&
                                rhs_ld % 16 == 0 && depth > 0 && ((uintptr_t)rhs % 16 == 0)),
            "padded right-hand panel must be ColMajor, 16-byte aligned, pitch a multiple of 16");
-  const bool rhs_direct = rhs_ld != 0 || (rhs_order == MACE_HIP_COL_MAJOR && depth % 16 == 0 &&
-                                          depth > 0 && ((uintptr_t)rhs % 16 == 0));
+  // cv: the right operand is not a matrix in memory but the patches of a convolution, gathered by
+  // the streaming kernel's loader (the caller has checked the geometry, see Q8ConvGather)
+  MH_CHECK(ctx, !cv || (rhs_ld == 0 && batch == 1 && out_order == MACE_HIP_COL_MAJOR &&
+                        lhs_order == MACE_HIP_ROW_MAJOR && depth % SLAB == 0 && depth >= 3 * SLAB &&
+                        cv->cin % SLAB == 0 && ((uintptr_t)rhs % 16 == 0) &&
+                        ((uintptr_t)lhs % 16 == 0)),
+           "convolution gather needs cin % 64 == 0, depth >= 192 and 16-byte aligned tensors");
+  const bool rhs_direct = cv || rhs_ld != 0 ||
+                          (rhs_order == MACE_HIP_COL_MAJOR && depth % 16 == 0 && depth > 0 &&
+                           ((uintptr_t)rhs % 16 == 0));
 
   // operands registered as constant weights keep their panel and sums in the context
   auto find_weight = [&](const uint8_t *src, size_t bytes) -> mh_weight * {
@@ -1048,9 +1092,9 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     return nullptr;
   };
   mh_weight *lhs_w = find_weight(lhs, (size_t)lhs_nb * rows * depth);
-  mh_weight *rhs_w = rhs_ld != 0 ? nullptr : find_weight(rhs, (size_t)rhs_nb * cols * depth);
+  mh_weight *rhs_w = (rhs_ld != 0 || cv) ? nullptr : find_weight(rhs, (size_t)rhs_nb * cols * depth);
 
-  size_t need = sizeof(int32_t) * ((size_t)lhs_nb * rows + (size_t)rhs_nb * cols) + 4096;
+  size_t need = sizeof(int32_t) * ((size_t)lhs_nb * rows + (size_t)rhs_nb * cols) + 4096 + 512;
   if (!lhs_direct && !lhs_w) need += (size_t)lhs_nb * rows * kp + 256;
   if (!rhs_direct && !rhs_w) need += (size_t)rhs_nb * cols * kp + 256;
   MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, need));
@@ -1153,8 +1197,8 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   // holds, which saves one pass over that operand.  The pass costs YN * K bytes of HBM traffic,
   // the in-kernel sums about 7 % of the GEMM's own time (measured at 8192^3: +37 us against an
   // 11 us pass), i.e. the ratio grows with XN only: in-kernel wins below XN of about 2500.
-  const bool sum_y = depth > 0 && (depth <= 1024 || (x_is_lhs ? rows : cols) <= 2048) &&
-                     !(x_is_lhs ? R.sums : L.sums);   // cached sums cost nothing
+  const bool sum_y = cv || (depth > 0 && (depth <= 1024 || (x_is_lhs ? rows : cols) <= 2048) &&
+                            !(x_is_lhs ? R.sums : L.sums));   // cached sums cost nothing
   const int32_t l_coef = (int32_t)(0u - zr), l_add = 0;
   const int32_t r_coef = (int32_t)(0u - zl), r_add = (int32_t)((uint32_t)depth * zl * zr);
   const int32_t *l_bias = out_u8 ? ep.bias : nullptr;
@@ -1162,7 +1206,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   // long Y panel goes to the streaming kernel, which also sums both panels itself.
   const int64_t xn = x_is_lhs ? rows : cols, yn = x_is_lhs ? cols : rows;
   // (Measured: it wins for K <= 64; from K = 128 on the tiled kernels are as fast.)
-  const bool stream = out_u8 && rq.table && lhs_direct && rhs_direct &&
+  const bool stream = !cv && out_u8 && rq.table && lhs_direct && rhs_direct &&
                       (depth == 32 || depth == 64) && (xn == 32 || xn == 64 || xn == 128) &&
                       yn >= 1024 && ((uintptr_t)out % 16 == 0);
   const int32_t *sumL = L.sums ? L.sums : corrL, *sumR = R.sums ? R.sums : corrR;
@@ -1200,6 +1244,17 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   p.xadd = x_is_lhs ? l_add : r_add;
   p.xbias = x_is_lhs ? l_bias : nullptr;
   p.tiles_x = p.tiles_y = 0;
+  p.conv = cv != nullptr;
+  p.cv_zero = nullptr;
+  if (cv) {
+    p.cv_in_h = cv->in_h; p.cv_in_w = cv->in_w; p.cv_cin = cv->cin; p.cv_kw = cv->k_w;
+    p.cv_sh = cv->stride_h; p.cv_sw = cv->stride_w; p.cv_pt = cv->pad_top; p.cv_pl = cv->pad_left;
+    p.cv_oh = cv->out_h; p.cv_ow = cv->out_w;
+    uint8_t *zero = (uint8_t *)mh_arena_take(ctx, 256);
+    if (!zero) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
+    MH_HIP(ctx, hipMemsetAsync(zero, cv->zero_point, 256, ctx->stream));
+    p.cv_zero = zero;
+  }
   if (stream) {
     switch (p.XN) {
       case 32: return launch_gemm_stream<1, 1>(ctx, p, tab, (int)batch);

@@ -74,6 +74,9 @@ CASES = [  # batch, cout, cin, in_h, in_w, k_h, k_w, padding, strides: the refer
     (2, 32, 3, 64, 64, 3, 3, S, (2, 2)), (2, 64, 32, 17, 17, 1, 1, V, (2, 2)),
     (2, 5, 3, 6, 11, 2, 4, Fu, (1, 2)), (1, 1, 1, 1, 1, 1, 1, S, (1, 1)),
     (3, 40, 16, 9, 9, 3, 3, S, (1, 1)), (1, 64, 32, 56, 56, 3, 3, S, (1, 1)),
+    # channel counts that are multiples of 64: gathered by the GEMM's loader, every tile shape
+    (2, 256, 128, 28, 28, 3, 3, S, (1, 1)), (1, 300, 64, 20, 20, 3, 3, S, (1, 1)),
+    (1, 48, 192, 13, 17, 3, 3, Fu, (2, 1)), (4, 64, 64, 56, 56, 3, 3, S, (1, 1)),
 ]
 
 
