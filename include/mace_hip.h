@@ -252,7 +252,8 @@ int mace_hip_conv1x1_q8_nhwc(mace_hip_ctx *ctx, const uint8_t *input, const uint
  * TOTAL paddings per dimension as MACE passes them: pad >> 1 rows / columns go on the top / left
  * (conv_2d.cc:345-348), the rest on the bottom / right; padded positions hold the input zero
  * point (Im2col, conv_2d.cc:321-412).  A 1x1 filter at stride 1 without padding multiplies the
- * input in place; everything else is gathered into an im2col matrix in the context arena first.
+ * input in place; with cin % 64 == 0 the GEMM gathers the patches while loading; otherwise they
+ * are gathered into an im2col matrix in the context arena first.
  * INVALID_ARGS where the reference CHECK-fails (multiplier outside (0,1)) and for a filter larger
  * than the padded input. */
 int mace_hip_conv2d_q8_nhwc(mace_hip_ctx *ctx, const uint8_t *input, const uint8_t *filter,
