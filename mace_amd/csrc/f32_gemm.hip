@@ -95,20 +95,28 @@ __global__ __launch_bounds__(256) void f32_gemm_kernel(F32GemmParams p) {
   for (int kt = 0; kt < nk; ++kt) {
     const int buf = kt & 1;
     if (kt + 1 < nk) load_global((kt + 1) * TK);
+    // v_mfma_f32_32x32x2: lane l supplies A[row l % 32][k = l / 32], B[k = l / 32][col l % 32].
+    // The fragments of step ks + 1 are read while the MFMAs of step ks run (one wavefront per
+    // SIMD has nobody else to hide the LDS latency behind).
+    float a[2][2], bb[2][2];
+    auto read_frags = [&](int ks, int slot) {
+      const int kk = ks * 2 + (lane >> 5);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) a[slot][i] = sA[buf][kk][wm * 64 + i * 32 + (lane & 31)];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) bb[slot][j] = sB[buf][kk][wn * 64 + j * 32 + (lane & 31)];
+    };
+    read_frags(0, 0);
 #pragma unroll
     for (int ks = 0; ks < TK / 2; ++ks) {
-      // v_mfma_f32_32x32x2: lane l supplies A[row l % 32][k = l / 32], B[k = l / 32][col l % 32]
-      const int kk = ks * 2 + (lane >> 5);
-      float a[2], bb[2];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) a[i] = sA[buf][kk][wm * 64 + i * 32 + (lane & 31)];
-#pragma unroll
-      for (int j = 0; j < 2; ++j) bb[j] = sB[buf][kk][wn * 64 + j * 32 + (lane & 31)];
+      if (ks + 1 < TK / 2) read_frags(ks + 1, (ks + 1) & 1);
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], bb[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ks & 1][i], bb[ks & 1][j], acc[i][j],
+                                                           0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
     if (kt + 1 < nk) store_lds(buf ^ 1);
     __syncthreads();
@@ -145,6 +153,135 @@ __global__ void f32_fill_kernel(F32GemmParams p, int64_t total) {
     const int n = (int)(i - bm * p.N);
     p.out[bb * p.obs + (int64_t)m * p.ors + (int64_t)n * p.ocs] = apply_act(v, p.act, p.limit);
   }
+}
+
+// The same tile for matrices whose sizes are multiples of the tile (M, N % 128 == 0, K % 16 == 0)
+// and whose rows are 16-byte aligned: no bounds checks, 16-byte global loads through pointers
+// advanced once per k tile (the general kernel spends about 85 vector instructions per k tile on
+// guarded 4-byte loads and their addresses, in front of 32 MFMAs).
+typedef float f4v __attribute__((ext_vector_type(4)));
+
+template <bool LK, bool RK>
+__global__ __launch_bounds__(256) void f32_gemm_vec_kernel(F32GemmParams p) {
+  __shared__ __align__(16) float sA[2][TK][LDT];
+  __shared__ __align__(16) float sB[2][TK][LDT];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave & 1, wn = wave >> 1;
+  const int m0 = (blockIdx.x % p.tiles_m) * TM, n0 = (blockIdx.x / p.tiles_m) * TN;
+  const int b = blockIdx.z;
+  const float *A = p.lhs + (int64_t)b * p.lbs;
+  const float *B = p.rhs + (int64_t)b * p.rbs;
+
+  // two 16-byte pieces per operand per thread and k tile
+  const float *pa[2], *pb[2];
+  int sa_off[2], sb_off[2];   // float offset of the piece inside one LDS buffer
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int f = tid + i * 256;
+    if (LK) {   // 4 consecutive k of row m
+      const int m = f >> 2, k4 = f & 3;
+      pa[i] = A + (int64_t)(m0 + m) * p.lrs + 4 * k4;
+      sa_off[i] = (4 * k4) * LDT + m;
+    } else {    // 4 consecutive m of depth k
+      const int k = f >> 5, m4 = f & 31;
+      pa[i] = A + (int64_t)k * p.lcs + m0 + 4 * m4;
+      sa_off[i] = k * LDT + 4 * m4;
+    }
+    if (RK) {
+      const int n = f >> 2, k4 = f & 3;
+      pb[i] = B + (int64_t)(n0 + n) * p.rcs + 4 * k4;
+      sb_off[i] = (4 * k4) * LDT + n;
+    } else {
+      const int k = f >> 5, n4 = f & 31;
+      pb[i] = B + (int64_t)k * p.rrs + n0 + 4 * n4;
+      sb_off[i] = k * LDT + 4 * n4;
+    }
+  }
+  const int64_t a_step = LK ? TK : (int64_t)TK * p.lcs;
+  const int64_t b_step = RK ? TK : (int64_t)TK * p.rrs;
+  f4v ra[2], rb[2];
+  auto load_global = [&]() {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      ra[i] = *(const f4v *)pa[i];
+      rb[i] = *(const f4v *)pb[i];
+      pa[i] += a_step;
+      pb[i] += b_step;
+    }
+  };
+  auto store_lds = [&](int buf) {
+    float *a = &sA[buf][0][0], *bq = &sB[buf][0][0];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      if (LK) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) a[sa_off[i] + e * LDT] = ra[i][e];
+      } else {
+        *(f4v *)(a + sa_off[i]) = ra[i];
+      }
+      if (RK) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) bq[sb_off[i] + e * LDT] = rb[i][e];
+      } else {
+        *(f4v *)(bq + sb_off[i]) = rb[i];
+      }
+    }
+  };
+
+  v16f acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int nk = p.K / TK;
+  load_global();
+  store_lds(0);
+  __syncthreads();
+  for (int kt = 0; kt < nk; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < nk) load_global();
+    float a[2][2], bb[2][2];
+    auto read_frags = [&](int ks, int slot) {
+      const int kk = ks * 2 + (lane >> 5);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) a[slot][i] = sA[buf][kk][wm * 64 + i * 32 + (lane & 31)];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) bb[slot][j] = sB[buf][kk][wn * 64 + j * 32 + (lane & 31)];
+    };
+    read_frags(0, 0);
+#pragma unroll
+    for (int ks = 0; ks < TK / 2; ++ks) {
+      if (ks + 1 < TK / 2) read_frags(ks + 1, (ks + 1) & 1);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ks & 1][i], bb[ks & 1][j], acc[i][j],
+                                                           0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (kt + 1 < nk) store_lds(buf ^ 1);
+    __syncthreads();
+  }
+
+  float *O = p.out + (int64_t)b * p.obs;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int n = n0 + wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        float v = acc[i][j][r];
+        if (p.bias_row) v = v + p.bias_row[m];
+        v = apply_act(v, p.act, p.limit);
+        O[(int64_t)m * p.ors + (int64_t)n * p.ocs] = v;
+      }
+    }
 }
 
 struct F32GemvParams {
@@ -217,7 +354,13 @@ int mh_f32_gemm(mace_hip_ctx *ctx, const float *lhs, const float *rhs, int64_t b
   const bool lk = lhs_major == MACE_HIP_ROW_MAJOR;   // depth contiguous
   const bool rk = rhs_major == MACE_HIP_COL_MAJOR;
   MH_PROF_BEGIN(ctx);
-  if (lk && rk) hipLaunchKernelGGL((f32_gemm_kernel<true, true>), grid, block, 0, ctx->stream, p);
+  const bool vec = rows % TM == 0 && cols % TN == 0 && depth % TK == 0 &&
+                   ((uintptr_t)lhs % 16 == 0) && ((uintptr_t)rhs % 16 == 0);
+  if (vec && lk && rk) hipLaunchKernelGGL((f32_gemm_vec_kernel<true, true>), grid, block, 0, ctx->stream, p);
+  else if (vec && lk) hipLaunchKernelGGL((f32_gemm_vec_kernel<true, false>), grid, block, 0, ctx->stream, p);
+  else if (vec && rk) hipLaunchKernelGGL((f32_gemm_vec_kernel<false, true>), grid, block, 0, ctx->stream, p);
+  else if (vec) hipLaunchKernelGGL((f32_gemm_vec_kernel<false, false>), grid, block, 0, ctx->stream, p);
+  else if (lk && rk) hipLaunchKernelGGL((f32_gemm_kernel<true, true>), grid, block, 0, ctx->stream, p);
   else if (lk) hipLaunchKernelGGL((f32_gemm_kernel<true, false>), grid, block, 0, ctx->stream, p);
   else if (rk) hipLaunchKernelGGL((f32_gemm_kernel<false, true>), grid, block, 0, ctx->stream, p);
   else hipLaunchKernelGGL((f32_gemm_kernel<false, false>), grid, block, 0, ctx->stream, p);
