@@ -172,14 +172,15 @@ __global__ __launch_bounds__(256) void f32_gemm_vec_kernel(F32GemmParams p) {
   const float *A = p.lhs + (int64_t)b * p.lbs;
   const float *B = p.rhs + (int64_t)b * p.rbs;
 
-  // two 16-byte pieces per operand per thread and k tile
-  const float *pa[2], *pb[2];
-  int sa_off[2], sb_off[2];   // float offset of the piece inside one LDS buffer
+  // NP 16-byte pieces per operand per thread and k tile; KQ pieces along k per row
+  constexpr int NP = TM * TK / 4 / 256, KQ = TK / 4;
+  const float *pa[NP], *pb[NP];
+  int sa_off[NP], sb_off[NP];   // float offset of the piece inside one LDS buffer
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < NP; ++i) {
     const int f = tid + i * 256;
     if (LK) {   // 4 consecutive k of row m
-      const int m = f >> 2, k4 = f & 3;
+      const int m = f / KQ, k4 = f % KQ;
       pa[i] = A + (int64_t)(m0 + m) * p.lrs + 4 * k4;
       sa_off[i] = (4 * k4) * LDT + m;
     } else {    // 4 consecutive m of depth k
@@ -188,7 +189,7 @@ __global__ __launch_bounds__(256) void f32_gemm_vec_kernel(F32GemmParams p) {
       sa_off[i] = k * LDT + 4 * m4;
     }
     if (RK) {
-      const int n = f >> 2, k4 = f & 3;
+      const int n = f / KQ, k4 = f % KQ;
       pb[i] = B + (int64_t)(n0 + n) * p.rcs + 4 * k4;
       sb_off[i] = (4 * k4) * LDT + n;
     } else {
@@ -199,10 +200,10 @@ __global__ __launch_bounds__(256) void f32_gemm_vec_kernel(F32GemmParams p) {
   }
   const int64_t a_step = LK ? TK : (int64_t)TK * p.lcs;
   const int64_t b_step = RK ? TK : (int64_t)TK * p.rrs;
-  f4v ra[2], rb[2];
+  f4v ra[NP], rb[NP];
   auto load_global = [&]() {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < NP; ++i) {
       ra[i] = *(const f4v *)pa[i];
       rb[i] = *(const f4v *)pb[i];
       pa[i] += a_step;
@@ -212,7 +213,7 @@ __global__ __launch_bounds__(256) void f32_gemm_vec_kernel(F32GemmParams p) {
   auto store_lds = [&](int buf) {
     float *a = &sA[buf][0][0], *bq = &sB[buf][0][0];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < NP; ++i) {
       if (LK) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) a[sa_off[i] + e * LDT] = ra[i][e];
@@ -236,13 +237,17 @@ __global__ __launch_bounds__(256) void f32_gemm_vec_kernel(F32GemmParams p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
+  // Tile kt + 1 sits in registers while tile kt is multiplied (it was requested a whole
+  // iteration earlier); it goes to LDS, and the request for tile kt + 2 goes out, in the middle
+  // of the MFMA sequence, so that neither the LDS stores nor the load issue leave the matrix
+  // core idle.  The other LDS buffer is free then: everybody passed the last barrier.
   const int nk = p.K / TK;
   load_global();
   store_lds(0);
+  if (nk > 1) load_global();
   __syncthreads();
   for (int kt = 0; kt < nk; ++kt) {
     const int buf = kt & 1;
-    if (kt + 1 < nk) load_global();
     float a[2][2], bb[2][2];
     auto read_frags = [&](int ks, int slot) {
       const int kk = ks * 2 + (lane >> 5);
@@ -261,9 +266,12 @@ __global__ __launch_bounds__(256) void f32_gemm_vec_kernel(F32GemmParams p) {
         for (int j = 0; j < 2; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ks & 1][i], bb[ks & 1][j], acc[i][j],
                                                            0, 0, 0);
+      if (ks == TK / 4 - 1 && kt + 1 < nk) {
+        store_lds(buf ^ 1);
+        if (kt + 2 < nk) load_global();
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (kt + 1 < nk) store_lds(buf ^ 1);
     __syncthreads();
   }
 
