@@ -44,6 +44,10 @@ GEMM_CASES += [(3, 47, 69, 37, lm, rm, om, True, True)
 GEMM_CASES += [(3, 47, 69, 37, R, R, R, True, False), (3, 47, 69, 37, R, R, R, False, True),
                (16, 31, 61, 67, R, Cm, R, True, True), (2, 300, 257, 129, R, R, R, True, True),
                (1, 1, 5, 1, R, R, R, True, True), (2, 128, 128, 16, Cm, Cm, Cm, True, True)]
+# sizes that are multiples of the tile (the aligned kernel): every layout, one-sided batching
+GEMM_CASES += [(2, 256, 128, 48, lm, rm, om, True, True)
+               for lm in (R, Cm) for rm in (R, Cm) for om in (R, Cm)]
+GEMM_CASES += [(3, 128, 384, 80, Cm, R, R, False, True), (3, 384, 128, 16, R, Cm, Cm, True, False)]
 
 
 @pytest.mark.parametrize("batch,rows,cols,depth,lm,rm,om,lb,rb", GEMM_CASES)
