@@ -427,19 +427,35 @@ __device__ inline void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
 }
 
+// KB = bytes of k per slab.  64: a ring of STAGES >= 3 slabs; the transfer issued while slab kt
+// is multiplied goes into the stage slab kt-1 occupied.  128: rows are fetched as whole 128-byte
+// cache lines (with 64-byte slabs the two halves of a line are fetched one slab period apart,
+// and in the 256 x 256 tile the line has left the 32 KB L1 by then, which doubles the
+// L2 -> L1 traffic), and the transfer goes into the stage of slab kt itself, which every
+// wavefront has finished reading at the barrier inside slab kt; two stages then suffice.
 template <int WX, int WY, int FX, int FY, int STAGES, typename OutT, int OCC = 1,
-          bool SUMY = false, bool CONV = false>
+          bool SUMY = false, bool CONV = false, int KB = SLAB>
 __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParams p, RequantTable) {
   constexpr int NW = WX * WY;
   constexpr int TX = WX * FX * 32;
   constexpr int TY = WY * FY * 32;
-  constexpr int LX = TX / 16 / NW;   // DMA instructions per wavefront per slab, X tile
-  constexpr int LY = TY / 16 / NW;
-  static_assert(TX % (16 * NW) == 0 && TY % (16 * NW) == 0, "uneven slab load");
-  constexpr int STAGE_BYTES = (TX + TY) * SLAB;
-  constexpr int Y_OFF = TX * SLAB;
-  static_assert(STAGES >= 3 && STAGES <= 5, "ring depth");
-  static_assert((STAGES - 2) * (LX + LY) < 64, "too many loads in flight for vmcnt");
+  static_assert(KB == 64 || KB == 128, "slab width");
+  static_assert(!CONV || KB == 64, "the gather addresses one filter tap per 64-byte slab");
+  constexpr bool REUSE = KB == 128;  // refill the stage of the slab being multiplied
+  constexpr int RPI = 1024 / KB;     // rows per DMA instruction (64 lanes x 16 bytes)
+  constexpr int CPR = KB / 16;       // 16-byte chunks per row
+  constexpr int KSN = KB / 32;       // k steps per slab
+  constexpr int LX = TX / RPI / NW;  // DMA instructions per wavefront per slab, X tile
+  constexpr int LY = TY / RPI / NW;
+  static_assert(TX % (RPI * NW) == 0 && TY % (RPI * NW) == 0, "uneven slab load");
+  constexpr int STAGE_BYTES = (TX + TY) * KB;
+  constexpr int Y_OFF = TX * KB;
+  constexpr int AHEAD = REUSE ? STAGES : STAGES - 1;   // slabs in flight or landed beyond slab kt
+  static_assert(AHEAD >= 2 && STAGES <= 8, "ring depth");
+  static_assert((AHEAD - 1) * (LX + LY) < 64, "too many loads in flight for vmcnt");
+  // chunk c of row r is stored in slot c ^ swizzle(r): the rows a 16-lane group reads together
+  // then cover all banks (pitch 64: four rows per 256 bytes; pitch 128: two)
+  auto swizzle = [](int row) { return KB == 64 ? (row >> 2) & 3 : (row >> 1) & 7; };
 
   extern __shared__ __align__(16) uint8_t lds[];
 
@@ -455,24 +471,30 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
   const uint8_t *Xb = p.X + (int64_t)b * p.xbs;
   const uint8_t *Yb = p.Y + (int64_t)b * p.ybs;
 
-  // DMA source pointers: instruction j of this wavefront fills rows [(j*NW + wave)*16, +16) of
-  // the slab; lane l lands in row l/4, slot l%4 and therefore fetches chunk slot ^ swizzle(row)
-  const uint8_t *gx[LX];
-  const uint8_t *gy[LY];
+  // DMA source pointers: instruction j of this wavefront fills rows [(j*NW + wave)*RPI, +RPI)
+  // of the slab; lane l lands in row l/CPR, slot l%CPR and therefore fetches chunk
+  // slot ^ swizzle(row)
+  // Addresses are kept as 32-bit byte offsets from the first row of the tile (the host checks
+  // that 256 rows fit), so that the transfers take a wave-uniform base plus a lane offset.
+  const uint8_t *Xt = Xb + (int64_t)x0 * p.ldx;
+  const uint8_t *Yt = Yb + (int64_t)y0 * p.ldy;
+  uint32_t ox[LX], oy[CONV ? 1 : LY];
+  const uint8_t *gy[CONV ? LY : 1];
 #pragma unroll
   for (int j = 0; j < LX; ++j) {
-    const int row = (j * NW + wave) * 16 + (lane >> 2);
-    const int kc = (lane & 3) ^ ((row >> 2) & 3);
-    gx[j] = Xb + (int64_t)min(x0 + row, p.XN - 1) * p.ldx + kc * 16;
+    const int row = (j * NW + wave) * RPI + lane / CPR;
+    const int kc = (lane % CPR) ^ swizzle(row);
+    ox[j] = (uint32_t)(min(x0 + row, p.XN - 1) - x0) * (uint32_t)p.ldx + kc * 16;
   }
+  auto x_src = [&](int j, int k0) -> const uint8_t * { return Xt + k0 + ox[j]; };
   // CONV: what the gather needs per row: top-left input position of the pixel's patch and the
   // lane's chunk offset; gy[j] is the image base.  A 64-byte slab lies inside one filter tap
   // (cin % 64 == 0), so the tap is the same for the whole wavefront.
   int cv_ih0[CONV ? LY : 1], cv_iw0[CONV ? LY : 1], cv_kc[CONV ? LY : 1];
 #pragma unroll
   for (int j = 0; j < LY; ++j) {
-    const int row = (j * NW + wave) * 16 + (lane >> 2);
-    const int kc = (lane & 3) ^ ((row >> 2) & 3);
+    const int row = (j * NW + wave) * RPI + lane / CPR;
+    const int kc = (lane % CPR) ^ swizzle(row);
     const int y = min(y0 + row, p.YN - 1);
     if constexpr (CONV) {
       const int ow = y % p.cv_ow, t = y / p.cv_ow;
@@ -482,7 +504,7 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
       cv_kc[j] = kc * 16;
       gy[j] = Yb + (int64_t)img * p.cv_in_h * p.cv_in_w * p.cv_cin;
     } else {
-      gy[j] = Yb + (int64_t)y * p.ldy + kc * 16;
+      oy[j] = (uint32_t)(y - y0) * (uint32_t)p.ldy + kc * 16;
     }
   }
   auto y_src = [&](int j, int k0) -> const uint8_t * {
@@ -494,13 +516,13 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
       const uint8_t *src = gy[j] + ((int64_t)ih * p.cv_in_w + iw) * p.cv_cin + c0 + cv_kc[j];
       return inside ? src : p.cv_zero + cv_kc[j];
     } else {
-      return gy[j] + k0;
+      return Yt + k0 + oy[j];
     }
   };
   auto issue_slab = [&](int stage, int k0) {
     uint8_t *sx = lds + stage * STAGE_BYTES + wave * 1024;
 #pragma unroll
-    for (int j = 0; j < LX; ++j) dma_16B(gx[j] + k0, sx + j * NW * 1024);
+    for (int j = 0; j < LX; ++j) dma_16B(x_src(j, k0), sx + j * NW * 1024);
 #pragma unroll
     for (int j = 0; j < LY; ++j) dma_16B(y_src(j, k0), sx + Y_OFF + j * NW * 1024);
   };
@@ -519,20 +541,20 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
   // fragment addresses: lane l reads row (l % 32) of a 32-row block, chunk 2*ks + l/32.
   // Block bases are multiples of 32 rows, so the swizzle depends on l only.
   const int frow = lane & 31;
-  const int fsw = (frow >> 2) & 3;
-  int foff[2];
+  const int fsw = swizzle(frow);
+  int foff[KSN];
 #pragma unroll
-  for (int ks = 0; ks < 2; ++ks) foff[ks] = frow * SLAB + (((2 * ks + (lane >> 5)) ^ fsw) << 4);
-  const int fx_base = wx * FX * 32 * SLAB;
-  const int fy_base = Y_OFF + wy * FY * 32 * SLAB;
+  for (int ks = 0; ks < KSN; ++ks) foff[ks] = frow * KB + (((2 * ks + (lane >> 5)) ^ fsw) << 4);
+  const int fx_base = wx * FX * 32 * KB;
+  const int fy_base = Y_OFF + wy * FY * 32 * KB;
   const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
 
   auto read_frags = [&](int stage, int ks, v4i (&a)[FX], v4i (&bf)[FY]) {
     const uint8_t *s = lds + stage * STAGE_BYTES + foff[ks];
 #pragma unroll
-    for (int i = 0; i < FX; ++i) a[i] = *(const v4i *)(s + fx_base + i * 32 * SLAB);
+    for (int i = 0; i < FX; ++i) a[i] = *(const v4i *)(s + fx_base + i * 32 * KB);
 #pragma unroll
-    for (int j = 0; j < FY; ++j) bf[j] = *(const v4i *)(s + fy_base + j * 32 * SLAB);
+    for (int j = 0; j < FY; ++j) bf[j] = *(const v4i *)(s + fy_base + j * 32 * KB);
   };
   auto flip_frags = [&](v4i (&a)[FX], v4i (&bf)[FY]) {
 #pragma unroll
@@ -551,7 +573,7 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
   constexpr int DELAY = NM - NF > 0 ? NM - NF : 0;
   auto frag_ptr = [&](int stage, int ks, int f) -> const v4i * {
     const uint8_t *s = lds + stage * STAGE_BYTES + foff[ks];
-    return (const v4i *)(f < FX ? s + fx_base + f * 32 * SLAB : s + fy_base + (f - FX) * 32 * SLAB);
+    return (const v4i *)(f < FX ? s + fx_base + f * 32 * KB : s + fy_base + (f - FX) * 32 * KB);
   };
   auto k_step = [&](auto dma_tag, v4i (&ca)[FX], v4i (&cb)[FY], v4i (&na)[FX], v4i (&nb)[FY],
                     int nstage, int nks, int dstage, int dk0) {
@@ -583,7 +605,7 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
         constexpr int PER_SLOT = (LX + LY + NM - 1) / NM;
 #pragma unroll
         for (int d = m * PER_SLOT; d < (m + 1) * PER_SLOT; ++d) {
-          if (d < LX) dma_16B(gx[d] + dk0, dsx + d * NW * 1024);
+          if (d < LX) dma_16B(x_src(d, dk0), dsx + d * NW * 1024);
           else if (d < LX + LY) dma_16B(y_src(d - LX, dk0), dsx + Y_OFF + (d - LX) * NW * 1024);
         }
       }
@@ -598,12 +620,12 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
       }
   };
 
-  const int nslab = p.K / SLAB;
-  // prologue: slabs 0 .. STAGES-2 in flight
+  const int nslab = p.K / KB;
+  // prologue: slabs 0 .. AHEAD-1 in flight
 #pragma unroll
-  for (int s = 0; s < STAGES - 1; ++s) issue_slab(s, s * SLAB);
-  wait_vmcnt<(STAGES - 2) * (LX + LY)>();   // slab 0 of this wavefront has landed
-  __builtin_amdgcn_s_barrier();             // ... and everybody else's part of it
+  for (int s = 0; s < AHEAD; ++s) issue_slab(s, s * KB);
+  wait_vmcnt<(AHEAD - 1) * (LX + LY)>();   // slab 0 of this wavefront has landed
+  __builtin_amdgcn_s_barrier();            // ... and everybody else's part of it
   asm volatile("" ::: "memory");
 
   v4i a0[FX], b0[FY], a1[FX], b1[FY];
@@ -611,26 +633,30 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
   flip_frags(a0, b0);
   int stage = 0;
   for (int kt = 0; kt < nslab; ++kt) {
-    // first half of slab kt; fetches its second half
+    // all k steps of slab kt but the last; each fetches the fragments of the one after it
     k_step(std::false_type{}, a0, b0, a1, b1, stage, 1, 0, 0);
-    // Slab kt+1 must be complete, and every wavefront must be done with slab kt-1 (whose
-    // stage the next DMA overwrites), before going on: one barrier covers both.
-    // Slabs 0 .. kt+STAGES-2 have been issued so far; those after slab kt+1 may stay in flight.
-    // Slabs up to kt+STAGES-2 have been issued (past the end: repeats of the last slab, see
-    // below), so exactly STAGES-3 slabs newer than kt+1 may stay in flight.
-    wait_vmcnt<(STAGES - 3) * (LX + LY)>();
+    if constexpr (KSN == 4) {
+      k_step(std::false_type{}, a1, b1, a0, b0, stage, 2, 0, 0);
+      k_step(std::false_type{}, a0, b0, a1, b1, stage, 3, 0, 0);
+    }
+    // Slab kt+1 must be complete, and every wavefront must be done reading the stage the next
+    // DMA overwrites (that of slab kt-1, or with REUSE that of slab kt, whose last fragments
+    // were fetched in the k step above), before going on: one barrier covers both.
+    // Slabs up to kt+AHEAD-1 have been issued (past the end: repeats of the last slab, see
+    // below), so exactly AHEAD-2 slabs newer than kt+1 may stay in flight.
+    wait_vmcnt<(AHEAD - 2) * (LX + LY)>();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     int next = stage + 1;
     if (next == STAGES) next = 0;
-    int dst = stage + STAGES - 1;
+    int dst = REUSE ? stage : stage + STAGES - 1;
     if (dst >= STAGES) dst -= STAGES;
-    // Second half of slab kt; fetches the first half of slab kt+1 and feeds the ring with slab
-    // kt+STAGES-1.  Near the end there is no such slab: the last one is fetched again into a
-    // stage nobody reads any more, which keeps the loop free of branches and the in-flight
+    // Last k step of slab kt; fetches the first fragments of slab kt+1 and feeds the ring with
+    // slab kt+AHEAD.  Near the end there is no such slab: the last one is fetched again into
+    // a stage nobody reads any more, which keeps the loop free of branches and the in-flight
     // count constant; likewise the fragments fetched after the last slab are never used.
-    const int ks = min(kt + STAGES - 1, nslab - 1);
-    k_step(std::true_type{}, a1, b1, a0, b0, next, 0, dst, ks * SLAB);
+    const int ks = min(kt + AHEAD, nslab - 1);
+    k_step(std::true_type{}, a1, b1, a0, b0, next, 0, dst, ks * KB);
     stage = next;
   }
 
@@ -983,13 +1009,13 @@ int launch_gemm(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, bool 
 }
 
 // the streaming kernel; the caller has checked K % 64 == 0 and K >= 64 * (STAGES - 1)
-template <int WX, int WY, int FX, int FY, int STAGES, int OCC>
+template <int WX, int WY, int FX, int FY, int STAGES, int OCC, int KB = SLAB>
 int launch_gemm_dma(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, bool out_u8,
                     int batch) {
   constexpr int TX = WX * FX * 32, TY = WY * FY * 32;
   p.tiles_x = (p.XN + TX - 1) / TX;
   p.tiles_y = (p.YN + TY - 1) / TY;
-  const size_t lds = (size_t)STAGES * (TX + TY) * SLAB;
+  const size_t lds = (size_t)STAGES * (TX + TY) * KB;
   dim3 grid(p.tiles_x * p.tiles_y, 1, batch), block(WX * WY * 64);
   auto launch = [&](auto k) -> int {
     if (lds > 64 * 1024)
@@ -999,19 +1025,27 @@ int launch_gemm_dma(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, b
     hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, tab);
     return MACE_HIP_SUCCESS;
   };
-  if (p.conv) {   // gathered convolution rows: always with in-kernel Y sums
-    if (out_u8)
-      MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, uint8_t, OCC, true, true>));
-    else
-      MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, int32_t, OCC, true, true>));
-  } else if (out_u8 && p.sum_y) {
-    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, uint8_t, OCC, true>));
+  if constexpr (KB == SLAB) {
+    if (p.conv) {   // gathered convolution rows: always with in-kernel Y sums
+      if (out_u8)
+        MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, uint8_t, OCC, true, true>));
+      else
+        MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, int32_t, OCC, true, true>));
+      MH_PROF_END(ctx);
+      MH_HIP(ctx, hipGetLastError());
+      return MACE_HIP_SUCCESS;
+    }
+  } else if (p.conv) {
+    return MACE_HIP_INVALID_ARGS;   // not dispatched: the gather works on 64-byte slabs
+  }
+  if (out_u8 && p.sum_y) {
+    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, uint8_t, OCC, true, false, KB>));
   } else if (out_u8) {
-    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, uint8_t, OCC, false>));
+    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, uint8_t, OCC, false, false, KB>));
   } else if (p.sum_y) {
-    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, int32_t, OCC, true>));
+    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, int32_t, OCC, true, false, KB>));
   } else {
-    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, int32_t, OCC, false>));
+    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, int32_t, OCC, false, false, KB>));
   }
   MH_PROF_END(ctx);
   MH_HIP(ctx, hipGetLastError());
@@ -1287,11 +1321,20 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   // the streaming kernel needs whole 64-byte slabs and enough of them to fill its ring
   // K = 128 is two slabs: a three-stage ring holds all of it (10 % faster than the
   // register-staged kernel on the 56x56x128 convolution)
-  if (p.K == 2 * SLAB && !p.conv) {
+  // the DMA kernels address a tile's rows with 32-bit offsets from its first row
+  const bool dma_ok = p.ldx < (1 << 24) && p.ldy < (1 << 24);
+  if (p.K == 2 * SLAB && !p.conv && dma_ok) {
     if (skinny) return launch_gemm_dma<1, 4, 2, 2, 3, 2>(ctx, p, tab, out_u8, (int)batch);
     if (big || medium) return launch_gemm_dma<2, 2, 2, 2, 3, 3>(ctx, p, tab, out_u8, (int)batch);
   }
-  if (p.K % SLAB == 0 && p.K >= SLAB * 3) {
+  // 128-byte slabs (whole cache lines per row) where they measure faster: the 256 x 256 tile
+  // (+5 % at 8192^3) and long-k 128 x 128 tiles; short k gains nothing from them
+  if (p.K % 128 == 0 && p.K >= 256 && !p.conv && dma_ok) {
+    if (big) return launch_gemm_dma<2, 2, 4, 4, 2, 1, 128>(ctx, p, tab, out_u8, (int)batch);
+    if (medium && p.K >= 1024)
+      return launch_gemm_dma<2, 2, 2, 2, 2, 2, 128>(ctx, p, tab, out_u8, (int)batch);
+  }
+  if (p.K % SLAB == 0 && p.K >= SLAB * 3 && dma_ok) {
     if (big) return launch_gemm_dma<2, 2, 4, 4, 4, 1>(ctx, p, tab, out_u8, (int)batch);
     if (skinny) return launch_gemm_dma<1, 4, 2, 2, 4, 2>(ctx, p, tab, out_u8, (int)batch);
     if (medium) return launch_gemm_dma<2, 2, 2, 2, 4, 2>(ctx, p, tab, out_u8, (int)batch);
