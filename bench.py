@@ -34,7 +34,7 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, published
 # Bytes that crossed the L2 <-> fabric boundary per launch of the dominant kernel, from rocprofv3
 # FETCH_SIZE / WRITE_SIZE runs of this benchmark scaled by the same counters' reading for a plain
 # 256 MiB copy (x2.0 and x1.0).  Keyed by M = N = K; a profiler run is needed to refresh them.
-GEMM_TRAFFIC_BYTES = {8192: 8.76e8}
+GEMM_TRAFFIC_BYTES = {8192: 8.80e8}
 GEMV_TRAFFIC_BYTES = {1: 1.69e7, 8: 1.73e7}
 
 
@@ -152,7 +152,7 @@ def main():
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_INT8_TOPS,
                      "unit": "TOP/s", "frac": round(achieved / PEAK_INT8_TOPS, 4),
                      "traffic": GEMM_TRAFFIC_BYTES.get(n), "traffic_unit": "B/launch",
-                     "kernel": "q8_gemm_dma_kernel<2,2,4,4,4,uint8_t>",
+                     "kernel": "q8_gemm_dma_kernel<2,2,4,4,2,uint8_t,1,false,false,128>",
                      "kernel_ms_avg": round(k_avg, 4), "kernel_ms_min": round(min(kms), 4),
                      "ops_per_launch": ops},
     }
@@ -192,6 +192,32 @@ def main():
             log("dominant kernel on %s operands: %.3f ms -> %.0f TOPS" % (name, k2, stats[-1]["TOPS"]))
             del A2, B2
         result["roofline"]["other_operand_statistics"] = stats
+        # For scale: the vendor library's int8 GEMM (hipBLASLt behind torch._int_mm) on the same
+        # shape, operand layout and uniform-random data.  It takes signed bytes and stores raw
+        # int32 (no zero points, no requantization), so it is a yardstick for what the board
+        # sustains on this shape, not an alternative path.
+        try:
+            A3 = torch.randint(-128, 128, (n, n), dtype=torch.int8, device="cuda", generator=g)
+            B3 = torch.randint(-128, 128, (n, n), dtype=torch.int8, device="cuda", generator=g)
+            Bv = B3.t() if rhs_order == mh.COL_MAJOR else B3     # [k][n] view of the same layout
+            for _ in range(3):
+                torch._int_mm(A3, Bv)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            for _ in range(10):
+                torch._int_mm(A3, Bv)
+            e1.record()
+            torch.cuda.synchronize()
+            lib_ms = e0.elapsed_time(e1) / 10
+            result["roofline"]["vendor_library_same_shape"] = {
+                "what": "torch._int_mm (hipBLASLt), int8 x int8 -> int32", "ms": round(lib_ms, 4),
+                "TOPS": round(ops / (lib_ms * 1e-3) / 1e12, 1),
+                "frac": round(ops / (lib_ms * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4)}
+            log("vendor library int8 GEMM, same shape: %.3f ms -> %.0f TOPS" % (lib_ms, ops / (lib_ms * 1e-3) / 1e12))
+            del A3, B3
+        except Exception as ex:   # informational only
+            log("vendor library comparison skipped: %s" % str(ex)[:120])
         step()          # out8 again holds the uniform-random result (checked by cpu_baseline)
         ctx.sync()
 
