@@ -218,6 +218,30 @@ def main():
             del A3, B3
         except Exception as ex:   # informational only
             log("vendor library comparison skipped: %s" % str(ex)[:120])
+        # What the matrix cores sustain with nothing else running (operands never leave the
+        # registers): constant bytes, then random bytes.  The second figure is the power-limited
+        # ceiling for an int8 GEMM on random operands on this board.
+        try:
+            import ctypes
+            probe = ctypes.CDLL(os.path.join(os.path.dirname(os.path.abspath(__file__)),
+                                             "mace_amd", "libmace_probe.so"))
+            probe.mace_probe_mfma_i8.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                 ctypes.POINTER(ctypes.c_double)]
+            ceil = {}
+            for name, rnd in (("constant_operands", 0), ("random_operands", 1)):
+                tops = ctypes.c_double(0.0)
+                rc = probe.mace_probe_mfma_i8(rnd, cus, 16384, ctypes.byref(tops))
+                if rc != 0:
+                    raise RuntimeError("probe returned %d" % rc)
+                ceil[name + "_TOPS"] = round(tops.value, 1)
+            ceil["achieved_over_random_ceiling"] = round(achieved / ceil["random_operands_TOPS"], 4)
+            ceil["what"] = ("v_mfma_i32_32x32x32_i8 alone, 16 accumulators per wavefront, one "
+                            "workgroup of 4 wavefronts per CU, no LDS or memory traffic")
+            result["roofline"]["mfma_only_probe"] = ceil
+            log("pure MFMA loop: %.0f TOPS on constant, %.0f TOPS on random operands" %
+                (ceil["constant_operands_TOPS"], ceil["random_operands_TOPS"]))
+        except Exception as ex:   # informational only
+            log("MFMA probe skipped: %s" % str(ex)[:120])
         step()          # out8 again holds the uniform-random result (checked by cpu_baseline)
         ctx.sync()
 
