@@ -203,6 +203,43 @@ def test_q8_gemm_large_device_pointers(ctx, n, lo, ro, oo):
     assert sat < 0.5, sat
 
 
+@pytest.mark.parametrize("batch,rows,depth,cols,lo,ro,oo,with_bias", [
+    (1, 3100, 384, 3300, R, Cm, R, True),     # 256 x 256 tiles, 128-byte slabs, ragged last tiles
+    (1, 3100, 256, 3300, R, Cm, Cm, False),   # ... shortest k that kernel takes (two slabs)
+    (2, 2100, 640, 2200, R, Cm, R, True),     # ... batched
+    (1, 1100, 1024, 1300, R, Cm, R, True),    # 128 x 128 tiles, 128-byte slabs
+    (1, 1100, 1152, 1300, R, R, Cm, False),   # ... through the repack, column-major result
+    (1, 2049, 448, 2305, R, Cm, R, True),     # 128 x 128 tiles, 64-byte slabs (k % 128 != 0)
+])
+def test_q8_gemm_ragged_tiled(ctx, batch, rows, depth, cols, lo, ro, oo, with_bias):
+    """Shapes large enough for the 256 x 256 and 128 x 128 tile kernels whose sides are not
+    multiples of the tile: every edge workgroup clamps its loads and masks its stores.  Both
+    outputs compared in full with the oracle."""
+    rng = np.random.default_rng(rows + depth + cols + batch)
+    A = rng.integers(0, 256, (batch, rows, depth), dtype=np.uint8)
+    B = rng.integers(0, 256, (batch, depth, cols), dtype=np.uint8)
+    za, zb, zc = int(rng.integers(120, 137)), int(rng.integers(120, 137)), int(rng.integers(100, 157))
+    l, r = as_major(A, lo), as_major(B, ro)
+    bias = rng.integers(-2 ** 14, 2 ** 14, rows).astype(np.int32) if with_bias else None
+    d = Dev()
+    dl, dr = d.put(l), d.put(r)
+    db = d.put(bias) if with_bias else None
+    t32, p32 = d.empty(batch * rows * cols, np.int32)
+    t8, p8 = d.empty(batch * rows * cols, np.uint8)
+    d.sync()
+    ctx.call("mace_hip_gemm_q8_i32", dl, lo, dr, ro, p32, oo, batch, rows, depth, cols, 1, 1, -za, -zb)
+    mult, shift = scales_for(depth)
+    ctx.call("mace_hip_gemm_q8_u8", dl, lo, dr, ro, p8, oo, batch, rows, depth, cols, 1, 1, -za, -zb,
+             db, mult, shift, zc, 0, 255)
+    ctx.sync()
+    want32 = orc.q8_gemm_i32(l, r, batch, rows, cols, depth, -za, -zb, lo, ro, oo)
+    np.testing.assert_array_equal(t32.cpu().numpy().reshape(want32.shape), want32)
+    want8 = orc.output_pipeline_u8(want32, batch, rows, cols, oo, bias, mult, shift, zc)
+    np.testing.assert_array_equal(t8.cpu().numpy().reshape(want8.shape), want8)
+    sat = (want8 == 0).mean() + (want8 == 255).mean()
+    assert sat < 0.5, sat
+
+
 def test_q8_gemm_batched_512(ctx):
     """BASELINE config 5's batched case in full: 32 x 512^3, int32 accumulators and uint8 output."""
     rng = np.random.default_rng(9)
