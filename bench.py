@@ -45,8 +45,10 @@ def log(*a):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--settle-ms", type=float, default=150.0,
+                    help="untimed run-in before the warm-up, until the board's clocks have settled")
     ap.add_argument("--size", type=int, default=8192, help="M = N = K of the uint8 GEMM")
     ap.add_argument("--rhs-order", choices=["row", "col"], default="row",
                     help="row = MatMul default; col = transpose_b (B is read in place, no repack)")
@@ -107,8 +109,28 @@ def main():
                  out8.data_ptr(), mh.ROW_MAJOR, 1, n, n, n, 1, 1, -za, -zb, None, mult, shift, zc,
                  0, 255)
 
+    # Bring the board to its sustained clocks first: after idling, the first ~3 launches run at
+    # boost, the next ~50 are throttled hard (the kernel takes up to 30 % longer) and only then
+    # does the power controller settle.  Untimed, like the warm-up; the timed region is exactly
+    # `steps` back-to-back steps.
+    settle_steps = 0
+    if args.settle_ms > 0:
+        for _ in range(3):
+            step()
+        ctx.sync()
+        ctx.timer_start()
+        for _ in range(5):
+            step()
+        est = max(ctx.timer_stop() / 5, 1e-3)
+        settle_steps = int(args.settle_ms / est) + 1
+        for _ in range(settle_steps):
+            step()
     for _ in range(args.warmup):
         step()
+    # The dominant kernel is timed inside the timed region itself: the library records a pair of
+    # HIP events around it on its stream (no waiting in between) and the durations are read
+    # after the last step.
+    ctx.profile(True)
     ctx.sync()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -119,28 +141,24 @@ def main():
     ctx.sync()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
+    ctx.profile(False)
+    kms = ctx.kernel_ms_list()
+    assert len(kms) == min(args.steps, 512), (len(kms), args.steps)
     ms_per_step = wall_ms / args.steps
     ops = 2.0 * n * n * n
     value = ops / (ms_per_step * 1e-3) / 1e12
     log("whole path: %.3f ms/step wall (%.3f ms by events) -> %.1f TOPS"
         % (ms_per_step, ev_ms / args.steps, value))
-
-    # dominant kernel alone, HIP events on the launch stream around that kernel
-    ctx.profile(True)
-    kms = []
-    for _ in range(args.steps):
-        step()
-        kms.append(ctx.last_kernel_ms())
-    ctx.profile(False)
     k_avg = sum(kms) / len(kms)
     achieved = ops / (k_avg * 1e-3) / 1e12
-    log("dominant kernel: avg %.3f ms (min %.3f) -> %.1f TOPS = %.1f%% of %.0f"
-        % (k_avg, min(kms), achieved, 100 * achieved / PEAK_INT8_TOPS, PEAK_INT8_TOPS))
+    log("dominant kernel: avg %.3f ms (min %.3f, max %.3f) -> %.1f TOPS = %.1f%% of %.0f"
+        % (k_avg, min(kms), max(kms), achieved, 100 * achieved / PEAK_INT8_TOPS, PEAK_INT8_TOPS))
     sat = float(((out8 == 0) | (out8 == 255)).float().mean().item())
 
     result = {
         "metric": METRIC, "value": round(value, 2), "unit": "TOPS", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "steps": args.steps, "warmup": args.warmup, "settle_steps": settle_steps,
+        "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8",
         "data": "synthetic",
         "config": {"workload": "q8_matmul_%dx%dx%d_u8out" % (n, n, n), "M": n, "N": n, "K": n,
@@ -154,15 +172,16 @@ def main():
                      "traffic": GEMM_TRAFFIC_BYTES.get(n), "traffic_unit": "B/launch",
                      "kernel": "q8_gemm_dma_kernel<2,2,4,4,2,uint8_t,1,false,false,128>",
                      "kernel_ms_avg": round(k_avg, 4), "kernel_ms_min": round(min(kms), 4),
+                     "kernel_ms_max": round(max(kms), 4),
+                     "timing": "one HIP event pair per launch, recorded inside the timed region",
                      "ops_per_launch": ops},
     }
 
     # The same step with B registered as a constant weight (the inference case: its repacked
     # panel and column sums are kept across calls).  Reported beside `value`, never as it.
     ctx.call("mace_hip_weight_register", B.data_ptr(), n * n)
-    for _ in range(max(2, args.warmup)):
+    for _ in range(max(2, args.warmup) + settle_steps):
         step()
-    ctx.sync()
     ctx.timer_start()
     for _ in range(args.steps):
         step()
@@ -200,16 +219,15 @@ def main():
             A3 = torch.randint(-128, 128, (n, n), dtype=torch.int8, device="cuda", generator=g)
             B3 = torch.randint(-128, 128, (n, n), dtype=torch.int8, device="cuda", generator=g)
             Bv = B3.t() if rhs_order == mh.COL_MAJOR else B3     # [k][n] view of the same layout
-            for _ in range(3):
+            for _ in range(3 + settle_steps):      # same run-in as our own step
                 torch._int_mm(A3, Bv)
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            torch.cuda.synchronize()
             e0.record()
-            for _ in range(10):
+            for _ in range(args.steps):
                 torch._int_mm(A3, Bv)
             e1.record()
             torch.cuda.synchronize()
-            lib_ms = e0.elapsed_time(e1) / 10
+            lib_ms = e0.elapsed_time(e1) / args.steps
             result["roofline"]["vendor_library_same_shape"] = {
                 "what": "torch._int_mm (hipBLASLt), int8 x int8 -> int32", "ms": round(lib_ms, 4),
                 "TOPS": round(ops / (lib_ms * 1e-3) / 1e12, 1),

@@ -69,9 +69,14 @@ int mace_hip_timer_stop(mace_hip_ctx *ctx, float *elapsed_ms);
 /* Dominant-kernel stopwatch (the counterpart of the per-op timing SerialNet::Run records into
  * RunMetadata, mace/core/net/serial_net.cc:122-168): while enabled, every GEMM / Gemv call
  * brackets its main kernel (not the repack or correction-vector passes) with HIP events on
- * the context's stream; last_kernel_ms waits for that kernel and returns its duration. */
+ * the context's stream; last_kernel_ms waits for that kernel and returns its duration.
+ * Enabling resets the count of timed launches; kernel_ms(i) returns the duration of the i-th
+ * timed launch since then (the most recent 512 are kept), so a run of calls can be timed
+ * without waiting between them. */
 int mace_hip_profile_enable(mace_hip_ctx *ctx, int on);
 int mace_hip_profile_last_kernel_ms(mace_hip_ctx *ctx, float *elapsed_ms);
+int mace_hip_profile_kernel_count(mace_hip_ctx *ctx, int *count);
+int mace_hip_profile_kernel_ms(mace_hip_ctx *ctx, int index, float *elapsed_ms);
 /* Test hook, the counterpart of MACE_RUNTIME_FAILURE_RATIO
  * (mace/core/runtime_failure_mock.cc:24-48): the next n arena allocations fail. */
 int mace_hip_ctx_fail_next_allocs(mace_hip_ctx *ctx, int n);

@@ -43,9 +43,11 @@ struct mace_hip_ctx {
   hipStream_t own_stream = nullptr;
   hipStream_t stream = nullptr;     // own_stream or a borrowed one
   hipEvent_t ev_start = nullptr, ev_stop = nullptr;
-  hipEvent_t ev_k0 = nullptr, ev_k1 = nullptr;   // dominant-kernel stopwatch
+  // dominant-kernel stopwatch: a ring of event pairs, one pair per timed launch, so that a run
+  // of launches can be timed without waiting for any of them in between
+  std::vector<hipEvent_t> prof_ev;   // 2 * MH_PROF_RING events, created when first enabled
   int prof_on = 0;
-  int prof_valid = 0;
+  int prof_count = 0;                // launches timed since profiling was enabled
   // grow-only device arena; offsets handed out per call by ArenaScope
   char *arena = nullptr;
   size_t arena_bytes = 0;
@@ -88,16 +90,20 @@ int mh_fail(mace_hip_ctx *ctx, int code, const char *fmt, ...);
   } while (0)
 
 // Brackets a kernel launch with the dominant-kernel stopwatch when profiling is enabled.
-#define MH_PROF_BEGIN(ctx)                                                           \
-  do {                                                                               \
-    if ((ctx)->prof_on) MH_HIP((ctx), hipEventRecord((ctx)->ev_k0, (ctx)->stream));  \
+#define MH_PROF_RING 512
+#define MH_PROF_BEGIN(ctx)                                                                       \
+  do {                                                                                           \
+    if ((ctx)->prof_on)                                                                          \
+      MH_HIP((ctx), hipEventRecord((ctx)->prof_ev[2 * ((ctx)->prof_count % MH_PROF_RING)],       \
+                                   (ctx)->stream));                                              \
   } while (0)
-#define MH_PROF_END(ctx)                                                             \
-  do {                                                                               \
-    if ((ctx)->prof_on) {                                                            \
-      MH_HIP((ctx), hipEventRecord((ctx)->ev_k1, (ctx)->stream));                    \
-      (ctx)->prof_valid = 1;                                                         \
-    }                                                                                \
+#define MH_PROF_END(ctx)                                                                         \
+  do {                                                                                           \
+    if ((ctx)->prof_on) {                                                                        \
+      MH_HIP((ctx), hipEventRecord((ctx)->prof_ev[2 * ((ctx)->prof_count % MH_PROF_RING) + 1],   \
+                                   (ctx)->stream));                                              \
+      (ctx)->prof_count++;                                                                       \
+    }                                                                                            \
   } while (0)
 
 // Arena: every call that needs scratch opens a scope, takes aligned slices and lets the

@@ -71,8 +71,7 @@ int mace_hip_ctx_create(int device, mace_hip_ctx **out) {
   if (hipSetDevice(device) != hipSuccess || hipGetDeviceProperties(&prop, device) != hipSuccess ||
       hipStreamCreate(&ctx->own_stream) != hipSuccess ||
       hipEventCreate(&ctx->ev_start) != hipSuccess ||
-      hipEventCreate(&ctx->ev_stop) != hipSuccess ||
-      hipEventCreate(&ctx->ev_k0) != hipSuccess || hipEventCreate(&ctx->ev_k1) != hipSuccess) {
+      hipEventCreate(&ctx->ev_stop) != hipSuccess) {
     (void)hipGetLastError();
     delete ctx;
     return MACE_HIP_RUNTIME_ERROR;
@@ -101,8 +100,7 @@ int mace_hip_ctx_destroy(mace_hip_ctx *ctx) {
   for (mh_weight &w : ctx->weights) mh_weight_drop_panels(&w);
   (void)hipEventDestroy(ctx->ev_start);
   (void)hipEventDestroy(ctx->ev_stop);
-  (void)hipEventDestroy(ctx->ev_k0);
-  (void)hipEventDestroy(ctx->ev_k1);
+  for (hipEvent_t e : ctx->prof_ev) (void)hipEventDestroy(e);
   (void)hipStreamDestroy(ctx->own_stream);
   delete ctx;
   return MACE_HIP_SUCCESS;
@@ -181,17 +179,41 @@ int mace_hip_timer_stop(mace_hip_ctx *ctx, float *elapsed_ms) {
 
 int mace_hip_profile_enable(mace_hip_ctx *ctx, int on) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  if (on && ctx->prof_ev.empty()) {
+    ctx->prof_ev.reserve(2 * MH_PROF_RING);
+    for (int i = 0; i < 2 * MH_PROF_RING; ++i) {
+      hipEvent_t e = nullptr;
+      MH_HIP(ctx, hipEventCreate(&e));
+      ctx->prof_ev.push_back(e);
+    }
+  }
   ctx->prof_on = on ? 1 : 0;
-  ctx->prof_valid = 0;
+  if (on) ctx->prof_count = 0;   // switching off keeps the recorded launches readable
+  return MACE_HIP_SUCCESS;
+}
+
+int mace_hip_profile_kernel_count(mace_hip_ctx *ctx, int *count) {
+  if (!ctx || !count) return MACE_HIP_INVALID_ARGS;
+  *count = ctx->prof_count;
+  return MACE_HIP_SUCCESS;
+}
+
+int mace_hip_profile_kernel_ms(mace_hip_ctx *ctx, int index, float *elapsed_ms) {
+  if (!ctx || !elapsed_ms) return MACE_HIP_INVALID_ARGS;
+  MH_CHECK(ctx, index >= 0 && index < ctx->prof_count,
+           "no timed launch with this index since profiling was enabled");
+  MH_CHECK(ctx, index >= ctx->prof_count - MH_PROF_RING,
+           "the stopwatch keeps only the most recent launches; this one has been overwritten");
+  const int slot = index % MH_PROF_RING;
+  MH_HIP(ctx, hipEventSynchronize(ctx->prof_ev[2 * slot + 1]));
+  MH_HIP(ctx, hipEventElapsedTime(elapsed_ms, ctx->prof_ev[2 * slot], ctx->prof_ev[2 * slot + 1]));
   return MACE_HIP_SUCCESS;
 }
 
 int mace_hip_profile_last_kernel_ms(mace_hip_ctx *ctx, float *elapsed_ms) {
   if (!ctx || !elapsed_ms) return MACE_HIP_INVALID_ARGS;
-  MH_CHECK(ctx, ctx->prof_valid, "no kernel has been timed since profiling was enabled");
-  MH_HIP(ctx, hipEventSynchronize(ctx->ev_k1));
-  MH_HIP(ctx, hipEventElapsedTime(elapsed_ms, ctx->ev_k0, ctx->ev_k1));
-  return MACE_HIP_SUCCESS;
+  MH_CHECK(ctx, ctx->prof_count > 0, "no kernel has been timed since profiling was enabled");
+  return mace_hip_profile_kernel_ms(ctx, ctx->prof_count - 1, elapsed_ms);
 }
 
 int mace_hip_ctx_fail_next_allocs(mace_hip_ctx *ctx, int n) {

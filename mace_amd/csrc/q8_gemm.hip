@@ -873,10 +873,12 @@ __device__ inline void transpose4x4_bytes(const uint32_t (&d)[4], uint32_t (&o)[
   o[3] = __builtin_amdgcn_perm(t3, t1, 0x07060302);
 }
 
+// With `sums` (zeroed beforehand, n entries per batch) the kernel also adds up what the panel
+// sums pass would: the shifted bytes of every output row, one atomic per row and tile.
 __global__ __launch_bounds__(256) void q8_pack_transpose128_kernel(const uint8_t *src,
                                                                    int64_t src_bs, uint8_t *dst,
                                                                    int64_t dst_bs, int n, int k,
-                                                                   int kp) {
+                                                                   int kp, int32_t *sums) {
   constexpr int PITCH = 130;
   __shared__ uint32_t tile[32 * PITCH];   // [n / 4][k]
   const uint8_t *s = src + (int64_t)blockIdx.z * src_bs;
@@ -915,7 +917,29 @@ __global__ __launch_bounds__(256) void q8_pack_transpose128_kernel(const uint8_t
           *(uint4 *)(d + (int64_t)gn * kp + gk) = uint4{o[0][j], o[1][j], o[2][j], o[3][j]};
       }
     }
+    if (sums) {
+      // bytes beyond k were loaded as 0x80 and count as zero; the 8 threads that share a row
+      // group are neighbouring lanes
+      int32_t *sb = sums + (int64_t)blockIdx.z * n;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        int v = 0;
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+          v = __builtin_amdgcn_sdot4((int)(o[b][j] ^ 0x80808080u), 0x01010101, v, false);
+        v += __shfl_xor(v, 1, 64);
+        v += __shfl_xor(v, 2, 64);
+        v += __shfl_xor(v, 4, 64);
+        const int gn = n0 + 4 * g + j;
+        if (kc == 0 && gn < n) atomicAdd(sb + gn, v);
+      }
+    }
   }
+}
+
+__global__ __launch_bounds__(256) void q8_zero_i32_kernel(int32_t *p, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0;
 }
 
 // ---- correction vectors --------------------------------------------------------------------
@@ -1141,7 +1165,11 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     const int32_t *sums;    // cached row sums of a registered weight, or nullptr
   } L, R;
 
-  auto pack = [&](const uint8_t *src, int order_is_kcontig, int nb, int64_t n, uint8_t *dst) -> int {
+  // fused_sums: where the repack may leave the panel's row sums as well (or nullptr); *fused
+  // tells whether it did
+  auto pack = [&](const uint8_t *src, int order_is_kcontig, int nb, int64_t n, uint8_t *dst,
+                  int32_t *fused_sums, bool *fused) -> int {
+    if (fused) *fused = false;
     if (order_is_kcontig) {
       const int64_t total = n * kp;
       dim3 grid((unsigned)std::min<int64_t>((total + 255) / 256, 65535), 1, nb);
@@ -1152,8 +1180,14 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
       const int vec_ok = (n % 16 == 0) && ((uintptr_t)src % 16 == 0);
       if (vec_ok) {
         dim3 grid((unsigned)((n + 127) / 128), (unsigned)((kp + 127) / 128), nb);
+        if (fused_sums) {
+          const int64_t cnt = (int64_t)nb * n;
+          hipLaunchKernelGGL(q8_zero_i32_kernel, dim3((unsigned)((cnt + 255) / 256)), dim3(256), 0,
+                             ctx->stream, fused_sums, cnt);
+          *fused = true;
+        }
         hipLaunchKernelGGL(q8_pack_transpose128_kernel, grid, dim3(256), 0, ctx->stream, src,
-                           n * depth, dst, n * kp, (int)n, (int)depth, (int)kp);
+                           n * depth, dst, n * kp, (int)n, (int)depth, (int)kp, fused_sums);
       } else {
         dim3 grid((unsigned)((n + 63) / 64), (unsigned)(kp / 64), nb);
         hipLaunchKernelGGL(q8_pack_transpose_kernel, grid, dim3(256), 0, ctx->stream, src,
@@ -1177,7 +1211,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
                       (int)(direct ? depth : kp), nullptr};
     if (!direct) {
       MH_HIP(ctx, hipMalloc((void **)&c.panel, (size_t)nb * n * kp));
-      const int rc = pack(src, order_is_kcontig, nb, n, c.panel);
+      const int rc = pack(src, order_is_kcontig, nb, n, c.panel, nullptr, nullptr);
       if (rc != MACE_HIP_SUCCESS) { (void)hipFree(c.panel); return rc; }
     }
     hipError_t e = hipMalloc((void **)&c.sums, sizeof(int32_t) * (size_t)nb * n);
@@ -1199,7 +1233,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   };
 
   auto prepare = [&](const uint8_t *src, int order_is_kcontig, bool direct, int nb, int64_t n,
-                     int64_t ld, mh_weight *w, Panel *P) -> int {
+                     int64_t ld, mh_weight *w, int32_t *corr, Panel *P) -> int {
     if (w) return prepare_weight(w, src, order_is_kcontig, direct, nb, n, P);
     if (direct) {
       // a caller-padded panel (ld > depth) is readable, and zero after the shift, up to ld
@@ -1210,29 +1244,35 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     if (!dst) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
     if (depth == 0) {
       MH_HIP(ctx, hipMemsetAsync(dst, 0x80, (size_t)nb * n * kp, ctx->stream));
-    } else {
-      MH_RETURN_IF_ERROR(pack(src, order_is_kcontig, nb, n, dst));
+      *P = Panel{dst, kp, nb > 1 ? n * kp : 0, (int)kp, nullptr};
+      return MACE_HIP_SUCCESS;
     }
-    *P = Panel{dst, kp, nb > 1 ? n * kp : 0, (int)kp, nullptr};
+    bool fused = false;
+    MH_RETURN_IF_ERROR(pack(src, order_is_kcontig, nb, n, dst, corr, &fused));
+    // sums the repack produced count like cached ones: no pass over the panel, none in the kernel
+    *P = Panel{dst, kp, nb > 1 ? n * kp : 0, (int)kp, fused ? corr : nullptr};
     return MACE_HIP_SUCCESS;
   };
-  MH_RETURN_IF_ERROR(prepare(lhs, lhs_order == MACE_HIP_ROW_MAJOR, lhs_direct, lhs_nb, rows, depth, lhs_w, &L));
-  MH_RETURN_IF_ERROR(prepare(rhs, rhs_order == MACE_HIP_COL_MAJOR, rhs_direct, rhs_nb, cols,
-                             rhs_ld != 0 ? rhs_ld : depth, rhs_w, &R));
-
   // correction vectors.  zl' = -lhs_offset - 128, zr' = -rhs_offset - 128.
   //   corrL[i] = -zr' * sum_k l'[i,k] + bias[i];   corrR[j] = -zl' * sum_k r'[k,j] + K zl' zr'
   int32_t *corrL = (int32_t *)mh_arena_take(ctx, sizeof(int32_t) * lhs_nb * rows);
   int32_t *corrR = (int32_t *)mh_arena_take(ctx, sizeof(int32_t) * rhs_nb * cols);
   if (!corrL || !corrR) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
-  const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
   const bool x_is_lhs = out_order == MACE_HIP_COL_MAJOR;
   // The Y operand's row sums can be taken inside the GEMM kernel from the fragments it already
   // holds, which saves one pass over that operand.  The pass costs YN * K bytes of HBM traffic,
   // the in-kernel sums about 7 % of the GEMM's own time (measured at 8192^3: +37 us against an
   // 11 us pass), i.e. the ratio grows with XN only: in-kernel wins below XN of about 2500.
-  const bool sum_y = cv || (depth > 0 && (depth <= 1024 || (x_is_lhs ? rows : cols) <= 2048) &&
-                            !(x_is_lhs ? R.sums : L.sums));   // cached sums cost nothing
+  const bool sum_y_shape = cv || (depth > 0 && (depth <= 1024 || (x_is_lhs ? rows : cols) <= 2048));
+  // A transposing repack can add up its rows on the way; worth its extra (zeroing) launch only
+  // where it replaces a pass, i.e. not for a Y operand whose sums the GEMM kernel takes anyway.
+  MH_RETURN_IF_ERROR(prepare(lhs, lhs_order == MACE_HIP_ROW_MAJOR, lhs_direct, lhs_nb, rows, depth,
+                             lhs_w, (!x_is_lhs && sum_y_shape) ? nullptr : corrL, &L));
+  MH_RETURN_IF_ERROR(prepare(rhs, rhs_order == MACE_HIP_COL_MAJOR, rhs_direct, rhs_nb, cols,
+                             rhs_ld != 0 ? rhs_ld : depth, rhs_w,
+                             (x_is_lhs && sum_y_shape) ? nullptr : corrR, &R));
+  const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
+  const bool sum_y = cv || (sum_y_shape && !(x_is_lhs ? R.sums : L.sums));   // cached sums cost nothing
   const int32_t l_coef = (int32_t)(0u - zr), l_add = 0;
   const int32_t r_coef = (int32_t)(0u - zl), r_add = (int32_t)((uint32_t)depth * zl * zr);
   const int32_t *l_bias = out_u8 ? ep.bias : nullptr;

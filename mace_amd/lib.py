@@ -46,6 +46,8 @@ SIGNATURES = {
     "mace_hip_timer_stop": (_int, [_p, C.POINTER(_f32)]),
     "mace_hip_profile_enable": (_int, [_p, _int]),
     "mace_hip_profile_last_kernel_ms": (_int, [_p, C.POINTER(_f32)]),
+    "mace_hip_profile_kernel_count": (_int, [_p, C.POINTER(_int)]),
+    "mace_hip_profile_kernel_ms": (_int, [_p, _int, C.POINTER(_f32)]),
     "mace_hip_ctx_fail_next_allocs": (_int, [_p, _int]),
     "mace_hip_malloc": (_int, [_p, C.c_size_t, C.POINTER(_p)]),
     "mace_hip_free": (_int, [_p, _p]),
@@ -198,6 +200,16 @@ class Context:
         ms = _f32()
         self.check(self.lib.mace_hip_profile_last_kernel_ms(self.handle, C.byref(ms)))
         return ms.value
+
+    def kernel_ms_list(self):
+        """Durations of the launches timed since profile(True), oldest first (waits for them)."""
+        n, ms = _int(), _f32()
+        self.check(self.lib.mace_hip_profile_kernel_count(self.handle, C.byref(n)))
+        out = []
+        for i in range(max(0, n.value - 512), n.value):
+            self.check(self.lib.mace_hip_profile_kernel_ms(self.handle, i, C.byref(ms)))
+            out.append(ms.value)
+        return out
 
 
 def get_output_multiplier_and_shift(lhs_scale, rhs_scale, out_scale):
