@@ -210,6 +210,8 @@ def test_q8_gemm_large_device_pointers(ctx, n, lo, ro, oo):
     (1, 1100, 1024, 1300, R, Cm, R, True),    # 128 x 128 tiles, 128-byte slabs
     (1, 1100, 1152, 1300, R, R, Cm, False),   # ... through the repack, column-major result
     (1, 2049, 448, 2305, R, Cm, R, True),     # 128 x 128 tiles, 64-byte slabs (k % 128 != 0)
+    (1, 4352, 256, 4608, R, Cm, R, True),     # 17 x 18 aligned 256 x 256 tiles: more than one per CU
+    (1, 4608, 384, 4352, R, Cm, Cm, False),   # ... odd number of slabs, column-major result
 ])
 def test_q8_gemm_ragged_tiled(ctx, batch, rows, depth, cols, lo, ro, oo, with_bias):
     """Shapes large enough for the 256 x 256 and 128 x 128 tile kernels whose sides are not
