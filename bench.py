@@ -448,6 +448,31 @@ def bench_other(ctx, mh, torch):
             tf = flops / (k * 1e-3) / 1e12
             out.append({"workload": "f32_gemm_4x1024^3_ta%d_tb%d" % (ta, tb), "kernel_ms": round(k, 4),
                         "TFLOPS": round(tf, 1), "frac_of_fp32_mfma_peak": round(tf / 157.3, 4)})
+    # The Gemv kernel where launch ramp and first-byte latency no longer dominate: 16384 x 16384
+    # weights (256 MiB per launch, rotating over three matrices), batch 1.
+    Hb = Wb = 16384
+    wbig = torch.randint(0, 256, (3, Hb, Wb), dtype=torch.uint8, device="cuda", generator=g)
+    xb = torch.randint(0, 256, (1, Wb), dtype=torch.uint8, device="cuda", generator=g)
+    bb = torch.zeros((Hb,), dtype=torch.int32, device="cuda")
+    yb = torch.empty((1, Hb), dtype=torch.uint8, device="cuda")
+    torch.cuda.synchronize()
+
+    def big_gemv(i):
+        ctx.call("mace_hip_gemv_q8_u8", wbig[i % 3].data_ptr(), xb.data_ptr(), bb.data_ptr(), 1, Hb, Wb,
+                 0, 1, 127, 128, 0.01, 0.02, 3.5, 128, mh.REQUANT_NEON, yb.data_ptr())
+
+    for i in range(6):
+        big_gemv(i)
+    ctx.sync()
+    ctx.timer_start()
+    for i in range(30):
+        big_gemv(i)
+    gms = ctx.timer_stop() / 30
+    gbytes = Hb * Wb + Wb + 4 * Hb + Hb
+    out.append({"workload": "q8_gemv_16384x16384_b1", "call_ms": round(gms, 4),
+                "GBps": round(gbytes / (gms * 1e-3) / 1e9, 1),
+                "frac_of_hbm_peak": round(gbytes / (gms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)})
+    del wbig
     # the steps either side of a quantized op: Quantize / Dequantize, 64 Mi elements each
     n = 64 << 20
     xf = torch.randn((n,), dtype=torch.float32, device="cuda", generator=g)
