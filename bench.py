@@ -353,7 +353,7 @@ def time_kernel(ctx, call, reps=10, warm=3):
 
 
 def bench_other(ctx, mh, torch):
-    """The remaining BASELINE configurations, timed the same way (device-resident inputs, HIP
+    """The remaining benchmark configurations, timed the same way (device-resident inputs, HIP
     events on the launch stream): not the headline, reported for coverage.  Each entry gives the
     dominant kernel's rate against the roofline that bounds it."""
     out = []

@@ -40,7 +40,7 @@ def test_conv_q8_known_answer(ctx):
     assert out.reshape(-1).tolist() == [k["expected"]]
 
 
-# MobileNetV1 pointwise shapes of BASELINE config 4 at batch 1-2 (batch 64 runs in the
+# MobileNetV1 pointwise shapes of benchmark configuration 4 at batch 1-2 (batch 64 runs in the
 # benchmark), the reference's random 1x1 case (conv_2d_test.cc:1383: batch 1, 128 <- 64, 32x32)
 # and ragged shapes
 CASES = [(2, 112, 112, 32, 64), (2, 56, 56, 128, 128), (2, 28, 28, 256, 256),
@@ -105,7 +105,7 @@ def test_conv1x1_q8_errors(ctx):
 @pytest.mark.parametrize("hw,cin,cout", [(112, 32, 64), (56, 128, 128), (28, 256, 256),
                                          (14, 512, 512), (7, 1024, 1024)])
 def test_conv1x1_q8_batch64_sampled(ctx, hw, cin, cout):
-    """BASELINE config 4 at its full batch of 64, device pointers: every output channel of 3000
+    """benchmark configuration 4 at its full batch of 64, device pointers: every output channel of 3000
     randomly chosen pixels (plus the first and last 64) against the oracle run on just those
     pixels -- a pixel's outputs depend on that pixel alone -- and a checksum identity over the
     whole tensor: the sum over pixels of the int32 outputs equals filter . (sum of the shifted

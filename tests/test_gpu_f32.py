@@ -1,7 +1,7 @@
 """fp32 Gemm / Gemv / Conv2D-1x1 on the GPU vs the CPU oracle.  Tolerance is the reference's
 own for this comparison (matmul_test.cc:142-143): |got - want| <= 1e-2 + 1e-4 * |want|,
 checked against both the binary32 serial oracle and the binary64-accumulated one; the
-BASELINE bound (1e-4 relative error) is asserted on the normwise relative error."""
+stated bound (1e-4 relative error) is asserted on the normwise relative error."""
 import json
 import os
 
@@ -83,7 +83,7 @@ def test_gemm_f32_reference_goldens(ctx, case):
 
 @pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
 def test_gemm_f32_config2(ctx, ta, tb):
-    """BASELINE config 2 at batch 4, 512^3 (the 1024^3 size runs in the benchmark; the
+    """benchmark configuration 2 at batch 4, 512^3 (the 1024^3 size runs in the benchmark; the
     scalar oracle needs ~1 s per 512^3 batch): N(0,1), all four transpose combinations,
     plus one non-batched lhs."""
     rng = np.random.default_rng(2)

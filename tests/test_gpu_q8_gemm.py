@@ -49,7 +49,7 @@ SHAPES = [  # batch, rows, depth, cols, lhs_batched, rhs_batched
     (1, 47, 37, 69, True, True), (3, 47, 37, 69, True, True), (16, 31, 61, 67, True, True),
     (6, 31, 61, 67, False, True), (6, 31, 61, 67, True, False),
     (1, 1, 3000, 256, True, True), (1, 3000, 256, 1, True, True), (3, 128, 256, 1, True, True),
-    (1, 128, 256, 128, True, True),          # BASELINE config 1
+    (1, 128, 256, 128, True, True),          # benchmark configuration 1
     (1, 300, 512, 260, True, True), (2, 257, 80, 513, True, True), (1, 5, 16, 7, True, True),
     (1, 1, 1, 1, True, True), (2, 130, 1000, 70, False, False),
 ]
@@ -80,7 +80,7 @@ def test_q8_gemm_parity(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo):
 
 
 def test_q8_gemm_config1_matmul(ctx):
-    """BASELINE config 1: A [128x256], B [256x128], zero points 128/128/128, scales
+    """benchmark configuration 1: A [128x256], B [256x128], zero points 128/128/128, scales
     0.02/0.015/0.05 -> (1649267328, shift 7)."""
     rng = np.random.default_rng(1)
     A = rng.integers(0, 256, (128, 256), dtype=np.uint8)
@@ -243,7 +243,7 @@ def test_q8_gemm_ragged_tiled(ctx, batch, rows, depth, cols, lo, ro, oo, with_bi
 
 
 def test_q8_gemm_batched_512(ctx):
-    """BASELINE config 5's batched case in full: 32 x 512^3, int32 accumulators and uint8 output."""
+    """benchmark configuration 5's batched case in full: 32 x 512^3, int32 accumulators and uint8 output."""
     rng = np.random.default_rng(9)
     b, n = 32, 512
     A = rng.integers(0, 256, (b, n, n), dtype=np.uint8)
@@ -260,7 +260,7 @@ def test_q8_gemm_batched_512(ctx):
 
 @pytest.mark.parametrize("n", [4096, 8192])
 def test_q8_gemm_freivalds_large(ctx, n):
-    """4096^3 and 8192^3 (BASELINE config 5): the oracle would take minutes, so (i) check
+    """4096^3 and 8192^3 (benchmark configuration 5): the oracle would take minutes, so (i) check
     C x == A (B x) exactly for random vectors x (a size-independent property; float64 holds these
     integers exactly), (ii) compare 32 full rows with the oracle, (iii) check the WHOLE uint8
     output by applying the oracle's output pipeline to the int32 output verified in (i)/(ii)."""

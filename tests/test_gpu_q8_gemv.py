@@ -65,7 +65,7 @@ def test_q8_gemv_parity(ctx, batch, h, w, lb, rb):
 
 
 def test_q8_gemv_config_4096(ctx):
-    """BASELINE config: weight [4096 x 4096], batch 1 and 8, weight_zp 127, input_zp 128,
+    """Benchmark configuration: weight [4096 x 4096], batch 1 and 8, weight_zp 127, input_zp 128,
     int32 bias in [-2^15, 2^15]; device-pointer path."""
     rng = np.random.default_rng(3)
     H = W = 4096
