@@ -34,6 +34,8 @@ def test_stopwatch_times_every_launch_without_waiting(ctx):
     small, large = _gemm(ctx, d, 256), _gemm(ctx, d, 2048)
     with pytest.raises(mh.MaceHipError):
         ctx.last_kernel_ms()                       # never enabled
+    small(), large()                               # first launches load the kernels' code
+    ctx.sync()
     ctx.profile(True)
     with pytest.raises(mh.MaceHipError):
         ctx.last_kernel_ms()                       # nothing timed yet
