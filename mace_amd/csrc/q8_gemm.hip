@@ -104,7 +104,9 @@ __device__ inline int sum16_i8(const v4i &f, int acc) {
 // so every lane owns runs of four consecutive x, stored as one 16-byte (int32) or 4-byte
 // (uint8) access.  The correction vectors of the tile are staged through LDS first (the
 // operand buffers are dead by then), so the stores do not wait on scattered global loads.
-template <int WX, int WY, int FX, int FY, typename OutT, bool SUMY>
+// PRESTAGED: the caller has already put the tile's x correction terms and the comparison table
+// into `lds` (same layout) and synchronised the workgroup.
+template <int WX, int WY, int FX, int FY, typename OutT, bool SUMY, bool PRESTAGED = false>
 __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[FX][FY], const int (&ysum)[FY],
                                      const GemmParams &p, uint8_t *lds, int b, int x0, int y0,
                                      int wx, int wy, int tid) {
@@ -114,6 +116,9 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[FX][FY], const int (&y
   const int32_t *cX = p.corrX + (int64_t)b * p.cxbs;
   const int32_t *cY = p.corrY + (int64_t)b * p.cybs;
   int32_t *sc = (int32_t *)lds;   // [TX] corrections along x, then [TY] along y
+  const RequantFixed rq = p.rq;
+  int32_t *tab = sc + TX + TY;    // [n + 2] comparison table of the threshold requantization
+  if constexpr (!PRESTAGED) {
   __syncthreads();                // every wavefront is done reading operand tiles
   // panel sums -> correction terms: coef * sum + add (+ bias on the side the result rows are on)
   for (int i = tid; i < TX; i += NT) {
@@ -129,8 +134,6 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[FX][FY], const int (&y
       if (p.ybias) c += (uint32_t)p.ybias[y];
       sc[TX + i] = (int32_t)c;
     }
-  const RequantFixed rq = p.rq;
-  int32_t *tab = sc + TX + TY;    // [n + 2] comparison table of the threshold requantization
   if constexpr (sizeof(OutT) == 1) {
     if (rq.table) {
       // The table is the kernel's second argument, placed right behind GemmParams in the
@@ -142,6 +145,7 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[FX][FY], const int (&y
     }
   }
   __syncthreads();
+  }
 
   OutT *outb = (OutT *)p.out + (int64_t)b * p.obs;
   const bool vec_ok = (p.ldo % 4 == 0) && (((uintptr_t)outb) % (4 * sizeof(OutT)) == 0);
@@ -400,6 +404,108 @@ __global__ __launch_bounds__(WX *WY * 64) void q8_gemm_kernel(GemmParams p, Requ
   gemm_epilogue<WX, WY, FX, FY, OutT, SUMY>(acc, ysum, p, lds, b, x0, y0, wx, wy, tid);
 }
 
+// ---- small problems: everything in one launch ---------------------------------------------
+//
+// A MatMul of a few hundred rows and columns is three launches in the general path (repack of
+// the operand that is not k-contiguous, row sums, GEMM) of a few microseconds each, most of it
+// launch latency.  This kernel does the whole call: 64 x 64 results per workgroup (four
+// wavefronts, one 32 x 32 accumulator each), operands read where they lie, in either layout --
+// XT / YT: the operand is stored k-major, [k][n] with n contiguous, and is transposed on its way
+// into LDS -- and both correction vectors taken from the fragments as they pass.
+// Requirements (checked by the host): a k-contiguous operand has K % 16 == 0 and 16-byte aligned
+// rows; a k-major operand has n % 16 == 0 and a 16-byte aligned base.
+template <typename OutT, bool XT, bool YT>
+__global__ __launch_bounds__(256) void q8_gemm_fused_small_kernel(GemmParams p, RequantTable) {
+  constexpr int T = 64;
+  __shared__ __align__(16) uint8_t tile[2][T * LDS_ROW];   // X rows, Y rows: [row][k], sign-flipped
+  __shared__ __align__(16) int32_t sc[2 * T + MH_REQUANT_TABLE_MAX + 2];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wx = wave % 2, wy = wave / 2;
+  const int tile_x = blockIdx.x % p.tiles_x, tile_y = blockIdx.x / p.tiles_x;
+  const int x0 = tile_x * T, y0 = tile_y * T;
+  const int b = blockIdx.z;
+  const uint8_t *Xb = p.X + (int64_t)b * p.xbs;
+  const uint8_t *Yb = p.Y + (int64_t)b * p.ybs;
+  const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+
+  // one 16-byte piece per thread, operand and k tile: row (or k) tid / 4, bytes 16 (tid % 4) ..
+  const int q = tid >> 2, c16 = (tid & 3) * 16;
+  auto fetch = [&](auto t_tag, const uint8_t *base, int64_t ld, int n, int n0, int k0) -> v4i {
+    if constexpr (decltype(t_tag)::value) {
+      // k-major: 16 consecutive n of row k0 + q
+      const bool ok = k0 + q < p.K && n0 + c16 < n;
+      return ok ? *(const v4i *)(base + (int64_t)(k0 + q) * ld + n0 + c16) : flip;
+    } else {
+      // k-contiguous: 16 consecutive k of row n0 + q (rows past the end: the last row again)
+      const bool ok = k0 + c16 < p.K;
+      return ok ? *(const v4i *)(base + (int64_t)min(n0 + q, n - 1) * ld + k0 + c16) : flip;
+    }
+  };
+  auto park = [&](auto t_tag, v4i v, uint8_t *dst) {
+    v ^= flip;
+    if constexpr (decltype(t_tag)::value) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+        dst[(c16 + e) * LDS_ROW + q] = (uint8_t)((uint32_t)v[e / 4] >> (8 * (e % 4)));
+    } else {
+      *(v4i *)(dst + q * LDS_ROW + c16) = v;
+    }
+  };
+  using XTag = std::integral_constant<bool, XT>;
+  using YTag = std::integral_constant<bool, YT>;
+
+  v16i acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0;
+  int xs = 0, ys = 0;
+  const int frag = (lane & 31) * LDS_ROW + (lane >> 5) * 16;
+  const uint8_t *fx = tile[0] + wx * 32 * LDS_ROW + frag;
+  const uint8_t *fy = tile[1] + wy * 32 * LDS_ROW + frag;
+
+  v4i rx = fetch(XTag{}, Xb, p.ldx, p.XN, x0, 0);
+  v4i ry = fetch(YTag{}, Yb, p.ldy, p.YN, y0, 0);
+  for (int k0 = 0; k0 < p.K; k0 += BK) {
+    park(XTag{}, rx, tile[0]);
+    park(YTag{}, ry, tile[1]);
+    __syncthreads();
+    if (k0 + BK < p.K) {   // next tile's loads fly during this tile's MFMAs
+      rx = fetch(XTag{}, Xb, p.ldx, p.XN, x0, k0 + BK);
+      ry = fetch(YTag{}, Yb, p.ldy, p.YN, y0, k0 + BK);
+    }
+#pragma unroll
+    for (int ks = 0; ks < BK / 32; ++ks) {
+      const v4i a = *(const v4i *)(fx + ks * 32), bf = *(const v4i *)(fy + ks * 32);
+      acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bf, acc, 0, 0, 0);
+      xs = sum16_i8(a, xs);
+      ys = sum16_i8(bf, ys);
+    }
+    __syncthreads();
+  }
+
+  // x corrections of the tile and the comparison table -> LDS; y corrections come from ys
+  xs += __shfl_xor(xs, 32, 64);
+  if (wy == 0 && lane < 32) {
+    const int xl = wx * 32 + lane;
+    uint32_t c = (uint32_t)p.xcoef * (uint32_t)xs + (uint32_t)p.xadd;
+    if (p.xbias) c += (uint32_t)p.xbias[min(x0 + xl, p.XN - 1)];
+    sc[xl] = (int32_t)c;
+  }
+  if constexpr (sizeof(OutT) == 1) {
+    if (p.rq.table) {
+      const int32_t *arg_tab = (const int32_t *)((const char *)__builtin_amdgcn_kernarg_segment_ptr() +
+                                                 sizeof(GemmParams));
+      for (int j = tid; j <= p.rq.n + 1; j += 256) sc[2 * T + j] = arg_tab[j];
+    }
+  }
+  __syncthreads();
+  v16i acc1[1][1] = {{acc}};
+  const int ysum[1] = {ys};
+  gemm_epilogue<2, 2, 1, 1, OutT, true, true>(acc1, ysum, p, (uint8_t *)sc, b, x0, y0, wx, wy, tid);
+}
+
 // ---- the streaming GEMM kernel: global -> LDS without passing through registers ----------
 //
 // A ring of STAGES LDS buffers, each one 64-byte k slab of the X and Y tiles, is filled by
@@ -413,6 +519,9 @@ __global__ __launch_bounds__(WX *WY * 64) void q8_gemm_kernel(GemmParams p, Requ
 //
 // Requirements (checked by the host): K % 64 == 0 and K >= 64 * (STAGES - 1).
 constexpr int SLAB = 64;   // bytes of k per ring stage
+// up to where the one-launch kernel for small problems is used
+constexpr int64_t MH_FUSED_SMALL_MAX_DEPTH = 1024;
+constexpr double MH_FUSED_SMALL_MAX_MACS = 1024.0 * 1024 * 1024;
 
 __device__ inline void dma_16B(const uint8_t *g, uint8_t *lds_wave_base) {
   __builtin_amdgcn_global_load_lds(
@@ -1076,6 +1185,31 @@ int launch_gemm_dma(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, b
   return MACE_HIP_SUCCESS;
 }
 
+// the one-launch kernel for small problems; the caller has checked its preconditions
+int launch_gemm_fused_small(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, bool out_u8,
+                            bool xt, bool yt, int batch) {
+  p.tiles_x = (p.XN + 63) / 64;
+  p.tiles_y = (p.YN + 63) / 64;
+  dim3 grid(p.tiles_x * p.tiles_y, 1, batch), block(256);
+  MH_PROF_BEGIN(ctx);
+#define MH_FUSED(OutT_, XT_, YT_) \
+  hipLaunchKernelGGL((q8_gemm_fused_small_kernel<OutT_, XT_, YT_>), grid, block, 0, ctx->stream, p, tab)
+  switch ((out_u8 ? 4 : 0) | (xt ? 2 : 0) | (yt ? 1 : 0)) {
+    case 0: MH_FUSED(int32_t, false, false); break;
+    case 1: MH_FUSED(int32_t, false, true); break;
+    case 2: MH_FUSED(int32_t, true, false); break;
+    case 3: MH_FUSED(int32_t, true, true); break;
+    case 4: MH_FUSED(uint8_t, false, false); break;
+    case 5: MH_FUSED(uint8_t, false, true); break;
+    case 6: MH_FUSED(uint8_t, true, false); break;
+    default: MH_FUSED(uint8_t, true, true); break;
+  }
+#undef MH_FUSED
+  MH_PROF_END(ctx);
+  MH_HIP(ctx, hipGetLastError());
+  return MACE_HIP_SUCCESS;
+}
+
 // the streaming kernel; the caller has checked its preconditions (see the kernel)
 template <int FX, int XW>
 int launch_gemm_stream(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, int batch) {
@@ -1151,6 +1285,54 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   };
   mh_weight *lhs_w = find_weight(lhs, (size_t)lhs_nb * rows * depth);
   mh_weight *rhs_w = (rhs_ld != 0 || cv) ? nullptr : find_weight(rhs, (size_t)rhs_nb * cols * depth);
+
+  // Small problems: one launch that reads both operands where they lie (k-contiguous, or k-major
+  // and transposed on the way into LDS) and takes both correction vectors itself.
+  {
+    const bool xl = out_order == MACE_HIP_COL_MAJOR;   // X = lhs rows, else X = rhs columns
+    const bool lhs_t = !lhs_direct && lhs_order == MACE_HIP_COL_MAJOR && rows % 16 == 0 &&
+                       ((uintptr_t)lhs % 16 == 0);
+    const bool rhs_t = !rhs_direct && rhs_order == MACE_HIP_ROW_MAJOR && cols % 16 == 0 &&
+                       ((uintptr_t)rhs % 16 == 0);
+    const int64_t cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
+    const int64_t wgs = ((rows + 63) / 64) * ((cols + 63) / 64) * batch;
+    const bool small = !cv && rhs_ld == 0 && depth > 0 && depth <= MH_FUSED_SMALL_MAX_DEPTH &&
+                       !lhs_w && !rhs_w && (lhs_direct || lhs_t) && (rhs_direct || rhs_t) &&
+                       wgs <= 4 * cus &&
+                       (double)batch * rows * cols * depth <= MH_FUSED_SMALL_MAX_MACS &&
+                       !getenv("MH_NO_FUSED");
+    if (small) {
+      GemmParams p{};
+      const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
+      const int32_t l_coef = (int32_t)(0u - zr), r_coef = (int32_t)(0u - zl);
+      const int32_t r_add = (int32_t)((uint32_t)depth * zl * zr);
+      const int32_t *l_bias = out_u8 ? ep.bias : nullptr;
+      const bool xt = xl ? lhs_t : rhs_t, yt = xl ? rhs_t : lhs_t;
+      p.X = xl ? lhs : rhs;
+      p.Y = xl ? rhs : lhs;
+      p.XN = (int)(xl ? rows : cols);
+      p.YN = (int)(xl ? cols : rows);
+      p.K = (int)depth;
+      p.ldx = xt ? p.XN : depth;    // k-major: bytes between consecutive k
+      p.ldy = yt ? p.YN : depth;
+      p.xbs = ((xl ? lhs_nb : rhs_nb) > 1) ? (int64_t)p.XN * depth : 0;
+      p.ybs = ((xl ? rhs_nb : lhs_nb) > 1) ? (int64_t)p.YN * depth : 0;
+      p.out = out;
+      p.ldo = p.XN;
+      p.obs = rows * cols;
+      p.rq = rq;
+      p.sum_y = true;
+      p.xcoef = xl ? l_coef : r_coef;
+      p.xadd = xl ? 0 : r_add;
+      p.xbias = xl ? l_bias : nullptr;
+      p.ycoef = xl ? r_coef : l_coef;
+      p.yadd = xl ? r_add : 0;
+      p.ybias = xl ? nullptr : l_bias;
+      RequantTable tab;
+      if (out_u8 && rq.table) mh_requant_table_cached(ctx, rq, tab.t);
+      return launch_gemm_fused_small(ctx, p, tab, out_u8, xt, yt, (int)batch);
+    }
+  }
 
   size_t need = sizeof(int32_t) * ((size_t)lhs_nb * rows + (size_t)rhs_nb * cols) + 4096 + 512;
   if (!lhs_direct && !lhs_w) need += (size_t)lhs_nb * rows * kp + 256;
