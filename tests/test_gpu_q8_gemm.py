@@ -52,6 +52,8 @@ SHAPES = [  # batch, rows, depth, cols, lhs_batched, rhs_batched
     (1, 128, 256, 128, True, True),          # benchmark configuration 1
     (1, 300, 512, 260, True, True), (2, 257, 80, 513, True, True), (1, 5, 16, 7, True, True),
     (1, 1, 1, 1, True, True), (2, 130, 1000, 70, False, False),
+    # aligned in every layout (the one-launch kernel for small problems), one side shared
+    (5, 64, 96, 80, False, True), (5, 80, 48, 144, True, False), (3, 16, 1024, 16, True, True),
 ]
 
 
