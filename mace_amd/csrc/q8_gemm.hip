@@ -465,40 +465,55 @@ __global__ __launch_bounds__(256) void q8_gemm_fused_small_kernel(GemmParams p, 
   const uint8_t *fx = tile[0] + wx * 32 * LDS_ROW + frag;
   const uint8_t *fy = tile[1] + wy * 32 * LDS_ROW + frag;
 
-  v4i rx = fetch(XTag{}, Xb, p.ldx, p.XN, x0, 0);
-  v4i ry = fetch(YTag{}, Yb, p.ldy, p.YN, y0, 0);
-  for (int k0 = 0; k0 < p.K; k0 += BK) {
-    park(XTag{}, rx, tile[0]);
-    park(YTag{}, ry, tile[1]);
-    __syncthreads();
-    if (k0 + BK < p.K) {   // next tile's loads fly during this tile's MFMAs
-      rx = fetch(XTag{}, Xb, p.ldx, p.XN, x0, k0 + BK);
-      ry = fetch(YTag{}, Yb, p.ldy, p.YN, y0, k0 + BK);
-    }
-#pragma unroll
-    for (int ks = 0; ks < BK / 32; ++ks) {
-      const v4i a = *(const v4i *)(fx + ks * 32), bf = *(const v4i *)(fy + ks * 32);
-      acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bf, acc, 0, 0, 0);
-      xs = sum16_i8(a, xs);
-      ys = sum16_i8(bf, ys);
-    }
-    __syncthreads();
-  }
-
-  // x corrections of the tile and the comparison table -> LDS; y corrections come from ys
-  xs += __shfl_xor(xs, 32, 64);
-  if (wy == 0 && lane < 32) {
-    const int xl = wx * 32 + lane;
-    uint32_t c = (uint32_t)p.xcoef * (uint32_t)xs + (uint32_t)p.xadd;
-    if (p.xbias) c += (uint32_t)p.xbias[min(x0 + xl, p.XN - 1)];
-    sc[xl] = (int32_t)c;
-  }
+  // Everything the epilogue needs from memory is asked for now, so that it arrives under the
+  // operand loads: the comparison table (into LDS) and this lane's bias.
   if constexpr (sizeof(OutT) == 1) {
     if (p.rq.table) {
       const int32_t *arg_tab = (const int32_t *)((const char *)__builtin_amdgcn_kernarg_segment_ptr() +
                                                  sizeof(GemmParams));
       for (int j = tid; j <= p.rq.n + 1; j += 256) sc[2 * T + j] = arg_tab[j];
     }
+  }
+  const int32_t xbias = p.xbias ? p.xbias[min(x0 + wx * 32 + (lane & 31), p.XN - 1)] : 0;
+
+  // NPRE k tiles of both operands are in flight at a time: with only a few tiles in all, what a
+  // call costs is the chain of load round trips, not bandwidth
+  constexpr int NPRE = 4;
+  v4i rx[NPRE], ry[NPRE];
+#pragma unroll
+  for (int s = 0; s < NPRE; ++s) {
+    rx[s] = fetch(XTag{}, Xb, p.ldx, p.XN, x0, s * BK);   // tiles past K come back as zeros
+    ry[s] = fetch(YTag{}, Yb, p.ldy, p.YN, y0, s * BK);
+  }
+  for (int kb = 0; kb < p.K; kb += NPRE * BK) {
+#pragma unroll
+    for (int s = 0; s < NPRE; ++s) {
+      const int k0 = kb + s * BK;
+      if (k0 < p.K) {   // uniform over the workgroup
+        park(XTag{}, rx[s], tile[0]);
+        park(YTag{}, ry[s], tile[1]);
+        __syncthreads();
+        if (k0 + NPRE * BK < p.K) {
+          rx[s] = fetch(XTag{}, Xb, p.ldx, p.XN, x0, k0 + NPRE * BK);
+          ry[s] = fetch(YTag{}, Yb, p.ldy, p.YN, y0, k0 + NPRE * BK);
+        }
+#pragma unroll
+        for (int ks = 0; ks < BK / 32; ++ks) {
+          const v4i a = *(const v4i *)(fx + ks * 32), bf = *(const v4i *)(fy + ks * 32);
+          acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bf, acc, 0, 0, 0);
+          xs = sum16_i8(a, xs);
+          ys = sum16_i8(bf, ys);
+        }
+        __syncthreads();
+      }
+    }
+  }
+
+  // x corrections of the tile and the comparison table -> LDS; y corrections come from ys
+  xs += __shfl_xor(xs, 32, 64);
+  if (wy == 0 && lane < 32) {
+    const int xl = wx * 32 + lane;
+    sc[xl] = (int32_t)((uint32_t)p.xcoef * (uint32_t)xs + (uint32_t)p.xadd + (uint32_t)xbias);
   }
   __syncthreads();
   v16i acc1[1][1] = {{acc}};
