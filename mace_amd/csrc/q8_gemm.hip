@@ -67,6 +67,9 @@ struct GemmParams {
   int cv_in_h, cv_in_w, cv_cin, cv_kw, cv_sh, cv_sw, cv_pt, cv_pl, cv_oh, cv_ow;
   const uint8_t *cv_zero;   // >= 64 bytes holding the input zero point (padding positions)
   bool conv;
+  // q8_gemm_fused_small_kernel: the operand's rows are not 16-byte pieces (odd depth or row
+  // length, unaligned base) and are read byte by byte
+  bool x_bytewise, y_bytewise;
 };
 
 // XCD-aware tile order: consecutive workgroup ids are dealt round-robin to the 8 XCDs, so
@@ -412,8 +415,8 @@ __global__ __launch_bounds__(WX *WY * 64) void q8_gemm_kernel(GemmParams p, Requ
 // wavefronts, one 32 x 32 accumulator each), operands read where they lie, in either layout --
 // XT / YT: the operand is stored k-major, [k][n] with n contiguous, and is transposed on its way
 // into LDS -- and both correction vectors taken from the fragments as they pass.
-// Requirements (checked by the host): a k-contiguous operand has K % 16 == 0 and 16-byte aligned
-// rows; a k-major operand has n % 16 == 0 and a 16-byte aligned base.
+// An operand whose rows do not consist of aligned 16-byte pieces (k-contiguous with K % 16 != 0,
+// k-major with n % 16 != 0, or an unaligned base) is read byte by byte (x_bytewise / y_bytewise).
 template <typename OutT, bool XT, bool YT>
 __global__ __launch_bounds__(256) void q8_gemm_fused_small_kernel(GemmParams p, RequantTable) {
   constexpr int T = 64;
@@ -433,7 +436,26 @@ __global__ __launch_bounds__(256) void q8_gemm_fused_small_kernel(GemmParams p, 
 
   // one 16-byte piece per thread, operand and k tile: row (or k) tid / 4, bytes 16 (tid % 4) ..
   const int q = tid >> 2, c16 = (tid & 3) * 16;
-  auto fetch = [&](auto t_tag, const uint8_t *base, int64_t ld, int n, int n0, int k0) -> v4i {
+  auto fetch = [&](auto t_tag, bool bytewise, const uint8_t *base, int64_t ld, int n, int n0,
+                   int k0) -> v4i {
+    if (bytewise) {   // uniform over the launch
+      uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        bool ok;
+        const uint8_t *src;
+        if constexpr (decltype(t_tag)::value) {
+          ok = k0 + q < p.K && n0 + c16 + e < n;
+          src = base + (int64_t)(k0 + q) * ld + n0 + c16 + e;
+        } else {
+          ok = k0 + c16 + e < p.K;
+          src = base + (int64_t)min(n0 + q, n - 1) * ld + k0 + c16 + e;
+        }
+        const uint32_t byte = ok ? (uint32_t)*src : 0x80u;
+        w[e / 4] |= byte << (8 * (e % 4));
+      }
+      return v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+    }
     if constexpr (decltype(t_tag)::value) {
       // k-major: 16 consecutive n of row k0 + q
       const bool ok = k0 + q < p.K && n0 + c16 < n;
@@ -482,8 +504,8 @@ __global__ __launch_bounds__(256) void q8_gemm_fused_small_kernel(GemmParams p, 
   v4i rx[NPRE], ry[NPRE];
 #pragma unroll
   for (int s = 0; s < NPRE; ++s) {
-    rx[s] = fetch(XTag{}, Xb, p.ldx, p.XN, x0, s * BK);   // tiles past K come back as zeros
-    ry[s] = fetch(YTag{}, Yb, p.ldy, p.YN, y0, s * BK);
+    rx[s] = fetch(XTag{}, p.x_bytewise, Xb, p.ldx, p.XN, x0, s * BK);   // tiles past K come back as zeros
+    ry[s] = fetch(YTag{}, p.y_bytewise, Yb, p.ldy, p.YN, y0, s * BK);
   }
   for (int kb = 0; kb < p.K; kb += NPRE * BK) {
 #pragma unroll
@@ -494,8 +516,8 @@ __global__ __launch_bounds__(256) void q8_gemm_fused_small_kernel(GemmParams p, 
         park(YTag{}, ry[s], tile[1]);
         __syncthreads();
         if (k0 + NPRE * BK < p.K) {
-          rx[s] = fetch(XTag{}, Xb, p.ldx, p.XN, x0, k0 + NPRE * BK);
-          ry[s] = fetch(YTag{}, Yb, p.ldy, p.YN, y0, k0 + NPRE * BK);
+          rx[s] = fetch(XTag{}, p.x_bytewise, Xb, p.ldx, p.XN, x0, k0 + NPRE * BK);
+          ry[s] = fetch(YTag{}, p.y_bytewise, Yb, p.ldy, p.YN, y0, k0 + NPRE * BK);
         }
 #pragma unroll
         for (int ks = 0; ks < BK / 32; ++ks) {
@@ -537,6 +559,9 @@ constexpr int SLAB = 64;   // bytes of k per ring stage
 // up to where the one-launch kernel for small problems is used
 constexpr int64_t MH_FUSED_SMALL_MAX_DEPTH = 1024;
 constexpr double MH_FUSED_SMALL_MAX_MACS = 1024.0 * 1024 * 1024;
+// ... when an operand has to be read byte by byte (measured: 600 x 600 x 300 still wins, depth 500 loses)
+constexpr int64_t MH_FUSED_SMALL_MAX_DEPTH_BYTEWISE = 320;
+constexpr double MH_FUSED_SMALL_MAX_MACS_BYTEWISE = 128.0 * 1024 * 1024;
 
 __device__ inline void dma_16B(const uint8_t *g, uint8_t *lds_wave_base) {
   __builtin_amdgcn_global_load_lds(
@@ -1305,16 +1330,19 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   // and transposed on the way into LDS) and takes both correction vectors itself.
   {
     const bool xl = out_order == MACE_HIP_COL_MAJOR;   // X = lhs rows, else X = rhs columns
-    const bool lhs_t = !lhs_direct && lhs_order == MACE_HIP_COL_MAJOR && rows % 16 == 0 &&
-                       ((uintptr_t)lhs % 16 == 0);
-    const bool rhs_t = !rhs_direct && rhs_order == MACE_HIP_ROW_MAJOR && cols % 16 == 0 &&
-                       ((uintptr_t)rhs % 16 == 0);
+    const bool lhs_t = lhs_order == MACE_HIP_COL_MAJOR, rhs_t = rhs_order == MACE_HIP_ROW_MAJOR;
+    // rows made of aligned 16-byte pieces are read as such, anything else byte by byte (which is
+    // only worth it while the whole problem is a few tiles)
+    const bool lhs_vec = lhs_t ? (rows % 16 == 0 && (uintptr_t)lhs % 16 == 0) : lhs_direct;
+    const bool rhs_vec = rhs_t ? (cols % 16 == 0 && (uintptr_t)rhs % 16 == 0) : rhs_direct;
+    const double macs = (double)batch * rows * cols * depth;
     const int64_t cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
     const int64_t wgs = ((rows + 63) / 64) * ((cols + 63) / 64) * batch;
-    const bool small = !cv && rhs_ld == 0 && depth > 0 && depth <= MH_FUSED_SMALL_MAX_DEPTH &&
-                       !lhs_w && !rhs_w && (lhs_direct || lhs_t) && (rhs_direct || rhs_t) &&
-                       wgs <= 4 * cus &&
-                       (double)batch * rows * cols * depth <= MH_FUSED_SMALL_MAX_MACS &&
+    const bool all_vec = lhs_vec && rhs_vec;
+    const bool small = !cv && rhs_ld == 0 && depth > 0 &&
+                       depth <= (all_vec ? MH_FUSED_SMALL_MAX_DEPTH : MH_FUSED_SMALL_MAX_DEPTH_BYTEWISE) &&
+                       !lhs_w && !rhs_w && wgs <= 4 * cus &&
+                       macs <= (all_vec ? MH_FUSED_SMALL_MAX_MACS : MH_FUSED_SMALL_MAX_MACS_BYTEWISE) &&
                        !getenv("MH_NO_FUSED");
     if (small) {
       GemmParams p{};
@@ -1337,6 +1365,8 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
       p.obs = rows * cols;
       p.rq = rq;
       p.sum_y = true;
+      p.x_bytewise = !(xl ? lhs_vec : rhs_vec);
+      p.y_bytewise = !(xl ? rhs_vec : lhs_vec);
       p.xcoef = xl ? l_coef : r_coef;
       p.xadd = xl ? 0 : r_add;
       p.xbias = xl ? l_bias : nullptr;
