@@ -420,24 +420,28 @@ def bench_other(ctx, mh, torch):
 
     # beyond the 1x1 shapes: 3x3 convolutions (SAME padding, stride 1); with cin % 64 == 0 the
     # GEMM's loader gathers the patches itself and no im2col matrix is written
-    for (hw, cin, cout, k) in ((56, 64, 64, 3), (28, 128, 128, 3)):
-        n = 64
+    # (batch 64, and single-image inference: one launch that gathers as it goes; the first entry is
+    # MobileNet's first layer, 224 x 224 x 3 at stride 2)
+    for (n, hw, cin, cout, k, st) in ((64, 56, 64, 64, 3, 1), (64, 28, 128, 128, 3, 1),
+                                      (1, 224, 3, 32, 3, 2), (1, 56, 64, 64, 3, 1), (1, 28, 128, 128, 3, 1)):
+        oh = (hw + st - 1) // st
+        pad = max((oh - 1) * st + k - hw, 0)      # SAME
         x, f = u8(n, hw, hw, cin), u8(cout, k, k, cin)
         bias = torch.randint(-2 ** 15, 2 ** 15, (cout,), dtype=torch.int32, device="cuda", generator=g)
-        y = torch.empty((n, hw, hw, cout), dtype=torch.uint8, device="cuda")
+        y = torch.empty((n, oh, oh, cout), dtype=torch.uint8, device="cuda")
         s_in, s_f = 0.02, 0.01
         s_out = max(6.0, 3 * 74.0 * 74.0 * (k * k * cin) ** 0.5 * s_in * s_f) / 255.0
         torch.cuda.synchronize()
         whole, kms = time_kernel(ctx, lambda: ctx.call(
             "mace_hip_conv2d_q8_nhwc", x.data_ptr(), f.data_ptr(), bias.data_ptr(), n, hw, hw, cin,
-            cout, k, k, 1, 1, k - 1, k - 1, s_in, 128, s_f, 127, s_in * s_f, s_out, 0, 0, 255,
+            cout, k, k, st, st, pad, pad, s_in, 128, s_f, 127, s_in * s_f, s_out, 0, 0, 255,
             y.data_ptr()))
-        pix = n * hw * hw
+        pix = n * oh * oh
         ops = 2.0 * pix * k * k * cin * cout
-        nbytes = pix * cin + cout * k * k * cin + 4 * cout + pix * cout
+        nbytes = n * hw * hw * cin + cout * k * k * cin + 4 * cout + pix * cout
         roof_tops = min(PEAK_INT8_TOPS, ops / nbytes * PEAK_HBM_GBS / 1e3)
         tops = ops / (whole * 1e-3) / 1e12
-        out.append({"workload": "q8_conv%dx%d_n64_%dx%dx%d_to_%d" % (k, k, hw, hw, cin, cout),
+        out.append({"workload": "q8_conv%dx%d_s%d_n%d_%dx%dx%d_to_%d" % (k, k, st, n, hw, hw, cin, cout),
                     "call_ms": round(whole, 4), "gemm_kernel_ms": round(kms, 4),
                     "TOPS_whole_call": round(tops, 1), "roofline_TOPS": round(roof_tops, 1),
                     "frac_of_roofline": round(tops / roof_tops, 4)})

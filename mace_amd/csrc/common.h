@@ -358,11 +358,26 @@ struct Q8GemmEpilogue {
 // (image, oh, ow) is the k_h x k_w x cin patch at (oh*stride_h - pad_top, ow*stride_w - pad_left)
 // of an NHWC input, k in (kh, kw, channel) order, positions outside the input = zero_point.
 // mh_q8_gemm takes it with rhs = the input tensor, cols = images*out_h*out_w, depth = k_h*k_w*cin,
-// lhs RowMajor, result ColMajor, batch 1; cin % 64 == 0 and depth >= 192.
+// lhs RowMajor, result ColMajor, batch 1; cin % 64 == 0 and depth >= 192 -- or any geometry when
+// the call is a small problem (mh_q8_small_problem with vec = filter rows and channel runs made of
+// aligned 16-byte pieces).
 struct Q8ConvGather {
   int in_h, in_w, cin, k_h, k_w, stride_h, stride_w, pad_top, pad_left, out_h, out_w;
   int zero_point;
 };
+
+// Whether a uint8 GEMM call is run by the one-launch kernel for small problems
+// (q8_gemm_fused_small_kernel).  vec: both operands consist of aligned 16-byte pieces; otherwise
+// at least one is read byte by byte, which pays only for shallower and smaller problems
+// (measured: 600 x 600 x 300 still wins, depth 500 loses; with 16-byte pieces 1024^3 still wins).
+inline bool mh_q8_small_problem(const mace_hip_ctx *ctx, int64_t batch, int64_t rows, int64_t cols,
+                                int64_t depth, bool vec) {
+  const int64_t cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
+  const int64_t wgs = ((rows + 63) / 64) * ((cols + 63) / 64) * batch;
+  const double macs = (double)batch * rows * cols * depth;
+  return depth > 0 && depth <= (vec ? 1024 : 320) && wgs <= 4 * cus &&
+         macs <= (vec ? 1024.0 : 128.0) * 1024 * 1024;
+}
 
 int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8_t *rhs,
                int rhs_order, void *out, int out_order, bool out_u8, int64_t batch,

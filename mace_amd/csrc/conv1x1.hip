@@ -149,8 +149,16 @@ extern "C" int mace_hip_conv2d_q8_nhwc(mace_hip_ctx *ctx, const uint8_t *input,
                         pad_w == 0;
   // With cin a multiple of 64 (and at least three 64-byte slabs of depth) the GEMM's loader
   // gathers the patches itself and no im2col matrix is written.
-  const bool gather = !in_place && cin % 64 == 0 && depth >= 192 && ((uintptr_t)input % 16 == 0) &&
-                      ((uintptr_t)filter % 16 == 0) && in_h * in_w * cin < (1ll << 31);
+  // A small problem is one launch of the kernel that does the whole GEMM call, which gathers too
+  // (any channel count).
+  const bool small_vec = depth % 16 == 0 && cin % 16 == 0 && ((uintptr_t)input % 16 == 0) &&
+                         ((uintptr_t)filter % 16 == 0);
+  const bool small_gather = !in_place && in_h * in_w * cin < (1ll << 31) &&
+                            mh_q8_small_problem(ctx, 1, cout, columns, depth, small_vec) &&
+                            !getenv("MH_NO_FUSED");
+  const bool gather = small_gather ||
+                      (!in_place && cin % 64 == 0 && depth >= 192 && ((uintptr_t)input % 16 == 0) &&
+                       ((uintptr_t)filter % 16 == 0) && in_h * in_w * cin < (1ll << 31));
   const int64_t kp = (int64_t)mh_align_up((size_t)(depth > 0 ? depth : 1), 64);
   size_t need = sizeof(int32_t) * cout + 4096 +
                 conv_gemm_scratch(cout, depth, columns, !in_place || depth % 16 == 0);

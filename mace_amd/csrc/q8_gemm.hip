@@ -66,6 +66,7 @@ struct GemmParams {
   // input, row y = (image, oh, ow), k = (kh, kw, channel) with cin % 64 == 0
   int cv_in_h, cv_in_w, cv_cin, cv_kw, cv_sh, cv_sw, cv_pt, cv_pl, cv_oh, cv_ow;
   const uint8_t *cv_zero;   // >= 64 bytes holding the input zero point (padding positions)
+  uint32_t cv_zp4;          // the input zero point in all four bytes (q8_gemm_fused_small_kernel)
   bool conv;
   // q8_gemm_fused_small_kernel: the operand's rows are not 16-byte pieces (odd depth or row
   // length, unaligned base) and are read byte by byte
@@ -417,6 +418,8 @@ __global__ __launch_bounds__(WX *WY * 64) void q8_gemm_kernel(GemmParams p, Requ
 // into LDS -- and both correction vectors taken from the fragments as they pass.
 // An operand whose rows do not consist of aligned 16-byte pieces (k-contiguous with K % 16 != 0,
 // k-major with n % 16 != 0, or an unaligned base) is read byte by byte (x_bytewise / y_bytewise).
+// With p.conv the Y rows are the patches of a convolution, gathered from the NHWC input (16 bytes
+// at a time when cin % 16 == 0, else byte by byte); positions in the padding read the zero point.
 template <typename OutT, bool XT, bool YT>
 __global__ __launch_bounds__(256) void q8_gemm_fused_small_kernel(GemmParams p, RequantTable) {
   constexpr int T = 64;
@@ -479,6 +482,57 @@ __global__ __launch_bounds__(256) void q8_gemm_fused_small_kernel(GemmParams p, 
   using XTag = std::integral_constant<bool, XT>;
   using YTag = std::integral_constant<bool, YT>;
 
+  // convolution gather: this thread's Y row is one output pixel; top-left corner of its patch
+  int cv_ih0 = 0, cv_iw0 = 0;
+  const uint8_t *cv_img = Yb;
+  if (p.conv) {
+    const int y = min(y0 + q, p.YN - 1);
+    const int ow = y % p.cv_ow, t = y / p.cv_ow;
+    const int oh = t % p.cv_oh, img = t / p.cv_oh;
+    cv_ih0 = oh * p.cv_sh - p.cv_pt;
+    cv_iw0 = ow * p.cv_sw - p.cv_pl;
+    cv_img = Yb + (int64_t)img * p.cv_in_h * p.cv_in_w * p.cv_cin;
+  }
+  auto fetch_patch = [&](int k0) -> v4i {
+    int kk = k0 + c16;
+    if (kk >= p.K) return flip;
+    // k = (kh, kw, channel); decoded once, then stepped
+    int tap = kk / p.cv_cin, c = kk - tap * p.cv_cin;
+    int kh = tap / p.cv_kw, kw = tap - kh * p.cv_kw;
+    auto at = [&](int kh_, int kw_, int c_, bool *inside) -> const uint8_t * {
+      const int ih = cv_ih0 + kh_, iw = cv_iw0 + kw_;
+      *inside = (unsigned)ih < (unsigned)p.cv_in_h && (unsigned)iw < (unsigned)p.cv_in_w;
+      return cv_img + ((int64_t)ih * p.cv_in_w + iw) * p.cv_cin + c_;
+    };
+    const int zp4 = (int)p.cv_zp4;
+    if (!p.y_bytewise) {   // cin % 16 == 0: the 16 bytes lie inside one tap
+      bool inside;
+      const uint8_t *src = at(kh, kw, c, &inside);
+      return inside ? *(const v4i *)src : v4i{zp4, zp4, zp4, zp4};
+    }
+    uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      uint32_t byte = 0x80u;
+      if (kk < p.K) {
+        bool inside;
+        const uint8_t *src = at(kh, kw, c, &inside);
+        byte = inside ? (uint32_t)*src : ((uint32_t)zp4 & 0xffu);
+      }
+      w[e / 4] |= byte << (8 * (e % 4));
+      ++kk;
+      if (++c == p.cv_cin) {
+        c = 0;
+        if (++kw == p.cv_kw) { kw = 0; ++kh; }
+      }
+    }
+    return v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+  };
+  auto fetch_y = [&](int k0) -> v4i {
+    if (p.conv) return fetch_patch(k0);   // uniform over the launch
+    return fetch(YTag{}, p.y_bytewise, Yb, p.ldy, p.YN, y0, k0);
+  };
+
   v16i acc;
 #pragma unroll
   for (int r = 0; r < 16; ++r) acc[r] = 0;
@@ -505,7 +559,7 @@ __global__ __launch_bounds__(256) void q8_gemm_fused_small_kernel(GemmParams p, 
 #pragma unroll
   for (int s = 0; s < NPRE; ++s) {
     rx[s] = fetch(XTag{}, p.x_bytewise, Xb, p.ldx, p.XN, x0, s * BK);   // tiles past K come back as zeros
-    ry[s] = fetch(YTag{}, p.y_bytewise, Yb, p.ldy, p.YN, y0, s * BK);
+    ry[s] = fetch_y(s * BK);
   }
   for (int kb = 0; kb < p.K; kb += NPRE * BK) {
 #pragma unroll
@@ -517,7 +571,7 @@ __global__ __launch_bounds__(256) void q8_gemm_fused_small_kernel(GemmParams p, 
         __syncthreads();
         if (k0 + NPRE * BK < p.K) {
           rx[s] = fetch(XTag{}, p.x_bytewise, Xb, p.ldx, p.XN, x0, k0 + NPRE * BK);
-          ry[s] = fetch(YTag{}, p.y_bytewise, Yb, p.ldy, p.YN, y0, k0 + NPRE * BK);
+          ry[s] = fetch_y(k0 + NPRE * BK);
         }
 #pragma unroll
         for (int ks = 0; ks < BK / 32; ++ks) {
@@ -556,12 +610,6 @@ __global__ __launch_bounds__(256) void q8_gemm_fused_small_kernel(GemmParams p, 
 //
 // Requirements (checked by the host): K % 64 == 0 and K >= 64 * (STAGES - 1).
 constexpr int SLAB = 64;   // bytes of k per ring stage
-// up to where the one-launch kernel for small problems is used
-constexpr int64_t MH_FUSED_SMALL_MAX_DEPTH = 1024;
-constexpr double MH_FUSED_SMALL_MAX_MACS = 1024.0 * 1024 * 1024;
-// ... when an operand has to be read byte by byte (measured: 600 x 600 x 300 still wins, depth 500 loses)
-constexpr int64_t MH_FUSED_SMALL_MAX_DEPTH_BYTEWISE = 320;
-constexpr double MH_FUSED_SMALL_MAX_MACS_BYTEWISE = 128.0 * 1024 * 1024;
 
 __device__ inline void dma_16B(const uint8_t *g, uint8_t *lds_wave_base) {
   __builtin_amdgcn_global_load_lds(
@@ -1307,10 +1355,16 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
            "padded right-hand panel must be ColMajor, 16-byte aligned, pitch a multiple of 16");
   // cv: the right operand is not a matrix in memory but the patches of a convolution, gathered by
   // the streaming kernel's loader (the caller has checked the geometry, see Q8ConvGather)
-  MH_CHECK(ctx, !cv || (rhs_ld == 0 && batch == 1 && out_order == MACE_HIP_COL_MAJOR &&
-                        lhs_order == MACE_HIP_ROW_MAJOR && depth % SLAB == 0 && depth >= 3 * SLAB &&
-                        cv->cin % SLAB == 0 && ((uintptr_t)rhs % 16 == 0) &&
-                        ((uintptr_t)lhs % 16 == 0)),
+  // ... or, for a small problem, by the one-launch kernel, which takes any geometry
+  const bool cv_vec = cv && lhs_direct && cv->cin % 16 == 0 && ((uintptr_t)rhs % 16 == 0);
+  const bool cv_small = cv && rhs_ld == 0 && batch == 1 && out_order == MACE_HIP_COL_MAJOR &&
+                        lhs_order == MACE_HIP_ROW_MAJOR &&
+                        mh_q8_small_problem(ctx, 1, rows, cols, depth, cv_vec) &&
+                        !getenv("MH_NO_FUSED");
+  MH_CHECK(ctx, !cv || cv_small ||
+                    (rhs_ld == 0 && batch == 1 && out_order == MACE_HIP_COL_MAJOR &&
+                     lhs_order == MACE_HIP_ROW_MAJOR && depth % SLAB == 0 && depth >= 3 * SLAB &&
+                     cv->cin % SLAB == 0 && ((uintptr_t)rhs % 16 == 0) && ((uintptr_t)lhs % 16 == 0)),
            "convolution gather needs cin % 64 == 0, depth >= 192 and 16-byte aligned tensors");
   const bool rhs_direct = cv || rhs_ld != 0 ||
                           (rhs_order == MACE_HIP_COL_MAJOR && depth % 16 == 0 && depth > 0 &&
@@ -1334,16 +1388,13 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     // rows made of aligned 16-byte pieces are read as such, anything else byte by byte (which is
     // only worth it while the whole problem is a few tiles)
     const bool lhs_vec = lhs_t ? (rows % 16 == 0 && (uintptr_t)lhs % 16 == 0) : lhs_direct;
-    const bool rhs_vec = rhs_t ? (cols % 16 == 0 && (uintptr_t)rhs % 16 == 0) : rhs_direct;
-    const double macs = (double)batch * rows * cols * depth;
-    const int64_t cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
-    const int64_t wgs = ((rows + 63) / 64) * ((cols + 63) / 64) * batch;
-    const bool all_vec = lhs_vec && rhs_vec;
-    const bool small = !cv && rhs_ld == 0 && depth > 0 &&
-                       depth <= (all_vec ? MH_FUSED_SMALL_MAX_DEPTH : MH_FUSED_SMALL_MAX_DEPTH_BYTEWISE) &&
-                       !lhs_w && !rhs_w && wgs <= 4 * cus &&
-                       macs <= (all_vec ? MH_FUSED_SMALL_MAX_MACS : MH_FUSED_SMALL_MAX_MACS_BYTEWISE) &&
-                       !getenv("MH_NO_FUSED");
+    const bool rhs_vec = cv ? (cv->cin % 16 == 0 && (uintptr_t)rhs % 16 == 0)
+                            : (rhs_t ? (cols % 16 == 0 && (uintptr_t)rhs % 16 == 0) : rhs_direct);
+    // (a registered weight keeps its sums and panel for the tiled kernels; the gather has no
+    // other kernel for a geometry that is not a multiple of 64 channels, so it always comes here)
+    const bool small = cv ? cv_small
+                          : (mh_q8_small_problem(ctx, batch, rows, cols, depth, lhs_vec && rhs_vec) &&
+                             !lhs_w && !rhs_w && !getenv("MH_NO_FUSED"));
     if (small) {
       GemmParams p{};
       const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
@@ -1356,15 +1407,25 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
       p.XN = (int)(xl ? rows : cols);
       p.YN = (int)(xl ? cols : rows);
       p.K = (int)depth;
-      p.ldx = xt ? p.XN : depth;    // k-major: bytes between consecutive k
-      p.ldy = yt ? p.YN : depth;
-      p.xbs = ((xl ? lhs_nb : rhs_nb) > 1) ? (int64_t)p.XN * depth : 0;
-      p.ybs = ((xl ? rhs_nb : lhs_nb) > 1) ? (int64_t)p.YN * depth : 0;
+      // row pitch: k-major: bytes between consecutive k; k-contiguous: depth, or the pitch of a
+      // caller-padded right-hand panel (whose padding bytes are zero after the shift)
+      const int64_t rhs_pitch = rhs_ld != 0 ? rhs_ld : depth;
+      p.ldx = xt ? p.XN : (xl ? depth : rhs_pitch);
+      p.ldy = yt ? p.YN : (xl ? rhs_pitch : depth);
+      p.xbs = ((xl ? lhs_nb : rhs_nb) > 1) ? (int64_t)p.XN * (xl ? depth : rhs_pitch) : 0;
+      p.ybs = ((xl ? rhs_nb : lhs_nb) > 1) ? (int64_t)p.YN * (xl ? rhs_pitch : depth) : 0;
       p.out = out;
       p.ldo = p.XN;
       p.obs = rows * cols;
       p.rq = rq;
       p.sum_y = true;
+      if (cv) {
+        p.conv = true;
+        p.cv_in_h = cv->in_h; p.cv_in_w = cv->in_w; p.cv_cin = cv->cin; p.cv_kw = cv->k_w;
+        p.cv_sh = cv->stride_h; p.cv_sw = cv->stride_w; p.cv_pt = cv->pad_top; p.cv_pl = cv->pad_left;
+        p.cv_oh = cv->out_h; p.cv_ow = cv->out_w;
+        p.cv_zp4 = (uint32_t)(cv->zero_point & 0xff) * 0x01010101u;
+      }
       p.x_bytewise = !(xl ? lhs_vec : rhs_vec);
       p.y_bytewise = !(xl ? rhs_vec : lhs_vec);
       p.xcoef = xl ? l_coef : r_coef;
