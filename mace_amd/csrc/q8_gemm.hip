@@ -1360,7 +1360,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   const bool cv_small = cv && rhs_ld == 0 && batch == 1 && out_order == MACE_HIP_COL_MAJOR &&
                         lhs_order == MACE_HIP_ROW_MAJOR &&
                         mh_q8_small_problem(ctx, 1, rows, cols, depth, cv_vec) &&
-                        !getenv("MH_NO_FUSED");
+                        !getenv("MACE_HIP_NO_SMALL_KERNEL");
   MH_CHECK(ctx, !cv || cv_small ||
                     (rhs_ld == 0 && batch == 1 && out_order == MACE_HIP_COL_MAJOR &&
                      lhs_order == MACE_HIP_ROW_MAJOR && depth % SLAB == 0 && depth >= 3 * SLAB &&
@@ -1390,11 +1390,13 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     const bool lhs_vec = lhs_t ? (rows % 16 == 0 && (uintptr_t)lhs % 16 == 0) : lhs_direct;
     const bool rhs_vec = cv ? (cv->cin % 16 == 0 && (uintptr_t)rhs % 16 == 0)
                             : (rhs_t ? (cols % 16 == 0 && (uintptr_t)rhs % 16 == 0) : rhs_direct);
+    // The environment variable MACE_HIP_NO_SMALL_KERNEL (any value) sends every call down the
+    // general path instead: a diagnostic switch, used by the tests to keep both paths covered.
     // (a registered weight keeps its sums and panel for the tiled kernels; the gather has no
     // other kernel for a geometry that is not a multiple of 64 channels, so it always comes here)
     const bool small = cv ? cv_small
                           : (mh_q8_small_problem(ctx, batch, rows, cols, depth, lhs_vec && rhs_vec) &&
-                             !lhs_w && !rhs_w && !getenv("MH_NO_FUSED"));
+                             !lhs_w && !rhs_w && !getenv("MACE_HIP_NO_SMALL_KERNEL"));
     if (small) {
       GemmParams p{};
       const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;

@@ -80,8 +80,18 @@ CASES = [  # batch, cout, cin, in_h, in_w, k_h, k_w, padding, strides: the refer
 ]
 
 
+@pytest.fixture(params=["default", "general_path"])
+def path(request, monkeypatch):
+    """A small convolution is one launch of the small-problem GEMM kernel, which gathers the
+    patches itself; MACE_HIP_NO_SMALL_KERNEL sends it through im2col / the gathering tiled kernel
+    instead, so that those stay covered on the same shapes."""
+    if request.param == "general_path":
+        monkeypatch.setenv("MACE_HIP_NO_SMALL_KERNEL", "1")
+    return request.param
+
+
 @pytest.mark.parametrize("n,cout,cin,in_h,in_w,k_h,k_w,pad,st", CASES)
-def test_conv2d_q8_parity(ctx, n, cout, cin, in_h, in_w, k_h, k_w, pad, st):
+def test_conv2d_q8_parity(ctx, path, n, cout, cin, in_h, in_w, k_h, k_w, pad, st):
     rng = np.random.default_rng(cout * 31 + cin + k_h * 7 + k_w + pad + st[0])
     x = rng.integers(0, 256, (n, in_h, in_w, cin), dtype=np.uint8)
     f = rng.integers(1, 256, (cout, k_h, k_w, cin), dtype=np.uint8)

@@ -57,10 +57,19 @@ SHAPES = [  # batch, rows, depth, cols, lhs_batched, rhs_batched
 ]
 
 
+@pytest.fixture(params=["default", "general_path"])
+def path(request, monkeypatch):
+    """Small problems are one launch of a kernel of their own; MACE_HIP_NO_SMALL_KERNEL sends them
+    through the general path (repack, row sums, tiled kernel) so that both stay covered."""
+    if request.param == "general_path":
+        monkeypatch.setenv("MACE_HIP_NO_SMALL_KERNEL", "1")
+    return request.param
+
+
 @pytest.mark.parametrize("batch,rows,depth,cols,lb,rb", SHAPES)
 @pytest.mark.parametrize("lo,ro,oo", [(R, R, R), (R, Cm, R), (Cm, R, R), (Cm, Cm, R),
                                       (R, Cm, Cm), (Cm, R, Cm), (R, R, Cm), (Cm, Cm, Cm)])
-def test_q8_gemm_parity(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo):
+def test_q8_gemm_parity(ctx, path, batch, rows, depth, cols, lb, rb, lo, ro, oo):
     rng = np.random.default_rng(rows * 31 + depth * 7 + cols + lo * 4 + ro * 2 + oo)
     L = rng.integers(0, 256, ((batch if lb else 1), rows, depth), dtype=np.uint8)
     Rr = rng.integers(0, 256, ((batch if rb else 1), depth, cols), dtype=np.uint8)
