@@ -48,6 +48,12 @@ GEMM_CASES += [(3, 47, 69, 37, R, R, R, True, False), (3, 47, 69, 37, R, R, R, F
 GEMM_CASES += [(2, 256, 128, 48, lm, rm, om, True, True)
                for lm in (R, Cm) for rm in (R, Cm) for om in (R, Cm)]
 GEMM_CASES += [(3, 128, 384, 80, Cm, R, R, False, True), (3, 384, 128, 16, R, Cm, Cm, True, False)]
+# the shapes of the Gemm call the reference's Winograd convolution makes
+# (mace/ops/arm/base/conv_2d_3x3_winograd.cc:191-204: batch = transformed tile area 16 or 64,
+# rows = output channels, depth = input channels, cols = number of tiles, all row-major, both
+# operands batched)
+GEMM_CASES += [(16, 32, 49, 16, R, R, R, True, True), (64, 64, 196, 32, R, R, R, True, True),
+               (16, 24, 9, 3, R, R, R, True, True), (64, 128, 256, 128, R, R, R, True, True)]
 
 
 @pytest.mark.parametrize("batch,rows,cols,depth,lm,rm,om,lb,rb", GEMM_CASES)
@@ -114,6 +120,10 @@ GEMV_CASES = [(1, 16, 4, True, True), (1, 16, 256, True, True), (2, 16, 256, Tru
               (3, 63, 257, True, True), (2, 16, 256, False, True), (3, 63, 257, False, True),
               (2, 16, 256, True, False), (3, 63, 257, True, False), (1, 253, 30001, False, True),
               (2, 300, 253, True, True)]
+# the two Gemv calls of the reference's DynamicLSTM step (mace/ops/dynamic_lstm.cc:301-310,
+# 328-337): batch 1, nothing batched, bias; affine a: [4 cell + ...] x [input + recurrent],
+# affine b: [output] x [cell]
+GEMV_CASES += [(1, 2048, 296, False, False), (1, 640, 512, False, False), (1, 1025, 115, False, False)]
 
 
 @pytest.mark.parametrize("batch,h,w,lb,rb", GEMV_CASES)
