@@ -471,6 +471,24 @@ class MatMulOpFloat {
 // uses the pipeline MakeNoBias(A.scale, B.scale, C.scale, C.zero_point), the int32 result
 // sets C.scale = A.scale * B.scale and C.zero_point = 0.  The gemmlowp call is not behind a
 // delegator in the reference, so the op calls the C ABI directly.
+// MatMulOp's constructor passes is_weight() of either operand to the Gemm delegator as
+// GemmParam::should_cache_pack_ (mace/ops/matmul.cc:101-108), which then keeps the packed operand
+// (arm/base/gemm.cc:560-576).  Counterpart: an operand that is a constant weight AND lives in device
+// memory is registered with the context once per op instance; its repacked panel and row sums are
+// then kept across Run() calls.  A weight whose buffer moves is registered afresh.
+class WeightRegistration {
+ public:
+  void Note(OpContext *context, const Tensor *t, size_t bytes) {
+    if (!t->is_weight() || !t->on_device()) return;
+    const void *ptr = t->data<uint8_t>();
+    if (ptr == registered_) return;
+    if (mace_hip_weight_register(context->hip(), ptr, bytes) == MACE_HIP_SUCCESS) registered_ = ptr;
+  }
+
+ private:
+  const void *registered_ = nullptr;
+};
+
 class MatMulOpQuant {
  public:
   MatMulOpQuant(bool transpose_a, bool transpose_b, DataType output_type)
@@ -482,6 +500,8 @@ class MatMulOpQuant {
     if ((st = C->Resize(s.output_shape)) != MaceStatus::MACE_SUCCESS) return st;
     const int a_order = transpose_a_ ? MACE_HIP_COL_MAJOR : MACE_HIP_ROW_MAJOR;
     const int b_order = transpose_b_ ? MACE_HIP_COL_MAJOR : MACE_HIP_ROW_MAJOR;
+    weight_a_.Note(context, A, static_cast<size_t>(A->size()));
+    weight_b_.Note(context, B, static_cast<size_t>(B->size()));
     if (output_type_ == DT_INT32) {
       C->SetScale(A->scale() * B->scale());
       C->SetZeroPoint(0);
@@ -506,6 +526,7 @@ class MatMulOpQuant {
  private:
   bool transpose_a_, transpose_b_;
   DataType output_type_;
+  WeightRegistration weight_a_, weight_b_;
 };
 
 // FullyConnectedOp<RT_CPU, uint8_t>::Run (mace/ops/fully_connected.cc:141-179) and the float op
@@ -580,6 +601,7 @@ class Conv2dOpQuant {
     }
     MaceStatus st = output->Resize({input->dim(0), out_h, out_w, filter->dim(0)});
     if (st != MaceStatus::MACE_SUCCESS) return st;
+    weight_.Note(context, filter, static_cast<size_t>(filter->size()));   // filters are constants
     auto fn = output->on_device() ? mace_hip_conv2d_q8_nhwc : mace_hip_conv2d_q8_nhwc_host;
     return ToStatus(fn(context->hip(), input->data<uint8_t>(), filter->data<uint8_t>(),
                        bias ? bias->data<int32_t>() : nullptr, input->dim(0), input->dim(1),
@@ -595,6 +617,7 @@ class Conv2dOpQuant {
   Padding padding_type_;
   std::vector<int> paddings_, dilations_;
   int clamp_min_, clamp_max_;
+  WeightRegistration weight_;
 };
 
 // The 1x1 / stride 1 / no padding case under its earlier name.

@@ -187,6 +187,35 @@ static int test_compute() {
     Tensor Cbad(c8.data(), DT_UINT8, {}, 1e-6f, 128);   // multiplier >= 1: the reference CHECKs
     EXPECT(op8.Run(&context, &A, &B, &Cbad) == MaceStatus::MACE_INVALID_ARGS);
 
+    // The same MatMul on device-resident tensors with B flagged as a constant weight: the op
+    // registers it once (matmul.cc:101-108 passes is_weight() as should_cache_pack_), the second
+    // Run() reuses its panel and sums, the result stays bit-exact.
+    {
+      mace_hip_ctx *h = context.hip();
+      void *da = nullptr, *db = nullptr, *dc = nullptr;
+      EXPECT(mace_hip_malloc(h, a.size(), &da) == MACE_HIP_SUCCESS);
+      EXPECT(mace_hip_malloc(h, b.size(), &db) == MACE_HIP_SUCCESS);
+      EXPECT(mace_hip_malloc(h, c8.size(), &dc) == MACE_HIP_SUCCESS);
+      EXPECT(mace_hip_memcpy_h2d(h, da, a.data(), a.size()) == MACE_HIP_SUCCESS);
+      EXPECT(mace_hip_memcpy_h2d(h, db, b.data(), b.size()) == MACE_HIP_SUCCESS);
+      Tensor dA(da, DT_UINT8, {batch, depth, rows}, 0.02f, 77, false, true);
+      Tensor dB(db, DT_UINT8, {cols, depth}, 0.015f, 201, /*is_weight=*/true, /*on_device=*/true);
+      Tensor dC(dc, DT_UINT8, {}, 40.f, 128, false, true);
+      ops::MatMulOpQuant dev_op(true, true, DT_UINT8);
+      int64_t builds0 = 0, hits0 = 0, builds1 = 0, hits1 = 0;
+      EXPECT(mace_hip_weight_cache_stats(h, &builds0, &hits0) == MACE_HIP_SUCCESS);
+      for (int run = 0; run < 3; ++run) {
+        EXPECT(dev_op.Run(&context, &dA, &dB, &dC) == MaceStatus::MACE_SUCCESS);
+        std::vector<uint8_t> got(c8.size());
+        EXPECT(mace_hip_memcpy_d2h(h, got.data(), dc, got.size()) == MACE_HIP_SUCCESS);
+        EXPECT(got == want8);
+      }
+      EXPECT(mace_hip_weight_cache_stats(h, &builds1, &hits1) == MACE_HIP_SUCCESS);
+      EXPECT(builds1 - builds0 == 1 && hits1 - hits0 == 2);
+      EXPECT(mace_hip_weight_unregister(h, db) == MACE_HIP_SUCCESS);
+      mace_hip_free(h, da); mace_hip_free(h, db); mace_hip_free(h, dc);
+    }
+
     const index_t n = 2, o = 40, isz = 7 * 7 * 32;
     std::vector<uint8_t> x(n * isz), w(o * isz), y(n * o), wanty(n * o);
     std::vector<int32_t> bias(o);
