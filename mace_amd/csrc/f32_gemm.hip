@@ -161,24 +161,32 @@ __global__ void f32_fill_kernel(F32GemmParams p, int64_t total) {
 // guarded 4-byte loads and their addresses, in front of 32 MFMAs).
 typedef float f4v __attribute__((ext_vector_type(4)));
 
-template <bool LK, bool RK>
-__global__ __launch_bounds__(256) void f32_gemm_vec_kernel(F32GemmParams p) {
+//
+// SPLIT = 2: eight wavefronts per tile instead of four.  Wavefronts 4..7 cover the same four
+// 64 x 64 quarters as 0..3 but take the second half of every k tile's k steps; their sums are
+// added to the first half's through LDS at the end (a fixed order).  Used when the launch has
+// no more tiles than CUs: one wavefront per SIMD leaves every LDS wait and barrier exposed
+// (matrix core busy 69 % of the time on 4 x 1024^3), two hide each other's.
+template <bool LK, bool RK, int SPLIT>
+__global__ __launch_bounds__(256 * SPLIT) void f32_gemm_vec_kernel(F32GemmParams p) {
+  constexpr int NT = 256 * SPLIT;
   __shared__ __align__(16) float sA[2][TK][LDT];
   __shared__ __align__(16) float sB[2][TK][LDT];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave & 1, wn = wave >> 1;
+  const int khalf = wave >> 2;           // which part of the k steps (0 when SPLIT == 1)
+  const int wm = wave & 1, wn = (wave >> 1) & 1;
   const int m0 = (blockIdx.x % p.tiles_m) * TM, n0 = (blockIdx.x / p.tiles_m) * TN;
   const int b = blockIdx.z;
   const float *A = p.lhs + (int64_t)b * p.lbs;
   const float *B = p.rhs + (int64_t)b * p.rbs;
 
   // NP 16-byte pieces per operand per thread and k tile; KQ pieces along k per row
-  constexpr int NP = TM * TK / 4 / 256, KQ = TK / 4;
+  constexpr int NP = TM * TK / 4 / NT, KQ = TK / 4;
   const float *pa[NP], *pb[NP];
   int sa_off[NP], sb_off[NP];   // float offset of the piece inside one LDS buffer
 #pragma unroll
   for (int i = 0; i < NP; ++i) {
-    const int f = tid + i * 256;
+    const int f = tid + i * NT;
     if (LK) {   // 4 consecutive k of row m
       const int m = f / KQ, k4 = f % KQ;
       pa[i] = A + (int64_t)(m0 + m) * p.lrs + 4 * k4;
@@ -256,23 +264,48 @@ __global__ __launch_bounds__(256) void f32_gemm_vec_kernel(F32GemmParams p) {
 #pragma unroll
       for (int j = 0; j < 2; ++j) bb[slot][j] = sB[buf][kk][wn * 64 + j * 32 + (lane & 31)];
     };
-    read_frags(0, 0);
+    constexpr int KS = TK / 2 / SPLIT;   // k steps of this wavefront per k tile
+    const int ks0 = khalf * KS;
+    read_frags(ks0, 0);
 #pragma unroll
-    for (int ks = 0; ks < TK / 2; ++ks) {
-      if (ks + 1 < TK / 2) read_frags(ks + 1, (ks + 1) & 1);
+    for (int ks = 0; ks < KS; ++ks) {
+      if (ks + 1 < KS) read_frags(ks0 + ks + 1, (ks + 1) & 1);
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ks & 1][i], bb[ks & 1][j], acc[i][j],
                                                            0, 0, 0);
-      if (ks == TK / 4 - 1 && kt + 1 < nk) {
+      if (ks == KS / 2 - 1 && kt + 1 < nk) {
         store_lds(buf ^ 1);
         if (kt + 2 < nk) load_global();
       }
       __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();
+  }
+
+  if constexpr (SPLIT == 2) {
+    // second half's sums -> first half, one accumulator block (16 values per lane) at a time
+    // through the A buffers (every wavefront is past the last barrier of the loop)
+    float *ex = &sA[0][0][0];
+    static_assert(sizeof(sA) >= 4 * 64 * 16 * sizeof(float), "exchange area");
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if (khalf == 1) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) ex[((wave & 3) * 16 + r) * 64 + lane] = acc[i][j][r];
+        }
+        __syncthreads();
+        if (khalf == 0) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[i][j][r] += ex[((wave & 3) * 16 + r) * 64 + lane];
+        }
+        __syncthreads();
+      }
+    if (khalf == 1) return;
   }
 
   float *O = p.out + (int64_t)b * p.obs;
@@ -358,16 +391,22 @@ int mh_f32_gemm(mace_hip_ctx *ctx, const float *lhs, const float *rhs, int64_t b
   p.tiles_m = (p.M + TM - 1) / TM;
   const int64_t tiles = (int64_t)p.tiles_m * ((p.N + TN - 1) / TN);
   MH_CHECK(ctx, tiles < (1ll << 31), "too many tiles");
-  dim3 grid((unsigned)tiles, 1, (unsigned)batch), block(256);
+  dim3 grid((unsigned)tiles, 1, (unsigned)batch), block(256), block2(512);
+  const int64_t cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
+  const bool split = tiles * batch <= cus;   // at most one tile per CU
   const bool lk = lhs_major == MACE_HIP_ROW_MAJOR;   // depth contiguous
   const bool rk = rhs_major == MACE_HIP_COL_MAJOR;
   MH_PROF_BEGIN(ctx);
   const bool vec = rows % TM == 0 && cols % TN == 0 && depth % TK == 0 &&
                    ((uintptr_t)lhs % 16 == 0) && ((uintptr_t)rhs % 16 == 0);
-  if (vec && lk && rk) hipLaunchKernelGGL((f32_gemm_vec_kernel<true, true>), grid, block, 0, ctx->stream, p);
-  else if (vec && lk) hipLaunchKernelGGL((f32_gemm_vec_kernel<true, false>), grid, block, 0, ctx->stream, p);
-  else if (vec && rk) hipLaunchKernelGGL((f32_gemm_vec_kernel<false, true>), grid, block, 0, ctx->stream, p);
-  else if (vec) hipLaunchKernelGGL((f32_gemm_vec_kernel<false, false>), grid, block, 0, ctx->stream, p);
+  if (vec && split && lk && rk) hipLaunchKernelGGL((f32_gemm_vec_kernel<true, true, 2>), grid, block2, 0, ctx->stream, p);
+  else if (vec && split && lk) hipLaunchKernelGGL((f32_gemm_vec_kernel<true, false, 2>), grid, block2, 0, ctx->stream, p);
+  else if (vec && split && rk) hipLaunchKernelGGL((f32_gemm_vec_kernel<false, true, 2>), grid, block2, 0, ctx->stream, p);
+  else if (vec && split) hipLaunchKernelGGL((f32_gemm_vec_kernel<false, false, 2>), grid, block2, 0, ctx->stream, p);
+  else if (vec && lk && rk) hipLaunchKernelGGL((f32_gemm_vec_kernel<true, true, 1>), grid, block, 0, ctx->stream, p);
+  else if (vec && lk) hipLaunchKernelGGL((f32_gemm_vec_kernel<true, false, 1>), grid, block, 0, ctx->stream, p);
+  else if (vec && rk) hipLaunchKernelGGL((f32_gemm_vec_kernel<false, true, 1>), grid, block, 0, ctx->stream, p);
+  else if (vec) hipLaunchKernelGGL((f32_gemm_vec_kernel<false, false, 1>), grid, block, 0, ctx->stream, p);
   else if (lk && rk) hipLaunchKernelGGL((f32_gemm_kernel<true, true>), grid, block, 0, ctx->stream, p);
   else if (lk) hipLaunchKernelGGL((f32_gemm_kernel<true, false>), grid, block, 0, ctx->stream, p);
   else if (rk) hipLaunchKernelGGL((f32_gemm_kernel<false, true>), grid, block, 0, ctx->stream, p);
