@@ -170,8 +170,8 @@ typedef float f4v __attribute__((ext_vector_type(4)));
 template <bool LK, bool RK, int SPLIT>
 __global__ __launch_bounds__(256 * SPLIT) void f32_gemm_vec_kernel(F32GemmParams p) {
   constexpr int NT = 256 * SPLIT;
-  __shared__ __align__(16) float sA[2][TK][LDT];
-  __shared__ __align__(16) float sB[2][TK][LDT];
+  __shared__ __align__(16) float sA[3][TK][LDT];
+  __shared__ __align__(16) float sB[3][TK][LDT];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int khalf = wave >> 2;           // which part of the k steps (0 when SPLIT == 1)
   const int wm = wave & 1, wn = (wave >> 1) & 1;
@@ -245,44 +245,56 @@ __global__ __launch_bounds__(256 * SPLIT) void f32_gemm_vec_kernel(F32GemmParams
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // Tile kt + 1 sits in registers while tile kt is multiplied (it was requested a whole
-  // iteration earlier); it goes to LDS, and the request for tile kt + 2 goes out, in the middle
-  // of the MFMA sequence, so that neither the LDS stores nor the load issue leave the matrix
-  // core idle.  The other LDS buffer is free then: everybody passed the last barrier.
+  // Three LDS buffers.  While tile kt is multiplied, tile kt + 1 is already in LDS (stored during
+  // tile kt - 1, visible since the barrier that ended it), tile kt + 2 sits in registers (requested
+  // a whole iteration earlier) and goes to LDS in the middle of the MFMA sequence, where the
+  // request for tile kt + 3 goes out too.  The first fragments of tile kt + 1 can therefore be
+  // read during the last k step of tile kt, in front of the barrier, and no LDS latency is
+  // exposed behind it.  The buffer written (tile kt + 2's = tile kt - 1's) is free: everybody
+  // passed the barrier that ended tile kt - 1.
   const int nk = p.K / TK;
   load_global();
   store_lds(0);
-  if (nk > 1) load_global();
+  if (nk > 1) {
+    load_global();
+    store_lds(1);
+  }
+  if (nk > 2) load_global();
   __syncthreads();
+  constexpr int KS = TK / 2 / SPLIT;   // k steps of this wavefront per k tile
+  const int ks0 = khalf * KS;
+  float a[2][2], bb[2][2];
+  auto read_frags = [&](int buf, int ks, int slot) {
+    const int kk = ks * 2 + (lane >> 5);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) a[slot][i] = sA[buf][kk][wm * 64 + i * 32 + (lane & 31)];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) bb[slot][j] = sB[buf][kk][wn * 64 + j * 32 + (lane & 31)];
+  };
+  static_assert(KS % 2 == 0, "fragment slots alternate; a tile must end on slot 1");
+  read_frags(0, ks0, 0);
+  int buf = 0;
   for (int kt = 0; kt < nk; ++kt) {
-    const int buf = kt & 1;
-    float a[2][2], bb[2][2];
-    auto read_frags = [&](int ks, int slot) {
-      const int kk = ks * 2 + (lane >> 5);
-#pragma unroll
-      for (int i = 0; i < 2; ++i) a[slot][i] = sA[buf][kk][wm * 64 + i * 32 + (lane & 31)];
-#pragma unroll
-      for (int j = 0; j < 2; ++j) bb[slot][j] = sB[buf][kk][wn * 64 + j * 32 + (lane & 31)];
-    };
-    constexpr int KS = TK / 2 / SPLIT;   // k steps of this wavefront per k tile
-    const int ks0 = khalf * KS;
-    read_frags(ks0, 0);
+    const int buf1 = buf == 2 ? 0 : buf + 1;    // tile kt + 1
+    const int buf2 = buf1 == 2 ? 0 : buf1 + 1;  // tile kt + 2 (= where tile kt - 1 was)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      if (ks + 1 < KS) read_frags(ks0 + ks + 1, (ks + 1) & 1);
+      if (ks + 1 < KS) read_frags(buf, ks0 + ks + 1, (ks + 1) & 1);
+      else read_frags(buf1, ks0, 0);   // past the last tile: stale data, never used
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ks & 1][i], bb[ks & 1][j], acc[i][j],
                                                            0, 0, 0);
-      if (ks == KS / 2 - 1 && kt + 1 < nk) {
-        store_lds(buf ^ 1);
-        if (kt + 2 < nk) load_global();
+      if (ks == KS / 2 - 1 && kt + 2 < nk) {
+        store_lds(buf2);
+        if (kt + 3 < nk) load_global();
       }
       __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();
+    buf = buf1;
   }
 
   if constexpr (SPLIT == 2) {
@@ -290,6 +302,7 @@ __global__ __launch_bounds__(256 * SPLIT) void f32_gemm_vec_kernel(F32GemmParams
     // through the A buffers (every wavefront is past the last barrier of the loop)
     float *ex = &sA[0][0][0];
     static_assert(sizeof(sA) >= 4 * 64 * 16 * sizeof(float), "exchange area");
+    __syncthreads();   // the fragment reads in front of the last barrier are done with
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
