@@ -1661,6 +1661,11 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   // (+5 % at 8192^3) and long-k 128 x 128 tiles; short k gains nothing from them
   if (p.K % 128 == 0 && p.K >= 256 && !p.conv && dma_ok) {
     if (big) return launch_gemm_dma<2, 2, 4, 4, 2, 1, 128>(ctx, p, tab, out_u8, (int)batch);
+    // Between half a round and one round of 128 x 128 tiles every CU has one workgroup and every
+    // SIMD one wavefront, with nothing to overlap its waits: eight wavefronts of 64 x 32 results
+    // instead of four of 64 x 64 (2048^3: -6 %; with a quarter of the CUs busy it is slower)
+    if (medium && p.K >= 1024 && tiles(128, 128) <= cu && 2 * tiles(128, 128) > cu)
+      return launch_gemm_dma<2, 4, 2, 1, 2, 1, 128>(ctx, p, tab, out_u8, (int)batch);
     if (medium && p.K >= 1024)
       return launch_gemm_dma<2, 2, 2, 2, 2, 2, 128>(ctx, p, tab, out_u8, (int)batch);
   }
