@@ -220,6 +220,8 @@ def test_q8_gemm_large_device_pointers(ctx, n, lo, ro, oo):
     (2, 2100, 640, 2200, R, Cm, R, True),     # ... batched
     (1, 1100, 1024, 1300, R, Cm, R, True),    # 128 x 128 tiles, 128-byte slabs
     (1, 1100, 1152, 1300, R, R, Cm, False),   # ... through the repack, column-major result
+    (1, 1700, 1024, 1800, R, Cm, R, True),    # ... 210 tiles: the eight-wavefront variant, ragged
+    (1, 1800, 1152, 1700, R, Cm, Cm, False),  # ... column-major result
     (1, 2049, 448, 2305, R, Cm, R, True),     # 128 x 128 tiles, 64-byte slabs (k % 128 != 0)
     (1, 4352, 256, 4608, R, Cm, R, True),     # 17 x 18 aligned 256 x 256 tiles: more than one per CU
     (1, 4608, 384, 4352, R, Cm, Cm, False),   # ... odd number of slabs, column-major result
