@@ -264,8 +264,63 @@ static int test_compute() {
   return g_fail;
 }
 
+// Per-call cost of small ops from a C++ caller (what MACE's engine thread would see): device
+// tensors, back-to-back calls, HIP events on the context's stream.  Prints, checks nothing.
+static int time_small_calls() {
+  mace_hip_ctx *h = nullptr;
+  if (mace_hip_ctx_create(0, &h) != MACE_HIP_SUCCESS) return 1;
+  struct Case { const char *name; int64_t m, k, n; int b_order; };
+  const Case cases[] = {{"uint8 MatMul 128x256 . 256x128 (B row-major)", 128, 256, 128, MACE_HIP_ROW_MAJOR},
+                        {"uint8 MatMul 256x256 . 256x256 (B k-contiguous)", 256, 256, 256, MACE_HIP_COL_MAJOR},
+                        {"uint8 MatMul 1024x512 . 512x1024 (B row-major)", 1024, 512, 1024, MACE_HIP_ROW_MAJOR}};
+  int32_t mult = 0; int shift = 0;
+  mace_hip_get_output_multiplier_and_shift(0.02f, 0.015f, 0.05f, &mult, &shift);
+  for (const Case &c : cases) {
+    void *a = nullptr, *b = nullptr, *o = nullptr;
+    mace_hip_malloc(h, (size_t)(c.m * c.k), &a);
+    mace_hip_malloc(h, (size_t)(c.k * c.n), &b);
+    mace_hip_malloc(h, (size_t)(c.m * c.n), &o);
+    std::vector<uint8_t> init((size_t)std::max(c.m * c.k, c.k * c.n), 77);
+    mace_hip_memcpy_h2d(h, a, init.data(), (size_t)(c.m * c.k));
+    mace_hip_memcpy_h2d(h, b, init.data(), (size_t)(c.k * c.n));
+    auto call = [&]() {
+      return mace_hip_gemm_q8_u8(h, (const uint8_t *)a, MACE_HIP_ROW_MAJOR, (const uint8_t *)b, c.b_order,
+                                 (uint8_t *)o, MACE_HIP_ROW_MAJOR, 1, c.m, c.k, c.n, 1, 1, -128, -128,
+                                 nullptr, mult, shift, 128, 0, 255);
+    };
+    for (int i = 0; i < 20; ++i) call();
+    mace_hip_sync(h);
+    const int reps = 2000;
+    float ms = 0.f;
+    mace_hip_timer_start(h);
+    for (int i = 0; i < reps; ++i) call();
+    mace_hip_timer_stop(h, &ms);
+    printf("%-52s %6.2f us per call\n", c.name, ms * 1e3 / reps);
+    mace_hip_free(h, a); mace_hip_free(h, b); mace_hip_free(h, o);
+  }
+  {  // the floor: a kernel with next to nothing to do (Quantize of 256 floats)
+    void *x = nullptr, *q = nullptr;
+    mace_hip_malloc(h, 1024, &x);
+    mace_hip_malloc(h, 256, &q);
+    std::vector<float> init(256, 1.5f);
+    mace_hip_memcpy_h2d(h, x, init.data(), 1024);
+    for (int i = 0; i < 20; ++i) mace_hip_quantize_tensor_u8(h, (const float *)x, 256, 0.03f, 128, (uint8_t *)q);
+    mace_hip_sync(h);
+    const int reps = 2000;
+    float ms = 0.f;
+    mace_hip_timer_start(h);
+    for (int i = 0; i < reps; ++i) mace_hip_quantize_tensor_u8(h, (const float *)x, 256, 0.03f, 128, (uint8_t *)q);
+    mace_hip_timer_stop(h, &ms);
+    printf("%-52s %6.2f us per call\n", "Quantize of 256 floats (launch floor)", ms * 1e3 / reps);
+    mace_hip_free(h, x); mace_hip_free(h, q);
+  }
+  mace_hip_ctx_destroy(h);
+  return 0;
+}
+
 int main(int argc, char **argv) {
   const char *mode = argc > 1 ? argv[1] : "registry";
+  if (strcmp(mode, "time") == 0) return time_small_calls();
   int fails = strcmp(mode, "compute") == 0 ? test_compute() : test_registry();
   printf("%s: %s (%d failures)\n", mode, fails ? "FAILED" : "ok", fails);
   return fails ? 1 : 0;
