@@ -379,6 +379,10 @@ inline bool mh_q8_small_problem(const mace_hip_ctx *ctx, int64_t batch, int64_t 
          macs <= (vec ? 1024.0 : 128.0) * 1024 * 1024;
 }
 
+// Fills device memory with one byte value on the context's stream, with a kernel (a memset node
+// recorded into a caller's graph capture has replayed wrongly on this hardware pool).
+int mh_fill_bytes(mace_hip_ctx *ctx, void *dst, uint8_t value, size_t bytes);
+
 int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8_t *rhs,
                int rhs_order, void *out, int out_order, bool out_u8, int64_t batch,
                int64_t rows, int64_t depth, int64_t cols, int lhs_batched, int rhs_batched,

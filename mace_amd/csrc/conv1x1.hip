@@ -184,7 +184,7 @@ extern "C" int mace_hip_conv2d_q8_nhwc(mace_hip_ctx *ctx, const uint8_t *input,
     const uint32_t zp4 = (uint32_t)input_zp * 0x01010101u;
     const bool fast = cin % 16 == 0 && cin > 0 && ((uintptr_t)input % 16 == 0);
     if (depth == 0) {
-      MH_HIP(ctx, hipMemsetAsync(cols, 0x80, (size_t)columns * kp, ctx->stream));
+      MH_RETURN_IF_ERROR(mh_fill_bytes(ctx, cols, 0x80, (size_t)columns * kp));
     } else if (fast) {
       hipLaunchKernelGGL(q8_im2col_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, ctx->stream,
                          input, cols, chunks, cpr, (int)kp, (int)depth, (int)in_h, (int)in_w,

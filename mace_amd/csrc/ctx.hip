@@ -54,6 +54,22 @@ void *mh_arena_take(mace_hip_ctx *ctx, size_t bytes) {
   return ctx->arena + at;
 }
 
+namespace {
+__global__ __launch_bounds__(256) void mh_fill_bytes_kernel(uint8_t *dst, uint8_t value, size_t bytes) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < bytes; i += (size_t)gridDim.x * 256)
+    dst[i] = value;
+}
+}  // namespace
+
+int mh_fill_bytes(mace_hip_ctx *ctx, void *dst, uint8_t value, size_t bytes) {
+  if (bytes == 0) return MACE_HIP_SUCCESS;
+  const size_t blocks = (bytes + 255) / 256;
+  hipLaunchKernelGGL(mh_fill_bytes_kernel, dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256), 0,
+                     ctx->stream, (uint8_t *)dst, value, bytes);
+  MH_HIP(ctx, hipGetLastError());
+  return MACE_HIP_SUCCESS;
+}
+
 extern "C" {
 
 int mace_hip_ctx_create(int device, mace_hip_ctx **out) {

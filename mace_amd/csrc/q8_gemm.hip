@@ -1533,7 +1533,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     uint8_t *dst = (uint8_t *)mh_arena_take(ctx, (size_t)nb * n * kp);
     if (!dst) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
     if (depth == 0) {
-      MH_HIP(ctx, hipMemsetAsync(dst, 0x80, (size_t)nb * n * kp, ctx->stream));
+      MH_RETURN_IF_ERROR(mh_fill_bytes(ctx, dst, 0x80, (size_t)nb * n * kp));
       *P = Panel{dst, kp, nb > 1 ? n * kp : 0, (int)kp, nullptr};
       return MACE_HIP_SUCCESS;
     }
@@ -1616,7 +1616,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     p.cv_oh = cv->out_h; p.cv_ow = cv->out_w;
     uint8_t *zero = (uint8_t *)mh_arena_take(ctx, 256);
     if (!zero) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
-    MH_HIP(ctx, hipMemsetAsync(zero, cv->zero_point, 256, ctx->stream));
+    MH_RETURN_IF_ERROR(mh_fill_bytes(ctx, zero, (uint8_t)cv->zero_point, 256));
     p.cv_zero = zero;
   }
   if (stream) {
