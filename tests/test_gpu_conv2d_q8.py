@@ -114,6 +114,42 @@ def test_conv2d_q8_parity(ctx, path, n, cout, cin, in_h, in_w, k_h, k_w, pad, st
         assert len(np.unique(want)) > 8
 
 
+def _random_conv_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        n = int(rng.integers(1, 4))
+        cin = int(rng.choice([1, 3, 8, 16, 24, 32, 48, 64, 128]))
+        cout = int(rng.choice([1, 7, 16, 32, 40, 64, 100, 128]))
+        k_h, k_w = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        in_h, in_w = int(rng.integers(k_h, 30)), int(rng.integers(k_w, 30))
+        st = (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+        pads = (int(rng.integers(0, k_h + 1)), int(rng.integers(0, k_w + 1)))
+        cases.append((n, cout, cin, in_h, in_w, k_h, k_w, pads, st, int(rng.integers(0, 1 << 30))))
+    return cases
+
+
+@pytest.mark.parametrize("n,cout,cin,in_h,in_w,k_h,k_w,pads,st,seed", _random_conv_cases(48, 77))
+def test_conv2d_q8_random_geometry(ctx, path, n, cout, cin, in_h, in_w, k_h, k_w, pads, st, seed):
+    """Seeded random geometries (channel counts on both sides of the 16- and 64-channel gather
+    conditions, filters 1..5, strides 1..3, arbitrary total paddings), in both modes."""
+    rng = np.random.default_rng(seed)
+    x = rng.integers(0, 256, (n, in_h, in_w, cin), dtype=np.uint8)
+    f = rng.integers(1, 256, (cout, k_h, k_w, cin), dtype=np.uint8)
+    bias = rng.integers(-2 ** 15, 2 ** 15, cout).astype(np.int32) if rng.integers(0, 2) else None
+    z_in, z_f = int(rng.integers(0, 256)), int(rng.integers(0, 256))
+    s_in, s_f = np.float32(0.02), np.float32(0.01)
+    depth = k_h * k_w * cin
+    s_out = np.float32(max(6.0, 3 * 74.0 * 74.0 * np.sqrt(depth) * float(s_in * s_f)) / 255.0)
+    s_b = np.float32(s_in * s_f) if bias is not None else np.float32(0)
+    z_o = int(rng.integers(0, 256))
+    want = orc.conv2d_q8_nhwc(x, f, bias, n, in_h, in_w, cin, cout, k_h, k_w, st, pads, s_in, z_in,
+                              s_f, z_f, s_b, s_out, z_o, 0, 255)
+    got = conv_host(ctx, x, f, bias, n, in_h, in_w, cin, cout, k_h, k_w, st, pads, s_in, z_in, s_f,
+                    z_f, s_b, s_out, z_o, 0, 255)
+    np.testing.assert_array_equal(got, want)
+
+
 def test_conv2d_q8_explicit_paddings_and_errors(ctx):
     """Asymmetric totals (odd paddings put the extra row / column at the bottom / right) and a
     padded 1x1 (which takes the gather path here)."""

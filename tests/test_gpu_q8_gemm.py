@@ -332,3 +332,41 @@ def test_q8_gemm_errors(ctx):
     ctx.call("mace_hip_ctx_fail_next_allocs", 0)
     assert st in (mh.OUT_OF_RESOURCES, mh.SUCCESS)   # SUCCESS only if the arena was already big
     assert ctx.status("mace_hip_gemm_q8_u8_host", *base, 2 ** 30, 1, 0, 0, 255) == mh.SUCCESS
+
+def _random_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    dims = [1, 2, 3, 15, 16, 17, 31, 32, 48, 63, 64, 65, 96, 127, 128, 129, 160, 200, 256, 257, 320, 400]
+    depths = [1, 3, 15, 16, 17, 27, 32, 48, 63, 64, 65, 100, 128, 129, 192, 256, 300, 320, 321, 500,
+              512, 640, 1000, 1024, 1025, 1100]
+    cases = []
+    for _ in range(count):
+        cases.append((int(rng.integers(1, 4)), int(rng.choice(dims)), int(rng.choice(depths)),
+                      int(rng.choice(dims)), int(rng.integers(0, 2)), int(rng.integers(0, 2)),
+                      int(rng.integers(0, 2)), bool(rng.integers(0, 4)), bool(rng.integers(0, 4)),
+                      int(rng.integers(0, 1 << 30))))
+    return cases
+
+
+@pytest.mark.parametrize("batch,rows,depth,cols,lo,ro,oo,lb,rb,seed", _random_cases(96, 2024))
+def test_q8_gemm_random_shapes(ctx, batch, rows, depth, cols, lo, ro, oo, lb, rb, seed):
+    """Seeded random shapes, orders and batching flags around every dispatch boundary (16-byte
+    alignment of rows, the small-problem limits on depth and size, tile sizes): int32 and uint8
+    results against the oracle, random zero points, bias and clamp."""
+    rng = np.random.default_rng(seed)
+    L = rng.integers(0, 256, ((batch if lb else 1), rows, depth), dtype=np.uint8)
+    Rr = rng.integers(0, 256, ((batch if rb else 1), depth, cols), dtype=np.uint8)
+    l, r = as_major(L, lo), as_major(Rr, ro)
+    lzp, rzp = int(rng.integers(0, 256)), int(rng.integers(0, 256))
+    want = orc.q8_gemm_i32(l, r, batch, rows, cols, depth, -lzp, -rzp, lo, ro, oo, lb, rb)
+    got = gemm_i32_host(ctx, l, lo, r, ro, oo, batch, rows, depth, cols, lb, rb, -lzp, -rzp)
+    np.testing.assert_array_equal(got, want)
+    mult, shift = scales_for(depth)
+    bias = rng.integers(-2 ** 15, 2 ** 15, rows).astype(np.int32) if rng.integers(0, 2) else None
+    zp = int(rng.integers(0, 256))
+    lo_c = int(rng.integers(0, 100))
+    hi_c = int(rng.integers(lo_c + 50, 256))
+    want8 = orc.q8_gemm_u8(l, r, batch, rows, cols, depth, -128, -125, bias, mult, shift, zp, lo_c, hi_c,
+                           lo, ro, oo, lb, rb)
+    got8 = gemm_u8_host(ctx, l, lo, r, ro, oo, batch, rows, depth, cols, lb, rb, -128, -125, bias,
+                        mult, shift, zp, lo_c, hi_c)
+    np.testing.assert_array_equal(got8, want8)
