@@ -370,3 +370,34 @@ def test_q8_gemm_random_shapes(ctx, batch, rows, depth, cols, lo, ro, oo, lb, rb
     got8 = gemm_u8_host(ctx, l, lo, r, ro, oo, batch, rows, depth, cols, lb, rb, -128, -125, bias,
                         mult, shift, zp, lo_c, hi_c)
     np.testing.assert_array_equal(got8, want8)
+
+def _random_mid_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(count):
+        cases.append((int(rng.integers(1, 3)), int(rng.integers(300, 1600)),
+                      int(rng.choice([192, 256, 320, 384, 448, 512, 1000, 1024, 1088, 1152, 2048, 2100])),
+                      int(rng.integers(300, 1600)), int(rng.integers(0, 2)), int(rng.integers(0, 2)),
+                      int(rng.integers(0, 2)), int(rng.integers(0, 1 << 30))))
+    return cases
+
+
+@pytest.mark.parametrize("batch,rows,depth,cols,lo,ro,oo,seed", _random_mid_cases(24, 4242))
+def test_q8_gemm_random_mid_sizes(ctx, batch, rows, depth, cols, lo, ro, oo, seed):
+    """Seeded random mid-size problems (a few hundred to 1600 rows and columns, depths on both
+    sides of the slab and ring conditions): the tiled kernels with ragged edges, both outputs in
+    full against the oracle."""
+    rng = np.random.default_rng(seed)
+    L = rng.integers(0, 256, (batch, rows, depth), dtype=np.uint8)
+    Rr = rng.integers(0, 256, (batch, depth, cols), dtype=np.uint8)
+    l, r = as_major(L, lo), as_major(Rr, ro)
+    lzp, rzp = int(rng.integers(100, 156)), int(rng.integers(100, 156))
+    want = orc.q8_gemm_i32(l, r, batch, rows, cols, depth, -lzp, -rzp, lo, ro, oo)
+    got = gemm_i32_host(ctx, l, lo, r, ro, oo, batch, rows, depth, cols, True, True, -lzp, -rzp)
+    np.testing.assert_array_equal(got, want)
+    mult, shift = scales_for(depth)
+    bias = rng.integers(-2 ** 15, 2 ** 15, rows).astype(np.int32)
+    want8 = orc.output_pipeline_u8(want, batch, rows, cols, oo, bias, mult, shift, 128)
+    got8 = gemm_u8_host(ctx, l, lo, r, ro, oo, batch, rows, depth, cols, True, True, -lzp, -rzp, bias,
+                        mult, shift, 128)
+    np.testing.assert_array_equal(got8, want8)
