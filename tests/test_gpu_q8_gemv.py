@@ -64,6 +64,35 @@ def test_q8_gemv_parity(ctx, batch, h, w, lb, rb):
     assert len(np.unique(got)) > min(10, h // 2)
 
 
+def _random_gemv_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    widths = [1, 15, 16, 17, 63, 64, 65, 127, 128, 200, 256, 1000, 1024, 1040, 2048, 4100, 5008, 9000]
+    return [(int(rng.integers(1, 21)), int(rng.integers(1, 400)), int(rng.choice(widths)),
+             bool(rng.integers(0, 3) == 0), bool(rng.integers(0, 4)), int(rng.integers(0, 1 << 30)))
+            for _ in range(count)]
+
+
+@pytest.mark.parametrize("batch,h,w,lb,rb,seed", _random_gemv_cases(40, 99))
+def test_q8_gemv_random_shapes(ctx, batch, h, w, lb, rb, seed):
+    """Seeded random batches, heights and widths around the kernels' dispatch boundaries (16-byte
+    rows, 64-byte minimum for the matrix-core kernel, LDS capacity, shared or per-batch weights)."""
+    rng = np.random.default_rng(seed)
+    L = rng.integers(0, 256, ((batch if lb else 1), h, w), dtype=np.uint8)
+    x = rng.integers(0, 256, ((batch if rb else 1), w), dtype=np.uint8)
+    bias = rng.integers(-2 ** 15, 2 ** 15, h).astype(np.int32) if rng.integers(0, 2) else None
+    lzp, rzp = int(rng.integers(0, 256)), int(rng.integers(0, 256))
+    want = orc.q8_gemv_i32(L, x, bias, batch, h, w, lzp, rzp, lb, rb)
+    got = run_host(ctx, L, x, bias, batch, h, w, lb, rb, lzp, rzp, False)
+    np.testing.assert_array_equal(got, want)
+    sigma = 74.0 * 74.0 * np.sqrt(w)
+    scales = (np.float32(0.01), np.float32(0.02), np.float32(0.0002 * sigma / 40.0))
+    ozp = int(rng.integers(0, 256))
+    for mode in (mh.REQUANT_REF, mh.REQUANT_NEON):
+        want = orc.q8_gemv_u8(L, x, bias, batch, h, w, 127, 128, *scales, ozp, mode, lb, rb)
+        got = run_host(ctx, L, x, bias, batch, h, w, lb, rb, 127, 128, True, scales, ozp, mode)
+        np.testing.assert_array_equal(got, want)
+
+
 def test_q8_gemv_config_4096(ctx):
     """Benchmark configuration: weight [4096 x 4096], batch 1 and 8, weight_zp 127, input_zp 128,
     int32 bias in [-2^15, 2^15]; device-pointer path."""
