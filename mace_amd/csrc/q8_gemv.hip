@@ -474,8 +474,14 @@ int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
   // a batched lhs gives every batch its own weights: one batch row per pass
   int nb = lhs_batched ? 1 : (p.batch >= 8 ? 8 : (p.batch >= 4 ? 4 : (p.batch >= 2 ? 2 : 1)));
   dim3 block(256);
-  // shared weights against two or more vectors: the batch goes through the matrix cores
-  if (vec && !lhs_batched && p.W >= 64 && p.batch >= 2 && p.rhs_bs % 16 == 0) {
+  // Two to four vectors against long rows stay on the row-block kernel (one pass, the weights
+  // streamed once: 5.6 us against 7.2 us at 4096 x 4096, batch 2); the matrix-core kernel's
+  // load-everything-then-multiply structure only pays from five vectors on, or on short rows.
+  const bool few = !lhs_batched && p.batch >= 2 && p.batch <= 4 && p.W >= 2048 &&
+                   (size_t)4 * p.W <= 64 * 1024;
+  if (few) nb = p.batch == 2 ? 2 : 4;
+  // shared weights against more vectors: the batch goes through the matrix cores
+  if (vec && !lhs_batched && !few && p.W >= 64 && p.batch >= 2 && p.rhs_bs % 16 == 0) {
     dim3 grid((unsigned)((p.H + 15) / 16), (unsigned)((p.batch + 14) / 15));
     MH_CHECK(ctx, grid.y <= 65535, "batch too large");
     const int nb_pass = (int)std::min<int64_t>(p.batch, 15);

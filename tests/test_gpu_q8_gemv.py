@@ -39,7 +39,11 @@ CASES = [(1, 16, 4, True, True), (1, 16, 256, True, True), (2, 16, 256, True, Tr
          (2, 3, 1, False, True), (3, 7, 48, False, False),
          # shared weights, batch >= 2: more than 15 vectors (two passes), width tails, shared rhs
          (16, 50, 272, False, True), (31, 17, 64, False, True), (3, 40, 128, False, False),
-         (15, 16, 80, False, True), (2, 100, 2000, False, True)]
+         (15, 16, 80, False, True), (2, 100, 2000, False, True),
+         # two to four vectors on rows of 2048 bytes and more: the row-block kernel in one pass
+         (2, 50, 2048, False, True), (3, 33, 2048 + 16, False, True), (4, 70, 4096, False, True),
+         (3, 19, 16384, False, True), (4, 20, 16384 + 16, False, True), (3, 40, 4096, False, False),
+         (2, 35, 4100, False, True)]
 
 
 @pytest.mark.parametrize("batch,h,w,lb,rb", CASES)
