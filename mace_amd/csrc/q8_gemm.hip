@@ -860,6 +860,187 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
   gemm_epilogue<WX, WY, FX, FY, OutT, SUMY>(acc, ysum, p, lds, b, x0, y0, wx, wy, tid);
 }
 
+// ---- the kernel for an X panel that fits in LDS ----------------------------------------------
+//
+// A 1x1 convolution's filter (or any operand of at most TX rows x K bytes <= ~128 KiB per tile)
+// against a long Y panel: the tiled kernels above pay a barrier per k slab and read 1 KiB of LDS
+// per MFMA at the 64 x 64 wavefront tile the medium shapes get.  Here the workgroup loads its X
+// tile (TX = 32 FX rows, all of k) into LDS once, flips it to int8 in place and takes its row
+// sums there; after that the four wavefronts never synchronise again: each walks over its own
+// blocks of 32 FY rows of Y, loading the Y fragments straight from global memory into registers
+// (one k group ahead) and reading only X fragments from LDS (1/FY KiB per MFMA).  Both
+// correction vectors are taken in the kernel, so the call is this one launch.
+//
+// k is walked in groups of G bytes.  Lane (row r, half h) loads the G/2 contiguous bytes
+// [G/2 h, G/2 (h+1)) of its row's group, so the loads of one group cover whole rows of G bytes
+// back to back; k step t of the group then multiplies chunk t of half 0 and chunk G/32 + t of
+// half 1, and the X fragment read picks the same chunks (any pairing of k positions is as good as
+// any other as long as both operands use it).
+//
+// LDS: [0, 2048): x correction terms [TX], unused [32 FY], comparison table (the layout
+// gemm_epilogue expects); then K/64 slabs of TX rows x 64 bytes, 16-byte chunk c of row r in
+// slot c ^ ((r >> 2) & 3) as in q8_gemm_dma_kernel.
+// Requirements (checked by the host): K % G == 0, 2048 + TX K bytes of LDS available.
+constexpr int XRES_SC_BYTES = 2048;
+template <int FX, int FY, int G, typename OutT, int OCC>
+__global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, RequantTable) {
+  constexpr int TX = FX * 32, TYW = FY * 32;
+  constexpr int KPG = G / 32;   // k steps per group
+  static_assert(G == 64 || G == 128, "group width");
+  static_assert(TX == 64 || TX == 128, "X tile rows");
+  static_assert((TX + TYW + MH_REQUANT_TABLE_MAX) * 4 <= XRES_SC_BYTES, "correction area");
+  extern __shared__ __align__(16) uint8_t lds[];
+  int32_t *sc = (int32_t *)lds;
+  uint8_t *xt = lds + XRES_SC_BYTES;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int h = lane >> 5, r32 = lane & 31;
+  const int x0 = blockIdx.y * TX;
+  const int b = blockIdx.z;
+  const uint8_t *Xb = p.X + (int64_t)b * p.xbs;
+  const uint8_t *Yb = p.Y + (int64_t)b * p.ybs;
+  const RequantFixed rq = p.rq;
+  const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+
+  const int nblk = (p.YN + TYW - 1) / TYW;
+  const int ngroup = p.K / G;
+  const int stride = gridDim.x * 4;
+  int blk = blockIdx.x * 4 + wave;
+  // rows past the end are clamped to the last one: always readable, never stored
+  auto row_ptr = [&](int bk, int j) -> const uint8_t * {
+    const int64_t row = min((int64_t)bk * TYW + j * 32 + r32, (int64_t)p.YN - 1);
+    return Yb + row * p.ldy + (G / 2) * h;
+  };
+  // the first block's first group is requested before anything else
+  v4i cur[KPG][FY], nxt[KPG][FY];
+  const uint8_t *yp[FY], *ypn[FY];
+#pragma unroll
+  for (int j = 0; j < FY; ++j) {
+    yp[j] = row_ptr(blk, j);
+#pragma unroll
+    for (int t = 0; t < KPG; ++t) cur[t][j] = *(const v4i *)(yp[j] + 16 * t);
+  }
+
+  // X tile -> LDS: one transfer instruction moves 16 rows x 64 bytes
+  {
+    constexpr int LX = TX / 64;   // instructions per wavefront per slab
+    const int nslab = p.K / 64;
+    const uint8_t *src[LX];
+#pragma unroll
+    for (int j = 0; j < LX; ++j) {
+      const int row = (j * 4 + wave) * 16 + (lane >> 2);
+      const int kc = (lane & 3) ^ ((row >> 2) & 3);
+      src[j] = Xb + (int64_t)min(x0 + row, p.XN - 1) * p.ldx + kc * 16;
+    }
+    for (int s = 0; s < nslab; ++s) {
+#pragma unroll
+      for (int j = 0; j < LX; ++j)
+        dma_16B(src[j] + s * 64, xt + s * (TX * 64) + (j * 4 + wave) * 1024);
+      // at most 32 transfers of this wavefront in flight (the counter has six bits)
+      if ((s & 15) == 15) wait_vmcnt<0>();
+    }
+    wait_vmcnt<0>();
+    __syncthreads();
+    // flip to int8 in place and add up the rows: 256 / TX threads per row, slabs dealt round robin
+    constexpr int TPR = 256 / TX;
+    const int row = tid / TPR, part = tid % TPR;
+    int xs = 0;
+    for (int s = part; s < nslab; s += TPR) {
+      uint8_t *q = xt + s * (TX * 64) + row * 64;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const v4i v = *(const v4i *)(q + c * 16) ^ flip;
+        xs = sum16_i8(v, xs);
+        *(v4i *)(q + c * 16) = v;
+      }
+    }
+#pragma unroll
+    for (int m = 1; m < TPR; m <<= 1) xs += __shfl_xor(xs, m, 64);
+    if (part == 0) {
+      const int x = min(x0 + row, p.XN - 1);
+      uint32_t c = (uint32_t)p.xcoef * (uint32_t)xs + (uint32_t)p.xadd;
+      if (p.xbias) c += (uint32_t)p.xbias[x];
+      sc[row] = (int32_t)c;
+    }
+    if constexpr (sizeof(OutT) == 1) {
+      if (rq.table) {
+        const int32_t *arg_tab = (const int32_t *)((const char *)__builtin_amdgcn_kernarg_segment_ptr() +
+                                                   sizeof(GemmParams));
+        int32_t *tab = sc + TX + TYW;
+        for (int j = tid; j <= rq.n + 1; j += 256) tab[j] = arg_tab[j];
+      }
+    }
+    __syncthreads();
+  }
+
+  // X fragment of k step t of group g, 32-row block i:
+  //   xfrag + g * GSTRIDE + i * 2048 + foff[t]
+  constexpr int GSTRIDE = (G / 64) * TX * 64;
+  const int fsw = (r32 >> 2) & 3;
+  const uint8_t *xfrag = xt + r32 * 64 + (G == 128 ? h * (TX * 64) : 0);
+  int foff[KPG];
+#pragma unroll
+  for (int t = 0; t < KPG; ++t) foff[t] = (((G == 128 ? t : 2 * h + t)) ^ fsw) << 4;
+
+  while (blk < nblk) {
+    const int nb = blk + stride;
+#pragma unroll
+    for (int j = 0; j < FY; ++j) ypn[j] = row_ptr(nb, j);
+    v16i acc[FX][FY];
+    int ysum[FY];
+#pragma unroll
+    for (int j = 0; j < FY; ++j) ysum[j] = 0;
+    // One group: request the whole next group (of this block, or the first of the next block),
+    // then multiply this one.  The block's very first k step takes a zero addend, which spares
+    // zeroing the accumulators.
+    auto group = [&](auto first_tag, int g) __attribute__((always_inline)) {
+      constexpr bool first = decltype(first_tag)::value;
+      const bool last = g + 1 == ngroup;
+#pragma unroll
+      for (int j = 0; j < FY; ++j) {
+        const uint8_t *src = last ? ypn[j] : yp[j] + (int64_t)(g + 1) * G;
+#pragma unroll
+        for (int t = 0; t < KPG; ++t) nxt[t][j] = *(const v4i *)(src + 16 * t);
+      }
+      const uint8_t *xg = xfrag + g * GSTRIDE;
+#pragma unroll
+      for (int t = 0; t < KPG; ++t) {
+        v4i xa[FX], yf[FY];
+#pragma unroll
+        for (int i = 0; i < FX; ++i) xa[i] = *(const v4i *)(xg + i * 2048 + foff[t]);
+#pragma unroll
+        for (int j = 0; j < FY; ++j) {
+          yf[j] = cur[t][j] ^ flip;
+          ysum[j] = sum16_i8(yf[j], ysum[j]);
+        }
+#pragma unroll
+        for (int i = 0; i < FX; ++i)
+#pragma unroll
+          for (int j = 0; j < FY; ++j) {
+            if (first && t == 0) {
+              const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+              acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa[i], yf[j], zero, 0, 0, 0);
+            } else {
+              acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa[i], yf[j], acc[i][j], 0, 0, 0);
+            }
+          }
+      }
+#pragma unroll
+      for (int t = 0; t < KPG; ++t)
+#pragma unroll
+        for (int j = 0; j < FY; ++j) cur[t][j] = nxt[t][j];
+    };
+    group(std::true_type{}, 0);
+    for (int g = 1; g < ngroup; ++g) group(std::false_type{}, g);
+    gemm_epilogue<1, 1, FX, FY, OutT, true, true>(acc, ysum, p, lds, b, x0, blk * TYW, 0, 0, tid);
+    blk = nb;
+#pragma unroll
+    for (int j = 0; j < FY; ++j) yp[j] = ypn[j];
+  }
+}
+
 // ---- the streaming kernel for a small X panel ------------------------------------------------
 //
 // When the X panel is small in both directions (a 1x1 convolution's filter; the host sends
@@ -1298,6 +1479,42 @@ int launch_gemm_fused_small(mace_hip_ctx *ctx, GemmParams &p, const RequantTable
   return MACE_HIP_SUCCESS;
 }
 
+// X panel resident in LDS; the caller has checked the preconditions (see the kernel)
+template <int FX, int FY>
+int launch_gemm_xres(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, bool out_u8,
+                     int batch) {
+  constexpr int TX = FX * 32, TYW = FY * 32;
+  const size_t lds = XRES_SC_BYTES + (size_t)TX * p.K;
+  const size_t lds_cu = ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536;
+  const int tiles_x = (p.XN + TX - 1) / TX;
+  const int nblk = (p.YN + TYW - 1) / TYW;
+  const int per_cu = (int)std::max<size_t>(1, std::min<size_t>(2, lds_cu / lds));
+  const int cu = ctx->cu_count > 0 ? ctx->cu_count : 256;
+  // workgroups along y: as many as fit at once
+  const int slots = std::max(1, cu * per_cu / std::max(1, tiles_x * batch));
+  const int need = (nblk + 3) / 4;
+  const int wgs = std::max(1, std::min(need, slots));
+  MH_CHECK(ctx, tiles_x <= 65535 && batch <= 65535, "grid too large");
+  dim3 grid(wgs, tiles_x, batch), block(256);
+  auto launch = [&](auto k) -> int {
+    if (lds > 64 * 1024)
+      MH_HIP(ctx, hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      (int)lds));
+    MH_PROF_BEGIN(ctx);
+    hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, tab);
+    MH_PROF_END(ctx);
+    MH_HIP(ctx, hipGetLastError());
+    return MACE_HIP_SUCCESS;
+  };
+  const bool g128 = p.K % 128 == 0;
+  if (out_u8) {
+    if (g128) return launch(q8_gemm_xres_kernel<FX, FY, 128, uint8_t, 2>);
+    return launch(q8_gemm_xres_kernel<FX, FY, 64, uint8_t, 2>);
+  }
+  if (g128) return launch(q8_gemm_xres_kernel<FX, FY, 128, int32_t, 2>);
+  return launch(q8_gemm_xres_kernel<FX, FY, 64, int32_t, 2>);
+}
+
 // the streaming kernel; the caller has checked its preconditions (see the kernel)
 template <int FX, int XW>
 int launch_gemm_stream(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, int batch) {
@@ -1574,7 +1791,22 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
                       (depth == 32 || depth == 64) && (xn == 32 || xn == 64 || xn == 128) &&
                       yn >= 1024 && ((uintptr_t)out % 16 == 0);
   const int32_t *sumL = L.sums ? L.sums : corrL, *sumR = R.sums ? R.sums : corrR;
-  if (!stream) {
+  // An X panel whose tile (64 or 128 rows, all of k) fits in LDS twice per CU goes to the kernel
+  // that keeps it there and sums both panels itself.  Measured against the tiled kernels (k from
+  // 64 to 1024, 64 to 512 X rows, 4 Ki to 256 Ki Y rows): it wins or ties throughout for
+  // k <= 256 and for X panels of at most 64 rows; for longer k it needs either at least two
+  // blocks of Y per SIMD or a problem so small that the saved launches decide.
+  // (MACE_HIP_NO_XRES_KERNEL, any value: diagnostic switch that keeps the tiled kernels in use.)
+  const int kk = L.k < R.k ? L.k : R.k;
+  const size_t lds_cu = ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536;
+  const int xres_tx = xn <= 64 ? 64 : 128;
+  const int64_t xres_blocks = ((xn + xres_tx - 1) / xres_tx) * ((yn + 63) / 64) * batch;
+  const int64_t cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
+  const bool xres = !cv && !stream && depth > 0 && kk % 64 == 0 && yn >= 256 &&
+                    2 * (XRES_SC_BYTES + (size_t)xres_tx * kk) <= lds_cu &&
+                    (kk <= 256 || xres_tx == 64 || xres_blocks >= 8 * cus || xres_blocks <= cus) &&
+                    !getenv("MACE_HIP_NO_XRES_KERNEL");
+  if (!stream && !xres) {
     if (!L.sums && !(sum_y && !x_is_lhs))
       MH_RETURN_IF_ERROR(launch_panel_sums(ctx, L.ptr, L.ld, L.bs, rows, L.k, lhs_nb, corrL));
     if (!R.sums && !(sum_y && x_is_lhs))
@@ -1618,6 +1850,11 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     if (!zero) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
     MH_RETURN_IF_ERROR(mh_fill_bytes(ctx, zero, (uint8_t)cv->zero_point, 256));
     p.cv_zero = zero;
+  }
+  if (xres) {
+    p.sum_y = true;
+    if (xres_tx == 64) return launch_gemm_xres<2, 2>(ctx, p, tab, out_u8, (int)batch);
+    return launch_gemm_xres<4, 2>(ctx, p, tab, out_u8, (int)batch);
   }
   if (stream) {
     switch (p.XN) {

@@ -87,6 +87,7 @@ def path(request, monkeypatch):
     instead, so that those stay covered on the same shapes."""
     if request.param == "general_path":
         monkeypatch.setenv("MACE_HIP_NO_SMALL_KERNEL", "1")
+        monkeypatch.setenv("MACE_HIP_NO_XRES_KERNEL", "1")
     return request.param
 
 

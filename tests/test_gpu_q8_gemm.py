@@ -59,10 +59,12 @@ SHAPES = [  # batch, rows, depth, cols, lhs_batched, rhs_batched
 
 @pytest.fixture(params=["default", "general_path"])
 def path(request, monkeypatch):
-    """Small problems are one launch of a kernel of their own; MACE_HIP_NO_SMALL_KERNEL sends them
-    through the general path (repack, row sums, tiled kernel) so that both stay covered."""
+    """Small problems are one launch of a kernel of their own, and an X panel that fits in LDS has
+    one too; MACE_HIP_NO_SMALL_KERNEL and MACE_HIP_NO_XRES_KERNEL send them through the general path
+    (repack, row sums, tiled kernel) so that all of them stay covered."""
     if request.param == "general_path":
         monkeypatch.setenv("MACE_HIP_NO_SMALL_KERNEL", "1")
+        monkeypatch.setenv("MACE_HIP_NO_XRES_KERNEL", "1")
     return request.param
 
 
@@ -70,6 +72,10 @@ def path(request, monkeypatch):
 @pytest.mark.parametrize("lo,ro,oo", [(R, R, R), (R, Cm, R), (Cm, R, R), (Cm, Cm, R),
                                       (R, Cm, Cm), (Cm, R, Cm), (R, R, Cm), (Cm, Cm, Cm)])
 def test_q8_gemm_parity(ctx, path, batch, rows, depth, cols, lb, rb, lo, ro, oo):
+    check_gemm(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo)
+
+
+def check_gemm(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo):
     rng = np.random.default_rng(rows * 31 + depth * 7 + cols + lo * 4 + ro * 2 + oo)
     L = rng.integers(0, 256, ((batch if lb else 1), rows, depth), dtype=np.uint8)
     Rr = rng.integers(0, 256, ((batch if rb else 1), depth, cols), dtype=np.uint8)
@@ -88,6 +94,22 @@ def test_q8_gemm_parity(ctx, path, batch, rows, depth, cols, lb, rb, lo, ro, oo)
         np.testing.assert_array_equal(got8, want8)
     if rows * cols >= 64:
         assert len(np.unique(want8)) > 8       # the uint8 check is not vacuous
+
+
+# The kernel that keeps the X panel in LDS (k a multiple of 64 after packing, at least 256 rows on
+# the other side): 64- and 128-row tiles, 64- and 128-byte k groups, ragged edges on both sides,
+# several blocks per wavefront, repacked operands, both result orders, batches.
+XRES_SHAPES = [  # batch, rows, depth, cols, lhs order, rhs order, out order
+    (1, 300, 128, 128, R, Cm, R), (1, 1000, 192, 100, R, Cm, R), (2, 260, 64, 40, R, Cm, R),
+    (1, 4096, 256, 256, R, Cm, R), (1, 140000, 64, 48, R, Cm, R), (1, 512, 100, 128, Cm, R, R),
+    (1, 96, 128, 700, R, Cm, Cm), (1, 300, 1024, 64, R, Cm, R), (1, 512, 512, 128, R, Cm, R),
+    (3, 333, 320, 130, R, R, R), (1, 70000, 128, 160, R, Cm, R),
+]
+
+
+@pytest.mark.parametrize("batch,rows,depth,cols,lo,ro,oo", XRES_SHAPES)
+def test_q8_gemm_x_panel_in_lds(ctx, path, batch, rows, depth, cols, lo, ro, oo):
+    check_gemm(ctx, batch, rows, depth, cols, True, True, lo, ro, oo)
 
 
 def test_q8_gemm_config1_matmul(ctx):
