@@ -386,7 +386,7 @@ def bench_other(ctx, mh, torch):
     torch.cuda.synchronize()
     whole, k = time_kernel(ctx, bind(ctx,
         "mace_hip_gemm_q8_u8", A.data_ptr(), 0, B.data_ptr(), 0, C.data_ptr(), 0, 1, 128, 256, 128,
-        1, 1, -128, -128, None, mult, shift, 128, 0, 255), reps=50)
+        1, 1, -128, -128, None, mult, shift, 128, 0, 255), reps=500, warm=100)
     # one launch does the whole call; call_us = back-to-back calls between two events, kernel_us =
     # one launch between its own pair of events (which costs more than it measures at this size)
     out.append({"workload": "q8_matmul_128x256x128", "call_us": round(whole * 1e3, 2),

@@ -77,16 +77,22 @@ CASES = [  # batch, cout, cin, in_h, in_w, k_h, k_w, padding, strides: the refer
     # channel counts that are multiples of 64: gathered by the GEMM's loader, every tile shape
     (2, 256, 128, 28, 28, 3, 3, S, (1, 1)), (1, 300, 64, 20, 20, 3, 3, S, (1, 1)),
     (1, 48, 192, 13, 17, 3, 3, Fu, (2, 1)), (4, 64, 64, 56, 56, 3, 3, S, (1, 1)),
+    # filter tile resident in LDS: 64 and 128 output channels, 64- and 128-byte k groups, ragged
+    # channel and pixel counts, strides, several blocks per wavefront
+    (3, 100, 64, 30, 31, 3, 3, S, (1, 1)), (2, 64, 128, 28, 28, 3, 3, V, (2, 2)),
+    (1, 40, 128, 33, 20, 2, 3, Fu, (1, 2)), (5, 128, 64, 40, 40, 3, 3, S, (1, 1)),
 ]
 
 
-@pytest.fixture(params=["default", "general_path"])
+@pytest.fixture(params=["default", "no_small_kernel", "general_path"])
 def path(request, monkeypatch):
     """A small convolution is one launch of the small-problem GEMM kernel, which gathers the
-    patches itself; MACE_HIP_NO_SMALL_KERNEL sends it through im2col / the gathering tiled kernel
-    instead, so that those stay covered on the same shapes."""
-    if request.param == "general_path":
+    patches itself; with MACE_HIP_NO_SMALL_KERNEL it goes to the kernel that keeps the filter in
+    LDS (cin a multiple of 64, filter tile fits) and with MACE_HIP_NO_XRES_KERNEL on top through
+    im2col / the gathering tiled kernel, so that all three stay covered on the same shapes."""
+    if request.param != "default":
         monkeypatch.setenv("MACE_HIP_NO_SMALL_KERNEL", "1")
+    if request.param == "general_path":
         monkeypatch.setenv("MACE_HIP_NO_XRES_KERNEL", "1")
     return request.param
 
@@ -113,6 +119,25 @@ def test_conv2d_q8_parity(ctx, path, n, cout, cin, in_h, in_w, k_h, k_w, pad, st
         np.testing.assert_array_equal(got, want)
     if want.size >= 64:
         assert len(np.unique(want)) > 8
+
+
+def test_conv2d_q8_filter_in_lds_many_blocks(ctx):
+    """More 64-pixel blocks than the kernel that keeps the filter in LDS has wavefronts: each
+    wavefront walks over several blocks, prefetching the next block's first filter tap."""
+    n, in_h, in_w, cin, cout, k_h, k_w, st = 44, 56, 56, 64, 64, 1, 3, (1, 1)
+    rng = np.random.default_rng(77)
+    x = rng.integers(0, 256, (n, in_h, in_w, cin), dtype=np.uint8)
+    f = rng.integers(1, 256, (cout, k_h, k_w, cin), dtype=np.uint8)
+    bias = rng.integers(-2 ** 15, 2 ** 15, cout).astype(np.int32)
+    s_in, s_f = np.float32(0.02), np.float32(0.01)
+    s_out = np.float32(max(6.0, 3 * 74.0 * 74.0 * np.sqrt(k_h * k_w * cin) * float(s_in * s_f)) / 255.0)
+    oh, ow, ph, pw = orc.calc_padding_and_output_size(in_h, in_w, k_h, k_w, st, S)
+    assert n * oh * ow > 64 * 2048
+    want = orc.conv2d_q8_nhwc(x, f, bias, n, in_h, in_w, cin, cout, k_h, k_w, st, (ph, pw), s_in,
+                              131, s_f, 122, np.float32(s_in * s_f), s_out, 7, 0, 255)
+    got = conv_host(ctx, x, f, bias, n, in_h, in_w, cin, cout, k_h, k_w, st, (ph, pw), s_in, 131,
+                    s_f, 122, np.float32(s_in * s_f), s_out, 7, 0, 255)
+    np.testing.assert_array_equal(got, want)
 
 
 def _random_conv_cases(count, seed):

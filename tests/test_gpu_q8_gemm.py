@@ -57,13 +57,14 @@ SHAPES = [  # batch, rows, depth, cols, lhs_batched, rhs_batched
 ]
 
 
-@pytest.fixture(params=["default", "general_path"])
+@pytest.fixture(params=["default", "no_small_kernel", "general_path"])
 def path(request, monkeypatch):
     """Small problems are one launch of a kernel of their own, and an X panel that fits in LDS has
-    one too; MACE_HIP_NO_SMALL_KERNEL and MACE_HIP_NO_XRES_KERNEL send them through the general path
-    (repack, row sums, tiled kernel) so that all of them stay covered."""
-    if request.param == "general_path":
+    one too; MACE_HIP_NO_SMALL_KERNEL leaves the second, MACE_HIP_NO_XRES_KERNEL on top of it only
+    the general path (repack, row sums, tiled kernel), so that all three stay covered."""
+    if request.param != "default":
         monkeypatch.setenv("MACE_HIP_NO_SMALL_KERNEL", "1")
+    if request.param == "general_path":
         monkeypatch.setenv("MACE_HIP_NO_XRES_KERNEL", "1")
     return request.param
 
