@@ -887,7 +887,34 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
 // slot c ^ ((r >> 2) & 3) as in q8_gemm_dma_kernel.
 // Requirements (checked by the host): K % G == 0, 2048 + TX K bytes of LDS available.
 constexpr int XRES_SC_BYTES = 2048;
-template <int FX, int FY, int G, typename OutT, int OCC, bool CONV = false>
+// 16 x 16 bytes held as 16 rows of 16 bytes, transposed in place (v_perm_b32: 4 x 4 byte blocks
+// in two stages, the blocks themselves change places by register renaming)
+__device__ __forceinline__ void transpose_16x16_bytes(v4i (&r)[16]) {
+  v4i q[16];
+#pragma unroll
+  for (int kq = 0; kq < 4; ++kq)
+#pragma unroll
+    for (int xq = 0; xq < 4; ++xq) {
+      const uint32_t d0 = (uint32_t)r[4 * kq + 0][xq], d1 = (uint32_t)r[4 * kq + 1][xq];
+      const uint32_t d2 = (uint32_t)r[4 * kq + 2][xq], d3 = (uint32_t)r[4 * kq + 3][xq];
+      const uint32_t u0 = __builtin_amdgcn_perm(d1, d0, 0x05010400u);
+      const uint32_t u1 = __builtin_amdgcn_perm(d1, d0, 0x07030602u);
+      const uint32_t u2 = __builtin_amdgcn_perm(d3, d2, 0x05010400u);
+      const uint32_t u3 = __builtin_amdgcn_perm(d3, d2, 0x07030602u);
+      q[4 * xq + 0][kq] = (int)__builtin_amdgcn_perm(u2, u0, 0x05040100u);
+      q[4 * xq + 1][kq] = (int)__builtin_amdgcn_perm(u2, u0, 0x07060302u);
+      q[4 * xq + 2][kq] = (int)__builtin_amdgcn_perm(u3, u1, 0x05040100u);
+      q[4 * xq + 3][kq] = (int)__builtin_amdgcn_perm(u3, u1, 0x07060302u);
+    }
+#pragma unroll
+  for (int i = 0; i < 16; ++i) r[i] = q[i];
+}
+
+// XT: the X operand lies k-major in memory (X(x, k) at X[k * ldx + x]: a RowMajor right-hand
+// matrix): the tile is read in 16 x 16 byte blocks, flipped, transposed in registers and written
+// into the same LDS layout, the row sums added up through LDS atomics; XN % 16 == 0, X 16-byte
+// aligned.
+template <int FX, int FY, int G, typename OutT, int OCC, bool CONV = false, bool XT = false>
 __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, RequantTable) {
   constexpr int TX = FX * 32, TYW = FY * 32;
   constexpr int KPG = G / 32;   // k steps per group
@@ -958,8 +985,46 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
     for (int t = 0; t < KPG; ++t) cur[t][j] = *(const v4i *)(src + 16 * t);
   }
 
-  // X tile -> LDS: one transfer instruction moves 16 rows x 64 bytes
-  {
+  if constexpr (XT) {
+    for (int i = tid; i < TX; i += 256) sc[i] = 0;
+    __syncthreads();
+    constexpr int XB = TX / 16;   // 16-row blocks of the tile
+    const int nblock = XB * (p.K / 16);
+    for (int id = tid; id < nblock; id += 256) {
+      const int xb = id % XB, kb = id / XB;
+      // blocks past the end of X re-read the last one (XN % 16 == 0: never a partial block)
+      const int xs = min(x0 + 16 * xb, p.XN - 16);
+      const uint8_t *src = Xb + (int64_t)(16 * kb) * p.ldx + xs;
+      v4i r[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) r[i] = *(const v4i *)(src + (int64_t)i * p.ldx) ^ flip;
+      transpose_16x16_bytes(r);
+      uint8_t *slab = xt + (kb >> 2) * (TX * 64);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int row = 16 * xb + i;
+        *(v4i *)(slab + row * 64 + (((kb & 3) ^ ((row >> 2) & 3)) << 4)) = r[i];
+        atomicAdd(&sc[row], sum16_i8(r[i], 0));
+      }
+    }
+    __syncthreads();
+    for (int i = tid; i < TX; i += 256) {
+      const int x = min(x0 + i, p.XN - 1);
+      uint32_t c = (uint32_t)p.xcoef * (uint32_t)sc[i] + (uint32_t)p.xadd;
+      if (p.xbias) c += (uint32_t)p.xbias[x];
+      sc[i] = (int32_t)c;
+    }
+    if constexpr (sizeof(OutT) == 1) {
+      if (rq.table) {
+        const int32_t *arg_tab = (const int32_t *)((const char *)__builtin_amdgcn_kernarg_segment_ptr() +
+                                                   sizeof(GemmParams));
+        int32_t *tab = sc + TX + TYW;
+        for (int j = tid; j <= rq.n + 1; j += 256) tab[j] = arg_tab[j];
+      }
+    }
+    __syncthreads();
+  } else {
+    // X tile -> LDS: one transfer instruction moves 16 rows x 64 bytes
     constexpr int LX = TX / 64;   // instructions per wavefront per slab
     const int nslab = p.K / 64;
     const uint8_t *src[LX];
@@ -1524,7 +1589,7 @@ int launch_gemm_fused_small(mace_hip_ctx *ctx, GemmParams &p, const RequantTable
 // X panel resident in LDS; the caller has checked the preconditions (see the kernel)
 template <int FX, int FY>
 int launch_gemm_xres(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, bool out_u8,
-                     int batch) {
+                     int batch, bool xt = false) {
   constexpr int TX = FX * 32, TYW = FY * 32;
   const size_t lds = XRES_SC_BYTES + (size_t)TX * p.K;
   const size_t lds_cu = ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536;
@@ -1554,6 +1619,14 @@ int launch_gemm_xres(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, 
     return launch(q8_gemm_xres_kernel<FX, FY, 64, uint8_t, 2, true>);
   }
   const bool g128 = p.K % 128 == 0;
+  if (xt) {   // X k-major in memory: transposed on its way into LDS
+    if (out_u8) {
+      if (g128) return launch(q8_gemm_xres_kernel<FX, FY, 128, uint8_t, 2, false, true>);
+      return launch(q8_gemm_xres_kernel<FX, FY, 64, uint8_t, 2, false, true>);
+    }
+    if (g128) return launch(q8_gemm_xres_kernel<FX, FY, 128, int32_t, 2, false, true>);
+    return launch(q8_gemm_xres_kernel<FX, FY, 64, int32_t, 2, false, true>);
+  }
   if (out_u8) {
     if (g128) return launch(q8_gemm_xres_kernel<FX, FY, 128, uint8_t, 2>);
     return launch(q8_gemm_xres_kernel<FX, FY, 64, uint8_t, 2>);
@@ -1703,6 +1776,58 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
       RequantTable tab;
       if (out_u8 && rq.table) mh_requant_table_cached(ctx, rq, tab.t);
       return launch_gemm_fused_small(ctx, p, tab, out_u8, xt, yt, (int)batch);
+    }
+  }
+
+  // An X operand that lies k-major in memory (the RowMajor right-hand matrix of a MatMul with
+  // RowMajor result) and whose tile fits in LDS twice per CU: the kernel that keeps the tile in
+  // LDS transposes it on the way in, so nothing is repacked and the call is one launch
+  // (32 x 512^3: repack + zeroing + GEMM 25.9 us -> one kernel).
+  {
+    const bool xl = out_order == MACE_HIP_COL_MAJOR;
+    const bool x_kmajor = xl ? lhs_order == MACE_HIP_COL_MAJOR : rhs_order == MACE_HIP_ROW_MAJOR;
+    const int64_t xn = xl ? rows : cols, yn = xl ? cols : rows;
+    const uint8_t *xp = xl ? lhs : rhs, *yp = xl ? rhs : lhs;
+    const bool y_direct = xl ? (rhs_direct && rhs_ld == 0) : lhs_direct;
+    const int tx = xn <= 64 ? 64 : 128;
+    const size_t lds_cu = ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536;
+    // at least one 64-row block of Y per SIMD (with fewer, the tiled kernels spread the work over
+    // more CUs and win even with the repack in front: 2048 x 512 x 2048 14.4 against 15.4 us)
+    const int64_t blocks = ((xn + tx - 1) / tx) * ((yn + 63) / 64) * batch;
+    const int64_t cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
+    if (!cv && x_kmajor && y_direct && rhs_ld == 0 && !lhs_w && !rhs_w && depth > 0 &&
+        depth % 64 == 0 && xn % 16 == 0 && (uintptr_t)xp % 16 == 0 && yn >= 256 &&
+        (blocks >= 4 * cus || blocks <= cus) &&
+        2 * (XRES_SC_BYTES + (size_t)tx * depth) <= lds_cu && !getenv("MACE_HIP_NO_XRES_KERNEL")) {
+      GemmParams p{};
+      const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
+      const int32_t l_coef = (int32_t)(0u - zr), r_coef = (int32_t)(0u - zl);
+      const int32_t r_add = (int32_t)((uint32_t)depth * zl * zr);
+      const int32_t *l_bias = out_u8 ? ep.bias : nullptr;
+      p.X = xp;
+      p.Y = yp;
+      p.XN = (int)xn;
+      p.YN = (int)yn;
+      p.K = (int)depth;
+      p.ldx = xn;      // bytes between consecutive k
+      p.ldy = depth;
+      p.xbs = ((xl ? lhs_nb : rhs_nb) > 1) ? xn * depth : 0;
+      p.ybs = ((xl ? rhs_nb : lhs_nb) > 1) ? yn * depth : 0;
+      p.out = out;
+      p.ldo = p.XN;
+      p.obs = rows * cols;
+      p.rq = rq;
+      p.sum_y = true;
+      p.xcoef = xl ? l_coef : r_coef;
+      p.xadd = xl ? 0 : r_add;
+      p.xbias = xl ? l_bias : nullptr;
+      p.ycoef = xl ? r_coef : l_coef;
+      p.yadd = xl ? r_add : 0;
+      p.ybias = xl ? nullptr : l_bias;
+      RequantTable tab;
+      if (out_u8 && rq.table) mh_requant_table_cached(ctx, rq, tab.t);
+      if (tx == 64) return launch_gemm_xres<2, 2>(ctx, p, tab, out_u8, (int)batch, true);
+      return launch_gemm_xres<4, 2>(ctx, p, tab, out_u8, (int)batch, true);
     }
   }
 

@@ -105,6 +105,10 @@ XRES_SHAPES = [  # batch, rows, depth, cols, lhs order, rhs order, out order
     (1, 4096, 256, 256, R, Cm, R), (1, 140000, 64, 48, R, Cm, R), (1, 512, 100, 128, Cm, R, R),
     (1, 96, 128, 700, R, Cm, Cm), (1, 300, 1024, 64, R, Cm, R), (1, 512, 512, 128, R, Cm, R),
     (3, 333, 320, 130, R, R, R), (1, 70000, 128, 160, R, Cm, R),
+    # X operand k-major in memory (RowMajor right-hand matrix, or ColMajor left-hand matrix with a
+    # ColMajor result): transposed on its way into LDS, nothing repacked
+    (1, 300, 128, 128, R, R, R), (4, 512, 512, 512, R, R, R), (1, 1000, 192, 112, R, R, R),
+    (2, 260, 64, 48, R, R, R), (1, 96, 128, 700, Cm, Cm, Cm), (1, 4100, 576, 272, R, R, R),
 ]
 
 
