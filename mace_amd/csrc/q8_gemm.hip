@@ -1614,9 +1614,11 @@ int launch_gemm_xres(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, 
     return MACE_HIP_SUCCESS;
   };
   if (p.conv) {
-    MH_CHECK(ctx, out_u8, "the convolution gather produces uint8 only");
-    if (p.cv_cin % 128 == 0) return launch(q8_gemm_xres_kernel<FX, FY, 128, uint8_t, 2, true>);
-    return launch(q8_gemm_xres_kernel<FX, FY, 64, uint8_t, 2, true>);
+    MH_CHECK(ctx, out_u8 && FY == 2, "the convolution gather produces uint8 only, 64 pixels per block");
+    if constexpr (FY == 2) {
+      if (p.cv_cin % 128 == 0) return launch(q8_gemm_xres_kernel<FX, FY, 128, uint8_t, 2, true>);
+      return launch(q8_gemm_xres_kernel<FX, FY, 64, uint8_t, 2, true>);
+    }
   }
   const bool g128 = p.K % 128 == 0;
   if (xt) {   // X k-major in memory: transposed on its way into LDS
@@ -1633,6 +1635,23 @@ int launch_gemm_xres(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, 
   }
   if (g128) return launch(q8_gemm_xres_kernel<FX, FY, 128, int32_t, 2>);
   return launch(q8_gemm_xres_kernel<FX, FY, 64, int32_t, 2>);
+}
+
+// Tile rows (64 / 128) and rows of Y per block.  64-row blocks read half the LDS per MFMA; 32-row
+// blocks give twice the wavefronts, which measured faster (or equal) from one block per CU up to
+// sixteen (56x56x128 -> 128 at batch 64: 22.2 -> 19.6 us; 4096 x 512 x 1024: 14.3 -> 9.6 us).
+// The gather variant is built for 64-row blocks only (32-row blocks measured within +-5 % there).
+int launch_gemm_xres_any(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, bool out_u8,
+                         int batch, int tx, bool xt) {
+  const int64_t blocks64 = (int64_t)((p.XN + tx - 1) / tx) * ((p.YN + 63) / 64) * batch;
+  const int64_t cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
+  const bool fy1 = !p.conv && blocks64 > cus && blocks64 < 16 * cus;
+  if (tx == 64) {
+    if (fy1) return launch_gemm_xres<2, 1>(ctx, p, tab, out_u8, batch, xt);
+    return launch_gemm_xres<2, 2>(ctx, p, tab, out_u8, batch, xt);
+  }
+  if (fy1) return launch_gemm_xres<4, 1>(ctx, p, tab, out_u8, batch, xt);
+  return launch_gemm_xres<4, 2>(ctx, p, tab, out_u8, batch, xt);
 }
 
 // the streaming kernel; the caller has checked its preconditions (see the kernel)
@@ -1791,13 +1810,8 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     const bool y_direct = xl ? (rhs_direct && rhs_ld == 0) : lhs_direct;
     const int tx = xn <= 64 ? 64 : 128;
     const size_t lds_cu = ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536;
-    // at least one 64-row block of Y per SIMD (with fewer, the tiled kernels spread the work over
-    // more CUs and win even with the repack in front: 2048 x 512 x 2048 14.4 against 15.4 us)
-    const int64_t blocks = ((xn + tx - 1) / tx) * ((yn + 63) / 64) * batch;
-    const int64_t cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
     if (!cv && x_kmajor && y_direct && rhs_ld == 0 && !lhs_w && !rhs_w && depth > 0 &&
         depth % 64 == 0 && xn % 16 == 0 && (uintptr_t)xp % 16 == 0 && yn >= 256 &&
-        (blocks >= 4 * cus || blocks <= cus) &&
         2 * (XRES_SC_BYTES + (size_t)tx * depth) <= lds_cu && !getenv("MACE_HIP_NO_XRES_KERNEL")) {
       GemmParams p{};
       const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
@@ -1826,8 +1840,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
       p.ybias = xl ? nullptr : l_bias;
       RequantTable tab;
       if (out_u8 && rq.table) mh_requant_table_cached(ctx, rq, tab.t);
-      if (tx == 64) return launch_gemm_xres<2, 2>(ctx, p, tab, out_u8, (int)batch, true);
-      return launch_gemm_xres<4, 2>(ctx, p, tab, out_u8, (int)batch, true);
+      return launch_gemm_xres_any(ctx, p, tab, out_u8, (int)batch, tx, true);
     }
   }
 
@@ -1965,10 +1978,10 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   const int32_t *sumL = L.sums ? L.sums : corrL, *sumR = R.sums ? R.sums : corrR;
   // An X panel whose tile (64 or 128 rows, all of k) fits in LDS twice per CU goes to the kernel
   // that keeps it there and sums both panels itself.  Measured against the tiled kernels (k from
-  // 64 to 1024, 64 to 512 X rows, 4 Ki to 256 Ki Y rows): it wins or ties throughout for
-  // k <= 256 and for X panels of at most 64 rows; for longer k it needs either at least two
-  // blocks of Y per SIMD or a problem so small that the saved launches decide.  A convolution
-  // whose patches the kernel gathers (cin % 64 == 0) takes it whenever the tile fits: 25 % faster
+  // 64 to 1024, 64 to 1024 X rows, 4 Ki to 256 Ki Y rows): with the block height chosen as in
+  // launch_gemm_xres_any it wins or ties throughout (where the tile only fits once, k >= 640 at
+  // 128 rows, the tiled kernels win by 10 - 35 % and keep the shape).  A convolution whose
+  // patches the kernel gathers (cin % 64 == 0) takes it whenever the tile fits: 25 % faster
   // than the gathering tiled kernel on 3x3, 56x56x64 -> 64 at batch 64 (splitting a 128-row tile
   // that does not fit into two of 64 rows was slower than the tiled kernel).
   // (MACE_HIP_NO_XRES_KERNEL, any value: diagnostic switch that keeps the tiled kernels in use.)
@@ -1976,12 +1989,9 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   const size_t lds_cu = ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536;
   auto xres_fits = [&](int tx) { return 2 * (XRES_SC_BYTES + (size_t)tx * kk) <= lds_cu; };
   const int xres_tx = xn <= 64 ? 64 : 128;
-  const int64_t xres_blocks = ((xn + xres_tx - 1) / xres_tx) * ((yn + 63) / 64) * batch;
-  const int64_t cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
   const bool xres_cv = cv && !cv_small && out_u8 && cv->cin % 64 == 0 && depth % 64 == 0;
   const bool xres = (!cv || xres_cv) && !stream && depth > 0 && kk % 64 == 0 && yn >= 256 &&
                     xres_fits(xres_tx) &&
-                    (cv || kk <= 256 || xres_tx == 64 || xres_blocks >= 8 * cus || xres_blocks <= cus) &&
                     !getenv("MACE_HIP_NO_XRES_KERNEL");
   if (!stream && !xres) {
     if (!L.sums && !(sum_y && !x_is_lhs))
@@ -2030,8 +2040,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   }
   if (xres) {
     p.sum_y = true;
-    if (xres_tx == 64) return launch_gemm_xres<2, 2>(ctx, p, tab, out_u8, (int)batch);
-    return launch_gemm_xres<4, 2>(ctx, p, tab, out_u8, (int)batch);
+    return launch_gemm_xres_any(ctx, p, tab, out_u8, (int)batch, xres_tx, false);
   }
   if (stream) {
     switch (p.XN) {
