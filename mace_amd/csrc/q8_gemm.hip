@@ -1988,7 +1988,13 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   const int kk = L.k < R.k ? L.k : R.k;
   const size_t lds_cu = ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536;
   auto xres_fits = [&](int tx) { return 2 * (XRES_SC_BYTES + (size_t)tx * kk) <= lds_cu; };
-  const int xres_tx = xn <= 64 ? 64 : 128;
+  // Where 128 rows of a long k do not fit, 64-row tiles (Y is then read once per 64 X rows) still
+  // win between one and two 64 x 64 blocks per CU, where the tiled kernels leave most of the chip
+  // idle (k = 1024, 512 X rows, 3136 Y rows: 16.0 -> 9.4 us); beyond that they lose.
+  const int64_t blocks_tx64 = ((xn + 63) / 64) * ((yn + 63) / 64) * batch;
+  const int64_t cu_n = ctx->cu_count > 0 ? ctx->cu_count : 256;
+  const bool xres_narrow = !cv && !xres_fits(128) && blocks_tx64 > cu_n && blocks_tx64 <= 2 * cu_n;
+  const int xres_tx = (xn <= 64 || xres_narrow) ? 64 : 128;
   const bool xres_cv = cv && !cv_small && out_u8 && cv->cin % 64 == 0 && depth % 64 == 0;
   const bool xres = (!cv || xres_cv) && !stream && depth > 0 && kk % 64 == 0 && yn >= 256 &&
                     xres_fits(xres_tx) &&

@@ -109,6 +109,8 @@ XRES_SHAPES = [  # batch, rows, depth, cols, lhs order, rhs order, out order
     # ColMajor result): transposed on its way into LDS, nothing repacked
     (1, 300, 128, 128, R, R, R), (4, 512, 512, 512, R, R, R), (1, 1000, 192, 112, R, R, R),
     (2, 260, 64, 48, R, R, R), (1, 96, 128, 700, Cm, Cm, Cm), (1, 4100, 576, 272, R, R, R),
+    # long k in 64-row tiles (128 rows would not fit in LDS twice)
+    (1, 3136, 1024, 500, R, Cm, R), (1, 4000, 768, 250, R, Cm, R),
 ]
 
 
