@@ -1163,8 +1163,12 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
 //
 // XN = 32 * FX * XW exactly, K = 32 * KS exactly, uint8 output by threshold look-up only,
 // result rows (ldo = XN bytes) and base 16-byte aligned: the host checks all of that.
+// (The occupancy in the launch bounds is what the host launches, see launch_gemm_stream; with at
+// most 256 registers per wavefront the compiler also keeps the MFMA results in ordinary VGPRs,
+// which spares the epilogue one register move per output.)
 template <int FX, int KS, int XW, int D>
-__global__ __launch_bounds__(256) void q8_gemm_stream_kernel(GemmParams p, RequantTable) {
+__global__ __launch_bounds__(256, (FX * KS <= 2 ? 4 : (FX * KS <= 4 ? 3 : (FX * KS <= 16 ? 2 : 1))))
+void q8_gemm_stream_kernel(GemmParams p, RequantTable) {
   constexpr int YW = 4 / XW;   // wavefronts of the workgroup along Y
   __shared__ int32_t s_cx[32 * FX * XW];
   __shared__ int32_t s_tab[MH_REQUANT_TABLE_MAX];
@@ -1616,7 +1620,9 @@ int launch_gemm_xres(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, 
   if (p.conv) {
     MH_CHECK(ctx, out_u8 && FY == 2, "the convolution gather produces uint8 only, 64 pixels per block");
     if constexpr (FY == 2) {
-      if (p.cv_cin % 128 == 0) return launch(q8_gemm_xres_kernel<FX, FY, 128, uint8_t, 2, true>);
+      // (128-byte groups with 128-row tiles would need more than 256 registers)
+      if constexpr (FX == 2)
+        if (p.cv_cin % 128 == 0) return launch(q8_gemm_xres_kernel<FX, FY, 128, uint8_t, 2, true>);
       return launch(q8_gemm_xres_kernel<FX, FY, 64, uint8_t, 2, true>);
     }
   }
@@ -1661,7 +1667,7 @@ int launch_gemm_stream(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab
   const int nblk = (p.YN + 31) / 32;
   const int ks = p.K / 32;
   // resident workgroups per CU by register footprint (X fragments dominate)
-  const int per_cu = FX * ks <= 4 ? 4 : (FX * ks <= 16 ? 2 : 1);
+  const int per_cu = FX * ks <= 2 ? 4 : (FX * ks <= 4 ? 3 : (FX * ks <= 16 ? 2 : 1));
   const int cu = ctx->cu_count > 0 ? ctx->cu_count : 256;
   const int wgs = std::max(1, std::min((nblk + YW - 1) / YW, cu * per_cu));
   dim3 grid(wgs, 1, batch), block(256);
