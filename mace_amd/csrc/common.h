@@ -189,8 +189,14 @@ struct RequantFixed {
   int32_t table;     // 1 = the kernels may requantize by threshold lookup
   int32_t n;         // bhi - blo: number of thresholds
   int32_t lo;        // lo = blo + zp: the output value below the first threshold
-  float inv, off;    // float estimate of the step index: floor(acc * inv + off)
+  float inv, off;    // float estimate of the step index, see mh_requant_step
+  float top;         // upper clamp of the estimate
 };
+// The estimate is formed as acc * inv + (2^20 - blo) in one fused multiply-add: at that magnitude
+// a float's last bit is worth 1/8, so the mantissa holds 8 * (estimate) and "bits & 0xFF8" is
+// 8 * floor(estimate): the byte offset of the step's entry in a table of 8-byte entries, with no
+// conversion back to integer and no shift.
+constexpr float MH_REQUANT_MAGIC = 1048576.0f;
 
 // The pipeline z(x) = clamp(RDivPOT(SRDHM(x, mult), shift), blo, bhi) is a non-decreasing step
 // function of x when mult > 0, so z(x) = blo + #{ j in 1..n : x >= T[j] } with
@@ -236,11 +242,13 @@ inline bool mh_make_requant(int32_t mult, int shift, int32_t zp, int lo, int hi,
   r->table = 0;
   r->inv = 0.f;
   r->off = 0.f;
+  r->top = 0.f;
   if (mult > 0 && blo >= -32768 && bhi <= 32768 && r->n + 2 <= 258 &&
       (r->n == 0 || mh_requant_threshold(mult, shift, r->blo, 1) > (int64_t)INT32_MIN)) {
     r->table = 1;
     r->inv = (float)((double)mult / 2147483648.0 / (double)((int64_t)1 << shift));
-    r->off = (float)(0.2 - (double)blo);
+    r->off = MH_REQUANT_MAGIC - (float)blo;              // an integer below 2^24: exact
+    r->top = MH_REQUANT_MAGIC + (float)r->n + 0.875f;    // floor(top - 2^20) = n
   }
   return true;
 }
@@ -268,20 +276,29 @@ inline void mh_requant_table_cached(mace_hip_ctx *ctx, const RequantFixed &q, in
   ctx->rq_cache_valid[e] = 1;
   memcpy(tab, ctx->rq_cache_tab[e], sizeof(int32_t) * (q.n + 2));
 }
-// Step index of accumulator x: k with z = blo + k, out = lo + k.  c = floor(x * inv + off),
-// clamped to [0, n], is k or k - 1 (SRDHM and RDivPOT each move the value by at most half a
-// step of their own, 0.75 output steps together; 0.2 centres that band), one look-up decides.
-__host__ __device__ inline int mh_requant_step(int32_t x, const RequantFixed &q,
-                                               const int32_t *table) {
+// Step index of accumulator x: k with z = blo + k, out = lo + k.  In exact arithmetic
+// u(x) = x * mult / 2^(31 + shift) - blo stays at least 1/4 below j for x = T[j] - 1 and at least
+// 1/4 above j - 1 for x = T[j] (SRDHM and RDivPOT each round to nearest; checked over random
+// parameter sets in exact rational arithmetic), so for an x of step k it lies in [k - 3/4, k + 3/4].
+// The float estimate adds at most 1/16 (the fused multiply-add rounds to a multiple of 1/8) plus
+// about 0.004 (rounding of x and of inv at |u| <= 2^15): c = floor(estimate), clamped to [0, n],
+// is k or k - 1, and one look-up decides.
+__host__ __device__ inline int mh_requant_step_estimate(int32_t x, const RequantFixed &q) {
 #if defined(__HIP_DEVICE_COMPILE__)
   float u = __fmaf_rn((float)x, q.inv, q.off);
-  u = __builtin_amdgcn_fmed3f(u, 0.0f, (float)q.n + 0.5f);
+  u = __builtin_amdgcn_fmed3f(u, MH_REQUANT_MAGIC, q.top);
+  return (int)((__float_as_uint(u) & 0xFF8u) >> 3);
 #else
   float u = fmaf((float)x, q.inv, q.off);
-  const float top = (float)q.n + 0.5f;
-  u = u < 0.0f ? 0.0f : (u > top ? top : u);
+  u = u < MH_REQUANT_MAGIC ? MH_REQUANT_MAGIC : (u > q.top ? q.top : u);
+  uint32_t bits;
+  memcpy(&bits, &u, sizeof(bits));
+  return (int)((bits & 0xFF8u) >> 3);
 #endif
-  const int c = (int)u;   // u >= 0: truncation is floor
+}
+__host__ __device__ inline int mh_requant_step(int32_t x, const RequantFixed &q,
+                                               const int32_t *table) {
+  const int c = mh_requant_step_estimate(x, q);
   return c + (x > table[c + 1] ? 1 : 0);
 }
 __host__ __device__ inline int32_t mh_requant_fixed(int32_t acc, const RequantFixed &q) {

@@ -101,6 +101,40 @@ __device__ inline int sum16_i8(const v4i &f, int acc) {
   return acc;
 }
 
+// The comparison table as the kernels keep it in LDS: entry c (8 bytes) = {largest accumulator
+// that does not reach step c + 1, output value of step c}.  The kernel's second argument holds the
+// first halves (see mh_requant_table_entry), placed right behind GemmParams in the argument
+// segment (indexing a by-value copy with a lane-dependent index would spill it).
+constexpr int MH_REQUANT_PAIRS_BYTES = 8 * (MH_REQUANT_TABLE_MAX - 1);
+__device__ inline void stage_requant_pairs(int32_t *pairs, const RequantFixed &rq, int tid,
+                                           int nthreads) {
+  static_assert(sizeof(GemmParams) % alignof(RequantTable) == 0, "argument layout");
+  const int32_t *arg_tab = (const int32_t *)((const char *)__builtin_amdgcn_kernarg_segment_ptr() +
+                                             sizeof(GemmParams));
+  for (int c = tid; c <= rq.n; c += nthreads) {
+    pairs[2 * c] = arg_tab[c + 1];
+    pairs[2 * c + 1] = rq.lo + c;
+  }
+}
+// Sixteen accumulators -> sixteen output bytes in four dwords.  Estimates first, then all
+// look-ups, then the compares: sixteen LDS reads in flight instead of one round trip per element.
+__device__ __forceinline__ void requant_16_by_table(const int32_t (&v)[16], const RequantFixed &rq,
+                                                    const int32_t *pairs, uint32_t (&packed)[4]) {
+  uint32_t a[16];
+  int2 e[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r)
+    a[r] = __float_as_uint(__builtin_amdgcn_fmed3f(__fmaf_rn((float)v[r], rq.inv, rq.off),
+                                                   MH_REQUANT_MAGIC, rq.top)) & 0xFF8u;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) e[r] = *(const int2 *)((const char *)pairs + a[r]);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) packed[q] = 0;
+#pragma unroll
+  for (int r = 0; r < 16; ++r)
+    packed[r / 4] |= (uint32_t)(e[r].y + (v[r] > e[r].x ? 1 : 0)) << (8 * (r % 4));
+}
+
 // Epilogue shared by the GEMM kernels: adds the correction vectors to the accumulators and
 // stores int32 results or requantized bytes.  Accumulator register r of a 32x32 tile holds
 //   x (MFMA row)    = 8 * (r / 4) + 4 * (lane / 32) + r % 4
@@ -121,7 +155,8 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[FX][FY], const int (&y
   const int32_t *cY = p.corrY + (int64_t)b * p.cybs;
   int32_t *sc = (int32_t *)lds;   // [TX] corrections along x, then [TY] along y
   const RequantFixed rq = p.rq;
-  int32_t *tab = sc + TX + TY;    // [n + 2] comparison table of the threshold requantization
+  static_assert((TX + TY) % 2 == 0, "the table entries are read as 8-byte pairs");
+  int32_t *tab = sc + TX + TY;    // [n + 1] 8-byte entries of the threshold requantization
   if constexpr (!PRESTAGED) {
   __syncthreads();                // every wavefront is done reading operand tiles
   // panel sums -> correction terms: coef * sum + add (+ bias on the side the result rows are on)
@@ -139,14 +174,7 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[FX][FY], const int (&y
       sc[TX + i] = (int32_t)c;
     }
   if constexpr (sizeof(OutT) == 1) {
-    if (rq.table) {
-      // The table is the kernel's second argument, placed right behind GemmParams in the
-      // argument segment (indexing a by-value copy with a lane-dependent index would spill it)
-      static_assert(sizeof(GemmParams) % alignof(RequantTable) == 0, "argument layout");
-      const int32_t *arg_tab = (const int32_t *)((const char *)__builtin_amdgcn_kernarg_segment_ptr() +
-                                                 sizeof(GemmParams));
-      for (int j = tid; j <= rq.n + 1; j += NT) tab[j] = arg_tab[j];
-    }
+    if (rq.table) stage_requant_pairs(tab, rq, tid, NT);
   }
   __syncthreads();
   }
@@ -201,21 +229,7 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[FX][FY], const int (&y
         } else {
           uint32_t packed[4] = {0, 0, 0, 0};
           if constexpr (TABLE) {
-            // estimates first, then all look-ups, then the compares: sixteen LDS reads in
-            // flight instead of one round trip per element
-            int c[16], t[16];
-            const float top = (float)rq.n + 0.5f;
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-              c[r] = (int)__builtin_amdgcn_fmed3f(__fmaf_rn((float)v[r], rq.inv, rq.off), 0.0f, top);
-#pragma unroll
-            for (int r = 0; r < 16; ++r) t[r] = tab[c[r] + 1];
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-              packed[r / 4] |= (uint32_t)(c[r] + (v[r] > t[r] ? 1 : 0)) << (8 * (r % 4));
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-              packed[q] += (uint32_t)rq.lo * 0x01010101u;   // lo + k <= 255: no carries
+            requant_16_by_table(v, rq, tab, packed);
           } else {
 #pragma unroll
             for (int r = 0; r < 16; ++r)
@@ -424,7 +438,7 @@ template <typename OutT, bool XT, bool YT>
 __global__ __launch_bounds__(256) void q8_gemm_fused_small_kernel(GemmParams p, RequantTable) {
   constexpr int T = 64;
   __shared__ __align__(16) uint8_t tile[2][T * LDS_ROW];   // X rows, Y rows: [row][k], sign-flipped
-  __shared__ __align__(16) int32_t sc[2 * T + MH_REQUANT_TABLE_MAX + 2];
+  __shared__ __align__(16) int32_t sc[2 * T + MH_REQUANT_PAIRS_BYTES / 4];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -544,11 +558,7 @@ __global__ __launch_bounds__(256) void q8_gemm_fused_small_kernel(GemmParams p, 
   // Everything the epilogue needs from memory is asked for now, so that it arrives under the
   // operand loads: the comparison table (into LDS) and this lane's bias.
   if constexpr (sizeof(OutT) == 1) {
-    if (p.rq.table) {
-      const int32_t *arg_tab = (const int32_t *)((const char *)__builtin_amdgcn_kernarg_segment_ptr() +
-                                                 sizeof(GemmParams));
-      for (int j = tid; j <= p.rq.n + 1; j += 256) sc[2 * T + j] = arg_tab[j];
-    }
+    if (p.rq.table) stage_requant_pairs(sc + 2 * T, p.rq, tid, 256);
   }
   const int32_t xbias = p.xbias ? p.xbias[min(x0 + wx * 32 + (lane & 31), p.XN - 1)] : 0;
 
@@ -882,11 +892,11 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
 // share of the group from the tap's pixel, or from a buffer of zero-point bytes where the tap
 // falls into the padding.
 //
-// LDS: [0, 2048): x correction terms [TX], unused [32 FY], comparison table (the layout
+// LDS: [0, 3072): x correction terms [TX], unused [32 FY], comparison table (the layout
 // gemm_epilogue expects); then K/64 slabs of TX rows x 64 bytes, 16-byte chunk c of row r in
 // slot c ^ ((r >> 2) & 3) as in q8_gemm_dma_kernel.
 // Requirements (checked by the host): K % G == 0, 2048 + TX K bytes of LDS available.
-constexpr int XRES_SC_BYTES = 2048;
+constexpr int XRES_SC_BYTES = 3072;
 // 16 x 16 bytes held as 16 rows of 16 bytes, transposed in place (v_perm_b32: 4 x 4 byte blocks
 // in two stages, the blocks themselves change places by register renaming)
 __device__ __forceinline__ void transpose_16x16_bytes(v4i (&r)[16]) {
@@ -920,7 +930,7 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
   constexpr int KPG = G / 32;   // k steps per group
   static_assert(G == 64 || G == 128, "group width");
   static_assert(TX == 64 || TX == 128, "X tile rows");
-  static_assert((TX + TYW + MH_REQUANT_TABLE_MAX) * 4 <= XRES_SC_BYTES, "correction area");
+  static_assert((TX + TYW) * 4 + MH_REQUANT_PAIRS_BYTES <= XRES_SC_BYTES, "correction area");
   extern __shared__ __align__(16) uint8_t lds[];
   int32_t *sc = (int32_t *)lds;
   uint8_t *xt = lds + XRES_SC_BYTES;
@@ -1015,12 +1025,7 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
       sc[i] = (int32_t)c;
     }
     if constexpr (sizeof(OutT) == 1) {
-      if (rq.table) {
-        const int32_t *arg_tab = (const int32_t *)((const char *)__builtin_amdgcn_kernarg_segment_ptr() +
-                                                   sizeof(GemmParams));
-        int32_t *tab = sc + TX + TYW;
-        for (int j = tid; j <= rq.n + 1; j += 256) tab[j] = arg_tab[j];
-      }
+      if (rq.table) stage_requant_pairs(sc + TX + TYW, rq, tid, 256);
     }
     __syncthreads();
   } else {
@@ -1065,12 +1070,7 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
       sc[row] = (int32_t)c;
     }
     if constexpr (sizeof(OutT) == 1) {
-      if (rq.table) {
-        const int32_t *arg_tab = (const int32_t *)((const char *)__builtin_amdgcn_kernarg_segment_ptr() +
-                                                   sizeof(GemmParams));
-        int32_t *tab = sc + TX + TYW;
-        for (int j = tid; j <= rq.n + 1; j += 256) tab[j] = arg_tab[j];
-      }
+      if (rq.table) stage_requant_pairs(sc + TX + TYW, rq, tid, 256);
     }
     __syncthreads();
   }
@@ -1171,7 +1171,7 @@ __global__ __launch_bounds__(256, (FX * KS <= 2 ? 4 : (FX * KS <= 4 ? 3 : (FX * 
 void q8_gemm_stream_kernel(GemmParams p, RequantTable) {
   constexpr int YW = 4 / XW;   // wavefronts of the workgroup along Y
   __shared__ int32_t s_cx[32 * FX * XW];
-  __shared__ int32_t s_tab[MH_REQUANT_TABLE_MAX];
+  __shared__ __align__(8) int32_t s_tab[MH_REQUANT_PAIRS_BYTES / 4];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -1204,11 +1204,7 @@ void q8_gemm_stream_kernel(GemmParams p, RequantTable) {
       s_cx[x] = (int32_t)c;
     }
   }
-  {
-    const int32_t *arg_tab = (const int32_t *)((const char *)__builtin_amdgcn_kernarg_segment_ptr() +
-                                               sizeof(GemmParams));
-    for (int j = tid; j <= rq.n + 1; j += 256) s_tab[j] = arg_tab[j];
-  }
+  stage_requant_pairs(s_tab, rq, tid, 256);
   __syncthreads();
 
   const int nblk = (p.YN + 31) / 32;
@@ -1224,8 +1220,6 @@ void q8_gemm_stream_kernel(GemmParams p, RequantTable) {
   v4i yf[D][KS];
 #pragma unroll
   for (int d = 0; d < D; ++d) load_y(blk + d * stride, yf[d]);
-  const float top = (float)rq.n + 0.5f;
-  const uint32_t lo4 = (uint32_t)rq.lo * 0x01010101u;
 
   while (blk < nblk) {
 #pragma unroll
@@ -1263,18 +1257,8 @@ void q8_gemm_stream_kernel(GemmParams p, RequantTable) {
             for (int e = 0; e < 4; ++e)
               v[q * 4 + e] = (int32_t)((uint32_t)acc[q * 4 + e] + (uint32_t)cx[e] + cy);
           }
-          int c[16], t[16];
-#pragma unroll
-          for (int r = 0; r < 16; ++r)
-            c[r] = (int)__builtin_amdgcn_fmed3f(__fmaf_rn((float)v[r], rq.inv, rq.off), 0.0f, top);
-#pragma unroll
-          for (int r = 0; r < 16; ++r) t[r] = s_tab[c[r] + 1];
-          uint32_t packed[4] = {0, 0, 0, 0};
-#pragma unroll
-          for (int r = 0; r < 16; ++r)
-            packed[r / 4] |= (uint32_t)(c[r] + (v[r] > t[r] ? 1 : 0)) << (8 * (r % 4));
-#pragma unroll
-          for (int q = 0; q < 4; ++q) packed[q] += lo4;
+          uint32_t packed[4];
+          requant_16_by_table(v, rq, s_tab, packed);
           const v2u s02 = __builtin_amdgcn_permlane32_swap(packed[0], packed[2], false, false);
           const v2u s13 = __builtin_amdgcn_permlane32_swap(packed[1], packed[3], false, false);
           const v4i w = {(int)s02.x, (int)s02.y, (int)s13.x, (int)s13.y};
