@@ -481,6 +481,46 @@ def bench_other(ctx, mh, torch):
             tf = flops / (k * 1e-3) / 1e12
             out.append({"workload": "f32_gemm_4x1024^3_ta%d_tb%d" % (ta, tb), "kernel_ms": round(k, 4),
                         "TFLOPS": round(tf, 1), "frac_of_fp32_mfma_peak": round(tf / 157.3, 4)})
+    # fp32 Gemv (FullyConnected) 4096 x 4096, batch 1: weights rotated over a set larger than the
+    # last-level cache; and the fp32 1x1 convolution (NCHW, bias + ReLU6 fused into the store) on
+    # two of the MobileNet shapes at batch 64
+    nbuf = 10
+    wf = [torch.randn((4096, 4096), dtype=torch.float32, device="cuda", generator=g) for _ in range(nbuf)]
+    xf = torch.randn((1, 4096), dtype=torch.float32, device="cuda", generator=g)
+    bf = torch.randn((4096,), dtype=torch.float32, device="cuda", generator=g)
+    yf = torch.empty((1, 4096), dtype=torch.float32, device="cuda")
+    fn = ctx.lib.mace_hip_gemv_f32
+    wp = [w.data_ptr() for w in wf]
+    torch.cuda.synchronize()
+    for i in range(30):
+        fn(ctx.handle, wp[i % nbuf], xf.data_ptr(), bf.data_ptr(), 1, 4096, 4096, 0, 1, yf.data_ptr())
+    ctx.sync()
+    ctx.timer_start()
+    for i in range(200):
+        fn(ctx.handle, wp[i % nbuf], xf.data_ptr(), bf.data_ptr(), 1, 4096, 4096, 0, 1, yf.data_ptr())
+    t = ctx.timer_stop() / 200
+    fb = 4096 * 4096 * 4 + 3 * 4096 * 4
+    out.append({"workload": "f32_gemv_4096x4096_b1", "call_us": round(t * 1e3, 2),
+                "GBps": round(fb / (t * 1e-3) / 1e9, 1),
+                "frac_of_hbm_peak": round(fb / (t * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)})
+    del wf
+    for (n, hw, cin, cout) in ((64, 56, 128, 128), (64, 14, 512, 512)):
+        x = torch.randn((n, cin, hw * hw), dtype=torch.float32, device="cuda", generator=g)
+        f = torch.randn((cout, cin), dtype=torch.float32, device="cuda", generator=g)
+        bias = torch.randn((cout,), dtype=torch.float32, device="cuda", generator=g)
+        y = torch.empty((n, cout, hw * hw), dtype=torch.float32, device="cuda")
+        torch.cuda.synchronize()
+        whole, k = time_kernel(ctx, bind(ctx, "mace_hip_conv1x1_f32_nchw", x.data_ptr(), f.data_ptr(),
+                                         bias.data_ptr(), n, cin, hw * hw, cout, mh.ACT_RELUX, 6.0,
+                                         y.data_ptr()))
+        flops = 2.0 * n * hw * hw * cin * cout
+        nbytes = 4.0 * (n * hw * hw * (cin + cout) + cout * cin + cout)
+        roof = min(157.3, flops / nbytes * PEAK_HBM_GBS / 1e3)
+        t = min(whole, k)
+        out.append({"workload": "f32_conv1x1_nchw_n%d_%dx%dx%d_to_%d" % (n, hw, hw, cin, cout),
+                    "call_ms": round(whole, 4), "kernel_ms": round(k, 4),
+                    "TFLOPS": round(flops / (t * 1e-3) / 1e12, 1), "roofline_TFLOPS": round(roof, 1),
+                    "frac_of_roofline": round(flops / (t * 1e-3) / 1e12 / roof, 4)})
     # The Gemv kernel where launch ramp and first-byte latency no longer dominate: 16384 x 16384
     # weights (256 MiB per launch, rotating over three matrices), batch 1.
     Hb = Wb = 16384

@@ -187,22 +187,24 @@ __global__ __launch_bounds__(256 * SPLIT) void f32_gemm_vec_kernel(F32GemmParams
 #pragma unroll
   for (int i = 0; i < NP; ++i) {
     const int f = tid + i * NT;
+    // Rows / columns past the end of a ragged last tile re-read the last valid ones (the host
+    // checks that those come in whole pieces of four); their results are not stored.
     if (LK) {   // 4 consecutive k of row m
       const int m = f / KQ, k4 = f % KQ;
-      pa[i] = A + (int64_t)(m0 + m) * p.lrs + 4 * k4;
+      pa[i] = A + (int64_t)min(m0 + m, p.M - 1) * p.lrs + 4 * k4;
       sa_off[i] = (4 * k4) * LDT + m;
     } else {    // 4 consecutive m of depth k
       const int k = f >> 5, m4 = f & 31;
-      pa[i] = A + (int64_t)k * p.lcs + m0 + 4 * m4;
+      pa[i] = A + (int64_t)k * p.lcs + min(m0 + 4 * m4, p.M - 4);
       sa_off[i] = k * LDT + 4 * m4;
     }
     if (RK) {
       const int n = f / KQ, k4 = f % KQ;
-      pb[i] = B + (int64_t)(n0 + n) * p.rcs + 4 * k4;
+      pb[i] = B + (int64_t)min(n0 + n, p.N - 1) * p.rcs + 4 * k4;
       sb_off[i] = (4 * k4) * LDT + n;
     } else {
       const int k = f >> 5, n4 = f & 31;
-      pb[i] = B + (int64_t)k * p.rrs + n0 + 4 * n4;
+      pb[i] = B + (int64_t)k * p.rrs + min(n0 + 4 * n4, p.N - 4);
       sb_off[i] = k * LDT + 4 * n4;
     }
   }
@@ -322,6 +324,7 @@ __global__ __launch_bounds__(256 * SPLIT) void f32_gemm_vec_kernel(F32GemmParams
   }
 
   float *O = p.out + (int64_t)b * p.obs;
+  const bool whole = m0 + TM <= p.M && n0 + TN <= p.N;
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -330,10 +333,12 @@ __global__ __launch_bounds__(256 * SPLIT) void f32_gemm_vec_kernel(F32GemmParams
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        float v = acc[i][j][r];
-        if (p.bias_row) v = v + p.bias_row[m];
-        v = apply_act(v, p.act, p.limit);
-        O[(int64_t)m * p.ors + (int64_t)n * p.ocs] = v;
+        if (whole || (m < p.M && n < p.N)) {
+          float v = acc[i][j][r];
+          if (p.bias_row) v = v + p.bias_row[m];
+          v = apply_act(v, p.act, p.limit);
+          O[(int64_t)m * p.ors + (int64_t)n * p.ocs] = v;
+        }
       }
     }
 }
@@ -410,8 +415,11 @@ int mh_f32_gemm(mace_hip_ctx *ctx, const float *lhs, const float *rhs, int64_t b
   const bool lk = lhs_major == MACE_HIP_ROW_MAJOR;   // depth contiguous
   const bool rk = rhs_major == MACE_HIP_COL_MAJOR;
   MH_PROF_BEGIN(ctx);
-  const bool vec = rows % TM == 0 && cols % TN == 0 && depth % TK == 0 &&
-                   ((uintptr_t)lhs % 16 == 0) && ((uintptr_t)rhs % 16 == 0);
+  // 16-byte pieces: whole k tiles; an operand whose rows run along k may have any number of rows
+  // (a ragged last tile re-reads its last row), one that runs along m / n needs them in fours
+  const bool vec = depth % TK == 0 && (lk || rows % 4 == 0) && (rk || cols % 4 == 0) &&
+                   rows >= 4 && cols >= 4 && ((uintptr_t)lhs % 16 == 0) &&
+                   ((uintptr_t)rhs % 16 == 0);
   if (vec && split && lk && rk) hipLaunchKernelGGL((f32_gemm_vec_kernel<true, true, 2>), grid, block2, 0, ctx->stream, p);
   else if (vec && split && lk) hipLaunchKernelGGL((f32_gemm_vec_kernel<true, false, 2>), grid, block2, 0, ctx->stream, p);
   else if (vec && split && rk) hipLaunchKernelGGL((f32_gemm_vec_kernel<false, true, 2>), grid, block2, 0, ctx->stream, p);

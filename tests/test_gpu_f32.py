@@ -48,6 +48,12 @@ GEMM_CASES += [(3, 47, 69, 37, R, R, R, True, False), (3, 47, 69, 37, R, R, R, F
 GEMM_CASES += [(2, 256, 128, 48, lm, rm, om, True, True)
                for lm in (R, Cm) for rm in (R, Cm) for om in (R, Cm)]
 GEMM_CASES += [(3, 128, 384, 80, Cm, R, R, False, True), (3, 384, 128, 16, R, Cm, Cm, True, False)]
+# ragged last tiles through the same kernel (depth a multiple of 16; rows / columns in fours
+# where the operand runs along them, any count where it runs along k)
+GEMM_CASES += [(2, 200, 260, 48, lm, rm, om, True, True)
+               for lm in (R, Cm) for rm in (R, Cm) for om in (R, Cm)]
+GEMM_CASES += [(1, 131, 77, 32, R, Cm, R, True, True), (3, 100, 324, 128, R, R, R, False, True),
+               (2, 4, 8, 16, Cm, R, Cm, True, True), (1, 260, 4, 64, R, R, R, True, True)]
 # the shapes of the Gemm call the reference's Winograd convolution makes
 # (mace/ops/arm/base/conv_2d_3x3_winograd.cc:191-204: batch = transformed tile area 16 or 64,
 # rows = output channels, depth = input channels, cols = number of tiles, all row-major, both
