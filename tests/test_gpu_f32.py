@@ -125,7 +125,11 @@ def test_gemm_f32_config2(ctx, ta, tb):
 GEMV_CASES = [(1, 16, 4, True, True), (1, 16, 256, True, True), (2, 16, 256, True, True),
               (3, 63, 257, True, True), (2, 16, 256, False, True), (3, 63, 257, False, True),
               (2, 16, 256, True, False), (3, 63, 257, True, False), (1, 253, 30001, False, True),
-              (2, 300, 253, True, True)]
+              (2, 300, 253, True, True),
+              # rows of whole 16-byte pieces: the 16-byte-load kernel, one, two and four vectors per
+              # pass, ragged batches, width tails of one to three 64-piece steps
+              (3, 70, 1024, False, True), (5, 33, 2052, False, True), (8, 9, 260, False, True),
+              (2, 300, 1024, True, True), (3, 63, 256, True, False), (1, 129, 4096 + 512, False, True)]
 # the two Gemv calls of the reference's DynamicLSTM step (mace/ops/dynamic_lstm.cc:301-310,
 # 328-337): batch 1, nothing batched, bias; affine a: [4 cell + ...] x [input + recurrent],
 # affine b: [output] x [cell]
