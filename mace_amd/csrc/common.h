@@ -387,13 +387,19 @@ struct Q8ConvGather {
 // (q8_gemm_fused_small_kernel).  vec: both operands consist of aligned 16-byte pieces; otherwise
 // at least one is read byte by byte, which pays only for shallower and smaller problems
 // (measured: 600 x 600 x 300 still wins, depth 500 loses; with 16-byte pieces 1024^3 still wins).
+// any_size: the call has no better kernel to go to however large it is (a convolution whose
+// channel count is not a multiple of 64 would otherwise be expanded by im2col; operands read in
+// place whose depth is not a multiple of 64 would take the register-staged tiled kernel):
+// measured on MobileNetV2's pointwise shapes at batch 64, the one-launch kernel wins on all of
+// them with 16-byte pieces (28x28x32 -> 192: 33.6 -> 9.2 us) and on the gathered ones
+// (224x224x3 -> 32, 3x3, stride 2: 160 -> 114 us).
 inline bool mh_q8_small_problem(const mace_hip_ctx *ctx, int64_t batch, int64_t rows, int64_t cols,
-                                int64_t depth, bool vec) {
+                                int64_t depth, bool vec, bool any_size = false) {
   const int64_t cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
   const int64_t wgs = ((rows + 63) / 64) * ((cols + 63) / 64) * batch;
   const double macs = (double)batch * rows * cols * depth;
-  return depth > 0 && depth <= (vec ? 1024 : 320) && wgs <= 4 * cus &&
-         macs <= (vec ? 1024.0 : 128.0) * 1024 * 1024;
+  if (depth <= 0 || depth > (vec ? 1024 : 320) || wgs >= (1ll << 31)) return false;
+  return any_size || (wgs <= 4 * cus && macs <= (vec ? 1024.0 : 128.0) * 1024 * 1024);
 }
 
 // Fills device memory with one byte value on the context's stream, with a kernel (a memset node

@@ -1705,7 +1705,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   const bool cv_vec = cv && lhs_direct && cv->cin % 16 == 0 && ((uintptr_t)rhs % 16 == 0);
   const bool cv_small = cv && rhs_ld == 0 && batch == 1 && out_order == MACE_HIP_COL_MAJOR &&
                         lhs_order == MACE_HIP_ROW_MAJOR &&
-                        mh_q8_small_problem(ctx, 1, rows, cols, depth, cv_vec) &&
+                        mh_q8_small_problem(ctx, 1, rows, cols, depth, cv_vec, cv->cin % 64 != 0) &&
                         !getenv("MACE_HIP_NO_SMALL_KERNEL");
   MH_CHECK(ctx, !cv || cv_small ||
                     (rhs_ld == 0 && batch == 1 && out_order == MACE_HIP_COL_MAJOR &&
@@ -1740,9 +1740,20 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     // general path instead: a diagnostic switch, used by the tests to keep both paths covered.
     // (a registered weight keeps its sums and panel for the tiled kernels; the gather has no
     // other kernel for a geometry that is not a multiple of 64 channels, so it always comes here)
+    // Operands read in place with a depth that is not a multiple of 64 have no streaming tiled
+    // kernel to go to: the one-launch kernel takes them at any size -- except the shapes of the
+    // streaming kernel for a small X panel (see `stream` below), which is faster there.
+    const int64_t xn_s = xl ? rows : cols, yn_s = xl ? cols : rows;
+    const bool stream_shape = out_u8 && rq.table && depth == 32 &&
+                              (xn_s == 32 || xn_s == 64 || xn_s == 128) && yn_s >= 1024 &&
+                              ((uintptr_t)out % 16 == 0);
+    const bool in_place = !lhs_t && !rhs_t && lhs_direct && rhs_direct && rhs_ld == 0;
+    const bool any_size = in_place && depth % 64 != 0 && !stream_shape;
     const bool small = cv ? cv_small
-                          : (mh_q8_small_problem(ctx, batch, rows, cols, depth, lhs_vec && rhs_vec) &&
-                             !lhs_w && !rhs_w && !getenv("MACE_HIP_NO_SMALL_KERNEL"));
+                          : (mh_q8_small_problem(ctx, batch, rows, cols, depth, lhs_vec && rhs_vec,
+                                                 any_size) &&
+                             ((!lhs_w && !rhs_w) || any_size) &&
+                             !getenv("MACE_HIP_NO_SMALL_KERNEL"));
     if (small) {
       GemmParams p{};
       const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;

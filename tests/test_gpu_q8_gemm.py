@@ -111,6 +111,9 @@ XRES_SHAPES = [  # batch, rows, depth, cols, lhs order, rhs order, out order
     (2, 260, 64, 48, R, R, R), (1, 96, 128, 700, Cm, Cm, Cm), (1, 4100, 576, 272, R, R, R),
     # long k in 64-row tiles (128 rows would not fit in LDS twice)
     (1, 3136, 1024, 500, R, Cm, R), (1, 4000, 768, 250, R, Cm, R),
+    # operands in place with a depth that is not a multiple of 64: the one-launch kernel at any
+    # size (more workgroups than it otherwise takes)
+    (1, 100000, 48, 40, R, Cm, R), (2, 70000, 144, 24, R, Cm, R),
 ]
 
 
