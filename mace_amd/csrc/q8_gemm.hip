@@ -1161,8 +1161,9 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
 // requantizing epilogue, 16-byte stores.  Both correction vectors are computed here (X once
 // per workgroup, into LDS; Y per block from the fragments), so the call is this one launch.
 //
-// XN = 32 * FX * XW exactly, K = 32 * KS exactly, uint8 output by threshold look-up only,
-// result rows (ldo = XN bytes) and base 16-byte aligned: the host checks all of that.
+// XN a multiple of 16 in (32 (FX XW - 1), 32 FX XW], K = 32 KS or 32 KS - 16, uint8 output by
+// threshold look-up only, result rows (ldo = XN bytes) and base 16-byte aligned: the host checks
+// all of that.
 // (The occupancy in the launch bounds is what the host launches, see launch_gemm_stream; with at
 // most 256 registers per wavefront the compiler also keeps the MFMA results in ordinary VGPRs,
 // which spares the epilogue one register move per output.)
@@ -1185,23 +1186,29 @@ void q8_gemm_stream_kernel(GemmParams p, RequantTable) {
   const RequantFixed rq = p.rq;
   const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
 
-  // this wavefront's X fragments, shifted to int8, and their row sums
+  // K = 32 KS, or 16 less: then the upper half (h = 1) of the last k step does not exist and
+  // counts as zeros (after the shift) on both sides
+  const bool tail_absent = (p.K & 16) && h == 1;
+  const v4i zero4 = {0, 0, 0, 0};
+  // this wavefront's X fragments, shifted to int8, and their row sums; rows past XN (a panel
+  // that does not fill its last 32-row block) repeat the last row and are never stored
   v4i xf[FX][KS];
 #pragma unroll
   for (int i = 0; i < FX; ++i) {
-    const int x = (wx * FX + i) * 32 + r32;
+    const int xi = (wx * FX + i) * 32 + r32;
+    const int x = min(xi, p.XN - 1);
     const uint8_t *src = Xb + (int64_t)x * p.ldx + 16 * h;
     int xs = 0;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      xf[i][ks] = *(const v4i *)(src + 32 * ks) ^ flip;
+      xf[i][ks] = (ks == KS - 1 && tail_absent) ? zero4 : (*(const v4i *)(src + 32 * ks) ^ flip);
       xs = sum16_i8(xf[i][ks], xs);
     }
     xs += __shfl_xor(xs, 32, 64);
     if (wy == 0 && h == 0) {
       uint32_t c = (uint32_t)p.xcoef * (uint32_t)xs + (uint32_t)p.xadd;
       if (p.xbias) c += (uint32_t)p.xbias[x];
-      s_cx[x] = (int32_t)c;
+      s_cx[xi] = (int32_t)c;
     }
   }
   stage_requant_pairs(s_tab, rq, tid, 256);
@@ -1215,7 +1222,9 @@ void q8_gemm_stream_kernel(GemmParams p, RequantTable) {
     const int row = min(bk * 32 + r32, p.YN - 1);
     const uint8_t *src = Yb + (int64_t)row * p.ldy + 16 * h;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) yf[ks] = __builtin_nontemporal_load((const v4i *)(src + 32 * ks));
+    for (int ks = 0; ks < KS; ++ks)
+      if (!(ks == KS - 1 && tail_absent))
+        yf[ks] = __builtin_nontemporal_load((const v4i *)(src + 32 * ks));
   };
   v4i yf[D][KS];
 #pragma unroll
@@ -1230,7 +1239,7 @@ void q8_gemm_stream_kernel(GemmParams p, RequantTable) {
         int ys = 0;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-          f[ks] = yf[d][ks] ^ flip;
+          f[ks] = (ks == KS - 1 && tail_absent) ? zero4 : (yf[d][ks] ^ flip);
           ys = sum16_i8(f[ks], ys);
         }
         load_y(cur + D * stride, yf[d]);   // refill this slot for D blocks ahead
@@ -1262,8 +1271,9 @@ void q8_gemm_stream_kernel(GemmParams p, RequantTable) {
           const v2u s02 = __builtin_amdgcn_permlane32_swap(packed[0], packed[2], false, false);
           const v2u s13 = __builtin_amdgcn_permlane32_swap(packed[1], packed[3], false, false);
           const v4i w = {(int)s02.x, (int)s02.y, (int)s13.x, (int)s13.y};
-          // plain stores: measured faster here than non-temporal ones
-          if (y < p.YN) *(v4i *)(orow + (wx * FX + i) * 32) = w;
+          // plain stores: measured faster here than non-temporal ones (XN is a multiple of 16:
+          // a lane's 16 bytes are inside the row or not at all)
+          if (y < p.YN && (wx * FX + i) * 32 + 16 * h < p.XN) *(v4i *)(orow + (wx * FX + i) * 32) = w;
         }
       }
     }
@@ -1649,7 +1659,7 @@ template <int FX, int XW>
 int launch_gemm_stream(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, int batch) {
   constexpr int YW = 4 / XW;
   const int nblk = (p.YN + 31) / 32;
-  const int ks = p.K / 32;
+  const int ks = (p.K + 31) / 32;
   // resident workgroups per CU by register footprint (X fragments dominate)
   const int per_cu = FX * ks <= 2 ? 4 : (FX * ks <= 4 ? 3 : (FX * ks <= 16 ? 2 : 1));
   const int cu = ctx->cu_count > 0 ? ctx->cu_count : 256;
@@ -1667,6 +1677,13 @@ int launch_gemm_stream(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab
 }
 
 }  // namespace
+
+// Shapes of the streaming kernel for a small X panel: depth 16 ... 64 in whole 16-byte pieces, at
+// most 128 X rows in whole 16-byte output pieces, a long Y panel.
+static bool mh_q8_stream_shape(int64_t depth, int64_t xn, int64_t yn) {
+  return depth >= 16 && depth <= 64 && depth % 16 == 0 && xn >= 16 && xn <= 128 && xn % 16 == 0 &&
+         yn >= 1024;
+}
 
 int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8_t *rhs,
                int rhs_order, void *out, int out_order, bool out_u8, int64_t batch,
@@ -1744,8 +1761,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     // kernel to go to: the one-launch kernel takes them at any size -- except the shapes of the
     // streaming kernel for a small X panel (see `stream` below), which is faster there.
     const int64_t xn_s = xl ? rows : cols, yn_s = xl ? cols : rows;
-    const bool stream_shape = out_u8 && rq.table && depth == 32 &&
-                              (xn_s == 32 || xn_s == 64 || xn_s == 128) && yn_s >= 1024 &&
+    const bool stream_shape = out_u8 && rq.table && mh_q8_stream_shape(depth, xn_s, yn_s) &&
                               ((uintptr_t)out % 16 == 0);
     const bool in_place = !lhs_t && !rhs_t && lhs_direct && rhs_direct && rhs_ld == 0;
     const bool any_size = in_place && depth % 64 != 0 && !stream_shape;
@@ -1973,9 +1989,8 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   // long Y panel goes to the streaming kernel, which also sums both panels itself.
   const int64_t xn = x_is_lhs ? rows : cols, yn = x_is_lhs ? cols : rows;
   // (Measured: it wins for K <= 64; from K = 128 on the tiled kernels are as fast.)
-  const bool stream = !cv && out_u8 && rq.table && lhs_direct && rhs_direct &&
-                      (depth == 32 || depth == 64) && (xn == 32 || xn == 64 || xn == 128) &&
-                      yn >= 1024 && ((uintptr_t)out % 16 == 0);
+  const bool stream = !cv && out_u8 && rq.table && lhs_direct && rhs_direct && rhs_ld == 0 &&
+                      mh_q8_stream_shape(depth, xn, yn) && ((uintptr_t)out % 16 == 0);
   const int32_t *sumL = L.sums ? L.sums : corrL, *sumR = R.sums ? R.sums : corrR;
   // An X panel whose tile (64 or 128 rows, all of k) fits in LDS twice per CU goes to the kernel
   // that keeps it there and sums both panels itself.  Measured against the tiled kernels (k from
@@ -2050,9 +2065,10 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     return launch_gemm_xres_any(ctx, p, tab, out_u8, (int)batch, xres_tx, false);
   }
   if (stream) {
-    switch (p.XN) {
-      case 32: return launch_gemm_stream<1, 1>(ctx, p, tab, (int)batch);
-      case 64: return launch_gemm_stream<2, 1>(ctx, p, tab, (int)batch);
+    switch ((p.XN + 31) / 32) {
+      case 1: return launch_gemm_stream<1, 1>(ctx, p, tab, (int)batch);
+      case 2: return launch_gemm_stream<2, 1>(ctx, p, tab, (int)batch);
+      case 3: return launch_gemm_stream<3, 1>(ctx, p, tab, (int)batch);
       default: return launch_gemm_stream<4, 1>(ctx, p, tab, (int)batch);
     }
   }

@@ -192,6 +192,9 @@ def test_q8_gemm_requant_at_every_step(ctx, mult, shift, zp, clamp, rows, cols, 
     (64, 32, 4096, 1), (32, 32, 1031, 1), (128, 128, 2048, 1), (256, 256, 1500, 1),
     (64, 64, 1024, 3), (128, 32, 5000, 1), (256, 64, 1111, 2), (32, 256, 1025, 1),
     (128, 64, 3000, 2), (64, 32, 2049, 1), (64, 128, 1056, 1), (32, 64, 40000, 1),
+    # panels that do not fill their last 32-row block, depths with half a k step at the tail
+    (16, 32, 3000, 1), (96, 16, 2500, 1), (48, 48, 1100, 2), (112, 64, 1500, 1), (80, 16, 1024, 1),
+    (128, 48, 20000, 1), (16, 16, 5000, 1),
 ])
 @pytest.mark.parametrize("x_is_lhs", [True, False])
 def test_q8_gemm_small_panel_streaming(ctx, xn, depth, yn, batch, x_is_lhs):
