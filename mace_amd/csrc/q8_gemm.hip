@@ -203,8 +203,12 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[FX][FY], const int (&y
         cy = (uint32_t)sc[TX + yl];
       }
       OutT *orow = outb + (int64_t)y * p.ldo + x0;
+      // 32 x 32 blocks that lie outside the matrix altogether (ragged last tiles) are skipped
+      // before their requantization, not after (uniform over the wavefront)
+      if (y0 + (wy * FY + j) * 32 >= p.YN) continue;
 #pragma unroll
       for (int i = 0; i < FX; ++i) {
+        if (x0 + (wx * FX + i) * 32 >= p.XN) continue;
         const int xb = (wx * FX + i) * 32 + 4 * (lane >> 5);   // x of register group q: xb + 8 q
         int32_t v[16];
 #pragma unroll
@@ -1299,6 +1303,26 @@ __global__ void q8_pack_rows_kernel(const uint8_t *src, int64_t src_bs, uint8_t 
   }
 }
 
+// The same for k % 4 == 0 and a 4-byte aligned base: one thread per 16 bytes of the padded row,
+// read as four dwords (a 24-channel activation tensor: rows of six dwords become rows of 64 bytes).
+__global__ void q8_pack_rows4_kernel(const uint8_t *src, int64_t src_bs, uint8_t *dst,
+                                     int64_t dst_bs, int n, int k, int kp) {
+  const int cpr = kp >> 4;   // 16-byte pieces per padded row
+  const int64_t total = (int64_t)n * cpr;
+  const uint32_t *s = (const uint32_t *)(src + (int64_t)blockIdx.z * src_bs);
+  uint8_t *d = dst + (int64_t)blockIdx.z * dst_bs;
+  const int k4 = k >> 2;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / cpr;
+    const int c4 = (int)(i - r * cpr) * 4;   // first dword of the piece inside the row
+    v4i v;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = c4 + e < k4 ? (int)s[r * k4 + c4 + e] : (int)0x80808080;
+    *(v4i *)(d + i * 16) = v;
+  }
+}
+
 // src is [k][n] with n contiguous (row stride = n): write dst [n][kp], padding k..kp with
 // 0x80.  64x64-byte tiles through LDS; 16-byte global accesses when n % 16 == 0 and the
 // base is aligned, byte accesses otherwise.
@@ -1880,10 +1904,17 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
                   int32_t *fused_sums, bool *fused) -> int {
     if (fused) *fused = false;
     if (order_is_kcontig) {
-      const int64_t total = n * kp;
-      dim3 grid((unsigned)std::min<int64_t>((total + 255) / 256, 65535), 1, nb);
-      hipLaunchKernelGGL(q8_pack_rows_kernel, grid, dim3(256), 0, ctx->stream, src,
-                         n * depth, dst, n * kp, (int)n, (int)depth, (int)kp);
+      if (depth % 4 == 0 && (uintptr_t)src % 4 == 0) {
+        const int64_t total = n * (kp / 16);
+        dim3 grid((unsigned)std::min<int64_t>((total + 255) / 256, 1 << 20), 1, nb);
+        hipLaunchKernelGGL(q8_pack_rows4_kernel, grid, dim3(256), 0, ctx->stream, src,
+                           n * depth, dst, n * kp, (int)n, (int)depth, (int)kp);
+      } else {
+        const int64_t total = n * kp;
+        dim3 grid((unsigned)std::min<int64_t>((total + 255) / 256, 65535), 1, nb);
+        hipLaunchKernelGGL(q8_pack_rows_kernel, grid, dim3(256), 0, ctx->stream, src,
+                           n * depth, dst, n * kp, (int)n, (int)depth, (int)kp);
+      }
     } else {
       MH_CHECK(ctx, (kp / 64) <= 65535, "depth too large to repack");
       const int vec_ok = (n % 16 == 0) && ((uintptr_t)src % 16 == 0);
