@@ -434,10 +434,21 @@ def bench_other(ctx, mh, torch):
         roof_tops = min(PEAK_INT8_TOPS, ai * PEAK_HBM_GBS / 1e3)
         t = min(whole, k)   # a one-launch call is rated by the call, not by the stopwatch around it
         tops = ops / (t * 1e-3) / 1e12
-        out.append({"workload": "q8_conv1x1_n%d_%dx%dx%d_to_%d" % (n, hw, hw, cin, cout),
-                    "call_ms": round(whole, 4), "kernel_ms": round(k, 4), "TOPS": round(tops, 1),
-                    "GBps": round(nbytes / (t * 1e-3) / 1e9, 1), "ops_per_byte": round(ai, 1),
-                    "roofline_TOPS": round(roof_tops, 1), "frac_of_roofline": round(tops / roof_tops, 4)})
+        entry = {"workload": "q8_conv1x1_n%d_%dx%dx%d_to_%d" % (n, hw, hw, cin, cout),
+                 "call_ms": round(whole, 4), "kernel_ms": round(k, 4), "TOPS": round(tops, 1),
+                 "GBps": round(nbytes / (t * 1e-3) / 1e9, 1), "ops_per_byte": round(ai, 1),
+                 "roofline_TOPS": round(roof_tops, 1), "frac_of_roofline": round(tops / roof_tops, 4)}
+        if n > 1:
+            # the same call with the filter registered as a constant weight, which is what the
+            # delegator adapter does for is_weight() tensors: its row sums are then kept by the
+            # context instead of being taken on every call
+            ctx.call("mace_hip_weight_register", f.data_ptr(), cout * cin)
+            whole_w, _ = time_kernel(ctx, bind(ctx,
+                "mace_hip_conv1x1_q8_nhwc", x.data_ptr(), f.data_ptr(), bias.data_ptr(), n, hw, hw, cin,
+                cout, s_in, 128, s_f, 127, s_in * s_f, s_out, 0, 0, 255, y.data_ptr()))
+            ctx.call("mace_hip_weight_unregister", f.data_ptr())
+            entry["call_ms_filter_registered"] = round(whole_w, 4)
+        out.append(entry)
 
     # beyond the 1x1 shapes: 3x3 convolutions (SAME padding, stride 1); with cin % 64 == 0 the
     # GEMM's loader gathers the patches itself and no im2col matrix is written
