@@ -410,6 +410,20 @@ def bench_other(ctx, mh, torch):
                     "kernel_ms": round(k, 4), "TOPS": round(ops / (t * 1e-3) / 1e12, 1),
                     "frac_of_int8_peak": round(ops / (t * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4)})
 
+    # config 5 with the raw int32 result (MatMulFixpointImpl<..., int32_t>): 4096^3, 256 MiB less
+    # to hold than 8192^3 and the same kernel
+    n = 4096
+    A, B = u8(n, n), u8(n, n)
+    C32 = torch.empty((n, n), dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()
+    whole, k = time_kernel(ctx, bind(ctx, "mace_hip_gemm_q8_i32", A.data_ptr(), 0, B.data_ptr(), 0,
+                                     C32.data_ptr(), 0, 1, n, n, n, 1, 1, -131, -122))
+    ops = 2.0 * n ** 3
+    out.append({"workload": "q8_matmul_1x4096^3_i32out", "call_ms": round(whole, 4),
+                "kernel_ms": round(k, 4), "TOPS": round(ops / (k * 1e-3) / 1e12, 1),
+                "frac_of_int8_peak": round(ops / (k * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4)})
+    del A, B, C32
+
     # config 4: quantized conv 1x1, NHWC, MobileNetV1 pointwise shapes, ReLU6 range: at batch 64 as
     # configured, and at batch 1 (single-image inference, where a call is one small launch)
     for (n, hw, cin, cout) in [(64, hw, ci, co) for (hw, ci, co) in
