@@ -8,6 +8,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <utility>
 #include <vector>
 
 #include "mace_hip.h"
@@ -55,6 +56,8 @@ struct mace_hip_ctx {
   int fail_allocs = 0;              // test hook
   int cu_count = 0;
   int lds_bytes = 0;
+  // kernels whose dynamic LDS limit has been raised, and to how many bytes
+  std::vector<std::pair<const void *, size_t>> big_lds_kernels;
   char arch[64] = {0};
   char err[512] = {0};
   // last few requantization comparison tables built on this context (mult, shift, blo, n)
@@ -400,6 +403,23 @@ inline bool mh_q8_small_problem(const mace_hip_ctx *ctx, int64_t batch, int64_t 
   const double macs = (double)batch * rows * cols * depth;
   if (depth <= 0 || depth > (vec ? 1024 : 320) || wgs >= (1ll << 31)) return false;
   return any_size || (wgs <= 4 * cus && macs <= (vec ? 1024.0 : 128.0) * 1024 * 1024);
+}
+
+// Raises a kernel's dynamic LDS limit to at least `bytes`; remembered per context and kernel, since
+// hipFuncSetAttribute costs about as much as a launch and the attribute stays set.
+inline hipError_t mh_allow_big_lds(mace_hip_ctx *ctx, const void *kernel, size_t bytes) {
+  for (auto &e : ctx->big_lds_kernels)
+    if (e.first == kernel) {
+      if (e.second >= bytes) return hipSuccess;
+      const hipError_t rc =
+          hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+      if (rc == hipSuccess) e.second = bytes;
+      return rc;
+    }
+  const hipError_t rc =
+      hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (rc == hipSuccess) ctx->big_lds_kernels.emplace_back(kernel, bytes);
+  return rc;
 }
 
 // Fills device memory with one byte value on the context's stream, with a kernel (a memset node

@@ -1518,9 +1518,7 @@ int launch_gemm(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, bool 
   const size_t lds = 2 * (size_t)(TX + TY) * LDS_ROW;
   dim3 grid(p.tiles_x * p.tiles_y, 1, batch), block(WX * WY * 64);
   auto launch = [&](auto k) -> int {
-    if (lds > 64 * 1024)
-      MH_HIP(ctx, hipFuncSetAttribute((const void *)k,
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    if (lds > 64 * 1024) MH_HIP(ctx, mh_allow_big_lds(ctx, (const void *)k, lds));
     MH_PROF_BEGIN(ctx);
     hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, tab);
     return MACE_HIP_SUCCESS;
@@ -1549,9 +1547,7 @@ int launch_gemm_dma(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, b
   const size_t lds = (size_t)STAGES * (TX + TY) * KB;
   dim3 grid(p.tiles_x * p.tiles_y, 1, batch), block(WX * WY * 64);
   auto launch = [&](auto k) -> int {
-    if (lds > 64 * 1024)
-      MH_HIP(ctx, hipFuncSetAttribute((const void *)k,
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    if (lds > 64 * 1024) MH_HIP(ctx, mh_allow_big_lds(ctx, (const void *)k, lds));
     MH_PROF_BEGIN(ctx);
     hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, tab);
     return MACE_HIP_SUCCESS;
@@ -1626,9 +1622,7 @@ int launch_gemm_xres(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, 
   MH_CHECK(ctx, tiles_x <= 65535 && batch <= 65535, "grid too large");
   dim3 grid(wgs, tiles_x, batch), block(256);
   auto launch = [&](auto k) -> int {
-    if (lds > 64 * 1024)
-      MH_HIP(ctx, hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      (int)lds));
+    if (lds > 64 * 1024) MH_HIP(ctx, mh_allow_big_lds(ctx, (const void *)k, lds));
     MH_PROF_BEGIN(ctx);
     hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, tab);
     MH_PROF_END(ctx);

@@ -490,9 +490,7 @@ int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
     const size_t lds_max = (ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536) - 2048;
     if (lds <= lds_max) {
       auto k = q8_gemv_mfma_lds_kernel<OutT>;
-      if (lds > 48 * 1024)
-        MH_HIP(ctx, hipFuncSetAttribute((const void *)k,
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      if (lds > 48 * 1024) MH_HIP(ctx, mh_allow_big_lds(ctx, (const void *)k, lds));
       MH_PROF_BEGIN(ctx);
       hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, pitch);
     } else {
