@@ -60,6 +60,15 @@ GEMM_CASES += [(1, 131, 77, 32, R, Cm, R, True, True), (3, 100, 324, 128, R, R, 
 # operands batched)
 GEMM_CASES += [(16, 32, 49, 16, R, R, R, True, True), (64, 64, 196, 32, R, R, R, True, True),
                (16, 24, 9, 3, R, R, R, True, True), (64, 128, 256, 128, R, R, R, True, True)]
+# more tiles than the chip has compute units (the four-wavefront variant of the 16-byte-load
+# kernel; every case above stays at or below 256 tiles and takes the eight-wavefront one):
+# whole tiles and ragged last tiles in every layout, one-sided batching, odd row counts where
+# the operand runs along k
+GEMM_CASES += [(1, 2304, 2304, 64, lm, rm, om, True, True)
+               for lm in (R, Cm) for rm in (R, Cm) for om in (R, Cm)]
+GEMM_CASES += [(3, 1100, 1300, 48, lm, rm, R, True, True) for lm in (R, Cm) for rm in (R, Cm)]
+GEMM_CASES += [(3, 1101, 1303, 48, R, Cm, Cm, True, True), (5, 900, 1028, 32, Cm, R, R, False, True),
+               (5, 1028, 900, 32, R, R, Cm, True, False), (2, 2048, 2304, 32, R, R, R, True, True)]
 
 
 @pytest.mark.parametrize("batch,rows,cols,depth,lm,rm,om,lb,rb", GEMM_CASES)
@@ -95,11 +104,12 @@ def test_gemm_f32_reference_goldens(ctx, case):
 
 @pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
 def test_gemm_f32_config2(ctx, ta, tb):
-    """benchmark configuration 2 at batch 4, 512^3 (the 1024^3 size runs in the benchmark; the
-    scalar oracle needs ~1 s per 512^3 batch): N(0,1), all four transpose combinations,
-    plus one non-batched lhs."""
+    """benchmark configuration 2 at its stated size (batch 4, 1024^3): N(0,1), all four
+    transpose combinations, plus one non-batched lhs.  Checked with the reference's own
+    tolerance form against the binary32 serial loop and the binary64-accumulated one, and
+    with the 1e-4 normwise bound."""
     rng = np.random.default_rng(2)
-    b, n = 4, 512
+    b, n = 4, 1024
     A = rng.standard_normal((b, n, n)).astype(np.float32)
     B = rng.standard_normal((b, n, n)).astype(np.float32)
     d = Dev()
@@ -110,8 +120,8 @@ def test_gemm_f32_config2(ctx, ta, tb):
     ctx.sync()
     got = t.cpu().numpy().copy()
     lm, rm = (Cm if ta else R), (Cm if tb else R)
-    want = orc.gemm_f32(A, B, b, n, n, n, lm, rm, R)
-    want64 = orc.gemm_f32(A, B, b, n, n, n, lm, rm, R, acc64=True)
+    want = orc.gemm_f32(A, B, b, n, n, n, lm, rm, R, nthreads=16)
+    want64 = orc.gemm_f32(A, B, b, n, n, n, lm, rm, R, acc64=True, nthreads=16)
     near(got, want)
     near(got, want64)
     rel = np.linalg.norm(got.astype(np.float64) - want64) / np.linalg.norm(want64)
@@ -119,7 +129,32 @@ def test_gemm_f32_config2(ctx, ta, tb):
     if ta == 0 and tb == 0:
         ctx.call("mace_hip_gemm_f32_transpose", dA, dB, b, n, n, n, n, 0, 0, 0, 0, 1, p)
         ctx.sync()
-        near(t.cpu().numpy(), orc.gemm_f32(A[0], B, b, n, n, n, R, R, R, False, True, acc64=True))
+        near(t.cpu().numpy(), orc.gemm_f32(A[0], B, b, n, n, n, R, R, R, False, True, acc64=True,
+                                           nthreads=16))
+
+
+def test_gemm_f32_config2_small(ctx):
+    """the same at 4 x 512^3: at most one tile per compute unit, i.e. the eight-wavefront
+    variant of the kernel, in all four transpose combinations."""
+    rng = np.random.default_rng(22)
+    b, n = 4, 512
+    A = rng.standard_normal((b, n, n)).astype(np.float32)
+    B = rng.standard_normal((b, n, n)).astype(np.float32)
+    d = Dev()
+    t, p = d.empty(b * n * n, np.float32)
+    dA, dB = d.put(A), d.put(B)
+    d.sync()
+    for ta in (0, 1):
+        for tb in (0, 1):
+            ctx.call("mace_hip_gemm_f32_transpose", dA, dB, b, n, n, n, n, ta, tb, 0, 1, 1, p)
+            ctx.sync()
+            got = t.cpu().numpy().copy()
+            lm, rm = (Cm if ta else R), (Cm if tb else R)
+            want64 = orc.gemm_f32(A, B, b, n, n, n, lm, rm, R, acc64=True, nthreads=16)
+            near(got, orc.gemm_f32(A, B, b, n, n, n, lm, rm, R, nthreads=16))
+            near(got, want64)
+            rel = np.linalg.norm(got.astype(np.float64) - want64) / np.linalg.norm(want64)
+            assert rel <= 1e-4, rel
 
 
 GEMV_CASES = [(1, 16, 4, True, True), (1, 16, 256, True, True), (2, 16, 256, True, True),
@@ -188,3 +223,32 @@ def test_conv1x1_f32_golden_and_random(ctx):
                 assert out.min() >= 0.0 and (act != mh.ACT_RELUX or out.max() <= limit)
     assert ctx.status("mace_hip_conv1x1_f32_nchw_host", ptr(x), ptr(f), None, n, cin, hw, cout,
                       9, 0.0, ptr(out)) == mh.INVALID_ARGS
+
+
+@pytest.mark.parametrize("n,cin,h,cout,act,limit,with_bias",
+                         [(64, 128, 56, 128, mh.ACT_RELUX, 6.0, True),
+                          (64, 512, 14, 512, mh.ACT_RELU, 0.0, True),
+                          (16, 64, 56, 256, mh.ACT_NOOP, 0.0, False)])
+def test_conv1x1_f32_nchw_batch64(ctx, n, cin, h, cout, act, limit, with_bias):
+    """MobileNet pointwise layers at batch 64 on device tensors: thousands of tiles with a
+    ragged last column tile (3136 and 196 are not multiples of 128), bias and activation
+    fused into the store."""
+    rng = np.random.default_rng(n * 31 + cin + h)
+    hw = h * h
+    x = rng.standard_normal((n, cin, hw)).astype(np.float32)
+    f = (rng.standard_normal((cout, cin)) / np.sqrt(cin)).astype(np.float32)
+    b = rng.standard_normal(cout).astype(np.float32) if with_bias else None
+    d = Dev()
+    t, p = d.empty(n * cout * hw, np.float32)
+    dx, df, db = d.put(x), d.put(f), d.put(b)
+    d.sync()
+    ctx.call("mace_hip_conv1x1_f32_nchw", dx, df, db, n, cin, hw, cout, act, limit, p)
+    ctx.sync()
+    got = t.cpu().numpy()
+    want = orc.conv1x1_f32_nchw(x, f, b, n, cin, hw, cout, act, limit, nthreads=16).reshape(-1)
+    near(got, want)
+    rel = np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want)
+    assert rel <= 1e-4, rel
+    if act != mh.ACT_NOOP:
+        assert got.min() >= 0.0 and (act != mh.ACT_RELUX or got.max() <= limit)
+        assert (got == 0.0).any() and (act != mh.ACT_RELUX or (got == limit).any() or limit > 5)
