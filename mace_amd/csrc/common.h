@@ -67,7 +67,11 @@ struct mace_hip_ctx {
   int rq_cache_next = 0;
   std::vector<mh_weight> weights;
   long weight_hits = 0, weight_builds = 0;   // statistics for tests
+  // Test hook (mace_hip_ctx_set_kernel_mask): kernel families switched off for this context, so
+  // that the tests reach every family on the same shapes.
+  int kernel_mask = 0;
 };
+constexpr int MH_MASK_NO_SMALL = 1, MH_MASK_NO_XRES = 2, MH_MASK_NO_SPLITK = 4;
 
 int mh_fail(mace_hip_ctx *ctx, int code, const char *fmt, ...);
 

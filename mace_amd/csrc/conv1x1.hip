@@ -155,7 +155,7 @@ extern "C" int mace_hip_conv2d_q8_nhwc(mace_hip_ctx *ctx, const uint8_t *input,
                          ((uintptr_t)filter % 16 == 0);
   const bool small_gather = !in_place && in_h * in_w * cin < (1ll << 31) &&
                             mh_q8_small_problem(ctx, 1, cout, columns, depth, small_vec, cin % 64 != 0) &&
-                            !getenv("MACE_HIP_NO_SMALL_KERNEL");
+                            !(ctx->kernel_mask & MH_MASK_NO_SMALL);
   const bool gather = small_gather ||
                       (!in_place && cin % 64 == 0 && depth >= 192 && ((uintptr_t)input % 16 == 0) &&
                        ((uintptr_t)filter % 16 == 0) && in_h * in_w * cin < (1ll << 31));

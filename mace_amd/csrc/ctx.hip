@@ -232,6 +232,12 @@ int mace_hip_profile_last_kernel_ms(mace_hip_ctx *ctx, float *elapsed_ms) {
   return mace_hip_profile_kernel_ms(ctx, ctx->prof_count - 1, elapsed_ms);
 }
 
+int mace_hip_ctx_set_kernel_mask(mace_hip_ctx *ctx, int mask) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  ctx->kernel_mask = mask;
+  return MACE_HIP_SUCCESS;
+}
+
 int mace_hip_ctx_fail_next_allocs(mace_hip_ctx *ctx, int n) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   ctx->fail_allocs = n;

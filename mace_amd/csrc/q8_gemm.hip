@@ -1741,7 +1741,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   const bool cv_small = cv && rhs_ld == 0 && batch == 1 && out_order == MACE_HIP_COL_MAJOR &&
                         lhs_order == MACE_HIP_ROW_MAJOR &&
                         mh_q8_small_problem(ctx, 1, rows, cols, depth, cv_vec, cv->cin % 64 != 0) &&
-                        !getenv("MACE_HIP_NO_SMALL_KERNEL");
+                        !(ctx->kernel_mask & MH_MASK_NO_SMALL);
   MH_CHECK(ctx, !cv || cv_small ||
                     (rhs_ld == 0 && batch == 1 && out_order == MACE_HIP_COL_MAJOR &&
                      lhs_order == MACE_HIP_ROW_MAJOR && depth % SLAB == 0 && depth >= 3 * SLAB &&
@@ -1771,8 +1771,8 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     const bool lhs_vec = lhs_t ? (rows % 16 == 0 && (uintptr_t)lhs % 16 == 0) : lhs_direct;
     const bool rhs_vec = cv ? (cv->cin % 16 == 0 && (uintptr_t)rhs % 16 == 0)
                             : (rhs_t ? (cols % 16 == 0 && (uintptr_t)rhs % 16 == 0) : rhs_direct);
-    // The environment variable MACE_HIP_NO_SMALL_KERNEL (any value) sends every call down the
-    // general path instead: a diagnostic switch, used by the tests to keep both paths covered.
+    // Bit MH_MASK_NO_SMALL of the context's kernel mask sends every call down the general path
+    // instead: a test hook, used by the tests to keep both paths covered.
     // (a registered weight keeps its sums and panel for the tiled kernels; the gather has no
     // other kernel for a geometry that is not a multiple of 64 channels, so it always comes here)
     // Operands read in place with a depth that is not a multiple of 64 have no streaming tiled
@@ -1787,7 +1787,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
                           : (mh_q8_small_problem(ctx, batch, rows, cols, depth, lhs_vec && rhs_vec,
                                                  any_size) &&
                              ((!lhs_w && !rhs_w) || any_size) &&
-                             !getenv("MACE_HIP_NO_SMALL_KERNEL"));
+                             !(ctx->kernel_mask & MH_MASK_NO_SMALL));
     if (small) {
       GemmParams p{};
       const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
@@ -1847,7 +1847,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     const size_t lds_cu = ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536;
     if (!cv && x_kmajor && y_direct && rhs_ld == 0 && !lhs_w && !rhs_w && depth > 0 &&
         depth % 64 == 0 && xn % 16 == 0 && (uintptr_t)xp % 16 == 0 && yn >= 256 &&
-        2 * (XRES_SC_BYTES + (size_t)tx * depth) <= lds_cu && !getenv("MACE_HIP_NO_XRES_KERNEL")) {
+        2 * (XRES_SC_BYTES + (size_t)tx * depth) <= lds_cu && !(ctx->kernel_mask & MH_MASK_NO_XRES)) {
       GemmParams p{};
       const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
       const int32_t l_coef = (int32_t)(0u - zr), r_coef = (int32_t)(0u - zl);
@@ -2025,7 +2025,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   // patches the kernel gathers (cin % 64 == 0) takes it whenever the tile fits: 25 % faster
   // than the gathering tiled kernel on 3x3, 56x56x64 -> 64 at batch 64 (splitting a 128-row tile
   // that does not fit into two of 64 rows was slower than the tiled kernel).
-  // (MACE_HIP_NO_XRES_KERNEL, any value: diagnostic switch that keeps the tiled kernels in use.)
+  // (Bit MH_MASK_NO_XRES of the kernel mask: test hook that keeps the tiled kernels in use.)
   const int kk = L.k < R.k ? L.k : R.k;
   const size_t lds_cu = ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536;
   auto xres_fits = [&](int tx) { return 2 * (XRES_SC_BYTES + (size_t)tx * kk) <= lds_cu; };
@@ -2038,8 +2038,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   const int xres_tx = (xn <= 64 || xres_narrow) ? 64 : 128;
   const bool xres_cv = cv && !cv_small && out_u8 && cv->cin % 64 == 0 && depth % 64 == 0;
   const bool xres = (!cv || xres_cv) && !stream && depth > 0 && kk % 64 == 0 && yn >= 256 &&
-                    xres_fits(xres_tx) &&
-                    !getenv("MACE_HIP_NO_XRES_KERNEL");
+                    xres_fits(xres_tx) && !(ctx->kernel_mask & MH_MASK_NO_XRES);
   if (!stream && !xres) {
     if (!L.sums && !(sum_y && !x_is_lhs))
       MH_RETURN_IF_ERROR(launch_panel_sums(ctx, L.ptr, L.ld, L.bs, rows, L.k, lhs_nb, corrL));

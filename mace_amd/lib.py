@@ -13,6 +13,7 @@ SUCCESS, INVALID_ARGS, OUT_OF_RESOURCES, UNSUPPORTED, RUNTIME_ERROR = range(5)
 ROW_MAJOR, COL_MAJOR = 0, 1
 REQUANT_REF, REQUANT_NEON = 0, 1
 ACT_NOOP, ACT_RELU, ACT_RELUX = 0, 1, 2
+MASK_NO_SMALL, MASK_NO_XRES, MASK_NO_SPLITK = 1, 2, 4
 
 _STATUS_NAMES = {0: "MACE_SUCCESS", 1: "MACE_INVALID_ARGS", 2: "MACE_OUT_OF_RESOURCES",
                  3: "MACE_UNSUPPORTED", 4: "MACE_RUNTIME_ERROR"}
@@ -49,6 +50,7 @@ SIGNATURES = {
     "mace_hip_profile_kernel_count": (_int, [_p, C.POINTER(_int)]),
     "mace_hip_profile_kernel_ms": (_int, [_p, _int, C.POINTER(_f32)]),
     "mace_hip_ctx_fail_next_allocs": (_int, [_p, _int]),
+    "mace_hip_ctx_set_kernel_mask": (_int, [_p, _int]),
     "mace_hip_malloc": (_int, [_p, C.c_size_t, C.POINTER(_p)]),
     "mace_hip_free": (_int, [_p, _p]),
     "mace_hip_memcpy_h2d": (_int, [_p, _p, _p, C.c_size_t]),

@@ -88,16 +88,16 @@ CASES = [  # batch, cout, cin, in_h, in_w, k_h, k_w, padding, strides: the refer
 
 
 @pytest.fixture(params=["default", "no_small_kernel", "general_path"])
-def path(request, monkeypatch):
+def path(request, ctx):
     """A small convolution is one launch of the small-problem GEMM kernel, which gathers the
-    patches itself; with MACE_HIP_NO_SMALL_KERNEL it goes to the kernel that keeps the filter in
-    LDS (cin a multiple of 64, filter tile fits) and with MACE_HIP_NO_XRES_KERNEL on top through
+    patches itself; with kernel-mask bit 0 it goes to the kernel that keeps the filter in
+    LDS (cin a multiple of 64, filter tile fits) and with bit 1 on top through
     im2col / the gathering tiled kernel, so that all three stay covered on the same shapes."""
-    if request.param != "default":
-        monkeypatch.setenv("MACE_HIP_NO_SMALL_KERNEL", "1")
-    if request.param == "general_path":
-        monkeypatch.setenv("MACE_HIP_NO_XRES_KERNEL", "1")
-    return request.param
+    mask = {"default": 0, "no_small_kernel": mh.MASK_NO_SMALL,
+            "general_path": mh.MASK_NO_SMALL | mh.MASK_NO_XRES}[request.param]
+    ctx.call("mace_hip_ctx_set_kernel_mask", mask)
+    yield request.param
+    ctx.call("mace_hip_ctx_set_kernel_mask", 0)
 
 
 @pytest.mark.parametrize("n,cout,cin,in_h,in_w,k_h,k_w,pad,st", CASES)

@@ -58,15 +58,15 @@ SHAPES = [  # batch, rows, depth, cols, lhs_batched, rhs_batched
 
 
 @pytest.fixture(params=["default", "no_small_kernel", "general_path"])
-def path(request, monkeypatch):
+def path(request, ctx):
     """Small problems are one launch of a kernel of their own, and an X panel that fits in LDS has
-    one too; MACE_HIP_NO_SMALL_KERNEL leaves the second, MACE_HIP_NO_XRES_KERNEL on top of it only
+    one too; kernel-mask bit 0 leaves the second, bit 1 on top of it only
     the general path (repack, row sums, tiled kernel), so that all three stay covered."""
-    if request.param != "default":
-        monkeypatch.setenv("MACE_HIP_NO_SMALL_KERNEL", "1")
-    if request.param == "general_path":
-        monkeypatch.setenv("MACE_HIP_NO_XRES_KERNEL", "1")
-    return request.param
+    mask = {"default": 0, "no_small_kernel": mh.MASK_NO_SMALL,
+            "general_path": mh.MASK_NO_SMALL | mh.MASK_NO_XRES}[request.param]
+    ctx.call("mace_hip_ctx_set_kernel_mask", mask)
+    yield request.param
+    ctx.call("mace_hip_ctx_set_kernel_mask", 0)
 
 
 @pytest.mark.parametrize("batch,rows,depth,cols,lb,rb", SHAPES)
