@@ -244,6 +244,27 @@ int mace_hip_gemm_q8_u8(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order,
                         int32_t rhs_offset, const int32_t *bias /* [rows] or NULL */,
                         int32_t multiplier, int right_shift, int32_t offset_after_shift,
                         int clamp_min, int clamp_max);
+
+/* mace_hip_gemm_q8_u8 for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same arguments, same kernels, same results; the repacked panels and correction
+ * vectors, which mace_hip_gemm_q8_u8 keeps in the context's growing arena, live in an array of
+ * MACE_HIP_NOALLOC_SCRATCH_BYTES that is part of the library's code object (every GPU the
+ * library runs on holds it until the process ends).  The call allocates and frees nothing;
+ * operands registered with mace_hip_weight_register are treated like any other (the weight
+ * cache allocates).  A shape that needs more scratch -- roughly 4 (rows + cols) bytes per batch
+ * plus rows x depth for a ColMajor lhs and depth x cols for a RowMajor rhs, depth rounded up to
+ * 64 -- returns MACE_INVALID_ARGS with the figures in mace_hip_last_error.  All contexts of a
+ * GPU share the one array: calls that overlap in time on one GPU (two contexts, two streams)
+ * race on it; the caller serializes them. */
+#define MACE_HIP_NOALLOC_SCRATCH_BYTES (32u << 20)
+int mace_hip_gemm_q8_u8_noalloc(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order,
+                                const uint8_t *rhs, int rhs_order, uint8_t *out, int out_order,
+                                int64_t batch, int64_t rows, int64_t depth, int64_t cols,
+                                int lhs_batched, int rhs_batched, int32_t lhs_offset,
+                                int32_t rhs_offset, const int32_t *bias /* or NULL */,
+                                int32_t multiplier, int right_shift,
+                                int32_t offset_after_shift, int clamp_min, int clamp_max);
 /* Conv2dOp<RT_CPU, uint8_t>::Run for a 1x1 filter, stride 1, dilation 1
  * (mace/ops/conv_2d.cc:201-318 with im2col_required == false): input NHWC, filter OHWI
  * [cout][cin], bias int32 [cout] or NULL with its own scale (rescaled as GetBiasData does,

@@ -67,6 +67,11 @@ struct mace_hip_ctx {
   int rq_cache_next = 0;
   std::vector<mh_weight> weights;
   long weight_hits = 0, weight_builds = 0;   // statistics for tests
+  // This device's copy of the library's static scratch array (see ctx.hip), and whether the call
+  // in progress is one that must not allocate: then the arena is that array, a reservation
+  // beyond its size is an error, and the weight cache (which allocates on first use) is bypassed.
+  char *static_scratch = nullptr;
+  bool no_alloc = false;
   // Test hook (mace_hip_ctx_set_kernel_mask): kernel families switched off for this context, so
   // that the tests reach every family on the same shapes.
   int kernel_mask = 0;

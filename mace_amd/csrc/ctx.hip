@@ -17,10 +17,35 @@ int mh_fail(mace_hip_ctx *ctx, int code, const char *fmt, ...) {
   return code;
 }
 
+// Scratch for the entry point that allocates nothing: one array per GPU, part of the code
+// object, held from the first use of the library on that GPU until the process ends.  Host
+// code never uses the array's name as an address; it asks the runtime for this device's copy
+// (mh_static_scratch) and passes that pointer on.
+static __device__ __align__(256) unsigned char scratch[MACE_HIP_NOALLOC_SCRATCH_BYTES];
+constexpr int MH_MAX_DEVICES = 64;
+static void *g_scratch_ptr[MH_MAX_DEVICES];
+
+// Address of `scratch` on `device` (which must be the current device), looked up once.
+static hipError_t mh_static_scratch(int device, void **ptr) {
+  if (device < 0 || device >= MH_MAX_DEVICES) return hipErrorInvalidDevice;
+  if (!g_scratch_ptr[device]) {
+    void *p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    g_scratch_ptr[device] = p;
+  }
+  *ptr = g_scratch_ptr[device];
+  return hipSuccess;
+}
+
 int mh_arena_reserve(mace_hip_ctx *ctx, size_t bytes) {
   // headroom for the per-slice alignment
   const size_t need = ctx->arena_used + bytes + 16 * 256;
   if (need <= ctx->arena_bytes) return MACE_HIP_SUCCESS;
+  if (ctx->no_alloc)
+    return mh_fail(ctx, MACE_HIP_INVALID_ARGS,
+                   "this call needs %zu bytes of scratch; the allocation-free entry point has %zu",
+                   need, ctx->arena_bytes);
   if (ctx->fail_allocs > 0) {
     --ctx->fail_allocs;
     return mh_fail(ctx, MACE_HIP_OUT_OF_RESOURCES, "arena allocation of %zu bytes failed (mock)",
@@ -92,6 +117,17 @@ int mace_hip_ctx_create(int device, mace_hip_ctx **out) {
     delete ctx;
     return MACE_HIP_RUNTIME_ERROR;
   }
+  void *sp = nullptr;
+  if (mh_static_scratch(device, &sp) != hipSuccess) {
+    (void)hipGetLastError();
+    (void)hipStreamDestroy(ctx->own_stream);
+    (void)hipEventDestroy(ctx->ev_start);
+    (void)hipEventDestroy(ctx->ev_stop);
+    delete ctx;
+    return MACE_HIP_RUNTIME_ERROR;
+  }
+  ctx->static_scratch = (char *)sp;
+  ctx->big_lds_kernels.reserve(128);   // so that raising a kernel's LDS limit never reallocates
   ctx->stream = ctx->own_stream;
   ctx->cu_count = prop.multiProcessorCount;
   ctx->lds_bytes = (int)prop.sharedMemPerBlock;
@@ -531,6 +567,34 @@ int mace_hip_gemm_q8_u8_host(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_orde
                                          (const int32_t *)db, multiplier, right_shift,
                                          offset_after_shift, clamp_min, clamp_max));
   return st.back(out, dout, ob);
+}
+
+int mace_hip_gemm_q8_u8_noalloc(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order,
+                                const uint8_t *rhs, int rhs_order, uint8_t *out, int out_order,
+                                int64_t batch, int64_t rows, int64_t depth, int64_t cols,
+                                int lhs_batched, int rhs_batched, int32_t lhs_offset,
+                                int32_t rhs_offset, const int32_t *bias, int32_t multiplier,
+                                int right_shift, int32_t offset_after_shift, int clamp_min,
+                                int clamp_max) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_CHECK(ctx, ctx->arena_used == 0 && !ctx->no_alloc, "another call is in progress on this context");
+  // For the length of this call the arena is this GPU's static array: the repacked panels and
+  // the correction vectors go there, the kernels are the ones mace_hip_gemm_q8_u8 launches.
+  // Everything taken from it is written before it is read (the panel sums that a repack adds up
+  // with atomics are cleared by a kernel first), so what the previous call left does not matter.
+  char *const saved_arena = ctx->arena;
+  const size_t saved_bytes = ctx->arena_bytes;
+  ctx->arena = ctx->static_scratch;
+  ctx->arena_bytes = MACE_HIP_NOALLOC_SCRATCH_BYTES;
+  ctx->no_alloc = true;
+  Q8GemmEpilogue ep{bias, multiplier, right_shift, offset_after_shift, clamp_min, clamp_max};
+  const int rc = mh_q8_gemm(ctx, lhs, lhs_order, rhs, rhs_order, out, out_order, true, batch, rows,
+                            depth, cols, lhs_batched, rhs_batched, lhs_offset, rhs_offset, ep);
+  ctx->no_alloc = false;
+  ctx->arena = saved_arena;
+  ctx->arena_bytes = saved_bytes;
+  ctx->arena_used = 0;
+  return rc;
 }
 
 int mace_hip_conv1x1_q8_nhwc_host(mace_hip_ctx *ctx, const uint8_t *input,

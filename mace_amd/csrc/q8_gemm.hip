@@ -1753,7 +1753,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
 
   // operands registered as constant weights keep their panel and sums in the context
   auto find_weight = [&](const uint8_t *src, size_t bytes) -> mh_weight * {
-    if (depth == 0) return nullptr;
+    if (depth == 0 || ctx->no_alloc) return nullptr;   // the cache allocates on first use
     for (mh_weight &w : ctx->weights)
       if (w.ptr == (const void *)src && bytes <= w.bytes) return &w;
     return nullptr;

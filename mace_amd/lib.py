@@ -14,6 +14,7 @@ ROW_MAJOR, COL_MAJOR = 0, 1
 REQUANT_REF, REQUANT_NEON = 0, 1
 ACT_NOOP, ACT_RELU, ACT_RELUX = 0, 1, 2
 MASK_NO_SMALL, MASK_NO_XRES, MASK_NO_SPLITK = 1, 2, 4
+NOALLOC_SCRATCH_BYTES = 32 << 20
 
 _STATUS_NAMES = {0: "MACE_SUCCESS", 1: "MACE_INVALID_ARGS", 2: "MACE_OUT_OF_RESOURCES",
                  3: "MACE_UNSUPPORTED", 4: "MACE_RUNTIME_ERROR"}
@@ -84,6 +85,7 @@ SIGNATURES = {
     "mace_hip_gemv_q8_i32": (_int, _GEMV_Q8_I32),
     "mace_hip_gemm_q8_i32": (_int, _GEMM_Q8_I32),
     "mace_hip_gemm_q8_u8": (_int, _GEMM_Q8_U8),
+    "mace_hip_gemm_q8_u8_noalloc": (_int, _GEMM_Q8_U8),
     "mace_hip_conv1x1_q8_nhwc": (_int, _CONV_Q8),
     "mace_hip_gemm_f32_host": (_int, _GEMM_F32),
     "mace_hip_gemv_f32_host": (_int, _GEMV_F32),
