@@ -31,11 +31,32 @@ if ROOT not in sys.path:
 METRIC = "uint8 GEMM int8-TOPS + q8 Gemv HBM GB/s, % of MI355X roofline, 1 GPU"
 PEAK_INT8_TOPS = 5000.0      # MI355X dense int8 MFMA, published
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, published
-# Bytes that crossed the L2 <-> fabric boundary per launch of the dominant kernel, from rocprofv3
-# FETCH_SIZE / WRITE_SIZE runs of this benchmark scaled by the same counters' reading for a plain
-# 256 MiB copy (x2.0 and x1.0).  Keyed by M = N = K; a profiler run is needed to refresh them.
-GEMM_TRAFFIC_BYTES = {8192: 8.80e8}
-GEMV_TRAFFIC_BYTES = {1: 1.69e7, 8: 1.73e7}
+
+
+def measured_traffic(key):
+    """Bytes that crossed the L2 <-> fabric boundary per launch of a kernel, from the rocprofv3
+    FETCH_SIZE / WRITE_SIZE runs recorded in profiles/traffic.json (written next to the profile
+    summaries from the counters of this benchmark's own command, scaled by the same counters'
+    reading for a plain 256 MiB copy).  None when no counter run covers the kernel."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            entry = json.load(f).get(key)
+        return None if entry is None else entry["bytes_per_launch"]
+    except (OSError, ValueError, KeyError):
+        return None
+
+
+def load_probes():
+    """bench_probes/libbench_probes.so: measurement aids (not part of the product library)."""
+    lib = C.CDLL(os.path.join(ROOT, "bench_probes", "libbench_probes.so"))
+    lib.mace_probe_mfma_i8.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double)]
+    lib.mace_probe_hbm_read.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_int,
+                                        C.POINTER(C.c_double)]
+    lib.mace_probe_gemv_loop.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_void_p,
+                                         C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float,
+                                         C.c_float, C.c_int, C.c_void_p, C.c_int,
+                                         C.POINTER(C.c_double)]
+    return lib
 
 
 def log(*a):
@@ -169,7 +190,7 @@ def main():
                    "saturated_fraction": round(sat, 4), "device": arch, "cus": cus},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_INT8_TOPS,
                      "unit": "TOP/s", "frac": round(achieved / PEAK_INT8_TOPS, 4),
-                     "traffic": GEMM_TRAFFIC_BYTES.get(n), "traffic_unit": "B/launch",
+                     "traffic": measured_traffic("q8_gemm_%d" % n), "traffic_unit": "B/launch",
                      "kernel": "q8_gemm_dma_kernel<2,2,4,4,2,uint8_t,1,false,false,128>",
                      "kernel_ms_avg": round(k_avg, 4), "kernel_ms_min": round(min(kms), 4),
                      "kernel_ms_max": round(max(kms), 4),
@@ -240,15 +261,11 @@ def main():
         # registers): constant bytes, then random bytes.  The second figure is the power-limited
         # ceiling for an int8 GEMM on random operands on this board.
         try:
-            import ctypes
-            probe = ctypes.CDLL(os.path.join(os.path.dirname(os.path.abspath(__file__)),
-                                             "mace_amd", "libmace_probe.so"))
-            probe.mace_probe_mfma_i8.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int,
-                                                 ctypes.POINTER(ctypes.c_double)]
+            probe = load_probes()
             ceil = {}
             for name, rnd in (("constant_operands", 0), ("random_operands", 1)):
-                tops = ctypes.c_double(0.0)
-                rc = probe.mace_probe_mfma_i8(rnd, cus, 16384, ctypes.byref(tops))
+                tops = C.c_double(0.0)
+                rc = probe.mace_probe_mfma_i8(rnd, cus, 16384, C.byref(tops))
                 if rc != 0:
                     raise RuntimeError("probe returned %d" % rc)
                 ceil[name + "_TOPS"] = round(tops.value, 1)
@@ -280,6 +297,7 @@ def bench_gemv(ctx, mh, torch, args):
     H*W weights + B*W input + 4*H bias + B*H output."""
     H = W = 4096
     nbuf = 40                                    # 40 x 16 MiB = 640 MiB > 256 MiB last-level cache
+    probes = load_probes()
     g = torch.Generator(device="cuda").manual_seed(3)
     weights = torch.randint(0, 256, (nbuf, H, W), dtype=torch.uint8, device="cuda", generator=g)
     bias = torch.randint(-2 ** 15, 2 ** 15, (H,), dtype=torch.int32, device="cuda", generator=g)
@@ -304,6 +322,7 @@ def bench_gemv(ctx, mh, torch, args):
                mh.REQUANT_NEON, yptr)
 
         res = {"bytes_per_launch": nbytes}
+        stride = H * W
         for name, rotate in (("hbm", True), ("cache_resident", False)):
             for i in range(nbuf):
                 call(i if rotate else 0)
@@ -313,31 +332,61 @@ def bench_gemv(ctx, mh, torch, args):
                 call(i % nbuf if rotate else 0)
                 ks.append(ctx.last_kernel_ms())
             ctx.profile(False)
-            # back-to-back launches, no host sync in between: what a serving loop sees
-            reps = 10 * nbuf
-            ctx.sync()
-            ctx.timer_start()
-            for i in range(reps):
-                call(i % nbuf if rotate else 0)
-            loop_ms = ctx.timer_stop() / reps
+            # back-to-back calls with no host synchronisation in between, issued from C (a Python
+            # loop needs about as long per call on the host as the kernel takes): what a serving
+            # loop sees, and -- consecutive launches on one stream do not overlap -- the kernel's
+            # duration including its launch
+            us = C.c_double(0.0)
+            best = None
+            for _ in range(3):
+                rc = probes.mace_probe_gemv_loop(ctx.handle, wptr[0], stride, nbuf if rotate else 1,
+                                                 xptr, bptr, batch, H, W, 0.01, 0.02, 1.75, 128, yptr,
+                                                 10 * nbuf, C.byref(us))
+                if rc != 0:
+                    raise RuntimeError("gemv loop returned %d: %s" % (rc, ctx.last_error()))
+                best = us.value if best is None else min(best, us.value)
+            loop_ms = best * 1e-3
             k_avg = sum(ks) / len(ks)
-            gbs = nbytes / (k_avg * 1e-3) / 1e9
-            res[name] = {"kernel_us_avg": round(k_avg * 1e3, 3),
-                         "kernel_us_min": round(min(ks) * 1e3, 3),
-                         "GBps": round(gbs, 1), "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBS, 4),
-                         "back_to_back_us": round(loop_ms * 1e3, 3),
-                         "back_to_back_GBps": round(nbytes / (loop_ms * 1e-3) / 1e9, 1)}
-            log("gemv batch %d %s: kernel %.2f us -> %.0f GB/s (%.1f%% of HBM peak); "
-                "back-to-back %.2f us" % (batch, name, k_avg * 1e3, gbs,
-                                          100 * gbs / PEAK_HBM_GBS, loop_ms * 1e3))
+            gbs = nbytes / (loop_ms * 1e-3) / 1e9
+            res[name] = {"back_to_back_us": round(loop_ms * 1e3, 3),
+                         "back_to_back_GBps": round(gbs, 1),
+                         "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBS, 4),
+                         "event_pair_per_launch_us_avg": round(k_avg * 1e3, 3),
+                         "event_pair_per_launch_us_min": round(min(ks) * 1e3, 3)}
+            log("gemv batch %d %s: %.2f us per launch back to back -> %.0f GB/s (%.1f%% of HBM "
+                "peak); %.2f us between an event pair of its own"
+                % (batch, name, loop_ms * 1e3, gbs, 100 * gbs / PEAK_HBM_GBS, k_avg * 1e3))
         out["batch%d" % batch] = res
+    # The ceiling for one launch of this size, measured: a read-only kernel of the same launch shape
+    # (one wavefront per 4 KiB row, all loads requested up front, a byte stored per row), launched
+    # back to back over the same rotating matrices.
+    us = C.c_double(0.0)
+    best = None
+    for _ in range(3):
+        rc = probes.mace_probe_hbm_read(weights.data_ptr(), H * W, nbuf, H, W, 10 * nbuf, C.byref(us))
+        if rc != 0:
+            raise RuntimeError("read probe returned %d" % rc)
+        best = us.value if best is None else min(best, us.value)
+    pbytes = H * W + H
+    out["hbm_read_probe"] = {
+        "us_per_launch": round(best, 3), "bytes_per_launch": pbytes,
+        "GBps": round(pbytes / (best * 1e-6) / 1e9, 1),
+        "frac_of_hbm_peak": round(pbytes / (best * 1e-6) / 1e9 / PEAK_HBM_GBS, 4),
+        "what": "read-only kernel (row sums, one byte stored per row), 400 back-to-back launches "
+                "rotating over the same 640 MiB of weights, kernel arguments preloaded"}
     hb = out["batch1"]["hbm"]
     out["roofline"] = {"bound": "hbm", "achieved": hb["back_to_back_GBps"], "peak": PEAK_HBM_GBS,
                        "unit": "GB/s", "frac": round(hb["back_to_back_GBps"] / PEAK_HBM_GBS, 4),
-                       "traffic": GEMV_TRAFFIC_BYTES[1], "traffic_unit": "B/launch",
-                       "kernel": "q8_gemv_rows_kernel<1,1,16,uint8_t>",
+                       "frac_of_read_probe": round(best / hb["back_to_back_us"], 4),
+                       "batch8_over_batch1": round(out["batch8"]["hbm"]["back_to_back_us"] /
+                                                   hb["back_to_back_us"], 4),
+                       "traffic": measured_traffic("q8_gemv_4096x4096_b1"),
+                       "traffic_unit": "B/launch",
+                       "kernel": "q8_gemv_row_kernel<4,false,true,uint8_t>",
                        "timing": "400 back-to-back launches between two HIP events, rotating "
                                  "over 640 MiB of weights"}
+    log("read probe: %.2f us per launch -> %.0f GB/s; gemv batch 1 at %.1f%% of it"
+        % (best, pbytes / (best * 1e-6) / 1e9, 100 * best / hb["back_to_back_us"]))
     return out
 
 
@@ -596,10 +645,10 @@ def cpu_baseline(np, torch, A, B, out8, n, za, zb, zc, mult, shift, rows, rhs_or
     the host cores.  The same rows of the GPU result are compared with it."""
     from oracle import mace_oracle as orc
     try:
-        cores = len(os.sched_getaffinity(0))
+        host_cores = len(os.sched_getaffinity(0))
     except AttributeError:
-        cores = os.cpu_count() or 1
-    cores = max(1, min(cores, 16))
+        host_cores = os.cpu_count() or 1
+    cores = max(1, min(host_cores, 16))   # the share of the host one GPU's job gets
     rows = min(rows, n)
     a = A[:rows].cpu().numpy()
     b = B.cpu().numpy()
@@ -615,7 +664,8 @@ def cpu_baseline(np, torch, A, B, out8, n, za, zb, zc, mult, shift, rows, rhs_or
     if not exact:
         log("ERROR: GPU result differs from the CPU oracle")
         sys.exit(3)
-    return {"value": round(tops, 5), "unit": "TOPS", "cores": cores, "kind": "port",
+    return {"value": round(tops, 5), "unit": "TOPS", "cores": cores, "host_cores_visible": host_cores,
+            "kind": "port",
             "sample": "rows 0..%d of A times all of B (%d x %d x %d), oracle/mace_oracle.c "
                       "q8_gemm_u8, gcc -O2 -fopenmp, %.2f s" % (rows - 1, rows, n, n, dt),
             "gpu_rows_bit_exact": exact}

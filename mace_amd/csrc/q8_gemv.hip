@@ -284,6 +284,81 @@ __global__ __launch_bounds__(NWAVES * 64) void q8_gemv_rows_kernel(GemvParams p)
   }
 }
 
+// One right-hand vector per pass (batch 1, or every batch with weights of its own) and rows of at
+// most U KiB: the whole call is one dependent chain per wavefront -- request, wait, reduce, store
+// -- so what the kernel adds to the transfer is whatever sits in front of the requests and behind
+// the last byte.  One wavefront per weight row, 16 per workgroup.  In front: only the row address.
+// The first wavefronts request the vector (one 16-byte chunk per lane) before their weights, so
+// that it can be parked in LDS for everybody while the weights are still on their way (loads
+// return in order; the other way round the parking would wait for the weights); the bias comes
+// through the scalar cache at the same time.  Behind the last byte: 8 dot instructions per chunk,
+// one wave reduction of the combined term dot - zr sum(l) - zl sum(r), requantization, one store.
+// The arguments the requests depend on come first and as scalars: this file is compiled with kernel
+// argument preloading, so they are in registers when a wavefront starts instead of behind a load
+// from the argument segment (about 0.1 us of the 4.3 us a 16 MiB call takes).  BATCHED: more than
+// one pass (grid.y), each with its own vector and, if lhs_bs != 0, its own weights.
+__device__ inline uint4 keep16(const uint4 &v, bool ok) {
+  return uint4{ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u};
+}
+// WHOLE: the row is U whole 1 KiB steps, so no chunk index needs clamping or masking.
+template <int U, bool BATCHED, bool WHOLE, typename OutT>
+__global__ __launch_bounds__(1024) void q8_gemv_row_kernel(
+    const uint8_t *lhs, const uint8_t *rhs, int H, int W, const int32_t *bias_ptr, void *out,
+    float mult, int32_t out_zp /* 0 for the flavour that does not add it: x + 0.0f == x */,
+    int32_t lhs_zp, int32_t rhs_zp, int64_t lhs_bs, int64_t rhs_bs) {
+  __shared__ __align__(16) uint8_t sx[U * 1024];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int h = blockIdx.x * 16 + wave;
+  const int hc = min(h, H - 1);   // rows past the end re-read the last row; nothing is stored
+  const int b = BATCHED ? blockIdx.y : 0;
+  const int nchunk = W >> 4;
+  const uint8_t *xrow = rhs, *lrow = lhs + (int64_t)hc * W;
+  if constexpr (BATCHED) {
+    xrow += (int64_t)b * rhs_bs;
+    lrow += (int64_t)b * lhs_bs;
+  }
+  const uint4 ones = {0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u};
+
+  // chunks past the end of the vector re-read its last chunk; nobody reads their LDS slot
+  const uint4 xv = *(const uint4 *)(xrow + min(tid, nchunk - 1) * 16);
+  uint4 w[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+    w[u] = load_stream16(lrow + (WHOLE ? lane + 64 * u : min(lane + 64 * u, nchunk - 1)) * 16);
+  const uint32_t bias = bias_ptr ? (uint32_t)bias_ptr[hc] : 0u;   // uniform: a scalar load
+  if (tid < 64 * U) *(uint4 *)(sx + tid * 16) = xv;
+  __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0) only: the weights stay in flight
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+
+  const uint32_t zl = (uint32_t)lhs_zp, zr = (uint32_t)rhs_zp;
+  uint4 x[U];
+  uint32_t sr = 0;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int c = lane + 64 * u;
+    x[u] = *(const uint4 *)(sx + c * 16);
+    if constexpr (!WHOLE) x[u] = keep16(x[u], c < nchunk);
+    sr = dot16(x[u], ones, sr);
+  }
+  uint32_t t = 0u - sr * zl;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    // a chunk past the end of the row has a zero x: its dot product vanishes, its sum must too
+    const uint4 wv = WHOLE ? w[u] : keep16(w[u], lane + 64 * u < nchunk);
+    t = dot16(wv, x[u], t);
+    t -= dot16(wv, ones, 0u) * zr;
+  }
+  t = wave_sum(t);
+  if (lane == 0 && h < H) {
+    const int32_t ret = (int32_t)(t + (uint32_t)W * zl * zr + bias);
+    OutT *o = (OutT *)out + (int64_t)b * H + h;
+    if constexpr (sizeof(OutT) == 4) *o = (OutT)ret;
+    else *o = (OutT)mh_requant_float(ret, mult, out_zp, 1);
+  }
+}
+
 // Shared weights against several right-hand vectors (batch >= 2): the per-lane dot products of
 // the kernel above cost NB LDS reads and NB dot instructions per weight chunk and become the
 // bound.  Here the batch rides on the matrix cores instead: one workgroup owns 16 weight rows,
@@ -384,9 +459,13 @@ __global__ __launch_bounds__(256) void q8_gemv_mfma_kernel(GemvParams p) {
 // (row pitch = a multiple of 1 KiB plus 16 bytes: the 16 rows of a fragment read fall into
 // 16 distinct bank groups).  Needs (16 + NB) rows of LDS: the host falls back to the direct
 // kernel when that does not fit.
-template <typename OutT>
-__global__ __launch_bounds__(256) void q8_gemv_mfma_lds_kernel(GemvParams p, int pitch) {
-  constexpr int NBMAX = 15, ONES_COL = 15;
+// NW wavefronts per workgroup: each moves 16 / NW weight rows and multiplies 1 / NW of the width.
+// Sixteen (rows of 1 KiB and more) keep a wavefront's share of the tail behind the last byte
+// short: 4 k steps on two accumulators instead of 16 on one.  The bias of the epilogue's rows is
+// requested before anything else.
+template <int NW, typename OutT>
+__global__ __launch_bounds__(NW * 64) void q8_gemv_mfma_lds_kernel(GemvParams p, int pitch) {
+  constexpr int NBMAX = 15, ONES_COL = 15, NT = NW * 64;
   extern __shared__ __align__(16) uint8_t lds_rows[];   // [16 + nb][pitch]
   __shared__ int32_t s_acc[16][17];
   __shared__ int32_t s_sx[16];
@@ -399,27 +478,30 @@ __global__ __launch_bounds__(256) void q8_gemv_mfma_lds_kernel(GemvParams p, int
   const int nchunk = p.W >> 4;
   const int nj = (nchunk + 63) >> 6;            // 1 KiB transfers per row
   const int nstep = (nchunk + 3) >> 2;
-  const int per_wave = (nstep + 3) >> 2;
+  const int per_wave = (nstep + NW - 1) / NW;
   const int ks0 = wave * per_wave, ks1 = min(nstep, ks0 + per_wave);
 
-  // rows 4 wave .. 4 wave + 3 of the weights, vectors wave, wave + 4, ...; chunks past the end
-  // of a row re-read its last chunk (never used: masked below)
-  for (int rr = 0; rr < 4; ++rr) {
-    const int row = 4 * wave + rr;
+  uint32_t bias_v = 0;
+  if (p.bias && tid < 16 * nb) bias_v = (uint32_t)p.bias[min(h0 + (tid & 15), p.H - 1)];
+
+  // weight rows wave, wave + NW, ..., vectors wave, wave + NW, ...; chunks past the end of a row
+  // re-read its last chunk (never used: masked below)
+  for (int row = wave; row < 16; row += NW) {
     const uint8_t *src = p.lhs + (int64_t)min(h0 + row, p.H - 1) * p.W;
     uint8_t *dst = lds_rows + row * pitch;
     for (int j = 0; j < nj; ++j)
       mh_dma_16B_stream(src + (int64_t)min(64 * j + lane, nchunk - 1) * 16, dst + j * 1024);
   }
-  for (int b = wave; b < nb; b += 4) {
+  for (int b = wave; b < nb; b += NW) {
     const uint8_t *src = p.rhs + (int64_t)(b0 + b) * p.rhs_bs;
     uint8_t *dst = lds_rows + (16 + b) * pitch;
     for (int j = 0; j < nj; ++j)
       mh_dma_16B(src + (int64_t)min(64 * j + lane, nchunk - 1) * 16, dst + j * 1024);
   }
-  for (int i = tid; i < 16 * 17; i += 256) (&s_acc[0][0])[i] = 0;
+  for (int i = tid; i < 16 * 17; i += NT) (&s_acc[0][0])[i] = 0;
   if (tid < 16) s_sx[tid] = 0;
-  __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0), lgkmcnt(0): own transfers and LDS stores done
+  // vmcnt(0), lgkmcnt(0): own transfers and LDS stores done (and the bias has arrived)
+  __builtin_amdgcn_s_waitcnt(0x0070);
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
 
@@ -431,25 +513,39 @@ __global__ __launch_bounds__(256) void q8_gemv_mfma_lds_kernel(GemvParams p, int
   const uint8_t *arow = lds_rows + r * pitch + q * 16;
   const uint8_t *xrow = lds_rows + (16 + (is_x ? r : 0)) * pitch + q * 16;
 
-  gv4i acc = zero;
+  // Four k steps at a time: all fragment reads first, then the multiplications on two
+  // accumulators (a chain of dependent MFMAs would wait for each result in turn).
+  gv4i acc0 = zero, acc1 = zero;
   int sx = 0;
-  for (int ks = ks0; ks < ks1; ++ks) {
-    const bool valid = 4 * ks + q < nchunk;
-    const gv4i av = valid ? (*(const gv4i *)(arow + ks * 64) ^ flip) : zero;
-    gv4i xv = other;
-    if (is_x) xv = *(const gv4i *)(xrow + ks * 64) ^ flip;
-    if (!valid) xv = zero;
-    if (is_x) {
-      sx = __builtin_amdgcn_sdot4(xv.x, 0x01010101, sx, false);
-      sx = __builtin_amdgcn_sdot4(xv.y, 0x01010101, sx, false);
-      sx = __builtin_amdgcn_sdot4(xv.z, 0x01010101, sx, false);
-      sx = __builtin_amdgcn_sdot4(xv.w, 0x01010101, sx, false);
-    }
-    acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, xv, acc, 0, 0, 0);
-  }
+  for (int kb = ks0; kb < ks1; kb += 4) {
+    gv4i av[4], xv[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) atomicAdd(&s_acc[4 * q + i][r], acc[i]);
-  if (is_x) atomicAdd(&s_sx[r], sx);
+    for (int u = 0; u < 4; ++u) {
+      const int ks = min(kb + u, ks1 - 1);   // past the wavefront's share: re-read, masked below
+      av[u] = *(const gv4i *)(arow + ks * 64);
+      xv[u] = *(const gv4i *)(xrow + ks * 64);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const bool valid = kb + u < ks1 && 4 * (kb + u) + q < nchunk;
+      const gv4i a = valid ? (av[u] ^ flip) : zero;
+      gv4i x = is_x ? (xv[u] ^ flip) : other;
+      if (!valid) x = zero;
+      if (is_x) {
+        sx = __builtin_amdgcn_sdot4(x.x, 0x01010101, sx, false);
+        sx = __builtin_amdgcn_sdot4(x.y, 0x01010101, sx, false);
+        sx = __builtin_amdgcn_sdot4(x.z, 0x01010101, sx, false);
+        sx = __builtin_amdgcn_sdot4(x.w, 0x01010101, sx, false);
+      }
+      if (u & 1) acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, x, acc1, 0, 0, 0);
+      else acc0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, x, acc0, 0, 0, 0);
+    }
+  }
+  if (ks0 < ks1) {   // uniform over the wavefront
+#pragma unroll
+    for (int i = 0; i < 4; ++i) atomicAdd(&s_acc[4 * q + i][r], acc0[i] + acc1[i]);
+    if (is_x) atomicAdd(&s_sx[r], sx);
+  }
   __syncthreads();
 
   if (tid < 16 * nb) {
@@ -458,11 +554,129 @@ __global__ __launch_bounds__(256) void q8_gemv_mfma_lds_kernel(GemvParams p, int
     if (h < p.H) {
       const uint32_t zl = (uint32_t)p.lhs_zp - 128u, zr = (uint32_t)p.rhs_zp - 128u;
       const uint32_t ret = (uint32_t)s_acc[row][b] - zr * (uint32_t)s_acc[row][ONES_COL] -
-                           zl * (uint32_t)s_sx[b] + (uint32_t)p.W * zl * zr +
-                           (p.bias ? (uint32_t)p.bias[h] : 0u);
+                           zl * (uint32_t)s_sx[b] + (uint32_t)p.W * zl * zr + bias_v;
       OutT *o = (OutT *)p.out + (int64_t)(b0 + b) * p.H + h;
       if constexpr (sizeof(OutT) == 4) *o = (OutT)(int32_t)ret;
       else *o = (OutT)mh_requant_float((int32_t)ret, p.mult, p.out_zp, p.neon_mode);
+    }
+  }
+}
+
+// The same product for rows of at most 4 KiB with nothing shared between the wavefronts until the
+// very end.  Wavefront w of 16 owns the k slice [64 SPW w, 64 SPW (w + 1)) of all 16 weight rows and
+// of the right-hand vectors: it moves exactly that into an LDS area of its own (one transfer
+// instruction covers 64 / (4 SPW) rows x 64 SPW bytes), waits for its own transfers only, and
+// multiplies while the other wavefronts' bytes are still on their way; the only barrier is the
+// one in front of the epilogue, after the 16 partial 16 x 16 results have met in LDS.  Inside a
+// wavefront's area 16-byte chunk c of row r sits in slot c ^ f(r) (chosen by which global chunk a
+// lane fetches), f such that the 16 rows a fragment read touches fall into 16 distinct bank groups.
+// Scalar leading arguments: preloaded into registers (see q8_gemv_row_kernel).
+template <int SPW, typename OutT>
+__global__ __launch_bounds__(1024) void q8_gemv_mfma_slice_kernel(
+    const uint8_t *lhs, const uint8_t *rhs, int H, int W, const int32_t *bias_ptr, void *out,
+    float mult, int32_t out_zp, int32_t lhs_zp, int32_t rhs_zp, int batch, int64_t rhs_bs) {
+  constexpr int NBMAX = 15, ONES_COL = 15;
+  constexpr int CH = 4 * SPW;        // 16-byte chunks per row of a slice
+  constexpr int RPI = 64 / CH;       // rows per transfer instruction
+  constexpr int NI = 16 / RPI;       // instructions for the 16 weight rows (and for 16 vectors)
+  constexpr int SH = SPW == 4 ? 0 : (SPW == 2 ? 1 : 2);   // f(r) = (r >> SH) & (CH - 1)
+  static_assert(SPW == 1 || SPW == 2 || SPW == 4, "slice width");
+  __shared__ __align__(16) uint8_t area[16][2][NI * 1024];   // [wavefront][weights, vectors]
+  __shared__ int32_t s_acc[16][17];
+  __shared__ int32_t s_sx[16];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, q = lane >> 4;
+  const int h0 = blockIdx.x * 16;
+  const int b0 = blockIdx.y * NBMAX;
+  const int nb = min(NBMAX, batch - b0);
+  const int nchunk = W >> 4;
+  const int c0 = wave * CH;          // first chunk of this wavefront's slice
+  const bool active = c0 < nchunk;   // uniform
+
+  // the epilogue's bias first: loads return in order, so it is back before the transfers are
+  uint32_t bias_v = 0;
+  if (bias_ptr && tid < 16 * nb) bias_v = (uint32_t)bias_ptr[min(h0 + (tid & 15), H - 1)];
+  if (active) {
+    const int rho = lane / CH, sig = lane % CH;
+    // weights first: their requests are the ones that go all the way to memory
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int row = j * RPI + rho;
+      const int c = min(c0 + (sig ^ ((row >> SH) & (CH - 1))), nchunk - 1);
+      mh_dma_16B_stream(lhs + (int64_t)min(h0 + row, H - 1) * W + c * 16, &area[wave][0][j * 1024]);
+    }
+    // Every workgroup reads the same vectors at the same moment; each starts with a different
+    // one so that they do not all queue up at the same cache lines.
+    const int nxj = (nb + RPI - 1) / RPI;
+    for (int jj = 0; jj < nxj; ++jj) {
+      int j = jj + (int)(blockIdx.x % (unsigned)nxj);
+      if (j >= nxj) j -= nxj;
+      const int vec = j * RPI + rho;
+      const int c = min(c0 + (sig ^ ((vec >> SH) & (CH - 1))), nchunk - 1);
+      mh_dma_16B(rhs + (int64_t)(b0 + min(vec, nb - 1)) * rhs_bs + c * 16, &area[wave][1][j * 1024]);
+    }
+  }
+  for (int i = tid; i < 16 * 17; i += 1024) (&s_acc[0][0])[i] = 0;
+  if (tid < 16) s_sx[tid] = 0;
+  // the zeroed sums are visible; lgkmcnt(0) only, so that the transfers stay in flight
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+
+  const bool is_x = r < nb;
+  const gv4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+  const gv4i zero = {0, 0, 0, 0};
+  const gv4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+  const gv4i other = r == ONES_COL ? ones : zero;
+  if (active) {
+    // row r of the area: transfer r / RPI, row r % RPI inside it, chunk c in slot c ^ f(r)
+    const int rbase = (r / RPI) * 1024 + (r % RPI) * (CH * 16);
+    const int fr = (r >> SH) & (CH - 1);
+    gv4i av[SPW], xv[SPW];
+    __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0), lgkmcnt(0): this wavefront's transfers landed
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int u = 0; u < SPW; ++u) {
+      const int slot = (4 * u + q) ^ fr;
+      av[u] = *(const gv4i *)(&area[wave][0][rbase + slot * 16]);
+      xv[u] = zero;
+      if (is_x) xv[u] = *(const gv4i *)(&area[wave][1][rbase + slot * 16]);
+    }
+    gv4i acc0 = zero, acc1 = zero;
+    int sx = 0;
+#pragma unroll
+    for (int u = 0; u < SPW; ++u) {
+      const bool valid = c0 + 4 * u + q < nchunk;
+      const gv4i a = valid ? (av[u] ^ flip) : zero;
+      gv4i x = is_x ? (xv[u] ^ flip) : other;
+      if (!valid) x = zero;
+      if (is_x) {
+        sx = __builtin_amdgcn_sdot4(x.x, 0x01010101, sx, false);
+        sx = __builtin_amdgcn_sdot4(x.y, 0x01010101, sx, false);
+        sx = __builtin_amdgcn_sdot4(x.z, 0x01010101, sx, false);
+        sx = __builtin_amdgcn_sdot4(x.w, 0x01010101, sx, false);
+      }
+      if (u & 1) acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, x, acc1, 0, 0, 0);
+      else acc0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, x, acc0, 0, 0, 0);
+    }
+    // result register i of lane l: row 4 (l / 16) + i, column l % 16
+#pragma unroll
+    for (int i = 0; i < 4; ++i) atomicAdd(&s_acc[4 * q + i][r], acc0[i] + acc1[i]);
+    if (is_x) atomicAdd(&s_sx[r], sx);
+  }
+  __syncthreads();
+
+  if (tid < 16 * nb) {
+    const int row = tid & 15, b = tid >> 4;
+    const int h = h0 + row;
+    if (h < H) {
+      const uint32_t zl = (uint32_t)lhs_zp - 128u, zr = (uint32_t)rhs_zp - 128u;
+      const uint32_t ret = (uint32_t)s_acc[row][b] - zr * (uint32_t)s_acc[row][ONES_COL] -
+                           zl * (uint32_t)s_sx[b] + (uint32_t)W * zl * zr + bias_v;
+      OutT *o = (OutT *)out + (int64_t)(b0 + b) * H + h;
+      if constexpr (sizeof(OutT) == 4) *o = (OutT)(int32_t)ret;
+      else *o = (OutT)mh_requant_float((int32_t)ret, mult, out_zp, 1);
     }
   }
 }
@@ -474,12 +688,10 @@ int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
   // a batched lhs gives every batch its own weights: one batch row per pass
   int nb = lhs_batched ? 1 : (p.batch >= 8 ? 8 : (p.batch >= 4 ? 4 : (p.batch >= 2 ? 2 : 1)));
   dim3 block(256);
-  // Two to four vectors against long rows stay on the row-block kernel (one pass, the weights
-  // streamed once: 5.6 us against 7.2 us at 4096 x 4096, batch 2); the matrix-core kernel's
-  // load-everything-then-multiply structure only pays from five vectors on, or on short rows.
-  const bool few = !lhs_batched && p.batch >= 2 && p.batch <= 4 && p.W >= 2048 &&
-                   (size_t)4 * p.W <= 64 * 1024;
-  if (few) nb = p.batch == 2 ? 2 : 4;
+  // Two vectors against long rows stay on the row-block kernel (one pass, the weights streamed
+  // once: 5.6 us against 5.9 us at 4096 x 4096); from three on the matrix-core kernels win.
+  const bool few = !lhs_batched && p.batch == 2 && p.W >= 2048 && (size_t)2 * p.W <= 64 * 1024;
+  if (few) nb = 2;
   // shared weights against more vectors: the batch goes through the matrix cores
   if (vec && !lhs_batched && !few && p.W >= 64 && p.batch >= 2 && p.rhs_bs % 16 == 0) {
     dim3 grid((unsigned)((p.H + 15) / 16), (unsigned)((p.batch + 14) / 15));
@@ -488,8 +700,25 @@ int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
     const int pitch = ((p.W / 16 + 63) / 64) * 1024 + 16;
     const size_t lds = (size_t)(16 + nb_pass) * pitch;
     const size_t lds_max = (ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536) - 2048;
-    if (lds <= lds_max) {
-      auto k = q8_gemv_mfma_lds_kernel<OutT>;
+    if (p.W <= 4096 && lds_max >= 140 * 1024) {
+      // rows of at most 4 KiB: every wavefront on a k slice of its own
+      const int spw = p.W <= 1024 ? 1 : (p.W <= 2048 ? 2 : 4);
+      MH_PROF_BEGIN(ctx);
+#define MH_SLICE_LAUNCH(S_)                                                                       \
+  hipLaunchKernelGGL((q8_gemv_mfma_slice_kernel<S_, OutT>), grid, dim3(1024), 0, ctx->stream,      \
+                     p.lhs, p.rhs, p.H, p.W, p.bias, p.out, p.mult, p.neon_mode ? p.out_zp : 0,   \
+                     p.lhs_zp, p.rhs_zp, p.batch, p.rhs_bs)
+      if (spw == 1) MH_SLICE_LAUNCH(1);
+      else if (spw == 2) MH_SLICE_LAUNCH(2);
+      else MH_SLICE_LAUNCH(4);
+#undef MH_SLICE_LAUNCH
+    } else if (lds <= lds_max && p.W >= 1024) {
+      auto k = q8_gemv_mfma_lds_kernel<16, OutT>;
+      if (lds > 48 * 1024) MH_HIP(ctx, mh_allow_big_lds(ctx, (const void *)k, lds));
+      MH_PROF_BEGIN(ctx);
+      hipLaunchKernelGGL(k, grid, dim3(1024), lds, ctx->stream, p, pitch);
+    } else if (lds <= lds_max) {
+      auto k = q8_gemv_mfma_lds_kernel<4, OutT>;
       if (lds > 48 * 1024) MH_HIP(ctx, mh_allow_big_lds(ctx, (const void *)k, lds));
       MH_PROF_BEGIN(ctx);
       hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, pitch);
@@ -497,6 +726,38 @@ int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
       MH_PROF_BEGIN(ctx);
       hipLaunchKernelGGL(q8_gemv_mfma_kernel<OutT>, grid, block, 0, ctx->stream, p);
     }
+    MH_PROF_END(ctx);
+    MH_HIP(ctx, hipGetLastError());
+    return MACE_HIP_SUCCESS;
+  }
+  // one vector per pass against rows of at most 8 KiB: the lean one-row-per-wavefront kernel
+  if (vec && nb == 1 && p.W >= 16 && p.W <= 8192 && p.batch <= 65535) {
+    dim3 grid((unsigned)((p.H + 15) / 16), (unsigned)p.batch);
+    const int u = (p.W + 1023) / 1024;
+    MH_PROF_BEGIN(ctx);
+#define MH_ROW_LAUNCH(U_, B_)                                                                      \
+  do {                                                                                             \
+    if (p.W == 1024 * U_)                                                                          \
+      hipLaunchKernelGGL((q8_gemv_row_kernel<U_, B_, true, OutT>), grid, dim3(1024), 0,            \
+                         ctx->stream, p.lhs, p.rhs, p.H, p.W, p.bias, p.out, p.mult,               \
+                         p.neon_mode ? p.out_zp : 0, p.lhs_zp, p.rhs_zp, p.lhs_bs, p.rhs_bs);      \
+    else                                                                                           \
+      hipLaunchKernelGGL((q8_gemv_row_kernel<U_, B_, false, OutT>), grid, dim3(1024), 0,           \
+                         ctx->stream, p.lhs, p.rhs, p.H, p.W, p.bias, p.out, p.mult,               \
+                         p.neon_mode ? p.out_zp : 0, p.lhs_zp, p.rhs_zp, p.lhs_bs, p.rhs_bs);      \
+  } while (0)
+    if (p.batch == 1) {
+      if (u <= 1) MH_ROW_LAUNCH(1, false);
+      else if (u <= 2) MH_ROW_LAUNCH(2, false);
+      else if (u <= 4) MH_ROW_LAUNCH(4, false);
+      else MH_ROW_LAUNCH(8, false);
+    } else {
+      if (u <= 1) MH_ROW_LAUNCH(1, true);
+      else if (u <= 2) MH_ROW_LAUNCH(2, true);
+      else if (u <= 4) MH_ROW_LAUNCH(4, true);
+      else MH_ROW_LAUNCH(8, true);
+    }
+#undef MH_ROW_LAUNCH
     MH_PROF_END(ctx);
     MH_HIP(ctx, hipGetLastError());
     return MACE_HIP_SUCCESS;
