@@ -191,6 +191,13 @@ int mace_hip_gemm_f32_transpose(mace_hip_ctx *ctx, const float *lhs, const float
                                 int64_t rhs_rows, int64_t rhs_cols, int transpose_lhs,
                                 int transpose_rhs, int transpose_out, int lhs_batched,
                                 int rhs_batched, float *out);
+/* The Gemm branch of MatMulOp<RT_CPU, float>::Run (mace/ops/matmul.cc:170-211): the
+ * transpose-form Gemm with a RowMajor result, then, when bias is given (length = result
+ * columns), c[i * cols + w] += bias[w] -- here added as the result is stored. */
+int mace_hip_matmul_f32(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
+                        const float *bias /* or NULL */, int64_t batch, int64_t lhs_rows,
+                        int64_t lhs_cols, int64_t rhs_rows, int64_t rhs_cols, int transpose_lhs,
+                        int transpose_rhs, int lhs_batched, int rhs_batched, float *out);
 /* delegator::Gemv::Compute for float (mace/ops/delegator/gemv.h:35-44;
  * mace/ops/ref/gemv.cc:46-81): out[b,h] = bias[h] + sum_w lhs[b?,h,w] * rhs[b?,w]. */
 int mace_hip_gemv_f32(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
@@ -203,6 +210,19 @@ int mace_hip_conv1x1_f32_nchw(mace_hip_ctx *ctx, const float *input, const float
                               const float *bias /* or NULL */, int64_t n, int64_t cin,
                               int64_t hw, int64_t cout, int activation, float max_limit,
                               float *out);
+/* delegator::Conv2d::Compute for float as Conv2dOp<RT_CPU, float>::Run calls it
+ * (mace/ops/conv_2d.cc:88-173), NCHW input, OIHW filter, followed by the BiasAdd and Activation
+ * delegators.  The case the op hands to Conv2dK1x1 (1x1 filter, stride 1, dilation 1, :101-105)
+ * runs on the GPU, including its padded form (pad_h / pad_w = total padding rows / columns:
+ * the input is copied into a zero-padded tensor, pad / 2 on top and left, and the result has
+ * (in_h + pad_h) x (in_w + pad_w) pixels, mace/ops/arm/base/conv_2d_1x1.cc:37-60).  Any other
+ * geometry returns MACE_UNSUPPORTED and writes nothing: the caller keeps its general
+ * convolution (ref::Conv2d) for it. */
+int mace_hip_conv2d_f32_nchw(mace_hip_ctx *ctx, const float *input, const float *filter,
+                             const float *bias /* or NULL */, int64_t n, int64_t cin,
+                             int64_t in_h, int64_t in_w, int64_t cout, int64_t k_h, int64_t k_w,
+                             int stride_h, int stride_w, int dilation_h, int dilation_w,
+                             int pad_h, int pad_w, int activation, float max_limit, float *out);
 
 /* ---- uint8 Gemv (FullyConnected) ------------------------------------------------------- */
 
@@ -315,6 +335,16 @@ int mace_hip_conv1x1_f32_nchw_host(mace_hip_ctx *ctx, const float *input,
                                    const float *filter, const float *bias, int64_t n,
                                    int64_t cin, int64_t hw, int64_t cout, int activation,
                                    float max_limit, float *out);
+int mace_hip_matmul_f32_host(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
+                             const float *bias, int64_t batch, int64_t lhs_rows, int64_t lhs_cols,
+                             int64_t rhs_rows, int64_t rhs_cols, int transpose_lhs,
+                             int transpose_rhs, int lhs_batched, int rhs_batched, float *out);
+int mace_hip_conv2d_f32_nchw_host(mace_hip_ctx *ctx, const float *input, const float *filter,
+                                  const float *bias, int64_t n, int64_t cin, int64_t in_h,
+                                  int64_t in_w, int64_t cout, int64_t k_h, int64_t k_w,
+                                  int stride_h, int stride_w, int dilation_h, int dilation_w,
+                                  int pad_h, int pad_w, int activation, float max_limit,
+                                  float *out);
 int mace_hip_gemv_q8_u8_host(mace_hip_ctx *ctx, const uint8_t *lhs, const uint8_t *rhs,
                              const int32_t *bias, int64_t batch, int64_t height,
                              int64_t width, int lhs_batched, int rhs_batched, int32_t lhs_zp,

@@ -19,7 +19,9 @@
 #ifndef MACE_HIP_DELEGATOR_H_
 #define MACE_HIP_DELEGATOR_H_
 
+#include <algorithm>
 #include <cstdint>
+#include <cstdlib>
 #include <functional>
 #include <cmath>
 #include <memory>
@@ -194,6 +196,8 @@ class OpDelegatorRegistry {
 #define MACE_HIP_REGISTER_DELEGATOR(registry, class_name, param_name, key) \
   (registry)->Register(key, ::mace_hip::OpDelegator::DefaultCreator<class_name, param_name>)
 
+enum Padding { VALID = 0, SAME = 1, FULL = 2 };   // mace/ops/common/conv_pool_2d_util.h
+
 // ---- abstract delegators ---------------------------------------------------------------------------
 namespace delegator {
 
@@ -233,14 +237,31 @@ class Gemv : public OpDelegator {              // mace/ops/delegator/gemv.h:27-4
                              Tensor *output) = 0;
 };
 
-struct Conv2dParam : public DelegatorParam {   // mace/ops/delegator/conv_2d.h:37-58 (subset)
-  Conv2dParam() = default;
+struct Conv2dParam : public DelegatorParam {   // mace/ops/delegator/conv_2d.h:46-58
+  explicit Conv2dParam(const std::vector<int> &strides = {1, 1},
+                       const std::vector<int> &dilations = {1, 1},
+                       const std::vector<int> &paddings = {},
+                       const Padding padding_type = SAME)
+      : strides_(strides), dilations_(dilations), paddings_(paddings),
+        padding_type_(padding_type) {}
+  const std::vector<int> strides_;
+  const std::vector<int> dilations_;
+  const std::vector<int> paddings_;   // empty: derive from padding_type_
+  const Padding padding_type_;
 };
 class Conv2d : public OpDelegator {            // mace/ops/delegator/conv_2d.h:60-82
  public:
-  explicit Conv2d(const Conv2dParam &param) : OpDelegator(param) {}
+  explicit Conv2d(const Conv2dParam &param)
+      : OpDelegator(param), strides_(param.strides_), dilations_(param.dilations_),
+        paddings_(param.paddings_), padding_type_(param.padding_type_) {}
   virtual MaceStatus Compute(const OpContext *context, const Tensor *input,
                              const Tensor *filter, Tensor *output) = 0;
+
+ protected:
+  const std::vector<int> strides_;
+  const std::vector<int> dilations_;
+  const std::vector<int> paddings_;
+  const Padding padding_type_;
 };
 
 }  // namespace delegator
@@ -334,27 +355,71 @@ class Gemv<int32_t> : public delegator::Gemv {   // replaces ref::q8::Gemv<int32
   }
 };
 
-// Replaces arm::Conv2dK1x1<float> (mace/ops/arm/base/conv_2d_1x1.cc:27-72): NCHW input
-// {n, cin, h, w}, OIHW filter {cout, cin, 1, 1}, output {n, cout, h, w}; the op adds bias and
-// activation afterwards (see Conv2dK1x1Op below), so the delegator itself computes the Gemm.
-template <typename T> class Conv2dK1x1;
+// The float Conv2d delegator, NCHW input {n, cin, h, w}, OIHW filter {cout, cin, kh, kw}, output
+// {n, cout, oh, ow}.  The output shape and padding come from the delegator's parameters exactly
+// as in ref::Conv2d / arm::Conv2dBase (mace/ops/ref/conv_2d.cc:44-66,
+// mace/ops/arm/base/conv_2d.cc:27-50): from the padding type, or from explicit paddings with the
+// FLOOR rule.  The geometry Conv2dOp hands to Conv2dK1x1 -- 1x1 filter, stride 1, dilation 1
+// (mace/ops/conv_2d.cc:101-105) -- runs on the GPU, a padded input included (the reference copies
+// it into a zero-padded tensor first, mace/ops/arm/base/conv_2d_1x1.cc:37-60).  Every other
+// geometry returns MACE_UNSUPPORTED without touching the output: in a MACE tree that branch is
+// `return ref::Conv2d<float>::Compute(...)`.
+// ComputeFused additionally applies the op's BiasAdd and Activation (mace/ops/conv_2d.cc:171-173)
+// as the result is stored; Compute (the virtual of the interface) is ComputeFused without them.
+template <typename T> class Conv2d;
 template <>
-class Conv2dK1x1<float> : public delegator::Conv2d {
+class Conv2d<float> : public delegator::Conv2d {
  public:
-  explicit Conv2dK1x1(const delegator::Conv2dParam &param) : delegator::Conv2d(param) {}
+  explicit Conv2d(const delegator::Conv2dParam &param) : delegator::Conv2d(param) {}
   MaceStatus Compute(const OpContext *context, const Tensor *input, const Tensor *filter,
                      Tensor *output) override {
-    if (input->dim_size() != 4 || filter->dim_size() != 4 || filter->dim(2) != 1 ||
-        filter->dim(3) != 1 || filter->dim(1) != input->dim(1))
-      return MaceStatus::MACE_INVALID_ARGS;
-    const index_t n = input->dim(0), cin = input->dim(1), hw = input->dim(2) * input->dim(3);
-    const index_t cout = filter->dim(0);
-    MaceStatus st = output->Resize({n, cout, input->dim(2), input->dim(3)});
-    if (st != MaceStatus::MACE_SUCCESS) return st;
-    auto fn = output->on_device() ? mace_hip_conv1x1_f32_nchw : mace_hip_conv1x1_f32_nchw_host;
-    return ToStatus(fn(context->hip(), input->data<float>(), filter->data<float>(), nullptr, n,
-                       cin, hw, cout, MACE_HIP_ACT_NOOP, 0.f, output->mutable_data<float>()));
+    return ComputeFused(context, input, filter, nullptr, NOOP, 0.f, output);
   }
+  MaceStatus ComputeFused(const OpContext *context, const Tensor *input, const Tensor *filter,
+                          const Tensor *bias, ActivationType activation, float max_limit,
+                          Tensor *output) {
+    if (input->dim_size() != 4 || filter->dim_size() != 4 || filter->dim(1) != input->dim(1))
+      return MaceStatus::MACE_INVALID_ARGS;
+    if (strides_.size() != 2 || dilations_.size() != 2) return MaceStatus::MACE_INVALID_ARGS;
+    if (bias && (bias->dim_size() != 1 || bias->dim(0) != filter->dim(0)))
+      return MaceStatus::MACE_INVALID_ARGS;
+    int64_t out_h = 0, out_w = 0;
+    int pads[2] = {0, 0};
+    if (paddings_.empty()) {
+      MaceStatus st = ToStatus(mace_hip_calc_padding_and_output_size(
+          input->dim(2), input->dim(3), filter->dim(2), filter->dim(3), dilations_[0],
+          dilations_[1], strides_[0], strides_[1], padding_type_, &out_h, &out_w, &pads[0],
+          &pads[1]));
+      if (st != MaceStatus::MACE_SUCCESS) return st;
+    } else {
+      if (paddings_.size() != 2 || strides_[0] <= 0 || strides_[1] <= 0)
+        return MaceStatus::MACE_INVALID_ARGS;
+      pads[0] = paddings_[0];
+      pads[1] = paddings_[1];
+      const index_t kh = (filter->dim(2) - 1) * dilations_[0] + 1;
+      const index_t kw = (filter->dim(3) - 1) * dilations_[1] + 1;
+      out_h = static_cast<int64_t>(std::floor(1.0 * (input->dim(2) + pads[0] - kh) / strides_[0]) + 1);
+      out_w = static_cast<int64_t>(std::floor(1.0 * (input->dim(3) + pads[1] - kw) / strides_[1]) + 1);
+    }
+    const bool k1x1 = filter->dim(2) == 1 && filter->dim(3) == 1 && strides_[0] == 1 &&
+                      strides_[1] == 1 && dilations_[0] == 1 && dilations_[1] == 1;
+    if (!k1x1) return MaceStatus::MACE_UNSUPPORTED;   // stays with ref::Conv2d
+    MaceStatus st = output->Resize({input->dim(0), filter->dim(0), out_h, out_w});
+    if (st != MaceStatus::MACE_SUCCESS) return st;
+    auto fn = output->on_device() ? mace_hip_conv2d_f32_nchw : mace_hip_conv2d_f32_nchw_host;
+    return ToStatus(fn(context->hip(), input->data<float>(), filter->data<float>(),
+                       bias ? bias->data<float>() : nullptr, input->dim(0), input->dim(1),
+                       input->dim(2), input->dim(3), filter->dim(0), 1, 1, 1, 1, 1, 1, pads[0],
+                       pads[1], activation, max_limit, output->mutable_data<float>()));
+  }
+};
+// The same delegator under the name the NEON build registers for the K1x1 tag
+// (mace/ops/arm/base/conv_2d_1x1.cc:74-88).
+template <typename T> class Conv2dK1x1;
+template <>
+class Conv2dK1x1<float> : public Conv2d<float> {
+ public:
+  explicit Conv2dK1x1(const delegator::Conv2dParam &param) : Conv2d<float>(param) {}
 };
 
 // mace/ops/registry/op_delegators_registry.cc:87-143 registers ref:: and arm:: delegators; this
@@ -372,6 +437,11 @@ inline MaceStatus RegisterAllHipDelegators(OpDelegatorRegistry *registry) {
   if (st != MaceStatus::MACE_SUCCESS) return st;
   st = MACE_HIP_REGISTER_DELEGATOR(registry, Gemv<int32_t>, DelegatorParam,
                                    MACE_HIP_DELEGATOR_KEY(Gemv, RT_CPU, int32_t, kCpuImplType));
+  if (st != MaceStatus::MACE_SUCCESS) return st;
+  // The general key is the one Conv2dOp asks for on a host without NEON -- the only kind an
+  // MI355X has (mace/ops/conv_2d.cc:88-91); the K1x1 tag serves a NEON build's request.
+  st = MACE_HIP_REGISTER_DELEGATOR(registry, Conv2d<float>, delegator::Conv2dParam,
+                                   MACE_HIP_DELEGATOR_KEY(Conv2d, RT_CPU, float, kCpuImplType));
   if (st != MaceStatus::MACE_SUCCESS) return st;
   return MACE_HIP_REGISTER_DELEGATOR(
       registry, Conv2dK1x1<float>, delegator::Conv2dParam,
@@ -423,7 +493,8 @@ inline MaceStatus MatMulInferShape(const Tensor *A, const Tensor *B, bool transp
 }
 
 // MatMulOp<RT_CPU, float>::Run (mace/ops/matmul.cc:110-215).  The optional bias of the Gemm
-// branch (:195-211) is a host loop in the reference and stays one here (host tensors only).
+// branch (:195-211), a loop over the finished result in the reference, is added by the GEMM
+// kernel as it stores the result (mace_hip_matmul_f32): one launch, host or device tensors.
 class MatMulOpFloat {
  public:
   MatMulOpFloat(OpDelegatorRegistry *registry, bool transpose_a, bool transpose_b)
@@ -446,18 +517,16 @@ class MatMulOpFloat {
     if (s.cols == 1 && !transpose_a_)
       return gemv_->Compute(context, lhs, rhs, bias, s.batch, s.rows, s.depth, s.lhs_batched,
                             s.rhs_batched, C);
-    st = gemm_->Compute(context, lhs, rhs, s.batch, s.lhs_rows, s.lhs_cols, s.rhs_rows,
-                        s.rhs_cols, transpose_a_, transpose_b_, false, s.lhs_batched,
-                        s.rhs_batched, C);
-    if (st == MaceStatus::MACE_SUCCESS && bias != nullptr) {
-      if (bias->dim_size() != 1 || bias->dim(0) != s.cols || C->on_device())
-        return MaceStatus::MACE_INVALID_ARGS;
-      const float *b = bias->data<float>();
-      float *c = C->mutable_data<float>();
-      for (index_t i = 0; i < s.batch * s.rows; ++i)
-        for (index_t w = 0; w < s.cols; ++w) c[i * s.cols + w] += b[w];
-    }
-    return st;
+    if (bias == nullptr)
+      return gemm_->Compute(context, lhs, rhs, s.batch, s.lhs_rows, s.lhs_cols, s.rhs_rows,
+                            s.rhs_cols, transpose_a_, transpose_b_, false, s.lhs_batched,
+                            s.rhs_batched, C);
+    // "bias' dim should be <= 2." (:196-197), checked before anything is written
+    if (bias->dim_size() != 1 || bias->dim(0) != s.cols) return MaceStatus::MACE_INVALID_ARGS;
+    auto fn = C->on_device() ? mace_hip_matmul_f32 : mace_hip_matmul_f32_host;
+    return ToStatus(fn(context->hip(), lhs->data<float>(), rhs->data<float>(), bias->data<float>(),
+                       s.batch, s.lhs_rows, s.lhs_cols, s.rhs_rows, s.rhs_cols, transpose_a_,
+                       transpose_b_, s.lhs_batched, s.rhs_batched, C->mutable_data<float>()));
   }
 
  private:
@@ -476,17 +545,35 @@ class MatMulOpFloat {
 // (arm/base/gemm.cc:560-576).  Counterpart: an operand that is a constant weight AND lives in device
 // memory is registered with the context once per op instance; its repacked panel and row sums are
 // then kept across Run() calls.  A weight whose buffer moves is registered afresh.
+// The registration ends with the op (or when the weight moves): the cache is keyed by address,
+// and once the weight's buffer has been freed the allocator may hand the same address to an
+// activation tensor, which must not find a stale panel.  The op must be destroyed before its
+// library context is.
 class WeightRegistration {
  public:
+  WeightRegistration() = default;
+  WeightRegistration(const WeightRegistration &) = delete;
+  WeightRegistration &operator=(const WeightRegistration &) = delete;
+  ~WeightRegistration() { Release(); }
   void Note(OpContext *context, const Tensor *t, size_t bytes) {
     if (!t->is_weight() || !t->on_device()) return;
     const void *ptr = t->data<uint8_t>();
-    if (ptr == registered_) return;
-    if (mace_hip_weight_register(context->hip(), ptr, bytes) == MACE_HIP_SUCCESS) registered_ = ptr;
+    if (ptr == registered_ && context->hip() == ctx_) return;
+    Release();
+    if (mace_hip_weight_register(context->hip(), ptr, bytes) == MACE_HIP_SUCCESS) {
+      registered_ = ptr;
+      ctx_ = context->hip();
+    }
+  }
+  void Release() {
+    if (registered_ != nullptr) (void)mace_hip_weight_unregister(ctx_, registered_);
+    registered_ = nullptr;
+    ctx_ = nullptr;
   }
 
  private:
   const void *registered_ = nullptr;
+  mace_hip_ctx *ctx_ = nullptr;
 };
 
 class MatMulOpQuant {
@@ -560,7 +647,10 @@ class FullyConnectedOp {
   std::unique_ptr<delegator::Gemv> gemv_;
 };
 
-enum Padding { VALID = 0, SAME = 1, FULL = 2 };   // mace/ops/common/conv_pool_2d_util.h
+using ::mace_hip::Padding;
+using ::mace_hip::VALID;
+using ::mace_hip::SAME;
+using ::mace_hip::FULL;
 
 // Conv2dOp<RT_CPU, uint8_t>::Run (mace/ops/conv_2d.cc:201-318): NHWC input, OHWI filter, NHWC
 // output, dilation 1.  The output shape comes from the padding type (CalcPaddingAndOutputSize)
@@ -634,6 +724,326 @@ class Conv2dK1x1OpQuant {
 
  private:
   Conv2dOpQuant op_;
+};
+
+// Conv2dOp<RT_CPU, float>::Run (mace/ops/conv_2d.cc:82-173): picks the delegator key on the first
+// run -- the general key, or on a NEON build the tag of the filter geometry (only the K1x1 tag
+// is mirrored) -- creates the delegator through the registry, runs it, then BiasAdd and
+// Activation (ref/bias_add.cc:74-100 NCHW, ref/activation.cc:61-75 NOOP / RELU / RELUX).  With the
+// GPU delegator the last two are applied as the result is stored; with any other delegator they
+// are the reference's host loops.
+class Conv2dOpFloat {
+ public:
+  Conv2dOpFloat(OpDelegatorRegistry *registry, std::vector<int> strides = {1, 1},
+                Padding padding_type = SAME, std::vector<int> paddings = {},
+                std::vector<int> dilations = {1, 1}, ActivationType activation = NOOP,
+                float max_limit = 0.f, ImplType impl = kCpuImplType)
+      : registry_(registry), strides_(std::move(strides)), padding_type_(padding_type),
+        paddings_(std::move(paddings)), dilations_(std::move(dilations)), activation_(activation),
+        max_limit_(max_limit), impl_(impl) {}
+  MaceStatus Run(OpContext *context, const Tensor *input, const Tensor *filter,
+                 const Tensor *bias, Tensor *output) {
+    if (input->dim_size() != 4 || filter->dim_size() != 4 || strides_.size() != 2 ||
+        dilations_.size() != 2)
+      return MaceStatus::MACE_INVALID_ARGS;
+    if (!conv_) {
+      DelegatorInfo tag = MACE_HIP_DELEGATOR_KEY(Conv2d, RT_CPU, float, impl_);
+      if (impl_ == NEON && filter->dim(2) == 1 && filter->dim(3) == 1 && strides_[0] == 1 &&
+          strides_[1] == 1 && dilations_[0] == 1 && dilations_[1] == 1)
+        tag = MACE_HIP_DELEGATOR_KEY_EX(Conv2d, RT_CPU, float, impl_, K1x1);
+      DelegatorCreator creator = registry_->GetCreator(tag);
+      if (!creator) return MaceStatus::MACE_RUNTIME_ERROR;   // LOG(FATAL) in the reference
+      delegator::Conv2dParam param(strides_, dilations_, paddings_, padding_type_);
+      conv_.reset(static_cast<delegator::Conv2d *>(creator(param).release()));
+    }
+    if (auto *fused = dynamic_cast<hip::Conv2d<float> *>(conv_.get()))
+      return fused->ComputeFused(context, input, filter, bias, activation_, max_limit_, output);
+    MaceStatus st = conv_->Compute(context, input, filter, output);
+    if (st != MaceStatus::MACE_SUCCESS) return st;
+    if (output->on_device()) return MaceStatus::MACE_UNSUPPORTED;   // host loops below
+    float *o = output->mutable_data<float>();
+    const index_t n = output->dim(0), c = output->dim(1), hw = output->dim(2) * output->dim(3);
+    for (index_t i = 0; i < n * c; ++i)
+      for (index_t p = 0; p < hw; ++p) {
+        float v = o[i * hw + p];
+        if (bias) v += bias->data<float>()[i % c];
+        if (activation_ == RELU) v = std::max(0.f, v);
+        if (activation_ == RELUX) v = std::max(0.f, std::min(max_limit_, v));
+        o[i * hw + p] = v;
+      }
+    return st;
+  }
+
+ private:
+  OpDelegatorRegistry *registry_;
+  std::vector<int> strides_;
+  Padding padding_type_;
+  std::vector<int> paddings_, dilations_;
+  ActivationType activation_;
+  float max_limit_;
+  ImplType impl_;
+  std::unique_ptr<delegator::Conv2d> conv_;
+};
+
+// arm::Conv2dK3x3Winograd<float>::Compute (mace/ops/arm/base/conv_2d_3x3_winograd.cc:31-236): a
+// caller of delegator::Gemm.  3x3 filter, stride 1, NCHW.  Output tiles of 2x2 (6x6 when the
+// input is larger than 16x16, :43-46); the input is zero-padded so that whole tiles cover the
+// (padded) output, every (tile + 2)^2 patch is transformed (B^T d B), the filter likewise
+// (G g G^T), and the products over the input channels are ONE batched Gemm per image --
+// batch = (tile + 2)^2, lhs = transformed filter [area][cout][cin], rhs = transformed input
+// [area][cin][tiles], both batched, row-major (:191-204) -- followed by the output transform
+// (A^T m A).  The transforms are host loops written from the standard matrices of the
+// algorithm (the reference has NEON code for the same matrices); the Gemm is the delegator's.
+class Conv2dK3x3WinogradOp {
+ public:
+  Conv2dK3x3WinogradOp(OpDelegatorRegistry *registry, Padding padding_type = SAME,
+                       std::vector<int> paddings = {})
+      : padding_type_(padding_type), paddings_(std::move(paddings)) {
+    auto gc = registry->GetCreator(MACE_HIP_DELEGATOR_KEY(Gemm, RT_CPU, float, kCpuImplType));
+    if (gc) gemm_.reset(static_cast<delegator::Gemm *>(gc(delegator::GemmParam()).release()));
+  }
+  MaceStatus Run(OpContext *context, const Tensor *input, const Tensor *filter, Tensor *output) {
+    if (!gemm_) return MaceStatus::MACE_RUNTIME_ERROR;
+    if (input->dim_size() != 4 || filter->dim_size() != 4 || filter->dim(2) != 3 ||
+        filter->dim(3) != 3 || filter->dim(1) != input->dim(1) || input->on_device())
+      return MaceStatus::MACE_INVALID_ARGS;
+    const index_t batch = input->dim(0), cin = input->dim(1), in_h = input->dim(2),
+                  in_w = input->dim(3), cout = filter->dim(0);
+    const int t = (in_h > 16 && in_w > 16) ? 6 : 2;   // output tile
+    const int a = t + 2, area = a * a;                 // input tile and its area
+    int64_t out_h = 0, out_w = 0;
+    int pads[2] = {0, 0};
+    if (paddings_.empty()) {
+      MaceStatus st = ToStatus(mace_hip_calc_padding_and_output_size(
+          in_h, in_w, 3, 3, 1, 1, 1, 1, padding_type_, &out_h, &out_w, &pads[0], &pads[1]));
+      if (st != MaceStatus::MACE_SUCCESS) return st;
+    } else {
+      if (paddings_.size() != 2) return MaceStatus::MACE_INVALID_ARGS;
+      pads[0] = paddings_[0]; pads[1] = paddings_[1];
+      out_h = in_h + pads[0] - 2; out_w = in_w + pads[1] - 2;
+    }
+    if (out_h <= 0 || out_w <= 0) return MaceStatus::MACE_INVALID_ARGS;
+    MaceStatus st = output->Resize({batch, cout, out_h, out_w});
+    if (st != MaceStatus::MACE_SUCCESS) return st;
+    // arm/base/conv_2d.cc:97-119: output rounded up to whole tiles, input padded to match
+    const index_t poh = (out_h + t - 1) / t * t, pow_ = (out_w + t - 1) / t * t;
+    const index_t pih = std::max<index_t>(in_h + pads[0], poh + 2);
+    const index_t piw = std::max<index_t>(in_w + pads[1], pow_ + 2);
+    const int top = pads[0] >> 1, left = pads[1] >> 1;
+    const index_t th = poh / t, tw = pow_ / t, tiles = th * tw;
+    const float *BT = t == 2 ? kBT4 : kBT8, *G = t == 2 ? kG4 : kG8, *AT = t == 2 ? kAT4 : kAT8;
+
+    // filter [cout][cin][3][3] -> U [area][cout][cin] = G g G^T
+    std::vector<float> U((size_t)area * cout * cin), V((size_t)area * cin * tiles),
+        M((size_t)area * cout * tiles), tmp(a * 3), d(area), w(area);
+    const float *f = filter->data<float>();
+    for (index_t oc = 0; oc < cout; ++oc)
+      for (index_t ic = 0; ic < cin; ++ic) {
+        const float *g = f + (oc * cin + ic) * 9;
+        for (int i = 0; i < a; ++i)
+          for (int j = 0; j < 3; ++j)
+            tmp[i * 3 + j] = G[i * 3] * g[j] + G[i * 3 + 1] * g[3 + j] + G[i * 3 + 2] * g[6 + j];
+        for (int i = 0; i < a; ++i)
+          for (int j = 0; j < a; ++j)
+            U[((size_t)(i * a + j) * cout + oc) * cin + ic] =
+                tmp[i * 3] * G[j * 3] + tmp[i * 3 + 1] * G[j * 3 + 1] + tmp[i * 3 + 2] * G[j * 3 + 2];
+      }
+    Tensor Ut(U.data(), DT_FLOAT, {area, cout, cin}), Vt(V.data(), DT_FLOAT, {area, cin, tiles}),
+        Mt(M.data(), DT_FLOAT, {area, cout, tiles});
+    const float *x = input->data<float>();
+    float *y = output->mutable_data<float>();
+    for (index_t b = 0; b < batch; ++b) {
+      // input patches -> V [area][cin][tiles] = B^T d B (zero outside the image)
+      for (index_t ic = 0; ic < cin; ++ic)
+        for (index_t ty = 0; ty < th; ++ty)
+          for (index_t tx = 0; tx < tw; ++tx) {
+            for (int i = 0; i < a; ++i)
+              for (int j = 0; j < a; ++j) {
+                const index_t py = ty * t + i, px = tx * t + j;   // in the padded image
+                const index_t iy = py - top, ix = px - left;
+                const bool in = py < pih && px < piw && iy >= 0 && iy < in_h && ix >= 0 && ix < in_w;
+                d[i * a + j] = in ? x[((b * cin + ic) * in_h + iy) * in_w + ix] : 0.f;
+              }
+            Sandwich(BT, d.data(), a, a, w.data());
+            for (int k = 0; k < area; ++k)
+              V[((size_t)k * cin + ic) * tiles + ty * tw + tx] = w[k];
+          }
+      // conv_2d_3x3_winograd.cc:191-204
+      st = gemm_->Compute(context, &Ut, &Vt, area, cout, cin, cin, tiles, false, false, false, true,
+                          true, &Mt);
+      if (st != MaceStatus::MACE_SUCCESS) return st;
+      // M [area][cout][tiles] -> output tiles = A^T m A, cropped to the output
+      for (index_t oc = 0; oc < cout; ++oc)
+        for (index_t ty = 0; ty < th; ++ty)
+          for (index_t tx = 0; tx < tw; ++tx) {
+            for (int k = 0; k < area; ++k) d[k] = M[((size_t)k * cout + oc) * tiles + ty * tw + tx];
+            Sandwich(AT, d.data(), t, a, w.data());
+            for (int i = 0; i < t; ++i)
+              for (int j = 0; j < t; ++j) {
+                const index_t oy = ty * t + i, ox = tx * t + j;
+                if (oy < out_h && ox < out_w)
+                  y[((b * cout + oc) * out_h + oy) * out_w + ox] = w[i * t + j];
+              }
+          }
+    }
+    return MaceStatus::MACE_SUCCESS;
+  }
+
+ private:
+  // out (r x r) = L (r x a) * m (a x a) * L^T
+  static void Sandwich(const float *L, const float *m, int r, int a, float *out) {
+    float tmp[64];
+    for (int i = 0; i < r; ++i)
+      for (int j = 0; j < a; ++j) {
+        float s = 0.f;
+        for (int k = 0; k < a; ++k) s += L[i * a + k] * m[k * a + j];
+        tmp[i * a + j] = s;
+      }
+    for (int i = 0; i < r; ++i)
+      for (int j = 0; j < r; ++j) {
+        float s = 0.f;
+        for (int k = 0; k < a; ++k) s += tmp[i * a + k] * L[j * a + k];
+        out[i * r + j] = s;
+      }
+  }
+  // F(2x2, 3x3) and F(6x6, 3x3): interpolation points 0, +-1 (and +-2, +-1/2), infinity
+  static constexpr float kBT4[16] = {1, 0, -1, 0, 0, 1, 1, 0, 0, -1, 1, 0, 0, 1, 0, -1};
+  static constexpr float kG4[12] = {1, 0, 0, .5f, .5f, .5f, .5f, -.5f, .5f, 0, 0, 1};
+  static constexpr float kAT4[8] = {1, 1, 1, 0, 0, 1, -1, -1};
+  static constexpr float kBT8[64] = {
+      1, 0, -5.25f, 0, 5.25f, 0, -1, 0,       0, 1, 1, -4.25f, -4.25f, 1, 1, 0,
+      0, -1, 1, 4.25f, -4.25f, -1, 1, 0,      0, .5f, .25f, -2.5f, -1.25f, 2, 1, 0,
+      0, -.5f, .25f, 2.5f, -1.25f, -2, 1, 0,  0, 2, 4, -2.5f, -5, .5f, 1, 0,
+      0, -2, 4, 2.5f, -5, -.5f, 1, 0,         0, -1, 0, 5.25f, 0, -5.25f, 0, 1};
+  static constexpr float kG8[24] = {
+      1, 0, 0,  -2.f / 9, -2.f / 9, -2.f / 9,  -2.f / 9, 2.f / 9, -2.f / 9,
+      1.f / 90, 1.f / 45, 2.f / 45,  1.f / 90, -1.f / 45, 2.f / 45,
+      32.f / 45, 16.f / 45, 8.f / 45,  32.f / 45, -16.f / 45, 8.f / 45,  0, 0, 1};
+  static constexpr float kAT8[48] = {
+      1, 1, 1, 1, 1, 1, 1, 0,               0, 1, -1, 2, -2, .5f, -.5f, 0,
+      0, 1, 1, 4, 4, .25f, .25f, 0,         0, 1, -1, 8, -8, .125f, -.125f, 0,
+      0, 1, 1, 16, 16, .0625f, .0625f, 0,   0, 1, -1, 32, -32, .03125f, -.03125f, 1};
+  Padding padding_type_;
+  std::vector<int> paddings_;
+  std::unique_ptr<delegator::Gemm> gemm_;
+};
+
+// DynamicLSTMOp<RT_CPU, float>::Run (mace/ops/dynamic_lstm.cc:160-372), a caller of
+// delegator::Gemv: per batch and output frame, affine a (weights_a [a_out][input_dim +
+// prev_out_dim] against the input frame appended with the delayed output, :296-310), the LSTM
+// nonlinearity with peephole parameters (mace/ops/common/lstm.h:29-84), the cell scaled
+// (:83-104), affine b (weights_b [out_dim][cell_dim], :328-337), and the delayed output / cell
+// ring buffers and caches (:339-366).  Both affines are batch-1 Gemv calls with nothing batched
+// and an optional bias; everything else is the reference's host code restated.
+struct DynamicLSTMArgs {
+  int prev_out_delay = 0, prev_cell_delay = 0, prev_out_offset = 0, prev_out_dim = 0,
+      prev_cell_dim = 0, subsample_factor = 1;
+  float scale = 1.0f;
+  std::vector<index_t> forward_indexes, cell_cache_indexes, out_cache_indexes;
+};
+class DynamicLSTMOp {
+ public:
+  DynamicLSTMOp(OpDelegatorRegistry *registry, DynamicLSTMArgs args) : a_(std::move(args)) {
+    auto vc = registry->GetCreator(MACE_HIP_DELEGATOR_KEY(Gemv, RT_CPU, float, kCpuImplType));
+    if (vc) gemv_.reset(static_cast<delegator::Gemv *>(vc(DelegatorParam()).release()));
+  }
+  MaceStatus Run(OpContext *context, const Tensor *input, const Tensor *prev_out,
+                 const Tensor *prev_cell, const Tensor *weights_a, const Tensor *lstm_params,
+                 const Tensor *weights_b, const Tensor *bias_a, const Tensor *bias_b,
+                 Tensor *output, Tensor *out_cache, Tensor *cell_cache) {
+    if (!gemv_) return MaceStatus::MACE_RUNTIME_ERROR;
+    const index_t rank = input->dim_size();
+    // Validate (:81-118)
+    if (rank < 2 || a_.prev_cell_delay >= 0 || a_.prev_out_delay >= 0 || a_.subsample_factor <= 0 ||
+        a_.prev_cell_delay % a_.subsample_factor != 0 || a_.prev_out_delay % a_.subsample_factor != 0 ||
+        a_.prev_out_dim <= 0 || a_.prev_cell_dim <= 0)
+      return MaceStatus::MACE_INVALID_ARGS;
+    const index_t chunk = input->dim(rank - 2), input_dim = input->dim(rank - 1);
+    for (index_t fi : a_.forward_indexes)
+      if (fi < 0 || fi >= chunk) return MaceStatus::MACE_INVALID_ARGS;
+    const index_t batch = std::accumulate(input->shape().begin(), input->shape().end() - 2,
+                                          index_t(1), std::multiplies<index_t>());
+    const index_t a_in = input_dim + a_.prev_out_dim, a_out = weights_a->dim(0);
+    if (a_in != weights_a->dim(1)) return MaceStatus::MACE_INVALID_ARGS;
+    const index_t lstm_in = a_out + a_.prev_cell_dim, cell_dim = lstm_in / 5;
+    if (lstm_in != cell_dim * 5 || lstm_params->dim(0) != 3 || lstm_params->dim(1) != cell_dim ||
+        cell_dim != a_.prev_cell_dim)
+      return MaceStatus::MACE_INVALID_ARGS;
+    const index_t out_dim = weights_b->dim(0);
+    if (weights_b->dim(1) != cell_dim || a_.prev_out_offset + a_.prev_out_dim > out_dim)
+      return MaceStatus::MACE_INVALID_ARGS;
+    const index_t out_buf_chunk = std::abs(a_.prev_out_delay / a_.subsample_factor);
+    const index_t cell_buf_chunk = std::abs(a_.prev_cell_delay / a_.subsample_factor);
+    const index_t out_chunk = (index_t)a_.forward_indexes.size();
+
+    std::vector<index_t> shape = input->shape();
+    shape[rank - 1] = out_dim;   // (the reference keeps the input's chunk here, :264-266)
+    MaceStatus st = output->Resize(shape);
+    shape[rank - 1] = a_.prev_out_dim; shape[rank - 2] = out_buf_chunk;
+    if (st == MaceStatus::MACE_SUCCESS) st = out_cache->Resize(shape);
+    shape[rank - 1] = a_.prev_cell_dim; shape[rank - 2] = cell_buf_chunk;
+    if (st == MaceStatus::MACE_SUCCESS) st = cell_cache->Resize(shape);
+    if (st != MaceStatus::MACE_SUCCESS) return st;
+
+    std::vector<float> out_buf(out_buf_chunk * a_.prev_out_dim), cell_buf(cell_buf_chunk * cell_dim),
+        va_in(a_in), va_out(a_out), vb_in(cell_dim), vb_out(out_dim);
+    Tensor a_in_t(va_in.data(), DT_FLOAT, {1, a_in}), a_out_t(va_out.data(), DT_FLOAT, {1, a_out}),
+        b_in_t(vb_in.data(), DT_FLOAT, {1, cell_dim}), b_out_t(vb_out.data(), DT_FLOAT, {1, out_dim});
+    const float *x = input->data<float>(), *params = lstm_params->data<float>();
+    float *y = output->mutable_data<float>();
+    const bool unit_scale = std::abs(a_.scale - 1.f) < 1e-6;
+    for (index_t b = 0; b < batch; ++b) {
+      std::copy_n(prev_out->data<float>() + b * out_buf_chunk * a_.prev_out_dim, out_buf.size(),
+                  out_buf.begin());
+      std::copy_n(prev_cell->data<float>() + b * cell_buf_chunk * cell_dim, cell_buf.size(),
+                  cell_buf.begin());
+      for (index_t i = 0; i < out_chunk; ++i) {
+        std::copy_n(x + (b * chunk + a_.forward_indexes[i]) * input_dim, input_dim, va_in.begin());
+        std::copy_n(out_buf.data() + i % out_buf_chunk * a_.prev_out_dim, a_.prev_out_dim,
+                    va_in.begin() + input_dim);
+        st = gemv_->Compute(context, weights_a, &a_in_t, bias_a, 1, a_out, a_in, false, false, &a_out_t);
+        if (st != MaceStatus::MACE_SUCCESS) return st;
+        float *cell = cell_buf.data() + i % cell_buf_chunk * cell_dim;
+        for (index_t c = 0; c < cell_dim; ++c) {   // common/lstm.h:64-81, embed_scales = false
+          const float i_part = va_out[c], f_part = va_out[c + cell_dim],
+                      c_part = va_out[c + 2 * cell_dim], o_part = va_out[c + 3 * cell_dim];
+          const float c_prev = cell[c];
+          const float i_t = Sigmoid(i_part + params[c] * c_prev);
+          const float f_t = Sigmoid(f_part + params[c + cell_dim] * c_prev);
+          const float c_t = f_t * 1.0f * c_prev + i_t * 1.0f * std::tanh(c_part);
+          const float o_t = Sigmoid(o_part + params[c + 2 * cell_dim] * c_t);
+          cell[c] = c_t;
+          vb_in[c] = o_t * 1.0f * std::tanh(c_t);
+        }
+        if (!unit_scale)
+          for (index_t c = 0; c < cell_dim; ++c) cell[c] *= a_.scale;
+        st = gemv_->Compute(context, weights_b, &b_in_t, bias_b, 1, out_dim, cell_dim, false, false, &b_out_t);
+        if (st != MaceStatus::MACE_SUCCESS) return st;
+        std::copy_n(vb_out.begin(), out_dim, y + (b * out_chunk + i) * out_dim);
+        float *cur_out = out_buf.data() + i % out_buf_chunk * a_.prev_out_dim;
+        for (index_t k = 0; k < a_.prev_out_dim; ++k)
+          cur_out[k] = unit_scale ? vb_out[a_.prev_out_offset + k] : vb_out[a_.prev_out_offset + k] * a_.scale;
+        for (size_t k = 0; k < a_.out_cache_indexes.size(); ++k)
+          if (i == a_.out_cache_indexes[k])
+            std::copy_n(cur_out, a_.prev_out_dim,
+                        out_cache->mutable_data<float>() + (b * out_buf_chunk + k) * a_.prev_out_dim);
+        for (size_t k = 0; k < a_.cell_cache_indexes.size(); ++k)
+          if (i == a_.cell_cache_indexes[k])
+            std::copy_n(cell, cell_dim,
+                        cell_cache->mutable_data<float>() + (b * cell_buf_chunk + k) * cell_dim);
+      }
+    }
+    return MaceStatus::MACE_SUCCESS;
+  }
+
+ private:
+  static float Sigmoid(float in) {   // mace/utils/math.h:63-70 ScalarSigmoid
+    if (in > 0) return 1 / (1 + std::exp(-in));
+    const float x = std::exp(in);
+    return x / (x + 1.f);
+  }
+  DynamicLSTMArgs a_;
+  std::unique_ptr<delegator::Gemv> gemv_;
 };
 
 // QuantizeOp<RT_CPU, uint8_t> (mace/ops/arm/q8/quantize.cc:31-72): float -> uint8.  An output

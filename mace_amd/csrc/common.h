@@ -445,6 +445,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
 
 struct F32Epilogue {
   const float *bias_row;    // added per result row (NCHW channel), or nullptr
+  const float *bias_col;    // added per result column (MatMul bias), or nullptr
   int act;
   float limit;
 };

@@ -464,6 +464,64 @@ int mace_hip_conv1x1_f32_nchw_host(mace_hip_ctx *ctx, const float *input,
   return st.back(out, dout, ob);
 }
 
+int mace_hip_matmul_f32_host(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
+                             const float *bias, int64_t batch, int64_t lhs_rows, int64_t lhs_cols,
+                             int64_t rhs_rows, int64_t rhs_cols, int transpose_lhs,
+                             int transpose_rhs, int lhs_batched, int rhs_batched, float *out) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_CHECK(ctx, nonneg(batch, lhs_rows, lhs_cols, 0) && nonneg(rhs_rows, rhs_cols, 0, 0),
+           "negative dimension");
+  const int64_t rows = transpose_lhs ? lhs_cols : lhs_rows;
+  const int64_t cols = transpose_rhs ? rhs_rows : rhs_cols;
+  const size_t lb = sizeof(float) * (lhs_batched ? batch : 1) * lhs_rows * lhs_cols;
+  const size_t rb = sizeof(float) * (rhs_batched ? batch : 1) * rhs_rows * rhs_cols;
+  const size_t bb = bias ? sizeof(float) * cols : 0;
+  const size_t ob = sizeof(float) * batch * rows * cols;
+  MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, lb + rb + bb + ob));
+  Stage st(ctx);
+  void *dl, *dr, *db, *dout;
+  MH_RETURN_IF_ERROR(st.in(lhs, lb, &dl));
+  MH_RETURN_IF_ERROR(st.in(rhs, rb, &dr));
+  MH_RETURN_IF_ERROR(st.in(bias, bb, &db));
+  MH_RETURN_IF_ERROR(st.out(ob, &dout));
+  MH_RETURN_IF_ERROR(mace_hip_matmul_f32(ctx, (const float *)dl, (const float *)dr,
+                                         (const float *)db, batch, lhs_rows, lhs_cols, rhs_rows,
+                                         rhs_cols, transpose_lhs, transpose_rhs, lhs_batched,
+                                         rhs_batched, (float *)dout));
+  return st.back(out, dout, ob);
+}
+
+int mace_hip_conv2d_f32_nchw_host(mace_hip_ctx *ctx, const float *input, const float *filter,
+                                  const float *bias, int64_t n, int64_t cin, int64_t in_h,
+                                  int64_t in_w, int64_t cout, int64_t k_h, int64_t k_w,
+                                  int stride_h, int stride_w, int dilation_h, int dilation_w,
+                                  int pad_h, int pad_w, int activation, float max_limit,
+                                  float *out) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_CHECK(ctx, nonneg(n, cin, in_h, in_w) && nonneg(cout, k_h, k_w, 0) && pad_h >= 0 && pad_w >= 0,
+           "negative dimension");
+  if (k_h != 1 || k_w != 1 || stride_h != 1 || stride_w != 1 || dilation_h != 1 || dilation_w != 1)
+    return mh_fail(ctx, MACE_HIP_UNSUPPORTED,
+                   "only 1x1 filters at stride 1, dilation 1 run on the GPU");
+  const int64_t ohw = (in_h + pad_h) * (in_w + pad_w);
+  const size_t ib = sizeof(float) * n * cin * in_h * in_w;
+  const size_t fb = sizeof(float) * cout * cin;
+  const size_t bb = bias ? sizeof(float) * cout : 0;
+  const size_t ob = sizeof(float) * n * cout * ohw;
+  MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, ib + fb + bb + ob + sizeof(float) * n * cin * ohw + 4096));
+  Stage st(ctx);
+  void *di, *df, *db, *dout;
+  MH_RETURN_IF_ERROR(st.in(input, ib, &di));
+  MH_RETURN_IF_ERROR(st.in(filter, fb, &df));
+  MH_RETURN_IF_ERROR(st.in(bias, bb, &db));
+  MH_RETURN_IF_ERROR(st.out(ob, &dout));
+  MH_RETURN_IF_ERROR(mace_hip_conv2d_f32_nchw(ctx, (const float *)di, (const float *)df,
+                                              (const float *)db, n, cin, in_h, in_w, cout, k_h, k_w,
+                                              stride_h, stride_w, dilation_h, dilation_w, pad_h,
+                                              pad_w, activation, max_limit, (float *)dout));
+  return st.back(out, dout, ob);
+}
+
 int mace_hip_gemv_q8_u8_host(mace_hip_ctx *ctx, const uint8_t *lhs, const uint8_t *rhs,
                              const int32_t *bias, int64_t batch, int64_t height,
                              int64_t width, int lhs_batched, int rhs_batched, int32_t lhs_zp,

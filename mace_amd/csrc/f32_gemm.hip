@@ -28,7 +28,8 @@ struct F32GemmParams {
   int64_t ors, ocs;   // out element strides for (row, col)
   int64_t lbs, rbs, obs;
   int M, N, K;
-  const float *bias_row;
+  const float *bias_row;   // added per result row (a convolution's output channel), or nullptr
+  const float *bias_col;   // added per result column (MatMul's bias), or nullptr
   int act;
   float limit;
   int tiles_m;
@@ -134,6 +135,7 @@ __global__ __launch_bounds__(256) void f32_gemm_kernel(F32GemmParams p) {
         if (m < p.M && n < p.N) {
           float v = acc[i][j][r];
           if (p.bias_row) v = v + p.bias_row[m];
+          if (p.bias_col) v = v + p.bias_col[n];
           v = apply_act(v, p.act, p.limit);
           O[(int64_t)m * p.ors + (int64_t)n * p.ocs] = v;
         }
@@ -151,6 +153,7 @@ __global__ void f32_fill_kernel(F32GemmParams p, int64_t total) {
     if (p.bias_row) v = v + p.bias_row[m];
     const int64_t bb = bm / p.M;
     const int n = (int)(i - bm * p.N);
+    if (p.bias_col) v = v + p.bias_col[n];
     p.out[bb * p.obs + (int64_t)m * p.ors + (int64_t)n * p.ocs] = apply_act(v, p.act, p.limit);
   }
 }
@@ -336,11 +339,25 @@ __global__ __launch_bounds__(256 * SPLIT) void f32_gemm_vec_kernel(F32GemmParams
         if (whole || (m < p.M && n < p.N)) {
           float v = acc[i][j][r];
           if (p.bias_row) v = v + p.bias_row[m];
+          if (p.bias_col) v = v + p.bias_col[n];
           v = apply_act(v, p.act, p.limit);
           O[(int64_t)m * p.ors + (int64_t)n * p.ocs] = v;
         }
       }
     }
+}
+
+// images of in_h x in_w copied into zero-filled images of ph x pw at (top, left)
+__global__ __launch_bounds__(256) void f32_pad_nchw_kernel(const float *src, float *dst,
+                                                           int64_t total, int in_h, int in_w, int ph,
+                                                           int pw, int top, int left) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t img = i / ((int64_t)ph * pw);
+    const int rem = (int)(i - img * ph * pw);
+    const int y = rem / pw - top, x = rem % pw - left;
+    dst[i] = ((unsigned)y < (unsigned)in_h && (unsigned)x < (unsigned)in_w)
+                 ? src[(img * in_h + y) * in_w + x] : 0.f;
+  }
 }
 
 struct F32GemvParams {
@@ -448,7 +465,7 @@ int mh_f32_gemm(mace_hip_ctx *ctx, const float *lhs, const float *rhs, int64_t b
   p.rbs = rhs_batched ? depth * cols : 0;
   p.obs = rows * cols;
   p.M = (int)rows; p.N = (int)cols; p.K = (int)depth;
-  p.bias_row = ep.bias_row; p.act = ep.act; p.limit = ep.limit;
+  p.bias_row = ep.bias_row; p.bias_col = ep.bias_col; p.act = ep.act; p.limit = ep.limit;
   if (depth == 0) {
     const int64_t total = batch * rows * cols;
     hipLaunchKernelGGL(f32_fill_kernel, dim3((unsigned)((total + 255) / 256 > 65535 ? 65535 : (total + 255) / 256)),
@@ -494,8 +511,29 @@ int mace_hip_gemm_f32(mace_hip_ctx *ctx, const float *lhs, const float *rhs, int
                       int rhs_major, int out_major, int lhs_batched, int rhs_batched,
                       float *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
-  F32Epilogue ep{nullptr, MACE_HIP_ACT_NOOP, 0.f};
+  F32Epilogue ep{nullptr, nullptr, MACE_HIP_ACT_NOOP, 0.f};
   return mh_f32_gemm(ctx, lhs, rhs, batch, rows, cols, depth, lhs_major, rhs_major, out_major,
+                     lhs_batched, rhs_batched, out, ep);
+}
+
+int mace_hip_matmul_f32(mace_hip_ctx *ctx, const float *lhs, const float *rhs, const float *bias,
+                        int64_t batch, int64_t lhs_rows, int64_t lhs_cols, int64_t rhs_rows,
+                        int64_t rhs_cols, int transpose_lhs, int transpose_rhs, int lhs_batched,
+                        int rhs_batched, float *out) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  // mace/ops/ref/gemm.cc:122-131, then mace/ops/matmul.cc:195-211: c[i * cols + w] += bias[w],
+  // i.e. one binary32 addition to the finished sum, done here as the sum is stored
+  const int64_t rows = transpose_lhs ? lhs_cols : lhs_rows;
+  const int64_t depth = transpose_lhs ? lhs_rows : lhs_cols;
+  const int64_t cols = transpose_rhs ? rhs_rows : rhs_cols;
+  const int64_t depth2 = transpose_rhs ? rhs_cols : rhs_rows;
+  MH_CHECK(ctx, depth == depth2,
+           "Matrices that multiply have inconsistent depth dim: %lld vs. %lld",
+           (long long)depth, (long long)depth2);
+  F32Epilogue ep{nullptr, bias, MACE_HIP_ACT_NOOP, 0.f};
+  return mh_f32_gemm(ctx, lhs, rhs, batch, rows, cols, depth,
+                     transpose_lhs ? MACE_HIP_COL_MAJOR : MACE_HIP_ROW_MAJOR,
+                     transpose_rhs ? MACE_HIP_COL_MAJOR : MACE_HIP_ROW_MAJOR, MACE_HIP_ROW_MAJOR,
                      lhs_batched, rhs_batched, out, ep);
 }
 
@@ -559,9 +597,48 @@ int mace_hip_conv1x1_f32_nchw(mace_hip_ctx *ctx, const float *input, const float
   // mace/ops/arm/base/conv_2d_1x1.cc:66-68: Gemm(filter, input, batch, cout, cin, cin, hw,
   // no transposes, lhs_batched = false, rhs_batched = true); bias and activation follow
   // (mace/ops/conv_2d.cc:171-173) and are fused into the store here.
-  F32Epilogue ep{bias, activation, max_limit};
+  F32Epilogue ep{bias, nullptr, activation, max_limit};
   return mh_f32_gemm(ctx, filter, input, n, cout, hw, cin, MACE_HIP_ROW_MAJOR,
                      MACE_HIP_ROW_MAJOR, MACE_HIP_ROW_MAJOR, 0, 1, out, ep);
+}
+
+int mace_hip_conv2d_f32_nchw(mace_hip_ctx *ctx, const float *input, const float *filter,
+                             const float *bias, int64_t n, int64_t cin, int64_t in_h, int64_t in_w,
+                             int64_t cout, int64_t k_h, int64_t k_w, int stride_h, int stride_w,
+                             int dilation_h, int dilation_w, int pad_h, int pad_w, int activation,
+                             float max_limit, float *out) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_CHECK(ctx, n >= 0 && cin >= 0 && in_h >= 0 && in_w >= 0 && cout >= 0, "negative dimension");
+  MH_CHECK(ctx, k_h >= 1 && k_w >= 1 && stride_h >= 1 && stride_w >= 1 && dilation_h >= 1 &&
+                    dilation_w >= 1 && pad_h >= 0 && pad_w >= 0,
+           "filter / stride / dilation < 1 or negative padding");
+  // the case mace/ops/conv_2d.cc:101-105 hands to Conv2dK1x1; everything else stays with the
+  // caller's general convolution
+  if (k_h != 1 || k_w != 1 || stride_h != 1 || stride_w != 1 || dilation_h != 1 || dilation_w != 1)
+    return mh_fail(ctx, MACE_HIP_UNSUPPORTED,
+                   "only 1x1 filters at stride 1, dilation 1 run on the GPU");
+  if (pad_h == 0 && pad_w == 0)
+    return mace_hip_conv1x1_f32_nchw(ctx, input, filter, bias, n, cin, in_h * in_w, cout,
+                                     activation, max_limit, out);
+  // mace/ops/arm/base/conv_2d_1x1.cc:37-60: the input is copied into a zero-padded tensor
+  // (pad / 2 rows above and columns to the left, the rest below and to the right) and the Gemm
+  // runs over the padded image
+  const int64_t ph = in_h + pad_h, pw = in_w + pad_w;
+  const int64_t total = n * cin * ph * pw;
+  MH_CHECK(ctx, total < (1ll << 40), "dimension too large");
+  if (total == 0 || cout == 0) return MACE_HIP_SUCCESS;
+  MH_CHECK(ctx, input && out, "null operand");
+  MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, sizeof(float) * (size_t)total));
+  ArenaScope scope(ctx);
+  float *padded = (float *)mh_arena_take(ctx, sizeof(float) * (size_t)total);
+  if (!padded) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
+  const int64_t blocks = (total + 255) / 256;
+  hipLaunchKernelGGL(f32_pad_nchw_kernel, dim3((unsigned)(blocks < 65535 ? blocks : 65535)),
+                     dim3(256), 0, ctx->stream, input, padded, total, (int)in_h, (int)in_w,
+                     (int)ph, (int)pw, pad_h >> 1, pad_w >> 1);
+  MH_HIP(ctx, hipGetLastError());
+  return mace_hip_conv1x1_f32_nchw(ctx, padded, filter, bias, n, cin, ph * pw, cout, activation,
+                                   max_limit, out);
 }
 
 }  // extern "C"

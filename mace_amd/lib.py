@@ -25,6 +25,8 @@ _i64, _i32, _f32, _int, _p = C.c_int64, C.c_int32, C.c_float, C.c_int, C.c_void_
 _GEMM_F32 = [_p, _p, _p, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _int, _p]
 _GEMV_F32 = [_p, _p, _p, _p, _i64, _i64, _i64, _int, _int, _p]
 _CONV_F32 = [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _int, _f32, _p]
+_CONV2D_F32 = [_p, _p, _p, _p] + [_i64] * 7 + [_int] * 6 + [_int, _f32, _p]
+_MATMUL_F32 = [_p, _p, _p, _p] + [_i64] * 5 + [_int] * 4 + [_p]
 _GEMV_Q8_U8 = [_p, _p, _p, _p, _i64, _i64, _i64, _int, _int, _i32, _i32, _f32, _f32, _f32,
                _i32, _int, _p]
 _GEMV_Q8_I32 = [_p, _p, _p, _p, _i64, _i64, _i64, _int, _int, _i32, _i32, _p]
@@ -81,6 +83,10 @@ SIGNATURES = {
                                            _int, _int, _int, _int, _p]),
     "mace_hip_gemv_f32": (_int, _GEMV_F32),
     "mace_hip_conv1x1_f32_nchw": (_int, _CONV_F32),
+    "mace_hip_conv2d_f32_nchw": (_int, _CONV2D_F32),
+    "mace_hip_conv2d_f32_nchw_host": (_int, _CONV2D_F32),
+    "mace_hip_matmul_f32": (_int, _MATMUL_F32),
+    "mace_hip_matmul_f32_host": (_int, _MATMUL_F32),
     "mace_hip_gemv_q8_u8": (_int, _GEMV_Q8_U8),
     "mace_hip_gemv_q8_i32": (_int, _GEMV_Q8_I32),
     "mace_hip_gemm_q8_i32": (_int, _GEMM_Q8_I32),

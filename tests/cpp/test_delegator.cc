@@ -42,8 +42,11 @@ static int test_registry() {
   EXPECT((bool)reg.GetCreator(MACE_HIP_DELEGATOR_KEY(Gemv, RT_CPU, float, NEON)));
   EXPECT((bool)reg.GetCreator(MACE_HIP_DELEGATOR_KEY_EX(Gemv, RT_CPU, float, NEON, K3x3)));
   EXPECT((bool)reg.GetCreator(MACE_HIP_DELEGATOR_KEY_EX(Conv2d, RT_CPU, float, NEON, K1x1)));
-  // a tagged-only registration does not serve the general key
-  EXPECT(!reg.GetCreator(MACE_HIP_DELEGATOR_KEY(Conv2d, RT_CPU, float, REF)));
+  // the float Conv2d delegator answers the general key (what Conv2dOp asks for on a host
+  // without NEON, conv_2d.cc:88-91) and the K1x1 tag of a NEON build
+  EXPECT((bool)reg.GetCreator(MACE_HIP_DELEGATOR_KEY(Conv2d, RT_CPU, float, REF)));
+  EXPECT((bool)reg.GetCreator(MACE_HIP_DELEGATOR_KEY_EX(Conv2d, RT_CPU, float, REF, K1x1)));
+  EXPECT(!reg.GetCreator(MACE_HIP_DELEGATOR_KEY(Conv2d, RT_CPU, uint8_t, REF)));
   EXPECT(!reg.GetCreator(MACE_HIP_DELEGATOR_KEY(Gemm, RT_OPENCL, float, REF)));
   // an exact NEON registration wins over the REF fallback
   EXPECT(MACE_HIP_REGISTER_DELEGATOR(&reg, DummyGemv, DelegatorParam,
@@ -69,6 +72,26 @@ static int test_registry() {
   EXPECT(ops::MatMulInferShape(&a2, &b5, false, true, &s) == MaceStatus::MACE_SUCCESS);
   EXPECT(s.rows == 3 && s.cols == 6 && s.depth == 4 && s.batch == 1);
   return g_fail;
+}
+
+// delegator::Gemv served by the CPU oracle: the yardstick the GPU-backed ops are compared with
+struct OracleGemv : public delegator::Gemv {
+  explicit OracleGemv(const DelegatorParam &p) : delegator::Gemv(p) {}
+  MaceStatus Compute(const OpContext *, const Tensor *lhs, const Tensor *rhs, const Tensor *bias,
+                     const index_t batch, const index_t h, const index_t w, const bool lb,
+                     const bool rb, Tensor *out) override {
+    orc_gemv_f32(lhs->data<float>(), rhs->data<float>(), bias ? bias->data<float>() : nullptr,
+                 batch, h, w, lb, rb, out->mutable_data<float>(), 1);
+    return MaceStatus::MACE_SUCCESS;
+  }
+};
+
+// reference tolerance of the float comparisons (matmul_test.cc:142-143)
+static bool close_enough(const std::vector<float> &got, const std::vector<float> &want) {
+  if (got.size() != want.size()) return false;
+  for (size_t i = 0; i < got.size(); ++i)
+    if (!(std::fabs(got[i] - want[i]) <= 1e-2 + 1e-4 * std::fabs(want[i]))) return false;
+  return true;
 }
 
 static bool near(const std::vector<float> &got, const std::vector<float> &want) {
@@ -212,7 +235,37 @@ static int test_compute() {
       }
       EXPECT(mace_hip_weight_cache_stats(h, &builds1, &hits1) == MACE_HIP_SUCCESS);
       EXPECT(builds1 - builds0 == 1 && hits1 - hits0 == 2);
-      EXPECT(mace_hip_weight_unregister(h, db) == MACE_HIP_SUCCESS);
+      mace_hip_free(h, da); mace_hip_free(h, db); mace_hip_free(h, dc);
+    }
+    // The registration ends with the op: once the op is gone the address is no longer a weight,
+    // and a tensor that reuses it (the allocator may hand a freed filter's address to an
+    // activation) is summed afresh.
+    {
+      mace_hip_ctx *h = context.hip();
+      void *da = nullptr, *db = nullptr, *dc = nullptr;
+      mace_hip_malloc(h, a.size(), &da); mace_hip_malloc(h, b.size(), &db); mace_hip_malloc(h, c8.size(), &dc);
+      mace_hip_memcpy_h2d(h, da, a.data(), a.size());
+      mace_hip_memcpy_h2d(h, db, b.data(), b.size());
+      Tensor dA(da, DT_UINT8, {batch, depth, rows}, 0.02f, 77, false, true);
+      Tensor dC(dc, DT_UINT8, {}, 40.f, 128, false, true);
+      {
+        Tensor dB(db, DT_UINT8, {cols, depth}, 0.015f, 201, true, true);
+        ops::MatMulOpQuant op(true, true, DT_UINT8);
+        EXPECT(op.Run(&context, &dA, &dB, &dC) == MaceStatus::MACE_SUCCESS);
+      }
+      // the op is gone; the same address now holds other bytes and is an activation
+      EXPECT(mace_hip_weight_unregister(h, db) == MACE_HIP_INVALID_ARGS);   // already released
+      std::vector<uint8_t> b2(b.size());
+      for (auto &v : b2) v = rng() & 255;
+      mace_hip_memcpy_h2d(h, db, b2.data(), b2.size());
+      Tensor dB2(db, DT_UINT8, {cols, depth}, 0.015f, 201, false, true);
+      ops::MatMulOpQuant op2(true, true, DT_UINT8);
+      EXPECT(op2.Run(&context, &dA, &dB2, &dC) == MaceStatus::MACE_SUCCESS);
+      std::vector<uint8_t> got(c8.size()), want2(c8.size());
+      mace_hip_memcpy_d2h(h, got.data(), dc, got.size());
+      orc_q8_gemm_u8(a.data(), b2.data(), batch, rows, cols, depth, ORC_COL_MAJOR, ORC_COL_MAJOR,
+                     ORC_ROW_MAJOR, 1, 0, -77, -201, nullptr, mult, shift, 128, 0, 255, want2.data(), 4);
+      EXPECT(got == want2);
       mace_hip_free(h, da); mace_hip_free(h, db); mace_hip_free(h, dc);
     }
 
@@ -230,6 +283,203 @@ static int test_compute() {
     orc_q8_gemv_u8(w.data(), x.data(), bias.data(), n, o, isz, 0, 1, 127, 128, 0.01f, 0.02f, 0.9f, 30,
                    ORC_REQUANT_NEON, wanty.data(), 4);
     EXPECT(y == wanty);
+  }
+  {  // float Conv2D through the registry's general key (what an x86 host asks for): 1x1 with
+     // bias + ReLUx fused, host and device tensors, a padded 1x1, and the geometry it forwards
+    std::mt19937 rng(21);
+    std::normal_distribution<float> nd(0.f, 1.f);
+    const index_t n = 3, cin = 40, h = 9, w = 7, cout = 24;
+    std::vector<float> x(n * cin * h * w), f(cout * cin), bias(cout);
+    for (auto &v : x) v = nd(rng);
+    for (auto &v : f) v = nd(rng);
+    for (auto &v : bias) v = nd(rng);
+    Tensor X(x.data(), DT_FLOAT, {n, cin, h, w}), F(f.data(), DT_FLOAT, {cout, cin, 1, 1}, 0, 0, true),
+        Bi(bias.data(), DT_FLOAT, {cout});
+    std::vector<float> y(n * cout * h * w), want(y.size());
+    Tensor Y(y.data(), DT_FLOAT, {});
+    ops::Conv2dOpFloat conv(&reg, {1, 1}, ops::SAME, {}, {1, 1}, RELUX, 1.5f);
+    EXPECT(conv.Run(&context, &X, &F, &Bi, &Y) == MaceStatus::MACE_SUCCESS);
+    EXPECT(Y.shape() == (std::vector<index_t>{n, cout, h, w}));
+    orc_conv1x1_f32_nchw(x.data(), f.data(), bias.data(), n, cin, h * w, cout, ORC_ACT_RELUX, 1.5f,
+                         want.data(), 2);
+    EXPECT(close_enough(y, want));
+    // the delegator alone (no bias, no activation), created through the NEON K1x1 tag as well
+    auto creator = reg.GetCreator(MACE_HIP_DELEGATOR_KEY_EX(Conv2d, RT_CPU, float, NEON, K1x1));
+    EXPECT((bool)creator);
+    std::unique_ptr<OpDelegator> d = creator(delegator::Conv2dParam({1, 1}, {1, 1}, {}, ops::VALID));
+    EXPECT(static_cast<delegator::Conv2d *>(d.get())->Compute(&context, &X, &F, &Y) == MaceStatus::MACE_SUCCESS);
+    orc_conv1x1_f32_nchw(x.data(), f.data(), nullptr, n, cin, h * w, cout, ORC_ACT_NOOP, 0.f, want.data(), 2);
+    EXPECT(close_enough(y, want));
+    // explicit paddings {2, 3}: the reference pads the input with zeros (1 row on top, 1 column
+    // on the left, conv_2d_1x1.cc:37-60) and the result has (h + 2) x (w + 3) pixels
+    {
+      const index_t ph = h + 2, pw = w + 3;
+      std::vector<float> xp(n * cin * ph * pw, 0.f), yp(n * cout * ph * pw), wantp(yp.size());
+      for (index_t i = 0; i < n * cin; ++i)
+        for (index_t r = 0; r < h; ++r)
+          for (index_t c = 0; c < w; ++c) xp[(i * ph + r + 1) * pw + c + 1] = x[(i * h + r) * w + c];
+      orc_conv1x1_f32_nchw(xp.data(), f.data(), bias.data(), n, cin, ph * pw, cout, ORC_ACT_RELU, 0.f,
+                           wantp.data(), 2);
+      Tensor Yp(yp.data(), DT_FLOAT, {});
+      ops::Conv2dOpFloat padded(&reg, {1, 1}, ops::VALID, {2, 3}, {1, 1}, RELU, 0.f);
+      EXPECT(padded.Run(&context, &X, &F, &Bi, &Yp) == MaceStatus::MACE_SUCCESS);
+      EXPECT(Yp.shape() == (std::vector<index_t>{n, cout, ph, pw}));
+      EXPECT(close_enough(yp, wantp));
+      // the same on device tensors
+      mace_hip_ctx *hc = context.hip();
+      void *dx = nullptr, *df = nullptr, *dbias = nullptr, *dy = nullptr;
+      mace_hip_malloc(hc, x.size() * 4, &dx); mace_hip_malloc(hc, f.size() * 4, &df);
+      mace_hip_malloc(hc, bias.size() * 4, &dbias); mace_hip_malloc(hc, yp.size() * 4, &dy);
+      mace_hip_memcpy_h2d(hc, dx, x.data(), x.size() * 4);
+      mace_hip_memcpy_h2d(hc, df, f.data(), f.size() * 4);
+      mace_hip_memcpy_h2d(hc, dbias, bias.data(), bias.size() * 4);
+      Tensor dX(dx, DT_FLOAT, {n, cin, h, w}, 0, 0, false, true), dF(df, DT_FLOAT, {cout, cin, 1, 1}, 0, 0, true, true),
+          dB(dbias, DT_FLOAT, {cout}, 0, 0, true, true), dY(dy, DT_FLOAT, {}, 0, 0, false, true);
+      EXPECT(padded.Run(&context, &dX, &dF, &dB, &dY) == MaceStatus::MACE_SUCCESS);
+      std::vector<float> got(yp.size());
+      mace_hip_memcpy_d2h(hc, got.data(), dy, got.size() * 4);
+      EXPECT(close_enough(got, wantp));
+      mace_hip_free(hc, dx); mace_hip_free(hc, df); mace_hip_free(hc, dbias); mace_hip_free(hc, dy);
+    }
+    // a 3x3 filter, a stride or a dilation is not this delegator's: it forwards (UNSUPPORTED,
+    // nothing written)
+    std::vector<float> f3(cout * cin * 9, 1.f);
+    Tensor F3(f3.data(), DT_FLOAT, {cout, cin, 3, 3});
+    y.assign(y.size(), -7.f);
+    EXPECT(conv.Run(&context, &X, &F3, &Bi, &Y) == MaceStatus::MACE_UNSUPPORTED);
+    EXPECT(y[0] == -7.f && y.back() == -7.f);
+    ops::Conv2dOpFloat strided(&reg, {2, 2}, ops::SAME);
+    EXPECT(strided.Run(&context, &X, &F, &Bi, &Y) == MaceStatus::MACE_UNSUPPORTED);
+    Tensor Fbad(f.data(), DT_FLOAT, {cout, cin + 1, 1, 1});
+    EXPECT(conv.Run(&context, &X, &Fbad, &Bi, &Y) == MaceStatus::MACE_INVALID_ARGS);
+  }
+  {  // float MatMul with the per-column bias on device tensors (matmul.cc:195-211), all transposes
+    std::mt19937 rng(31);
+    std::normal_distribution<float> nd(0.f, 1.f);
+    const index_t batch = 3, rows = 70, depth = 48, cols = 52;
+    std::vector<float> a(batch * rows * depth), b(batch * depth * cols), bias(cols);
+    for (auto &v : a) v = nd(rng);
+    for (auto &v : b) v = nd(rng);
+    for (auto &v : bias) v = nd(rng);
+    mace_hip_ctx *hc = context.hip();
+    void *da = nullptr, *db = nullptr, *dbias = nullptr, *dc = nullptr;
+    mace_hip_malloc(hc, a.size() * 4, &da); mace_hip_malloc(hc, b.size() * 4, &db);
+    mace_hip_malloc(hc, bias.size() * 4, &dbias); mace_hip_malloc(hc, batch * rows * cols * 4, &dc);
+    mace_hip_memcpy_h2d(hc, da, a.data(), a.size() * 4);
+    mace_hip_memcpy_h2d(hc, db, b.data(), b.size() * 4);
+    mace_hip_memcpy_h2d(hc, dbias, bias.data(), bias.size() * 4);
+    for (int ta = 0; ta < 2; ++ta)
+      for (int tb = 0; tb < 2; ++tb) {
+        Tensor A(da, DT_FLOAT, ta ? std::vector<index_t>{batch, depth, rows} : std::vector<index_t>{batch, rows, depth}, 0, 0, false, true);
+        Tensor B(db, DT_FLOAT, tb ? std::vector<index_t>{batch, cols, depth} : std::vector<index_t>{batch, depth, cols}, 0, 0, false, true);
+        Tensor Bi(dbias, DT_FLOAT, {cols}, 0, 0, false, true), Cc(dc, DT_FLOAT, {}, 0, 0, false, true);
+        ops::MatMulOpFloat op(&reg, ta != 0, tb != 0);
+        EXPECT(op.Run(&context, &A, &B, &Bi, &Cc) == MaceStatus::MACE_SUCCESS);
+        std::vector<float> got(batch * rows * cols), want(got.size());
+        mace_hip_memcpy_d2h(hc, got.data(), dc, got.size() * 4);
+        orc_gemm_f32(a.data(), b.data(), batch, rows, cols, depth, ta ? ORC_COL_MAJOR : ORC_ROW_MAJOR,
+                     tb ? ORC_COL_MAJOR : ORC_ROW_MAJOR, ORC_ROW_MAJOR, 1, 1, want.data(), 2);
+        for (index_t i = 0; i < batch * rows; ++i)
+          for (index_t w2 = 0; w2 < cols; ++w2) want[i * cols + w2] += bias[w2];
+        EXPECT(close_enough(got, want));
+        Tensor BadBias(dbias, DT_FLOAT, {cols - 1}, 0, 0, false, true);
+        EXPECT(op.Run(&context, &A, &B, &BadBias, &Cc) == MaceStatus::MACE_INVALID_ARGS);
+      }
+    mace_hip_free(hc, da); mace_hip_free(hc, db); mace_hip_free(hc, dbias); mace_hip_free(hc, dc);
+  }
+  {  // the Winograd caller of Gemm (conv_2d_3x3_winograd.cc): 2x2 tiles on a small image, 6x6
+     // tiles on a larger one, against the textbook 3x3 convolution sum
+    std::mt19937 rng(41);
+    std::uniform_real_distribution<float> ud(-1.f, 1.f);
+    struct Geo { index_t n, cin, h, w, cout; ops::Padding pad; };
+    for (const Geo &g : {Geo{2, 5, 11, 13, 7, ops::SAME}, Geo{1, 8, 12, 9, 16, ops::VALID},
+                         Geo{2, 6, 23, 19, 9, ops::SAME}, Geo{1, 16, 30, 30, 8, ops::VALID}}) {
+      std::vector<float> x(g.n * g.cin * g.h * g.w), f(g.cout * g.cin * 9);
+      for (auto &v : x) v = ud(rng);
+      for (auto &v : f) v = ud(rng);
+      const index_t oh = g.pad == ops::SAME ? g.h : g.h - 2, ow = g.pad == ops::SAME ? g.w : g.w - 2;
+      const int top = g.pad == ops::SAME ? 1 : 0;
+      std::vector<float> y(g.n * g.cout * oh * ow), want(y.size());
+      for (index_t b = 0; b < g.n; ++b)
+        for (index_t oc = 0; oc < g.cout; ++oc)
+          for (index_t r = 0; r < oh; ++r)
+            for (index_t c = 0; c < ow; ++c) {
+              double s = 0;
+              for (index_t ic = 0; ic < g.cin; ++ic)
+                for (int kh = 0; kh < 3; ++kh)
+                  for (int kw = 0; kw < 3; ++kw) {
+                    const index_t iy = r + kh - top, ix = c + kw - top;
+                    if (iy >= 0 && iy < g.h && ix >= 0 && ix < g.w)
+                      s += (double)x[((b * g.cin + ic) * g.h + iy) * g.w + ix] * f[((oc * g.cin + ic) * 3 + kh) * 3 + kw];
+                  }
+              want[((b * g.cout + oc) * oh + r) * ow + c] = (float)s;
+            }
+      Tensor X(x.data(), DT_FLOAT, {g.n, g.cin, g.h, g.w}), F(f.data(), DT_FLOAT, {g.cout, g.cin, 3, 3}, 0, 0, true),
+          Y(y.data(), DT_FLOAT, {});
+      ops::Conv2dK3x3WinogradOp wino(&reg, g.pad);
+      EXPECT(wino.Run(&context, &X, &F, &Y) == MaceStatus::MACE_SUCCESS);
+      EXPECT(Y.shape() == (std::vector<index_t>{g.n, g.cout, oh, ow}));
+      // the reference compares its Winograd with the direct convolution at 1e-3 / 1e-5
+      // (conv_2d_test.cc: ExpectTensorNear); the 6x6 transform loses a few more bits
+      bool ok = true;
+      for (size_t i = 0; i < y.size(); ++i) ok = ok && std::fabs(y[i] - want[i]) <= 2e-3 + 1e-3 * std::fabs(want[i]);
+      EXPECT(ok);
+    }
+  }
+  {  // DynamicLSTM (dynamic_lstm.cc:160-372): the op with the GPU Gemv against the same op with a
+     // Gemv served by the CPU oracle; with zero weights the step has a closed form
+    std::mt19937 rng(51);
+    std::normal_distribution<float> nd(0.f, 0.3f);
+    OpDelegatorRegistry cpu_reg;
+    EXPECT(MACE_HIP_REGISTER_DELEGATOR(&cpu_reg, OracleGemv, DelegatorParam,
+                                       MACE_HIP_DELEGATOR_KEY(Gemv, RT_CPU, float, kCpuImplType)) ==
+           MaceStatus::MACE_SUCCESS);
+    ops::DynamicLSTMArgs args;
+    const index_t batch = 2, chunk = 7, input_dim = 40, cell = 64, out_dim = 48;
+    args.prev_out_delay = -3; args.prev_cell_delay = -3; args.prev_out_offset = 8; args.prev_out_dim = 24;
+    args.prev_cell_dim = cell; args.subsample_factor = 3; args.scale = 0.9f;
+    args.forward_indexes = {0, 1, 2, 4, 6};
+    args.out_cache_indexes = {4}; args.cell_cache_indexes = {4};
+    const index_t a_in = input_dim + args.prev_out_dim, a_out = 4 * cell;
+    std::vector<float> x(batch * chunk * input_dim), po(batch * 1 * args.prev_out_dim), pc(batch * 1 * cell),
+        wa(a_out * a_in), params(3 * cell), wb(out_dim * cell), ba(a_out), bb(out_dim);
+    for (auto *v : {&x, &po, &pc, &wa, &params, &wb, &ba, &bb}) for (auto &e : *v) e = nd(rng);
+    Tensor X(x.data(), DT_FLOAT, {batch, chunk, input_dim}), PO(po.data(), DT_FLOAT, {batch, 1, args.prev_out_dim}),
+        PC(pc.data(), DT_FLOAT, {batch, 1, cell}), WA(wa.data(), DT_FLOAT, {a_out, a_in}, 0, 0, true),
+        P(params.data(), DT_FLOAT, {3, cell}), WB(wb.data(), DT_FLOAT, {out_dim, cell}, 0, 0, true),
+        BA(ba.data(), DT_FLOAT, {a_out}), BB(bb.data(), DT_FLOAT, {out_dim});
+    std::vector<float> y[2], oc[2], cc[2];
+    for (int which = 0; which < 2; ++which) {
+      y[which].assign(batch * chunk * out_dim, 0.f);
+      oc[which].assign(batch * args.prev_out_dim, 0.f);
+      cc[which].assign(batch * cell, 0.f);
+      Tensor Y(y[which].data(), DT_FLOAT, {}), OC(oc[which].data(), DT_FLOAT, {}), CC(cc[which].data(), DT_FLOAT, {});
+      ops::DynamicLSTMOp op(which == 0 ? &reg : &cpu_reg, args);
+      EXPECT(op.Run(&context, &X, &PO, &PC, &WA, &P, &WB, &BA, &BB, &Y, &OC, &CC) == MaceStatus::MACE_SUCCESS);
+      EXPECT(Y.shape() == (std::vector<index_t>{batch, chunk, out_dim}));
+      EXPECT(OC.shape() == (std::vector<index_t>{batch, 1, args.prev_out_dim}));
+      EXPECT(CC.shape() == (std::vector<index_t>{batch, 1, cell}));
+    }
+    EXPECT(close_enough(y[0], y[1]) && close_enough(oc[0], oc[1]) && close_enough(cc[0], cc[1]));
+    float energy = 0.f;
+    for (float v : y[0]) energy += v * v;
+    EXPECT(energy > 1.f);
+    // closed form: zero weights, biases and peepholes, first frame, c_prev given:
+    // i = f = o = sigmoid(0) = 1/2, c = c_prev / 2 + tanh(0) / 2, m = tanh(c) / 2, out = 0 (+ bias_b)
+    std::vector<float> zwa(wa.size(), 0.f), zwb(wb.size(), 0.f), zp(params.size(), 0.f), y0(batch * chunk * out_dim),
+        oc0(batch * args.prev_out_dim), cc0(batch * cell);
+    Tensor ZWA(zwa.data(), DT_FLOAT, {a_out, a_in}), ZWB(zwb.data(), DT_FLOAT, {out_dim, cell}), ZP(zp.data(), DT_FLOAT, {3, cell}),
+        Y0(y0.data(), DT_FLOAT, {}), OC0(oc0.data(), DT_FLOAT, {}), CC0(cc0.data(), DT_FLOAT, {});
+    ops::DynamicLSTMArgs one = args;
+    one.forward_indexes = {0}; one.out_cache_indexes = {0}; one.cell_cache_indexes = {0}; one.scale = 1.0f;
+    ops::DynamicLSTMOp op1(&reg, one);
+    EXPECT(op1.Run(&context, &X, &PO, &PC, &ZWA, &ZP, &ZWB, nullptr, &BB, &Y0, &OC0, &CC0) == MaceStatus::MACE_SUCCESS);
+    bool ok = true;
+    for (index_t b = 0; b < batch; ++b) {
+      for (index_t c = 0; c < cell; ++c) ok = ok && std::fabs(cc0[b * cell + c] - 0.5f * pc[b * cell + c]) < 1e-6f;
+      for (index_t k = 0; k < out_dim; ++k) ok = ok && std::fabs(y0[b * out_dim + k] - bb[k]) < 1e-6f;
+    }
+    EXPECT(ok);
   }
   {
     // Quantize -> Dequantize as in the reference's test (quantize_test.cc:24-76): round trip

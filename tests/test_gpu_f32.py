@@ -252,3 +252,37 @@ def test_conv1x1_f32_nchw_batch64(ctx, n, cin, h, cout, act, limit, with_bias):
     if act != mh.ACT_NOOP:
         assert got.min() >= 0.0 and (act != mh.ACT_RELUX or got.max() <= limit)
         assert (got == 0.0).any() and (act != mh.ACT_RELUX or (got == limit).any() or limit > 5)
+
+
+def test_matmul_f32_bias_and_padded_conv2d(ctx):
+    """mace_hip_matmul_f32 (the Gemm branch of MatMulOp with its per-column bias,
+    matmul.cc:170-211) and mace_hip_conv2d_f32_nchw (1x1 with explicit padding,
+    arm/base/conv_2d_1x1.cc:37-60; other geometries are refused) against the oracle."""
+    rng = np.random.default_rng(77)
+    b, rows, depth, cols = 2, 300, 64, 260
+    A = rng.standard_normal((b, rows, depth)).astype(np.float32)
+    B = rng.standard_normal((depth, cols)).astype(np.float32)
+    bias = rng.standard_normal(cols).astype(np.float32)
+    out = np.empty(b * rows * cols, np.float32)
+    ctx.call("mace_hip_matmul_f32_host", ptr(A), ptr(B), ptr(bias), b, rows, depth, depth, cols,
+             0, 0, 1, 0, ptr(out))
+    want = orc.gemm_f32(A, B, b, rows, cols, depth, R, R, R, True, False).reshape(b * rows, cols)
+    near(out, (want + bias[None, :]).astype(np.float32).reshape(-1))
+    assert ctx.status("mace_hip_matmul_f32_host", ptr(A), ptr(B), ptr(bias), b, rows, depth,
+                      depth + 1, cols, 0, 0, 1, 0, ptr(out)) == mh.INVALID_ARGS
+    n, cin, h, w, cout, ph, pw = 2, 48, 10, 6, 20, 3, 2
+    x = rng.standard_normal((n, cin, h, w)).astype(np.float32)
+    f = rng.standard_normal((cout, cin)).astype(np.float32)
+    cb = rng.standard_normal(cout).astype(np.float32)
+    xp = np.zeros((n, cin, h + ph, w + pw), np.float32)
+    xp[:, :, ph // 2:ph // 2 + h, pw // 2:pw // 2 + w] = x
+    got = np.empty(n * cout * (h + ph) * (w + pw), np.float32)
+    ctx.call("mace_hip_conv2d_f32_nchw_host", ptr(x), ptr(f), ptr(cb), n, cin, h, w, cout, 1, 1,
+             1, 1, 1, 1, ph, pw, mh.ACT_RELUX, 2.0, ptr(got))
+    want = orc.conv1x1_f32_nchw(xp, f, cb, n, cin, (h + ph) * (w + pw), cout, mh.ACT_RELUX, 2.0)
+    near(got, want.reshape(-1))
+    got.fill(-3.0)
+    for geometry in ((3, 3, 1, 1, 1, 1), (1, 1, 2, 1, 1, 1), (1, 1, 1, 1, 1, 2)):
+        assert ctx.status("mace_hip_conv2d_f32_nchw_host", ptr(x), ptr(f), ptr(cb), n, cin, h, w,
+                          cout, *geometry, 0, 0, mh.ACT_NOOP, 0.0, ptr(got)) == mh.UNSUPPORTED
+    assert (got == -3.0).all()
