@@ -553,8 +553,19 @@ def bench_other(ctx, mh, torch):
                 ta, tb, 0, 1, 1, C.data_ptr()))
             flops = 2.0 * 4 * 1024 ** 3
             tf = flops / (k * 1e-3) / 1e12
+            # a sample of the result against a binary64 product of the same operands (rows of
+            # every batch; the 1e-4 bound of the benchmark configuration, normwise)
+            rows = torch.arange(0, 1024, 37, device="cuda")
+            a64 = (A.transpose(1, 2) if ta else A).double()[:, rows]
+            b64 = (B.transpose(1, 2) if tb else B).double()
+            ref = a64 @ b64
+            rel = float(((C[:, rows].double() - ref).norm() / ref.norm()).item())
+            if not rel <= 1e-4:
+                log("ERROR: fp32 Gemm result off by %.3g (normwise) from the binary64 product" % rel)
+                sys.exit(3)
             out.append({"workload": "f32_gemm_4x1024^3_ta%d_tb%d" % (ta, tb), "kernel_ms": round(k, 4),
-                        "TFLOPS": round(tf, 1), "frac_of_fp32_mfma_peak": round(tf / 157.3, 4)})
+                        "TFLOPS": round(tf, 1), "frac_of_fp32_mfma_peak": round(tf / 157.3, 4),
+                        "sample_rel_err_vs_f64": float("%.3g" % rel)})
     # fp32 Gemv (FullyConnected) 4096 x 4096, batch 1: weights rotated over a set larger than the
     # last-level cache; and the fp32 1x1 convolution (NCHW, bias + ReLU6 fused into the store) on
     # two of the MobileNet shapes at batch 64
@@ -591,7 +602,15 @@ def bench_other(ctx, mh, torch):
         nbytes = 4.0 * (n * hw * hw * (cin + cout) + cout * cin + cout)
         roof = min(157.3, flops / nbytes * PEAK_HBM_GBS / 1e3)
         t = min(whole, k)
+        # a sample of images against the binary64 convolution with bias and ReLU6
+        imgs = torch.tensor([0, n // 2, n - 1], device="cuda")
+        ref = ((f.double() @ x[imgs].double()) + bias.double()[None, :, None]).clamp(0.0, 6.0)
+        rel = float(((y[imgs].double() - ref).norm() / ref.norm()).item())
+        if not rel <= 1e-4:
+            log("ERROR: fp32 conv1x1 result off by %.3g (normwise) from the binary64 one" % rel)
+            sys.exit(3)
         out.append({"workload": "f32_conv1x1_nchw_n%d_%dx%dx%d_to_%d" % (n, hw, hw, cin, cout),
+                    "sample_rel_err_vs_f64": float("%.3g" % rel),
                     "call_ms": round(whole, 4), "kernel_ms": round(k, 4),
                     "TFLOPS": round(flops / (t * 1e-3) / 1e12, 1), "roofline_TFLOPS": round(roof, 1),
                     "frac_of_roofline": round(flops / (t * 1e-3) / 1e12 / roof, 4)})
