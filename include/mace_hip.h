@@ -77,6 +77,22 @@ int mace_hip_profile_enable(mace_hip_ctx *ctx, int on);
 int mace_hip_profile_last_kernel_ms(mace_hip_ctx *ctx, float *elapsed_ms);
 int mace_hip_profile_kernel_count(mace_hip_ctx *ctx, int *count);
 int mace_hip_profile_kernel_ms(mace_hip_ctx *ctx, int index, float *elapsed_ms);
+/* HIP graphs.  MACE runs a net as a fixed sequence of ops on one engine thread
+ * (mace/core/net/serial_net.cc:93-124); for small tensors every op costs a kernel launch or
+ * three, and the launch, not the kernel, is what a step takes.  The counterpart here: the
+ * device-pointer calls made on a context between capture_begin and capture_end are recorded
+ * instead of run, and the recorded sequence is then replayed by one graph launch, on the
+ * context's stream.  The recorded calls must not wait for the stream or grow the context's
+ * scratch arena (host-pointer entry points, mace_hip_sync, the dynamic-range Quantize and a first
+ * call that needs more scratch do; such a call fails and the capture ends in an error), so run
+ * the sequence once eagerly first.  A replay reads and writes the same device buffers the
+ * recorded calls named; scalar arguments (scales, zero points, shapes) are frozen. */
+typedef struct mace_hip_graph mace_hip_graph;
+int mace_hip_graph_capture_begin(mace_hip_ctx *ctx);
+int mace_hip_graph_capture_end(mace_hip_ctx *ctx, mace_hip_graph **graph);
+int mace_hip_graph_launch(mace_hip_ctx *ctx, mace_hip_graph *graph);
+int mace_hip_graph_destroy(mace_hip_ctx *ctx, mace_hip_graph *graph);
+
 /* Test hook: switches kernel families off for this context so that the parity tests reach every
  * family on the same shapes (no counterpart in the reference).  Bit 0: the one-launch kernel for
  * small uint8 GEMM / Conv2D calls; bit 1: the kernel that keeps one operand's tile in LDS.

@@ -72,6 +72,9 @@ struct mace_hip_ctx {
   // beyond its size is an error, and the weight cache (which allocates on first use) is bypassed.
   char *static_scratch = nullptr;
   bool no_alloc = false;
+  // A HIP graph is being captured from this context's stream: nothing may wait for the stream
+  // or reallocate the arena until the capture ends.
+  bool capturing = false;
   // Test hook (mace_hip_ctx_set_kernel_mask): kernel families switched off for this context, so
   // that the tests reach every family on the same shapes.
   int kernel_mask = 0;
@@ -105,13 +108,13 @@ int mh_fail(mace_hip_ctx *ctx, int code, const char *fmt, ...);
 #define MH_PROF_RING 512
 #define MH_PROF_BEGIN(ctx)                                                                       \
   do {                                                                                           \
-    if ((ctx)->prof_on)                                                                          \
+    if ((ctx)->prof_on && !(ctx)->capturing)                                                     \
       MH_HIP((ctx), hipEventRecord((ctx)->prof_ev[2 * ((ctx)->prof_count % MH_PROF_RING)],       \
                                    (ctx)->stream));                                              \
   } while (0)
 #define MH_PROF_END(ctx)                                                                         \
   do {                                                                                           \
-    if ((ctx)->prof_on) {                                                                        \
+    if ((ctx)->prof_on && !(ctx)->capturing) {                                                   \
       MH_HIP((ctx), hipEventRecord((ctx)->prof_ev[2 * ((ctx)->prof_count % MH_PROF_RING) + 1],   \
                                    (ctx)->stream));                                              \
       (ctx)->prof_count++;                                                                       \

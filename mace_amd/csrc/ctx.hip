@@ -51,6 +51,10 @@ int mh_arena_reserve(mace_hip_ctx *ctx, size_t bytes) {
     return mh_fail(ctx, MACE_HIP_OUT_OF_RESOURCES, "arena allocation of %zu bytes failed (mock)",
                    need);
   }
+  if (ctx->capturing)
+    return mh_fail(ctx, MACE_HIP_INVALID_ARGS,
+                   "this call needs %zu bytes of scratch, more than the context holds; run it once "
+                   "before capturing it into a graph", need);
   if (ctx->arena_used != 0)
     return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena grown while slices are live");
   MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
@@ -266,6 +270,59 @@ int mace_hip_profile_last_kernel_ms(mace_hip_ctx *ctx, float *elapsed_ms) {
   if (!ctx || !elapsed_ms) return MACE_HIP_INVALID_ARGS;
   MH_CHECK(ctx, ctx->prof_count > 0, "no kernel has been timed since profiling was enabled");
   return mace_hip_profile_kernel_ms(ctx, ctx->prof_count - 1, elapsed_ms);
+}
+
+// ---- HIP graphs ---------------------------------------------------------------------------------
+
+struct mace_hip_graph {
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+};
+
+int mace_hip_graph_capture_begin(mace_hip_ctx *ctx) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_CHECK(ctx, !ctx->capturing, "a capture is already in progress on this context");
+  MH_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+  ctx->capturing = true;
+  return MACE_HIP_SUCCESS;
+}
+
+int mace_hip_graph_capture_end(mace_hip_ctx *ctx, mace_hip_graph **out) {
+  if (!ctx || !out) return MACE_HIP_INVALID_ARGS;
+  *out = nullptr;
+  MH_CHECK(ctx, ctx->capturing, "no capture in progress on this context");
+  ctx->capturing = false;
+  hipGraph_t g = nullptr;
+  // (ends the capture also when a call in between has invalidated it: the error comes back here)
+  MH_HIP(ctx, hipStreamEndCapture(ctx->stream, &g));
+  mace_hip_graph *h = new (std::nothrow) mace_hip_graph();
+  if (!h) { (void)hipGraphDestroy(g); return MACE_HIP_OUT_OF_RESOURCES; }
+  h->graph = g;
+  const hipError_t e = hipGraphInstantiate(&h->exec, g, nullptr, nullptr, 0);
+  if (e != hipSuccess) {
+    (void)hipGraphDestroy(g);
+    delete h;
+    MH_HIP(ctx, e);
+  }
+  *out = h;
+  return MACE_HIP_SUCCESS;
+}
+
+int mace_hip_graph_launch(mace_hip_ctx *ctx, mace_hip_graph *graph) {
+  if (!ctx || !graph || !graph->exec) return MACE_HIP_INVALID_ARGS;
+  MH_CHECK(ctx, !ctx->capturing, "a capture is in progress on this context");
+  MH_HIP(ctx, hipGraphLaunch(graph->exec, ctx->stream));
+  return MACE_HIP_SUCCESS;
+}
+
+int mace_hip_graph_destroy(mace_hip_ctx *ctx, mace_hip_graph *graph) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  if (!graph) return MACE_HIP_SUCCESS;
+  MH_HIP(ctx, hipStreamSynchronize(ctx->stream));   // a launch of it may still be running
+  if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
+  if (graph->graph) (void)hipGraphDestroy(graph->graph);
+  delete graph;
+  return MACE_HIP_SUCCESS;
 }
 
 int mace_hip_ctx_set_kernel_mask(mace_hip_ctx *ctx, int mask) {

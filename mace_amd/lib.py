@@ -54,6 +54,10 @@ SIGNATURES = {
     "mace_hip_profile_kernel_ms": (_int, [_p, _int, C.POINTER(_f32)]),
     "mace_hip_ctx_fail_next_allocs": (_int, [_p, _int]),
     "mace_hip_ctx_set_kernel_mask": (_int, [_p, _int]),
+    "mace_hip_graph_capture_begin": (_int, [_p]),
+    "mace_hip_graph_capture_end": (_int, [_p, C.POINTER(_p)]),
+    "mace_hip_graph_launch": (_int, [_p, _p]),
+    "mace_hip_graph_destroy": (_int, [_p, _p]),
     "mace_hip_malloc": (_int, [_p, C.c_size_t, C.POINTER(_p)]),
     "mace_hip_free": (_int, [_p, _p]),
     "mace_hip_memcpy_h2d": (_int, [_p, _p, _p, C.c_size_t]),
