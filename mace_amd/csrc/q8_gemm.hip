@@ -631,6 +631,21 @@ __device__ inline void dma_16B(const uint8_t *g, uint8_t *lds_wave_base) {
       (void __attribute__((address_space(3))) *)lds_wave_base, 16, 0, 0);
 }
 
+// The same transfer addressed through a buffer descriptor: base (wave-uniform) + lane offset + scalar
+// offset.  Preferred where the rows can be addressed this way: the compiler treats the global
+// form as a FLAT access that may return through the LDS counter and then waits for ALL outstanding
+// LDS reads (lgkmcnt(0)) wherever it needs one of them, for as long as a transfer is in flight,
+// i.e. throughout the loops below; with the buffer form its waits name the read they need.
+typedef __amdgpu_buffer_rsrc_t mh_rsrc;
+__device__ inline mh_rsrc dma_rsrc(const uint8_t *base) {
+  // raw buffer: stride 0, every 32-bit offset in range, DATA_FORMAT = 32-bit
+  return __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, -1, 0x00020000);
+}
+__device__ inline void dma_16B(mh_rsrc rs, uint32_t lane_off, uint32_t uniform_off, uint8_t *lds_wave_base) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (void __attribute__((address_space(3))) *)lds_wave_base,
+                                           16, (int)lane_off, (int)uniform_off, 0, 0);
+}
+
 // s_waitcnt vmcnt(N) alone (expcnt / lgkmcnt fields left at "no wait")
 template <int N>
 __device__ inline void wait_vmcnt() {
@@ -697,7 +712,8 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
     const int kc = (lane % CPR) ^ swizzle(row);
     ox[j] = (uint32_t)(min(x0 + row, p.XN - 1) - x0) * (uint32_t)p.ldx + kc * 16;
   }
-  auto x_src = [&](int j, int k0) -> const uint8_t * { return Xt + k0 + ox[j]; };
+  const mh_rsrc rsx = dma_rsrc(Xt), rsy = dma_rsrc(Yt);
+  auto dma_x = [&](int j, int k0, uint8_t *dst) { dma_16B(rsx, ox[j], (uint32_t)k0, dst); };
   // CONV: what the gather needs per row: top-left input position of the pixel's patch and the
   // lane's chunk offset; gy[j] is the image base.  A 64-byte slab lies inside one filter tap
   // (cin % 64 == 0), so the tap is the same for the whole wavefront.
@@ -718,24 +734,24 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
       oy[j] = (uint32_t)(y - y0) * (uint32_t)p.ldy + kc * 16;
     }
   }
-  auto y_src = [&](int j, int k0) -> const uint8_t * {
+  auto dma_y = [&](int j, int k0, uint8_t *dst) {
     if constexpr (CONV) {
       const int tap = k0 / p.cv_cin, c0 = k0 - tap * p.cv_cin;   // wave-uniform
       const int kh = tap / p.cv_kw, kw = tap - kh * p.cv_kw;
       const int ih = cv_ih0[j] + kh, iw = cv_iw0[j] + kw;
       const bool inside = (unsigned)ih < (unsigned)p.cv_in_h && (unsigned)iw < (unsigned)p.cv_in_w;
       const uint8_t *src = gy[j] + ((int64_t)ih * p.cv_in_w + iw) * p.cv_cin + c0 + cv_kc[j];
-      return inside ? src : p.cv_zero + cv_kc[j];
+      dma_16B(inside ? src : p.cv_zero + cv_kc[j], dst);   // per-lane addresses: the global form
     } else {
-      return Yt + k0 + oy[j];
+      dma_16B(rsy, oy[j], (uint32_t)k0, dst);
     }
   };
   auto issue_slab = [&](int stage, int k0) {
     uint8_t *sx = lds + stage * STAGE_BYTES + wave * 1024;
 #pragma unroll
-    for (int j = 0; j < LX; ++j) dma_16B(x_src(j, k0), sx + j * NW * 1024);
+    for (int j = 0; j < LX; ++j) dma_x(j, k0, sx + j * NW * 1024);
 #pragma unroll
-    for (int j = 0; j < LY; ++j) dma_16B(y_src(j, k0), sx + Y_OFF + j * NW * 1024);
+    for (int j = 0; j < LY; ++j) dma_y(j, k0, sx + Y_OFF + j * NW * 1024);
   };
 
   v16i acc[FX][FY];
@@ -816,8 +832,8 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
         constexpr int PER_SLOT = (LX + LY + NM - 1) / NM;
 #pragma unroll
         for (int d = m * PER_SLOT; d < (m + 1) * PER_SLOT; ++d) {
-          if (d < LX) dma_16B(x_src(d, dk0), dsx + d * NW * 1024);
-          else if (d < LX + LY) dma_16B(y_src(d - LX, dk0), dsx + Y_OFF + (d - LX) * NW * 1024);
+          if (d < LX) dma_x(d, dk0, dsx + d * NW * 1024);
+          else if (d < LX + LY) dma_y(d - LX, dk0, dsx + Y_OFF + (d - LX) * NW * 1024);
         }
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -872,6 +888,207 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
   }
 
   gemm_epilogue<WX, WY, FX, FY, OutT, SUMY>(acc, ysum, p, lds, b, x0, y0, wx, wy, tid);
+}
+
+// ---- one round of 128 x 128 tiles ------------------------------------------------------------
+//
+// Shapes whose 128 x 128 tiles fill the CUs at most once (2048 x 2048 results and the like) give
+// every SIMD a single wavefront with a 64 x 64 tile, and nothing else hides that wavefront's waits.
+// Measured on the ring kernel above at 2048 x 8192 x 2048 (one tile per CU): a k step took 350 cycles
+// where its four MFMAs need 128, because the fragments of step g + 1 were read during step g and
+// flipped behind its last MFMA, so every step ended with an LDS round trip in the open; and the
+// transfers had one slab period to land.  This kernel keeps the slab layout and the DMA transfers
+// and changes the schedule:
+//   * fragments are read two k steps ahead and flipped one step ahead (three register sets in
+//     rotation), so neither the LDS latency nor the flips sit between MFMAs;
+//   * a ring of STAGES 128-byte slabs with STAGES - 1 slabs ahead of the one multiplied: a
+//     transfer has two slab periods to land;
+//   * both correction vectors are taken in the kernel from the flipped fragments: every wavefront
+//     sums its X fragments on even step positions and its Y fragments on odd ones, and wavefronts
+//     with wx ^ wy = 1 walk the two 32-byte k steps of each 64-byte pair in the opposite order, so
+//     the two wavefronts that hold the same rows cover all of k between them without a branch in
+//     the loop; the call is this one launch.
+// Requirements (checked by the host): K % 128 == 0, rows addressable with 32-bit offsets.
+template <typename OutT, int STAGES>
+__global__ __launch_bounds__(256, 1) void q8_gemm_mid_kernel(GemmParams p, RequantTable) {
+  constexpr int KB = 128, T = 128, NW = 4;
+  constexpr int RPI = 1024 / KB, CPR = KB / 16;
+  constexpr int NL = 2 * T / RPI / NW;            // transfers per wavefront per slab (X then Y rows)
+  constexpr int STAGE_BYTES = 2 * T * KB, Y_OFF = T * KB;
+  constexpr int AHEAD = STAGES - 1;
+  static_assert(STAGES >= 3 && STAGES <= 4, "ring depth");
+  static_assert(NL == 8, "slot layout below");
+
+  extern __shared__ __align__(16) uint8_t lds[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wx = wave & 1, wy = wave >> 1;
+  const int par = wx ^ wy;   // order of the two k steps inside each 64-byte pair
+
+  int tile_x, tile_y;
+  tile_of_block(blockIdx.x, gridDim.x, p.tiles_x, p.tiles_y, &tile_x, &tile_y);
+  const int x0 = tile_x * T, y0 = tile_y * T;
+  const int b = blockIdx.z;
+  const uint8_t *Xt = p.X + (int64_t)b * p.xbs + (int64_t)x0 * p.ldx;
+  const uint8_t *Yt = p.Y + (int64_t)b * p.ybs + (int64_t)y0 * p.ldy;
+
+  // transfer j of this wavefront fills slab rows [(j*NW + wave)*RPI, +RPI): rows 0..127 are X rows,
+  // 128..255 Y rows; lane l lands in row l / CPR, slot l % CPR and fetches chunk slot ^ swizzle
+  uint32_t off[NL];
+#pragma unroll
+  for (int j = 0; j < NL; ++j) {
+    const int r = (j * NW + wave) * RPI + lane / CPR;
+    const int kc = (lane % CPR) ^ ((r >> 1) & 7);
+    if (j < NL / 2) off[j] = (uint32_t)(min(x0 + r, p.XN - 1) - x0) * (uint32_t)p.ldx + kc * 16;
+    else off[j] = (uint32_t)(min(y0 + r - T, p.YN - 1) - y0) * (uint32_t)p.ldy + kc * 16;
+  }
+  const mh_rsrc rsx = dma_rsrc(Xt), rsy = dma_rsrc(Yt);
+  auto dma_one = [&](int j, int stage, int k0) {
+    dma_16B(j < NL / 2 ? rsx : rsy, off[j], (uint32_t)k0, lds + stage * STAGE_BYTES + (j * NW + wave) * 1024);
+  };
+
+  v16i acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+  int xs[2] = {0, 0}, ys[2] = {0, 0};
+
+  // fragment addresses inside a stage: lane l reads row l % 32 of a 32-row block, chunk 2 ks + l / 32
+  const int frow = lane & 31, fsw = (frow >> 1) & 7;
+  int foff[4], rx[4], ry[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks)   // step position ks multiplies chunk pair ks ^ par (see the sums)
+    foff[ks] = frow * KB + (((2 * (ks ^ par) + (lane >> 5)) ^ fsw) << 4);
+  const int xbase = wx * 2 * 32 * KB, ybase = Y_OFF + wy * 2 * 32 * KB;
+  auto point_reads_at = [&](int stage) {
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      rx[ks] = foff[ks] + stage * STAGE_BYTES + xbase;
+      ry[ks] = foff[ks] + stage * STAGE_BYTES + ybase;
+    }
+  };
+  const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+  v4i fa[3][2], fb[3][2];   // three fragment sets in rotation: multiplied / flipped / in flight
+
+  // k step S of a slab.  Slot m: MFMA m on set CUR, the read of fragment m of step S + 2 into set
+  // NN, the flip of fragment m of set NXT (read one step earlier), and (DMA) one transfer.
+  auto k_step = [&](auto s_tag, auto cur_tag, auto dma_tag, int dstage, int dk0) {
+    constexpr int S = decltype(s_tag)::value, CUR = decltype(cur_tag)::value;
+    constexpr int NXT = (CUR + 1) % 3, NN = (CUR + 2) % 3, RK = (S + 2) & 3;
+    constexpr int DJ = decltype(dma_tag)::value;   // first transfer of this step, or -1
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      acc[m >> 1][m & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[CUR][m >> 1], fb[CUR][m & 1],
+                                                                 acc[m >> 1][m & 1], 0, 0, 0);
+      if (m < 2) fa[NN][m] = *(const v4i *)(lds + rx[RK] + m * 32 * KB);
+      else fb[NN][m - 2] = *(const v4i *)(lds + ry[RK] + (m - 2) * 32 * KB);
+      if (m < 2) fa[NXT][m] ^= flip;
+      else fb[NXT][m - 2] ^= flip;
+      if constexpr (DJ >= 0) dma_one(DJ + m, dstage, dk0);
+      // even step positions sum the X fragments, odd ones the Y fragments (one fragment per slot pair)
+      if constexpr ((S & 1) == 0) {
+        if (m == 1) xs[0] = sum16_i8(fa[CUR][0], xs[0]);
+        if (m == 3) xs[1] = sum16_i8(fa[CUR][1], xs[1]);
+      } else {
+        if (m == 1) ys[0] = sum16_i8(fb[CUR][0], ys[0]);
+        if (m == 3) ys[1] = sum16_i8(fb[CUR][1], ys[1]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  const int nslab = p.K / KB;
+  // prologue: slabs 0 .. AHEAD-1 in flight (past the end: the last slab again, see below)
+#pragma unroll
+  for (int s = 0; s < AHEAD; ++s)
+#pragma unroll
+    for (int j = 0; j < NL; ++j) dma_one(j, s, min(s, nslab - 1) * KB);
+  wait_vmcnt<(AHEAD - 1) * NL>();
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  point_reads_at(0);
+#pragma unroll
+  for (int m = 0; m < 2; ++m) {
+    fa[0][m] = *(const v4i *)(lds + rx[0] + m * 32 * KB) ^ flip;
+    fb[0][m] = *(const v4i *)(lds + ry[0] + m * 32 * KB) ^ flip;
+    fa[1][m] = *(const v4i *)(lds + rx[1] + m * 32 * KB);
+    fb[1][m] = *(const v4i *)(lds + ry[1] + m * 32 * KB);
+  }
+
+  // One slab: k steps 0 and 1 fetch the last fragments of its stage; then slab kt+1 must be complete
+  // and every wavefront past its reads of slab kt-1 (whose stage the next transfers overwrite; those
+  // reads were consumed by flips before this point): one barrier covers both.  k steps 2 and 3 fetch
+  // the first fragments of slab kt+1 and feed the ring with slab kt+AHEAD.  Near the end there is no
+  // such slab: the last one is fetched again into a stage nobody reads any more, which keeps the
+  // in-flight count constant; fragments fetched beyond the last slab are never multiplied.
+  int stage = 0;
+  auto slab = [&](auto phase_tag, int kt) {
+    constexpr int PH = decltype(phase_tag)::value;
+    k_step(std::integral_constant<int, 0>{}, std::integral_constant<int, (PH + 0) % 3>{},
+           std::integral_constant<int, -1>{}, 0, 0);
+    k_step(std::integral_constant<int, 1>{}, std::integral_constant<int, (PH + 1) % 3>{},
+           std::integral_constant<int, -1>{}, 0, 0);
+    wait_vmcnt<(AHEAD - 2) * NL>();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    int next = stage + 1;
+    if (next == STAGES) next = 0;
+    int dst = stage + AHEAD;
+    if (dst >= STAGES) dst -= STAGES;
+    const int dk0 = min(kt + AHEAD, nslab - 1) * KB;
+    point_reads_at(next);
+    k_step(std::integral_constant<int, 2>{}, std::integral_constant<int, (PH + 2) % 3>{},
+           std::integral_constant<int, 0>{}, dst, dk0);
+    k_step(std::integral_constant<int, 3>{}, std::integral_constant<int, (PH + 3) % 3>{},
+           std::integral_constant<int, 4>{}, dst, dk0);
+    stage = next;
+  };
+  for (int kt = 0;;) {
+    slab(std::integral_constant<int, 0>{}, kt);
+    if (++kt >= nslab) break;
+    slab(std::integral_constant<int, 1>{}, kt);
+    if (++kt >= nslab) break;
+    slab(std::integral_constant<int, 2>{}, kt);
+    if (++kt >= nslab) break;
+  }
+
+  // the ring is dead: correction terms and the comparison table go where the epilogue expects them
+  wait_vmcnt<0>();
+  __syncthreads();
+  int32_t *sc = (int32_t *)lds;                       // [T] x terms, [T] y terms, then the table
+  int32_t *part = (int32_t *)(lds + 16384);           // [2][T] partial X sums, [2][T] partial Y sums
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int sx = xs[i] + __shfl_xor(xs[i], 32, 64);
+    const int sy = ys[i] + __shfl_xor(ys[i], 32, 64);
+    if (lane < 32) {
+      part[wy * T + (wx * 2 + i) * 32 + lane] = sx;
+      part[2 * T + wx * T + (wy * 2 + i) * 32 + lane] = sy;
+    }
+  }
+  if constexpr (sizeof(OutT) == 1) {
+    if (p.rq.table) stage_requant_pairs(sc + 2 * T, p.rq, tid, 256);
+  }
+  __syncthreads();
+  if (tid < T) {
+    const int x = min(x0 + tid, p.XN - 1);
+    uint32_t c = (uint32_t)p.xcoef * (uint32_t)(part[tid] + part[T + tid]) + (uint32_t)p.xadd;
+    if (p.xbias) c += (uint32_t)p.xbias[x];
+    sc[tid] = (int32_t)c;
+  } else {
+    const int t = tid - T;
+    const int y = min(y0 + t, p.YN - 1);
+    uint32_t c = (uint32_t)p.ycoef * (uint32_t)(part[2 * T + t] + part[3 * T + t]) + (uint32_t)p.yadd;
+    if (p.ybias) c += (uint32_t)p.ybias[y];
+    sc[T + t] = (int32_t)c;
+  }
+  __syncthreads();
+  const int none[2] = {0, 0};
+  gemm_epilogue<2, 2, 2, 2, OutT, false, true>(acc, none, p, lds, b, x0, y0, wx, wy, tid);
 }
 
 // ---- the kernel for an X panel that fits in LDS ----------------------------------------------
@@ -1579,6 +1796,26 @@ int launch_gemm_dma(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, b
   return MACE_HIP_SUCCESS;
 }
 
+// one round of 128 x 128 tiles; the caller has checked K % 128 == 0 and the 32-bit row offsets
+int launch_gemm_mid(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, bool out_u8, int batch) {
+  constexpr int STAGES = 4;
+  p.tiles_x = (p.XN + 127) / 128;
+  p.tiles_y = (p.YN + 127) / 128;
+  const size_t lds = (size_t)STAGES * 256 * 128;
+  dim3 grid(p.tiles_x * p.tiles_y, 1, batch), block(256);
+  auto launch = [&](auto k) -> int {
+    MH_HIP(ctx, mh_allow_big_lds(ctx, (const void *)k, lds));
+    MH_PROF_BEGIN(ctx);
+    hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, tab);
+    return MACE_HIP_SUCCESS;
+  };
+  if (out_u8) MH_RETURN_IF_ERROR(launch(q8_gemm_mid_kernel<uint8_t, STAGES>));
+  else MH_RETURN_IF_ERROR(launch(q8_gemm_mid_kernel<int32_t, STAGES>));
+  MH_PROF_END(ctx);
+  MH_HIP(ctx, hipGetLastError());
+  return MACE_HIP_SUCCESS;
+}
+
 // the one-launch kernel for small problems; the caller has checked its preconditions
 int launch_gemm_fused_small(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, bool out_u8,
                             bool xt, bool yt, int batch) {
@@ -2039,7 +2276,13 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   const bool xres_cv = cv && !cv_small && out_u8 && cv->cin % 64 == 0 && depth % 64 == 0;
   const bool xres = (!cv || xres_cv) && !stream && depth > 0 && kk % 64 == 0 && yn >= 256 &&
                     xres_fits(xres_tx) && !(ctx->kernel_mask & MH_MASK_NO_XRES);
-  if (!stream && !xres) {
+  // At most one round of 128 x 128 tiles (and more than half a round), long k: the kernel that sums
+  // both panels itself, so no pass over either operand is launched.
+  const int64_t tiles128 = ((xn + 127) / 128) * ((yn + 127) / 128) * batch;
+  const bool mid = !cv && !stream && !xres && kk % 128 == 0 && kk >= 512 && xn > 64 && yn > 64 &&
+                   tiles128 <= cu_n && 2 * tiles128 > cu_n && L.ld < (1 << 24) && R.ld < (1 << 24) &&
+                   (size_t)4 * 256 * 128 <= lds_cu && !(ctx->kernel_mask & MH_MASK_NO_MID);
+  if (!stream && !xres && !mid) {
     if (!L.sums && !(sum_y && !x_is_lhs))
       MH_RETURN_IF_ERROR(launch_panel_sums(ctx, L.ptr, L.ld, L.bs, rows, L.k, lhs_nb, corrL));
     if (!R.sums && !(sum_y && x_is_lhs))
@@ -2088,6 +2331,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     p.sum_y = true;
     return launch_gemm_xres_any(ctx, p, tab, out_u8, (int)batch, xres_tx, false);
   }
+  if (mid) return launch_gemm_mid(ctx, p, tab, out_u8, (int)batch);
   if (stream) {
     switch ((p.XN + 31) / 32) {
       case 1: return launch_gemm_stream<1, 1>(ctx, p, tab, (int)batch);

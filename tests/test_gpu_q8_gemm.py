@@ -122,6 +122,30 @@ def test_q8_gemm_x_panel_in_lds(ctx, path, batch, rows, depth, cols, lo, ro, oo)
     check_gemm(ctx, batch, rows, depth, cols, True, True, lo, ro, oo)
 
 
+# The kernel for at most one round of 128 x 128 tiles (more than 128 and at most 256 of them, k a
+# multiple of 128 from 512 on): it sums both panels itself, reads fragments two k steps ahead and
+# leaves its 3-slab unrolled loop at every phase (4, 5, 6 and 7 slabs); ragged edges on both sides,
+# repacked and in-place operands, both result orders, batches, one side shared.
+MID_SHAPES = [  # batch, rows, depth, cols, lhs batched, rhs batched, lhs order, rhs order, out order
+    (1, 1500, 640, 1410, True, True, R, Cm, R), (1, 1408, 512, 1536, True, True, R, R, R),
+    (1, 1537, 768, 1300, True, True, Cm, R, Cm), (2, 1100, 896, 1000, True, True, R, Cm, R),
+    (2, 1024, 512, 1100, False, True, Cm, Cm, R), (1, 2048, 1024, 2048, True, True, R, Cm, Cm),
+    (3, 900, 512, 1000, True, False, R, R, Cm),
+]
+
+
+@pytest.mark.parametrize("batch,rows,depth,cols,lb,rb,lo,ro,oo", MID_SHAPES)
+@pytest.mark.parametrize("mid", ["one_round_kernel", "tiled_kernels"])
+def test_q8_gemm_one_round_of_tiles(ctx, mid, batch, rows, depth, cols, lb, rb, lo, ro, oo):
+    # (the kernel that keeps one panel in LDS would take the 512-deep shapes: switched off here)
+    ctx.call("mace_hip_ctx_set_kernel_mask",
+             mh.MASK_NO_XRES | (0 if mid == "one_round_kernel" else mh.MASK_NO_MID))
+    try:
+        check_gemm(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo)
+    finally:
+        ctx.call("mace_hip_ctx_set_kernel_mask", 0)
+
+
 def test_q8_gemm_config1_matmul(ctx):
     """benchmark configuration 1: A [128x256], B [256x128], zero points 128/128/128, scales
     0.02/0.015/0.05 -> (1649267328, shift 7)."""
