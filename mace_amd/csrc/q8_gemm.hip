@@ -92,6 +92,19 @@ __device__ inline void tile_of_block(int bid, int nblocks, int tiles_x, int tile
   *tx = r / gsize;
 }
 
+// Sum of the 16 bytes of a fragment as read from memory (unsigned, before the flip), added to acc.
+// The sum of the shifted bytes the corrections need is this minus 128 per byte.  v_sad_u8 is an
+// ordinary vector-ALU instruction; the dot-product instructions (sum16_i8 below) do not run next to
+// an MFMA of the same wavefront: two of them per MFMA stretch a 32-cycle MFMA slot to 60 cycles
+// (measured), so loops that issue MFMAs sum with this one.
+__device__ inline int sum16_u8(const v4i &raw, int acc) {
+  uint32_t a = (uint32_t)acc;
+  a = __builtin_amdgcn_sad_u8((uint32_t)raw.x, 0u, a);
+  a = __builtin_amdgcn_sad_u8((uint32_t)raw.y, 0u, a);
+  a = __builtin_amdgcn_sad_u8((uint32_t)raw.z, 0u, a);
+  a = __builtin_amdgcn_sad_u8((uint32_t)raw.w, 0u, a);
+  return (int)a;
+}
 // sum of the 16 signed bytes of a (flipped) fragment, added to acc
 __device__ inline int sum16_i8(const v4i &f, int acc) {
   acc = __builtin_amdgcn_sdot4(f.x, 0x01010101, acc, false);
@@ -810,12 +823,6 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
     for (int m = 0; m < NM; ++m) {
       acc[m / FY][m % FY] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ca[m / FY], cb[m % FY],
                                                                   acc[m / FY][m % FY], 0, 0, 0);
-      if constexpr (SUMY) {
-        constexpr int SUMS_PER_SLOT = (FY + NM - 1) / NM;
-#pragma unroll
-        for (int j = m * SUMS_PER_SLOT; j < (m + 1) * SUMS_PER_SLOT; ++j)
-          if (j < FY) ysum[j] = sum16_i8(cb[j], ysum[j]);
-      }
       constexpr int READS_PER_SLOT = (NF + NM - 1) / NM;
 #pragma unroll
       for (int f = m * READS_PER_SLOT; f < (m + 1) * READS_PER_SLOT; ++f) {
@@ -824,6 +831,8 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
       }
       if (DELAY > 0 && m >= DELAY && m - DELAY < NF) {
         const int f = m - DELAY;
+        if constexpr (SUMY)
+          if (f >= FX) ysum[f - FX] = sum16_u8(nb[f - FX], ysum[f - FX]);   // as read, before the flip
         if (f < FX) na[f] ^= flip;
         else nb[f - FX] ^= flip;
       }
@@ -842,6 +851,8 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
 #pragma unroll
     for (int f = 0; f < NF; ++f)
       if (DELAY == 0 || f + DELAY >= NM) {
+        if constexpr (SUMY)
+          if (f >= FX) ysum[f - FX] = sum16_u8(nb[f - FX], ysum[f - FX]);
         if (f < FX) na[f] ^= flip;
         else nb[f - FX] ^= flip;
       }
@@ -857,6 +868,10 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
 
   v4i a0[FX], b0[FY], a1[FX], b1[FY];
   read_frags(0, 0, a0, b0);
+  if constexpr (SUMY) {
+#pragma unroll
+    for (int j = 0; j < FY; ++j) ysum[j] = sum16_u8(b0[j], ysum[j]);
+  }
   flip_frags(a0, b0);
   int stage = 0;
   for (int kt = 0; kt < nslab; ++kt) {
@@ -886,6 +901,12 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
     k_step(std::true_type{}, a1, b1, a0, b0, next, 0, dst, ks * KB);
     stage = next;
   }
+  if constexpr (SUMY) {
+    // The sums are of the bytes as read: minus the fragments the last step fetched beyond the last
+    // slab (still in b0, flipped), minus 128 per byte of this lane's half of every k step.
+#pragma unroll
+    for (int j = 0; j < FY; ++j) ysum[j] -= sum16_u8(b0[j] ^ flip, 0) + 64 * p.K;
+  }
 
   gemm_epilogue<WX, WY, FX, FY, OutT, SUMY>(acc, ysum, p, lds, b, x0, y0, wx, wy, tid);
 }
@@ -903,8 +924,8 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
 //     rotation), so neither the LDS latency nor the flips sit between MFMAs;
 //   * a ring of STAGES 128-byte slabs with STAGES - 1 slabs ahead of the one multiplied: a
 //     transfer has two slab periods to land;
-//   * both correction vectors are taken in the kernel from the flipped fragments: every wavefront
-//     sums its X fragments on even step positions and its Y fragments on odd ones, and wavefronts
+//   * both correction vectors are taken in the kernel from the fragments as read (v_sad_u8, before
+//     the flip): every wavefront sums its X fragments on even step positions and its Y fragments on odd ones, and wavefronts
 //     with wx ^ wy = 1 walk the two 32-byte k steps of each 64-byte pair in the opposite order, so
 //     the two wavefronts that hold the same rows cover all of k between them without a branch in
 //     the loop; the call is this one launch.
@@ -978,7 +999,7 @@ __global__ __launch_bounds__(256, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
   // NN, the flip of fragment m of set NXT (read one step earlier), and (DMA) one transfer.
   auto k_step = [&](auto s_tag, auto cur_tag, auto dma_tag, int dstage, int dk0) {
     constexpr int S = decltype(s_tag)::value, CUR = decltype(cur_tag)::value;
-    constexpr int NXT = (CUR + 1) % 3, NN = (CUR + 2) % 3, RK = (S + 2) & 3;
+    constexpr int NXT = (CUR + 1) % 3, NN = (CUR + 2) % 3, RK = (S + 2) & 3, PN = (S + 1) & 3;
     constexpr int DJ = decltype(dma_tag)::value;   // first transfer of this step, or -1
 #pragma unroll
     for (int m = 0; m < 4; ++m) {
@@ -986,17 +1007,16 @@ __global__ __launch_bounds__(256, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
                                                                  acc[m >> 1][m & 1], 0, 0, 0);
       if (m < 2) fa[NN][m] = *(const v4i *)(lds + rx[RK] + m * 32 * KB);
       else fb[NN][m - 2] = *(const v4i *)(lds + ry[RK] + (m - 2) * 32 * KB);
-      if (m < 2) fa[NXT][m] ^= flip;
-      else fb[NXT][m - 2] ^= flip;
-      if constexpr (DJ >= 0) dma_one(DJ + m, dstage, dk0);
-      // even step positions sum the X fragments, odd ones the Y fragments (one fragment per slot pair)
-      if constexpr ((S & 1) == 0) {
-        if (m == 1) xs[0] = sum16_i8(fa[CUR][0], xs[0]);
-        if (m == 3) xs[1] = sum16_i8(fa[CUR][1], xs[1]);
+      // fragment m of the next step: summed as read where its step position takes that operand's
+      // sums (even positions X, odd ones Y), then flipped
+      if (m < 2) {
+        if constexpr ((PN & 1) == 0) xs[m] = sum16_u8(fa[NXT][m], xs[m]);
+        fa[NXT][m] ^= flip;
       } else {
-        if (m == 1) ys[0] = sum16_i8(fb[CUR][0], ys[0]);
-        if (m == 3) ys[1] = sum16_i8(fb[CUR][1], ys[1]);
+        if constexpr ((PN & 1) == 1) ys[m - 2] = sum16_u8(fb[NXT][m - 2], ys[m - 2]);
+        fb[NXT][m - 2] ^= flip;
       }
+      if constexpr (DJ >= 0) dma_one(DJ + m, dstage, dk0);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -1013,10 +1033,13 @@ __global__ __launch_bounds__(256, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
   point_reads_at(0);
 #pragma unroll
   for (int m = 0; m < 2; ++m) {
-    fa[0][m] = *(const v4i *)(lds + rx[0] + m * 32 * KB) ^ flip;
-    fb[0][m] = *(const v4i *)(lds + ry[0] + m * 32 * KB) ^ flip;
+    fa[0][m] = *(const v4i *)(lds + rx[0] + m * 32 * KB);
+    fb[0][m] = *(const v4i *)(lds + ry[0] + m * 32 * KB);
     fa[1][m] = *(const v4i *)(lds + rx[1] + m * 32 * KB);
     fb[1][m] = *(const v4i *)(lds + ry[1] + m * 32 * KB);
+    xs[m] = sum16_u8(fa[0][m], xs[m]);    // step position 0
+    fa[0][m] ^= flip;
+    fb[0][m] ^= flip;
   }
 
   // One slab: k steps 0 and 1 fetch the last fragments of its stage; then slab kt+1 must be complete
@@ -1047,13 +1070,20 @@ __global__ __launch_bounds__(256, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
            std::integral_constant<int, 4>{}, dst, dk0);
     stage = next;
   };
+  // The last step of the last slab has summed and flipped the X fragments of a step that does not
+  // exist (set (phase + 1) % 3): taken out again where the loop is left.
+  auto unsum = [&](auto set_tag) {
+    constexpr int G = decltype(set_tag)::value;
+#pragma unroll
+    for (int m = 0; m < 2; ++m) xs[m] -= sum16_u8(fa[G][m] ^ flip, 0);
+  };
   for (int kt = 0;;) {
     slab(std::integral_constant<int, 0>{}, kt);
-    if (++kt >= nslab) break;
+    if (++kt >= nslab) { unsum(std::integral_constant<int, 1>{}); break; }
     slab(std::integral_constant<int, 1>{}, kt);
-    if (++kt >= nslab) break;
+    if (++kt >= nslab) { unsum(std::integral_constant<int, 2>{}); break; }
     slab(std::integral_constant<int, 2>{}, kt);
-    if (++kt >= nslab) break;
+    if (++kt >= nslab) { unsum(std::integral_constant<int, 0>{}); break; }
   }
 
   // the ring is dead: correction terms and the comparison table go where the epilogue expects them
@@ -1076,13 +1106,13 @@ __global__ __launch_bounds__(256, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
   __syncthreads();
   if (tid < T) {
     const int x = min(x0 + tid, p.XN - 1);
-    uint32_t c = (uint32_t)p.xcoef * (uint32_t)(part[tid] + part[T + tid]) + (uint32_t)p.xadd;
+    uint32_t c = (uint32_t)p.xcoef * (uint32_t)(part[tid] + part[T + tid] - 128 * p.K) + (uint32_t)p.xadd;
     if (p.xbias) c += (uint32_t)p.xbias[x];
     sc[tid] = (int32_t)c;
   } else {
     const int t = tid - T;
     const int y = min(y0 + t, p.YN - 1);
-    uint32_t c = (uint32_t)p.ycoef * (uint32_t)(part[2 * T + t] + part[3 * T + t]) + (uint32_t)p.yadd;
+    uint32_t c = (uint32_t)p.ycoef * (uint32_t)(part[2 * T + t] + part[3 * T + t] - 128 * p.K) + (uint32_t)p.yadd;
     if (p.ybias) c += (uint32_t)p.ybias[y];
     sc[T + t] = (int32_t)c;
   }
@@ -1341,8 +1371,8 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
         for (int i = 0; i < FX; ++i) xa[i] = *(const v4i *)(xg + i * 2048 + foff[t]);
 #pragma unroll
         for (int j = 0; j < FY; ++j) {
+          ysum[j] = sum16_u8(cur[t][j], ysum[j]);   // as read; the 128 per byte comes off below
           yf[j] = cur[t][j] ^ flip;
-          ysum[j] = sum16_i8(yf[j], ysum[j]);
         }
 #pragma unroll
         for (int i = 0; i < FX; ++i)
@@ -1363,6 +1393,8 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
     };
     group(std::true_type{}, 0);
     for (int g = 1; g < ngroup; ++g) group(std::false_type{}, g);
+#pragma unroll
+    for (int j = 0; j < FY; ++j) ysum[j] -= 64 * p.K;   // this lane's half of every row: K / 2 bytes
     gemm_epilogue<1, 1, FX, FY, OutT, true, true>(acc, ysum, p, lds, b, x0, blk * TYW, 0, 0, tid);
     blk = nb;
     yr = yrn;
@@ -1460,9 +1492,11 @@ void q8_gemm_stream_kernel(GemmParams p, RequantTable) {
         int ys = 0;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-          f[ks] = (ks == KS - 1 && tail_absent) ? zero4 : (yf[d][ks] ^ flip);
-          ys = sum16_i8(f[ks], ys);
+          const bool absent = ks == KS - 1 && tail_absent;
+          f[ks] = absent ? zero4 : (yf[d][ks] ^ flip);
+          if (!absent) ys = sum16_u8(yf[d][ks], ys);   // as read: 128 too much per byte
         }
+        ys -= 128 * 16 * (KS - (tail_absent ? 1 : 0));
         load_y(cur + D * stride, yf[d]);   // refill this slot for D blocks ahead
         ys += __shfl_xor(ys, 32, 64);
         const int y = cur * 32 + r32;
