@@ -913,39 +913,43 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
 
 // ---- one round of 128 x 128 tiles ------------------------------------------------------------
 //
-// Shapes whose 128 x 128 tiles fill the CUs at most once (2048 x 2048 results and the like) give
-// every SIMD a single wavefront with a 64 x 64 tile, and nothing else hides that wavefront's waits.
-// Measured on the ring kernel above at 2048 x 8192 x 2048 (one tile per CU): a k step took 350 cycles
-// where its four MFMAs need 128, because the fragments of step g + 1 were read during step g and
-// flipped behind its last MFMA, so every step ended with an LDS round trip in the open; and the
-// transfers had one slab period to land.  This kernel keeps the slab layout and the DMA transfers
-// and changes the schedule:
-//   * fragments are read two k steps ahead and flipped one step ahead (three register sets in
-//     rotation), so neither the LDS latency nor the flips sit between MFMAs;
-//   * a ring of STAGES 128-byte slabs with STAGES - 1 slabs ahead of the one multiplied: a
-//     transfer has two slab periods to land;
+// Shapes whose 128 x 128 tiles fill the CUs at most once (2048 x 2048 results and the like) leave
+// every CU one workgroup, and with four wavefronts of 64 x 64 results every SIMD a single
+// wavefront.  A wavefront issues in order, an MFMA holds its issue for about 16 of its 32 cycles,
+// and roughly four other instructions fit behind it; a 64 x 64 tile needs per MFMA one fragment
+// read, four flips, its share of the sums and of the transfers.  Measured on the ring kernel
+// above at 2048 x 8192 x 2048 (one tile per CU): a k step of four MFMAs took 350 cycles instead of
+// 128, the parts adding up as if nothing overlapped.  This kernel therefore runs EIGHT wavefronts
+// per tile, two per SIMD, so that one wavefront's reads, flips and transfers issue while the other's
+// MFMA holds its own issue.  The two wavefronts of a SIMD own the same 64 x 64 results and split k:
+// of the four 32-byte k steps of a 128-byte slab, group 0 multiplies the first two and group 1 the
+// last two, each into accumulators of its own, added through LDS at the end (each group then
+// finishes half of the results).  Further:
+//   * a ring of STAGES 128-byte slabs filled by DMA, STAGES - 1 slabs ahead: a transfer has two
+//     slab periods to land;
 //   * both correction vectors are taken in the kernel from the fragments as read (v_sad_u8, before
-//     the flip): every wavefront sums its X fragments on even step positions and its Y fragments on odd ones, and wavefronts
-//     with wx ^ wy = 1 walk the two 32-byte k steps of each 64-byte pair in the opposite order, so
-//     the two wavefronts that hold the same rows cover all of k between them without a branch in
-//     the loop; the call is this one launch.
+//     the flip): a wavefront sums its X fragments on the first of its two k steps and its Y
+//     fragments on the second, and wavefronts with wx ^ wy = 1 take their two k steps in the
+//     opposite order, so the wavefronts that hold the same rows cover all of k between them
+//     without a branch in the loop; the call is this one launch.
 // Requirements (checked by the host): K % 128 == 0, rows addressable with 32-bit offsets.
 template <typename OutT, int STAGES>
-__global__ __launch_bounds__(256, 1) void q8_gemm_mid_kernel(GemmParams p, RequantTable) {
-  constexpr int KB = 128, T = 128, NW = 4;
+__global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel(GemmParams p, RequantTable) {
+  constexpr int KB = 128, T = 128, NW = 8;
   constexpr int RPI = 1024 / KB, CPR = KB / 16;
-  constexpr int NL = 2 * T / RPI / NW;            // transfers per wavefront per slab (X then Y rows)
+  constexpr int NL = 2 * T / RPI / NW;            // transfers per wavefront per slab
   constexpr int STAGE_BYTES = 2 * T * KB, Y_OFF = T * KB;
   constexpr int AHEAD = STAGES - 1;
   static_assert(STAGES >= 3 && STAGES <= 4, "ring depth");
-  static_assert(NL == 8, "slot layout below");
+  static_assert(NL == 4, "one transfer per MFMA slot of the second k step");
 
   extern __shared__ __align__(16) uint8_t lds[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wx = wave & 1, wy = wave >> 1;
-  const int par = wx ^ wy;   // order of the two k steps inside each 64-byte pair
+  const int grp = wave >> 2;                      // which half of every slab's k steps
+  const int wx = wave & 1, wy = (wave >> 1) & 1;
+  const int par = wx ^ wy;                        // order of this wavefront's two k steps
 
   int tile_x, tile_y;
   tile_of_block(blockIdx.x, gridDim.x, p.tiles_x, p.tiles_y, &tile_x, &tile_y);
@@ -978,46 +982,49 @@ __global__ __launch_bounds__(256, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
   int xs[2] = {0, 0}, ys[2] = {0, 0};
 
-  // fragment addresses inside a stage: lane l reads row l % 32 of a 32-row block, chunk 2 ks + l / 32
+  // fragment addresses inside a stage: lane l reads row l % 32 of a 32-row block, chunk 2 ks + l / 32;
+  // this wavefront's first k step is ks = 2 grp + par, its second 2 grp + 1 - par
   const int frow = lane & 31, fsw = (frow >> 1) & 7;
-  int foff[4], rx[4], ry[4];
+  int foff[2], rx[2], ry[2];
 #pragma unroll
-  for (int ks = 0; ks < 4; ++ks)   // step position ks multiplies chunk pair ks ^ par (see the sums)
-    foff[ks] = frow * KB + (((2 * (ks ^ par) + (lane >> 5)) ^ fsw) << 4);
+  for (int q = 0; q < 2; ++q)
+    foff[q] = frow * KB + (((2 * (2 * grp + (q ^ par)) + (lane >> 5)) ^ fsw) << 4);
   const int xbase = wx * 2 * 32 * KB, ybase = Y_OFF + wy * 2 * 32 * KB;
   auto point_reads_at = [&](int stage) {
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      rx[ks] = foff[ks] + stage * STAGE_BYTES + xbase;
-      ry[ks] = foff[ks] + stage * STAGE_BYTES + ybase;
+    for (int q = 0; q < 2; ++q) {
+      rx[q] = foff[q] + stage * STAGE_BYTES + xbase;
+      ry[q] = foff[q] + stage * STAGE_BYTES + ybase;
     }
   };
   const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
-  v4i fa[3][2], fb[3][2];   // three fragment sets in rotation: multiplied / flipped / in flight
+  v4i fa[2][2], fb[2][2];   // set 0: first k step of a slab, set 1: second
 
-  // k step S of a slab.  Slot m: MFMA m on set CUR, the read of fragment m of step S + 2 into set
-  // NN, the flip of fragment m of set NXT (read one step earlier), and (DMA) one transfer.
-  auto k_step = [&](auto s_tag, auto cur_tag, auto dma_tag, int dstage, int dk0) {
-    constexpr int S = decltype(s_tag)::value, CUR = decltype(cur_tag)::value;
-    constexpr int NXT = (CUR + 1) % 3, NN = (CUR + 2) % 3, RK = (S + 2) & 3, PN = (S + 1) & 3;
-    constexpr int DJ = decltype(dma_tag)::value;   // first transfer of this step, or -1
+  // One k step.  Slot m: MFMA m on set CUR, the read of fragment m of the other set (the wavefront's
+  // next k step: Q says which of its two, from the stage rx / ry point at), and (DMA) one transfer.
+  // Fragments of the other set are summed where their step takes that operand's sums (first step X,
+  // second step Y) and flipped once they have landed: the X ones two slots after their read, the Y
+  // ones behind the last MFMA.
+  auto k_step = [&](auto cur_tag, auto dma_tag, int dstage, int dk0) {
+    constexpr int CUR = decltype(cur_tag)::value, OTH = 1 - CUR;
+    constexpr bool dma = decltype(dma_tag)::value;
 #pragma unroll
     for (int m = 0; m < 4; ++m) {
       acc[m >> 1][m & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[CUR][m >> 1], fb[CUR][m & 1],
                                                                  acc[m >> 1][m & 1], 0, 0, 0);
-      if (m < 2) fa[NN][m] = *(const v4i *)(lds + rx[RK] + m * 32 * KB);
-      else fb[NN][m - 2] = *(const v4i *)(lds + ry[RK] + (m - 2) * 32 * KB);
-      // fragment m of the next step: summed as read where its step position takes that operand's
-      // sums (even positions X, odd ones Y), then flipped
-      if (m < 2) {
-        if constexpr ((PN & 1) == 0) xs[m] = sum16_u8(fa[NXT][m], xs[m]);
-        fa[NXT][m] ^= flip;
-      } else {
-        if constexpr ((PN & 1) == 1) ys[m - 2] = sum16_u8(fb[NXT][m - 2], ys[m - 2]);
-        fb[NXT][m - 2] ^= flip;
+      if (m < 2) fa[OTH][m] = *(const v4i *)(lds + rx[OTH] + m * 32 * KB);
+      else fb[OTH][m - 2] = *(const v4i *)(lds + ry[OTH] + (m - 2) * 32 * KB);
+      if (m >= 2) {
+        if constexpr (OTH == 0) xs[m - 2] = sum16_u8(fa[OTH][m - 2], xs[m - 2]);
+        fa[OTH][m - 2] ^= flip;
       }
-      if constexpr (DJ >= 0) dma_one(DJ + m, dstage, dk0);
+      if constexpr (dma) dma_one(m, dstage, dk0);
       __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      if constexpr (OTH == 1) ys[j] = sum16_u8(fb[OTH][j], ys[j]);
+      fb[OTH][j] ^= flip;
     }
   };
 
@@ -1035,26 +1042,21 @@ __global__ __launch_bounds__(256, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
   for (int m = 0; m < 2; ++m) {
     fa[0][m] = *(const v4i *)(lds + rx[0] + m * 32 * KB);
     fb[0][m] = *(const v4i *)(lds + ry[0] + m * 32 * KB);
-    fa[1][m] = *(const v4i *)(lds + rx[1] + m * 32 * KB);
-    fb[1][m] = *(const v4i *)(lds + ry[1] + m * 32 * KB);
-    xs[m] = sum16_u8(fa[0][m], xs[m]);    // step position 0
+    xs[m] = sum16_u8(fa[0][m], xs[m]);
     fa[0][m] ^= flip;
     fb[0][m] ^= flip;
   }
 
-  // One slab: k steps 0 and 1 fetch the last fragments of its stage; then slab kt+1 must be complete
-  // and every wavefront past its reads of slab kt-1 (whose stage the next transfers overwrite; those
-  // reads were consumed by flips before this point): one barrier covers both.  k steps 2 and 3 fetch
-  // the first fragments of slab kt+1 and feed the ring with slab kt+AHEAD.  Near the end there is no
-  // such slab: the last one is fetched again into a stage nobody reads any more, which keeps the
-  // in-flight count constant; fragments fetched beyond the last slab are never multiplied.
+  // One slab: the first k step fetches the second one's fragments from the same stage; then slab
+  // kt+1 must be complete and every wavefront past its reads of slab kt-1 (whose stage the next
+  // transfers overwrite; those reads were consumed by flips before this point): one barrier covers
+  // both.  The second k step fetches the first fragments of slab kt+1 and feeds the ring with slab
+  // kt+AHEAD.  Near the end there is no such slab: the last one is fetched again into a stage nobody
+  // reads any more, which keeps the in-flight count constant; the fragments fetched beyond the last
+  // slab are never multiplied, and their sums are taken out again below.
   int stage = 0;
-  auto slab = [&](auto phase_tag, int kt) {
-    constexpr int PH = decltype(phase_tag)::value;
-    k_step(std::integral_constant<int, 0>{}, std::integral_constant<int, (PH + 0) % 3>{},
-           std::integral_constant<int, -1>{}, 0, 0);
-    k_step(std::integral_constant<int, 1>{}, std::integral_constant<int, (PH + 1) % 3>{},
-           std::integral_constant<int, -1>{}, 0, 0);
+  for (int kt = 0; kt < nslab; ++kt) {
+    k_step(std::integral_constant<int, 0>{}, std::false_type{}, 0, 0);
     wait_vmcnt<(AHEAD - 2) * NL>();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
@@ -1062,63 +1064,73 @@ __global__ __launch_bounds__(256, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
     if (next == STAGES) next = 0;
     int dst = stage + AHEAD;
     if (dst >= STAGES) dst -= STAGES;
-    const int dk0 = min(kt + AHEAD, nslab - 1) * KB;
     point_reads_at(next);
-    k_step(std::integral_constant<int, 2>{}, std::integral_constant<int, (PH + 2) % 3>{},
-           std::integral_constant<int, 0>{}, dst, dk0);
-    k_step(std::integral_constant<int, 3>{}, std::integral_constant<int, (PH + 3) % 3>{},
-           std::integral_constant<int, 4>{}, dst, dk0);
+    k_step(std::integral_constant<int, 1>{}, std::true_type{}, dst, min(kt + AHEAD, nslab - 1) * KB);
     stage = next;
-  };
-  // The last step of the last slab has summed and flipped the X fragments of a step that does not
-  // exist (set (phase + 1) % 3): taken out again where the loop is left.
-  auto unsum = [&](auto set_tag) {
-    constexpr int G = decltype(set_tag)::value;
-#pragma unroll
-    for (int m = 0; m < 2; ++m) xs[m] -= sum16_u8(fa[G][m] ^ flip, 0);
-  };
-  for (int kt = 0;;) {
-    slab(std::integral_constant<int, 0>{}, kt);
-    if (++kt >= nslab) { unsum(std::integral_constant<int, 1>{}); break; }
-    slab(std::integral_constant<int, 1>{}, kt);
-    if (++kt >= nslab) { unsum(std::integral_constant<int, 2>{}); break; }
-    slab(std::integral_constant<int, 2>{}, kt);
-    if (++kt >= nslab) { unsum(std::integral_constant<int, 0>{}); break; }
   }
+#pragma unroll
+  for (int m = 0; m < 2; ++m) xs[m] -= sum16_u8(fa[0][m] ^ flip, 0);
 
-  // the ring is dead: correction terms and the comparison table go where the epilogue expects them
+  // The ring is dead.  Sums: every row has four partial sums (two wavefronts per group that hold it,
+  // two groups).  Accumulators: group 0 finishes X blocks 2 wx, group 1 blocks 2 wx + 1; each sends
+  // the other half to the wavefront of the other group on the same SIMD.
   wait_vmcnt<0>();
   __syncthreads();
   int32_t *sc = (int32_t *)lds;                       // [T] x terms, [T] y terms, then the table
-  int32_t *part = (int32_t *)(lds + 16384);           // [2][T] partial X sums, [2][T] partial Y sums
+  int32_t *part = (int32_t *)(lds + 16384);           // [4][T] partial X sums, [4][T] partial Y sums
+  int32_t *ex = (int32_t *)(lds + 32768);             // [8 wavefronts][32 registers][64 lanes]
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int sx = xs[i] + __shfl_xor(xs[i], 32, 64);
     const int sy = ys[i] + __shfl_xor(ys[i], 32, 64);
     if (lane < 32) {
-      part[wy * T + (wx * 2 + i) * 32 + lane] = sx;
-      part[2 * T + wx * T + (wy * 2 + i) * 32 + lane] = sy;
+      part[(wy * 2 + grp) * T + (wx * 2 + i) * 32 + lane] = sx;
+      part[4 * T + (wx * 2 + grp) * T + (wy * 2 + i) * 32 + lane] = sy;
     }
   }
-  if constexpr (sizeof(OutT) == 1) {
-    if (p.rq.table) stage_requant_pairs(sc + 2 * T, p.rq, tid, 256);
+  v16i fin[1][2];
+  {
+    int32_t *mine = ex + wave * 2048 + lane;
+    const int32_t *theirs = ex + (wave ^ 4) * 2048 + lane;
+    if (grp == 0) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mine[(j * 16 + r) * 64] = acc[1][j][r];
+    } else {
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mine[(j * 16 + r) * 64] = acc[0][j][r];
+    }
+    if constexpr (sizeof(OutT) == 1) {
+      if (p.rq.table) stage_requant_pairs(sc + 2 * T, p.rq, tid, 512);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        fin[0][j][r] = (grp == 0 ? acc[0][j][r] : acc[1][j][r]) + theirs[(j * 16 + r) * 64];
   }
-  __syncthreads();
   if (tid < T) {
     const int x = min(x0 + tid, p.XN - 1);
-    uint32_t c = (uint32_t)p.xcoef * (uint32_t)(part[tid] + part[T + tid] - 128 * p.K) + (uint32_t)p.xadd;
+    const int sum = part[tid] + part[T + tid] + part[2 * T + tid] + part[3 * T + tid] - 128 * p.K;
+    uint32_t c = (uint32_t)p.xcoef * (uint32_t)sum + (uint32_t)p.xadd;
     if (p.xbias) c += (uint32_t)p.xbias[x];
     sc[tid] = (int32_t)c;
-  } else {
+  } else if (tid < 2 * T) {
     const int t = tid - T;
     const int y = min(y0 + t, p.YN - 1);
-    uint32_t c = (uint32_t)p.ycoef * (uint32_t)(part[2 * T + t] + part[3 * T + t] - 128 * p.K) + (uint32_t)p.yadd;
+    const int32_t *py = part + 4 * T;
+    const int sum = py[t] + py[T + t] + py[2 * T + t] + py[3 * T + t] - 128 * p.K;
+    uint32_t c = (uint32_t)p.ycoef * (uint32_t)sum + (uint32_t)p.yadd;
     if (p.ybias) c += (uint32_t)p.ybias[y];
     sc[T + t] = (int32_t)c;
   }
   __syncthreads();
   const int none[2] = {0, 0};
-  gemm_epilogue<2, 2, 2, 2, OutT, false, true>(acc, none, p, lds, b, x0, y0, wx, wy, tid);
+  gemm_epilogue<4, 2, 1, 2, OutT, false, true>(fin, none, p, lds, b, x0, y0, wx * 2 + grp, wy, tid);
 }
 
 // ---- the kernel for an X panel that fits in LDS ----------------------------------------------
@@ -1836,7 +1848,7 @@ int launch_gemm_mid(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, b
   p.tiles_x = (p.XN + 127) / 128;
   p.tiles_y = (p.YN + 127) / 128;
   const size_t lds = (size_t)STAGES * 256 * 128;
-  dim3 grid(p.tiles_x * p.tiles_y, 1, batch), block(256);
+  dim3 grid(p.tiles_x * p.tiles_y, 1, batch), block(512);
   auto launch = [&](auto k) -> int {
     MH_HIP(ctx, mh_allow_big_lds(ctx, (const void *)k, lds));
     MH_PROF_BEGIN(ctx);
