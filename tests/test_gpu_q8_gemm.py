@@ -122,15 +122,17 @@ def test_q8_gemm_x_panel_in_lds(ctx, path, batch, rows, depth, cols, lo, ro, oo)
     check_gemm(ctx, batch, rows, depth, cols, True, True, lo, ro, oo)
 
 
-# The kernel for at most one round of 128 x 128 tiles (more than 128 and at most 256 of them, k a
-# multiple of 128 from 512 on): it sums both panels itself, reads fragments two k steps ahead and
-# leaves its 3-slab unrolled loop at every phase (4, 5, 6 and 7 slabs); ragged edges on both sides,
-# repacked and in-place operands, both result orders, batches, one side shared.
+# The kernel with eight wavefronts per 128 x 128 tile (64 to 640 tiles, k a multiple of 128 from 512
+# on): it sums both panels itself and splits every slab's k steps between two groups of wavefronts;
+# 4, 5, 6, 7 and 8 slabs, ragged edges on both sides, repacked and in-place operands, both result
+# orders, batches, one side shared.
 MID_SHAPES = [  # batch, rows, depth, cols, lhs batched, rhs batched, lhs order, rhs order, out order
     (1, 1500, 640, 1410, True, True, R, Cm, R), (1, 1408, 512, 1536, True, True, R, R, R),
     (1, 1537, 768, 1300, True, True, Cm, R, Cm), (2, 1100, 896, 1000, True, True, R, Cm, R),
     (2, 1024, 512, 1100, False, True, Cm, Cm, R), (1, 2048, 1024, 2048, True, True, R, Cm, Cm),
     (3, 900, 512, 1000, True, False, R, R, Cm),
+    # both ends of the range of tile counts it takes: a quarter of a round, more than one round
+    (1, 1000, 512, 1024, True, True, R, Cm, R), (1, 2500, 640, 2300, True, True, R, Cm, R),
 ]
 
 
