@@ -2322,15 +2322,17 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   const bool xres_cv = cv && !cv_small && out_u8 && cv->cin % 64 == 0 && depth % 64 == 0;
   const bool xres = (!cv || xres_cv) && !stream && depth > 0 && kk % 64 == 0 && yn >= 256 &&
                     xres_fits(xres_tx) && !(ctx->kernel_mask & MH_MASK_NO_XRES);
-  // From a quarter of a round to two and a half rounds of 128 x 128 tiles, long k: the kernel with
-  // eight wavefronts per tile that sums both panels itself, so no pass over either operand is
-  // launched.  Measured against the other tiled kernels (k-contiguous operands): 1024 x 4096 x 1024
+  // From a quarter of a round to one round of 128 x 128 tiles, and up to two and a half rounds where
+  // k is long (with short k and several rounds the two-workgroups-per-CU kernel, which overlaps one
+  // tile's epilogue with another's loop, wins: 32 x 512 x 1024 x 512 29.8 against 33.7 us): the
+  // kernel with eight wavefronts per tile that sums both panels itself, so no pass over either
+  // operand is launched.  Measured against the other tiled kernels (k-contiguous operands): 1024 x 4096 x 1024
   // (64 tiles) 19.2 -> 18.7 us, 1280 x 2048 x 1280 (100) 16.3 -> 12.2, 2048^3 (256) 19.3 -> 14.8,
   // 2560 x 2048 x 2560 (400) 25.8 -> 23.8, 3072 x 1024 x 3072 (576) 26.6 -> 24.9; at 1024 tiles
   // (4096 x 1024 x 4096, 4096^3) the 256 x 256 tiles win by 8 - 13 %.
   const int64_t tiles128 = ((xn + 127) / 128) * ((yn + 127) / 128) * batch;
   const bool mid = !cv && !stream && !xres && kk % 128 == 0 && kk >= 512 && xn > 64 && yn > 64 &&
-                   4 * tiles128 >= cu_n && 2 * tiles128 <= 5 * cu_n && L.ld < (1 << 24) && R.ld < (1 << 24) &&
+                   4 * tiles128 >= cu_n && (tiles128 <= cu_n || (kk >= 2048 && 2 * tiles128 <= 5 * cu_n)) && L.ld < (1 << 24) && R.ld < (1 << 24) &&
                    (size_t)4 * 256 * 128 <= lds_cu && !(ctx->kernel_mask & MH_MASK_NO_MID);
   if (!stream && !xres && !mid) {
     if (!L.sums && !(sum_y && !x_is_lhs))

@@ -132,7 +132,7 @@ MID_SHAPES = [  # batch, rows, depth, cols, lhs batched, rhs batched, lhs order,
     (2, 1024, 512, 1100, False, True, Cm, Cm, R), (1, 2048, 1024, 2048, True, True, R, Cm, Cm),
     (3, 900, 512, 1000, True, False, R, R, Cm),
     # both ends of the range of tile counts it takes: a quarter of a round, more than one round
-    (1, 1000, 512, 1024, True, True, R, Cm, R), (1, 2500, 640, 2300, True, True, R, Cm, R),
+    (1, 1000, 512, 1024, True, True, R, Cm, R), (1, 2300, 2048, 2200, True, True, R, Cm, R),
 ]
 
 
