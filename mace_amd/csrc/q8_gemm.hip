@@ -2283,11 +2283,19 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   const bool sum_y_shape = cv || (depth > 0 && (depth <= 1024 || (x_is_lhs ? rows : cols) <= 2048));
   // A transposing repack can add up its rows on the way; worth its extra (zeroing) launch only
   // where it replaces a pass, i.e. not for a Y operand whose sums the GEMM kernel takes anyway.
+  // ... nor where the call will go to the kernel that sums both panels itself (the shape test of
+  // the dispatch below, with a depth too long for the kernel that keeps a panel in LDS)
+  const int64_t tiles128_pre = (((x_is_lhs ? rows : cols) + 127) / 128) * (((x_is_lhs ? cols : rows) + 127) / 128) * batch;
+  const int64_t cu_pre = ctx->cu_count > 0 ? ctx->cu_count : 256;
+  const bool sums_in_kernel = !cv && depth % 128 == 0 && depth >= 1280 && rows > 64 && cols > 64 &&
+                              4 * tiles128_pre >= cu_pre &&
+                              (tiles128_pre <= cu_pre || (depth >= 2048 && 2 * tiles128_pre <= 5 * cu_pre)) &&
+                              !(ctx->kernel_mask & MH_MASK_NO_MID);
   MH_RETURN_IF_ERROR(prepare(lhs, lhs_order == MACE_HIP_ROW_MAJOR, lhs_direct, lhs_nb, rows, depth,
-                             lhs_w, (!x_is_lhs && sum_y_shape) ? nullptr : corrL, &L));
+                             lhs_w, ((!x_is_lhs && sum_y_shape) || sums_in_kernel) ? nullptr : corrL, &L));
   MH_RETURN_IF_ERROR(prepare(rhs, rhs_order == MACE_HIP_COL_MAJOR, rhs_direct, rhs_nb, cols,
                              rhs_ld != 0 ? rhs_ld : depth, rhs_w,
-                             (x_is_lhs && sum_y_shape) ? nullptr : corrR, &R));
+                             ((x_is_lhs && sum_y_shape) || sums_in_kernel) ? nullptr : corrR, &R));
   const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
   const bool sum_y = cv || (sum_y_shape && !(x_is_lhs ? R.sums : L.sums));   // cached sums cost nothing
   const int32_t l_coef = (int32_t)(0u - zr), l_add = 0;
