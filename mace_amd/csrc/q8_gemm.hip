@@ -932,8 +932,20 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
 //     fragments on the second, and wavefronts with wx ^ wy = 1 take their two k steps in the
 //     opposite order, so the wavefronts that hold the same rows cover all of k between them
 //     without a branch in the loop; the call is this one launch.
-// Requirements (checked by the host): K % 128 == 0, rows addressable with 32-bit offsets.
-template <typename OutT, int STAGES>
+//   * XT: the X operand lies k-major in memory (X(x, k) at X[k * ldx + x]: the RowMajor right-hand
+//     matrix of a MatMul with RowMajor result) and is not repacked.  Its slab is 128 k rows of the
+//     tile's 128 bytes; a transfer instruction moves 8 k rows of 8 chunks, chunk c of row k to slot
+//     (c + k) % 8 of the row.  A fragment is two ds_read_b64_tr_b8: within 16 lanes the instruction
+//     takes 8 bytes at each lane's address and hands lane j < 8 byte j of the even lanes' pieces,
+//     lane 8 + j byte j of the odd lanes' pieces (measured with a pattern in LDS).  Even lanes
+//     point at 8 consecutive k rows of the fragment's first 8 x bytes, odd lanes at the same rows
+//     of the next 8 x bytes, so every lane receives 8 consecutive k of its own x: exactly the
+//     register contents the k-contiguous layout gives, and everything behind the read is shared.
+//     The rotation puts the 16 pieces of two neighbouring 16-lane groups into 16 distinct bank
+//     groups.
+// Requirements (checked by the host): K % 128 == 0, rows addressable with 32-bit offsets; XT: XN a
+// multiple of 16, 16-byte aligned base, the whole operand within 32-bit offsets.
+template <typename OutT, int STAGES, bool XT>
 __global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel(GemmParams p, RequantTable) {
   constexpr int KB = 128, T = 128, NW = 8;
   constexpr int RPI = 1024 / KB, CPR = KB / 16;
@@ -955,22 +967,29 @@ __global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
   tile_of_block(blockIdx.x, gridDim.x, p.tiles_x, p.tiles_y, &tile_x, &tile_y);
   const int x0 = tile_x * T, y0 = tile_y * T;
   const int b = blockIdx.z;
-  const uint8_t *Xt = p.X + (int64_t)b * p.xbs + (int64_t)x0 * p.ldx;
+  const uint8_t *Xt = XT ? p.X + (int64_t)b * p.xbs + x0 : p.X + (int64_t)b * p.xbs + (int64_t)x0 * p.ldx;
   const uint8_t *Yt = p.Y + (int64_t)b * p.ybs + (int64_t)y0 * p.ldy;
 
   // transfer j of this wavefront fills slab rows [(j*NW + wave)*RPI, +RPI): rows 0..127 are X rows,
-  // 128..255 Y rows; lane l lands in row l / CPR, slot l % CPR and fetches chunk slot ^ swizzle
+  // 128..255 Y rows; lane l lands in row l / CPR, slot l % CPR and fetches chunk slot ^ swizzle.
+  // XT: the X rows of the slab are k rows, chunk (slot - row) % 8 of the tile's 128 bytes.
   uint32_t off[NL];
 #pragma unroll
   for (int j = 0; j < NL; ++j) {
     const int r = (j * NW + wave) * RPI + lane / CPR;
     const int kc = (lane % CPR) ^ ((r >> 1) & 7);
-    if (j < NL / 2) off[j] = (uint32_t)(min(x0 + r, p.XN - 1) - x0) * (uint32_t)p.ldx + kc * 16;
-    else off[j] = (uint32_t)(min(y0 + r - T, p.YN - 1) - y0) * (uint32_t)p.ldy + kc * 16;
+    if (j < NL / 2) {
+      if constexpr (XT)   // pieces beyond the end of a k row: the row's last piece again (never stored)
+        off[j] = (uint32_t)r * (uint32_t)p.ldx + min((((lane % CPR) - r) & 7) * 16, p.XN - 16 - x0);
+      else off[j] = (uint32_t)(min(x0 + r, p.XN - 1) - x0) * (uint32_t)p.ldx + kc * 16;
+    } else {
+      off[j] = (uint32_t)(min(y0 + r - T, p.YN - 1) - y0) * (uint32_t)p.ldy + kc * 16;
+    }
   }
   const mh_rsrc rsx = dma_rsrc(Xt), rsy = dma_rsrc(Yt);
   auto dma_one = [&](int j, int stage, int k0) {
-    dma_16B(j < NL / 2 ? rsx : rsy, off[j], (uint32_t)k0, lds + stage * STAGE_BYTES + (j * NW + wave) * 1024);
+    const uint32_t uo = (XT && j < NL / 2) ? (uint32_t)k0 * (uint32_t)p.ldx : (uint32_t)k0;
+    dma_16B(j < NL / 2 ? rsx : rsy, off[j], uo, lds + stage * STAGE_BYTES + (j * NW + wave) * 1024);
   };
 
   v16i acc[2][2];
@@ -990,11 +1009,41 @@ __global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
   for (int q = 0; q < 2; ++q)
     foff[q] = frow * KB + (((2 * (2 * grp + (q ^ par)) + (lane >> 5)) ^ fsw) << 4);
   const int xbase = wx * 2 * 32 * KB, ybase = Y_OFF + wy * 2 * 32 * KB;
+  // XT: lane l of a 16-lane group points at k row 16 (l / 32) + (l % 16) / 2 of the k step, 8 bytes at
+  // x = 32 (2 wx + i) + 16 ((l / 16) % 2) + 8 (l % 2); the second read is 8 k rows (1 KiB) further
+  int xt_off[2][2], rxt[2][2];   // [step of the wavefront][32-row block i]
+  if constexpr (XT) {
+    const int t = (lane & 15) >> 1;
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int c = (wx * 2 + i) * 2 + ((lane >> 4) & 1);
+        const int krow = 32 * (2 * grp + (q ^ par)) + 16 * (lane >> 5) + t;
+        xt_off[q][i] = (krow * 8 + ((c + t) & 7)) * 16 + 8 * (lane & 1);
+      }
+  }
   auto point_reads_at = [&](int stage) {
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
       rx[q] = foff[q] + stage * STAGE_BYTES + xbase;
       ry[q] = foff[q] + stage * STAGE_BYTES + ybase;
+      if constexpr (XT) {
+        rxt[q][0] = xt_off[q][0] + stage * STAGE_BYTES;
+        rxt[q][1] = xt_off[q][1] + stage * STAGE_BYTES;
+      }
+    }
+  };
+  auto read_x = [&](int q, int i) -> v4i {
+    if constexpr (XT) {
+      typedef int v2i_t __attribute__((ext_vector_type(2)));
+      const v2i_t lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+          (v2i_t __attribute__((address_space(3))) *)(lds + rxt[q][i]));
+      const v2i_t hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+          (v2i_t __attribute__((address_space(3))) *)(lds + rxt[q][i] + 1024));
+      return v4i{lo.x, lo.y, hi.x, hi.y};
+    } else {
+      return *(const v4i *)(lds + rx[q] + i * 32 * KB);
     }
   };
   const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
@@ -1012,7 +1061,7 @@ __global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
     for (int m = 0; m < 4; ++m) {
       acc[m >> 1][m & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[CUR][m >> 1], fb[CUR][m & 1],
                                                                  acc[m >> 1][m & 1], 0, 0, 0);
-      if (m < 2) fa[OTH][m] = *(const v4i *)(lds + rx[OTH] + m * 32 * KB);
+      if (m < 2) fa[OTH][m] = read_x(OTH, m);
       else fb[OTH][m - 2] = *(const v4i *)(lds + ry[OTH] + (m - 2) * 32 * KB);
       if (m >= 2) {
         if constexpr (OTH == 0) xs[m - 2] = sum16_u8(fa[OTH][m - 2], xs[m - 2]);
@@ -1040,7 +1089,7 @@ __global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
   point_reads_at(0);
 #pragma unroll
   for (int m = 0; m < 2; ++m) {
-    fa[0][m] = *(const v4i *)(lds + rx[0] + m * 32 * KB);
+    fa[0][m] = read_x(0, m);
     fb[0][m] = *(const v4i *)(lds + ry[0] + m * 32 * KB);
     xs[m] = sum16_u8(fa[0][m], xs[m]);
     fa[0][m] ^= flip;
@@ -1843,7 +1892,8 @@ int launch_gemm_dma(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, b
 }
 
 // one round of 128 x 128 tiles; the caller has checked K % 128 == 0 and the 32-bit row offsets
-int launch_gemm_mid(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, bool out_u8, int batch) {
+int launch_gemm_mid(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, bool out_u8, int batch,
+                    bool xt = false) {
   constexpr int STAGES = 4;
   p.tiles_x = (p.XN + 127) / 128;
   p.tiles_y = (p.YN + 127) / 128;
@@ -1855,8 +1905,13 @@ int launch_gemm_mid(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, b
     hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, tab);
     return MACE_HIP_SUCCESS;
   };
-  if (out_u8) MH_RETURN_IF_ERROR(launch(q8_gemm_mid_kernel<uint8_t, STAGES>));
-  else MH_RETURN_IF_ERROR(launch(q8_gemm_mid_kernel<int32_t, STAGES>));
+  if (xt) {
+    if (out_u8) MH_RETURN_IF_ERROR(launch(q8_gemm_mid_kernel<uint8_t, STAGES, true>));
+    else MH_RETURN_IF_ERROR(launch(q8_gemm_mid_kernel<int32_t, STAGES, true>));
+  } else {
+    if (out_u8) MH_RETURN_IF_ERROR(launch(q8_gemm_mid_kernel<uint8_t, STAGES, false>));
+    else MH_RETURN_IF_ERROR(launch(q8_gemm_mid_kernel<int32_t, STAGES, false>));
+  }
   MH_PROF_END(ctx);
   MH_HIP(ctx, hipGetLastError());
   return MACE_HIP_SUCCESS;
@@ -2159,6 +2214,44 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
       RequantTable tab;
       if (out_u8 && rq.table) mh_requant_table_cached(ctx, rq, tab.t);
       return launch_gemm_xres_any(ctx, p, tab, out_u8, (int)batch, tx, true);
+    }
+    // The same operand layout with a longer k, in the tile-count range of the eight-wavefront
+    // 128 x 128 kernel (see below): its transposing LDS reads take the operand as it lies, so the
+    // repack (2048^3: zeroing 2.4 + repack 7.5 us of a 22 us call) is not launched.
+    const int64_t tiles128 = ((xn + 127) / 128) * ((yn + 127) / 128) * batch;
+    const int64_t cu_n = ctx->cu_count > 0 ? ctx->cu_count : 256;
+    if (!cv && x_kmajor && y_direct && rhs_ld == 0 && !lhs_w && !rhs_w && depth >= 512 &&
+        depth % 128 == 0 && xn % 16 == 0 && (uintptr_t)xp % 16 == 0 && xn > 64 && yn > 64 &&
+        4 * tiles128 >= cu_n && (tiles128 <= cu_n || (depth >= 2048 && 2 * tiles128 <= 5 * cu_n)) &&
+        xn * depth < ((int64_t)1 << 32) && depth < (1 << 24) && (size_t)4 * 256 * 128 <= lds_cu &&
+        !(ctx->kernel_mask & MH_MASK_NO_MID)) {
+      GemmParams p{};
+      const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
+      const int32_t l_coef = (int32_t)(0u - zr), r_coef = (int32_t)(0u - zl);
+      const int32_t r_add = (int32_t)((uint32_t)depth * zl * zr);
+      const int32_t *l_bias = out_u8 ? ep.bias : nullptr;
+      p.X = xp;
+      p.Y = yp;
+      p.XN = (int)xn;
+      p.YN = (int)yn;
+      p.K = (int)depth;
+      p.ldx = xn;      // bytes between consecutive k
+      p.ldy = depth;
+      p.xbs = ((xl ? lhs_nb : rhs_nb) > 1) ? xn * depth : 0;
+      p.ybs = ((xl ? rhs_nb : lhs_nb) > 1) ? yn * depth : 0;
+      p.out = out;
+      p.ldo = p.XN;
+      p.obs = rows * cols;
+      p.rq = rq;
+      p.xcoef = xl ? l_coef : r_coef;
+      p.xadd = xl ? 0 : r_add;
+      p.xbias = xl ? l_bias : nullptr;
+      p.ycoef = xl ? r_coef : l_coef;
+      p.yadd = xl ? r_add : 0;
+      p.ybias = xl ? nullptr : l_bias;
+      RequantTable tab;
+      if (out_u8 && rq.table) mh_requant_table_cached(ctx, rq, tab.t);
+      return launch_gemm_mid(ctx, p, tab, out_u8, (int)batch, true);
     }
   }
 

@@ -133,6 +133,12 @@ MID_SHAPES = [  # batch, rows, depth, cols, lhs batched, rhs batched, lhs order,
     (3, 900, 512, 1000, True, False, R, R, Cm),
     # both ends of the range of tile counts it takes: a quarter of a round, more than one round
     (1, 1000, 512, 1024, True, True, R, Cm, R), (1, 2300, 2048, 2200, True, True, R, Cm, R),
+    # X operand k-major in memory (RowMajor right-hand matrix with a RowMajor result, ColMajor
+    # left-hand matrix with a ColMajor result): read through the transposing LDS loads, nothing
+    # repacked; ragged last tiles in both directions, batches, one side shared
+    (1, 1536, 1024, 1488, True, True, R, R, R), (2, 1000, 640, 1040, True, True, R, R, R),
+    (1, 1296, 1280, 1500, True, True, Cm, Cm, Cm), (2, 1100, 512, 1200, True, False, R, R, R),
+    (1, 2048, 2048, 2048, True, True, R, R, R),
 ]
 
 
