@@ -659,6 +659,33 @@ __device__ inline void dma_16B(mh_rsrc rs, uint32_t lane_off, uint32_t uniform_o
                                            16, (int)lane_off, (int)uniform_off, 0, 0);
 }
 
+// ds_read_b64_tr_b8 (see q8_gemm_mid_kernel for what it returns) as inline assembly: through the
+// builtin the compiler cannot tell the read from the DMA transfers' LDS writes and puts
+// s_waitcnt vmcnt(0) in front of every such read, which drains the ring once per k step (4096^3:
+// 78 -> 102 us).  The price: the compiler does not know that the result arrives later, so whoever
+// reads it first calls lds_wait_tr with the number of LDS instructions the wavefront has issued
+// since (both carry a memory clobber, so no LDS access moves across them and the count is exact).
+typedef int v2i_t __attribute__((ext_vector_type(2)));
+template <int OFF>
+__device__ inline v2i_t lds_read_tr8(int lds_byte_address) {
+  v2i_t r;
+  asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(r) : "v"(lds_byte_address), "n"(OFF) : "memory");
+  return r;
+}
+__device__ __forceinline__ void lds_wait_tr(v4i &frag, int younger) {   // a constant once unrolled
+  switch (younger) {
+#define MH_WAIT_CASE(N) case N: asm volatile("s_waitcnt lgkmcnt(" #N ")" : "+v"(frag) : : "memory"); break;
+    MH_WAIT_CASE(1) MH_WAIT_CASE(2) MH_WAIT_CASE(3) MH_WAIT_CASE(4) MH_WAIT_CASE(5) MH_WAIT_CASE(6)
+    MH_WAIT_CASE(7) MH_WAIT_CASE(8) MH_WAIT_CASE(9) MH_WAIT_CASE(10) MH_WAIT_CASE(11) MH_WAIT_CASE(12)
+    MH_WAIT_CASE(13) MH_WAIT_CASE(14) MH_WAIT_CASE(15)
+#undef MH_WAIT_CASE
+    default: asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(frag) : : "memory"); break;
+  }
+}
+__device__ inline int lds_address_of(const uint8_t *p) {
+  return (int)(uintptr_t)(const __attribute__((address_space(3))) uint8_t *)p;
+}
+
 // s_waitcnt vmcnt(N) alone (expcnt / lgkmcnt fields left at "no wait")
 template <int N>
 __device__ inline void wait_vmcnt() {
@@ -672,14 +699,25 @@ __device__ inline void wait_vmcnt() {
 // and in the 256 x 256 tile the line has left the 32 KB L1 by then, which doubles the
 // L2 -> L1 traffic), and the transfer goes into the stage of slab kt itself, which every
 // wavefront has finished reading at the barrier inside slab kt; two stages then suffice.
+// XT (128-byte slabs only): the X operand lies k-major in memory (X(x, k) at X[k * ldx + x]) and is
+// not repacked.  Its slab is 128 k rows of the tile's TX bytes; a transfer instruction moves 1 KiB
+// of consecutive k rows, chunk c of row k to slot c ^ swz(k) of the row, and a fragment is two
+// ds_read_b64_tr_b8 (see q8_gemm_mid_kernel): the swizzle puts the 16 pieces two neighbouring
+// 16-lane groups read into 16 distinct bank groups.
 template <int WX, int WY, int FX, int FY, int STAGES, typename OutT, int OCC = 1,
-          bool SUMY = false, bool CONV = false, int KB = SLAB>
+          bool SUMY = false, bool CONV = false, int KB = SLAB, bool XT = false>
 __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParams p, RequantTable) {
   constexpr int NW = WX * WY;
   constexpr int TX = WX * FX * 32;
   constexpr int TY = WY * FY * 32;
   static_assert(KB == 64 || KB == 128, "slab width");
   static_assert(!CONV || KB == 64, "the gather addresses one filter tap per 64-byte slab");
+  static_assert(!XT || (KB == 128 && !CONV && (TX == 128 || TX == 256)), "k-major X: 128-byte slabs");
+  constexpr int CX = TX / 16;        // XT: 16-byte chunks per k row of the X slab
+  // XT: chunk c of k row k sits in slot c ^ xt_swz(k) of the row.  XOR by an even number keeps the
+  // four chunks of an aligned 64-byte piece together (in some order), so a transfer instruction
+  // still touches whole 64-byte pieces of memory; a rotation measured 45 % slower at 4096^3.
+  auto xt_swz = [](int k) { return CX == 16 ? (k & 7) << 1 : k & 6; };
   constexpr bool REUSE = KB == 128;  // refill the stage of the slab being multiplied
   constexpr int RPI = 1024 / KB;     // rows per DMA instruction (64 lanes x 16 bytes)
   constexpr int CPR = KB / 16;       // 16-byte chunks per row
@@ -715,18 +753,28 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
   // slot ^ swizzle(row)
   // Addresses are kept as 32-bit byte offsets from the first row of the tile (the host checks
   // that 256 rows fit), so that the transfers take a wave-uniform base plus a lane offset.
-  const uint8_t *Xt = Xb + (int64_t)x0 * p.ldx;
+  const uint8_t *Xt = XT ? Xb + x0 : Xb + (int64_t)x0 * p.ldx;
   const uint8_t *Yt = Yb + (int64_t)y0 * p.ldy;
   uint32_t ox[LX], oy[CONV ? 1 : LY];
   const uint8_t *gy[CONV ? LY : 1];
 #pragma unroll
   for (int j = 0; j < LX; ++j) {
-    const int row = (j * NW + wave) * RPI + lane / CPR;
-    const int kc = (lane % CPR) ^ swizzle(row);
-    ox[j] = (uint32_t)(min(x0 + row, p.XN - 1) - x0) * (uint32_t)p.ldx + kc * 16;
+    if constexpr (XT) {
+      // instruction q = j * NW + wave: k rows [q * 1024 / TX, +1024 / TX) of the slab; pieces beyond
+      // the end of a k row fetch the row's last piece again (never stored)
+      const int kr = (j * NW + wave) * (64 / CX) + lane / CX;
+      const int c = (lane % CX) ^ xt_swz(kr);
+      ox[j] = (uint32_t)kr * (uint32_t)p.ldx + min(c * 16, p.XN - 16 - x0);
+    } else {
+      const int row = (j * NW + wave) * RPI + lane / CPR;
+      const int kc = (lane % CPR) ^ swizzle(row);
+      ox[j] = (uint32_t)(min(x0 + row, p.XN - 1) - x0) * (uint32_t)p.ldx + kc * 16;
+    }
   }
   const mh_rsrc rsx = dma_rsrc(Xt), rsy = dma_rsrc(Yt);
-  auto dma_x = [&](int j, int k0, uint8_t *dst) { dma_16B(rsx, ox[j], (uint32_t)k0, dst); };
+  auto dma_x = [&](int j, int k0, uint8_t *dst) {
+    dma_16B(rsx, ox[j], XT ? (uint32_t)k0 * (uint32_t)p.ldx : (uint32_t)k0, dst);
+  };
   // CONV: what the gather needs per row: top-left input position of the pixel's patch and the
   // lane's chunk offset; gy[j] is the image base.  A 64-byte slab lies inside one filter tap
   // (cin % 64 == 0), so the tap is the same for the whole wavefront.
@@ -789,12 +837,40 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
   const int fy_base = Y_OFF + wy * FY * 32 * KB;
   const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
 
-  auto read_frags = [&](int stage, int ks, v4i (&a)[FX], v4i (&bf)[FY]) {
+  // XT: lane l of a 16-lane group points at k row 16 (l / 32) + (l % 16) / 2 of the k step, 8 bytes at
+  // x = 32 (FX wx + i) + 16 ((l / 16) % 2) + 8 (l % 2); the second read is 8 k rows further
+  int xt_off[XT ? FX : 1];
+  if constexpr (XT) {
+    const int t = (lane & 15) >> 1;
+#pragma unroll
+    for (int i = 0; i < FX; ++i) {
+      const int c = (wx * FX + i) * 2 + ((lane >> 4) & 1);
+      xt_off[i] = ((16 * (lane >> 5) + t) * CX + (c ^ xt_swz(t))) * 16 + 8 * (lane & 1);
+    }
+  }
+  const int lds_base = lds_address_of(lds);
+  auto read_frag = [&](int stage, auto ks_tag, int f) -> v4i {
+    constexpr int ks = decltype(ks_tag)::value;
+    if constexpr (XT) {
+      if (f < FX) {
+        const int a = lds_base + stage * STAGE_BYTES + xt_off[f];
+        const v2i_t lo = lds_read_tr8<ks * 32 * TX>(a);
+        const v2i_t hi = lds_read_tr8<ks * 32 * TX + 8 * TX>(a);
+        return v4i{lo.x, lo.y, hi.x, hi.y};
+      }
+    }
     const uint8_t *s = lds + stage * STAGE_BYTES + foff[ks];
+    return *(const v4i *)(f < FX ? s + fx_base + f * 32 * KB : s + fy_base + (f - FX) * 32 * KB);
+  };
+  auto read_frags = [&](int stage, auto ks_tag, v4i (&a)[FX], v4i (&bf)[FY]) {
 #pragma unroll
-    for (int i = 0; i < FX; ++i) a[i] = *(const v4i *)(s + fx_base + i * 32 * KB);
+    for (int i = 0; i < FX; ++i) a[i] = read_frag(stage, ks_tag, i);
 #pragma unroll
-    for (int j = 0; j < FY; ++j) bf[j] = *(const v4i *)(s + fy_base + j * 32 * KB);
+    for (int j = 0; j < FY; ++j) bf[j] = read_frag(stage, ks_tag, FX + j);
+    if constexpr (XT) {
+#pragma unroll
+      for (int i = 0; i < FX; ++i) lds_wait_tr(a[i], 0);
+    }
   };
   auto flip_frags = [&](v4i (&a)[FX], v4i (&bf)[FY]) {
 #pragma unroll
@@ -811,12 +887,10 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
   // front of a wait nor the flips behind the last MFMA.
   constexpr int NM = FX * FY, NF = FX + FY;
   constexpr int DELAY = NM - NF > 0 ? NM - NF : 0;
-  auto frag_ptr = [&](int stage, int ks, int f) -> const v4i * {
-    const uint8_t *s = lds + stage * STAGE_BYTES + foff[ks];
-    return (const v4i *)(f < FX ? s + fx_base + f * 32 * KB : s + fy_base + (f - FX) * 32 * KB);
-  };
+  static_assert(!XT || (NM >= 2 * NF && (FX - 1) * 2 + FY < 16),
+                "k-major X: every read of a step is issued before its first flip");
   auto k_step = [&](auto dma_tag, v4i (&ca)[FX], v4i (&cb)[FY], v4i (&na)[FX], v4i (&nb)[FY],
-                    int nstage, int nks, int dstage, int dk0) {
+                    int nstage, auto nks, int dstage, int dk0) {
     constexpr bool dma = decltype(dma_tag)::value;
     uint8_t *dsx = lds + dstage * STAGE_BYTES + wave * 1024;
 #pragma unroll
@@ -826,13 +900,17 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
       constexpr int READS_PER_SLOT = (NF + NM - 1) / NM;
 #pragma unroll
       for (int f = m * READS_PER_SLOT; f < (m + 1) * READS_PER_SLOT; ++f) {
-        if (f < FX) na[f] = *frag_ptr(nstage, nks, f);
-        else if (f < NF) nb[f - FX] = *frag_ptr(nstage, nks, f);
+        if (f < FX) na[f] = read_frag(nstage, nks, f);
+        else if (f < NF) nb[f - FX] = read_frag(nstage, nks, f);
       }
       if (DELAY > 0 && m >= DELAY && m - DELAY < NF) {
         const int f = m - DELAY;
         if constexpr (SUMY)
           if (f >= FX) ysum[f - FX] = sum16_u8(nb[f - FX], ysum[f - FX]);   // as read, before the flip
+        if constexpr (XT) {
+          // issued since this fragment's two reads: two per later X fragment, one per Y fragment
+          if (f < FX) lds_wait_tr(na[f], (FX - 1 - f) * 2 + FY);
+        }
         if (f < FX) na[f] ^= flip;
         else nb[f - FX] ^= flip;
       }
@@ -867,7 +945,7 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
   asm volatile("" ::: "memory");
 
   v4i a0[FX], b0[FY], a1[FX], b1[FY];
-  read_frags(0, 0, a0, b0);
+  read_frags(0, std::integral_constant<int, 0>{}, a0, b0);
   if constexpr (SUMY) {
 #pragma unroll
     for (int j = 0; j < FY; ++j) ysum[j] = sum16_u8(b0[j], ysum[j]);
@@ -876,10 +954,10 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
   int stage = 0;
   for (int kt = 0; kt < nslab; ++kt) {
     // all k steps of slab kt but the last; each fetches the fragments of the one after it
-    k_step(std::false_type{}, a0, b0, a1, b1, stage, 1, 0, 0);
+    k_step(std::false_type{}, a0, b0, a1, b1, stage, std::integral_constant<int, 1>{}, 0, 0);
     if constexpr (KSN == 4) {
-      k_step(std::false_type{}, a1, b1, a0, b0, stage, 2, 0, 0);
-      k_step(std::false_type{}, a0, b0, a1, b1, stage, 3, 0, 0);
+      k_step(std::false_type{}, a1, b1, a0, b0, stage, std::integral_constant<int, 2>{}, 0, 0);
+      k_step(std::false_type{}, a0, b0, a1, b1, stage, std::integral_constant<int, 3>{}, 0, 0);
     }
     // Slab kt+1 must be complete, and every wavefront must be done reading the stage the next
     // DMA overwrites (that of slab kt-1, or with REUSE that of slab kt, whose last fragments
@@ -898,7 +976,7 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
     // a stage nobody reads any more, which keeps the loop free of branches and the in-flight
     // count constant; likewise the fragments fetched after the last slab are never used.
     const int ks = min(kt + AHEAD, nslab - 1);
-    k_step(std::true_type{}, a1, b1, a0, b0, next, 0, dst, ks * KB);
+    k_step(std::true_type{}, a1, b1, a0, b0, next, std::integral_constant<int, 0>{}, dst, ks * KB);
     stage = next;
   }
   if constexpr (SUMY) {
@@ -935,13 +1013,14 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
 //   * XT: the X operand lies k-major in memory (X(x, k) at X[k * ldx + x]: the RowMajor right-hand
 //     matrix of a MatMul with RowMajor result) and is not repacked.  Its slab is 128 k rows of the
 //     tile's 128 bytes; a transfer instruction moves 8 k rows of 8 chunks, chunk c of row k to slot
-//     (c + k) % 8 of the row.  A fragment is two ds_read_b64_tr_b8: within 16 lanes the instruction
+//     c ^ (k & 6) of the row (XOR by an even number: the four chunks of an aligned 64-byte piece of
+//     memory stay together, so the transfer still touches whole 64-byte pieces).  A fragment is two ds_read_b64_tr_b8: within 16 lanes the instruction
 //     takes 8 bytes at each lane's address and hands lane j < 8 byte j of the even lanes' pieces,
 //     lane 8 + j byte j of the odd lanes' pieces (measured with a pattern in LDS).  Even lanes
 //     point at 8 consecutive k rows of the fragment's first 8 x bytes, odd lanes at the same rows
 //     of the next 8 x bytes, so every lane receives 8 consecutive k of its own x: exactly the
 //     register contents the k-contiguous layout gives, and everything behind the read is shared.
-//     The rotation puts the 16 pieces of two neighbouring 16-lane groups into 16 distinct bank
+//     The swizzle puts the 16 pieces of two neighbouring 16-lane groups into 16 distinct bank
 //     groups.
 // Requirements (checked by the host): K % 128 == 0, rows addressable with 32-bit offsets; XT: XN a
 // multiple of 16, 16-byte aligned base, the whole operand within 32-bit offsets.
@@ -972,7 +1051,7 @@ __global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
 
   // transfer j of this wavefront fills slab rows [(j*NW + wave)*RPI, +RPI): rows 0..127 are X rows,
   // 128..255 Y rows; lane l lands in row l / CPR, slot l % CPR and fetches chunk slot ^ swizzle.
-  // XT: the X rows of the slab are k rows, chunk (slot - row) % 8 of the tile's 128 bytes.
+  // XT: the X rows of the slab are k rows, chunk slot ^ (row & 6) of the tile's 128 bytes.
   uint32_t off[NL];
 #pragma unroll
   for (int j = 0; j < NL; ++j) {
@@ -980,7 +1059,7 @@ __global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
     const int kc = (lane % CPR) ^ ((r >> 1) & 7);
     if (j < NL / 2) {
       if constexpr (XT)   // pieces beyond the end of a k row: the row's last piece again (never stored)
-        off[j] = (uint32_t)r * (uint32_t)p.ldx + min((((lane % CPR) - r) & 7) * 16, p.XN - 16 - x0);
+        off[j] = (uint32_t)r * (uint32_t)p.ldx + min(((lane % CPR) ^ (r & 6)) * 16, p.XN - 16 - x0);
       else off[j] = (uint32_t)(min(x0 + r, p.XN - 1) - x0) * (uint32_t)p.ldx + kc * 16;
     } else {
       off[j] = (uint32_t)(min(y0 + r - T, p.YN - 1) - y0) * (uint32_t)p.ldy + kc * 16;
@@ -1020,7 +1099,7 @@ __global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
       for (int i = 0; i < 2; ++i) {
         const int c = (wx * 2 + i) * 2 + ((lane >> 4) & 1);
         const int krow = 32 * (2 * grp + (q ^ par)) + 16 * (lane >> 5) + t;
-        xt_off[q][i] = (krow * 8 + ((c + t) & 7)) * 16 + 8 * (lane & 1);
+        xt_off[q][i] = (krow * 8 + (c ^ (t & 6))) * 16 + 8 * (lane & 1);
       }
   }
   auto point_reads_at = [&](int stage) {
@@ -1034,13 +1113,11 @@ __global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
       }
     }
   };
+  const int lds_base = lds_address_of(lds);
   auto read_x = [&](int q, int i) -> v4i {
     if constexpr (XT) {
-      typedef int v2i_t __attribute__((ext_vector_type(2)));
-      const v2i_t lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-          (v2i_t __attribute__((address_space(3))) *)(lds + rxt[q][i]));
-      const v2i_t hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-          (v2i_t __attribute__((address_space(3))) *)(lds + rxt[q][i] + 1024));
+      const v2i_t lo = lds_read_tr8<0>(lds_base + rxt[q][i]);
+      const v2i_t hi = lds_read_tr8<1024>(lds_base + rxt[q][i]);
       return v4i{lo.x, lo.y, hi.x, hi.y};
     } else {
       return *(const v4i *)(lds + rx[q] + i * 32 * KB);
@@ -1064,6 +1141,9 @@ __global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
       if (m < 2) fa[OTH][m] = read_x(OTH, m);
       else fb[OTH][m - 2] = *(const v4i *)(lds + ry[OTH] + (m - 2) * 32 * KB);
       if (m >= 2) {
+        // XT: issued since X fragment m - 2 was read: the other X fragment's two reads (m = 2 only)
+        // and the Y fragments' reads so far
+        if constexpr (XT) lds_wait_tr(fa[OTH][m - 2], m == 2 ? 3 : 2);
         if constexpr (OTH == 0) xs[m - 2] = sum16_u8(fa[OTH][m - 2], xs[m - 2]);
         fa[OTH][m - 2] ^= flip;
       }
@@ -1091,6 +1171,7 @@ __global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
   for (int m = 0; m < 2; ++m) {
     fa[0][m] = read_x(0, m);
     fb[0][m] = *(const v4i *)(lds + ry[0] + m * 32 * KB);
+    if constexpr (XT) lds_wait_tr(fa[0][m], 0);
     xs[m] = sum16_u8(fa[0][m], xs[m]);
     fa[0][m] ^= flip;
     fb[0][m] ^= flip;
@@ -1821,6 +1902,66 @@ int launch_panel_sums(mace_hip_ctx *ctx, const uint8_t *P, int64_t ld, int64_t p
   return MACE_HIP_SUCCESS;
 }
 
+// The same sums for an operand that lies k-major ([k][n], n contiguous, n a multiple of 16): a
+// workgroup owns 256 neighbouring columns over a range of k rows; thread (c, q) adds up 16 columns
+// over every 16th row of the range in 16-bit halves (even and odd bytes of every dword apart, at
+// most 256 rows per thread), the 16 row groups meet in LDS, and one atomic per column adds the
+// workgroup's sum to the zeroed result.
+__global__ __launch_bounds__(256) void q8_kmajor_sums_kernel(const uint8_t *P, int64_t ld, int64_t pbs,
+                                                             int n, int k, int rows_per_block,
+                                                             int32_t *sums) {
+  __shared__ int32_t part[16][256 + 4];
+  const int tid = threadIdx.x, c = tid & 15, q = tid >> 4;
+  const int col0 = blockIdx.x * 256 + c * 16;
+  const int k0 = blockIdx.y * rows_per_block, k1 = min(k, k0 + rows_per_block);
+  uint32_t even[4] = {0, 0, 0, 0}, odd[4] = {0, 0, 0, 0};
+  int cnt = 0;
+  if (col0 < n) {
+    const uint8_t *src = P + (int64_t)blockIdx.z * pbs + col0;
+    for (int r = k0 + q; r < k1; r += 16, ++cnt) {
+      const v4i v = __builtin_nontemporal_load((const v4i *)(src + (int64_t)r * ld));
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        even[d] += (uint32_t)v[d] & 0x00ff00ffu;
+        odd[d] += ((uint32_t)v[d] >> 8) & 0x00ff00ffu;
+      }
+    }
+  }
+  const int shift = 128 * cnt;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    part[q][c * 16 + 4 * d + 0] = (int)(even[d] & 0xffffu) - shift;
+    part[q][c * 16 + 4 * d + 1] = (int)(odd[d] & 0xffffu) - shift;
+    part[q][c * 16 + 4 * d + 2] = (int)(even[d] >> 16) - shift;
+    part[q][c * 16 + 4 * d + 3] = (int)(odd[d] >> 16) - shift;
+  }
+  __syncthreads();
+  const int col = blockIdx.x * 256 + tid;
+  if (col < n) {
+    int s = 0;
+#pragma unroll
+    for (int g = 0; g < 16; ++g) s += part[g][tid];
+    atomicAdd(sums + (int64_t)blockIdx.z * n + col, s);
+  }
+}
+
+int launch_kmajor_sums(mace_hip_ctx *ctx, const uint8_t *P, int64_t ld, int64_t pbs, int64_t n,
+                       int64_t k, int nb, int32_t *sums) {
+  const int64_t cnt = (int64_t)nb * n;
+  hipLaunchKernelGGL(q8_zero_i32_kernel, dim3((unsigned)((cnt + 255) / 256)), dim3(256), 0, ctx->stream,
+                     sums, cnt);
+  const int gx = (int)((n + 255) / 256);
+  const int64_t cu = ctx->cu_count > 0 ? ctx->cu_count : 256;
+  // about four workgroups per CU, at most 4096 rows each (256 per thread: the 16-bit halves hold)
+  const int64_t want = std::max<int64_t>(1, 4 * cu / std::max<int64_t>(1, (int64_t)gx * nb));
+  const int rpb = (int)std::min<int64_t>(4096, std::max<int64_t>(64, (k + want - 1) / want));
+  dim3 grid((unsigned)gx, (unsigned)((k + rpb - 1) / rpb), (unsigned)nb);
+  hipLaunchKernelGGL(q8_kmajor_sums_kernel, grid, dim3(256), 0, ctx->stream, P, ld, pbs, (int)n, (int)k,
+                     rpb, sums);
+  MH_HIP(ctx, hipGetLastError());
+  return MACE_HIP_SUCCESS;
+}
+
 template <int WX, int WY, int FX, int FY>
 int launch_gemm(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, bool out_u8,
                 int batch) {
@@ -1911,6 +2052,33 @@ int launch_gemm_mid(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, b
   } else {
     if (out_u8) MH_RETURN_IF_ERROR(launch(q8_gemm_mid_kernel<uint8_t, STAGES, false>));
     else MH_RETURN_IF_ERROR(launch(q8_gemm_mid_kernel<int32_t, STAGES, false>));
+  }
+  MH_PROF_END(ctx);
+  MH_HIP(ctx, hipGetLastError());
+  return MACE_HIP_SUCCESS;
+}
+
+// 256 x 256 tiles, X operand k-major in memory; the caller has checked the preconditions
+int launch_gemm_big_xt(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, bool out_u8,
+                       int batch) {
+  p.tiles_x = (p.XN + 255) / 256;
+  p.tiles_y = (p.YN + 255) / 256;
+  const size_t lds = (size_t)2 * 512 * 128;
+  dim3 grid(p.tiles_x * p.tiles_y, 1, batch), block(256);
+  auto launch = [&](auto k) -> int {
+    MH_HIP(ctx, mh_allow_big_lds(ctx, (const void *)k, lds));
+    MH_PROF_BEGIN(ctx);
+    hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, tab);
+    return MACE_HIP_SUCCESS;
+  };
+  if (out_u8 && p.sum_y) {
+    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<2, 2, 4, 4, 2, uint8_t, 1, true, false, 128, true>));
+  } else if (out_u8) {
+    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<2, 2, 4, 4, 2, uint8_t, 1, false, false, 128, true>));
+  } else if (p.sum_y) {
+    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<2, 2, 4, 4, 2, int32_t, 1, true, false, 128, true>));
+  } else {
+    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<2, 2, 4, 4, 2, int32_t, 1, false, false, 128, true>));
   }
   MH_PROF_END(ctx);
   MH_HIP(ctx, hipGetLastError());
@@ -2036,6 +2204,27 @@ int launch_gemm_stream(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab
 
 // Shapes of the streaming kernel for a small X panel: depth 16 ... 64 in whole 16-byte pieces, at
 // most 128 X rows in whole 16-byte output pieces, a long Y panel.
+// Tile shape of the tiled kernels: bigger tiles do more MFMA work per byte moved and per barrier,
+// smaller ones keep more CUs busy.  Score = relative efficiency of the shape x the fraction of CU
+// slots its last round of workgroups fills.
+enum MhTile { MH_TILE_BIG, MH_TILE_SKINNY, MH_TILE_MEDIUM, MH_TILE_SMALL };
+static MhTile mh_q8_tile_choice(int64_t xn, int64_t yn, int64_t batch, int64_t cu) {
+  auto score = [&](int tx, int ty, double weight) {
+    const int64_t t = ((xn + tx - 1) / tx) * ((yn + ty - 1) / ty) * batch;
+    const int64_t rounds = (t + cu - 1) / cu;
+    return weight * (double)t / (double)(rounds * cu);
+  };
+  const double s_big = (xn > 128 && yn > 128) ? score(256, 256, 1.0) : 0.0;
+  const double s_skinny = (xn <= 64 && yn > 128) ? score(64, 256, 0.6) : 0.0;
+  const double s_medium = (xn > 64 && yn > 64) ? score(128, 128, 0.6) : 0.0;
+  const double s_small = score(64, 64, 0.3);
+  const double best = std::max(std::max(s_big, s_skinny), std::max(s_medium, s_small));
+  if (s_big == best) return MH_TILE_BIG;
+  if (s_skinny == best) return MH_TILE_SKINNY;
+  if (s_medium == best) return MH_TILE_MEDIUM;
+  return MH_TILE_SMALL;
+}
+
 static bool mh_q8_stream_shape(int64_t depth, int64_t xn, int64_t yn) {
   return depth >= 16 && depth <= 64 && depth % 16 == 0 && xn >= 16 && xn <= 128 && xn % 16 == 0 &&
          yn >= 1024;
@@ -2252,6 +2441,61 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
       RequantTable tab;
       if (out_u8 && rq.table) mh_requant_table_cached(ctx, rq, tab.t);
       return launch_gemm_mid(ctx, p, tab, out_u8, (int)batch, true);
+    }
+    // ... and where the 256 x 256 tiles are the choice: the ring kernel's k-major variant; the
+    // operand's sums come from a pass over it as it lies.  Measured against repack + k-contiguous
+    // kernel: 4096^3 86.7 -> 84.6 us, 3000 x 1024 x 4000 52.7 -> 51.6; at 8192^3 the repack's 31 us
+    // are saved but the kernel, at its power limit, pays 22 us for the twice as many LDS read
+    // instructions of the k-major operand (512.7 -> 518 us per call), so from k = 8192 on the
+    // repack stays unless the arena may not grow (no repacked copy is needed here).
+    if (!cv && x_kmajor && y_direct && rhs_ld == 0 && !lhs_w && !rhs_w && depth >= 256 &&
+        (depth < 8192 || ctx->no_alloc || ctx->capturing) &&
+        depth % 128 == 0 && xn % 16 == 0 && (uintptr_t)xp % 16 == 0 &&
+        mh_q8_tile_choice(xn, yn, batch, cu_n) == MH_TILE_BIG &&
+        xn * depth < ((int64_t)1 << 32) && depth < (1 << 24) && (size_t)2 * 512 * 128 <= lds_cu &&
+        !(ctx->kernel_mask & MH_MASK_NO_MID)) {
+      const int x_nb = xl ? lhs_nb : rhs_nb, y_nb = xl ? rhs_nb : lhs_nb;
+      MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, sizeof(int32_t) * ((size_t)x_nb * xn + (size_t)y_nb * yn) + 1024));
+      ArenaScope scope(ctx);
+      int32_t *sum_x = (int32_t *)mh_arena_take(ctx, sizeof(int32_t) * x_nb * xn);
+      int32_t *sum_y_buf = (int32_t *)mh_arena_take(ctx, sizeof(int32_t) * y_nb * yn);
+      if (!sum_x || !sum_y_buf) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
+      GemmParams p{};
+      const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
+      const int32_t l_coef = (int32_t)(0u - zr), r_coef = (int32_t)(0u - zl);
+      const int32_t r_add = (int32_t)((uint32_t)depth * zl * zr);
+      const int32_t *l_bias = out_u8 ? ep.bias : nullptr;
+      p.X = xp;
+      p.Y = yp;
+      p.XN = (int)xn;
+      p.YN = (int)yn;
+      p.K = (int)depth;
+      p.ldx = xn;      // bytes between consecutive k
+      p.ldy = depth;
+      p.xbs = (x_nb > 1) ? xn * depth : 0;
+      p.ybs = (y_nb > 1) ? yn * depth : 0;
+      p.out = out;
+      p.ldo = p.XN;
+      p.obs = rows * cols;
+      p.rq = rq;
+      p.xcoef = xl ? l_coef : r_coef;
+      p.xadd = xl ? 0 : r_add;
+      p.xbias = xl ? l_bias : nullptr;
+      p.ycoef = xl ? r_coef : l_coef;
+      p.yadd = xl ? r_add : 0;
+      p.ybias = xl ? nullptr : l_bias;
+      p.corrX = sum_x;
+      p.corrY = sum_y_buf;
+      p.cxbs = x_nb > 1 ? p.XN : 0;
+      p.cybs = y_nb > 1 ? p.YN : 0;
+      // the Y sums in the kernel where that is cheaper than a pass (see sum_y_shape below)
+      p.sum_y = depth <= 1024 || xn <= 2048;
+      MH_RETURN_IF_ERROR(launch_kmajor_sums(ctx, xp, xn, p.xbs, xn, depth, x_nb, sum_x));
+      if (!p.sum_y)
+        MH_RETURN_IF_ERROR(launch_panel_sums(ctx, yp, depth, p.ybs, yn, (int)depth, y_nb, sum_y_buf));
+      RequantTable tab;
+      if (out_u8 && rq.table) mh_requant_table_cached(ctx, rq, tab.t);
+      return launch_gemm_big_xt(ctx, p, tab, out_u8, (int)batch);
     }
   }
 
@@ -2499,22 +2743,8 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   auto tiles = [&](int tx, int ty) {
     return (int64_t)((p.XN + tx - 1) / tx) * ((p.YN + ty - 1) / ty) * batch;
   };
-  // Tile shape: bigger tiles do more MFMA work per byte moved and per barrier, smaller ones
-  // keep more CUs busy.  Score = relative efficiency of the shape x the fraction of CU slots
-  // its last round of workgroups fills.
-  auto score = [&](int tx, int ty, double weight) {
-    const int64_t t = tiles(tx, ty);
-    const int64_t rounds = (t + cu - 1) / cu;
-    return weight * (double)t / (double)(rounds * cu);
-  };
-  const double s_big = (p.XN > 128 && p.YN > 128) ? score(256, 256, 1.0) : 0.0;
-  const double s_skinny = (p.XN <= 64 && p.YN > 128) ? score(64, 256, 0.6) : 0.0;
-  const double s_medium = (p.XN > 64 && p.YN > 64) ? score(128, 128, 0.6) : 0.0;
-  const double s_small = score(64, 64, 0.3);
-  const double best = std::max(std::max(s_big, s_skinny), std::max(s_medium, s_small));
-  const bool big = s_big == best;
-  const bool skinny = !big && s_skinny == best;
-  const bool medium = !big && !skinny && s_medium == best;
+  const MhTile tile = mh_q8_tile_choice(p.XN, p.YN, batch, cu);
+  const bool big = tile == MH_TILE_BIG, skinny = tile == MH_TILE_SKINNY, medium = tile == MH_TILE_MEDIUM;
   // the streaming kernel needs whole 64-byte slabs and enough of them to fill its ring
   // K = 128 is two slabs: a three-stage ring holds all of it (10 % faster than the
   // register-staged kernel on the 56x56x128 convolution)

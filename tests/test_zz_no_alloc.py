@@ -61,14 +61,19 @@ def test_noalloc_rejects_what_does_not_fit():
     ctx = mh.Context(0)
     try:
         d = Dev()
-        n = 8192   # a RowMajor 8192 x 8192 rhs needs a 64 MiB panel
+        n = 8192   # a ColMajor 8192 x 8192 lhs with a RowMajor result needs a 64 MiB panel
         t, p = d.empty(n * n, np.uint8)
         o, po = d.empty(n * n, np.uint8)
         d.sync()
-        st = ctx.status("mace_hip_gemm_q8_u8_noalloc", p, R, p, R, po, R, 1, n, n, n, 1, 1, -1, -1,
+        st = ctx.status("mace_hip_gemm_q8_u8_noalloc", p, Cm, p, R, po, R, 1, n, n, n, 1, 1, -1, -1,
                         None, 1 << 30, 8, 0, 0, 255)
         assert st == mh.INVALID_ARGS
         assert "scratch" in ctx.last_error()
+        # the same size with the k-major operand on the side the kernels read in place (RowMajor
+        # rhs, RowMajor result) needs the correction vectors only and fits
+        st = ctx.status("mace_hip_gemm_q8_u8_noalloc", p, R, p, R, po, R, 1, n, n, n, 1, 1, -1, -1,
+                        None, 1 << 30, 8, 0, 0, 255)
+        assert st == mh.SUCCESS, ctx.last_error()
         # the context is usable afterwards, by either entry point
         run_pair(ctx, 1, 200, 1100, 300, Cm, R, R, 5, check_oracle=True)
     finally:
