@@ -651,11 +651,15 @@ __global__ __launch_bounds__(1024) void q8_gemv_mfma_slice_kernel(
       const gv4i a = valid ? (av[u] ^ flip) : zero;
       gv4i x = is_x ? (xv[u] ^ flip) : other;
       if (!valid) x = zero;
-      if (is_x) {
-        sx = __builtin_amdgcn_sdot4(x.x, 0x01010101, sx, false);
-        sx = __builtin_amdgcn_sdot4(x.y, 0x01010101, sx, false);
-        sx = __builtin_amdgcn_sdot4(x.z, 0x01010101, sx, false);
-        sx = __builtin_amdgcn_sdot4(x.w, 0x01010101, sx, false);
+      if (is_x && valid) {
+        // the bytes as read, 128 too much each (v_sad_u8: a dot-product instruction would not run
+        // beside the MFMAs)
+        uint32_t t = (uint32_t)sx;
+        t = __builtin_amdgcn_sad_u8((uint32_t)xv[u].x, 0u, t);
+        t = __builtin_amdgcn_sad_u8((uint32_t)xv[u].y, 0u, t);
+        t = __builtin_amdgcn_sad_u8((uint32_t)xv[u].z, 0u, t);
+        t = __builtin_amdgcn_sad_u8((uint32_t)xv[u].w, 0u, t);
+        sx = (int)t - 2048;
       }
       if (u & 1) acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, x, acc1, 0, 0, 0);
       else acc0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, x, acc0, 0, 0, 0);
