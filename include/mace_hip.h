@@ -96,7 +96,8 @@ int mace_hip_graph_destroy(mace_hip_ctx *ctx, mace_hip_graph *graph);
 /* Test hook: switches kernel families off for this context so that the parity tests reach every
  * family on the same shapes (no counterpart in the reference).  Bit 0: the one-launch kernel for
  * small uint8 GEMM / Conv2D calls; bit 1: the kernel that keeps one operand's tile in LDS; bit 2:
- * the kernel for at most one round of 128 x 128 tiles.  0 restores normal dispatch. */
+ * the eight-wavefront 128 x 128 kernel and the in-place reading of k-major operands; bit 3: the
+ * repack that writes a panel already shifted to int8.  0 restores normal dispatch. */
 int mace_hip_ctx_set_kernel_mask(mace_hip_ctx *ctx, int mask);
 /* Test hook, the counterpart of MACE_RUNTIME_FAILURE_RATIO
  * (mace/core/runtime_failure_mock.cc:24-48): the next n arena allocations fail. */

@@ -79,7 +79,7 @@ struct mace_hip_ctx {
   // that the tests reach every family on the same shapes.
   int kernel_mask = 0;
 };
-constexpr int MH_MASK_NO_SMALL = 1, MH_MASK_NO_XRES = 2, MH_MASK_NO_MID = 4;
+constexpr int MH_MASK_NO_SMALL = 1, MH_MASK_NO_XRES = 2, MH_MASK_NO_MID = 4, MH_MASK_NO_XFLIP = 8;
 
 int mh_fail(mace_hip_ctx *ctx, int code, const char *fmt, ...);
 

@@ -704,8 +704,9 @@ __device__ inline void wait_vmcnt() {
 // of consecutive k rows, chunk c of row k to slot c ^ swz(k) of the row, and a fragment is two
 // ds_read_b64_tr_b8 (see q8_gemm_mid_kernel): the swizzle puts the 16 pieces two neighbouring
 // 16-lane groups read into 16 distinct bank groups.
+// XF: the X panel was repacked already shifted to int8; its fragments are not flipped here.
 template <int WX, int WY, int FX, int FY, int STAGES, typename OutT, int OCC = 1,
-          bool SUMY = false, bool CONV = false, int KB = SLAB, bool XT = false>
+          bool SUMY = false, bool CONV = false, int KB = SLAB, bool XT = false, bool XF = false>
 __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParams p, RequantTable) {
   constexpr int NW = WX * WY;
   constexpr int TX = WX * FX * 32;
@@ -874,7 +875,8 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
   };
   auto flip_frags = [&](v4i (&a)[FX], v4i (&bf)[FY]) {
 #pragma unroll
-    for (int i = 0; i < FX; ++i) a[i] ^= flip;
+    for (int i = 0; i < FX; ++i)
+      if (!XF) a[i] ^= flip;
 #pragma unroll
     for (int j = 0; j < FY; ++j) bf[j] ^= flip;
   };
@@ -911,7 +913,7 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
           // issued since this fragment's two reads: two per later X fragment, one per Y fragment
           if (f < FX) lds_wait_tr(na[f], (FX - 1 - f) * 2 + FY);
         }
-        if (f < FX) na[f] ^= flip;
+        if (f < FX) { if (!XF) na[f] ^= flip; }
         else nb[f - FX] ^= flip;
       }
       if constexpr (dma) {
@@ -931,7 +933,7 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
       if (DELAY == 0 || f + DELAY >= NM) {
         if constexpr (SUMY)
           if (f >= FX) ysum[f - FX] = sum16_u8(nb[f - FX], ysum[f - FX]);
-        if (f < FX) na[f] ^= flip;
+        if (f < FX) { if (!XF) na[f] ^= flip; }
         else nb[f - FX] ^= flip;
       }
   };
@@ -1778,7 +1780,10 @@ __device__ inline void transpose4x4_bytes(const uint32_t (&d)[4], uint32_t (&o)[
 __global__ __launch_bounds__(256) void q8_pack_transpose128_kernel(const uint8_t *src,
                                                                    int64_t src_bs, uint8_t *dst,
                                                                    int64_t dst_bs, int n, int k,
-                                                                   int kp, int32_t *sums) {
+                                                                   int kp, int32_t *sums,
+                                                                   uint32_t flip) {
+  // flip = 0x80808080: the panel is written already shifted to int8 (for the kernel variant that
+  // then leaves this operand's fragments alone); 0: as read
   constexpr int PITCH = 130;
   __shared__ uint32_t tile[32 * PITCH];   // [n / 4][k]
   const uint8_t *s = src + (int64_t)blockIdx.z * src_bs;
@@ -1814,7 +1819,8 @@ __global__ __launch_bounds__(256) void q8_pack_transpose128_kernel(const uint8_t
       for (int j = 0; j < 4; ++j) {
         const int gn = n0 + 4 * g + j;
         if (gn < n)
-          *(uint4 *)(d + (int64_t)gn * kp + gk) = uint4{o[0][j], o[1][j], o[2][j], o[3][j]};
+          *(uint4 *)(d + (int64_t)gn * kp + gk) =
+              uint4{o[0][j] ^ flip, o[1][j] ^ flip, o[2][j] ^ flip, o[3][j] ^ flip};
       }
     }
     if (sums) {
@@ -2079,6 +2085,33 @@ int launch_gemm_big_xt(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab
     MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<2, 2, 4, 4, 2, int32_t, 1, true, false, 128, true>));
   } else {
     MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<2, 2, 4, 4, 2, int32_t, 1, false, false, 128, true>));
+  }
+  MH_PROF_END(ctx);
+  MH_HIP(ctx, hipGetLastError());
+  return MACE_HIP_SUCCESS;
+}
+
+// 256 x 256 tiles, X panel repacked already shifted to int8; the caller has checked the preconditions
+int launch_gemm_big_xf(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, bool out_u8,
+                       int batch) {
+  p.tiles_x = (p.XN + 255) / 256;
+  p.tiles_y = (p.YN + 255) / 256;
+  const size_t lds = (size_t)2 * 512 * 128;
+  dim3 grid(p.tiles_x * p.tiles_y, 1, batch), block(256);
+  auto launch = [&](auto k) -> int {
+    MH_HIP(ctx, mh_allow_big_lds(ctx, (const void *)k, lds));
+    MH_PROF_BEGIN(ctx);
+    hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, tab);
+    return MACE_HIP_SUCCESS;
+  };
+  if (out_u8 && p.sum_y) {
+    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<2, 2, 4, 4, 2, uint8_t, 1, true, false, 128, false, true>));
+  } else if (out_u8) {
+    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<2, 2, 4, 4, 2, uint8_t, 1, false, false, 128, false, true>));
+  } else if (p.sum_y) {
+    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<2, 2, 4, 4, 2, int32_t, 1, true, false, 128, false, true>));
+  } else {
+    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<2, 2, 4, 4, 2, int32_t, 1, false, false, 128, false, true>));
   }
   MH_PROF_END(ctx);
   MH_HIP(ctx, hipGetLastError());
@@ -2510,13 +2543,16 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     int64_t ld, bs;
     int k;                  // readable bytes of k per row
     const int32_t *sums;    // cached row sums of a registered weight, or nullptr
+    bool flipped = false;   // repacked already shifted to int8 (X operand of the 256 x 256 kernel)
   } L, R;
 
   // fused_sums: where the repack may leave the panel's row sums as well (or nullptr); *fused
   // tells whether it did
   auto pack = [&](const uint8_t *src, int order_is_kcontig, int nb, int64_t n, uint8_t *dst,
-                  int32_t *fused_sums, bool *fused) -> int {
+                  int32_t *fused_sums, bool *fused, bool want_flipped = false,
+                  bool *flipped = nullptr) -> int {
     if (fused) *fused = false;
+    if (flipped) *flipped = false;
     if (order_is_kcontig) {
       if (depth % 4 == 0 && (uintptr_t)src % 4 == 0) {
         const int64_t total = n * (kp / 16);
@@ -2540,8 +2576,11 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
                              ctx->stream, fused_sums, cnt);
           *fused = true;
         }
+        const bool fl = want_flipped && flipped;
         hipLaunchKernelGGL(q8_pack_transpose128_kernel, grid, dim3(256), 0, ctx->stream, src,
-                           n * depth, dst, n * kp, (int)n, (int)depth, (int)kp, fused_sums);
+                           n * depth, dst, n * kp, (int)n, (int)depth, (int)kp, fused_sums,
+                           fl ? 0x80808080u : 0u);
+        if (fl) *flipped = true;
       } else {
         dim3 grid((unsigned)((n + 63) / 64), (unsigned)(kp / 64), nb);
         hipLaunchKernelGGL(q8_pack_transpose_kernel, grid, dim3(256), 0, ctx->stream, src,
@@ -2587,7 +2626,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   };
 
   auto prepare = [&](const uint8_t *src, int order_is_kcontig, bool direct, int nb, int64_t n,
-                     int64_t ld, mh_weight *w, int32_t *corr, Panel *P) -> int {
+                     int64_t ld, mh_weight *w, int32_t *corr, Panel *P, bool want_flipped = false) -> int {
     if (w) return prepare_weight(w, src, order_is_kcontig, direct, nb, n, P);
     if (direct) {
       // a caller-padded panel (ld > depth) is readable, and zero after the shift, up to ld
@@ -2601,10 +2640,10 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
       *P = Panel{dst, kp, nb > 1 ? n * kp : 0, (int)kp, nullptr};
       return MACE_HIP_SUCCESS;
     }
-    bool fused = false;
-    MH_RETURN_IF_ERROR(pack(src, order_is_kcontig, nb, n, dst, corr, &fused));
+    bool fused = false, flipped = false;
+    MH_RETURN_IF_ERROR(pack(src, order_is_kcontig, nb, n, dst, corr, &fused, want_flipped, &flipped));
     // sums the repack produced count like cached ones: no pass over the panel, none in the kernel
-    *P = Panel{dst, kp, nb > 1 ? n * kp : 0, (int)kp, fused ? corr : nullptr};
+    *P = Panel{dst, kp, nb > 1 ? n * kp : 0, (int)kp, fused ? corr : nullptr, flipped};
     return MACE_HIP_SUCCESS;
   };
   // correction vectors.  zl' = -lhs_offset - 128, zr' = -rhs_offset - 128.
@@ -2628,11 +2667,21 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
                               4 * tiles128_pre >= cu_pre &&
                               (tiles128_pre <= cu_pre || (depth >= 2048 && 2 * tiles128_pre <= 5 * cu_pre)) &&
                               !(ctx->kernel_mask & MH_MASK_NO_MID);
+  // An X operand that is repacked for the 256 x 256 kernel with 128-byte slabs is written already
+  // shifted to int8, which spares that kernel half of its sign flips (8192^3, same box: 505.3 ->
+  // 498.5 us per call).  The test
+  // repeats the dispatch below: a depth too long for the kernel that keeps a panel in LDS, not the
+  // eight-wavefront kernel's range, 256 x 256 tiles chosen, rows within the ring's 32-bit offsets.
+  const bool x_flip = !(ctx->kernel_mask & MH_MASK_NO_XFLIP) && !cv && depth % 128 == 0 && depth >= 1280 && depth < (1 << 24) && !sums_in_kernel &&
+                      mh_q8_tile_choice(x_is_lhs ? rows : cols, x_is_lhs ? cols : rows, batch, cu_pre) ==
+                          MH_TILE_BIG;
   MH_RETURN_IF_ERROR(prepare(lhs, lhs_order == MACE_HIP_ROW_MAJOR, lhs_direct, lhs_nb, rows, depth,
-                             lhs_w, ((!x_is_lhs && sum_y_shape) || sums_in_kernel) ? nullptr : corrL, &L));
+                             lhs_w, ((!x_is_lhs && sum_y_shape) || sums_in_kernel) ? nullptr : corrL, &L,
+                             x_flip && x_is_lhs));
   MH_RETURN_IF_ERROR(prepare(rhs, rhs_order == MACE_HIP_COL_MAJOR, rhs_direct, rhs_nb, cols,
                              rhs_ld != 0 ? rhs_ld : depth, rhs_w,
-                             ((x_is_lhs && sum_y_shape) || sums_in_kernel) ? nullptr : corrR, &R));
+                             ((x_is_lhs && sum_y_shape) || sums_in_kernel) ? nullptr : corrR, &R,
+                             x_flip && !x_is_lhs));
   const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
   const bool sum_y = cv || (sum_y_shape && !(x_is_lhs ? R.sums : L.sums));   // cached sums cost nothing
   const int32_t l_coef = (int32_t)(0u - zr), l_add = 0;
@@ -2690,6 +2739,9 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   GemmParams p;
   const Panel &PX = x_is_lhs ? L : R;
   const Panel &PY = x_is_lhs ? R : L;
+  // a panel written already shifted to int8 has exactly one consumer (see x_flip above)
+  MH_CHECK(ctx, !PY.flipped && (!PX.flipped || (!xres && !stream && !mid)),
+           "internal: shifted panel outside the 256 x 256 kernel");
   p.X = PX.ptr; p.ldx = PX.ld; p.xbs = PX.bs;
   p.Y = PY.ptr; p.ldy = PY.ld; p.ybs = PY.bs;
   p.XN = (int)(x_is_lhs ? rows : cols);
@@ -2757,6 +2809,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   // 128-byte slabs (whole cache lines per row) where they measure faster: the 256 x 256 tile
   // (+5 % at 8192^3) and long-k 128 x 128 tiles; short k gains nothing from them
   if (p.K % 128 == 0 && p.K >= 256 && !p.conv && dma_ok) {
+    if (big && PX.flipped) return launch_gemm_big_xf(ctx, p, tab, out_u8, (int)batch);
     if (big) return launch_gemm_dma<2, 2, 4, 4, 2, 1, 128>(ctx, p, tab, out_u8, (int)batch);
     // Between half a round and one round of 128 x 128 tiles every CU has one workgroup and every
     // SIMD one wavefront, with nothing to overlap its waits: eight wavefronts of 64 x 32 results
@@ -2766,6 +2819,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     if (medium && p.K >= 1024)
       return launch_gemm_dma<2, 2, 2, 2, 2, 2, 128>(ctx, p, tab, out_u8, (int)batch);
   }
+  MH_CHECK(ctx, !PX.flipped, "internal: shifted panel outside the 256 x 256 kernel");
   if (p.K % SLAB == 0 && p.K >= SLAB * 3 && dma_ok) {
     if (big) return launch_gemm_dma<2, 2, 4, 4, 4, 1>(ctx, p, tab, out_u8, (int)batch);
     if (skinny) return launch_gemm_dma<1, 4, 2, 2, 4, 2>(ctx, p, tab, out_u8, (int)batch);

@@ -13,7 +13,7 @@ SUCCESS, INVALID_ARGS, OUT_OF_RESOURCES, UNSUPPORTED, RUNTIME_ERROR = range(5)
 ROW_MAJOR, COL_MAJOR = 0, 1
 REQUANT_REF, REQUANT_NEON = 0, 1
 ACT_NOOP, ACT_RELU, ACT_RELUX = 0, 1, 2
-MASK_NO_SMALL, MASK_NO_XRES, MASK_NO_MID = 1, 2, 4
+MASK_NO_SMALL, MASK_NO_XRES, MASK_NO_MID, MASK_NO_XFLIP = 1, 2, 4, 8
 NOALLOC_SCRATCH_BYTES = 32 << 20
 
 _STATUS_NAMES = {0: "MACE_SUCCESS", 1: "MACE_INVALID_ARGS", 2: "MACE_OUT_OF_RESOURCES",

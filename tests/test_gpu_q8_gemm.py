@@ -143,6 +143,8 @@ MID_SHAPES = [  # batch, rows, depth, cols, lhs batched, rhs batched, lhs order,
     # and from a pass of their own, ragged last tiles, ColMajor everything
     (1, 3000, 256, 4000, True, True, R, R, R), (1, 4000, 384, 3024, True, True, Cm, Cm, Cm),
     (1, 2900, 1152, 4112, True, True, R, R, R),
+    # long enough k that the repacked panel of the tiled path is written already shifted to int8
+    (1, 2900, 1280, 4112, True, True, R, R, R),
 ]
 
 
