@@ -24,6 +24,7 @@ struct mh_weight_panel {
   int64_t ld;
   int k;
   int32_t *sums;        // [nb][n], device memory owned by the cache
+  bool flipped;         // the panel holds the bytes already shifted to int8 (one consumer only)
 };
 struct mh_weight {
   const void *ptr;

@@ -2593,41 +2593,50 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
 
   // a registered weight: reuse (or build once, in memory of its own) its panel and row sums
   auto prepare_weight = [&](mh_weight *w, const uint8_t *src, int order_is_kcontig, bool direct,
-                            int nb, int64_t n, Panel *P) -> int {
+                            int nb, int64_t n, Panel *P, bool want_flipped) -> int {
+    // a panel written already shifted serves only the caller that asked for one; a plain one anybody
+    const mh_weight_panel *hit = nullptr;
     for (const mh_weight_panel &c : w->panels)
-      if (c.kcontig == order_is_kcontig && c.n == n && c.depth == depth && c.nb == nb) {
-        *P = Panel{c.panel ? c.panel : src, c.ld, nb > 1 ? n * c.ld : 0, c.k, c.sums};
-        ++ctx->weight_hits;
-        return MACE_HIP_SUCCESS;
-      }
+      if (c.kcontig == order_is_kcontig && c.n == n && c.depth == depth && c.nb == nb &&
+          (c.flipped ? want_flipped : !hit))
+        hit = &c;
+    if (hit) {
+      *P = Panel{hit->panel ? hit->panel : src, hit->ld, nb > 1 ? n * hit->ld : 0, hit->k, hit->sums,
+                 hit->flipped};
+      ++ctx->weight_hits;
+      return MACE_HIP_SUCCESS;
+    }
     mh_weight_panel c{order_is_kcontig, n, depth, nb, nullptr, direct ? depth : kp,
-                      (int)(direct ? depth : kp), nullptr};
+                      (int)(direct ? depth : kp), nullptr, false};
+    MH_HIP(ctx, hipMalloc((void **)&c.sums, sizeof(int32_t) * (size_t)nb * n));
+    bool fused = false;
     if (!direct) {
-      MH_HIP(ctx, hipMalloc((void **)&c.panel, (size_t)nb * n * kp));
-      const int rc = pack(src, order_is_kcontig, nb, n, c.panel, nullptr, nullptr);
-      if (rc != MACE_HIP_SUCCESS) { (void)hipFree(c.panel); return rc; }
+      hipError_t e = hipMalloc((void **)&c.panel, (size_t)nb * n * kp);
+      if (e != hipSuccess) { (void)hipFree(c.sums); MH_HIP(ctx, e); }
+      // the sums come from the repack where it can take them (always where it shifts the bytes)
+      const int rc = pack(src, order_is_kcontig, nb, n, c.panel, want_flipped ? c.sums : nullptr, &fused,
+                          want_flipped, &c.flipped);
+      if (rc != MACE_HIP_SUCCESS) { (void)hipFree(c.panel); (void)hipFree(c.sums); return rc; }
     }
-    hipError_t e = hipMalloc((void **)&c.sums, sizeof(int32_t) * (size_t)nb * n);
-    if (e != hipSuccess) {
-      if (c.panel) (void)hipFree(c.panel);
-      MH_HIP(ctx, e);
-    }
-    const int rc = launch_panel_sums(ctx, c.panel ? c.panel : src, c.ld, nb > 1 ? n * c.ld : 0, n,
-                                     c.k, nb, c.sums);
-    if (rc != MACE_HIP_SUCCESS) {
-      if (c.panel) (void)hipFree(c.panel);
-      (void)hipFree(c.sums);
-      return rc;
+    if (!fused) {
+      const int rc = c.flipped ? MACE_HIP_RUNTIME_ERROR
+                               : launch_panel_sums(ctx, c.panel ? c.panel : src, c.ld,
+                                                   nb > 1 ? n * c.ld : 0, n, c.k, nb, c.sums);
+      if (rc != MACE_HIP_SUCCESS) {
+        if (c.panel) (void)hipFree(c.panel);
+        (void)hipFree(c.sums);
+        return rc;
+      }
     }
     w->panels.push_back(c);
     ++ctx->weight_builds;
-    *P = Panel{c.panel ? c.panel : src, c.ld, nb > 1 ? n * c.ld : 0, c.k, c.sums};
+    *P = Panel{c.panel ? c.panel : src, c.ld, nb > 1 ? n * c.ld : 0, c.k, c.sums, c.flipped};
     return MACE_HIP_SUCCESS;
   };
 
   auto prepare = [&](const uint8_t *src, int order_is_kcontig, bool direct, int nb, int64_t n,
                      int64_t ld, mh_weight *w, int32_t *corr, Panel *P, bool want_flipped = false) -> int {
-    if (w) return prepare_weight(w, src, order_is_kcontig, direct, nb, n, P);
+    if (w) return prepare_weight(w, src, order_is_kcontig, direct, nb, n, P, want_flipped);
     if (direct) {
       // a caller-padded panel (ld > depth) is readable, and zero after the shift, up to ld
       *P = Panel{src, ld, nb > 1 ? n * ld : 0, (int)ld, nullptr};

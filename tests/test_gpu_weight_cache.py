@@ -47,6 +47,8 @@ def gemm_dev(ctx, torch, dl, lo, dr, ro, oo, batch, rows, depth, cols, lb, rb, l
     (128, 256, 4000, R, Cm, Cm, "lhs"),   # conv-like: the filter is the weight
     (64, 64, 2048, R, Cm, Cm, "lhs"),     # streaming-kernel shape
     (130, 300, 70, Cm, R, R, "lhs"),
+    # 256 x 256 tiles and a long k: the cached panel is written already shifted to int8
+    (2900, 1280, 4112, R, R, R, "rhs"),
 ])
 def test_cached_weight_matches_uncached_and_oracle(ctx, rows, depth, cols, lo, ro, oo, weight_side):
     import torch
