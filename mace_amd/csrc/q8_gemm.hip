@@ -705,9 +705,13 @@ __device__ inline void wait_vmcnt() {
 // ds_read_b64_tr_b8 (see q8_gemm_mid_kernel): the swizzle puts the 16 pieces two neighbouring
 // 16-lane groups read into 16 distinct bank groups.
 // XF: the X panel was repacked already shifted to int8; its fragments are not flipped here.
+// SUMX: the X panel's sums are taken here too (like SUMY, from the fragments as read), so that no
+// pass over that operand is launched.
 template <int WX, int WY, int FX, int FY, int STAGES, typename OutT, int OCC = 1,
-          bool SUMY = false, bool CONV = false, int KB = SLAB, bool XT = false, bool XF = false>
+          bool SUMY = false, bool CONV = false, int KB = SLAB, bool XT = false, bool XF = false,
+          bool SUMX = false>
 __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParams p, RequantTable) {
+  static_assert(!SUMX || !XF, "a panel written already shifted comes with its sums");
   constexpr int NW = WX * WY;
   constexpr int TX = WX * FX * 32;
   constexpr int TY = WY * FY * 32;
@@ -826,6 +830,9 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
   int ysum[FY];
 #pragma unroll
   for (int j = 0; j < FY; ++j) ysum[j] = 0;
+  int xsum[SUMX ? FX : 1];
+#pragma unroll
+  for (int i = 0; i < (SUMX ? FX : 1); ++i) xsum[i] = 0;
 
   // fragment addresses: lane l reads row (l % 32) of a 32-row block, chunk 2*ks + l/32.
   // Block bases are multiples of 32 rows, so the swizzle depends on l only.
@@ -913,8 +920,12 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
           // issued since this fragment's two reads: two per later X fragment, one per Y fragment
           if (f < FX) lds_wait_tr(na[f], (FX - 1 - f) * 2 + FY);
         }
-        if (f < FX) { if (!XF) na[f] ^= flip; }
-        else nb[f - FX] ^= flip;
+        if (f < FX) {
+          if constexpr (SUMX) xsum[f] = sum16_u8(na[f], xsum[f]);
+          if (!XF) na[f] ^= flip;
+        } else {
+          nb[f - FX] ^= flip;
+        }
       }
       if constexpr (dma) {
         // LX + LY transfers spread over the slots from slot 0 on
@@ -933,8 +944,12 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
       if (DELAY == 0 || f + DELAY >= NM) {
         if constexpr (SUMY)
           if (f >= FX) ysum[f - FX] = sum16_u8(nb[f - FX], ysum[f - FX]);
-        if (f < FX) { if (!XF) na[f] ^= flip; }
-        else nb[f - FX] ^= flip;
+        if (f < FX) {
+          if constexpr (SUMX) xsum[f] = sum16_u8(na[f], xsum[f]);
+          if (!XF) na[f] ^= flip;
+        } else {
+          nb[f - FX] ^= flip;
+        }
       }
   };
 
@@ -951,6 +966,10 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
   if constexpr (SUMY) {
 #pragma unroll
     for (int j = 0; j < FY; ++j) ysum[j] = sum16_u8(b0[j], ysum[j]);
+  }
+  if constexpr (SUMX) {
+#pragma unroll
+    for (int i = 0; i < FX; ++i) xsum[i] = sum16_u8(a0[i], xsum[i]);
   }
   flip_frags(a0, b0);
   int stage = 0;
@@ -988,7 +1007,40 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
     for (int j = 0; j < FY; ++j) ysum[j] -= sum16_u8(b0[j] ^ flip, 0) + 64 * p.K;
   }
 
-  gemm_epilogue<WX, WY, FX, FY, OutT, SUMY>(acc, ysum, p, lds, b, x0, y0, wx, wy, tid);
+  if constexpr (SUMX) {
+    // x terms from the sums taken here (both wavefront rows hold them; wy == 0 writes), y terms and
+    // the comparison table staged as the epilogue would, then the epilogue on what is in LDS
+#pragma unroll
+    for (int i = 0; i < FX; ++i) xsum[i] -= sum16_u8(a0[i] ^ flip, 0) + 64 * p.K;
+    __syncthreads();   // every wavefront is done reading operand tiles, every transfer has landed
+    int32_t *sc = (int32_t *)lds;
+#pragma unroll
+    for (int i = 0; i < FX; ++i) {
+      const int total = xsum[i] + __shfl_xor(xsum[i], 32, 64);
+      if (wy == 0 && lane < 32) {
+        const int xl = (wx * FX + i) * 32 + lane;
+        uint32_t c = (uint32_t)p.xcoef * (uint32_t)total + (uint32_t)p.xadd;
+        if (p.xbias) c += (uint32_t)p.xbias[min(x0 + xl, p.XN - 1)];
+        sc[xl] = (int32_t)c;
+      }
+    }
+    if constexpr (!SUMY) {
+      const int32_t *cY = p.corrY + (int64_t)b * p.cybs;
+      for (int i = tid; i < TY; i += NW * 64) {
+        const int y = min(y0 + i, p.YN - 1);
+        uint32_t c = (uint32_t)p.ycoef * (uint32_t)cY[y] + (uint32_t)p.yadd;
+        if (p.ybias) c += (uint32_t)p.ybias[y];
+        sc[TX + i] = (int32_t)c;
+      }
+    }
+    if constexpr (sizeof(OutT) == 1) {
+      if (p.rq.table) stage_requant_pairs(sc + TX + TY, p.rq, tid, NW * 64);
+    }
+    __syncthreads();
+    gemm_epilogue<WX, WY, FX, FY, OutT, SUMY, true>(acc, ysum, p, lds, b, x0, y0, wx, wy, tid);
+  } else {
+    gemm_epilogue<WX, WY, FX, FY, OutT, SUMY>(acc, ysum, p, lds, b, x0, y0, wx, wy, tid);
+  }
 }
 
 // ---- one round of 128 x 128 tiles ------------------------------------------------------------
@@ -2066,7 +2118,7 @@ int launch_gemm_mid(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, b
 
 // 256 x 256 tiles, X operand k-major in memory; the caller has checked the preconditions
 int launch_gemm_big_xt(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, bool out_u8,
-                       int batch) {
+                       int batch, bool sum_x) {
   p.tiles_x = (p.XN + 255) / 256;
   p.tiles_y = (p.YN + 255) / 256;
   const size_t lds = (size_t)2 * 512 * 128;
@@ -2077,15 +2129,20 @@ int launch_gemm_big_xt(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab
     hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, tab);
     return MACE_HIP_SUCCESS;
   };
-  if (out_u8 && p.sum_y) {
-    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<2, 2, 4, 4, 2, uint8_t, 1, true, false, 128, true>));
-  } else if (out_u8) {
-    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<2, 2, 4, 4, 2, uint8_t, 1, false, false, 128, true>));
-  } else if (p.sum_y) {
-    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<2, 2, 4, 4, 2, int32_t, 1, true, false, 128, true>));
+#define MH_XT(OUT_, SY_, SX_) \
+  MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<2, 2, 4, 4, 2, OUT_, 1, SY_, false, 128, true, false, SX_>))
+  if (out_u8) {
+    if (p.sum_y && sum_x) MH_XT(uint8_t, true, true);
+    else if (p.sum_y) MH_XT(uint8_t, true, false);
+    else if (sum_x) MH_XT(uint8_t, false, true);
+    else MH_XT(uint8_t, false, false);
   } else {
-    MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<2, 2, 4, 4, 2, int32_t, 1, false, false, 128, true>));
+    if (p.sum_y && sum_x) MH_XT(int32_t, true, true);
+    else if (p.sum_y) MH_XT(int32_t, true, false);
+    else if (sum_x) MH_XT(int32_t, false, true);
+    else MH_XT(int32_t, false, false);
   }
+#undef MH_XT
   MH_PROF_END(ctx);
   MH_HIP(ctx, hipGetLastError());
   return MACE_HIP_SUCCESS;
@@ -2521,14 +2578,18 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
       p.corrY = sum_y_buf;
       p.cxbs = x_nb > 1 ? p.XN : 0;
       p.cybs = y_nb > 1 ? p.YN : 0;
-      // the Y sums in the kernel where that is cheaper than a pass (see sum_y_shape below)
-      p.sum_y = depth <= 1024 || xn <= 2048;
-      MH_RETURN_IF_ERROR(launch_kmajor_sums(ctx, xp, xn, p.xbs, xn, depth, x_nb, sum_x));
+      // Either operand's sums in the kernel where that is cheaper than a pass: the kernel pays
+      // about 3.6 % of its time per operand (8192^3: +17 us), a pass its launch plus the operand's
+      // bytes at 6 TB/s, so the kernel wins while the other dimension is at most about 4096.
+      p.sum_y = depth <= 1024 || xn <= 4096;
+      const bool sum_x_in_kernel = depth <= 1024 || yn <= 4096;
+      if (!sum_x_in_kernel)
+        MH_RETURN_IF_ERROR(launch_kmajor_sums(ctx, xp, xn, p.xbs, xn, depth, x_nb, sum_x));
       if (!p.sum_y)
         MH_RETURN_IF_ERROR(launch_panel_sums(ctx, yp, depth, p.ybs, yn, (int)depth, y_nb, sum_y_buf));
       RequantTable tab;
       if (out_u8 && rq.table) mh_requant_table_cached(ctx, rq, tab.t);
-      return launch_gemm_big_xt(ctx, p, tab, out_u8, (int)batch);
+      return launch_gemm_big_xt(ctx, p, tab, out_u8, (int)batch, sum_x_in_kernel);
     }
   }
 
@@ -2663,9 +2724,9 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   const bool x_is_lhs = out_order == MACE_HIP_COL_MAJOR;
   // The Y operand's row sums can be taken inside the GEMM kernel from the fragments it already
   // holds, which saves one pass over that operand.  The pass costs YN * K bytes of HBM traffic,
-  // the in-kernel sums about 7 % of the GEMM's own time (measured at 8192^3: +37 us against an
-  // 11 us pass), i.e. the ratio grows with XN only: in-kernel wins below XN of about 2500.
-  const bool sum_y_shape = cv || (depth > 0 && (depth <= 1024 || (x_is_lhs ? rows : cols) <= 2048));
+  // the in-kernel sums about 3.6 % of the GEMM's own time (measured at 8192^3: +17 us against an
+  // 11 us pass), i.e. the ratio grows with XN only: in-kernel wins up to XN of about 4096.
+  const bool sum_y_shape = cv || (depth > 0 && (depth <= 1024 || (x_is_lhs ? rows : cols) <= 4096));
   // A transposing repack can add up its rows on the way; worth its extra (zeroing) launch only
   // where it replaces a pass, i.e. not for a Y operand whose sums the GEMM kernel takes anyway.
   // ... nor where the call will go to the kernel that sums both panels itself (the shape test of

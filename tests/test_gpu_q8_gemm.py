@@ -139,10 +139,11 @@ MID_SHAPES = [  # batch, rows, depth, cols, lhs batched, rhs batched, lhs order,
     (1, 1536, 1024, 1488, True, True, R, R, R), (2, 1000, 640, 1040, True, True, R, R, R),
     (1, 1296, 1280, 1500, True, True, Cm, Cm, Cm), (2, 1100, 512, 1200, True, False, R, R, R),
     (1, 2048, 2048, 2048, True, True, R, R, R),
-    # the same operand layout at sizes that take 256 x 256 tiles: Y sums in the kernel (k <= 1024)
-    # and from a pass of their own, ragged last tiles, ColMajor everything
+    # the same operand layout at sizes that take 256 x 256 tiles: each operand's sums in the kernel
+    # (k <= 1024 or the other dimension <= 4096) or from a pass of their own, ragged last tiles,
+    # ColMajor everything
     (1, 3000, 256, 4000, True, True, R, R, R), (1, 4000, 384, 3024, True, True, Cm, Cm, Cm),
-    (1, 2900, 1152, 4112, True, True, R, R, R),
+    (1, 2900, 1152, 4112, True, True, R, R, R), (1, 4200, 1152, 2048, True, True, R, R, R),
     # long enough k that the repacked panel of the tiled path is written already shifted to int8
     (1, 2900, 1280, 4112, True, True, R, R, R),
 ]
