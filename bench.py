@@ -191,7 +191,7 @@ def main():
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_INT8_TOPS,
                      "unit": "TOP/s", "frac": round(achieved / PEAK_INT8_TOPS, 4),
                      "traffic": measured_traffic("q8_gemm_%d" % n), "traffic_unit": "B/launch",
-                     "kernel": "q8_gemm_dma_kernel<2,2,4,4,2,uint8_t,1,false,false,128,false>",
+                     "kernel": "q8_gemm_dma_kernel<2,2,4,4,2,uint8_t,1,false,false,128,false,true,false>",
                      "kernel_ms_avg": round(k_avg, 4), "kernel_ms_min": round(min(kms), 4),
                      "kernel_ms_max": round(max(kms), 4),
                      "timing": "one HIP event pair per launch, recorded inside the timed region",
