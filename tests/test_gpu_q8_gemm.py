@@ -475,3 +475,55 @@ def test_q8_gemm_random_mid_sizes(ctx, batch, rows, depth, cols, lo, ro, oo, see
     got8 = gemm_u8_host(ctx, l, lo, r, ro, oo, batch, rows, depth, cols, True, True, -lzp, -rzp, bias,
                         mult, shift, 128)
     np.testing.assert_array_equal(got8, want8)
+
+
+def _random_large_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        rows, cols = int(rng.integers(32, 289)) * 16, int(rng.integers(32, 289)) * 16
+        depth = int(rng.choice([512, 640, 1024, 1280, 2048, 2176, 4096]))
+        batch = int(rng.integers(1, 3))
+        if batch * rows * cols * depth > 3e10:
+            continue
+        cases.append((batch, rows, depth, cols, int(rng.integers(0, 2)), int(rng.integers(0, 2)),
+                      int(rng.integers(0, 2)), bool(rng.integers(0, 2)), int(rng.integers(0, 1 << 30))))
+    return cases
+
+
+@pytest.mark.parametrize("batch,rows,depth,cols,lo,ro,oo,rb,seed", _random_large_cases(28, 777))
+def test_q8_gemm_kernel_families_agree_on_large_shapes(ctx, batch, rows, depth, cols, lo, ro, oo, rb, seed):
+    """Seeded random shapes of 512 to 4608 rows and columns (multiples of 16, so that a k-major
+    operand can be read in place) on device buffers: normal dispatch (eight-wavefront 128 x 128
+    kernel, 256 x 256 kernel with a k-major or pre-shifted X panel, in-kernel sums) against the
+    general path that the smaller cases pin to the oracle (repack, sum passes, plain tiled kernels),
+    int32 and uint8 results bit for bit."""
+    import torch
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    nl = batch * rows * depth
+    nr = (batch if rb else 1) * depth * cols
+    dl = torch.randint(0, 256, (nl,), dtype=torch.uint8, device="cuda", generator=g)
+    dr = torch.randint(0, 256, (nr,), dtype=torch.uint8, device="cuda", generator=g)
+    bias = torch.randint(-2 ** 15, 2 ** 15, (rows,), dtype=torch.int32, device="cuda", generator=g)
+    mult, shift = scales_for(depth)
+    lzp, rzp = 100 + seed % 56, 100 + (seed >> 8) % 56
+    res = {}
+    for name, mask in (("normal", 0),
+                       ("general", mh.MASK_NO_SMALL | mh.MASK_NO_XRES | mh.MASK_NO_MID | mh.MASK_NO_XFLIP)):
+        ctx.call("mace_hip_ctx_set_kernel_mask", mask)
+        try:
+            o8 = torch.zeros(batch * rows * cols, dtype=torch.uint8, device="cuda")
+            o32 = torch.zeros(batch * rows * cols, dtype=torch.int32, device="cuda")
+            torch.cuda.synchronize()
+            ctx.call("mace_hip_gemm_q8_u8", dl.data_ptr(), lo, dr.data_ptr(), ro, o8.data_ptr(), oo, batch,
+                     rows, depth, cols, 1, int(rb), -lzp, -rzp, bias.data_ptr(), mult, shift, 128, 0, 255)
+            ctx.call("mace_hip_gemm_q8_i32", dl.data_ptr(), lo, dr.data_ptr(), ro, o32.data_ptr(), oo,
+                     batch, rows, depth, cols, 1, int(rb), -lzp, -rzp)
+            ctx.sync()
+            res[name] = (o8, o32)
+        finally:
+            ctx.call("mace_hip_ctx_set_kernel_mask", 0)
+    assert bool((res["normal"][1] == res["general"][1]).all())
+    assert bool((res["normal"][0] == res["general"][0]).all())
+    assert int(res["normal"][0].max()) - int(res["normal"][0].min()) > 64   # not saturated away
+
