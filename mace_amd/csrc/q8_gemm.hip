@@ -2496,12 +2496,16 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     }
     // The same operand layout with a longer k, in the tile-count range of the eight-wavefront
     // 128 x 128 kernel (see below): its transposing LDS reads take the operand as it lies, so the
-    // repack (2048^3: zeroing 2.4 + repack 7.5 us of a 22 us call) is not launched.
+    // repack (2048^3: zeroing 2.4 + repack 7.5 us of a 22 us call) is not launched.  Because of that
+    // saving the range is wider here: two rounds of tiles from k = 1024 on (8 x 1024^3 25.7 -> 23.4 us,
+    // 32 x 512 x 1024 x 512 30.1 -> 24.8; 3072 x 1024 x 3072, 576 tiles, loses 5 % and is left out).
     const int64_t tiles128 = ((xn + 127) / 128) * ((yn + 127) / 128) * batch;
     const int64_t cu_n = ctx->cu_count > 0 ? ctx->cu_count : 256;
     if (!cv && x_kmajor && y_direct && rhs_ld == 0 && !lhs_w && !rhs_w && depth >= 512 &&
         depth % 128 == 0 && xn % 16 == 0 && (uintptr_t)xp % 16 == 0 && xn > 64 && yn > 64 &&
-        4 * tiles128 >= cu_n && (tiles128 <= cu_n || (depth >= 2048 && 2 * tiles128 <= 5 * cu_n)) &&
+        4 * tiles128 >= cu_n &&
+        (tiles128 <= cu_n || (depth >= 2048 && 2 * tiles128 <= 5 * cu_n) ||
+         (depth >= 1024 && tiles128 <= 2 * cu_n)) &&
         xn * depth < ((int64_t)1 << 32) && depth < (1 << 24) && (size_t)4 * 256 * 128 <= lds_cu &&
         !(ctx->kernel_mask & MH_MASK_NO_MID)) {
       GemmParams p{};
