@@ -1386,8 +1386,18 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int h = lane >> 5, r32 = lane & 31;
-  const int x0 = blockIdx.y * TX;
-  const int b = blockIdx.z;
+  // Consecutive workgroup ids go round-robin to the 8 XCDs: every XCD gets a contiguous span of
+  // the sequence (batch, share of the Y blocks, X tile), X tile fastest, so that the workgroups
+  // that read the same Y rows, and a batch's workgroups, share an L2
+  // (32 x 512^3: 18.8 -> 16.2 us).
+  int wg = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+  {
+    const int nwg = gridDim.x * gridDim.y * gridDim.z;
+    if (nwg % 8 == 0) wg = (wg % 8) * (nwg / 8) + wg / 8;
+  }
+  const int wg_y = (wg / gridDim.y) % gridDim.x;   // share of the Y blocks
+  const int x0 = (wg % gridDim.y) * TX;
+  const int b = wg / (gridDim.y * gridDim.x);
   const uint8_t *Xb = p.X + (int64_t)b * p.xbs;
   const uint8_t *Yb = p.Y + (int64_t)b * p.ybs;
   const RequantFixed rq = p.rq;
@@ -1396,7 +1406,7 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
   const int nblk = (p.YN + TYW - 1) / TYW;
   const int ngroup = p.K / G;
   const int stride = gridDim.x * 4;
-  int blk = blockIdx.x * 4 + wave;
+  int blk = wg_y * 4 + wave;
   // What a lane needs to address its row of a block.  Plain: the row's first byte (+ the lane's
   // half).  CONV: the image base (+ the lane's half) and the top-left input position of the
   // pixel's patch.  Rows past the end are clamped to the last one: always readable, never stored.
@@ -2378,6 +2388,35 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   mh_weight *lhs_w = find_weight(lhs, (size_t)lhs_nb * rows * depth);
   mh_weight *rhs_w = (rhs_ld != 0 || cv) ? nullptr : find_weight(rhs, (size_t)rhs_nb * cols * depth);
 
+  // At most one round of 128 x 128 tiles (and at least a quarter of one) with k >= 512: the
+  // eight-wavefront kernel (q8_gemm_mid_kernel) is one launch as well and goes first where it
+  // measured faster than the kernels below (8 buffer sets in rotation, us per call):
+  //   X k-major, against the one-launch kernel: 4 x 512^3 8.4 -> 8.0, 8 x 512^3 11.6 -> 8.4,
+  //     1024^3 12.8 -> 9.6, 4 x 512 x 1024 x 512 13.1 -> 9.4, 1024 x 768 x 1024 10.6 -> 8.8;
+  //   X k-major, against the kernel with the X tile resident in LDS: 16 x 512^3 12.7 -> 10.2,
+  //     2048 x 512 x 2048 12.7 -> 8.5, 1536 x 512 x 1536 12.0 -> 8.2;
+  //   k-contiguous operands, against the resident-tile kernel (which leaves most CUs idle at these
+  //     sizes): 16 x 512^3 11.3 -> 9.9, 2048 x 512 x 2048 11.2 -> 8.3, 8 x 512^3 14.6 -> 8.7;
+  //   k-contiguous operands, against the one-launch kernel: ties or loses at k = 512 (4 x 512^3
+  //     6.8 against 8.1) and wins from k = 1024 on (1024^3 9.7 -> 9.2, 4 x 512 x 1024 x 512 9.7 -> 9.0).
+  const bool mid_xl = out_order == MACE_HIP_COL_MAJOR;
+  const int64_t mid_xn = mid_xl ? rows : cols, mid_yn = mid_xl ? cols : rows;
+  const int64_t mid_tiles = ((mid_xn + 127) / 128) * ((mid_yn + 127) / 128) * batch;
+  const int64_t mid_cu = ctx->cu_count > 0 ? ctx->cu_count : 256;
+  const bool mid_one_round =
+      !cv && !lhs_w && !rhs_w && rhs_ld == 0 && depth >= 512 && depth % 128 == 0 &&
+      depth < (1 << 24) && mid_xn > 64 && mid_yn > 64 && 4 * mid_tiles >= mid_cu &&
+      mid_tiles <= mid_cu &&
+      (size_t)4 * 256 * 128 <= (ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536) &&
+      !(ctx->kernel_mask & MH_MASK_NO_MID);
+  const bool mid_y_direct = mid_xl ? (rhs_direct && rhs_order == MACE_HIP_COL_MAJOR) : lhs_direct;
+  const bool mid_x_direct = mid_xl ? lhs_direct : (rhs_direct && rhs_order == MACE_HIP_COL_MAJOR);
+  const bool mid_x_kmajor = mid_xl ? lhs_order == MACE_HIP_COL_MAJOR : rhs_order == MACE_HIP_ROW_MAJOR;
+  const bool mid_first_xt = mid_one_round && mid_x_kmajor && mid_y_direct && mid_xn % 16 == 0 &&
+                            (uintptr_t)(mid_xl ? lhs : rhs) % 16 == 0 &&
+                            mid_xn * depth < ((int64_t)1 << 32);
+  const bool mid_first_kc = mid_one_round && mid_x_direct && mid_y_direct && depth >= 1024;
+
   // Small problems: one launch that reads both operands where they lie (k-contiguous, or k-major
   // and transposed on the way into LDS) and takes both correction vectors itself.
   {
@@ -2403,7 +2442,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     const bool small = cv ? cv_small
                           : (mh_q8_small_problem(ctx, batch, rows, cols, depth, lhs_vec && rhs_vec,
                                                  any_size) &&
-                             ((!lhs_w && !rhs_w) || any_size) &&
+                             ((!lhs_w && !rhs_w) || any_size) && !mid_first_xt && !mid_first_kc &&
                              !(ctx->kernel_mask & MH_MASK_NO_SMALL));
     if (small) {
       GemmParams p{};
@@ -2464,7 +2503,8 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     const size_t lds_cu = ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536;
     if (!cv && x_kmajor && y_direct && rhs_ld == 0 && !lhs_w && !rhs_w && depth > 0 &&
         depth % 64 == 0 && xn % 16 == 0 && (uintptr_t)xp % 16 == 0 && yn >= 256 &&
-        2 * (XRES_SC_BYTES + (size_t)tx * depth) <= lds_cu && !(ctx->kernel_mask & MH_MASK_NO_XRES)) {
+        2 * (XRES_SC_BYTES + (size_t)tx * depth) <= lds_cu && !mid_first_xt &&
+        !(ctx->kernel_mask & MH_MASK_NO_XRES)) {
       GemmParams p{};
       const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
       const int32_t l_coef = (int32_t)(0u - zr), r_coef = (int32_t)(0u - zl);
@@ -2788,8 +2828,14 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   const bool xres_narrow = !cv && !xres_fits(128) && blocks_tx64 > cu_n && blocks_tx64 <= 2 * cu_n;
   const int xres_tx = (xn <= 64 || xres_narrow) ? 64 : 128;
   const bool xres_cv = cv && !cv_small && out_u8 && cv->cin % 64 == 0 && depth % 64 == 0;
+  const int64_t tiles128 = ((xn + 127) / 128) * ((yn + 127) / 128) * batch;
+  // (one round of 128 x 128 tiles at k >= 512 is faster on the eight-wavefront kernel, see above)
+  const bool mid_shape = !cv && !stream && kk % 128 == 0 && kk >= 512 && xn > 64 && yn > 64 &&
+                         4 * tiles128 >= cu_n && L.ld < (1 << 24) && R.ld < (1 << 24) &&
+                         (size_t)4 * 256 * 128 <= lds_cu && !(ctx->kernel_mask & MH_MASK_NO_MID);
   const bool xres = (!cv || xres_cv) && !stream && depth > 0 && kk % 64 == 0 && yn >= 256 &&
-                    xres_fits(xres_tx) && !(ctx->kernel_mask & MH_MASK_NO_XRES);
+                    xres_fits(xres_tx) && !(mid_shape && tiles128 <= cu_n) &&
+                    !(ctx->kernel_mask & MH_MASK_NO_XRES);
   // From a quarter of a round to one round of 128 x 128 tiles, and up to two and a half rounds where
   // k is long (with short k and several rounds the two-workgroups-per-CU kernel, which overlaps one
   // tile's epilogue with another's loop, wins: 32 x 512 x 1024 x 512 29.8 against 33.7 us): the
@@ -2798,10 +2844,8 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   // (64 tiles) 19.2 -> 18.7 us, 1280 x 2048 x 1280 (100) 16.3 -> 12.2, 2048^3 (256) 19.3 -> 14.8,
   // 2560 x 2048 x 2560 (400) 25.8 -> 23.8, 3072 x 1024 x 3072 (576) 26.6 -> 24.9; at 1024 tiles
   // (4096 x 1024 x 4096, 4096^3) the 256 x 256 tiles win by 8 - 13 %.
-  const int64_t tiles128 = ((xn + 127) / 128) * ((yn + 127) / 128) * batch;
-  const bool mid = !cv && !stream && !xres && kk % 128 == 0 && kk >= 512 && xn > 64 && yn > 64 &&
-                   4 * tiles128 >= cu_n && (tiles128 <= cu_n || (kk >= 2048 && 2 * tiles128 <= 5 * cu_n)) && L.ld < (1 << 24) && R.ld < (1 << 24) &&
-                   (size_t)4 * 256 * 128 <= lds_cu && !(ctx->kernel_mask & MH_MASK_NO_MID);
+  const bool mid = mid_shape && !xres &&
+                   (tiles128 <= cu_n || (kk >= 2048 && 2 * tiles128 <= 5 * cu_n));
   if (!stream && !xres && !mid) {
     if (!L.sums && !(sum_y && !x_is_lhs))
       MH_RETURN_IF_ERROR(launch_panel_sums(ctx, L.ptr, L.ld, L.bs, rows, L.k, lhs_nb, corrL));
