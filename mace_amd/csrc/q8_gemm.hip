@@ -1917,11 +1917,20 @@ __global__ __launch_bounds__(256) void q8_zero_i32_kernel(int32_t *p, int64_t n)
 // conv with few channels) pack several rows into one wavefront so that every 16-byte load is
 // useful, long rows get the whole wavefront.  Rows are consecutive in memory whenever
 // ld == k, which then makes a wavefront's loads one contiguous run.
+// `zero` (or nullptr): zero_n words that this launch clears on the way -- the buffer into which
+// the next launch, a transposing repack, adds up the other operand's sums with atomics.
 template <int LPR>
 __global__ __launch_bounds__(256) void q8_panel_sums_kernel(const uint8_t *P, int64_t ld,
                                                             int64_t pbs, int n, int k,
-                                                            int32_t *sums) {
+                                                            int32_t *sums, int32_t *zero,
+                                                            int64_t zero_n) {
   constexpr int RPW = 64 / LPR;   // rows per wavefront
+  if (zero) {
+    const int64_t nthreads = (int64_t)gridDim.x * gridDim.z * 256;
+    for (int64_t i = ((int64_t)blockIdx.z * gridDim.x + blockIdx.x) * 256 + threadIdx.x; i < zero_n;
+         i += nthreads)
+      zero[i] = 0;
+  }
   const int lane = threadIdx.x & 63;
   const int sub = lane % LPR;
   const int64_t row = ((int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * RPW +
@@ -1945,7 +1954,7 @@ __global__ __launch_bounds__(256) void q8_panel_sums_kernel(const uint8_t *P, in
 }
 
 int launch_panel_sums(mace_hip_ctx *ctx, const uint8_t *P, int64_t ld, int64_t pbs, int64_t n,
-                      int k, int nb, int32_t *sums) {
+                      int k, int nb, int32_t *sums, int32_t *zero = nullptr, int64_t zero_n = 0) {
   const int chunks = k / 16;
   int lpr = 1;
   while (lpr < 64 && lpr < chunks) lpr *= 2;
@@ -1955,7 +1964,7 @@ int launch_panel_sums(mace_hip_ctx *ctx, const uint8_t *P, int64_t ld, int64_t p
   dim3 grid((unsigned)blocks, 1, nb), block(256);
 #define MH_SUMS(L_)                                                                       \
   hipLaunchKernelGGL((q8_panel_sums_kernel<L_>), grid, block, 0, ctx->stream, P, ld, pbs, \
-                     (int)n, k, sums)
+                     (int)n, k, sums, zero, zero_n)
   switch (lpr) {
     case 1: MH_SUMS(1); break;
     case 2: MH_SUMS(2); break;
@@ -2653,6 +2662,8 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
 
   // fused_sums: where the repack may leave the panel's row sums as well (or nullptr); *fused
   // tells whether it did
+  // sums_cleared: an earlier launch of this call has zeroed fused_sums already
+  bool sums_cleared = false;
   auto pack = [&](const uint8_t *src, int order_is_kcontig, int nb, int64_t n, uint8_t *dst,
                   int32_t *fused_sums, bool *fused, bool want_flipped = false,
                   bool *flipped = nullptr) -> int {
@@ -2677,8 +2688,9 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
         dim3 grid((unsigned)((n + 127) / 128), (unsigned)((kp + 127) / 128), nb);
         if (fused_sums) {
           const int64_t cnt = (int64_t)nb * n;
-          hipLaunchKernelGGL(q8_zero_i32_kernel, dim3((unsigned)((cnt + 255) / 256)), dim3(256), 0,
-                             ctx->stream, fused_sums, cnt);
+          if (!sums_cleared)
+            hipLaunchKernelGGL(q8_zero_i32_kernel, dim3((unsigned)((cnt + 255) / 256)), dim3(256), 0,
+                               ctx->stream, fused_sums, cnt);
           *fused = true;
         }
         const bool fl = want_flipped && flipped;
@@ -2789,6 +2801,19 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   const bool x_flip = !(ctx->kernel_mask & MH_MASK_NO_XFLIP) && !cv && depth % 128 == 0 && depth >= 1280 && depth < (1 << 24) && !sums_in_kernel &&
                       mh_q8_tile_choice(x_is_lhs ? rows : cols, x_is_lhs ? cols : rows, batch, cu_pre) ==
                           MH_TILE_BIG;
+  // Where the left-hand matrix is read in place and needs a pass for its sums (the Y operand of the
+  // 256 x 256 kernel on a shape too large for in-kernel sums) while the right-hand one is repacked
+  // with fused sums, the pass goes first and clears the repack's sums buffer on the way: one launch
+  // less in front of the GEMM kernel (8192^3, same process: 502.3 -> 500.3 us per call).
+  // x_flip repeats the dispatch's shape test: none of the kernels that sum their own panels applies.
+  const bool l_sums_first = x_flip && !x_is_lhs && !sum_y_shape && lhs_direct && !lhs_w && !rhs_w &&
+                            !rhs_direct && rhs_order == MACE_HIP_ROW_MAJOR && cols % 16 == 0 &&
+                            (uintptr_t)rhs % 16 == 0;
+  if (l_sums_first) {
+    MH_RETURN_IF_ERROR(launch_panel_sums(ctx, lhs, depth, lhs_nb > 1 ? rows * depth : 0, rows, (int)depth,
+                                         lhs_nb, corrL, corrR, (int64_t)rhs_nb * cols));
+    sums_cleared = true;
+  }
   MH_RETURN_IF_ERROR(prepare(lhs, lhs_order == MACE_HIP_ROW_MAJOR, lhs_direct, lhs_nb, rows, depth,
                              lhs_w, ((!x_is_lhs && sum_y_shape) || sums_in_kernel) ? nullptr : corrL, &L,
                              x_flip && x_is_lhs));
@@ -2846,8 +2871,10 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   // (4096 x 1024 x 4096, 4096^3) the 256 x 256 tiles win by 8 - 13 %.
   const bool mid = mid_shape && !xres &&
                    (tiles128 <= cu_n || (kk >= 2048 && 2 * tiles128 <= 5 * cu_n));
+  MH_CHECK(ctx, !l_sums_first || (!stream && !xres && !mid && !L.sums && !sum_y),
+           "internal: early sums pass on a shape whose kernel takes its own");
   if (!stream && !xres && !mid) {
-    if (!L.sums && !(sum_y && !x_is_lhs))
+    if (!L.sums && !(sum_y && !x_is_lhs) && !l_sums_first)
       MH_RETURN_IF_ERROR(launch_panel_sums(ctx, L.ptr, L.ld, L.bs, rows, L.k, lhs_nb, corrL));
     if (!R.sums && !(sum_y && x_is_lhs))
       MH_RETURN_IF_ERROR(launch_panel_sums(ctx, R.ptr, R.ld, R.bs, cols, R.k, rhs_nb, corrR));
