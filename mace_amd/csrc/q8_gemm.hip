@@ -2510,7 +2510,22 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     const bool y_direct = xl ? (rhs_direct && rhs_ld == 0) : lhs_direct;
     const int tx = xn <= 64 ? 64 : 128;
     const size_t lds_cu = ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536;
-    if (!cv && x_kmajor && y_direct && rhs_ld == 0 && !lhs_w && !rhs_w && depth > 0 &&
+    const int64_t tiles128 = ((xn + 127) / 128) * ((yn + 127) / 128) * batch;
+    const int64_t tiles256 = ((xn + 255) / 256) * ((yn + 255) / 256) * batch;
+    const int64_t cu_n = ctx->cu_count > 0 ? ctx->cu_count : 256;
+    // the 256 x 256 ring kernel's k-major variant applies (third block below)
+    const bool big_xt = !cv && x_kmajor && y_direct && rhs_ld == 0 && !lhs_w && !rhs_w && depth >= 256 &&
+                        (depth < 8192 || ctx->no_alloc || ctx->capturing) && depth % 128 == 0 &&
+                        xn % 16 == 0 && (uintptr_t)xp % 16 == 0 &&
+                        mh_q8_tile_choice(xn, yn, batch, cu_n) == MH_TILE_BIG &&
+                        xn * depth < ((int64_t)1 << 32) && depth < (1 << 24) &&
+                        (size_t)2 * 512 * 128 <= lds_cu && !(ctx->kernel_mask & MH_MASK_NO_MID);
+    // ... and wins over the resident-tile kernel while its tiles are at most one round (us per call,
+    // three buffer sets in rotation: 4096 x 512 x 4096 27.0 -> 23.1, 2048 x 512 x 8192 26.8 -> 22.3,
+    // 3072 x 512 x 3072 22.9 -> 20.1, 4096 x 384 x 4096 22.8 -> 21.1, 4 x 2048 x 512 x 2048 25.3 -> 23.7;
+    // k = 256 ties; four rounds, 8192 x 512 x 8192, lose 64 against 79)
+    const bool big_xt_first = big_xt && depth >= 384 && tiles256 <= cu_n;
+    if (!cv && x_kmajor && y_direct && rhs_ld == 0 && !lhs_w && !rhs_w && depth > 0 && !big_xt_first &&
         depth % 64 == 0 && xn % 16 == 0 && (uintptr_t)xp % 16 == 0 && yn >= 256 &&
         2 * (XRES_SC_BYTES + (size_t)tx * depth) <= lds_cu && !mid_first_xt &&
         !(ctx->kernel_mask & MH_MASK_NO_XRES)) {
@@ -2548,8 +2563,6 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     // repack (2048^3: zeroing 2.4 + repack 7.5 us of a 22 us call) is not launched.  Because of that
     // saving the range is wider here: two rounds of tiles from k = 1024 on (8 x 1024^3 25.7 -> 23.4 us,
     // 32 x 512 x 1024 x 512 30.1 -> 24.8; 3072 x 1024 x 3072, 576 tiles, loses 5 % and is left out).
-    const int64_t tiles128 = ((xn + 127) / 128) * ((yn + 127) / 128) * batch;
-    const int64_t cu_n = ctx->cu_count > 0 ? ctx->cu_count : 256;
     if (!cv && x_kmajor && y_direct && rhs_ld == 0 && !lhs_w && !rhs_w && depth >= 512 &&
         depth % 128 == 0 && xn % 16 == 0 && (uintptr_t)xp % 16 == 0 && xn > 64 && yn > 64 &&
         4 * tiles128 >= cu_n &&
@@ -2591,12 +2604,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     // are saved but the kernel, at its power limit, pays 22 us for the twice as many LDS read
     // instructions of the k-major operand (512.7 -> 518 us per call), so from k = 8192 on the
     // repack stays unless the arena may not grow (no repacked copy is needed here).
-    if (!cv && x_kmajor && y_direct && rhs_ld == 0 && !lhs_w && !rhs_w && depth >= 256 &&
-        (depth < 8192 || ctx->no_alloc || ctx->capturing) &&
-        depth % 128 == 0 && xn % 16 == 0 && (uintptr_t)xp % 16 == 0 &&
-        mh_q8_tile_choice(xn, yn, batch, cu_n) == MH_TILE_BIG &&
-        xn * depth < ((int64_t)1 << 32) && depth < (1 << 24) && (size_t)2 * 512 * 128 <= lds_cu &&
-        !(ctx->kernel_mask & MH_MASK_NO_MID)) {
+    if (big_xt) {
       const int x_nb = xl ? lhs_nb : rhs_nb, y_nb = xl ? rhs_nb : lhs_nb;
       MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, sizeof(int32_t) * ((size_t)x_nb * xn + (size_t)y_nb * yn) + 1024));
       ArenaScope scope(ctx);

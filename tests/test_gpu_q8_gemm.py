@@ -161,6 +161,26 @@ def test_q8_gemm_one_round_of_tiles(ctx, mid, batch, rows, depth, cols, lb, rb, 
         ctx.call("mace_hip_ctx_set_kernel_mask", 0)
 
 
+# Shapes on the boundaries between the one-launch kernels under the normal dispatch: the
+# eight-wavefront kernel ahead of the one-launch and the resident-tile kernels (one round of
+# 128 x 128 tiles, k >= 512; k-contiguous against the one-launch kernel from k = 1024), the
+# 256 x 256 kernel with a k-major operand in place ahead of the resident-tile kernel (at most one
+# round of its tiles, k >= 384), and their neighbours just outside.
+DISPATCH_SHAPES = [
+    (16, 512, 512, 512, True, True, R, R, R), (4, 512, 512, 512, True, True, R, R, R),
+    (1, 2048, 512, 2048, True, True, R, Cm, R), (1, 1024, 1024, 1024, True, True, R, Cm, R),
+    (1, 1024, 896, 1024, True, True, R, Cm, R), (1, 1100, 640, 1200, True, True, R, R, R),
+    (1, 3000, 512, 4000, True, True, R, R, R), (1, 4000, 384, 3024, True, True, Cm, Cm, Cm),
+    (1, 3000, 256, 4000, True, True, R, R, R), (2, 2048, 512, 2064, True, False, R, R, R),
+    (1, 760, 512, 1024, True, True, R, R, R),
+]
+
+
+@pytest.mark.parametrize("batch,rows,depth,cols,lb,rb,lo,ro,oo", DISPATCH_SHAPES)
+def test_q8_gemm_dispatch_boundaries(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo):
+    check_gemm(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo)
+
+
 def test_q8_gemm_config1_matmul(ctx):
     """benchmark configuration 1: A [128x256], B [256x128], zero points 128/128/128, scales
     0.02/0.015/0.05 -> (1649267328, shift 7)."""
