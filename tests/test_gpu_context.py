@@ -31,7 +31,7 @@ def _gemm(ctx, d, n):
 
 def test_stopwatch_times_every_launch_without_waiting(ctx):
     d = Dev()
-    small, large = _gemm(ctx, d, 256), _gemm(ctx, d, 2048)
+    small, large = _gemm(ctx, d, 256), _gemm(ctx, d, 4096)
     with pytest.raises(mh.MaceHipError):
         ctx.last_kernel_ms()                       # never enabled
     small(), large()                               # first launches load the kernels' code
@@ -44,7 +44,7 @@ def test_stopwatch_times_every_launch_without_waiting(ctx):
     ctx.profile(False)
     ms = ctx.kernel_ms_list()
     assert len(ms) == 5 and all(m > 0 for m in ms)
-    # 2048^3 is 512 times the work of 256^3: the per-launch durations tell them apart
+    # 4096^3 is 4096 times the work of 256^3: the per-launch durations tell them apart
     assert min(ms[1], ms[3], ms[4]) > 2 * max(ms[0], ms[2]), ms
     assert ctx.last_kernel_ms() == pytest.approx(ms[4])
     v = C.c_float()
