@@ -129,23 +129,53 @@ __device__ inline void stage_requant_pairs(int32_t *pairs, const RequantFixed &r
     pairs[2 * c + 1] = rq.lo + c;
   }
 }
+// The float estimate of the step index with the table's LDS address folded in: the mantissa trick
+// of mh_requant_step_estimate yields 8 * (step index) as the low bits of the float; adding the
+// table's address / 8 to the offset and to both clamp bounds makes those bits the entry's LDS
+// address itself, so the look-up needs no address arithmetic (a vector add per output otherwise).
+// All values stay integers (+ 7/8) below 2^21, where a float's last bit is worth 1/8: exact.
+struct RequantLds {
+  float inv, off, lo, top;
+};
+__device__ __forceinline__ RequantLds requant_lds(const RequantFixed &rq, const int32_t *pairs) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const uint32_t addr = (uint32_t)(const __attribute__((address_space(3))) int32_t *)pairs;
+#else
+  const uint32_t addr = 0;
+#endif
+  const float t0 = (float)(addr >> 3);   // the table is 8-byte aligned; LDS addresses are below 2^18
+  return RequantLds{rq.inv, rq.off + t0, MH_REQUANT_MAGIC + t0, rq.top + t0};
+}
 // Sixteen accumulators -> sixteen output bytes in four dwords.  Estimates first, then all
 // look-ups, then the compares: sixteen LDS reads in flight instead of one round trip per element.
-__device__ __forceinline__ void requant_16_by_table(const int32_t (&v)[16], const RequantFixed &rq,
-                                                    const int32_t *pairs, uint32_t (&packed)[4]) {
+__device__ __forceinline__ void requant_16_by_table(const int32_t (&v)[16], const RequantLds &rq,
+                                                    uint32_t (&packed)[4]) {
+  typedef int pair_t __attribute__((ext_vector_type(2)));
   uint32_t a[16];
-  int2 e[16];
+  pair_t e[16];
 #pragma unroll
   for (int r = 0; r < 16; ++r)
-    a[r] = __float_as_uint(__builtin_amdgcn_fmed3f(__fmaf_rn((float)v[r], rq.inv, rq.off),
-                                                   MH_REQUANT_MAGIC, rq.top)) & 0xFF8u;
+    a[r] = __float_as_uint(__builtin_amdgcn_fmed3f(__fmaf_rn((float)v[r], rq.inv, rq.off), rq.lo,
+                                                   rq.top)) & 0x3FFF8u;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) e[r] = *(const int2 *)((const char *)pairs + a[r]);
+  for (int r = 0; r < 16; ++r) {
+#if defined(__HIP_DEVICE_COMPILE__)   // (an LDS pointer is 32 bits wide in the device pass only)
+    e[r] = *(const __attribute__((address_space(3))) pair_t *)a[r];
+#else
+    e[r] = pair_t{0, 0};
+#endif
+  }
 #pragma unroll
-  for (int q = 0; q < 4; ++q) packed[q] = 0;
+  for (int q = 0; q < 4; ++q) {
+    uint32_t o[4];
 #pragma unroll
-  for (int r = 0; r < 16; ++r)
-    packed[r / 4] |= (uint32_t)(e[r].y + (v[r] > e[r].x ? 1 : 0)) << (8 * (r % 4));
+    for (int i = 0; i < 4; ++i) o[i] = (uint32_t)(e[4 * q + i].y + (v[4 * q + i] > e[4 * q + i].x ? 1 : 0));
+    // bytes 0 of o[0..3] side by side (v_perm_b32: selector 0..3 = bytes of the second operand,
+    // 4..7 of the first, 0x0c = zero)
+    const uint32_t p10 = __builtin_amdgcn_perm(o[1], o[0], 0x0c0c0400u);
+    const uint32_t p32 = __builtin_amdgcn_perm(o[3], o[2], 0x0c0c0400u);
+    packed[q] = (p32 << 16) | p10;
+  }
 }
 
 // Epilogue shared by the GEMM kernels: adds the correction vectors to the accumulators and
@@ -197,6 +227,7 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[FX][FY], const int (&y
   const bool interior = vec_ok && x0 + TX <= p.XN && y0 + TY <= p.YN;
   const bool interior16 = interior && (p.ldo % 16 == 0) && (((uintptr_t)outb) % 16 == 0);
 
+  const RequantLds rql = requant_lds(rq, tab);
   // One fully unrolled copy of the store loop per combination that occurs: TABLE = threshold
   // requantization, WIDE = whole tile inside the matrix and 16-byte aligned rows.
   auto store_tile = [&](auto table_tag, auto wide_tag) __attribute__((always_inline)) {
@@ -246,7 +277,7 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[FX][FY], const int (&y
         } else {
           uint32_t packed[4] = {0, 0, 0, 0};
           if constexpr (TABLE) {
-            requant_16_by_table(v, rq, tab, packed);
+            requant_16_by_table(v, rql, packed);
           } else {
 #pragma unroll
             for (int r = 0; r < 16; ++r)
@@ -1671,6 +1702,7 @@ void q8_gemm_stream_kernel(GemmParams p, RequantTable) {
     }
   }
   stage_requant_pairs(s_tab, rq, tid, 256);
+  const RequantLds rql = requant_lds(rq, s_tab);
   __syncthreads();
 
   const int nblk = (p.YN + 31) / 32;
@@ -1728,7 +1760,7 @@ void q8_gemm_stream_kernel(GemmParams p, RequantTable) {
               v[q * 4 + e] = (int32_t)((uint32_t)acc[q * 4 + e] + (uint32_t)cx[e] + cy);
           }
           uint32_t packed[4];
-          requant_16_by_table(v, rq, s_tab, packed);
+          requant_16_by_table(v, rql, packed);
           const v2u s02 = __builtin_amdgcn_permlane32_swap(packed[0], packed[2], false, false);
           const v2u s13 = __builtin_amdgcn_permlane32_swap(packed[1], packed[3], false, false);
           const v4i w = {(int)s02.x, (int)s02.y, (int)s13.x, (int)s13.y};
