@@ -59,6 +59,9 @@ struct mace_hip_ctx {
   int lds_bytes = 0;
   // kernels whose dynamic LDS limit has been raised, and to how many bytes
   std::vector<std::pair<const void *, size_t>> big_lds_kernels;
+  // workgroups of a kernel that fit on one CU at a given dynamic LDS size (mh_blocks_per_cu)
+  struct Occupancy { const void *kernel; size_t lds; int blocks; };
+  std::vector<Occupancy> occupancy;
   char arch[64] = {0};
   char err[512] = {0};
   // last few requantization comparison tables built on this context (mult, shift, blo, n)
@@ -433,6 +436,20 @@ inline hipError_t mh_allow_big_lds(mace_hip_ctx *ctx, const void *kernel, size_t
       hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
   if (rc == hipSuccess) ctx->big_lds_kernels.emplace_back(kernel, bytes);
   return rc;
+}
+
+// How many workgroups of `threads` threads and `lds` bytes of dynamic LDS the runtime fits on one
+// CU for this kernel (registers included); asked once per kernel and size, 1 if the query fails.
+inline int mh_blocks_per_cu(mace_hip_ctx *ctx, const void *kernel, int threads, size_t lds) {
+  for (const auto &e : ctx->occupancy)
+    if (e.kernel == kernel && e.lds == lds) return e.blocks;
+  int n = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, threads, lds) != hipSuccess || n < 1) {
+    (void)hipGetLastError();
+    n = 1;
+  }
+  ctx->occupancy.push_back({kernel, lds, n});
+  return n;
 }
 
 // Fills device memory with one byte value on the context's stream, with a kernel (a memset node
