@@ -272,7 +272,8 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[FX][FY], const int (&y
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
             const int xl = xb + 8 * q;
-            if (interior) {
+            // (rows of whole, aligned 16-byte pieces: a ragged tile stores them whole as well)
+            if (interior || (vec_ok && p.XN % 4 == 0 && y < p.YN && x0 + xl < p.XN)) {
               *(v4i *)(orow + xl) = v4i{v[q * 4], v[q * 4 + 1], v[q * 4 + 2], v[q * 4 + 3]};
             } else if (y < p.YN) {
 #pragma unroll
@@ -302,7 +303,8 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[FX][FY], const int (&y
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
               const int xl = xb + 8 * q;
-              if (interior) {
+              // (rows of whole, aligned dwords: a ragged tile stores them whole as well)
+              if (interior || (vec_ok && p.XN % 4 == 0 && y < p.YN && x0 + xl < p.XN)) {
                 *(uint32_t *)(orow + xl) = packed[q];
               } else if (y < p.YN) {
 #pragma unroll
