@@ -1416,8 +1416,10 @@ __device__ __forceinline__ void transpose_16x16_bytes(v4i (&r)[16]) {
 // matrix): the tile is read in 16 x 16 byte blocks, flipped, transposed in registers and written
 // into the same LDS layout, the row sums added up through LDS atomics; XN % 16 == 0, X 16-byte
 // aligned.
-template <int FX, int FY, int G, typename OutT, int OCC, bool CONV = false, bool XT = false>
+template <int FX, int FY, int G, typename OutT, int OCC, bool CONV = false, bool XT = false,
+          bool TAIL = false>
 __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, RequantTable) {
+  static_assert(!TAIL || (!CONV && !XT && G == 64), "the depth tail: plain operands, 64-byte groups");
   constexpr int TX = FX * 32, TYW = FY * 32;
   constexpr int KPG = G / 32;   // k steps per group
   static_assert(G == 64 || G == 128, "group width");
@@ -1449,7 +1451,11 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
   const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
 
   const int nblk = (p.YN + TYW - 1) / TYW;
-  const int ngroup = p.K / G;
+  // TAIL: K is a multiple of 16 but not of 64.  k is walked up to the next multiple of 64; the
+  // 16-byte pieces past K are not fetched (their addresses are clamped to the row's first piece)
+  // and count as zeros after the shift on both sides.
+  const int KP = TAIL ? (p.K + 63) & ~63 : p.K;
+  const int ngroup = KP / G;
   const int stride = gridDim.x * 4;
   int blk = wg_y * 4 + wave;
   // What a lane needs to address its row of a block.  Plain: the row's first byte (+ the lane's
@@ -1486,6 +1492,17 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
       return r.ptr[j] + (int64_t)g * G;
     }
   };
+  // piece t of this lane's share of group g (k = G g + G/2 h + 16 t); TAIL: past K it is 0x80 bytes
+  const v4i raw_zero = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+  auto load_piece = [&](const uint8_t *src, int g, int t) -> v4i {
+    if constexpr (TAIL) {
+      const int k = g * G + (G / 2) * h + 16 * t;
+      const v4i v = *(const v4i *)(k < p.K ? src + 16 * t : src - (int64_t)g * G - (G / 2) * h);
+      return k < p.K ? v : raw_zero;
+    } else {
+      return *(const v4i *)(src + 16 * t);
+    }
+  };
   // the first block's first group is requested before anything else
   v4i cur[KPG][FY], nxt[KPG][FY];
   Rows yr, yrn;
@@ -1494,7 +1511,7 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
   for (int j = 0; j < FY; ++j) {
     const uint8_t *src = group_src(yr, j, 0, 0, 0, 0);
 #pragma unroll
-    for (int t = 0; t < KPG; ++t) cur[t][j] = *(const v4i *)(src + 16 * t);
+    for (int t = 0; t < KPG; ++t) cur[t][j] = load_piece(src, 0, t);
   }
 
   if constexpr (XT) {
@@ -1533,18 +1550,23 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
   } else {
     // X tile -> LDS: one transfer instruction moves 16 rows x 64 bytes
     constexpr int LX = TX / 64;   // instructions per wavefront per slab
-    const int nslab = p.K / 64;
+    const int nslab = KP / 64;
     const uint8_t *src[LX];
+    int src_kc[LX];
 #pragma unroll
     for (int j = 0; j < LX; ++j) {
       const int row = (j * 4 + wave) * 16 + (lane >> 2);
       const int kc = (lane & 3) ^ ((row >> 2) & 3);
+      src_kc[j] = kc * 16;
       src[j] = Xb + (int64_t)min(x0 + row, p.XN - 1) * p.ldx + kc * 16;
     }
     for (int s = 0; s < nslab; ++s) {
 #pragma unroll
-      for (int j = 0; j < LX; ++j)
-        dma_16B(src[j] + s * 64, xt + s * (TX * 64) + (j * 4 + wave) * 1024);
+      for (int j = 0; j < LX; ++j) {
+        // TAIL: a piece past K fetches the row's first piece instead; the pass below zeroes it
+        const bool past = TAIL && s * 64 + src_kc[j] >= p.K;
+        dma_16B(past ? src[j] - src_kc[j] : src[j] + s * 64, xt + s * (TX * 64) + (j * 4 + wave) * 1024);
+      }
       // at most 32 transfers of this wavefront in flight (the counter has six bits)
       if ((s & 15) == 15) wait_vmcnt<0>();
     }
@@ -1558,7 +1580,10 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
       uint8_t *q = xt + s * (TX * 64) + row * 64;
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
-        const v4i v = *(const v4i *)(q + c * 16) ^ flip;
+        v4i v = *(const v4i *)(q + c * 16) ^ flip;
+        if constexpr (TAIL) {   // slot c holds piece c ^ swizzle(row) of the slab
+          if (s * 64 + ((c ^ ((row >> 2) & 3)) << 4) >= p.K) v = v4i{0, 0, 0, 0};
+        }
         xs = sum16_i8(v, xs);
         *(v4i *)(q + c * 16) = v;
       }
@@ -1612,7 +1637,7 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
       for (int j = 0; j < FY; ++j) {
         const uint8_t *src = last ? group_src(yrn, j, 0, 0, 0, 0) : group_src(yr, j, g + 1, kh, kw, c0);
 #pragma unroll
-        for (int t = 0; t < KPG; ++t) nxt[t][j] = *(const v4i *)(src + 16 * t);
+        for (int t = 0; t < KPG; ++t) nxt[t][j] = load_piece(src, last ? 0 : g + 1, t);
       }
       const uint8_t *xg = xfrag + g * GSTRIDE;
 #pragma unroll
@@ -1645,7 +1670,7 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
     group(std::true_type{}, 0);
     for (int g = 1; g < ngroup; ++g) group(std::false_type{}, g);
 #pragma unroll
-    for (int j = 0; j < FY; ++j) ysum[j] -= 64 * p.K;   // this lane's half of every row: K / 2 bytes
+    for (int j = 0; j < FY; ++j) ysum[j] -= 64 * KP;   // this lane's half of every row: KP / 2 bytes
     gemm_epilogue<1, 1, FX, FY, OutT, true, true>(acc, ysum, p, lds, b, x0, blk * TYW, 0, 0, tid);
     blk = nb;
     yr = yrn;
@@ -2270,7 +2295,8 @@ template <int FX, int FY>
 int launch_gemm_xres(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, bool out_u8,
                      int batch, bool xt = false) {
   constexpr int TX = FX * 32, TYW = FY * 32;
-  const size_t lds = XRES_SC_BYTES + (size_t)TX * p.K;
+  const bool tail = p.K % 64 != 0;   // (a multiple of 16: checked by the caller)
+  const size_t lds = XRES_SC_BYTES + (size_t)TX * ((p.K + 63) & ~63);
   const int tiles_x = (p.XN + TX - 1) / TX;
   const int nblk = (p.YN + TYW - 1) / TYW;
   const int cu = ctx->cu_count > 0 ? ctx->cu_count : 256;
@@ -2308,6 +2334,10 @@ int launch_gemm_xres(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, 
     }
     if (g128) return launch(q8_gemm_xres_kernel<FX, FY, 128, int32_t, 2, false, true>);
     return launch(q8_gemm_xres_kernel<FX, FY, 64, int32_t, 2, false, true>);
+  }
+  if (tail) {
+    if (out_u8) return launch(q8_gemm_xres_kernel<FX, FY, 64, uint8_t, 2, false, false, true>);
+    return launch(q8_gemm_xres_kernel<FX, FY, 64, int32_t, 2, false, false, true>);
   }
   if (out_u8) {
     if (g128) return launch(q8_gemm_xres_kernel<FX, FY, 128, uint8_t, 2>);
@@ -2473,6 +2503,21 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
                             mid_xn * depth < ((int64_t)1 << 32);
   const bool mid_first_kc = mid_one_round && mid_x_direct && mid_y_direct && depth >= 1024;
 
+  // A depth that is a multiple of 16 but not of 64, both operands k-contiguous and read in place, a
+  // long Y panel and an X tile that fits in LDS: the resident-tile kernel walks k up to the next
+  // multiple of 64 itself (pieces past the end count as zeros), so nothing is repacked and the
+  // one-launch kernel, which otherwise takes such depths at any size, keeps the small problems
+  // (200704 x 96 x 128: 25.8 us there).
+  const int64_t tail_kp = (depth + 63) & ~(int64_t)63;
+  const bool tail_xres =
+      !cv && !lhs_w && !rhs_w && rhs_ld == 0 && depth > 64 && depth % 64 != 0 && depth % 16 == 0 &&
+      lhs_direct && rhs_direct && lhs_order == MACE_HIP_ROW_MAJOR && rhs_order == MACE_HIP_COL_MAJOR &&
+      mid_yn >= 256 &&
+      2 * (XRES_SC_BYTES + (size_t)(mid_xn <= 64 ? 64 : 128) * tail_kp) <=
+          (ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536) &&
+      !mh_q8_small_problem(ctx, batch, rows, cols, depth, true, false) &&
+      !(ctx->kernel_mask & MH_MASK_NO_XRES);
+
   // Small problems: one launch that reads both operands where they lie (k-contiguous, or k-major
   // and transposed on the way into LDS) and takes both correction vectors itself.
   {
@@ -2494,7 +2539,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     const bool stream_shape = out_u8 && rq.table && mh_q8_stream_shape(depth, xn_s, yn_s) &&
                               ((uintptr_t)out % 16 == 0);
     const bool in_place = !lhs_t && !rhs_t && lhs_direct && rhs_direct && rhs_ld == 0;
-    const bool any_size = in_place && depth % 64 != 0 && !stream_shape;
+    const bool any_size = in_place && depth % 64 != 0 && !stream_shape && !tail_xres;
     const bool small = cv ? cv_small
                           : (mh_q8_small_problem(ctx, batch, rows, cols, depth, lhs_vec && rhs_vec,
                                                  any_size) &&
@@ -2899,7 +2944,9 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   // (Bit MH_MASK_NO_XRES of the kernel mask: test hook that keeps the tiled kernels in use.)
   const int kk = L.k < R.k ? L.k : R.k;
   const size_t lds_cu = ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536;
-  auto xres_fits = [&](int tx) { return 2 * (XRES_SC_BYTES + (size_t)tx * kk) <= lds_cu; };
+  auto xres_fits = [&](int tx) {
+    return 2 * (XRES_SC_BYTES + (size_t)tx * ((kk + 63) & ~63)) <= lds_cu;
+  };
   // Where 128 rows of a long k do not fit, 64-row tiles (Y is then read once per 64 X rows) still
   // win between one and two 64 x 64 blocks per CU, where the tiled kernels leave most of the chip
   // idle (k = 1024, 512 X rows, 3136 Y rows: 16.0 -> 9.4 us); beyond that they lose.
@@ -2913,7 +2960,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   const bool mid_shape = !cv && !stream && kk % 128 == 0 && kk >= 512 && xn > 64 && yn > 64 &&
                          4 * tiles128 >= cu_n && L.ld < (1 << 24) && R.ld < (1 << 24) &&
                          (size_t)4 * 256 * 128 <= lds_cu && !(ctx->kernel_mask & MH_MASK_NO_MID);
-  const bool xres = (!cv || xres_cv) && !stream && depth > 0 && kk % 64 == 0 && yn >= 256 &&
+  const bool xres = (!cv || xres_cv) && !stream && depth > 0 && (kk % 64 == 0 || tail_xres) && yn >= 256 &&
                     xres_fits(xres_tx) && !(mid_shape && tiles128 <= cu_n) &&
                     !(ctx->kernel_mask & MH_MASK_NO_XRES);
   // From a quarter of a round to one round of 128 x 128 tiles, and up to two and a half rounds where
@@ -2926,6 +2973,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   // (4096 x 1024 x 4096, 4096^3) the 256 x 256 tiles win by 8 - 13 %.
   const bool mid = mid_shape && !xres &&
                    (tiles128 <= cu_n || (kk >= 2048 && 2 * tiles128 <= 5 * cu_n));
+  MH_CHECK(ctx, !tail_xres || xres, "internal: depth tail outside the resident-tile kernel");
   MH_CHECK(ctx, !l_sums_first || (!stream && !xres && !mid && !L.sums && !sum_y),
            "internal: early sums pass on a shape whose kernel takes its own");
   if (!stream && !xres && !mid) {

@@ -181,6 +181,29 @@ def test_q8_gemm_dispatch_boundaries(ctx, batch, rows, depth, cols, lb, rb, lo, 
     check_gemm(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo)
 
 
+# Depths that are a multiple of 16 but not of 64 with both operands k-contiguous: read in place by
+# the resident-tile kernel, which walks k to the next multiple of 64 (tails of 16, 32 and 48 bytes;
+# 64- and 128-row tiles; 32- and 64-row blocks; ragged rows and columns; the result transposed;
+# batches), and the same shapes through the other kernels.
+TAIL_SHAPES = [
+    (1, 9000, 96, 128, True, True, R, Cm, R), (1, 9000, 144, 128, True, True, R, Cm, R),
+    (1, 9000, 176, 64, True, True, R, Cm, R), (1, 70000, 80, 48, True, True, R, Cm, R),
+    (1, 5003, 208, 200, True, True, R, Cm, R), (2, 3000, 112, 130, True, True, R, Cm, R),
+    (1, 128, 160, 9000, True, True, R, Cm, Cm), (1, 20000, 336, 256, True, True, R, Cm, R),
+    (3, 4000, 96, 128, True, False, R, Cm, R),
+]
+
+
+@pytest.mark.parametrize("batch,rows,depth,cols,lb,rb,lo,ro,oo", TAIL_SHAPES)
+@pytest.mark.parametrize("kernels", ["normal", "no_resident_tile"])
+def test_q8_gemm_depth_tail_in_place(ctx, kernels, batch, rows, depth, cols, lb, rb, lo, ro, oo):
+    ctx.call("mace_hip_ctx_set_kernel_mask", 0 if kernels == "normal" else mh.MASK_NO_XRES)
+    try:
+        check_gemm(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo)
+    finally:
+        ctx.call("mace_hip_ctx_set_kernel_mask", 0)
+
+
 def test_q8_gemm_config1_matmul(ctx):
     """benchmark configuration 1: A [128x256], B [256x128], zero points 128/128/128, scales
     0.02/0.015/0.05 -> (1649267328, shift 7)."""
