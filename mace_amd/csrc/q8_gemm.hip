@@ -233,12 +233,10 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[FX][FY], const int (&y
 
   const RequantLds rql = requant_lds(rq, tab);
   // One fully unrolled copy of the store loop per combination that occurs: TABLE = threshold
-  // requantization, WIDE = 16-byte stores (aligned rows of whole 16-byte pieces), EDGE = the tile
-  // is not wholly inside the matrix.
-  auto store_tile = [&](auto table_tag, auto wide_tag, auto edge_tag) __attribute__((always_inline)) {
+  // requantization, WIDE = whole tile inside the matrix and 16-byte aligned rows.
+  auto store_tile = [&](auto table_tag, auto wide_tag) __attribute__((always_inline)) {
     constexpr bool TABLE = decltype(table_tag)::value;
     constexpr bool WIDE = decltype(wide_tag)::value;
-    constexpr bool EDGE = decltype(edge_tag)::value;   // WIDE: every lane checks its own 16-byte piece
 #pragma unroll
     for (int j = 0; j < FY; ++j) {
       const int yl = (wy * FY + j) * 32 + (lane & 31);
@@ -297,8 +295,16 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[FX][FY], const int (&y
             const v2u s02 = __builtin_amdgcn_permlane32_swap(packed[0], packed[2], false, false);
             const v2u s13 = __builtin_amdgcn_permlane32_swap(packed[1], packed[3], false, false);
             const v4i w = {(int)s02.x, (int)s02.y, (int)s13.x, (int)s13.y};
+            *(v4i *)(orow + (wx * FX + i) * 32 + 16 * (lane >> 5)) = w;
+          } else if (wide16) {
+            // the same 16-byte pieces in a tile that is not wholly inside the matrix: every lane
+            // checks its own piece (uniform branch; the requantization above is shared with the
+            // dword / byte stores below, so no further unrolled copy of it exists)
+            const v2u s02 = __builtin_amdgcn_permlane32_swap(packed[0], packed[2], false, false);
+            const v2u s13 = __builtin_amdgcn_permlane32_swap(packed[1], packed[3], false, false);
+            const v4i w = {(int)s02.x, (int)s02.y, (int)s13.x, (int)s13.y};
             const int xh = (wx * FX + i) * 32 + 16 * (lane >> 5);
-            if (!EDGE || (y < p.YN && x0 + xh < p.XN)) *(v4i *)(orow + xh) = w;
+            if (y < p.YN && x0 + xh < p.XN) *(v4i *)(orow + xh) = w;
           } else {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
@@ -321,16 +327,11 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[FX][FY], const int (&y
     }
   };
   if constexpr (sizeof(OutT) == 4) {
-    store_tile(std::false_type{}, std::false_type{}, std::false_type{});
+    store_tile(std::false_type{}, std::false_type{});
   } else {
-    // (not for 4 x 4 blocks per wavefront: with all 512 registers taken by accumulators and fragments
-    // a fourth copy of the unrolled loop costs spills that slow the other three down, 4096^3 by 2.6 %)
-    constexpr bool EDGE_COPY = FX * FY < 16;
-    if (rq.table && interior16) store_tile(std::true_type{}, std::true_type{}, std::false_type{});
-    else if (EDGE_COPY && rq.table && wide16)
-      store_tile(std::true_type{}, std::true_type{}, std::integral_constant<bool, EDGE_COPY>{});
-    else if (rq.table) store_tile(std::true_type{}, std::false_type{}, std::false_type{});
-    else store_tile(std::false_type{}, std::false_type{}, std::false_type{});
+    if (rq.table && interior16) store_tile(std::true_type{}, std::true_type{});
+    else if (rq.table) store_tile(std::true_type{}, std::false_type{});
+    else store_tile(std::false_type{}, std::false_type{});
   }
 }
 
