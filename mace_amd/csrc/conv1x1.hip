@@ -156,9 +156,20 @@ extern "C" int mace_hip_conv2d_q8_nhwc(mace_hip_ctx *ctx, const uint8_t *input,
   const bool small_gather = !in_place && in_h * in_w * cin < (1ll << 31) &&
                             mh_q8_small_problem(ctx, 1, cout, columns, depth, small_vec, cin % 64 != 0) &&
                             !(ctx->kernel_mask & MH_MASK_NO_SMALL);
+  // ... unless the patches make at most one round of 128 x 128 tiles with a long k: the gathering
+  // tiled kernel then leaves most CUs without a tile for its whole length, while the patch matrix
+  // is small and the eight-wavefront GEMM kernel takes it (7x7x512 -> 512, 3 x 3, batch 64: 46.4 ->
+  // 31.6 us; 7x7x1024 -> 1024: 86.7 -> 52.2; 14x14x256 -> 512 at stride 2: 28.4 -> 20.4; ties at 196
+  // tiles of depth 2304, loses at 392 tiles of depth 1152).  Not where the arena may not grow.
+  const int64_t tiles128 = ((cout + 127) / 128) * ((columns + 127) / 128);
+  const int64_t cu_n = ctx->cu_count > 0 ? ctx->cu_count : 256;
+  const bool im2col_one_round = depth >= 2048 && depth % 128 == 0 && cout > 64 && columns > 64 &&
+                                4 * tiles128 >= cu_n && tiles128 <= cu_n && !ctx->no_alloc &&
+                                !ctx->capturing && !(ctx->kernel_mask & MH_MASK_NO_MID);
   const bool gather = small_gather ||
-                      (!in_place && cin % 64 == 0 && depth >= 192 && ((uintptr_t)input % 16 == 0) &&
-                       ((uintptr_t)filter % 16 == 0) && in_h * in_w * cin < (1ll << 31));
+                      (!im2col_one_round && !in_place && cin % 64 == 0 && depth >= 192 &&
+                       ((uintptr_t)input % 16 == 0) && ((uintptr_t)filter % 16 == 0) &&
+                       in_h * in_w * cin < (1ll << 31));
   const int64_t kp = (int64_t)mh_align_up((size_t)(depth > 0 ? depth : 1), 64);
   size_t need = sizeof(int32_t) * cout + 4096 +
                 conv_gemm_scratch(cout, depth, columns, !in_place || depth % 16 == 0);

@@ -84,6 +84,9 @@ CASES = [  # batch, cout, cin, in_h, in_w, k_h, k_w, padding, strides: the refer
     # channel counts that are not multiples of 64, larger than a small problem: still gathered by
     # the one-launch kernel (first layer of a MobileNet at batch 8; 48 channels, 3x3)
     (8, 32, 3, 224, 224, 3, 3, S, (2, 2)), (6, 48, 48, 56, 56, 3, 3, S, (1, 1)),
+    # a long depth on at most one round of 128 x 128 tiles: patch matrix written out, then the
+    # eight-wavefront GEMM kernel (ragged in both directions in the second case)
+    (16, 512, 256, 14, 14, 3, 3, S, (1, 1)), (48, 300, 256, 15, 15, 3, 3, S, (2, 2)),
 ]
 
 
