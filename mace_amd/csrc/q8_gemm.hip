@@ -829,7 +829,7 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
   // CONV: what the gather needs per row: top-left input position of the pixel's patch and the
   // lane's chunk offset; gy[j] is the image base.  A 64-byte slab lies inside one filter tap
   // (cin % 64 == 0), so the tap is the same for the whole wavefront.
-  int cv_ih0[CONV ? LY : 1], cv_iw0[CONV ? LY : 1], cv_kc[CONV ? LY : 1];
+  int cv_ih0[CONV ? LY : 1], cv_iw0[CONV ? LY : 1], cv_kc[CONV ? LY : 1], cv_pad[CONV ? LY : 1];
 #pragma unroll
   for (int j = 0; j < LY; ++j) {
     const int row = (j * NW + wave) * RPI + lane / CPR;
@@ -840,7 +840,10 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
       const int oh = t % p.cv_oh, img = t / p.cv_oh;
       cv_ih0[j] = oh * p.cv_sh - p.cv_pt;
       cv_iw0[j] = ow * p.cv_sw - p.cv_pl;
-      cv_kc[j] = kc * 16;
+      // byte offset of the patch's top-left position in its image plus the lane's chunk (32 bits:
+      // host-checked), multiplied out once; the tap's part is wave-uniform
+      cv_kc[j] = (cv_ih0[j] * p.cv_in_w + cv_iw0[j]) * p.cv_cin + kc * 16;
+      cv_pad[j] = kc * 16;
       gy[j] = Yb + (int64_t)img * p.cv_in_h * p.cv_in_w * p.cv_cin;
     } else {
       oy[j] = (uint32_t)(y - y0) * (uint32_t)p.ldy + kc * 16;
@@ -852,8 +855,8 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
       const int kh = tap / p.cv_kw, kw = tap - kh * p.cv_kw;
       const int ih = cv_ih0[j] + kh, iw = cv_iw0[j] + kw;
       const bool inside = (unsigned)ih < (unsigned)p.cv_in_h && (unsigned)iw < (unsigned)p.cv_in_w;
-      const uint8_t *src = gy[j] + ((int64_t)ih * p.cv_in_w + iw) * p.cv_cin + c0 + cv_kc[j];
-      dma_16B(inside ? src : p.cv_zero + cv_kc[j], dst);   // per-lane addresses: the global form
+      const uint8_t *src = gy[j] + (cv_kc[j] + (kh * p.cv_in_w + kw) * p.cv_cin + c0);
+      dma_16B(inside ? src : p.cv_zero + cv_pad[j], dst);   // per-lane addresses: the global form
     } else {
       dma_16B(rsy, oy[j], (uint32_t)k0, dst);
     }
@@ -1465,6 +1468,7 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
   struct Rows {
     const uint8_t *ptr[FY];
     int ih0[CONV ? FY : 1], iw0[CONV ? FY : 1];
+    int off0[CONV ? FY : 1];   // byte offset of the patch's top-left position in its image (32 bits: host-checked)
   };
   auto rows_of = [&](int bk, Rows &r) {
 #pragma unroll
@@ -1476,6 +1480,7 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
         const int oh = t % p.cv_oh, img = t / p.cv_oh;
         r.ih0[j] = oh * p.cv_sh - p.cv_pt;
         r.iw0[j] = ow * p.cv_sw - p.cv_pl;
+        r.off0[j] = (r.ih0[j] * p.cv_in_w + r.iw0[j]) * p.cv_cin;
         r.ptr[j] = Yb + (int64_t)img * p.cv_in_h * p.cv_in_w * p.cv_cin + (G / 2) * h;
       } else {
         r.ptr[j] = Yb + row * p.ldy + (G / 2) * h;
@@ -1487,7 +1492,10 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
     if constexpr (CONV) {
       const int ih = r.ih0[j] + kh, iw = r.iw0[j] + kw;
       const bool inside = (unsigned)ih < (unsigned)p.cv_in_h && (unsigned)iw < (unsigned)p.cv_in_w;
-      const uint8_t *src = r.ptr[j] + ((int64_t)ih * p.cv_in_w + iw) * p.cv_cin + c0;
+      // the tap's offset is the same for the whole wavefront (scalar arithmetic); the per-lane part
+      // was multiplied out once per block (64-bit multiplies per group cost as much as the MFMAs)
+      const int tap = (kh * p.cv_in_w + kw) * p.cv_cin + c0;
+      const uint8_t *src = r.ptr[j] + (r.off0[j] + tap);
       return inside ? src : p.cv_zero + (G / 2) * h;
     } else {
       return r.ptr[j] + (int64_t)g * G;
