@@ -519,6 +519,14 @@ __global__ __launch_bounds__(256) void q8_gemm_fused_small_kernel(GemmParams p, 
   auto fetch = [&](auto t_tag, bool bytewise, const uint8_t *base, int64_t ld, int n, int n0,
                    int k0) -> v4i {
     if (bytewise) {   // uniform over the launch
+      // Nothing of this piece lies inside the operand (a k tile past the depth, asked for ahead of
+      // time, or the pieces past a short depth): a wavefront whose lanes all say so skips the 16
+      // predicated loads and their address arithmetic.
+      if constexpr (decltype(t_tag)::value) {
+        if (k0 + q >= p.K || n0 + c16 >= n) return flip;
+      } else {
+        if (k0 + c16 >= p.K) return flip;
+      }
       uint32_t w[4] = {0, 0, 0, 0};
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
