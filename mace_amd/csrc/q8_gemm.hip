@@ -71,6 +71,10 @@ struct GemmParams {
   // q8_gemm_fused_small_kernel: the operand's rows are not 16-byte pieces (odd depth or row
   // length, unaligned base) and are read byte by byte
   bool x_bytewise, y_bytewise;
+  // ... but in aligned 4-byte groups where the operand allows it (base, row pitch and batch stride
+  // multiples of 4; K % 4 == 0 for k-contiguous rows, n % 4 == 0 for k-major ones; a convolution's
+  // patches: cin % 4 == 0, so that a group lies inside one filter tap)
+  bool x_dword, y_dword;
 };
 
 // XCD-aware tile order: consecutive workgroup ids are dealt round-robin to the 8 XCDs, so
@@ -497,8 +501,14 @@ __global__ __launch_bounds__(WX *WY * 64) void q8_gemm_kernel(GemmParams p, Requ
 // k-major with n % 16 != 0, or an unaligned base) is read byte by byte (x_bytewise / y_bytewise).
 // With p.conv the Y rows are the patches of a convolution, gathered from the NHWC input (16 bytes
 // at a time when cin % 16 == 0, else byte by byte); positions in the padding read the zero point.
-template <typename OutT, bool XT, bool YT>
-__global__ __launch_bounds__(256) void q8_gemm_fused_small_kernel(GemmParams p, RequantTable) {
+// BW: the launch reads an operand byte by byte or in 4-byte groups.  Those loops are long and hold
+// many registers, so they are compiled into kernels of their own, which keep two k tiles in flight
+// instead of four (their depths are short) and are held to 96 registers, i.e. five wavefronts per
+// SIMD: one kernel for both took 104 and ran four, and the byte-wise launches are bound by latency
+// (MobileNet's first convolution at batch 64: 79 us at five wavefronts, 92 at four).  The same bound
+// on the other instantiations makes the k-major ones spill.
+template <typename OutT, bool XT, bool YT, bool BW>
+__global__ __launch_bounds__(256, BW ? 5 : 1) void q8_gemm_fused_small_kernel(GemmParams p, RequantTable) {
   constexpr int T = 64;
   __shared__ __align__(16) uint8_t tile[2][T * LDS_ROW];   // X rows, Y rows: [row][k], sign-flipped
   __shared__ __align__(16) int32_t sc[2 * T + MH_REQUANT_PAIRS_BYTES / 4];
@@ -516,9 +526,9 @@ __global__ __launch_bounds__(256) void q8_gemm_fused_small_kernel(GemmParams p, 
 
   // one 16-byte piece per thread, operand and k tile: row (or k) tid / 4, bytes 16 (tid % 4) ..
   const int q = tid >> 2, c16 = (tid & 3) * 16;
-  auto fetch = [&](auto t_tag, bool bytewise, const uint8_t *base, int64_t ld, int n, int n0,
-                   int k0) -> v4i {
-    if (bytewise) {   // uniform over the launch
+  auto fetch = [&](auto t_tag, bool bytewise, bool dword, const uint8_t *base, int64_t ld, int n,
+                   int n0, int k0) -> v4i {
+    if (BW && bytewise) {   // uniform over the launch
       // Nothing of this piece lies inside the operand (a k tile past the depth, asked for ahead of
       // time, or the pieces past a short depth): a wavefront whose lanes all say so skips the 16
       // predicated loads and their address arithmetic.
@@ -526,6 +536,23 @@ __global__ __launch_bounds__(256) void q8_gemm_fused_small_kernel(GemmParams p, 
         if (k0 + q >= p.K || n0 + c16 >= n) return flip;
       } else {
         if (k0 + c16 >= p.K) return flip;
+      }
+      if (dword) {   // uniform over the launch: every group is wholly inside or wholly outside
+        v4i w4;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          bool ok;
+          const uint8_t *src;
+          if constexpr (decltype(t_tag)::value) {
+            ok = n0 + c16 + 4 * g < n;
+            src = base + (int64_t)(k0 + q) * ld + n0 + c16 + 4 * g;
+          } else {
+            ok = k0 + c16 + 4 * g < p.K;
+            src = base + (int64_t)min(n0 + q, n - 1) * ld + k0 + c16 + 4 * g;
+          }
+          w4[g] = ok ? *(const int *)src : (int)0x80808080;
+        }
+        return w4;
       }
       uint32_t w[4] = {0, 0, 0, 0};
 #pragma unroll
@@ -590,10 +617,29 @@ __global__ __launch_bounds__(256) void q8_gemm_fused_small_kernel(GemmParams p, 
       return cv_img + ((int64_t)ih * p.cv_in_w + iw) * p.cv_cin + c_;
     };
     const int zp4 = (int)p.cv_zp4;
-    if (!p.y_bytewise) {   // cin % 16 == 0: the 16 bytes lie inside one tap
+    if (!BW || !p.y_bytewise) {   // cin % 16 == 0: the 16 bytes lie inside one tap
       bool inside;
       const uint8_t *src = at(kh, kw, c, &inside);
       return inside ? *(const v4i *)src : v4i{zp4, zp4, zp4, zp4};
+    }
+    if (p.y_dword) {   // cin % 4 == 0: each aligned 4-byte group of k lies inside one tap
+      v4i w4;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        int word = (int)0x80808080;
+        if (kk < p.K) {
+          bool inside;
+          const uint8_t *src = at(kh, kw, c, &inside);
+          word = inside ? *(const int *)src : zp4;
+        }
+        w4[g] = word;
+        kk += 4;
+        if ((c += 4) == p.cv_cin) {
+          c = 0;
+          if (++kw == p.cv_kw) { kw = 0; ++kh; }
+        }
+      }
+      return w4;
     }
     uint32_t w[4] = {0, 0, 0, 0};
 #pragma unroll
@@ -615,7 +661,7 @@ __global__ __launch_bounds__(256) void q8_gemm_fused_small_kernel(GemmParams p, 
   };
   auto fetch_y = [&](int k0) -> v4i {
     if (p.conv) return fetch_patch(k0);   // uniform over the launch
-    return fetch(YTag{}, p.y_bytewise, Yb, p.ldy, p.YN, y0, k0);
+    return fetch(YTag{}, p.y_bytewise, p.y_dword, Yb, p.ldy, p.YN, y0, k0);
   };
 
   v16i acc;
@@ -635,11 +681,11 @@ __global__ __launch_bounds__(256) void q8_gemm_fused_small_kernel(GemmParams p, 
 
   // NPRE k tiles of both operands are in flight at a time: with only a few tiles in all, what a
   // call costs is the chain of load round trips, not bandwidth
-  constexpr int NPRE = 4;
+  constexpr int NPRE = BW ? 2 : 4;
   v4i rx[NPRE], ry[NPRE];
 #pragma unroll
   for (int s = 0; s < NPRE; ++s) {
-    rx[s] = fetch(XTag{}, p.x_bytewise, Xb, p.ldx, p.XN, x0, s * BK);   // tiles past K come back as zeros
+    rx[s] = fetch(XTag{}, p.x_bytewise, p.x_dword, Xb, p.ldx, p.XN, x0, s * BK);   // tiles past K come back as zeros
     ry[s] = fetch_y(s * BK);
   }
   for (int kb = 0; kb < p.K; kb += NPRE * BK) {
@@ -651,7 +697,7 @@ __global__ __launch_bounds__(256) void q8_gemm_fused_small_kernel(GemmParams p, 
         park(YTag{}, ry[s], tile[1]);
         __syncthreads();
         if (k0 + NPRE * BK < p.K) {
-          rx[s] = fetch(XTag{}, p.x_bytewise, Xb, p.ldx, p.XN, x0, k0 + NPRE * BK);
+          rx[s] = fetch(XTag{}, p.x_bytewise, p.x_dword, Xb, p.ldx, p.XN, x0, k0 + NPRE * BK);
           ry[s] = fetch_y(k0 + NPRE * BK);
         }
 #pragma unroll
@@ -2289,8 +2335,14 @@ int launch_gemm_fused_small(mace_hip_ctx *ctx, GemmParams &p, const RequantTable
   p.tiles_y = (p.YN + 63) / 64;
   dim3 grid(p.tiles_x * p.tiles_y, 1, batch), block(256);
   MH_PROF_BEGIN(ctx);
-#define MH_FUSED(OutT_, XT_, YT_) \
-  hipLaunchKernelGGL((q8_gemm_fused_small_kernel<OutT_, XT_, YT_>), grid, block, 0, ctx->stream, p, tab)
+  const bool bw = p.x_bytewise || p.y_bytewise;
+#define MH_FUSED(OutT_, XT_, YT_)                                                                 \
+  if (bw)                                                                                         \
+    hipLaunchKernelGGL((q8_gemm_fused_small_kernel<OutT_, XT_, YT_, true>), grid, block, 0,       \
+                       ctx->stream, p, tab);                                                      \
+  else                                                                                            \
+    hipLaunchKernelGGL((q8_gemm_fused_small_kernel<OutT_, XT_, YT_, false>), grid, block, 0,      \
+                       ctx->stream, p, tab)
   switch ((out_u8 ? 4 : 0) | (xt ? 2 : 0) | (yt ? 1 : 0)) {
     case 0: MH_FUSED(int32_t, false, false); break;
     case 1: MH_FUSED(int32_t, false, true); break;
@@ -2595,6 +2647,12 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
       }
       p.x_bytewise = !(xl ? lhs_vec : rhs_vec);
       p.y_bytewise = !(xl ? rhs_vec : lhs_vec);
+      auto by_dwords = [&](const uint8_t *base, int64_t ld, int64_t bs, bool t, int n) {
+        return (uintptr_t)base % 4 == 0 && ld % 4 == 0 && bs % 4 == 0 && (t ? n : p.K) % 4 == 0;
+      };
+      p.x_dword = p.x_bytewise && by_dwords(p.X, p.ldx, p.xbs, xt, p.XN);
+      p.y_dword = p.y_bytewise && (cv ? (uintptr_t)p.Y % 4 == 0 && cv->cin % 4 == 0
+                                      : by_dwords(p.Y, p.ldy, p.ybs, yt, p.YN));
       p.xcoef = xl ? l_coef : r_coef;
       p.xadd = xl ? 0 : r_add;
       p.xbias = xl ? l_bias : nullptr;

@@ -87,6 +87,9 @@ CASES = [  # batch, cout, cin, in_h, in_w, k_h, k_w, padding, strides: the refer
     # a long depth on at most one round of 128 x 128 tiles: patch matrix written out, then the
     # eight-wavefront GEMM kernel (ragged in both directions in the second case)
     (16, 512, 256, 14, 14, 3, 3, S, (1, 1)), (48, 300, 256, 15, 15, 3, 3, S, (2, 2)),
+    # channel counts that are multiples of 4 but not of 16: patches gathered in 4-byte groups
+    (3, 16, 8, 30, 30, 3, 3, S, (1, 1)), (2, 24, 24, 19, 17, 3, 3, S, (2, 1)),
+    (2, 20, 4, 33, 33, 5, 5, Fu, (2, 2)), (1, 24, 12, 9, 9, 3, 3, V, (1, 1)),
 ]
 
 

@@ -54,6 +54,8 @@ SHAPES = [  # batch, rows, depth, cols, lhs_batched, rhs_batched
     (1, 1, 1, 1, True, True), (2, 130, 1000, 70, False, False),
     # aligned in every layout (the one-launch kernel for small problems), one side shared
     (5, 64, 96, 80, False, True), (5, 80, 48, 144, True, False), (3, 16, 1024, 16, True, True),
+    # multiples of 4 that are not multiples of 16 in every extent (read in 4-byte groups)
+    (3, 100, 36, 68, True, True), (2, 52, 100, 44, True, False),
 ]
 
 
