@@ -554,20 +554,31 @@ __global__ __launch_bounds__(256, BW ? 5 : 1) void q8_gemm_fused_small_kernel(Ge
         }
         return w4;
       }
+      // A group of four bytes that lies wholly inside the row is one 4-byte load at whatever
+      // alignment it has (the hardware reads unaligned dwords from global memory); only the group
+      // that straddles the end of the row is read byte by byte.  What a launch of this kind costs
+      // is the number of loads.
       uint32_t w[4] = {0, 0, 0, 0};
+      const uint8_t *src;
+      int left;   // bytes of this piece inside the operand (> 0 after the test above)
+      if constexpr (decltype(t_tag)::value) {
+        src = base + (int64_t)(k0 + q) * ld + n0 + c16;
+        left = n - (n0 + c16);
+      } else {
+        src = base + (int64_t)min(n0 + q, n - 1) * ld + k0 + c16;
+        left = p.K - (k0 + c16);
+      }
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        bool ok;
-        const uint8_t *src;
-        if constexpr (decltype(t_tag)::value) {
-          ok = k0 + q < p.K && n0 + c16 + e < n;
-          src = base + (int64_t)(k0 + q) * ld + n0 + c16 + e;
+      for (int g = 0; g < 4; ++g) {
+        if (4 * g + 4 <= left) {
+          __builtin_memcpy(&w[g], src + 4 * g, 4);
         } else {
-          ok = k0 + c16 + e < p.K;
-          src = base + (int64_t)min(n0 + q, n - 1) * ld + k0 + c16 + e;
+          uint32_t word = 0x80808080u;
+#pragma unroll
+          for (int e = 0; e < 3; ++e)   // a straddling group holds at most three bytes
+            if (4 * g + e < left) word = (word & ~(0xffu << (8 * e))) | ((uint32_t)src[4 * g + e] << (8 * e));
+          w[g] = word;
         }
-        const uint32_t byte = ok ? (uint32_t)*src : 0x80u;
-        w[e / 4] |= byte << (8 * (e % 4));
       }
       return v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
     }
