@@ -122,7 +122,26 @@ __global__ __launch_bounds__(256) void q8_gemv_kernel(GemvParams p) {
       }
     }
   } else {
-    for (int w = lane; w < p.W; w += 64) {
+    // Rows at any alignment and of any width: whole 16-byte pieces through unaligned 16-byte
+    // loads (the hardware reads them from global memory at any address), the last W % 16 bytes
+    // one at a time.
+    const uint4 ones = {0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u};
+    const int nchunk = p.W >> 4;
+    for (int c = lane; c < nchunk; c += 64) {
+      uint4 w0;
+      __builtin_memcpy(&w0, l + (int64_t)c * 16, 16);
+      sum_l = dot16(w0, ones, sum_l);
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        if (b < nb) {
+          uint4 x0;
+          __builtin_memcpy(&x0, r + (int64_t)b * p.rhs_bs + (int64_t)c * 16, 16);
+          dot[b] = dot16(w0, x0, dot[b]);
+          sum_r[b] = dot16(x0, ones, sum_r[b]);
+        }
+      }
+    }
+    for (int w = nchunk * 16 + lane; w < p.W; w += 64) {
       const uint32_t lv = l[w];
       sum_l += lv;
 #pragma unroll
