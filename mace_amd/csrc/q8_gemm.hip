@@ -1891,17 +1891,32 @@ void q8_gemm_stream_kernel(GemmParams p, RequantTable) {
 // ---- repacking ---------------------------------------------------------------------------
 
 // src is k-contiguous already ([n][k], row stride = k) but k is not a multiple of 16 or the
-// base is misaligned: copy into [n][kp] rows padded with 0x80.
+// base is misaligned: copy into [n][kp] rows padded with 0x80.  One thread per 16 bytes of the
+// padded row: a piece that lies wholly inside the source row is one unaligned 16-byte load (the
+// hardware reads those from global memory at any address), the piece at the row end is put
+// together from single bytes.
 __global__ void q8_pack_rows_kernel(const uint8_t *src, int64_t src_bs, uint8_t *dst,
                                     int64_t dst_bs, int n, int k, int kp) {
-  const int64_t total = (int64_t)n * kp;
+  const int cpr = kp >> 4;   // 16-byte pieces per padded row
+  const int64_t total = (int64_t)n * cpr;
   const uint8_t *s = src + (int64_t)blockIdx.z * src_bs;
   uint8_t *d = dst + (int64_t)blockIdx.z * dst_bs;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
        i += (int64_t)gridDim.x * blockDim.x) {
-    const int64_t r = i / kp;
-    const int c = (int)(i - r * kp);
-    d[i] = c < k ? s[r * k + c] : (uint8_t)0x80;
+    const int64_t r = i / cpr;
+    const int c = (int)(i - r * cpr) * 16;   // first byte of the piece inside the row
+    const uint8_t *from = s + r * k + c;
+    const int left = k - c;
+    v4i v;
+    if (left >= 16) {
+      __builtin_memcpy(&v, from, 16);
+    } else {
+      uint32_t w[4] = {0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u};
+      for (int e = 0; e < left; ++e)
+        w[e >> 2] = (w[e >> 2] & ~(0xffu << (8 * (e & 3)))) | ((uint32_t)from[e] << (8 * (e & 3)));
+      v = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+    }
+    *(v4i *)(d + i * 16) = v;
   }
 }
 
@@ -2862,8 +2877,8 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
         hipLaunchKernelGGL(q8_pack_rows4_kernel, grid, dim3(256), 0, ctx->stream, src,
                            n * depth, dst, n * kp, (int)n, (int)depth, (int)kp);
       } else {
-        const int64_t total = n * kp;
-        dim3 grid((unsigned)std::min<int64_t>((total + 255) / 256, 65535), 1, nb);
+        const int64_t total = n * (kp / 16);
+        dim3 grid((unsigned)std::min<int64_t>((total + 255) / 256, 1 << 20), 1, nb);
         hipLaunchKernelGGL(q8_pack_rows_kernel, grid, dim3(256), 0, ctx->stream, src,
                            n * depth, dst, n * kp, (int)n, (int)depth, (int)kp);
       }
