@@ -99,6 +99,81 @@ int mace_hip_graph_destroy(mace_hip_ctx *ctx, mace_hip_graph *graph);
  * the eight-wavefront 128 x 128 kernel and the in-place reading of k-major operands; bit 3: the
  * repack that writes a panel already shifted to int8.  0 restores normal dispatch. */
 int mace_hip_ctx_set_kernel_mask(mace_hip_ctx *ctx, int mask);
+/* ---- kernel plans (test and measurement hook; no counterpart in the reference) ----------------
+ * Which kernel a compute call runs is chosen on the host from the shapes, layouts, alignments and
+ * the device's CU count and LDS size.  The choice is observable: after any compute call,
+ * mace_hip_last_plan reports the family and template variant of the call's main kernel (the one
+ * that does the multiply-accumulate work), the number of kernel launches the call made and which
+ * auxiliary passes (repacks, sum passes, im2col ...) were among them.  A plan-only context
+ * (mace_hip_plan_ctx_create) runs the same host code for a device it only describes -- it needs no
+ * GPU, launches nothing and never touches its pointer arguments -- so the choice can be tested on
+ * a CPU-only machine: pass any non-null addresses with the alignment the case is about.
+ * mace_hip_plan_coverage counts, process-wide, the real launches of every (family, variant). */
+enum {
+  MACE_HIP_KF_NONE = 0,
+  MACE_HIP_KF_Q8_GEMM_FUSED_SMALL,   /* q8_gemm_fused_small_kernel: whole call in one launch      */
+  MACE_HIP_KF_Q8_GEMM_XRES,          /* q8_gemm_xres_kernel: X tile resident in LDS               */
+  MACE_HIP_KF_Q8_GEMM_MID,           /* q8_gemm_mid_kernel: eight wavefronts per 128 x 128 tile   */
+  MACE_HIP_KF_Q8_GEMM_STREAM,        /* q8_gemm_stream_kernel: X panel in registers               */
+  MACE_HIP_KF_Q8_GEMM_RING,          /* q8_gemm_dma_kernel: LDS ring filled by buffer_load..lds   */
+  MACE_HIP_KF_Q8_GEMM_RING_XT,       /* ... 256 x 256, k-major X read in place                    */
+  MACE_HIP_KF_Q8_GEMM_RING_XF,       /* ... 256 x 256, X panel repacked already shifted to int8   */
+  MACE_HIP_KF_Q8_GEMM_TILED,         /* q8_gemm_kernel: register-staged fallback                  */
+  MACE_HIP_KF_Q8_GEMV_ROW,           /* q8_gemv_row_kernel: one weight row per wavefront          */
+  MACE_HIP_KF_Q8_GEMV_SLICE,         /* q8_gemv_mfma_slice_kernel: batch >= 2, rows <= 4 KiB      */
+  MACE_HIP_KF_Q8_GEMV_MFMA_LDS,      /* q8_gemv_mfma_lds_kernel: batch >= 2, wider rows           */
+  MACE_HIP_KF_Q8_GEMV_MFMA,          /* q8_gemv_mfma_kernel: rows too wide for LDS                */
+  MACE_HIP_KF_Q8_GEMV_ROWS,          /* q8_gemv_rows_kernel: vectors of one pass in LDS           */
+  MACE_HIP_KF_Q8_GEMV_GENERAL,       /* q8_gemv_kernel: any width and alignment                   */
+  MACE_HIP_KF_F32_GEMM_VEC,          /* f32_gemm_vec_kernel: 16-byte loads, fp32 MFMA             */
+  MACE_HIP_KF_F32_GEMM_GENERAL,      /* f32_gemm_kernel: bounds-checked                           */
+  MACE_HIP_KF_F32_GEMM_FILL,         /* depth 0: the epilogue alone                               */
+  MACE_HIP_KF_F32_GEMV_VEC,          /* f32_gemv_vec_kernel                                       */
+  MACE_HIP_KF_F32_GEMV_GENERAL,      /* f32_gemv_kernel                                           */
+  MACE_HIP_KF_COUNT
+};
+/* auxiliary passes of a call (bits of mace_hip_plan.aux) */
+enum {
+  MACE_HIP_AUX_PACK_ROWS = 1,            /* k-contiguous operand copied into a padded panel       */
+  MACE_HIP_AUX_PACK_TRANSPOSE = 2,       /* k-major operand transposed into a padded panel        */
+  MACE_HIP_AUX_PACK_SHIFTED = 4,         /* ... written already shifted to int8                   */
+  MACE_HIP_AUX_PANEL_SUMS = 8,           /* row sums of a k-contiguous panel                      */
+  MACE_HIP_AUX_KMAJOR_SUMS = 16,         /* sums over k of a k-major operand                      */
+  MACE_HIP_AUX_ZERO = 32,                /* clearing of a sums buffer                             */
+  MACE_HIP_AUX_IM2COL = 64,              /* patch matrix of a convolution written out             */
+  MACE_HIP_AUX_BIAS_RESCALE = 128,       /* GetBiasData's rescaling                               */
+  MACE_HIP_AUX_F32_PAD = 256,            /* zero-padded copy of an NCHW input                     */
+  MACE_HIP_AUX_FILL = 512,               /* constant fill (zero-point page, empty depth)          */
+  MACE_HIP_AUX_WEIGHT_HIT = 1024,        /* a registered weight's panel / sums were reused        */
+  MACE_HIP_AUX_WEIGHT_BUILD = 2048       /* ... were built by this call                           */
+};
+typedef struct mace_hip_plan {
+  int family;      /* MACE_HIP_KF_*; NONE when the call launched no main kernel (empty result)    */
+  int variant;     /* index of the template instantiation within the family, see
+                      mace_hip_plan_describe; 0 <= variant < mace_hip_plan_variant_count(family)  */
+  int launches;    /* kernel launches of the call, auxiliary passes included                      */
+  int aux;         /* MACE_HIP_AUX_* bits                                                         */
+  int grid[3];     /* launch geometry of the main kernel                                          */
+  int block;
+  int lds_bytes;   /* dynamic LDS of the main kernel                                              */
+} mace_hip_plan;
+/* A context that plans for a device with `cu_count` CUs and `lds_bytes` of LDS per workgroup
+ * (MI355X: 256 and 163840) without using one.  Compute entry points with device-pointer
+ * arguments work on it (and do nothing but plan); the host-pointer variants, the memory helpers,
+ * graphs, timers and the data-dependent Quantize entry points return MACE_HIP_UNSUPPORTED.
+ * Destroy it with mace_hip_ctx_destroy. */
+int mace_hip_plan_ctx_create(int cu_count, int lds_bytes, mace_hip_ctx **out);
+/* Plan of the most recent compute call on this context (plan-only or real). */
+int mace_hip_last_plan(const mace_hip_ctx *ctx, mace_hip_plan *plan);
+/* Number of variant indices of a family, and whether an index names an instantiation the library
+ * can launch (some combinations of template parameters are not built). */
+int mace_hip_plan_variant_count(int family);
+int mace_hip_plan_variant_valid(int family, int variant);
+/* "kernel<template arguments>" of a (family, variant), as a profiler would name it. */
+int mace_hip_plan_describe(int family, int variant, char *buf, size_t len);
+/* Real launches of (family, variant) in this process so far. */
+int64_t mace_hip_plan_coverage(int family, int variant);
+
 /* Test hook, the counterpart of MACE_RUNTIME_FAILURE_RATIO
  * (mace/core/runtime_failure_mock.cc:24-48): the next n arena allocations fail. */
 int mace_hip_ctx_fail_next_allocs(mace_hip_ctx *ctx, int n);
@@ -220,6 +295,14 @@ int mace_hip_matmul_f32(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
 int mace_hip_gemv_f32(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
                       const float *bias /* or NULL */, int64_t batch, int64_t height,
                       int64_t width, int lhs_batched, int rhs_batched, float *out);
+/* The Gemv of FullyConnectedOp<RT_CPU, float>::Run followed by its Activation delegator
+ * (mace/ops/fully_connected.cc:62-75,108-121; mace/ops/ref/activation.cc:61-75): NOOP, RELU =
+ * max(0, v) and RELUX = max(0, min(max_limit, v)) are applied to bias + sum as it is stored;
+ * any other activation type returns MACE_UNSUPPORTED and writes nothing. */
+int mace_hip_gemv_f32_act(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
+                          const float *bias /* or NULL */, int64_t batch, int64_t height,
+                          int64_t width, int lhs_batched, int rhs_batched, int activation,
+                          float max_limit, float *out);
 /* arm::Conv2dK1x1<float>::Compute (mace/ops/arm/base/conv_2d_1x1.cc:27-72) followed by the
  * BiasAdd and Activation delegators as Conv2dOp runs them (mace/ops/conv_2d.cc:171-173):
  * input [n][cin][hw], filter [cout][cin], out [n][cout][hw]. */
@@ -348,6 +431,10 @@ int mace_hip_gemm_f32_host(mace_hip_ctx *ctx, const float *lhs, const float *rhs
 int mace_hip_gemv_f32_host(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
                            const float *bias, int64_t batch, int64_t height, int64_t width,
                            int lhs_batched, int rhs_batched, float *out);
+int mace_hip_gemv_f32_act_host(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
+                               const float *bias, int64_t batch, int64_t height, int64_t width,
+                               int lhs_batched, int rhs_batched, int activation, float max_limit,
+                               float *out);
 int mace_hip_conv1x1_f32_nchw_host(mace_hip_ctx *ctx, const float *input,
                                    const float *filter, const float *bias, int64_t n,
                                    int64_t cin, int64_t hw, int64_t cout, int activation,

@@ -8,6 +8,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <algorithm>
 #include <utility>
 #include <vector>
 
@@ -32,10 +33,15 @@ struct mh_weight {
   std::vector<mh_weight_panel> panels;
 };
 
-inline void mh_weight_drop_panels(mh_weight *w) {
+// Frees what was derived from a weight -- or, while a captured graph may still read it (or on a
+// plan-only context, whose panels are not real memory), hands it to `retired` / forgets it.
+inline void mh_weight_drop_panels(mh_weight *w, bool real_memory, std::vector<void *> *retired) {
   for (mh_weight_panel &c : w->panels) {
-    if (c.panel) (void)hipFree(c.panel);
-    if (c.sums) (void)hipFree(c.sums);
+    for (void *p : {(void *)c.panel, (void *)c.sums}) {
+      if (!p || !real_memory) continue;
+      if (retired) retired->push_back(p);
+      else (void)hipFree(p);
+    }
   }
   w->panels.clear();
 }
@@ -82,6 +88,19 @@ struct mace_hip_ctx {
   // Test hook (mace_hip_ctx_set_kernel_mask): kernel families switched off for this context, so
   // that the tests reach every family on the same shapes.
   int kernel_mask = 0;
+  // What the compute call in progress (or the last one) launches: see mace_hip_last_plan.
+  mace_hip_plan plan = {};
+  int plan_depth = 0;               // nesting of compute entry points (PlanScope)
+  // A context made by mace_hip_plan_ctx_create: every compute entry point runs its host logic
+  // (validation, kernel choice, scratch accounting) and records the plan, but calls nothing of the
+  // HIP runtime and launches nothing.  It needs no GPU.
+  bool plan_only = false;
+  // Instantiated HIP graphs that were captured from this context and still exist: they hold raw
+  // pointers into the arena and the weight cache, so neither may be freed while one is alive.
+  int live_graphs = 0;
+  // device memory (an outgrown arena, panels of an unregistered weight) that such a graph may
+  // still use; freed when the last graph is destroyed or with the context
+  std::vector<void *> retired;
 };
 constexpr int MH_MASK_NO_SMALL = 1, MH_MASK_NO_XRES = 2, MH_MASK_NO_MID = 4, MH_MASK_NO_XFLIP = 8;
 
@@ -107,6 +126,94 @@ int mh_fail(mace_hip_ctx *ctx, int code, const char *fmt, ...);
     int s__ = (expr);                                                                \
     if (s__ != MACE_HIP_SUCCESS) return s__;                                         \
   } while (0)
+
+// ---- kernel plan ----------------------------------------------------------------------------------
+// Every kernel launch of the library goes through MH_KLAUNCH, which counts it in the context's plan
+// and skips it on a plan-only context; the launch of a call's main kernel (the one that does the
+// multiply-accumulate work) is announced with mh_plan_main(family, variant) first.  Variants are
+// dense indices per family, formed next to the template dispatch they mirror, so that
+// "which instantiation ran" is a fact the tests can check (mace_hip_last_plan) and count
+// (mace_hip_plan_coverage).
+void mh_plan_count(int family, int variant);   // process-wide tally of real launches
+inline void mh_plan_reset(mace_hip_ctx *ctx) { ctx->plan = mace_hip_plan{}; }
+inline void mh_plan_main(mace_hip_ctx *ctx, int family, int variant, dim3 grid, dim3 block,
+                         size_t lds) {
+  ctx->plan.family = family;
+  ctx->plan.variant = variant;
+  ctx->plan.grid[0] = (int)grid.x; ctx->plan.grid[1] = (int)grid.y; ctx->plan.grid[2] = (int)grid.z;
+  ctx->plan.block = (int)(block.x * block.y * block.z);
+  ctx->plan.lds_bytes = (int)lds;
+  if (!ctx->plan_only) mh_plan_count(family, variant);
+}
+inline void mh_plan_aux(mace_hip_ctx *ctx, int aux_bit) { ctx->plan.aux |= aux_bit; }
+// Opened by every compute entry point: the outermost one of a call starts a fresh plan (entry points
+// call one another: a host-pointer variant its device-pointer twin, a convolution the GEMM).
+struct PlanScope {
+  mace_hip_ctx *ctx;
+  explicit PlanScope(mace_hip_ctx *c) : ctx(c) { if (ctx->plan_depth++ == 0) mh_plan_reset(ctx); }
+  ~PlanScope() { --ctx->plan_depth; }
+};
+#define MH_KLAUNCH(ctx, ...)                                                                     \
+  do {                                                                                           \
+    ++(ctx)->plan.launches;                                                                      \
+    if (!(ctx)->plan_only) hipLaunchKernelGGL(__VA_ARGS__);                                      \
+  } while (0)
+// after a launch: the runtime's verdict on it (nothing to ask on a plan-only context)
+#define MH_LAUNCH_CHECK(ctx)                                                                     \
+  do {                                                                                           \
+    if (!(ctx)->plan_only) MH_HIP((ctx), hipGetLastError());                                     \
+  } while (0)
+
+// Variant indices: one function per family, used by the launcher that picks the instantiation and
+// decoded by mace_hip_plan_describe / mace_hip_plan_variant_valid (plan.hip).
+namespace mhv {
+inline int fused_small(bool out_u8, bool xt, bool yt, bool bytewise) {
+  return (out_u8 ? 8 : 0) | (xt ? 4 : 0) | (yt ? 2 : 0) | (bytewise ? 1 : 0);
+}
+enum { XRES_PLAIN = 0, XRES_XT = 1, XRES_TAIL = 2, XRES_CONV = 3 };
+inline int xres(int mode, int fx, int fy, int group, bool out_u8) {
+  return ((((mode * 2 + (fx == 4)) * 2 + (fy == 2)) * 2 + (group == 128)) * 2) + (out_u8 ? 1 : 0);
+}
+inline int mid(bool out_u8, bool xt) { return (xt ? 2 : 0) | (out_u8 ? 1 : 0); }
+inline int stream(int fx, int ks) { return (fx - 1) * 2 + (ks - 1); }
+// tile configurations of the ring kernel: <WX, WY, FX, FY, STAGES, OCC, KB>
+enum { RING_1422_3_2 = 0, RING_2222_3_3, RING_2244_2_1_128, RING_2421_2_1_128, RING_2222_2_2_128,
+       RING_2244_4_1, RING_1422_4_2, RING_2222_4_2, RING_2211_4_4, RING_CONFIGS };
+inline int ring_config(int wx, int wy, int fx, int fy, int stages, int occ, int kb) {
+  if (kb == 128) return fx == 4 ? RING_2244_2_1_128 : (wy == 4 ? RING_2421_2_1_128 : RING_2222_2_2_128);
+  if (stages == 3) return wx == 1 ? RING_1422_3_2 : RING_2222_3_3;
+  if (fx == 4) return RING_2244_4_1;
+  if (wx == 1) return RING_1422_4_2;
+  (void)occ;
+  return fx == 2 ? RING_2222_4_2 : RING_2211_4_4;
+}
+inline int ring(int config, bool conv, bool sum_y, bool out_u8) {
+  return config * 8 + (conv ? 4 : 0) + (sum_y ? 2 : 0) + (out_u8 ? 1 : 0);
+}
+inline int ring_xt(bool out_u8, bool sum_y, bool sum_x) {
+  return (sum_x ? 4 : 0) | (sum_y ? 2 : 0) | (out_u8 ? 1 : 0);
+}
+inline int ring_xf(bool out_u8, bool sum_y) { return (sum_y ? 2 : 0) | (out_u8 ? 1 : 0); }
+enum { TILED_BIG = 0, TILED_SKINNY, TILED_MEDIUM, TILED_SMALL };
+inline int tiled(int shape, bool sum_y, bool out_u8) {
+  return shape * 4 + (sum_y ? 2 : 0) + (out_u8 ? 1 : 0);
+}
+inline int log2i(int v) { int l = 0; while ((1 << (l + 1)) <= v) ++l; return l; }
+inline int gemv_row(int u, bool batched, bool whole, bool out_u8) {
+  return ((log2i(u) * 2 + (batched ? 1 : 0)) * 2 + (whole ? 1 : 0)) * 2 + (out_u8 ? 1 : 0);
+}
+inline int gemv_slice(int spw, bool out_u8) { return log2i(spw) * 2 + (out_u8 ? 1 : 0); }
+inline int gemv_out(bool out_u8) { return out_u8 ? 1 : 0; }
+inline int gemv_rows(int nb, bool out_u8) { return log2i(nb) * 2 + (out_u8 ? 1 : 0); }
+inline int gemv_general(int nb, bool vec, bool out_u8) {
+  return (log2i(nb) * 2 + (vec ? 1 : 0)) * 2 + (out_u8 ? 1 : 0);
+}
+inline int f32_gemm_vec(bool split, bool lk, bool rk) {
+  return (split ? 4 : 0) | (lk ? 2 : 0) | (rk ? 1 : 0);
+}
+inline int f32_gemm_general(bool lk, bool rk) { return (lk ? 2 : 0) | (rk ? 1 : 0); }
+inline int f32_gemv_vec(int nb) { return log2i(nb); }
+}  // namespace mhv
 
 // Brackets a kernel launch with the dominant-kernel stopwatch when profiling is enabled.
 #define MH_PROF_RING 512
@@ -424,6 +531,7 @@ inline bool mh_q8_small_problem(const mace_hip_ctx *ctx, int64_t batch, int64_t 
 // Raises a kernel's dynamic LDS limit to at least `bytes`; remembered per context and kernel, since
 // hipFuncSetAttribute costs about as much as a launch and the attribute stays set.
 inline hipError_t mh_allow_big_lds(mace_hip_ctx *ctx, const void *kernel, size_t bytes) {
+  if (ctx->plan_only) return hipSuccess;
   for (auto &e : ctx->big_lds_kernels)
     if (e.first == kernel) {
       if (e.second >= bytes) return hipSuccess;
@@ -441,6 +549,9 @@ inline hipError_t mh_allow_big_lds(mace_hip_ctx *ctx, const void *kernel, size_t
 // How many workgroups of `threads` threads and `lds` bytes of dynamic LDS the runtime fits on one
 // CU for this kernel (registers included); asked once per kernel and size, 1 if the query fails.
 inline int mh_blocks_per_cu(mace_hip_ctx *ctx, const void *kernel, int threads, size_t lds) {
+  // (a plan-only context has no runtime to ask: LDS alone bounds the figure there; it shapes a
+  // grid, never the choice of kernel)
+  if (ctx->plan_only) return (int)std::max<size_t>(1, (size_t)ctx->lds_bytes / std::max<size_t>(lds, 1));
   for (const auto &e : ctx->occupancy)
     if (e.kernel == kernel && e.lds == lds) return e.blocks;
   int n = 0;

@@ -92,9 +92,10 @@ int conv_gemm(mace_hip_ctx *ctx, const uint8_t *filter, const uint8_t *rhs, int6
     int32_t *scaled = (int32_t *)mh_arena_take(ctx, sizeof(int32_t) * cout);
     if (!scaled) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
     volatile float adjust_scale = bias_scale / prod;
-    hipLaunchKernelGGL(q8_bias_rescale_kernel, dim3((unsigned)((cout + 255) / 256)), dim3(256),
+    mh_plan_aux(ctx, MACE_HIP_AUX_BIAS_RESCALE);
+    MH_KLAUNCH(ctx, q8_bias_rescale_kernel, dim3((unsigned)((cout + 255) / 256)), dim3(256),
                        0, ctx->stream, bias, adjust_scale, scaled, (int)cout);
-    MH_HIP(ctx, hipGetLastError());
+    MH_LAUNCH_CHECK(ctx);
     bias_used = scaled;
   }
   Q8GemmEpilogue ep{bias_used, mult, shift, out_zp, clamp_min, clamp_max};
@@ -122,6 +123,7 @@ extern "C" int mace_hip_conv2d_q8_nhwc(mace_hip_ctx *ctx, const uint8_t *input,
                                        float bias_scale, float out_scale, int32_t out_zp,
                                        int clamp_min, int clamp_max, uint8_t *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  PlanScope plan_scope(ctx);
   MH_CHECK(ctx, n >= 0 && in_h >= 0 && in_w >= 0 && cin >= 0 && cout >= 0, "negative dimension");
   MH_CHECK(ctx, k_h >= 1 && k_w >= 1 && stride_h >= 1 && stride_w >= 1, "filter / stride < 1");
   MH_CHECK(ctx, pad_h >= 0 && pad_w >= 0, "negative padding");
@@ -197,17 +199,19 @@ extern "C" int mace_hip_conv2d_q8_nhwc(mace_hip_ctx *ctx, const uint8_t *input,
     if (depth == 0) {
       MH_RETURN_IF_ERROR(mh_fill_bytes(ctx, cols, 0x80, (size_t)columns * kp));
     } else if (fast) {
-      hipLaunchKernelGGL(q8_im2col_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, ctx->stream,
+      mh_plan_aux(ctx, MACE_HIP_AUX_IM2COL);
+      MH_KLAUNCH(ctx, q8_im2col_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, ctx->stream,
                          input, cols, chunks, cpr, (int)kp, (int)depth, (int)in_h, (int)in_w,
                          (int)cin, (int)k_w, stride_h, stride_w, pad_h >> 1, pad_w >> 1,
                          (int)out_h, (int)out_w, zp4);
     } else {
-      hipLaunchKernelGGL(q8_im2col_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, ctx->stream,
+      mh_plan_aux(ctx, MACE_HIP_AUX_IM2COL);
+      MH_KLAUNCH(ctx, q8_im2col_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, ctx->stream,
                          input, cols, chunks, cpr, (int)kp, (int)depth, (int)in_h, (int)in_w,
                          (int)cin, (int)k_w, stride_h, stride_w, pad_h >> 1, pad_w >> 1,
                          (int)out_h, (int)out_w, zp4);
     }
-    MH_HIP(ctx, hipGetLastError());
+    MH_LAUNCH_CHECK(ctx);
     rhs = cols;
     rhs_ld = kp;
   }

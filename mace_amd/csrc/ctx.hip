@@ -42,6 +42,12 @@ int mh_arena_reserve(mace_hip_ctx *ctx, size_t bytes) {
   // headroom for the per-slice alignment
   const size_t need = ctx->arena_used + bytes + 16 * 256;
   if (need <= ctx->arena_bytes) return MACE_HIP_SUCCESS;
+  if (ctx->plan_only) {
+    // nothing is ever read or written through a plan-only context's arena: addresses only
+    ctx->arena = (char *)(uintptr_t)0x100000000ull;
+    ctx->arena_bytes = mh_align_up(need + need / 4, 1 << 20);
+    return MACE_HIP_SUCCESS;
+  }
   if (ctx->no_alloc)
     return mh_fail(ctx, MACE_HIP_INVALID_ARGS,
                    "this call needs %zu bytes of scratch; the allocation-free entry point has %zu",
@@ -59,7 +65,10 @@ int mh_arena_reserve(mace_hip_ctx *ctx, size_t bytes) {
     return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena grown while slices are live");
   MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
   if (ctx->arena) {
-    MH_HIP(ctx, hipFree(ctx->arena));
+    // An instantiated graph captured from this context replays with the old arena's addresses:
+    // while one exists the old arena stays allocated (retired) and only new calls move on.
+    if (ctx->live_graphs > 0) ctx->retired.push_back(ctx->arena);
+    else MH_HIP(ctx, hipFree(ctx->arena));
     ctx->arena = nullptr;
     ctx->arena_bytes = 0;
   }
@@ -93,10 +102,24 @@ __global__ __launch_bounds__(256) void mh_fill_bytes_kernel(uint8_t *dst, uint8_
 int mh_fill_bytes(mace_hip_ctx *ctx, void *dst, uint8_t value, size_t bytes) {
   if (bytes == 0) return MACE_HIP_SUCCESS;
   const size_t blocks = (bytes + 255) / 256;
-  hipLaunchKernelGGL(mh_fill_bytes_kernel, dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256), 0,
-                     ctx->stream, (uint8_t *)dst, value, bytes);
-  MH_HIP(ctx, hipGetLastError());
+  mh_plan_aux(ctx, MACE_HIP_AUX_FILL);
+  MH_KLAUNCH(ctx, mh_fill_bytes_kernel, dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256), 0,
+             ctx->stream, (uint8_t *)dst, value, bytes);
+  MH_LAUNCH_CHECK(ctx);
   return MACE_HIP_SUCCESS;
+}
+
+// Entry points that move data or need a stream have nothing to do on a plan-only context.
+#define MH_NEEDS_GPU(ctx)                                                                       \
+  do {                                                                                          \
+    if ((ctx)->plan_only)                                                                       \
+      return mh_fail((ctx), MACE_HIP_UNSUPPORTED, "%s needs a GPU: this is a plan-only context", \
+                     __func__);                                                                 \
+  } while (0)
+
+static void mh_free_retired(mace_hip_ctx *ctx) {
+  for (void *p : ctx->retired) (void)hipFree(p);
+  ctx->retired.clear();
 }
 
 extern "C" {
@@ -150,10 +173,15 @@ int mace_hip_ctx_create(int device, mace_hip_ctx **out) {
 
 int mace_hip_ctx_destroy(mace_hip_ctx *ctx) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  if (ctx->plan_only) {
+    delete ctx;
+    return MACE_HIP_SUCCESS;
+  }
   (void)hipSetDevice(ctx->device);
   (void)hipStreamSynchronize(ctx->stream);
   if (ctx->arena) (void)hipFree(ctx->arena);
-  for (mh_weight &w : ctx->weights) mh_weight_drop_panels(&w);
+  for (mh_weight &w : ctx->weights) mh_weight_drop_panels(&w, true, nullptr);
+  mh_free_retired(ctx);
   (void)hipEventDestroy(ctx->ev_start);
   (void)hipEventDestroy(ctx->ev_stop);
   for (hipEvent_t e : ctx->prof_ev) (void)hipEventDestroy(e);
@@ -167,8 +195,8 @@ int mace_hip_weight_register(mace_hip_ctx *ctx, const void *device_ptr, size_t b
   MH_CHECK(ctx, device_ptr && bytes > 0, "null or empty weight");
   for (mh_weight &w : ctx->weights)
     if (w.ptr == device_ptr) {   // registered again: whatever was derived from it is stale
-      MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
-      mh_weight_drop_panels(&w);
+      if (!ctx->plan_only) MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
+      mh_weight_drop_panels(&w, !ctx->plan_only, ctx->live_graphs > 0 ? &ctx->retired : nullptr);
       w.bytes = bytes;
       return MACE_HIP_SUCCESS;
     }
@@ -180,8 +208,10 @@ int mace_hip_weight_unregister(mace_hip_ctx *ctx, const void *device_ptr) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   for (size_t i = 0; i < ctx->weights.size(); ++i)
     if (ctx->weights[i].ptr == device_ptr) {
-      MH_HIP(ctx, hipStreamSynchronize(ctx->stream));   // kernels may still read the panels
-      mh_weight_drop_panels(&ctx->weights[i]);
+      // kernels may still read the panels; so may a captured graph, until it is destroyed
+      if (!ctx->plan_only) MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
+      mh_weight_drop_panels(&ctx->weights[i], !ctx->plan_only,
+                            ctx->live_graphs > 0 ? &ctx->retired : nullptr);
       ctx->weights.erase(ctx->weights.begin() + (long)i);
       return MACE_HIP_SUCCESS;
     }
@@ -197,6 +227,7 @@ int mace_hip_weight_cache_stats(mace_hip_ctx *ctx, int64_t *builds, int64_t *hit
 
 int mace_hip_ctx_set_stream(mace_hip_ctx *ctx, void *hip_stream) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
   MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
   ctx->stream = hip_stream ? (hipStream_t)hip_stream : ctx->own_stream;
   return MACE_HIP_SUCCESS;
@@ -204,6 +235,7 @@ int mace_hip_ctx_set_stream(mace_hip_ctx *ctx, void *hip_stream) {
 
 int mace_hip_sync(mace_hip_ctx *ctx) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
   MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
   return MACE_HIP_SUCCESS;
 }
@@ -221,12 +253,14 @@ int mace_hip_device_info(mace_hip_ctx *ctx, char *arch, size_t arch_len, int *cu
 
 int mace_hip_timer_start(mace_hip_ctx *ctx) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
   MH_HIP(ctx, hipEventRecord(ctx->ev_start, ctx->stream));
   return MACE_HIP_SUCCESS;
 }
 
 int mace_hip_timer_stop(mace_hip_ctx *ctx, float *elapsed_ms) {
   if (!ctx || !elapsed_ms) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
   MH_HIP(ctx, hipEventRecord(ctx->ev_stop, ctx->stream));
   MH_HIP(ctx, hipEventSynchronize(ctx->ev_stop));
   MH_HIP(ctx, hipEventElapsedTime(elapsed_ms, ctx->ev_start, ctx->ev_stop));
@@ -235,6 +269,7 @@ int mace_hip_timer_stop(mace_hip_ctx *ctx, float *elapsed_ms) {
 
 int mace_hip_profile_enable(mace_hip_ctx *ctx, int on) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
   if (on && ctx->prof_ev.empty()) {
     ctx->prof_ev.reserve(2 * MH_PROF_RING);
     for (int i = 0; i < 2 * MH_PROF_RING; ++i) {
@@ -281,6 +316,7 @@ struct mace_hip_graph {
 
 int mace_hip_graph_capture_begin(mace_hip_ctx *ctx) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
   MH_CHECK(ctx, !ctx->capturing, "a capture is already in progress on this context");
   MH_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
   ctx->capturing = true;
@@ -305,11 +341,13 @@ int mace_hip_graph_capture_end(mace_hip_ctx *ctx, mace_hip_graph **out) {
     MH_HIP(ctx, e);
   }
   *out = h;
+  ++ctx->live_graphs;
   return MACE_HIP_SUCCESS;
 }
 
 int mace_hip_graph_launch(mace_hip_ctx *ctx, mace_hip_graph *graph) {
   if (!ctx || !graph || !graph->exec) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
   MH_CHECK(ctx, !ctx->capturing, "a capture is in progress on this context");
   MH_HIP(ctx, hipGraphLaunch(graph->exec, ctx->stream));
   return MACE_HIP_SUCCESS;
@@ -322,6 +360,8 @@ int mace_hip_graph_destroy(mace_hip_ctx *ctx, mace_hip_graph *graph) {
   if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
   if (graph->graph) (void)hipGraphDestroy(graph->graph);
   delete graph;
+  // memory that was kept only because a graph might still replay with its address
+  if (ctx->live_graphs > 0 && --ctx->live_graphs == 0) mh_free_retired(ctx);
   return MACE_HIP_SUCCESS;
 }
 
@@ -339,6 +379,7 @@ int mace_hip_ctx_fail_next_allocs(mace_hip_ctx *ctx, int n) {
 
 int mace_hip_malloc(mace_hip_ctx *ctx, size_t bytes, void **dev_ptr) {
   if (!ctx || !dev_ptr) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
   *dev_ptr = nullptr;
   if (bytes == 0) return MACE_HIP_SUCCESS;
   hipError_t e = hipMalloc(dev_ptr, bytes);
@@ -352,6 +393,7 @@ int mace_hip_malloc(mace_hip_ctx *ctx, size_t bytes, void **dev_ptr) {
 
 int mace_hip_free(mace_hip_ctx *ctx, void *dev_ptr) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
   if (!dev_ptr) return MACE_HIP_SUCCESS;
   MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
   MH_HIP(ctx, hipFree(dev_ptr));
@@ -360,6 +402,7 @@ int mace_hip_free(mace_hip_ctx *ctx, void *dev_ptr) {
 
 int mace_hip_memcpy_h2d(mace_hip_ctx *ctx, void *dst, const void *src, size_t bytes) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
   if (bytes == 0) return MACE_HIP_SUCCESS;
   MH_HIP(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
   MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
@@ -368,6 +411,7 @@ int mace_hip_memcpy_h2d(mace_hip_ctx *ctx, void *dst, const void *src, size_t by
 
 int mace_hip_memcpy_d2h(mace_hip_ctx *ctx, void *dst, const void *src, size_t bytes) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
   if (bytes == 0) return MACE_HIP_SUCCESS;
   MH_HIP(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
   MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
@@ -460,6 +504,7 @@ int mace_hip_gemm_f32_host(mace_hip_ctx *ctx, const float *lhs, const float *rhs
                            int lhs_major, int rhs_major, int out_major, int lhs_batched,
                            int rhs_batched, float *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
   MH_CHECK(ctx, nonneg(batch, rows, cols, depth), "negative dimension");
   const size_t lb = sizeof(float) * (lhs_batched ? batch : 1) * rows * depth;
   const size_t rb = sizeof(float) * (rhs_batched ? batch : 1) * depth * cols;
@@ -479,7 +524,16 @@ int mace_hip_gemm_f32_host(mace_hip_ctx *ctx, const float *lhs, const float *rhs
 int mace_hip_gemv_f32_host(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
                            const float *bias, int64_t batch, int64_t height, int64_t width,
                            int lhs_batched, int rhs_batched, float *out) {
+  return mace_hip_gemv_f32_act_host(ctx, lhs, rhs, bias, batch, height, width, lhs_batched,
+                                    rhs_batched, MACE_HIP_ACT_NOOP, 0.f, out);
+}
+
+int mace_hip_gemv_f32_act_host(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
+                               const float *bias, int64_t batch, int64_t height, int64_t width,
+                               int lhs_batched, int rhs_batched, int activation, float max_limit,
+                               float *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
   MH_CHECK(ctx, nonneg(batch, height, width, 0), "negative dimension");
   const size_t lb = sizeof(float) * (lhs_batched ? batch : 1) * height * width;
   const size_t rb = sizeof(float) * (rhs_batched ? batch : 1) * width;
@@ -492,9 +546,9 @@ int mace_hip_gemv_f32_host(mace_hip_ctx *ctx, const float *lhs, const float *rhs
   MH_RETURN_IF_ERROR(st.in(rhs, rb, &dr));
   MH_RETURN_IF_ERROR(st.in(bias, bb, &db));
   MH_RETURN_IF_ERROR(st.out(ob, &dout));
-  MH_RETURN_IF_ERROR(mace_hip_gemv_f32(ctx, (const float *)dl, (const float *)dr,
-                                       (const float *)db, batch, height, width, lhs_batched,
-                                       rhs_batched, (float *)dout));
+  MH_RETURN_IF_ERROR(mace_hip_gemv_f32_act(ctx, (const float *)dl, (const float *)dr,
+                                           (const float *)db, batch, height, width, lhs_batched,
+                                           rhs_batched, activation, max_limit, (float *)dout));
   return st.back(out, dout, ob);
 }
 
@@ -503,6 +557,7 @@ int mace_hip_conv1x1_f32_nchw_host(mace_hip_ctx *ctx, const float *input,
                                    int64_t cin, int64_t hw, int64_t cout, int activation,
                                    float max_limit, float *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
   MH_CHECK(ctx, nonneg(n, cin, hw, cout), "negative dimension");
   const size_t ib = sizeof(float) * n * cin * hw;
   const size_t fb = sizeof(float) * cout * cin;
@@ -526,6 +581,7 @@ int mace_hip_matmul_f32_host(mace_hip_ctx *ctx, const float *lhs, const float *r
                              int64_t rhs_rows, int64_t rhs_cols, int transpose_lhs,
                              int transpose_rhs, int lhs_batched, int rhs_batched, float *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
   MH_CHECK(ctx, nonneg(batch, lhs_rows, lhs_cols, 0) && nonneg(rhs_rows, rhs_cols, 0, 0),
            "negative dimension");
   const int64_t rows = transpose_lhs ? lhs_cols : lhs_rows;
@@ -555,6 +611,7 @@ int mace_hip_conv2d_f32_nchw_host(mace_hip_ctx *ctx, const float *input, const f
                                   int pad_h, int pad_w, int activation, float max_limit,
                                   float *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
   MH_CHECK(ctx, nonneg(n, cin, in_h, in_w) && nonneg(cout, k_h, k_w, 0) && pad_h >= 0 && pad_w >= 0,
            "negative dimension");
   if (k_h != 1 || k_w != 1 || stride_h != 1 || stride_w != 1 || dilation_h != 1 || dilation_w != 1)
@@ -586,6 +643,7 @@ int mace_hip_gemv_q8_u8_host(mace_hip_ctx *ctx, const uint8_t *lhs, const uint8_
                              float out_scale, int32_t out_zp, int requant_mode,
                              uint8_t *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
   MH_CHECK(ctx, nonneg(batch, height, width, 0), "negative dimension");
   const size_t lb = (size_t)(lhs_batched ? batch : 1) * height * width;
   const size_t rb = (size_t)(rhs_batched ? batch : 1) * width;
@@ -611,6 +669,7 @@ int mace_hip_gemv_q8_i32_host(mace_hip_ctx *ctx, const uint8_t *lhs, const uint8
                               int64_t width, int lhs_batched, int rhs_batched,
                               int32_t lhs_zp, int32_t rhs_zp, int32_t *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
   MH_CHECK(ctx, nonneg(batch, height, width, 0), "negative dimension");
   const size_t lb = (size_t)(lhs_batched ? batch : 1) * height * width;
   const size_t rb = (size_t)(rhs_batched ? batch : 1) * width;
@@ -636,6 +695,7 @@ int mace_hip_gemm_q8_i32_host(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_ord
                               int64_t cols, int lhs_batched, int rhs_batched,
                               int32_t lhs_offset, int32_t rhs_offset) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
   MH_CHECK(ctx, nonneg(batch, rows, depth, cols), "negative dimension");
   const size_t lb = (size_t)(lhs_batched ? batch : 1) * rows * depth;
   const size_t rb = (size_t)(rhs_batched ? batch : 1) * depth * cols;
@@ -662,6 +722,7 @@ int mace_hip_gemm_q8_u8_host(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_orde
                              int right_shift, int32_t offset_after_shift, int clamp_min,
                              int clamp_max) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
   MH_CHECK(ctx, nonneg(batch, rows, depth, cols), "negative dimension");
   const size_t lb = (size_t)(lhs_batched ? batch : 1) * rows * depth;
   const size_t rb = (size_t)(rhs_batched ? batch : 1) * depth * cols;
@@ -692,6 +753,7 @@ int mace_hip_gemm_q8_u8_noalloc(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_o
                                 int right_shift, int32_t offset_after_shift, int clamp_min,
                                 int clamp_max) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  PlanScope plan_scope(ctx);
   MH_CHECK(ctx, ctx->arena_used == 0 && !ctx->no_alloc, "another call is in progress on this context");
   // For the length of this call the arena is this GPU's static array: the repacked panels and
   // the correction vectors go there, the kernels are the ones mace_hip_gemm_q8_u8 launches.
@@ -720,6 +782,7 @@ int mace_hip_conv1x1_q8_nhwc_host(mace_hip_ctx *ctx, const uint8_t *input,
                                   int32_t out_zp, int clamp_min, int clamp_max,
                                   uint8_t *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
   MH_CHECK(ctx, nonneg(n, h, w, 0) && nonneg(cin, cout, 0, 0), "negative dimension");
   const int64_t pix = n * h * w;
   const size_t ib = (size_t)pix * cin, fb = (size_t)cout * cin;
@@ -748,6 +811,7 @@ int mace_hip_conv2d_q8_nhwc_host(mace_hip_ctx *ctx, const uint8_t *input, const 
                                  int32_t filter_zp, float bias_scale, float out_scale,
                                  int32_t out_zp, int clamp_min, int clamp_max, uint8_t *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
   MH_CHECK(ctx, nonneg(n, in_h, in_w, 0) && nonneg(cin, cout, 0, 0), "negative dimension");
   MH_CHECK(ctx, k_h >= 1 && k_w >= 1 && stride_h >= 1 && stride_w >= 1 && pad_h >= 0 &&
                     pad_w >= 0, "filter / stride < 1 or negative padding");

@@ -365,6 +365,8 @@ struct F32GemvParams {
   float *out;
   int64_t lbs, rbs;
   int H, W;
+  int act;        // applied to the finished sum as it is stored (FullyConnected's Activation)
+  float limit;
 };
 
 __global__ __launch_bounds__(256) void f32_gemv_kernel(F32GemvParams p) {
@@ -386,7 +388,7 @@ __global__ __launch_bounds__(256) void f32_gemv_kernel(F32GemvParams p) {
   float s = (s0 + s1) + (s2 + s3);
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
-  if (lane == 0) p.out[(int64_t)b * p.H + h] = (p.bias ? p.bias[h] : 0.f) + s;
+  if (lane == 0) p.out[(int64_t)b * p.H + h] = apply_act((p.bias ? p.bias[h] : 0.f) + s, p.act, p.limit);
 }
 
 // The same with 16-byte loads (W % 4 == 0, aligned bases), four weight loads in flight per lane
@@ -435,7 +437,8 @@ __global__ __launch_bounds__(256) void f32_gemv_vec_kernel(F32GemvParams p, int 
     float t = (s[j][0] + s[j][1]) + (s[j][2] + s[j][3]);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) t += __shfl_xor(t, off, 64);
-    if (lane == 0 && b0 + j < batch) p.out[(int64_t)(b0 + j) * p.H + h] = (p.bias ? p.bias[h] : 0.f) + t;
+    if (lane == 0 && b0 + j < batch)
+      p.out[(int64_t)(b0 + j) * p.H + h] = apply_act((p.bias ? p.bias[h] : 0.f) + t, p.act, p.limit);
   }
 }
 
@@ -468,9 +471,10 @@ int mh_f32_gemm(mace_hip_ctx *ctx, const float *lhs, const float *rhs, int64_t b
   p.bias_row = ep.bias_row; p.bias_col = ep.bias_col; p.act = ep.act; p.limit = ep.limit;
   if (depth == 0) {
     const int64_t total = batch * rows * cols;
-    hipLaunchKernelGGL(f32_fill_kernel, dim3((unsigned)((total + 255) / 256 > 65535 ? 65535 : (total + 255) / 256)),
+    mh_plan_main(ctx, MACE_HIP_KF_F32_GEMM_FILL, 0, dim3(1), dim3(256), 0);
+    MH_KLAUNCH(ctx, f32_fill_kernel, dim3((unsigned)((total + 255) / 256 > 65535 ? 65535 : (total + 255) / 256)),
                        dim3(256), 0, ctx->stream, p, total);
-    MH_HIP(ctx, hipGetLastError());
+    MH_LAUNCH_CHECK(ctx);
     return MACE_HIP_SUCCESS;
   }
   p.tiles_m = (p.M + TM - 1) / TM;
@@ -481,26 +485,29 @@ int mh_f32_gemm(mace_hip_ctx *ctx, const float *lhs, const float *rhs, int64_t b
   const bool split = tiles * batch <= cus;   // at most one tile per CU
   const bool lk = lhs_major == MACE_HIP_ROW_MAJOR;   // depth contiguous
   const bool rk = rhs_major == MACE_HIP_COL_MAJOR;
-  MH_PROF_BEGIN(ctx);
   // 16-byte pieces: whole k tiles; an operand whose rows run along k may have any number of rows
   // (a ragged last tile re-reads its last row), one that runs along m / n needs them in fours
   const bool vec = depth % TK == 0 && (lk || rows % 4 == 0) && (rk || cols % 4 == 0) &&
                    rows >= 4 && cols >= 4 && ((uintptr_t)lhs % 16 == 0) &&
                    ((uintptr_t)rhs % 16 == 0);
-  if (vec && split && lk && rk) hipLaunchKernelGGL((f32_gemm_vec_kernel<true, true, 2>), grid, block2, 0, ctx->stream, p);
-  else if (vec && split && lk) hipLaunchKernelGGL((f32_gemm_vec_kernel<true, false, 2>), grid, block2, 0, ctx->stream, p);
-  else if (vec && split && rk) hipLaunchKernelGGL((f32_gemm_vec_kernel<false, true, 2>), grid, block2, 0, ctx->stream, p);
-  else if (vec && split) hipLaunchKernelGGL((f32_gemm_vec_kernel<false, false, 2>), grid, block2, 0, ctx->stream, p);
-  else if (vec && lk && rk) hipLaunchKernelGGL((f32_gemm_vec_kernel<true, true, 1>), grid, block, 0, ctx->stream, p);
-  else if (vec && lk) hipLaunchKernelGGL((f32_gemm_vec_kernel<true, false, 1>), grid, block, 0, ctx->stream, p);
-  else if (vec && rk) hipLaunchKernelGGL((f32_gemm_vec_kernel<false, true, 1>), grid, block, 0, ctx->stream, p);
-  else if (vec) hipLaunchKernelGGL((f32_gemm_vec_kernel<false, false, 1>), grid, block, 0, ctx->stream, p);
-  else if (lk && rk) hipLaunchKernelGGL((f32_gemm_kernel<true, true>), grid, block, 0, ctx->stream, p);
-  else if (lk) hipLaunchKernelGGL((f32_gemm_kernel<true, false>), grid, block, 0, ctx->stream, p);
-  else if (rk) hipLaunchKernelGGL((f32_gemm_kernel<false, true>), grid, block, 0, ctx->stream, p);
-  else hipLaunchKernelGGL((f32_gemm_kernel<false, false>), grid, block, 0, ctx->stream, p);
+  if (vec) mh_plan_main(ctx, MACE_HIP_KF_F32_GEMM_VEC, mhv::f32_gemm_vec(split, lk, rk), grid,
+                        split ? block2 : block, 0);
+  else mh_plan_main(ctx, MACE_HIP_KF_F32_GEMM_GENERAL, mhv::f32_gemm_general(lk, rk), grid, block, 0);
+  MH_PROF_BEGIN(ctx);
+  if (vec && split && lk && rk) MH_KLAUNCH(ctx, (f32_gemm_vec_kernel<true, true, 2>), grid, block2, 0, ctx->stream, p);
+  else if (vec && split && lk) MH_KLAUNCH(ctx, (f32_gemm_vec_kernel<true, false, 2>), grid, block2, 0, ctx->stream, p);
+  else if (vec && split && rk) MH_KLAUNCH(ctx, (f32_gemm_vec_kernel<false, true, 2>), grid, block2, 0, ctx->stream, p);
+  else if (vec && split) MH_KLAUNCH(ctx, (f32_gemm_vec_kernel<false, false, 2>), grid, block2, 0, ctx->stream, p);
+  else if (vec && lk && rk) MH_KLAUNCH(ctx, (f32_gemm_vec_kernel<true, true, 1>), grid, block, 0, ctx->stream, p);
+  else if (vec && lk) MH_KLAUNCH(ctx, (f32_gemm_vec_kernel<true, false, 1>), grid, block, 0, ctx->stream, p);
+  else if (vec && rk) MH_KLAUNCH(ctx, (f32_gemm_vec_kernel<false, true, 1>), grid, block, 0, ctx->stream, p);
+  else if (vec) MH_KLAUNCH(ctx, (f32_gemm_vec_kernel<false, false, 1>), grid, block, 0, ctx->stream, p);
+  else if (lk && rk) MH_KLAUNCH(ctx, (f32_gemm_kernel<true, true>), grid, block, 0, ctx->stream, p);
+  else if (lk) MH_KLAUNCH(ctx, (f32_gemm_kernel<true, false>), grid, block, 0, ctx->stream, p);
+  else if (rk) MH_KLAUNCH(ctx, (f32_gemm_kernel<false, true>), grid, block, 0, ctx->stream, p);
+  else MH_KLAUNCH(ctx, (f32_gemm_kernel<false, false>), grid, block, 0, ctx->stream, p);
   MH_PROF_END(ctx);
-  MH_HIP(ctx, hipGetLastError());
+  MH_LAUNCH_CHECK(ctx);
   return MACE_HIP_SUCCESS;
 }
 
@@ -511,6 +518,7 @@ int mace_hip_gemm_f32(mace_hip_ctx *ctx, const float *lhs, const float *rhs, int
                       int rhs_major, int out_major, int lhs_batched, int rhs_batched,
                       float *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  PlanScope plan_scope(ctx);
   F32Epilogue ep{nullptr, nullptr, MACE_HIP_ACT_NOOP, 0.f};
   return mh_f32_gemm(ctx, lhs, rhs, batch, rows, cols, depth, lhs_major, rhs_major, out_major,
                      lhs_batched, rhs_batched, out, ep);
@@ -521,6 +529,7 @@ int mace_hip_matmul_f32(mace_hip_ctx *ctx, const float *lhs, const float *rhs, c
                         int64_t rhs_cols, int transpose_lhs, int transpose_rhs, int lhs_batched,
                         int rhs_batched, float *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  PlanScope plan_scope(ctx);
   // mace/ops/ref/gemm.cc:122-131, then mace/ops/matmul.cc:195-211: c[i * cols + w] += bias[w],
   // i.e. one binary32 addition to the finished sum, done here as the sum is stored
   const int64_t rows = transpose_lhs ? lhs_cols : lhs_rows;
@@ -543,6 +552,7 @@ int mace_hip_gemm_f32_transpose(mace_hip_ctx *ctx, const float *lhs, const float
                                 int transpose_rhs, int transpose_out, int lhs_batched,
                                 int rhs_batched, float *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  PlanScope plan_scope(ctx);
   // mace/ops/ref/gemm.cc:122-131
   const int64_t rows = transpose_lhs ? lhs_cols : lhs_rows;
   const int64_t depth = transpose_lhs ? lhs_rows : lhs_cols;
@@ -561,30 +571,43 @@ int mace_hip_gemm_f32_transpose(mace_hip_ctx *ctx, const float *lhs, const float
 int mace_hip_gemv_f32(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
                       const float *bias, int64_t batch, int64_t height, int64_t width,
                       int lhs_batched, int rhs_batched, float *out) {
+  return mace_hip_gemv_f32_act(ctx, lhs, rhs, bias, batch, height, width, lhs_batched, rhs_batched,
+                               MACE_HIP_ACT_NOOP, 0.f, out);
+}
+
+int mace_hip_gemv_f32_act(mace_hip_ctx *ctx, const float *lhs, const float *rhs,
+                          const float *bias, int64_t batch, int64_t height, int64_t width,
+                          int lhs_batched, int rhs_batched, int activation, float max_limit,
+                          float *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  PlanScope plan_scope(ctx);
+  if (activation < MACE_HIP_ACT_NOOP || activation > MACE_HIP_ACT_RELUX)
+    return mh_fail(ctx, MACE_HIP_UNSUPPORTED, "activation %d is not applied by this library", activation);
   MH_CHECK(ctx, batch >= 0 && height >= 0 && width >= 0, "negative dimension");
   MH_CHECK(ctx, height < (1ll << 31) && width < (1ll << 31) && batch <= 65535,
            "dimension too large");
   if (batch == 0 || height == 0) return MACE_HIP_SUCCESS;
   MH_CHECK(ctx, out && (width == 0 || (lhs && rhs)), "null operand");
   F32GemvParams p{lhs, rhs, bias, out, lhs_batched ? height * width : 0,
-                  rhs_batched ? width : 0, (int)height, (int)width};
+                  rhs_batched ? width : 0, (int)height, (int)width, activation, max_limit};
   dim3 grid((unsigned)((height + 3) / 4), (unsigned)batch);
-  MH_PROF_BEGIN(ctx);
   const bool vec = width % 4 == 0 && (uintptr_t)lhs % 16 == 0 && (uintptr_t)rhs % 16 == 0;
-  if (vec && !lhs_batched && rhs_batched && batch >= 2) {
-    // shared weights: up to four vectors per pass
-    const int nb = batch >= 3 ? 4 : 2;
-    grid.y = (unsigned)((batch + nb - 1) / nb);
-    if (nb == 4) hipLaunchKernelGGL(f32_gemv_vec_kernel<4>, grid, dim3(256), 0, ctx->stream, p, (int)batch);
-    else hipLaunchKernelGGL(f32_gemv_vec_kernel<2>, grid, dim3(256), 0, ctx->stream, p, (int)batch);
+  const bool shared = vec && !lhs_batched && rhs_batched && batch >= 2;
+  const int nb = shared ? (batch >= 3 ? 4 : 2) : 1;   // shared weights: up to four vectors per pass
+  if (shared) grid.y = (unsigned)((batch + nb - 1) / nb);
+  if (vec) mh_plan_main(ctx, MACE_HIP_KF_F32_GEMV_VEC, mhv::f32_gemv_vec(nb), grid, dim3(256), 0);
+  else mh_plan_main(ctx, MACE_HIP_KF_F32_GEMV_GENERAL, 0, grid, dim3(256), 0);
+  MH_PROF_BEGIN(ctx);
+  if (shared) {
+    if (nb == 4) MH_KLAUNCH(ctx, f32_gemv_vec_kernel<4>, grid, dim3(256), 0, ctx->stream, p, (int)batch);
+    else MH_KLAUNCH(ctx, f32_gemv_vec_kernel<2>, grid, dim3(256), 0, ctx->stream, p, (int)batch);
   } else if (vec) {
-    hipLaunchKernelGGL(f32_gemv_vec_kernel<1>, grid, dim3(256), 0, ctx->stream, p, (int)batch);
+    MH_KLAUNCH(ctx, f32_gemv_vec_kernel<1>, grid, dim3(256), 0, ctx->stream, p, (int)batch);
   } else {
-    hipLaunchKernelGGL(f32_gemv_kernel, grid, dim3(256), 0, ctx->stream, p);
+    MH_KLAUNCH(ctx, f32_gemv_kernel, grid, dim3(256), 0, ctx->stream, p);
   }
   MH_PROF_END(ctx);
-  MH_HIP(ctx, hipGetLastError());
+  MH_LAUNCH_CHECK(ctx);
   return MACE_HIP_SUCCESS;
 }
 
@@ -592,6 +615,7 @@ int mace_hip_conv1x1_f32_nchw(mace_hip_ctx *ctx, const float *input, const float
                               const float *bias, int64_t n, int64_t cin, int64_t hw,
                               int64_t cout, int activation, float max_limit, float *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  PlanScope plan_scope(ctx);
   MH_CHECK(ctx, activation >= MACE_HIP_ACT_NOOP && activation <= MACE_HIP_ACT_RELUX,
            "unsupported activation %d", activation);
   // mace/ops/arm/base/conv_2d_1x1.cc:66-68: Gemm(filter, input, batch, cout, cin, cin, hw,
@@ -608,6 +632,7 @@ int mace_hip_conv2d_f32_nchw(mace_hip_ctx *ctx, const float *input, const float 
                              int dilation_h, int dilation_w, int pad_h, int pad_w, int activation,
                              float max_limit, float *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  PlanScope plan_scope(ctx);
   MH_CHECK(ctx, n >= 0 && cin >= 0 && in_h >= 0 && in_w >= 0 && cout >= 0, "negative dimension");
   MH_CHECK(ctx, k_h >= 1 && k_w >= 1 && stride_h >= 1 && stride_w >= 1 && dilation_h >= 1 &&
                     dilation_w >= 1 && pad_h >= 0 && pad_w >= 0,
@@ -633,10 +658,11 @@ int mace_hip_conv2d_f32_nchw(mace_hip_ctx *ctx, const float *input, const float 
   float *padded = (float *)mh_arena_take(ctx, sizeof(float) * (size_t)total);
   if (!padded) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
   const int64_t blocks = (total + 255) / 256;
-  hipLaunchKernelGGL(f32_pad_nchw_kernel, dim3((unsigned)(blocks < 65535 ? blocks : 65535)),
+  mh_plan_aux(ctx, MACE_HIP_AUX_F32_PAD);
+  MH_KLAUNCH(ctx, f32_pad_nchw_kernel, dim3((unsigned)(blocks < 65535 ? blocks : 65535)),
                      dim3(256), 0, ctx->stream, input, padded, total, (int)in_h, (int)in_w,
                      (int)ph, (int)pw, pad_h >> 1, pad_w >> 1);
-  MH_HIP(ctx, hipGetLastError());
+  MH_LAUNCH_CHECK(ctx);
   return mace_hip_conv1x1_f32_nchw(ctx, padded, filter, bias, n, cin, ph * pw, cout, activation,
                                    max_limit, out);
 }

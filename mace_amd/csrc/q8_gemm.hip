@@ -2123,8 +2123,9 @@ int launch_panel_sums(mace_hip_ctx *ctx, const uint8_t *P, int64_t ld, int64_t p
   MH_CHECK(ctx, blocks < (1ll << 31), "panel too tall");
   dim3 grid((unsigned)blocks, 1, nb), block(256);
 #define MH_SUMS(L_)                                                                       \
-  hipLaunchKernelGGL((q8_panel_sums_kernel<L_>), grid, block, 0, ctx->stream, P, ld, pbs, \
-                     (int)n, k, sums, zero, zero_n)
+  MH_KLAUNCH(ctx, (q8_panel_sums_kernel<L_>), grid, block, 0, ctx->stream, P, ld, pbs, \
+             (int)n, k, sums, zero, zero_n)
+  mh_plan_aux(ctx, MACE_HIP_AUX_PANEL_SUMS);
   switch (lpr) {
     case 1: MH_SUMS(1); break;
     case 2: MH_SUMS(2); break;
@@ -2135,7 +2136,7 @@ int launch_panel_sums(mace_hip_ctx *ctx, const uint8_t *P, int64_t ld, int64_t p
     default: MH_SUMS(64); break;
   }
 #undef MH_SUMS
-  MH_HIP(ctx, hipGetLastError());
+  MH_LAUNCH_CHECK(ctx);
   return MACE_HIP_SUCCESS;
 }
 
@@ -2185,17 +2186,18 @@ __global__ __launch_bounds__(256) void q8_kmajor_sums_kernel(const uint8_t *P, i
 int launch_kmajor_sums(mace_hip_ctx *ctx, const uint8_t *P, int64_t ld, int64_t pbs, int64_t n,
                        int64_t k, int nb, int32_t *sums) {
   const int64_t cnt = (int64_t)nb * n;
-  hipLaunchKernelGGL(q8_zero_i32_kernel, dim3((unsigned)((cnt + 255) / 256)), dim3(256), 0, ctx->stream,
-                     sums, cnt);
+  mh_plan_aux(ctx, MACE_HIP_AUX_ZERO | MACE_HIP_AUX_KMAJOR_SUMS);
+  MH_KLAUNCH(ctx, q8_zero_i32_kernel, dim3((unsigned)((cnt + 255) / 256)), dim3(256), 0, ctx->stream,
+             sums, cnt);
   const int gx = (int)((n + 255) / 256);
   const int64_t cu = ctx->cu_count > 0 ? ctx->cu_count : 256;
   // about four workgroups per CU, at most 4096 rows each (256 per thread: the 16-bit halves hold)
   const int64_t want = std::max<int64_t>(1, 4 * cu / std::max<int64_t>(1, (int64_t)gx * nb));
   const int rpb = (int)std::min<int64_t>(4096, std::max<int64_t>(64, (k + want - 1) / want));
   dim3 grid((unsigned)gx, (unsigned)((k + rpb - 1) / rpb), (unsigned)nb);
-  hipLaunchKernelGGL(q8_kmajor_sums_kernel, grid, dim3(256), 0, ctx->stream, P, ld, pbs, (int)n, (int)k,
+  MH_KLAUNCH(ctx, q8_kmajor_sums_kernel, grid, dim3(256), 0, ctx->stream, P, ld, pbs, (int)n, (int)k,
                      rpb, sums);
-  MH_HIP(ctx, hipGetLastError());
+  MH_LAUNCH_CHECK(ctx);
   return MACE_HIP_SUCCESS;
 }
 
@@ -2207,10 +2209,13 @@ int launch_gemm(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, bool 
   p.tiles_y = (p.YN + TY - 1) / TY;
   const size_t lds = 2 * (size_t)(TX + TY) * LDS_ROW;
   dim3 grid(p.tiles_x * p.tiles_y, 1, batch), block(WX * WY * 64);
+  constexpr int shape = FX == 4 ? mhv::TILED_BIG : (WX == 1 ? mhv::TILED_SKINNY
+                                                            : (FX == 2 ? mhv::TILED_MEDIUM : mhv::TILED_SMALL));
+  mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMM_TILED, mhv::tiled(shape, p.sum_y, out_u8), grid, block, lds);
   auto launch = [&](auto k) -> int {
     if (lds > 64 * 1024) MH_HIP(ctx, mh_allow_big_lds(ctx, (const void *)k, lds));
     MH_PROF_BEGIN(ctx);
-    hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, tab);
+    MH_KLAUNCH(ctx, k, grid, block, lds, ctx->stream, p, tab);
     return MACE_HIP_SUCCESS;
   };
   if (out_u8 && p.sum_y) {
@@ -2223,7 +2228,7 @@ int launch_gemm(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, bool 
     MH_RETURN_IF_ERROR(launch(q8_gemm_kernel<WX, WY, FX, FY, int32_t, false>));
   }
   MH_PROF_END(ctx);
-  MH_HIP(ctx, hipGetLastError());
+  MH_LAUNCH_CHECK(ctx);
   return MACE_HIP_SUCCESS;
 }
 
@@ -2236,10 +2241,14 @@ int launch_gemm_dma(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, b
   p.tiles_y = (p.YN + TY - 1) / TY;
   const size_t lds = (size_t)STAGES * (TX + TY) * KB;
   dim3 grid(p.tiles_x * p.tiles_y, 1, batch), block(WX * WY * 64);
+  if (p.conv && KB != SLAB) return MACE_HIP_INVALID_ARGS;   // not dispatched: the gather works on 64-byte slabs
+  mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMM_RING,
+               mhv::ring(mhv::ring_config(WX, WY, FX, FY, STAGES, OCC, KB), p.conv, p.conv || p.sum_y, out_u8),
+               grid, block, lds);
   auto launch = [&](auto k) -> int {
     if (lds > 64 * 1024) MH_HIP(ctx, mh_allow_big_lds(ctx, (const void *)k, lds));
     MH_PROF_BEGIN(ctx);
-    hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, tab);
+    MH_KLAUNCH(ctx, k, grid, block, lds, ctx->stream, p, tab);
     return MACE_HIP_SUCCESS;
   };
   if constexpr (KB == SLAB) {
@@ -2249,11 +2258,9 @@ int launch_gemm_dma(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, b
       else
         MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, int32_t, OCC, true, true>));
       MH_PROF_END(ctx);
-      MH_HIP(ctx, hipGetLastError());
+      MH_LAUNCH_CHECK(ctx);
       return MACE_HIP_SUCCESS;
     }
-  } else if (p.conv) {
-    return MACE_HIP_INVALID_ARGS;   // not dispatched: the gather works on 64-byte slabs
   }
   if (out_u8 && p.sum_y) {
     MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, uint8_t, OCC, true, false, KB>));
@@ -2265,7 +2272,7 @@ int launch_gemm_dma(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, b
     MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, int32_t, OCC, false, false, KB>));
   }
   MH_PROF_END(ctx);
-  MH_HIP(ctx, hipGetLastError());
+  MH_LAUNCH_CHECK(ctx);
   return MACE_HIP_SUCCESS;
 }
 
@@ -2277,10 +2284,11 @@ int launch_gemm_mid(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, b
   p.tiles_y = (p.YN + 127) / 128;
   const size_t lds = (size_t)STAGES * 256 * 128;
   dim3 grid(p.tiles_x * p.tiles_y, 1, batch), block(512);
+  mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMM_MID, mhv::mid(out_u8, xt), grid, block, lds);
   auto launch = [&](auto k) -> int {
     MH_HIP(ctx, mh_allow_big_lds(ctx, (const void *)k, lds));
     MH_PROF_BEGIN(ctx);
-    hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, tab);
+    MH_KLAUNCH(ctx, k, grid, block, lds, ctx->stream, p, tab);
     return MACE_HIP_SUCCESS;
   };
   if (xt) {
@@ -2291,7 +2299,7 @@ int launch_gemm_mid(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, b
     else MH_RETURN_IF_ERROR(launch(q8_gemm_mid_kernel<int32_t, STAGES, false>));
   }
   MH_PROF_END(ctx);
-  MH_HIP(ctx, hipGetLastError());
+  MH_LAUNCH_CHECK(ctx);
   return MACE_HIP_SUCCESS;
 }
 
@@ -2302,10 +2310,11 @@ int launch_gemm_big_xt(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab
   p.tiles_y = (p.YN + 255) / 256;
   const size_t lds = (size_t)2 * 512 * 128;
   dim3 grid(p.tiles_x * p.tiles_y, 1, batch), block(256);
+  mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMM_RING_XT, mhv::ring_xt(out_u8, p.sum_y, sum_x), grid, block, lds);
   auto launch = [&](auto k) -> int {
     MH_HIP(ctx, mh_allow_big_lds(ctx, (const void *)k, lds));
     MH_PROF_BEGIN(ctx);
-    hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, tab);
+    MH_KLAUNCH(ctx, k, grid, block, lds, ctx->stream, p, tab);
     return MACE_HIP_SUCCESS;
   };
 #define MH_XT(OUT_, SY_, SX_) \
@@ -2323,7 +2332,7 @@ int launch_gemm_big_xt(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab
   }
 #undef MH_XT
   MH_PROF_END(ctx);
-  MH_HIP(ctx, hipGetLastError());
+  MH_LAUNCH_CHECK(ctx);
   return MACE_HIP_SUCCESS;
 }
 
@@ -2334,10 +2343,11 @@ int launch_gemm_big_xf(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab
   p.tiles_y = (p.YN + 255) / 256;
   const size_t lds = (size_t)2 * 512 * 128;
   dim3 grid(p.tiles_x * p.tiles_y, 1, batch), block(256);
+  mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMM_RING_XF, mhv::ring_xf(out_u8, p.sum_y), grid, block, lds);
   auto launch = [&](auto k) -> int {
     MH_HIP(ctx, mh_allow_big_lds(ctx, (const void *)k, lds));
     MH_PROF_BEGIN(ctx);
-    hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, tab);
+    MH_KLAUNCH(ctx, k, grid, block, lds, ctx->stream, p, tab);
     return MACE_HIP_SUCCESS;
   };
   if (out_u8 && p.sum_y) {
@@ -2350,7 +2360,7 @@ int launch_gemm_big_xf(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab
     MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<2, 2, 4, 4, 2, int32_t, 1, false, false, 128, false, true>));
   }
   MH_PROF_END(ctx);
-  MH_HIP(ctx, hipGetLastError());
+  MH_LAUNCH_CHECK(ctx);
   return MACE_HIP_SUCCESS;
 }
 
@@ -2360,14 +2370,15 @@ int launch_gemm_fused_small(mace_hip_ctx *ctx, GemmParams &p, const RequantTable
   p.tiles_x = (p.XN + 63) / 64;
   p.tiles_y = (p.YN + 63) / 64;
   dim3 grid(p.tiles_x * p.tiles_y, 1, batch), block(256);
-  MH_PROF_BEGIN(ctx);
   const bool bw = p.x_bytewise || p.y_bytewise;
+  mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMM_FUSED_SMALL, mhv::fused_small(out_u8, xt, yt, bw), grid, block, 0);
+  MH_PROF_BEGIN(ctx);
 #define MH_FUSED(OutT_, XT_, YT_)                                                                 \
   if (bw)                                                                                         \
-    hipLaunchKernelGGL((q8_gemm_fused_small_kernel<OutT_, XT_, YT_, true>), grid, block, 0,       \
+    MH_KLAUNCH(ctx, (q8_gemm_fused_small_kernel<OutT_, XT_, YT_, true>), grid, block, 0,       \
                        ctx->stream, p, tab);                                                      \
   else                                                                                            \
-    hipLaunchKernelGGL((q8_gemm_fused_small_kernel<OutT_, XT_, YT_, false>), grid, block, 0,      \
+    MH_KLAUNCH(ctx, (q8_gemm_fused_small_kernel<OutT_, XT_, YT_, false>), grid, block, 0,      \
                        ctx->stream, p, tab)
   switch ((out_u8 ? 4 : 0) | (xt ? 2 : 0) | (yt ? 1 : 0)) {
     case 0: MH_FUSED(int32_t, false, false); break;
@@ -2381,7 +2392,7 @@ int launch_gemm_fused_small(mace_hip_ctx *ctx, GemmParams &p, const RequantTable
   }
 #undef MH_FUSED
   MH_PROF_END(ctx);
-  MH_HIP(ctx, hipGetLastError());
+  MH_LAUNCH_CHECK(ctx);
   return MACE_HIP_SUCCESS;
 }
 
@@ -2397,7 +2408,8 @@ int launch_gemm_xres(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, 
   const int cu = ctx->cu_count > 0 ? ctx->cu_count : 256;
   const int need = (nblk + 3) / 4;
   MH_CHECK(ctx, tiles_x <= 65535 && batch <= 65535, "grid too large");
-  auto launch = [&](auto k) -> int {
+  auto launch = [&](auto k, int mode, int group) -> int {
+    const int variant = mhv::xres(mode, FX, FY, group, out_u8);
     if (lds > 64 * 1024) MH_HIP(ctx, mh_allow_big_lds(ctx, (const void *)k, lds));
     // workgroups along y: as many as are resident at once -- up to three per CU where registers
     // and LDS allow (two against three: 56x56x128 -> 128 at batch 64 19.2 -> 18.6 us, 28x28x256 ->
@@ -2406,10 +2418,11 @@ int launch_gemm_xres(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, 
     const int slots = std::max(1, cu * per_cu / std::max(1, tiles_x * batch));
     const int wgs = std::max(1, std::min(need, slots));
     dim3 grid(wgs, tiles_x, batch), block(256);
+    mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMM_XRES, variant, grid, block, lds);
     MH_PROF_BEGIN(ctx);
-    hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, tab);
+    MH_KLAUNCH(ctx, k, grid, block, lds, ctx->stream, p, tab);
     MH_PROF_END(ctx);
-    MH_HIP(ctx, hipGetLastError());
+    MH_LAUNCH_CHECK(ctx);
     return MACE_HIP_SUCCESS;
   };
   if (p.conv) {
@@ -2417,29 +2430,30 @@ int launch_gemm_xres(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, 
     if constexpr (FY == 2) {
       // (128-byte groups with 128-row tiles would need more than 256 registers)
       if constexpr (FX == 2)
-        if (p.cv_cin % 128 == 0) return launch(q8_gemm_xres_kernel<FX, FY, 128, uint8_t, 2, true>);
-      return launch(q8_gemm_xres_kernel<FX, FY, 64, uint8_t, 2, true>);
+        if (p.cv_cin % 128 == 0)
+          return launch(q8_gemm_xres_kernel<FX, FY, 128, uint8_t, 2, true>, mhv::XRES_CONV, 128);
+      return launch(q8_gemm_xres_kernel<FX, FY, 64, uint8_t, 2, true>, mhv::XRES_CONV, 64);
     }
   }
   const bool g128 = p.K % 128 == 0;
   if (xt) {   // X k-major in memory: transposed on its way into LDS
     if (out_u8) {
-      if (g128) return launch(q8_gemm_xres_kernel<FX, FY, 128, uint8_t, 2, false, true>);
-      return launch(q8_gemm_xres_kernel<FX, FY, 64, uint8_t, 2, false, true>);
+      if (g128) return launch(q8_gemm_xres_kernel<FX, FY, 128, uint8_t, 2, false, true>, mhv::XRES_XT, 128);
+      return launch(q8_gemm_xres_kernel<FX, FY, 64, uint8_t, 2, false, true>, mhv::XRES_XT, 64);
     }
-    if (g128) return launch(q8_gemm_xres_kernel<FX, FY, 128, int32_t, 2, false, true>);
-    return launch(q8_gemm_xres_kernel<FX, FY, 64, int32_t, 2, false, true>);
+    if (g128) return launch(q8_gemm_xres_kernel<FX, FY, 128, int32_t, 2, false, true>, mhv::XRES_XT, 128);
+    return launch(q8_gemm_xres_kernel<FX, FY, 64, int32_t, 2, false, true>, mhv::XRES_XT, 64);
   }
   if (tail) {
-    if (out_u8) return launch(q8_gemm_xres_kernel<FX, FY, 64, uint8_t, 2, false, false, true>);
-    return launch(q8_gemm_xres_kernel<FX, FY, 64, int32_t, 2, false, false, true>);
+    if (out_u8) return launch(q8_gemm_xres_kernel<FX, FY, 64, uint8_t, 2, false, false, true>, mhv::XRES_TAIL, 64);
+    return launch(q8_gemm_xres_kernel<FX, FY, 64, int32_t, 2, false, false, true>, mhv::XRES_TAIL, 64);
   }
   if (out_u8) {
-    if (g128) return launch(q8_gemm_xres_kernel<FX, FY, 128, uint8_t, 2>);
-    return launch(q8_gemm_xres_kernel<FX, FY, 64, uint8_t, 2>);
+    if (g128) return launch(q8_gemm_xres_kernel<FX, FY, 128, uint8_t, 2>, mhv::XRES_PLAIN, 128);
+    return launch(q8_gemm_xres_kernel<FX, FY, 64, uint8_t, 2>, mhv::XRES_PLAIN, 64);
   }
-  if (g128) return launch(q8_gemm_xres_kernel<FX, FY, 128, int32_t, 2>);
-  return launch(q8_gemm_xres_kernel<FX, FY, 64, int32_t, 2>);
+  if (g128) return launch(q8_gemm_xres_kernel<FX, FY, 128, int32_t, 2>, mhv::XRES_PLAIN, 128);
+  return launch(q8_gemm_xres_kernel<FX, FY, 64, int32_t, 2>, mhv::XRES_PLAIN, 64);
 }
 
 // Tile rows (64 / 128) and rows of Y per block.  64-row blocks read half the LDS per MFMA; 32-row
@@ -2470,14 +2484,16 @@ int launch_gemm_stream(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab
   const int cu = ctx->cu_count > 0 ? ctx->cu_count : 256;
   const int wgs = std::max(1, std::min((nblk + YW - 1) / YW, cu * per_cu));
   dim3 grid(wgs, 1, batch), block(256);
+  if (ks < 1 || ks > 2) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "streaming kernel: unsupported depth");
+  mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMM_STREAM, mhv::stream(FX, ks), grid, block, 0);
   MH_PROF_BEGIN(ctx);
   switch (ks) {
-    case 1: hipLaunchKernelGGL((q8_gemm_stream_kernel<FX, 1, XW, 4>), grid, block, 0, ctx->stream, p, tab); break;
-    case 2: hipLaunchKernelGGL((q8_gemm_stream_kernel<FX, 2, XW, 4>), grid, block, 0, ctx->stream, p, tab); break;
+    case 1: MH_KLAUNCH(ctx, (q8_gemm_stream_kernel<FX, 1, XW, 4>), grid, block, 0, ctx->stream, p, tab); break;
+    case 2: MH_KLAUNCH(ctx, (q8_gemm_stream_kernel<FX, 2, XW, 4>), grid, block, 0, ctx->stream, p, tab); break;
     default: return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "streaming kernel: unsupported depth");
   }
   MH_PROF_END(ctx);
-  MH_HIP(ctx, hipGetLastError());
+  MH_LAUNCH_CHECK(ctx);
   return MACE_HIP_SUCCESS;
 }
 
@@ -2871,41 +2887,45 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     if (fused) *fused = false;
     if (flipped) *flipped = false;
     if (order_is_kcontig) {
+      mh_plan_aux(ctx, MACE_HIP_AUX_PACK_ROWS);
       if (depth % 4 == 0 && (uintptr_t)src % 4 == 0) {
         const int64_t total = n * (kp / 16);
         dim3 grid((unsigned)std::min<int64_t>((total + 255) / 256, 1 << 20), 1, nb);
-        hipLaunchKernelGGL(q8_pack_rows4_kernel, grid, dim3(256), 0, ctx->stream, src,
+        MH_KLAUNCH(ctx, q8_pack_rows4_kernel, grid, dim3(256), 0, ctx->stream, src,
                            n * depth, dst, n * kp, (int)n, (int)depth, (int)kp);
       } else {
         const int64_t total = n * (kp / 16);
         dim3 grid((unsigned)std::min<int64_t>((total + 255) / 256, 1 << 20), 1, nb);
-        hipLaunchKernelGGL(q8_pack_rows_kernel, grid, dim3(256), 0, ctx->stream, src,
+        MH_KLAUNCH(ctx, q8_pack_rows_kernel, grid, dim3(256), 0, ctx->stream, src,
                            n * depth, dst, n * kp, (int)n, (int)depth, (int)kp);
       }
     } else {
       MH_CHECK(ctx, (kp / 64) <= 65535, "depth too large to repack");
       const int vec_ok = (n % 16 == 0) && ((uintptr_t)src % 16 == 0);
+      mh_plan_aux(ctx, MACE_HIP_AUX_PACK_TRANSPOSE);
       if (vec_ok) {
         dim3 grid((unsigned)((n + 127) / 128), (unsigned)((kp + 127) / 128), nb);
         if (fused_sums) {
           const int64_t cnt = (int64_t)nb * n;
+          if (!sums_cleared) mh_plan_aux(ctx, MACE_HIP_AUX_ZERO);
           if (!sums_cleared)
-            hipLaunchKernelGGL(q8_zero_i32_kernel, dim3((unsigned)((cnt + 255) / 256)), dim3(256), 0,
+            MH_KLAUNCH(ctx, q8_zero_i32_kernel, dim3((unsigned)((cnt + 255) / 256)), dim3(256), 0,
                                ctx->stream, fused_sums, cnt);
           *fused = true;
         }
         const bool fl = want_flipped && flipped;
-        hipLaunchKernelGGL(q8_pack_transpose128_kernel, grid, dim3(256), 0, ctx->stream, src,
+        MH_KLAUNCH(ctx, q8_pack_transpose128_kernel, grid, dim3(256), 0, ctx->stream, src,
                            n * depth, dst, n * kp, (int)n, (int)depth, (int)kp, fused_sums,
                            fl ? 0x80808080u : 0u);
+        if (fl) mh_plan_aux(ctx, MACE_HIP_AUX_PACK_SHIFTED);
         if (fl) *flipped = true;
       } else {
         dim3 grid((unsigned)((n + 63) / 64), (unsigned)(kp / 64), nb);
-        hipLaunchKernelGGL(q8_pack_transpose_kernel, grid, dim3(256), 0, ctx->stream, src,
+        MH_KLAUNCH(ctx, q8_pack_transpose_kernel, grid, dim3(256), 0, ctx->stream, src,
                            n * depth, dst, n * kp, (int)n, (int)depth, (int)kp, 0);
       }
     }
-    MH_HIP(ctx, hipGetLastError());
+    MH_LAUNCH_CHECK(ctx);
     return MACE_HIP_SUCCESS;
   };
 
@@ -2922,27 +2942,36 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
       *P = Panel{hit->panel ? hit->panel : src, hit->ld, nb > 1 ? n * hit->ld : 0, hit->k, hit->sums,
                  hit->flipped};
       ++ctx->weight_hits;
+      mh_plan_aux(ctx, MACE_HIP_AUX_WEIGHT_HIT);
       return MACE_HIP_SUCCESS;
     }
+    mh_plan_aux(ctx, MACE_HIP_AUX_WEIGHT_BUILD);
     mh_weight_panel c{order_is_kcontig, n, depth, nb, nullptr, direct ? depth : kp,
                       (int)(direct ? depth : kp), nullptr, false};
-    MH_HIP(ctx, hipMalloc((void **)&c.sums, sizeof(int32_t) * (size_t)nb * n));
+    // (a plan-only context derives nothing real: addresses stand in for the two buffers)
+    auto dev_alloc = [&](void **ptr, size_t bytes) -> hipError_t {
+      if (!ctx->plan_only) return hipMalloc(ptr, bytes);
+      *ptr = (void *)(uintptr_t)0x300000000ull;
+      return hipSuccess;
+    };
+    auto dev_free = [&](void *ptr) { if (!ctx->plan_only) (void)hipFree(ptr); };
+    MH_HIP(ctx, dev_alloc((void **)&c.sums, sizeof(int32_t) * (size_t)nb * n));
     bool fused = false;
     if (!direct) {
-      hipError_t e = hipMalloc((void **)&c.panel, (size_t)nb * n * kp);
-      if (e != hipSuccess) { (void)hipFree(c.sums); MH_HIP(ctx, e); }
+      hipError_t e = dev_alloc((void **)&c.panel, (size_t)nb * n * kp);
+      if (e != hipSuccess) { dev_free(c.sums); MH_HIP(ctx, e); }
       // the sums come from the repack where it can take them (always where it shifts the bytes)
       const int rc = pack(src, order_is_kcontig, nb, n, c.panel, want_flipped ? c.sums : nullptr, &fused,
                           want_flipped, &c.flipped);
-      if (rc != MACE_HIP_SUCCESS) { (void)hipFree(c.panel); (void)hipFree(c.sums); return rc; }
+      if (rc != MACE_HIP_SUCCESS) { dev_free(c.panel); dev_free(c.sums); return rc; }
     }
     if (!fused) {
       const int rc = c.flipped ? MACE_HIP_RUNTIME_ERROR
                                : launch_panel_sums(ctx, c.panel ? c.panel : src, c.ld,
                                                    nb > 1 ? n * c.ld : 0, n, c.k, nb, c.sums);
       if (rc != MACE_HIP_SUCCESS) {
-        if (c.panel) (void)hipFree(c.panel);
-        (void)hipFree(c.sums);
+        if (c.panel) dev_free(c.panel);
+        dev_free(c.sums);
         return rc;
       }
     }
@@ -3082,7 +3111,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
       MH_RETURN_IF_ERROR(launch_panel_sums(ctx, L.ptr, L.ld, L.bs, rows, L.k, lhs_nb, corrL));
     if (!R.sums && !(sum_y && x_is_lhs))
       MH_RETURN_IF_ERROR(launch_panel_sums(ctx, R.ptr, R.ld, R.bs, cols, R.k, rhs_nb, corrR));
-    MH_HIP(ctx, hipGetLastError());
+    MH_LAUNCH_CHECK(ctx);
   }
 
   GemmParams p;
@@ -3189,6 +3218,7 @@ int mace_hip_gemm_q8_i32(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order,
                          int lhs_batched, int rhs_batched, int32_t lhs_offset,
                          int32_t rhs_offset) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  PlanScope plan_scope(ctx);
   Q8GemmEpilogue ep{nullptr, 0, 0, 0, 0, 255};
   return mh_q8_gemm(ctx, lhs, lhs_order, rhs, rhs_order, out, out_order, false, batch, rows,
                     depth, cols, lhs_batched, rhs_batched, lhs_offset, rhs_offset, ep);
@@ -3202,6 +3232,7 @@ int mace_hip_gemm_q8_u8(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order,
                         int right_shift, int32_t offset_after_shift, int clamp_min,
                         int clamp_max) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  PlanScope plan_scope(ctx);
   Q8GemmEpilogue ep{bias, multiplier, right_shift, offset_after_shift, clamp_min, clamp_max};
   return mh_q8_gemm(ctx, lhs, lhs_order, rhs, rhs_order, out, out_order, true, batch, rows,
                     depth, cols, lhs_batched, rhs_batched, lhs_offset, rhs_offset, ep);

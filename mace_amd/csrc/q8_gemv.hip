@@ -711,6 +711,7 @@ int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
   // a batched lhs gives every batch its own weights: one batch row per pass
   int nb = lhs_batched ? 1 : (p.batch >= 8 ? 8 : (p.batch >= 4 ? 4 : (p.batch >= 2 ? 2 : 1)));
   dim3 block(256);
+  constexpr bool out_u8 = sizeof(OutT) == 1;
   // Two vectors against long rows stay on the row-block kernel (one pass, the weights streamed
   // once: 5.6 us against 5.9 us at 4096 x 4096); from three on the matrix-core kernels win.
   const bool few = !lhs_batched && p.batch == 2 && p.W >= 2048 && (size_t)2 * p.W <= 64 * 1024;
@@ -726,9 +727,10 @@ int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
     if (p.W <= 4096 && lds_max >= 140 * 1024) {
       // rows of at most 4 KiB: every wavefront on a k slice of its own
       const int spw = p.W <= 1024 ? 1 : (p.W <= 2048 ? 2 : 4);
+      mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMV_SLICE, mhv::gemv_slice(spw, out_u8), grid, dim3(1024), 0);
       MH_PROF_BEGIN(ctx);
 #define MH_SLICE_LAUNCH(S_)                                                                       \
-  hipLaunchKernelGGL((q8_gemv_mfma_slice_kernel<S_, OutT>), grid, dim3(1024), 0, ctx->stream,      \
+  MH_KLAUNCH(ctx, (q8_gemv_mfma_slice_kernel<S_, OutT>), grid, dim3(1024), 0, ctx->stream,      \
                      p.lhs, p.rhs, p.H, p.W, p.bias, p.out, p.mult, p.neon_mode ? p.out_zp : 0,   \
                      p.lhs_zp, p.rhs_zp, p.batch, p.rhs_bs)
       if (spw == 1) MH_SLICE_LAUNCH(1);
@@ -738,34 +740,34 @@ int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
     } else if (lds <= lds_max && p.W >= 1024) {
       auto k = q8_gemv_mfma_lds_kernel<16, OutT>;
       if (lds > 48 * 1024) MH_HIP(ctx, mh_allow_big_lds(ctx, (const void *)k, lds));
+      mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMV_MFMA_LDS, mhv::gemv_out(out_u8), grid, dim3(1024), lds);
       MH_PROF_BEGIN(ctx);
-      hipLaunchKernelGGL(k, grid, dim3(1024), lds, ctx->stream, p, pitch);
-    } else if (lds <= lds_max) {
-      auto k = q8_gemv_mfma_lds_kernel<4, OutT>;
-      if (lds > 48 * 1024) MH_HIP(ctx, mh_allow_big_lds(ctx, (const void *)k, lds));
-      MH_PROF_BEGIN(ctx);
-      hipLaunchKernelGGL(k, grid, block, lds, ctx->stream, p, pitch);
+      MH_KLAUNCH(ctx, k, grid, dim3(1024), lds, ctx->stream, p, pitch);
     } else {
+      mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMV_MFMA, mhv::gemv_out(out_u8), grid, block, 0);
       MH_PROF_BEGIN(ctx);
-      hipLaunchKernelGGL(q8_gemv_mfma_kernel<OutT>, grid, block, 0, ctx->stream, p);
+      MH_KLAUNCH(ctx, q8_gemv_mfma_kernel<OutT>, grid, block, 0, ctx->stream, p);
     }
     MH_PROF_END(ctx);
-    MH_HIP(ctx, hipGetLastError());
+    MH_LAUNCH_CHECK(ctx);
     return MACE_HIP_SUCCESS;
   }
   // one vector per pass against rows of at most 8 KiB: the lean one-row-per-wavefront kernel
   if (vec && nb == 1 && p.W >= 16 && p.W <= 8192 && p.batch <= 65535) {
     dim3 grid((unsigned)((p.H + 15) / 16), (unsigned)p.batch);
     const int u = (p.W + 1023) / 1024;
+    const int u_t = u <= 1 ? 1 : (u <= 2 ? 2 : (u <= 4 ? 4 : 8));
+    mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMV_ROW, mhv::gemv_row(u_t, p.batch != 1, p.W == 1024 * u_t, out_u8),
+                 grid, dim3(1024), 0);
     MH_PROF_BEGIN(ctx);
 #define MH_ROW_LAUNCH(U_, B_)                                                                      \
   do {                                                                                             \
     if (p.W == 1024 * U_)                                                                          \
-      hipLaunchKernelGGL((q8_gemv_row_kernel<U_, B_, true, OutT>), grid, dim3(1024), 0,            \
+      MH_KLAUNCH(ctx, (q8_gemv_row_kernel<U_, B_, true, OutT>), grid, dim3(1024), 0,            \
                          ctx->stream, p.lhs, p.rhs, p.H, p.W, p.bias, p.out, p.mult,               \
                          p.neon_mode ? p.out_zp : 0, p.lhs_zp, p.rhs_zp, p.lhs_bs, p.rhs_bs);      \
     else                                                                                           \
-      hipLaunchKernelGGL((q8_gemv_row_kernel<U_, B_, false, OutT>), grid, dim3(1024), 0,           \
+      MH_KLAUNCH(ctx, (q8_gemv_row_kernel<U_, B_, false, OutT>), grid, dim3(1024), 0,           \
                          ctx->stream, p.lhs, p.rhs, p.H, p.W, p.bias, p.out, p.mult,               \
                          p.neon_mode ? p.out_zp : 0, p.lhs_zp, p.rhs_zp, p.lhs_bs, p.rhs_bs);      \
   } while (0)
@@ -782,7 +784,7 @@ int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
     }
 #undef MH_ROW_LAUNCH
     MH_PROF_END(ctx);
-    MH_HIP(ctx, hipGetLastError());
+    MH_LAUNCH_CHECK(ctx);
     return MACE_HIP_SUCCESS;
   }
   // shared weights, aligned rows, right-hand vectors of one pass fit in LDS: row-block kernel
@@ -792,25 +794,27 @@ int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
               (unsigned)((p.batch + nb - 1) / nb));
     dim3 wg(NWAVES * 64);
     const size_t lds = (size_t)nb * p.W;
+    mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMV_ROWS, mhv::gemv_rows(nb, out_u8), grid, wg, lds);
     MH_PROF_BEGIN(ctx);
     switch (nb) {
-      case 8: hipLaunchKernelGGL((q8_gemv_rows_kernel<R, 8, NWAVES, OutT>), grid, wg, lds, ctx->stream, p); break;
-      case 4: hipLaunchKernelGGL((q8_gemv_rows_kernel<R, 4, NWAVES, OutT>), grid, wg, lds, ctx->stream, p); break;
-      case 2: hipLaunchKernelGGL((q8_gemv_rows_kernel<R, 2, NWAVES, OutT>), grid, wg, lds, ctx->stream, p); break;
-      default: hipLaunchKernelGGL((q8_gemv_rows_kernel<R, 1, NWAVES, OutT>), grid, wg, lds, ctx->stream, p); break;
+      case 8: MH_KLAUNCH(ctx, (q8_gemv_rows_kernel<R, 8, NWAVES, OutT>), grid, wg, lds, ctx->stream, p); break;
+      case 4: MH_KLAUNCH(ctx, (q8_gemv_rows_kernel<R, 4, NWAVES, OutT>), grid, wg, lds, ctx->stream, p); break;
+      case 2: MH_KLAUNCH(ctx, (q8_gemv_rows_kernel<R, 2, NWAVES, OutT>), grid, wg, lds, ctx->stream, p); break;
+      default: MH_KLAUNCH(ctx, (q8_gemv_rows_kernel<R, 1, NWAVES, OutT>), grid, wg, lds, ctx->stream, p); break;
     }
     MH_PROF_END(ctx);
-    MH_HIP(ctx, hipGetLastError());
+    MH_LAUNCH_CHECK(ctx);
     return MACE_HIP_SUCCESS;
   }
   dim3 grid((unsigned)((p.H + 3) / 4), (unsigned)((p.batch + nb - 1) / nb));
 #define MH_GEMV_LAUNCH(NB_)                                                              \
   do {                                                                                   \
     if (vec)                                                                             \
-      hipLaunchKernelGGL((q8_gemv_kernel<NB_, true, OutT>), grid, block, 0, ctx->stream, p); \
+      MH_KLAUNCH(ctx, (q8_gemv_kernel<NB_, true, OutT>), grid, block, 0, ctx->stream, p); \
     else                                                                                 \
-      hipLaunchKernelGGL((q8_gemv_kernel<NB_, false, OutT>), grid, block, 0, ctx->stream, p); \
+      MH_KLAUNCH(ctx, (q8_gemv_kernel<NB_, false, OutT>), grid, block, 0, ctx->stream, p); \
   } while (0)
+  mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMV_GENERAL, mhv::gemv_general(nb, vec, out_u8), grid, block, 0);
   MH_PROF_BEGIN(ctx);
   switch (nb) {
     case 8: MH_GEMV_LAUNCH(8); break;
@@ -820,7 +824,7 @@ int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
   }
 #undef MH_GEMV_LAUNCH
   MH_PROF_END(ctx);
-  MH_HIP(ctx, hipGetLastError());
+  MH_LAUNCH_CHECK(ctx);
   return MACE_HIP_SUCCESS;
 }
 
@@ -851,6 +855,7 @@ int mace_hip_gemv_q8_u8(mace_hip_ctx *ctx, const uint8_t *lhs, const uint8_t *rh
                         float lhs_scale, float rhs_scale, float out_scale, int32_t out_zp,
                         int requant_mode, uint8_t *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  PlanScope plan_scope(ctx);
   MH_CHECK(ctx, requant_mode == MACE_HIP_REQUANT_REF || requant_mode == MACE_HIP_REQUANT_NEON,
            "unknown requant mode %d", requant_mode);
   MH_CHECK(ctx, out_scale > 0.f, "output scale must not be zero");
@@ -873,6 +878,7 @@ int mace_hip_gemv_q8_i32(mace_hip_ctx *ctx, const uint8_t *lhs, const uint8_t *r
                          int lhs_batched, int rhs_batched, int32_t lhs_zp, int32_t rhs_zp,
                          int32_t *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  PlanScope plan_scope(ctx);
   GemvParams p{};
   p.lhs = lhs; p.rhs = rhs; p.bias = bias; p.out = out;
   p.lhs_zp = lhs_zp; p.rhs_zp = rhs_zp;

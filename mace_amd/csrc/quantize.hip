@@ -206,25 +206,29 @@ void mace_hip_adjust_range_u8(float in_min, float in_max, int non_zero, float *s
 int mace_hip_quantize_tensor_u8(mace_hip_ctx *ctx, const float *input, int64_t size,
                                 float scale, int32_t zero_point, uint8_t *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  PlanScope plan_scope(ctx);
   MH_RETURN_IF_ERROR(check_size(ctx, size, input, out));
   if (size == 0) return MACE_HIP_SUCCESS;
   volatile float recip = 1 / scale;
   const unsigned blocks = (unsigned)((size + 4095) / 4096);
   MH_PROF_BEGIN(ctx);
   if (aligned16(input, out))
-    hipLaunchKernelGGL(quantize_u8_kernel<true>, dim3(blocks), dim3(256), 0, ctx->stream, input,
+    MH_KLAUNCH(ctx, quantize_u8_kernel<true>, dim3(blocks), dim3(256), 0, ctx->stream, input,
                        size, (float)recip, (float)zero_point, out);
   else
-    hipLaunchKernelGGL(quantize_u8_kernel<false>, dim3(blocks), dim3(256), 0, ctx->stream, input,
+    MH_KLAUNCH(ctx, quantize_u8_kernel<false>, dim3(blocks), dim3(256), 0, ctx->stream, input,
                        size, (float)recip, (float)zero_point, out);
   MH_PROF_END(ctx);
-  MH_HIP(ctx, hipGetLastError());
+  MH_LAUNCH_CHECK(ctx);
   return MACE_HIP_SUCCESS;
 }
 
 int mace_hip_find_min_max_f32(mace_hip_ctx *ctx, const float *input, int64_t size,
                               float *min_val, float *max_val) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  if (ctx->plan_only)
+    return mh_fail(ctx, MACE_HIP_UNSUPPORTED, "%s needs a GPU: this is a plan-only context", __func__);
+  PlanScope plan_scope(ctx);
   MH_CHECK(ctx, size > 0 && input && min_val && max_val, "empty or null tensor");
   MH_CHECK(ctx, size < (1ll << 40), "tensor too large");
   const int cu = ctx->cu_count > 0 ? ctx->cu_count : 256;
@@ -236,15 +240,15 @@ int mace_hip_find_min_max_f32(mace_hip_ctx *ctx, const float *input, int64_t siz
   float *result = partial + 2 * blocks;
   MH_PROF_BEGIN(ctx);
   if (((uintptr_t)input & 15) == 0)
-    hipLaunchKernelGGL(min_max_kernel<true>, dim3(blocks), dim3(256), 0, ctx->stream, input, size,
+    MH_KLAUNCH(ctx, min_max_kernel<true>, dim3(blocks), dim3(256), 0, ctx->stream, input, size,
                        partial);
   else
-    hipLaunchKernelGGL(min_max_kernel<false>, dim3(blocks), dim3(256), 0, ctx->stream, input,
+    MH_KLAUNCH(ctx, min_max_kernel<false>, dim3(blocks), dim3(256), 0, ctx->stream, input,
                        size, partial);
   MH_PROF_END(ctx);
-  hipLaunchKernelGGL(min_max_fold_kernel, dim3(1), dim3(256), 0, ctx->stream, partial, blocks,
+  MH_KLAUNCH(ctx, min_max_fold_kernel, dim3(1), dim3(256), 0, ctx->stream, partial, blocks,
                      result);
-  MH_HIP(ctx, hipGetLastError());
+  MH_LAUNCH_CHECK(ctx);
   float host[2];
   MH_HIP(ctx, hipMemcpyAsync(host, result, sizeof(host), hipMemcpyDeviceToHost, ctx->stream));
   MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
@@ -257,6 +261,9 @@ int mace_hip_quantize_tensor_dynamic_u8(mace_hip_ctx *ctx, const float *input, i
                                         int non_zero, uint8_t *out, float *scale,
                                         int32_t *zero_point) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  if (ctx->plan_only)
+    return mh_fail(ctx, MACE_HIP_UNSUPPORTED, "%s needs a GPU: this is a plan-only context", __func__);
+  PlanScope plan_scope(ctx);
   MH_CHECK(ctx, scale && zero_point, "null result pointer");
   float mn, mx;
   MH_RETURN_IF_ERROR(mace_hip_find_min_max_f32(ctx, input, size, &mn, &mx));
@@ -267,36 +274,38 @@ int mace_hip_quantize_tensor_dynamic_u8(mace_hip_ctx *ctx, const float *input, i
 int mace_hip_dequantize_tensor_u8(mace_hip_ctx *ctx, const uint8_t *input, int64_t size,
                                   float scale, int32_t zero_point, float *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  PlanScope plan_scope(ctx);
   MH_RETURN_IF_ERROR(check_size(ctx, size, input, out));
   if (size == 0) return MACE_HIP_SUCCESS;
   const unsigned blocks = (unsigned)((size + 4095) / 4096);
   MH_PROF_BEGIN(ctx);
   if (aligned16(input, out))
-    hipLaunchKernelGGL(dequantize_u8_kernel<true>, dim3(blocks), dim3(256), 0, ctx->stream,
+    MH_KLAUNCH(ctx, dequantize_u8_kernel<true>, dim3(blocks), dim3(256), 0, ctx->stream,
                        input, size, scale, zero_point, out);
   else
-    hipLaunchKernelGGL(dequantize_u8_kernel<false>, dim3(blocks), dim3(256), 0, ctx->stream,
+    MH_KLAUNCH(ctx, dequantize_u8_kernel<false>, dim3(blocks), dim3(256), 0, ctx->stream,
                        input, size, scale, zero_point, out);
   MH_PROF_END(ctx);
-  MH_HIP(ctx, hipGetLastError());
+  MH_LAUNCH_CHECK(ctx);
   return MACE_HIP_SUCCESS;
 }
 
 int mace_hip_dequantize_tensor_i32(mace_hip_ctx *ctx, const int32_t *input, int64_t size,
                                    float scale, int32_t zero_point, float *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  PlanScope plan_scope(ctx);
   MH_RETURN_IF_ERROR(check_size(ctx, size, input, out));
   if (size == 0) return MACE_HIP_SUCCESS;
   const unsigned blocks = (unsigned)((size + 4 * 256 - 1) / (4 * 256));
   MH_PROF_BEGIN(ctx);
   if (aligned16(input, out))
-    hipLaunchKernelGGL(dequantize_i32_kernel<true>, dim3(blocks), dim3(256), 0, ctx->stream,
+    MH_KLAUNCH(ctx, dequantize_i32_kernel<true>, dim3(blocks), dim3(256), 0, ctx->stream,
                        input, size, scale, zero_point, out);
   else
-    hipLaunchKernelGGL(dequantize_i32_kernel<false>, dim3(blocks), dim3(256), 0, ctx->stream,
+    MH_KLAUNCH(ctx, dequantize_i32_kernel<false>, dim3(blocks), dim3(256), 0, ctx->stream,
                        input, size, scale, zero_point, out);
   MH_PROF_END(ctx);
-  MH_HIP(ctx, hipGetLastError());
+  MH_LAUNCH_CHECK(ctx);
   return MACE_HIP_SUCCESS;
 }
 
@@ -305,6 +314,9 @@ int mace_hip_dequantize_tensor_i32(mace_hip_ctx *ctx, const int32_t *input, int6
 int mace_hip_quantize_tensor_u8_host(mace_hip_ctx *ctx, const float *input, int64_t size,
                                      float scale, int32_t zero_point, uint8_t *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  if (ctx->plan_only)
+    return mh_fail(ctx, MACE_HIP_UNSUPPORTED, "%s needs a GPU: this is a plan-only context", __func__);
+  PlanScope plan_scope(ctx);
   MH_RETURN_IF_ERROR(check_size(ctx, size, input, out));
   if (size == 0) return MACE_HIP_SUCCESS;
   MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, (size_t)size * 5));
@@ -321,6 +333,9 @@ int mace_hip_quantize_tensor_dynamic_u8_host(mace_hip_ctx *ctx, const float *inp
                                              int64_t size, int non_zero, uint8_t *out,
                                              float *scale, int32_t *zero_point) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  if (ctx->plan_only)
+    return mh_fail(ctx, MACE_HIP_UNSUPPORTED, "%s needs a GPU: this is a plan-only context", __func__);
+  PlanScope plan_scope(ctx);
   MH_CHECK(ctx, size > 0 && input && out && scale && zero_point, "empty or null tensor");
   MH_CHECK(ctx, size < (1ll << 40), "tensor too large");
   MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, (size_t)size * 5 + (1 << 16)));
@@ -336,6 +351,9 @@ int mace_hip_quantize_tensor_dynamic_u8_host(mace_hip_ctx *ctx, const float *inp
 int mace_hip_dequantize_tensor_u8_host(mace_hip_ctx *ctx, const uint8_t *input, int64_t size,
                                        float scale, int32_t zero_point, float *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  if (ctx->plan_only)
+    return mh_fail(ctx, MACE_HIP_UNSUPPORTED, "%s needs a GPU: this is a plan-only context", __func__);
+  PlanScope plan_scope(ctx);
   MH_RETURN_IF_ERROR(check_size(ctx, size, input, out));
   if (size == 0) return MACE_HIP_SUCCESS;
   MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, (size_t)size * 5));
@@ -351,6 +369,9 @@ int mace_hip_dequantize_tensor_u8_host(mace_hip_ctx *ctx, const uint8_t *input, 
 int mace_hip_dequantize_tensor_i32_host(mace_hip_ctx *ctx, const int32_t *input, int64_t size,
                                         float scale, int32_t zero_point, float *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  if (ctx->plan_only)
+    return mh_fail(ctx, MACE_HIP_UNSUPPORTED, "%s needs a GPU: this is a plan-only context", __func__);
+  PlanScope plan_scope(ctx);
   MH_RETURN_IF_ERROR(check_size(ctx, size, input, out));
   if (size == 0) return MACE_HIP_SUCCESS;
   MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, (size_t)size * 8));

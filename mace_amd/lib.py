@@ -24,6 +24,7 @@ _i64, _i32, _f32, _int, _p = C.c_int64, C.c_int32, C.c_float, C.c_int, C.c_void_
 # name -> (restype, argtypes); must list every symbol of include/mace_hip.h
 _GEMM_F32 = [_p, _p, _p, _i64, _i64, _i64, _i64, _int, _int, _int, _int, _int, _p]
 _GEMV_F32 = [_p, _p, _p, _p, _i64, _i64, _i64, _int, _int, _p]
+_GEMV_F32_ACT = [_p, _p, _p, _p, _i64, _i64, _i64, _int, _int, _int, _f32, _p]
 _CONV_F32 = [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _int, _f32, _p]
 _CONV2D_F32 = [_p, _p, _p, _p] + [_i64] * 7 + [_int] * 6 + [_int, _f32, _p]
 _MATMUL_F32 = [_p, _p, _p, _p] + [_i64] * 5 + [_int] * 4 + [_p]
@@ -53,6 +54,12 @@ SIGNATURES = {
     "mace_hip_profile_kernel_count": (_int, [_p, C.POINTER(_int)]),
     "mace_hip_profile_kernel_ms": (_int, [_p, _int, C.POINTER(_f32)]),
     "mace_hip_ctx_fail_next_allocs": (_int, [_p, _int]),
+    "mace_hip_plan_ctx_create": (_int, [_int, _int, C.POINTER(_p)]),
+    "mace_hip_last_plan": (_int, [_p, _p]),
+    "mace_hip_plan_variant_count": (_int, [_int]),
+    "mace_hip_plan_variant_valid": (_int, [_int, _int]),
+    "mace_hip_plan_describe": (_int, [_int, _int, C.c_char_p, C.c_size_t]),
+    "mace_hip_plan_coverage": (C.c_int64, [_int, _int]),
     "mace_hip_ctx_set_kernel_mask": (_int, [_p, _int]),
     "mace_hip_graph_capture_begin": (_int, [_p]),
     "mace_hip_graph_capture_end": (_int, [_p, C.POINTER(_p)]),
@@ -86,6 +93,8 @@ SIGNATURES = {
     "mace_hip_gemm_f32_transpose": (_int, [_p, _p, _p, _i64, _i64, _i64, _i64, _i64, _int,
                                            _int, _int, _int, _int, _p]),
     "mace_hip_gemv_f32": (_int, _GEMV_F32),
+    "mace_hip_gemv_f32_act": (_int, _GEMV_F32_ACT),
+    "mace_hip_gemv_f32_act_host": (_int, _GEMV_F32_ACT),
     "mace_hip_conv1x1_f32_nchw": (_int, _CONV_F32),
     "mace_hip_conv2d_f32_nchw": (_int, _CONV2D_F32),
     "mace_hip_conv2d_f32_nchw_host": (_int, _CONV2D_F32),
@@ -112,6 +121,52 @@ SIGNATURES = {
                                                      C.POINTER(C.c_int64), C.POINTER(_int),
                                                      C.POINTER(_int)]),
 }
+
+
+# kernel families (MACE_HIP_KF_*) and auxiliary passes (MACE_HIP_AUX_*) of include/mace_hip.h
+(KF_NONE, KF_Q8_GEMM_FUSED_SMALL, KF_Q8_GEMM_XRES, KF_Q8_GEMM_MID, KF_Q8_GEMM_STREAM, KF_Q8_GEMM_RING,
+ KF_Q8_GEMM_RING_XT, KF_Q8_GEMM_RING_XF, KF_Q8_GEMM_TILED, KF_Q8_GEMV_ROW, KF_Q8_GEMV_SLICE,
+ KF_Q8_GEMV_MFMA_LDS, KF_Q8_GEMV_MFMA, KF_Q8_GEMV_ROWS, KF_Q8_GEMV_GENERAL, KF_F32_GEMM_VEC,
+ KF_F32_GEMM_GENERAL, KF_F32_GEMM_FILL, KF_F32_GEMV_VEC, KF_F32_GEMV_GENERAL, KF_COUNT) = range(21)
+(AUX_PACK_ROWS, AUX_PACK_TRANSPOSE, AUX_PACK_SHIFTED, AUX_PANEL_SUMS, AUX_KMAJOR_SUMS, AUX_ZERO,
+ AUX_IM2COL, AUX_BIAS_RESCALE, AUX_F32_PAD, AUX_FILL, AUX_WEIGHT_HIT, AUX_WEIGHT_BUILD) = (
+    1 << i for i in range(12))
+
+
+class PlanStruct(C.Structure):
+    _fields_ = [("family", _int), ("variant", _int), ("launches", _int), ("aux", _int),
+                ("grid", _int * 3), ("block", _int), ("lds_bytes", _int)]
+
+
+class Plan:
+    """mace_hip_plan of a call: family / variant of its main kernel, launches, auxiliary passes."""
+
+    def __init__(self, st):
+        self.family, self.variant, self.launches, self.aux = st.family, st.variant, st.launches, st.aux
+        self.grid, self.block, self.lds_bytes = tuple(st.grid), st.block, st.lds_bytes
+        self.kernel = describe(self.family, self.variant)
+
+    def __repr__(self):
+        return "Plan(%s, launches=%d, aux=0x%x, grid=%s)" % (self.kernel, self.launches, self.aux,
+                                                             self.grid)
+
+
+def describe(family, variant):
+    buf = C.create_string_buffer(256)
+    if load().mace_hip_plan_describe(family, variant, buf, 256) != SUCCESS:
+        raise ValueError("no kernel (family %d, variant %d)" % (family, variant))
+    return buf.value.decode()
+
+
+def variants(family):
+    """Variant indices of a family that name an instantiation the library can launch."""
+    lib = load()
+    return [v for v in range(lib.mace_hip_plan_variant_count(family))
+            if lib.mace_hip_plan_variant_valid(family, v)]
+
+
+def coverage(family, variant):
+    return load().mace_hip_plan_coverage(family, variant)
 
 
 class MaceHipError(RuntimeError):
@@ -150,13 +205,22 @@ def load():
 class Context:
     """One stream + one scratch arena on one GPU (mace_hip_ctx)."""
 
-    def __init__(self, device=0):
+    def __init__(self, device=0, plan_only=None):
+        """plan_only=(cu_count, lds_bytes): a context that only plans (needs no GPU)."""
         self.lib = load()
         h = _p()
-        st = self.lib.mace_hip_ctx_create(device, C.byref(h))
+        if plan_only is not None:
+            st = self.lib.mace_hip_plan_ctx_create(plan_only[0], plan_only[1], C.byref(h))
+        else:
+            st = self.lib.mace_hip_ctx_create(device, C.byref(h))
         if st != SUCCESS:
             raise MaceHipError(st, "mace_hip_ctx_create(device=%d) failed" % device)
         self.handle = h
+
+    def last_plan(self):
+        st = PlanStruct()
+        self.check(self.lib.mace_hip_last_plan(self.handle, C.byref(st)))
+        return Plan(st)
 
     def close(self):
         if getattr(self, "handle", None):
