@@ -98,9 +98,13 @@ int mace_hip_plan_variant_valid(int family, int v) {
     case MACE_HIP_KF_Q8_GEMM_RING: {
       const int cfg = v >> 3, conv = (v >> 2) & 1, sum_y = (v >> 1) & 1;
       // the gather works on 64-byte slabs in a four-stage ring and always sums Y in the kernel
-      if (conv) return sum_y && kRing[cfg][6] == 64 && kRing[cfg][4] == 4;
+      // and stores uint8 (a convolution has no int32 result)
+      if (conv) return sum_y && (v & 1) && kRing[cfg][6] == 64 && kRing[cfg][4] == 4;
       return 1;
     }
+    case MACE_HIP_KF_Q8_GEMV_GENERAL:
+      // 16-byte pieces (VEC) reach the general kernel with one vector per pass only
+      return !((v & 2) && (v >> 2) != 0);
     default:
       return 1;
   }

@@ -2253,10 +2253,8 @@ int launch_gemm_dma(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, b
   };
   if constexpr (KB == SLAB) {
     if (p.conv) {   // gathered convolution rows: always with in-kernel Y sums
-      if (out_u8)
-        MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, uint8_t, OCC, true, true>));
-      else
-        MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, int32_t, OCC, true, true>));
+      MH_CHECK(ctx, out_u8, "the convolution gather produces uint8 only");
+      MH_RETURN_IF_ERROR(launch(q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, uint8_t, OCC, true, true>));
       MH_PROF_END(ctx);
       MH_LAUNCH_CHECK(ctx);
       return MACE_HIP_SUCCESS;
@@ -2527,18 +2525,97 @@ static bool mh_q8_stream_shape(int64_t depth, int64_t xn, int64_t yn) {
          yn >= 1024;
 }
 
-int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8_t *rhs,
-               int rhs_order, void *out, int out_order, bool out_u8, int64_t batch,
-               int64_t rows, int64_t depth, int64_t cols, int lhs_batched, int rhs_batched,
-               int32_t lhs_offset, int32_t rhs_offset, const Q8GemmEpilogue &ep,
-               int64_t rhs_ld, const Q8ConvGather *cv) {
+// What every kernel family reads of a call, in the kernels' own terms: X is the operand along
+// the contiguous dimension of the result (x_is_lhs: the left-hand matrix of a ColMajor result,
+// else the right-hand matrix of a RowMajor one), Y the other.  Zero points: with z' = z - 128
+// (zl' = -lhs_offset - 128, zr' = -rhs_offset - 128) the correction of result (i, j) is
+//   -zr' * sum_k l'[i,k] + bias[i]   (left-hand side)   -zl' * sum_k r'[k,j] + K zl' zr'   (right).
+struct Q8Operand {
+  const uint8_t *ptr;
+  int64_t ld;     // k-contiguous: bytes between rows; k-major: bytes between consecutive k
+  int64_t bs;     // bytes between batches, 0 = shared
+};
+static GemmParams q8_params(bool x_is_lhs, const Q8Operand &L, const Q8Operand &R, int64_t rows,
+                            int64_t cols, int64_t depth, int k_bytes, void *out, bool out_u8,
+                            const RequantFixed &rq, int32_t lhs_offset, int32_t rhs_offset,
+                            const int32_t *bias) {
+  GemmParams p{};
+  const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
+  const int32_t l_coef = (int32_t)(0u - zr), r_coef = (int32_t)(0u - zl);
+  const int32_t r_add = (int32_t)((uint32_t)depth * zl * zr);
+  const int32_t *l_bias = out_u8 ? bias : nullptr;
+  const Q8Operand &X = x_is_lhs ? L : R, &Y = x_is_lhs ? R : L;
+  p.X = X.ptr; p.ldx = X.ld; p.xbs = X.bs;
+  p.Y = Y.ptr; p.ldy = Y.ld; p.ybs = Y.bs;
+  p.XN = (int)(x_is_lhs ? rows : cols);
+  p.YN = (int)(x_is_lhs ? cols : rows);
+  p.K = k_bytes;
+  p.out = out;
+  p.ldo = p.XN;
+  p.obs = rows * cols;
+  p.rq = rq;
+  p.xcoef = x_is_lhs ? l_coef : r_coef;
+  p.xadd = x_is_lhs ? 0 : r_add;
+  p.xbias = x_is_lhs ? l_bias : nullptr;
+  p.ycoef = x_is_lhs ? r_coef : l_coef;
+  p.yadd = x_is_lhs ? r_add : 0;
+  p.ybias = x_is_lhs ? nullptr : l_bias;
+  return p;
+}
+static void q8_params_conv(GemmParams *p, const Q8ConvGather &cv) {
+  p->conv = true;
+  p->cv_in_h = cv.in_h; p->cv_in_w = cv.in_w; p->cv_cin = cv.cin; p->cv_kw = cv.k_w;
+  p->cv_sh = cv.stride_h; p->cv_sw = cv.stride_w; p->cv_pt = cv.pad_top; p->cv_pl = cv.pad_left;
+  p->cv_oh = cv.out_h; p->cv_ow = cv.out_w;
+  p->cv_zp4 = (uint32_t)(cv.zero_point & 0xff) * 0x01010101u;
+}
+
+// One uint8 GEMM call on its way to a kernel: the arguments of mh_q8_gemm, what prepare() derives
+// from them, and the three stages of the dispatch.  Every stage is host logic only (a plan-only
+// context runs it without a GPU): small_problem() and kmajor_in_place() each either launch the
+// whole call as one kernel and set *done, or leave it to the next stage; general() repacks what
+// cannot be read in place, takes the panel sums the chosen kernel does not take itself, and
+// launches one of the tiled kernels.
+struct Q8Call {
+  mace_hip_ctx *ctx;
+  const uint8_t *lhs;
+  int lhs_order;
+  const uint8_t *rhs;
+  int rhs_order;
+  void *out;
+  int out_order;
+  bool out_u8;
+  int64_t batch, rows, depth, cols;
+  int lhs_batched, rhs_batched;
+  int32_t lhs_offset, rhs_offset;
+  const Q8GemmEpilogue &ep;
+  int64_t rhs_ld;
+  const Q8ConvGather *cv;
+  // derived by prepare()
+  RequantFixed rq{};
+  int lhs_nb = 1, rhs_nb = 1;
+  int64_t kp = 64;                       // depth rounded up to whole 64-byte slabs
+  bool lhs_direct = false, rhs_direct = false;   // the operand can be read in place
+  bool cv_small = false;                 // a gathered convolution that is a small problem
+  mh_weight *lhs_w = nullptr, *rhs_w = nullptr;  // registered as constant weights
+  bool mid_first_xt = false, mid_first_kc = false;   // the eight-wavefront kernel goes first
+  bool tail_xres = false;                // depth % 64 != 0 read in place by the resident-tile kernel
+
+  int prepare(bool *done);
+  int small_problem(bool *done);
+  int kmajor_in_place(bool *done);
+  int general();
+};
+
+// Validation (the reference's MACE_CHECKs come back as MACE_HIP_INVALID_ARGS) and the facts the
+// stages share.  *done: the result is empty.
+int Q8Call::prepare(bool *done) {
   MH_CHECK(ctx, batch >= 0 && rows >= 0 && depth >= 0 && cols >= 0, "negative dimension");
   MH_CHECK(ctx, (lhs_order | 1) == 1 && (rhs_order | 1) == 1 && (out_order | 1) == 1,
            "matrix order must be RowMajor (0) or ColMajor (1)");
   MH_CHECK(ctx, rows < (1ll << 31) && cols < (1ll << 31) && depth < (1ll << 31) - 64 &&
                     batch < 65536,
            "dimension too large");
-  RequantFixed rq{};
   if (out_u8) {
     MH_CHECK(ctx, ep.shift >= 0 && ep.shift <= 31, "right shift %d outside [0,31]", ep.shift);
     MH_CHECK(ctx, ep.lo >= 0 && ep.hi <= 255 && ep.lo <= ep.hi, "clamp range [%d,%d] invalid",
@@ -2546,14 +2623,15 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     MH_CHECK(ctx, mh_make_requant(ep.mult, ep.shift, ep.zp, ep.lo, ep.hi, &rq),
              "offset_after_shift %d outside the supported range", ep.zp);
   }
-  if (batch == 0 || rows == 0 || cols == 0) return MACE_HIP_SUCCESS;
+  if (batch == 0 || rows == 0 || cols == 0) { *done = true; return MACE_HIP_SUCCESS; }
   MH_CHECK(ctx, lhs && rhs && out, "null operand");
 
-  const int lhs_nb = lhs_batched ? (int)batch : 1, rhs_nb = rhs_batched ? (int)batch : 1;
-  const int64_t kp = (int64_t)mh_align_up((size_t)(depth > 0 ? depth : 1), 64);
+  lhs_nb = lhs_batched ? (int)batch : 1;
+  rhs_nb = rhs_batched ? (int)batch : 1;
+  kp = (int64_t)mh_align_up((size_t)(depth > 0 ? depth : 1), 64);
 
   // which operands can be read in place
-  const bool lhs_direct = lhs_order == MACE_HIP_ROW_MAJOR && depth % 16 == 0 && depth > 0 &&
+  lhs_direct = lhs_order == MACE_HIP_ROW_MAJOR && depth % 16 == 0 && depth > 0 &&
                           ((uintptr_t)lhs % 16 == 0);
   MH_CHECK(ctx, rhs_ld == 0 || (rhs_order == MACE_HIP_COL_MAJOR && rhs_ld >= depth &&
                                rhs_ld % 16 == 0 && depth > 0 && ((uintptr_t)rhs % 16 == 0)),
@@ -2562,7 +2640,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   // the streaming kernel's loader (the caller has checked the geometry, see Q8ConvGather)
   // ... or, for a small problem, by the one-launch kernel, which takes any geometry
   const bool cv_vec = cv && lhs_direct && cv->cin % 16 == 0 && ((uintptr_t)rhs % 16 == 0);
-  const bool cv_small = cv && rhs_ld == 0 && batch == 1 && out_order == MACE_HIP_COL_MAJOR &&
+  cv_small = cv && rhs_ld == 0 && batch == 1 && out_order == MACE_HIP_COL_MAJOR &&
                         lhs_order == MACE_HIP_ROW_MAJOR &&
                         mh_q8_small_problem(ctx, 1, rows, cols, depth, cv_vec, cv->cin % 64 != 0) &&
                         !(ctx->kernel_mask & MH_MASK_NO_SMALL);
@@ -2571,7 +2649,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
                      lhs_order == MACE_HIP_ROW_MAJOR && depth % SLAB == 0 && depth >= 3 * SLAB &&
                      cv->cin % SLAB == 0 && ((uintptr_t)rhs % 16 == 0) && ((uintptr_t)lhs % 16 == 0)),
            "convolution gather needs cin % 64 == 0, depth >= 192 and 16-byte aligned tensors");
-  const bool rhs_direct = cv || rhs_ld != 0 ||
+  rhs_direct = cv || rhs_ld != 0 ||
                           (rhs_order == MACE_HIP_COL_MAJOR && depth % 16 == 0 && depth > 0 &&
                            ((uintptr_t)rhs % 16 == 0));
 
@@ -2582,8 +2660,8 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
       if (w.ptr == (const void *)src && bytes <= w.bytes) return &w;
     return nullptr;
   };
-  mh_weight *lhs_w = find_weight(lhs, (size_t)lhs_nb * rows * depth);
-  mh_weight *rhs_w = (rhs_ld != 0 || cv) ? nullptr : find_weight(rhs, (size_t)rhs_nb * cols * depth);
+  lhs_w = find_weight(lhs, (size_t)lhs_nb * rows * depth);
+  rhs_w = (rhs_ld != 0 || cv) ? nullptr : find_weight(rhs, (size_t)rhs_nb * cols * depth);
 
   // At most one round of 128 x 128 tiles (and at least a quarter of one) with k >= 512: the
   // eight-wavefront kernel (q8_gemm_mid_kernel) is one launch as well and goes first where it
@@ -2609,10 +2687,10 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   const bool mid_y_direct = mid_xl ? (rhs_direct && rhs_order == MACE_HIP_COL_MAJOR) : lhs_direct;
   const bool mid_x_direct = mid_xl ? lhs_direct : (rhs_direct && rhs_order == MACE_HIP_COL_MAJOR);
   const bool mid_x_kmajor = mid_xl ? lhs_order == MACE_HIP_COL_MAJOR : rhs_order == MACE_HIP_ROW_MAJOR;
-  const bool mid_first_xt = mid_one_round && mid_x_kmajor && mid_y_direct && mid_xn % 16 == 0 &&
+  mid_first_xt = mid_one_round && mid_x_kmajor && mid_y_direct && mid_xn % 16 == 0 &&
                             (uintptr_t)(mid_xl ? lhs : rhs) % 16 == 0 &&
                             mid_xn * depth < ((int64_t)1 << 32);
-  const bool mid_first_kc = mid_one_round && mid_x_direct && mid_y_direct && depth >= 1024;
+  mid_first_kc = mid_one_round && mid_x_direct && mid_y_direct && depth >= 1024;
 
   // A depth that is a multiple of 16 but not of 64, both operands k-contiguous and read in place, a
   // long Y panel and an X tile that fits in LDS: the resident-tile kernel walks k up to the next
@@ -2620,7 +2698,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   // one-launch kernel, which otherwise takes such depths at any size, keeps the small problems
   // (200704 x 96 x 128: 25.8 us there).
   const int64_t tail_kp = (depth + 63) & ~(int64_t)63;
-  const bool tail_xres =
+  tail_xres =
       !cv && !lhs_w && !rhs_w && rhs_ld == 0 && depth > 64 && depth % 64 != 0 && depth % 16 == 0 &&
       lhs_direct && rhs_direct && lhs_order == MACE_HIP_ROW_MAJOR && rhs_order == MACE_HIP_COL_MAJOR &&
       mid_yn >= 256 &&
@@ -2628,7 +2706,10 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
           (ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536) &&
       !mh_q8_small_problem(ctx, batch, rows, cols, depth, true, false) &&
       !(ctx->kernel_mask & MH_MASK_NO_XRES);
+  return MACE_HIP_SUCCESS;
+}
 
+int Q8Call::small_problem(bool *done) {
   // Small problems: one launch that reads both operands where they lie (k-contiguous, or k-major
   // and transposed on the way into LDS) and takes both correction vectors itself.
   {
@@ -2657,36 +2738,16 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
                              ((!lhs_w && !rhs_w) || any_size) && !mid_first_xt && !mid_first_kc &&
                              !(ctx->kernel_mask & MH_MASK_NO_SMALL));
     if (small) {
-      GemmParams p{};
-      const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
-      const int32_t l_coef = (int32_t)(0u - zr), r_coef = (int32_t)(0u - zl);
-      const int32_t r_add = (int32_t)((uint32_t)depth * zl * zr);
-      const int32_t *l_bias = out_u8 ? ep.bias : nullptr;
       const bool xt = xl ? lhs_t : rhs_t, yt = xl ? rhs_t : lhs_t;
-      p.X = xl ? lhs : rhs;
-      p.Y = xl ? rhs : lhs;
-      p.XN = (int)(xl ? rows : cols);
-      p.YN = (int)(xl ? cols : rows);
-      p.K = (int)depth;
       // row pitch: k-major: bytes between consecutive k; k-contiguous: depth, or the pitch of a
       // caller-padded right-hand panel (whose padding bytes are zero after the shift)
       const int64_t rhs_pitch = rhs_ld != 0 ? rhs_ld : depth;
-      p.ldx = xt ? p.XN : (xl ? depth : rhs_pitch);
-      p.ldy = yt ? p.YN : (xl ? rhs_pitch : depth);
-      p.xbs = ((xl ? lhs_nb : rhs_nb) > 1) ? (int64_t)p.XN * (xl ? depth : rhs_pitch) : 0;
-      p.ybs = ((xl ? rhs_nb : lhs_nb) > 1) ? (int64_t)p.YN * (xl ? rhs_pitch : depth) : 0;
-      p.out = out;
-      p.ldo = p.XN;
-      p.obs = rows * cols;
-      p.rq = rq;
+      const Q8Operand L{lhs, lhs_t ? rows : depth, lhs_nb > 1 ? rows * depth : 0};
+      const Q8Operand R{rhs, rhs_t ? cols : rhs_pitch, rhs_nb > 1 ? cols * rhs_pitch : 0};
+      GemmParams p = q8_params(xl, L, R, rows, cols, depth, (int)depth, out, out_u8, rq, lhs_offset,
+                               rhs_offset, ep.bias);
       p.sum_y = true;
-      if (cv) {
-        p.conv = true;
-        p.cv_in_h = cv->in_h; p.cv_in_w = cv->in_w; p.cv_cin = cv->cin; p.cv_kw = cv->k_w;
-        p.cv_sh = cv->stride_h; p.cv_sw = cv->stride_w; p.cv_pt = cv->pad_top; p.cv_pl = cv->pad_left;
-        p.cv_oh = cv->out_h; p.cv_ow = cv->out_w;
-        p.cv_zp4 = (uint32_t)(cv->zero_point & 0xff) * 0x01010101u;
-      }
+      if (cv) q8_params_conv(&p, *cv);
       p.x_bytewise = !(xl ? lhs_vec : rhs_vec);
       p.y_bytewise = !(xl ? rhs_vec : lhs_vec);
       auto by_dwords = [&](const uint8_t *base, int64_t ld, int64_t bs, bool t, int n) {
@@ -2695,18 +2756,16 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
       p.x_dword = p.x_bytewise && by_dwords(p.X, p.ldx, p.xbs, xt, p.XN);
       p.y_dword = p.y_bytewise && (cv ? (uintptr_t)p.Y % 4 == 0 && cv->cin % 4 == 0
                                       : by_dwords(p.Y, p.ldy, p.ybs, yt, p.YN));
-      p.xcoef = xl ? l_coef : r_coef;
-      p.xadd = xl ? 0 : r_add;
-      p.xbias = xl ? l_bias : nullptr;
-      p.ycoef = xl ? r_coef : l_coef;
-      p.yadd = xl ? r_add : 0;
-      p.ybias = xl ? nullptr : l_bias;
       RequantTable tab;
       if (out_u8 && rq.table) mh_requant_table_cached(ctx, rq, tab.t);
+      *done = true;
       return launch_gemm_fused_small(ctx, p, tab, out_u8, xt, yt, (int)batch);
     }
   }
+  return MACE_HIP_SUCCESS;
+}
 
+int Q8Call::kmajor_in_place(bool *done) {
   // An X operand that lies k-major in memory (the RowMajor right-hand matrix of a MatMul with
   // RowMajor result) and whose tile fits in LDS twice per CU: the kernel that keeps the tile in
   // LDS transposes it on the way in, so nothing is repacked and the call is one launch
@@ -2722,6 +2781,14 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     const int64_t tiles128 = ((xn + 127) / 128) * ((yn + 127) / 128) * batch;
     const int64_t tiles256 = ((xn + 255) / 256) * ((yn + 255) / 256) * batch;
     const int64_t cu_n = ctx->cu_count > 0 ? ctx->cu_count : 256;
+    // the call in the kernels' terms when X is read as it lies: k-major X (xn bytes between
+    // consecutive k), k-contiguous Y
+    auto kmajor_params = [&]() {
+      const Q8Operand Xo{xp, xn, (xl ? lhs_nb : rhs_nb) > 1 ? xn * depth : 0};
+      const Q8Operand Yo{yp, depth, (xl ? rhs_nb : lhs_nb) > 1 ? yn * depth : 0};
+      return q8_params(xl, xl ? Xo : Yo, xl ? Yo : Xo, rows, cols, depth, (int)depth, out, out_u8, rq,
+                       lhs_offset, rhs_offset, ep.bias);
+    };
     // the 256 x 256 ring kernel's k-major variant applies (third block below)
     const bool big_xt = !cv && x_kmajor && y_direct && rhs_ld == 0 && !lhs_w && !rhs_w && depth >= 256 &&
                         (depth < 8192 || ctx->no_alloc || ctx->capturing) && depth % 128 == 0 &&
@@ -2738,33 +2805,11 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
         depth % 64 == 0 && xn % 16 == 0 && (uintptr_t)xp % 16 == 0 && yn >= 256 &&
         2 * (XRES_SC_BYTES + (size_t)tx * depth) <= lds_cu && !mid_first_xt &&
         !(ctx->kernel_mask & MH_MASK_NO_XRES)) {
-      GemmParams p{};
-      const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
-      const int32_t l_coef = (int32_t)(0u - zr), r_coef = (int32_t)(0u - zl);
-      const int32_t r_add = (int32_t)((uint32_t)depth * zl * zr);
-      const int32_t *l_bias = out_u8 ? ep.bias : nullptr;
-      p.X = xp;
-      p.Y = yp;
-      p.XN = (int)xn;
-      p.YN = (int)yn;
-      p.K = (int)depth;
-      p.ldx = xn;      // bytes between consecutive k
-      p.ldy = depth;
-      p.xbs = ((xl ? lhs_nb : rhs_nb) > 1) ? xn * depth : 0;
-      p.ybs = ((xl ? rhs_nb : lhs_nb) > 1) ? yn * depth : 0;
-      p.out = out;
-      p.ldo = p.XN;
-      p.obs = rows * cols;
-      p.rq = rq;
+      GemmParams p = kmajor_params();
       p.sum_y = true;
-      p.xcoef = xl ? l_coef : r_coef;
-      p.xadd = xl ? 0 : r_add;
-      p.xbias = xl ? l_bias : nullptr;
-      p.ycoef = xl ? r_coef : l_coef;
-      p.yadd = xl ? r_add : 0;
-      p.ybias = xl ? nullptr : l_bias;
       RequantTable tab;
       if (out_u8 && rq.table) mh_requant_table_cached(ctx, rq, tab.t);
+      *done = true;
       return launch_gemm_xres_any(ctx, p, tab, out_u8, (int)batch, tx, true);
     }
     // The same operand layout with a longer k, in the tile-count range of the eight-wavefront
@@ -2779,32 +2824,10 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
          (depth >= 1024 && tiles128 <= 2 * cu_n)) &&
         xn * depth < ((int64_t)1 << 32) && depth < (1 << 24) && (size_t)4 * 256 * 128 <= lds_cu &&
         !(ctx->kernel_mask & MH_MASK_NO_MID)) {
-      GemmParams p{};
-      const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
-      const int32_t l_coef = (int32_t)(0u - zr), r_coef = (int32_t)(0u - zl);
-      const int32_t r_add = (int32_t)((uint32_t)depth * zl * zr);
-      const int32_t *l_bias = out_u8 ? ep.bias : nullptr;
-      p.X = xp;
-      p.Y = yp;
-      p.XN = (int)xn;
-      p.YN = (int)yn;
-      p.K = (int)depth;
-      p.ldx = xn;      // bytes between consecutive k
-      p.ldy = depth;
-      p.xbs = ((xl ? lhs_nb : rhs_nb) > 1) ? xn * depth : 0;
-      p.ybs = ((xl ? rhs_nb : lhs_nb) > 1) ? yn * depth : 0;
-      p.out = out;
-      p.ldo = p.XN;
-      p.obs = rows * cols;
-      p.rq = rq;
-      p.xcoef = xl ? l_coef : r_coef;
-      p.xadd = xl ? 0 : r_add;
-      p.xbias = xl ? l_bias : nullptr;
-      p.ycoef = xl ? r_coef : l_coef;
-      p.yadd = xl ? r_add : 0;
-      p.ybias = xl ? nullptr : l_bias;
+      GemmParams p = kmajor_params();
       RequantTable tab;
       if (out_u8 && rq.table) mh_requant_table_cached(ctx, rq, tab.t);
+      *done = true;
       return launch_gemm_mid(ctx, p, tab, out_u8, (int)batch, true);
     }
     // ... and where the 256 x 256 tiles are the choice: the ring kernel's k-major variant; the
@@ -2820,30 +2843,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
       int32_t *sum_x = (int32_t *)mh_arena_take(ctx, sizeof(int32_t) * x_nb * xn);
       int32_t *sum_y_buf = (int32_t *)mh_arena_take(ctx, sizeof(int32_t) * y_nb * yn);
       if (!sum_x || !sum_y_buf) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
-      GemmParams p{};
-      const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
-      const int32_t l_coef = (int32_t)(0u - zr), r_coef = (int32_t)(0u - zl);
-      const int32_t r_add = (int32_t)((uint32_t)depth * zl * zr);
-      const int32_t *l_bias = out_u8 ? ep.bias : nullptr;
-      p.X = xp;
-      p.Y = yp;
-      p.XN = (int)xn;
-      p.YN = (int)yn;
-      p.K = (int)depth;
-      p.ldx = xn;      // bytes between consecutive k
-      p.ldy = depth;
-      p.xbs = (x_nb > 1) ? xn * depth : 0;
-      p.ybs = (y_nb > 1) ? yn * depth : 0;
-      p.out = out;
-      p.ldo = p.XN;
-      p.obs = rows * cols;
-      p.rq = rq;
-      p.xcoef = xl ? l_coef : r_coef;
-      p.xadd = xl ? 0 : r_add;
-      p.xbias = xl ? l_bias : nullptr;
-      p.ycoef = xl ? r_coef : l_coef;
-      p.yadd = xl ? r_add : 0;
-      p.ybias = xl ? nullptr : l_bias;
+      GemmParams p = kmajor_params();
       p.corrX = sum_x;
       p.corrY = sum_y_buf;
       p.cxbs = x_nb > 1 ? p.XN : 0;
@@ -2859,10 +2859,14 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
         MH_RETURN_IF_ERROR(launch_panel_sums(ctx, yp, depth, p.ybs, yn, (int)depth, y_nb, sum_y_buf));
       RequantTable tab;
       if (out_u8 && rq.table) mh_requant_table_cached(ctx, rq, tab.t);
+      *done = true;
       return launch_gemm_big_xt(ctx, p, tab, out_u8, (int)batch, sum_x_in_kernel);
     }
   }
+  return MACE_HIP_SUCCESS;
+}
 
+int Q8Call::general() {
   size_t need = sizeof(int32_t) * ((size_t)lhs_nb * rows + (size_t)rhs_nb * cols) + 4096 + 512;
   if (!lhs_direct && !lhs_w) need += (size_t)lhs_nb * rows * kp + 256;
   if (!rhs_direct && !rhs_w) need += (size_t)rhs_nb * cols * kp + 256;
@@ -3051,11 +3055,7 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
                              rhs_ld != 0 ? rhs_ld : depth, rhs_w,
                              ((x_is_lhs && sum_y_shape) || sums_in_kernel) ? nullptr : corrR, &R,
                              x_flip && !x_is_lhs));
-  const uint32_t zl = (uint32_t)(-lhs_offset) - 128u, zr = (uint32_t)(-rhs_offset) - 128u;
   const bool sum_y = cv || (sum_y_shape && !(x_is_lhs ? R.sums : L.sums));   // cached sums cost nothing
-  const int32_t l_coef = (int32_t)(0u - zr), l_add = 0;
-  const int32_t r_coef = (int32_t)(0u - zl), r_add = (int32_t)((uint32_t)depth * zl * zr);
-  const int32_t *l_bias = out_u8 ? ep.bias : nullptr;
   // A small X panel (at most 128 rows of at most 64 bytes: an early 1x1 convolution's filter) against a
   // long Y panel goes to the streaming kernel, which also sums both panels itself.
   const int64_t xn = x_is_lhs ? rows : cols, yn = x_is_lhs ? cols : rows;
@@ -3114,41 +3114,24 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
     MH_LAUNCH_CHECK(ctx);
   }
 
-  GemmParams p;
   const Panel &PX = x_is_lhs ? L : R;
   const Panel &PY = x_is_lhs ? R : L;
   // a panel written already shifted to int8 has exactly one consumer (see x_flip above)
   MH_CHECK(ctx, !PY.flipped && (!PX.flipped || (!xres && !stream && !mid)),
            "internal: shifted panel outside the 256 x 256 kernel");
-  p.X = PX.ptr; p.ldx = PX.ld; p.xbs = PX.bs;
-  p.Y = PY.ptr; p.ldy = PY.ld; p.ybs = PY.bs;
-  p.XN = (int)(x_is_lhs ? rows : cols);
-  p.YN = (int)(x_is_lhs ? cols : rows);
-  p.K = L.k < R.k ? L.k : R.k;    // padded tails are zero after the shift, so the shorter wins
+  // (padded tails are zero after the shift, so the shorter of the two readable lengths wins)
+  GemmParams p = q8_params(x_is_lhs, Q8Operand{L.ptr, L.ld, L.bs}, Q8Operand{R.ptr, R.ld, R.bs}, rows,
+                           cols, depth, L.k < R.k ? L.k : R.k, out, out_u8, rq, lhs_offset, rhs_offset,
+                           ep.bias);
   p.corrX = x_is_lhs ? sumL : sumR;
   p.corrY = x_is_lhs ? sumR : sumL;
   p.cxbs = (x_is_lhs ? lhs_nb : rhs_nb) > 1 ? p.XN : 0;
   p.cybs = (x_is_lhs ? rhs_nb : lhs_nb) > 1 ? p.YN : 0;
-  p.out = out;
-  p.ldo = p.XN;
-  p.obs = rows * cols;
-  p.rq = rq;
   RequantTable tab;
   if (out_u8 && rq.table) mh_requant_table_cached(ctx, rq, tab.t);
   p.sum_y = sum_y;
-  p.ycoef = x_is_lhs ? r_coef : l_coef;
-  p.yadd = x_is_lhs ? r_add : l_add;
-  p.ybias = x_is_lhs ? nullptr : l_bias;
-  p.xcoef = x_is_lhs ? l_coef : r_coef;
-  p.xadd = x_is_lhs ? l_add : r_add;
-  p.xbias = x_is_lhs ? l_bias : nullptr;
-  p.tiles_x = p.tiles_y = 0;
-  p.conv = cv != nullptr;
-  p.cv_zero = nullptr;
   if (cv) {
-    p.cv_in_h = cv->in_h; p.cv_in_w = cv->in_w; p.cv_cin = cv->cin; p.cv_kw = cv->k_w;
-    p.cv_sh = cv->stride_h; p.cv_sw = cv->stride_w; p.cv_pt = cv->pad_top; p.cv_pl = cv->pad_left;
-    p.cv_oh = cv->out_h; p.cv_ow = cv->out_w;
+    q8_params_conv(&p, *cv);
     uint8_t *zero = (uint8_t *)mh_arena_take(ctx, 256);
     if (!zero) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
     MH_RETURN_IF_ERROR(mh_fill_bytes(ctx, zero, (uint8_t)cv->zero_point, 256));
@@ -3208,6 +3191,23 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   if (skinny) return launch_gemm<1, 4, 2, 2>(ctx, p, tab, out_u8, (int)batch);
   if (medium) return launch_gemm<2, 2, 2, 2>(ctx, p, tab, out_u8, (int)batch);
   return launch_gemm<2, 2, 1, 1>(ctx, p, tab, out_u8, (int)batch);
+}
+
+int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8_t *rhs,
+               int rhs_order, void *out, int out_order, bool out_u8, int64_t batch,
+               int64_t rows, int64_t depth, int64_t cols, int lhs_batched, int rhs_batched,
+               int32_t lhs_offset, int32_t rhs_offset, const Q8GemmEpilogue &ep,
+               int64_t rhs_ld, const Q8ConvGather *cv) {
+  Q8Call call{ctx, lhs, lhs_order, rhs, rhs_order, out, out_order, out_u8, batch, rows, depth, cols,
+              lhs_batched, rhs_batched, lhs_offset, rhs_offset, ep, rhs_ld, cv};
+  bool done = false;
+  MH_RETURN_IF_ERROR(call.prepare(&done));
+  if (done) return MACE_HIP_SUCCESS;
+  MH_RETURN_IF_ERROR(call.small_problem(&done));
+  if (done) return MACE_HIP_SUCCESS;
+  MH_RETURN_IF_ERROR(call.kmajor_in_place(&done));
+  if (done) return MACE_HIP_SUCCESS;
+  return call.general();
 }
 
 extern "C" {

@@ -807,20 +807,21 @@ int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
     return MACE_HIP_SUCCESS;
   }
   dim3 grid((unsigned)((p.H + 3) / 4), (unsigned)((p.batch + nb - 1) / nb));
-#define MH_GEMV_LAUNCH(NB_)                                                              \
-  do {                                                                                   \
-    if (vec)                                                                             \
-      MH_KLAUNCH(ctx, (q8_gemv_kernel<NB_, true, OutT>), grid, block, 0, ctx->stream, p); \
-    else                                                                                 \
-      MH_KLAUNCH(ctx, (q8_gemv_kernel<NB_, false, OutT>), grid, block, 0, ctx->stream, p); \
-  } while (0)
-  mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMV_GENERAL, mhv::gemv_general(nb, vec, out_u8), grid, block, 0);
+  // (rows made of aligned 16-byte pieces reach this kernel with one vector per pass only: with
+  // more, one of the kernels above has taken the call)
+  const bool vec1 = vec && nb == 1;
+#define MH_GEMV_LAUNCH(NB_) MH_KLAUNCH(ctx, (q8_gemv_kernel<NB_, false, OutT>), grid, block, 0, ctx->stream, p)
+  mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMV_GENERAL, mhv::gemv_general(nb, vec1, out_u8), grid, block, 0);
   MH_PROF_BEGIN(ctx);
-  switch (nb) {
-    case 8: MH_GEMV_LAUNCH(8); break;
-    case 4: MH_GEMV_LAUNCH(4); break;
-    case 2: MH_GEMV_LAUNCH(2); break;
-    default: MH_GEMV_LAUNCH(1); break;
+  if (vec1) {
+    MH_KLAUNCH(ctx, (q8_gemv_kernel<1, true, OutT>), grid, block, 0, ctx->stream, p);
+  } else {
+    switch (nb) {
+      case 8: MH_GEMV_LAUNCH(8); break;
+      case 4: MH_GEMV_LAUNCH(4); break;
+      case 2: MH_GEMV_LAUNCH(2); break;
+      default: MH_GEMV_LAUNCH(1); break;
+    }
   }
 #undef MH_GEMV_LAUNCH
   MH_PROF_END(ctx);

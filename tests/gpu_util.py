@@ -45,3 +45,19 @@ def as_major(mat, major):
     if major == mh.ROW_MAJOR:
         return np.ascontiguousarray(mat).reshape(-1)
     return np.ascontiguousarray(np.swapaxes(mat, -1, -2)).reshape(-1)
+
+
+_TAGS = {mh.KF_Q8_GEMM_FUSED_SMALL: "small", mh.KF_Q8_GEMM_XRES: "xres", mh.KF_Q8_GEMM_MID: "mid",
+         mh.KF_Q8_GEMM_STREAM: "stream", mh.KF_Q8_GEMM_RING: "ring", mh.KF_Q8_GEMM_RING_XT: "ring_xt",
+         mh.KF_Q8_GEMM_RING_XF: "ring_xf", mh.KF_Q8_GEMM_TILED: "tiled"}
+
+
+def kernel_tag(plan):
+    """Short name of the uint8 GEMM kernel family a call ran (mace_hip_last_plan), with /XT where
+    a k-major operand was read in place, /TAIL where a depth tail was, /CONV where patches were
+    gathered: what the family-aimed parity tests assert."""
+    tag = _TAGS.get(plan.family, plan.kernel)
+    for flag in ("XT", "TAIL", "CONV"):
+        if (flag + "=true") in plan.kernel and plan.family != mh.KF_Q8_GEMM_RING_XT:
+            tag += "/" + flag
+    return tag

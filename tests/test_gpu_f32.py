@@ -78,6 +78,14 @@ def test_gemm_f32_parity(ctx, batch, rows, cols, depth, lm, rm, om, lb, rb):
     Rr = rng.standard_normal(((batch if rb else 1), depth, cols)).astype(np.float32)
     l, r = as_major(L, lm), as_major(Rr, rm)
     got = gemm_host(ctx, l, r, batch, rows, cols, depth, lm, rm, om, lb, rb)
+    plan = ctx.last_plan()
+    # the groups of GEMM_CASES aimed at one variant of the 16-byte-load kernel reach it
+    if (batch, rows, cols, depth) in ((2, 256, 128, 48), (2, 200, 260, 48), (64, 128, 256, 128)):
+        assert plan.family == mh.KF_F32_GEMM_VEC and "SPLIT=2" in plan.kernel, plan
+    if (rows, cols) in ((2304, 2304), (1100, 1300), (2048, 2304)) or (batch, rows) == (5, 1028):
+        assert plan.family == mh.KF_F32_GEMM_VEC and "SPLIT=1" in plan.kernel, plan
+    if (rows, cols, depth) == (47, 69, 37):
+        assert plan.family == mh.KF_F32_GEMM_GENERAL, plan
     near(got, orc.gemm_f32(l, r, batch, rows, cols, depth, lm, rm, om, lb, rb))
     near(got, orc.gemm_f32(l, r, batch, rows, cols, depth, lm, rm, om, lb, rb, acc64=True))
 
@@ -117,6 +125,8 @@ def test_gemm_f32_config2(ctx, ta, tb):
     dA, dB = d.put(A), d.put(B)
     d.sync()
     ctx.call("mace_hip_gemm_f32_transpose", dA, dB, b, n, n, n, n, ta, tb, 0, 1, 1, p)
+    assert ctx.last_plan().kernel == "f32_gemm_vec_kernel<LK=%s,RK=%s,SPLIT=2>" % (
+        "false" if ta else "true", "true" if tb else "false")
     ctx.sync()
     got = t.cpu().numpy().copy()
     lm, rm = (Cm if ta else R), (Cm if tb else R)
@@ -147,6 +157,7 @@ def test_gemm_f32_config2_small(ctx):
     for ta in (0, 1):
         for tb in (0, 1):
             ctx.call("mace_hip_gemm_f32_transpose", dA, dB, b, n, n, n, n, ta, tb, 0, 1, 1, p)
+            assert "SPLIT=2" in ctx.last_plan().kernel
             ctx.sync()
             got = t.cpu().numpy().copy()
             lm, rm = (Cm if ta else R), (Cm if tb else R)

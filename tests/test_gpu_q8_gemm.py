@@ -7,7 +7,7 @@ import pytest
 
 from mace_amd import lib as mh
 from oracle import mace_oracle as orc
-from gpu_util import Dev, as_major, c_, ptr
+from gpu_util import Dev, as_major, c_, kernel_tag, ptr
 
 pytestmark = pytest.mark.gpu
 R, Cm = mh.ROW_MAJOR, mh.COL_MAJOR
@@ -79,6 +79,8 @@ def test_q8_gemm_parity(ctx, path, batch, rows, depth, cols, lb, rb, lo, ro, oo)
 
 
 def check_gemm(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo):
+    """int32 and uint8 results against the oracle; returns what mace_hip_last_plan named as the kernel
+    of the int32 call and of the last uint8 call (gpu_util.kernel_tag)."""
     rng = np.random.default_rng(rows * 31 + depth * 7 + cols + lo * 4 + ro * 2 + oo)
     L = rng.integers(0, 256, ((batch if lb else 1), rows, depth), dtype=np.uint8)
     Rr = rng.integers(0, 256, ((batch if rb else 1), depth, cols), dtype=np.uint8)
@@ -86,6 +88,7 @@ def check_gemm(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo):
     lzp, rzp = int(rng.integers(0, 256)), int(rng.integers(0, 256))
     want = orc.q8_gemm_i32(l, r, batch, rows, cols, depth, -lzp, -rzp, lo, ro, oo, lb, rb)
     got = gemm_i32_host(ctx, l, lo, r, ro, oo, batch, rows, depth, cols, lb, rb, -lzp, -rzp)
+    tag32 = kernel_tag(ctx.last_plan())
     np.testing.assert_array_equal(got, want)
     mult, shift = scales_for(depth)
     bias = rng.integers(-2 ** 15, 2 ** 15, rows).astype(np.int32)
@@ -97,70 +100,88 @@ def check_gemm(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo):
         np.testing.assert_array_equal(got8, want8)
     if rows * cols >= 64:
         assert len(np.unique(want8)) > 8       # the uint8 check is not vacuous
+    return tag32, kernel_tag(ctx.last_plan())
 
 
 # The kernel that keeps the X panel in LDS (k a multiple of 64 after packing, at least 256 rows on
 # the other side): 64- and 128-row tiles, 64- and 128-byte k groups, ragged edges on both sides,
 # several blocks per wavefront, repacked operands, both result orders, batches.
-XRES_SHAPES = [  # batch, rows, depth, cols, lhs order, rhs order, out order
-    (1, 300, 128, 128, R, Cm, R), (1, 1000, 192, 100, R, Cm, R), (2, 260, 64, 40, R, Cm, R),
-    (1, 4096, 256, 256, R, Cm, R), (1, 140000, 64, 48, R, Cm, R), (1, 512, 100, 128, Cm, R, R),
-    (1, 96, 128, 700, R, Cm, Cm), (1, 300, 1024, 64, R, Cm, R), (1, 512, 512, 128, R, Cm, R),
-    (3, 333, 320, 130, R, R, R), (1, 70000, 128, 160, R, Cm, R),
+XRES_SHAPES = [  # batch, rows, depth, cols, lhs order, rhs order, out order, kernel without the one-launch kernel
+    (1, 300, 128, 128, R, Cm, R, "xres"), (1, 1000, 192, 100, R, Cm, R, "xres"),
+    (2, 260, 64, 40, R, Cm, R, "xres"), (1, 4096, 256, 256, R, Cm, R, "xres"),
+    (1, 512, 100, 128, Cm, R, R, "xres"), (1, 96, 128, 700, R, Cm, Cm, "xres"),
+    (1, 300, 1024, 64, R, Cm, R, "xres"), (1, 512, 512, 128, R, Cm, R, "xres"),
+    (3, 333, 320, 130, R, R, R, "xres"), (1, 70000, 128, 160, R, Cm, R, "xres"),
     # X operand k-major in memory (RowMajor right-hand matrix, or ColMajor left-hand matrix with a
     # ColMajor result): transposed on its way into LDS, nothing repacked
-    (1, 300, 128, 128, R, R, R), (4, 512, 512, 512, R, R, R), (1, 1000, 192, 112, R, R, R),
-    (2, 260, 64, 48, R, R, R), (1, 96, 128, 700, Cm, Cm, Cm), (1, 4100, 576, 272, R, R, R),
-    # long k in 64-row tiles (128 rows would not fit in LDS twice)
-    (1, 3136, 1024, 500, R, Cm, R), (1, 4000, 768, 250, R, Cm, R),
-    # operands in place with a depth that is not a multiple of 64: the one-launch kernel at any
-    # size (more workgroups than it otherwise takes)
-    (1, 100000, 48, 40, R, Cm, R), (2, 70000, 144, 24, R, Cm, R),
+    (1, 300, 128, 128, R, R, R, "xres/XT"), (1, 1000, 192, 112, R, R, R, "xres/XT"),
+    (2, 260, 64, 48, R, R, R, "xres/XT"), (1, 96, 128, 700, Cm, Cm, Cm, "xres/XT"),
+    (1, 4100, 576, 272, R, R, R, "xres/XT"),
+    # long k in 64-row tiles (128 rows would not fit in LDS twice; k % 128 != 0 keeps the
+    # eight-wavefront kernel away)
+    (1, 3136, 960, 500, R, Cm, R, "xres"), (1, 5000, 960, 250, R, Cm, R, "xres"),
+    # a depth tail read in place
+    (2, 70000, 144, 24, R, Cm, R, "xres/TAIL"),
+    # neighbours that other kernels take: a short, narrow X panel (uint8 only), one round of
+    # 128 x 128 tiles, a depth below 64 that is not a multiple of 64
+    (1, 140000, 64, 48, R, Cm, R, "stream"), (4, 512, 512, 512, R, R, R, "mid/XT"),
+    (1, 3136, 1024, 500, R, Cm, R, "mid"), (1, 100000, 48, 40, R, Cm, R, "tiled"),
 ]
 
 
-@pytest.mark.parametrize("batch,rows,depth,cols,lo,ro,oo", XRES_SHAPES)
-def test_q8_gemm_x_panel_in_lds(ctx, path, batch, rows, depth, cols, lo, ro, oo):
-    check_gemm(ctx, batch, rows, depth, cols, True, True, lo, ro, oo)
+@pytest.mark.parametrize("batch,rows,depth,cols,lo,ro,oo,kernel", XRES_SHAPES)
+def test_q8_gemm_x_panel_in_lds(ctx, path, batch, rows, depth, cols, lo, ro, oo, kernel):
+    tag32, tag8 = check_gemm(ctx, batch, rows, depth, cols, True, True, lo, ro, oo)
+    if path == "no_small_kernel":      # (by default most of these are one launch of the small-problem kernel)
+        assert tag8 == kernel
+        assert tag32 == ("xres" if kernel == "stream" else kernel)     # the streaming kernel stores uint8 only
+    if path == "general_path":
+        assert tag8.split("/")[0] in ("ring", "tiled", "mid", "stream") and tag32.split("/")[0] != "xres"
 
 
 # The kernel with eight wavefronts per 128 x 128 tile (64 to 640 tiles, k a multiple of 128 from 512
 # on): it sums both panels itself and splits every slab's k steps between two groups of wavefronts;
 # 4, 5, 6, 7 and 8 slabs, ragged edges on both sides, repacked and in-place operands, both result
 # orders, batches, one side shared.
-MID_SHAPES = [  # batch, rows, depth, cols, lhs batched, rhs batched, lhs order, rhs order, out order
-    (1, 1500, 640, 1410, True, True, R, Cm, R), (1, 1408, 512, 1536, True, True, R, R, R),
-    (1, 1537, 768, 1300, True, True, Cm, R, Cm), (2, 1100, 896, 1000, True, True, R, Cm, R),
-    (2, 1024, 512, 1100, False, True, Cm, Cm, R), (1, 2048, 1024, 2048, True, True, R, Cm, Cm),
-    (3, 900, 512, 1000, True, False, R, R, Cm),
+MID_SHAPES = [  # batch, rows, depth, cols, lhs batched, rhs batched, lhs order, rhs order, out order, kernel
+    (1, 1500, 640, 1410, True, True, R, Cm, R, "mid"), (1, 1408, 512, 1536, True, True, R, R, R, "mid/XT"),
+    (1, 1537, 768, 1300, True, True, Cm, R, Cm, "mid"), (2, 1100, 896, 1000, True, True, R, Cm, R, "mid"),
+    (2, 1024, 512, 1100, False, True, Cm, Cm, R, "mid"), (1, 2048, 1024, 2048, True, True, R, Cm, Cm, "mid"),
+    (3, 900, 512, 1000, True, False, R, R, Cm, "mid"),
     # both ends of the range of tile counts it takes: a quarter of a round, more than one round
-    (1, 1000, 512, 1024, True, True, R, Cm, R), (1, 2300, 2048, 2200, True, True, R, Cm, R),
+    (1, 1000, 512, 1024, True, True, R, Cm, R, "mid"), (1, 2300, 2048, 2200, True, True, R, Cm, R, "mid"),
     # X operand k-major in memory (RowMajor right-hand matrix with a RowMajor result, ColMajor
     # left-hand matrix with a ColMajor result): read through the transposing LDS loads, nothing
     # repacked; ragged last tiles in both directions, batches, one side shared
-    (1, 1536, 1024, 1488, True, True, R, R, R), (2, 1000, 640, 1040, True, True, R, R, R),
-    (1, 1296, 1280, 1500, True, True, Cm, Cm, Cm), (2, 1100, 512, 1200, True, False, R, R, R),
-    (1, 2048, 2048, 2048, True, True, R, R, R),
+    (1, 1536, 1024, 1488, True, True, R, R, R, "mid/XT"), (2, 1000, 640, 1040, True, True, R, R, R, "mid/XT"),
+    (1, 1296, 1280, 1500, True, True, Cm, Cm, Cm, "mid/XT"), (2, 1100, 512, 1200, True, False, R, R, R, "mid/XT"),
+    (1, 2048, 2048, 2048, True, True, R, R, R, "mid/XT"),
     # the same operand layout at sizes that take 256 x 256 tiles: each operand's sums in the kernel
     # (k <= 1024 or the other dimension <= 4096) or from a pass of their own, ragged last tiles,
     # ColMajor everything
-    (1, 3000, 256, 4000, True, True, R, R, R), (1, 4000, 384, 3024, True, True, Cm, Cm, Cm),
-    (1, 2900, 1152, 4112, True, True, R, R, R), (1, 4200, 1152, 2048, True, True, R, R, R),
+    (1, 3000, 256, 4000, True, True, R, R, R, "ring_xt"), (1, 4000, 384, 3024, True, True, Cm, Cm, Cm, "ring_xt"),
+    (1, 2900, 1152, 4112, True, True, R, R, R, "ring_xt"), (1, 4200, 1152, 2048, True, True, R, R, R, "ring_xt"),
     # long enough k that the repacked panel of the tiled path is written already shifted to int8
-    (1, 2900, 1280, 4112, True, True, R, R, R),
+    (1, 2900, 1280, 4112, True, True, R, R, R, "ring_xt"),
 ]
 
 
-@pytest.mark.parametrize("batch,rows,depth,cols,lb,rb,lo,ro,oo", MID_SHAPES)
+@pytest.mark.parametrize("batch,rows,depth,cols,lb,rb,lo,ro,oo,kernel", MID_SHAPES)
 @pytest.mark.parametrize("mid", ["one_round_kernel", "tiled_kernels"])
-def test_q8_gemm_one_round_of_tiles(ctx, mid, batch, rows, depth, cols, lb, rb, lo, ro, oo):
-    # (the kernel that keeps one panel in LDS would take the 512-deep shapes: switched off here)
-    ctx.call("mace_hip_ctx_set_kernel_mask",
-             mh.MASK_NO_XRES | (0 if mid == "one_round_kernel" else mh.MASK_NO_MID))
+def test_q8_gemm_one_round_of_tiles(ctx, mid, batch, rows, depth, cols, lb, rb, lo, ro, oo, kernel):
+    # (the one-launch kernel and the kernel that keeps one panel in LDS would take the shallower
+    # shapes: switched off here)
+    ctx.call("mace_hip_ctx_set_kernel_mask", mh.MASK_NO_SMALL | mh.MASK_NO_XRES |
+             (0 if mid == "one_round_kernel" else mh.MASK_NO_MID))
     try:
-        check_gemm(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo)
+        tag32, tag8 = check_gemm(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo)
     finally:
         ctx.call("mace_hip_ctx_set_kernel_mask", 0)
+    if mid == "one_round_kernel":
+        assert (tag32, tag8) == (kernel, kernel)
+    else:   # the ring kernel on repacked / in-place k-contiguous panels
+        want = "ring_xf" if depth >= 1280 and kernel == "ring_xt" else "ring"
+        assert (tag32, tag8) == (want, want)
 
 
 # Shapes on the boundaries between the one-launch kernels under the normal dispatch: the
@@ -169,18 +190,18 @@ def test_q8_gemm_one_round_of_tiles(ctx, mid, batch, rows, depth, cols, lb, rb, 
 # 256 x 256 kernel with a k-major operand in place ahead of the resident-tile kernel (at most one
 # round of its tiles, k >= 384), and their neighbours just outside.
 DISPATCH_SHAPES = [
-    (16, 512, 512, 512, True, True, R, R, R), (4, 512, 512, 512, True, True, R, R, R),
-    (1, 2048, 512, 2048, True, True, R, Cm, R), (1, 1024, 1024, 1024, True, True, R, Cm, R),
-    (1, 1024, 896, 1024, True, True, R, Cm, R), (1, 1100, 640, 1200, True, True, R, R, R),
-    (1, 3000, 512, 4000, True, True, R, R, R), (1, 4000, 384, 3024, True, True, Cm, Cm, Cm),
-    (1, 3000, 256, 4000, True, True, R, R, R), (2, 2048, 512, 2064, True, False, R, R, R),
-    (1, 760, 512, 1024, True, True, R, R, R),
+    (16, 512, 512, 512, True, True, R, R, R, "mid/XT"), (4, 512, 512, 512, True, True, R, R, R, "mid/XT"),
+    (1, 2048, 512, 2048, True, True, R, Cm, R, "mid"), (1, 1024, 1024, 1024, True, True, R, Cm, R, "mid"),
+    (1, 1024, 896, 1024, True, True, R, Cm, R, "small"), (1, 1100, 640, 1200, True, True, R, R, R, "mid/XT"),
+    (1, 3000, 512, 4000, True, True, R, R, R, "ring_xt"), (1, 4000, 384, 3024, True, True, Cm, Cm, Cm, "ring_xt"),
+    (1, 3000, 256, 4000, True, True, R, R, R, "xres/XT"), (2, 2048, 512, 2064, True, False, R, R, R, "ring_xt"),
+    (1, 760, 512, 1024, True, True, R, R, R, "small/XT"),
 ]
 
 
-@pytest.mark.parametrize("batch,rows,depth,cols,lb,rb,lo,ro,oo", DISPATCH_SHAPES)
-def test_q8_gemm_dispatch_boundaries(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo):
-    check_gemm(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo)
+@pytest.mark.parametrize("batch,rows,depth,cols,lb,rb,lo,ro,oo,kernel", DISPATCH_SHAPES)
+def test_q8_gemm_dispatch_boundaries(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo, kernel):
+    assert check_gemm(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo) == (kernel, kernel)
 
 
 # Depths that are a multiple of 16 but not of 64 with both operands k-contiguous: read in place by
@@ -188,11 +209,11 @@ def test_q8_gemm_dispatch_boundaries(ctx, batch, rows, depth, cols, lb, rb, lo, 
 # 64- and 128-row tiles; 32- and 64-row blocks; ragged rows and columns; the result transposed;
 # batches), and the same shapes through the other kernels.
 TAIL_SHAPES = [
-    (1, 9000, 96, 128, True, True, R, Cm, R), (1, 9000, 144, 128, True, True, R, Cm, R),
-    (1, 9000, 176, 64, True, True, R, Cm, R), (1, 70000, 80, 48, True, True, R, Cm, R),
-    (1, 5003, 208, 200, True, True, R, Cm, R), (2, 3000, 112, 130, True, True, R, Cm, R),
-    (1, 128, 160, 9000, True, True, R, Cm, Cm), (1, 20000, 336, 256, True, True, R, Cm, R),
-    (3, 4000, 96, 128, True, False, R, Cm, R),
+    (1, 40000, 96, 128, True, True, R, Cm, R), (1, 40000, 144, 128, True, True, R, Cm, R),
+    (1, 70000, 176, 64, True, True, R, Cm, R), (1, 70000, 80, 48, True, True, R, Cm, R),
+    (1, 35003, 208, 200, True, True, R, Cm, R), (2, 20000, 112, 130, True, True, R, Cm, R),
+    (1, 128, 160, 40000, True, True, R, Cm, Cm), (1, 20000, 336, 256, True, True, R, Cm, R),
+    (3, 14000, 96, 128, True, False, R, Cm, R), (1, 280000, 96, 64, True, True, R, Cm, R),
 ]
 
 
@@ -201,9 +222,11 @@ TAIL_SHAPES = [
 def test_q8_gemm_depth_tail_in_place(ctx, kernels, batch, rows, depth, cols, lb, rb, lo, ro, oo):
     ctx.call("mace_hip_ctx_set_kernel_mask", 0 if kernels == "normal" else mh.MASK_NO_XRES)
     try:
-        check_gemm(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo)
+        tags = check_gemm(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo)
     finally:
         ctx.call("mace_hip_ctx_set_kernel_mask", 0)
+    # (without the resident-tile kernel such depths go to the one-launch kernel at any size)
+    assert tags == (("xres/TAIL", "xres/TAIL") if kernels == "normal" else ("small", "small"))
 
 
 def test_q8_gemm_config1_matmul(ctx):
@@ -272,20 +295,26 @@ def test_q8_gemm_requant_at_every_step(ctx, mult, shift, zp, clamp, rows, cols, 
         assert len(np.unique(want8)) > 100
 
 
-@pytest.mark.parametrize("xn,depth,yn,batch", [
-    (64, 32, 4096, 1), (32, 32, 1031, 1), (128, 128, 2048, 1), (256, 256, 1500, 1),
-    (64, 64, 1024, 3), (128, 32, 5000, 1), (256, 64, 1111, 2), (32, 256, 1025, 1),
-    (128, 64, 3000, 2), (64, 32, 2049, 1), (64, 128, 1056, 1), (32, 64, 40000, 1),
+@pytest.mark.parametrize("xn,depth,yn,batch,kernel", [
+    (64, 32, 4096, 1, "stream"), (32, 32, 1031, 1, "stream"), (128, 128, 2048, 1, "xres"),
+    (256, 256, 1500, 1, "xres"), (64, 64, 1024, 3, "stream"), (128, 32, 5000, 1, "stream"),
+    (256, 64, 1111, 2, "xres"), (32, 256, 1025, 1, "xres"), (128, 64, 3000, 2, "stream"),
+    (64, 32, 2049, 1, "stream"), (64, 128, 1056, 1, "xres"), (32, 64, 40000, 1, "stream"),
     # panels that do not fill their last 32-row block, depths with half a k step at the tail
-    (16, 32, 3000, 1), (96, 16, 2500, 1), (48, 48, 1100, 2), (112, 64, 1500, 1), (80, 16, 1024, 1),
-    (128, 48, 20000, 1), (16, 16, 5000, 1),
+    (16, 32, 3000, 1, "stream"), (96, 16, 2500, 1, "stream"), (48, 48, 1100, 2, "stream"),
+    (112, 64, 1500, 1, "stream"), (80, 16, 1024, 1, "stream"), (128, 48, 20000, 1, "stream"),
+    (16, 16, 5000, 1, "stream"),
+    # long enough that the normal dispatch itself picks the streaming kernel
+    (64, 32, 70000, 1, "stream"), (128, 64, 40000, 1, "stream"),
 ])
 @pytest.mark.parametrize("x_is_lhs", [True, False])
-def test_q8_gemm_small_panel_streaming(ctx, xn, depth, yn, batch, x_is_lhs):
+def test_q8_gemm_small_panel_streaming(ctx, xn, depth, yn, batch, x_is_lhs, kernel):
     """A small operand (at most 256 x 256) against a long one, both k-contiguous, uint8 result
     with the small dimension contiguous: the shapes of a 1x1 convolution (filter as the
     left-hand side, column-major result) and of a MatMul with a narrow right-hand side.  Long
-    dimensions include non-multiples of 32; the bias runs along either side."""
+    dimensions include non-multiples of 32; the bias runs along either side.  The one-launch
+    kernel, which takes most of these sizes by default, is switched off, so that the streaming
+    kernel (panels of at most 128 rows x 64 bytes) and the resident-tile kernel (the others) run."""
     rng = np.random.default_rng(xn * 7 + depth * 3 + yn + batch)
     if x_is_lhs:    # lhs [xn x depth] RowMajor, rhs [depth x yn] ColMajor, result ColMajor
         rows, cols, oo = xn, yn, Cm
@@ -297,12 +326,17 @@ def test_q8_gemm_small_panel_streaming(ctx, xn, depth, yn, batch, x_is_lhs):
     lzp, rzp = int(rng.integers(120, 136)), int(rng.integers(120, 136))   # keeps the mean small
     mult, shift = scales_for(depth)
     bias = rng.integers(-2 ** 15, 2 ** 15, rows).astype(np.int32)
-    for bb, zp, clamp in ((bias, 90, (90, 200)), (None, 0, (0, 255)), (bias, 128, (0, 255))):
-        want8 = orc.q8_gemm_u8(l, r, batch, rows, cols, depth, -lzp, -rzp, bb, mult, shift, zp,
-                               clamp[0], clamp[1], R, Cm, oo, True, True)
-        got8 = gemm_u8_host(ctx, l, R, r, Cm, oo, batch, rows, depth, cols, True, True, -lzp,
-                            -rzp, bb, mult, shift, zp, clamp[0], clamp[1])
-        np.testing.assert_array_equal(got8, want8)
+    ctx.call("mace_hip_ctx_set_kernel_mask", 0 if yn >= 40000 and xn >= 64 else mh.MASK_NO_SMALL)
+    try:
+        for bb, zp, clamp in ((bias, 90, (90, 200)), (None, 0, (0, 255)), (bias, 128, (0, 255))):
+            want8 = orc.q8_gemm_u8(l, r, batch, rows, cols, depth, -lzp, -rzp, bb, mult, shift, zp,
+                                   clamp[0], clamp[1], R, Cm, oo, True, True)
+            got8 = gemm_u8_host(ctx, l, R, r, Cm, oo, batch, rows, depth, cols, True, True, -lzp,
+                                -rzp, bb, mult, shift, zp, clamp[0], clamp[1])
+            assert kernel_tag(ctx.last_plan()) == kernel
+            np.testing.assert_array_equal(got8, want8)
+    finally:
+        ctx.call("mace_hip_ctx_set_kernel_mask", 0)
     assert len(np.unique(want8)) > 8       # zero point 128: both signs of the sums survive
 
 
@@ -333,22 +367,23 @@ def test_q8_gemm_large_device_pointers(ctx, n, lo, ro, oo):
     assert sat < 0.5, sat
 
 
-@pytest.mark.parametrize("batch,rows,depth,cols,lo,ro,oo,with_bias", [
-    (1, 3100, 384, 3300, R, Cm, R, True),     # 256 x 256 tiles, 128-byte slabs, ragged last tiles
-    (1, 3100, 256, 3300, R, Cm, Cm, False),   # ... shortest k that kernel takes (two slabs)
-    (2, 2100, 640, 2200, R, Cm, R, True),     # ... batched
-    (1, 1100, 1024, 1300, R, Cm, R, True),    # 128 x 128 tiles, 128-byte slabs
-    (1, 1100, 1152, 1300, R, R, Cm, False),   # ... through the repack, column-major result
-    (1, 1700, 1024, 1800, R, Cm, R, True),    # ... 210 tiles: the eight-wavefront variant, ragged
-    (1, 1800, 1152, 1700, R, Cm, Cm, False),  # ... column-major result
-    (1, 2049, 448, 2305, R, Cm, R, True),     # 128 x 128 tiles, 64-byte slabs (k % 128 != 0)
-    (1, 4352, 256, 4608, R, Cm, R, True),     # 17 x 18 aligned 256 x 256 tiles: more than one per CU
-    (1, 4608, 384, 4352, R, Cm, Cm, False),   # ... odd number of slabs, column-major result
+@pytest.mark.parametrize("batch,rows,depth,cols,lo,ro,oo,with_bias,tile", [
+    (1, 3100, 384, 3300, R, Cm, R, True, "2,2,4,4,STAGES=2"),    # 256 x 256 tiles, 128-byte slabs, ragged last tiles
+    (1, 3100, 256, 3300, R, Cm, Cm, False, "2,2,4,4,STAGES=2"),  # ... shortest k that kernel takes (two slabs)
+    (2, 2100, 640, 2200, R, Cm, R, True, "2,2,4,4,STAGES=2"),    # ... batched
+    (1, 1100, 1024, 1300, R, Cm, R, True, "2,2,2,2,STAGES=2"),   # 128 x 128 tiles, 128-byte slabs
+    (1, 1100, 1152, 1300, R, R, Cm, False, "2,2,2,2,STAGES=2"),  # ... through the repack, column-major result
+    (1, 1700, 1024, 1800, R, Cm, R, True, "2,4,2,1,STAGES=2"),   # ... 210 tiles: the eight-wavefront variant, ragged
+    (1, 1800, 1152, 1700, R, Cm, Cm, False, "2,4,2,1,STAGES=2"), # ... column-major result
+    (1, 2049, 448, 2305, R, Cm, R, True, "2,2,2,2,STAGES=4"),    # 128 x 128 tiles, 64-byte slabs (k % 128 != 0)
+    (1, 4352, 256, 4608, R, Cm, R, True, "2,2,4,4,STAGES=2"),    # 17 x 18 aligned 256 x 256 tiles: more than one per CU
+    (1, 4608, 384, 4352, R, Cm, Cm, False, "2,2,4,4,STAGES=2"),  # ... odd number of slabs, column-major result
 ])
-def test_q8_gemm_ragged_tiled(ctx, batch, rows, depth, cols, lo, ro, oo, with_bias):
-    """Shapes large enough for the 256 x 256 and 128 x 128 tile kernels whose sides are not
-    multiples of the tile: every edge workgroup clamps its loads and masks its stores.  Both
-    outputs compared in full with the oracle."""
+def test_q8_gemm_ragged_tiled(ctx, batch, rows, depth, cols, lo, ro, oo, with_bias, tile):
+    """Shapes large enough for the 256 x 256 and 128 x 128 tiles of the ring kernel whose sides are
+    not multiples of the tile: every edge workgroup clamps its loads and masks its stores.  Both
+    outputs compared in full with the oracle.  (The one-launch, resident-tile and eight-wavefront
+    kernels, which the normal dispatch prefers on these shapes, are switched off.)"""
     rng = np.random.default_rng(rows + depth + cols + batch)
     A = rng.integers(0, 256, (batch, rows, depth), dtype=np.uint8)
     B = rng.integers(0, 256, (batch, depth, cols), dtype=np.uint8)
@@ -361,11 +396,19 @@ def test_q8_gemm_ragged_tiled(ctx, batch, rows, depth, cols, lo, ro, oo, with_bi
     t32, p32 = d.empty(batch * rows * cols, np.int32)
     t8, p8 = d.empty(batch * rows * cols, np.uint8)
     d.sync()
-    ctx.call("mace_hip_gemm_q8_i32", dl, lo, dr, ro, p32, oo, batch, rows, depth, cols, 1, 1, -za, -zb)
     mult, shift = scales_for(depth)
-    ctx.call("mace_hip_gemm_q8_u8", dl, lo, dr, ro, p8, oo, batch, rows, depth, cols, 1, 1, -za, -zb,
-             db, mult, shift, zc, 0, 255)
+    ctx.call("mace_hip_ctx_set_kernel_mask", mh.MASK_NO_SMALL | mh.MASK_NO_XRES | mh.MASK_NO_MID)
+    try:
+        ctx.call("mace_hip_gemm_q8_i32", dl, lo, dr, ro, p32, oo, batch, rows, depth, cols, 1, 1, -za, -zb)
+        plan32 = ctx.last_plan()
+        ctx.call("mace_hip_gemm_q8_u8", dl, lo, dr, ro, p8, oo, batch, rows, depth, cols, 1, 1, -za, -zb,
+                 db, mult, shift, zc, 0, 255)
+        plan8 = ctx.last_plan()
+    finally:
+        ctx.call("mace_hip_ctx_set_kernel_mask", 0)
     ctx.sync()
+    for plan in (plan32, plan8):
+        assert plan.family == mh.KF_Q8_GEMM_RING and ("<" + tile) in plan.kernel, plan
     want32 = orc.q8_gemm_i32(l, r, batch, rows, cols, depth, -za, -zb, lo, ro, oo)
     np.testing.assert_array_equal(t32.cpu().numpy().reshape(want32.shape), want32)
     want8 = orc.output_pipeline_u8(want32, batch, rows, cols, oo, bias, mult, shift, zc)

@@ -143,3 +143,55 @@ def test_q8_gemv_errors(ctx):
     # empty problems succeed and write nothing
     assert ctx.status("mace_hip_gemv_q8_i32_host", ptr(z), ptr(z), None, 0, 4, 4, 0, 1, 0, 0,
                       ptr(np.zeros(1, np.int32))) == mh.SUCCESS
+
+
+# One case (at least) per kernel family and row-length class of the dispatch, with the kernel that
+# ran asserted: rows of exactly U KiB and in between (WHOLE or not), per-batch weights (BATCHED),
+# the matrix-core kernels for shared weights (k slices, LDS-staged, straight from memory), the
+# row-block kernel, and the general kernel on rows that are not 16-byte pieces.
+FAMILY_CASES = [  # batch, h, w, lhs batched, kernel (without the output type)
+    (1, 77, 1024, False, "q8_gemv_row_kernel<U=1,BATCHED=false,WHOLE=true"),
+    (1, 77, 1008, False, "q8_gemv_row_kernel<U=1,BATCHED=false,WHOLE=false"),
+    (1, 77, 2048, False, "q8_gemv_row_kernel<U=2,BATCHED=false,WHOLE=true"),
+    (1, 77, 1536, False, "q8_gemv_row_kernel<U=2,BATCHED=false,WHOLE=false"),
+    (1, 77, 3072, False, "q8_gemv_row_kernel<U=4,BATCHED=false,WHOLE=false"),
+    (1, 77, 4096, False, "q8_gemv_row_kernel<U=4,BATCHED=false,WHOLE=true"),
+    (1, 77, 5120, False, "q8_gemv_row_kernel<U=8,BATCHED=false,WHOLE=false"),
+    (1, 77, 8192, False, "q8_gemv_row_kernel<U=8,BATCHED=false,WHOLE=true"),
+    (3, 45, 8192, True, "q8_gemv_row_kernel<U=8,BATCHED=true,WHOLE=true"),
+    (3, 45, 4096, True, "q8_gemv_row_kernel<U=4,BATCHED=true,WHOLE=true"),
+    (3, 45, 2048, True, "q8_gemv_row_kernel<U=2,BATCHED=true,WHOLE=true"),
+    (3, 45, 1008, True, "q8_gemv_row_kernel<U=1,BATCHED=true,WHOLE=false"),
+    (8, 77, 4096, False, "q8_gemv_mfma_slice_kernel<SPW=4"),
+    (5, 77, 2048, False, "q8_gemv_mfma_slice_kernel<SPW=2"),
+    (15, 33, 1024, False, "q8_gemv_mfma_slice_kernel<SPW=1"),
+    (3, 45, 8192, False, "q8_gemv_mfma_lds_kernel<16"),
+    (8, 45, 9216, False, "q8_gemv_mfma_kernel<"),
+    (2, 77, 4096, False, "q8_gemv_rows_kernel<R=1,NB=2,NWAVES=16"),
+    (1, 50, 9216, False, "q8_gemv_rows_kernel<R=1,NB=1,NWAVES=16"),
+    (1, 77, 4001, False, "q8_gemv_kernel<NB=1,VEC=false"),
+    (8, 20, 4001, False, "q8_gemv_kernel<NB=8,VEC=false"),
+    (1, 9, 70000, False, "q8_gemv_kernel<NB=1,VEC=true"),
+]
+
+
+@pytest.mark.parametrize("batch,h,w,lb,kernel", FAMILY_CASES)
+def test_q8_gemv_kernel_families(ctx, batch, h, w, lb, kernel):
+    rng = np.random.default_rng(77 + batch * 5 + h + w)
+    L = rng.integers(0, 256, ((batch if lb else 1), h, w), dtype=np.uint8)
+    x = rng.integers(0, 256, (batch, w), dtype=np.uint8)
+    bias = rng.integers(-2 ** 15, 2 ** 15, h).astype(np.int32)
+    sigma = 74.0 * 74.0 * np.sqrt(w)
+    scales = (np.float32(0.01), np.float32(0.02), np.float32(0.0002 * sigma / 40.0))
+    for bb in (bias, None):
+        lzp, rzp = int(rng.integers(0, 256)), int(rng.integers(0, 256))
+        want = orc.q8_gemv_i32(L, x, bb, batch, h, w, lzp, rzp, lb, True)
+        got = run_host(ctx, L, x, bb, batch, h, w, lb, True, lzp, rzp, False)
+        assert ctx.last_plan().kernel == kernel + ("," if kernel[-1] != "<" else "") + "int32_t>"
+        np.testing.assert_array_equal(got, want)
+        for mode, ozp in ((mh.REQUANT_REF, 57), (mh.REQUANT_NEON, 57), (mh.REQUANT_NEON, 0)):
+            want = orc.q8_gemv_u8(L, x, bb, batch, h, w, 127, 128, *scales, ozp, mode, lb, True)
+            got = run_host(ctx, L, x, bb, batch, h, w, lb, True, 127, 128, True, scales, ozp, mode)
+            assert ctx.last_plan().kernel == kernel + ("," if kernel[-1] != "<" else "") + "uint8_t>"
+            np.testing.assert_array_equal(got, want)
+    assert len(np.unique(got)) > min(10, h // 2)
