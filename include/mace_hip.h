@@ -196,6 +196,19 @@ int mace_hip_memcpy_d2h(mace_hip_ctx *ctx, void *dst_host, const void *src_dev, 
  * was derived (after synchronizing the stream); so does destroying the context. */
 int mace_hip_weight_register(mace_hip_ctx *ctx, const void *device_ptr, size_t bytes);
 int mace_hip_weight_unregister(mace_hip_ctx *ctx, const void *device_ptr);
+/* The same for a constant operand that lives in HOST memory -- MACE's weights when the ops are
+ * bound through the *_host entry points.  Registering uploads `bytes` from host_ptr into device
+ * memory owned by the context once (and registers that copy as above); from then on every
+ * *_host call on this context whose lhs, rhs, filter, weight or bias pointer equals host_ptr (and
+ * reads at most `bytes`) uses the copy instead of staging the operand again, so a call moves its
+ * activations only.  The counterpart of the reference's pack cache, which likewise stops reading
+ * the original weight once packed (it even AdviseFree()s it, mace/ops/arm/base/gemm.cc:612-617).
+ * The caller registers again after changing the weight (the copy is refreshed and what was
+ * derived from it dropped) and unregisters before freeing it. */
+int mace_hip_host_weight_register(mace_hip_ctx *ctx, const void *host_ptr, size_t bytes);
+int mace_hip_host_weight_unregister(mace_hip_ctx *ctx, const void *host_ptr);
+/* Uploads made / operands found resident by *_host calls so far (for tests). */
+int mace_hip_host_weight_stats(mace_hip_ctx *ctx, int64_t *uploads, int64_t *hits);
 /* Number of times a registered weight's panel was built / reused so far (for tests). */
 int mace_hip_weight_cache_stats(mace_hip_ctx *ctx, int64_t *builds, int64_t *hits);
 

@@ -23,6 +23,7 @@
 #include <cstdint>
 #include <cstdlib>
 #include <functional>
+#include <initializer_list>
 #include <cmath>
 #include <memory>
 #include <numeric>
@@ -53,8 +54,18 @@ enum RuntimeType { RT_CPU = 0, RT_OPENCL = 2 };            // include/mace/publi
 enum ImplType { REF = 0, NEON };                            // mace/core/ops/op_delegator.h:25-28
 const ImplType kCpuImplType = ImplType::REF;                // :30-34 on a non-NEON host
 enum MatrixMajor { RowMajor = MACE_HIP_ROW_MAJOR, ColMajor = MACE_HIP_COL_MAJOR };
+// mace/ops/common/activation_type.h; the kernels of this library apply the first three
 enum ActivationType { NOOP = MACE_HIP_ACT_NOOP, RELU = MACE_HIP_ACT_RELU,
-                      RELUX = MACE_HIP_ACT_RELUX };
+                      RELUX = MACE_HIP_ACT_RELUX, PRELU = 3, TANH = 4, SIGMOID = 5, LEAKYRELU = 6,
+                      ELU = 7, HARDSIGMOID = 8 };
+// mace/ops/common/activation_type.h StringToActivationType; false for a name it does not know
+inline bool StringToActivationType(const std::string &name, ActivationType *type) {
+  static const char *const names[] = {"NOOP", "RELU", "RELUX", "PRELU", "TANH", "SIGMOID",
+                                      "LEAKYRELU", "ELU", "HARDSIGMOID"};
+  for (int i = 0; i < 9; ++i)
+    if (name == names[i]) { *type = static_cast<ActivationType>(i); return true; }
+  return false;
+}
 
 template <typename T> struct DataTypeToEnum;
 template <> struct DataTypeToEnum<float> { static const DataType value = DT_FLOAT; };
@@ -266,6 +277,72 @@ class Conv2d : public OpDelegator {            // mace/ops/delegator/conv_2d.h:6
 
 }  // namespace delegator
 
+// Where the operands of a call live.  The C ABI has two families of entry points -- device
+// pointers, ordered on the context's stream, and host pointers, staged and synchronous -- and a
+// call must go to one of them as a whole: every operand has to live where the output does.  A mix
+// (say a device output with a weight still in host memory, the natural state of a half-migrated
+// integration) would hand a host address to a kernel, so it is refused before anything is launched.
+inline bool SamePlacement(const Tensor *output, std::initializer_list<const Tensor *> inputs) {
+  for (const Tensor *t : inputs)
+    if (t != nullptr && t->on_device() != output->on_device()) return false;
+  return true;
+}
+
+// A constant operand kept resident across calls.  MACE's delegators may keep a packed copy of a
+// weight (GemmParam::should_cache_pack_ with Tensor::is_weight(), mace/ops/delegator/gemm.h:28-33,
+// mace/ops/arm/base/gemm.cc:560-576, which then stops reading the original).  Counterpart: an
+// operand that is_weight() is registered with the library context once per op instance --
+//   * in device memory: its repacked uint8 panel and row sums are kept across Run() calls;
+//   * in host memory: it is uploaded once, and the host-pointer entry points then move only the
+//     activations (the registered copy also keeps its panel and sums).
+// A weight whose buffer moves is registered afresh; Refresh() re-registers one whose contents the
+// caller has changed.  The registration ends with the op (or when the weight moves): the caches are
+// keyed by address, and once the weight's buffer has been freed the allocator may hand the same
+// address to an activation tensor, which must not find a stale copy.  The op must be destroyed
+// before its library context is.
+class WeightRegistration {
+ public:
+  WeightRegistration() = default;
+  WeightRegistration(const WeightRegistration &) = delete;
+  WeightRegistration &operator=(const WeightRegistration &) = delete;
+  ~WeightRegistration() { Release(); }
+  void Note(const OpContext *context, const Tensor *t, size_t bytes) {
+    if (t == nullptr || !t->is_weight() || bytes == 0) return;
+    const void *ptr = t->data<uint8_t>();
+    if (ptr == registered_ && context->hip() == ctx_ && bytes == bytes_ && t->on_device() == device_)
+      return;
+    Release();
+    const int rc = t->on_device() ? mace_hip_weight_register(context->hip(), ptr, bytes)
+                                  : mace_hip_host_weight_register(context->hip(), ptr, bytes);
+    if (rc == MACE_HIP_SUCCESS) {
+      registered_ = ptr;
+      ctx_ = context->hip();
+      bytes_ = bytes;
+      device_ = t->on_device();
+    }
+  }
+  // the caller has written new values into the registered weight
+  void Refresh() {
+    if (registered_ == nullptr) return;
+    if (device_) (void)mace_hip_weight_register(ctx_, registered_, bytes_);
+    else (void)mace_hip_host_weight_register(ctx_, registered_, bytes_);
+  }
+  void Release() {
+    if (registered_ != nullptr) {
+      if (device_) (void)mace_hip_weight_unregister(ctx_, registered_);
+      else (void)mace_hip_host_weight_unregister(ctx_, registered_);
+    }
+    registered_ = nullptr;
+    ctx_ = nullptr;
+  }
+
+ private:
+  const void *registered_ = nullptr;
+  mace_hip_ctx *ctx_ = nullptr;
+  size_t bytes_ = 0;
+  bool device_ = false;
+};
+
 // ---- the GPU delegators --------------------------------------------------------------------------------
 namespace hip {
 
@@ -273,13 +350,23 @@ template <typename T> class Gemm;
 template <>
 class Gemm<float> : public delegator::Gemm {   // replaces ref::Gemm<float> / arm::Gemm<float>
  public:
-  explicit Gemm(const delegator::GemmParam &param) : delegator::Gemm(param) {}
+  explicit Gemm(const delegator::GemmParam &param)
+      : delegator::Gemm(param), should_cache_pack_(param.should_cache_pack_) {}
   MaceStatus Compute(const OpContext *context, const Tensor *lhs, const Tensor *rhs,
                      const index_t batch, const index_t rows, const index_t cols,
                      const index_t depth, const MatrixMajor lhs_major,
                      const MatrixMajor rhs_major, const MatrixMajor output_major,
                      const bool lhs_batched, const bool rhs_batched,
                      Tensor *output) override {
+    if (!SamePlacement(output, {lhs, rhs})) return MaceStatus::MACE_INVALID_ARGS;
+    // mace/ops/arm/base/gemm.cc:560-576: with should_cache_pack_, the weight side (the left one
+    // first) is kept across calls unless it differs per batch
+    if (should_cache_pack_) {
+      if (lhs->is_weight() && (!lhs_batched || batch == 1))
+        cache_.Note(context, lhs, sizeof(float) * static_cast<size_t>(rows * depth));
+      else if (rhs->is_weight() && (!rhs_batched || batch == 1))
+        cache_.Note(context, rhs, sizeof(float) * static_cast<size_t>(depth * cols));
+    }
     auto fn = output->on_device() ? mace_hip_gemm_f32 : mace_hip_gemm_f32_host;
     return ToStatus(fn(context->hip(), lhs->data<float>(), rhs->data<float>(), batch, rows,
                        cols, depth, lhs_major, rhs_major, output_major, lhs_batched,
@@ -301,6 +388,10 @@ class Gemm<float> : public delegator::Gemm {   // replaces ref::Gemm<float> / ar
                    transpose_lhs ? ColMajor : RowMajor, transpose_rhs ? ColMajor : RowMajor,
                    transpose_out ? ColMajor : RowMajor, lhs_batched, rhs_batched, output);
   }
+
+ private:
+  const bool should_cache_pack_;
+  WeightRegistration cache_;
 };
 
 template <typename T> class Gemv;
@@ -312,11 +403,28 @@ class Gemv<float> : public delegator::Gemv {   // replaces ref::Gemv<float> / ar
                      const Tensor *bias, const index_t batch, const index_t lhs_height,
                      const index_t lhs_width, const bool lhs_batched, const bool rhs_batched,
                      Tensor *output) override {
-    auto fn = output->on_device() ? mace_hip_gemv_f32 : mace_hip_gemv_f32_host;
+    return ComputeFused(context, lhs, rhs, bias, batch, lhs_height, lhs_width, lhs_batched,
+                        rhs_batched, NOOP, 0.f, output);
+  }
+  // Compute followed by the Activation delegator as FullyConnectedOp runs it
+  // (mace/ops/fully_connected.cc:108-121), applied as the sums are stored.
+  MaceStatus ComputeFused(const OpContext *context, const Tensor *lhs, const Tensor *rhs,
+                          const Tensor *bias, const index_t batch, const index_t lhs_height,
+                          const index_t lhs_width, const bool lhs_batched, const bool rhs_batched,
+                          ActivationType activation, float max_limit, Tensor *output) {
+    if (!SamePlacement(output, {lhs, rhs, bias})) return MaceStatus::MACE_INVALID_ARGS;
+    // a constant weight matrix (and bias) stays on the GPU between calls
+    if (!lhs_batched) weight_.Note(context, lhs, sizeof(float) * static_cast<size_t>(lhs_height * lhs_width));
+    if (bias) bias_.Note(context, bias, sizeof(float) * static_cast<size_t>(lhs_height));
+    auto fn = output->on_device() ? mace_hip_gemv_f32_act : mace_hip_gemv_f32_act_host;
     return ToStatus(fn(context->hip(), lhs->data<float>(), rhs->data<float>(),
                        bias ? bias->data<float>() : nullptr, batch, lhs_height, lhs_width,
-                       lhs_batched, rhs_batched, output->mutable_data<float>()));
+                       lhs_batched, rhs_batched, activation, max_limit,
+                       output->mutable_data<float>()));
   }
+
+ private:
+  WeightRegistration weight_, bias_;
 };
 // Replaces ref::q8::Gemv<uint8_t> (requant_mode REF) / arm::q8::Gemv<uint8_t> (NEON).
 template <>
@@ -328,6 +436,9 @@ class Gemv<uint8_t> : public delegator::Gemv {
                      const Tensor *bias, const index_t batch, const index_t lhs_height,
                      const index_t lhs_width, const bool lhs_batched, const bool rhs_batched,
                      Tensor *output) override {
+    if (!SamePlacement(output, {lhs, rhs, bias})) return MaceStatus::MACE_INVALID_ARGS;
+    if (!lhs_batched) weight_.Note(context, lhs, static_cast<size_t>(lhs_height * lhs_width));
+    if (bias) bias_.Note(context, bias, sizeof(int32_t) * static_cast<size_t>(lhs_height));
     auto fn = output->on_device() ? mace_hip_gemv_q8_u8 : mace_hip_gemv_q8_u8_host;
     return ToStatus(fn(context->hip(), lhs->data<uint8_t>(), rhs->data<uint8_t>(),
                        bias ? bias->data<int32_t>() : nullptr, batch, lhs_height, lhs_width,
@@ -338,6 +449,7 @@ class Gemv<uint8_t> : public delegator::Gemv {
 
  private:
   int requant_mode_;
+  WeightRegistration weight_, bias_;
 };
 template <>
 class Gemv<int32_t> : public delegator::Gemv {   // replaces ref::q8::Gemv<int32_t>
@@ -347,12 +459,18 @@ class Gemv<int32_t> : public delegator::Gemv {   // replaces ref::q8::Gemv<int32
                      const Tensor *bias, const index_t batch, const index_t lhs_height,
                      const index_t lhs_width, const bool lhs_batched, const bool rhs_batched,
                      Tensor *output) override {
+    if (!SamePlacement(output, {lhs, rhs, bias})) return MaceStatus::MACE_INVALID_ARGS;
+    if (!lhs_batched) weight_.Note(context, lhs, static_cast<size_t>(lhs_height * lhs_width));
+    if (bias) bias_.Note(context, bias, sizeof(int32_t) * static_cast<size_t>(lhs_height));
     auto fn = output->on_device() ? mace_hip_gemv_q8_i32 : mace_hip_gemv_q8_i32_host;
     return ToStatus(fn(context->hip(), lhs->data<uint8_t>(), rhs->data<uint8_t>(),
                        bias ? bias->data<int32_t>() : nullptr, batch, lhs_height, lhs_width,
                        lhs_batched, rhs_batched, lhs->zero_point(), rhs->zero_point(),
                        output->mutable_data<int32_t>()));
   }
+
+ private:
+  WeightRegistration weight_, bias_;
 };
 
 // The float Conv2d delegator, NCHW input {n, cin, h, w}, OIHW filter {cout, cin, kh, kw}, output
@@ -404,14 +522,20 @@ class Conv2d<float> : public delegator::Conv2d {
     const bool k1x1 = filter->dim(2) == 1 && filter->dim(3) == 1 && strides_[0] == 1 &&
                       strides_[1] == 1 && dilations_[0] == 1 && dilations_[1] == 1;
     if (!k1x1) return MaceStatus::MACE_UNSUPPORTED;   // stays with ref::Conv2d
+    if (!SamePlacement(output, {input, filter, bias})) return MaceStatus::MACE_INVALID_ARGS;
     MaceStatus st = output->Resize({input->dim(0), filter->dim(0), out_h, out_w});
     if (st != MaceStatus::MACE_SUCCESS) return st;
+    filter_.Note(context, filter, sizeof(float) * static_cast<size_t>(filter->size()));
+    if (bias) bias_.Note(context, bias, sizeof(float) * static_cast<size_t>(bias->size()));
     auto fn = output->on_device() ? mace_hip_conv2d_f32_nchw : mace_hip_conv2d_f32_nchw_host;
     return ToStatus(fn(context->hip(), input->data<float>(), filter->data<float>(),
                        bias ? bias->data<float>() : nullptr, input->dim(0), input->dim(1),
                        input->dim(2), input->dim(3), filter->dim(0), 1, 1, 1, 1, 1, 1, pads[0],
                        pads[1], activation, max_limit, output->mutable_data<float>()));
   }
+
+ private:
+  WeightRegistration filter_, bias_;
 };
 // The same delegator under the name the NEON build registers for the K1x1 tag
 // (mace/ops/arm/base/conv_2d_1x1.cc:74-88).
@@ -523,6 +647,7 @@ class MatMulOpFloat {
                             s.rhs_batched, C);
     // "bias' dim should be <= 2." (:196-197), checked before anything is written
     if (bias->dim_size() != 1 || bias->dim(0) != s.cols) return MaceStatus::MACE_INVALID_ARGS;
+    if (!SamePlacement(C, {lhs, rhs, bias})) return MaceStatus::MACE_INVALID_ARGS;
     auto fn = C->on_device() ? mace_hip_matmul_f32 : mace_hip_matmul_f32_host;
     return ToStatus(fn(context->hip(), lhs->data<float>(), rhs->data<float>(), bias->data<float>(),
                        s.batch, s.lhs_rows, s.lhs_cols, s.rhs_rows, s.rhs_cols, transpose_a_,
@@ -540,42 +665,7 @@ class MatMulOpFloat {
 // uses the pipeline MakeNoBias(A.scale, B.scale, C.scale, C.zero_point), the int32 result
 // sets C.scale = A.scale * B.scale and C.zero_point = 0.  The gemmlowp call is not behind a
 // delegator in the reference, so the op calls the C ABI directly.
-// MatMulOp's constructor passes is_weight() of either operand to the Gemm delegator as
-// GemmParam::should_cache_pack_ (mace/ops/matmul.cc:101-108), which then keeps the packed operand
-// (arm/base/gemm.cc:560-576).  Counterpart: an operand that is a constant weight AND lives in device
-// memory is registered with the context once per op instance; its repacked panel and row sums are
-// then kept across Run() calls.  A weight whose buffer moves is registered afresh.
-// The registration ends with the op (or when the weight moves): the cache is keyed by address,
-// and once the weight's buffer has been freed the allocator may hand the same address to an
-// activation tensor, which must not find a stale panel.  The op must be destroyed before its
-// library context is.
-class WeightRegistration {
- public:
-  WeightRegistration() = default;
-  WeightRegistration(const WeightRegistration &) = delete;
-  WeightRegistration &operator=(const WeightRegistration &) = delete;
-  ~WeightRegistration() { Release(); }
-  void Note(OpContext *context, const Tensor *t, size_t bytes) {
-    if (!t->is_weight() || !t->on_device()) return;
-    const void *ptr = t->data<uint8_t>();
-    if (ptr == registered_ && context->hip() == ctx_) return;
-    Release();
-    if (mace_hip_weight_register(context->hip(), ptr, bytes) == MACE_HIP_SUCCESS) {
-      registered_ = ptr;
-      ctx_ = context->hip();
-    }
-  }
-  void Release() {
-    if (registered_ != nullptr) (void)mace_hip_weight_unregister(ctx_, registered_);
-    registered_ = nullptr;
-    ctx_ = nullptr;
-  }
-
- private:
-  const void *registered_ = nullptr;
-  mace_hip_ctx *ctx_ = nullptr;
-};
-
+// A constant operand (is_weight()) is kept resident across Run() calls (WeightRegistration).
 class MatMulOpQuant {
  public:
   MatMulOpQuant(bool transpose_a, bool transpose_b, DataType output_type)
@@ -585,6 +675,7 @@ class MatMulOpQuant {
     MaceStatus st = MatMulInferShape(A, B, transpose_a_, transpose_b_, &s);
     if (st != MaceStatus::MACE_SUCCESS) return st;
     if ((st = C->Resize(s.output_shape)) != MaceStatus::MACE_SUCCESS) return st;
+    if (!SamePlacement(C, {A, B})) return MaceStatus::MACE_INVALID_ARGS;
     const int a_order = transpose_a_ ? MACE_HIP_COL_MAJOR : MACE_HIP_ROW_MAJOR;
     const int b_order = transpose_b_ ? MACE_HIP_COL_MAJOR : MACE_HIP_ROW_MAJOR;
     weight_a_.Note(context, A, static_cast<size_t>(A->size()));
@@ -617,11 +708,18 @@ class MatMulOpQuant {
 };
 
 // FullyConnectedOp<RT_CPU, uint8_t>::Run (mace/ops/fully_connected.cc:141-179) and the float op
-// (:82-121) up to the Gemv call: weight OIHW, output {N,1,1,O} (uint8) / {N,O,1,1} (float).
+// (:82-121): weight OIHW, output {N,1,1,O} (uint8) / {N,O,1,1} (float).  The float op runs its
+// Activation delegator on the Gemv's output (:62-75,121: the op's "activation" / "max_limit"
+// arguments; mace/ops/ref/activation.cc:61-75); the quantized op has none (the converter folds a
+// quantized ReLU into the output range).  With the GPU Gemv the activation is applied as the sums
+// are stored; with any other Gemv delegator it is the reference's host loop.  NOOP, RELU and RELUX
+// are applied; any other type makes Run return MACE_UNSUPPORTED before anything is computed.
 template <typename T>
 class FullyConnectedOp {
  public:
-  explicit FullyConnectedOp(OpDelegatorRegistry *registry) {
+  explicit FullyConnectedOp(OpDelegatorRegistry *registry, ActivationType activation = NOOP,
+                            float max_limit = 0.f)
+      : activation_(activation), max_limit_(max_limit) {
     auto vc = registry->GetCreator(MACE_HIP_DELEGATOR_KEY(Gemv, RT_CPU, T, kCpuImplType));
     if (vc) gemv_.reset(static_cast<delegator::Gemv *>(vc(DelegatorParam()).release()));
   }
@@ -639,11 +737,27 @@ class FullyConnectedOp {
     MaceStatus st = output->Resize(out_shape);
     if (st != MaceStatus::MACE_SUCCESS) return st;
     const index_t input_size = weight->dim(1) * weight->dim(2) * weight->dim(3);
-    return gemv_->Compute(context, weight, input, bias, input->dim(0), weight->dim(0),
-                          input_size, false, true, output);
+    if (std::is_same<T, float>::value) {
+      if (activation_ != NOOP && activation_ != RELU && activation_ != RELUX)
+        return MaceStatus::MACE_UNSUPPORTED;
+      if (auto *fused = dynamic_cast<hip::Gemv<float> *>(gemv_.get()))
+        return fused->ComputeFused(context, weight, input, bias, input->dim(0), weight->dim(0),
+                                   input_size, false, true, activation_, max_limit_, output);
+    }
+    st = gemv_->Compute(context, weight, input, bias, input->dim(0), weight->dim(0), input_size,
+                        false, true, output);
+    if (st != MaceStatus::MACE_SUCCESS || !std::is_same<T, float>::value || activation_ == NOOP)
+      return st;
+    if (output->on_device()) return MaceStatus::MACE_UNSUPPORTED;   // host loop below
+    float *o = output->template mutable_data<float>();
+    for (index_t i = 0; i < output->size(); ++i)
+      o[i] = std::max(0.f, activation_ == RELUX ? std::min(max_limit_, o[i]) : o[i]);
+    return st;
   }
 
  private:
+  ActivationType activation_;
+  float max_limit_;
   std::unique_ptr<delegator::Gemv> gemv_;
 };
 
@@ -689,9 +803,11 @@ class Conv2dOpQuant {
       out_w = static_cast<int64_t>(
           std::floor(1.0 * (input->dim(2) + pads[1] - filter->dim(2)) / strides_[1]) + 1);
     }
+    if (!SamePlacement(output, {input, filter, bias})) return MaceStatus::MACE_INVALID_ARGS;
     MaceStatus st = output->Resize({input->dim(0), out_h, out_w, filter->dim(0)});
     if (st != MaceStatus::MACE_SUCCESS) return st;
     weight_.Note(context, filter, static_cast<size_t>(filter->size()));   // filters are constants
+    if (bias) bias_.Note(context, bias, sizeof(int32_t) * static_cast<size_t>(bias->size()));
     auto fn = output->on_device() ? mace_hip_conv2d_q8_nhwc : mace_hip_conv2d_q8_nhwc_host;
     return ToStatus(fn(context->hip(), input->data<uint8_t>(), filter->data<uint8_t>(),
                        bias ? bias->data<int32_t>() : nullptr, input->dim(0), input->dim(1),
@@ -707,7 +823,7 @@ class Conv2dOpQuant {
   Padding padding_type_;
   std::vector<int> paddings_, dilations_;
   int clamp_min_, clamp_max_;
-  WeightRegistration weight_;
+  WeightRegistration weight_, bias_;
 };
 
 // The 1x1 / stride 1 / no padding case under its earlier name.
@@ -794,6 +910,7 @@ class Conv2dOpFloat {
 // [area][cin][tiles], both batched, row-major (:191-204) -- followed by the output transform
 // (A^T m A).  The transforms are host loops written from the standard matrices of the
 // algorithm (the reference has NEON code for the same matrices); the Gemm is the delegator's.
+// Host tensors only: the transforms read and write the tensors' memory directly.
 class Conv2dK3x3WinogradOp {
  public:
   Conv2dK3x3WinogradOp(OpDelegatorRegistry *registry, Padding padding_type = SAME,
@@ -833,23 +950,35 @@ class Conv2dK3x3WinogradOp {
     const index_t th = poh / t, tw = pow_ / t, tiles = th * tw;
     const float *BT = t == 2 ? kBT4 : kBT8, *G = t == 2 ? kG4 : kG8, *AT = t == 2 ? kAT4 : kAT8;
 
-    // filter [cout][cin][3][3] -> U [area][cout][cin] = G g G^T
-    std::vector<float> U((size_t)area * cout * cin), V((size_t)area * cin * tiles),
-        M((size_t)area * cout * tiles), tmp(a * 3), d(area), w(area);
+    // filter [cout][cin][3][3] -> U [area][cout][cin] = G g G^T.  As in the reference, the
+    // transformed filter of a constant filter is computed once and kept (conv_2d_3x3_winograd.cc:
+    // 120-143: redone only when the filter is not a weight or the tile size changes); it is the
+    // constant left-hand side of every Gemm call below, so it also stays on the GPU.
+    std::vector<float> V((size_t)area * cin * tiles), M((size_t)area * cout * tiles), tmp(a * 3), d(area),
+        w(area);
     const float *f = filter->data<float>();
-    for (index_t oc = 0; oc < cout; ++oc)
-      for (index_t ic = 0; ic < cin; ++ic) {
-        const float *g = f + (oc * cin + ic) * 9;
-        for (int i = 0; i < a; ++i)
-          for (int j = 0; j < 3; ++j)
-            tmp[i * 3 + j] = G[i * 3] * g[j] + G[i * 3 + 1] * g[3 + j] + G[i * 3 + 2] * g[6 + j];
-        for (int i = 0; i < a; ++i)
-          for (int j = 0; j < a; ++j)
-            U[((size_t)(i * a + j) * cout + oc) * cin + ic] =
-                tmp[i * 3] * G[j * 3] + tmp[i * 3 + 1] * G[j * 3 + 1] + tmp[i * 3 + 2] * G[j * 3 + 2];
-      }
-    Tensor Ut(U.data(), DT_FLOAT, {area, cout, cin}), Vt(V.data(), DT_FLOAT, {area, cin, tiles}),
-        Mt(M.data(), DT_FLOAT, {area, cout, tiles});
+    const bool keep = filter->is_weight() && t == u_tile_ && f == u_filter_ &&
+                      U_.size() == (size_t)area * cout * cin;
+    if (!keep) {
+      u_resident_.Release();
+      U_.assign((size_t)area * cout * cin, 0.f);
+      for (index_t oc = 0; oc < cout; ++oc)
+        for (index_t ic = 0; ic < cin; ++ic) {
+          const float *g = f + (oc * cin + ic) * 9;
+          for (int i = 0; i < a; ++i)
+            for (int j = 0; j < 3; ++j)
+              tmp[i * 3 + j] = G[i * 3] * g[j] + G[i * 3 + 1] * g[3 + j] + G[i * 3 + 2] * g[6 + j];
+          for (int i = 0; i < a; ++i)
+            for (int j = 0; j < a; ++j)
+              U_[((size_t)(i * a + j) * cout + oc) * cin + ic] =
+                  tmp[i * 3] * G[j * 3] + tmp[i * 3 + 1] * G[j * 3 + 1] + tmp[i * 3 + 2] * G[j * 3 + 2];
+        }
+      u_tile_ = t;
+      u_filter_ = f;
+    }
+    Tensor Ut(U_.data(), DT_FLOAT, {area, cout, cin}, 0.f, 0, /*is_weight=*/filter->is_weight()),
+        Vt(V.data(), DT_FLOAT, {area, cin, tiles}), Mt(M.data(), DT_FLOAT, {area, cout, tiles});
+    u_resident_.Note(context, &Ut, sizeof(float) * U_.size());
     const float *x = input->data<float>();
     float *y = output->mutable_data<float>();
     for (index_t b = 0; b < batch; ++b) {
@@ -926,6 +1055,10 @@ class Conv2dK3x3WinogradOp {
   Padding padding_type_;
   std::vector<int> paddings_;
   std::unique_ptr<delegator::Gemm> gemm_;
+  std::vector<float> U_;              // transformed filter, kept while the filter is a constant
+  int u_tile_ = 0;
+  const float *u_filter_ = nullptr;
+  WeightRegistration u_resident_;
 };
 
 // DynamicLSTMOp<RT_CPU, float>::Run (mace/ops/dynamic_lstm.cc:160-372), a caller of
@@ -1055,6 +1188,7 @@ class QuantizeOp {
   explicit QuantizeOp(bool non_zero = false, bool find_range_every_time = false)
       : non_zero_(non_zero), find_range_every_time_(find_range_every_time) {}
   MaceStatus Run(OpContext *context, const Tensor *input, Tensor *output) {
+    if (!SamePlacement(output, {input})) return MaceStatus::MACE_INVALID_ARGS;
     MaceStatus st = output->Resize(input->shape());   // ResizeLike
     if (st != MaceStatus::MACE_SUCCESS) return st;
     if (!find_range_every_time_ && output->scale() > 0.f) {
@@ -1083,6 +1217,7 @@ template <typename T>
 class DequantizeOp {
  public:
   MaceStatus Run(OpContext *context, const Tensor *input, Tensor *output) {
+    if (!SamePlacement(output, {input})) return MaceStatus::MACE_INVALID_ARGS;
     MaceStatus st = output->Resize(input->shape());
     if (st != MaceStatus::MACE_SUCCESS) return st;
     return ToStatus(Call(context->hip(), input->data<T>(), input->size(), input->scale(),

@@ -13,10 +13,13 @@
 //     tensors their scale and zero point;
 //   * SerialNet::Init / Run (mace/core/net/serial_net.cc:39-124): ops are created once, in the
 //     order of the NetDef, and run one after the other on the caller's thread.
-// The ops it can create are the ones this library computes: Quantize, Dequantize, Conv2D
+// The ops it creates itself are the ones this library computes: Quantize, Dequantize, Conv2D
 // (uint8 NHWC any geometry; float NCHW 1x1), MatMul, FullyConnected, and the shape-only Reshape /
-// Squeeze / Identity.  Any other op type makes Init return MACE_UNSUPPORTED and names the op
-// (a MobileNet also needs DepthwiseConv2d, Pooling and Softmax, which are outside this library).
+// Squeeze / Identity.  Other op types come from the host: RegisterOp(type, creator) adds an op
+// factory, as the reference creates every op through its registry (serial_net.cc:39-91), so a
+// host can supply DepthwiseConv2d, Pooling, Softmax ... (on the CPU, or with kernels of its own)
+// and run a whole MobileNet with this library's ops on the GPU.  An op type nobody provides makes
+// Init return MACE_UNSUPPORTED and names the op.
 // Output tensors get a device buffer each, sized from the op's output_shape and output_type
 // (the reference's memory optimizer, which lets ops share buffers, is not mirrored).
 //
@@ -27,6 +30,7 @@
 #define MACE_HIP_NET_H_
 
 #include <cstring>
+#include <functional>
 #include <map>
 #include <memory>
 #include <string>
@@ -304,6 +308,19 @@ inline std::vector<int> GetIntsArg(const OperatorDef &op, const char *name, std:
 inline size_t SizeOfType(int dt) {
   return dt == DT_FLOAT || dt == DT_INT32 ? 4 : (dt == DT_UINT8 ? 1 : 0);
 }
+// Elements of a shape times `elem` bytes; false for a negative dimension or a product that does
+// not fit (shapes come from a file: nothing about them is trusted).
+inline bool CheckedBytes(const std::vector<int64_t> &dims, size_t elem, int64_t *count, size_t *bytes) {
+  int64_t n = 1;
+  for (int64_t d : dims) {
+    if (d < 0 || __builtin_mul_overflow(n, d, &n)) return false;
+  }
+  int64_t b = 0;
+  if (__builtin_mul_overflow(n, (int64_t)elem, &b) || b > ((int64_t)1 << 46)) return false;
+  *count = n;
+  *bytes = (size_t)b;
+  return true;
+}
 
 // ---- the runner ------------------------------------------------------------------------------------
 class SerialNet {
@@ -320,24 +337,28 @@ class SerialNet {
   }
   const std::string &error() const { return error_; }
 
+  // An op supplied by the host.  The creator is called once per OperatorDef of its type during
+  // Init, after every tensor of the net exists (GetTensor: device tensors, the outputs sized from
+  // the def's output_shape / output_type and carrying its quantize_info), and returns the function
+  // Run() calls in the op's place.  An op that computes on the CPU moves its operands itself
+  // (mace_hip_memcpy_d2h / _h2d, which wait for the stream); such an op cannot be captured into a
+  // graph.  Register before Init; a type registered here takes precedence over a built-in one.
+  typedef std::function<MaceStatus(OpContext *)> OpRun;
+  typedef std::function<MaceStatus(const OperatorDef &, SerialNet *, OpRun *)> OpCreator;
+  void RegisterOp(const std::string &type, OpCreator creator) { custom_ops_[type] = std::move(creator); }
+
   // Workspace::LoadModelTensor + AddQuantizeInfoForOutputTensor + SerialNet::Init
   MaceStatus Init(const NetDef &net, const void *model_data, size_t model_data_size) {
     if (!ops_.empty() || weights_) return Fail(MaceStatus::MACE_INVALID_ARGS, "Init called twice");
-    // weights: one buffer on the device, every ConstTensor a slice of it (workspace.cc:170-205)
-    if (model_data_size > 0) {
-      if (mace_hip_malloc(ctx_, model_data_size, &weights_) != MACE_HIP_SUCCESS ||
-          mace_hip_memcpy_h2d(ctx_, weights_, model_data, model_data_size) != MACE_HIP_SUCCESS)
-        return Fail(MaceStatus::MACE_OUT_OF_RESOURCES, mace_hip_last_error(ctx_));
-    }
+    // Everything the file says is checked before anything is allocated.
+    // weights: every ConstTensor is a slice of ONE buffer (workspace.cc:170-205)
     for (const ConstTensor &c : net.tensors) {
       const size_t es = SizeOfType(c.data_type);
-      int64_t count = 1;
-      for (int64_t d : c.dims) count *= d;
-      if (es == 0 || c.offset < 0 || count != c.data_size ||
-          (uint64_t)c.offset + (uint64_t)count * es > model_data_size)
+      int64_t count = 0;
+      size_t bytes = 0;
+      if (es == 0 || c.offset < 0 || !CheckedBytes(c.dims, es, &count, &bytes) || count != c.data_size ||
+          (uint64_t)c.offset > model_data_size || bytes > model_data_size - (uint64_t)c.offset)
         return Fail(MaceStatus::MACE_INVALID_ARGS, "tensor " + c.name + ": bad type, size or offset");
-      tensors_[c.name] = Tensor((char *)weights_ + c.offset, (DataType)c.data_type, c.dims, c.scale,
-                                c.zero_point, /*is_weight=*/true, /*on_device=*/true);
     }
     // activations: the net's inputs and every op output, a 256-byte aligned slice each
     struct Want { std::string name; std::vector<index_t> shape; int dt; float scale; int32_t zp; size_t off; };
@@ -345,12 +366,12 @@ class SerialNet {
     size_t total = 0;
     auto want = [&](const std::string &name, const std::vector<int64_t> &shape, int dt, float scale,
                     int32_t zp) -> bool {
-      size_t n = SizeOfType(dt);
-      if (n == 0) return false;
-      for (int64_t d : shape) { if (d < 0) return false; n *= (size_t)d; }
+      int64_t count = 0;
+      size_t n = 0;
+      if (SizeOfType(dt) == 0 || !CheckedBytes(shape, SizeOfType(dt), &count, &n)) return false;
       wants.push_back(Want{name, shape, dt, scale, zp, total});
       total += (n + 255) / 256 * 256 + 256;
-      return true;
+      return total < ((size_t)1 << 47);
     };
     for (const InputOutputInfo &i : net.input_info)
       if (!want(i.name, i.dims, i.data_type, i.scale, i.zero_point))
@@ -377,6 +398,15 @@ class SerialNet {
         }
       }
     }
+    // the weights buffer is copied to the GPU once and the slices point into it
+    if (model_data_size > 0) {
+      if (mace_hip_malloc(ctx_, model_data_size, &weights_) != MACE_HIP_SUCCESS ||
+          mace_hip_memcpy_h2d(ctx_, weights_, model_data, model_data_size) != MACE_HIP_SUCCESS)
+        return Fail(MaceStatus::MACE_OUT_OF_RESOURCES, mace_hip_last_error(ctx_));
+    }
+    for (const ConstTensor &c : net.tensors)
+      tensors_[c.name] = Tensor((char *)weights_ + c.offset, (DataType)c.data_type, c.dims, c.scale,
+                                c.zero_point, /*is_weight=*/true, /*on_device=*/true);
     if (total > 0 && mace_hip_malloc(ctx_, total, &activations_) != MACE_HIP_SUCCESS)
       return Fail(MaceStatus::MACE_OUT_OF_RESOURCES, mace_hip_last_error(ctx_));
     for (const Want &w : wants)
@@ -386,9 +416,9 @@ class SerialNet {
       auto it = tensors_.find(v.of);
       if (it == tensors_.end()) return Fail(MaceStatus::MACE_INVALID_ARGS, "no tensor " + v.of);
       Tensor t = it->second;
-      int64_t n = 1;
-      for (int64_t d : v.shape) n *= d;
-      if (n != t.size()) return Fail(MaceStatus::MACE_INVALID_ARGS, v.name + ": a view cannot change the size");
+      int64_t n = 0;
+      size_t unused = 0;
+      if (!CheckedBytes(v.shape, 1, &n, &unused) || n != t.size()) return Fail(MaceStatus::MACE_INVALID_ARGS, v.name + ": a view cannot change the size");
       tensors_[v.name] = Tensor(t.mutable_data<char>(), t.dtype(), v.shape, t.scale(), t.zero_point(),
                                 t.is_weight(), true);
     }
@@ -470,6 +500,21 @@ class SerialNet {
 
   MaceStatus Fail(MaceStatus st, const std::string &why) { error_ = why; return st; }
 
+  // The "activation" / "max_limit" arguments of a float op.  An activation this library does not
+  // apply is refused here, at Init, never dropped.
+  MaceStatus ParseActivation(const OperatorDef &def, ActivationType *act, float *limit) {
+    const Argument *a = FindArg(def, "activation");
+    if (a && a->has_s) {
+      if (!StringToActivationType(a->s, act))
+        return Fail(MaceStatus::MACE_INVALID_ARGS, def.name + ": unknown activation type: " + a->s);
+      if (*act != NOOP && *act != RELU && *act != RELUX)
+        return Fail(MaceStatus::MACE_UNSUPPORTED, def.name + ": activation " + a->s + " is not applied by this library");
+    }
+    const Argument *lim = FindArg(def, "max_limit");
+    *limit = (lim && lim->has_f) ? lim->f : 0.f;
+    return MaceStatus::MACE_SUCCESS;
+  }
+
   MaceStatus CreateOp(const OperatorDef &def, std::unique_ptr<Op> *out) {
     auto in = [&](size_t k) -> Tensor * { return k < def.input.size() ? GetTensor(def.input[k]) : nullptr; };
     auto outt = [&](size_t k) -> Tensor * { return k < def.output.size() ? GetTensor(def.output[k]) : nullptr; };
@@ -477,7 +522,19 @@ class SerialNet {
       if (!GetTensor(n)) return Fail(MaceStatus::MACE_INVALID_ARGS, def.name + ": no tensor " + n);
     const int T = (int)GetIntArg(def, "T", DT_FLOAT);
     const std::string &type = def.type;
+    auto custom = custom_ops_.find(type);
+    if (custom != custom_ops_.end()) {
+      OpRun run;
+      MaceStatus st = custom->second(def, this, &run);
+      if (st != MaceStatus::MACE_SUCCESS) return error_.empty() ? Fail(st, def.name + ": the host's op creator failed") : st;
+      if (!run) return Fail(MaceStatus::MACE_INVALID_ARGS, def.name + ": the host's op creator returned no op");
+      *out = Make(def.name, std::move(run));
+      return MaceStatus::MACE_SUCCESS;
+    }
     if (type == "Reshape" || type == "Squeeze" || type == "Identity") return MaceStatus::MACE_SUCCESS;
+    // every built-in op reads input 0 and writes output 0
+    if (!in(0) || !outt(0))
+      return Fail(MaceStatus::MACE_INVALID_ARGS, def.name + ": " + type + " needs an input and an output");
     if (type == "Quantize") {
       auto op = std::make_shared<ops::QuantizeOp>(GetIntArg(def, "non_zero", 0) != 0,
                                                   GetIntArg(def, "find_range_every_time", 0) != 0);
@@ -506,15 +563,10 @@ class SerialNet {
         *out = Make(def.name, [op, x, f, b, y](OpContext *c) { return op->Run(c, x, f, b, y); });
       } else {
         ActivationType act = NOOP;
-        const Argument *a = FindArg(def, "activation");
-        if (a && a->has_s) {
-          if (a->s == "RELU") act = RELU;
-          else if (a->s == "RELUX") act = RELUX;
-          else if (a->s != "NOOP") return Fail(MaceStatus::MACE_UNSUPPORTED, def.name + ": activation " + a->s);
-        }
-        const Argument *lim = FindArg(def, "max_limit");
-        auto op = std::make_shared<ops::Conv2dOpFloat>(registry_, strides, pad, pads, dil, act,
-                                                       (lim && lim->has_f) ? lim->f : 0.f);
+        float limit = 0.f;
+        MaceStatus ast = ParseActivation(def, &act, &limit);
+        if (ast != MaceStatus::MACE_SUCCESS) return ast;
+        auto op = std::make_shared<ops::Conv2dOpFloat>(registry_, strides, pad, pads, dil, act, limit);
         *out = Make(def.name, [op, x, f, b, y](OpContext *c) { return op->Run(c, x, f, b, y); });
       }
     } else if (type == "MatMul") {
@@ -535,7 +587,12 @@ class SerialNet {
         auto op = std::make_shared<ops::FullyConnectedOp<uint8_t>>(registry_);
         *out = Make(def.name, [op, x, w, b, y](OpContext *c) { return op->Run(c, x, w, b, y); });
       } else {
-        auto op = std::make_shared<ops::FullyConnectedOp<float>>(registry_);
+        // FullyConnectedOpBase reads "activation" / "max_limit" (mace/ops/fully_connected.cc:40-47)
+        ActivationType act = NOOP;
+        float limit = 0.f;
+        MaceStatus ast = ParseActivation(def, &act, &limit);
+        if (ast != MaceStatus::MACE_SUCCESS) return ast;
+        auto op = std::make_shared<ops::FullyConnectedOp<float>>(registry_, act, limit);
         *out = Make(def.name, [op, x, w, b, y](OpContext *c) { return op->Run(c, x, w, b, y); });
       }
     } else {
@@ -554,6 +611,7 @@ class SerialNet {
   std::map<std::string, Tensor> tensors_;
   std::vector<View> views_;
   std::vector<std::unique_ptr<Op>> ops_;
+  std::map<std::string, OpCreator> custom_ops_;
   mace_hip_graph *graph_ = nullptr;
 };
 

@@ -46,6 +46,14 @@ inline void mh_weight_drop_panels(mh_weight *w, bool real_memory, std::vector<vo
   w->panels.clear();
 }
 
+// A constant operand in HOST memory (mace_hip_host_weight_register): its device copy, which the
+// host-pointer entry points use instead of staging the operand on every call.
+struct mh_host_weight {
+  const void *host;
+  size_t bytes;
+  void *dev;
+};
+
 struct mace_hip_ctx {
   int device = 0;
   hipStream_t own_stream = nullptr;
@@ -77,6 +85,12 @@ struct mace_hip_ctx {
   int rq_cache_next = 0;
   std::vector<mh_weight> weights;
   long weight_hits = 0, weight_builds = 0;   // statistics for tests
+  std::vector<mh_host_weight> host_weights;
+  long host_weight_uploads = 0, host_weight_hits = 0;
+  // pinned host memory the host-pointer entry points route small transfers through (a copy
+  // from or to pageable memory is staged by the runtime itself, synchronously and more slowly)
+  char *pinned = nullptr;
+  size_t pinned_bytes = 0, pinned_used = 0;
   // This device's copy of the library's static scratch array (see ctx.hip), and whether the call
   // in progress is one that must not allocate: then the arena is that array, a reservation
   // beyond its size is an error, and the weight cache (which allocates on first use) is bypassed.
@@ -245,17 +259,41 @@ struct ArenaScope {
   ~ArenaScope() { ctx->arena_used = mark; }
 };
 
+constexpr size_t MH_PINNED_BYTES = 4u << 20, MH_PINNED_MAX_TRANSFER = 1u << 20;
 struct Stage {
   mace_hip_ctx *ctx;
   ArenaScope scope;
   explicit Stage(mace_hip_ctx *c) : ctx(c), scope(c) {}
   // returns nullptr for a null/empty host pointer
+  ~Stage() { ctx->pinned_used = 0; }
+  // A slice of the context's pinned staging buffer, or nullptr when the transfer is too large for
+  // it (then the copy goes straight from / to the caller's memory).
+  void *pinned_slice(size_t bytes) {
+    if (!ctx->pinned || bytes > MH_PINNED_MAX_TRANSFER) return nullptr;
+    const size_t at = mh_align_up(ctx->pinned_used, 64);
+    if (at + bytes > ctx->pinned_bytes) return nullptr;
+    ctx->pinned_used = at + bytes;
+    return ctx->pinned + at;
+  }
+  // returns nullptr for a null/empty host pointer
   int in(const void *host, size_t bytes, void **dev) {
     *dev = nullptr;
     if (!host || bytes == 0) return MACE_HIP_SUCCESS;
+    // a registered constant operand is on the device already
+    for (const mh_host_weight &w : ctx->host_weights)
+      if (w.host == host && bytes <= w.bytes) {
+        *dev = w.dev;
+        ++ctx->host_weight_hits;
+        return MACE_HIP_SUCCESS;
+      }
     *dev = mh_arena_take(ctx, bytes);
     if (!*dev) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
-    MH_HIP(ctx, hipMemcpyAsync(*dev, host, bytes, hipMemcpyHostToDevice, ctx->stream));
+    const void *src = host;
+    if (void *p = pinned_slice(bytes)) {
+      memcpy(p, host, bytes);
+      src = p;
+    }
+    MH_HIP(ctx, hipMemcpyAsync(*dev, src, bytes, hipMemcpyHostToDevice, ctx->stream));
     return MACE_HIP_SUCCESS;
   }
   int out(size_t bytes, void **dev) {
@@ -264,8 +302,10 @@ struct Stage {
     return MACE_HIP_SUCCESS;
   }
   int back(void *host, const void *dev, size_t bytes) {
-    if (bytes) MH_HIP(ctx, hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    void *p = bytes ? pinned_slice(bytes) : nullptr;
+    if (bytes) MH_HIP(ctx, hipMemcpyAsync(p ? p : host, dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
     MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (p) memcpy(host, p, bytes);
     return MACE_HIP_SUCCESS;
   }
 };

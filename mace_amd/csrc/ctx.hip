@@ -117,6 +117,17 @@ int mh_fill_bytes(mace_hip_ctx *ctx, void *dst, uint8_t value, size_t bytes) {
                      __func__);                                                                 \
   } while (0)
 
+// Entry points that wait for the stream (or copy from or to host memory) cannot be recorded into
+// a graph; while one is being captured from this context they are refused before they touch the
+// runtime, so the capture itself stays valid.
+#define MH_NOT_CAPTURING(ctx)                                                                  \
+  do {                                                                                         \
+    if ((ctx)->capturing)                                                                      \
+      return mh_fail((ctx), MACE_HIP_INVALID_ARGS,                                             \
+                     "%s waits for the stream: not possible while a graph is being captured", \
+                     __func__);                                                                \
+  } while (0)
+
 static void mh_free_retired(mace_hip_ctx *ctx) {
   for (void *p : ctx->retired) (void)hipFree(p);
   ctx->retired.clear();
@@ -154,6 +165,14 @@ int mace_hip_ctx_create(int device, mace_hip_ctx **out) {
     return MACE_HIP_RUNTIME_ERROR;
   }
   ctx->static_scratch = (char *)sp;
+  // (staging through pinned memory is an optimisation: without the buffer, copies go direct)
+  void *pin = nullptr;
+  if (hipHostMalloc(&pin, MH_PINNED_BYTES, hipHostMallocDefault) == hipSuccess) {
+    ctx->pinned = (char *)pin;
+    ctx->pinned_bytes = MH_PINNED_BYTES;
+  } else {
+    (void)hipGetLastError();
+  }
   ctx->big_lds_kernels.reserve(128);   // so that raising a kernel's LDS limit never reallocates
   ctx->stream = ctx->own_stream;
   ctx->cu_count = prop.multiProcessorCount;
@@ -181,6 +200,8 @@ int mace_hip_ctx_destroy(mace_hip_ctx *ctx) {
   (void)hipStreamSynchronize(ctx->stream);
   if (ctx->arena) (void)hipFree(ctx->arena);
   for (mh_weight &w : ctx->weights) mh_weight_drop_panels(&w, true, nullptr);
+  for (mh_host_weight &w : ctx->host_weights) (void)hipFree(w.dev);
+  if (ctx->pinned) (void)hipHostFree(ctx->pinned);
   mh_free_retired(ctx);
   (void)hipEventDestroy(ctx->ev_start);
   (void)hipEventDestroy(ctx->ev_stop);
@@ -206,6 +227,7 @@ int mace_hip_weight_register(mace_hip_ctx *ctx, const void *device_ptr, size_t b
 
 int mace_hip_weight_unregister(mace_hip_ctx *ctx, const void *device_ptr) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_NOT_CAPTURING(ctx);
   for (size_t i = 0; i < ctx->weights.size(); ++i)
     if (ctx->weights[i].ptr == device_ptr) {
       // kernels may still read the panels; so may a captured graph, until it is destroyed
@@ -218,6 +240,60 @@ int mace_hip_weight_unregister(mace_hip_ctx *ctx, const void *device_ptr) {
   return mh_fail(ctx, MACE_HIP_INVALID_ARGS, "weight %p is not registered", device_ptr);
 }
 
+int mace_hip_host_weight_register(mace_hip_ctx *ctx, const void *host_ptr, size_t bytes) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
+  MH_CHECK(ctx, host_ptr && bytes > 0, "null or empty weight");
+  MH_CHECK(ctx, !ctx->capturing, "a capture is in progress on this context");
+  mh_host_weight *w = nullptr;
+  for (mh_host_weight &e : ctx->host_weights)
+    if (e.host == host_ptr) w = &e;
+  if (w && w->bytes != bytes) {   // same address, another size: start over
+    MH_RETURN_IF_ERROR(mace_hip_host_weight_unregister(ctx, host_ptr));
+    w = nullptr;
+  }
+  if (!w) {
+    void *dev = nullptr;
+    const hipError_t e = hipMalloc(&dev, bytes);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      return mh_fail(ctx, MACE_HIP_OUT_OF_RESOURCES, "hipMalloc(%zu) failed: %s", bytes,
+                     hipGetErrorString(e));
+    }
+    ctx->host_weights.push_back(mh_host_weight{host_ptr, bytes, dev});
+    w = &ctx->host_weights.back();
+  }
+  // (registered again: the caller has changed the weight; the copy and whatever the uint8 GEMM
+  // derived from it are refreshed)
+  MH_HIP(ctx, hipMemcpyAsync(w->dev, host_ptr, bytes, hipMemcpyHostToDevice, ctx->stream));
+  MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  ++ctx->host_weight_uploads;
+  return mace_hip_weight_register(ctx, w->dev, bytes);
+}
+
+int mace_hip_host_weight_unregister(mace_hip_ctx *ctx, const void *host_ptr) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  MH_NEEDS_GPU(ctx);
+  MH_NOT_CAPTURING(ctx);
+  for (size_t i = 0; i < ctx->host_weights.size(); ++i)
+    if (ctx->host_weights[i].host == host_ptr) {
+      void *dev = ctx->host_weights[i].dev;
+      (void)mace_hip_weight_unregister(ctx, dev);   // synchronizes the stream
+      if (ctx->live_graphs > 0) ctx->retired.push_back(dev);
+      else (void)hipFree(dev);
+      ctx->host_weights.erase(ctx->host_weights.begin() + (long)i);
+      return MACE_HIP_SUCCESS;
+    }
+  return mh_fail(ctx, MACE_HIP_INVALID_ARGS, "host weight %p is not registered", host_ptr);
+}
+
+int mace_hip_host_weight_stats(mace_hip_ctx *ctx, int64_t *uploads, int64_t *hits) {
+  if (!ctx) return MACE_HIP_INVALID_ARGS;
+  if (uploads) *uploads = ctx->host_weight_uploads;
+  if (hits) *hits = ctx->host_weight_hits;
+  return MACE_HIP_SUCCESS;
+}
+
 int mace_hip_weight_cache_stats(mace_hip_ctx *ctx, int64_t *builds, int64_t *hits) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   if (builds) *builds = ctx->weight_builds;
@@ -228,6 +304,7 @@ int mace_hip_weight_cache_stats(mace_hip_ctx *ctx, int64_t *builds, int64_t *hit
 int mace_hip_ctx_set_stream(mace_hip_ctx *ctx, void *hip_stream) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   MH_NEEDS_GPU(ctx);
+  MH_NOT_CAPTURING(ctx);
   MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
   ctx->stream = hip_stream ? (hipStream_t)hip_stream : ctx->own_stream;
   return MACE_HIP_SUCCESS;
@@ -236,6 +313,7 @@ int mace_hip_ctx_set_stream(mace_hip_ctx *ctx, void *hip_stream) {
 int mace_hip_sync(mace_hip_ctx *ctx) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   MH_NEEDS_GPU(ctx);
+  MH_NOT_CAPTURING(ctx);
   MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
   return MACE_HIP_SUCCESS;
 }
@@ -261,6 +339,7 @@ int mace_hip_timer_start(mace_hip_ctx *ctx) {
 int mace_hip_timer_stop(mace_hip_ctx *ctx, float *elapsed_ms) {
   if (!ctx || !elapsed_ms) return MACE_HIP_INVALID_ARGS;
   MH_NEEDS_GPU(ctx);
+  MH_NOT_CAPTURING(ctx);
   MH_HIP(ctx, hipEventRecord(ctx->ev_stop, ctx->stream));
   MH_HIP(ctx, hipEventSynchronize(ctx->ev_stop));
   MH_HIP(ctx, hipEventElapsedTime(elapsed_ms, ctx->ev_start, ctx->ev_stop));
@@ -394,6 +473,7 @@ int mace_hip_malloc(mace_hip_ctx *ctx, size_t bytes, void **dev_ptr) {
 int mace_hip_free(mace_hip_ctx *ctx, void *dev_ptr) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   MH_NEEDS_GPU(ctx);
+  MH_NOT_CAPTURING(ctx);
   if (!dev_ptr) return MACE_HIP_SUCCESS;
   MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
   MH_HIP(ctx, hipFree(dev_ptr));
@@ -403,6 +483,7 @@ int mace_hip_free(mace_hip_ctx *ctx, void *dev_ptr) {
 int mace_hip_memcpy_h2d(mace_hip_ctx *ctx, void *dst, const void *src, size_t bytes) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   MH_NEEDS_GPU(ctx);
+  MH_NOT_CAPTURING(ctx);
   if (bytes == 0) return MACE_HIP_SUCCESS;
   MH_HIP(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
   MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
@@ -412,6 +493,7 @@ int mace_hip_memcpy_h2d(mace_hip_ctx *ctx, void *dst, const void *src, size_t by
 int mace_hip_memcpy_d2h(mace_hip_ctx *ctx, void *dst, const void *src, size_t bytes) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   MH_NEEDS_GPU(ctx);
+  MH_NOT_CAPTURING(ctx);
   if (bytes == 0) return MACE_HIP_SUCCESS;
   MH_HIP(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
   MH_HIP(ctx, hipStreamSynchronize(ctx->stream));
@@ -505,6 +587,7 @@ int mace_hip_gemm_f32_host(mace_hip_ctx *ctx, const float *lhs, const float *rhs
                            int rhs_batched, float *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   MH_NEEDS_GPU(ctx);
+  MH_NOT_CAPTURING(ctx);
   MH_CHECK(ctx, nonneg(batch, rows, cols, depth), "negative dimension");
   const size_t lb = sizeof(float) * (lhs_batched ? batch : 1) * rows * depth;
   const size_t rb = sizeof(float) * (rhs_batched ? batch : 1) * depth * cols;
@@ -534,6 +617,7 @@ int mace_hip_gemv_f32_act_host(mace_hip_ctx *ctx, const float *lhs, const float 
                                float *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   MH_NEEDS_GPU(ctx);
+  MH_NOT_CAPTURING(ctx);
   MH_CHECK(ctx, nonneg(batch, height, width, 0), "negative dimension");
   const size_t lb = sizeof(float) * (lhs_batched ? batch : 1) * height * width;
   const size_t rb = sizeof(float) * (rhs_batched ? batch : 1) * width;
@@ -558,6 +642,7 @@ int mace_hip_conv1x1_f32_nchw_host(mace_hip_ctx *ctx, const float *input,
                                    float max_limit, float *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   MH_NEEDS_GPU(ctx);
+  MH_NOT_CAPTURING(ctx);
   MH_CHECK(ctx, nonneg(n, cin, hw, cout), "negative dimension");
   const size_t ib = sizeof(float) * n * cin * hw;
   const size_t fb = sizeof(float) * cout * cin;
@@ -582,6 +667,7 @@ int mace_hip_matmul_f32_host(mace_hip_ctx *ctx, const float *lhs, const float *r
                              int transpose_rhs, int lhs_batched, int rhs_batched, float *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   MH_NEEDS_GPU(ctx);
+  MH_NOT_CAPTURING(ctx);
   MH_CHECK(ctx, nonneg(batch, lhs_rows, lhs_cols, 0) && nonneg(rhs_rows, rhs_cols, 0, 0),
            "negative dimension");
   const int64_t rows = transpose_lhs ? lhs_cols : lhs_rows;
@@ -612,6 +698,7 @@ int mace_hip_conv2d_f32_nchw_host(mace_hip_ctx *ctx, const float *input, const f
                                   float *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   MH_NEEDS_GPU(ctx);
+  MH_NOT_CAPTURING(ctx);
   MH_CHECK(ctx, nonneg(n, cin, in_h, in_w) && nonneg(cout, k_h, k_w, 0) && pad_h >= 0 && pad_w >= 0,
            "negative dimension");
   if (k_h != 1 || k_w != 1 || stride_h != 1 || stride_w != 1 || dilation_h != 1 || dilation_w != 1)
@@ -644,6 +731,7 @@ int mace_hip_gemv_q8_u8_host(mace_hip_ctx *ctx, const uint8_t *lhs, const uint8_
                              uint8_t *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   MH_NEEDS_GPU(ctx);
+  MH_NOT_CAPTURING(ctx);
   MH_CHECK(ctx, nonneg(batch, height, width, 0), "negative dimension");
   const size_t lb = (size_t)(lhs_batched ? batch : 1) * height * width;
   const size_t rb = (size_t)(rhs_batched ? batch : 1) * width;
@@ -670,6 +758,7 @@ int mace_hip_gemv_q8_i32_host(mace_hip_ctx *ctx, const uint8_t *lhs, const uint8
                               int32_t lhs_zp, int32_t rhs_zp, int32_t *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   MH_NEEDS_GPU(ctx);
+  MH_NOT_CAPTURING(ctx);
   MH_CHECK(ctx, nonneg(batch, height, width, 0), "negative dimension");
   const size_t lb = (size_t)(lhs_batched ? batch : 1) * height * width;
   const size_t rb = (size_t)(rhs_batched ? batch : 1) * width;
@@ -696,6 +785,7 @@ int mace_hip_gemm_q8_i32_host(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_ord
                               int32_t lhs_offset, int32_t rhs_offset) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   MH_NEEDS_GPU(ctx);
+  MH_NOT_CAPTURING(ctx);
   MH_CHECK(ctx, nonneg(batch, rows, depth, cols), "negative dimension");
   const size_t lb = (size_t)(lhs_batched ? batch : 1) * rows * depth;
   const size_t rb = (size_t)(rhs_batched ? batch : 1) * depth * cols;
@@ -723,6 +813,7 @@ int mace_hip_gemm_q8_u8_host(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_orde
                              int clamp_max) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   MH_NEEDS_GPU(ctx);
+  MH_NOT_CAPTURING(ctx);
   MH_CHECK(ctx, nonneg(batch, rows, depth, cols), "negative dimension");
   const size_t lb = (size_t)(lhs_batched ? batch : 1) * rows * depth;
   const size_t rb = (size_t)(rhs_batched ? batch : 1) * depth * cols;
@@ -783,6 +874,7 @@ int mace_hip_conv1x1_q8_nhwc_host(mace_hip_ctx *ctx, const uint8_t *input,
                                   uint8_t *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   MH_NEEDS_GPU(ctx);
+  MH_NOT_CAPTURING(ctx);
   MH_CHECK(ctx, nonneg(n, h, w, 0) && nonneg(cin, cout, 0, 0), "negative dimension");
   const int64_t pix = n * h * w;
   const size_t ib = (size_t)pix * cin, fb = (size_t)cout * cin;
@@ -812,6 +904,7 @@ int mace_hip_conv2d_q8_nhwc_host(mace_hip_ctx *ctx, const uint8_t *input, const 
                                  int32_t out_zp, int clamp_min, int clamp_max, uint8_t *out) {
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   MH_NEEDS_GPU(ctx);
+  MH_NOT_CAPTURING(ctx);
   MH_CHECK(ctx, nonneg(n, in_h, in_w, 0) && nonneg(cin, cout, 0, 0), "negative dimension");
   MH_CHECK(ctx, k_h >= 1 && k_w >= 1 && stride_h >= 1 && stride_w >= 1 && pad_h >= 0 &&
                     pad_w >= 0, "filter / stride < 1 or negative padding");

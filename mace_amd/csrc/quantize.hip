@@ -228,6 +228,9 @@ int mace_hip_find_min_max_f32(mace_hip_ctx *ctx, const float *input, int64_t siz
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   if (ctx->plan_only)
     return mh_fail(ctx, MACE_HIP_UNSUPPORTED, "%s needs a GPU: this is a plan-only context", __func__);
+  if (ctx->capturing)
+    return mh_fail(ctx, MACE_HIP_INVALID_ARGS,
+                   "%s waits for the stream: not possible while a graph is being captured", __func__);
   PlanScope plan_scope(ctx);
   MH_CHECK(ctx, size > 0 && input && min_val && max_val, "empty or null tensor");
   MH_CHECK(ctx, size < (1ll << 40), "tensor too large");
@@ -263,6 +266,9 @@ int mace_hip_quantize_tensor_dynamic_u8(mace_hip_ctx *ctx, const float *input, i
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   if (ctx->plan_only)
     return mh_fail(ctx, MACE_HIP_UNSUPPORTED, "%s needs a GPU: this is a plan-only context", __func__);
+  if (ctx->capturing)
+    return mh_fail(ctx, MACE_HIP_INVALID_ARGS,
+                   "%s waits for the stream: not possible while a graph is being captured", __func__);
   PlanScope plan_scope(ctx);
   MH_CHECK(ctx, scale && zero_point, "null result pointer");
   float mn, mx;
@@ -316,6 +322,9 @@ int mace_hip_quantize_tensor_u8_host(mace_hip_ctx *ctx, const float *input, int6
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   if (ctx->plan_only)
     return mh_fail(ctx, MACE_HIP_UNSUPPORTED, "%s needs a GPU: this is a plan-only context", __func__);
+  if (ctx->capturing)
+    return mh_fail(ctx, MACE_HIP_INVALID_ARGS,
+                   "%s waits for the stream: not possible while a graph is being captured", __func__);
   PlanScope plan_scope(ctx);
   MH_RETURN_IF_ERROR(check_size(ctx, size, input, out));
   if (size == 0) return MACE_HIP_SUCCESS;
@@ -335,6 +344,9 @@ int mace_hip_quantize_tensor_dynamic_u8_host(mace_hip_ctx *ctx, const float *inp
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   if (ctx->plan_only)
     return mh_fail(ctx, MACE_HIP_UNSUPPORTED, "%s needs a GPU: this is a plan-only context", __func__);
+  if (ctx->capturing)
+    return mh_fail(ctx, MACE_HIP_INVALID_ARGS,
+                   "%s waits for the stream: not possible while a graph is being captured", __func__);
   PlanScope plan_scope(ctx);
   MH_CHECK(ctx, size > 0 && input && out && scale && zero_point, "empty or null tensor");
   MH_CHECK(ctx, size < (1ll << 40), "tensor too large");
@@ -353,6 +365,9 @@ int mace_hip_dequantize_tensor_u8_host(mace_hip_ctx *ctx, const uint8_t *input, 
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   if (ctx->plan_only)
     return mh_fail(ctx, MACE_HIP_UNSUPPORTED, "%s needs a GPU: this is a plan-only context", __func__);
+  if (ctx->capturing)
+    return mh_fail(ctx, MACE_HIP_INVALID_ARGS,
+                   "%s waits for the stream: not possible while a graph is being captured", __func__);
   PlanScope plan_scope(ctx);
   MH_RETURN_IF_ERROR(check_size(ctx, size, input, out));
   if (size == 0) return MACE_HIP_SUCCESS;
@@ -371,6 +386,9 @@ int mace_hip_dequantize_tensor_i32_host(mace_hip_ctx *ctx, const int32_t *input,
   if (!ctx) return MACE_HIP_INVALID_ARGS;
   if (ctx->plan_only)
     return mh_fail(ctx, MACE_HIP_UNSUPPORTED, "%s needs a GPU: this is a plan-only context", __func__);
+  if (ctx->capturing)
+    return mh_fail(ctx, MACE_HIP_INVALID_ARGS,
+                   "%s waits for the stream: not possible while a graph is being captured", __func__);
   PlanScope plan_scope(ctx);
   MH_RETURN_IF_ERROR(check_size(ctx, size, input, out));
   if (size == 0) return MACE_HIP_SUCCESS;

@@ -71,6 +71,9 @@ SIGNATURES = {
     "mace_hip_memcpy_d2h": (_int, [_p, _p, _p, C.c_size_t]),
     "mace_hip_weight_register": (_int, [_p, _p, C.c_size_t]),
     "mace_hip_weight_unregister": (_int, [_p, _p]),
+    "mace_hip_host_weight_register": (_int, [_p, _p, C.c_size_t]),
+    "mace_hip_host_weight_unregister": (_int, [_p, _p]),
+    "mace_hip_host_weight_stats": (_int, [_p, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
     "mace_hip_weight_cache_stats": (_int, [_p, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
     "mace_hip_quantize_multiplier": (None, [C.c_double, C.POINTER(_i32), C.POINTER(_int)]),
     "mace_hip_get_output_multiplier_and_shift": (_int, [_f32, _f32, _f32, C.POINTER(_i32),

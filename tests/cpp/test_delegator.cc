@@ -27,6 +27,85 @@ struct DummyGemv : public delegator::Gemv {
                      Tensor *) override { return MaceStatus::MACE_UNSUPPORTED; }
 };
 
+// Every operand of a call has to live where the output does: a device output with a host weight
+// or bias (or the other way round) is refused before anything reaches the library -- the context
+// here is null, so any call that got through would fail differently.
+static void test_placement(OpDelegatorRegistry *reg) {
+  OpContext context(nullptr);
+  const MaceStatus bad = MaceStatus::MACE_INVALID_ARGS;
+  float f[64] = {0};
+  uint8_t q[64] = {0};
+  int32_t i32[8] = {0};
+  auto T = [&](void *p, DataType dt, std::vector<index_t> shape, bool dev, bool weight = false) {
+    return Tensor(p, dt, std::move(shape), 0.5f, 3, weight, dev);
+  };
+  for (int mix = 0; mix < 3; ++mix) {     // which operand sits on the other side
+    const bool out_dev = mix != 2;
+    Tensor out_f = T(f, DT_FLOAT, {}, out_dev), out_q = T(q, DT_UINT8, {}, out_dev),
+           out_i = T(i32, DT_INT32, {}, out_dev);
+    Tensor lhs_f = T(f, DT_FLOAT, {4, 4}, mix == 0 ? !out_dev : out_dev, true);
+    Tensor rhs_f = T(f, DT_FLOAT, {4, 4}, mix == 1 ? !out_dev : out_dev);
+    Tensor bias_f = T(f, DT_FLOAT, {4}, mix == 2 ? !out_dev : out_dev, true);
+    hip::Gemm<float> gemm((delegator::GemmParam(true)));
+    if (mix < 2) {
+      EXPECT(gemm.Compute(&context, &lhs_f, &rhs_f, 1, 4, 4, 4, RowMajor, RowMajor, RowMajor, true, true,
+                          &out_f) == bad);
+      EXPECT(gemm.Compute(&context, &lhs_f, &rhs_f, 1, 4, 4, 4, 4, false, false, false, true, true,
+                          &out_f) == bad);
+    }
+    hip::Gemv<float> gemv((DelegatorParam()));
+    EXPECT(gemv.Compute(&context, &lhs_f, &rhs_f, &bias_f, 1, 4, 4, false, true, &out_f) == bad);
+    Tensor lhs_q = T(q, DT_UINT8, {4, 4}, mix == 0 ? !out_dev : out_dev, true);
+    Tensor rhs_q = T(q, DT_UINT8, {1, 4}, mix == 1 ? !out_dev : out_dev);
+    Tensor bias_i = T(i32, DT_INT32, {4}, mix == 2 ? !out_dev : out_dev, true);
+    hip::Gemv<uint8_t> gemv_q((DelegatorParam()));
+    hip::Gemv<int32_t> gemv_i((DelegatorParam()));
+    EXPECT(gemv_q.Compute(&context, &lhs_q, &rhs_q, &bias_i, 1, 4, 4, false, true, &out_q) == bad);
+    EXPECT(gemv_i.Compute(&context, &lhs_q, &rhs_q, &bias_i, 1, 4, 4, false, true, &out_i) == bad);
+    // ops
+    Tensor in4 = T(f, DT_FLOAT, {1, 4, 1, 1}, rhs_f.on_device());
+    Tensor w4 = T(f, DT_FLOAT, {4, 4, 1, 1}, lhs_f.on_device(), true);
+    ops::FullyConnectedOp<float> fc(reg, RELU);
+    EXPECT(fc.Run(&context, &in4, &w4, &bias_f, &out_f) == bad);
+    Tensor in4q = T(q, DT_UINT8, {1, 4, 1, 1}, rhs_q.on_device());
+    Tensor w4q = T(q, DT_UINT8, {4, 4, 1, 1}, lhs_q.on_device(), true);
+    ops::FullyConnectedOp<uint8_t> fcq(reg);
+    EXPECT(fcq.Run(&context, &in4q, &w4q, &bias_i, &out_q) == bad);
+    ops::Conv2dOpFloat conv(reg, {1, 1}, VALID);
+    Tensor img = T(f, DT_FLOAT, {1, 4, 2, 2}, rhs_f.on_device());
+    EXPECT(conv.Run(&context, &img, &w4, &bias_f, &out_f) == bad);
+    ops::Conv2dOpQuant convq({1, 1}, VALID);
+    Tensor imgq = T(q, DT_UINT8, {1, 2, 2, 4}, rhs_q.on_device());
+    Tensor filtq = T(q, DT_UINT8, {4, 1, 1, 4}, lhs_q.on_device(), true);
+    EXPECT(convq.Run(&context, &imgq, &filtq, &bias_i, &out_q) == bad);
+    if (mix < 2) {
+      ops::MatMulOpQuant mm(false, false, DT_UINT8), mm32(false, false, DT_INT32);
+      Tensor bq = T(q, DT_UINT8, {4, 4}, rhs_q.on_device());
+      EXPECT(mm.Run(&context, &lhs_q, &bq, &out_q) == bad);
+      EXPECT(mm32.Run(&context, &lhs_q, &bq, &out_i) == bad);
+      ops::MatMulOpFloat mmf(reg, false, false);
+      Tensor bias_ok = T(f, DT_FLOAT, {4}, out_dev);
+      EXPECT(mmf.Run(&context, &lhs_f, &rhs_f, &bias_ok, &out_f) == bad);
+      EXPECT(mmf.Run(&context, &lhs_f, &rhs_f, nullptr, &out_f) == bad);
+      ops::QuantizeOp qop;
+      Tensor qout = T(q, DT_UINT8, {}, out_dev), qin = T(f, DT_FLOAT, {16}, !out_dev);
+      EXPECT(qop.Run(&context, &qin, &qout) == bad);
+      ops::DequantizeOp<uint8_t> dq;
+      Tensor dqin = T(q, DT_UINT8, {16}, !out_dev);
+      EXPECT(dq.Run(&context, &dqin, &out_f) == bad);
+    }
+  }
+  // the float FullyConnected names an activation it does not apply instead of dropping it
+  float w[16] = {0}, x[4] = {0}, y[4];
+  Tensor W(w, DT_FLOAT, {4, 4, 1, 1}), X(x, DT_FLOAT, {1, 4, 1, 1}), Y(y, DT_FLOAT, {});
+  ops::FullyConnectedOp<float> tanh_fc(reg, TANH);
+  EXPECT(tanh_fc.Run(&context, &X, &W, nullptr, &Y) == MaceStatus::MACE_UNSUPPORTED);
+  ActivationType t = NOOP;
+  EXPECT(StringToActivationType("RELUX", &t) && t == RELUX);
+  EXPECT(StringToActivationType("HARDSIGMOID", &t) && t == HARDSIGMOID);
+  EXPECT(!StringToActivationType("relu", &t));
+}
+
 static int test_registry() {
   OpDelegatorRegistry reg;
   // key string: name_dtype_runtime_impl_tag (op_delegator_registry.cc:39-44)
@@ -71,6 +150,7 @@ static int test_registry() {
   Tensor b5(nullptr, DT_FLOAT, {6, 4});
   EXPECT(ops::MatMulInferShape(&a2, &b5, false, true, &s) == MaceStatus::MACE_SUCCESS);
   EXPECT(s.rows == 3 && s.cols == 6 && s.depth == 4 && s.batch == 1);
+  test_placement(&reg);
   return g_fail;
 }
 
@@ -140,6 +220,156 @@ static int test_compute() {
     EXPECT(near(y, {387, 3853}));
     Tensor Wbad(w.data(), DT_FLOAT, {2, 1, 5, 2});
     EXPECT(fc.Run(&context, &X, &Wbad, &Bi, &Y) == MaceStatus::MACE_INVALID_ARGS);
+  }
+  {  // float FullyConnected with its activation (fully_connected.cc:62-75,121): NOOP / RELU / RELUX
+     // against the oracle's Gemv followed by the oracle's activation, host and device tensors,
+     // batch 1 (one vector per pass) and batch 5 (shared weights, four vectors per pass), a width
+     // that is not a multiple of 4 (the general kernel)
+    std::mt19937 rng(99);
+    std::normal_distribution<float> nd(0.f, 1.f);
+    mace_hip_ctx *hc = context.hip();
+    for (index_t in_size : {256, 203}) {
+      for (index_t batch : {1, 5}) {
+        const index_t out_size = 77;
+        std::vector<float> x(batch * in_size), w(out_size * in_size), bias(out_size);
+        for (auto &v : x) v = nd(rng);
+        for (auto &v : w) v = nd(rng);
+        for (auto &v : bias) v = nd(rng);
+        for (int act = 0; act < 3; ++act) {
+          const float limit = 1.5f;
+          std::vector<float> want(batch * out_size), y(want.size(), -99.f);
+          orc_gemv_f32(w.data(), x.data(), bias.data(), batch, out_size, in_size, 0, 1, want.data(), 1);
+          orc_activation_f32(want.data(), (int64_t)want.size(), act, limit);
+          Tensor X(x.data(), DT_FLOAT, {batch, in_size, 1, 1}), W(w.data(), DT_FLOAT, {out_size, in_size, 1, 1}, 0, 0, true),
+              Bi(bias.data(), DT_FLOAT, {out_size}, 0, 0, true), Y(y.data(), DT_FLOAT, {});
+          ops::FullyConnectedOp<float> fc(&reg, (ActivationType)act, limit);
+          EXPECT(fc.Run(&context, &X, &W, &Bi, &Y) == MaceStatus::MACE_SUCCESS);
+          EXPECT(Y.shape() == (std::vector<index_t>{batch, out_size, 1, 1}));
+          EXPECT(close_enough(y, want));
+          if (act == 1) { float lo = 0.f; for (float v : y) lo = std::min(lo, v); EXPECT(lo == 0.f); }
+          if (act == 2) { float hi = 0.f; for (float v : y) hi = std::max(hi, v); EXPECT(hi == limit); }
+          // device tensors
+          void *dx = nullptr, *dw = nullptr, *db = nullptr, *dy = nullptr;
+          mace_hip_malloc(hc, x.size() * 4, &dx); mace_hip_malloc(hc, w.size() * 4, &dw);
+          mace_hip_malloc(hc, bias.size() * 4, &db); mace_hip_malloc(hc, y.size() * 4, &dy);
+          mace_hip_memcpy_h2d(hc, dx, x.data(), x.size() * 4);
+          mace_hip_memcpy_h2d(hc, dw, w.data(), w.size() * 4);
+          mace_hip_memcpy_h2d(hc, db, bias.data(), bias.size() * 4);
+          Tensor dX(dx, DT_FLOAT, {batch, in_size, 1, 1}, 0, 0, false, true), dW(dw, DT_FLOAT, {out_size, in_size, 1, 1}, 0, 0, true, true),
+              dB(db, DT_FLOAT, {out_size}, 0, 0, true, true), dY(dy, DT_FLOAT, {}, 0, 0, false, true);
+          {
+            ops::FullyConnectedOp<float> dfc(&reg, (ActivationType)act, limit);
+            EXPECT(dfc.Run(&context, &dX, &dW, &dB, &dY) == MaceStatus::MACE_SUCCESS);
+            std::vector<float> got(y.size());
+            mace_hip_memcpy_d2h(hc, got.data(), dy, got.size() * 4);
+            EXPECT(close_enough(got, want));
+          }
+          mace_hip_free(hc, dx); mace_hip_free(hc, dw); mace_hip_free(hc, db); mace_hip_free(hc, dy);
+        }
+      }
+    }
+    // the C entry point names an activation it does not apply
+    float one = 1.f, out1 = 0.f;
+    EXPECT(mace_hip_gemv_f32_act_host(hc, &one, &one, nullptr, 1, 1, 1, 0, 1, 4 /* TANH */, 0.f, &out1) ==
+           MACE_HIP_UNSUPPORTED);
+  }
+  {  // Constant operands in host memory stay on the GPU between calls (the counterpart of the
+     // reference's pack cache, gemm.h:28-33, arm/base/gemm.cc:560-576): a uint8 FullyConnected on
+     // host tensors uploads its weight matrix and bias once per op instance, later Run() calls move
+     // the input and the output only; results stay bit-exact.  A weight changed in place is stale
+     // until it is registered again; the registration ends with the op.
+    std::mt19937 rng(123);
+    mace_hip_ctx *hc = context.hip();
+    const index_t out_size = 200, in_size = 1024, batch = 3;
+    std::vector<uint8_t> w(out_size * in_size), x(batch * in_size), y(batch * out_size), want(y.size());
+    std::vector<int32_t> bias(out_size);
+    for (auto &v : w) v = rng() & 255;
+    for (auto &v : bias) v = (int32_t)(rng() % 65536) - 32768;
+    Tensor W(w.data(), DT_UINT8, {out_size, in_size, 1, 1}, 0.01f, 127, true), Bi(bias.data(), DT_INT32, {out_size}, 0.0002f, 0, true),
+        Y(y.data(), DT_UINT8, {}, 1.0f, 128);
+    int64_t up0 = 0, hit0 = 0, up1 = 0, hit1 = 0;
+    EXPECT(mace_hip_host_weight_stats(hc, &up0, &hit0) == MACE_HIP_SUCCESS);
+    {
+      ops::FullyConnectedOp<uint8_t> fc(&reg);
+      for (int round = 0; round < 4; ++round) {
+        for (auto &v : x) v = rng() & 255;
+        Tensor X(x.data(), DT_UINT8, {batch, in_size, 1, 1}, 0.02f, 128);
+        EXPECT(fc.Run(&context, &X, &W, &Bi, &Y) == MaceStatus::MACE_SUCCESS);
+        orc_q8_gemv_u8(w.data(), x.data(), bias.data(), batch, out_size, in_size, 0, 1, 127, 128, 0.01f, 0.02f,
+                       1.0f, 128, ORC_REQUANT_NEON, want.data(), 2);
+        EXPECT(y == want);
+      }
+      EXPECT(mace_hip_host_weight_stats(hc, &up1, &hit1) == MACE_HIP_SUCCESS);
+      EXPECT(up1 - up0 == 2);            // the weight matrix and the bias, once each
+      EXPECT(hit1 - hit0 == 8);          // ... and found resident by every one of the four calls
+      // a weight changed in place: the resident copy is what the calls keep using ...
+      std::vector<uint8_t> stale = want;
+      for (auto &v : w) v = rng() & 255;
+      Tensor X(x.data(), DT_UINT8, {batch, in_size, 1, 1}, 0.02f, 128);
+      EXPECT(fc.Run(&context, &X, &W, &Bi, &Y) == MaceStatus::MACE_SUCCESS);
+      EXPECT(y == stale);
+      // ... until it is registered again
+      EXPECT(mace_hip_host_weight_register(hc, w.data(), w.size()) == MACE_HIP_SUCCESS);
+      EXPECT(fc.Run(&context, &X, &W, &Bi, &Y) == MaceStatus::MACE_SUCCESS);
+      orc_q8_gemv_u8(w.data(), x.data(), bias.data(), batch, out_size, in_size, 0, 1, 127, 128, 0.01f, 0.02f,
+                     1.0f, 128, ORC_REQUANT_NEON, want.data(), 2);
+      EXPECT(y == want && y != stale);
+    }
+    // the op is gone: so are its registrations (unregistering again is an error), and the same
+    // address now holds other values that a fresh op must see
+    EXPECT(mace_hip_host_weight_unregister(hc, w.data()) == MACE_HIP_INVALID_ARGS);
+    for (auto &v : w) v = rng() & 255;
+    ops::FullyConnectedOp<uint8_t> fresh(&reg);
+    Tensor X(x.data(), DT_UINT8, {batch, in_size, 1, 1}, 0.02f, 128);
+    EXPECT(fresh.Run(&context, &X, &W, &Bi, &Y) == MaceStatus::MACE_SUCCESS);
+    orc_q8_gemv_u8(w.data(), x.data(), bias.data(), batch, out_size, in_size, 0, 1, 127, 128, 0.01f, 0.02f,
+                   1.0f, 128, ORC_REQUANT_NEON, want.data(), 2);
+    EXPECT(y == want);
+    // a uint8 MatMul with a constant host right-hand matrix: uploaded once, repacked once
+    const index_t rows = 300, depth = 512, cols = 260;
+    std::vector<uint8_t> a(rows * depth), b(depth * cols), c(rows * cols), cw(c.size());
+    for (auto &v : b) v = rng() & 255;
+    Tensor B(b.data(), DT_UINT8, {depth, cols}, 0.015f, 120, true), Cc(c.data(), DT_UINT8, {}, 40.f, 128);
+    int32_t mult; int shift;
+    EXPECT(orc_get_output_multiplier_and_shift(0.02f, 0.015f, 40.f, &mult, &shift) == 0);
+    int64_t builds0 = 0, builds1 = 0, h0 = 0, h1 = 0;
+    EXPECT(mace_hip_ctx_set_kernel_mask(hc, 1 | 2 | 4) == MACE_HIP_SUCCESS);   // the path that repacks
+    EXPECT(mace_hip_weight_cache_stats(hc, &builds0, &h0) == MACE_HIP_SUCCESS);
+    {
+      ops::MatMulOpQuant mm(false, false, DT_UINT8);
+      for (int round = 0; round < 3; ++round) {
+        for (auto &v : a) v = rng() & 255;
+        Tensor A(a.data(), DT_UINT8, {rows, depth}, 0.02f, 131);
+        EXPECT(mm.Run(&context, &A, &B, &Cc) == MaceStatus::MACE_SUCCESS);
+        orc_q8_gemm_u8(a.data(), b.data(), 1, rows, cols, depth, ORC_ROW_MAJOR, ORC_ROW_MAJOR, ORC_ROW_MAJOR, 1, 1,
+                       -131, -120, nullptr, mult, shift, 128, 0, 255, cw.data(), 4);
+        EXPECT(c == cw);
+      }
+    }
+    EXPECT(mace_hip_weight_cache_stats(hc, &builds1, &h1) == MACE_HIP_SUCCESS);
+    EXPECT(builds1 - builds0 == 1 && h1 - h0 == 2);
+    EXPECT(mace_hip_ctx_set_kernel_mask(hc, 0) == MACE_HIP_SUCCESS);
+    // float Gemm delegator created with should_cache_pack_: the constant side is uploaded once
+    std::normal_distribution<float> nd(0.f, 1.f);
+    std::vector<float> fl(64 * 48), fr(48 * 80), fo(64 * 80), fw(fo.size());
+    for (auto &v : fl) v = nd(rng);
+    Tensor FL(fl.data(), DT_FLOAT, {64, 48}, 0, 0, true), FO(fo.data(), DT_FLOAT, {});
+    EXPECT(mace_hip_host_weight_stats(hc, &up0, &hit0) == MACE_HIP_SUCCESS);
+    {
+      auto creator = reg.GetCreator(MACE_HIP_DELEGATOR_KEY(Gemm, RT_CPU, float, kCpuImplType));
+      std::unique_ptr<OpDelegator> d = creator(delegator::GemmParam(true));
+      auto *gemm = static_cast<delegator::Gemm *>(d.get());
+      for (int round = 0; round < 3; ++round) {
+        for (auto &v : fr) v = nd(rng);
+        Tensor FR(fr.data(), DT_FLOAT, {48, 80});
+        EXPECT(gemm->Compute(&context, &FL, &FR, 1, 64, 80, 48, RowMajor, RowMajor, RowMajor, true, true, &FO) ==
+               MaceStatus::MACE_SUCCESS);
+        orc_gemm_f32(fl.data(), fr.data(), 1, 64, 80, 48, ORC_ROW_MAJOR, ORC_ROW_MAJOR, ORC_ROW_MAJOR, 1, 1, fw.data(), 2);
+        EXPECT(close_enough(fo, fw));
+      }
+    }
+    EXPECT(mace_hip_host_weight_stats(hc, &up1, &hit1) == MACE_HIP_SUCCESS);
+    EXPECT(up1 - up0 == 1 && hit1 - hit0 == 3);
   }
   {  // conv_2d_test.cc:1240-1275: the quantized known answer 230, as a 1x1 conv over 18 channels
     std::vector<uint8_t> f = {102, 150, 123, 135, 1, 216, 137, 47, 53, 75, 145, 130, 171, 62, 255, 122, 72, 211};

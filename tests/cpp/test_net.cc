@@ -6,6 +6,7 @@
 //                          as a HIP graph, against the CPU oracle's ops chained by hand
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <random>
 #include <vector>
@@ -164,6 +165,141 @@ static int test_wire() {
   return g_fail;
 }
 
+// A NetDef serialized by an independent implementation of the wire format (the google.protobuf
+// package, tests/golden/make_netdef_fixture.py), in the schema's own encoding and with every
+// repeated scalar packed: both must parse to the same messages, with the values the script wrote.
+static std::string ReadFile(const std::string &path) {
+  std::string out;
+  if (FILE *f = fopen(path.c_str(), "rb")) {
+    char buf[4096];
+    size_t n;
+    while ((n = fread(buf, 1, sizeof(buf), f)) > 0) out.append(buf, n);
+    fclose(f);
+  }
+  return out;
+}
+
+static int test_fixture(const char *dir) {
+  for (const char *name : {"netdef_unpacked.pb", "netdef_packed.pb"}) {
+    const std::string bytes = ReadFile(std::string(dir) + "/" + name);
+    EXPECT(bytes.size() > 500);
+    NetDef net;
+    EXPECT(ParseNetDef(bytes.data(), bytes.size(), &net));
+    EXPECT(net.name == "fixture_net" && net.op.size() == 2 && net.tensors.size() == 3);
+    if (net.op.size() != 2 || net.tensors.size() != 3) continue;
+    const OperatorDef &op = net.op[0];
+    EXPECT(op.name == "conv_a" && op.type == "Conv2D");
+    EXPECT(op.input == (std::vector<std::string>{"in_q", "conv_a/filter", "conv_a/bias"}));
+    EXPECT(op.output == (std::vector<std::string>{"act_a"}));
+    EXPECT(op.arg.size() == 8);
+    EXPECT(GetIntArg(op, "T", 0) == 2);
+    EXPECT(GetIntsArg(op, "strides") == (std::vector<int>{2, 1}));
+    const Argument *pv = FindArg(op, "padding_values");
+    EXPECT(pv && pv->ints == (std::vector<int64_t>{-1, 0, 70000000000ll}));
+    const Argument *ml = FindArg(op, "max_limit");
+    EXPECT(ml && ml->has_f && ml->f == 6.0f && !ml->has_i);
+    const Argument *act = FindArg(op, "activation");
+    EXPECT(act && act->has_s && act->s == "RELUX");
+    const Argument *co = FindArg(op, "coeffs");
+    EXPECT(co && co->floats == (std::vector<float>{0.25f, -1.5f, 3.0e-5f}));
+    EXPECT(GetIntArg(op, "neg", 0) == -123456789012ll);
+    const Argument *empty = FindArg(op, "");
+    EXPECT(empty && empty->has_s && empty->s.empty());
+    EXPECT(op.output_shape.size() == 1 && op.output_shape[0] == (std::vector<int64_t>{64, 56, 56, 128}));
+    EXPECT(op.output_type == (std::vector<int>{DT_UINT8}));
+    EXPECT(op.quantize_info.size() == 1 && op.quantize_info[0].scale == 0.023529412f &&
+           op.quantize_info[0].zero_point == -7 && op.quantize_info[0].minval == -0.5f &&
+           op.quantize_info[0].maxval == 6.0f);
+    const OperatorDef &op2 = net.op[1];
+    EXPECT(op2.type == "Split" && op2.output == (std::vector<std::string>{"s0", "s1"}));
+    EXPECT(op2.output_shape.size() == 2 && op2.output_shape[0] == (std::vector<int64_t>{64, 56, 56, 64}) &&
+           op2.output_shape[1].empty());
+    EXPECT(op2.output_type == (std::vector<int>{DT_UINT8, DT_INT32}));
+    EXPECT(op2.quantize_info.size() == 2 && op2.quantize_info[0].zero_point == 255 &&
+           op2.quantize_info[1].zero_point == INT32_MIN && op2.quantize_info[1].scale == 1.0e-3f);
+    const ConstTensor &t = net.tensors[0];
+    EXPECT(t.name == "conv_a/filter" && t.dims == (std::vector<int64_t>{128, 1, 1, 128}) && t.data_type == DT_UINT8 &&
+           t.offset == 256 && t.data_size == 128 * 128 && t.scale == 0.0123f && t.zero_point == 131);
+    const ConstTensor &t2 = net.tensors[1];
+    EXPECT(t2.name == "conv_a/bias" && t2.dims == (std::vector<int64_t>{128}) && t2.data_type == DT_INT32 &&
+           t2.offset == 256 + 128 * 128 && t2.data_size == 128 && t2.scale == 2.5e-4f && t2.zero_point == -3);
+    EXPECT(net.tensors[2].name == "inline_floats" && net.tensors[2].data_type == DT_FLOAT);
+    EXPECT(net.input_info.size() == 1 && net.input_info[0].name == "in" &&
+           net.input_info[0].dims == (std::vector<int64_t>{64, 112, 112, 3}) && net.input_info[0].data_type == DT_FLOAT);
+    EXPECT(net.output_info.size() == 1 && net.output_info[0].name == "s1" && net.output_info[0].data_type == DT_INT32 &&
+           net.output_info[0].dims == (std::vector<int64_t>{64, 10}) && net.output_info[0].scale == 7.5f &&
+           net.output_info[0].zero_point == -9);
+    // every truncation of the independent writer's bytes is either refused or parses without
+    // reading past the end (run under the address sanitizer in the CPU suite)
+    for (size_t cut = 0; cut < bytes.size(); cut += 3) {
+      NetDef part;
+      (void)ParseNetDef(bytes.data(), cut, &part);
+    }
+  }
+  return g_fail;
+}
+
+// Malformed model descriptions (crafted dims, sizes and offsets) make Init return
+// MACE_INVALID_ARGS before it allocates anything.  This needs no GPU: the context is a plan-only
+// one, on which the first allocation of a well-formed model fails with OUT_OF_RESOURCES instead.
+static int test_malformed() {
+  OpDelegatorRegistry reg;
+  hip::RegisterAllHipDelegators(&reg);
+  mace_hip_ctx *plan = nullptr;
+  EXPECT(mace_hip_plan_ctx_create(256, 160 * 1024, &plan) == MACE_HIP_SUCCESS);
+  std::vector<uint8_t> data(4096, 1);
+  auto with_tensor = [&](std::vector<int64_t> dims, int64_t data_size, int64_t offset, int dt = DT_UINT8) {
+    NetDef n;
+    ConstTensor c; c.name = "w"; c.dims = std::move(dims); c.data_type = dt; c.offset = offset; c.data_size = data_size;
+    n.tensors.push_back(c);
+    SerialNet net(&reg, plan);
+    return net.Init(n, data.data(), data.size());
+  };
+  const MaceStatus bad = MaceStatus::MACE_INVALID_ARGS, fine = MaceStatus::MACE_OUT_OF_RESOURCES;
+  EXPECT(with_tensor({16, 16}, 256, 0) == fine);                        // well-formed: gets as far as the allocation
+  EXPECT(with_tensor({16, 16}, 256, 3840) == fine);                     // ends exactly at the end of the buffer
+  EXPECT(with_tensor({16, 16}, 256, 3841) == bad);                      // one byte past it
+  EXPECT(with_tensor({-1, -256}, 256, 0) == bad);                       // negative dims whose product is positive
+  EXPECT(with_tensor({-16, 16}, -256, 0) == bad);
+  EXPECT(with_tensor({1ll << 40, 1ll << 40}, 0, 0) == bad);             // product wraps to 0
+  EXPECT(with_tensor({1ll << 32, 1ll << 32, 256}, 256, 0) == bad);      // ... wraps to a small positive count
+  EXPECT(with_tensor({1ll << 62, 4}, 0, 0, DT_INT32) == bad);           // byte count overflows
+  EXPECT(with_tensor({16, 16}, 256, -4) == bad);                        // negative offset
+  EXPECT(with_tensor({16, 16}, 255, 0) == bad);                         // data_size disagrees with dims
+  EXPECT(with_tensor({0}, 0, INT64_MAX) == bad);                        // offset beyond the buffer
+  EXPECT(with_tensor({16}, 16, 0, 3 /* DT_HALF */) == bad);             // a type this runner does not hold
+  auto with_input = [&](std::vector<int64_t> dims, int dt) {
+    NetDef n;
+    InputOutputInfo in; in.name = "x"; in.dims = std::move(dims); in.data_type = dt;
+    n.input_info.push_back(in);
+    SerialNet net(&reg, plan);
+    return net.Init(n, nullptr, 0);
+  };
+  EXPECT(with_input({4, 4}, DT_FLOAT) == fine);
+  EXPECT(with_input({4, -4}, DT_FLOAT) == bad);
+  EXPECT(with_input({1ll << 31, 1ll << 31, 16}, DT_FLOAT) == bad);
+  EXPECT(with_input({1ll << 45, 8}, DT_UINT8) == bad);                  // no overflow, but no such tensor either
+  EXPECT(with_input({4}, 3) == bad);
+  {  // an op's outputs: a shape per output, quantize_info for all or none, sane shapes
+    NetDef n;
+    InputOutputInfo in; in.name = "x"; in.dims = {4}; in.data_type = DT_FLOAT;
+    n.input_info.push_back(in);
+    OperatorDef op; op.type = "Quantize"; op.name = "q"; op.input = {"x"}; op.output = {"y"};
+    op.output_type = {DT_UINT8};
+    n.op.push_back(op);
+    { SerialNet net(&reg, plan); EXPECT(net.Init(n, nullptr, 0) == bad); }           // no output_shape
+    n.op[0].output_shape = {{4, -1}};
+    { SerialNet net(&reg, plan); EXPECT(net.Init(n, nullptr, 0) == bad); }
+    n.op[0].output_shape = {{4}};
+    n.op[0].quantize_info.resize(2);
+    { SerialNet net(&reg, plan); EXPECT(net.Init(n, nullptr, 0) == bad); }
+    n.op[0].quantize_info.resize(1);
+    { SerialNet net(&reg, plan); EXPECT(net.Init(n, nullptr, 0) == fine); }
+  }
+  mace_hip_ctx_destroy(plan);
+  return g_fail;
+}
+
 static int test_run() {
   mace_hip_ctx *hctx = nullptr;
   if (mace_hip_ctx_create(0, &hctx) != MACE_HIP_SUCCESS) { printf("FAIL: no context\n"); return 1; }
@@ -244,9 +380,419 @@ static int test_run() {
   return g_fail;
 }
 
+static Argument FloatArg(const char *name, float v) { Argument a; a.name = name; a.f = v; a.has_f = true; return a; }
+static Argument StrArg(const char *name, const char *v) { Argument a; a.name = name; a.s = v; a.has_s = true; return a; }
+
+static void AddConst(NetDef *net, std::vector<uint8_t> *data, const char *name, std::vector<int64_t> dims, int dt,
+                     const void *bytes, size_t nbytes, float scale = 0.f, int32_t zp = 0) {
+  ConstTensor c;
+  c.name = name; c.dims = std::move(dims); c.data_type = dt; c.scale = scale; c.zero_point = zp;
+  while (data->size() % 16) data->push_back(0);
+  c.offset = (int64_t)data->size();
+  c.data_size = (int64_t)(nbytes / (dt == DT_UINT8 ? 1 : 4));
+  data->insert(data->end(), (const uint8_t *)bytes, (const uint8_t *)bytes + nbytes);
+  net->tensors.push_back(c);
+}
+static void AddOp(NetDef *net, const char *type, const char *name, std::vector<std::string> ins, const char *o,
+                  std::vector<int64_t> shape, int dt, float scale, int32_t zp, std::vector<Argument> args) {
+  OperatorDef d;
+  d.type = type; d.name = name; d.input = std::move(ins); d.output = {o};
+  d.output_shape = {std::move(shape)}; d.output_type = {dt};
+  if (scale > 0.f) { QuantizeActivationInfo q; q.scale = scale; q.zero_point = zp; d.quantize_info = {q}; }
+  d.arg = std::move(args);
+  net->op.push_back(d);
+}
+static bool close_f32(const std::vector<float> &got, const std::vector<float> &want) {
+  if (got.size() != want.size()) return false;
+  for (size_t i = 0; i < got.size(); ++i)
+    if (!(std::fabs(got[i] - want[i]) <= 1e-2 + 1e-4 * std::fabs(want[i]))) return false;
+  return true;
+}
+
+// The branches of the op factory the quantized toy net does not reach: float Conv2D (1x1, bias,
+// RELUX), Reshape / Identity views, float MatMul with bias, float FullyConnected with RELU,
+// Quantize, uint8 MatMul with a uint8 and with an int32 result, Dequantize of either -- one net,
+// every intermediate tensor against the oracle's ops chained by hand.
+static int test_mixed_net() {
+  mace_hip_ctx *hctx = nullptr;
+  if (mace_hip_ctx_create(0, &hctx) != MACE_HIP_SUCCESS) { printf("FAIL: no context\n"); return 1; }
+  OpDelegatorRegistry reg;
+  EXPECT(hip::RegisterAllHipDelegators(&reg) == MaceStatus::MACE_SUCCESS);
+  std::mt19937 rng(2024);
+  std::normal_distribution<float> nd(0.f, 1.f);
+  const index_t n = 2, cin = 8, hw = 36, cout = 16, mm_cols = 20, fc_in = cout * mm_cols, fc_out = 10, q_cols = 12;
+  std::vector<float> filt(cout * cin), cbias(cout), mm_w(hw * mm_cols), mm_b(mm_cols), fc_w(fc_out * fc_in), fc_b(fc_out);
+  for (auto *v : {&filt, &cbias, &mm_w, &mm_b, &fc_w, &fc_b}) for (auto &e : *v) e = nd(rng) * 0.3f;
+  std::vector<uint8_t> qw(fc_out * q_cols);
+  for (auto &e : qw) e = rng() & 255;
+  const float s_q = 0.05f, s_w = 0.02f, s_o = 1.5f; const int32_t z_q = 20, z_w = 119, z_o = 77;
+  NetDef net; std::vector<uint8_t> data;
+  net.name = "mixed";
+  AddConst(&net, &data, "conv/filter", {cout, cin, 1, 1}, DT_FLOAT, filt.data(), filt.size() * 4);
+  AddConst(&net, &data, "conv/bias", {cout}, DT_FLOAT, cbias.data(), cbias.size() * 4);
+  AddConst(&net, &data, "mm/w", {hw, mm_cols}, DT_FLOAT, mm_w.data(), mm_w.size() * 4);
+  AddConst(&net, &data, "mm/bias", {mm_cols}, DT_FLOAT, mm_b.data(), mm_b.size() * 4);
+  AddConst(&net, &data, "fc/w", {fc_out, fc_in, 1, 1}, DT_FLOAT, fc_w.data(), fc_w.size() * 4);
+  AddConst(&net, &data, "fc/bias", {fc_out}, DT_FLOAT, fc_b.data(), fc_b.size() * 4);
+  AddConst(&net, &data, "qmm/w", {fc_out, q_cols}, DT_UINT8, qw.data(), qw.size(), s_w, z_w);
+  InputOutputInfo in; in.name = "x"; in.dims = {n, cin, 6, 6}; in.data_type = DT_FLOAT;
+  net.input_info.push_back(in);
+  AddOp(&net, "Conv2D", "conv", {"x", "conv/filter", "conv/bias"}, "c", {n, cout, 6, 6}, DT_FLOAT, 0.f, 0,
+        {IntArg("T", DT_FLOAT), IntsArg("strides", {1, 1}), IntArg("padding", VALID), StrArg("activation", "RELUX"),
+         FloatArg("max_limit", 0.8f)});
+  AddOp(&net, "Reshape", "r0", {"c"}, "c3", {n, cout, hw}, DT_FLOAT, 0.f, 0, {});
+  AddOp(&net, "Identity", "id", {"c3"}, "c3i", {n, cout, hw}, DT_FLOAT, 0.f, 0, {});
+  AddOp(&net, "MatMul", "mm", {"c3i", "mm/w", "mm/bias"}, "m", {n, cout, mm_cols}, DT_FLOAT, 0.f, 0, {IntArg("T", DT_FLOAT)});
+  AddOp(&net, "Reshape", "r1", {"m"}, "m4", {n, fc_in, 1, 1}, DT_FLOAT, 0.f, 0, {});
+  AddOp(&net, "FullyConnected", "fc", {"m4", "fc/w", "fc/bias"}, "f", {n, fc_out, 1, 1}, DT_FLOAT, 0.f, 0,
+        {IntArg("T", DT_FLOAT), StrArg("activation", "RELU")});
+  AddOp(&net, "Quantize", "quant", {"f"}, "fq", {n, fc_out, 1, 1}, DT_UINT8, s_q, z_q, {IntArg("T", DT_UINT8)});
+  AddOp(&net, "Reshape", "r2", {"fq"}, "fq2", {n, fc_out}, DT_UINT8, 0.f, 0, {});
+  AddOp(&net, "MatMul", "qmm8", {"fq2", "qmm/w"}, "q8", {n, q_cols}, DT_UINT8, s_o, z_o, {IntArg("T", DT_UINT8)});
+  AddOp(&net, "MatMul", "qmm32", {"fq2", "qmm/w"}, "q32", {n, q_cols}, DT_INT32, 0.f, 0, {IntArg("T", DT_UINT8)});
+  AddOp(&net, "Dequantize", "deq8", {"q8"}, "d8", {n, q_cols}, DT_FLOAT, 0.f, 0, {IntArg("T", DT_UINT8)});
+  AddOp(&net, "Dequantize", "deq32", {"q32"}, "d32", {n, q_cols}, DT_FLOAT, 0.f, 0, {IntArg("T", DT_INT32)});
+  const std::string bytes = SerializeNetDef(net);
+  NetDef parsed;
+  EXPECT(ParseNetDef(bytes.data(), bytes.size(), &parsed));
+  SerialNet sn(&reg, hctx);
+  MaceStatus st = sn.Init(parsed, data.data(), data.size());
+  if (st != MaceStatus::MACE_SUCCESS) printf("Init: %s\n", sn.error().c_str());
+  EXPECT(st == MaceStatus::MACE_SUCCESS);
+  EXPECT(sn.op_count() == 8);    // four views create no op
+  std::vector<float> x(n * cin * hw);
+  for (auto &v : x) v = nd(rng);
+  EXPECT(sn.SetInput("x", x.data(), x.size() * 4) == MaceStatus::MACE_SUCCESS);
+  st = sn.Run();
+  if (st != MaceStatus::MACE_SUCCESS) printf("Run: %s\n", sn.error().c_str());
+  EXPECT(st == MaceStatus::MACE_SUCCESS);
+  // the oracle's chain
+  std::vector<float> c(n * cout * hw), m(n * cout * mm_cols), f(n * fc_out);
+  orc_conv1x1_f32_nchw(x.data(), filt.data(), cbias.data(), n, cin, hw, cout, ORC_ACT_RELUX, 0.8f, c.data(), 2);
+  orc_gemm_f32(c.data(), mm_w.data(), n, cout, mm_cols, hw, ORC_ROW_MAJOR, ORC_ROW_MAJOR, ORC_ROW_MAJOR, 1, 0, m.data(), 2);
+  for (size_t i = 0; i < m.size(); ++i) m[i] += mm_b[i % mm_cols];
+  orc_gemv_f32(fc_w.data(), m.data(), fc_b.data(), n, fc_out, fc_in, 0, 1, f.data(), 1);
+  orc_activation_f32(f.data(), (int64_t)f.size(), ORC_ACT_RELU, 0.f);
+  std::vector<float> got_c(c.size()), got_m(m.size()), got_f(f.size());
+  EXPECT(sn.GetOutput("c3i", got_c.data(), got_c.size() * 4) == MaceStatus::MACE_SUCCESS);
+  EXPECT(sn.GetOutput("m4", got_m.data(), got_m.size() * 4) == MaceStatus::MACE_SUCCESS);
+  EXPECT(sn.GetOutput("f", got_f.data(), got_f.size() * 4) == MaceStatus::MACE_SUCCESS);
+  EXPECT(close_f32(got_c, c) && close_f32(got_m, m) && close_f32(got_f, f));
+  float cmax = 0.f, fmin = 1.f;
+  for (float v : got_c) cmax = std::max(cmax, v);
+  for (float v : got_f) fmin = std::min(fmin, v);
+  EXPECT(cmax == 0.8f && fmin == 0.f);     // both activations bite
+  // the quantized tail starts from the GPU's own float values (so that a last-bit difference in f
+  // cannot flip a quantized byte of the comparison)
+  std::vector<uint8_t> fq(f.size()), got_fq(f.size()), q8(n * q_cols), got_q8(q8.size());
+  std::vector<int32_t> q32(n * q_cols), got_q32(q32.size());
+  orc_quantize_with_scale_u8(got_f.data(), (int64_t)got_f.size(), s_q, z_q, fq.data());
+  int32_t mult; int shift;
+  EXPECT(orc_get_output_multiplier_and_shift(s_q, s_w, s_o, &mult, &shift) == 0);
+  orc_q8_gemm_u8(fq.data(), qw.data(), 1, n, q_cols, fc_out, ORC_ROW_MAJOR, ORC_ROW_MAJOR, ORC_ROW_MAJOR, 1, 1, -z_q, -z_w,
+                 nullptr, mult, shift, z_o, 0, 255, q8.data(), 1);
+  orc_q8_gemm_i32(fq.data(), qw.data(), 1, n, q_cols, fc_out, ORC_ROW_MAJOR, ORC_ROW_MAJOR, ORC_ROW_MAJOR, 1, 1, -z_q, -z_w,
+                  q32.data(), 1);
+  EXPECT(sn.GetOutput("fq2", got_fq.data(), got_fq.size()) == MaceStatus::MACE_SUCCESS);
+  EXPECT(sn.GetOutput("q8", got_q8.data(), got_q8.size()) == MaceStatus::MACE_SUCCESS);
+  EXPECT(sn.GetOutput("q32", got_q32.data(), got_q32.size() * 4) == MaceStatus::MACE_SUCCESS);
+  EXPECT(got_fq == fq && got_q8 == q8 && got_q32 == q32);
+  std::vector<float> d8(q8.size()), d32(q32.size()), got_d8(d8.size()), got_d32(d32.size());
+  orc_dequantize_u8(q8.data(), (int64_t)q8.size(), s_o, z_o, d8.data());
+  // MatMulFixpointImpl<..., int32_t> gives its result scale = a.scale * b.scale, zero point 0
+  orc_dequantize_i32(q32.data(), (int64_t)q32.size(), s_q * s_w, 0, d32.data());
+  EXPECT(sn.GetOutput("d8", got_d8.data(), got_d8.size() * 4) == MaceStatus::MACE_SUCCESS);
+  EXPECT(sn.GetOutput("d32", got_d32.data(), got_d32.size() * 4) == MaceStatus::MACE_SUCCESS);
+  EXPECT(got_d8 == d8 && got_d32 == d32);
+  {  // a float FullyConnected whose activation this library does not apply is refused at Init
+    NetDef bad = parsed;
+    for (auto &a : bad.op[5].arg) if (a.name == "activation") a.s = "TANH";
+    SerialNet n2(&reg, hctx);
+    EXPECT(n2.Init(bad, data.data(), data.size()) == MaceStatus::MACE_UNSUPPORTED);
+    EXPECT(n2.error().find("TANH") != std::string::npos);
+    for (auto &a : bad.op[5].arg) if (a.name == "activation") a.s = "Relu";
+    SerialNet n3(&reg, hctx);
+    EXPECT(n3.Init(bad, data.data(), data.size()) == MaceStatus::MACE_INVALID_ARGS);
+  }
+  {  // ops that lack an input or an output are refused, not dereferenced
+    for (int which = 0; which < 3; ++which) {
+      NetDef bad = parsed;
+      if (which == 0) bad.op[6].input.clear();            // Quantize without input
+      if (which == 1) bad.op[11].output.clear(), bad.op[11].output_shape.clear(), bad.op[11].output_type.clear();
+      if (which == 2) bad.op[8].input.resize(1);          // MatMul with one input
+      SerialNet n2(&reg, hctx);
+      EXPECT(n2.Init(bad, data.data(), data.size()) == MaceStatus::MACE_INVALID_ARGS);
+    }
+  }
+  mace_hip_ctx_destroy(hctx);
+  return g_fail;
+}
+
+// The five pointwise layers of MobileNetV1-224 (benchmark configuration 4) inside a NetDef, through
+// the serial runner: per layer Quantize -> Conv2D 1x1 with a ReLU6 output range (zero point 0,
+// scale 6 / 255, so that the saturating cast is the clamp) -> Dequantize.  In the real network a
+// depthwise convolution sits between two of them and changes the shape, so here each layer is a
+// branch with an input of its own; the runner executes the fifteen ops in order, eagerly and as a
+// replayed HIP graph, and every branch is compared with the oracle's chain.  `timing`: also prints
+// the time per pass over all five layers (JSON, for bench.py).
+struct C4Layer { index_t hw, cin, cout; };
+static const C4Layer kC4[5] = {{112, 32, 64}, {56, 128, 128}, {28, 256, 256}, {14, 512, 512}, {7, 1024, 1024}};
+
+static int test_c4_net(index_t batch, bool timing) {
+  mace_hip_ctx *hctx = nullptr;
+  if (mace_hip_ctx_create(0, &hctx) != MACE_HIP_SUCCESS) { printf("FAIL: no context\n"); return 1; }
+  OpDelegatorRegistry reg;
+  EXPECT(hip::RegisterAllHipDelegators(&reg) == MaceStatus::MACE_SUCCESS);
+  std::mt19937 rng(4);
+  NetDef net; std::vector<uint8_t> data;
+  net.name = "mobilenet_v1_pointwise_layers";
+  const float s_in = 6.f / 255.f, s_f = 0.01f, s_out = 6.f / 255.f;
+  const int32_t z_in = 0, z_out = 0;
+  std::vector<std::vector<uint8_t>> filt(5);
+  std::vector<std::vector<int32_t>> bias(5);
+  int32_t z_f[5];
+  for (int l = 0; l < 5; ++l) {
+    const C4Layer &L = kC4[l];
+    filt[l].resize(L.cout * L.cin); bias[l].resize(L.cout);
+    for (auto &e : filt[l]) e = (uint8_t)(rng() % 255 + 1);
+    for (auto &e : bias[l]) e = (int32_t)(rng() % 65536) - 32768;
+    z_f[l] = 100 + (int)(rng() % 56);
+    char name[64];
+    snprintf(name, sizeof(name), "pw%d/filter", l);
+    AddConst(&net, &data, name, {L.cout, 1, 1, L.cin}, DT_UINT8, filt[l].data(), filt[l].size(), s_f, z_f[l]);
+    snprintf(name, sizeof(name), "pw%d/bias", l);
+    AddConst(&net, &data, name, {L.cout}, DT_INT32, bias[l].data(), bias[l].size() * 4, s_in * s_f, 0);
+  }
+  for (int l = 0; l < 5; ++l) {
+    const C4Layer &L = kC4[l];
+    char x[32], xq[32], y[32], yf[32], f[32], b[32], nq[32], nc[32], nd[32];
+    snprintf(x, 32, "in%d", l); snprintf(xq, 32, "in%d_q", l); snprintf(y, 32, "act%d", l); snprintf(yf, 32, "out%d", l);
+    snprintf(f, 32, "pw%d/filter", l); snprintf(b, 32, "pw%d/bias", l);
+    snprintf(nq, 32, "quantize%d", l); snprintf(nc, 32, "pointwise%d", l); snprintf(nd, 32, "dequantize%d", l);
+    InputOutputInfo in; in.name = x; in.dims = {batch, L.hw, L.hw, L.cin}; in.data_type = DT_FLOAT;
+    net.input_info.push_back(in);
+    AddOp(&net, "Quantize", nq, {x}, xq, {batch, L.hw, L.hw, L.cin}, DT_UINT8, s_in, z_in, {IntArg("T", DT_UINT8)});
+    AddOp(&net, "Conv2D", nc, {xq, f, b}, y, {batch, L.hw, L.hw, L.cout}, DT_UINT8, s_out, z_out,
+          {IntArg("T", DT_UINT8), IntsArg("strides", {1, 1}), IntArg("padding", VALID), StrArg("activation", "RELUX"),
+           FloatArg("max_limit", 6.f)});
+    AddOp(&net, "Dequantize", nd, {y}, yf, {batch, L.hw, L.hw, L.cout}, DT_FLOAT, 0.f, 0, {IntArg("T", DT_UINT8)});
+  }
+  const std::string bytes = SerializeNetDef(net);
+  NetDef parsed;
+  EXPECT(ParseNetDef(bytes.data(), bytes.size(), &parsed));
+  SerialNet sn(&reg, hctx);
+  MaceStatus st = sn.Init(parsed, data.data(), data.size());
+  if (st != MaceStatus::MACE_SUCCESS) printf("Init: %s\n", sn.error().c_str());
+  EXPECT(st == MaceStatus::MACE_SUCCESS && sn.op_count() == 15);
+  std::uniform_real_distribution<float> ud(-0.5f, 6.5f);
+  std::vector<std::vector<float>> x(5);
+  for (int l = 0; l < 5; ++l) {
+    x[l].resize((size_t)batch * kC4[l].hw * kC4[l].hw * kC4[l].cin);
+    for (auto &v : x[l]) v = ud(rng);
+  }
+  auto check = [&](const char *what) {
+    for (int l = 0; l < 5; ++l) {
+      const C4Layer &L = kC4[l];
+      const size_t pix = (size_t)batch * L.hw * L.hw;
+      std::vector<uint8_t> q(x[l].size()), a(pix * L.cout);
+      std::vector<float> want(a.size()), got(a.size());
+      orc_quantize_with_scale_u8(x[l].data(), (int64_t)x[l].size(), s_in, z_in, q.data());
+      EXPECT(orc_conv2d_q8_nhwc(q.data(), filt[l].data(), bias[l].data(), batch, L.hw, L.hw, L.cin, L.cout, 1, 1, 1, 1, 0, 0,
+                                s_in, z_in, s_f, z_f[l], s_in * s_f, s_out, z_out, 0, 255, a.data(), 16) == 0);
+      orc_dequantize_u8(a.data(), (int64_t)a.size(), s_out, z_out, want.data());
+      char name[32]; snprintf(name, 32, "out%d", l);
+      EXPECT(sn.GetOutput(name, got.data(), got.size() * 4) == MaceStatus::MACE_SUCCESS);
+      const bool same = got == want;
+      if (!same) printf("%s: layer %d differs\n", what, l);
+      EXPECT(same);
+      size_t lo = 0, hi = 0;
+      for (uint8_t v : a) { lo += v == 0; hi += v == 255; }
+      EXPECT(lo + hi < a.size() * 9 / 10 && lo + hi > 0);   // the ReLU6 clamp bites, but not everywhere
+    }
+  };
+  auto set_inputs = [&]() {
+    for (int l = 0; l < 5; ++l) {
+      char name[32]; snprintf(name, 32, "in%d", l);
+      EXPECT(sn.SetInput(name, x[l].data(), x[l].size() * 4) == MaceStatus::MACE_SUCCESS);
+    }
+  };
+  set_inputs();
+  EXPECT(sn.Run() == MaceStatus::MACE_SUCCESS);
+  check("eager");
+  st = sn.CaptureGraph();
+  if (st != MaceStatus::MACE_SUCCESS) printf("CaptureGraph: %s\n", sn.error().c_str());
+  EXPECT(st == MaceStatus::MACE_SUCCESS);
+  for (int replay = 0; replay < 2; ++replay) {
+    for (int l = 0; l < 5; ++l) for (size_t i = replay; i < x[l].size(); i += 7) x[l][i] = ud(rng);
+    set_inputs();
+    EXPECT(sn.RunGraph() == MaceStatus::MACE_SUCCESS);
+    check("graph");
+    if (replay == 0) { EXPECT(sn.Run() == MaceStatus::MACE_SUCCESS); EXPECT(mace_hip_sync(hctx) == MACE_HIP_SUCCESS); }
+  }
+  if (timing) {
+    float ms_eager = 0.f, ms_graph = 0.f;
+    const int reps = 30;
+    for (int i = 0; i < 5; ++i) sn.Run();
+    mace_hip_timer_start(hctx);
+    for (int i = 0; i < reps; ++i) sn.Run();
+    mace_hip_timer_stop(hctx, &ms_eager);
+    for (int i = 0; i < 5; ++i) sn.RunGraph();
+    mace_hip_timer_start(hctx);
+    for (int i = 0; i < reps; ++i) sn.RunGraph();
+    mace_hip_timer_stop(hctx, &ms_graph);
+    double ops = 0;
+    for (const C4Layer &L : kC4) ops += 2.0 * batch * L.hw * L.hw * L.cin * L.cout;
+    printf("{\"workload\": \"c4_chain_n%d\", \"ops_in_net\": 15, \"eager_us\": %.1f, \"graph_us\": %.1f, "
+           "\"conv_ops\": %.4g, \"parity\": %s}\n", (int)batch, ms_eager * 1e3 / reps, ms_graph * 1e3 / reps, ops,
+           g_fail ? "false" : "true");
+  }
+  mace_hip_ctx_destroy(hctx);
+  return g_fail;
+}
+
+// An op supplied by the host (SerialNet::RegisterOp): a 2x2 average pool computed on the CPU sits
+// between two of this library's convolutions, so a net with an op type outside the library runs.
+static int test_host_op() {
+  mace_hip_ctx *hctx = nullptr;
+  if (mace_hip_ctx_create(0, &hctx) != MACE_HIP_SUCCESS) { printf("FAIL: no context\n"); return 1; }
+  OpDelegatorRegistry reg;
+  EXPECT(hip::RegisterAllHipDelegators(&reg) == MaceStatus::MACE_SUCCESS);
+  std::mt19937 rng(8);
+  const index_t n = 2, hw = 8, c0 = 32, c1 = 64, c2 = 48;
+  std::vector<uint8_t> f0(c1 * c0), f1(c2 * c1);
+  for (auto &e : f0) e = rng() & 255;
+  for (auto &e : f1) e = rng() & 255;
+  NetDef net; std::vector<uint8_t> data;
+  AddConst(&net, &data, "f0", {c1, 1, 1, c0}, DT_UINT8, f0.data(), f0.size(), 0.01f, 125);
+  AddConst(&net, &data, "f1", {c2, 1, 1, c1}, DT_UINT8, f1.data(), f1.size(), 0.012f, 130);
+  InputOutputInfo in; in.name = "x"; in.dims = {n, hw, hw, c0}; in.data_type = DT_UINT8; in.scale = 0.05f; in.zero_point = 128;
+  net.input_info.push_back(in);
+  AddOp(&net, "Conv2D", "conv0", {"x", "f0"}, "a", {n, hw, hw, c1}, DT_UINT8, 0.8f, 120, {IntArg("T", DT_UINT8), IntArg("padding", VALID)});
+  AddOp(&net, "Pooling", "pool", {"a"}, "p", {n, hw / 2, hw / 2, c1}, DT_UINT8, 0.8f, 120, {IntArg("T", DT_UINT8), IntsArg("kernels", {2, 2})});
+  AddOp(&net, "Conv2D", "conv1", {"p", "f1"}, "y", {n, hw / 2, hw / 2, c2}, DT_UINT8, 6.0f, 110, {IntArg("T", DT_UINT8), IntArg("padding", VALID)});
+  auto pool = [](const std::vector<uint8_t> &a, index_t n, index_t hw, index_t c) {
+    std::vector<uint8_t> p((size_t)n * (hw / 2) * (hw / 2) * c);
+    for (index_t b = 0; b < n; ++b)
+      for (index_t y = 0; y < hw / 2; ++y)
+        for (index_t x = 0; x < hw / 2; ++x)
+          for (index_t k = 0; k < c; ++k) {
+            int s = 2;   // rounds to nearest
+            for (int dy = 0; dy < 2; ++dy) for (int dx = 0; dx < 2; ++dx) s += a[((b * hw + 2 * y + dy) * hw + 2 * x + dx) * c + k];
+            p[((b * (hw / 2) + y) * (hw / 2) + x) * c + k] = (uint8_t)(s / 4);
+          }
+    return p;
+  };
+  {  // without the host's op the net cannot be initialised
+    SerialNet sn(&reg, hctx);
+    EXPECT(sn.Init(net, data.data(), data.size()) == MaceStatus::MACE_UNSUPPORTED);
+    EXPECT(sn.error().find("Pooling") != std::string::npos);
+  }
+  SerialNet sn(&reg, hctx);
+  int created = 0;
+  sn.RegisterOp("Pooling", [&](const OperatorDef &def, SerialNet *self, SerialNet::OpRun *run) {
+    Tensor *src = self->GetTensor(def.input[0]), *dst = self->GetTensor(def.output[0]);
+    if (!src || !dst || GetIntsArg(def, "kernels") != std::vector<int>{2, 2}) return MaceStatus::MACE_INVALID_ARGS;
+    ++created;
+    *run = [src, dst, pool](OpContext *c) {
+      std::vector<uint8_t> a((size_t)src->size());
+      if (mace_hip_memcpy_d2h(c->hip(), a.data(), src->data<uint8_t>(), a.size()) != MACE_HIP_SUCCESS)
+        return MaceStatus::MACE_RUNTIME_ERROR;
+      const std::vector<uint8_t> p = pool(a, src->dim(0), src->dim(1), src->dim(3));
+      return ToStatus(mace_hip_memcpy_h2d(c->hip(), dst->mutable_data<uint8_t>(), p.data(), p.size()));
+    };
+    return MaceStatus::MACE_SUCCESS;
+  });
+  MaceStatus st = sn.Init(net, data.data(), data.size());
+  if (st != MaceStatus::MACE_SUCCESS) printf("Init: %s\n", sn.error().c_str());
+  EXPECT(st == MaceStatus::MACE_SUCCESS && created == 1 && sn.op_count() == 3);
+  std::vector<uint8_t> x((size_t)n * hw * hw * c0), got((size_t)n * (hw / 2) * (hw / 2) * c2), a((size_t)n * hw * hw * c1), want(got.size());
+  for (auto &e : x) e = rng() & 255;
+  EXPECT(sn.SetInput("x", x.data(), x.size()) == MaceStatus::MACE_SUCCESS);
+  EXPECT(sn.Run() == MaceStatus::MACE_SUCCESS);
+  EXPECT(sn.GetOutput("y", got.data(), got.size()) == MaceStatus::MACE_SUCCESS);
+  EXPECT(orc_conv2d_q8_nhwc(x.data(), f0.data(), nullptr, n, hw, hw, c0, c1, 1, 1, 1, 1, 0, 0, 0.05f, 128, 0.01f, 125, 0.f, 0.8f,
+                            120, 0, 255, a.data(), 2) == 0);
+  const std::vector<uint8_t> p = pool(a, n, hw, c1);
+  EXPECT(orc_conv2d_q8_nhwc(p.data(), f1.data(), nullptr, n, hw / 2, hw / 2, c1, c2, 1, 1, 1, 1, 0, 0, 0.8f, 120, 0.012f, 130, 0.f,
+                            6.0f, 110, 0, 255, want.data(), 2) == 0);
+  EXPECT(got == want);
+  // a host op that waits for the stream cannot be part of a captured graph: the capture fails cleanly
+  EXPECT(sn.CaptureGraph() != MaceStatus::MACE_SUCCESS);
+  EXPECT(sn.Run() == MaceStatus::MACE_SUCCESS);   // ... and the context stays usable
+  EXPECT(sn.GetOutput("y", got.data(), got.size()) == MaceStatus::MACE_SUCCESS);
+  EXPECT(got == want);
+  mace_hip_ctx_destroy(hctx);
+  return g_fail;
+}
+
+// An instantiated graph holds raw pointers into the context's arena.  Eager work that outgrows
+// the arena afterwards must not pull it from under the graph: the old arena is kept until the
+// graph is destroyed, and a replay after the growth still matches the oracle.
+static int test_graph_outlives_arena_growth() {
+  mace_hip_ctx *hctx = nullptr;
+  if (mace_hip_ctx_create(0, &hctx) != MACE_HIP_SUCCESS) { printf("FAIL: no context\n"); return 1; }
+  OpDelegatorRegistry reg;
+  EXPECT(hip::RegisterAllHipDelegators(&reg) == MaceStatus::MACE_SUCCESS);
+  Weights wt;
+  Model m = BuildModel(&wt);
+  std::mt19937 rng(77);
+  std::normal_distribution<float> nd(0.f, 2.f);
+  {
+    SerialNet net(&reg, hctx);
+    EXPECT(net.Init(m.net, m.data.data(), m.data.size()) == MaceStatus::MACE_SUCCESS);
+    std::vector<float> x((size_t)m.n * m.h * m.w * m.c0), got(m.n * m.classes);
+    for (auto &v : x) v = nd(rng);
+    EXPECT(net.SetInput("data", x.data(), x.size() * 4) == MaceStatus::MACE_SUCCESS);
+    EXPECT(net.Run() == MaceStatus::MACE_SUCCESS);
+    EXPECT(net.CaptureGraph() == MaceStatus::MACE_SUCCESS);
+    // an eager GEMM whose repacked panels need far more scratch than the toy net ever took:
+    // ColMajor lhs and RowMajor rhs with an odd depth are both repacked (2 x 3000 x 1088 bytes)
+    const index_t rows = 3000, depth = 1031, cols = 3000;
+    std::vector<uint8_t> a(rows * depth), b(depth * cols);
+    for (auto &e : a) e = rng() & 255;
+    for (auto &e : b) e = rng() & 255;
+    void *da = nullptr, *db = nullptr, *dc = nullptr;
+    EXPECT(mace_hip_malloc(hctx, a.size(), &da) == MACE_HIP_SUCCESS && mace_hip_malloc(hctx, b.size(), &db) == MACE_HIP_SUCCESS &&
+           mace_hip_malloc(hctx, (size_t)rows * cols * 4, &dc) == MACE_HIP_SUCCESS);
+    mace_hip_memcpy_h2d(hctx, da, a.data(), a.size());
+    mace_hip_memcpy_h2d(hctx, db, b.data(), b.size());
+    EXPECT(mace_hip_gemm_q8_i32(hctx, (const uint8_t *)da, MACE_HIP_COL_MAJOR, (const uint8_t *)db, MACE_HIP_ROW_MAJOR,
+                                (int32_t *)dc, MACE_HIP_ROW_MAJOR, 1, rows, depth, cols, 1, 1, -100, -90) == MACE_HIP_SUCCESS);
+    mace_hip_plan plan;
+    EXPECT(mace_hip_last_plan(hctx, &plan) == MACE_HIP_SUCCESS && (plan.aux & MACE_HIP_AUX_PACK_TRANSPOSE));
+    std::vector<int32_t> c32((size_t)rows * cols), w32(c32.size());
+    mace_hip_memcpy_d2h(hctx, c32.data(), dc, c32.size() * 4);
+    orc_q8_gemm_i32(a.data(), b.data(), 1, rows, cols, depth, ORC_COL_MAJOR, ORC_ROW_MAJOR, ORC_ROW_MAJOR, 1, 1, -100, -90,
+                    w32.data(), 16);
+    EXPECT(c32 == w32);
+    // the graph, recorded against the arena of before, still computes the net
+    for (int replay = 0; replay < 2; ++replay) {
+      for (auto &v : x) v = nd(rng);
+      EXPECT(net.SetInput("data", x.data(), x.size() * 4) == MaceStatus::MACE_SUCCESS);
+      EXPECT(net.RunGraph() == MaceStatus::MACE_SUCCESS);
+      EXPECT(net.GetOutput("prob", got.data(), got.size() * 4) == MaceStatus::MACE_SUCCESS);
+      EXPECT(got == OracleRun(m, wt, x));
+      EXPECT(net.Run() == MaceStatus::MACE_SUCCESS);     // eager runs use the new arena
+      EXPECT(net.GetOutput("prob", got.data(), got.size() * 4) == MaceStatus::MACE_SUCCESS);
+      EXPECT(got == OracleRun(m, wt, x));
+    }
+    mace_hip_free(hctx, da); mace_hip_free(hctx, db); mace_hip_free(hctx, dc);
+  }
+  mace_hip_ctx_destroy(hctx);
+  return g_fail;
+}
+
 int main(int argc, char **argv) {
   const char *mode = argc > 1 ? argv[1] : "wire";
-  const int fails = strcmp(mode, "run") == 0 ? test_run() : test_wire();
+  int fails;
+  if (strcmp(mode, "run") == 0) fails = test_run();
+  else if (strcmp(mode, "fixture") == 0) fails = test_fixture(argc > 2 ? argv[2] : "tests/golden");
+  else if (strcmp(mode, "malformed") == 0) fails = test_malformed();
+  else if (strcmp(mode, "mixed") == 0) fails = test_mixed_net();
+  else if (strcmp(mode, "c4") == 0) fails = test_c4_net(argc > 2 ? atoi(argv[2]) : 2, argc > 3);
+  else if (strcmp(mode, "hostop") == 0) fails = test_host_op();
+  else if (strcmp(mode, "graph_arena") == 0) fails = test_graph_outlives_arena_growth();
+  else fails = test_wire();
   printf("%s: %s (%d failures)\n", mode, fails ? "FAILED" : "ok", fails);
   return fails ? 1 : 0;
 }

@@ -475,6 +475,48 @@ def test_q8_gemm_freivalds_large(ctx, n):
     assert 0 < ((got8 == 0) | (got8 == 255)).mean() < 0.1 and len(np.unique(got8)) > 200
 
 
+@pytest.mark.parametrize("batch,n,kernel", [(1, 2048, "mid/XT"), (32, 512, "xres/XT")])
+def test_q8_gemm_config5_random_zero_points(ctx, batch, n, kernel):
+    """Benchmark configuration 5 with all three zero points drawn from U{0..255} and the output
+    scale derived from the data.  With zero points far from the operands' mean the accumulators sit
+    at K (127.5 - za)(127.5 - zb), dozens of standard deviations from zero, so the real multiplier
+    is taken as 100 / (|mean| + 3 sigma) of the oracle's accumulators: the uint8 outputs then lie
+    around zc +- 100 with a few levels of spread.  The zero points are the first draw of the seeded
+    stream for which that window stays inside [0, 255] (a property of the three scalars and K
+    alone), so that the uint8 comparison is not a comparison of saturated bytes: the saturated
+    fraction is asserted below one half.  int32 and uint8 results in full against the oracle."""
+    rng = np.random.default_rng(5)
+    A = rng.integers(0, 256, (batch, n, n), dtype=np.uint8)
+    B = rng.integers(0, 256, (batch, n, n), dtype=np.uint8)
+    for _ in range(64):
+        za, zb, zc = (int(v) for v in rng.integers(0, 256, 3))
+        centre = zc + 100.0 * np.sign((127.5 - za) * (127.5 - zb))
+        if 20 <= centre <= 235:
+            break
+    want32 = orc.q8_gemm_i32(A, B, batch, n, n, n, -za, -zb, nthreads=16)
+    real = 100.0 / (abs(float(want32.mean())) + 3.0 * float(want32.std()))
+    mult, e = orc.quantize_multiplier(real)
+    shift = -e
+    assert 0 < real < 1 and shift >= 0
+    d = Dev()
+    dl, dr = d.put(A), d.put(B)
+    t32, p32 = d.empty(batch * n * n, np.int32)
+    t8, p8 = d.empty(batch * n * n, np.uint8)
+    d.sync()
+    ctx.call("mace_hip_gemm_q8_i32", dl, R, dr, R, p32, R, batch, n, n, n, 1, 1, -za, -zb)
+    assert kernel_tag(ctx.last_plan()) == kernel
+    ctx.call("mace_hip_gemm_q8_u8", dl, R, dr, R, p8, R, batch, n, n, n, 1, 1, -za, -zb, None, mult,
+             shift, zc, 0, 255)
+    assert kernel_tag(ctx.last_plan()) == kernel
+    ctx.sync()
+    np.testing.assert_array_equal(t32.cpu().numpy(), want32)
+    want8 = orc.q8_gemm_u8(A, B, batch, n, n, n, -za, -zb, None, mult, shift, zc, nthreads=16)
+    np.testing.assert_array_equal(t8.cpu().numpy(), want8)
+    sat = float(((want8 == 0) | (want8 == 255)).mean())
+    assert sat < 0.5, (za, zb, zc, sat)
+    assert len(np.unique(want8)) >= 4
+
+
 def test_q8_gemm_errors(ctx):
     z = np.zeros(64, np.uint8)
     o = np.zeros(64, np.uint8)
