@@ -380,6 +380,13 @@ static int test_run() {
   return g_fail;
 }
 
+// Destroys the library context after everything declared later in the scope (nets and ops release
+// their registrations and device memory through it, so they have to go first).
+struct ContextHolder {
+  mace_hip_ctx *ctx = nullptr;
+  ~ContextHolder() { if (ctx) mace_hip_ctx_destroy(ctx); }
+};
+
 static Argument FloatArg(const char *name, float v) { Argument a; a.name = name; a.f = v; a.has_f = true; return a; }
 static Argument StrArg(const char *name, const char *v) { Argument a; a.name = name; a.s = v; a.has_s = true; return a; }
 
@@ -414,8 +421,9 @@ static bool close_f32(const std::vector<float> &got, const std::vector<float> &w
 // Quantize, uint8 MatMul with a uint8 and with an int32 result, Dequantize of either -- one net,
 // every intermediate tensor against the oracle's ops chained by hand.
 static int test_mixed_net() {
-  mace_hip_ctx *hctx = nullptr;
-  if (mace_hip_ctx_create(0, &hctx) != MACE_HIP_SUCCESS) { printf("FAIL: no context\n"); return 1; }
+  ContextHolder holder;
+  if (mace_hip_ctx_create(0, &holder.ctx) != MACE_HIP_SUCCESS) { printf("FAIL: no context\n"); return 1; }
+  mace_hip_ctx *hctx = holder.ctx;
   OpDelegatorRegistry reg;
   EXPECT(hip::RegisterAllHipDelegators(&reg) == MaceStatus::MACE_SUCCESS);
   std::mt19937 rng(2024);
@@ -524,7 +532,6 @@ static int test_mixed_net() {
       EXPECT(n2.Init(bad, data.data(), data.size()) == MaceStatus::MACE_INVALID_ARGS);
     }
   }
-  mace_hip_ctx_destroy(hctx);
   return g_fail;
 }
 
@@ -539,14 +546,18 @@ struct C4Layer { index_t hw, cin, cout; };
 static const C4Layer kC4[5] = {{112, 32, 64}, {56, 128, 128}, {28, 256, 256}, {14, 512, 512}, {7, 1024, 1024}};
 
 static int test_c4_net(index_t batch, bool timing) {
-  mace_hip_ctx *hctx = nullptr;
-  if (mace_hip_ctx_create(0, &hctx) != MACE_HIP_SUCCESS) { printf("FAIL: no context\n"); return 1; }
+  ContextHolder holder;
+  if (mace_hip_ctx_create(0, &holder.ctx) != MACE_HIP_SUCCESS) { printf("FAIL: no context\n"); return 1; }
+  mace_hip_ctx *hctx = holder.ctx;
   OpDelegatorRegistry reg;
   EXPECT(hip::RegisterAllHipDelegators(&reg) == MaceStatus::MACE_SUCCESS);
   std::mt19937 rng(4);
   NetDef net; std::vector<uint8_t> data;
   net.name = "mobilenet_v1_pointwise_layers";
-  const float s_in = 6.f / 255.f, s_f = 0.01f, s_out = 6.f / 255.f;
+  // filter scales such that the real-valued sums have a standard deviation of about 3: the ReLU6
+  // range [0, 6] then clamps a good part of the outputs at either end, but not most of them
+  const float s_in = 6.f / 255.f, s_out = 6.f / 255.f;
+  float s_f[5];
   const int32_t z_in = 0, z_out = 0;
   std::vector<std::vector<uint8_t>> filt(5);
   std::vector<std::vector<int32_t>> bias(5);
@@ -556,12 +567,13 @@ static int test_c4_net(index_t batch, bool timing) {
     filt[l].resize(L.cout * L.cin); bias[l].resize(L.cout);
     for (auto &e : filt[l]) e = (uint8_t)(rng() % 255 + 1);
     for (auto &e : bias[l]) e = (int32_t)(rng() % 65536) - 32768;
-    z_f[l] = 100 + (int)(rng() % 56);
+    z_f[l] = 126 + (int)(rng() % 5);
+    s_f[l] = 3.f / (74.f * std::sqrt(12.f * (float)L.cin));
     char name[64];
     snprintf(name, sizeof(name), "pw%d/filter", l);
-    AddConst(&net, &data, name, {L.cout, 1, 1, L.cin}, DT_UINT8, filt[l].data(), filt[l].size(), s_f, z_f[l]);
+    AddConst(&net, &data, name, {L.cout, 1, 1, L.cin}, DT_UINT8, filt[l].data(), filt[l].size(), s_f[l], z_f[l]);
     snprintf(name, sizeof(name), "pw%d/bias", l);
-    AddConst(&net, &data, name, {L.cout}, DT_INT32, bias[l].data(), bias[l].size() * 4, s_in * s_f, 0);
+    AddConst(&net, &data, name, {L.cout}, DT_INT32, bias[l].data(), bias[l].size() * 4, s_in * s_f[l], 0);
   }
   for (int l = 0; l < 5; ++l) {
     const C4Layer &L = kC4[l];
@@ -598,7 +610,7 @@ static int test_c4_net(index_t batch, bool timing) {
       std::vector<float> want(a.size()), got(a.size());
       orc_quantize_with_scale_u8(x[l].data(), (int64_t)x[l].size(), s_in, z_in, q.data());
       EXPECT(orc_conv2d_q8_nhwc(q.data(), filt[l].data(), bias[l].data(), batch, L.hw, L.hw, L.cin, L.cout, 1, 1, 1, 1, 0, 0,
-                                s_in, z_in, s_f, z_f[l], s_in * s_f, s_out, z_out, 0, 255, a.data(), 16) == 0);
+                                s_in, z_in, s_f[l], z_f[l], s_in * s_f[l], s_out, z_out, 0, 255, a.data(), 16) == 0);
       orc_dequantize_u8(a.data(), (int64_t)a.size(), s_out, z_out, want.data());
       char name[32]; snprintf(name, 32, "out%d", l);
       EXPECT(sn.GetOutput(name, got.data(), got.size() * 4) == MaceStatus::MACE_SUCCESS);
@@ -646,15 +658,15 @@ static int test_c4_net(index_t batch, bool timing) {
            "\"conv_ops\": %.4g, \"parity\": %s}\n", (int)batch, ms_eager * 1e3 / reps, ms_graph * 1e3 / reps, ops,
            g_fail ? "false" : "true");
   }
-  mace_hip_ctx_destroy(hctx);
   return g_fail;
 }
 
 // An op supplied by the host (SerialNet::RegisterOp): a 2x2 average pool computed on the CPU sits
 // between two of this library's convolutions, so a net with an op type outside the library runs.
 static int test_host_op() {
-  mace_hip_ctx *hctx = nullptr;
-  if (mace_hip_ctx_create(0, &hctx) != MACE_HIP_SUCCESS) { printf("FAIL: no context\n"); return 1; }
+  ContextHolder holder;
+  if (mace_hip_ctx_create(0, &holder.ctx) != MACE_HIP_SUCCESS) { printf("FAIL: no context\n"); return 1; }
+  mace_hip_ctx *hctx = holder.ctx;
   OpDelegatorRegistry reg;
   EXPECT(hip::RegisterAllHipDelegators(&reg) == MaceStatus::MACE_SUCCESS);
   std::mt19937 rng(8);
@@ -721,7 +733,6 @@ static int test_host_op() {
   EXPECT(sn.Run() == MaceStatus::MACE_SUCCESS);   // ... and the context stays usable
   EXPECT(sn.GetOutput("y", got.data(), got.size()) == MaceStatus::MACE_SUCCESS);
   EXPECT(got == want);
-  mace_hip_ctx_destroy(hctx);
   return g_fail;
 }
 
@@ -729,8 +740,9 @@ static int test_host_op() {
 // the arena afterwards must not pull it from under the graph: the old arena is kept until the
 // graph is destroyed, and a replay after the growth still matches the oracle.
 static int test_graph_outlives_arena_growth() {
-  mace_hip_ctx *hctx = nullptr;
-  if (mace_hip_ctx_create(0, &hctx) != MACE_HIP_SUCCESS) { printf("FAIL: no context\n"); return 1; }
+  ContextHolder holder;
+  if (mace_hip_ctx_create(0, &holder.ctx) != MACE_HIP_SUCCESS) { printf("FAIL: no context\n"); return 1; }
+  mace_hip_ctx *hctx = holder.ctx;
   OpDelegatorRegistry reg;
   EXPECT(hip::RegisterAllHipDelegators(&reg) == MaceStatus::MACE_SUCCESS);
   Weights wt;
@@ -778,7 +790,6 @@ static int test_graph_outlives_arena_growth() {
     }
     mace_hip_free(hctx, da); mace_hip_free(hctx, db); mace_hip_free(hctx, dc);
   }
-  mace_hip_ctx_destroy(hctx);
   return g_fail;
 }
 
