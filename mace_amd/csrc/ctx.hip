@@ -3,6 +3,7 @@
 #include <stdarg.h>
 #include <string.h>
 
+#include <mutex>
 #include <new>
 
 #include "common.h"
@@ -24,10 +25,12 @@ int mh_fail(mace_hip_ctx *ctx, int code, const char *fmt, ...) {
 static __device__ __align__(256) unsigned char scratch[MACE_HIP_NOALLOC_SCRATCH_BYTES];
 constexpr int MH_MAX_DEVICES = 64;
 static void *g_scratch_ptr[MH_MAX_DEVICES];
+static std::mutex g_scratch_mutex;   // contexts may be created from several threads at once
 
 // Address of `scratch` on `device` (which must be the current device), looked up once.
 static hipError_t mh_static_scratch(int device, void **ptr) {
   if (device < 0 || device >= MH_MAX_DEVICES) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
   if (!g_scratch_ptr[device]) {
     void *p = nullptr;
     const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
@@ -173,7 +176,10 @@ int mace_hip_ctx_create(int device, mace_hip_ctx **out) {
   } else {
     (void)hipGetLastError();
   }
-  ctx->big_lds_kernels.reserve(128);   // so that raising a kernel's LDS limit never reallocates
+  // so that raising a kernel's LDS limit or asking for its occupancy never reallocates (host
+  // memory either: the allocation-free entry point allocates nothing at all)
+  ctx->big_lds_kernels.reserve(128);
+  ctx->occupancy.reserve(256);
   ctx->stream = ctx->own_stream;
   ctx->cu_count = prop.multiProcessorCount;
   ctx->lds_bytes = (int)prop.sharedMemPerBlock;

@@ -78,3 +78,44 @@ def test_noalloc_rejects_what_does_not_fit():
         run_pair(ctx, 1, 200, 1100, 300, Cm, R, R, 5, check_oracle=True)
     finally:
         ctx.close()
+
+
+def test_noalloc_allocates_nothing():
+    """The property the entry point exists for.  On a fresh context (whose own arena is still
+    empty) the free device memory the runtime reports is the same after a series of noalloc calls
+    as before -- the arena did not grow, no panel was built for the weight cache although an
+    operand of the calls is a registered weight -- and then it does shrink when the allocating
+    entry point runs the same shape, which shows that the probe sees such allocations."""
+    import ctypes as C
+    import torch
+
+    ctx = mh.Context(0)
+    try:
+        rng = np.random.default_rng(11)
+        rows, depth, cols = 1024, 2048, 1536
+        l = rng.integers(0, 256, rows * depth, dtype=np.uint8)
+        r = rng.integers(0, 256, depth * cols, dtype=np.uint8)
+        d = Dev()
+        dl, dr = d.put(l), d.put(r)
+        t, po = d.empty(rows * cols, np.uint8)
+        ctx.call("mace_hip_weight_register", dr, r.size)     # the cache would allocate a panel for it
+        mult, e = orc.quantize_multiplier(1e-5)
+        tail = (R, 1, rows, depth, cols, 1, 1, -128, -127, None, mult, -e, 128, 0, 255)
+        builds, hits = C.c_int64(), C.c_int64()
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
+        for lo, ro in ((Cm, R), (R, R), (R, Cm), (Cm, R)):    # repacks of either side, in place
+            ctx.call("mace_hip_gemm_q8_u8_noalloc", dl, lo, dr, ro, po, *tail)
+            assert ctx.last_plan().launches >= 1
+        ctx.sync()
+        assert torch.cuda.mem_get_info()[0] == free_before
+        ctx.call("mace_hip_weight_cache_stats", C.byref(builds), C.byref(hits))
+        assert (builds.value, hits.value) == (0, 0)
+        ctx.call("mace_hip_gemm_q8_u8", dl, Cm, dr, R, po, *tail)     # arena + cached panel: allocates
+        ctx.sync()
+        ctx.call("mace_hip_weight_cache_stats", C.byref(builds), C.byref(hits))
+        assert builds.value == 1
+        assert torch.cuda.mem_get_info()[0] < free_before
+        ctx.call("mace_hip_weight_unregister", dr)
+    finally:
+        ctx.close()
