@@ -56,6 +56,9 @@ def load_probes():
                                          C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float,
                                          C.c_float, C.c_int, C.c_void_p, C.c_int,
                                          C.POINTER(C.c_double)]
+    lib.mace_probe_gemv_host_loop.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
+                                              C.c_int, C.c_int, C.c_float, C.c_float, C.c_float, C.c_int,
+                                              C.c_void_p, C.c_int, C.POINTER(C.c_double)]
     return lib
 
 
@@ -130,6 +133,18 @@ def main():
                  out8.data_ptr(), mh.ROW_MAJOR, 1, n, n, n, 1, 1, -za, -zb, None, mult, shift, zc,
                  0, 255)
 
+    # What a caller sees who starts from an idle board: the plain warm-up and the same number of
+    # timed steps, before any run-in (reported beside the settled figure, never as it).
+    for _ in range(args.warmup):
+        step()
+    ctx.sync()
+    ctx.timer_start()
+    for _ in range(args.steps):
+        step()
+    cold_ms_per_step = ctx.timer_stop() / args.steps
+    gemm_plan = ctx.last_plan()     # the kernel this step runs, as the library itself reports it
+    log("from idle (no run-in): %.3f ms/step" % cold_ms_per_step)
+
     # Bring the board to its sustained clocks first: after idling, the first ~3 launches run at
     # boost, the next ~50 are throttled hard (the kernel takes up to 30 % longer) and only then
     # does the power controller settle.  Untimed, like the warm-up; the timed region is exactly
@@ -180,6 +195,7 @@ def main():
         "metric": METRIC, "value": round(value, 2), "unit": "TOPS", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "settle_steps": settle_steps,
         "ms_per_step": round(ms_per_step, 4),
+        "cold_ms_per_step": round(cold_ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8",
         "data": "synthetic",
         "config": {"workload": "q8_matmul_%dx%dx%d_u8out" % (n, n, n), "M": n, "N": n, "K": n,
@@ -191,7 +207,7 @@ def main():
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_INT8_TOPS,
                      "unit": "TOP/s", "frac": round(achieved / PEAK_INT8_TOPS, 4),
                      "traffic": measured_traffic("q8_gemm_%d" % n), "traffic_unit": "B/launch",
-                     "kernel": "q8_gemm_dma_kernel<2,2,4,4,2,uint8_t,1,false,false,128,false,true,false>",
+                     "kernel": gemm_plan.kernel, "launches_per_step": gemm_plan.launches,
                      "kernel_ms_avg": round(k_avg, 4), "kernel_ms_min": round(min(kms), 4),
                      "kernel_ms_max": round(max(kms), 4),
                      "timing": "one HIP event pair per launch, recorded inside the timed region",
@@ -270,6 +286,7 @@ def main():
                     raise RuntimeError("probe returned %d" % rc)
                 ceil[name + "_TOPS"] = round(tops.value, 1)
             ceil["achieved_over_random_ceiling"] = round(achieved / ceil["random_operands_TOPS"], 4)
+            result["roofline"]["frac_of_random_mfma_ceiling"] = ceil["achieved_over_random_ceiling"]
             ceil["what"] = ("v_mfma_i32_32x32x32_i8 alone, 16 accumulators per wavefront, one "
                             "workgroup of 4 wavefronts per CU, no LDS or memory traffic")
             result["roofline"]["mfma_only_probe"] = ceil
@@ -284,10 +301,16 @@ def main():
         result["gemv"] = bench_gemv(ctx, mh, torch, args)
     if not args.no_other:
         result["other_configs"] = bench_other(ctx, mh, torch)
+        result["host_pointer_calls"] = bench_host_pointers(ctx, mh, np)
+        chain = bench_c4_net()
+        if chain is not None:
+            result["other_configs"].append(chain)
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(np, torch, A, B, out8, n, za, zb, zc, mult, shift,
                                               args.cpu_rows, rhs_order)
+        if not args.no_other:
+            result["cpu_baseline"]["other_configs"] = cpu_baselines_other(np)
     ctx.close()
     print(json.dumps(result), flush=True)
 
@@ -298,6 +321,7 @@ def bench_gemv(ctx, mh, torch, args):
     H = W = 4096
     nbuf = 40                                    # 40 x 16 MiB = 640 MiB > 256 MiB last-level cache
     probes = load_probes()
+    kernels = {}
     g = torch.Generator(device="cuda").manual_seed(3)
     weights = torch.randint(0, 256, (nbuf, H, W), dtype=torch.uint8, device="cuda", generator=g)
     bias = torch.randint(-2 ** 15, 2 ** 15, (H,), dtype=torch.int32, device="cuda", generator=g)
@@ -316,12 +340,13 @@ def bench_gemv(ctx, mh, torch, args):
         xptr, bptr, yptr = x.data_ptr(), bias.data_ptr(), y.data_ptr()
         ctx.call("mace_hip_gemv_q8_u8", wptr[0], xptr, bptr, batch, H, W, 0, 1, 127, 128, 0.01, 0.02,
                  1.75, 128, mh.REQUANT_NEON, yptr)      # once through the checking wrapper
+        kernels[batch] = ctx.last_plan().kernel
 
         def call(i):
             fn(ctx.handle, wptr[i], xptr, bptr, batch, H, W, 0, 1, 127, 128, 0.01, 0.02, 1.75, 128,
                mh.REQUANT_NEON, yptr)
 
-        res = {"bytes_per_launch": nbytes}
+        res = {"bytes_per_launch": nbytes, "kernel": kernels[batch]}
         stride = H * W
         for name, rotate in (("hbm", True), ("cache_resident", False)):
             for i in range(nbuf):
@@ -382,11 +407,42 @@ def bench_gemv(ctx, mh, torch, args):
                                                    hb["back_to_back_us"], 4),
                        "traffic": measured_traffic("q8_gemv_4096x4096_b1"),
                        "traffic_unit": "B/launch",
-                       "kernel": "q8_gemv_row_kernel<4,false,true,uint8_t>",
+                       "kernel": kernels[1],
                        "timing": "400 back-to-back launches between two HIP events, rotating "
                                  "over 640 MiB of weights"}
     log("read probe: %.2f us per launch -> %.0f GB/s; gemv batch 1 at %.1f%% of it"
         % (best, pbytes / (best * 1e-6) / 1e9, 100 * best / hb["back_to_back_us"]))
+    del weights
+    # The fraction of the HBM peak against the size of the matrix, batch 1 and 8: back-to-back
+    # launches from C, weights rotating over a set larger than the last-level cache.
+    curve = []
+    for n in (4096, 8192, 16384):
+        nb = max(3, (640 << 20) // (n * n))
+        wts = torch.randint(0, 256, (nb, n, n), dtype=torch.uint8, device="cuda", generator=g)
+        bias_n = torch.randint(-2 ** 15, 2 ** 15, (n,), dtype=torch.int32, device="cuda", generator=g)
+        for batch in (1, 8):
+            x = torch.randint(0, 256, (batch, n), dtype=torch.uint8, device="cuda", generator=g)
+            y = torch.empty((batch, n), dtype=torch.uint8, device="cuda")
+            torch.cuda.synchronize()
+            us = C.c_double(0.0)
+            best = None
+            for _ in range(3):
+                rc = probes.mace_probe_gemv_loop(ctx.handle, wts.data_ptr(), n * n, nb, x.data_ptr(),
+                                                 bias_n.data_ptr(), batch, n, n, 0.01, 0.02,
+                                                 1.75 * (n / 4096) ** 0.5, 128, y.data_ptr(), 10 * nb,
+                                                 C.byref(us))
+                if rc != 0:
+                    raise RuntimeError("gemv loop returned %d: %s" % (rc, ctx.last_error()))
+                best = us.value if best is None else min(best, us.value)
+            nbytes = n * n + batch * n + 4 * n + batch * n
+            gbs = nbytes / (best * 1e-6) / 1e9
+            curve.append({"H": n, "W": n, "batch": batch, "us_per_launch": round(best, 3),
+                          "GBps": round(gbs, 1), "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBS, 4),
+                          "kernel": ctx.last_plan().kernel})
+            log("gemv %d x %d batch %d: %.2f us -> %.0f GB/s (%.1f%%)" % (n, n, batch, best, gbs,
+                                                                        100 * gbs / PEAK_HBM_GBS))
+        del wts
+    out["size_curve"] = curve
     return out
 
 
@@ -655,6 +711,197 @@ def bench_other(ctx, mh, torch):
                     "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBS, 4)})
     for o in out:
         log("other:", json.dumps(o))
+    return out
+
+
+def bench_host_pointers(ctx, mh, np):
+    """What the documented drop-in costs per call: the *_host entry points on tensors in host
+    memory (synchronous: operands staged, kernel, result copied back), with the constant operands
+    staged on every call and with them registered as resident (mace_hip_host_weight_register, what
+    the adapter does for is_weight() tensors), beside the device-pointer call on resident tensors.
+    Wall-clock time per call on the host."""
+    import torch
+    probes = load_probes()
+    rng = np.random.default_rng(3)
+    out = []
+    H = W = 4096
+    wt = rng.integers(0, 256, (H, W), dtype=np.uint8)
+    bias = rng.integers(-2 ** 15, 2 ** 15, H).astype(np.int32)
+    dwt, dbias = torch.from_numpy(wt).cuda(), torch.from_numpy(bias).cuda()
+    for batch in (1, 8):
+        x = rng.integers(0, 256, (batch, W), dtype=np.uint8)
+        y = np.empty((batch, H), np.uint8)
+        dx = torch.from_numpy(x).cuda()
+        dy = torch.empty((batch, H), dtype=torch.uint8, device="cuda")
+        torch.cuda.synchronize()
+        entry = {"workload": "q8_fully_connected_4096x4096_b%d" % batch}
+        us = C.c_double(0.0)
+
+        def host_loop(calls):
+            rc = probes.mace_probe_gemv_host_loop(ctx.handle, wt.ctypes.data, x.ctypes.data, bias.ctypes.data,
+                                                  batch, H, W, 0.01, 0.02, 1.75, 128, y.ctypes.data, calls,
+                                                  C.byref(us))
+            if rc != 0:
+                raise RuntimeError("host gemv loop returned %d: %s" % (rc, ctx.last_error()))
+            return us.value
+
+        entry["host_pointers_weights_staged_us"] = round(host_loop(10), 1)
+        ctx.call("mace_hip_host_weight_register", wt.ctypes.data, wt.size)
+        ctx.call("mace_hip_host_weight_register", bias.ctypes.data, bias.nbytes)
+        entry["host_pointers_weights_resident_us"] = round(min(host_loop(200) for _ in range(3)), 1)
+        got = y.copy()
+        ctx.call("mace_hip_host_weight_unregister", wt.ctypes.data)
+        ctx.call("mace_hip_host_weight_unregister", bias.ctypes.data)
+        # the device-pointer call followed by a wait, i.e. the same synchronous contract
+        fn, sync = ctx.lib.mace_hip_gemv_q8_u8, ctx.lib.mace_hip_sync
+        args = (ctx.handle, dwt.data_ptr(), dx.data_ptr(), dbias.data_ptr(), batch, H, W, 0, 1, 127, 128,
+                0.01, 0.02, 1.75, 128, mh.REQUANT_NEON, dy.data_ptr())
+        for _ in range(20):
+            fn(*args)
+            sync(ctx.handle)
+        t0 = time.perf_counter()
+        for _ in range(500):
+            fn(*args)
+            sync(ctx.handle)
+        entry["device_pointers_call_and_wait_us"] = round((time.perf_counter() - t0) / 500 * 1e6, 1)
+        entry["resident_over_device"] = round(entry["host_pointers_weights_resident_us"] /
+                                              entry["device_pointers_call_and_wait_us"], 2)
+        if not np.array_equal(got, dy.cpu().numpy()):
+            log("ERROR: host-pointer and device-pointer results differ")
+            sys.exit(3)
+        out.append(entry)
+    # configuration 1 through the host-pointer MatMul entry point, B constant
+    A = rng.integers(0, 256, (128, 256), dtype=np.uint8)
+    B = rng.integers(0, 256, (256, 128), dtype=np.uint8)
+    Cq = np.empty((128, 128), np.uint8)
+    mult, shift = mh.get_output_multiplier_and_shift(0.02, 0.015, 0.05)
+    fn = ctx.lib.mace_hip_gemm_q8_u8_host
+    args = (ctx.handle, A.ctypes.data, 0, B.ctypes.data, 0, Cq.ctypes.data, 0, 1, 128, 256, 128, 1, 1, -128,
+            -128, None, mult, shift, 128, 0, 255)
+    entry = {"workload": "q8_matmul_128x256x128"}
+    for key, resident in (("host_pointers_weights_staged_us", False), ("host_pointers_weights_resident_us", True)):
+        if resident:
+            ctx.call("mace_hip_host_weight_register", B.ctypes.data, B.size)
+        for _ in range(20):
+            ctx.check(fn(*args))
+        t0 = time.perf_counter()
+        for _ in range(300):
+            fn(*args)
+        entry[key] = round((time.perf_counter() - t0) / 300 * 1e6, 1)
+        if resident:
+            ctx.call("mace_hip_host_weight_unregister", B.ctypes.data)
+    out.append(entry)
+    for o in out:
+        log("host pointers:", json.dumps(o))
+    return out
+
+
+def bench_c4_net():
+    """Benchmark configuration 4's five layers inside a NetDef through the serial runner (Quantize ->
+    Conv2D 1x1 with a ReLU6 range -> Dequantize per layer, fifteen ops), at batch 64, eagerly and as
+    a replayed HIP graph, each compared with the oracle's chain.  The runner is C++
+    (include/mace_hip_net.h): its test binary times the net and prints one JSON line."""
+    import subprocess
+    exe = os.path.join(ROOT, "tests", "cpp", "test_net.bin")
+    if not os.path.exists(exe):
+        log("c4 net: tests/cpp/test_net.bin is not built; skipped")
+        return None
+    try:
+        r = subprocess.run([exe, "c4", "64", "timing"], capture_output=True, text=True, timeout=240)
+        line = [ln for ln in r.stdout.splitlines() if ln.startswith("{")][-1]
+        entry = json.loads(line)
+        if r.returncode != 0 or not entry.get("parity"):
+            log("ERROR: the pointwise-layer net differs from the oracle:\n" + r.stdout[-400:])
+            sys.exit(3)
+        log("other:", json.dumps(entry))
+        return entry
+    except (OSError, IndexError, ValueError, subprocess.TimeoutExpired) as ex:
+        log("c4 net skipped: %s" % str(ex)[:120])
+        return None
+
+
+def time_cpu(fn, budget_s=2.5):
+    """Seconds per call of a CPU function by the reference harness's rule (at least 10 iterations,
+    at least 0.5 s: test/ccbenchmark/mace/benchmark_utils/test_benchmark.cc:85-108 in the reference
+    tree) -- cut short, and flagged, where a call is so long that the rule would not fit the
+    benchmark's time limit.  Returns (seconds per call, iterations, rule_met)."""
+    fn()                       # warm the caches, page the operands in
+    t0 = time.perf_counter()
+    fn()
+    one = time.perf_counter() - t0
+    iters = max(10, int(0.5 / max(one, 1e-9)) + 1)
+    met = True
+    if iters * one > budget_s:
+        iters = max(1, int(budget_s / one))
+        met = iters >= 10
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        fn()
+    return (time.perf_counter() - t0) / iters, iters, met
+
+
+def cpu_baselines_other(np):
+    """The CPU oracle (a port of the reference's CPU path) timed on the host cores for the other
+    benchmark configurations, single-threaded as the reference's REF delegators run and row-parallel
+    over the job's cores as its thread pool would split the rows; bounded samples where the whole
+    configuration would take too long (stated per entry)."""
+    from oracle import mace_oracle as orc
+    try:
+        host_cores = len(os.sched_getaffinity(0))
+    except AttributeError:
+        host_cores = os.cpu_count() or 1
+    cores = max(1, min(host_cores, 16))
+    rng = np.random.default_rng(17)
+    out = []
+
+    def entry(workload, code, sample, ops_or_bytes, unit, fn_of_threads):
+        e = {"workload": workload, "code": code, "sample": sample, "host_cores_visible": host_cores}
+        for threads in (1, cores):
+            sec, iters, met = time_cpu(lambda: fn_of_threads(threads))
+            rate = ops_or_bytes / sec / (1e9 if unit == "GB/s" else 1e12)
+            e["threads_%d" % threads] = {"ns_per_iter": round(sec * 1e9), "iterations": iters,
+                                         "rule_10_iters_0.5s_met": met, unit: float("%.4g" % rate)}
+        out.append(e)
+        log("cpu baseline:", json.dumps(e))
+
+    # C1: uint8 MatMul 128 x 256 x 128
+    A = rng.integers(0, 256, (128, 256), dtype=np.uint8)
+    B = rng.integers(0, 256, (256, 128), dtype=np.uint8)
+    m, s_ = orc.get_output_multiplier_and_shift(0.02, 0.015, 0.05)
+    entry("q8_matmul_128x256x128", "orc_q8_gemm_u8 (exact integer GEMM + fixed-point pipeline)", "whole",
+          2.0 * 128 * 256 * 128, "TOPS",
+          lambda t: orc.q8_gemm_u8(A, B, 1, 128, 128, 256, -128, -128, None, m, s_, 128, nthreads=t))
+    # C2: fp32 Gemm, the serial loop of ref/gemm.cc (strided reads of the right-hand matrix make it
+    # slow: a whole 1024^3 batch takes one thread about six seconds), 128 rows of one batch per call
+    L = rng.standard_normal((1, 128, 1024)).astype(np.float32)
+    Rm = rng.standard_normal((1, 1024, 1024)).astype(np.float32)
+    entry("f32_gemm_4x1024^3", "orc_gemm_f32 (ref/gemm.cc:92-102 loop)",
+          "128 of the 1024 rows of one of the four batches (x 32 for the configuration)",
+          2.0 * 128 * 1024 * 1024, "TFLOPS", lambda t: orc.gemm_f32(L, Rm, 1, 128, 1024, 1024, nthreads=t))
+    # C3: uint8 Gemv 4096 x 4096, batch 1 and 8
+    W = rng.integers(0, 256, (4096, 4096), dtype=np.uint8)
+    bias = rng.integers(-2 ** 15, 2 ** 15, 4096).astype(np.int32)
+    for batch in (1, 8):
+        x = rng.integers(0, 256, (batch, 4096), dtype=np.uint8)
+        nbytes = 4096 * 4096 + batch * 4096 * 2 + 4 * 4096
+        entry("q8_gemv_4096x4096_b%d" % batch, "orc_q8_gemv_u8 (arm/q8/gemv.cc flavour)", "whole", nbytes, "GB/s",
+              lambda t: orc.q8_gemv_u8(W, x, bias, batch, 4096, 4096, 127, 128, 0.01, 0.02, 1.75, 128,
+                                       orc.REQUANT_NEON, nthreads=t))
+    # C4: 56 x 56 x 128 -> 128 at batch 64 would take a single thread tens of seconds: 4 images
+    n = 4
+    xin = rng.integers(0, 256, (n, 56, 56, 128), dtype=np.uint8)
+    f = rng.integers(0, 256, (128, 128), dtype=np.uint8)
+    b4 = rng.integers(-2 ** 15, 2 ** 15, 128).astype(np.int32)
+    entry("q8_conv1x1_56x56x128_to_128", "orc_conv1x1_q8_nhwc", "4 of the 64 images (x 16 for the configuration)",
+          2.0 * n * 56 * 56 * 128 * 128, "TOPS",
+          lambda t: orc.conv1x1_q8_nhwc(xin, f, b4, n, 56, 56, 128, 128, 0.02, 128, 0.01, 127, 0.0002, 0.05, 0,
+                                        nthreads=t))
+    # C5: 2048^3 by 256 rows of A
+    A2 = rng.integers(0, 256, (256, 2048), dtype=np.uint8)
+    B2 = rng.integers(0, 256, (2048, 2048), dtype=np.uint8)
+    entry("q8_matmul_2048^3", "orc_q8_gemm_u8", "256 of the 2048 rows of A (x 8 for the configuration)",
+          2.0 * 256 * 2048 * 2048, "TOPS",
+          lambda t: orc.q8_gemm_u8(A2, B2, 1, 256, 2048, 2048, -131, -122, None, 1 << 30, 12, 128, nthreads=t))
     return out
 
 

@@ -19,6 +19,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <chrono>
+
 #include "mace_hip.h"
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -150,6 +152,30 @@ int mace_probe_gemv_loop(mace_hip_ctx *ctx, const void *weights, int64_t stride,
   float ms = 0.f;
   if (mace_hip_timer_stop(ctx, &ms) != MACE_HIP_SUCCESS) return 3;
   *us_per_launch = (double)ms * 1e3 / launches;
+  return 0;
+}
+
+// `calls` synchronous calls of mace_hip_gemv_q8_u8_host (host pointers in, result back in host
+// memory when the call returns) timed by the host's clock: what a caller holding MACE's CPU
+// tensors sees per FullyConnected, transfers included.  Whether the weights are staged on every
+// call or found resident depends on mace_hip_host_weight_register, which the caller of this probe
+// does or does not do beforehand.
+int mace_probe_gemv_host_loop(mace_hip_ctx *ctx, const void *weights, const void *x, const void *bias,
+                              int batch, int H, int W, float lhs_scale, float rhs_scale, float out_scale,
+                              int out_zp, void *out, int calls, double *us_per_call) {
+  if (!ctx || !weights || !us_per_call || calls <= 0) return 1;
+  auto call = [&]() {
+    return mace_hip_gemv_q8_u8_host(ctx, (const uint8_t *)weights, (const uint8_t *)x, (const int32_t *)bias,
+                                    batch, H, W, 0, 1, 127, 128, lhs_scale, rhs_scale, out_scale, out_zp,
+                                    MACE_HIP_REQUANT_NEON, (uint8_t *)out);
+  };
+  for (int i = 0; i < 3; ++i)
+    if (call() != MACE_HIP_SUCCESS) return 2;
+  const auto t0 = std::chrono::steady_clock::now();
+  for (int i = 0; i < calls; ++i)
+    if (call() != MACE_HIP_SUCCESS) return 2;
+  const auto t1 = std::chrono::steady_clock::now();
+  *us_per_call = std::chrono::duration<double, std::micro>(t1 - t0).count() / calls;
   return 0;
 }
 
