@@ -23,7 +23,7 @@ const int kVariantCount[MACE_HIP_KF_COUNT] = {
     32,                       // Q8_GEMV_ROW
     6,                        // Q8_GEMV_SLICE
     2,                        // Q8_GEMV_MFMA_LDS
-    2,                        // Q8_GEMV_MFMA
+    6,                        // Q8_GEMV_MFMA
     8,                        // Q8_GEMV_ROWS
     16,                       // Q8_GEMV_GENERAL
     8,                        // F32_GEMM_VEC
@@ -163,7 +163,7 @@ int mace_hip_plan_describe(int family, int v, char *buf, size_t len) {
       snprintf(buf, len, "%s<16,%s>", k, out_name(v & 1));
       break;
     case MACE_HIP_KF_Q8_GEMV_MFMA:
-      snprintf(buf, len, "%s<%s>", k, out_name(v & 1));
+      snprintf(buf, len, "%s<NW=%d,GROUP=2,NBUF=4,%s>", k, 4 << (v >> 1), out_name(v & 1));
       break;
     case MACE_HIP_KF_Q8_GEMV_ROWS:
       snprintf(buf, len, "%s<R=1,NB=%d,NWAVES=16,%s>", k, 1 << (v >> 1), out_name(v & 1));

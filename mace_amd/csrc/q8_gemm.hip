@@ -172,8 +172,28 @@ __device__ __forceinline__ void requant_16_by_table(const int32_t (&v)[16], cons
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     uint32_t o[4];
+#if defined(__HIP_DEVICE_COMPILE__)
+    // o = out + (v > limit), four at a time: the compares first, each into a lane mask of its own,
+    // then the four additions with the mask as carry.  A compare's mask cannot be consumed by the
+    // very next instructions (the compiler, left alone, reuses one mask register and waits
+    // between every compare and its addition).
+    uint64_t m0, m1, m2, m3;
+    asm("v_cmp_gt_i32_e64 %4, %8, %12\n\t"
+        "v_cmp_gt_i32_e64 %5, %9, %13\n\t"
+        "v_cmp_gt_i32_e64 %6, %10, %14\n\t"
+        "v_cmp_gt_i32_e64 %7, %11, %15\n\t"
+        "v_addc_co_u32_e64 %0, %4, 0, %16, %4\n\t"
+        "v_addc_co_u32_e64 %1, %5, 0, %17, %5\n\t"
+        "v_addc_co_u32_e64 %2, %6, 0, %18, %6\n\t"
+        "v_addc_co_u32_e64 %3, %7, 0, %19, %7"
+        : "=&v"(o[0]), "=&v"(o[1]), "=&v"(o[2]), "=&v"(o[3]), "=&s"(m0), "=&s"(m1), "=&s"(m2), "=&s"(m3)
+        : "v"(v[4 * q]), "v"(v[4 * q + 1]), "v"(v[4 * q + 2]), "v"(v[4 * q + 3]), "v"(e[4 * q].x),
+          "v"(e[4 * q + 1].x), "v"(e[4 * q + 2].x), "v"(e[4 * q + 3].x), "v"(e[4 * q].y),
+          "v"(e[4 * q + 1].y), "v"(e[4 * q + 2].y), "v"(e[4 * q + 3].y));
+#else
 #pragma unroll
     for (int i = 0; i < 4; ++i) o[i] = (uint32_t)(e[4 * q + i].y + (v[4 * q + i] > e[4 * q + i].x ? 1 : 0));
+#endif
     // bytes 0 of o[0..3] side by side (v_perm_b32: selector 0..3 = bytes of the second operand,
     // 4..7 of the first, 0x0c = zero)
     const uint32_t p10 = __builtin_amdgcn_perm(o[1], o[0], 0x0c0c0400u);
@@ -2412,6 +2432,8 @@ int launch_gemm_xres(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, 
     // workgroups along y: as many as are resident at once -- up to three per CU where registers
     // and LDS allow (two against three: 56x56x128 -> 128 at batch 64 19.2 -> 18.6 us, 28x28x256 ->
     // 256 16.4 -> 15.2)
+    // (Fewer workgroups so that every wavefront walks the same number of blocks -- 523 instead of
+    // 768 for 6272 blocks -- measured slower, 22.7 against 19.8 us; so did a few more than fit.)
     const int per_cu = std::max(1, std::min(3, mh_blocks_per_cu(ctx, (const void *)k, 256, lds)));
     const int slots = std::max(1, cu * per_cu / std::max(1, tiles_x * batch));
     const int wgs = std::max(1, std::min(need, slots));

@@ -392,22 +392,30 @@ __global__ __launch_bounds__(1024) void q8_gemv_row_kernel(
 // partial 16 x 16 results meet in LDS (integer atomics: the order does not matter).
 typedef int gv4i __attribute__((ext_vector_type(4)));
 
-template <typename OutT>
-__global__ __launch_bounds__(256) void q8_gemv_mfma_kernel(GemvParams p) {
-  constexpr int NBMAX = 15, ONES_COL = 15, STEPS = 16;   // k steps in flight per wavefront
+// NW wavefronts share a block of 16 rows, each on a contiguous share of the k steps, walked as a
+// ring of NBUF groups of GROUP steps: while one group is multiplied the loads of the other
+// NBUF - 1 are on their way, and the group just consumed is requested again, NBUF groups ahead,
+// before the next one is touched.  (Burst-wise loading -- 16 steps requested, all awaited, all
+// multiplied -- ran at 3.4 TB/s at 8192 x 8192 against 8 vectors; this at 4.0.  Groups of 2 to 8
+// steps, rings of 2 to 8, 4 to 16 wavefronts and 32 rows per workgroup all lie within 5 % of each
+// other; what is left is the vectors' traffic, re-read from L2 by every workgroup.)
+template <int NW, int GROUP, int NBUF, typename OutT>
+__global__ __launch_bounds__(NW * 64) void q8_gemv_mfma_kernel(GemvParams p) {
+  constexpr int NBMAX = 15, ONES_COL = 15;
   __shared__ int32_t s_acc[16][17];
   __shared__ int32_t s_sx[16];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, q = lane >> 4;
   const int h0 = blockIdx.x * 16;
   const int b0 = blockIdx.y * NBMAX;
   const int nb = min(NBMAX, p.batch - b0);
   const int nchunk = p.W >> 4;
   const int nstep = (nchunk + 3) >> 2;
-  const int per_wave = (nstep + 3) >> 2;
+  const int per_wave = (nstep + NW - 1) / NW;
   const int ks0 = wave * per_wave, ks1 = min(nstep, ks0 + per_wave);
 
-  for (int i = tid; i < 16 * 17; i += 256) (&s_acc[0][0])[i] = 0;
+  for (int i = tid; i < 16 * 17; i += NW * 64) (&s_acc[0][0])[i] = 0;
   if (tid < 16) s_sx[tid] = 0;
 
   const uint8_t *arow = p.lhs + (int64_t)min(h0 + r, p.H - 1) * p.W;
@@ -418,40 +426,70 @@ __global__ __launch_bounds__(256) void q8_gemv_mfma_kernel(GemvParams p) {
   const gv4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
   const gv4i other = r == ONES_COL ? ones : zero;
 
-  gv4i acc = zero;
-  int sx = 0;
-  for (int ks = ks0; ks < ks1; ks += STEPS) {
-    gv4i a[STEPS], x[STEPS];
+  gv4i acc[2] = {zero, zero};
+  uint32_t sx_raw = 0;   // the vector's bytes as read, 128 too much each
+  int sx_bytes = 0;
+  // steps past the wavefront's share or the end of the row re-read the row's last chunk (masked
+  // when multiplied)
+  auto fetch = [&](gv4i (&a)[GROUP], gv4i (&x)[GROUP], int ks) {
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int u = 0; u < STEPS; ++u) {
-      const int c = min(4 * (ks + u) + q, nchunk - 1);
+    for (int u = 0; u < GROUP; ++u) {
+      const int c = min(4 * min(ks + u, ks1 - 1) + q, nchunk - 1);
       a[u] = __builtin_nontemporal_load((const gv4i *)(arow + (int64_t)c * 16));
     }
 #pragma unroll
-    for (int u = 0; u < STEPS; ++u) {
-      const int c = min(4 * (ks + u) + q, nchunk - 1);
-      x[u] = flip;
-      if (is_x) x[u] = *(const gv4i *)(xrow + (int64_t)c * 16);
+    for (int u = 0; u < GROUP; ++u) {
+      // (every lane loads: columns past the batch re-read the last vector and are replaced below;
+      // a load under a lane mask would cost a branch each)
+      const int c = min(4 * min(ks + u, ks1 - 1) + q, nchunk - 1);
+      x[u] = *(const gv4i *)(xrow + (int64_t)c * 16);
     }
+    // the group's loads stay together: one of them issued late, among the other group's, would
+    // make this group's last step wait for those as well (loads return in order)
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto multiply = [&](const gv4i (&a)[GROUP], const gv4i (&x)[GROUP], int ks) {
 #pragma unroll
-    for (int u = 0; u < STEPS; ++u) {
+    for (int u = 0; u < GROUP; ++u) {
       const bool valid = (ks + u < ks1) && (4 * (ks + u) + q < nchunk);
-      const gv4i av = valid ? (a[u] ^ flip) : zero;
       gv4i xv = is_x ? (x[u] ^ flip) : other;
       if (!valid) xv = zero;
-      if (is_x) {
-        sx = __builtin_amdgcn_sdot4(xv.x, 0x01010101, sx, false);
-        sx = __builtin_amdgcn_sdot4(xv.y, 0x01010101, sx, false);
-        sx = __builtin_amdgcn_sdot4(xv.z, 0x01010101, sx, false);
-        sx = __builtin_amdgcn_sdot4(xv.w, 0x01010101, sx, false);
+      if (is_x && valid) {
+        // v_sad_u8: a dot-product instruction would not run beside the MFMAs
+        sx_raw = __builtin_amdgcn_sad_u8((uint32_t)x[u].x, 0u, sx_raw);
+        sx_raw = __builtin_amdgcn_sad_u8((uint32_t)x[u].y, 0u, sx_raw);
+        sx_raw = __builtin_amdgcn_sad_u8((uint32_t)x[u].z, 0u, sx_raw);
+        sx_raw = __builtin_amdgcn_sad_u8((uint32_t)x[u].w, 0u, sx_raw);
+        sx_bytes += 16;
       }
-      acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, xv, acc, 0, 0, 0);
+      const gv4i av = valid ? (a[u] ^ flip) : zero;
+      acc[u & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, xv, acc[u & 1], 0, 0, 0);
     }
+  };
+  if (ks0 < ks1) {   // uniform over the wavefront
+    gv4i a[NBUF][GROUP], x[NBUF][GROUP];
+#pragma unroll
+    for (int g = 0; g < NBUF; ++g) fetch(a[g], x[g], ks0 + g * GROUP);
+    // No fetch sits under a condition: the wait counts in front of each group then leave the
+    // other groups' loads in flight.  (The last fetches of the loop may lie wholly past the share:
+    // they re-read one chunk.)
+    int ks = ks0;
+    for (; ks + NBUF * GROUP < ks1; ks += NBUF * GROUP) {
+#pragma unroll
+      for (int g = 0; g < NBUF; ++g) {
+        multiply(a[g], x[g], ks + g * GROUP);
+        fetch(a[g], x[g], ks + (NBUF + g) * GROUP);
+      }
+    }
+#pragma unroll
+    for (int g = 0; g < NBUF; ++g) multiply(a[g], x[g], ks + g * GROUP);
   }
+  const int sx = (int)sx_raw - 128 * sx_bytes;
   __syncthreads();   // the zeroed LDS is visible
   // result register i of lane l: row 4 (l / 16) + i, column l % 16
 #pragma unroll
-  for (int i = 0; i < 4; ++i) atomicAdd(&s_acc[4 * q + i][r], acc[i]);
+  for (int i = 0; i < 4; ++i) atomicAdd(&s_acc[4 * q + i][r], acc[0][i] + acc[1][i]);
   if (is_x) atomicAdd(&s_sx[r], sx);
   __syncthreads();
 
@@ -737,16 +775,23 @@ int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
       else if (spw == 2) MH_SLICE_LAUNCH(2);
       else MH_SLICE_LAUNCH(4);
 #undef MH_SLICE_LAUNCH
-    } else if (lds <= lds_max && p.W >= 1024) {
+    } else if (lds <= lds_max && p.W >= 1024 && (int)grid.x <= ctx->cu_count) {
       auto k = q8_gemv_mfma_lds_kernel<16, OutT>;
       if (lds > 48 * 1024) MH_HIP(ctx, mh_allow_big_lds(ctx, (const void *)k, lds));
       mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMV_MFMA_LDS, mhv::gemv_out(out_u8), grid, dim3(1024), lds);
       MH_PROF_BEGIN(ctx);
       MH_KLAUNCH(ctx, k, grid, dim3(1024), lds, ctx->stream, p, pitch);
     } else {
-      mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMV_MFMA, mhv::gemv_out(out_u8), grid, block, 0);
+      // eight wavefronts per block of 16 rows once there are four blocks per CU and more
+      // (16384 x 16384: 57.5 against 61.3 us; 4096 x 9216: 13.2 against 11.7)
+      // and sixteen where the blocks of rows reach a quarter of the CUs at most: the bytes in
+      // flight per CU are then all that keeps the few busy CUs fed
+      const int nw = (int)grid.x >= 4 * ctx->cu_count ? 8 : ((int)grid.x * 4 <= ctx->cu_count ? 16 : 4);
+      mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMV_MFMA, mhv::gemv_mfma(nw, out_u8), grid, dim3(nw * 64), 0);
       MH_PROF_BEGIN(ctx);
-      MH_KLAUNCH(ctx, q8_gemv_mfma_kernel<OutT>, grid, block, 0, ctx->stream, p);
+      if (nw == 8) MH_KLAUNCH(ctx, (q8_gemv_mfma_kernel<8, 2, 4, OutT>), grid, dim3(512), 0, ctx->stream, p);
+      else if (nw == 16) MH_KLAUNCH(ctx, (q8_gemv_mfma_kernel<16, 2, 4, OutT>), grid, dim3(1024), 0, ctx->stream, p);
+      else MH_KLAUNCH(ctx, (q8_gemv_mfma_kernel<4, 2, 4, OutT>), grid, dim3(256), 0, ctx->stream, p);
     }
     MH_PROF_END(ctx);
     MH_LAUNCH_CHECK(ctx);

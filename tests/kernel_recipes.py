@@ -125,6 +125,10 @@ def candidates():
                         for u8 in (1, 0):
                             yield {"kind": "gemv", "batch": b, "H": H, "W": W, "lb": lb, "off": off,
                                    "u8": u8}, (b if lb else 1) * H * W / 1e9 + off
+    # the wide-row kernel's forms for many and for a middling number of blocks of 16 rows
+    for u8 in (1, 0):
+        yield {"kind": "gemv", "batch": 3, "H": 16400, "W": 4608, "lb": 0, "off": 0, "u8": u8}, 0.5
+        yield {"kind": "gemv", "batch": 3, "H": 1100, "W": 9216, "lb": 0, "off": 0, "u8": u8}, 0.1
     for m in (4, 31, 64, 300, 1024, 2304):
         for n in (4, 31, 64, 300, 1024, 2304):
             for k in (0, 16, 100, 256):

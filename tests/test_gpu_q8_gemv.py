@@ -166,7 +166,11 @@ FAMILY_CASES = [  # batch, h, w, lhs batched, kernel (without the output type)
     (5, 77, 2048, False, "q8_gemv_mfma_slice_kernel<SPW=2"),
     (15, 33, 1024, False, "q8_gemv_mfma_slice_kernel<SPW=1"),
     (3, 45, 8192, False, "q8_gemv_mfma_lds_kernel<16"),
-    (8, 45, 9216, False, "q8_gemv_mfma_kernel<"),
+    (8, 45, 9216, False, "q8_gemv_mfma_kernel<NW=16,GROUP=2,NBUF=4"),
+    (15, 45, 9232, False, "q8_gemv_mfma_kernel<NW=16,GROUP=2,NBUF=4"),   # a ragged last k step
+    (8, 1100, 8208, False, "q8_gemv_mfma_kernel<NW=4,GROUP=2,NBUF=4"),   # shares of 32.25 k steps
+    (4, 4112, 8192, False, "q8_gemv_mfma_kernel<NW=4,GROUP=2,NBUF=4"),   # more row blocks than CUs
+    (3, 16400, 4608, False, "q8_gemv_mfma_kernel<NW=8,GROUP=2,NBUF=4"),
     (2, 77, 4096, False, "q8_gemv_rows_kernel<R=1,NB=2,NWAVES=16"),
     (1, 50, 9216, False, "q8_gemv_rows_kernel<R=1,NB=1,NWAVES=16"),
     (1, 77, 4001, False, "q8_gemv_kernel<NB=1,VEC=false"),

@@ -296,7 +296,7 @@ def test_variant_tables_are_consistent():
         total += len(vs)
         assert not lib.mace_hip_plan_variant_valid(f, n) and not lib.mace_hip_plan_variant_valid(f, -1)
         assert mh.coverage(f, 0) == 0              # nothing is launched by planning
-    assert total == 216
+    assert total == 220
     assert lib.mace_hip_plan_variant_count(0) == 0 and lib.mace_hip_plan_variant_count(mh.KF_COUNT) == 0
 
 
