@@ -571,10 +571,10 @@ def bench_other(ctx, mh, torch):
 
     # beyond the 1x1 shapes: 3x3 convolutions (SAME padding, stride 1); with cin % 64 == 0 the
     # GEMM's loader gathers the patches itself and no im2col matrix is written
-    # (batch 64, and single-image inference: one launch that gathers as it goes; the first entry is
-    # MobileNet's first layer, 224 x 224 x 3 at stride 2)
+    # (batch 64, and single-image inference: one launch that gathers as it goes; 224 x 224 x 3 at
+    # stride 2 is MobileNet's first layer: patches of 27 bytes, the strip kernel)
     for (n, hw, cin, cout, k, st) in ((64, 56, 64, 64, 3, 1), (64, 28, 128, 128, 3, 1),
-                                      (1, 224, 3, 32, 3, 2), (1, 56, 64, 64, 3, 1), (1, 28, 128, 128, 3, 1)):
+                                      (64, 224, 3, 32, 3, 2), (1, 224, 3, 32, 3, 2), (1, 56, 64, 64, 3, 1), (1, 28, 128, 128, 3, 1)):
         oh = (hw + st - 1) // st
         pad = max((oh - 1) * st + k - hw, 0)      # SAME
         x, f = u8(n, hw, hw, cin), u8(cout, k, k, cin)

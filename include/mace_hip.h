@@ -97,7 +97,8 @@ int mace_hip_graph_destroy(mace_hip_ctx *ctx, mace_hip_graph *graph);
  * family on the same shapes (no counterpart in the reference).  Bit 0: the one-launch kernel for
  * small uint8 GEMM / Conv2D calls; bit 1: the kernel that keeps one operand's tile in LDS; bit 2:
  * the eight-wavefront 128 x 128 kernel and the in-place reading of k-major operands; bit 3: the
- * repack that writes a panel already shifted to int8.  0 restores normal dispatch. */
+ * repack that writes a panel already shifted to int8; bit 4: the convolution kernel for patches
+ * of at most 32 bytes.  0 restores normal dispatch. */
 int mace_hip_ctx_set_kernel_mask(mace_hip_ctx *ctx, int mask);
 /* ---- kernel plans (test and measurement hook; no counterpart in the reference) ----------------
  * Which kernel a compute call runs is chosen on the host from the shapes, layouts, alignments and
@@ -130,6 +131,7 @@ enum {
   MACE_HIP_KF_F32_GEMM_FILL,         /* depth 0: the epilogue alone                               */
   MACE_HIP_KF_F32_GEMV_VEC,          /* f32_gemv_vec_kernel                                       */
   MACE_HIP_KF_F32_GEMV_GENERAL,      /* f32_gemv_kernel                                           */
+  MACE_HIP_KF_Q8_CONV_SHORT,         /* q8_conv_short_kernel: patches of at most 32 bytes        */
   MACE_HIP_KF_COUNT
 };
 /* auxiliary passes of a call (bits of mace_hip_plan.aux) */

@@ -116,7 +116,8 @@ struct mace_hip_ctx {
   // still use; freed when the last graph is destroyed or with the context
   std::vector<void *> retired;
 };
-constexpr int MH_MASK_NO_SMALL = 1, MH_MASK_NO_XRES = 2, MH_MASK_NO_MID = 4, MH_MASK_NO_XFLIP = 8;
+constexpr int MH_MASK_NO_SMALL = 1, MH_MASK_NO_XRES = 2, MH_MASK_NO_MID = 4, MH_MASK_NO_XFLIP = 8,
+              MH_MASK_NO_CONV_SHORT = 16;
 
 int mh_fail(mace_hip_ctx *ctx, int code, const char *fmt, ...);
 
@@ -218,6 +219,7 @@ inline int gemv_row(int u, bool batched, bool whole, bool out_u8) {
 }
 inline int gemv_slice(int spw, bool out_u8) { return log2i(spw) * 2 + (out_u8 ? 1 : 0); }
 inline int gemv_out(bool out_u8) { return out_u8 ? 1 : 0; }
+inline int conv_short(int fx) { return log2i(fx); }
 inline int gemv_mfma(int nw, bool out_u8) { return (log2i(nw) - 2) * 2 + (out_u8 ? 1 : 0); }
 inline int gemv_rows(int nb, bool out_u8) { return log2i(nb) * 2 + (out_u8 ? 1 : 0); }
 inline int gemv_general(int nb, bool vec, bool out_u8) {

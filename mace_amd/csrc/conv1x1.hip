@@ -8,7 +8,10 @@
 // moves before the GEMM.  The bias is per result row (= output channel).
 #include <math.h>
 
+#include <algorithm>
+
 #include "common.h"
+#include "q8_requant.h"
 
 namespace {
 
@@ -73,21 +76,223 @@ __global__ __launch_bounds__(256) void q8_im2col_kernel(const uint8_t *in, uint8
   *(uint4 *)(out + p * (int64_t)kp + k0) = v;
 }
 
+
+// ---- convolutions with a short patch (k_h * k_w * cin <= 32 bytes) ------------------------------
+//
+// MobileNet's first layer (3 x 3, 3 channels, stride 2) and its like: a patch is one MFMA k step, so
+// the product is nothing and the call is bound by gathering patches whose channel runs are not
+// made of aligned pieces, by the requantization and by the stores.  A workgroup takes a strip of
+// output rows of one image: it stages the input rows the strip needs in LDS with aligned 4-byte
+// copies -- left / right padding and rows outside the image materialised as zero-point bytes, so
+// the gather never checks bounds -- and its four wavefronts then walk the strip's pixels in blocks
+// of 32.  Lane (pixel r, half h) puts the 16 bytes k = 16 h .. 16 h + 15 of its pixel's patch
+// together from single LDS bytes (k in (kh, kw, channel) order: the k_w * cin bytes of one kh lie
+// side by side in a staged row; bytes past the depth are 0x80, zero after the shift).  The filter
+// stays in registers as MFMA fragments for the whole kernel; the epilogue is the streaming GEMM
+// kernel's (threshold requantization, 16-byte stores).
+struct ConvShortParams {
+  const uint8_t *in, *filter;
+  const int32_t *bias;
+  uint8_t *out;
+  int in_h, in_w, cin, cout, k_h, sh, sw, pt, out_h, out_w;
+  int depth;    // k_h * k_w * cin
+  int run;      // k_w * cin
+  int strip;    // output rows per workgroup
+  int strips;   // strips per image
+  int pitch;    // LDS bytes per staged input row (a multiple of 4)
+  int lead;     // offset of an input row's first byte inside its staged row (a multiple of 4)
+  int gbase;    // lead - pad_left * cin: where output column 0's patches start
+  uint32_t zp4; // the input zero point in all four bytes
+  int32_t xcoef, ycoef, yadd;
+  RequantFixed rq;
+};
+static_assert(sizeof(ConvShortParams) % alignof(RequantTable) == 0, "argument layout");
+
+// (Occupancy 3 in the launch bounds: with at most 170 registers the compiler keeps the MFMA results
+// in ordinary registers, which spares the epilogue a move per output.)
+template <int FX>
+__global__ __launch_bounds__(256, 3) void q8_conv_short_kernel(ConvShortParams p, RequantTable) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  int32_t *s_cx = (int32_t *)lds;                                 // [32 FX]
+  int32_t *s_tab = s_cx + 32 * FX;                                // the comparison table's pairs
+  uint8_t *rows = lds + 128 * FX + MH_REQUANT_PAIRS_BYTES;        // staged input rows
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int h = lane >> 5, r32 = lane & 31;
+  const int img = blockIdx.x / p.strips, strip_i = blockIdx.x - img * p.strips;
+  const int oh0 = strip_i * p.strip;
+  const int nrows = min(p.strip, p.out_h - oh0);
+  const int npix = nrows * p.out_w;
+  const int staged = (nrows - 1) * p.sh + p.k_h;
+  const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+
+  // The strip's input rows go to LDS BATCH dwords per thread at a time: all loads of a turn are
+  // requested before the first is stored, and the first turn's before anything else of the
+  // prologue, so that the filter's and the table's loads travel with them (one load per turn of a
+  // loop would put a dozen memory round trips in front of every workgroup's first block).  No
+  // load sits under a condition: padding and rows outside the image load from a clamped address
+  // and are replaced; a row's last, partial dword is taken from the dword that ends at the row's
+  // end (rows are at least 4 bytes long).
+  constexpr int BATCH = 12;
+  const int row_len = p.in_w * p.cin;
+  const int dpr = p.pitch >> 2;
+  const int ih_first = oh0 * p.sh - p.pt;
+  const int stage_total = staged * dpr;
+  const uint8_t *image = p.in + (int64_t)img * p.in_h * row_len;
+  uint32_t sv[BATCH];
+  int sdst[BATCH], sshift[BATCH];
+  bool sinside[BATCH];
+  auto stage_issue = [&](int base) {
+#pragma unroll
+    for (int u = 0; u < BATCH; ++u) {
+      const int d = min(base + u * 256, stage_total - 1);
+      const int sr = d / dpr, dw = d - sr * dpr;
+      const int ih = ih_first + sr;
+      const int o = dw * 4 - p.lead;   // byte offset inside the input row
+      sinside[u] = (unsigned)ih < (unsigned)p.in_h && o >= 0 && o < row_len;
+      const int oc = min(max(o, 0), row_len - 4);
+      sshift[u] = sinside[u] ? 8 * (o - oc) : 0;   // > 0 for the partial dword at the row's end
+      sdst[u] = base + u * 256 < stage_total ? sr * p.pitch + dw * 4 : -1;
+      __builtin_memcpy(&sv[u], image + (int64_t)min(max(ih, 0), p.in_h - 1) * row_len + oc, 4);
+    }
+  };
+  auto stage_commit = [&]() {
+#pragma unroll
+    for (int u = 0; u < BATCH; ++u) {
+      // bytes past the row's end: the zero point
+      uint32_t w = sshift[u] ? ((sv[u] >> sshift[u]) | (p.zp4 << (32 - sshift[u]))) : sv[u];
+      if (!sinside[u]) w = p.zp4;
+      if (sdst[u] >= 0) *(uint32_t *)(rows + sdst[u]) = w;
+    }
+  };
+  stage_issue(tid);
+
+  // the filter: fragment i holds output channels 32 i .. 32 i + 31 (rows past cout repeat the last)
+  v4i xf[FX];
+#pragma unroll
+  for (int i = 0; i < FX; ++i) {
+    const int ci = i * 32 + r32;
+    const int c = min(ci, p.cout - 1);
+    // the row's bytes 16 h .. 16 h + 15 as four dwords, no load under a condition (a load per byte,
+    // each waiting in a branch of its own, put sixteen memory round trips in front of every
+    // workgroup): a dword that straddles the row's end is taken from the dword that ends there
+    // (the depth is at least 4), one past the end is 0x80 bytes, zero after the shift
+    const uint8_t *row = p.filter + (int64_t)c * p.depth;
+    uint32_t w[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int o = 16 * h + 4 * j;
+      const int oc = min(o, p.depth - 4);
+      uint32_t got;
+      __builtin_memcpy(&got, row + oc, 4);
+      const int shift = 8 * (o - oc);
+      w[j] = o >= p.depth ? 0x80808080u
+                          : (shift ? ((got >> shift) | (0x80808080u << (32 - shift))) : got);
+    }
+    uint32_t xs = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) xs = __builtin_amdgcn_sad_u8(w[j], 0u, xs);
+    int sum = (int)xs - 128 * 16;   // of the shifted bytes
+    sum += __shfl_xor(sum, 32, 64);
+    xf[i] = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]} ^ flip;
+    if (wave == 0 && h == 0) {
+      uint32_t cx = (uint32_t)p.xcoef * (uint32_t)sum;
+      if (p.bias) cx += (uint32_t)p.bias[c];
+      s_cx[ci] = (int32_t)cx;
+    }
+  }
+  stage_requant_pairs_from((const int32_t *)((const char *)__builtin_amdgcn_kernarg_segment_ptr() +
+                                             sizeof(ConvShortParams)),
+                           s_tab, p.rq, tid, 256);
+  // the rest of the strip's input rows (a strip of MobileNet's first layer is done with the
+  // first turn)
+  stage_commit();
+  for (int base = tid + 256 * BATCH; base < stage_total; base += 256 * BATCH) {
+    stage_issue(base);
+    stage_commit();
+  }
+  // where byte e of this lane's 16 lies relative to its pixel's first patch byte, and which bytes
+  // exist at all.  (Single LDS bytes: LDS takes dword reads at any byte address, but gathering
+  // with those -- two per dword, merged under a mask -- ran at 39.7 us where this takes 23.4.)
+  int koff[16];
+  uint32_t keep[4] = {0, 0, 0, 0};
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    const int k = 16 * h + e;
+    const int kh = k / p.run;
+    koff[e] = k < p.depth ? kh * p.pitch + (k - kh * p.run) : 0;
+    if (k < p.depth) keep[e >> 2] |= 0xffu << (8 * (e & 3));
+  }
+  const RequantLds rql = requant_lds(p.rq, s_tab);
+  __syncthreads();
+
+  const int nblk = (npix + 31) >> 5;
+  int q = wave * 32 + r32;   // this lane's pixel within the strip
+  int ohl = q / p.out_w, ow = q - ohl * p.out_w;
+  const int dq = 128 / p.out_w, dr = 128 - dq * p.out_w;   // four blocks on
+  uint8_t *out0 = p.out + (((int64_t)img * p.out_h + oh0) * p.out_w) * p.cout + 16 * h;
+  const int step_h = p.sh * p.pitch, step_w = p.sw * p.cin;
+  for (int blk = wave; blk < nblk; blk += 4) {
+    // pixels past the strip's end read its last pixel's patch and store nothing
+    const bool live = q < npix;
+    const uint8_t *src = rows + p.gbase + (live ? ohl : nrows - 1) * step_h +
+                         (live ? ow : p.out_w - 1) * step_w;
+    uint32_t w[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t b0 = src[koff[4 * j]], b1 = src[koff[4 * j + 1]];
+      const uint32_t b2 = src[koff[4 * j + 2]], b3 = src[koff[4 * j + 3]];
+      const uint32_t got = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+      w[j] = (got & keep[j]) | (0x80808080u & ~keep[j]);
+    }
+    uint32_t ysr = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) ysr = __builtin_amdgcn_sad_u8(w[j], 0u, ysr);
+    int ys = (int)ysr - 128 * 16;
+    ys += __shfl_xor(ys, 32, 64);
+    const uint32_t cy = (uint32_t)p.ycoef * (uint32_t)ys + (uint32_t)p.yadd;
+    const v4i yf = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]} ^ flip;
+    uint8_t *orow = out0 + (int64_t)q * p.cout;
+#pragma unroll
+    for (int i = 0; i < FX; ++i) {
+      v16i acc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = 0;
+      acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(xf[i], yf, acc, 0, 0, 0);
+      // register r: channel 8 (r / 4) + 4 h + r % 4 of this block of 32, pixel lane % 32
+      const int xb = i * 32 + 4 * h;
+      int32_t v[16];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const v4i cx = *(const v4i *)(s_cx + xb + 8 * g);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[g * 4 + e] = (int32_t)((uint32_t)acc[g * 4 + e] + (uint32_t)cx[e] + cy);
+      }
+      uint32_t packed[4];
+      requant_16_by_table(v, rql, packed);
+      const v2u s02 = __builtin_amdgcn_permlane32_swap(packed[0], packed[2], false, false);
+      const v2u s13 = __builtin_amdgcn_permlane32_swap(packed[1], packed[3], false, false);
+      const v4i o = {(int)s02.x, (int)s02.y, (int)s13.x, (int)s13.y};
+      if (live && i * 32 + 16 * h < p.cout) *(v4i *)(orow + i * 32) = o;
+    }
+    q += 128;
+    ow += dr;
+    ohl += dq;
+    if (ow >= p.out_w) { ow -= p.out_w; ++ohl; }
+  }
+}
+
 // floor(a / b) for b > 0
 inline int64_t floor_div(int64_t a, int64_t b) { return a >= 0 ? a / b : -((-a + b - 1) / b); }
 
-// bias rescaling + GEMM shared by the 1x1 and the im2col paths; rhs is the [columns][rhs_ld]
-// panel (rhs_ld = 0: dense, row length = depth)
-int conv_gemm(mace_hip_ctx *ctx, const uint8_t *filter, const uint8_t *rhs, int64_t rhs_ld,
-              const int32_t *bias, int64_t cout, int64_t depth, int64_t columns,
-              float input_scale, int32_t input_zp, float filter_scale, int32_t filter_zp,
-              float bias_scale, int32_t mult, int shift, int32_t out_zp, int clamp_min,
-              int clamp_max, uint8_t *out, const Q8ConvGather *cv = nullptr) {
-  // GetBiasData (mace/ops/arm/q8/quantization_util.cc:20-46)
+// GetBiasData (mace/ops/arm/q8/quantization_util.cc:20-46): the bias as the GEMM adds it, rescaled
+// into an arena slice where its scale is not input_scale * filter_scale
+int conv_bias(mace_hip_ctx *ctx, const int32_t *bias, int64_t cout, float input_scale,
+              float filter_scale, float bias_scale, const int32_t **used) {
   volatile float prod = input_scale * filter_scale;
   volatile float diff = prod - bias_scale;
   const bool adjust = bias != nullptr && fabs((double)diff) > 1e-6;
-  const int32_t *bias_used = bias;   // a null bias adds nothing, like the zero vector
+  *used = bias;   // a null bias adds nothing, like the zero vector
   if (adjust) {
     int32_t *scaled = (int32_t *)mh_arena_take(ctx, sizeof(int32_t) * cout);
     if (!scaled) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
@@ -96,12 +301,100 @@ int conv_gemm(mace_hip_ctx *ctx, const uint8_t *filter, const uint8_t *rhs, int6
     MH_KLAUNCH(ctx, q8_bias_rescale_kernel, dim3((unsigned)((cout + 255) / 256)), dim3(256),
                        0, ctx->stream, bias, adjust_scale, scaled, (int)cout);
     MH_LAUNCH_CHECK(ctx);
-    bias_used = scaled;
+    *used = scaled;
   }
+  return MACE_HIP_SUCCESS;
+}
+
+// bias rescaling + GEMM shared by the 1x1 and the im2col paths; rhs is the [columns][rhs_ld]
+// panel (rhs_ld = 0: dense, row length = depth)
+int conv_gemm(mace_hip_ctx *ctx, const uint8_t *filter, const uint8_t *rhs, int64_t rhs_ld,
+              const int32_t *bias, int64_t cout, int64_t depth, int64_t columns,
+              float input_scale, int32_t input_zp, float filter_scale, int32_t filter_zp,
+              float bias_scale, int32_t mult, int shift, int32_t out_zp, int clamp_min,
+              int clamp_max, uint8_t *out, const Q8ConvGather *cv = nullptr) {
+  const int32_t *bias_used = nullptr;
+  MH_RETURN_IF_ERROR(conv_bias(ctx, bias, cout, input_scale, filter_scale, bias_scale, &bias_used));
   Q8GemmEpilogue ep{bias_used, mult, shift, out_zp, clamp_min, clamp_max};
   return mh_q8_gemm(ctx, filter, MACE_HIP_ROW_MAJOR, rhs, MACE_HIP_COL_MAJOR, out,
                     MACE_HIP_COL_MAJOR, true, 1, cout, depth, columns, 0, 0, -filter_zp,
                     -input_zp, ep, rhs_ld, cv);
+}
+
+// The strip kernel for patches of at most 32 bytes.  *taken = false: the call is not one for it
+// (nothing has been launched).
+int conv_short(mace_hip_ctx *ctx, const uint8_t *input, const uint8_t *filter, const int32_t *bias,
+               int64_t n, int64_t in_h, int64_t in_w, int64_t cin, int64_t cout, int64_t k_h,
+               int64_t k_w, int stride_h, int stride_w, int pad_top, int pad_left, int64_t out_h,
+               int64_t out_w, float input_scale, int32_t input_zp, float filter_scale,
+               int32_t filter_zp, float bias_scale, int32_t mult, int shift, int32_t out_zp,
+               int clamp_min, int clamp_max, uint8_t *out, bool *taken) {
+  *taken = false;
+  const int64_t depth = k_h * k_w * cin, columns = n * out_h * out_w;
+  if (depth > 32 || cout % 16 != 0 || cout > 128 || (uintptr_t)out % 16 != 0 ||
+      columns < 1024 || in_w * cin < 4 || depth < 4 || (ctx->kernel_mask & MH_MASK_NO_CONV_SHORT))
+    return MACE_HIP_SUCCESS;
+  if (shift < 0 || shift > 31 || clamp_min < 0 || clamp_max > 255 || clamp_min > clamp_max)
+    return MACE_HIP_SUCCESS;   // (the general path reports these)
+  RequantFixed rq;
+  if (!mh_make_requant(mult, shift, out_zp, clamp_min, clamp_max, &rq) || !rq.table)
+    return MACE_HIP_SUCCESS;
+  // staged rows: pixel positions -pad_left ... up to the last one any patch or the image reaches
+  const int64_t reach = std::max<int64_t>(in_w + pad_left, (out_w - 1) * stride_w + k_w);
+  const int lead = (int)mh_align_up((size_t)(pad_left * cin), 4);
+  const int gbase = lead - (int)(pad_left * cin);
+  const int64_t pitch = (int64_t)mh_align_up((size_t)(gbase + reach * cin), 4);
+  const int fx = cout <= 32 ? 1 : (cout <= 64 ? 2 : 4);
+  const int64_t fixed = 128 * fx + MH_REQUANT_PAIRS_BYTES;
+  auto lds_of = [&](int64_t r) { return fixed + ((r - 1) * stride_h + k_h) * pitch; };
+  if (lds_of(1) > 64 * 1024 || n * in_h >= (1ll << 31) || in_w * cin >= (1ll << 30)) return MACE_HIP_SUCCESS;
+  // Rows per strip: about columns / (2 CUs) pixels per workgroup, between 128 and 1024, and what
+  // fits in 64 KiB of LDS; among the heights from half of that up, the one that leaves the fewest
+  // blocks of 32 pixels.  (224 x 224 x 3 -> 32 at stride 2, batch 64, strips of 2 / 4 / 8 / 16
+  // output rows: 37.2 / 26.8 / 23.4 / 24.6 us -- workgroups cost about 5 ns each to start, and 448
+  // of them leave CUs idle.)
+  const int64_t cu = ctx->cu_count > 0 ? ctx->cu_count : 256;
+  const int64_t target = std::min<int64_t>(1024, std::max<int64_t>(128, columns / (2 * cu)));
+  int64_t r_hi = std::min<int64_t>(out_h, std::max<int64_t>(1, (target + out_w / 2) / out_w));
+  while (r_hi > 1 && lds_of(r_hi) > 64 * 1024) --r_hi;
+  int64_t strip = r_hi, best = -1;
+  for (int64_t r = r_hi; r >= std::max<int64_t>(1, r_hi / 2); --r) {
+    const int64_t strips = (out_h + r - 1) / r, last = out_h - (strips - 1) * r;
+    const int64_t blocks = (strips - 1) * ((r * out_w + 31) / 32) + (last * out_w + 31) / 32;
+    if (best < 0 || blocks < best) { best = blocks; strip = r; }
+  }
+  const int64_t strips = (out_h + strip - 1) / strip;
+  if (n * strips >= (1ll << 31)) return MACE_HIP_SUCCESS;
+  *taken = true;
+
+  MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, sizeof(int32_t) * cout + 4096));
+  ArenaScope scope(ctx);
+  const int32_t *bias_used = nullptr;
+  MH_RETURN_IF_ERROR(conv_bias(ctx, bias, cout, input_scale, filter_scale, bias_scale, &bias_used));
+  RequantTable tab;
+  mh_requant_table_cached(ctx, rq, tab.t);
+  const uint32_t zl = (uint32_t)filter_zp - 128u, zr = (uint32_t)input_zp - 128u;
+  ConvShortParams p{};
+  p.in = input; p.filter = filter; p.bias = bias_used; p.out = out;
+  p.in_h = (int)in_h; p.in_w = (int)in_w; p.cin = (int)cin; p.cout = (int)cout; p.k_h = (int)k_h;
+  p.sh = stride_h; p.sw = stride_w; p.pt = pad_top; p.out_h = (int)out_h; p.out_w = (int)out_w;
+  p.depth = (int)depth; p.run = (int)(k_w * cin); p.strip = (int)strip; p.strips = (int)strips;
+  p.pitch = (int)pitch; p.lead = lead; p.gbase = gbase;
+  p.zp4 = (uint32_t)(input_zp & 0xff) * 0x01010101u;
+  p.xcoef = (int32_t)(0u - zr);
+  p.ycoef = (int32_t)(0u - zl);
+  p.yadd = (int32_t)((uint32_t)depth * zl * zr);
+  p.rq = rq;
+  const size_t lds = (size_t)lds_of(strip);
+  dim3 grid((unsigned)(n * strips)), block(256);
+  mh_plan_main(ctx, MACE_HIP_KF_Q8_CONV_SHORT, mhv::conv_short(fx), grid, block, (int)lds);
+  MH_PROF_BEGIN(ctx);
+  if (fx == 1) MH_KLAUNCH(ctx, q8_conv_short_kernel<1>, grid, block, lds, ctx->stream, p, tab);
+  else if (fx == 2) MH_KLAUNCH(ctx, q8_conv_short_kernel<2>, grid, block, lds, ctx->stream, p, tab);
+  else MH_KLAUNCH(ctx, q8_conv_short_kernel<4>, grid, block, lds, ctx->stream, p, tab);
+  MH_PROF_END(ctx);
+  MH_LAUNCH_CHECK(ctx);
+  return MACE_HIP_SUCCESS;
 }
 
 // scratch the GEMM takes from the arena for a [cout x depth] . [depth x columns] product
@@ -149,6 +442,14 @@ extern "C" int mace_hip_conv2d_q8_nhwc(mace_hip_ctx *ctx, const uint8_t *input,
   // still skips it and reads past the input; here a padded 1x1 takes the im2col path.)
   const bool in_place = k_h == 1 && k_w == 1 && stride_h == 1 && stride_w == 1 && pad_h == 0 &&
                         pad_w == 0;
+  if (!in_place) {
+    bool taken = false;
+    MH_RETURN_IF_ERROR(conv_short(ctx, input, filter, bias, n, in_h, in_w, cin, cout, k_h, k_w,
+                                  stride_h, stride_w, pad_h >> 1, pad_w >> 1, out_h, out_w,
+                                  input_scale, input_zp, filter_scale, filter_zp, bias_scale, mult,
+                                  shift, out_zp, clamp_min, clamp_max, out, &taken));
+    if (taken) return MACE_HIP_SUCCESS;
+  }
   // With cin a multiple of 64 (and at least three 64-byte slabs of depth) the GEMM's loader
   // gathers the patches itself and no im2col matrix is written.
   // A small problem is one launch of the kernel that does the whole GEMM call, which gathers too

@@ -31,6 +31,7 @@ const int kVariantCount[MACE_HIP_KF_COUNT] = {
     1,                        // F32_GEMM_FILL
     3,                        // F32_GEMV_VEC
     1,                        // F32_GEMV_GENERAL
+    3,                        // Q8_CONV_SHORT
 };
 static_assert(mhv::RING_CONFIGS * 8 <= kMaxVariants, "coverage table too narrow");
 
@@ -39,7 +40,8 @@ const char *const kFamilyName[MACE_HIP_KF_COUNT] = {
     "q8_gemm_stream_kernel", "q8_gemm_dma_kernel", "q8_gemm_dma_kernel", "q8_gemm_dma_kernel",
     "q8_gemm_kernel", "q8_gemv_row_kernel", "q8_gemv_mfma_slice_kernel", "q8_gemv_mfma_lds_kernel",
     "q8_gemv_mfma_kernel", "q8_gemv_rows_kernel", "q8_gemv_kernel", "f32_gemm_vec_kernel",
-    "f32_gemm_kernel", "f32_fill_kernel", "f32_gemv_vec_kernel", "f32_gemv_kernel"};
+    "f32_gemm_kernel", "f32_fill_kernel", "f32_gemv_vec_kernel", "f32_gemv_kernel",
+    "q8_conv_short_kernel"};
 
 // <WX, WY, FX, FY, STAGES, OCC, KB> of the ring kernel's tile configurations (mhv::RING_*)
 const int kRing[mhv::RING_CONFIGS][7] = {
@@ -176,6 +178,9 @@ int mace_hip_plan_describe(int family, int v, char *buf, size_t len) {
       break;
     case MACE_HIP_KF_F32_GEMM_GENERAL:
       snprintf(buf, len, "%s<LK=%s,RK=%s>", k, tf(v & 2), tf(v & 1));
+      break;
+    case MACE_HIP_KF_Q8_CONV_SHORT:
+      snprintf(buf, len, "%s<FX=%d>", k, 1 << v);
       break;
     case MACE_HIP_KF_F32_GEMV_VEC:
       snprintf(buf, len, "%s<NB=%d>", k, 1 << v);

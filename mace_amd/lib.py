@@ -13,7 +13,7 @@ SUCCESS, INVALID_ARGS, OUT_OF_RESOURCES, UNSUPPORTED, RUNTIME_ERROR = range(5)
 ROW_MAJOR, COL_MAJOR = 0, 1
 REQUANT_REF, REQUANT_NEON = 0, 1
 ACT_NOOP, ACT_RELU, ACT_RELUX = 0, 1, 2
-MASK_NO_SMALL, MASK_NO_XRES, MASK_NO_MID, MASK_NO_XFLIP = 1, 2, 4, 8
+MASK_NO_SMALL, MASK_NO_XRES, MASK_NO_MID, MASK_NO_XFLIP, MASK_NO_CONV_SHORT = 1, 2, 4, 8, 16
 NOALLOC_SCRATCH_BYTES = 32 << 20
 
 _STATUS_NAMES = {0: "MACE_SUCCESS", 1: "MACE_INVALID_ARGS", 2: "MACE_OUT_OF_RESOURCES",
@@ -130,7 +130,8 @@ SIGNATURES = {
 (KF_NONE, KF_Q8_GEMM_FUSED_SMALL, KF_Q8_GEMM_XRES, KF_Q8_GEMM_MID, KF_Q8_GEMM_STREAM, KF_Q8_GEMM_RING,
  KF_Q8_GEMM_RING_XT, KF_Q8_GEMM_RING_XF, KF_Q8_GEMM_TILED, KF_Q8_GEMV_ROW, KF_Q8_GEMV_SLICE,
  KF_Q8_GEMV_MFMA_LDS, KF_Q8_GEMV_MFMA, KF_Q8_GEMV_ROWS, KF_Q8_GEMV_GENERAL, KF_F32_GEMM_VEC,
- KF_F32_GEMM_GENERAL, KF_F32_GEMM_FILL, KF_F32_GEMV_VEC, KF_F32_GEMV_GENERAL, KF_COUNT) = range(21)
+ KF_F32_GEMM_GENERAL, KF_F32_GEMM_FILL, KF_F32_GEMV_VEC, KF_F32_GEMV_GENERAL, KF_Q8_CONV_SHORT,
+ KF_COUNT) = range(22)
 (AUX_PACK_ROWS, AUX_PACK_TRANSPOSE, AUX_PACK_SHIFTED, AUX_PANEL_SUMS, AUX_KMAJOR_SUMS, AUX_ZERO,
  AUX_IM2COL, AUX_BIAS_RESCALE, AUX_F32_PAD, AUX_FILL, AUX_WEIGHT_HIT, AUX_WEIGHT_BUILD) = (
     1 << i for i in range(12))

@@ -29,7 +29,7 @@ DIMS = [16, 48, 64, 80, 96, 100, 128, 255, 256, 300, 512, 1000, 1024, 1100, 1536
 DEPTHS = [16, 32, 48, 64, 96, 100, 128, 192, 256, 320, 384, 448, 512, 576, 640, 960, 1024, 1152, 1280,
           2048, 2176, 4096, 8192]
 ORDERS = list(itertools.product((0, 1), repeat=3))
-MASKS = [0, 1, 2, 3, 4, 7, 15]
+MASKS = [0, 1, 2, 3, 4, 7, 15, 16, 31]
 
 
 def plan_call(c, call):

@@ -99,8 +99,10 @@ def path(request, ctx):
     patches itself; with kernel-mask bit 0 it goes to the kernel that keeps the filter in
     LDS (cin a multiple of 64, filter tile fits) and with bit 1 on top through
     im2col / the gathering tiled kernel, so that all three stay covered on the same shapes."""
-    mask = {"default": 0, "no_small_kernel": mh.MASK_NO_SMALL,
-            "general_path": mh.MASK_NO_SMALL | mh.MASK_NO_XRES}[request.param]
+    # (both masked modes also switch off the strip kernel for patches of at most 32 bytes, which
+    # the default mode runs on the shapes it applies to)
+    mask = {"default": 0, "no_small_kernel": mh.MASK_NO_SMALL | mh.MASK_NO_CONV_SHORT,
+            "general_path": mh.MASK_NO_SMALL | mh.MASK_NO_XRES | mh.MASK_NO_CONV_SHORT}[request.param]
     ctx.call("mace_hip_ctx_set_kernel_mask", mask)
     yield request.param
     ctx.call("mace_hip_ctx_set_kernel_mask", 0)
@@ -128,6 +130,47 @@ def test_conv2d_q8_parity(ctx, path, n, cout, cin, in_h, in_w, k_h, k_w, pad, st
         np.testing.assert_array_equal(got, want)
     if want.size >= 64:
         assert len(np.unique(want)) > 8
+
+
+SHORT_CASES = [  # batch, cout, cin, in_h, in_w, k_h, k_w, padding, strides, filter blocks of 32
+    (8, 32, 3, 224, 224, 3, 3, S, (2, 2), 1),     # MobileNet's first layer
+    (1, 32, 3, 224, 224, 3, 3, S, (2, 2), 1),     # ... one image: strips of a single output row
+    (3, 16, 3, 65, 67, 3, 3, S, (2, 2), 1),       # half a block of channels, odd sizes
+    (2, 64, 3, 64, 64, 3, 3, V, (1, 1), 2),
+    (2, 128, 1, 40, 40, 5, 5, S, (1, 1), 4),      # depth 25
+    (3, 48, 8, 41, 41, 1, 1, V, (2, 2), 2),       # 1 x 1 at stride 2
+    (4, 32, 2, 50, 50, 4, 4, Fu, (3, 3), 1),      # depth 32 exactly, padding of 3 on every side
+    (5, 96, 4, 30, 30, 2, 3, S, (1, 2), 4),
+    (2, 32, 16, 33, 33, 1, 2, S, (1, 1), 1),      # two whole 16-byte channel runs
+    (64, 32, 3, 20, 20, 3, 3, S, (2, 2), 1),      # a strip is a whole (small) image
+    (1, 112, 3, 40, 300, 3, 3, S, (1, 1), 4),     # wide rows, ragged channel count
+]
+
+
+@pytest.mark.parametrize("n,cout,cin,in_h,in_w,k_h,k_w,pad,st,fx", SHORT_CASES)
+def test_conv2d_q8_short_patches(ctx, n, cout, cin, in_h, in_w, k_h, k_w, pad, st, fx):
+    """Patches of at most 32 bytes: the kernel that stages a strip's input rows in LDS.  Against the
+    oracle bit for bit, the kernel that ran asserted, three bias / clamp settings each."""
+    rng = np.random.default_rng(cout * 13 + cin + k_h * 5 + k_w + in_w)
+    x = rng.integers(0, 256, (n, in_h, in_w, cin), dtype=np.uint8)
+    f = rng.integers(1, 256, (cout, k_h, k_w, cin), dtype=np.uint8)
+    bias = rng.integers(-2 ** 15, 2 ** 15, cout).astype(np.int32)
+    z_in, z_f = int(rng.integers(0, 256)), int(rng.integers(0, 256))
+    s_in, s_f = np.float32(0.02), np.float32(0.01)
+    depth = k_h * k_w * cin
+    s_out = np.float32(max(6.0, 3 * 74.0 * 74.0 * np.sqrt(depth) * float(s_in * s_f)) / 255.0)
+    oh, ow, ph, pw = orc.calc_padding_and_output_size(in_h, in_w, k_h, k_w, st, pad)
+    for (bb, s_b, z_o, lo, hi) in ((bias, np.float32(s_in * s_f), 0, 0, 255),
+                                   (bias, np.float32(2.5 * float(s_in * s_f)), 100, 100, 230),
+                                   (None, np.float32(0), 128, 0, 255)):
+        want = orc.conv2d_q8_nhwc(x, f, bb, n, in_h, in_w, cin, cout, k_h, k_w, st, (ph, pw), s_in,
+                                  z_in, s_f, z_f, s_b, s_out, z_o, lo, hi, nthreads=16)
+        got = conv_host(ctx, x, f, bb, n, in_h, in_w, cin, cout, k_h, k_w, st, (ph, pw), s_in,
+                        z_in, s_f, z_f, s_b, s_out, z_o, lo, hi)
+        assert ctx.last_plan().kernel == "q8_conv_short_kernel<FX=%d>" % fx
+        assert got.shape == (n, oh, ow, cout)
+        np.testing.assert_array_equal(got, want)
+    assert len(np.unique(want)) > 8
 
 
 def test_conv2d_q8_filter_in_lds_many_blocks(ctx):

@@ -252,9 +252,25 @@ def test_convolution_gather_and_im2col(ctx):
     assert p.family == mh.KF_Q8_GEMM_RING and "CONV=true" in p.kernel
     p = conv(ctx, 64, 7, 512, 512, k=3, pad=2)          # one round of tiles, long depth: patch matrix
     assert p.family == mh.KF_Q8_GEMM_MID and p.aux & mh.AUX_IM2COL
-    p = conv(ctx, 64, 224, 3, 32, k=3, stride=2, pad=1)  # MobileNet's first layer: gathered byte-wise
-    assert p.family == mh.KF_Q8_GEMM_FUSED_SMALL and "BW=true" in p.kernel and p.launches == 1
-    p = conv(ctx, 64, 224, 3, 32, k=3, stride=2, pad=1, mask=mh.MASK_NO_SMALL)
+    # MobileNet's first layer: a patch of 27 bytes, the strip kernel; one workgroup per strip
+    p = conv(ctx, 64, 224, 3, 32, k=3, stride=2, pad=1)
+    assert p.kernel == "q8_conv_short_kernel<FX=1>" and p.launches == 1 and p.lds_bytes <= 64 * 1024
+    assert p.grid[0] % 64 == 0 and 2 * 256 <= p.grid[0] <= 64 * 112
+    assert conv(ctx, 1, 224, 3, 32, k=3, stride=2, pad=1).kernel == "q8_conv_short_kernel<FX=1>"
+    assert conv(ctx, 64, 224, 3, 64, k=3, stride=2, pad=1).kernel == "q8_conv_short_kernel<FX=2>"
+    assert conv(ctx, 64, 224, 3, 128, k=3, stride=2, pad=1).kernel == "q8_conv_short_kernel<FX=4>"
+    assert conv(ctx, 8, 64, 2, 32, k=4, stride=1, pad=3).family == mh.KF_Q8_CONV_SHORT       # depth 32
+    # not for it: 33 bytes of patch, channel counts that are not whole 16-byte pieces of the output
+    # row or more than 128, fewer than 1024 pixels; those stay with the one-launch kernel
+    small = mh.KF_Q8_GEMM_FUSED_SMALL
+    assert conv(ctx, 8, 64, 3, 32, k=3, stride=1, pad=2, mask=0).family == mh.KF_Q8_CONV_SHORT
+    assert conv(ctx, 8, 64, 11, 32, k=3, stride=3, pad=0).family == small     # depth 99
+    assert conv(ctx, 8, 64, 3, 24, k=3, stride=2, pad=1).family == small
+    assert conv(ctx, 8, 64, 3, 144, k=3, stride=2, pad=1).family == small
+    assert conv(ctx, 1, 40, 3, 32, k=3, stride=2, pad=1).family == small      # 400 pixels
+    p = conv(ctx, 64, 224, 3, 32, k=3, stride=2, pad=1, mask=mh.MASK_NO_CONV_SHORT)
+    assert p.family == small and "BW=true" in p.kernel and p.launches == 1   # gathered byte-wise
+    p = conv(ctx, 64, 224, 3, 32, k=3, stride=2, pad=1, mask=mh.MASK_NO_SMALL | mh.MASK_NO_CONV_SHORT)
     assert p.aux & mh.AUX_IM2COL
 
 
@@ -296,7 +312,7 @@ def test_variant_tables_are_consistent():
         total += len(vs)
         assert not lib.mace_hip_plan_variant_valid(f, n) and not lib.mace_hip_plan_variant_valid(f, -1)
         assert mh.coverage(f, 0) == 0              # nothing is launched by planning
-    assert total == 220
+    assert total == 223
     assert lib.mace_hip_plan_variant_count(0) == 0 and lib.mace_hip_plan_variant_count(mh.KF_COUNT) == 0
 
 
