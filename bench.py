@@ -80,6 +80,8 @@ def main():
     ap.add_argument("--no-gemv", action="store_true")
     ap.add_argument("--no-other", action="store_true",
                     help="skip the secondary configurations (conv1x1, smaller GEMMs, fp32)")
+    ap.add_argument("--no-net", action="store_true",
+                    help="skip the pointwise-layer net (a child process; leave it out under a profiler)")
     ap.add_argument("--only-gemv", action="store_true", help="development: skip the GEMM part")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a kernel of known traffic, for "
@@ -302,7 +304,7 @@ def main():
     if not args.no_other:
         result["other_configs"] = bench_other(ctx, mh, torch)
         result["host_pointer_calls"] = bench_host_pointers(ctx, mh, np)
-        chain = bench_c4_net()
+        chain = None if args.no_net else bench_c4_net()
         if chain is not None:
             result["other_configs"].append(chain)
 

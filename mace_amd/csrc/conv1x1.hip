@@ -142,18 +142,23 @@ __global__ __launch_bounds__(256, 3) void q8_conv_short_kernel(ConvShortParams p
   uint32_t sv[BATCH];
   int sdst[BATCH], sshift[BATCH];
   bool sinside[BATCH];
+  // dword d = (staged row sr, dword dw of it); a thread's dwords are 256 apart, walked without a
+  // division per dword (those divisions were a quarter of the kernel's vector instructions)
+  const int sr_step = 256 / dpr, dw_step = 256 - sr_step * dpr;
+  int sr = tid / dpr, dw = tid - sr * dpr;
   auto stage_issue = [&](int base) {
 #pragma unroll
     for (int u = 0; u < BATCH; ++u) {
-      const int d = min(base + u * 256, stage_total - 1);
-      const int sr = d / dpr, dw = d - sr * dpr;
-      const int ih = ih_first + sr;
+      const int ih = ih_first + sr;   // (past the last staged row for dwords past the total: clamped, not stored)
       const int o = dw * 4 - p.lead;   // byte offset inside the input row
       sinside[u] = (unsigned)ih < (unsigned)p.in_h && o >= 0 && o < row_len;
       const int oc = min(max(o, 0), row_len - 4);
       sshift[u] = sinside[u] ? 8 * (o - oc) : 0;   // > 0 for the partial dword at the row's end
       sdst[u] = base + u * 256 < stage_total ? sr * p.pitch + dw * 4 : -1;
       __builtin_memcpy(&sv[u], image + (int64_t)min(max(ih, 0), p.in_h - 1) * row_len + oc, 4);
+      sr += sr_step;
+      dw += dw_step;
+      if (dw >= dpr) { dw -= dpr; ++sr; }
     }
   };
   auto stage_commit = [&]() {
@@ -216,12 +221,16 @@ __global__ __launch_bounds__(256, 3) void q8_conv_short_kernel(ConvShortParams p
   // with those -- two per dword, merged under a mask -- ran at 39.7 us where this takes 23.4.)
   int koff[16];
   uint32_t keep[4] = {0, 0, 0, 0};
+  {
+    const int kh16 = 16 / p.run;   // (uniform: one scalar division)
+    int kh_off = h ? kh16 * p.pitch : 0, off = h ? 16 - kh16 * p.run : 0;
 #pragma unroll
-  for (int e = 0; e < 16; ++e) {
-    const int k = 16 * h + e;
-    const int kh = k / p.run;
-    koff[e] = k < p.depth ? kh * p.pitch + (k - kh * p.run) : 0;
-    if (k < p.depth) keep[e >> 2] |= 0xffu << (8 * (e & 3));
+    for (int e = 0; e < 16; ++e) {
+      const int k = 16 * h + e;
+      koff[e] = k < p.depth ? kh_off + off : 0;
+      if (k < p.depth) keep[e >> 2] |= 0xffu << (8 * (e & 3));
+      if (++off == p.run) { off = 0; kh_off += p.pitch; }
+    }
   }
   const RequantLds rql = requant_lds(p.rq, s_tab);
   __syncthreads();
@@ -232,11 +241,15 @@ __global__ __launch_bounds__(256, 3) void q8_conv_short_kernel(ConvShortParams p
   const int dq = 128 / p.out_w, dr = 128 - dq * p.out_w;   // four blocks on
   uint8_t *out0 = p.out + (((int64_t)img * p.out_h + oh0) * p.out_w) * p.cout + 16 * h;
   const int step_h = p.sh * p.pitch, step_w = p.sw * p.cin;
+  // LDS offset of this lane's pixel's first patch byte, advanced with the pixel (no multiplication
+  // per block), and that of the strip's last pixel
+  int at = p.gbase + ohl * step_h + ow * step_w;
+  const int at_step = dq * step_h + dr * step_w, at_wrap = step_h - p.out_w * step_w;
+  const int at_last = p.gbase + (nrows - 1) * step_h + (p.out_w - 1) * step_w;
   for (int blk = wave; blk < nblk; blk += 4) {
     // pixels past the strip's end read its last pixel's patch and store nothing
     const bool live = q < npix;
-    const uint8_t *src = rows + p.gbase + (live ? ohl : nrows - 1) * step_h +
-                         (live ? ow : p.out_w - 1) * step_w;
+    const uint8_t *src = rows + (live ? at : at_last);
     uint32_t w[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -250,7 +263,8 @@ __global__ __launch_bounds__(256, 3) void q8_conv_short_kernel(ConvShortParams p
     for (int j = 0; j < 4; ++j) ysr = __builtin_amdgcn_sad_u8(w[j], 0u, ysr);
     int ys = (int)ysr - 128 * 16;
     ys += __shfl_xor(ys, 32, 64);
-    const uint32_t cy = (uint32_t)p.ycoef * (uint32_t)ys + (uint32_t)p.yadd;
+    // (both factors fit in 24 bits: a zero point and the sum of 32 bytes)
+    const uint32_t cy = (uint32_t)__mul24(p.ycoef, ys) + (uint32_t)p.yadd;
     const v4i yf = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]} ^ flip;
     uint8_t *orow = out0 + (int64_t)q * p.cout;
 #pragma unroll
@@ -277,8 +291,8 @@ __global__ __launch_bounds__(256, 3) void q8_conv_short_kernel(ConvShortParams p
     }
     q += 128;
     ow += dr;
-    ohl += dq;
-    if (ow >= p.out_w) { ow -= p.out_w; ++ohl; }
+    at += at_step;
+    if (ow >= p.out_w) { ow -= p.out_w; at += at_wrap; }
   }
 }
 
