@@ -23,7 +23,7 @@ const int kVariantCount[MACE_HIP_KF_COUNT] = {
     32,                       // Q8_GEMV_ROW
     6,                        // Q8_GEMV_SLICE
     2,                        // Q8_GEMV_MFMA_LDS
-    6,                        // Q8_GEMV_MFMA
+    4,                        // Q8_GEMV_MFMA
     8,                        // Q8_GEMV_ROWS
     16,                       // Q8_GEMV_GENERAL
     8,                        // F32_GEMM_VEC

@@ -2715,6 +2715,8 @@ int Q8Call::kmajor_in_place(bool *done) {
     const int64_t xn = xl ? rows : cols, yn = xl ? cols : rows;
     const uint8_t *xp = xl ? lhs : rhs, *yp = xl ? rhs : lhs;
     const bool y_direct = xl ? (rhs_direct && rhs_ld == 0) : lhs_direct;
+    // (32 x 512^3: 64-row tiles, 64-row blocks and one to three workgroups per tile all land within
+    // 17.9 - 19.2 us: the redundant transposes of a tile shared by four workgroups are not the cost)
     const int tx = xn <= 64 ? 64 : 128;
     const size_t lds_cu = ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536;
     const int64_t tiles128 = ((xn + 127) / 128) * ((yn + 127) / 128) * batch;

@@ -385,8 +385,8 @@ __global__ __launch_bounds__(1024) void q8_gemv_row_kernel(
 // v_mfma_i32_16x16x64_i8 with the weights as the 16 x 64 A operand (lane l: row l % 16, bytes
 // [16 (l / 16), +16) of the step, loaded straight from global memory) and, as the 64 x 16 B
 // operand, column b < NB = right-hand vector b (same bytes of the step, loaded from global /
-// L2), column 15 = all ones (its result column is the row sum of the weights), other columns
-// zero.  Bytes are shifted to int8 (XOR 0x80) on the way in:
+// L2), other columns zero.  (The weights' row sums come from v_sad_u8 on the fragments as read: a
+// column of ones would yield them for nothing but costs the sixteenth vector of a pass.)  Bytes are shifted to int8 (XOR 0x80) on the way in:
 //   sum (w - zl)(x - zr) = sum w'x' - zr' sum w' - zl' sum x' + W zl' zr',  z' = z - 128.
 // A k step past the end of the row contributes zeros on the weight side.  The wavefronts'
 // partial 16 x 16 results meet in LDS (integer atomics: the order does not matter).
@@ -401,9 +401,9 @@ typedef int gv4i __attribute__((ext_vector_type(4)));
 // other; what is left is the vectors' traffic, re-read from L2 by every workgroup.)
 template <int NW, int GROUP, int NBUF, typename OutT>
 __global__ __launch_bounds__(NW * 64) void q8_gemv_mfma_kernel(GemvParams p) {
-  constexpr int NBMAX = 15, ONES_COL = 15;
+  constexpr int NBMAX = 16;
   __shared__ int32_t s_acc[16][17];
-  __shared__ int32_t s_sx[16];
+  __shared__ int32_t s_sx[16], s_sl[16];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, q = lane >> 4;
@@ -416,19 +416,17 @@ __global__ __launch_bounds__(NW * 64) void q8_gemv_mfma_kernel(GemvParams p) {
   const int ks0 = wave * per_wave, ks1 = min(nstep, ks0 + per_wave);
 
   for (int i = tid; i < 16 * 17; i += NW * 64) (&s_acc[0][0])[i] = 0;
-  if (tid < 16) s_sx[tid] = 0;
+  if (tid < 16) s_sx[tid] = s_sl[tid] = 0;
 
   const uint8_t *arow = p.lhs + (int64_t)min(h0 + r, p.H - 1) * p.W;
   const uint8_t *xrow = p.rhs + (int64_t)min(b0 + r, p.batch - 1) * p.rhs_bs;
   const bool is_x = r < nb;
   const gv4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
   const gv4i zero = {0, 0, 0, 0};
-  const gv4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
-  const gv4i other = r == ONES_COL ? ones : zero;
 
   gv4i acc[2] = {zero, zero};
-  uint32_t sx_raw = 0;   // the vector's bytes as read, 128 too much each
-  int sx_bytes = 0;
+  uint32_t sx_raw = 0, sl_raw = 0;   // the vector's / the row's bytes as read, 128 too much each
+  int sx_bytes = 0, sl_bytes = 0;
   // steps past the wavefront's share or the end of the row re-read the row's last chunk (masked
   // when multiplied)
   auto fetch = [&](gv4i (&a)[GROUP], gv4i (&x)[GROUP], int ks) {
@@ -453,7 +451,7 @@ __global__ __launch_bounds__(NW * 64) void q8_gemv_mfma_kernel(GemvParams p) {
 #pragma unroll
     for (int u = 0; u < GROUP; ++u) {
       const bool valid = (ks + u < ks1) && (4 * (ks + u) + q < nchunk);
-      gv4i xv = is_x ? (x[u] ^ flip) : other;
+      gv4i xv = is_x ? (x[u] ^ flip) : zero;
       if (!valid) xv = zero;
       if (is_x && valid) {
         // v_sad_u8: a dot-product instruction would not run beside the MFMAs
@@ -462,6 +460,13 @@ __global__ __launch_bounds__(NW * 64) void q8_gemv_mfma_kernel(GemvParams p) {
         sx_raw = __builtin_amdgcn_sad_u8((uint32_t)x[u].z, 0u, sx_raw);
         sx_raw = __builtin_amdgcn_sad_u8((uint32_t)x[u].w, 0u, sx_raw);
         sx_bytes += 16;
+      }
+      if (valid) {
+        sl_raw = __builtin_amdgcn_sad_u8((uint32_t)a[u].x, 0u, sl_raw);
+        sl_raw = __builtin_amdgcn_sad_u8((uint32_t)a[u].y, 0u, sl_raw);
+        sl_raw = __builtin_amdgcn_sad_u8((uint32_t)a[u].z, 0u, sl_raw);
+        sl_raw = __builtin_amdgcn_sad_u8((uint32_t)a[u].w, 0u, sl_raw);
+        sl_bytes += 16;
       }
       const gv4i av = valid ? (a[u] ^ flip) : zero;
       acc[u & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, xv, acc[u & 1], 0, 0, 0);
@@ -491,6 +496,7 @@ __global__ __launch_bounds__(NW * 64) void q8_gemv_mfma_kernel(GemvParams p) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) atomicAdd(&s_acc[4 * q + i][r], acc[0][i] + acc[1][i]);
   if (is_x) atomicAdd(&s_sx[r], sx);
+  atomicAdd(&s_sl[r], (int)sl_raw - 128 * sl_bytes);   // this lane's bytes of row r
   __syncthreads();
 
   if (tid < 16 * nb) {
@@ -498,7 +504,7 @@ __global__ __launch_bounds__(NW * 64) void q8_gemv_mfma_kernel(GemvParams p) {
     const int h = h0 + row;
     if (h < p.H) {
       const uint32_t zl = (uint32_t)p.lhs_zp - 128u, zr = (uint32_t)p.rhs_zp - 128u;
-      const uint32_t ret = (uint32_t)s_acc[row][b] - zr * (uint32_t)s_acc[row][ONES_COL] -
+      const uint32_t ret = (uint32_t)s_acc[row][b] - zr * (uint32_t)s_sl[row] -
                            zl * (uint32_t)s_sx[b] + (uint32_t)p.W * zl * zr +
                            (p.bias ? (uint32_t)p.bias[h] : 0u);
       OutT *o = (OutT *)p.out + (int64_t)(b0 + b) * p.H + h;
@@ -522,10 +528,10 @@ __global__ __launch_bounds__(NW * 64) void q8_gemv_mfma_kernel(GemvParams p) {
 // requested before anything else.
 template <int NW, typename OutT>
 __global__ __launch_bounds__(NW * 64) void q8_gemv_mfma_lds_kernel(GemvParams p, int pitch) {
-  constexpr int NBMAX = 15, ONES_COL = 15, NT = NW * 64;
+  constexpr int NBMAX = 16, NT = NW * 64;
   extern __shared__ __align__(16) uint8_t lds_rows[];   // [16 + nb][pitch]
   __shared__ int32_t s_acc[16][17];
-  __shared__ int32_t s_sx[16];
+  __shared__ int32_t s_sx[16], s_sl[16];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, q = lane >> 4;
@@ -556,7 +562,7 @@ __global__ __launch_bounds__(NW * 64) void q8_gemv_mfma_lds_kernel(GemvParams p,
       mh_dma_16B(src + (int64_t)min(64 * j + lane, nchunk - 1) * 16, dst + j * 1024);
   }
   for (int i = tid; i < 16 * 17; i += NT) (&s_acc[0][0])[i] = 0;
-  if (tid < 16) s_sx[tid] = 0;
+  if (tid < 16) s_sx[tid] = s_sl[tid] = 0;
   // vmcnt(0), lgkmcnt(0): own transfers and LDS stores done (and the bias has arrived)
   __builtin_amdgcn_s_waitcnt(0x0070);
   __builtin_amdgcn_s_barrier();
@@ -565,15 +571,13 @@ __global__ __launch_bounds__(NW * 64) void q8_gemv_mfma_lds_kernel(GemvParams p,
   const bool is_x = r < nb;
   const gv4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
   const gv4i zero = {0, 0, 0, 0};
-  const gv4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
-  const gv4i other = r == ONES_COL ? ones : zero;
   const uint8_t *arow = lds_rows + r * pitch + q * 16;
   const uint8_t *xrow = lds_rows + (16 + (is_x ? r : 0)) * pitch + q * 16;
 
   // Four k steps at a time: all fragment reads first, then the multiplications on two
   // accumulators (a chain of dependent MFMAs would wait for each result in turn).
   gv4i acc0 = zero, acc1 = zero;
-  int sx = 0;
+  int sx = 0, sl = 0;
   for (int kb = ks0; kb < ks1; kb += 4) {
     gv4i av[4], xv[4];
 #pragma unroll
@@ -586,7 +590,7 @@ __global__ __launch_bounds__(NW * 64) void q8_gemv_mfma_lds_kernel(GemvParams p,
     for (int u = 0; u < 4; ++u) {
       const bool valid = kb + u < ks1 && 4 * (kb + u) + q < nchunk;
       const gv4i a = valid ? (av[u] ^ flip) : zero;
-      gv4i x = is_x ? (xv[u] ^ flip) : other;
+      gv4i x = is_x ? (xv[u] ^ flip) : zero;
       if (!valid) x = zero;
       if (is_x) {
         sx = __builtin_amdgcn_sdot4(x.x, 0x01010101, sx, false);
@@ -594,6 +598,10 @@ __global__ __launch_bounds__(NW * 64) void q8_gemv_mfma_lds_kernel(GemvParams p,
         sx = __builtin_amdgcn_sdot4(x.z, 0x01010101, sx, false);
         sx = __builtin_amdgcn_sdot4(x.w, 0x01010101, sx, false);
       }
+      sl = __builtin_amdgcn_sdot4(a.x, 0x01010101, sl, false);   // (zero where the step does not exist)
+      sl = __builtin_amdgcn_sdot4(a.y, 0x01010101, sl, false);
+      sl = __builtin_amdgcn_sdot4(a.z, 0x01010101, sl, false);
+      sl = __builtin_amdgcn_sdot4(a.w, 0x01010101, sl, false);
       if (u & 1) acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, x, acc1, 0, 0, 0);
       else acc0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, x, acc0, 0, 0, 0);
     }
@@ -602,6 +610,7 @@ __global__ __launch_bounds__(NW * 64) void q8_gemv_mfma_lds_kernel(GemvParams p,
 #pragma unroll
     for (int i = 0; i < 4; ++i) atomicAdd(&s_acc[4 * q + i][r], acc0[i] + acc1[i]);
     if (is_x) atomicAdd(&s_sx[r], sx);
+    atomicAdd(&s_sl[r], sl);
   }
   __syncthreads();
 
@@ -610,7 +619,7 @@ __global__ __launch_bounds__(NW * 64) void q8_gemv_mfma_lds_kernel(GemvParams p,
     const int h = h0 + row;
     if (h < p.H) {
       const uint32_t zl = (uint32_t)p.lhs_zp - 128u, zr = (uint32_t)p.rhs_zp - 128u;
-      const uint32_t ret = (uint32_t)s_acc[row][b] - zr * (uint32_t)s_acc[row][ONES_COL] -
+      const uint32_t ret = (uint32_t)s_acc[row][b] - zr * (uint32_t)s_sl[row] -
                            zl * (uint32_t)s_sx[b] + (uint32_t)p.W * zl * zr + bias_v;
       OutT *o = (OutT *)p.out + (int64_t)(b0 + b) * p.H + h;
       if constexpr (sizeof(OutT) == 4) *o = (OutT)(int32_t)ret;
@@ -632,7 +641,7 @@ template <int SPW, typename OutT>
 __global__ __launch_bounds__(1024) void q8_gemv_mfma_slice_kernel(
     const uint8_t *lhs, const uint8_t *rhs, int H, int W, const int32_t *bias_ptr, void *out,
     float mult, int32_t out_zp, int32_t lhs_zp, int32_t rhs_zp, int batch, int64_t rhs_bs) {
-  constexpr int NBMAX = 15, ONES_COL = 15;
+  constexpr int NBMAX = 16;
   constexpr int CH = 4 * SPW;        // 16-byte chunks per row of a slice
   constexpr int RPI = 64 / CH;       // rows per transfer instruction
   constexpr int NI = 16 / RPI;       // instructions for the 16 weight rows (and for 16 vectors)
@@ -640,7 +649,7 @@ __global__ __launch_bounds__(1024) void q8_gemv_mfma_slice_kernel(
   static_assert(SPW == 1 || SPW == 2 || SPW == 4, "slice width");
   __shared__ __align__(16) uint8_t area[16][2][NI * 1024];   // [wavefront][weights, vectors]
   __shared__ int32_t s_acc[16][17];
-  __shared__ int32_t s_sx[16];
+  __shared__ int32_t s_sx[16], s_sl[16];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, q = lane >> 4;
@@ -675,7 +684,7 @@ __global__ __launch_bounds__(1024) void q8_gemv_mfma_slice_kernel(
     }
   }
   for (int i = tid; i < 16 * 17; i += 1024) (&s_acc[0][0])[i] = 0;
-  if (tid < 16) s_sx[tid] = 0;
+  if (tid < 16) s_sx[tid] = s_sl[tid] = 0;
   // the zeroed sums are visible; lgkmcnt(0) only, so that the transfers stay in flight
   __builtin_amdgcn_s_waitcnt(0xC07F);
   __builtin_amdgcn_s_barrier();
@@ -684,8 +693,6 @@ __global__ __launch_bounds__(1024) void q8_gemv_mfma_slice_kernel(
   const bool is_x = r < nb;
   const gv4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
   const gv4i zero = {0, 0, 0, 0};
-  const gv4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
-  const gv4i other = r == ONES_COL ? ones : zero;
   if (active) {
     // row r of the area: transfer r / RPI, row r % RPI inside it, chunk c in slot c ^ f(r)
     const int rbase = (r / RPI) * 1024 + (r % RPI) * (CH * 16);
@@ -701,13 +708,21 @@ __global__ __launch_bounds__(1024) void q8_gemv_mfma_slice_kernel(
       if (is_x) xv[u] = *(const gv4i *)(&area[wave][1][rbase + slot * 16]);
     }
     gv4i acc0 = zero, acc1 = zero;
-    int sx = 0;
+    int sx = 0, sl = 0;
 #pragma unroll
     for (int u = 0; u < SPW; ++u) {
       const bool valid = c0 + 4 * u + q < nchunk;
       const gv4i a = valid ? (av[u] ^ flip) : zero;
-      gv4i x = is_x ? (xv[u] ^ flip) : other;
+      gv4i x = is_x ? (xv[u] ^ flip) : zero;
       if (!valid) x = zero;
+      if (valid) {   // this lane's 16 bytes of weight row r, as read
+        uint32_t t = (uint32_t)sl;
+        t = __builtin_amdgcn_sad_u8((uint32_t)av[u].x, 0u, t);
+        t = __builtin_amdgcn_sad_u8((uint32_t)av[u].y, 0u, t);
+        t = __builtin_amdgcn_sad_u8((uint32_t)av[u].z, 0u, t);
+        t = __builtin_amdgcn_sad_u8((uint32_t)av[u].w, 0u, t);
+        sl = (int)t - 2048;
+      }
       if (is_x && valid) {
         // the bytes as read, 128 too much each (v_sad_u8: a dot-product instruction would not run
         // beside the MFMAs)
@@ -725,6 +740,7 @@ __global__ __launch_bounds__(1024) void q8_gemv_mfma_slice_kernel(
 #pragma unroll
     for (int i = 0; i < 4; ++i) atomicAdd(&s_acc[4 * q + i][r], acc0[i] + acc1[i]);
     if (is_x) atomicAdd(&s_sx[r], sx);
+    atomicAdd(&s_sl[r], sl);
   }
   __syncthreads();
 
@@ -733,7 +749,7 @@ __global__ __launch_bounds__(1024) void q8_gemv_mfma_slice_kernel(
     const int h = h0 + row;
     if (h < H) {
       const uint32_t zl = (uint32_t)lhs_zp - 128u, zr = (uint32_t)rhs_zp - 128u;
-      const uint32_t ret = (uint32_t)s_acc[row][b] - zr * (uint32_t)s_acc[row][ONES_COL] -
+      const uint32_t ret = (uint32_t)s_acc[row][b] - zr * (uint32_t)s_sl[row] -
                            zl * (uint32_t)s_sx[b] + (uint32_t)W * zl * zr + bias_v;
       OutT *o = (OutT *)out + (int64_t)(b0 + b) * H + h;
       if constexpr (sizeof(OutT) == 4) *o = (OutT)(int32_t)ret;
@@ -756,9 +772,9 @@ int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
   if (few) nb = 2;
   // shared weights against more vectors: the batch goes through the matrix cores
   if (vec && !lhs_batched && !few && p.W >= 64 && p.batch >= 2 && p.rhs_bs % 16 == 0) {
-    dim3 grid((unsigned)((p.H + 15) / 16), (unsigned)((p.batch + 14) / 15));
+    dim3 grid((unsigned)((p.H + 15) / 16), (unsigned)((p.batch + 15) / 16));
     MH_CHECK(ctx, grid.y <= 65535, "batch too large");
-    const int nb_pass = (int)std::min<int64_t>(p.batch, 15);
+    const int nb_pass = (int)std::min<int64_t>(p.batch, 16);
     const int pitch = ((p.W / 16 + 63) / 64) * 1024 + 16;
     const size_t lds = (size_t)(16 + nb_pass) * pitch;
     const size_t lds_max = (ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536) - 2048;
@@ -784,13 +800,12 @@ int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
     } else {
       // eight wavefronts per block of 16 rows once there are four blocks per CU and more
       // (16384 x 16384: 57.5 against 61.3 us; 4096 x 9216: 13.2 against 11.7)
-      // and sixteen where the blocks of rows reach a quarter of the CUs at most: the bytes in
-      // flight per CU are then all that keeps the few busy CUs fed
-      const int nw = (int)grid.x >= 4 * ctx->cu_count ? 8 : ((int)grid.x * 4 <= ctx->cu_count ? 16 : 4);
+      // (sixteen where the blocks of rows reach a quarter of the CUs at most were slower: 1000 x
+      // 25088 against 8 vectors 29.4 against 24.1 us)
+      const int nw = (int)grid.x >= 4 * ctx->cu_count ? 8 : 4;
       mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMV_MFMA, mhv::gemv_mfma(nw, out_u8), grid, dim3(nw * 64), 0);
       MH_PROF_BEGIN(ctx);
       if (nw == 8) MH_KLAUNCH(ctx, (q8_gemv_mfma_kernel<8, 2, 4, OutT>), grid, dim3(512), 0, ctx->stream, p);
-      else if (nw == 16) MH_KLAUNCH(ctx, (q8_gemv_mfma_kernel<16, 2, 4, OutT>), grid, dim3(1024), 0, ctx->stream, p);
       else MH_KLAUNCH(ctx, (q8_gemv_mfma_kernel<4, 2, 4, OutT>), grid, dim3(256), 0, ctx->stream, p);
     }
     MH_PROF_END(ctx);

@@ -166,8 +166,8 @@ FAMILY_CASES = [  # batch, h, w, lhs batched, kernel (without the output type)
     (5, 77, 2048, False, "q8_gemv_mfma_slice_kernel<SPW=2"),
     (15, 33, 1024, False, "q8_gemv_mfma_slice_kernel<SPW=1"),
     (3, 45, 8192, False, "q8_gemv_mfma_lds_kernel<16"),
-    (8, 45, 9216, False, "q8_gemv_mfma_kernel<NW=16,GROUP=2,NBUF=4"),
-    (15, 45, 9232, False, "q8_gemv_mfma_kernel<NW=16,GROUP=2,NBUF=4"),   # a ragged last k step
+    (8, 45, 9216, False, "q8_gemv_mfma_kernel<NW=4,GROUP=2,NBUF=4"),
+    (16, 45, 9232, False, "q8_gemv_mfma_kernel<NW=4,GROUP=2,NBUF=4"),    # a ragged last k step, a full pass
     (8, 1100, 8208, False, "q8_gemv_mfma_kernel<NW=4,GROUP=2,NBUF=4"),   # shares of 32.25 k steps
     (4, 4112, 8192, False, "q8_gemv_mfma_kernel<NW=4,GROUP=2,NBUF=4"),   # more row blocks than CUs
     (3, 16400, 4608, False, "q8_gemv_mfma_kernel<NW=8,GROUP=2,NBUF=4"),
