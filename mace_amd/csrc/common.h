@@ -189,7 +189,7 @@ enum { XRES_PLAIN = 0, XRES_XT = 1, XRES_TAIL = 2, XRES_CONV = 3 };
 inline int xres(int mode, int fx, int fy, int group, bool out_u8) {
   return ((((mode * 2 + (fx == 4)) * 2 + (fy == 2)) * 2 + (group == 128)) * 2) + (out_u8 ? 1 : 0);
 }
-inline int mid(bool out_u8, bool xt) { return (xt ? 2 : 0) | (out_u8 ? 1 : 0); }
+inline int mid(bool out_u8, bool xt, bool yt = false) { return (yt ? 4 : 0) | (xt ? 2 : 0) | (out_u8 ? 1 : 0); }
 inline int stream(int fx, int ks) { return (fx - 1) * 2 + (ks - 1); }
 // tile configurations of the ring kernel: <WX, WY, FX, FY, STAGES, OCC, KB>
 enum { RING_1422_3_2 = 0, RING_2222_3_3, RING_2244_2_1_128, RING_2421_2_1_128, RING_2222_2_2_128,

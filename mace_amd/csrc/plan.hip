@@ -14,7 +14,7 @@ const int kVariantCount[MACE_HIP_KF_COUNT] = {
     0,
     16,                       // Q8_GEMM_FUSED_SMALL
     64,                       // Q8_GEMM_XRES
-    4,                        // Q8_GEMM_MID
+    8,                        // Q8_GEMM_MID
     8,                        // Q8_GEMM_STREAM
     mhv::RING_CONFIGS * 8,    // Q8_GEMM_RING
     8,                        // Q8_GEMM_RING_XT
@@ -130,7 +130,7 @@ int mace_hip_plan_describe(int family, int v, char *buf, size_t len) {
       break;
     }
     case MACE_HIP_KF_Q8_GEMM_MID:
-      snprintf(buf, len, "%s<%s,STAGES=4,XT=%s>", k, out_name(v & 1), tf(v & 2));
+      snprintf(buf, len, "%s<%s,STAGES=4,XT=%s,YT=%s>", k, out_name(v & 1), tf(v & 2), tf(v & 4));
       break;
     case MACE_HIP_KF_Q8_GEMM_STREAM:
       snprintf(buf, len, "%s<FX=%d,KS=%d,XW=1,4>", k, v / 2 + 1, v % 2 + 1);

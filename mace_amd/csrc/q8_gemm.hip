@@ -1127,9 +1127,12 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
 //     register contents the k-contiguous layout gives, and everything behind the read is shared.
 //     The swizzle puts the 16 pieces of two neighbouring 16-lane groups into 16 distinct bank
 //     groups.
-// Requirements (checked by the host): K % 128 == 0, rows addressable with 32-bit offsets; XT: XN a
-// multiple of 16, 16-byte aligned base, the whole operand within 32-bit offsets.
-template <typename OutT, int STAGES, bool XT>
+//   * YT: the same for the Y operand (Y(y, k) at Y[k * ldy + y]: the ColMajor left-hand matrix of a
+//     MatMul with transpose_a and a RowMajor result); the MFMA's two operands have the same register
+//     layout, so the Y half of a slab and its fragment reads mirror the X half's.
+// Requirements (checked by the host): K % 128 == 0, rows addressable with 32-bit offsets; XT / YT:
+// XN / YN a multiple of 16, 16-byte aligned base, the whole operand within 32-bit offsets.
+template <typename OutT, int STAGES, bool XT, bool YT = false>
 __global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel(GemmParams p, RequantTable) {
   constexpr int KB = 128, T = 128, NW = 8;
   constexpr int RPI = 1024 / KB, CPR = KB / 16;
@@ -1152,7 +1155,7 @@ __global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
   const int x0 = tile_x * T, y0 = tile_y * T;
   const int b = blockIdx.z;
   const uint8_t *Xt = XT ? p.X + (int64_t)b * p.xbs + x0 : p.X + (int64_t)b * p.xbs + (int64_t)x0 * p.ldx;
-  const uint8_t *Yt = p.Y + (int64_t)b * p.ybs + (int64_t)y0 * p.ldy;
+  const uint8_t *Yt = YT ? p.Y + (int64_t)b * p.ybs + y0 : p.Y + (int64_t)b * p.ybs + (int64_t)y0 * p.ldy;
 
   // transfer j of this wavefront fills slab rows [(j*NW + wave)*RPI, +RPI): rows 0..127 are X rows,
   // 128..255 Y rows; lane l lands in row l / CPR, slot l % CPR and fetches chunk slot ^ swizzle.
@@ -1167,12 +1170,16 @@ __global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
         off[j] = (uint32_t)r * (uint32_t)p.ldx + min(((lane % CPR) ^ (r & 6)) * 16, p.XN - 16 - x0);
       else off[j] = (uint32_t)(min(x0 + r, p.XN - 1) - x0) * (uint32_t)p.ldx + kc * 16;
     } else {
-      off[j] = (uint32_t)(min(y0 + r - T, p.YN - 1) - y0) * (uint32_t)p.ldy + kc * 16;
+      if constexpr (YT)
+        off[j] = (uint32_t)(r - T) * (uint32_t)p.ldy + min(((lane % CPR) ^ (r & 6)) * 16, p.YN - 16 - y0);
+      else off[j] = (uint32_t)(min(y0 + r - T, p.YN - 1) - y0) * (uint32_t)p.ldy + kc * 16;
     }
   }
   const mh_rsrc rsx = dma_rsrc(Xt), rsy = dma_rsrc(Yt);
   auto dma_one = [&](int j, int stage, int k0) {
-    const uint32_t uo = (XT && j < NL / 2) ? (uint32_t)k0 * (uint32_t)p.ldx : (uint32_t)k0;
+    const uint32_t uo = (XT && j < NL / 2)    ? (uint32_t)k0 * (uint32_t)p.ldx
+                        : (YT && j >= NL / 2) ? (uint32_t)k0 * (uint32_t)p.ldy
+                                              : (uint32_t)k0;
     dma_16B(j < NL / 2 ? rsx : rsy, off[j], uo, lds + stage * STAGE_BYTES + (j * NW + wave) * 1024);
   };
 
@@ -1196,15 +1203,17 @@ __global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
   // XT: lane l of a 16-lane group points at k row 16 (l / 32) + (l % 16) / 2 of the k step, 8 bytes at
   // x = 32 (2 wx + i) + 16 ((l / 16) % 2) + 8 (l % 2); the second read is 8 k rows (1 KiB) further
   int xt_off[2][2], rxt[2][2];   // [step of the wavefront][32-row block i]
-  if constexpr (XT) {
+  int yt_off[2][2], ryt[2][2];   // YT: the same inside the Y half of a stage
+  if constexpr (XT || YT) {
     const int t = (lane & 15) >> 1;
 #pragma unroll
     for (int q = 0; q < 2; ++q)
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
-        const int c = (wx * 2 + i) * 2 + ((lane >> 4) & 1);
         const int krow = 32 * (2 * grp + (q ^ par)) + 16 * (lane >> 5) + t;
-        xt_off[q][i] = (krow * 8 + (c ^ (t & 6))) * 16 + 8 * (lane & 1);
+        const int cx = (wx * 2 + i) * 2 + ((lane >> 4) & 1), cy = (wy * 2 + i) * 2 + ((lane >> 4) & 1);
+        xt_off[q][i] = (krow * 8 + (cx ^ (t & 6))) * 16 + 8 * (lane & 1);
+        yt_off[q][i] = Y_OFF + (krow * 8 + (cy ^ (t & 6))) * 16 + 8 * (lane & 1);
       }
   }
   auto point_reads_at = [&](int stage) {
@@ -1215,6 +1224,10 @@ __global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
       if constexpr (XT) {
         rxt[q][0] = xt_off[q][0] + stage * STAGE_BYTES;
         rxt[q][1] = xt_off[q][1] + stage * STAGE_BYTES;
+      }
+      if constexpr (YT) {
+        ryt[q][0] = yt_off[q][0] + stage * STAGE_BYTES;
+        ryt[q][1] = yt_off[q][1] + stage * STAGE_BYTES;
       }
     }
   };
@@ -1228,6 +1241,17 @@ __global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
       return *(const v4i *)(lds + rx[q] + i * 32 * KB);
     }
   };
+  auto read_y = [&](int q, int j) -> v4i {
+    if constexpr (YT) {
+      const v2i_t lo = lds_read_tr8<0>(lds_base + ryt[q][j]);
+      const v2i_t hi = lds_read_tr8<1024>(lds_base + ryt[q][j]);
+      return v4i{lo.x, lo.y, hi.x, hi.y};
+    } else {
+      return *(const v4i *)(lds + ry[q] + j * 32 * KB);
+    }
+  };
+  // LDS instructions per fragment read: what the explicit waits for the transposing reads count
+  constexpr int NX = XT ? 2 : 1, NY = YT ? 2 : 1;
   const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
   v4i fa[2][2], fb[2][2];   // set 0: first k step of a slab, set 1: second
 
@@ -1244,11 +1268,11 @@ __global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
       acc[m >> 1][m & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[CUR][m >> 1], fb[CUR][m & 1],
                                                                  acc[m >> 1][m & 1], 0, 0, 0);
       if (m < 2) fa[OTH][m] = read_x(OTH, m);
-      else fb[OTH][m - 2] = *(const v4i *)(lds + ry[OTH] + (m - 2) * 32 * KB);
+      else fb[OTH][m - 2] = read_y(OTH, m - 2);
       if (m >= 2) {
-        // XT: issued since X fragment m - 2 was read: the other X fragment's two reads (m = 2 only)
-        // and the Y fragments' reads so far
-        if constexpr (XT) lds_wait_tr(fa[OTH][m - 2], m == 2 ? 3 : 2);
+        // XT: issued since X fragment m - 2 was read: the other X fragment's reads (m = 2 only) and
+        // the Y fragments' reads so far
+        if constexpr (XT) lds_wait_tr(fa[OTH][m - 2], m == 2 ? NX + NY : 2 * NY);
         if constexpr (OTH == 0) xs[m - 2] = sum16_u8(fa[OTH][m - 2], xs[m - 2]);
         fa[OTH][m - 2] ^= flip;
       }
@@ -1257,6 +1281,7 @@ __global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
+      if constexpr (YT) lds_wait_tr(fb[OTH][j], j == 0 ? NY : 0);   // (nothing was read after the Y fragments)
       if constexpr (OTH == 1) ys[j] = sum16_u8(fb[OTH][j], ys[j]);
       fb[OTH][j] ^= flip;
     }
@@ -1275,8 +1300,9 @@ __global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
 #pragma unroll
   for (int m = 0; m < 2; ++m) {
     fa[0][m] = read_x(0, m);
-    fb[0][m] = *(const v4i *)(lds + ry[0] + m * 32 * KB);
+    fb[0][m] = read_y(0, m);
     if constexpr (XT) lds_wait_tr(fa[0][m], 0);
+    if constexpr (YT) lds_wait_tr(fb[0][m], 0);
     xs[m] = sum16_u8(fa[0][m], xs[m]);
     fa[0][m] ^= flip;
     fb[0][m] ^= flip;
@@ -2213,20 +2239,28 @@ int launch_gemm_dma(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, b
 
 // one round of 128 x 128 tiles; the caller has checked K % 128 == 0 and the 32-bit row offsets
 int launch_gemm_mid(mace_hip_ctx *ctx, GemmParams &p, const RequantTable &tab, bool out_u8, int batch,
-                    bool xt = false) {
+                    bool xt = false, bool yt = false) {
   constexpr int STAGES = 4;
   p.tiles_x = (p.XN + 127) / 128;
   p.tiles_y = (p.YN + 127) / 128;
   const size_t lds = (size_t)STAGES * 256 * 128;
   dim3 grid(p.tiles_x * p.tiles_y, 1, batch), block(512);
-  mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMM_MID, mhv::mid(out_u8, xt), grid, block, lds);
+  mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMM_MID, mhv::mid(out_u8, xt, yt), grid, block, lds);
   auto launch = [&](auto k) -> int {
     MH_HIP(ctx, mh_allow_big_lds(ctx, (const void *)k, lds));
     MH_PROF_BEGIN(ctx);
     MH_KLAUNCH(ctx, k, grid, block, lds, ctx->stream, p, tab);
     return MACE_HIP_SUCCESS;
   };
-  if (xt) {
+  if (yt) {
+    if (xt) {
+      if (out_u8) MH_RETURN_IF_ERROR(launch(q8_gemm_mid_kernel<uint8_t, STAGES, true, true>));
+      else MH_RETURN_IF_ERROR(launch(q8_gemm_mid_kernel<int32_t, STAGES, true, true>));
+    } else {
+      if (out_u8) MH_RETURN_IF_ERROR(launch(q8_gemm_mid_kernel<uint8_t, STAGES, false, true>));
+      else MH_RETURN_IF_ERROR(launch(q8_gemm_mid_kernel<int32_t, STAGES, false, true>));
+    }
+  } else if (xt) {
     if (out_u8) MH_RETURN_IF_ERROR(launch(q8_gemm_mid_kernel<uint8_t, STAGES, true>));
     else MH_RETURN_IF_ERROR(launch(q8_gemm_mid_kernel<int32_t, STAGES, true>));
   } else {
@@ -2537,7 +2571,7 @@ struct Q8Call {
   bool lhs_direct = false, rhs_direct = false;   // the operand can be read in place
   bool cv_small = false;                 // a gathered convolution that is a small problem
   mh_weight *lhs_w = nullptr, *rhs_w = nullptr;  // registered as constant weights
-  bool mid_first_xt = false, mid_first_kc = false;   // the eight-wavefront kernel goes first
+  bool mid_first_xt = false, mid_first_kc = false, mid_first_yt = false;   // the eight-wavefront kernel goes first
   bool tail_xres = false;                // depth % 64 != 0 read in place by the resident-tile kernel
 
   int prepare(bool *done);
@@ -2630,6 +2664,14 @@ int Q8Call::prepare(bool *done) {
                             (uintptr_t)(mid_xl ? lhs : rhs) % 16 == 0 &&
                             mid_xn * depth < ((int64_t)1 << 32);
   mid_first_kc = mid_one_round && mid_x_direct && mid_y_direct && depth >= 1024;
+  //   Y k-major (X k-major or k-contiguous), against the one-launch kernel: 1024^3 with both
+  //     operands k-major 15.6 -> 10.4
+  const bool mid_y_kmajor = mid_xl ? rhs_order == MACE_HIP_ROW_MAJOR : lhs_order == MACE_HIP_COL_MAJOR;
+  const bool mid_x_in_place = mid_x_kmajor ? (mid_xn % 16 == 0 && (uintptr_t)(mid_xl ? lhs : rhs) % 16 == 0 &&
+                                              mid_xn * depth < ((int64_t)1 << 32))
+                                           : mid_x_direct;
+  mid_first_yt = mid_one_round && mid_y_kmajor && mid_x_in_place && mid_yn % 16 == 0 &&
+                 (uintptr_t)(mid_xl ? rhs : lhs) % 16 == 0 && mid_yn * depth < ((int64_t)1 << 32);
 
   // A depth that is a multiple of 16 but not of 64, both operands k-contiguous and read in place, a
   // long Y panel and an X tile that fits in LDS: the resident-tile kernel walks k up to the next
@@ -2675,6 +2717,7 @@ int Q8Call::small_problem(bool *done) {
                           : (mh_q8_small_problem(ctx, batch, rows, cols, depth, lhs_vec && rhs_vec,
                                                  any_size) &&
                              ((!lhs_w && !rhs_w) || any_size) && !mid_first_xt && !mid_first_kc &&
+                             !mid_first_yt &&
                              !(ctx->kernel_mask & MH_MASK_NO_SMALL));
     if (small) {
       const bool xt = xl ? lhs_t : rhs_t, yt = xl ? rhs_t : lhs_t;
@@ -2770,6 +2813,31 @@ int Q8Call::kmajor_in_place(bool *done) {
       if (out_u8 && rq.table) mh_requant_table_cached(ctx, rq, tab.t);
       *done = true;
       return launch_gemm_mid(ctx, p, tab, out_u8, (int)batch, true);
+    }
+    // A k-major Y operand (the ColMajor left-hand matrix of a transpose_a MatMul with a RowMajor
+    // result; X k-major as well, or k-contiguous and read in place) in the same tile-count range:
+    // the eight-wavefront kernel's Y half mirrors its X half, so neither operand is repacked.
+    {
+      const bool y_kmajor = xl ? rhs_order == MACE_HIP_ROW_MAJOR : lhs_order == MACE_HIP_COL_MAJOR;
+      const bool x_direct = xl ? lhs_direct : (rhs_direct && rhs_order == MACE_HIP_COL_MAJOR);
+      const bool x_ok = x_kmajor ? (xn % 16 == 0 && (uintptr_t)xp % 16 == 0 && xn * depth < ((int64_t)1 << 32))
+                                 : x_direct;
+      if (!cv && y_kmajor && x_ok && rhs_ld == 0 && !lhs_w && !rhs_w && depth >= 512 &&
+          depth % 128 == 0 && yn % 16 == 0 && (uintptr_t)yp % 16 == 0 && xn > 64 && yn > 64 &&
+          4 * tiles128 >= cu_n &&
+          (tiles128 <= cu_n || (depth >= 2048 && 2 * tiles128 <= 5 * cu_n) ||
+           (depth >= 1024 && tiles128 <= 2 * cu_n)) &&
+          yn * depth < ((int64_t)1 << 32) && depth < (1 << 24) && (size_t)4 * 256 * 128 <= lds_cu &&
+          !(ctx->kernel_mask & MH_MASK_NO_MID)) {
+        const Q8Operand Xo{xp, x_kmajor ? xn : depth, (xl ? lhs_nb : rhs_nb) > 1 ? xn * depth : 0};
+        const Q8Operand Yo{yp, yn, (xl ? rhs_nb : lhs_nb) > 1 ? yn * depth : 0};
+        GemmParams p = q8_params(xl, xl ? Xo : Yo, xl ? Yo : Xo, rows, cols, depth, (int)depth, out,
+                                 out_u8, rq, lhs_offset, rhs_offset, ep.bias);
+        RequantTable tab;
+        if (out_u8 && rq.table) mh_requant_table_cached(ctx, rq, tab.t);
+        *done = true;
+        return launch_gemm_mid(ctx, p, tab, out_u8, (int)batch, x_kmajor, true);
+      }
     }
     // ... and where the 256 x 256 tiles are the choice: the ring kernel's k-major variant; the
     // operand's sums come from a pass over it as it lies.  Measured against repack + k-contiguous

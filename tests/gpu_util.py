@@ -57,7 +57,9 @@ def kernel_tag(plan):
     a k-major operand was read in place, /TAIL where a depth tail was, /CONV where patches were
     gathered: what the family-aimed parity tests assert."""
     tag = _TAGS.get(plan.family, plan.kernel)
-    for flag in ("XT", "TAIL", "CONV"):
+    for flag in ("XT", "YT", "TAIL", "CONV"):
+        if flag == "YT" and plan.family != mh.KF_Q8_GEMM_MID:
+            continue      # (only the eight-wavefront kernel's k-major Y is told apart)
         if (flag + "=true") in plan.kernel and plan.family != mh.KF_Q8_GEMM_RING_XT:
             tag += "/" + flag
     return tag

@@ -146,7 +146,7 @@ def test_q8_gemm_x_panel_in_lds(ctx, path, batch, rows, depth, cols, lo, ro, oo,
 MID_SHAPES = [  # batch, rows, depth, cols, lhs batched, rhs batched, lhs order, rhs order, out order, kernel
     (1, 1500, 640, 1410, True, True, R, Cm, R, "mid"), (1, 1408, 512, 1536, True, True, R, R, R, "mid/XT"),
     (1, 1537, 768, 1300, True, True, Cm, R, Cm, "mid"), (2, 1100, 896, 1000, True, True, R, Cm, R, "mid"),
-    (2, 1024, 512, 1100, False, True, Cm, Cm, R, "mid"), (1, 2048, 1024, 2048, True, True, R, Cm, Cm, "mid"),
+    (2, 1024, 512, 1100, False, True, Cm, Cm, R, "mid/YT"), (1, 2048, 1024, 2048, True, True, R, Cm, Cm, "mid"),
     (3, 900, 512, 1000, True, False, R, R, Cm, "mid"),
     # both ends of the range of tile counts it takes: a quarter of a round, more than one round
     (1, 1000, 512, 1024, True, True, R, Cm, R, "mid"), (1, 2300, 2048, 2200, True, True, R, Cm, R, "mid"),
@@ -156,6 +156,13 @@ MID_SHAPES = [  # batch, rows, depth, cols, lhs batched, rhs batched, lhs order,
     (1, 1536, 1024, 1488, True, True, R, R, R, "mid/XT"), (2, 1000, 640, 1040, True, True, R, R, R, "mid/XT"),
     (1, 1296, 1280, 1500, True, True, Cm, Cm, Cm, "mid/XT"), (2, 1100, 512, 1200, True, False, R, R, R, "mid/XT"),
     (1, 2048, 2048, 2048, True, True, R, R, R, "mid/XT"),
+    # Y operand k-major in memory (ColMajor left-hand matrix with a RowMajor result: a transpose_a
+    # MatMul; RowMajor right-hand matrix with a ColMajor result), X k-major as well or k-contiguous:
+    # neither is repacked; ragged last tiles, batches, one side shared
+    (1, 1536, 1024, 1488, True, True, Cm, R, R, "mid/XT/YT"), (1, 1408, 512, 1500, True, True, Cm, Cm, R, "mid/YT"),
+    (2, 1040, 640, 1008, True, True, Cm, R, R, "mid/XT/YT"), (1, 1296, 1280, 1504, True, True, R, R, Cm, "mid/YT"),
+    (1, 2048, 2048, 2048, True, True, Cm, R, R, "mid/XT/YT"), (3, 912, 512, 1008, True, False, Cm, R, R, "mid/XT/YT"),
+    (2, 1024, 768, 1100, False, True, Cm, Cm, R, "mid/YT"),
     # the same operand layout at sizes that take 256 x 256 tiles: each operand's sums in the kernel
     # (k <= 1024 or the other dimension <= 4096) or from a pass of their own, ragged last tiles,
     # ColMajor everything

@@ -64,7 +64,7 @@ def test_config1_matmul_is_one_launch(ctx):
 
 def test_config5_gemm_sweep(ctx):
     p = gemm(ctx, 1, 2048, 2048, 2048)
-    assert p.kernel == "q8_gemm_mid_kernel<uint8_t,STAGES=4,XT=true>" and p.launches == 1
+    assert p.kernel == "q8_gemm_mid_kernel<uint8_t,STAGES=4,XT=true,YT=false>" and p.launches == 1
     assert p.grid == (256, 1, 1) and p.block == 512
     p = gemm(ctx, 1, 4096, 4096, 4096)
     assert p.family == mh.KF_Q8_GEMM_RING_XT and p.launches == 1
@@ -98,7 +98,7 @@ def test_config4_conv1x1_batch64(ctx):
             (56, 128, 128): "q8_gemm_xres_kernel<FX=4,FY=1,G=128,uint8_t,OCC=2,CONV=false,XT=false,TAIL=false>",
             (28, 256, 256): "q8_gemm_xres_kernel<FX=4,FY=1,G=128,uint8_t,OCC=2,CONV=false,XT=false,TAIL=false>",
             (14, 512, 512): "q8_gemm_xres_kernel<FX=4,FY=1,G=128,uint8_t,OCC=2,CONV=false,XT=false,TAIL=false>",
-            (7, 1024, 1024): "q8_gemm_mid_kernel<uint8_t,STAGES=4,XT=false>"}
+            (7, 1024, 1024): "q8_gemm_mid_kernel<uint8_t,STAGES=4,XT=false,YT=false>"}
     for (hw, cin, cout), kernel in want.items():
         p = conv(ctx, 64, hw, cin, cout)
         assert p.kernel == kernel, (hw, p)
@@ -160,11 +160,20 @@ def test_eight_wavefront_kernel_range(ctx):
     # k-contiguous operands at k = 512 stay with the one-launch kernel; a k-major X does not
     assert fam(gemm(ctx, 4, 512, 512, 512, ro=Cm)) == mh.KF_Q8_GEMM_FUSED_SMALL
     p = gemm(ctx, 4, 512, 512, 512)
-    assert p.kernel == "q8_gemm_mid_kernel<uint8_t,STAGES=4,XT=true>"
+    assert p.kernel == "q8_gemm_mid_kernel<uint8_t,STAGES=4,XT=true,YT=false>"
     # k-major X: two rounds of tiles from k = 1024 on
     assert fam(gemm(ctx, 8, 1024, 1024, 1024)) == mid and gemm(ctx, 8, 1024, 1024, 1024).grid == (64, 1, 8)
     assert fam(gemm(ctx, 1, 3072, 1024, 3072)) != mid                 # 576 tiles
     assert fam(gemm(ctx, 1, 2048, 2048, 2048, mask=mh.MASK_NO_MID)) != mid
+    # k-major Y (transpose_a with a RowMajor result), X k-major or k-contiguous: read as they lie
+    p = gemm(ctx, 1, 2048, 2048, 2048, lo=Cm)
+    assert p.kernel == "q8_gemm_mid_kernel<uint8_t,STAGES=4,XT=true,YT=true>" and p.launches == 1 and p.aux == 0
+    p = gemm(ctx, 1, 2048, 2048, 2048, lo=Cm, ro=Cm, u8=False)
+    assert p.kernel == "q8_gemm_mid_kernel<int32_t,STAGES=4,XT=false,YT=true>" and p.launches == 1
+    p = gemm(ctx, 1, 2048, 2048, 2048, lo=R, ro=R, oo=Cm)            # ColMajor result: Y is the right-hand matrix
+    assert p.kernel == "q8_gemm_mid_kernel<uint8_t,STAGES=4,XT=false,YT=true>"
+    p = gemm(ctx, 1, 2040, 2048, 2048, lo=Cm)                        # rows not in whole 16-byte pieces: repacked
+    assert "YT=true" not in p.kernel and p.launches > 1
 
 
 def test_resident_tile_kernel_range(ctx):
@@ -313,7 +322,7 @@ def test_variant_tables_are_consistent():
         total += len(vs)
         assert not lib.mace_hip_plan_variant_valid(f, n) and not lib.mace_hip_plan_variant_valid(f, -1)
         assert mh.coverage(f, 0) == 0              # nothing is launched by planning
-    assert total == 221
+    assert total == 225
     assert lib.mace_hip_plan_variant_count(0) == 0 and lib.mace_hip_plan_variant_count(mh.KF_COUNT) == 0
 
 
