@@ -780,6 +780,7 @@ int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
     const size_t lds_max = (ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536) - 2048;
     if (p.W <= 4096 && lds_max >= 140 * 1024) {
       // rows of at most 4 KiB: every wavefront on a k slice of its own
+      // (the ring of direct loads below takes 4096 x 4096 against 8 vectors in 6.13 us, this 5.99)
       const int spw = p.W <= 1024 ? 1 : (p.W <= 2048 ? 2 : 4);
       mh_plan_main(ctx, MACE_HIP_KF_Q8_GEMV_SLICE, mhv::gemv_slice(spw, out_u8), grid, dim3(1024), 0);
       MH_PROF_BEGIN(ctx);
