@@ -104,6 +104,9 @@ int mace_hip_plan_variant_valid(int family, int v) {
       if (conv) return sum_y && (v & 1) && kRing[cfg][6] == 64 && kRing[cfg][4] == 4;
       return 1;
     }
+    case MACE_HIP_KF_Q8_GEMM_TILED:
+      // the 256 x 256 instantiation is switched off (see the end of Q8Call::general)
+      return (v >> 2) != mhv::TILED_BIG;
     case MACE_HIP_KF_Q8_GEMV_GENERAL:
       // 16-byte pieces (VEC) reach the general kernel with one vector per pass only
       return !((v & 2) && (v >> 2) != 0);

@@ -102,6 +102,35 @@ def test_conv1x1_q8_errors(ctx):
     assert st == mh.INVALID_ARGS and "multiplier" in ctx.last_error()
 
 
+# Channel counts that are odd multiples of 8 (MobileNetV2's 24, 40, 72, 120 ...): read in place by the
+# resident-tile kernel's depth tail; small cases go to the one-launch kernel unless it is masked out.
+@pytest.mark.parametrize("n,hw,cin,cout", [(2, 56, 24, 144), (3, 28, 40, 64), (1, 30, 72, 200),
+                                           (2, 20, 120, 128), (1, 17, 24, 16), (1, 64, 88, 48),
+                                           (5, 14, 200, 96), (8, 56, 24, 144)])
+@pytest.mark.parametrize("one_launch_kernel", [True, False])
+def test_conv1x1_q8_channels_odd_multiple_of_8(ctx, one_launch_kernel, n, hw, cin, cout):
+    rng = np.random.default_rng(hw * 5 + cin)
+    x = rng.integers(0, 256, (n, hw, hw, cin), dtype=np.uint8)
+    f = rng.integers(0, 256, (cout, cin), dtype=np.uint8)
+    bias = rng.integers(-2 ** 15, 2 ** 15, cout).astype(np.int32)
+    z_in, z_f, z_o = int(rng.integers(0, 256)), int(rng.integers(0, 256)), int(rng.integers(0, 256))
+    s_in, s_f = np.float32(0.02), np.float32(0.01)
+    s_o = np.float32(max(1.0, 3 * 74.0 * 74.0 * np.sqrt(cin) * float(s_in * s_f)) / 255.0)
+    want = orc.conv1x1_q8_nhwc(x, f, bias, n, hw, hw, cin, cout, s_in, z_in, s_f, z_f,
+                               np.float32(s_in * s_f), s_o, z_o)
+    ctx.call("mace_hip_ctx_set_kernel_mask", 0 if one_launch_kernel else mh.MASK_NO_SMALL)
+    try:
+        got = conv_host(ctx, x, f, bias, n, hw, hw, cin, cout, s_in, z_in, s_f, z_f,
+                        np.float32(s_in * s_f), s_o, z_o)
+        plan = ctx.last_plan()
+    finally:
+        ctx.call("mace_hip_ctx_set_kernel_mask", 0)
+    np.testing.assert_array_equal(got, want)
+    assert len(np.unique(want)) > 20
+    if not one_launch_kernel and n * hw * hw >= 256:
+        assert "TAIL=true" in plan.kernel and plan.launches == 1
+
+
 @pytest.mark.parametrize("hw,cin,cout", [(112, 32, 64), (56, 128, 128), (28, 256, 256),
                                          (14, 512, 512), (7, 1024, 1024)])
 def test_conv1x1_q8_batch64_sampled(ctx, hw, cin, cout):

@@ -236,6 +236,23 @@ def test_q8_gemm_depth_tail_in_place(ctx, kernels, batch, rows, depth, cols, lb,
     assert tags == (("xres/TAIL", "xres/TAIL") if kernels == "normal" else ("small", "small"))
 
 
+# Depths that are odd multiples of 8 (24, 40, 72 ... channels): the same kernel reads half a piece
+# at the end of every row, and rows start at 8-byte boundaries only.  64- and 128-row tiles, ragged
+# rows and columns, the result transposed, batches (shared and per-batch operands).
+HALF_TAIL_SHAPES = [
+    (1, 40000, 24, 128, True, True, R, Cm, R), (1, 70000, 88, 64, True, True, R, Cm, R),
+    (1, 35003, 104, 200, True, True, R, Cm, R), (2, 20000, 40, 130, True, True, R, Cm, R),
+    (1, 128, 72, 40000, True, True, R, Cm, Cm), (1, 20000, 328, 256, True, True, R, Cm, R),
+    (3, 14000, 56, 128, True, False, R, Cm, R), (1, 280000, 24, 48, True, True, R, Cm, R),
+    (1, 90000, 120, 17, True, True, R, Cm, R),
+]
+
+
+@pytest.mark.parametrize("batch,rows,depth,cols,lb,rb,lo,ro,oo", HALF_TAIL_SHAPES)
+def test_q8_gemm_depth_tail_of_half_a_piece(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo):
+    assert check_gemm(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo) == ("xres/TAIL", "xres/TAIL")
+
+
 def test_q8_gemm_config1_matmul(ctx):
     """benchmark configuration 1: A [128x256], B [256x128], zero points 128/128/128, scales
     0.02/0.015/0.05 -> (1649267328, shift 7)."""

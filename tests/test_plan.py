@@ -200,6 +200,23 @@ def test_resident_tile_kernel_range(ctx):
     assert fam(gemm(ctx, 1, 200704, 128, 128, ro=Cm, mask=mh.MASK_NO_XRES)) == mh.KF_Q8_GEMM_RING
 
 
+def test_depth_that_is_an_odd_multiple_of_8_in_place(ctx):
+    # 24, 40, 72 ... input channels of a 1x1 convolution: the resident-tile kernel's depth tail reads
+    # both operands as they lie (half a 16-byte piece at the end of every row), one launch
+    for (n, hw, cin, cout) in ((64, 56, 24, 144), (64, 28, 40, 240), (64, 14, 72, 432), (16, 28, 120, 128)):
+        p = conv(ctx, n, hw, cin, cout)
+        assert p.family == mh.KF_Q8_GEMM_XRES and "TAIL=true" in p.kernel and p.launches == 1, (cin, p.kernel)
+    p = gemm(ctx, 1, 40000, 88, 64, ro=Cm)
+    assert "TAIL=true" in p.kernel and p.launches == 1
+    # not for it: a short Y panel, 8 channels (no whole piece in front of the half one), an operand
+    # that is not k-contiguous, an address that is not a multiple of 8
+    assert "TAIL=true" not in conv(ctx, 1, 10, 24, 144).kernel
+    assert "TAIL=true" not in conv(ctx, 64, 56, 8, 144).kernel
+    assert "TAIL=true" not in gemm(ctx, 1, 40000, 88, 64).kernel
+    assert "TAIL=true" not in gemm(ctx, 1, 40000, 88, 64, ro=Cm, b=B + 4).kernel
+    assert "TAIL=true" not in gemm(ctx, 1, 40000, 88, 64, ro=Cm, mask=mh.MASK_NO_XRES).kernel
+
+
 def test_streaming_kernel_shapes(ctx):
     st = mh.KF_Q8_GEMM_STREAM
     p = gemm(ctx, 1, 64, 32, 802816, lo=R, ro=Cm, oo=Cm)
@@ -252,6 +269,14 @@ def test_tile_shapes_of_the_ring_kernel(ctx):
     # depths the ring cannot take (not whole slabs, or fewer than three): the register-staged kernel
     p = gemm(ctx, 1, 300, 100, 260, ro=Cm, mask=off)
     assert p.family == mh.KF_Q8_GEMM_TILED and p.aux & mh.AUX_PACK_ROWS
+    # the 256 x 256 instantiation of that kernel is switched off: the shapes whose tile choice is
+    # 256 x 256 take 128 x 128 tiles
+    p = conv(ctx, 64, 56, 24, 144, mask=mh.MASK_NO_XRES)
+    assert p.family == mh.KF_Q8_GEMM_TILED and "<2,2,2,2," in p.kernel
+    p = gemm(ctx, 1, 200704, 24, 144, ro=Cm, oo=Cm)       # a short Y panel: no resident-tile kernel
+    assert p.family == mh.KF_Q8_GEMM_TILED and "<2,2,2,2," in p.kernel
+    for v in range(4):
+        assert not mh.load().mace_hip_plan_variant_valid(mh.KF_Q8_GEMM_TILED, v)
 
 
 def test_convolution_gather_and_im2col(ctx):
@@ -322,7 +347,7 @@ def test_variant_tables_are_consistent():
         total += len(vs)
         assert not lib.mace_hip_plan_variant_valid(f, n) and not lib.mace_hip_plan_variant_valid(f, -1)
         assert mh.coverage(f, 0) == 0              # nothing is launched by planning
-    assert total == 225
+    assert total == 221
     assert lib.mace_hip_plan_variant_count(0) == 0 and lib.mace_hip_plan_variant_count(mh.KF_COUNT) == 0
 
 
