@@ -1486,8 +1486,8 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
   // TAIL: K is a multiple of 8 (from 24 on) but not of 64.  k is walked up to the next multiple of 64;
   // the 16-byte pieces past K are not fetched (their addresses are clamped to the row's first piece)
   // and count as zeros after the shift on both sides; where K is an odd multiple of 8 the last
-  // piece is half a piece (rows then start at 8-byte boundaries only: the 16-byte loads and
-  // transfers take any 4-byte aligned address).
+  // piece is half a piece (rows then start at 8-byte boundaries only, which ordinary 16-byte loads
+  // accept; the X tile is then staged through registers, see below).
   const int KP = TAIL ? (p.K + 63) & ~63 : p.K;
   const int ngroup = KP / G;
   const int stride = gridDim.x * 4;
@@ -1604,6 +1604,10 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
       src_kc[j] = kc * 16;
       src[j] = Xb + (int64_t)min(x0 + row, p.XN - 1) * p.ldx + kc * 16;
     }
+    // TAIL with K an odd multiple of 8: rows start at 8-byte boundaries only.  The transfers into
+    // LDS are kept to 16-byte aligned addresses; such a tile goes through registers instead
+    // (ordinary 16-byte loads take any address), same slots.
+    const bool by_registers = TAIL && (p.K & 15) != 0;
     for (int s = 0; s < nslab; ++s) {
 #pragma unroll
       for (int j = 0; j < LX; ++j) {
@@ -1611,8 +1615,10 @@ __global__ __launch_bounds__(256, OCC) void q8_gemm_xres_kernel(GemmParams p, Re
         // halfway starts 8 bytes early; the pass below zeroes the one and moves the other down
         const bool past = TAIL && s * 64 + src_kc[j] >= p.K;
         const bool half = TAIL && !past && s * 64 + src_kc[j] + 16 > p.K;
-        dma_16B(past ? src[j] - src_kc[j] : src[j] + s * 64 - (half ? 8 : 0),
-                xt + s * (TX * 64) + (j * 4 + wave) * 1024);
+        const uint8_t *from = past ? src[j] - src_kc[j] : src[j] + s * 64 - (half ? 8 : 0);
+        uint8_t *to = xt + s * (TX * 64) + (j * 4 + wave) * 1024;
+        if (TAIL && by_registers) *(v4i *)(to + 16 * lane) = *(const v4i *)from;
+        else dma_16B(from, to);
       }
       // at most 32 transfers of this wavefront in flight (the counter has six bits)
       if ((s & 15) == 15) wait_vmcnt<0>();
