@@ -1,15 +1,17 @@
-// Runs the SOURCE of a few GPU kernels of mace_amd/csrc/q8_gemm.hip on the CPU: kernel_emu_extract.py
-// cuts their text out, this file supplies what the text needs from the GPU (thread and block
-// indices, LDS, barriers, and the wavefront-wide instructions -- MFMA, lane shuffles, the
-// transfer into LDS -- as collectives over 64 host threads), and every case runs one launch with
-// operands allocated at exactly their size.  Built with AddressSanitizer: an access outside an
-// operand aborts the run.  int32 results are compared with sums formed directly from the
-// operands; uint8 launches must write every byte of the result (the table look-up of the
-// requantization reads LDS through a 32-bit LDS pointer and has no host form, so their values are
-// not compared here; the GPU parity tests do that).
+// Runs the SOURCE of the uint8 GEMM kernels of mace_amd/csrc/q8_gemm.hip on the CPU:
+// kernel_emu_extract.py cuts their text out, this file supplies what the text needs from the GPU
+// (thread and block indices, LDS, barriers, and the wavefront-wide instructions -- MFMA, lane
+// shuffles, transfers into LDS, the transposing LDS read -- as collectives over the 64 host threads
+// of a wavefront), and every case runs one launch with operands allocated at exactly their size.
+// Built with AddressSanitizer: an access outside an operand aborts the run.  int32 results are
+// compared with sums formed directly from the operands; uint8 launches must write every byte of
+// the result (the table look-up of the requantization reads LDS through a 32-bit LDS pointer and
+// has no host form, so their values are not compared here; the GPU parity tests do that).
 //
-// What this covers is indexing: row clamps, ragged tiles, depth tails, store guards.  What it
-// cannot cover: the compiler's GPU code, timing, anything written in GPU assembly.
+// What this covers is indexing and arithmetic of the source: row clamps, ragged tiles, depth
+// tails, swizzles, store guards.  A transfer into LDS lands at once here, so the order of
+// asynchronous transfers and reads is not covered, nor the compiler's GPU code, nor anything
+// written in GPU assembly.
 #include <algorithm>
 #include <barrier>
 #include <cmath>
@@ -29,7 +31,8 @@ using std::min;
 #define __host__
 #define __forceinline__ inline __attribute__((always_inline))
 #define __launch_bounds__(...)
-#define __align__(n)
+#define __align__(n) __attribute__((aligned(n)))
+#define __shared__ static   // one workgroup runs at a time: a function's static is that workgroup's LDS
 
 struct dim3 {
   unsigned x, y, z;
@@ -43,22 +46,23 @@ typedef int e16i __attribute__((ext_vector_type(16)));
 typedef unsigned e2u __attribute__((ext_vector_type(2)));
 typedef unsigned uint4 __attribute__((ext_vector_type(4)));
 
-constexpr int THREADS = 256;   // every kernel here runs workgroups of four wavefronts
 struct Wave {
   std::barrier<> bar{64};
   e4i a[64], b[64];
   uint32_t w[64][2];
+  uint64_t piece[64];
 };
 struct Block {
-  std::barrier<> bar{THREADS};
-  Wave waves[THREADS / 64];
+  std::barrier<> *bar = nullptr;   // of the launch's workgroup size
+  Wave waves[8];
   alignas(16) uint8_t lds[160 * 1024];
 };
 static Block g_block;
 static inline Wave &wave_of_thread() { return g_block.waves[threadIdx.x >> 6]; }
 static inline int lane_of_thread() { return threadIdx.x & 63; }
 uint8_t *emu_lds() { return g_block.lds; }
-void __syncthreads() { g_block.bar.arrive_and_wait(); }
+void __syncthreads() { g_block.bar->arrive_and_wait(); }
+void emu_s_barrier() { g_block.bar->arrive_and_wait(); }
 
 // ---- wavefront-wide instructions: every lane of the wavefront calls them together ---------------
 int __shfl_xor(int v, int m, int = 64) {
@@ -106,6 +110,25 @@ e16i emu_mfma(e4i a, e4i b, e16i c, int, int, int) {
   w.bar.arrive_and_wait();
   return c;
 }
+// ds_read_b64_tr_b8: within 16 lanes the instruction takes 8 bytes at each lane's address and hands
+// lane j < 8 byte j of the even lanes' pieces, lane 8 + j byte j of the odd lanes' pieces
+typedef int v2i_t __attribute__((ext_vector_type(2)));
+template <int OFF>
+v2i_t lds_read_tr8(int lds_byte_address) {
+  Wave &w = wave_of_thread();
+  const int l = lane_of_thread();
+  memcpy(&w.piece[l], g_block.lds + lds_byte_address + OFF, 8);
+  w.bar.arrive_and_wait();
+  const int g = l & ~15, j = l & 7, odd = (l >> 3) & 1;
+  uint8_t out[8];
+  for (int i = 0; i < 8; ++i) out[i] = (uint8_t)(w.piece[g + 2 * i + odd] >> (8 * j));
+  w.bar.arrive_and_wait();
+  v2i_t r;
+  memcpy(&r, out, 8);
+  return r;
+}
+inline void lds_wait_tr(e4i &, int) {}
+inline int lds_address_of(const uint8_t *p) { return (int)(p - g_block.lds); }
 // ---- per-lane instructions ------------------------------------------------------------------------
 uint32_t emu_sad_u8(uint32_t a, uint32_t b, uint32_t c) {
   for (int i = 0; i < 4; ++i) c += (uint32_t)std::abs((int)((a >> (8 * i)) & 255) - (int)((b >> (8 * i)) & 255));
@@ -142,6 +165,7 @@ const void *emu_kernarg();
 #define __builtin_amdgcn_fmed3f emu_fmed3f
 #define __builtin_amdgcn_readfirstlane emu_readfirstlane
 #define __builtin_amdgcn_sched_barrier(x) ((void)0)
+#define __builtin_amdgcn_s_barrier emu_s_barrier
 #define __builtin_amdgcn_kernarg_segment_ptr emu_kernarg
 
 // ---- what the kernels' text takes from common.h and from other parts of q8_gemm.hip --------------
@@ -163,6 +187,13 @@ template <int N> inline void wait_vmcnt() {}
 inline void dma_16B(const uint8_t *g, uint8_t *lds_wave_base) {
   memcpy(lds_wave_base + 16 * (threadIdx.x & 63), g, 16);
 }
+// ... addressed as base (the same for the wavefront) + lane offset + another offset
+struct mh_rsrc { const uint8_t *base; };
+inline mh_rsrc dma_rsrc(const uint8_t *base) { return mh_rsrc{base}; }
+inline void dma_16B(mh_rsrc rs, uint32_t lane_off, uint32_t uniform_off, uint8_t *lds_wave_base) {
+  memcpy(lds_wave_base + 16 * (threadIdx.x & 63), rs.base + lane_off + uniform_off, 16);
+}
+constexpr int SLAB = 64;
 #include "kernels.inc"
 }  // namespace
 
@@ -172,12 +203,14 @@ static struct KernArgs {
 } g_args;
 const void *emu_kernarg() { return &g_args; }
 
-// all workgroups of a grid, one after the other, on THREADS host threads
-static void run_grid(dim3 grid, const std::function<void()> &body) {
+// all workgroups of a grid, one after the other, on as many host threads as a workgroup has
+static void run_grid(dim3 grid, const std::function<void()> &body, int threads = 256) {
   gridDim = grid;
-  blockDim = dim3(THREADS);
+  blockDim = dim3(threads);
+  std::barrier<> bar(threads);
+  g_block.bar = &bar;
   std::vector<std::thread> th;
-  for (int t = 0; t < THREADS; ++t)
+  for (int t = 0; t < threads; ++t)
     th.emplace_back([&, t] {
       threadIdx = dim3(t, 0, 0);
       for (unsigned z = 0; z < grid.z; ++z)
@@ -185,7 +218,7 @@ static void run_grid(dim3 grid, const std::function<void()> &body) {
           for (unsigned x = 0; x < grid.x; ++x) {
             blockIdx = dim3(x, y, z);
             body();
-            g_block.bar.arrive_and_wait();
+            g_block.bar->arrive_and_wait();
           }
     });
   for (auto &t : th) t.join();
@@ -202,32 +235,39 @@ static int g_failures = 0, g_cases = 0;
 static uint32_t g_seed = 12345;
 static uint8_t rnd() { g_seed = g_seed * 1664525u + 1013904223u; return (uint8_t)(g_seed >> 24); }
 
-// ---- one GEMM problem: OUT[y][x] = sum_k (X[x][k] - 128)(Y[y][k] - 128) + corrections -------------
+// ---- one GEMM problem: OUT[y][x] = sum_k (X(x,k) - 128)(Y(y,k) - 128) + corrections --------------
+// An operand is k-contiguous (row pitch ld >= k, the last row ending at its k-th byte: nothing
+// readable behind it) or k-major ([k][n], n contiguous); X may be stored already shifted to int8.
 struct Problem {
   int xn, yn, k;
   int64_t ldx, ldy;
-  std::vector<uint8_t *> owned;
+  bool xt, yt, xf;
+  int64_t xbytes, ybytes;
   uint8_t *X, *Y;
   int32_t *sumx, *sumy, *bias;
   GemmParams p{};
-  Problem(int xn_, int yn_, int k_, int64_t ldx_, int64_t ldy_) : xn(xn_), yn(yn_), k(k_), ldx(ldx_), ldy(ldy_) {
-    // the last row ends at its k-th byte: nothing readable behind it
-    X = new uint8_t[(int64_t)(xn - 1) * ldx + k];
-    Y = new uint8_t[(int64_t)(yn - 1) * ldy + k];
-    for (int64_t i = 0; i < (int64_t)(xn - 1) * ldx + k; ++i) X[i] = rnd();
-    for (int64_t i = 0; i < (int64_t)(yn - 1) * ldy + k; ++i) Y[i] = rnd();
+  int xat(int x, int c) const { return (int)((xt ? X[(int64_t)c * ldx + x] : X[(int64_t)x * ldx + c]) ^ (xf ? 0x80 : 0)) - 128; }
+  int yat(int y, int c) const { return (int)(yt ? Y[(int64_t)c * ldy + y] : Y[(int64_t)y * ldy + c]) - 128; }
+  Problem(int xn_, int yn_, int k_, int64_t ldx_, int64_t ldy_, bool xt_ = false, bool yt_ = false, bool xf_ = false)
+      : xn(xn_), yn(yn_), k(k_), ldx(ldx_), ldy(ldy_), xt(xt_), yt(yt_), xf(xf_) {
+    xbytes = xt ? (int64_t)(k - 1) * ldx + xn : (int64_t)(xn - 1) * ldx + k;
+    ybytes = yt ? (int64_t)(k - 1) * ldy + yn : (int64_t)(yn - 1) * ldy + k;
+    X = new uint8_t[xbytes];
+    Y = new uint8_t[ybytes];
+    for (int64_t i = 0; i < xbytes; ++i) X[i] = rnd();
+    for (int64_t i = 0; i < ybytes; ++i) Y[i] = rnd();
     sumx = new int32_t[xn];
     sumy = new int32_t[yn];
     bias = new int32_t[xn];
     for (int x = 0; x < xn; ++x) {
       int s = 0;
-      for (int c = 0; c < k; ++c) s += (int)X[x * ldx + c] - 128;
+      for (int c = 0; c < k; ++c) s += xat(x, c);
       sumx[x] = s;
       bias[x] = (int)rnd() * 37 - 4000;
     }
     for (int y = 0; y < yn; ++y) {
       int s = 0;
-      for (int c = 0; c < k; ++c) s += (int)Y[y * ldy + c] - 128;
+      for (int c = 0; c < k; ++c) s += yat(y, c);
       sumy[y] = s;
     }
     p.X = X; p.ldx = ldx; p.Y = Y; p.ldy = ldy;
@@ -245,7 +285,7 @@ struct Problem {
   }
   int32_t expected(int x, int y) const {
     int64_t acc = 0;
-    for (int c = 0; c < k; ++c) acc += ((int)X[x * ldx + c] - 128) * ((int)Y[y * ldy + c] - 128);
+    for (int c = 0; c < k; ++c) acc += xat(x, c) * yat(y, c);
     return (int32_t)((uint32_t)acc + (uint32_t)p.xcoef * (uint32_t)sumx[x] + (uint32_t)p.xadd + (uint32_t)bias[x] +
                      (uint32_t)p.ycoef * (uint32_t)sumy[y] + (uint32_t)p.yadd);
   }
@@ -279,6 +319,46 @@ struct Problem {
     }
   }
 };
+
+// the ring kernel: slabs of KB bytes of k moved into LDS by transfers; X k-contiguous, k-major (XT)
+// or repacked already shifted (XF); the panels' sums taken by the kernel or handed in
+template <int WX, int WY, int FX, int FY, int STAGES, int KB, bool SUMY, bool XT = false, bool XF = false,
+          bool SUMX = false>
+static void ring_case(int xn, int yn, int k) {
+  Problem pr(xn, yn, k, XT ? xn : k, k, XT, false, XF);
+  constexpr int TX = WX * FX * 32, TY = WY * FY * 32;
+  pr.p.tiles_x = (xn + TX - 1) / TX;
+  pr.p.tiles_y = (yn + TY - 1) / TY;
+  pr.p.sum_y = SUMY;
+  const dim3 grid(pr.p.tiles_x * pr.p.tiles_y, 1, 1);
+  char what[96];
+  snprintf(what, sizeof what, "q8_gemm_dma_kernel<%d,%d,%d,%d,STAGES=%d,KB=%d,SUMY=%d,XT=%d,XF=%d,SUMX=%d>", WX, WY,
+           FX, FY, STAGES, KB, (int)SUMY, (int)XT, (int)XF, (int)SUMX);
+  pr.check(what,
+           [&](GemmParams &p) {
+             run_grid(grid, [&] { q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, int32_t, 1, SUMY, false, KB, XT, XF, SUMX>(p, g_args.t); },
+                      WX * WY * 64);
+           },
+           [&](GemmParams &p) {
+             run_grid(grid, [&] { q8_gemm_dma_kernel<WX, WY, FX, FY, STAGES, uint8_t, 1, SUMY, false, KB, XT, XF, SUMX>(p, g_args.t); },
+                      WX * WY * 64);
+           });
+}
+
+// the eight-wavefront kernel: either operand k-contiguous or k-major
+template <bool XT, bool YT>
+static void mid_case(int xn, int yn, int k) {
+  Problem pr(xn, yn, k, XT ? xn : k, YT ? yn : k, XT, YT);
+  pr.p.tiles_x = (xn + 127) / 128;
+  pr.p.tiles_y = (yn + 127) / 128;
+  pr.p.sum_y = true;
+  const dim3 grid(pr.p.tiles_x * pr.p.tiles_y, 1, 1);
+  char what[64];
+  snprintf(what, sizeof what, "q8_gemm_mid_kernel<STAGES=4,XT=%d,YT=%d>", (int)XT, (int)YT);
+  pr.check(what,
+           [&](GemmParams &p) { run_grid(grid, [&] { q8_gemm_mid_kernel<int32_t, 4, XT, YT>(p, g_args.t); }, 512); },
+           [&](GemmParams &p) { run_grid(grid, [&] { q8_gemm_mid_kernel<uint8_t, 4, XT, YT>(p, g_args.t); }, 512); });
+}
 
 template <int WX, int WY, int FX, int FY>
 static void tiled_case(int xn, int yn, int k, bool sum_y) {
@@ -319,6 +399,104 @@ static void xres_case(int xn, int yn, int k, int wgs) {
            });
 }
 
+// The one-launch kernel: either operand k-contiguous ([n][k]) or k-major ([k][n]), rows of whole
+// aligned 16-byte pieces or not (then read in 4-byte groups where everything is a multiple of 4,
+// else byte by byte), or Y gathered from the NHWC input of a convolution.
+struct Conv { int in_h, in_w, cin, k, stride, pad, out_h, out_w, zp; };
+template <bool XT, bool YT>
+static void small_case(int xn, int yn, int k, const Conv *cv = nullptr) {
+  ++g_cases;
+  const int64_t ldx = XT ? xn : k, ldy = cv ? 0 : (YT ? yn : k);
+  const int64_t xbytes = XT ? (int64_t)k * xn : (int64_t)xn * k;
+  const int64_t ybytes = cv ? (int64_t)(yn / (cv->out_h * cv->out_w)) * cv->in_h * cv->in_w * cv->cin
+                            : (YT ? (int64_t)k * yn : (int64_t)yn * k);
+  uint8_t *X = new uint8_t[xbytes], *Y = new uint8_t[ybytes];
+  for (int64_t i = 0; i < xbytes; ++i) X[i] = rnd();
+  for (int64_t i = 0; i < ybytes; ++i) Y[i] = rnd();
+  auto xat = [&](int x, int c) { return (int)(XT ? X[(int64_t)c * xn + x] : X[(int64_t)x * k + c]) - 128; };
+  auto yat = [&](int y, int c) {
+    if (!cv) return (int)(YT ? Y[(int64_t)c * yn + y] : Y[(int64_t)y * k + c]) - 128;
+    const int ow = y % cv->out_w, t = y / cv->out_w, oh = t % cv->out_h, img = t / cv->out_h;
+    const int tap = c / cv->cin, ch = c % cv->cin, kh = tap / cv->k, kw = tap % cv->k;
+    const int ih = oh * cv->stride - cv->pad + kh, iw = ow * cv->stride - cv->pad + kw;
+    if (ih < 0 || ih >= cv->in_h || iw < 0 || iw >= cv->in_w) return cv->zp - 128;
+    return (int)Y[(((int64_t)img * cv->in_h + ih) * cv->in_w + iw) * cv->cin + ch] - 128;
+  };
+  std::vector<int32_t> bias(xn), sumx(xn), sumy(yn);
+  for (int x = 0; x < xn; ++x) {
+    bias[x] = (int)rnd() * 91 - 9000;
+    for (int c = 0; c < k; ++c) sumx[x] += xat(x, c);
+  }
+  for (int y = 0; y < yn; ++y)
+    for (int c = 0; c < k; ++c) sumy[y] += yat(y, c);
+  GemmParams p{};
+  p.X = X; p.ldx = ldx; p.Y = Y; p.ldy = ldy;
+  p.XN = xn; p.YN = yn; p.K = k;
+  p.ldo = xn; p.obs = (int64_t)xn * yn;
+  p.rq = RequantFixed{1 << 30, 8, 255, 127, -128, 127, 128, 1, 255, 0, 1e-3f, MH_REQUANT_MAGIC + 128.0f,
+                      MH_REQUANT_MAGIC + 255.875f};
+  p.xcoef = -3; p.xadd = 11; p.xbias = bias.data();
+  p.ycoef = 5; p.yadd = -7; p.ybias = nullptr;
+  p.sum_y = true;
+  p.tiles_x = (xn + 63) / 64;
+  p.tiles_y = (yn + 63) / 64;
+  // the host's rules (Q8Call::small_problem): whole aligned pieces, else 4-byte groups, else bytes
+  auto vec = [&](bool t, int n) { return (t ? n : k) % 16 == 0; };
+  auto dwords = [&](bool t, int n) { return (t ? n : k) % 4 == 0; };
+  p.x_bytewise = !vec(XT, xn);
+  p.x_dword = p.x_bytewise && dwords(XT, xn);
+  if (cv) {
+    p.conv = true;
+    p.cv_in_h = cv->in_h; p.cv_in_w = cv->in_w; p.cv_cin = cv->cin; p.cv_kw = cv->k;
+    p.cv_sh = p.cv_sw = cv->stride; p.cv_pt = p.cv_pl = cv->pad; p.cv_oh = cv->out_h; p.cv_ow = cv->out_w;
+    p.cv_zp4 = (uint32_t)cv->zp * 0x01010101u;
+    p.y_bytewise = cv->cin % 16 != 0;
+    p.y_dword = p.y_bytewise && cv->cin % 4 == 0;
+  } else {
+    p.y_bytewise = !vec(YT, yn);
+    p.y_dword = p.y_bytewise && dwords(YT, yn);
+  }
+  for (int i = 0; i < MH_REQUANT_TABLE_MAX; ++i) g_args.t.t[i] = i * 1000 - 100000;
+  const bool bw = p.x_bytewise || p.y_bytewise;
+  const dim3 grid(p.tiles_x * p.tiles_y, 1, 1);
+  {
+    std::vector<int32_t> out((int64_t)xn * yn, 0x5EEDBEEF);
+    p.out = out.data();
+    g_args.p = p;
+    if (bw) run_grid(grid, [&] { q8_gemm_fused_small_kernel<int32_t, XT, YT, true>(p, g_args.t); });
+    else run_grid(grid, [&] { q8_gemm_fused_small_kernel<int32_t, XT, YT, false>(p, g_args.t); });
+    int64_t bad = 0;
+    for (int y = 0; y < yn; ++y)
+      for (int x = 0; x < xn; ++x) {
+        int64_t acc = 0;
+        for (int c = 0; c < k; ++c) acc += xat(x, c) * yat(y, c);
+        const int32_t want = (int32_t)((uint32_t)acc + (uint32_t)p.xcoef * (uint32_t)sumx[x] + (uint32_t)p.xadd +
+                                       (uint32_t)bias[x] + (uint32_t)p.ycoef * (uint32_t)sumy[y] + (uint32_t)p.yadd);
+        bad += out[(int64_t)y * xn + x] != want;
+      }
+    EXPECT(bad == 0, "fused_small<XT=%d,YT=%d,BW=%d>%s XN %d YN %d K %d: %lld int32 results differ", (int)XT,
+           (int)YT, (int)bw, cv ? " conv" : "", xn, yn, k, (long long)bad);
+  }
+  {
+    std::vector<uint8_t> out((int64_t)xn * yn, 0xEE);
+    p.out = out.data();
+    g_args.p = p;
+    if (bw) run_grid(grid, [&] { q8_gemm_fused_small_kernel<uint8_t, XT, YT, true>(p, g_args.t); });
+    else run_grid(grid, [&] { q8_gemm_fused_small_kernel<uint8_t, XT, YT, false>(p, g_args.t); });
+    int64_t untouched = 0;
+    for (uint8_t v : out) untouched += v == 0xEE;
+    EXPECT(untouched == 0, "fused_small<XT=%d,YT=%d,BW=%d> XN %d YN %d K %d: %lld uint8 results not written",
+           (int)XT, (int)YT, (int)bw, xn, yn, k, (long long)untouched);
+  }
+  delete[] X;
+  delete[] Y;
+}
+static void small_conv_case(int n, int hw, int cin, int cout, int k, int stride, int pad) {
+  const int out = (hw + 2 * pad - k) / stride + 1;
+  const Conv cv{hw, hw, cin, k, stride, pad, out, out, 77};
+  small_case<false, false>(cout, n * out * out, k * k * cin, &cv);
+}
+
 static void pack_case(int n, int k, bool by_dwords) {
   ++g_cases;
   const int kp = (k + 63) & ~63;
@@ -357,7 +535,13 @@ static void sums_case(int n, int k) {
   delete[] sums;
 }
 
+// PART (compile-time): 1 = everything but the ring and eight-wavefront kernels, 2 = those two; the
+// test builds and runs the parts side by side.
+#ifndef PART
+#define PART 0
+#endif
 int main() {
+#if PART != 2
   // the repacks of k-contiguous rows (any k; k % 4 == 0 by dwords)
   for (int k : {1, 3, 15, 16, 17, 24, 63, 64, 65, 100, 127}) pack_case(37, k, false);
   for (int k : {4, 8, 24, 40, 60, 64, 68, 120}) pack_case(301, k, true);
@@ -380,6 +564,26 @@ int main() {
     tiled_case<2, 2, 4, 4>(144, 520, 64, sum_y);
     tiled_case<2, 2, 4, 4>(300, 290, 16, sum_y);
   }
+  // the one-launch kernel: both layouts of both operands; rows of whole pieces, of 4-byte groups, of
+  // single bytes; ragged tiles; depths from one byte to several k tiles; gathered convolutions
+  small_case<false, false>(128, 128, 256);
+  small_case<false, false>(70, 130, 48);
+  small_case<false, false>(33, 65, 100);
+  small_case<false, false>(64, 17, 27);
+  small_case<false, false>(5, 3, 1);
+  small_case<false, false>(100, 90, 333);
+  small_case<true, false>(128, 64, 128);
+  small_case<true, false>(100, 70, 96);
+  small_case<true, false>(37, 64, 50);
+  small_case<false, true>(64, 112, 80);
+  small_case<false, true>(48, 101, 64);
+  small_case<true, true>(80, 48, 144);
+  small_case<true, true>(31, 29, 67);
+  small_conv_case(2, 9, 16, 24, 3, 1, 1);
+  small_conv_case(1, 12, 8, 16, 3, 2, 1);
+  small_conv_case(1, 10, 3, 32, 3, 2, 0);
+  small_conv_case(2, 7, 5, 17, 2, 1, 1);
+  small_conv_case(1, 8, 32, 64, 1, 1, 0);
   // the resident-tile kernel: 64- and 128-row tiles, 32- and 64-row blocks, more blocks than
   // wavefronts and fewer, whole groups, depth tails of whole pieces and of half a piece
   xres_case<2, 1, false>(48, 700, 64, 3);
@@ -393,6 +597,29 @@ int main() {
   xres_case<4, 1, true>(130, 515, 72, 2);
   xres_case<2, 1, true>(24, 4000, 120, 40);
   xres_case<4, 2, true>(128, 256, 328, 1);
+#endif
+#if PART != 1
+  // the ring kernel in the tile shapes, ring depths and slab widths the dispatch uses; ragged tiles
+  ring_case<2, 2, 4, 4, 2, 128, false>(300, 260, 384);
+  ring_case<2, 2, 4, 4, 2, 128, true>(256, 257, 256);
+  ring_case<2, 2, 4, 4, 2, 128, false, true>(304, 200, 384);           // X k-major, read in place
+  ring_case<2, 2, 4, 4, 2, 128, true, true, false, true>(272, 300, 256);   // ... and summed in the kernel
+  ring_case<2, 2, 4, 4, 2, 128, false, false, true>(260, 300, 384);    // X repacked already shifted
+  ring_case<2, 4, 2, 1, 2, 128, true>(130, 140, 1024);
+  ring_case<2, 2, 2, 2, 2, 128, false>(200, 129, 1024);
+  ring_case<2, 2, 4, 4, 4, 64, true>(257, 300, 192);
+  ring_case<1, 4, 2, 2, 4, 64, false>(48, 300, 256);
+  ring_case<2, 2, 2, 2, 4, 64, true>(130, 200, 448);
+  ring_case<2, 2, 1, 1, 4, 64, false>(70, 65, 192);
+  ring_case<1, 4, 2, 2, 3, 64, true>(64, 513, 128);
+  ring_case<2, 2, 2, 2, 3, 64, false>(129, 131, 128);
+  // the eight-wavefront kernel: every layout of both operands, ragged tiles, the shortest depth
+  mid_case<false, false>(200, 130, 512);
+  mid_case<true, false>(144, 129, 640);
+  mid_case<false, true>(129, 208, 512);
+  mid_case<true, true>(272, 144, 512);
+  mid_case<false, false>(128, 128, 128);
+#endif
   if (g_failures) {
     printf("kernel_emu: %d failures in %d cases\n", g_failures, g_cases);
     return 1;

@@ -12,6 +12,12 @@ PIECES = [
     ("__device__ inline int sum16_u8", "// Epilogue shared by the GEMM kernels"),
     ("template <int WX, int WY, int FX, int FY, typename OutT, bool SUMY, bool PRESTAGED = false>",
      "// ---- small problems: everything in one launch"),
+    ("template <typename OutT, bool XT, bool YT, bool BW>\n__global__ __launch_bounds__(256, BW ? 5 : 1) void q8_gemm_fused_small_kernel",
+     "// ---- the streaming GEMM kernel: global -> LDS"),
+    ("template <int WX, int WY, int FX, int FY, int STAGES, typename OutT, int OCC = 1,",
+     "// ---- one round of 128 x 128 tiles"),
+    ("template <typename OutT, int STAGES, bool XT, bool YT = false>\n__global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel",
+     "// ---- the kernel for an X panel that fits in LDS"),
     ("template <int FX, int FY, int G, typename OutT, int OCC, bool CONV = false, bool XT = false,",
      "// ---- the streaming kernel for a small X panel"),
     ("__global__ void q8_pack_rows_kernel", "// src is [k][n] with n contiguous"),
@@ -22,6 +28,9 @@ PIECES = [
 PATCHES = [
     ("extern __shared__ __align__(16) uint8_t lds[];", "uint8_t *lds = emu_lds();"),
     ("__launch_bounds__(256, OCC)", ""),
+    ("__launch_bounds__(WX *WY * 64, OCC)", ""),
+    ("__launch_bounds__(512, 1)", ""),
+    ('asm volatile("" ::: "memory");', ""),
     # 16-byte accesses at addresses that are multiples of 8 only: fine on the GPU, not for SSE
     ("v4i v = *(const v4i *)at;", "v4i v; memcpy(&v, at, 16);"),
     ("*(v4i *)(to + 16 * lane) = *(const v4i *)from;", "memcpy(to + 16 * lane, from, 16);"),
