@@ -87,6 +87,24 @@ __device__ inline void tile_of_block(int bid, int nblocks, int tiles_x, int tile
   *tx = r / gsize;
 }
 
+// The same for a launch over a batch (grid.z = batches): workgroup ids run over the tiles of a
+// batch first, then over the batches, and go round-robin to the 8 XCDs, so left alone every XCD
+// would hold a few tiles of EVERY batch and pull all of the operands through its L2.  Every XCD
+// gets a contiguous span of (batch, tile) instead (eight-wavefront kernel, k-major X, us per call:
+// 16 x 512 x 768 x 512 11.8 -> 10.1, 32 x 512^3 in two rounds 19.2 -> 16.5).
+__device__ inline void tile_and_batch_of_block(int tiles_x, int tiles_y, int *tx, int *ty, int *b) {
+  *b = blockIdx.z;
+  if (gridDim.z > 1 && (gridDim.x * gridDim.z) % 8 == 0) {
+    const int nwg = gridDim.x * gridDim.z;
+    int wg = blockIdx.x + gridDim.x * blockIdx.z;
+    wg = (wg % 8) * (nwg / 8) + wg / 8;
+    *b = wg / gridDim.x;
+    tile_of_block(wg - *b * gridDim.x, 1, tiles_x, tiles_y, tx, ty);
+  } else {
+    tile_of_block(blockIdx.x, gridDim.x, tiles_x, tiles_y, tx, ty);
+  }
+}
+
 // Sum of the 16 bytes of a fragment as read from memory (unsigned, before the flip), added to acc.
 // The sum of the shifted bytes the corrections need is this minus 128 per byte.  v_sad_u8 is an
 // ordinary vector-ALU instruction; the dot-product instructions (sum16_i8 below) do not run next to
@@ -295,10 +313,9 @@ __global__ __launch_bounds__(WX *WY * 64) void q8_gemm_kernel(GemmParams p, Requ
   const int wave = tid >> 6;
   const int wx = wave % WX, wy = wave / WX;
 
-  int tile_x, tile_y;
-  tile_of_block(blockIdx.x, gridDim.x, p.tiles_x, p.tiles_y, &tile_x, &tile_y);
+  int tile_x, tile_y, b;
+  tile_and_batch_of_block(p.tiles_x, p.tiles_y, &tile_x, &tile_y, &b);
   const int x0 = tile_x * TX, y0 = tile_y * TY;
-  const int b = blockIdx.z;
 
   const uint8_t *Xb = p.X + (int64_t)b * p.xbs;
   const uint8_t *Yb = p.Y + (int64_t)b * p.ybs;
@@ -794,10 +811,9 @@ __global__ __launch_bounds__(WX *WY * 64, OCC) void q8_gemm_dma_kernel(GemmParam
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wx = wave % WX, wy = wave / WX;
 
-  int tile_x, tile_y;
-  tile_of_block(blockIdx.x, gridDim.x, p.tiles_x, p.tiles_y, &tile_x, &tile_y);
+  int tile_x, tile_y, b;
+  tile_and_batch_of_block(p.tiles_x, p.tiles_y, &tile_x, &tile_y, &b);
   const int x0 = tile_x * TX, y0 = tile_y * TY;
-  const int b = blockIdx.z;
   const uint8_t *Xb = p.X + (int64_t)b * p.xbs;
   const uint8_t *Yb = p.Y + (int64_t)b * p.ybs;
 
@@ -1150,10 +1166,9 @@ __global__ __launch_bounds__(512, 1) void q8_gemm_mid_kernel(GemmParams p, Requa
   const int wx = wave & 1, wy = (wave >> 1) & 1;
   const int par = wx ^ wy;                        // order of this wavefront's two k steps
 
-  int tile_x, tile_y;
-  tile_of_block(blockIdx.x, gridDim.x, p.tiles_x, p.tiles_y, &tile_x, &tile_y);
+  int tile_x, tile_y, b;
+  tile_and_batch_of_block(p.tiles_x, p.tiles_y, &tile_x, &tile_y, &b);
   const int x0 = tile_x * T, y0 = tile_y * T;
-  const int b = blockIdx.z;
   const uint8_t *Xt = XT ? p.X + (int64_t)b * p.xbs + x0 : p.X + (int64_t)b * p.xbs + (int64_t)x0 * p.ldx;
   const uint8_t *Yt = YT ? p.Y + (int64_t)b * p.ybs + y0 : p.Y + (int64_t)b * p.ybs + (int64_t)y0 * p.ldy;
 
@@ -2803,9 +2818,17 @@ int Q8Call::kmajor_in_place(bool *done) {
     // 3072 x 512 x 3072 22.9 -> 20.1, 4096 x 384 x 4096 22.8 -> 21.1, 4 x 2048 x 512 x 2048 25.3 -> 23.7;
     // k = 256 ties; four rounds, 8192 x 512 x 8192, lose 64 against 79)
     const bool big_xt_first = big_xt && depth >= 384 && tiles256 <= cu_n;
+    // The eight-wavefront 128 x 128 kernel reads the same layout in place (second block below): one
+    // round of tiles, up to two rounds from k = 512 on, two and a half from k = 2048 on.
+    const bool mid_xt = !cv && x_kmajor && y_direct && rhs_ld == 0 && !lhs_w && !rhs_w && depth >= 512 &&
+                        depth % 128 == 0 && xn % 16 == 0 && (uintptr_t)xp % 16 == 0 && xn > 64 && yn > 64 &&
+                        4 * tiles128 >= cu_n &&
+                        (tiles128 <= 2 * cu_n || (depth >= 2048 && 2 * tiles128 <= 5 * cu_n)) &&
+                        xn * depth < ((int64_t)1 << 32) && depth < (1 << 24) &&
+                        (size_t)4 * 256 * 128 <= lds_cu && !(ctx->kernel_mask & MH_MASK_NO_MID);
     if (!cv && x_kmajor && y_direct && rhs_ld == 0 && !lhs_w && !rhs_w && depth > 0 && !big_xt_first &&
         depth % 64 == 0 && xn % 16 == 0 && (uintptr_t)xp % 16 == 0 && yn >= 256 &&
-        2 * (XRES_SC_BYTES + (size_t)tx * depth) <= lds_cu && !mid_first_xt &&
+        2 * (XRES_SC_BYTES + (size_t)tx * depth) <= lds_cu && !mid_first_xt && !(mid_xt && tiles128 > cu_n) &&
         !(ctx->kernel_mask & MH_MASK_NO_XRES)) {
       GemmParams p = kmajor_params();
       p.sum_y = true;
@@ -2814,18 +2837,15 @@ int Q8Call::kmajor_in_place(bool *done) {
       *done = true;
       return launch_gemm_xres_any(ctx, p, tab, out_u8, (int)batch, tx, true);
     }
-    // The same operand layout with a longer k, in the tile-count range of the eight-wavefront
-    // 128 x 128 kernel (see below): its transposing LDS reads take the operand as it lies, so the
-    // repack (2048^3: zeroing 2.4 + repack 7.5 us of a 22 us call) is not launched.  Because of that
-    // saving the range is wider here: two rounds of tiles from k = 1024 on (8 x 1024^3 25.7 -> 23.4 us,
-    // 32 x 512 x 1024 x 512 30.1 -> 24.8; 3072 x 1024 x 3072, 576 tiles, loses 5 % and is left out).
-    if (!cv && x_kmajor && y_direct && rhs_ld == 0 && !lhs_w && !rhs_w && depth >= 512 &&
-        depth % 128 == 0 && xn % 16 == 0 && (uintptr_t)xp % 16 == 0 && xn > 64 && yn > 64 &&
-        4 * tiles128 >= cu_n &&
-        (tiles128 <= cu_n || (depth >= 2048 && 2 * tiles128 <= 5 * cu_n) ||
-         (depth >= 1024 && tiles128 <= 2 * cu_n)) &&
-        xn * depth < ((int64_t)1 << 32) && depth < (1 << 24) && (size_t)4 * 256 * 128 <= lds_cu &&
-        !(ctx->kernel_mask & MH_MASK_NO_MID)) {
+    // The same operand layout in the tile-count range of the eight-wavefront 128 x 128 kernel (see
+    // below): its transposing LDS reads take the operand as it lies, so the repack (2048^3: zeroing
+    // 2.4 + repack 7.5 us of a 22 us call) is not launched.  Because of that saving the range is
+    // wider here: two rounds of tiles from k = 512 on (us per call, six buffer sets in rotation,
+    // against the kernel that had the shape before: 8 x 1024^3 25.7 -> 23.4, 32 x 512 x 1024 x 512 30.1
+    // -> 24.8, 4096 x 512 x 2048 18.1 -> 15.8, 2048 x 640 x 3072 19.7 -> 16.1, 20 x 640 x 512 x 512 21.3
+    // -> 17.8, 32 x 512^3 17.6 -> 16.5, 24 x 512^3 16.7 -> 15.6; 3072 x 1024 x 3072, 576 tiles, loses 5 %
+    // and is left out; with k-contiguous operands two rounds lose by 2 - 5 % and stay where they were).
+    if (mid_xt) {
       GemmParams p = kmajor_params();
       RequantTable tab;
       if (out_u8 && rq.table) mh_requant_table_cached(ctx, rq, tab.t);

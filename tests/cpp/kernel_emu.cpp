@@ -399,6 +399,46 @@ static void xres_case(int xn, int yn, int k, int wgs) {
            });
 }
 
+// ... on a batch of small products (per-batch operands): every (batch, tile) is computed exactly once
+// whatever order the kernel walks them in
+static void mid_batched_case(int batch, int xn, int yn, int k) {
+  ++g_cases;
+  std::vector<uint8_t> X((int64_t)batch * xn * k), Y((int64_t)batch * yn * k);
+  for (auto &v : X) v = rnd();
+  for (auto &v : Y) v = rnd();
+  std::vector<int32_t> bias(xn), out((int64_t)batch * xn * yn, 0x5EEDBEEF);
+  for (auto &v : bias) v = (int)rnd() * 37 - 4000;
+  GemmParams p{};
+  p.X = X.data(); p.ldx = k; p.xbs = (int64_t)xn * k;
+  p.Y = Y.data(); p.ldy = k; p.ybs = (int64_t)yn * k;
+  p.XN = xn; p.YN = yn; p.K = k;
+  p.out = out.data(); p.ldo = xn; p.obs = (int64_t)xn * yn;
+  p.xcoef = -3; p.xadd = 11; p.xbias = bias.data();
+  p.ycoef = 5; p.yadd = -7;
+  p.sum_y = true;
+  p.tiles_x = (xn + 127) / 128;
+  p.tiles_y = (yn + 127) / 128;
+  g_args.p = p;
+  run_grid(dim3(p.tiles_x * p.tiles_y, 1, batch), [&] { q8_gemm_mid_kernel<int32_t, 4, false, false>(p, g_args.t); }, 512);
+  int64_t bad = 0;
+  for (int b = 0; b < batch; ++b)
+    for (int y = 0; y < yn; ++y)
+      for (int x = 0; x < xn; ++x) {
+        const uint8_t *xr = &X[((int64_t)b * xn + x) * k], *yr = &Y[((int64_t)b * yn + y) * k];
+        int64_t acc = 0, sx = 0, sy = 0;
+        for (int c = 0; c < k; ++c) {
+          acc += ((int)xr[c] - 128) * ((int)yr[c] - 128);
+          sx += (int)xr[c] - 128;
+          sy += (int)yr[c] - 128;
+        }
+        const int32_t want = (int32_t)((uint32_t)acc + (uint32_t)p.xcoef * (uint32_t)sx + (uint32_t)p.xadd +
+                                       (uint32_t)bias[x] + (uint32_t)p.ycoef * (uint32_t)sy + (uint32_t)p.yadd);
+        bad += out[((int64_t)b * yn + y) * xn + x] != want;
+      }
+  EXPECT(bad == 0, "q8_gemm_mid_kernel batch %d XN %d YN %d K %d: %lld int32 results differ", batch, xn, yn, k,
+         (long long)bad);
+}
+
 // The one-launch kernel: either operand k-contiguous ([n][k]) or k-major ([k][n]), rows of whole
 // aligned 16-byte pieces or not (then read in 4-byte groups where everything is a multiple of 4,
 // else byte by byte), or Y gathered from the NHWC input of a convolution.
@@ -619,6 +659,8 @@ int main() {
   mid_case<false, true>(129, 208, 512);
   mid_case<true, true>(272, 144, 512);
   mid_case<false, false>(128, 128, 128);
+  mid_batched_case(8, 200, 128, 128);    // 16 workgroups: dealt to the XCDs in spans of (batch, tile)
+  mid_batched_case(3, 129, 130, 128);    // a workgroup count that is not a multiple of 8
 #endif
   if (g_failures) {
     printf("kernel_emu: %d failures in %d cases\n", g_failures, g_cases);

@@ -156,6 +156,11 @@ MID_SHAPES = [  # batch, rows, depth, cols, lhs batched, rhs batched, lhs order,
     (1, 1536, 1024, 1488, True, True, R, R, R, "mid/XT"), (2, 1000, 640, 1040, True, True, R, R, R, "mid/XT"),
     (1, 1296, 1280, 1500, True, True, Cm, Cm, Cm, "mid/XT"), (2, 1100, 512, 1200, True, False, R, R, R, "mid/XT"),
     (1, 2048, 2048, 2048, True, True, R, R, R, "mid/XT"),
+    # ... up to two rounds of tiles from k = 512 on; batches whose workgroups are dealt to the XCDs in
+    # spans of (batch, tile) (a workgroup count that is a multiple of 8) and batches that are not
+    (24, 512, 512, 512, True, True, R, R, R, "mid/XT"), (1, 2100, 640, 3008, True, True, R, R, R, "mid/XT"),
+    (13, 640, 512, 640, True, True, R, R, R, "mid/XT"), (6, 640, 512, 1024, False, True, R, R, R, "mid/XT"),
+    (8, 600, 1024, 500, True, True, R, Cm, R, "mid"), (5, 640, 640, 600, True, True, R, Cm, R, "mid"),
     # Y operand k-major in memory (ColMajor left-hand matrix with a RowMajor result: a transpose_a
     # MatMul; RowMajor right-hand matrix with a ColMajor result), X k-major as well or k-contiguous:
     # neither is repacked; ragged last tiles, batches, one side shared
@@ -499,7 +504,7 @@ def test_q8_gemm_freivalds_large(ctx, n):
     assert 0 < ((got8 == 0) | (got8 == 255)).mean() < 0.1 and len(np.unique(got8)) > 200
 
 
-@pytest.mark.parametrize("batch,n,kernel", [(1, 2048, "mid/XT"), (32, 512, "xres/XT")])
+@pytest.mark.parametrize("batch,n,kernel", [(1, 2048, "mid/XT"), (32, 512, "mid/XT")])
 def test_q8_gemm_config5_random_zero_points(ctx, batch, n, kernel):
     """Benchmark configuration 5 with all three zero points drawn from U{0..255} and the output
     scale derived from the data.  With zero points far from the operands' mean the accumulators sit

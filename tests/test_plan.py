@@ -80,8 +80,8 @@ def test_config5_gemm_sweep(ctx):
     p = gemm(ctx, 1, 8192, 8192, 8192, ro=Cm)
     assert p.family == mh.KF_Q8_GEMM_RING and "2,2,4,4,STAGES=2" in p.kernel and "KB=128" in p.kernel
     assert p.aux == mh.AUX_PANEL_SUMS and p.launches == 3     # one pass per operand at this size
-    p = gemm(ctx, 32, 512, 512, 512)
-    assert p.family == mh.KF_Q8_GEMM_XRES and "XT=true" in p.kernel and p.launches == 1
+    p = gemm(ctx, 32, 512, 512, 512)      # two rounds of 128 x 128 tiles, B read as it lies
+    assert p.family == mh.KF_Q8_GEMM_MID and "XT=true" in p.kernel and p.launches == 1
 
 
 def test_config3_gemv(ctx):
@@ -161,9 +161,14 @@ def test_eight_wavefront_kernel_range(ctx):
     assert fam(gemm(ctx, 4, 512, 512, 512, ro=Cm)) == mh.KF_Q8_GEMM_FUSED_SMALL
     p = gemm(ctx, 4, 512, 512, 512)
     assert p.kernel == "q8_gemm_mid_kernel<uint8_t,STAGES=4,XT=true,YT=false>"
-    # k-major X: two rounds of tiles from k = 1024 on
+    # k-major X: two rounds of tiles from k = 512 on (with k-contiguous operands two rounds lose)
     assert fam(gemm(ctx, 8, 1024, 1024, 1024)) == mid and gemm(ctx, 8, 1024, 1024, 1024).grid == (64, 1, 8)
+    assert fam(gemm(ctx, 1, 4096, 512, 2048)) == mid and fam(gemm(ctx, 1, 2048, 640, 3072)) == mid
+    assert fam(gemm(ctx, 32, 512, 512, 512)) == mid and fam(gemm(ctx, 20, 640, 512, 512)) == mid
+    assert fam(gemm(ctx, 32, 512, 512, 512, ro=Cm)) == mh.KF_Q8_GEMM_XRES
+    assert fam(gemm(ctx, 32, 512, 384, 512)) == mh.KF_Q8_GEMM_XRES    # k < 512
     assert fam(gemm(ctx, 1, 3072, 1024, 3072)) != mid                 # 576 tiles
+    assert fam(gemm(ctx, 36, 512, 512, 512)) != mid                   # 576 tiles
     assert fam(gemm(ctx, 1, 2048, 2048, 2048, mask=mh.MASK_NO_MID)) != mid
     # k-major Y (transpose_a with a RowMajor result), X k-major or k-contiguous: read as they lie
     p = gemm(ctx, 1, 2048, 2048, 2048, lo=Cm)
