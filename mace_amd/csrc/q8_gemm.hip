@@ -92,17 +92,22 @@ __device__ inline void tile_of_block(int bid, int nblocks, int tiles_x, int tile
 // would hold a few tiles of EVERY batch and pull all of the operands through its L2.  Every XCD
 // gets a contiguous span of (batch, tile) instead (eight-wavefront kernel, k-major X, us per call:
 // 16 x 512 x 768 x 512 11.8 -> 10.1, 32 x 512^3 in two rounds 19.2 -> 16.5).
-__device__ inline void tile_and_batch_of_block(int tiles_x, int tiles_y, int *tx, int *ty, int *b) {
+// (returns whether the launch is dealt that way; *bid: the workgroup's index within batch *b)
+__device__ inline bool batch_span_of_block(int *bid, int *b) {
+  *bid = blockIdx.x;
   *b = blockIdx.z;
-  if (gridDim.z > 1 && (gridDim.x * gridDim.z) % 8 == 0) {
-    const int nwg = gridDim.x * gridDim.z;
-    int wg = blockIdx.x + gridDim.x * blockIdx.z;
-    wg = (wg % 8) * (nwg / 8) + wg / 8;
-    *b = wg / gridDim.x;
-    tile_of_block(wg - *b * gridDim.x, 1, tiles_x, tiles_y, tx, ty);
-  } else {
-    tile_of_block(blockIdx.x, gridDim.x, tiles_x, tiles_y, tx, ty);
-  }
+  if (gridDim.z == 1 || (gridDim.x * gridDim.z) % 8 != 0) return false;
+  const int nwg = gridDim.x * gridDim.z;
+  int wg = blockIdx.x + gridDim.x * blockIdx.z;
+  wg = (wg % 8) * (nwg / 8) + wg / 8;
+  *b = wg / gridDim.x;
+  *bid = wg - *b * gridDim.x;
+  return true;
+}
+__device__ inline void tile_and_batch_of_block(int tiles_x, int tiles_y, int *tx, int *ty, int *b) {
+  int bid;
+  if (batch_span_of_block(&bid, b)) tile_of_block(bid, 1, tiles_x, tiles_y, tx, ty);
+  else tile_of_block(blockIdx.x, gridDim.x, tiles_x, tiles_y, tx, ty);
 }
 
 // Sum of the 16 bytes of a fragment as read from memory (unsigned, before the flip), added to acc.
@@ -471,9 +476,10 @@ __global__ __launch_bounds__(256, BW ? 5 : 1) void q8_gemm_fused_small_kernel(Ge
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int wx = wave % 2, wy = wave / 2;
-  const int tile_x = blockIdx.x % p.tiles_x, tile_y = blockIdx.x / p.tiles_x;
+  int bid, b;
+  batch_span_of_block(&bid, &b);
+  const int tile_x = bid % p.tiles_x, tile_y = bid / p.tiles_x;
   const int x0 = tile_x * T, y0 = tile_y * T;
-  const int b = blockIdx.z;
   const uint8_t *Xb = p.X + (int64_t)b * p.xbs;
   const uint8_t *Yb = p.Y + (int64_t)b * p.ybs;
   const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
