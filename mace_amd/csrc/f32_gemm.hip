@@ -35,6 +35,21 @@ struct F32GemmParams {
   int tiles_m;
 };
 
+// Which tile of which batch a workgroup computes.  Workgroup ids (tiles of a batch first, then the
+// batches) go round-robin to the 8 XCDs, each with an L2 of its own: left alone every XCD would
+// hold a few tiles of every batch and pull all operands through its L2.  Every XCD gets a
+// contiguous span of (batch, tile) instead.
+__device__ inline void span_of_block(int *bid, int *b) {
+  *bid = blockIdx.x;
+  *b = blockIdx.z;
+  const int nwg = gridDim.x * gridDim.z;
+  if (nwg % 8 != 0) return;
+  int wg = blockIdx.x + gridDim.x * blockIdx.z;
+  wg = (wg % 8) * (nwg / 8) + wg / 8;
+  *b = wg / gridDim.x;
+  *bid = wg - *b * gridDim.x;
+}
+
 __device__ inline float apply_act(float v, int act, float limit) {
   // mace/ops/ref/activation.cc:61-75
   if (act == MACE_HIP_ACT_RELU) return fmaxf(0.f, v);
@@ -50,8 +65,9 @@ __global__ __launch_bounds__(256) void f32_gemm_kernel(F32GemmParams p) {
   __shared__ float sB[2][TK][LDT];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave & 1, wn = wave >> 1;
-  const int m0 = (blockIdx.x % p.tiles_m) * TM, n0 = (blockIdx.x / p.tiles_m) * TN;
-  const int b = blockIdx.z;
+  int bid, b;
+  span_of_block(&bid, &b);
+  const int m0 = (bid % p.tiles_m) * TM, n0 = (bid / p.tiles_m) * TN;
   const float *A = p.lhs + (int64_t)b * p.lbs;
   const float *B = p.rhs + (int64_t)b * p.rbs;
 
@@ -178,8 +194,9 @@ __global__ __launch_bounds__(256 * SPLIT) void f32_gemm_vec_kernel(F32GemmParams
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int khalf = wave >> 2;           // which part of the k steps (0 when SPLIT == 1)
   const int wm = wave & 1, wn = (wave >> 1) & 1;
-  const int m0 = (blockIdx.x % p.tiles_m) * TM, n0 = (blockIdx.x / p.tiles_m) * TN;
-  const int b = blockIdx.z;
+  int bid, b;
+  span_of_block(&bid, &b);
+  const int m0 = (bid % p.tiles_m) * TM, n0 = (bid / p.tiles_m) * TN;
   const float *A = p.lhs + (int64_t)b * p.lbs;
   const float *B = p.rhs + (int64_t)b * p.rbs;
 
