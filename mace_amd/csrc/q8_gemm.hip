@@ -2883,6 +2883,9 @@ int Q8Call::kmajor_in_place(bool *done) {
     // A k-major Y operand (the ColMajor left-hand matrix of a transpose_a MatMul with a RowMajor
     // result; X k-major as well, or k-contiguous and read in place) in the same tile-count range:
     // the eight-wavefront kernel's Y half mirrors its X half, so neither operand is repacked.
+    // Two rounds of tiles from k = 512 on here as well (us per call with both operands k-major,
+    // six buffer sets in rotation, against the kernel the shape had before: 32 x 512^3 32.8 -> 16.5,
+    // 4096 x 512 x 2048 26.0 -> 16.4, 2048 x 640 x 3072 23.8 -> 16.7, 24 x 512 x 768 x 512 32.6 -> 18.0).
     {
       const bool y_kmajor = xl ? rhs_order == MACE_HIP_ROW_MAJOR : lhs_order == MACE_HIP_COL_MAJOR;
       const bool x_direct = xl ? lhs_direct : (rhs_direct && rhs_order == MACE_HIP_COL_MAJOR);
@@ -2891,8 +2894,7 @@ int Q8Call::kmajor_in_place(bool *done) {
       if (!cv && y_kmajor && x_ok && rhs_ld == 0 && !lhs_w && !rhs_w && depth >= 512 &&
           depth % 128 == 0 && yn % 16 == 0 && (uintptr_t)yp % 16 == 0 && xn > 64 && yn > 64 &&
           4 * tiles128 >= cu_n &&
-          (tiles128 <= cu_n || (depth >= 2048 && 2 * tiles128 <= 5 * cu_n) ||
-           (depth >= 1024 && tiles128 <= 2 * cu_n)) &&
+          (tiles128 <= 2 * cu_n || (depth >= 2048 && 2 * tiles128 <= 5 * cu_n)) &&
           yn * depth < ((int64_t)1 << 32) && depth < (1 << 24) && (size_t)4 * 256 * 128 <= lds_cu &&
           !(ctx->kernel_mask & MH_MASK_NO_MID)) {
         const Q8Operand Xo{xp, x_kmajor ? xn : depth, (xl ? lhs_nb : rhs_nb) > 1 ? xn * depth : 0};

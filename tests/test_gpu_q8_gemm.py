@@ -168,6 +168,7 @@ MID_SHAPES = [  # batch, rows, depth, cols, lhs batched, rhs batched, lhs order,
     (2, 1040, 640, 1008, True, True, Cm, R, R, "mid/XT/YT"), (1, 1296, 1280, 1504, True, True, R, R, Cm, "mid/YT"),
     (1, 2048, 2048, 2048, True, True, Cm, R, R, "mid/XT/YT"), (3, 912, 512, 1008, True, False, Cm, R, R, "mid/XT/YT"),
     (2, 1024, 768, 1100, False, True, Cm, Cm, R, "mid/YT"),
+    (20, 512, 512, 640, True, True, Cm, R, R, "mid/XT/YT"), (1, 4000, 512, 2000, True, True, Cm, Cm, R, "mid/YT"),
     # the same operand layout at sizes that take 256 x 256 tiles: each operand's sums in the kernel
     # (k <= 1024 or the other dimension <= 4096) or from a pass of their own, ragged last tiles,
     # ColMajor everything

@@ -177,6 +177,11 @@ def test_eight_wavefront_kernel_range(ctx):
     assert p.kernel == "q8_gemm_mid_kernel<int32_t,STAGES=4,XT=false,YT=true>" and p.launches == 1
     p = gemm(ctx, 1, 2048, 2048, 2048, lo=R, ro=R, oo=Cm)            # ColMajor result: Y is the right-hand matrix
     assert p.kernel == "q8_gemm_mid_kernel<uint8_t,STAGES=4,XT=false,YT=true>"
+    # ... two rounds of tiles from k = 512 on, as for a k-major X alone
+    p = gemm(ctx, 32, 512, 512, 512, lo=Cm)
+    assert p.kernel == "q8_gemm_mid_kernel<uint8_t,STAGES=4,XT=true,YT=true>" and p.launches == 1
+    assert "YT=true" in gemm(ctx, 1, 4096, 512, 2048, lo=Cm).kernel and "YT=true" in gemm(ctx, 24, 512, 768, 512, lo=Cm).kernel
+    assert "YT=true" not in gemm(ctx, 36, 512, 512, 512, lo=Cm).kernel   # 576 tiles
     p = gemm(ctx, 1, 2040, 2048, 2048, lo=Cm)                        # rows not in whole 16-byte pieces: repacked
     assert "YT=true" not in p.kernel and p.launches > 1
 
