@@ -131,6 +131,40 @@ def test_conv1x1_q8_channels_odd_multiple_of_8(ctx, one_launch_kernel, n, hw, ci
         assert "TAIL=true" in plan.kernel and plan.launches == 1
 
 
+def _random_conv1x1_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        n = int(rng.choice([1, 2, 5, 16, 64]))
+        hw = int(rng.choice([7, 9, 14, 28, 33, 56]))
+        cin = int(rng.choice([16, 20, 24, 32, 36, 40, 48, 64, 72, 96, 128, 144, 192, 256, 384, 512]))
+        cout = int(rng.choice([16, 24, 32, 40, 64, 96, 100, 128, 144, 160, 256, 320]))
+        if n * hw * hw * cin * cout > 3e9:
+            continue
+        cases.append((n, hw, cin, cout, int(rng.integers(1 << 30))))
+    return cases
+
+
+@pytest.mark.parametrize("n,hw,cin,cout,seed", _random_conv1x1_cases(48, 2024))
+def test_conv1x1_q8_random_shapes(ctx, n, hw, cin, cout, seed):
+    """Seeded random batches, image sizes and channel counts (MobileNet's, odd multiples of 8,
+    multiples of 4 only) under the normal dispatch, zero points over the whole uint8 range, with
+    and without a clamp narrower than the output type."""
+    rng = np.random.default_rng(seed)
+    x = rng.integers(0, 256, (n, hw, hw, cin), dtype=np.uint8)
+    f = rng.integers(0, 256, (cout, cin), dtype=np.uint8)
+    bias = rng.integers(-2 ** 15, 2 ** 15, cout).astype(np.int32)
+    z_in, z_f, z_o = int(rng.integers(0, 256)), int(rng.integers(0, 256)), int(rng.integers(0, 256))
+    s_in, s_f = np.float32(0.02), np.float32(0.01)
+    s_o = np.float32(3 * 74.0 * 74.0 * np.sqrt(cin) * float(s_in * s_f) / 255.0)
+    lo, hi = (0, 255) if rng.integers(0, 2) else (min(z_o, 200), 255)
+    want = orc.conv1x1_q8_nhwc(x, f, bias, n, hw, hw, cin, cout, s_in, z_in, s_f, z_f,
+                               np.float32(s_in * s_f), s_o, z_o, lo, hi)
+    got = conv_host(ctx, x, f, bias, n, hw, hw, cin, cout, s_in, z_in, s_f, z_f,
+                    np.float32(s_in * s_f), s_o, z_o, lo, hi)
+    np.testing.assert_array_equal(got, want, err_msg=ctx.last_plan().kernel)
+
+
 @pytest.mark.parametrize("hw,cin,cout", [(112, 32, 64), (56, 128, 128), (28, 256, 256),
                                          (14, 512, 512), (7, 1024, 1024)])
 def test_conv1x1_q8_batch64_sampled(ctx, hw, cin, cout):
