@@ -26,6 +26,7 @@
 #include "common.h"
 #include "q8_requant.h"
 
+
 namespace {
 
 
@@ -2692,17 +2693,23 @@ int Q8Call::prepare(bool *done) {
   const int64_t mid_cu = ctx->cu_count > 0 ? ctx->cu_count : 256;
   const bool mid_one_round =
       !cv && !lhs_w && !rhs_w && rhs_ld == 0 && depth >= 512 && depth % 128 == 0 &&
-      depth < (1 << 24) && mid_xn > 64 && mid_yn > 64 && 4 * mid_tiles >= mid_cu &&
-      mid_tiles <= mid_cu &&
+      depth < (1 << 24) && mid_xn > 64 && mid_yn > 64 && mid_tiles <= mid_cu &&
       (size_t)4 * 256 * 128 <= (ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536) &&
       !(ctx->kernel_mask & MH_MASK_NO_MID);
   const bool mid_y_direct = mid_xl ? (rhs_direct && rhs_order == MACE_HIP_COL_MAJOR) : lhs_direct;
   const bool mid_x_direct = mid_xl ? lhs_direct : (rhs_direct && rhs_order == MACE_HIP_COL_MAJOR);
   const bool mid_x_kmajor = mid_xl ? lhs_order == MACE_HIP_COL_MAJOR : rhs_order == MACE_HIP_ROW_MAJOR;
-  mid_first_xt = mid_one_round && mid_x_kmajor && mid_y_direct && mid_xn % 16 == 0 &&
+  // Fewer tiles than a quarter of a round (a grid of shapes from 1 to 63 tiles, us per call against
+  // the kernel that had them, six buffer sets in rotation): the kernel's time hardly depends on the
+  // tile count, so it keeps winning wherever the alternative pays for the depth -- X k-major from
+  // k = 1024 on (against the one-launch kernel 15 - 25 % faster at every tile count; at k = 512 - 640
+  // +-8 % and a batch of four 512^2 x 512 loses 9 %, so those stay), Y k-major at every depth (k = 512
+  // 8 - 18 %, k = 1024 33 - 40 % faster); k-contiguous operands tie at k = 1024 and stay.
+  const bool mid_quarter = 4 * mid_tiles >= mid_cu;
+  mid_first_xt = mid_one_round && (mid_quarter || depth >= 1024) && mid_x_kmajor && mid_y_direct && mid_xn % 16 == 0 &&
                             (uintptr_t)(mid_xl ? lhs : rhs) % 16 == 0 &&
                             mid_xn * depth < ((int64_t)1 << 32);
-  mid_first_kc = mid_one_round && mid_x_direct && mid_y_direct && depth >= 1024;
+  mid_first_kc = mid_one_round && mid_quarter && mid_x_direct && mid_y_direct && depth >= 1024;
   //   Y k-major (X k-major or k-contiguous), against the one-launch kernel: 1024^3 with both
   //     operands k-major 15.6 -> 10.4
   const bool mid_y_kmajor = mid_xl ? rhs_order == MACE_HIP_ROW_MAJOR : lhs_order == MACE_HIP_COL_MAJOR;
@@ -2825,10 +2832,12 @@ int Q8Call::kmajor_in_place(bool *done) {
     // k = 256 ties; four rounds, 8192 x 512 x 8192, lose 64 against 79)
     const bool big_xt_first = big_xt && depth >= 384 && tiles256 <= cu_n;
     // The eight-wavefront 128 x 128 kernel reads the same layout in place (second block below): one
-    // round of tiles, up to two rounds from k = 512 on, two and a half from k = 2048 on.
+    // round of tiles, up to two rounds from k = 512 on, two and a half from k = 2048 on; from
+    // k = 1024 on any number of tiles below that (1 to 63 tiles at k = 2048: 24 - 30 % faster than
+    // repack + sums + 64 x 64 tiles, at k = 4096 15 - 24 %).
     const bool mid_xt = !cv && x_kmajor && y_direct && rhs_ld == 0 && !lhs_w && !rhs_w && depth >= 512 &&
                         depth % 128 == 0 && xn % 16 == 0 && (uintptr_t)xp % 16 == 0 && xn > 64 && yn > 64 &&
-                        4 * tiles128 >= cu_n &&
+                        (4 * tiles128 >= cu_n || depth >= 1024) &&
                         (tiles128 <= 2 * cu_n || (depth >= 2048 && 2 * tiles128 <= 5 * cu_n)) &&
                         xn * depth < ((int64_t)1 << 32) && depth < (1 << 24) &&
                         (size_t)4 * 256 * 128 <= lds_cu && !(ctx->kernel_mask & MH_MASK_NO_MID);
@@ -2893,7 +2902,6 @@ int Q8Call::kmajor_in_place(bool *done) {
                                  : x_direct;
       if (!cv && y_kmajor && x_ok && rhs_ld == 0 && !lhs_w && !rhs_w && depth >= 512 &&
           depth % 128 == 0 && yn % 16 == 0 && (uintptr_t)yp % 16 == 0 && xn > 64 && yn > 64 &&
-          4 * tiles128 >= cu_n &&
           (tiles128 <= 2 * cu_n || (depth >= 2048 && 2 * tiles128 <= 5 * cu_n)) &&
           yn * depth < ((int64_t)1 << 32) && depth < (1 << 24) && (size_t)4 * 256 * 128 <= lds_cu &&
           !(ctx->kernel_mask & MH_MASK_NO_MID)) {
@@ -3163,9 +3171,11 @@ int Q8Call::general() {
   const int xres_tx = (xn <= 64 || xres_narrow) ? 64 : 128;
   const bool xres_cv = cv && !cv_small && out_u8 && cv->cin % 64 == 0 && depth % 64 == 0;
   const int64_t tiles128 = ((xn + 127) / 128) * ((yn + 127) / 128) * batch;
-  // (one round of 128 x 128 tiles at k >= 512 is faster on the eight-wavefront kernel, see above)
+  // (one round of 128 x 128 tiles at k >= 512 is faster on the eight-wavefront kernel, see above;
+  // from k = 2048 on also below a quarter of a round, where the 64 x 64 tiles and their sums pass took
+  // the shape: 6 - 11 % faster with k-contiguous operands at 1 to 63 tiles)
   const bool mid_shape = !cv && !stream && kk % 128 == 0 && kk >= 512 && xn > 64 && yn > 64 &&
-                         4 * tiles128 >= cu_n && L.ld < (1 << 24) && R.ld < (1 << 24) &&
+                         (4 * tiles128 >= cu_n || kk >= 2048) && L.ld < (1 << 24) && R.ld < (1 << 24) &&
                          (size_t)4 * 256 * 128 <= lds_cu && !(ctx->kernel_mask & MH_MASK_NO_MID);
   const bool xres = (!cv || xres_cv) && !stream && depth > 0 && (kk % 64 == 0 || tail_xres) && yn >= 256 &&
                     xres_fits(xres_tx) && !(mid_shape && tiles128 <= cu_n) &&

@@ -169,6 +169,10 @@ MID_SHAPES = [  # batch, rows, depth, cols, lhs batched, rhs batched, lhs order,
     (1, 2048, 2048, 2048, True, True, Cm, R, R, "mid/XT/YT"), (3, 912, 512, 1008, True, False, Cm, R, R, "mid/XT/YT"),
     (2, 1024, 768, 1100, False, True, Cm, Cm, R, "mid/YT"),
     (20, 512, 512, 640, True, True, Cm, R, R, "mid/XT/YT"), (1, 4000, 512, 2000, True, True, Cm, Cm, R, "mid/YT"),
+    # a handful of tiles, one tile, fewer workgroups than XCDs: long depths keep the kernel
+    (1, 130, 1024, 208, True, True, R, R, R, "mid/XT"), (1, 128, 2048, 144, True, True, R, Cm, R, "mid"),
+    (2, 112, 512, 176, True, True, Cm, R, R, "mid/XT/YT"), (1, 300, 1152, 112, True, True, R, R, Cm, "mid/YT"),
+    (3, 260, 1024, 144, True, False, R, R, R, "mid/XT"), (1, 65, 2176, 65, True, True, Cm, Cm, Cm, "mid"),
     # the same operand layout at sizes that take 256 x 256 tiles: each operand's sums in the kernel
     # (k <= 1024 or the other dimension <= 4096) or from a pass of their own, ragged last tiles,
     # ColMajor everything

@@ -170,6 +170,14 @@ def test_eight_wavefront_kernel_range(ctx):
     assert fam(gemm(ctx, 1, 3072, 1024, 3072)) != mid                 # 576 tiles
     assert fam(gemm(ctx, 36, 512, 512, 512)) != mid                   # 576 tiles
     assert fam(gemm(ctx, 1, 2048, 2048, 2048, mask=mh.MASK_NO_MID)) != mid
+    # fewer tiles than a quarter of a round: a k-major X from k = 1024 on, k-contiguous operands from
+    # k = 2048 on (a k-major Y at any depth, below)
+    assert fam(gemm(ctx, 1, 256, 1024, 256)) == mid and gemm(ctx, 1, 256, 1024, 256).launches == 1
+    assert fam(gemm(ctx, 1, 128, 2048, 384)) == mid and fam(gemm(ctx, 4, 256, 4096, 256)) == mid
+    assert fam(gemm(ctx, 1, 256, 512, 256)) == mh.KF_Q8_GEMM_FUSED_SMALL
+    assert fam(gemm(ctx, 1, 256, 2048, 256, ro=Cm)) == mid
+    assert fam(gemm(ctx, 1, 256, 1024, 256, ro=Cm)) == mh.KF_Q8_GEMM_FUSED_SMALL
+    assert "YT=true" in gemm(ctx, 1, 256, 512, 256, lo=Cm).kernel and "YT=true" in gemm(ctx, 1, 128, 640, 144, lo=Cm, ro=Cm).kernel
     # k-major Y (transpose_a with a RowMajor result), X k-major or k-contiguous: read as they lie
     p = gemm(ctx, 1, 2048, 2048, 2048, lo=Cm)
     assert p.kernel == "q8_gemm_mid_kernel<uint8_t,STAGES=4,XT=true,YT=true>" and p.launches == 1 and p.aux == 0
