@@ -2723,15 +2723,20 @@ int Q8Call::prepare(bool *done) {
   // long Y panel and an X tile that fits in LDS: the resident-tile kernel walks k up to the next
   // multiple of 64 itself (pieces past the end count as zeros), so nothing is repacked and the
   // one-launch kernel, which otherwise takes such depths at any size, keeps the small problems
-  // (200704 x 96 x 128: 25.8 us there).
+  // (200704 x 96 x 128: 25.8 us there).  Depths of 16 to 48 as well, where the X panel has more rows
+  // than the streaming kernel takes (one k group, mostly padding, still beats the one-launch kernel:
+  // 200704 x 32 x 256 35.4 -> 25.5 us, 50176 x 16 x 1024 36.6 -> 25.8, 50176 x 32 x 512 20.6 -> 15.9,
+  // 200704 x 16 x 24 11.2 -> 9.0).
   const int64_t tail_kp = (depth + 63) & ~(int64_t)63;
   tail_xres =
-      !cv && !lhs_w && !rhs_w && rhs_ld == 0 && depth > 64 && depth % 64 != 0 && depth % 16 == 0 &&
+      !cv && !lhs_w && !rhs_w && rhs_ld == 0 && depth >= 16 && depth % 64 != 0 && depth % 16 == 0 &&
       lhs_direct && rhs_direct && lhs_order == MACE_HIP_ROW_MAJOR && rhs_order == MACE_HIP_COL_MAJOR &&
       mid_yn >= 256 &&
       2 * (XRES_SC_BYTES + (size_t)(mid_xn <= 64 ? 64 : 128) * tail_kp) <=
           (ctx->lds_bytes > 0 ? (size_t)ctx->lds_bytes : 65536) &&
       !mh_q8_small_problem(ctx, batch, rows, cols, depth, true, false) &&
+      // (depths of 16 to 48 against at most 128 X rows are the streaming kernel's, see `stream`)
+      !(out_u8 && rq.table && mh_q8_stream_shape(depth, mid_xn, mid_yn) && (uintptr_t)out % 16 == 0) &&
       !(ctx->kernel_mask & MH_MASK_NO_XRES);
   return MACE_HIP_SUCCESS;
 }

@@ -120,12 +120,15 @@ XRES_SHAPES = [  # batch, rows, depth, cols, lhs order, rhs order, out order, ke
     # long k in 64-row tiles (128 rows would not fit in LDS twice; k % 128 != 0 keeps the
     # eight-wavefront kernel away)
     (1, 3136, 960, 500, R, Cm, R, "xres"), (1, 5000, 960, 250, R, Cm, R, "xres"),
-    # a depth tail read in place
-    (2, 70000, 144, 24, R, Cm, R, "xres/TAIL"),
+    # a depth tail read in place; depths below 64 against more X rows than the streaming kernel takes
+    (2, 70000, 144, 24, R, Cm, R, "xres/TAIL"), (1, 30000, 32, 192, R, Cm, R, "xres/TAIL"),
+    (1, 24000, 16, 300, R, Cm, R, "xres/TAIL"), (2, 12000, 48, 144, R, Cm, R, "xres/TAIL"),
+    (1, 256, 32, 70000, R, Cm, Cm, "xres/TAIL"),
+    (1, 100000, 48, 40, R, Cm, R, "xres/TAIL"),
     # neighbours that other kernels take: a short, narrow X panel (uint8 only), one round of
-    # 128 x 128 tiles, a depth below 64 that is not a multiple of 64
+    # 128 x 128 tiles, a depth below 64 that is not a multiple of 64 against fewer than 256 Y rows
     (1, 140000, 64, 48, R, Cm, R, "stream"), (4, 512, 512, 512, R, R, R, "mid/XT"),
-    (1, 3136, 1024, 500, R, Cm, R, "mid"), (1, 100000, 48, 40, R, Cm, R, "tiled"),
+    (1, 3136, 1024, 500, R, Cm, R, "mid"), (1, 200, 48, 100000, R, Cm, R, "tiled"),
 ]
 
 

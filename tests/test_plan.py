@@ -170,6 +170,12 @@ def test_eight_wavefront_kernel_range(ctx):
     assert fam(gemm(ctx, 1, 3072, 1024, 3072)) != mid                 # 576 tiles
     assert fam(gemm(ctx, 36, 512, 512, 512)) != mid                   # 576 tiles
     assert fam(gemm(ctx, 1, 2048, 2048, 2048, mask=mh.MASK_NO_MID)) != mid
+    # depths of 16 to 48 (not whole 64-byte groups) against more X rows than the streaming kernel takes:
+    # the resident-tile kernel's depth tail, one launch; with at most 128 X rows the streaming kernel
+    p = gemm(ctx, 1, 200704, 32, 256, ro=Cm)
+    assert "TAIL=true" in p.kernel and p.launches == 1
+    assert "TAIL=true" in gemm(ctx, 1, 50176, 16, 1024, ro=Cm).kernel
+    assert fam(gemm(ctx, 1, 200704, 32, 64, ro=Cm)) == mh.KF_Q8_GEMM_STREAM
     # fewer tiles than a quarter of a round: a k-major X from k = 1024 on, k-contiguous operands from
     # k = 2048 on (a k-major Y at any depth, below)
     assert fam(gemm(ctx, 1, 256, 1024, 256)) == mid and gemm(ctx, 1, 256, 1024, 256).launches == 1
