@@ -768,7 +768,10 @@ int launch_gemv(mace_hip_ctx *ctx, GemvParams &p, int lhs_batched) {
   constexpr bool out_u8 = sizeof(OutT) == 1;
   // Two vectors against long rows stay on the row-block kernel (one pass, the weights streamed
   // once: 5.6 us against 5.9 us at 4096 x 4096); from three on the matrix-core kernels win.
-  const bool few = !lhs_batched && p.batch == 2 && p.W >= 2048 && (size_t)2 * p.W <= 64 * 1024;
+  // (rows of 2 KiB from 4096 rows on go the other way: 8192 x 2048 7.4 against 5.4 us, 4096 x 2048
+  // 5.4 against 4.9)
+  const bool few = !lhs_batched && p.batch == 2 && p.W >= 2048 && (size_t)2 * p.W <= 64 * 1024 &&
+                   (p.W >= 3072 || p.H < 4096);
   if (few) nb = 2;
   // shared weights against more vectors: the batch goes through the matrix cores
   if (vec && !lhs_batched && !few && p.W >= 64 && p.batch >= 2 && p.rhs_bs % 16 == 0) {
