@@ -147,7 +147,8 @@ enum {
   MACE_HIP_AUX_F32_PAD = 256,            /* zero-padded copy of an NCHW input                     */
   MACE_HIP_AUX_FILL = 512,               /* constant fill (zero-point page, empty depth)          */
   MACE_HIP_AUX_WEIGHT_HIT = 1024,        /* a registered weight's panel / sums were reused        */
-  MACE_HIP_AUX_WEIGHT_BUILD = 2048       /* ... were built by this call                           */
+  MACE_HIP_AUX_WEIGHT_BUILD = 2048,      /* ... were built by this call                           */
+  MACE_HIP_AUX_F32_KSPLIT = 4096         /* fp32 GEMM: parts of the depth added up by a second launch */
 };
 typedef struct mace_hip_plan {
   int family;      /* MACE_HIP_KF_*; NONE when the call launched no main kernel (empty result)    */

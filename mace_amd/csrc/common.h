@@ -571,6 +571,26 @@ inline bool mh_q8_small_problem(const mace_hip_ctx *ctx, int64_t batch, int64_t 
   return any_size || (wgs <= 4 * cus && macs <= (vec ? 1024.0 : 128.0) * 1024 * 1024);
 }
 
+// Into how many parts the fp32 GEMM deals a tile's k range (1: no split): only while at most half
+// the CUs would have a tile, at least four k tiles of 16 per part, at most 16 parts.
+inline int mh_f32_ksplit(const mace_hip_ctx *ctx, int64_t batch, int64_t rows, int64_t cols,
+                         int64_t depth) {
+  const int64_t cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
+  const int64_t wgs = ((rows + 127) / 128) * ((cols + 127) / 128) * batch;
+  const int64_t nk = (depth + 15) / 16;
+  if (wgs <= 0 || 2 * wgs > cus || nk < 8) return 1;
+  int64_t parts = cus / wgs;
+  if (parts > nk / 4) parts = nk / 4;
+  if (parts > 16) parts = 16;
+  return parts < 2 ? 1 : (int)parts;
+}
+// scratch of that split (0 without one)
+inline size_t mh_f32_ksplit_bytes(const mace_hip_ctx *ctx, int64_t batch, int64_t rows, int64_t cols,
+                                  int64_t depth) {
+  const int parts = mh_f32_ksplit(ctx, batch, rows, cols, depth);
+  return parts > 1 ? sizeof(float) * (size_t)parts * batch * rows * cols + 256 : 0;
+}
+
 // Raises a kernel's dynamic LDS limit to at least `bytes`; remembered per context and kernel, since
 // hipFuncSetAttribute costs about as much as a launch and the attribute stays set.
 inline hipError_t mh_allow_big_lds(mace_hip_ctx *ctx, const void *kernel, size_t bytes) {

@@ -598,7 +598,7 @@ int mace_hip_gemm_f32_host(mace_hip_ctx *ctx, const float *lhs, const float *rhs
   const size_t lb = sizeof(float) * (lhs_batched ? batch : 1) * rows * depth;
   const size_t rb = sizeof(float) * (rhs_batched ? batch : 1) * depth * cols;
   const size_t ob = sizeof(float) * batch * rows * cols;
-  MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, lb + rb + ob));
+  MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, lb + rb + ob + mh_f32_ksplit_bytes(ctx, batch, rows, cols, depth) + 4096));
   Stage st(ctx);
   void *dl, *dr, *dout;
   MH_RETURN_IF_ERROR(st.in(lhs, lb, &dl));
@@ -654,7 +654,7 @@ int mace_hip_conv1x1_f32_nchw_host(mace_hip_ctx *ctx, const float *input,
   const size_t fb = sizeof(float) * cout * cin;
   const size_t bb = bias ? sizeof(float) * cout : 0;
   const size_t ob = sizeof(float) * n * cout * hw;
-  MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, ib + fb + bb + ob));
+  MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, ib + fb + bb + ob + mh_f32_ksplit_bytes(ctx, n, cout, hw, cin) + 4096));
   Stage st(ctx);
   void *di, *df, *db, *dout;
   MH_RETURN_IF_ERROR(st.in(input, ib, &di));
@@ -682,7 +682,8 @@ int mace_hip_matmul_f32_host(mace_hip_ctx *ctx, const float *lhs, const float *r
   const size_t rb = sizeof(float) * (rhs_batched ? batch : 1) * rhs_rows * rhs_cols;
   const size_t bb = bias ? sizeof(float) * cols : 0;
   const size_t ob = sizeof(float) * batch * rows * cols;
-  MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, lb + rb + bb + ob));
+  MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, lb + rb + bb + ob +
+                                           mh_f32_ksplit_bytes(ctx, batch, rows, cols, transpose_lhs ? lhs_rows : lhs_cols) + 4096));
   Stage st(ctx);
   void *dl, *dr, *db, *dout;
   MH_RETURN_IF_ERROR(st.in(lhs, lb, &dl));
@@ -715,7 +716,8 @@ int mace_hip_conv2d_f32_nchw_host(mace_hip_ctx *ctx, const float *input, const f
   const size_t fb = sizeof(float) * cout * cin;
   const size_t bb = bias ? sizeof(float) * cout : 0;
   const size_t ob = sizeof(float) * n * cout * ohw;
-  MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, ib + fb + bb + ob + sizeof(float) * n * cin * ohw + 4096));
+  MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, ib + fb + bb + ob + sizeof(float) * n * cin * ohw +
+                                           mh_f32_ksplit_bytes(ctx, n, cout, ohw, cin) + 8192));
   Stage st(ctx);
   void *di, *df, *db, *dout;
   MH_RETURN_IF_ERROR(st.in(input, ib, &di));

@@ -33,6 +33,12 @@ struct F32GemmParams {
   int act;
   float limit;
   int tiles_m;
+  // k split: blockIdx.y takes k tiles [y kt_split, (y + 1) kt_split) and
+  // stores its raw sums into part[(y batches + b) obs + ...] with the result's own strides;
+  // f32_ksplit_reduce_kernel adds the parts in the order of y and applies bias and activation.
+  // kt_split = 0: no split.
+  float *part;
+  int kt_split;
 };
 
 // Which tile of which batch a workgroup computes.  Workgroup ids (tiles of a batch first, then the
@@ -105,12 +111,15 @@ __global__ __launch_bounds__(256) void f32_gemm_kernel(F32GemmParams p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  const int nk = (p.K + TK - 1) / TK;
-  load_global(0);
+  // (k split: this workgroup's k tiles are [kt0, nk), see F32GemmParams)
+  const int kt0 = p.kt_split * (int)blockIdx.y;
+  const int nk_all = (p.K + TK - 1) / TK;
+  const int nk = p.kt_split ? min(kt0 + p.kt_split, nk_all) : nk_all;
+  load_global(kt0 * TK);
   store_lds(0);
   __syncthreads();
-  for (int kt = 0; kt < nk; ++kt) {
-    const int buf = kt & 1;
+  for (int kt = kt0; kt < nk; ++kt) {
+    const int buf = (kt - kt0) & 1;
     if (kt + 1 < nk) load_global((kt + 1) * TK);
     // v_mfma_f32_32x32x2: lane l supplies A[row l % 32][k = l / 32], B[k = l / 32][col l % 32].
     // The fragments of step ks + 1 are read while the MFMAs of step ks run (one wavefront per
@@ -139,7 +148,8 @@ __global__ __launch_bounds__(256) void f32_gemm_kernel(F32GemmParams p) {
     __syncthreads();
   }
 
-  float *O = p.out + (int64_t)b * p.obs;
+  const bool raw = p.kt_split != 0;   // a part of the k range: bias and activation come with the sum of the parts
+  float *O = raw ? p.part + ((int64_t)blockIdx.y * gridDim.z + b) * p.obs : p.out + (int64_t)b * p.obs;
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -150,9 +160,11 @@ __global__ __launch_bounds__(256) void f32_gemm_kernel(F32GemmParams p) {
         const int m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
         if (m < p.M && n < p.N) {
           float v = acc[i][j][r];
-          if (p.bias_row) v = v + p.bias_row[m];
-          if (p.bias_col) v = v + p.bias_col[n];
-          v = apply_act(v, p.act, p.limit);
+          if (!raw) {
+            if (p.bias_row) v = v + p.bias_row[m];
+            if (p.bias_col) v = v + p.bias_col[n];
+            v = apply_act(v, p.act, p.limit);
+          }
           O[(int64_t)m * p.ors + (int64_t)n * p.ocs] = v;
         }
       }
@@ -230,6 +242,14 @@ __global__ __launch_bounds__(256 * SPLIT) void f32_gemm_vec_kernel(F32GemmParams
   }
   const int64_t a_step = LK ? TK : (int64_t)TK * p.lcs;
   const int64_t b_step = RK ? TK : (int64_t)TK * p.rrs;
+  const int kt0 = p.kt_split * (int)blockIdx.y;   // this workgroup's first k tile
+  if (p.kt_split) {
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      pa[i] += kt0 * a_step;
+      pb[i] += kt0 * b_step;
+    }
+  }
   f4v ra[NP], rb[NP];
   auto load_global = [&]() {
 #pragma unroll
@@ -274,7 +294,7 @@ __global__ __launch_bounds__(256 * SPLIT) void f32_gemm_vec_kernel(F32GemmParams
   // read during the last k step of tile kt, in front of the barrier, and no LDS latency is
   // exposed behind it.  The buffer written (tile kt + 2's = tile kt - 1's) is free: everybody
   // passed the barrier that ended tile kt - 1.
-  const int nk = p.K / TK;
+  const int nk = p.kt_split ? min(p.kt_split, p.K / TK - kt0) : p.K / TK;
   load_global();
   store_lds(0);
   if (nk > 1) {
@@ -343,7 +363,8 @@ __global__ __launch_bounds__(256 * SPLIT) void f32_gemm_vec_kernel(F32GemmParams
     if (khalf == 1) return;
   }
 
-  float *O = p.out + (int64_t)b * p.obs;
+  const bool raw = p.kt_split != 0;   // a part of the k range: bias and activation come with the sum of the parts
+  float *O = raw ? p.part + ((int64_t)blockIdx.y * gridDim.z + b) * p.obs : p.out + (int64_t)b * p.obs;
   const bool whole = m0 + TM <= p.M && n0 + TN <= p.N;
 #pragma unroll
   for (int i = 0; i < 2; ++i)
@@ -355,13 +376,31 @@ __global__ __launch_bounds__(256 * SPLIT) void f32_gemm_vec_kernel(F32GemmParams
         const int m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
         if (whole || (m < p.M && n < p.N)) {
           float v = acc[i][j][r];
-          if (p.bias_row) v = v + p.bias_row[m];
-          if (p.bias_col) v = v + p.bias_col[n];
-          v = apply_act(v, p.act, p.limit);
+          if (!raw) {
+            if (p.bias_row) v = v + p.bias_row[m];
+            if (p.bias_col) v = v + p.bias_col[n];
+            v = apply_act(v, p.act, p.limit);
+          }
           O[(int64_t)m * p.ors + (int64_t)n * p.ocs] = v;
         }
       }
     }
+}
+
+// The sum of a k split's parts, in the order of the parts, with the bias and the activation of the
+// call: element i of batch b lies at b obs + i in every part and in the result (dense M x N).
+__global__ __launch_bounds__(256) void f32_ksplit_reduce_kernel(F32GemmParams p, int parts, int64_t total) {
+  const int64_t mn = (int64_t)p.M * p.N;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    float v = p.part[i];
+    for (int s = 1; s < parts; ++s) v = v + p.part[(int64_t)s * total + i];
+    const int64_t j = i % mn;
+    const int m = p.ocs == 1 ? (int)(j / p.N) : (int)(j % p.M);
+    const int n = p.ocs == 1 ? (int)(j % p.N) : (int)(j / p.M);
+    if (p.bias_row) v = v + p.bias_row[m];
+    if (p.bias_col) v = v + p.bias_col[n];
+    p.out[i] = apply_act(v, p.act, p.limit);
+  }
 }
 
 // images of in_h x in_w copied into zero-filled images of ph x pw at (top, left)
@@ -507,6 +546,25 @@ int mh_f32_gemm(mace_hip_ctx *ctx, const float *lhs, const float *rhs, int64_t b
   const bool vec = depth % TK == 0 && (lk || rows % 4 == 0) && (rk || cols % 4 == 0) &&
                    rows >= 4 && cols >= 4 && ((uintptr_t)lhs % 16 == 0) &&
                    ((uintptr_t)rhs % 16 == 0);
+  // Few tiles and a long depth: the k tiles are dealt to several workgroups per tile, whose parts a
+  // second launch adds up in a fixed order.  (A tile's time is its k tiles at about 1 us each
+  // whatever else runs: 512^3, 16 tiles, took 43.7 us with 240 CUs idle.)
+  ArenaScope scope(ctx);
+  const int parts = mh_f32_ksplit(ctx, batch, rows, cols, depth);
+  if (parts > 1) {
+    const size_t bytes = mh_f32_ksplit_bytes(ctx, batch, rows, cols, depth);
+    const bool room = ctx->arena_used + bytes + 16 * 256 <= ctx->arena_bytes;
+    // (scratch that does not fit while other slices of the arena are in use: no split)
+    if (room || ctx->arena_used == 0) {
+      MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, bytes));
+      p.part = (float *)mh_arena_take(ctx, bytes);
+      if (!p.part) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
+      const int64_t nk = (depth + TK - 1) / TK;
+      p.kt_split = (int)((nk + parts - 1) / parts);
+      grid.y = (unsigned)((nk + p.kt_split - 1) / p.kt_split);
+      mh_plan_aux(ctx, MACE_HIP_AUX_F32_KSPLIT);
+    }
+  }
   if (vec) mh_plan_main(ctx, MACE_HIP_KF_F32_GEMM_VEC, mhv::f32_gemm_vec(split, lk, rk), grid,
                         split ? block2 : block, 0);
   else mh_plan_main(ctx, MACE_HIP_KF_F32_GEMM_GENERAL, mhv::f32_gemm_general(lk, rk), grid, block, 0);
@@ -524,6 +582,12 @@ int mh_f32_gemm(mace_hip_ctx *ctx, const float *lhs, const float *rhs, int64_t b
   else if (rk) MH_KLAUNCH(ctx, (f32_gemm_kernel<false, true>), grid, block, 0, ctx->stream, p);
   else MH_KLAUNCH(ctx, (f32_gemm_kernel<false, false>), grid, block, 0, ctx->stream, p);
   MH_PROF_END(ctx);
+  if (p.kt_split) {
+    const int64_t total = batch * rows * cols;
+    const int64_t blocks = (total + 255) / 256;
+    MH_KLAUNCH(ctx, f32_ksplit_reduce_kernel, dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256), 0,
+               ctx->stream, p, (int)grid.y, total);
+  }
   MH_LAUNCH_CHECK(ctx);
   return MACE_HIP_SUCCESS;
 }
@@ -670,7 +734,8 @@ int mace_hip_conv2d_f32_nchw(mace_hip_ctx *ctx, const float *input, const float 
   MH_CHECK(ctx, total < (1ll << 40), "dimension too large");
   if (total == 0 || cout == 0) return MACE_HIP_SUCCESS;
   MH_CHECK(ctx, input && out, "null operand");
-  MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, sizeof(float) * (size_t)total));
+  MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, sizeof(float) * (size_t)total +
+                                           mh_f32_ksplit_bytes(ctx, n, cout, ph * pw, cin) + 4096));
   ArenaScope scope(ctx);
   float *padded = (float *)mh_arena_take(ctx, sizeof(float) * (size_t)total);
   if (!padded) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");

@@ -90,6 +90,91 @@ def test_gemm_f32_parity(ctx, batch, rows, cols, depth, lm, rm, om, lb, rb):
     near(got, orc.gemm_f32(l, r, batch, rows, cols, depth, lm, rm, om, lb, rb, acc64=True))
 
 
+# Few tiles and a long depth: the k tiles of a tile are dealt to several workgroups and a second
+# launch adds their parts up (with the bias and the activation).  Both kernels (16-byte loads;
+# bounds-checked: extents that are not multiples of 4, a depth that is not a multiple of 16, whose
+# last k tile is partial), every layout, batches, one side shared.
+KSPLIT_CASES = [(1, 300, 260, 1024, lm, rm, om, True, True, "vec")
+                for lm in (R, Cm) for rm in (R, Cm) for om in (R, Cm)]
+KSPLIT_CASES += [(2, 131, 77, 512, R, Cm, R, True, True, "vec"), (3, 128, 128, 2048, R, R, Cm, False, True, "vec"),
+                 (1, 512, 512, 512, R, R, R, True, True, "vec"), (2, 260, 4, 640, Cm, R, R, True, False, "vec")]
+KSPLIT_CASES += [(1, 47, 69, 640, lm, rm, om, True, True, "general")
+                 for lm in (R, Cm) for rm in (R, Cm) for om in (R, Cm)]
+KSPLIT_CASES += [(1, 49, 130, 1000, R, R, R, True, True, "general"), (2, 1024, 49, 200, R, R, R, False, True, "general"),
+                 (3, 33, 35, 129, Cm, Cm, Cm, True, True, "general")]
+
+
+@pytest.mark.parametrize("batch,rows,cols,depth,lm,rm,om,lb,rb,kernel", KSPLIT_CASES)
+def test_gemm_f32_k_split(ctx, batch, rows, cols, depth, lm, rm, om, lb, rb, kernel):
+    rng = np.random.default_rng(rows * 1000 + cols + depth + lm * 4 + rm * 2 + om)
+    L = rng.standard_normal(((batch if lb else 1), rows, depth)).astype(np.float32)
+    Rr = rng.standard_normal(((batch if rb else 1), depth, cols)).astype(np.float32)
+    l, r = as_major(L, lm), as_major(Rr, rm)
+    got = gemm_host(ctx, l, r, batch, rows, cols, depth, lm, rm, om, lb, rb)
+    plan = ctx.last_plan()
+    # (an operand that runs along k may have any number of rows: those layouts of the "general"
+    # group with a depth in whole k tiles take the 16-byte loads after all)
+    vec = depth % 16 == 0 and (lm == R or rows % 4 == 0) and (rm == Cm or cols % 4 == 0)
+    assert (kernel == "vec") <= vec
+    assert plan.family == (mh.KF_F32_GEMM_VEC if vec else mh.KF_F32_GEMM_GENERAL), plan
+    assert plan.aux & mh.AUX_F32_KSPLIT and plan.launches == 2 and plan.grid[1] >= 2, plan
+    near(got, orc.gemm_f32(l, r, batch, rows, cols, depth, lm, rm, om, lb, rb))
+    want = orc.gemm_f32(l, r, batch, rows, cols, depth, lm, rm, om, lb, rb, acc64=True)
+    near(got, want)
+    assert np.linalg.norm(got.astype(np.float64) - want) <= 1e-4 * np.linalg.norm(want)
+
+
+def test_k_split_bias_and_activation(ctx):
+    """The second launch of a k split applies MatMul's per-column bias and a convolution's
+    per-channel bias and activation: batch-1 pointwise layers (a handful of tiles, depths of 256 to
+    1024), on host and on device tensors, and through the padded Conv2D."""
+    rng = np.random.default_rng(5)
+    b, rows, depth, cols = 2, 200, 768, 132
+    A = rng.standard_normal((b, rows, depth)).astype(np.float32)
+    B = rng.standard_normal((depth, cols)).astype(np.float32)
+    bias = rng.standard_normal(cols).astype(np.float32)
+    out = np.empty(b * rows * cols, np.float32)
+    ctx.call("mace_hip_matmul_f32_host", ptr(A), ptr(B), ptr(bias), b, rows, depth, depth, cols,
+             0, 0, 1, 0, ptr(out))
+    assert ctx.last_plan().aux & mh.AUX_F32_KSPLIT
+    want = orc.gemm_f32(A, B, b, rows, cols, depth, R, R, R, True, False, acc64=True).reshape(b * rows, cols)
+    near(out, (want + bias[None, :]).reshape(-1))
+    for (n, cin, h, cout, act, limit, with_bias) in ((1, 1024, 7, 1024, mh.ACT_RELUX, 6.0, True),
+                                                     (1, 512, 14, 512, mh.ACT_RELU, 0.0, True),
+                                                     (2, 256, 28, 256, mh.ACT_NOOP, 0.0, False),
+                                                     (1, 300, 5, 70, mh.ACT_RELUX, 1.0, True)):
+        hw = h * h
+        x = rng.standard_normal((n, cin, hw)).astype(np.float32)
+        f = (rng.standard_normal((cout, cin)) / np.sqrt(cin)).astype(np.float32)
+        cb = rng.standard_normal(cout).astype(np.float32) if with_bias else None
+        want = orc.conv1x1_f32_nchw(x, f, cb, n, cin, hw, cout, act, limit, nthreads=16).reshape(-1)
+        got = np.empty(n * cout * hw, np.float32)
+        ctx.call("mace_hip_conv1x1_f32_nchw_host", ptr(x), ptr(f), ptr(cb), n, cin, hw, cout, act, limit, ptr(got))
+        assert ctx.last_plan().aux & mh.AUX_F32_KSPLIT, ctx.last_plan()
+        near(got, want)
+        d = Dev()
+        t, p = d.empty(n * cout * hw, np.float32)
+        dx, df, db = d.put(x), d.put(f), d.put(cb)
+        d.sync()
+        ctx.call("mace_hip_conv1x1_f32_nchw", dx, df, db, n, cin, hw, cout, act, limit, p)
+        assert ctx.last_plan().aux & mh.AUX_F32_KSPLIT and ctx.last_plan().launches == 2
+        ctx.sync()
+        near(t.cpu().numpy(), want)
+        if act != mh.ACT_NOOP:
+            assert got.min() >= 0.0 and (got == 0.0).any() and (act != mh.ACT_RELUX or got.max() <= limit)
+    n, cin, h, w, cout, ph, pw = 1, 384, 10, 6, 130, 3, 2
+    x = rng.standard_normal((n, cin, h, w)).astype(np.float32)
+    f = (rng.standard_normal((cout, cin)) / np.sqrt(cin)).astype(np.float32)
+    cb = rng.standard_normal(cout).astype(np.float32)
+    xp = np.zeros((n, cin, h + ph, w + pw), np.float32)
+    xp[:, :, ph // 2:ph // 2 + h, pw // 2:pw // 2 + w] = x
+    got = np.empty(n * cout * (h + ph) * (w + pw), np.float32)
+    ctx.call("mace_hip_conv2d_f32_nchw_host", ptr(x), ptr(f), ptr(cb), n, cin, h, w, cout, 1, 1,
+             1, 1, 1, 1, ph, pw, mh.ACT_RELUX, 2.0, ptr(got))
+    assert ctx.last_plan().aux & mh.AUX_F32_KSPLIT and ctx.last_plan().aux & mh.AUX_F32_PAD
+    near(got, orc.conv1x1_f32_nchw(xp, f, cb, n, cin, (h + ph) * (w + pw), cout, mh.ACT_RELUX, 2.0).reshape(-1))
+
+
 @pytest.mark.parametrize("case", GOLDEN["matmul_f32"], ids=lambda c: c["source"][-20:])
 def test_gemm_f32_reference_goldens(ctx, case):
     """matmul_test.cc:55-72 through the transpose-form entry point, as MatMulOp calls it."""

@@ -118,6 +118,18 @@ def test_config2_f32_gemm(ctx):
             assert p.grid == (64, 1, 4) and p.block == 512
     ctx.call("mace_hip_gemm_f32", A, B, 5, 1024, 1024, 1024, 0, 0, 0, 1, 1, O)    # 320 tiles: SPLIT = 1
     assert "SPLIT=1" in ctx.last_plan().kernel and ctx.last_plan().block == 256
+    # few tiles and a long depth: the k tiles go to several workgroups per tile and a second launch
+    # adds the parts up; not when more than half the CUs have a tile, nor below eight k tiles
+    ctx.call("mace_hip_gemm_f32", A, B, 1, 512, 512, 512, 0, 0, 0, 1, 1, O)
+    p = ctx.last_plan()
+    assert p.aux == mh.AUX_F32_KSPLIT and p.launches == 2 and p.grid == (16, 8, 1) and "SPLIT=2" in p.kernel, p
+    ctx.call("mace_hip_gemm_f32", A, B, 1, 1024, 49, 1024, 0, 0, 0, 1, 1, O)      # 7 x 7 x 1024 -> 1024 at batch 1
+    p = ctx.last_plan()
+    assert p.family == mh.KF_F32_GEMM_GENERAL and p.aux == mh.AUX_F32_KSPLIT and p.grid == (8, 16, 1), p
+    ctx.call("mace_hip_gemm_f32", A, B, 3, 1024, 1024, 1024, 0, 0, 0, 1, 1, O)    # 192 tiles
+    assert ctx.last_plan().aux == 0 and ctx.last_plan().launches == 1
+    ctx.call("mace_hip_gemm_f32", A, B, 1, 512, 512, 112, 0, 0, 0, 1, 1, O)       # seven k tiles
+    assert ctx.last_plan().aux == 0 and ctx.last_plan().grid == (16, 1, 1)
     ctx.call("mace_hip_gemv_f32", A, B, BIAS, 1, 4096, 4096, 0, 1, O)
     assert ctx.last_plan().kernel == "f32_gemv_vec_kernel<NB=1>"
     ctx.call("mace_hip_gemv_f32_act", A, B, BIAS, 8, 4096, 4096, 0, 1, mh.ACT_RELUX, 6.0, O)
