@@ -296,6 +296,183 @@ __global__ __launch_bounds__(256, 3) void q8_conv_short_kernel(ConvShortParams p
   }
 }
 
+// ---- convolutions with several taps of whole 16-byte channel pieces (3 x 3 on 16 or 32 channels) ----
+//
+// The same arrangement as the short-patch kernel above -- a strip of output rows per workgroup,
+// its input rows staged in LDS with padding materialised, the filter in registers as MFMA
+// fragments, the streaming kernel's epilogue -- for patches of KS k steps of 32 bytes.  With the
+// channel count a multiple of 16 a patch is a sequence of 16-byte pieces (tap, 16 channels), each
+// contiguous in a staged row at a 16-byte aligned address (the host pads `lead` and `pitch` to
+// multiples of 16): lane (pixel r, half h) reads piece 2 ks + h of its pixel's patch with one
+// 16-byte LDS read per k step; a piece past the depth (an odd number of pieces) is 0x80 bytes,
+// zero after the shift, on both sides.  Where the gathering GEMM kernels need 64 channels per
+// filter tap, such layers went through the one-launch kernel (3 x 3, 112 x 112 x 32 -> 64 at batch
+// 64: 78 us).
+template <int FX, int KS>
+__global__ __launch_bounds__(256, 2) void q8_conv_rows_kernel(ConvShortParams p, RequantTable) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  int32_t *s_cx = (int32_t *)lds;                                 // [32 FX]
+  int32_t *s_tab = s_cx + 32 * FX;                                // the comparison table's pairs
+  uint8_t *rows = lds + ((128 * FX + MH_REQUANT_PAIRS_BYTES + 15) & ~15);   // staged input rows
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int h = lane >> 5, r32 = lane & 31;
+  const int img = blockIdx.x / p.strips, strip_i = blockIdx.x - img * p.strips;
+  const int oh0 = strip_i * p.strip;
+  const int nrows = min(p.strip, p.out_h - oh0);
+  const int npix = nrows * p.out_w;
+  const int staged = (nrows - 1) * p.sh + p.k_h;
+  const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+
+  // staging of the strip's input rows: as in q8_conv_short_kernel (all loads of a turn requested
+  // before the first store, none under a condition, no division per dword)
+  constexpr int BATCH = 12;
+  const int row_len = p.in_w * p.cin;
+  const int dpr = p.pitch >> 2;
+  const int ih_first = oh0 * p.sh - p.pt;
+  const int stage_total = staged * dpr;
+  const uint8_t *image = p.in + (int64_t)img * p.in_h * row_len;
+  uint32_t sv[BATCH];
+  int sdst[BATCH];
+  bool sinside[BATCH];
+  const int sr_step = 256 / dpr, dw_step = 256 - sr_step * dpr;
+  int sr = tid / dpr, dw = tid - sr * dpr;
+  auto stage_issue = [&](int base) {
+#pragma unroll
+    for (int u = 0; u < BATCH; ++u) {
+      const int ih = ih_first + sr;
+      const int o = dw * 4 - p.lead;   // byte offset inside the input row (rows are whole dwords here)
+      sinside[u] = (unsigned)ih < (unsigned)p.in_h && o >= 0 && o < row_len;
+      const int oc = min(max(o, 0), row_len - 4);
+      sdst[u] = base + u * 256 < stage_total ? sr * p.pitch + dw * 4 : -1;
+      __builtin_memcpy(&sv[u], image + (int64_t)min(max(ih, 0), p.in_h - 1) * row_len + oc, 4);
+      sr += sr_step;
+      dw += dw_step;
+      if (dw >= dpr) { dw -= dpr; ++sr; }
+    }
+  };
+  auto stage_commit = [&]() {
+#pragma unroll
+    for (int u = 0; u < BATCH; ++u)
+      if (sdst[u] >= 0) *(uint32_t *)(rows + sdst[u]) = sinside[u] ? sv[u] : p.zp4;
+  };
+  stage_issue(tid);
+
+  // the filter: fragment (i, ks) holds bytes 32 ks + 16 h .. + 15 of output channels 32 i .. 32 i + 31
+  // (rows past cout repeat the last; a piece past the depth is 0x80 bytes)
+  const int npieces = p.depth >> 4;
+  v4i xf[FX][KS];
+#pragma unroll
+  for (int i = 0; i < FX; ++i) {
+    const int ci = i * 32 + r32;
+    const int c = min(ci, p.cout - 1);
+    const uint8_t *row = p.filter + (int64_t)c * p.depth;
+    uint32_t xs = 0;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int piece = min(2 * ks + h, npieces - 1);   // (clamped: no load under a condition)
+      uint32_t w[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) __builtin_memcpy(&w[j], row + 16 * piece + 4 * j, 4);
+      if (2 * ks + h >= npieces) w[0] = w[1] = w[2] = w[3] = 0x80808080u;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) xs = __builtin_amdgcn_sad_u8(w[j], 0u, xs);
+      xf[i][ks] = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]} ^ flip;
+    }
+    int sum = (int)xs - 128 * 16 * KS;   // of the shifted bytes
+    sum += __shfl_xor(sum, 32, 64);
+    if (wave == 0 && h == 0) {
+      uint32_t cx = (uint32_t)p.xcoef * (uint32_t)sum;
+      if (p.bias) cx += (uint32_t)p.bias[c];
+      s_cx[ci] = (int32_t)cx;
+    }
+  }
+  stage_requant_pairs_from((const int32_t *)((const char *)__builtin_amdgcn_kernarg_segment_ptr() +
+                                             sizeof(ConvShortParams)),
+                           s_tab, p.rq, tid, 256);
+  stage_commit();
+  for (int base = tid + 256 * BATCH; base < stage_total; base += 256 * BATCH) {
+    stage_issue(base);
+    stage_commit();
+  }
+  // where piece 2 ks + h of a patch lies relative to the patch's first byte
+  int koff[KS];
+  {
+    const int cpt = p.cin >> 4;          // pieces per tap
+    const int k_w = p.run / p.cin;       // (uniform: scalar divisions)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int piece = min(2 * ks + h, npieces - 1);
+      const int tap = piece / cpt, c16 = piece - tap * cpt;
+      const int kh = tap / k_w, kw = tap - kh * k_w;
+      koff[ks] = kh * p.pitch + kw * p.cin + 16 * c16;
+    }
+  }
+  const RequantLds rql = requant_lds(p.rq, s_tab);
+  __syncthreads();
+
+  const int nblk = (npix + 31) >> 5;
+  int q = wave * 32 + r32;   // this lane's pixel within the strip
+  int ohl = q / p.out_w, ow = q - ohl * p.out_w;
+  const int dq = 128 / p.out_w, dr = 128 - dq * p.out_w;   // four blocks on
+  uint8_t *out0 = p.out + (((int64_t)img * p.out_h + oh0) * p.out_w) * p.cout + 16 * h;
+  const int step_h = p.sh * p.pitch, step_w = p.sw * p.cin;
+  int at = p.gbase + ohl * step_h + ow * step_w;
+  const int at_step = dq * step_h + dr * step_w, at_wrap = step_h - p.out_w * step_w;
+  const int at_last = p.gbase + (nrows - 1) * step_h + (p.out_w - 1) * step_w;
+  const bool odd = (npieces & 1) != 0;   // the last k step's upper half does not exist
+  for (int blk = wave; blk < nblk; blk += 4) {
+    // pixels past the strip's end read its last pixel's patch and store nothing
+    const bool live = q < npix;
+    const uint8_t *src = rows + (live ? at : at_last);
+    v16i acc[FX];
+#pragma unroll
+    for (int i = 0; i < FX; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][r] = 0;
+    uint32_t ysr = 0;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      v4i w = *(const v4i *)(src + koff[ks]);
+      if (ks == KS - 1 && odd && h == 1) w = flip;   // (0x80 bytes)
+      ysr = __builtin_amdgcn_sad_u8((uint32_t)w.x, 0u, ysr);
+      ysr = __builtin_amdgcn_sad_u8((uint32_t)w.y, 0u, ysr);
+      ysr = __builtin_amdgcn_sad_u8((uint32_t)w.z, 0u, ysr);
+      ysr = __builtin_amdgcn_sad_u8((uint32_t)w.w, 0u, ysr);
+      const v4i yf = w ^ flip;
+#pragma unroll
+      for (int i = 0; i < FX; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xf[i][ks], yf, acc[i], 0, 0, 0);
+    }
+    int ys = (int)ysr - 128 * 16 * KS;
+    ys += __shfl_xor(ys, 32, 64);
+    // (both factors fit in 24 bits: a zero point and the sum of at most 32 KS bytes)
+    const uint32_t cy = (uint32_t)__mul24(p.ycoef, ys) + (uint32_t)p.yadd;
+    uint8_t *orow = out0 + (int64_t)q * p.cout;
+#pragma unroll
+    for (int i = 0; i < FX; ++i) {
+      // register r: channel 8 (r / 4) + 4 h + r % 4 of this block of 32, pixel lane % 32
+      const int xb = i * 32 + 4 * h;
+      int32_t v[16];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const v4i cx = *(const v4i *)(s_cx + xb + 8 * g);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[g * 4 + e] = (int32_t)((uint32_t)acc[i][g * 4 + e] + (uint32_t)cx[e] + cy);
+      }
+      uint32_t packed[4];
+      requant_16_by_table(v, rql, packed);
+      const v2u s02 = __builtin_amdgcn_permlane32_swap(packed[0], packed[2], false, false);
+      const v2u s13 = __builtin_amdgcn_permlane32_swap(packed[1], packed[3], false, false);
+      const v4i o = {(int)s02.x, (int)s02.y, (int)s13.x, (int)s13.y};
+      if (live && i * 32 + 16 * h < p.cout) *(v4i *)(orow + i * 32) = o;
+    }
+    q += 128;
+    ow += dr;
+    at += at_step;
+    if (ow >= p.out_w) { ow -= p.out_w; at += at_wrap; }
+  }
+}
+
 // floor(a / b) for b > 0
 inline int64_t floor_div(int64_t a, int64_t b) { return a >= 0 ? a / b : -((-a + b - 1) / b); }
 
@@ -412,6 +589,88 @@ int conv_short(mace_hip_ctx *ctx, const uint8_t *input, const uint8_t *filter, c
   return MACE_HIP_SUCCESS;
 }
 
+// The strip kernel for 16-channel pieces: patches of 9 - 10 or 17 - 18 pieces (3 x 3 on 16 or 32
+// channels and their like).  *taken = false: the call is not one for it (nothing has been launched).
+int conv_rows(mace_hip_ctx *ctx, const uint8_t *input, const uint8_t *filter, const int32_t *bias,
+              int64_t n, int64_t in_h, int64_t in_w, int64_t cin, int64_t cout, int64_t k_h,
+              int64_t k_w, int stride_h, int stride_w, int pad_top, int pad_left, int64_t out_h,
+              int64_t out_w, float input_scale, int32_t input_zp, float filter_scale,
+              int32_t filter_zp, float bias_scale, int32_t mult, int shift, int32_t out_zp,
+              int clamp_min, int clamp_max, uint8_t *out, bool *taken) {
+  *taken = false;
+  const int64_t depth = k_h * k_w * cin, columns = n * out_h * out_w;
+  const int64_t ks = (depth / 16 + 1) / 2;
+  // (17 - 18 pieces against more than 64 output channels would hold 36 filter fragments and 64
+  // accumulators per lane, one workgroup per CU: measured no faster than the one-launch kernel on
+  // 56 x 56 x 32 -> 128 at batch 64, 42.2 against 41.2 us, and 34 % slower on 28 x 28; not built)
+  if (cin % 16 != 0 || depth <= 32 || (ks != 5 && ks != 9) || cout % 16 != 0 || cout > 128 ||
+      (ks == 9 && cout > 64) ||
+      (uintptr_t)out % 16 != 0 || columns < 1024 || (ctx->kernel_mask & MH_MASK_NO_CONV_SHORT))
+    return MACE_HIP_SUCCESS;
+  if (shift < 0 || shift > 31 || clamp_min < 0 || clamp_max > 255 || clamp_min > clamp_max)
+    return MACE_HIP_SUCCESS;   // (the general path reports these)
+  RequantFixed rq;
+  if (!mh_make_requant(mult, shift, out_zp, clamp_min, clamp_max, &rq) || !rq.table)
+    return MACE_HIP_SUCCESS;
+  // staged rows: pixel positions -pad_left ... up to the last one any patch or the image reaches
+  // (cin is a multiple of 16, so every position starts a 16-byte piece)
+  const int64_t reach = std::max<int64_t>(in_w + pad_left, (out_w - 1) * stride_w + k_w);
+  const int lead = (int)(pad_left * cin);
+  const int64_t pitch = reach * cin;
+  const int fx = cout <= 32 ? 1 : (cout <= 64 ? 2 : 4);
+  const int64_t fixed = (128 * fx + MH_REQUANT_PAIRS_BYTES + 15) & ~(int64_t)15;
+  auto lds_of = [&](int64_t r) { return fixed + ((r - 1) * stride_h + k_h) * pitch; };
+  if (lds_of(1) > 64 * 1024 || n * in_h >= (1ll << 31) || in_w * cin >= (1ll << 30) || pitch >= (1 << 24))
+    return MACE_HIP_SUCCESS;
+  // rows per strip: as for the short-patch kernel
+  const int64_t cu = ctx->cu_count > 0 ? ctx->cu_count : 256;
+  const int64_t target = std::min<int64_t>(1024, std::max<int64_t>(128, columns / (2 * cu)));
+  int64_t r_hi = std::min<int64_t>(out_h, std::max<int64_t>(1, (target + out_w / 2) / out_w));
+  while (r_hi > 1 && lds_of(r_hi) > 64 * 1024) --r_hi;
+  int64_t strip = r_hi, best = -1;
+  for (int64_t r = r_hi; r >= std::max<int64_t>(1, r_hi / 2); --r) {
+    const int64_t strips = (out_h + r - 1) / r, last = out_h - (strips - 1) * r;
+    const int64_t blocks = (strips - 1) * ((r * out_w + 31) / 32) + (last * out_w + 31) / 32;
+    if (best < 0 || blocks < best) { best = blocks; strip = r; }
+  }
+  const int64_t strips = (out_h + strip - 1) / strip;
+  if (n * strips >= (1ll << 31)) return MACE_HIP_SUCCESS;
+  *taken = true;
+
+  MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, sizeof(int32_t) * cout + 4096));
+  ArenaScope scope(ctx);
+  const int32_t *bias_used = nullptr;
+  MH_RETURN_IF_ERROR(conv_bias(ctx, bias, cout, input_scale, filter_scale, bias_scale, &bias_used));
+  RequantTable tab;
+  mh_requant_table_cached(ctx, rq, tab.t);
+  const uint32_t zl = (uint32_t)filter_zp - 128u, zr = (uint32_t)input_zp - 128u;
+  ConvShortParams p{};
+  p.in = input; p.filter = filter; p.bias = bias_used; p.out = out;
+  p.in_h = (int)in_h; p.in_w = (int)in_w; p.cin = (int)cin; p.cout = (int)cout; p.k_h = (int)k_h;
+  p.sh = stride_h; p.sw = stride_w; p.pt = pad_top; p.out_h = (int)out_h; p.out_w = (int)out_w;
+  p.depth = (int)depth; p.run = (int)(k_w * cin); p.strip = (int)strip; p.strips = (int)strips;
+  p.pitch = (int)pitch; p.lead = lead; p.gbase = 0;
+  p.zp4 = (uint32_t)(input_zp & 0xff) * 0x01010101u;
+  p.xcoef = (int32_t)(0u - zr);
+  p.ycoef = (int32_t)(0u - zl);
+  p.yadd = (int32_t)((uint32_t)depth * zl * zr);
+  p.rq = rq;
+  const size_t lds = (size_t)lds_of(strip);
+  dim3 grid((unsigned)(n * strips)), block(256);
+  mh_plan_main(ctx, MACE_HIP_KF_Q8_CONV_ROWS, mhv::conv_rows(fx, (int)ks), grid, block, (int)lds);
+  MH_PROF_BEGIN(ctx);
+#define MH_ROWS(FX_, KS_) MH_KLAUNCH(ctx, (q8_conv_rows_kernel<FX_, KS_>), grid, block, lds, ctx->stream, p, tab)
+  if (ks == 5) {
+    if (fx == 1) MH_ROWS(1, 5); else if (fx == 2) MH_ROWS(2, 5); else MH_ROWS(4, 5);
+  } else {
+    if (fx == 1) MH_ROWS(1, 9); else MH_ROWS(2, 9);
+  }
+#undef MH_ROWS
+  MH_PROF_END(ctx);
+  MH_LAUNCH_CHECK(ctx);
+  return MACE_HIP_SUCCESS;
+}
+
 // scratch the GEMM takes from the arena for a [cout x depth] . [depth x columns] product
 inline size_t conv_gemm_scratch(int64_t cout, int64_t depth, int64_t columns, bool rhs_in_place) {
   const size_t kp = mh_align_up((size_t)(depth > 0 ? depth : 1), 64);
@@ -463,6 +722,11 @@ extern "C" int mace_hip_conv2d_q8_nhwc(mace_hip_ctx *ctx, const uint8_t *input,
                                   stride_h, stride_w, pad_h >> 1, pad_w >> 1, out_h, out_w,
                                   input_scale, input_zp, filter_scale, filter_zp, bias_scale, mult,
                                   shift, out_zp, clamp_min, clamp_max, out, &taken));
+    if (taken) return MACE_HIP_SUCCESS;
+    MH_RETURN_IF_ERROR(conv_rows(ctx, input, filter, bias, n, in_h, in_w, cin, cout, k_h, k_w,
+                                 stride_h, stride_w, pad_h >> 1, pad_w >> 1, out_h, out_w,
+                                 input_scale, input_zp, filter_scale, filter_zp, bias_scale, mult,
+                                 shift, out_zp, clamp_min, clamp_max, out, &taken));
     if (taken) return MACE_HIP_SUCCESS;
   }
   // With cin a multiple of 64 (and at least three 64-byte slabs of depth) the GEMM's loader

@@ -173,6 +173,47 @@ def test_conv2d_q8_short_patches(ctx, n, cout, cin, in_h, in_w, k_h, k_w, pad, s
     assert len(np.unique(want)) > 8
 
 
+ROWS_CASES = [  # batch, cout, cin, in_h, in_w, k_h, k_w, padding, strides, FX, KS
+    (8, 64, 32, 56, 56, 3, 3, S, (1, 1), 2, 9),      # SqueezeNet-like expand 3 x 3 on 32 channels
+    (2, 16, 16, 57, 59, 3, 3, S, (2, 2), 1, 5),      # nine pieces: the last k step's upper half is absent
+    (1, 128, 16, 40, 300, 3, 3, V, (1, 1), 4, 5),    # wide rows, one image
+    (3, 48, 32, 33, 31, 3, 3, Fu, (1, 1), 2, 9),     # ragged channel count, padding of 2 on every side
+    (12, 32, 32, 30, 30, 3, 3, S, (3, 3), 1, 9),
+    (4, 48, 16, 41, 41, 2, 5, S, (1, 2), 2, 5),      # ten pieces
+    (3, 64, 16, 20, 64, 5, 2, V, (2, 1), 2, 5),
+    (64, 32, 32, 14, 14, 3, 3, S, (1, 1), 1, 9),     # a strip is a whole (small) image
+    (1, 64, 96, 64, 64, 1, 3, S, (1, 1), 2, 9),      # 1 x 3 on 96 channels: 18 pieces, 6 per tap
+]
+
+
+@pytest.mark.parametrize("n,cout,cin,in_h,in_w,k_h,k_w,pad,st,fx,ks", ROWS_CASES)
+def test_conv2d_q8_pieces_of_16_channels(ctx, n, cout, cin, in_h, in_w, k_h, k_w, pad, st, fx, ks):
+    """Patches of 9 - 10 or 17 - 18 pieces of 16 channels (3 x 3 on 16 or 32 channels and their like):
+    the strip kernel with several k steps.  Against the oracle bit for bit, the kernel that ran
+    asserted, three bias / clamp settings each (zero points near the middle of the range, so that
+    the outputs do not all saturate; the random sweep below draws them from all of it)."""
+    rng = np.random.default_rng(cout * 13 + cin + k_h * 5 + k_w + in_w)
+    x = rng.integers(0, 256, (n, in_h, in_w, cin), dtype=np.uint8)
+    f = rng.integers(0, 256, (cout, k_h, k_w, cin), dtype=np.uint8)
+    bias = rng.integers(-2 ** 15, 2 ** 15, cout).astype(np.int32)
+    z_in, z_f = int(rng.integers(110, 147)), int(rng.integers(110, 147))
+    s_in, s_f = np.float32(0.02), np.float32(0.01)
+    depth = k_h * k_w * cin
+    s_out = np.float32(max(6.0, 3 * 74.0 * 74.0 * np.sqrt(depth) * float(s_in * s_f)) / 255.0)
+    oh, ow, ph, pw = orc.calc_padding_and_output_size(in_h, in_w, k_h, k_w, st, pad)
+    for (bb, s_b, z_o, lo, hi) in ((bias, np.float32(s_in * s_f), 0, 0, 255),
+                                   (bias, np.float32(2.5 * float(s_in * s_f)), 100, 100, 230),
+                                   (None, np.float32(0), 128, 0, 255)):
+        want = orc.conv2d_q8_nhwc(x, f, bb, n, in_h, in_w, cin, cout, k_h, k_w, st, (ph, pw), s_in,
+                                  z_in, s_f, z_f, s_b, s_out, z_o, lo, hi, nthreads=16)
+        got = conv_host(ctx, x, f, bb, n, in_h, in_w, cin, cout, k_h, k_w, st, (ph, pw), s_in,
+                        z_in, s_f, z_f, s_b, s_out, z_o, lo, hi)
+        assert ctx.last_plan().kernel == "q8_conv_rows_kernel<FX=%d,KS=%d>" % (fx, ks), ctx.last_plan()
+        assert got.shape == (n, oh, ow, cout)
+        np.testing.assert_array_equal(got, want)
+    assert len(np.unique(want)) > 8
+
+
 def test_conv2d_q8_filter_in_lds_many_blocks(ctx):
     """More 64-pixel blocks than the kernel that keeps the filter in LDS has wavefronts: each
     wavefront walks over several blocks, prefetching the next block's first filter tap."""

@@ -330,6 +330,13 @@ def test_convolution_gather_and_im2col(ctx):
     assert conv(ctx, 64, 224, 3, 64, k=3, stride=2, pad=1).kernel == "q8_conv_short_kernel<FX=2>"
     assert conv(ctx, 64, 224, 3, 128, k=3, stride=2, pad=1).kernel == "q8_conv_short_kernel<FX=4>"
     assert conv(ctx, 8, 64, 2, 32, k=4, stride=1, pad=3).family == mh.KF_Q8_CONV_SHORT       # depth 32
+    # patches of several taps of 16-channel pieces (3 x 3 on 16 or 32 channels): the strip kernel's sibling
+    p = conv(ctx, 64, 112, 32, 64, k=3, stride=1, pad=2)
+    assert p.kernel == "q8_conv_rows_kernel<FX=2,KS=9>" and p.launches == 1 and p.lds_bytes <= 64 * 1024, p
+    assert conv(ctx, 8, 56, 16, 128, k=3, stride=2, pad=2).kernel == "q8_conv_rows_kernel<FX=4,KS=5>"
+    assert conv(ctx, 8, 56, 48, 64, k=3, stride=1, pad=2).family != mh.KF_Q8_CONV_ROWS      # 27 pieces
+    assert conv(ctx, 8, 56, 32, 128, k=3, stride=1, pad=2).family != mh.KF_Q8_CONV_ROWS     # 18 pieces, > 64 output channels
+    assert conv(ctx, 64, 112, 32, 64, k=3, stride=1, pad=2, mask=mh.MASK_NO_CONV_SHORT).family != mh.KF_Q8_CONV_ROWS
     # not for it: 33 bytes of patch, channel counts that are not whole 16-byte pieces of the output
     # row or more than 128, fewer than 1024 pixels; those stay with the one-launch kernel
     small = mh.KF_Q8_GEMM_FUSED_SMALL
@@ -383,7 +390,7 @@ def test_variant_tables_are_consistent():
         total += len(vs)
         assert not lib.mace_hip_plan_variant_valid(f, n) and not lib.mace_hip_plan_variant_valid(f, -1)
         assert mh.coverage(f, 0) == 0              # nothing is launched by planning
-    assert total == 221
+    assert total == 226
     assert lib.mace_hip_plan_variant_count(0) == 0 and lib.mace_hip_plan_variant_count(mh.KF_COUNT) == 0
 
 
