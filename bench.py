@@ -517,6 +517,19 @@ def bench_other(ctx, mh, torch):
                     "kernel_ms": round(k, 4), "TOPS": round(ops / (t * 1e-3) / 1e12, 1),
                     "frac_of_int8_peak": round(ops / (t * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4)})
 
+    # a handful of 128 x 128 tiles with a long depth (MACE's RowMajor operands): the eight-wavefront
+    # kernel's lower range
+    for (m, kk, n) in ((256, 2048, 3072), (512, 1024, 1024)):
+        A, B = u8(m, kk), u8(kk, n)
+        C = torch.empty((m, n), dtype=torch.uint8, device="cuda")
+        e = mh.quantize_multiplier(min(0.9, 40.0 / (74.0 * 74.0 * kk ** 0.5)))
+        torch.cuda.synchronize()
+        whole, k = time_kernel(ctx, bind(ctx,
+            "mace_hip_gemm_q8_u8", A.data_ptr(), 0, B.data_ptr(), 0, C.data_ptr(), 0, 1, m, kk, n, 1,
+            1, -131, -122, None, e[0], -e[1], 128, 0, 255))
+        out.append({"workload": "q8_matmul_%dx%dx%d" % (m, kk, n), "call_ms": round(whole, 4),
+                    "kernel": ctx.last_plan().kernel, "launches": ctx.last_plan().launches})
+
     # config 5 with the raw int32 result (MatMulFixpointImpl<..., int32_t>): 4096^3, 256 MiB less
     # to hold than 8192^3 and the same kernel
     n = 4096
@@ -576,7 +589,8 @@ def bench_other(ctx, mh, torch):
     # (batch 64, and single-image inference: one launch that gathers as it goes; 224 x 224 x 3 at
     # stride 2 is MobileNet's first layer: patches of 27 bytes, the strip kernel)
     for (n, hw, cin, cout, k, st) in ((64, 56, 64, 64, 3, 1), (64, 28, 128, 128, 3, 1),
-                                      (64, 224, 3, 32, 3, 2), (1, 224, 3, 32, 3, 2), (1, 56, 64, 64, 3, 1), (1, 28, 128, 128, 3, 1)):
+                                      (64, 224, 3, 32, 3, 2), (1, 224, 3, 32, 3, 2), (1, 56, 64, 64, 3, 1), (1, 28, 128, 128, 3, 1),
+                                      (64, 112, 32, 32, 3, 1)):   # 18 pieces of 16 channels: q8_conv_rows_kernel
         oh = (hw + st - 1) // st
         pad = max((oh - 1) * st + k - hw, 0)      # SAME
         x, f = u8(n, hw, hw, cin), u8(cout, k, k, cin)
@@ -624,6 +638,22 @@ def bench_other(ctx, mh, torch):
             out.append({"workload": "f32_gemm_4x1024^3_ta%d_tb%d" % (ta, tb), "kernel_ms": round(k, 4),
                         "TFLOPS": round(tf, 1), "frac_of_fp32_mfma_peak": round(tf / 157.3, 4),
                         "sample_rel_err_vs_f64": float("%.3g" % rel)})
+    # fp32 GEMMs with few tiles: the depth is dealt to several workgroups per tile (two launches)
+    for (m, kk, n) in ((512, 512, 512), (1024, 1024, 49)):
+        Af = torch.randn((m, kk), dtype=torch.float32, device="cuda", generator=g)
+        Bf = torch.randn((kk, n), dtype=torch.float32, device="cuda", generator=g)
+        Cf = torch.empty((m, n), dtype=torch.float32, device="cuda")
+        torch.cuda.synchronize()
+        whole, k = time_kernel(ctx, bind(ctx, "mace_hip_gemm_f32", Af.data_ptr(), Bf.data_ptr(), 1, m, n, kk,
+                                         0, 0, 0, 1, 1, Cf.data_ptr()))
+        ref = Af.double() @ Bf.double()
+        rel = float(((Cf.double() - ref).norm() / ref.norm()).item())
+        if not rel <= 1e-4:
+            log("ERROR: fp32 Gemm (k split) result off by %.3g (normwise) from the binary64 product" % rel)
+            sys.exit(3)
+        out.append({"workload": "f32_gemm_%dx%dx%d" % (m, kk, n), "call_ms": round(whole, 4),
+                    "TFLOPS": round(2.0 * m * kk * n / (whole * 1e-3) / 1e12, 1),
+                    "launches": ctx.last_plan().launches, "sample_rel_err_vs_f64": float("%.3g" % rel)})
     # fp32 Gemv (FullyConnected) 4096 x 4096, batch 1: weights rotated over a set larger than the
     # last-level cache; and the fp32 1x1 convolution (NCHW, bias + ReLU6 fused into the store) on
     # two of the MobileNet shapes at batch 64
