@@ -174,25 +174,36 @@ __global__ __launch_bounds__(256, 3) void q8_conv_short_kernel(ConvShortParams p
 
   // the filter: fragment i holds output channels 32 i .. 32 i + 31 (rows past cout repeat the last)
   v4i xf[FX];
+  // a lane's bytes 16 h .. 16 h + 15 of its row as four dwords, no load under a condition (a load
+  // per byte, each waiting in a branch of its own, put sixteen memory round trips in front of every
+  // workgroup) and all of them, with the bias's, requested before the first is used: a dword that
+  // straddles the row's end is taken from the dword that ends there (the depth is at least 4), one
+  // past the end is 0x80 bytes, zero after the shift
+  uint32_t got[FX][4];
+  int32_t bias_v[FX];
 #pragma unroll
   for (int i = 0; i < FX; ++i) {
-    const int ci = i * 32 + r32;
-    const int c = min(ci, p.cout - 1);
-    // the row's bytes 16 h .. 16 h + 15 as four dwords, no load under a condition (a load per byte,
-    // each waiting in a branch of its own, put sixteen memory round trips in front of every
-    // workgroup): a dword that straddles the row's end is taken from the dword that ends there
-    // (the depth is at least 4), one past the end is 0x80 bytes, zero after the shift
+    const int c = min(i * 32 + r32, p.cout - 1);
     const uint8_t *row = p.filter + (int64_t)c * p.depth;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) __builtin_memcpy(&got[i][j], row + min(16 * h + 4 * j, p.depth - 4), 4);
+    bias_v[i] = 0;
+    if (p.bias) bias_v[i] = p.bias[c];
+  }
+  // (the comparison table's load travels with them)
+  stage_requant_pairs_from((const int32_t *)((const char *)__builtin_amdgcn_kernarg_segment_ptr() +
+                                             sizeof(ConvShortParams)),
+                           s_tab, p.rq, tid, 256);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int i = 0; i < FX; ++i) {
     uint32_t w[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int o = 16 * h + 4 * j;
-      const int oc = min(o, p.depth - 4);
-      uint32_t got;
-      __builtin_memcpy(&got, row + oc, 4);
-      const int shift = 8 * (o - oc);
+      const int shift = 8 * (o - min(o, p.depth - 4));
       w[j] = o >= p.depth ? 0x80808080u
-                          : (shift ? ((got >> shift) | (0x80808080u << (32 - shift))) : got);
+                          : (shift ? ((got[i][j] >> shift) | (0x80808080u << (32 - shift))) : got[i][j]);
     }
     uint32_t xs = 0;
 #pragma unroll
@@ -200,15 +211,8 @@ __global__ __launch_bounds__(256, 3) void q8_conv_short_kernel(ConvShortParams p
     int sum = (int)xs - 128 * 16;   // of the shifted bytes
     sum += __shfl_xor(sum, 32, 64);
     xf[i] = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]} ^ flip;
-    if (wave == 0 && h == 0) {
-      uint32_t cx = (uint32_t)p.xcoef * (uint32_t)sum;
-      if (p.bias) cx += (uint32_t)p.bias[c];
-      s_cx[ci] = (int32_t)cx;
-    }
+    if (wave == 0 && h == 0) s_cx[i * 32 + r32] = (int32_t)((uint32_t)p.xcoef * (uint32_t)sum + (uint32_t)bias_v[i]);
   }
-  stage_requant_pairs_from((const int32_t *)((const char *)__builtin_amdgcn_kernarg_segment_ptr() +
-                                             sizeof(ConvShortParams)),
-                           s_tab, p.rq, tid, 256);
   // the rest of the strip's input rows (a strip of MobileNet's first layer is done with the
   // first turn)
   stage_commit();
@@ -304,8 +308,9 @@ __global__ __launch_bounds__(256, 3) void q8_conv_short_kernel(ConvShortParams p
 // channel count a multiple of 16 a patch is a sequence of 16-byte pieces (tap, 16 channels), each
 // contiguous in a staged row at a 16-byte aligned address (the host pads `lead` and `pitch` to
 // multiples of 16): lane (pixel r, half h) reads piece 2 ks + h of its pixel's patch with one
-// 16-byte LDS read per k step; a piece past the depth (an odd number of pieces) is 0x80 bytes,
-// zero after the shift, on both sides.  Where the gathering GEMM kernels need 64 channels per
+// 16-byte LDS read per k step; a piece past the depth (an odd number of pieces) is zero after the
+// shift on both sides.  The rows are staged already shifted (x ^ 0x80), 16 bytes per load, so a
+// block's k steps are LDS read, four v_dot4c for the patch sum, MFMA.  Where the gathering GEMM kernels need 64 channels per
 // filter tap, such layers went through the one-launch kernel (3 x 3, 112 x 112 x 32 -> 64 at batch
 // 64: 78 us).
 template <int FX, int KS>
@@ -324,89 +329,120 @@ __global__ __launch_bounds__(256, 2) void q8_conv_rows_kernel(ConvShortParams p,
   const int staged = (nrows - 1) * p.sh + p.k_h;
   const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
 
-  // staging of the strip's input rows: as in q8_conv_short_kernel (all loads of a turn requested
-  // before the first store, none under a condition, no division per dword)
-  constexpr int BATCH = 12;
+  // Staging of the strip's input rows, as in q8_conv_short_kernel (all loads of a turn requested
+  // before the first store, none under a per-lane condition, no division per unit) but 16 bytes at
+  // a time: rows, the left padding and the pitch are whole 16-byte pieces here, so a piece lies
+  // inside the image or is padding as a whole.  The bytes are stored shifted (x ^ 0x80), as the
+  // MFMA takes them.  A turn covers 256 BATCH pieces (40 KiB: most strips); its upper half is
+  // skipped, by a branch the whole workgroup takes alike, where the strip ends before.
+  constexpr int BATCH = 10, HALF = BATCH / 2;
   const int row_len = p.in_w * p.cin;
-  const int dpr = p.pitch >> 2;
+  const int qpr = p.pitch >> 4;
   const int ih_first = oh0 * p.sh - p.pt;
-  const int stage_total = staged * dpr;
+  const int stage_total = staged * qpr;
   const uint8_t *image = p.in + (int64_t)img * p.in_h * row_len;
-  uint32_t sv[BATCH];
+  v4i sv[BATCH];
   int sdst[BATCH];
   bool sinside[BATCH];
-  const int sr_step = 256 / dpr, dw_step = 256 - sr_step * dpr;
-  int sr = tid / dpr, dw = tid - sr * dpr;
-  auto stage_issue = [&](int base) {
+  const int sr_step = 256 / qpr, qu_step = 256 - sr_step * qpr;
+  int sr = tid / qpr, qu = tid - sr * qpr;
+  auto stage_issue_one = [&](int base0, int u) {
+    const int ih = ih_first + sr;
+    const int o = qu * 16 - p.lead;   // byte offset inside the input row
+    sinside[u] = (unsigned)ih < (unsigned)p.in_h && o >= 0 && o < row_len;
+    const int oc = min(max(o, 0), row_len - 16);
+    // (24-bit factors and an image of less than 2 GiB: the host checks)
+    sdst[u] = base0 + tid + u * 256 < stage_total ? __mul24(sr, p.pitch) + qu * 16 : -1;
+    sv[u] = *(const v4i *)(image + ((uint32_t)__mul24(min(max(ih, 0), p.in_h - 1), row_len) + (uint32_t)oc));
+    sr += sr_step;
+    qu += qu_step;
+    if (qu >= qpr) { qu -= qpr; ++sr; }
+  };
+  auto stage_issue = [&](int base0) {   // (base0: the same in every lane)
 #pragma unroll
-    for (int u = 0; u < BATCH; ++u) {
-      const int ih = ih_first + sr;
-      const int o = dw * 4 - p.lead;   // byte offset inside the input row (rows are whole dwords here)
-      sinside[u] = (unsigned)ih < (unsigned)p.in_h && o >= 0 && o < row_len;
-      const int oc = min(max(o, 0), row_len - 4);
-      sdst[u] = base + u * 256 < stage_total ? sr * p.pitch + dw * 4 : -1;
-      __builtin_memcpy(&sv[u], image + (int64_t)min(max(ih, 0), p.in_h - 1) * row_len + oc, 4);
-      sr += sr_step;
-      dw += dw_step;
-      if (dw >= dpr) { dw -= dpr; ++sr; }
+    for (int u = 0; u < HALF; ++u) stage_issue_one(base0, u);
+    if (base0 + HALF * 256 < stage_total) {
+#pragma unroll
+      for (int u = HALF; u < BATCH; ++u) stage_issue_one(base0, u);
+    } else {
+#pragma unroll
+      for (int u = HALF; u < BATCH; ++u) sdst[u] = -1;
     }
   };
+  const int zpf = (int)(p.zp4 ^ 0x80808080u);
   auto stage_commit = [&]() {
 #pragma unroll
     for (int u = 0; u < BATCH; ++u)
-      if (sdst[u] >= 0) *(uint32_t *)(rows + sdst[u]) = sinside[u] ? sv[u] : p.zp4;
+      if (sdst[u] >= 0) *(v4i *)(rows + sdst[u]) = sinside[u] ? (sv[u] ^ flip) : v4i{zpf, zpf, zpf, zpf};
   };
-  stage_issue(tid);
+  stage_issue(0);
 
   // the filter: fragment (i, ks) holds bytes 32 ks + 16 h .. + 15 of output channels 32 i .. 32 i + 31
-  // (rows past cout repeat the last; a piece past the depth is 0x80 bytes)
+  // (rows past cout repeat the last; a piece past the depth is 0x80 bytes).  All of its loads and
+  // the bias's are requested behind the rows', before anything waits.
   const int npieces = p.depth >> 4;
   v4i xf[FX][KS];
+  int32_t bias_v[FX];
 #pragma unroll
   for (int i = 0; i < FX; ++i) {
-    const int ci = i * 32 + r32;
-    const int c = min(ci, p.cout - 1);
-    const uint8_t *row = p.filter + (int64_t)c * p.depth;
-    uint32_t xs = 0;
+    const int c = min(i * 32 + r32, p.cout - 1);
+    const uint8_t *row = p.filter + (uint32_t)__mul24(c, p.depth);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int piece = min(2 * ks + h, npieces - 1);   // (clamped: no load under a condition)
-      uint32_t w[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) __builtin_memcpy(&w[j], row + 16 * piece + 4 * j, 4);
-      if (2 * ks + h >= npieces) w[0] = w[1] = w[2] = w[3] = 0x80808080u;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) xs = __builtin_amdgcn_sad_u8(w[j], 0u, xs);
-      xf[i][ks] = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]} ^ flip;
+      __builtin_memcpy(&xf[i][ks], row + 16 * piece, 16);
     }
-    int sum = (int)xs - 128 * 16 * KS;   // of the shifted bytes
-    sum += __shfl_xor(sum, 32, 64);
-    if (wave == 0 && h == 0) {
-      uint32_t cx = (uint32_t)p.xcoef * (uint32_t)sum;
-      if (p.bias) cx += (uint32_t)p.bias[c];
-      s_cx[ci] = (int32_t)cx;
-    }
+    bias_v[i] = 0;
+    if (p.bias) bias_v[i] = p.bias[c];
   }
+  // (the comparison table's load travels with them)
   stage_requant_pairs_from((const int32_t *)((const char *)__builtin_amdgcn_kernarg_segment_ptr() +
                                              sizeof(ConvShortParams)),
                            s_tab, p.rq, tid, 256);
-  stage_commit();
-  for (int base = tid + 256 * BATCH; base < stage_total; base += 256 * BATCH) {
-    stage_issue(base);
-    stage_commit();
-  }
-  // where piece 2 ks + h of a patch lies relative to the patch's first byte
+  __builtin_amdgcn_sched_barrier(0);
+  // where piece 2 ks + h of a patch lies relative to the patch's first byte: pieces follow one
+  // another along a filter row and step by the pitch from row to row (the same in every lane but
+  // for h: scalar arithmetic, no division)
   int koff[KS];
   {
-    const int cpt = p.cin >> 4;          // pieces per tap
-    const int k_w = p.run / p.cin;       // (uniform: scalar divisions)
+    const int per_row = p.run >> 4;   // pieces per filter row
+    int along = 0, off = 0, row_off = 0;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const int piece = min(2 * ks + h, npieces - 1);
-      const int tap = piece / cpt, c16 = piece - tap * cpt;
-      const int kh = tap / k_w, kw = tap - kh * k_w;
-      koff[ks] = kh * p.pitch + kw * p.cin + 16 * c16;
+      int pair[2];
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        pair[e] = off;
+        if (2 * ks + e + 1 < npieces) {
+          ++along;
+          off += 16;
+          if (along == per_row) { along = 0; row_off += p.pitch; off = row_off; }
+        }
+      }
+      koff[ks] = h ? pair[1] : pair[0];
     }
+  }
+#pragma unroll
+  for (int i = 0; i < FX; ++i) {
+    uint32_t xs = 0;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      v4i w = xf[i][ks];
+      if (2 * ks + h >= npieces) w = flip;
+      xs = __builtin_amdgcn_sad_u8((uint32_t)w.x, 0u, xs);
+      xs = __builtin_amdgcn_sad_u8((uint32_t)w.y, 0u, xs);
+      xs = __builtin_amdgcn_sad_u8((uint32_t)w.z, 0u, xs);
+      xs = __builtin_amdgcn_sad_u8((uint32_t)w.w, 0u, xs);
+      xf[i][ks] = w ^ flip;
+    }
+    int sum = (int)xs - 128 * 16 * KS;   // of the shifted bytes
+    sum += __shfl_xor(sum, 32, 64);
+    if (wave == 0 && h == 0) s_cx[i * 32 + r32] = (int32_t)((uint32_t)p.xcoef * (uint32_t)sum + (uint32_t)bias_v[i]);
+  }
+  stage_commit();
+  for (int base0 = 256 * BATCH; base0 < stage_total; base0 += 256 * BATCH) {
+    stage_issue(base0);
+    stage_commit();
   }
   const RequantLds rql = requant_lds(p.rq, s_tab);
   __syncthreads();
@@ -424,30 +460,39 @@ __global__ __launch_bounds__(256, 2) void q8_conv_rows_kernel(ConvShortParams p,
   for (int blk = wave; blk < nblk; blk += 4) {
     // pixels past the strip's end read its last pixel's patch and store nothing
     const bool live = q < npix;
-    const uint8_t *src = rows + (live ? at : at_last);
     v16i acc[FX];
 #pragma unroll
     for (int i = 0; i < FX; ++i)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][r] = 0;
-    uint32_t ysr = 0;
+    // all of the patch's pieces are requested before the first is used
+    v4i ya[KS];
+    {
+      const uint8_t *src = rows + (live ? at : at_last);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) ya[ks] = *(const v4i *)(src + koff[ks]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    int ys = 0;   // the sum of the patch's shifted bytes
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      v4i w = *(const v4i *)(src + koff[ks]);
-      if (ks == KS - 1 && odd && h == 1) w = flip;   // (0x80 bytes)
-      ysr = __builtin_amdgcn_sad_u8((uint32_t)w.x, 0u, ysr);
-      ysr = __builtin_amdgcn_sad_u8((uint32_t)w.y, 0u, ysr);
-      ysr = __builtin_amdgcn_sad_u8((uint32_t)w.z, 0u, ysr);
-      ysr = __builtin_amdgcn_sad_u8((uint32_t)w.w, 0u, ysr);
-      const v4i yf = w ^ flip;
+      v4i yf = ya[ks];
+      if (ks == KS - 1 && odd && h == 1) yf = v4i{0, 0, 0, 0};
+      ys = __builtin_amdgcn_sdot4(yf.x, 0x01010101, ys, false);
+      ys = __builtin_amdgcn_sdot4(yf.y, 0x01010101, ys, false);
+      ys = __builtin_amdgcn_sdot4(yf.z, 0x01010101, ys, false);
+      ys = __builtin_amdgcn_sdot4(yf.w, 0x01010101, ys, false);
 #pragma unroll
       for (int i = 0; i < FX; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xf[i][ks], yf, acc[i], 0, 0, 0);
     }
-    int ys = (int)ysr - 128 * 16 * KS;
+    uint8_t *orow = out0 + (int64_t)q * p.cout;
+    q += 128;
+    ow += dr;
+    at += at_step;
+    if (ow >= p.out_w) { ow -= p.out_w; at += at_wrap; }
     ys += __shfl_xor(ys, 32, 64);
     // (both factors fit in 24 bits: a zero point and the sum of at most 32 KS bytes)
     const uint32_t cy = (uint32_t)__mul24(p.ycoef, ys) + (uint32_t)p.yadd;
-    uint8_t *orow = out0 + (int64_t)q * p.cout;
 #pragma unroll
     for (int i = 0; i < FX; ++i) {
       // register r: channel 8 (r / 4) + 4 h + r % 4 of this block of 32, pixel lane % 32
@@ -466,10 +511,6 @@ __global__ __launch_bounds__(256, 2) void q8_conv_rows_kernel(ConvShortParams p,
       const v4i o = {(int)s02.x, (int)s02.y, (int)s13.x, (int)s13.y};
       if (live && i * 32 + 16 * h < p.cout) *(v4i *)(orow + i * 32) = o;
     }
-    q += 128;
-    ow += dr;
-    at += at_step;
-    if (ow >= p.out_w) { ow -= p.out_w; at += at_wrap; }
   }
 }
 
@@ -605,7 +646,8 @@ int conv_rows(mace_hip_ctx *ctx, const uint8_t *input, const uint8_t *filter, co
   // 56 x 56 x 32 -> 128 at batch 64, 42.2 against 41.2 us, and 34 % slower on 28 x 28; not built)
   if (cin % 16 != 0 || depth <= 32 || (ks != 5 && ks != 9) || cout % 16 != 0 || cout > 128 ||
       (ks == 9 && cout > 64) ||
-      (uintptr_t)out % 16 != 0 || columns < 1024 || (ctx->kernel_mask & MH_MASK_NO_CONV_SHORT))
+      (uintptr_t)out % 16 != 0 || (uintptr_t)input % 16 != 0 || columns < 1024 ||
+      (ctx->kernel_mask & MH_MASK_NO_CONV_SHORT))
     return MACE_HIP_SUCCESS;
   if (shift < 0 || shift > 31 || clamp_min < 0 || clamp_max > 255 || clamp_min > clamp_max)
     return MACE_HIP_SUCCESS;   // (the general path reports these)
@@ -620,7 +662,10 @@ int conv_rows(mace_hip_ctx *ctx, const uint8_t *input, const uint8_t *filter, co
   const int fx = cout <= 32 ? 1 : (cout <= 64 ? 2 : 4);
   const int64_t fixed = (128 * fx + MH_REQUANT_PAIRS_BYTES + 15) & ~(int64_t)15;
   auto lds_of = [&](int64_t r) { return fixed + ((r - 1) * stride_h + k_h) * pitch; };
-  if (lds_of(1) > 64 * 1024 || n * in_h >= (1ll << 31) || in_w * cin >= (1ll << 30) || pitch >= (1 << 24))
+  // (the kernel multiplies row numbers by row lengths with 24-bit factors and keeps offsets inside
+  // an image and inside the filter in 32 bits)
+  if (lds_of(1) > 64 * 1024 || n * in_h >= (1ll << 31) || in_w * cin >= (1ll << 23) || in_h >= (1ll << 23) ||
+      in_h * in_w * cin >= (1ll << 31) || pitch >= (1 << 23) || cout * depth >= (1ll << 23))
     return MACE_HIP_SUCCESS;
   // rows per strip: as for the short-patch kernel
   const int64_t cu = ctx->cu_count > 0 ? ctx->cu_count : 256;

@@ -214,6 +214,39 @@ def test_conv2d_q8_pieces_of_16_channels(ctx, n, cout, cin, in_h, in_w, k_h, k_w
     assert len(np.unique(want)) > 8
 
 
+def test_conv2d_q8_pieces_of_16_channels_operand_alignment(ctx):
+    """The strip kernel stages rows in 16-byte pieces: an input that does not start on a 16-byte
+    boundary takes another kernel, a filter or bias that does not still takes the strip kernel;
+    all exact against the oracle (device pointers, operands placed inside larger allocations)."""
+    import torch
+    n, cout, cin, in_h, in_w, k, st = 4, 32, 32, 28, 28, 3, (1, 1)
+    rng = np.random.default_rng(5)
+    x = rng.integers(0, 256, (n, in_h, in_w, cin), dtype=np.uint8)
+    f = rng.integers(0, 256, (cout, k, k, cin), dtype=np.uint8)
+    bias = rng.integers(-2 ** 15, 2 ** 15, cout).astype(np.int32)
+    s_in, s_f = np.float32(0.02), np.float32(0.01)
+    s_out = np.float32(3 * 74.0 * 74.0 * np.sqrt(k * k * cin) * float(s_in * s_f) / 255.0)
+    oh, ow, ph, pw = orc.calc_padding_and_output_size(in_h, in_w, k, k, st, S)
+    want = orc.conv2d_q8_nhwc(x, f, bias, n, in_h, in_w, cin, cout, k, k, st, (ph, pw), s_in, 120,
+                              s_f, 131, np.float32(s_in * s_f), s_out, 3, 0, 255, nthreads=16)
+    for (x_off, f_off, rows) in ((0, 0, True), (0, 1, True), (4, 0, False), (1, 3, False)):
+        xb = torch.zeros(x.size + 64, dtype=torch.uint8, device="cuda")
+        fb = torch.zeros(f.size + 64, dtype=torch.uint8, device="cuda")
+        xb[x_off:x_off + x.size] = torch.from_numpy(x.reshape(-1)).cuda()
+        fb[f_off:f_off + f.size] = torch.from_numpy(f.reshape(-1)).cuda()
+        bd = torch.from_numpy(bias).cuda()
+        out = torch.zeros(n * oh * ow * cout, dtype=torch.uint8, device="cuda")
+        assert xb.data_ptr() % 16 == 0 and fb.data_ptr() % 16 == 0
+        torch.cuda.synchronize()
+        ctx.call("mace_hip_conv2d_q8_nhwc", xb.data_ptr() + x_off, fb.data_ptr() + f_off, bd.data_ptr(),
+                 n, in_h, in_w, cin, cout, k, k, st[0], st[1], ph, pw, float(s_in), 120, float(s_f),
+                 131, float(s_in * s_f), float(s_out), 3, 0, 255, out.data_ptr())
+        ctx.sync()
+        assert (ctx.last_plan().kernel == "q8_conv_rows_kernel<FX=1,KS=9>") == rows, (x_off, f_off, ctx.last_plan())
+        np.testing.assert_array_equal(out.cpu().numpy().reshape(n, oh, ow, cout), want)
+    assert len(np.unique(want)) > 8
+
+
 def test_conv2d_q8_filter_in_lds_many_blocks(ctx):
     """More 64-pixel blocks than the kernel that keeps the filter in LDS has wavefronts: each
     wavefront walks over several blocks, prefetching the next block's first filter tap."""
