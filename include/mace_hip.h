@@ -133,6 +133,7 @@ enum {
   MACE_HIP_KF_F32_GEMV_GENERAL,      /* f32_gemv_kernel                                           */
   MACE_HIP_KF_Q8_CONV_SHORT,         /* q8_conv_short_kernel: patches of at most 32 bytes        */
   MACE_HIP_KF_Q8_CONV_ROWS,          /* q8_conv_rows_kernel: several taps of 16-channel pieces   */
+  MACE_HIP_KF_Q8_CONV_KSPLIT,        /* q8_conv_ksplit_kernel: few pixels, the depth in slices   */
   MACE_HIP_KF_COUNT
 };
 /* auxiliary passes of a call (bits of mace_hip_plan.aux) */
@@ -149,7 +150,8 @@ enum {
   MACE_HIP_AUX_FILL = 512,               /* constant fill (zero-point page, empty depth)          */
   MACE_HIP_AUX_WEIGHT_HIT = 1024,        /* a registered weight's panel / sums were reused        */
   MACE_HIP_AUX_WEIGHT_BUILD = 2048,      /* ... were built by this call                           */
-  MACE_HIP_AUX_F32_KSPLIT = 4096         /* fp32 GEMM: parts of the depth added up by a second launch */
+  MACE_HIP_AUX_F32_KSPLIT = 4096,        /* fp32 GEMM: parts of the depth added up by a second launch */
+  MACE_HIP_AUX_Q8_KSPLIT = 8192          /* uint8 convolution: slices of the depth added up and requantized by a second launch */
 };
 typedef struct mace_hip_plan {
   int family;      /* MACE_HIP_KF_*; NONE when the call launched no main kernel (empty result)    */

@@ -514,6 +514,157 @@ __global__ __launch_bounds__(256, 2) void q8_conv_rows_kernel(ConvShortParams p,
   }
 }
 
+// ---- few pixels against a long patch (the deep layers of a single image): the depth split ----
+//
+// A 3 x 3 convolution of 7 x 7 x 512 -> 512 on one image is 49 pixels against patches of 4608
+// bytes: as a GEMM it has eight 64 x 64 tiles, and a kernel that gives a tile to a workgroup walks
+// 72 k steps on 8 of 256 CUs (27.6 us).  Here a wavefront owns a 32 x 32 tile (32 output channels
+// x 32 pixels) over a slice of the depth, `kb_per` blocks of 64 bytes: every block lies inside one
+// filter tap (the channel count is a multiple of 64), so lane (row or pixel r, half h) loads its
+// 16 bytes of two k steps straight from the filter row and from the input pixel the tap selects
+// (a pixel of the padding is the zero point), no LDS, all loads of four blocks in flight.  The
+// zero-point terms are linear in k, so each wavefront adds those of its own slice to its sums
+// before it stores them; a second launch adds the slices in a fixed order, the bias and the
+// constant term, requantizes and stores bytes.
+struct ConvSplitParams {
+  const uint8_t *in, *filter;
+  int32_t *part;   // [task][lane][16] partial sums
+  int in_h, in_w, cin, cout, k_w, sh, sw, pt, pl, out_h, out_w;
+  int depth, columns, tiles_c, tiles_p, kblocks, kb_per, tasks;
+  int32_t xcoef, ycoef;
+  uint32_t zpf4;   // the input zero point ^ 0x80 in all four bytes
+};
+
+__global__ __launch_bounds__(256) void q8_conv_ksplit_kernel(ConvSplitParams p) {
+  __shared__ __align__(16) int32_t s_xs[4][32];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int h = lane >> 5, r32 = lane & 31;
+  const int task = (int)blockIdx.x * 4 + wave;   // (tile of channels fastest, then pixels, then slice)
+  if (task >= p.tasks) return;                   // (no workgroup barrier below)
+  const int tc = task % p.tiles_c, t2 = task / p.tiles_c;
+  const int tp = t2 % p.tiles_p, slice = t2 / p.tiles_p;
+  const int kb0 = slice * p.kb_per, kb1 = min(kb0 + p.kb_per, p.kblocks);
+  const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+  const v4i zero = {0, 0, 0, 0};
+  const int zpf = (int)p.zpf4;
+
+  const int c = min(tc * 32 + r32, p.cout - 1);
+  const uint8_t *frow = p.filter + (int64_t)c * p.depth + 16 * h;
+  const int pix = min(tp * 32 + r32, p.columns - 1);
+  const int per_img = p.out_h * p.out_w;
+  const int img = pix / per_img, rem = pix - img * per_img;
+  const int oh = rem / p.out_w, ow = rem - oh * p.out_w;
+  const int ih0 = oh * p.sh - p.pt, iw0 = ow * p.sw - p.pl;
+  const uint8_t *ibase = p.in + (int64_t)img * p.in_h * p.in_w * p.cin + 16 * h;
+
+  v16i acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0;
+  int xs = 0, ys = 0;   // sums of this lane's shifted filter / input bytes
+  constexpr int UN = 4;
+  for (int kb = kb0; kb < kb1; kb += UN) {
+    v4i a[UN][2], b[UN][2];
+    bool inside[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int k = min(kb + u, kb1 - 1) * 64;          // (the same in every lane: scalar)
+      const int tap = k / p.cin, c0 = k - tap * p.cin;
+      const int kh = tap / p.k_w, kw = tap - kh * p.k_w;
+      const int ih = ih0 + kh, iw = iw0 + kw;
+      inside[u] = (unsigned)ih < (unsigned)p.in_h && (unsigned)iw < (unsigned)p.in_w;
+      const int ihc = min(max(ih, 0), p.in_h - 1), iwc = min(max(iw, 0), p.in_w - 1);
+      const uint8_t *src = ibase + ((uint32_t)(ihc * p.in_w + iwc) * (uint32_t)p.cin + (uint32_t)c0);
+      b[u][0] = *(const v4i *)src;
+      b[u][1] = *(const v4i *)(src + 32);
+      a[u][0] = *(const v4i *)(frow + k);
+      a[u][1] = *(const v4i *)(frow + k + 32);
+    }
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const bool live = kb + u < kb1;   // (scalar)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const v4i x = live ? (a[u][j] ^ flip) : zero;
+        const v4i y = live ? (inside[u] ? (b[u][j] ^ flip) : v4i{zpf, zpf, zpf, zpf}) : zero;
+        xs = __builtin_amdgcn_sdot4(x.x, 0x01010101, xs, false);
+        xs = __builtin_amdgcn_sdot4(x.y, 0x01010101, xs, false);
+        xs = __builtin_amdgcn_sdot4(x.z, 0x01010101, xs, false);
+        xs = __builtin_amdgcn_sdot4(x.w, 0x01010101, xs, false);
+        ys = __builtin_amdgcn_sdot4(y.x, 0x01010101, ys, false);
+        ys = __builtin_amdgcn_sdot4(y.y, 0x01010101, ys, false);
+        ys = __builtin_amdgcn_sdot4(y.z, 0x01010101, ys, false);
+        ys = __builtin_amdgcn_sdot4(y.w, 0x01010101, ys, false);
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(x, y, acc, 0, 0, 0);
+      }
+    }
+  }
+  xs += __shfl_xor(xs, 32, 64);
+  ys += __shfl_xor(ys, 32, 64);
+  // register r of the result: channel 8 (r / 4) + 4 h + r % 4, pixel lane % 32.  The channels'
+  // sums change lanes through LDS (this wavefront's 32 words: written and read by it alone).
+  if (h == 0) s_xs[wave][r32] = (int32_t)((uint32_t)p.xcoef * (uint32_t)xs);
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const uint32_t cy = (uint32_t)p.ycoef * (uint32_t)ys;
+  int32_t *dst = p.part + ((int64_t)task * 64 + lane) * 16;
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const v4i cx = *(const v4i *)&s_xs[wave][8 * g + 4 * h];
+    v4i o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = (int)((uint32_t)acc[g * 4 + e] + (uint32_t)cx[e] + cy);
+    *(v4i *)(dst + 4 * g) = o;
+  }
+}
+
+// adds the slices in order, then bias, constant term and requantization: one thread per four
+// output channels of a pixel (a dwordx4 of every slice's partial tile)
+struct ConvSplitReduceParams {
+  const int32_t *part;
+  const int32_t *bias;
+  uint8_t *out;
+  int cout, columns, tiles_c, tiles_p, slices, total;   // total: threads with work
+  int32_t yadd;
+  RequantFixed rq;
+};
+
+__global__ __launch_bounds__(256) void q8_conv_ksplit_reduce_kernel(ConvSplitReduceParams p) {
+  const int idx = (int)blockIdx.x * 256 + (int)threadIdx.x;
+  if (idx >= p.total) return;
+  const int g = idx & 3, lane = (idx >> 2) & 63, tile = idx >> 8;
+  const int tc = tile % p.tiles_c, tp = tile / p.tiles_c;
+  const int64_t stride = (int64_t)p.tiles_c * p.tiles_p * 1024;   // words per slice
+  const int32_t *src = p.part + (int64_t)tile * 1024 + lane * 16 + g * 4;
+  uint32_t sum[4] = {0, 0, 0, 0};
+  int s = 0;
+  for (; s + 4 <= p.slices; s += 4) {   // (four loads in flight)
+    v4i v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = *(const v4i *)(src + (s + u) * stride);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) sum[e] += (uint32_t)v[u][e];
+  }
+  for (; s < p.slices; ++s) {
+    const v4i v = *(const v4i *)(src + s * stride);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) sum[e] += (uint32_t)v[e];
+  }
+  const int ch = tc * 32 + 8 * g + 4 * (lane >> 5), pix = tp * 32 + (lane & 31);
+  if (ch >= p.cout || pix >= p.columns) return;   // (cout is a multiple of 4)
+  uint32_t packed = 0;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    uint32_t v = sum[e] + (uint32_t)p.yadd;
+    if (p.bias) v += (uint32_t)p.bias[ch + e];
+    packed |= (uint32_t)(mh_requant_fixed((int32_t)v, p.rq) & 0xff) << (8 * e);
+  }
+  *(uint32_t *)(p.out + (int64_t)pix * p.cout + ch) = packed;
+}
+
 // floor(a / b) for b > 0
 inline int64_t floor_div(int64_t a, int64_t b) { return a >= 0 ? a / b : -((-a + b - 1) / b); }
 
@@ -716,6 +867,80 @@ int conv_rows(mace_hip_ctx *ctx, const uint8_t *input, const uint8_t *filter, co
   return MACE_HIP_SUCCESS;
 }
 
+// The depth split for few pixels against long patches.  *taken = false: not a call for it.
+int conv_ksplit(mace_hip_ctx *ctx, const uint8_t *input, const uint8_t *filter, const int32_t *bias,
+                int64_t n, int64_t in_h, int64_t in_w, int64_t cin, int64_t cout, int64_t k_h,
+                int64_t k_w, int stride_h, int stride_w, int pad_top, int pad_left, int64_t out_h,
+                int64_t out_w, float input_scale, int32_t input_zp, float filter_scale,
+                int32_t filter_zp, float bias_scale, int32_t mult, int shift, int32_t out_zp,
+                int clamp_min, int clamp_max, uint8_t *out, bool *taken) {
+  *taken = false;
+  const int64_t depth = k_h * k_w * cin, columns = n * out_h * out_w;
+  const int64_t tiles_c = (cout + 31) / 32, tiles_p = (columns + 31) / 32, tiles = tiles_c * tiles_p;
+  const int64_t kblocks = depth / 64;
+  const int64_t cu = ctx->cu_count > 0 ? ctx->cu_count : 256;
+  // Few tiles (a wavefront each would leave most SIMDs idle) and a depth worth splitting.  Measured
+  // against the kernels that take these calls otherwise, 3 x 3 on one image: 7 x 7 x 512 -> 512
+  // 27.9 -> 11.1 us, 14 x 14 x 256 -> 256 18.1 -> 9.1, 28 x 28 x 128 -> 128 14.2 -> 9.7, 28 x 28 x 256 ->
+  // 512 at stride 2 18.4 -> 10.1; at batch 4 27.0 -> 11.6, 18.3 -> 11.3, 14.3 -> 12.8, 18.7 -> 16.2; at
+  // batch 16, 7 x 7 x 512 -> 512 27.5 -> 22.6.  A 1 x 1 filter read in place has the one-launch
+  // kernel to beat: 7 x 7 x 1024 -> 1024 8.7 -> 8.1 and 7 x 7 x 2048 -> 512 12.5 -> 8.2 on one image,
+  // 8.9 -> 9.5 at batch 4 (224 tiles): taken there from 2048 channels and up to half a tile per CU.
+  const bool in_place = k_h == 1 && k_w == 1 && stride_h == 1 && stride_w == 1 && pad_top == 0 && pad_left == 0;
+  if (cin % 64 != 0 || cout % 4 != 0 || kblocks < (in_place ? 32 : 16) || tiles > (in_place ? cu / 2 : 2 * cu) ||
+      (uintptr_t)input % 16 != 0 || (uintptr_t)filter % 16 != 0 || (uintptr_t)out % 4 != 0 ||
+      n * in_h * in_w * cin >= (1ll << 40) || in_h * in_w * cin >= (1ll << 31) || ctx->no_alloc ||
+      ctx->capturing || (ctx->kernel_mask & MH_MASK_NO_CONV_SHORT))
+    return MACE_HIP_SUCCESS;
+  if (shift < 0 || shift > 31 || clamp_min < 0 || clamp_max > 255 || clamp_min > clamp_max)
+    return MACE_HIP_SUCCESS;   // (the general path reports these)
+  RequantFixed rq;
+  if (!mh_make_requant(mult, shift, out_zp, clamp_min, clamp_max, &rq)) return MACE_HIP_SUCCESS;
+  // slices: about four wavefronts per CU, at least four blocks of 64 bytes each (one turn of the
+  // kernel's loads), at most 16 (the second launch reads them all)
+  int64_t slices = std::min<int64_t>(std::min<int64_t>(kblocks / 4, 16), std::max<int64_t>(1, (4 * cu) / tiles));
+  const int64_t kb_per = (kblocks + slices - 1) / slices;
+  slices = (kblocks + kb_per - 1) / kb_per;
+  if (slices < 2) return MACE_HIP_SUCCESS;
+  const int64_t tasks = tiles * slices;
+  *taken = true;
+
+  const size_t part_bytes = (size_t)tasks * 4096;
+  MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, part_bytes + sizeof(int32_t) * cout + 8192));
+  ArenaScope scope(ctx);
+  const int32_t *bias_used = nullptr;
+  MH_RETURN_IF_ERROR(conv_bias(ctx, bias, cout, input_scale, filter_scale, bias_scale, &bias_used));
+  int32_t *part = (int32_t *)mh_arena_take(ctx, part_bytes);
+  if (!part) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
+  const uint32_t zl = (uint32_t)filter_zp - 128u, zr = (uint32_t)input_zp - 128u;
+  ConvSplitParams p{};
+  p.in = input; p.filter = filter; p.part = part;
+  p.in_h = (int)in_h; p.in_w = (int)in_w; p.cin = (int)cin; p.cout = (int)cout; p.k_w = (int)k_w;
+  p.sh = stride_h; p.sw = stride_w; p.pt = pad_top; p.pl = pad_left;
+  p.out_h = (int)out_h; p.out_w = (int)out_w; p.depth = (int)depth; p.columns = (int)columns;
+  p.tiles_c = (int)tiles_c; p.tiles_p = (int)tiles_p; p.kblocks = (int)kblocks;
+  p.kb_per = (int)kb_per; p.tasks = (int)tasks;
+  p.xcoef = (int32_t)(0u - zr);
+  p.ycoef = (int32_t)(0u - zl);
+  p.zpf4 = ((uint32_t)(input_zp & 0xff) * 0x01010101u) ^ 0x80808080u;
+  dim3 grid((unsigned)((tasks + 3) / 4)), block(256);
+  mh_plan_main(ctx, MACE_HIP_KF_Q8_CONV_KSPLIT, 0, grid, block, 512);
+  mh_plan_aux(ctx, MACE_HIP_AUX_Q8_KSPLIT);
+  MH_PROF_BEGIN(ctx);
+  MH_KLAUNCH(ctx, q8_conv_ksplit_kernel, grid, block, 0, ctx->stream, p);
+  MH_PROF_END(ctx);
+  MH_LAUNCH_CHECK(ctx);
+  ConvSplitReduceParams r{};
+  r.part = part; r.bias = bias_used; r.out = out;
+  r.cout = (int)cout; r.columns = (int)columns; r.tiles_c = (int)tiles_c; r.tiles_p = (int)tiles_p;
+  r.slices = (int)slices; r.total = (int)(tiles * 256);
+  r.yadd = (int32_t)((uint32_t)depth * zl * zr);
+  r.rq = rq;
+  MH_KLAUNCH(ctx, q8_conv_ksplit_reduce_kernel, dim3((unsigned)tiles), dim3(256), 0, ctx->stream, r);
+  MH_LAUNCH_CHECK(ctx);
+  return MACE_HIP_SUCCESS;
+}
+
 // scratch the GEMM takes from the arena for a [cout x depth] . [depth x columns] product
 inline size_t conv_gemm_scratch(int64_t cout, int64_t depth, int64_t columns, bool rhs_in_place) {
   const size_t kp = mh_align_up((size_t)(depth > 0 ? depth : 1), 64);
@@ -772,6 +997,14 @@ extern "C" int mace_hip_conv2d_q8_nhwc(mace_hip_ctx *ctx, const uint8_t *input,
                                  stride_h, stride_w, pad_h >> 1, pad_w >> 1, out_h, out_w,
                                  input_scale, input_zp, filter_scale, filter_zp, bias_scale, mult,
                                  shift, out_zp, clamp_min, clamp_max, out, &taken));
+    if (taken) return MACE_HIP_SUCCESS;
+  }
+  {
+    bool taken = false;
+    MH_RETURN_IF_ERROR(conv_ksplit(ctx, input, filter, bias, n, in_h, in_w, cin, cout, k_h, k_w,
+                                   stride_h, stride_w, pad_h >> 1, pad_w >> 1, out_h, out_w,
+                                   input_scale, input_zp, filter_scale, filter_zp, bias_scale, mult,
+                                   shift, out_zp, clamp_min, clamp_max, out, &taken));
     if (taken) return MACE_HIP_SUCCESS;
   }
   // With cin a multiple of 64 (and at least three 64-byte slabs of depth) the GEMM's loader

@@ -247,6 +247,48 @@ def test_conv2d_q8_pieces_of_16_channels_operand_alignment(ctx):
     assert len(np.unique(want)) > 8
 
 
+KSPLIT_CASES = [  # batch, cout, cin, in_h, in_w, k_h, k_w, padding, strides
+    (1, 512, 512, 7, 7, 3, 3, S, (1, 1)),       # the deep layers of a single image
+    (1, 256, 256, 14, 14, 3, 3, S, (1, 1)),
+    (1, 128, 128, 28, 28, 3, 3, S, (1, 1)),
+    (1, 512, 512, 14, 14, 3, 3, S, (2, 2)),
+    (2, 100, 192, 9, 11, 3, 3, Fu, (1, 1)),     # ragged tiles of channels and pixels, padding of 2
+    (1, 512, 2048, 7, 7, 1, 1, V, (1, 1)),      # a 1 x 1 filter read in place
+    (3, 36, 320, 5, 6, 2, 3, S, (1, 2)),        # 30 blocks of 64 bytes: slices of unequal length
+    (1, 48, 64, 13, 13, 5, 5, S, (1, 1)),       # every block a tap of its own
+    (1, 260, 128, 10, 10, 3, 3, V, (3, 3)),
+]
+
+
+@pytest.mark.parametrize("n,cout,cin,in_h,in_w,k_h,k_w,pad,st", KSPLIT_CASES)
+def test_conv2d_q8_depth_in_slices(ctx, n, cout, cin, in_h, in_w, k_h, k_w, pad, st):
+    """Few pixels against a long patch: wavefronts take 32 x 32 tiles over slices of the depth and a
+    second launch adds the slices up and requantizes.  Against the oracle bit for bit, the kernel
+    that ran asserted, three bias / clamp settings each."""
+    rng = np.random.default_rng(cout * 7 + cin + k_h * 5 + k_w + in_w)
+    x = rng.integers(0, 256, (n, in_h, in_w, cin), dtype=np.uint8)
+    f = rng.integers(0, 256, (cout, k_h, k_w, cin), dtype=np.uint8)
+    bias = rng.integers(-2 ** 15, 2 ** 15, cout).astype(np.int32)
+    z_in, z_f = int(rng.integers(100, 156)), int(rng.integers(100, 156))
+    s_in, s_f = np.float32(0.02), np.float32(0.01)
+    depth = k_h * k_w * cin
+    s_out = np.float32(max(6.0, 3 * 74.0 * 74.0 * np.sqrt(depth) * float(s_in * s_f)) / 255.0)
+    oh, ow, ph, pw = orc.calc_padding_and_output_size(in_h, in_w, k_h, k_w, st, pad)
+    for (bb, s_b, z_o, lo, hi) in ((bias, np.float32(s_in * s_f), 0, 0, 255),
+                                   (bias, np.float32(2.5 * float(s_in * s_f)), 100, 100, 230),
+                                   (None, np.float32(0), 128, 0, 255)):
+        want = orc.conv2d_q8_nhwc(x, f, bb, n, in_h, in_w, cin, cout, k_h, k_w, st, (ph, pw), s_in,
+                                  z_in, s_f, z_f, s_b, s_out, z_o, lo, hi, nthreads=16)
+        got = conv_host(ctx, x, f, bb, n, in_h, in_w, cin, cout, k_h, k_w, st, (ph, pw), s_in,
+                        z_in, s_f, z_f, s_b, s_out, z_o, lo, hi)
+        plan = ctx.last_plan()
+        assert plan.kernel == "q8_conv_ksplit_kernel" and plan.aux & mh.AUX_Q8_KSPLIT, plan
+        assert plan.launches == (3 if plan.aux & mh.AUX_BIAS_RESCALE else 2), plan
+        assert got.shape == (n, oh, ow, cout)
+        np.testing.assert_array_equal(got, want)
+    assert len(np.unique(want)) > 8
+
+
 def test_conv2d_q8_filter_in_lds_many_blocks(ctx):
     """More 64-pixel blocks than the kernel that keeps the filter in LDS has wavefronts: each
     wavefront walks over several blocks, prefetching the next block's first filter tap."""

@@ -337,6 +337,23 @@ def test_convolution_gather_and_im2col(ctx):
     assert conv(ctx, 8, 56, 48, 64, k=3, stride=1, pad=2).family != mh.KF_Q8_CONV_ROWS      # 27 pieces
     assert conv(ctx, 8, 56, 32, 128, k=3, stride=1, pad=2).family != mh.KF_Q8_CONV_ROWS     # 18 pieces, > 64 output channels
     assert conv(ctx, 64, 112, 32, 64, k=3, stride=1, pad=2, mask=mh.MASK_NO_CONV_SHORT).family != mh.KF_Q8_CONV_ROWS
+
+
+def test_conv_depth_in_slices_for_few_pixels(ctx):
+    """Few 32 x 32 tiles against a depth of at least 16 blocks of 64 bytes: wavefronts take slices of
+    the depth and a second launch adds them up (the deep 3 x 3 layers of one image; a 1 x 1 filter
+    read in place only from 32 blocks and up to half a tile per CU)."""
+    p = conv(ctx, 1, 7, 512, 512, k=3, stride=1, pad=2)
+    assert p.kernel == "q8_conv_ksplit_kernel" and p.aux == mh.AUX_Q8_KSPLIT and p.launches == 2, p
+    assert p.grid == (120, 1, 1), p                                   # 32 tiles x 15 slices / 4 wavefronts
+    assert conv(ctx, 4, 14, 256, 256, k=3, stride=1, pad=2).family == mh.KF_Q8_CONV_KSPLIT
+    assert conv(ctx, 16, 7, 512, 512, k=3, stride=1, pad=2).family == mh.KF_Q8_CONV_KSPLIT      # 400 tiles
+    assert conv(ctx, 64, 7, 512, 512, k=3, stride=1, pad=2).family != mh.KF_Q8_CONV_KSPLIT      # 1568 tiles
+    assert conv(ctx, 1, 7, 2048, 512).family == mh.KF_Q8_CONV_KSPLIT                              # 32 tiles, in place
+    assert conv(ctx, 1, 7, 1024, 1024).family != mh.KF_Q8_CONV_KSPLIT                             # in place, 16 blocks of depth
+    assert conv(ctx, 16, 7, 2048, 512).family != mh.KF_Q8_CONV_KSPLIT                             # 400 tiles, in place
+    assert conv(ctx, 1, 14, 64, 64, k=3, stride=1, pad=2).family != mh.KF_Q8_CONV_KSPLIT        # 9 blocks of depth
+    assert conv(ctx, 1, 7, 512, 512, k=3, stride=1, pad=2, mask=mh.MASK_NO_CONV_SHORT).family != mh.KF_Q8_CONV_KSPLIT
     # not for it: 33 bytes of patch, channel counts that are not whole 16-byte pieces of the output
     # row or more than 128, fewer than 1024 pixels; those stay with the one-launch kernel
     small = mh.KF_Q8_GEMM_FUSED_SMALL
@@ -390,7 +407,7 @@ def test_variant_tables_are_consistent():
         total += len(vs)
         assert not lib.mace_hip_plan_variant_valid(f, n) and not lib.mace_hip_plan_variant_valid(f, -1)
         assert mh.coverage(f, 0) == 0              # nothing is launched by planning
-    assert total == 226
+    assert total == 227
     assert lib.mace_hip_plan_variant_count(0) == 0 and lib.mace_hip_plan_variant_count(mh.KF_COUNT) == 0
 
 
