@@ -590,7 +590,8 @@ def bench_other(ctx, mh, torch):
     # stride 2 is MobileNet's first layer: patches of 27 bytes, the strip kernel)
     for (n, hw, cin, cout, k, st) in ((64, 56, 64, 64, 3, 1), (64, 28, 128, 128, 3, 1),
                                       (64, 224, 3, 32, 3, 2), (1, 224, 3, 32, 3, 2), (1, 56, 64, 64, 3, 1), (1, 28, 128, 128, 3, 1),
-                                      (64, 112, 32, 32, 3, 1)):   # 18 pieces of 16 channels: q8_conv_rows_kernel
+                                      (64, 112, 32, 32, 3, 1),    # 18 pieces of 16 channels: q8_conv_rows_kernel
+                                      (1, 14, 256, 256, 3, 1), (1, 7, 512, 512, 3, 1)):   # few pixels, long patches: the depth in slices
         oh = (hw + st - 1) // st
         pad = max((oh - 1) * st + k - hw, 0)      # SAME
         x, f = u8(n, hw, hw, cin), u8(cout, k, k, cin)
