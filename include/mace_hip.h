@@ -133,7 +133,8 @@ enum {
   MACE_HIP_KF_F32_GEMV_GENERAL,      /* f32_gemv_kernel                                           */
   MACE_HIP_KF_Q8_CONV_SHORT,         /* q8_conv_short_kernel: patches of at most 32 bytes        */
   MACE_HIP_KF_Q8_CONV_ROWS,          /* q8_conv_rows_kernel: several taps of 16-channel pieces   */
-  MACE_HIP_KF_Q8_CONV_KSPLIT,        /* q8_conv_ksplit_kernel: few pixels, the depth in slices   */
+  MACE_HIP_KF_Q8_CONV_KSPLIT,        /* q8_conv_ksplit_kernel: few pixels, a wavefront per slice of the depth */
+  MACE_HIP_KF_Q8_CONV_KSLICES,       /* q8_conv_kslices_kernel: ... over the whole device, two launches */
   MACE_HIP_KF_COUNT
 };
 /* auxiliary passes of a call (bits of mace_hip_plan.aux) */

@@ -221,6 +221,7 @@ inline int gemv_slice(int spw, bool out_u8) { return log2i(spw) * 2 + (out_u8 ? 
 inline int gemv_out(bool out_u8) { return out_u8 ? 1 : 0; }
 inline int conv_short(int fx) { return log2i(fx); }
 inline int conv_rows(int fx, int ks) { return log2i(fx) * 2 + (ks == 9 ? 1 : 0); }
+inline int conv_ksplit(int waves) { return waves == 16 ? 1 : 0; }
 inline int gemv_mfma(int nw, bool out_u8) { return (log2i(nw) - 2) * 2 + (out_u8 ? 1 : 0); }
 inline int gemv_rows(int nb, bool out_u8) { return log2i(nb) * 2 + (out_u8 ? 1 : 0); }
 inline int gemv_general(int nb, bool vec, bool out_u8) {

@@ -517,16 +517,142 @@ __global__ __launch_bounds__(256, 2) void q8_conv_rows_kernel(ConvShortParams p,
 // ---- few pixels against a long patch (the deep layers of a single image): the depth split ----
 //
 // A 3 x 3 convolution of 7 x 7 x 512 -> 512 on one image is 49 pixels against patches of 4608
-// bytes: as a GEMM it has eight 64 x 64 tiles, and a kernel that gives a tile to a workgroup walks
-// 72 k steps on 8 of 256 CUs (27.6 us).  Here a wavefront owns a 32 x 32 tile (32 output channels
-// x 32 pixels) over a slice of the depth, `kb_per` blocks of 64 bytes: every block lies inside one
-// filter tap (the channel count is a multiple of 64), so lane (row or pixel r, half h) loads its
-// 16 bytes of two k steps straight from the filter row and from the input pixel the tap selects
-// (a pixel of the padding is the zero point), no LDS, all loads of four blocks in flight.  The
-// zero-point terms are linear in k, so each wavefront adds those of its own slice to its sums
-// before it stores them; a second launch adds the slices in a fixed order, the bias and the
-// constant term, requantizes and stores bytes.
+// bytes: as a GEMM it has eight 64 x 64 tiles, and a kernel that gives a tile to four wavefronts
+// walks 72 k steps on 8 of 256 CUs (27.6 us).  Here a workgroup of 8 or 16 wavefronts owns a
+// 32 x 32 tile (32 output channels x 32 pixels) and each wavefront a slice of the depth, `kb_per`
+// blocks of 64 bytes: every block lies inside one filter tap (the channel count is a multiple of
+// 64), so lane (row or pixel r, half h) loads its 16 bytes of two k steps straight from the filter
+// row and from the input pixel the tap selects (a pixel of the padding is the zero point), no LDS,
+// all loads of four blocks in flight.  The zero-point terms are linear in k, so each wavefront adds
+// those of its own slice to its sums; the sums meet in LDS, where 256 threads add the slices in
+// their fixed order, then the bias and the constant term, requantize and store four bytes each.
 struct ConvSplitParams {
+  const uint8_t *in, *filter;
+  const int32_t *bias;
+  uint8_t *out;
+  int in_h, in_w, cin, cout, k_w, sh, sw, pt, pl, out_h, out_w;
+  int depth, columns, tiles_c, kblocks, kb_per;
+  int32_t xcoef, ycoef, yadd;
+  uint32_t zpf4;   // the input zero point ^ 0x80 in all four bytes
+  RequantFixed rq;
+};
+
+template <int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void q8_conv_ksplit_kernel(ConvSplitParams p) {
+  __shared__ __align__(16) int32_t s_xs[WAVES][32];
+  __shared__ __align__(16) int32_t s_part[WAVES][4][64][4];   // [slice][register group][lane]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int h = lane >> 5, r32 = lane & 31;
+  const int tc = (int)blockIdx.x % p.tiles_c, tp = (int)blockIdx.x / p.tiles_c;
+  const int kb0 = wave * p.kb_per, kb1 = min(kb0 + p.kb_per, p.kblocks);   // (empty for late slices)
+  const v4i flip = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+  const v4i zero = {0, 0, 0, 0};
+  const int zpf = (int)p.zpf4;
+
+  const int c = min(tc * 32 + r32, p.cout - 1);
+  const uint8_t *frow = p.filter + (int64_t)c * p.depth + 16 * h;
+  const int pix = min(tp * 32 + r32, p.columns - 1);
+  const int per_img = p.out_h * p.out_w;
+  const int img = pix / per_img, rem = pix - img * per_img;
+  const int oh = rem / p.out_w, ow = rem - oh * p.out_w;
+  const int ih0 = oh * p.sh - p.pt, iw0 = ow * p.sw - p.pl;
+  const uint8_t *ibase = p.in + (int64_t)img * p.in_h * p.in_w * p.cin + 16 * h;
+
+  v16i acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0;
+  int xs = 0, ys = 0;   // sums of this lane's shifted filter / input bytes
+  constexpr int UN = 4;
+  for (int kb = kb0; kb < kb1; kb += UN) {
+    v4i a[UN][2], b[UN][2];
+    bool inside[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int k = min(kb + u, kb1 - 1) * 64;          // (the same in every lane: scalar)
+      const int tap = k / p.cin, c0 = k - tap * p.cin;
+      const int kh = tap / p.k_w, kw = tap - kh * p.k_w;
+      const int ih = ih0 + kh, iw = iw0 + kw;
+      inside[u] = (unsigned)ih < (unsigned)p.in_h && (unsigned)iw < (unsigned)p.in_w;
+      const int ihc = min(max(ih, 0), p.in_h - 1), iwc = min(max(iw, 0), p.in_w - 1);
+      const uint8_t *src = ibase + ((uint32_t)(ihc * p.in_w + iwc) * (uint32_t)p.cin + (uint32_t)c0);
+      b[u][0] = *(const v4i *)src;
+      b[u][1] = *(const v4i *)(src + 32);
+      a[u][0] = *(const v4i *)(frow + k);
+      a[u][1] = *(const v4i *)(frow + k + 32);
+    }
+    // (all sixteen loads are requested before the first is used: left to itself the compiler
+    // keeps two in flight and waits for memory before every MFMA)
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const bool live = kb + u < kb1;   // (scalar)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const v4i x = live ? (a[u][j] ^ flip) : zero;
+        const v4i y = live ? (inside[u] ? (b[u][j] ^ flip) : v4i{zpf, zpf, zpf, zpf}) : zero;
+        xs = __builtin_amdgcn_sdot4(x.x, 0x01010101, xs, false);
+        xs = __builtin_amdgcn_sdot4(x.y, 0x01010101, xs, false);
+        xs = __builtin_amdgcn_sdot4(x.z, 0x01010101, xs, false);
+        xs = __builtin_amdgcn_sdot4(x.w, 0x01010101, xs, false);
+        ys = __builtin_amdgcn_sdot4(y.x, 0x01010101, ys, false);
+        ys = __builtin_amdgcn_sdot4(y.y, 0x01010101, ys, false);
+        ys = __builtin_amdgcn_sdot4(y.z, 0x01010101, ys, false);
+        ys = __builtin_amdgcn_sdot4(y.w, 0x01010101, ys, false);
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(x, y, acc, 0, 0, 0);
+      }
+    }
+  }
+  xs += __shfl_xor(xs, 32, 64);
+  ys += __shfl_xor(ys, 32, 64);
+  // register r of the result: channel 8 (r / 4) + 4 h + r % 4, pixel lane % 32.  The channels'
+  // sums change lanes through LDS.
+  if (h == 0) s_xs[wave][r32] = (int32_t)((uint32_t)p.xcoef * (uint32_t)xs);
+  __syncthreads();
+  const uint32_t cy = (uint32_t)p.ycoef * (uint32_t)ys;
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const v4i cx = *(const v4i *)&s_xs[wave][8 * g + 4 * h];
+    v4i o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = (int)((uint32_t)acc[g * 4 + e] + (uint32_t)cx[e] + cy);
+    *(v4i *)&s_part[wave][g][lane][0] = o;
+  }
+  __syncthreads();
+  if (tid >= 256) return;
+  // thread (register group g, lane l): four channels of a pixel
+  const int g = tid >> 6;
+  const int ch = tc * 32 + 8 * g + 4 * h, pixel = tp * 32 + r32;
+  int32_t bias_v[4] = {0, 0, 0, 0};
+  if (p.bias) {   // (requested together, ahead of the sums)
+    const int cb = min(ch, p.cout - 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) bias_v[e] = p.bias[cb + e];
+  }
+  uint32_t sum[4] = {0, 0, 0, 0};
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w) {
+    const v4i v = *(const v4i *)&s_part[w][g][lane][0];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) sum[e] += (uint32_t)v[e];
+  }
+  if (ch >= p.cout || pixel >= p.columns) return;   // (cout is a multiple of 4)
+  uint32_t packed = 0;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const uint32_t v = sum[e] + (uint32_t)p.yadd + (uint32_t)bias_v[e];
+    packed |= (uint32_t)(mh_requant_fixed((int32_t)v, p.rq) & 0xff) << (8 * e);
+  }
+  *(uint32_t *)(p.out + (int64_t)pixel * p.cout + ch) = packed;
+}
+
+// The same tile and the same slices where the depth is too long for one workgroup's wavefronts
+// (more than 48 blocks of 64 bytes: the loads of a 32-row tile touch 32 cache lines each, and
+// one CU's memory pipeline is what 8 or 16 wavefronts then wait for): a wavefront per (tile,
+// slice) spread over the whole device, the sums of a slice stored (4 KiB, L2-resident), and a
+// second launch that adds the slices in their fixed order, then bias and constant term,
+// requantizes and stores bytes.
+struct ConvSlicesParams {
   const uint8_t *in, *filter;
   int32_t *part;   // [task][lane][16] partial sums
   int in_h, in_w, cin, cout, k_w, sh, sw, pt, pl, out_h, out_w;
@@ -535,7 +661,7 @@ struct ConvSplitParams {
   uint32_t zpf4;   // the input zero point ^ 0x80 in all four bytes
 };
 
-__global__ __launch_bounds__(256) void q8_conv_ksplit_kernel(ConvSplitParams p) {
+__global__ __launch_bounds__(256) void q8_conv_kslices_kernel(ConvSlicesParams p) {
   __shared__ __align__(16) int32_t s_xs[4][32];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -580,6 +706,7 @@ __global__ __launch_bounds__(256) void q8_conv_ksplit_kernel(ConvSplitParams p) 
       a[u][0] = *(const v4i *)(frow + k);
       a[u][1] = *(const v4i *)(frow + k + 32);
     }
+    __builtin_amdgcn_sched_barrier(0);   // (all loads requested before the first is used)
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
       const bool live = kb + u < kb1;   // (scalar)
@@ -621,7 +748,7 @@ __global__ __launch_bounds__(256) void q8_conv_ksplit_kernel(ConvSplitParams p) 
 
 // adds the slices in order, then bias, constant term and requantization: one thread per four
 // output channels of a pixel (a dwordx4 of every slice's partial tile)
-struct ConvSplitReduceParams {
+struct ConvSlicesReduceParams {
   const int32_t *part;
   const int32_t *bias;
   uint8_t *out;
@@ -630,7 +757,7 @@ struct ConvSplitReduceParams {
   RequantFixed rq;
 };
 
-__global__ __launch_bounds__(256) void q8_conv_ksplit_reduce_kernel(ConvSplitReduceParams p) {
+__global__ __launch_bounds__(256) void q8_conv_kslices_reduce_kernel(ConvSlicesReduceParams p) {
   const int idx = (int)blockIdx.x * 256 + (int)threadIdx.x;
   if (idx >= p.total) return;
   const int g = idx & 3, lane = (idx >> 2) & 63, tile = idx >> 8;
@@ -868,6 +995,18 @@ int conv_rows(mace_hip_ctx *ctx, const uint8_t *input, const uint8_t *filter, co
 }
 
 // The depth split for few pixels against long patches.  *taken = false: not a call for it.
+//
+// Measured on one image against the kernels that take these calls otherwise (3 x 3 unless said;
+// blocks = depth / 64): one workgroup per tile with 8 wavefronts up to 32 blocks (28 x 28 x 128 ->
+// 128, 18 blocks: 13.0 -> 5.9 us; 1 x 1 on 7 x 7 x 2048 -> 512, 32 blocks: 11.9 -> 6.6), with 16
+// up to 48 (14 x 14 x 256 -> 256, 36 blocks: 17.9 -> 8.5 against 9.7 with 8; 28 x 28 x 256 -> 512 at
+// stride 2: 17.8 -> 8.8), a wavefront per (tile, slice) over the whole device and a second launch
+// beyond (7 x 7 x 512 -> 512, 72 blocks: 27.9 -> 11.1 against 13.2 / 15.8 in one launch).  At batch
+// 4: 13.1 -> 8.8, 18.0 -> 8.8, 18.2 -> 16.6, 27.2 -> 11.6; at batch 16, 7 x 7 x 512 -> 512 27.5 -> 22.6.
+// From 9 blocks on: 56 x 56 x 64 -> 64 (9 blocks) 8.5 -> 5.2, 28 x 28 x 64 -> 128 8.6 -> 5.2.  A 1 x 1 filter
+// read in place has the one-launch GEMM kernel to beat: 7 x 7 x 1024 -> 1024 8.8 -> 6.7, 14 x 14 x 640 ->
+// 128 (10 blocks) 6.9 -> 6.0, but 14 x 14 x 512 -> 512 (8 blocks) 6.6 -> 6.9: from 10 blocks there, up to
+// one tile per CU (7 x 7 x 1024 -> 1024 at batch 4, 224 tiles: 8.7 -> 7.1).
 int conv_ksplit(mace_hip_ctx *ctx, const uint8_t *input, const uint8_t *filter, const int32_t *bias,
                 int64_t n, int64_t in_h, int64_t in_w, int64_t cin, int64_t cout, int64_t k_h,
                 int64_t k_w, int stride_h, int stride_w, int pad_top, int pad_left, int64_t out_h,
@@ -879,32 +1018,56 @@ int conv_ksplit(mace_hip_ctx *ctx, const uint8_t *input, const uint8_t *filter, 
   const int64_t tiles_c = (cout + 31) / 32, tiles_p = (columns + 31) / 32, tiles = tiles_c * tiles_p;
   const int64_t kblocks = depth / 64;
   const int64_t cu = ctx->cu_count > 0 ? ctx->cu_count : 256;
-  // Few tiles (a wavefront each would leave most SIMDs idle) and a depth worth splitting.  Measured
-  // against the kernels that take these calls otherwise, 3 x 3 on one image: 7 x 7 x 512 -> 512
-  // 27.9 -> 11.1 us, 14 x 14 x 256 -> 256 18.1 -> 9.1, 28 x 28 x 128 -> 128 14.2 -> 9.7, 28 x 28 x 256 ->
-  // 512 at stride 2 18.4 -> 10.1; at batch 4 27.0 -> 11.6, 18.3 -> 11.3, 14.3 -> 12.8, 18.7 -> 16.2; at
-  // batch 16, 7 x 7 x 512 -> 512 27.5 -> 22.6.  A 1 x 1 filter read in place has the one-launch
-  // kernel to beat: 7 x 7 x 1024 -> 1024 8.7 -> 8.1 and 7 x 7 x 2048 -> 512 12.5 -> 8.2 on one image,
-  // 8.9 -> 9.5 at batch 4 (224 tiles): taken there from 2048 channels and up to half a tile per CU.
   const bool in_place = k_h == 1 && k_w == 1 && stride_h == 1 && stride_w == 1 && pad_top == 0 && pad_left == 0;
-  if (cin % 64 != 0 || cout % 4 != 0 || kblocks < (in_place ? 32 : 16) || tiles > (in_place ? cu / 2 : 2 * cu) ||
+  if (cin % 64 != 0 || cout % 4 != 0 || kblocks < (in_place ? 10 : 9) || tiles > (in_place ? cu : 2 * cu) ||
       (uintptr_t)input % 16 != 0 || (uintptr_t)filter % 16 != 0 || (uintptr_t)out % 4 != 0 ||
-      n * in_h * in_w * cin >= (1ll << 40) || in_h * in_w * cin >= (1ll << 31) || ctx->no_alloc ||
-      ctx->capturing || (ctx->kernel_mask & MH_MASK_NO_CONV_SHORT))
+      n * in_h * in_w * cin >= (1ll << 40) || in_h * in_w * cin >= (1ll << 31) ||
+      (ctx->kernel_mask & MH_MASK_NO_CONV_SHORT))
     return MACE_HIP_SUCCESS;
   if (shift < 0 || shift > 31 || clamp_min < 0 || clamp_max > 255 || clamp_min > clamp_max)
     return MACE_HIP_SUCCESS;   // (the general path reports these)
   RequantFixed rq;
   if (!mh_make_requant(mult, shift, out_zp, clamp_min, clamp_max, &rq)) return MACE_HIP_SUCCESS;
+  // (the slices' sums of the two-launch form live in the arena)
+  const bool spread = kblocks > 48 && !ctx->no_alloc && !ctx->capturing;
+  const uint32_t zl = (uint32_t)filter_zp - 128u, zr = (uint32_t)input_zp - 128u;
+  const int32_t yadd = (int32_t)((uint32_t)depth * zl * zr);
+  *taken = true;
+
+  if (!spread) {
+    const int waves = kblocks > 32 ? 16 : 8;
+    const int64_t kb_per = (kblocks + waves - 1) / waves;
+    MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, sizeof(int32_t) * cout + 4096));
+    ArenaScope scope(ctx);
+    const int32_t *bias_used = nullptr;
+    MH_RETURN_IF_ERROR(conv_bias(ctx, bias, cout, input_scale, filter_scale, bias_scale, &bias_used));
+    ConvSplitParams p{};
+    p.in = input; p.filter = filter; p.bias = bias_used; p.out = out;
+    p.in_h = (int)in_h; p.in_w = (int)in_w; p.cin = (int)cin; p.cout = (int)cout; p.k_w = (int)k_w;
+    p.sh = stride_h; p.sw = stride_w; p.pt = pad_top; p.pl = pad_left;
+    p.out_h = (int)out_h; p.out_w = (int)out_w; p.depth = (int)depth; p.columns = (int)columns;
+    p.tiles_c = (int)tiles_c; p.kblocks = (int)kblocks; p.kb_per = (int)kb_per;
+    p.xcoef = (int32_t)(0u - zr);
+    p.ycoef = (int32_t)(0u - zl);
+    p.yadd = yadd;
+    p.zpf4 = ((uint32_t)(input_zp & 0xff) * 0x01010101u) ^ 0x80808080u;
+    p.rq = rq;
+    dim3 grid((unsigned)tiles), block(64 * waves);
+    mh_plan_main(ctx, MACE_HIP_KF_Q8_CONV_KSPLIT, mhv::conv_ksplit(waves), grid, block, waves * (4096 + 128));
+    MH_PROF_BEGIN(ctx);
+    if (waves == 16) MH_KLAUNCH(ctx, q8_conv_ksplit_kernel<16>, grid, block, 0, ctx->stream, p);
+    else MH_KLAUNCH(ctx, q8_conv_ksplit_kernel<8>, grid, block, 0, ctx->stream, p);
+    MH_PROF_END(ctx);
+    MH_LAUNCH_CHECK(ctx);
+    return MACE_HIP_SUCCESS;
+  }
+
   // slices: about four wavefronts per CU, at least four blocks of 64 bytes each (one turn of the
   // kernel's loads), at most 16 (the second launch reads them all)
   int64_t slices = std::min<int64_t>(std::min<int64_t>(kblocks / 4, 16), std::max<int64_t>(1, (4 * cu) / tiles));
   const int64_t kb_per = (kblocks + slices - 1) / slices;
   slices = (kblocks + kb_per - 1) / kb_per;
-  if (slices < 2) return MACE_HIP_SUCCESS;
   const int64_t tasks = tiles * slices;
-  *taken = true;
-
   const size_t part_bytes = (size_t)tasks * 4096;
   MH_RETURN_IF_ERROR(mh_arena_reserve(ctx, part_bytes + sizeof(int32_t) * cout + 8192));
   ArenaScope scope(ctx);
@@ -912,8 +1075,7 @@ int conv_ksplit(mace_hip_ctx *ctx, const uint8_t *input, const uint8_t *filter, 
   MH_RETURN_IF_ERROR(conv_bias(ctx, bias, cout, input_scale, filter_scale, bias_scale, &bias_used));
   int32_t *part = (int32_t *)mh_arena_take(ctx, part_bytes);
   if (!part) return mh_fail(ctx, MACE_HIP_RUNTIME_ERROR, "arena slice unavailable");
-  const uint32_t zl = (uint32_t)filter_zp - 128u, zr = (uint32_t)input_zp - 128u;
-  ConvSplitParams p{};
+  ConvSlicesParams p{};
   p.in = input; p.filter = filter; p.part = part;
   p.in_h = (int)in_h; p.in_w = (int)in_w; p.cin = (int)cin; p.cout = (int)cout; p.k_w = (int)k_w;
   p.sh = stride_h; p.sw = stride_w; p.pt = pad_top; p.pl = pad_left;
@@ -924,19 +1086,19 @@ int conv_ksplit(mace_hip_ctx *ctx, const uint8_t *input, const uint8_t *filter, 
   p.ycoef = (int32_t)(0u - zl);
   p.zpf4 = ((uint32_t)(input_zp & 0xff) * 0x01010101u) ^ 0x80808080u;
   dim3 grid((unsigned)((tasks + 3) / 4)), block(256);
-  mh_plan_main(ctx, MACE_HIP_KF_Q8_CONV_KSPLIT, 0, grid, block, 512);
+  mh_plan_main(ctx, MACE_HIP_KF_Q8_CONV_KSLICES, 0, grid, block, 512);
   mh_plan_aux(ctx, MACE_HIP_AUX_Q8_KSPLIT);
   MH_PROF_BEGIN(ctx);
-  MH_KLAUNCH(ctx, q8_conv_ksplit_kernel, grid, block, 0, ctx->stream, p);
+  MH_KLAUNCH(ctx, q8_conv_kslices_kernel, grid, block, 0, ctx->stream, p);
   MH_PROF_END(ctx);
   MH_LAUNCH_CHECK(ctx);
-  ConvSplitReduceParams r{};
+  ConvSlicesReduceParams r{};
   r.part = part; r.bias = bias_used; r.out = out;
   r.cout = (int)cout; r.columns = (int)columns; r.tiles_c = (int)tiles_c; r.tiles_p = (int)tiles_p;
   r.slices = (int)slices; r.total = (int)(tiles * 256);
-  r.yadd = (int32_t)((uint32_t)depth * zl * zr);
+  r.yadd = yadd;
   r.rq = rq;
-  MH_KLAUNCH(ctx, q8_conv_ksplit_reduce_kernel, dim3((unsigned)tiles), dim3(256), 0, ctx->stream, r);
+  MH_KLAUNCH(ctx, q8_conv_kslices_reduce_kernel, dim3((unsigned)tiles), dim3(256), 0, ctx->stream, r);
   MH_LAUNCH_CHECK(ctx);
   return MACE_HIP_SUCCESS;
 }

@@ -33,7 +33,8 @@ const int kVariantCount[MACE_HIP_KF_COUNT] = {
     1,                        // F32_GEMV_GENERAL
     3,                        // Q8_CONV_SHORT
     5,                        // Q8_CONV_ROWS (FX = 4 exists with KS = 5 only)
-    1,                        // Q8_CONV_KSPLIT
+    2,                        // Q8_CONV_KSPLIT
+    1,                        // Q8_CONV_KSLICES
 };
 static_assert(mhv::RING_CONFIGS * 8 <= kMaxVariants, "coverage table too narrow");
 
@@ -43,7 +44,8 @@ const char *const kFamilyName[MACE_HIP_KF_COUNT] = {
     "q8_gemm_kernel", "q8_gemv_row_kernel", "q8_gemv_mfma_slice_kernel", "q8_gemv_mfma_lds_kernel",
     "q8_gemv_mfma_kernel", "q8_gemv_rows_kernel", "q8_gemv_kernel", "f32_gemm_vec_kernel",
     "f32_gemm_kernel", "f32_fill_kernel", "f32_gemv_vec_kernel", "f32_gemv_kernel",
-    "q8_conv_short_kernel", "q8_conv_rows_kernel", "q8_conv_ksplit_kernel"};
+    "q8_conv_short_kernel", "q8_conv_rows_kernel", "q8_conv_ksplit_kernel",
+    "q8_conv_kslices_kernel"};
 
 // <WX, WY, FX, FY, STAGES, OCC, KB> of the ring kernel's tile configurations (mhv::RING_*)
 const int kRing[mhv::RING_CONFIGS][7] = {
@@ -189,6 +191,9 @@ int mace_hip_plan_describe(int family, int v, char *buf, size_t len) {
       break;
     case MACE_HIP_KF_Q8_CONV_ROWS:
       snprintf(buf, len, "%s<FX=%d,KS=%d>", k, 1 << (v >> 1), (v & 1) ? 9 : 5);
+      break;
+    case MACE_HIP_KF_Q8_CONV_KSPLIT:
+      snprintf(buf, len, "%s<WAVES=%d>", k, v ? 16 : 8);
       break;
     case MACE_HIP_KF_F32_GEMV_VEC:
       snprintf(buf, len, "%s<NB=%d>", k, 1 << v);

@@ -131,7 +131,7 @@ SIGNATURES = {
  KF_Q8_GEMM_RING_XT, KF_Q8_GEMM_RING_XF, KF_Q8_GEMM_TILED, KF_Q8_GEMV_ROW, KF_Q8_GEMV_SLICE,
  KF_Q8_GEMV_MFMA_LDS, KF_Q8_GEMV_MFMA, KF_Q8_GEMV_ROWS, KF_Q8_GEMV_GENERAL, KF_F32_GEMM_VEC,
  KF_F32_GEMM_GENERAL, KF_F32_GEMM_FILL, KF_F32_GEMV_VEC, KF_F32_GEMV_GENERAL, KF_Q8_CONV_SHORT,
- KF_Q8_CONV_ROWS, KF_Q8_CONV_KSPLIT, KF_COUNT) = range(24)
+ KF_Q8_CONV_ROWS, KF_Q8_CONV_KSPLIT, KF_Q8_CONV_KSLICES, KF_COUNT) = range(25)
 (AUX_PACK_ROWS, AUX_PACK_TRANSPOSE, AUX_PACK_SHIFTED, AUX_PANEL_SUMS, AUX_KMAJOR_SUMS, AUX_ZERO,
  AUX_IM2COL, AUX_BIAS_RESCALE, AUX_F32_PAD, AUX_FILL, AUX_WEIGHT_HIT, AUX_WEIGHT_BUILD,
  AUX_F32_KSPLIT, AUX_Q8_KSPLIT) = (1 << i for i in range(14))

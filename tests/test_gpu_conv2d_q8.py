@@ -256,14 +256,19 @@ KSPLIT_CASES = [  # batch, cout, cin, in_h, in_w, k_h, k_w, padding, strides
     (1, 512, 2048, 7, 7, 1, 1, V, (1, 1)),      # a 1 x 1 filter read in place
     (3, 36, 320, 5, 6, 2, 3, S, (1, 2)),        # 30 blocks of 64 bytes: slices of unequal length
     (1, 48, 64, 13, 13, 5, 5, S, (1, 1)),       # every block a tap of its own
+    (2, 64, 256, 14, 14, 3, 3, S, (1, 1)),      # 36 blocks: sixteen wavefronts per tile
+    (1, 96, 192, 12, 12, 4, 4, V, (2, 2)),      # 48 blocks, three per wavefront
+    (1, 64, 64, 56, 56, 3, 3, S, (1, 1)),       # 9 blocks: the eighth wavefront has none
+    (1, 1024, 1024, 7, 7, 1, 1, V, (1, 1)),     # 16 blocks, in place
     (1, 260, 128, 10, 10, 3, 3, V, (3, 3)),
 ]
 
 
 @pytest.mark.parametrize("n,cout,cin,in_h,in_w,k_h,k_w,pad,st", KSPLIT_CASES)
 def test_conv2d_q8_depth_in_slices(ctx, n, cout, cin, in_h, in_w, k_h, k_w, pad, st):
-    """Few pixels against a long patch: wavefronts take 32 x 32 tiles over slices of the depth and a
-    second launch adds the slices up and requantizes.  Against the oracle bit for bit, the kernel
+    """Few pixels against a long patch: a wavefront per slice of the depth of a 32 x 32 tile, the
+    slices added up in their fixed order and requantized -- in LDS by the tile's workgroup up to 48
+    blocks of 64 bytes, by a second launch beyond.  Against the oracle bit for bit, the kernel
     that ran asserted, three bias / clamp settings each."""
     rng = np.random.default_rng(cout * 7 + cin + k_h * 5 + k_w + in_w)
     x = rng.integers(0, 256, (n, in_h, in_w, cin), dtype=np.uint8)
@@ -282,8 +287,12 @@ def test_conv2d_q8_depth_in_slices(ctx, n, cout, cin, in_h, in_w, k_h, k_w, pad,
         got = conv_host(ctx, x, f, bb, n, in_h, in_w, cin, cout, k_h, k_w, st, (ph, pw), s_in,
                         z_in, s_f, z_f, s_b, s_out, z_o, lo, hi)
         plan = ctx.last_plan()
-        assert plan.kernel == "q8_conv_ksplit_kernel" and plan.aux & mh.AUX_Q8_KSPLIT, plan
-        assert plan.launches == (3 if plan.aux & mh.AUX_BIAS_RESCALE else 2), plan
+        blocks = depth // 64
+        if blocks > 48:     # a wavefront per (tile, slice) over the whole device, then the sum
+            assert plan.kernel == "q8_conv_kslices_kernel" and plan.aux & mh.AUX_Q8_KSPLIT, plan
+        else:               # a workgroup per tile, a wavefront per slice
+            assert plan.kernel == "q8_conv_ksplit_kernel<WAVES=%d>" % (16 if blocks > 32 else 8), plan
+        assert plan.launches == (1 if blocks <= 48 else 2) + (1 if plan.aux & mh.AUX_BIAS_RESCALE else 0), plan
         assert got.shape == (n, oh, ow, cout)
         np.testing.assert_array_equal(got, want)
     assert len(np.unique(want)) > 8

@@ -104,8 +104,9 @@ def test_config4_conv1x1_batch64(ctx):
         assert p.kernel == kernel, (hw, p)
         assert p.launches == 1 and p.aux == 0      # nothing but the GEMM kernel is launched
     for (hw, cin, cout) in want:                   # single-image inference: one small launch each
-        p = conv(ctx, 1, hw, cin, cout)
-        assert p.family == mh.KF_Q8_GEMM_FUSED_SMALL and p.launches == 1, (hw, p)
+        p = conv(ctx, 1, hw, cin, cout)            # (1024 channels: a wavefront per slice of the depth)
+        assert p.family == (mh.KF_Q8_CONV_KSPLIT if cin == 1024 else mh.KF_Q8_GEMM_FUSED_SMALL), (hw, p)
+        assert p.launches == 1, (hw, p)
 
 
 def test_config2_f32_gemm(ctx):
@@ -340,32 +341,29 @@ def test_convolution_gather_and_im2col(ctx):
 
 
 def test_conv_depth_in_slices_for_few_pixels(ctx):
-    """Few 32 x 32 tiles against a depth of at least 16 blocks of 64 bytes: wavefronts take slices of
-    the depth and a second launch adds them up (the deep 3 x 3 layers of one image; a 1 x 1 filter
-    read in place only from 32 blocks and up to half a tile per CU)."""
-    p = conv(ctx, 1, 7, 512, 512, k=3, stride=1, pad=2)
-    assert p.kernel == "q8_conv_ksplit_kernel" and p.aux == mh.AUX_Q8_KSPLIT and p.launches == 2, p
-    assert p.grid == (120, 1, 1), p                                   # 32 tiles x 15 slices / 4 wavefronts
-    assert conv(ctx, 4, 14, 256, 256, k=3, stride=1, pad=2).family == mh.KF_Q8_CONV_KSPLIT
-    assert conv(ctx, 16, 7, 512, 512, k=3, stride=1, pad=2).family == mh.KF_Q8_CONV_KSPLIT      # 400 tiles
-    assert conv(ctx, 64, 7, 512, 512, k=3, stride=1, pad=2).family != mh.KF_Q8_CONV_KSPLIT      # 1568 tiles
-    assert conv(ctx, 1, 7, 2048, 512).family == mh.KF_Q8_CONV_KSPLIT                              # 32 tiles, in place
-    assert conv(ctx, 1, 7, 1024, 1024).family != mh.KF_Q8_CONV_KSPLIT                             # in place, 16 blocks of depth
-    assert conv(ctx, 16, 7, 2048, 512).family != mh.KF_Q8_CONV_KSPLIT                             # 400 tiles, in place
-    assert conv(ctx, 1, 14, 64, 64, k=3, stride=1, pad=2).family != mh.KF_Q8_CONV_KSPLIT        # 9 blocks of depth
-    assert conv(ctx, 1, 7, 512, 512, k=3, stride=1, pad=2, mask=mh.MASK_NO_CONV_SHORT).family != mh.KF_Q8_CONV_KSPLIT
-    # not for it: 33 bytes of patch, channel counts that are not whole 16-byte pieces of the output
-    # row or more than 128, fewer than 1024 pixels; those stay with the one-launch kernel
-    small = mh.KF_Q8_GEMM_FUSED_SMALL
-    assert conv(ctx, 8, 64, 3, 32, k=3, stride=1, pad=2, mask=0).family == mh.KF_Q8_CONV_SHORT
-    assert conv(ctx, 8, 64, 11, 32, k=3, stride=3, pad=0).family == small     # depth 99
-    assert conv(ctx, 8, 64, 3, 24, k=3, stride=2, pad=1).family == small
-    assert conv(ctx, 8, 64, 3, 144, k=3, stride=2, pad=1).family == small
-    assert conv(ctx, 1, 40, 3, 32, k=3, stride=2, pad=1).family == small      # 400 pixels
-    p = conv(ctx, 64, 224, 3, 32, k=3, stride=2, pad=1, mask=mh.MASK_NO_CONV_SHORT)
-    assert p.family == small and "BW=true" in p.kernel and p.launches == 1   # gathered byte-wise
-    p = conv(ctx, 64, 224, 3, 32, k=3, stride=2, pad=1, mask=mh.MASK_NO_SMALL | mh.MASK_NO_CONV_SHORT)
-    assert p.aux & mh.AUX_IM2COL
+    """Few 32 x 32 tiles against a depth of at least 9 blocks of 64 bytes (the 3 x 3 layers of
+    one image): a wavefront per slice of the depth; one workgroup per tile up to 48 blocks (8
+    wavefronts up to 32, then 16), spread over the device with a second launch beyond.  A 1 x 1
+    filter read in place from 10 blocks, up to a tile per CU; other filters from 9 blocks."""
+    KS = (mh.KF_Q8_CONV_KSPLIT, mh.KF_Q8_CONV_KSLICES)
+    p = conv(ctx, 1, 28, 128, 128, k=3, stride=1, pad=2)                  # 18 blocks
+    assert p.kernel == "q8_conv_ksplit_kernel<WAVES=8>" and p.aux == 0 and p.launches == 1, p
+    assert p.grid == (100, 1, 1) and p.block == 512, p                     # a workgroup per 32 x 32 tile
+    p = conv(ctx, 4, 14, 256, 256, k=3, stride=1, pad=2)                  # 36 blocks
+    assert p.kernel == "q8_conv_ksplit_kernel<WAVES=16>" and p.launches == 1 and p.block == 1024, p
+    p = conv(ctx, 1, 7, 512, 512, k=3, stride=1, pad=2)                   # 72 blocks
+    assert p.kernel == "q8_conv_kslices_kernel" and p.aux == mh.AUX_Q8_KSPLIT and p.launches == 2, p
+    assert p.grid == (120, 1, 1), p                                        # 32 tiles x 15 slices / 4 wavefronts
+    assert conv(ctx, 16, 7, 512, 512, k=3, stride=1, pad=2).family == mh.KF_Q8_CONV_KSLICES      # 400 tiles
+    assert conv(ctx, 64, 7, 512, 512, k=3, stride=1, pad=2).family not in KS                      # 1568 tiles
+    assert conv(ctx, 1, 7, 2048, 512).kernel == "q8_conv_ksplit_kernel<WAVES=8>"                  # 32 tiles, in place
+    assert conv(ctx, 1, 14, 640, 128).family == mh.KF_Q8_CONV_KSPLIT                              # in place, 10 blocks
+    assert conv(ctx, 1, 14, 512, 512).family not in KS                                            # in place, 8 blocks
+    assert conv(ctx, 16, 7, 2048, 512).family not in KS                                           # 400 tiles, in place
+    assert conv(ctx, 1, 56, 64, 64, k=3, stride=1, pad=2).family == mh.KF_Q8_CONV_KSPLIT          # 9 blocks of depth
+    assert conv(ctx, 1, 14, 128, 64, k=2, stride=1, pad=0).family not in KS                       # 8 blocks of depth
+    assert conv(ctx, 1, 7, 512, 512, k=3, stride=1, pad=2, mask=mh.MASK_NO_CONV_SHORT).family not in KS
+    assert conv(ctx, 1, 28, 128, 128, k=3, stride=1, pad=2, mask=mh.MASK_NO_CONV_SHORT).family not in KS
 
 
 def test_gemv_dispatch(ctx):
@@ -407,7 +405,7 @@ def test_variant_tables_are_consistent():
         total += len(vs)
         assert not lib.mace_hip_plan_variant_valid(f, n) and not lib.mace_hip_plan_variant_valid(f, -1)
         assert mh.coverage(f, 0) == 0              # nothing is launched by planning
-    assert total == 227
+    assert total == 229
     assert lib.mace_hip_plan_variant_count(0) == 0 and lib.mace_hip_plan_variant_count(mh.KF_COUNT) == 0
 
 
