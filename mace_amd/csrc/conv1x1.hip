@@ -559,6 +559,17 @@ __global__ __launch_bounds__(64 * WAVES) void q8_conv_ksplit_kernel(ConvSplitPar
   const int ih0 = oh * p.sh - p.pt, iw0 = ow * p.sw - p.pl;
   const uint8_t *ibase = p.in + (int64_t)img * p.in_h * p.in_w * p.cin + 16 * h;
 
+  // thread (register group g_out, lane) of the first four wavefronts stores four channels of a
+  // pixel at the end: their bias is requested here, with the operands
+  const int g_out = tid >> 6;
+  const int ch = tc * 32 + 8 * g_out + 4 * h, pixel = tp * 32 + r32;
+  int32_t bias_v[4] = {0, 0, 0, 0};
+  if (p.bias && tid < 256) {
+    const int cb = min(ch, p.cout - 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) bias_v[e] = p.bias[cb + e];
+  }
+
   v16i acc;
 #pragma unroll
   for (int r = 0; r < 16; ++r) acc[r] = 0;
@@ -620,19 +631,10 @@ __global__ __launch_bounds__(64 * WAVES) void q8_conv_ksplit_kernel(ConvSplitPar
   }
   __syncthreads();
   if (tid >= 256) return;
-  // thread (register group g, lane l): four channels of a pixel
-  const int g = tid >> 6;
-  const int ch = tc * 32 + 8 * g + 4 * h, pixel = tp * 32 + r32;
-  int32_t bias_v[4] = {0, 0, 0, 0};
-  if (p.bias) {   // (requested together, ahead of the sums)
-    const int cb = min(ch, p.cout - 4);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) bias_v[e] = p.bias[cb + e];
-  }
   uint32_t sum[4] = {0, 0, 0, 0};
 #pragma unroll
   for (int w = 0; w < WAVES; ++w) {
-    const v4i v = *(const v4i *)&s_part[w][g][lane][0];
+    const v4i v = *(const v4i *)&s_part[w][g_out][lane][0];
 #pragma unroll
     for (int e = 0; e < 4; ++e) sum[e] += (uint32_t)v[e];
   }
