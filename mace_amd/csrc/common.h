@@ -632,6 +632,13 @@ inline int mh_blocks_per_cu(mace_hip_ctx *ctx, const void *kernel, int threads, 
 // recorded into a caller's graph capture has replayed wrongly on this hardware pool).
 int mh_fill_bytes(mace_hip_ctx *ctx, void *dst, uint8_t value, size_t bytes);
 
+// conv1x1.hip: a GEMM with both operands k-contiguous, few 32 x 32 tiles and a long depth, by the
+// convolution kernels that deal the depth to wavefronts.  *taken = false: not a call for them.
+int mh_q8_gemm_depth_split(mace_hip_ctx *ctx, const uint8_t *lhs, const uint8_t *rhs, uint8_t *out,
+                           int out_order, int64_t rows, int64_t depth, int64_t cols,
+                           int32_t lhs_offset, int32_t rhs_offset, const int32_t *bias,
+                           int32_t mult, int shift, int32_t out_zp, int clamp_min, int clamp_max,
+                           bool *taken);
 int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8_t *rhs,
                int rhs_order, void *out, int out_order, bool out_u8, int64_t batch,
                int64_t rows, int64_t depth, int64_t cols, int lhs_batched, int rhs_batched,

@@ -534,6 +534,7 @@ struct ConvSplitParams {
   int depth, columns, tiles_c, kblocks, kb_per;
   int32_t xcoef, ycoef, yadd;
   uint32_t zpf4;   // the input zero point ^ 0x80 in all four bytes
+  int bias_px;     // the bias is one word per pixel, not per output channel (a MatMul's rows)
   RequantFixed rq;
 };
 
@@ -565,9 +566,9 @@ __global__ __launch_bounds__(64 * WAVES) void q8_conv_ksplit_kernel(ConvSplitPar
   const int ch = tc * 32 + 8 * g_out + 4 * h, pixel = tp * 32 + r32;
   int32_t bias_v[4] = {0, 0, 0, 0};
   if (p.bias && tid < 256) {
-    const int cb = min(ch, p.cout - 4);
+    const int cb = min(ch, p.cout - 4), pb = min(pixel, p.columns - 1);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) bias_v[e] = p.bias[cb + e];
+    for (int e = 0; e < 4; ++e) bias_v[e] = p.bias[p.bias_px ? pb : cb + e];
   }
 
   v16i acc;
@@ -755,6 +756,7 @@ struct ConvSlicesReduceParams {
   const int32_t *bias;
   uint8_t *out;
   int cout, columns, tiles_c, tiles_p, slices, total;   // total: threads with work
+  int bias_px;   // the bias is one word per pixel, not per output channel
   int32_t yadd;
   RequantFixed rq;
 };
@@ -788,7 +790,7 @@ __global__ __launch_bounds__(256) void q8_conv_kslices_reduce_kernel(ConvSlicesR
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     uint32_t v = sum[e] + (uint32_t)p.yadd;
-    if (p.bias) v += (uint32_t)p.bias[ch + e];
+    if (p.bias) v += (uint32_t)p.bias[p.bias_px ? pix : ch + e];
     packed |= (uint32_t)(mh_requant_fixed((int32_t)v, p.rq) & 0xff) << (8 * e);
   }
   *(uint32_t *)(p.out + (int64_t)pix * p.cout + ch) = packed;
@@ -1014,7 +1016,7 @@ int conv_ksplit(mace_hip_ctx *ctx, const uint8_t *input, const uint8_t *filter, 
                 int64_t k_w, int stride_h, int stride_w, int pad_top, int pad_left, int64_t out_h,
                 int64_t out_w, float input_scale, int32_t input_zp, float filter_scale,
                 int32_t filter_zp, float bias_scale, int32_t mult, int shift, int32_t out_zp,
-                int clamp_min, int clamp_max, uint8_t *out, bool *taken) {
+                int clamp_min, int clamp_max, uint8_t *out, bool *taken, bool bias_per_pixel = false) {
   *taken = false;
   const int64_t depth = k_h * k_w * cin, columns = n * out_h * out_w;
   const int64_t tiles_c = (cout + 31) / 32, tiles_p = (columns + 31) / 32, tiles = tiles_c * tiles_p;
@@ -1053,6 +1055,7 @@ int conv_ksplit(mace_hip_ctx *ctx, const uint8_t *input, const uint8_t *filter, 
     p.ycoef = (int32_t)(0u - zl);
     p.yadd = yadd;
     p.zpf4 = ((uint32_t)(input_zp & 0xff) * 0x01010101u) ^ 0x80808080u;
+    p.bias_px = bias_per_pixel ? 1 : 0;
     p.rq = rq;
     dim3 grid((unsigned)tiles), block(64 * waves);
     mh_plan_main(ctx, MACE_HIP_KF_Q8_CONV_KSPLIT, mhv::conv_ksplit(waves), grid, block, waves * (4096 + 128));
@@ -1098,12 +1101,41 @@ int conv_ksplit(mace_hip_ctx *ctx, const uint8_t *input, const uint8_t *filter, 
   r.part = part; r.bias = bias_used; r.out = out;
   r.cout = (int)cout; r.columns = (int)columns; r.tiles_c = (int)tiles_c; r.tiles_p = (int)tiles_p;
   r.slices = (int)slices; r.total = (int)(tiles * 256);
+  r.bias_px = bias_per_pixel ? 1 : 0;
   r.yadd = yadd;
   r.rq = rq;
   MH_KLAUNCH(ctx, q8_conv_kslices_reduce_kernel, dim3((unsigned)tiles), dim3(256), 0, ctx->stream, r);
   MH_LAUNCH_CHECK(ctx);
   return MACE_HIP_SUCCESS;
 }
+
+}  // namespace
+
+// A uint8 GEMM whose operands are both k-contiguous (RowMajor lhs, ColMajor rhs: a MatMul against
+// transposed weights) is the 1 x 1 convolution above: the operand whose index runs along the
+// result's contiguous direction plays the filter (for a ColMajor result the lhs, bias per output
+// channel; for a RowMajor one the rhs, and the bias goes by "pixel").  FullyConnected batches of
+// 16 - 64 rows through the tiled kernels against this: 32 x 4096 x 4096 20.1 -> 12.2 us,
+// 64 x 2048 x 1024 11.7 -> 6.7, 16 x 9216 x 4096 37.3 -> 15.6, 32 x 1024 x 4096 8.7 -> 7.0.
+int mh_q8_gemm_depth_split(mace_hip_ctx *ctx, const uint8_t *lhs, const uint8_t *rhs, uint8_t *out,
+                           int out_order, int64_t rows, int64_t depth, int64_t cols,
+                           int32_t lhs_offset, int32_t rhs_offset, const int32_t *bias,
+                           int32_t mult, int shift, int32_t out_zp, int clamp_min, int clamp_max,
+                           bool *taken) {
+  *taken = false;
+  if (!lhs || !rhs || !out || rows <= 0 || cols <= 0 || depth <= 0 || rows >= (1 << 24) ||
+      cols >= (1 << 24) || depth >= (1 << 24) || lhs_offset > 0 || lhs_offset < -255 ||
+      rhs_offset > 0 || rhs_offset < -255)
+    return MACE_HIP_SUCCESS;
+  const bool x_is_lhs = out_order == MACE_HIP_COL_MAJOR;
+  const uint8_t *x = x_is_lhs ? lhs : rhs, *y = x_is_lhs ? rhs : lhs;
+  const int64_t xn = x_is_lhs ? rows : cols, yn = x_is_lhs ? cols : rows;
+  const int32_t x_zp = x_is_lhs ? -lhs_offset : -rhs_offset, y_zp = x_is_lhs ? -rhs_offset : -lhs_offset;
+  return conv_ksplit(ctx, y, x, bias, 1, 1, yn, depth, xn, 1, 1, 1, 1, 0, 0, 1, yn, 1.0f, y_zp, 1.0f,
+                     x_zp, 1.0f, mult, shift, out_zp, clamp_min, clamp_max, out, taken, !x_is_lhs);
+}
+
+namespace {
 
 // scratch the GEMM takes from the arena for a [cout x depth] . [depth x columns] product
 inline size_t conv_gemm_scratch(int64_t cout, int64_t depth, int64_t columns, bool rhs_in_place) {

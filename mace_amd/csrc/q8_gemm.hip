@@ -3297,6 +3297,13 @@ int mh_q8_gemm(mace_hip_ctx *ctx, const uint8_t *lhs, int lhs_order, const uint8
   Q8Call call{ctx, lhs, lhs_order, rhs, rhs_order, out, out_order, out_u8, batch, rows, depth, cols,
               lhs_batched, rhs_batched, lhs_offset, rhs_offset, ep, rhs_ld, cv};
   bool done = false;
+  if (out_u8 && batch == 1 && !cv && rhs_ld == 0 && lhs_order == MACE_HIP_ROW_MAJOR &&
+      rhs_order == MACE_HIP_COL_MAJOR) {
+    MH_RETURN_IF_ERROR(mh_q8_gemm_depth_split(ctx, lhs, rhs, (uint8_t *)out, out_order, rows, depth, cols,
+                                              lhs_offset, rhs_offset, ep.bias, ep.mult, ep.shift,
+                                              ep.zp, ep.lo, ep.hi, &done));
+    if (done) return MACE_HIP_SUCCESS;
+  }
   MH_RETURN_IF_ERROR(call.prepare(&done));
   if (done) return MACE_HIP_SUCCESS;
   MH_RETURN_IF_ERROR(call.small_problem(&done));

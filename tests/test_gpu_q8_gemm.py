@@ -64,8 +64,10 @@ def path(request, ctx):
     """Small problems are one launch of a kernel of their own, and an X panel that fits in LDS has
     one too; kernel-mask bit 0 leaves the second, bit 1 on top of it only
     the general path (repack, row sums, tiled kernel), so that all three stay covered."""
-    mask = {"default": 0, "no_small_kernel": mh.MASK_NO_SMALL,
-            "general_path": mh.MASK_NO_SMALL | mh.MASK_NO_XRES}[request.param]
+    # (both also without the kernels that deal the depth of a few 32 x 32 tiles to wavefronts, which
+    # take uint8 calls with two k-contiguous operands under the default dispatch)
+    mask = {"default": 0, "no_small_kernel": mh.MASK_NO_SMALL | mh.MASK_NO_CONV_SHORT,
+            "general_path": mh.MASK_NO_SMALL | mh.MASK_NO_XRES | mh.MASK_NO_CONV_SHORT}[request.param]
     ctx.call("mace_hip_ctx_set_kernel_mask", mask)
     yield request.param
     ctx.call("mace_hip_ctx_set_kernel_mask", 0)
@@ -191,7 +193,7 @@ MID_SHAPES = [  # batch, rows, depth, cols, lhs batched, rhs batched, lhs order,
 def test_q8_gemm_one_round_of_tiles(ctx, mid, batch, rows, depth, cols, lb, rb, lo, ro, oo, kernel):
     # (the one-launch kernel and the kernel that keeps one panel in LDS would take the shallower
     # shapes: switched off here)
-    ctx.call("mace_hip_ctx_set_kernel_mask", mh.MASK_NO_SMALL | mh.MASK_NO_XRES |
+    ctx.call("mace_hip_ctx_set_kernel_mask", mh.MASK_NO_SMALL | mh.MASK_NO_XRES | mh.MASK_NO_CONV_SHORT |
              (0 if mid == "one_round_kernel" else mh.MASK_NO_MID))
     try:
         tag32, tag8 = check_gemm(ctx, batch, rows, depth, cols, lb, rb, lo, ro, oo)
@@ -202,6 +204,30 @@ def test_q8_gemm_one_round_of_tiles(ctx, mid, batch, rows, depth, cols, lb, rb, 
     else:   # the ring kernel on repacked / in-place k-contiguous panels
         want = "ring_xf" if depth >= 1280 and kernel == "ring_xt" else "ring"
         assert (tag32, tag8) == (want, want)
+
+
+# Both operands k-contiguous (RowMajor lhs, ColMajor rhs: a MatMul against transposed weights), few
+# 32 x 32 tiles, a depth of ten 64-byte blocks or more: the uint8 call is the 1 x 1 convolution whose
+# depth is dealt to wavefronts -- one workgroup per tile up to 48 blocks, two launches beyond; with a
+# RowMajor result the rhs plays the filter and the bias goes by result row all the same.
+KSPLIT_GEMM_SHAPES = [  # rows, depth, cols, out order, kernel of the uint8 call
+    (32, 1024, 512, R, "q8_conv_ksplit_kernel<WAVES=8>"), (300, 1024, 64, R, "q8_conv_ksplit_kernel<WAVES=8>"),
+    (64, 2048, 96, Cm, "q8_conv_ksplit_kernel<WAVES=8>"), (20, 640, 36, Cm, "q8_conv_ksplit_kernel<WAVES=8>"),
+    (49, 2304, 100, R, "q8_conv_ksplit_kernel<WAVES=16>"), (20, 3072, 260, Cm, "q8_conv_ksplit_kernel<WAVES=16>"),
+    (16, 4096, 256, R, "q8_conv_kslices_kernel"), (36, 9216, 128, Cm, "q8_conv_kslices_kernel"),
+]
+
+
+@pytest.mark.parametrize("rows,depth,cols,oo,kernel", KSPLIT_GEMM_SHAPES)
+def test_q8_gemm_depth_dealt_to_wavefronts(ctx, rows, depth, cols, oo, kernel):
+    tag32, tag8 = check_gemm(ctx, 1, rows, depth, cols, True, True, R, Cm, oo)
+    assert tag8 == kernel and not tag32.startswith("q8_conv"), (tag32, tag8)
+    ctx.call("mace_hip_ctx_set_kernel_mask", mh.MASK_NO_CONV_SHORT)
+    try:
+        _, masked = check_gemm(ctx, 1, rows, depth, cols, True, True, R, Cm, oo)
+    finally:
+        ctx.call("mace_hip_ctx_set_kernel_mask", 0)
+    assert not masked.startswith("q8_conv"), masked
 
 
 # Shapes on the boundaries between the one-launch kernels under the normal dispatch: the

@@ -147,7 +147,8 @@ def fam(p):
 
 def test_small_problem_limits(ctx):
     # depth 1024 is the last the one-launch kernel takes with 16-byte pieces
-    assert fam(gemm(ctx, 1, 256, 1024, 256, ro=Cm)) == mh.KF_Q8_GEMM_FUSED_SMALL
+    assert fam(gemm(ctx, 1, 256, 1024, 256, ro=Cm, u8=False)) == mh.KF_Q8_GEMM_FUSED_SMALL
+    assert fam(gemm(ctx, 1, 256, 1024, 256, ro=Cm)) == mh.KF_Q8_CONV_KSPLIT     # (uint8 result: the depth dealt to wavefronts)
     assert fam(gemm(ctx, 1, 256, 1088, 256, ro=Cm)) != mh.KF_Q8_GEMM_FUSED_SMALL
     # ... depth 320 when an operand is read byte by byte (odd extent)
     assert fam(gemm(ctx, 1, 255, 320, 255)) == mh.KF_Q8_GEMM_FUSED_SMALL
@@ -194,8 +195,11 @@ def test_eight_wavefront_kernel_range(ctx):
     assert fam(gemm(ctx, 1, 256, 1024, 256)) == mid and gemm(ctx, 1, 256, 1024, 256).launches == 1
     assert fam(gemm(ctx, 1, 128, 2048, 384)) == mid and fam(gemm(ctx, 4, 256, 4096, 256)) == mid
     assert fam(gemm(ctx, 1, 256, 512, 256)) == mh.KF_Q8_GEMM_FUSED_SMALL
-    assert fam(gemm(ctx, 1, 256, 2048, 256, ro=Cm)) == mid
-    assert fam(gemm(ctx, 1, 256, 1024, 256, ro=Cm)) == mh.KF_Q8_GEMM_FUSED_SMALL
+    assert fam(gemm(ctx, 1, 256, 2048, 256, ro=Cm, u8=False)) == mid
+    assert fam(gemm(ctx, 1, 256, 2048, 256, ro=Cm)) == mh.KF_Q8_CONV_KSPLIT
+    assert fam(gemm(ctx, 1, 512, 2048, 1024, ro=Cm)) == mid                      # 512 tiles of 32 x 32
+    assert fam(gemm(ctx, 1, 64, 4096, 4096, ro=Cm)) == mh.KF_Q8_CONV_KSLICES and fam(gemm(ctx, 1, 64, 4096, 4096)) != mh.KF_Q8_CONV_KSLICES
+    assert fam(gemm(ctx, 1, 256, 1024, 256, ro=Cm, u8=False)) == mh.KF_Q8_GEMM_FUSED_SMALL
     assert "YT=true" in gemm(ctx, 1, 256, 512, 256, lo=Cm).kernel and "YT=true" in gemm(ctx, 1, 128, 640, 144, lo=Cm, ro=Cm).kernel
     # k-major Y (transpose_a with a RowMajor result), X k-major or k-contiguous: read as they lie
     p = gemm(ctx, 1, 2048, 2048, 2048, lo=Cm)
