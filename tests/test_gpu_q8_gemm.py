@@ -230,6 +230,34 @@ def test_q8_gemm_depth_dealt_to_wavefronts(ctx, rows, depth, cols, oo, kernel):
     assert not masked.startswith("q8_conv"), masked
 
 
+@pytest.mark.parametrize("rows,depth,cols,oo", [(40, 1024, 96, R), (40, 1024, 96, Cm), (12, 4096, 64, R),
+                                                (64, 2304, 36, Cm)])
+def test_q8_gemm_depth_dealt_to_wavefronts_zero_points(ctx, rows, depth, cols, oo):
+    """The same route with two different zero points far from 128, a bias per result row and a clamp:
+    the operands change roles with the result's order (the filter is the one along the result's
+    contiguous direction), the zero points and the bias must follow.  Multiplier and bias are taken
+    from the oracle's accumulators so that the outputs are not saturated bytes."""
+    rng = np.random.default_rng(rows + depth + cols + oo)
+    L = rng.integers(0, 256, (1, rows, depth), dtype=np.uint8)
+    Rr = rng.integers(0, 256, (1, depth, cols), dtype=np.uint8)
+    l, r = as_major(L, R), as_major(Rr, Cm)
+    for (lzp, rzp) in ((23, 201), (250, 7)):
+        acc = orc.q8_gemm_i32(l, r, 1, rows, cols, depth, -lzp, -rzp, R, Cm, oo, True, True).astype(np.float64)
+        # (zero points far from the data's mean put the accumulators dozens of standard deviations
+        # from zero: the bias takes the mean out, row by row with a spread of its own)
+        sigma = float(acc.std())
+        bias = (-np.round(acc.mean()) + rng.integers(-int(2 * sigma), int(2 * sigma), rows)).astype(np.int32)
+        mult, rshift = mh.quantize_multiplier(min(100.0 / (4 * sigma), 0.99))
+        zp = 131
+        want8 = orc.q8_gemm_u8(l, r, 1, rows, cols, depth, -lzp, -rzp, bias, mult, -rshift, zp, 5, 250,
+                               R, Cm, oo, True, True)
+        got8 = gemm_u8_host(ctx, l, R, r, Cm, oo, 1, rows, depth, cols, True, True, -lzp, -rzp, bias,
+                            mult, -rshift, zp, 5, 250)
+        assert ctx.last_plan().kernel.startswith("q8_conv_ks"), ctx.last_plan()
+        np.testing.assert_array_equal(got8, want8)
+        assert len(np.unique(want8)) > 16 and ((want8 == 5) | (want8 == 250)).mean() < 0.5
+
+
 # Shapes on the boundaries between the one-launch kernels under the normal dispatch: the
 # eight-wavefront kernel ahead of the one-launch and the resident-tile kernels (one round of
 # 128 x 128 tiles, k >= 512; k-contiguous against the one-launch kernel from k = 1024), the
