@@ -530,6 +530,19 @@ def bench_other(ctx, mh, torch):
         out.append({"workload": "q8_matmul_%dx%dx%d" % (m, kk, n), "call_ms": round(whole, 4),
                     "kernel": ctx.last_plan().kernel, "launches": ctx.last_plan().launches})
 
+    # few rows against transposed weights (RowMajor . ColMajor, a FullyConnected-like batch): the depth
+    # dealt to wavefronts, 32 x 32 tiles
+    for (m, kk, n) in ((32, 4096, 4096), (64, 2048, 1024)):
+        A, B = u8(m, kk), u8(n, kk)
+        C = torch.empty((m, n), dtype=torch.uint8, device="cuda")
+        e = mh.quantize_multiplier(min(0.9, 40.0 / (74.0 * 74.0 * kk ** 0.5)))
+        torch.cuda.synchronize()
+        whole, k = time_kernel(ctx, bind(ctx,
+            "mace_hip_gemm_q8_u8", A.data_ptr(), 0, B.data_ptr(), 1, C.data_ptr(), 0, 1, m, kk, n, 1,
+            1, -131, -122, None, e[0], -e[1], 128, 0, 255))
+        out.append({"workload": "q8_matmul_%dx%dx%d_rhs_colmajor" % (m, kk, n), "call_ms": round(whole, 4),
+                    "kernel": ctx.last_plan().kernel, "launches": ctx.last_plan().launches})
+
     # config 5 with the raw int32 result (MatMulFixpointImpl<..., int32_t>): 4096^3, 256 MiB less
     # to hold than 8192^3 and the same kernel
     n = 4096
