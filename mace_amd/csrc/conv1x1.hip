@@ -1125,8 +1125,9 @@ int mh_q8_gemm_depth_split(mace_hip_ctx *ctx, const uint8_t *lhs, const uint8_t 
   *taken = false;
   if (!lhs || !rhs || !out || rows <= 0 || cols <= 0 || depth <= 0 || rows >= (1 << 24) ||
       cols >= (1 << 24) || depth >= (1 << 24) || lhs_offset > 0 || lhs_offset < -255 ||
-      rhs_offset > 0 || rhs_offset < -255)
-    return MACE_HIP_SUCCESS;
+      rhs_offset > 0 || rhs_offset < -255 ||
+      (out_order != MACE_HIP_ROW_MAJOR && out_order != MACE_HIP_COL_MAJOR))
+    return MACE_HIP_SUCCESS;   // (the general path reports what is invalid)
   const bool x_is_lhs = out_order == MACE_HIP_COL_MAJOR;
   const uint8_t *x = x_is_lhs ? lhs : rhs, *y = x_is_lhs ? rhs : lhs;
   const int64_t xn = x_is_lhs ? rows : cols, yn = x_is_lhs ? cols : rows;
