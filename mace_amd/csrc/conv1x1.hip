@@ -1010,7 +1010,8 @@ int conv_rows(mace_hip_ctx *ctx, const uint8_t *input, const uint8_t *filter, co
 // From 9 blocks on: 56 x 56 x 64 -> 64 (9 blocks) 8.5 -> 5.2, 28 x 28 x 64 -> 128 8.6 -> 5.2.  A 1 x 1 filter
 // read in place has the one-launch GEMM kernel to beat: 7 x 7 x 1024 -> 1024 8.8 -> 6.7, 14 x 14 x 640 ->
 // 128 (10 blocks) 6.9 -> 6.0, but 14 x 14 x 512 -> 512 (8 blocks) 6.6 -> 6.9: from 10 blocks there, up to
-// one tile per CU (7 x 7 x 1024 -> 1024 at batch 4, 224 tiles: 8.7 -> 7.1).
+// one tile per CU (7 x 7 x 1024 -> 1024 at batch 4, 224 tiles: 8.7 -> 7.1; with 384 - 512 tiles 48 of 60
+// k-contiguous GEMM shapes of a sweep lose, e.g. 128 x 4096 x 4096 17.9 -> 22.4, 256 x 1024 x 2048 8.7 -> 10.5).
 int conv_ksplit(mace_hip_ctx *ctx, const uint8_t *input, const uint8_t *filter, const int32_t *bias,
                 int64_t n, int64_t in_h, int64_t in_w, int64_t cin, int64_t cout, int64_t k_h,
                 int64_t k_w, int stride_h, int stride_w, int pad_top, int pad_left, int64_t out_h,
